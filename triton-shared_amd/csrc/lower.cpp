@@ -1,0 +1,837 @@
+// TTIR -> structured program.
+//
+// Restates, for structured (non-gather, non-wraparound) accesses:
+//   * tts::PtrAnalysis / PtrState  lib/AnalysisStructured/PtrAnalysis.cpp:276-503
+//     (addState), :539-625 (mulState), :901-1100 (make_range, expand_dims,
+//     broadcast, splat, addptr, const splat), :1200-1303 (visitOperand dispatch),
+//     :1480-1602 (loop-carried pointer state becomes loop-carried offsets/strides),
+//     :1672-1733 / :1813-1862 (load / store rewriting);
+//   * triton::MaskState  lib/Analysis/MaskAnalysis.cpp:32-59 (dispatch), :181-222
+//     (add), :269-286 (min), :288-338 (constants, scalars), :461-603 (cmp; the
+//     max(min(end, n), start) - start rule at :568-585), :696-846 (make_range,
+//     broadcast, splat, expand_dims);
+//   * the op lowering table of include/triton-shared/Conversion/
+//     TritonArithToLinalg/ConversionPatterns.hpp: splat :629-650, broadcast
+//     :674-719, expand_dims :721-749, make_range :764-805, matmul :1128-1201,
+//     reduce :1203-1440, dense constant :1919-1939; elementwise arith/math ops
+//     become one whole-tile map each (TritonArithToLinalg.cpp:104).
+// Ops whose results feed only address or mask computations are dropped at the
+// end, as the reference's final remove-dead-values/CSE/canonicalize does
+// (TritonToLinalgExperimentalPass.cpp:80-86).
+#include <cmath>
+#include <cstring>
+#include <functional>
+#include <set>
+
+#include "structured.h"
+
+namespace tts {
+
+namespace {
+
+struct PtrState {   // PtrAnalysis.h:52-129, structured fields only
+  int source = -1;  // kernel argument index
+  int scalar = -1;  // index expr
+  std::vector<int> offsets, strides;
+  std::vector<int64_t> sizes;
+  size_t rank() const { return sizes.size(); }
+};
+
+struct MaskState {  // MaskAnalysis.h:63-180
+  int start = -1, end = -1, scalar = -1;
+  std::vector<int> dims;
+  size_t rank() const { return dims.size(); }
+};
+
+struct Def {
+  const Op *op = nullptr;  // defining op, null for function / region arguments
+  int index = 0;           // result number
+  Type type;
+  int func_arg = -1;       // >= 0 for kernel arguments
+};
+
+static double parse_float_literal(const std::string &lit, const std::string &elem) {
+  // MLIR prints non-finite and some exact values as hex bit patterns.
+  if (lit.rfind("0x", 0) == 0 || lit.rfind("0X", 0) == 0) {
+    uint64_t bits = std::stoull(lit, nullptr, 16);
+    if (elem == "f32") {
+      uint32_t b = (uint32_t)bits;
+      float f;
+      memcpy(&f, &b, 4);
+      return f;
+    }
+    if (elem == "f64") {
+      double d;
+      memcpy(&d, &bits, 8);
+      return d;
+    }
+    if (elem == "f16") {
+      uint32_t h = (uint32_t)bits, s = (h >> 15) & 1, e = (h >> 10) & 31, m = h & 1023;
+      double v = e == 31 ? (m ? NAN : INFINITY) : e == 0 ? std::ldexp((double)m, -24) : std::ldexp(1024.0 + m, (int)e - 25);
+      return s ? -v : v;
+    }
+    if (elem == "bf16") {
+      uint32_t b = (uint32_t)bits << 16;
+      float f;
+      memcpy(&f, &b, 4);
+      return f;
+    }
+    throw Unsupported("hex float literal of type " + elem);
+  }
+  return std::stod(lit);
+}
+
+class Lowerer {
+ public:
+  explicit Lowerer(const Func &f) : f_(f) {}
+
+  Program run() {
+    P.name = f_.name;
+    P.arg_names = f_.arg_names;
+    P.arg_types = f_.arg_types;
+    for (size_t i = 0; i < f_.arg_names.size(); i++) {
+      Def d;
+      d.type = f_.arg_types[i];
+      d.func_arg = (int)i;
+      if (d.type.is_tensor) throw Unsupported("tensor-typed kernel argument");
+      defs_[f_.arg_names[i]] = d;
+    }
+    cur_ = &P.body;
+    lower_block(f_.body);
+    dce();
+    return std::move(P);
+  }
+
+ private:
+  const Func &f_;
+  Program P;
+  std::map<std::string, Def> defs_;
+  std::map<std::string, int> int_memo_;       // scalar integer SSA name -> expr
+  std::map<std::string, PtrState> known_ptr_; // loop-carried / loop-result pointer states
+  std::map<std::string, int> data_;           // SSA name -> value id
+  std::vector<SOp> *cur_ = nullptr;
+
+  // ---------------------------------------------------------------- helpers
+  const Def &def(const std::string &name) const {
+    auto it = defs_.find(name);
+    if (it == defs_.end()) throw Unsupported("use of unknown SSA value " + name);
+    return it->second;
+  }
+  int c64(int64_t v) { return P.pool.constant(v, 64); }
+
+  int new_value(const Type &t) {
+    Value v;
+    v.shape = t.shape;
+    v.dtype = t.elem;
+    P.values.push_back(v);
+    return (int)P.values.size() - 1;
+  }
+
+  static Type result_type(const Op &op) {
+    if (!op.result_types.empty()) return op.result_types[0];
+    if (op.types.empty()) throw Unsupported("cannot infer the result type of " + op.name);
+    if (op.name == "tt.load") {
+      Type t = op.types[0];
+      t.ptr = false;
+      return t;
+    }
+    if (op.name == "arith.cmpi" || op.name == "arith.cmpf") {
+      Type t = op.types[0];
+      t.elem = "i1";
+      return t;
+    }
+    if (op.name == "tt.addptr") return op.types[0];
+    return op.types.back();
+  }
+
+  // ------------------------------------------------- scalar integer values
+  int int_of(const std::string &name) {
+    auto it = int_memo_.find(name);
+    if (it != int_memo_.end()) return it->second;
+    const Def &d = def(name);
+    if (d.type.is_tensor || !d.type.is_int()) throw Unsupported(name + " is not a scalar integer");
+    int bits = (d.type.elem == "i64" || d.type.elem == "index") ? 64 : 32;
+    int e = -1;
+    if (d.func_arg >= 0) {
+      e = P.pool.arg(d.func_arg, bits);
+    } else if (!d.op) {
+      throw Unsupported("integer region argument " + name + " has no known value");
+    } else {
+      const Op &op = *d.op;
+      auto opnd = [&](int i) { return int_of(op.operands.at(i)); };
+      static const std::map<std::string, EK> bins = {
+          {"arith.addi", EK::Add}, {"arith.subi", EK::Sub},   {"arith.muli", EK::Mul}, {"arith.divsi", EK::DivS},
+          {"arith.remsi", EK::RemS}, {"arith.minsi", EK::MinS}, {"arith.maxsi", EK::MaxS}};
+      if (op.name == "arith.constant") {
+        if (op.literal == "true") e = P.pool.constant(1, 32);
+        else if (op.literal == "false") e = P.pool.constant(0, 32);
+        else e = P.pool.constant(std::stoll(op.literal), bits);
+      } else if (op.name == "tt.get_program_id" || op.name == "tt.get_num_programs") {
+        int axis = op.words.empty() ? 0 : (op.words[0] == "x" ? 0 : op.words[0] == "y" ? 1 : 2);
+        e = op.name == "tt.get_program_id" ? P.pool.pid(axis) : P.pool.nprog(axis);
+      } else if (bins.count(op.name)) {
+        e = P.pool.bin(bins.at(op.name), opnd(0), opnd(1));
+      } else if (op.name == "arith.extsi" || op.name == "arith.index_cast") {
+        int a = opnd(0);
+        e = bits == 64 ? P.pool.sext(a) : P.pool.trunc(a);
+      } else if (op.name == "arith.trunci") {
+        e = P.pool.trunc(opnd(0));
+      } else if (op.name == "arith.select") {
+        const Def &c = def(op.operands[0]);
+        if (!c.op || c.op->name != "arith.cmpi") throw Unsupported("scalar select on a non-cmpi condition");
+        static const std::map<std::string, int> preds = {{"slt", 0}, {"sle", 1}, {"sgt", 2}, {"sge", 3}, {"eq", 4}, {"ne", 5}};
+        auto pit = preds.find(c.op->words.at(0));
+        if (pit == preds.end()) throw Unsupported("scalar cmpi predicate " + c.op->words[0]);
+        e = P.pool.cmpsel(pit->second, int_of(c.op->operands[0]), int_of(c.op->operands[1]), opnd(1), opnd(2));
+      } else {
+        throw Unsupported("scalar integer op " + op.name + " (line " + std::to_string(op.line) + ")");
+      }
+    }
+    int_memo_[name] = e;
+    return e;
+  }
+
+  // ------------------------------------------------------------ PtrAnalysis
+  PtrState add_state(const PtrState &l, const PtrState &r, const Op &op) {  // PtrAnalysis.cpp:276-503
+    if (l.rank() != r.rank()) throw Unsupported("PtrAnalysis: rank mismatch at line " + std::to_string(op.line));
+    if (l.source >= 0 && r.source >= 0) throw Unsupported("PtrAnalysis: adding two states that both have a base pointer");
+    PtrState s;
+    s.source = l.source >= 0 ? l.source : r.source;
+    if (l.scalar >= 0 && r.scalar >= 0) s.scalar = P.pool.bin(EK::Add, l.scalar, r.scalar);
+    else if (l.rank() == 0) s.scalar = l.scalar >= 0 ? l.scalar : r.scalar;
+    for (size_t i = 0; i < l.rank(); i++) {
+      s.offsets.push_back(P.pool.bin(EK::Add, l.offsets[i], r.offsets[i]));
+      s.strides.push_back(P.pool.bin(EK::Add, l.strides[i], r.strides[i]));
+      s.sizes.push_back(l.sizes[i]);
+    }
+    return s;
+  }
+
+  PtrState mul_state(const PtrState &lhs, const PtrState &rhs, const Op &op) {  // PtrAnalysis.cpp:539-625
+    if (lhs.source >= 0 || rhs.source >= 0) throw Unsupported("PtrAnalysis: multiplying a base pointer");
+    if (lhs.scalar < 0 && rhs.scalar < 0)
+      throw Unsupported("PtrAnalysis: product of two non-scalar index tensors (line " + std::to_string(op.line) + ")");
+    const PtrState *l = &lhs, *r = &rhs;
+    if (r->scalar < 0 && l->scalar >= 0) std::swap(l, r);
+    PtrState s;
+    if (lhs.scalar >= 0 && rhs.scalar >= 0) s.scalar = P.pool.bin(EK::Mul, lhs.scalar, rhs.scalar);
+    for (size_t i = 0; i < l->rank(); i++) {
+      s.offsets.push_back(P.pool.bin(EK::Mul, l->offsets[i], r->scalar));
+      s.strides.push_back(P.pool.bin(EK::Mul, l->strides[i], r->scalar));
+      s.sizes.push_back(l->sizes[i]);
+    }
+    return s;
+  }
+
+  PtrState visit(const std::string &name) {  // PtrAnalysis.cpp:1200-1303
+    auto kp = known_ptr_.find(name);
+    if (kp != known_ptr_.end()) return kp->second;
+    const Def &d = def(name);
+    PtrState s;
+    if (!d.type.is_tensor && d.type.is_int()) {
+      s.scalar = P.pool.to_index(int_of(name));
+      return s;
+    }
+    if (!d.type.is_tensor && d.type.ptr) {
+      if (d.func_arg >= 0) {
+        s.source = d.func_arg;
+        return s;
+      }
+      if (d.op && d.op->name == "tt.addptr") return visit_addptr(*d.op);
+      throw Unsupported("scalar pointer produced by " + (d.op ? d.op->name : std::string("a region argument")));
+    }
+    if (!d.op) throw Unsupported("PtrAnalysis: tensor region argument " + name + " without a known state");
+    const Op &op = *d.op;
+    if (op.name == "arith.addi") return add_state(visit(op.operands[0]), visit(op.operands[1]), op);
+    if (op.name == "arith.muli") return mul_state(visit(op.operands[0]), visit(op.operands[1]), op);
+    if (op.name == "tt.addptr") return visit_addptr(op);
+    if (op.name == "arith.extsi") return visit(op.operands[0]);
+    if (op.name == "tt.make_range") {  // :901-919
+      int64_t start = std::stoll(op.attrs.at("start")), end = std::stoll(op.attrs.at("end"));
+      int64_t n = d.type.shape.at(0);
+      if ((end - start + n - 1) / n != 1) throw Unsupported("make_range with stride != 1");
+      s.offsets.push_back(c64(start));
+      s.sizes.push_back(n);
+      s.strides.push_back(c64(1));
+      return s;
+    }
+    if (op.name == "tt.expand_dims") {  // :921-952
+      s = visit(op.operands[0]);
+      int axis = std::stoi(op.attrs.at("axis"));
+      s.offsets.insert(s.offsets.begin() + axis, c64(0));
+      s.sizes.insert(s.sizes.begin() + axis, 1);
+      s.strides.insert(s.strides.begin() + axis, c64(0));
+      return s;
+    }
+    if (op.name == "tt.broadcast") {  // :954-989
+      s = visit(op.operands[0]);
+      const Type &src = def(op.operands[0]).type;
+      for (size_t i = 0; i < d.type.shape.size(); i++)
+        if (src.shape[i] < d.type.shape[i]) s.sizes[i] = d.type.shape[i];
+      return s;
+    }
+    if (op.name == "tt.splat") {  // :991-1030
+      s = visit(op.operands[0]);
+      if (s.rank() != 0) throw Unsupported("splat of a non-scalar");
+      for (auto n : d.type.shape) {
+        s.offsets.push_back(c64(0));
+        s.sizes.push_back(n);
+        s.strides.push_back(c64(0));
+      }
+      if (s.scalar >= 0) s.offsets[0] = s.scalar;
+      return s;
+    }
+    if (op.name == "arith.constant") {  // :1068-1100
+      int64_t v = dense_int(op);
+      s.scalar = c64(v);
+      for (size_t i = 0; i < d.type.shape.size(); i++) {
+        s.offsets.push_back(i == 0 ? s.scalar : c64(0));
+        s.sizes.push_back(d.type.shape[i]);
+        s.strides.push_back(c64(0));
+      }
+      return s;
+    }
+    if (op.name == "arith.remsi")
+      throw Unsupported("PtrAnalysis: modulo (wraparound) addressing is not supported by this backend");
+    throw Unsupported("PtrAnalysis: address computed by " + op.name + " (line " + std::to_string(op.line) +
+                      ") is not a structured access");
+  }
+
+  PtrState visit_addptr(const Op &op) {  // :1032-1066
+    PtrState p = visit(op.operands[0]);
+    PtrState o = visit(op.operands[1]);
+    if (p.source < 0) throw Unsupported("tt.addptr whose pointer operand has no base");
+    return add_state(p, o, op);
+  }
+
+  static int64_t dense_int(const Op &op) {
+    const std::string &lit = op.literal;
+    if (lit.rfind("dense<", 0) != 0) throw Unsupported("non-splat constant " + lit);
+    std::string in = lit.substr(6, lit.size() - 7);
+    if (in == "true") return 1;
+    if (in == "false") return 0;
+    if (in.find('[') != std::string::npos) throw Unsupported("non-splat dense constant");
+    return std::stoll(in);
+  }
+
+  // ----------------------------------------------------------- MaskAnalysis
+  MaskState mask_parse(const std::string &name) {  // MaskAnalysis.cpp:32-59
+    const Def &d = def(name);
+    MaskState m;
+    if (d.op && d.op->name == "arith.constant") {  // :288-310
+      m.scalar = d.type.is_tensor ? c64(dense_int(*d.op)) : P.pool.to_index(int_of(name));
+      return m;
+    }
+    if (!d.type.is_tensor && d.type.is_int()) {  // :312-324
+      if (d.type.elem == "i1") throw Unsupported("MaskAnalysis: scalar boolean in a mask is not supported");
+      m.scalar = P.pool.to_index(int_of(name));
+      return m;
+    }
+    if (!d.op) throw Unsupported("MaskAnalysis: loop-carried mask operand");
+    const Op &op = *d.op;
+    if (op.name == "arith.addi") {  // :181-222, :340-353
+      MaskState l = mask_parse(op.operands[0]), r = mask_parse(op.operands[1]);
+      if ((l.scalar >= 0) == (r.scalar >= 0)) throw Unsupported("MaskAnalysis: add needs exactly one scalar side");
+      const MaskState &t = l.scalar >= 0 ? r : l;
+      int sc = l.scalar >= 0 ? l.scalar : r.scalar;
+      if (t.start < 0) throw Unsupported("MaskAnalysis: add on a state without a range");
+      m.start = P.pool.bin(EK::Add, t.start, sc);
+      m.end = P.pool.bin(EK::Add, t.end, sc);
+      m.dims = t.dims;
+      return m;
+    }
+    if (op.name == "arith.andi") {  // :355-453, :269-286
+      MaskState l = mask_parse(op.operands[0]), r = mask_parse(op.operands[1]);
+      if (l.scalar >= 0 || r.scalar >= 0) throw Unsupported("MaskAnalysis: conjunction with a scalar condition");
+      if (l.rank() != r.rank()) throw Unsupported("MaskAnalysis: conjunction of different ranks");
+      for (size_t i = 0; i < l.rank(); i++) m.dims.push_back(P.pool.bin(EK::MinS, l.dims[i], r.dims[i]));
+      return m;
+    }
+    if (op.name == "arith.cmpi") return mask_cmp(op);
+    if (op.name == "arith.extsi") return mask_parse(op.operands[0]);
+    if (op.name == "tt.make_range") {  // :696-720
+      int64_t start = std::stoll(op.attrs.at("start")), end = std::stoll(op.attrs.at("end"));
+      int64_t n = d.type.shape.at(0);
+      if ((end - start + n - 1) / n != 1) throw Unsupported("MaskAnalysis: make_range with stride != 1");
+      m.start = c64(start);
+      m.end = c64(end);
+      m.dims.push_back(c64(n));
+      return m;
+    }
+    if (op.name == "tt.broadcast") {  // :722-750
+      m = mask_parse(op.operands[0]);
+      const Type &src = def(op.operands[0]).type;
+      for (size_t i = 0; i < d.type.shape.size(); i++)
+        if (src.shape[i] < d.type.shape[i]) m.dims[i] = c64(d.type.shape[i]);
+      return m;
+    }
+    if (op.name == "tt.splat") {  // :752-783
+      const Def &src = def(op.operands[0]);
+      if (src.type.is_tensor || !src.type.is_int()) throw Unsupported("MaskAnalysis: splat of a non-integer");
+      m = mask_parse(op.operands[0]);
+      for (auto n : d.type.shape) m.dims.push_back(c64(n));
+      return m;
+    }
+    if (op.name == "tt.expand_dims") {  // :785-846
+      m = mask_parse(op.operands[0]);
+      int axis = std::stoi(op.attrs.at("axis"));
+      m.dims.insert(m.dims.begin() + axis, c64(1));
+      return m;
+    }
+    throw Unsupported("MaskAnalysis: mask computed by " + op.name + " (line " + std::to_string(op.line) + ")");
+  }
+
+  MaskState mask_cmp(const Op &op) {  // MaskAnalysis.cpp:461-603
+    const std::string &pred = op.words.at(0);
+    if (pred != "slt" && pred != "ult" && pred != "sge") throw Unsupported("MaskAnalysis: cmpi " + pred);
+    MaskState l = mask_parse(op.operands[0]), r = mask_parse(op.operands[1]);
+    int64_t zero;
+    if (pred == "sge" && !(r.scalar >= 0 && P.pool.is_const(r.scalar, &zero) && zero == 0))
+      throw Unsupported("MaskAnalysis: sge against a non-zero bound");
+    if (l.scalar >= 0) throw Unsupported("MaskAnalysis: comparison of two scalars");
+    if (r.scalar < 0) throw Unsupported("MaskAnalysis: comparison against a non-scalar");
+    int cmp_dim = -1;
+    for (size_t i = 0; i < l.rank(); i++) {
+      int64_t v;
+      if (!(P.pool.is_const(l.dims[i], &v) && v == 1)) {
+        if (cmp_dim != -1) throw Unsupported("MaskAnalysis: cmpi over more than one non-unit dimension");
+        cmp_dim = (int)i;
+      }
+    }
+    if (cmp_dim < 0) throw Unsupported("MaskAnalysis: cmpi over a unit tensor");
+    int new_dim;
+    if (pred == "sge") {
+      new_dim = l.dims[cmp_dim];
+    } else {
+      if (l.start < 0) throw Unsupported("MaskAnalysis: cmpi lhs without a range");
+      // :568-585  an entirely masked-off block must give 0, hence the max with start
+      int new_end = P.pool.bin(EK::MinS, l.end, r.scalar);
+      new_end = P.pool.bin(EK::MaxS, new_end, l.start);
+      new_dim = P.pool.bin(EK::Sub, new_end, l.start);
+    }
+    MaskState m;
+    m.dims = l.dims;
+    m.dims[cmp_dim] = new_dim;
+    return m;
+  }
+
+  // --------------------------------------------------------- data lowering
+  int data_of(const std::string &name) {
+    auto it = data_.find(name);
+    if (it != data_.end()) return it->second;
+    const Def &d = def(name);
+    if (!d.type.is_tensor && d.type.is_int()) {  // integer scalar used as data
+      SOp s;
+      s.kind = SK::FromIndex;
+      s.expr = int_of(name);
+      s.result = new_value(d.type);
+      cur_->push_back(s);
+      // not memoised across scopes: an expression may depend on a loop's state
+      return s.result;
+    }
+    if (!d.type.is_tensor && d.type.is_float() && d.func_arg >= 0) {
+      SOp s;
+      s.kind = SK::ScalarArg;
+      s.ival = d.func_arg;
+      s.result = new_value(d.type);
+      cur_->push_back(s);
+      data_[name] = s.result;
+      return s.result;
+    }
+    throw Unsupported("value " + name + " (" + d.type.str() + ") is not available as data");
+  }
+
+  Access make_access(const PtrState &st, const Type &elem_type) {
+    if (st.source < 0) throw Unsupported("memory access without a base pointer");
+    Access a;
+    a.base_arg = st.source;
+    a.elem = elem_type.elem;
+    a.sizes = st.sizes;
+    a.offsets = st.offsets;
+    a.strides = st.strides;
+    if (st.rank() == 0) a.offsets.push_back(st.scalar >= 0 ? st.scalar : c64(0));
+    return a;
+  }
+
+  void scalar_other(const std::string &name, Access &a) {  // TritonStructuredOps.cpp:38-98
+    const Def &d = def(name);
+    const Op *op = d.op;
+    if (op && op->name == "tt.splat") op = def(op->operands[0]).op;
+    if (!op || op->name != "arith.constant") throw Unsupported("masked load whose `other` is not a constant");
+    std::string lit = op->literal;
+    if (lit.rfind("dense<", 0) == 0) lit = lit.substr(6, lit.size() - 7);
+    a.has_other = true;
+    if (d.type.is_float()) a.other_f = parse_float_literal(lit, d.type.elem);
+    else a.other_i = lit == "true" ? 1 : lit == "false" ? 0 : std::stoll(lit);
+  }
+
+  void lower_load(const Op &op) {
+    const Def &p = def(op.operands[0]);
+    Type rt = result_type(op);
+    SOp s;
+    PtrState st = visit(op.operands[0]);
+    s.acc = make_access(st, rt);
+    if (!p.type.is_tensor) {
+      if (op.operands.size() > 1) throw Unsupported("masked scalar load");
+      s.kind = SK::ScalarLoad;
+    } else {
+      s.kind = SK::Load;
+      if (op.operands.size() >= 2) {
+        MaskState m = mask_parse(op.operands[1]);
+        if (m.rank() != st.rank()) throw Unsupported("mask rank differs from pointer rank");
+        s.acc.dims = m.dims;
+      }
+      if (op.operands.size() >= 3) scalar_other(op.operands[2], s.acc);
+    }
+    s.result = new_value(rt);
+    data_[op.results[0]] = s.result;
+    cur_->push_back(s);
+  }
+
+  void lower_store(const Op &op) {
+    const Def &p = def(op.operands[0]);
+    SOp s;
+    PtrState st = visit(op.operands[0]);
+    Type vt = def(op.operands[1]).type;
+    s.acc = make_access(st, vt);
+    s.operands.push_back(data_of(op.operands[1]));
+    if (!p.type.is_tensor) {
+      if (op.operands.size() > 2) throw Unsupported("masked scalar store");
+      s.kind = SK::ScalarStore;
+    } else {
+      s.kind = SK::Store;
+      if (op.operands.size() >= 3) {
+        MaskState m = mask_parse(op.operands[2]);
+        if (m.rank() != st.rank()) throw Unsupported("mask rank differs from pointer rank");
+        s.acc.dims = m.dims;
+      }
+    }
+    cur_->push_back(s);
+  }
+
+  void emit_simple(const Op &op, SK kind, const std::string &name, std::vector<std::string> operand_names) {
+    SOp s;
+    s.kind = kind;
+    s.name = name;
+    for (auto &n : operand_names) s.operands.push_back(data_of(n));
+    s.result = new_value(result_type(op));
+    data_[op.results[0]] = s.result;
+    cur_->push_back(s);
+  }
+
+  void lower_for(const Op &op) {  // PtrAnalysis.cpp:1480-1602 + TritonToStructuredPass.cpp:72-171
+    SOp s;
+    s.kind = SK::For;
+    s.loop = P.num_loops++;
+    s.lb = int_of(op.operands[0]);
+    s.ub = int_of(op.operands[1]);
+    s.step = int_of(op.operands[2]);
+    const Def &lbd = def(op.operands[0]);
+    int iv_bits = (lbd.type.elem == "i64" || lbd.type.elem == "index") ? 64 : 32;
+    {
+      Def d;
+      d.type = lbd.type;
+      defs_[op.iv] = d;
+      int_memo_[op.iv] = P.pool.iv(s.loop, iv_bits);
+    }
+    struct Carried { int kind; PtrState st; size_t first_slot; int tile_index; };  // 0 ptr, 1 int, 2 tile
+    std::vector<Carried> carried;
+    for (size_t j = 0; j < op.iter_names.size(); j++) {
+      const Type &t = op.result_types[j];
+      Def d;
+      d.type = t;
+      defs_[op.iter_names[j]] = d;
+      Carried c{};
+      if (t.ptr) {
+        c.kind = 0;
+        PtrState init = visit(op.iter_inits[j]);
+        c.first_slot = s.int_iters.size();
+        PtrState inside = init;
+        auto carry = [&](int init_expr) {
+          IntIter it;
+          int slot = (int)s.int_iters.size();
+          it.init = init_expr;
+          it.iter_expr = P.pool.iter(s.loop, slot, 64);
+          it.result_expr = P.pool.result(s.loop, slot, 64);
+          s.int_iters.push_back(it);
+          return it.iter_expr;
+        };
+        if (init.rank() == 0) {
+          inside.scalar = carry(init.scalar >= 0 ? init.scalar : c64(0));
+        } else {
+          for (auto &o : inside.offsets) o = carry(o);
+          for (auto &st : inside.strides) st = carry(st);
+        }
+        c.st = inside;
+        known_ptr_[op.iter_names[j]] = inside;
+      } else if (!t.is_tensor && t.is_int()) {
+        c.kind = 1;
+        c.first_slot = s.int_iters.size();
+        int bits = (t.elem == "i64" || t.elem == "index") ? 64 : 32;
+        IntIter it;
+        it.init = int_of(op.iter_inits[j]);
+        it.iter_expr = P.pool.iter(s.loop, (int)c.first_slot, bits);
+        it.result_expr = P.pool.result(s.loop, (int)c.first_slot, bits);
+        s.int_iters.push_back(it);
+        int_memo_[op.iter_names[j]] = it.iter_expr;
+      } else if (t.is_tensor && t.is_int()) {
+        throw Unsupported("loop-carried integer tensors are not supported");
+      } else {
+        c.kind = 2;
+        c.tile_index = (int)s.tile_args.size();
+        s.tile_inits.push_back(data_of(op.iter_inits[j]));
+        int v = new_value(t);
+        s.tile_args.push_back(v);
+        data_[op.iter_names[j]] = v;
+      }
+      carried.push_back(c);
+    }
+    // body
+    std::vector<SOp> *saved = cur_;
+    cur_ = &s.body;
+    const Block &body = op.regions.at(0);
+    const Op *yield = nullptr;
+    for (auto &bop : body.ops) {
+      if (bop->name == "scf.yield") {
+        yield = bop.get();
+        break;
+      }
+      lower_op(*bop);
+    }
+    if (!op.iter_names.empty()) {
+      if (!yield || yield->operands.size() != op.iter_names.size()) throw Unsupported("scf.for without a matching scf.yield");
+      s.tile_yields.resize(s.tile_args.size());
+      for (size_t j = 0; j < carried.size(); j++) {
+        const Carried &c = carried[j];
+        const std::string &y = yield->operands[j];
+        if (c.kind == 0) {
+          PtrState ns = visit(y);
+          if (ns.source != c.st.source || ns.sizes != c.st.sizes)
+            throw Unsupported("loop-carried pointer changes its base or block shape");
+          size_t slot = c.first_slot;
+          if (ns.rank() == 0) {
+            s.int_iters[slot].next = ns.scalar;
+          } else {
+            for (auto o : ns.offsets) s.int_iters[slot++].next = o;
+            for (auto st : ns.strides) s.int_iters[slot++].next = st;
+          }
+        } else if (c.kind == 1) {
+          s.int_iters[c.first_slot].next = int_of(y);
+        } else {
+          s.tile_yields[c.tile_index] = data_of(y);
+        }
+      }
+    }
+    cur_ = saved;
+    // results
+    s.results.resize(s.tile_args.size());
+    for (size_t j = 0; j < carried.size(); j++) {
+      const Carried &c = carried[j];
+      const std::string &rname = op.results.at(j);
+      Def d;
+      d.type = op.result_types[j];
+      d.op = &op;
+      d.index = (int)j;
+      defs_[rname] = d;
+      if (c.kind == 0) {
+        PtrState after = c.st;
+        size_t slot = c.first_slot;
+        if (after.rank() == 0) {
+          after.scalar = s.int_iters[slot].result_expr;
+        } else {
+          for (auto &o : after.offsets) o = s.int_iters[slot++].result_expr;
+          for (auto &st : after.strides) st = s.int_iters[slot++].result_expr;
+        }
+        known_ptr_[rname] = after;
+      } else if (c.kind == 1) {
+        int_memo_[rname] = s.int_iters[c.first_slot].result_expr;
+      } else {
+        int v = new_value(d.type);
+        s.results[c.tile_index] = v;
+        data_[rname] = v;
+      }
+    }
+    cur_->push_back(std::move(s));
+  }
+
+  void lower_reduce(const Op &op) {  // ConversionPatterns.hpp:1203-1440
+    if (op.operands.size() != 1 || op.regions.size() != 1) throw Unsupported("tt.reduce with several operands (argmin/argmax)");
+    const Block &rb = op.regions[0];
+    if (rb.ops.size() != 2 || rb.ops[1]->name != "tt.reduce.return") throw Unsupported("tt.reduce with a compound combiner");
+    const Op &comb = *rb.ops[0];
+    static const std::set<std::string> ok = {"arith.addf", "arith.addi", "arith.maxnumf", "arith.maximumf",
+                                             "arith.minnumf", "arith.minimumf", "arith.mulf", "arith.maxsi",
+                                             "arith.minsi", "arith.maxui", "arith.minui", "arith.ori",
+                                             "arith.andi", "arith.xori", "arith.muli"};
+    if (!ok.count(comb.name)) throw Unsupported("tt.reduce combiner " + comb.name);
+    std::set<std::string> ins(comb.operands.begin(), comb.operands.end());
+    if (comb.operands.size() != 2 || !ins.count(rb.arg_names.at(0)) || !ins.count(rb.arg_names.at(1)))
+      throw Unsupported("tt.reduce combiner does not combine the two block arguments");
+    SOp s;
+    s.kind = SK::Reduce;
+    s.name = comb.name;
+    s.axis = std::stoi(op.attrs.at("axis"));
+    s.operands.push_back(data_of(op.operands[0]));
+    s.result = new_value(result_type(op));
+    data_[op.results[0]] = s.result;
+    cur_->push_back(s);
+  }
+
+  void lower_constant(const Op &op) {
+    Type t = result_type(op);
+    if (!t.is_tensor && t.is_int()) return;  // reached through int_of on demand
+    SOp s;
+    s.kind = SK::Const;
+    std::string lit = op.literal;
+    if (t.is_tensor) {
+      if (lit.rfind("dense<", 0) != 0) throw Unsupported("non-dense tensor constant");
+      lit = lit.substr(6, lit.size() - 7);
+      if (lit.find('[') != std::string::npos) throw Unsupported("non-splat tensor constant");
+    }
+    if (t.is_float()) s.fval = parse_float_literal(lit, t.elem);
+    else s.ival = lit == "true" ? 1 : lit == "false" ? 0 : std::stoll(lit);
+    s.result = new_value(t);
+    data_[op.results[0]] = s.result;
+    cur_->push_back(s);
+  }
+
+  void lower_op(const Op &op) {
+    // record definitions first so later uses can find types
+    if (op.name != "scf.for")
+      for (size_t i = 0; i < op.results.size(); i++) {
+        Def d;
+        d.op = &op;
+        d.index = (int)i;
+        d.type = result_type(op);
+        defs_[op.results[i]] = d;
+      }
+    const std::string &n = op.name;
+    if (n == "tt.return") return;
+    if (n == "scf.for") return lower_for(op);
+    if (n == "tt.load") return lower_load(op);
+    if (n == "tt.store") return lower_store(op);
+    if (n == "tt.reduce") return lower_reduce(op);
+    if (n == "arith.constant") return lower_constant(op);
+    if (op.results.size() != 1) throw Unsupported("operation " + n + " (line " + std::to_string(op.line) + ")");
+    Type rt = result_type(op);
+    if (rt.ptr) return;                          // address computation: PtrAnalysis reads it on demand
+    if (!rt.is_tensor && rt.is_int()) return;    // scalar integer: int_of reads it on demand
+    if (n == "tt.make_range") {
+      SOp s;
+      s.kind = SK::Iota;
+      s.ival = std::stoll(op.attrs.at("start"));
+      s.result = new_value(rt);
+      data_[op.results[0]] = s.result;
+      cur_->push_back(s);
+      return;
+    }
+    if (n == "tt.splat") return emit_simple(op, SK::Splat, "", {op.operands[0]});
+    if (n == "tt.broadcast") return emit_simple(op, SK::Broadcast, "", {op.operands[0]});
+    if (n == "tt.expand_dims") {
+      emit_simple(op, SK::ExpandDims, "", {op.operands[0]});
+      cur_->back().axis = std::stoi(op.attrs.at("axis"));
+      return;
+    }
+    if (n == "tt.dot") {  // ConversionPatterns.hpp:1128-1201
+      if (op.operands.size() != 3) throw Unsupported("tt.dot without an accumulator operand");
+      return emit_simple(op, SK::Dot, "", op.operands);
+    }
+    if (n.rfind("arith.", 0) == 0 || n.rfind("math.", 0) == 0) {
+      std::string name = n;
+      if (n == "arith.cmpi" || n == "arith.cmpf") name += "." + op.words.at(0);
+      return emit_simple(op, SK::Map, name, op.operands);
+    }
+    throw Unsupported("operation " + n + " (line " + std::to_string(op.line) + ") has no structured lowering");
+  }
+
+  void lower_block(const Block &b) {
+    for (auto &op : b.ops) lower_op(*op);
+  }
+
+  // ------------------------------------------------------------------ DCE
+  void dce() {
+    std::vector<char> live(P.values.size(), 0);
+    bool changed = true;
+    std::function<bool(std::vector<SOp> &)> mark = [&](std::vector<SOp> &ops) {
+      bool any_effect = false;
+      for (auto it = ops.rbegin(); it != ops.rend(); ++it) {
+        SOp &s = *it;
+        auto use = [&](int v) {
+          if (v >= 0 && !live[v]) {
+            live[v] = 1;
+            changed = true;
+          }
+        };
+        if (s.kind == SK::Store || s.kind == SK::ScalarStore) {
+          any_effect = true;
+          for (int v : s.operands) use(v);
+        } else if (s.kind == SK::For) {
+          bool eff = mark(s.body);
+          bool res_live = false;
+          for (int r : s.results) res_live |= (r >= 0 && live[r]);
+          if (eff || res_live) {
+            any_effect |= eff;
+            for (size_t j = 0; j < s.tile_args.size(); j++) {
+              // a carried tile matters if its result or its region value is read
+              if ((s.results[j] >= 0 && live[s.results[j]]) || live[s.tile_args[j]]) {
+                use(s.tile_yields[j]);
+                use(s.tile_inits[j]);
+                use(s.tile_args[j]);
+              }
+            }
+            mark(s.body);
+          }
+        } else if (s.result >= 0 && live[s.result]) {
+          for (int v : s.operands) use(v);
+        }
+      }
+      return any_effect;
+    };
+    while (changed) {
+      changed = false;
+      mark(P.body);
+    }
+    std::function<bool(std::vector<SOp> &)> sweep = [&](std::vector<SOp> &ops) {
+      bool keep_any = false;
+      std::vector<SOp> out;
+      for (auto &s : ops) {
+        bool keep;
+        if (s.kind == SK::Store || s.kind == SK::ScalarStore) keep = true;
+        else if (s.kind == SK::For) {
+          bool eff = sweep(s.body);
+          bool res_live = false;
+          for (int r : s.results) res_live |= (r >= 0 && live[r]);
+          keep = eff || res_live;
+          if (keep) {
+            // drop carried tiles nobody reads
+            std::vector<int> a, i, y, r;
+            for (size_t j = 0; j < s.tile_args.size(); j++)
+              if (live[s.tile_args[j]] || (s.results[j] >= 0 && live[s.results[j]])) {
+                a.push_back(s.tile_args[j]);
+                i.push_back(s.tile_inits[j]);
+                y.push_back(s.tile_yields[j]);
+                r.push_back(s.results[j]);
+              }
+            s.tile_args = a;
+            s.tile_inits = i;
+            s.tile_yields = y;
+            s.results = r;
+          }
+        } else keep = s.result >= 0 && live[s.result];
+        if (keep) {
+          out.push_back(std::move(s));
+          keep_any = true;
+        }
+      }
+      ops = std::move(out);
+      return keep_any;
+    };
+    sweep(P.body);
+  }
+};
+
+}  // namespace
+
+Program lower_ttir(const Func &f) { return Lowerer(f).run(); }
+
+}  // namespace tts

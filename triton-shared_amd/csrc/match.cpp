@@ -1,0 +1,566 @@
+// Family recognition and binding extraction: see match.h.
+#include "match.h"
+
+#include <functional>
+#include <sstream>
+
+namespace tts {
+
+const char *family_name(Family f) {
+  switch (f) {
+    case Family::Map1D: return "map1d";
+    case Family::RowSoftmax: return "row_softmax";
+    case Family::LayerNormFwd: return "layernorm_fwd";
+    case Family::Gemm: return "gemm";
+    case Family::GemmW8A16: return "gemm_w8a16";
+  }
+  return "?";
+}
+
+// ---------------------------------------------------------------- signature
+
+std::string signature(const Program &p) {
+  std::map<int, int> num;  // value id -> normalised number
+  auto V = [&](int v) {
+    auto it = num.find(v);
+    if (it == num.end()) return std::string("v?");
+    return "v" + std::to_string(it->second);
+  };
+  auto def = [&](int v) {
+    int n = (int)num.size();
+    num[v] = n;
+    return "v" + std::to_string(n);
+  };
+  std::ostringstream os;
+  std::function<void(const std::vector<SOp> &)> walk = [&](const std::vector<SOp> &ops) {
+    for (auto &s : ops) {
+      auto operands = [&]() {
+        std::string r = "(";
+        for (size_t i = 0; i < s.operands.size(); i++) r += (i ? "," : "") + V(s.operands[i]);
+        return r + ")";
+      };
+      auto acc = [&]() {
+        std::string r = ":" + s.acc.elem + ".r" + std::to_string(s.acc.sizes.size());
+        if (!s.acc.dims.empty()) r += ".m";
+        if (s.acc.has_other) r += ".o";
+        return r;
+      };
+      switch (s.kind) {
+        case SK::Load: os << def(s.result) << "=load" << acc() << ";"; break;
+        case SK::ScalarLoad: os << def(s.result) << "=sload" << acc() << ";"; break;
+        case SK::Store: os << "store" << acc() << operands() << ";"; break;
+        case SK::ScalarStore: os << "sstore" << acc() << operands() << ";"; break;
+        case SK::Map: {
+          std::string o = operands();
+          os << def(s.result) << "=" << s.name << ":" << p.values[s.result].dtype << o << ";";
+          break;
+        }
+        case SK::Splat: { std::string o = operands(); os << def(s.result) << "=splat" << o << ";"; break; }
+        case SK::Const: os << def(s.result) << "=const:" << p.values[s.result].dtype << ";"; break;
+        case SK::Iota: os << def(s.result) << "=iota;"; break;
+        case SK::FromIndex: os << def(s.result) << "=index;"; break;
+        case SK::ScalarArg: os << def(s.result) << "=farg;"; break;
+        case SK::Reduce: { std::string o = operands(); os << def(s.result) << "=reduce." << s.name << "." << s.axis << o << ";"; break; }
+        case SK::Dot: { std::string o = operands(); os << def(s.result) << "=dot" << o << ";"; break; }
+        case SK::ExpandDims: { std::string o = operands(); os << def(s.result) << "=expand." << s.axis << o << ";"; break; }
+        case SK::Broadcast: { std::string o = operands(); os << def(s.result) << "=bcast" << o << ";"; break; }
+        case SK::For: {
+          os << "for[";
+          for (size_t j = 0; j < s.tile_args.size(); j++) {
+            std::string init = V(s.tile_inits[j]);
+            os << (j ? "," : "") << def(s.tile_args[j]) << "<-" << init;
+          }
+          os << "]{";
+          walk(s.body);
+          os << "yield(";
+          for (size_t j = 0; j < s.tile_yields.size(); j++) os << (j ? "," : "") << V(s.tile_yields[j]);
+          os << ")}";
+          if (!s.results.empty()) {
+            os << "->";
+            for (size_t j = 0; j < s.results.size(); j++) os << (j ? "," : "") << def(s.results[j]);
+          }
+          os << ";";
+          break;
+        }
+      }
+    }
+  };
+  walk(p.body);
+  return os.str();
+}
+
+// ------------------------------------------------------------ expr helpers
+
+namespace {
+
+struct LinIv : Lin {
+  int iv = -1;  // coefficient of the designated loop's induction variable
+};
+
+struct Matcher {
+  Program &P;
+  ExprPool &X;
+  explicit Matcher(Program &p) : P(p), X(p.pool) { index_ops(P.body); }
+
+  int c64(int64_t v) { return X.constant(v, 64); }
+
+  bool pid_free(int e) { return !X.depends_on(e, EK::Pid); }
+  bool loop_free(int e) {
+    return !X.depends_on(e, EK::IV) && !X.depends_on(e, EK::Iter) && !X.depends_on(e, EK::Result);
+  }
+  bool is_const(int e, int64_t want) {
+    int64_t v;
+    return X.is_const(e, &v) && v == want;
+  }
+
+  // Decomposes e into c0 + sum coef[a]*pid[a] + iv*IV(loop) with parts that read
+  // neither the program id nor any loop state.  Sign extension is looked
+  // through: a 32-bit product that overflowed would differ, which the launcher
+  // rules out by evaluating the original expression at the last program of the
+  // grid and comparing.
+  bool linear(int e, LinIv &out, int loop = -1) {
+    const Expr x = X.at(e);
+    auto zero = [&](LinIv &l) {
+      l.c0 = c64(0);
+      for (int a = 0; a < 3; a++) l.coef[a] = c64(0);
+      l.iv = c64(0);
+    };
+    if (pid_free(e) && loop_free(e)) {
+      zero(out);
+      out.c0 = X.to_index(e);
+      return true;
+    }
+    if (x.k == EK::Pid) {
+      zero(out);
+      out.coef[x.a] = c64(1);
+      return true;
+    }
+    if (x.k == EK::IV && x.a == loop) {
+      zero(out);
+      out.iv = c64(1);
+      return true;
+    }
+    if (x.k == EK::Sext) return linear(x.a, out, loop);
+    if (x.k == EK::Add || x.k == EK::Sub) {
+      LinIv l, r;
+      if (!linear(x.a, l, loop) || !linear(x.b, r, loop)) return false;
+      out.c0 = X.bin(x.k, l.c0, r.c0);
+      for (int a = 0; a < 3; a++) out.coef[a] = X.bin(x.k, l.coef[a], r.coef[a]);
+      out.iv = X.bin(x.k, l.iv, r.iv);
+      return true;
+    }
+    if (x.k == EK::Mul) {
+      bool fa = pid_free(x.a) && loop_free(x.a), fb = pid_free(x.b) && loop_free(x.b);
+      if (!fa && !fb) return false;
+      int free_side = fa ? x.a : x.b, other = fa ? x.b : x.a;
+      LinIv l;
+      if (!linear(other, l, loop)) return false;
+      int s = X.to_index(free_side);
+      out.c0 = X.bin(EK::Mul, l.c0, s);
+      for (int a = 0; a < 3; a++) out.coef[a] = X.bin(EK::Mul, l.coef[a], s);
+      out.iv = X.bin(EK::Mul, l.iv, s);
+      return true;
+    }
+    return false;
+  }
+
+  // Recognises the valid extent MaskAnalysis derives for `start + arange(size) <
+  // bound`:  max(start, min(start+size, bound)) - start, possibly wrapped in
+  // min(size, .) by a conjunction with a broadcast mask.
+  bool extent(int e, int64_t size, int &start, int &bound) {
+    for (int guard = 0; guard < 4; guard++) {
+      const Expr x = X.at(e);
+      if (x.k != EK::MinS) break;
+      int64_t v;
+      if (X.is_const(x.a, &v) && v == size) e = x.b;
+      else if (X.is_const(x.b, &v) && v == size) e = x.a;
+      else break;
+    }
+    const Expr x = X.at(e);
+    auto min_with_end = [&](int m, int s, int &b) {
+      const Expr mm = X.at(m);
+      if (mm.k != EK::MinS) return false;
+      int end = X.bin(EK::Add, s, c64(size));
+      if (mm.a == end) { b = mm.b; return true; }
+      if (mm.b == end) { b = mm.a; return true; }
+      return false;
+    };
+    if (x.k == EK::Sub) {
+      int s = x.b;
+      const Expr mx = X.at(x.a);
+      if (mx.k != EK::MaxS) return false;
+      int m = mx.a == s ? mx.b : mx.b == s ? mx.a : -1;
+      if (m < 0) return false;
+      if (!min_with_end(m, s, bound)) return false;
+      start = s;
+      return true;
+    }
+    if (x.k == EK::MaxS) {  // start == 0: the subtraction folded away
+      int zero = c64(0);
+      int m = x.a == zero ? x.b : x.b == zero ? x.a : -1;
+      if (m < 0) return false;
+      if (!min_with_end(m, zero, bound)) return false;
+      start = zero;
+      return true;
+    }
+    return false;
+  }
+
+  int sum(const std::vector<int> &v) {
+    int s = c64(0);
+    for (int e : v) s = X.bin(EK::Add, s, X.to_index(e));
+    return s;
+  }
+
+  // flattened views of the program
+  std::vector<SOp *> accesses, loops, all;
+  void index_ops(std::vector<SOp> &ops) {
+    for (auto &s : ops) {
+      all.push_back(&s);
+      if (s.kind == SK::Load || s.kind == SK::Store || s.kind == SK::ScalarLoad || s.kind == SK::ScalarStore)
+        accesses.push_back(&s);
+      if (s.kind == SK::For) {
+        loops.push_back(&s);
+        index_ops(s.body);
+      }
+    }
+  }
+  std::vector<SOp *> of_kind(SK k) {
+    std::vector<SOp *> r;
+    for (auto s : all)
+      if (s->kind == k) r.push_back(s);
+    return r;
+  }
+};
+
+[[noreturn]] void refuse(const char *family, const std::string &why) {
+  throw Unsupported(std::string("the program has the op structure of family '") + family + "' but " + why);
+}
+
+void unit_stride(Matcher &m, const Access &a, const char *family) {
+  if (!m.is_const(a.strides.back(), 1)) refuse(family, "its innermost stride is not 1");
+}
+
+Lin as_lin(const LinIv &l) { return (Lin)l; }
+
+// ------------------------------------------------------------------ map1d
+// load, load, one binary f32 op, store: z[i] = x[i] op y[i] over each program's block.
+bool try_map1d(Plan &pl) {
+  Matcher m(pl.prog);
+  if (m.all.size() != 4) return false;
+  SOp *l0 = m.all[0], *l1 = m.all[1], *op = m.all[2], *st = m.all[3];
+  if (l0->kind != SK::Load || l1->kind != SK::Load || op->kind != SK::Map || st->kind != SK::Store) return false;
+  static const std::map<std::string, int> ops = {{"arith.addf", 0}, {"arith.subf", 1}, {"arith.mulf", 2},
+                                                 {"arith.divf", 3}, {"arith.maximumf", 4}, {"arith.minimumf", 5}};
+  auto it = ops.find(op->name);
+  if (it == ops.end() || op->operands.size() != 2) return false;
+  bool direct = op->operands[0] == l0->result && op->operands[1] == l1->result;
+  bool swapped = op->operands[0] == l1->result && op->operands[1] == l0->result;
+  if (!direct && !swapped) return false;
+  if (st->operands[0] != op->result) return false;
+  const char *F = "map1d";
+  for (SOp *a : {l0, l1, st}) {
+    if (a->acc.sizes.size() != 1) return false;
+    if (a->acc.elem != "f32") refuse(F, "its element type is " + a->acc.elem + " (only f32 is implemented)");
+    if (a->acc.sizes[0] != st->acc.sizes[0]) return false;
+    unit_stride(m, a->acc, F);
+    if (a->acc.dims != st->acc.dims) refuse(F, "its loads and its store are masked differently");
+  }
+  int64_t B = st->acc.sizes[0];
+  pl.family = Family::Map1D;
+  pl.k["op"] = it->second;
+  pl.k["swap"] = swapped;
+  pl.k["block"] = B;
+  pl.k["x_arg"] = l0->acc.base_arg;
+  pl.k["y_arg"] = l1->acc.base_arg;
+  pl.k["z_arg"] = st->acc.base_arg;
+  const char *names[] = {"x_off", "y_off", "z_off"};
+  int i = 0;
+  for (SOp *a : {l0, l1, st}) {
+    LinIv l;
+    if (!m.linear(a->acc.offsets[0], l)) refuse(F, "a block offset is not linear in the program id");
+    pl.lin[names[i++]] = as_lin(l);
+  }
+  pl.k["masked"] = !st->acc.dims.empty();
+  if (!st->acc.dims.empty()) {
+    int start, bound;
+    if (!m.extent(st->acc.dims[0], B, start, bound)) refuse(F, "its mask is not of the form start+arange < bound");
+    LinIv l;
+    if (!m.linear(start, l)) refuse(F, "its mask start is not linear in the program id");
+    if (!m.pid_free(bound) || !m.loop_free(bound)) refuse(F, "its mask bound depends on the program id");
+    pl.lin["m_start"] = as_lin(l);
+    pl.e["bound"] = bound;
+  }
+  return true;
+}
+
+// ------------------------------------------------------------ row softmax
+const char *SIG_SOFTMAX =
+    "v0=load:f32.r1.m.o;v1=reduce.arith.{MAX}.0(v0);v2=splat(v1);v3=arith.subf:f32(v0,v2);v4=math.exp:f32(v3);"
+    "v5=reduce.arith.addf.0(v4);v6=splat(v5);v7=arith.divf:f32(v4,v6);store:f32.r1.m(v7);";
+
+std::string subst(std::string s, const std::string &key, const std::string &val) {
+  for (size_t p = s.find(key); p != std::string::npos; p = s.find(key, p + val.size())) s.replace(p, key.size(), val);
+  return s;
+}
+
+bool try_softmax(Plan &pl) {
+  if (pl.signature != subst(SIG_SOFTMAX, "{MAX}", "maxnumf") && pl.signature != subst(SIG_SOFTMAX, "{MAX}", "maximumf"))
+    return false;
+  const char *F = "row_softmax";
+  Matcher m(pl.prog);
+  SOp *ld = m.accesses.at(0), *st = m.accesses.at(1);
+  unit_stride(m, ld->acc, F);
+  unit_stride(m, st->acc, F);
+  if (ld->acc.sizes != st->acc.sizes) refuse(F, "its load and store blocks differ in size");
+  pl.family = Family::RowSoftmax;
+  pl.k["block"] = ld->acc.sizes[0];
+  pl.k["in_arg"] = ld->acc.base_arg;
+  pl.k["out_arg"] = st->acc.base_arg;
+  pl.f["other"] = ld->acc.other_f;
+  LinIv li, lo;
+  if (!m.linear(ld->acc.offsets[0], li) || !m.linear(st->acc.offsets[0], lo))
+    refuse(F, "a row offset is not linear in the program id");
+  pl.lin["in_off"] = as_lin(li);
+  pl.lin["out_off"] = as_lin(lo);
+  for (SOp *a : {ld, st})
+    if (!m.pid_free(a->acc.dims[0]) || !m.loop_free(a->acc.dims[0])) refuse(F, "its column mask depends on the program id");
+  pl.e["in_dims"] = ld->acc.dims[0];
+  pl.e["out_dims"] = st->acc.dims[0];
+  return true;
+}
+
+// ---------------------------------------------------------- layernorm fwd
+const char *SIG_LAYERNORM = 
+    "v0=const:f32;v1=const:f32;v2=iota;v3=index;v4=splat(v3);for[v5<-v1]{v6=load:{T}.r1.m.o;v7=arith.extf"
+    ":f32(v6);v8=arith.addf:f32(v5,v7);yield(v8)}->v9;v10=reduce.arith.addf.0(v9);v11=index;v12=arith.sit"
+    "ofp:f32(v11);v13=arith.divf:f32(v10,v12);v14=splat(v13);for[v15<-v1]{v16=index;v17=splat(v16);v18=ar"
+    "ith.addi:i32(v17,v2);v19=arith.cmpi.slt:i1(v18,v4);v20=load:{T}.r1.m.o;v21=arith.extf:f32(v20);v22=a"
+    "rith.subf:f32(v21,v14);v23=arith.select:f32(v19,v22,v1);v24=arith.mulf:f32(v23,v23);v25=arith.addf:f"
+    "32(v15,v24);yield(v25)}->v26;v27=reduce.arith.addf.0(v26);v28=arith.divf:f32(v27,v12);v29=farg;v30=a"
+    "rith.addf:f32(v28,v29);v31=math.sqrt:f32(v30);v32=arith.divf:f32(v0,v31);sstore:f32.r0(v13);sstore:f"
+    "32.r0(v32);v33=splat(v32);for[]{v34=load:{T}.r1.m;v35=load:{T}.r1.m;v36=load:{T}.r1.m.o;v37=arith.ex"
+    "tf:f32(v36);v38=arith.subf:f32(v37,v14);v39=arith.mulf:f32(v38,v33);v40=arith.extf:f32(v34);v41=arit"
+    "h.mulf:f32(v39,v40);v42=arith.extf:f32(v35);v43=arith.addf:f32(v41,v42);v44=arith.truncf:{T}(v43);st"
+    "ore:{T}.r1.m(v44);yield()};";
+
+bool try_layernorm(Plan &pl) {
+  if (pl.signature != subst(SIG_LAYERNORM, "{T}", "f16") && pl.signature != subst(SIG_LAYERNORM, "{T}", "bf16")) return false;
+  const char *F = "layernorm_fwd";
+  Matcher m(pl.prog);
+  if (m.loops.size() != 3 || m.accesses.size() != 8) return false;
+  SOp *x0 = m.accesses[0], *x1 = m.accesses[1], *mean_st = m.accesses[2], *rstd_st = m.accesses[3];
+  SOp *w = m.accesses[4], *b = m.accesses[5], *x2 = m.accesses[6], *y = m.accesses[7];
+  int64_t B = x0->acc.sizes[0];
+  ExprPool &X = pl.prog.pool;
+  int N = m.loops[0]->ub;
+  for (size_t i = 0; i < 3; i++) {
+    SOp *lp = m.loops[i];
+    if (lp->ub != N) refuse(F, "its three column loops have different bounds");
+    if (!m.is_const(lp->lb, 0) || !m.is_const(lp->step, B)) refuse(F, "a column loop does not run from 0 in steps of the block size");
+  }
+  if (!m.pid_free(N) || !m.loop_free(N)) refuse(F, "its column count depends on the program id");
+  int Nidx = X.to_index(N);
+  // every block access: unit stride, same block, extent = clamp(N - iv)
+  SOp *blocks[] = {x0, x1, w, b, x2, y};
+  int loop_of[] = {0, 1, 2, 2, 2, 2};
+  const char *names[] = {"x_off", "x_off1", "w_off", "b_off", "x_off2", "y_off"};
+  for (int i = 0; i < 6; i++) {
+    SOp *a = blocks[i];
+    int loop = m.loops[loop_of[i]]->loop;
+    if (a->acc.sizes.size() != 1 || a->acc.sizes[0] != B) refuse(F, "its blocks differ in size");
+    unit_stride(m, a->acc, F);
+    int start, bound;
+    if (a->acc.dims.empty() || !m.extent(a->acc.dims[0], B, start, bound)) refuse(F, "a column mask is not start+arange < N");
+    if (start != X.to_index(X.iv(loop, 32)) || bound != Nidx) refuse(F, "a column mask is not (loop offset + arange) < N");
+    LinIv l;
+    if (!m.linear(a->acc.offsets[0], l, loop) || !m.is_const(l.iv, 1)) refuse(F, "a block offset is not row offset + loop offset");
+    pl.lin[names[i]] = as_lin(l);
+  }
+  auto same = [&](const Lin &a, const Lin &c) {
+    return a.c0 == c.c0 && a.coef[0] == c.coef[0] && a.coef[1] == c.coef[1] && a.coef[2] == c.coef[2];
+  };
+  if (!same(pl.lin["x_off"], pl.lin["x_off1"]) || !same(pl.lin["x_off"], pl.lin["x_off2"]))
+    refuse(F, "its three passes read different rows");
+  if (x0->acc.base_arg != x1->acc.base_arg || x0->acc.base_arg != x2->acc.base_arg) refuse(F, "its three passes read different tensors");
+  for (SOp *a : {x0, x1, x2})
+    if (!a->acc.has_other || a->acc.other_f != 0.0) refuse(F, "its input loads do not pad with 0");
+  // the select mask of the variance pass and the float N: every integer that
+  // reaches the data path must be the loop offset or N
+  auto from_index = m.of_kind(SK::FromIndex);
+  for (SOp *fi : from_index) {
+    int e = fi->expr;
+    bool is_n = e == N;
+    bool is_iv = X.at(e).k == EK::IV && X.at(e).a == m.loops[1]->loop;
+    if (!is_n && !is_iv) refuse(F, "an unexpected integer feeds its arithmetic");
+  }
+  for (SOp *io : m.of_kind(SK::Iota))
+    if (io->ival != 0) refuse(F, "its lane index does not start at 0");
+  auto consts = m.of_kind(SK::Const);
+  if (consts.size() != 2 || consts[0]->fval != 1.0 || consts[1]->fval != 0.0) refuse(F, "its constants are not 1 and 0");
+  for (SOp *s : {mean_st, rstd_st}) {
+    LinIv l;
+    if (!m.linear(s->acc.offsets[0], l)) refuse(F, "a statistics offset is not linear in the program id");
+    pl.lin[s == mean_st ? "mean_off" : "rstd_off"] = as_lin(l);
+  }
+  pl.family = Family::LayerNormFwd;
+  pl.k["block"] = B;
+  pl.k["x_arg"] = x0->acc.base_arg;
+  pl.k["y_arg"] = y->acc.base_arg;
+  pl.k["w_arg"] = w->acc.base_arg;
+  pl.k["b_arg"] = b->acc.base_arg;
+  pl.k["mean_arg"] = mean_st->acc.base_arg;
+  pl.k["rstd_arg"] = rstd_st->acc.base_arg;
+  pl.k["eps_arg"] = m.of_kind(SK::ScalarArg).at(0)->ival;
+  pl.k["half_is_bf16"] = x0->acc.elem == "bf16";
+  pl.e["N"] = N;
+  return true;
+}
+
+// ------------------------------------------------------------------- gemm
+const char *SIG_GEMM = 
+    "v0=const:f32;for[v1<-v0]{v2=load:{T}.r2.m.o;v3=load:{T}.r2.m.o;v4=dot(v2,v3,v1);yield(v4)}->v5;v6=ar"
+    "ith.truncf:{T}(v5);store:{T}.r2.m(v6);";
+const char *SIG_W8A16 = 
+    "v0=const:f32;v1=load:f16.r1.m.o;v2=expand.0(v1);v3=bcast(v2);for[v4<-v0]{v5=load:f16.r2.m.o;v6=load:"
+    "i8.r2.m.o;v7=arith.sitofp:f16(v6);v8=arith.mulf:f16(v7,v3);v9=dot(v5,v8,v4);yield(v9)}->v10;v11=arit"
+    "h.truncf:f16(v10);store:f16.r2.m(v11);";
+
+// Loop-carried pointer state of a 2-D block: strides must not change, offsets
+// advance by a loop-invariant amount per iteration.
+struct Carried2D {
+  int base = -1;   // sum of the offsets at iteration 0
+  int kstep = -1;  // sum of the per-iteration advances
+  int stride[2] = {-1, -1};
+};
+
+bool carried_state(Matcher &m, SOp *loop, const Access &a, Carried2D &out) {
+  ExprPool &X = m.X;
+  auto slot_of = [&](int e) -> IntIter * {
+    for (auto &it : loop->int_iters)
+      if (it.iter_expr == e) return &it;
+    return nullptr;
+  };
+  std::vector<int> inits, steps;
+  for (int e : a.offsets) {
+    IntIter *it = slot_of(e);
+    if (!it) {
+      if (!m.loop_free(e)) return false;
+      inits.push_back(e);
+      continue;
+    }
+    inits.push_back(it->init);
+    if (it->next == it->iter_expr) continue;
+    const Expr n = X.at(it->next);
+    if (n.k != EK::Add) return false;
+    int delta = n.a == it->iter_expr ? n.b : n.b == it->iter_expr ? n.a : -1;
+    if (delta < 0 || !m.loop_free(delta) || !m.pid_free(delta)) return false;
+    steps.push_back(delta);
+  }
+  for (int d = 0; d < 2; d++) {
+    int e = a.strides[d];
+    IntIter *it = slot_of(e);
+    if (it) {
+      if (it->next != it->iter_expr) return false;
+      e = it->init;
+    }
+    if (!m.loop_free(e) || !m.pid_free(e)) return false;
+    out.stride[d] = e;
+  }
+  out.base = m.sum(inits);
+  out.kstep = m.sum(steps);
+  return true;
+}
+
+bool try_gemm(Plan &pl, bool w8a16) {
+  std::string sig = pl.signature;
+  std::string T;
+  if (!w8a16) {
+    if (sig == subst(SIG_GEMM, "{T}", "bf16")) T = "bf16";
+    else if (sig == subst(SIG_GEMM, "{T}", "f16")) T = "f16";
+    else return false;
+  } else {
+    if (sig != SIG_W8A16) return false;
+    T = "f16";
+  }
+  const char *F = w8a16 ? "gemm_w8a16" : "gemm";
+  Matcher m(pl.prog);
+  if (m.loops.size() != 1) return false;
+  SOp *loop = m.loops[0];
+  size_t o = w8a16 ? 1 : 0;
+  if (m.accesses.size() != 3 + o) return false;
+  SOp *A = m.accesses[o], *Bm = m.accesses[o + 1], *C = m.accesses[o + 2];
+  if (A->acc.sizes.size() != 2 || Bm->acc.sizes.size() != 2 || C->acc.sizes.size() != 2) return false;
+  int64_t BM = A->acc.sizes[0], BK = A->acc.sizes[1], BN = Bm->acc.sizes[1];
+  if (Bm->acc.sizes[0] != BK || C->acc.sizes[0] != BM || C->acc.sizes[1] != BN) refuse(F, "its block shapes do not compose");
+  if (!m.is_const(loop->lb, 0) || !m.is_const(loop->step, 1)) refuse(F, "its K loop does not count 0,1,2,...");
+  if (!m.pid_free(loop->ub)) refuse(F, "its K trip count depends on the program id");
+  Carried2D ca, cb;
+  if (!carried_state(m, loop, A->acc, ca) || !carried_state(m, loop, Bm->acc, cb))
+    refuse(F, "its operand pointers do not advance by a constant per K step");
+  for (int e : C->acc.strides)
+    if (!m.pid_free(e) || !m.loop_free(e)) refuse(F, "its output strides depend on the program id");
+  // masks: rows against M, columns against N, K against what is left
+  int r0, Mb, c0, Nb, r0c, Mc, c0c, Nc;
+  if (A->acc.dims.size() != 2 || !m.extent(A->acc.dims[0], BM, r0, Mb)) refuse(F, "its A rows are not masked as row0+arange < M");
+  if (Bm->acc.dims.size() != 2 || !m.extent(Bm->acc.dims[1], BN, c0, Nb)) refuse(F, "its B columns are not masked as col0+arange < N");
+  if (C->acc.dims.size() != 2 || !m.extent(C->acc.dims[0], BM, r0c, Mc) || !m.extent(C->acc.dims[1], BN, c0c, Nc))
+    refuse(F, "its output is not masked as (row0+arange < M) & (col0+arange < N)");
+  if (r0 != r0c || c0 != c0c || Mb != Mc || Nb != Nc) refuse(F, "its operand masks and its output mask disagree");
+  if (A->acc.dims[1] != Bm->acc.dims[0]) refuse(F, "A and B mask the K dimension differently");
+  if (!m.pid_free(A->acc.dims[1])) refuse(F, "its K mask depends on the program id");
+  for (int e : {Mb, Nb})
+    if (!m.pid_free(e) || !m.loop_free(e)) refuse(F, "its problem size depends on the program id");
+  for (SOp *a : {A, Bm})
+    if (!a->acc.has_other || a->acc.other_f != 0.0 || a->acc.other_i != 0) refuse(F, "its operand loads do not pad with 0");
+  auto consts = m.of_kind(SK::Const);
+  if (consts.size() != 1 || consts[0]->fval != 0.0) refuse(F, "its accumulator does not start at 0");
+  if (w8a16) {
+    SOp *S = m.accesses[0];
+    int s0, Ns;
+    if (S->acc.sizes.size() != 1 || S->acc.sizes[0] != BN || S->acc.dims.empty() || !m.extent(S->acc.dims[0], BN, s0, Ns) ||
+        s0 != c0 || Ns != Nb || S->acc.offsets[0] != c0)
+      refuse(F, "its scale vector is not indexed and masked like the output columns");
+    unit_stride(m, S->acc, F);
+    pl.k["s_arg"] = S->acc.base_arg;
+  }
+  pl.family = w8a16 ? Family::GemmW8A16 : Family::Gemm;
+  pl.k["BM"] = BM;
+  pl.k["BN"] = BN;
+  pl.k["BK"] = BK;
+  pl.k["a_arg"] = A->acc.base_arg;
+  pl.k["b_arg"] = Bm->acc.base_arg;
+  pl.k["c_arg"] = C->acc.base_arg;
+  pl.k["is_bf16"] = T == "bf16";
+  pl.k["loop"] = loop->loop;
+  pl.e["a_base"] = ca.base;
+  pl.e["a_kstep"] = ca.kstep;
+  pl.e["sam"] = ca.stride[0];
+  pl.e["sak"] = ca.stride[1];
+  pl.e["b_base"] = cb.base;
+  pl.e["b_kstep"] = cb.kstep;
+  pl.e["sbk"] = cb.stride[0];
+  pl.e["sbn"] = cb.stride[1];
+  pl.e["c_base"] = m.sum(C->acc.offsets);
+  pl.e["scm"] = C->acc.strides[0];
+  pl.e["scn"] = C->acc.strides[1];
+  pl.e["r0"] = r0;
+  pl.e["c0"] = c0;
+  pl.e["M"] = Mb;
+  pl.e["N"] = Nb;
+  pl.e["kdim"] = A->acc.dims[1];
+  pl.e["trip"] = loop->ub;
+  return true;
+}
+
+}  // namespace
+
+Plan make_plan(Program &&p) {
+  Plan pl;
+  pl.prog = std::move(p);
+  pl.signature = signature(pl.prog);
+  if (try_map1d(pl) || try_softmax(pl) || try_layernorm(pl) || try_gemm(pl, false) || try_gemm(pl, true)) return pl;
+  throw Unsupported("no hand-written kernel family matches this structured program; signature: " + pl.signature);
+}
+
+}  // namespace tts

@@ -1,0 +1,43 @@
+// Pattern matcher: structured program -> kernel family + symbolic bindings.
+//
+// The reference lowers the structured program generically (mlir-opt pipeline,
+// backend/compiler.py:75-124) and runs it one Triton program at a time
+// (backend/driver.py:116-133).  This backend instead recognises the shape of
+// the whole structured program and hands the whole grid to one hand-written
+// gfx950 kernel of the matching family.  A program that matches no family is
+// refused (tts::Unsupported); nothing falls back to a slower path.
+#pragma once
+#include <map>
+#include <string>
+
+#include "structured.h"
+
+namespace tts {
+
+enum class Family { Map1D, RowSoftmax, LayerNormFwd, Gemm, GemmW8A16 };
+const char *family_name(Family f);
+
+// value(pid) = c0 + cx*pid.x + cy*pid.y + cz*pid.z ; all four are index
+// expressions that do not read the program id.
+struct Lin {
+  int c0 = -1;
+  int coef[3] = {-1, -1, -1};
+};
+
+struct Plan {
+  Program prog;
+  Family family;
+  std::string signature;            // normalised op listing the family was recognised from
+  std::map<std::string, int> e;     // named index expressions
+  std::map<std::string, Lin> lin;   // named pid-linear forms
+  std::map<std::string, int64_t> k; // named compile-time constants (block sizes, arg indices)
+  std::map<std::string, double> f;  // named float constants
+};
+
+// Normalised listing of a program's ops (no shapes, no expression ids).
+std::string signature(const Program &p);
+
+// Recognises the family and extracts its bindings.  Throws Unsupported.
+Plan make_plan(Program &&p);
+
+}  // namespace tts

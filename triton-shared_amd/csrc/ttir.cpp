@@ -1,0 +1,430 @@
+// TTIR text reader: see ttir.h.  Line oriented, because the MLIR printer
+// emits one operation per line and opens/closes regions on lines of their own.
+#include "ttir.h"
+
+#include <cctype>
+#include <sstream>
+
+namespace tts {
+
+std::string Type::str() const {
+  std::string e = ptr ? "!tt.ptr<" + elem + ">" : elem;
+  if (!is_tensor) return e;
+  std::string s = "tensor<";
+  for (auto d : shape) s += std::to_string(d) + "x";
+  return s + e + ">";
+}
+
+static std::string trim(const std::string &s) {
+  size_t a = 0, b = s.size();
+  while (a < b && isspace((unsigned char)s[a])) a++;
+  while (b > a && isspace((unsigned char)s[b - 1])) b--;
+  return s.substr(a, b - a);
+}
+
+static bool starts_with(const std::string &s, const char *p) { return s.rfind(p, 0) == 0; }
+
+Type parse_type(const std::string &raw) {
+  std::string s = trim(raw);
+  Type t;
+  if (starts_with(s, "tensor<")) {
+    t.is_tensor = true;
+    std::string in = s.substr(7, s.size() - 8);
+    // dims are separated by 'x' up to the first token that is not a number
+    size_t p = 0;
+    while (p < in.size() && isdigit((unsigned char)in[p])) {
+      size_t q = p;
+      while (q < in.size() && isdigit((unsigned char)in[q])) q++;
+      if (q >= in.size() || in[q] != 'x') break;
+      t.shape.push_back(std::stoll(in.substr(p, q - p)));
+      p = q + 1;
+    }
+    Type e = parse_type(in.substr(p));
+    t.ptr = e.ptr;
+    t.elem = e.elem;
+    return t;
+  }
+  if (starts_with(s, "!tt.ptr<")) {
+    t.ptr = true;
+    std::string in = s.substr(8, s.size() - 9);
+    size_t comma = in.find(',');  // address space suffix, if printed
+    if (comma != std::string::npos) in = in.substr(0, comma);
+    t.elem = trim(in);
+    if (starts_with(t.elem, "tensor<") || starts_with(t.elem, "!tt.ptr"))
+      throw Unsupported("block pointers / pointer-to-pointer are not supported: " + s);
+    return t;
+  }
+  static const char *known[] = {"i1", "i8", "i16", "i32", "i64", "f16", "bf16", "f32", "f64", "index"};
+  for (auto k : known)
+    if (s == k) {
+      t.elem = s;
+      return t;
+    }
+  throw Unsupported("unsupported type '" + s + "'");
+}
+
+// Removes "#loc..." definition lines and every " loc(...)" trailer.
+static std::string strip_locations(const std::string &text) {
+  std::string out;
+  out.reserve(text.size());
+  size_t i = 0, n = text.size();
+  bool line_start = true;
+  while (i < n) {
+    if (line_start && text.compare(i, 4, "#loc") == 0) {
+      while (i < n && text[i] != '\n') i++;
+      continue;
+    }
+    if (text.compare(i, 5, " loc(") == 0) {
+      size_t j = i + 5;
+      int depth = 1;
+      bool in_str = false;
+      while (j < n && depth) {
+        char c = text[j];
+        if (c == '"') in_str = !in_str;
+        else if (!in_str && c == '(') depth++;
+        else if (!in_str && c == ')') depth--;
+        j++;
+      }
+      i = j;
+      continue;
+    }
+    line_start = text[i] == '\n';
+    out.push_back(text[i++]);
+  }
+  return out;
+}
+
+static bool ssa_char(char c) {
+  return isalnum((unsigned char)c) || c == '_' || c == '.' || c == '$' || c == '#';
+}
+
+// Splits at top-level occurrences of any separator in seps (each a literal).
+static std::vector<std::string> split_top(const std::string &s, const std::vector<std::string> &seps) {
+  std::vector<std::string> out;
+  int depth = 0;
+  size_t last = 0, i = 0;
+  while (i < s.size()) {
+    char c = s[i];
+    if (depth == 0) {
+      bool hit = false;
+      for (auto &sep : seps)
+        if (s.compare(i, sep.size(), sep) == 0) {
+          out.push_back(trim(s.substr(last, i - last)));
+          i += sep.size();
+          last = i;
+          hit = true;
+          break;
+        }
+      if (hit) continue;
+    }
+    if (c == '-' && i + 1 < s.size() && s[i + 1] == '>') { i += 2; continue; }
+    if (c == '(' || c == '{' || c == '<' || c == '[') depth++;
+    else if (c == ')' || c == '}' || c == '>' || c == ']') depth--;
+    i++;
+  }
+  out.push_back(trim(s.substr(last)));
+  return out;
+}
+
+static std::vector<Type> parse_type_list(const std::string &s) {
+  std::vector<Type> out;
+  for (auto &piece : split_top(s, {"->", ",", " to ", " * "})) {
+    std::string p = piece;
+    if (p.empty()) continue;
+    if (p.front() == '(' && p.back() == ')') {
+      for (auto &t : parse_type_list(p.substr(1, p.size() - 2))) out.push_back(t);
+      continue;
+    }
+    out.push_back(parse_type(p));
+  }
+  return out;
+}
+
+static void collect_operands(const std::string &s, std::vector<std::string> &out) {
+  for (size_t i = 0; i < s.size(); i++) {
+    if (s[i] != '%') continue;
+    size_t j = i + 1;
+    while (j < s.size() && ssa_char(s[j])) j++;
+    out.push_back(s.substr(i, j - i));
+    i = j - 1;
+  }
+}
+
+static void parse_attr_dict(const std::string &body, std::map<std::string, std::string> &attrs) {
+  for (auto &ent : split_top(body, {","})) {
+    if (ent.empty()) continue;
+    size_t eq = ent.find('=');
+    if (eq == std::string::npos) {
+      attrs[trim(ent)] = "unit";
+      continue;
+    }
+    std::string key = trim(ent.substr(0, eq));
+    std::string val = trim(ent.substr(eq + 1));
+    auto parts = split_top(val, {" : "});
+    attrs[key] = parts[0];
+  }
+}
+
+// Finds the first ':' that is outside every bracket.  Returns npos if none.
+static size_t top_colon(const std::string &s) {
+  int depth = 0;
+  for (size_t i = 0; i < s.size(); i++) {
+    char c = s[i];
+    if (c == '-' && i + 1 < s.size() && s[i + 1] == '>') { i++; continue; }
+    if (c == '(' || c == '{' || c == '<' || c == '[') depth++;
+    else if (c == ')' || c == '}' || c == '>' || c == ']') depth--;
+    else if (c == ':' && depth == 0) return i;
+  }
+  return std::string::npos;
+}
+
+struct Lines {
+  std::vector<std::string> v;
+  size_t i = 0;
+};
+
+static void parse_block(Lines &L, Block &blk);
+
+static void parse_results(const std::string &lhs, Op &op) {
+  for (auto &r : split_top(lhs, {","})) {
+    size_t colon = r.find(':');
+    if (colon == std::string::npos) {
+      op.results.push_back(r);
+    } else {
+      int n = std::stoi(r.substr(colon + 1));
+      std::string base = r.substr(0, colon);
+      for (int k = 0; k < n; k++) op.results.push_back(base + "#" + std::to_string(k));
+    }
+  }
+}
+
+static void parse_for(const std::string &rest, Op &op, Lines &L) {
+  // %iv = %lb to %ub step %st [iter_args(%a = %x, ...) -> (types)] : i32 {
+  size_t eq = rest.find(" = ");
+  size_t to = rest.find(" to ");
+  size_t st = rest.find(" step ");
+  if (eq == std::string::npos || to == std::string::npos || st == std::string::npos)
+    throw Unsupported("malformed scf.for: " + rest);
+  op.iv = trim(rest.substr(0, eq));
+  op.operands.push_back(trim(rest.substr(eq + 3, to - eq - 3)));
+  op.operands.push_back(trim(rest.substr(to + 4, st - to - 4)));
+  size_t after = st + 6;
+  size_t e = after;
+  while (e < rest.size() && (rest[e] == '%' || ssa_char(rest[e]))) e++;
+  op.operands.push_back(rest.substr(after, e - after));
+  size_t ia = rest.find("iter_args(", e);
+  if (ia != std::string::npos) {
+    size_t open = ia + 9;
+    int depth = 0;
+    size_t close = open;
+    for (; close < rest.size(); close++) {
+      if (rest[close] == '(') depth++;
+      if (rest[close] == ')' && --depth == 0) break;
+    }
+    std::string inner = rest.substr(open + 1, close - open - 1);
+    for (auto &pair : split_top(inner, {","})) {
+      size_t q = pair.find('=');
+      op.iter_names.push_back(trim(pair.substr(0, q)));
+      op.iter_inits.push_back(trim(pair.substr(q + 1)));
+    }
+    size_t arrow = rest.find("->", close);
+    size_t tcolon = rest.rfind(" : ");
+    std::string tys = trim(rest.substr(arrow + 2, tcolon - arrow - 2));
+    op.result_types = parse_type_list(tys);
+    if (op.result_types.size() != op.iter_names.size())
+      throw Unsupported("scf.for: iter_args/result type count mismatch");
+  }
+  op.regions.emplace_back();
+  parse_block(L, op.regions.back());
+  if (L.i >= L.v.size() || L.v[L.i] != "}") throw Unsupported("scf.for region not closed");
+  L.i++;
+}
+
+static void parse_op(Lines &L, Block &blk) {
+  std::string line = L.v[L.i];
+  int line_no = (int)L.i + 1;
+  L.i++;
+  auto op = std::make_unique<Op>();
+  op->line = line_no;
+  std::string rest = line;
+  if (line[0] == '%') {
+    size_t eq = line.find(" = ");
+    if (eq == std::string::npos) throw Unsupported("cannot parse: " + line);
+    parse_results(line.substr(0, eq), *op);
+    rest = trim(line.substr(eq + 3));
+  }
+  // operation name (quoted for the generic form)
+  size_t p = 0;
+  if (rest[0] == '"') {
+    size_t q = rest.find('"', 1);
+    op->name = rest.substr(1, q - 1);
+    p = q + 1;
+  } else {
+    while (p < rest.size() && !isspace((unsigned char)rest[p]) && rest[p] != '(') p++;
+    op->name = rest.substr(0, p);
+  }
+  rest = trim(rest.substr(p));
+
+  if (op->name == "scf.for") {
+    parse_for(rest, *op, L);
+    blk.ops.push_back(std::move(op));
+    return;
+  }
+  if (op->name == "arith.constant") {
+    size_t c = std::string::npos;
+    {
+      // last top-level " : "
+      int depth = 0;
+      for (size_t i = 0; i + 2 < rest.size(); i++) {
+        char ch = rest[i];
+        if (ch == '<' || ch == '(' || ch == '[') depth++;
+        else if (ch == '>' || ch == ')' || ch == ']') depth--;
+        else if (depth == 0 && rest.compare(i, 3, " : ") == 0) c = i;
+      }
+    }
+    if (c == std::string::npos) {
+      op->literal = rest;
+      Type t;
+      t.elem = "i1";
+      op->result_types.push_back(t);
+    } else {
+      op->literal = trim(rest.substr(0, c));
+      op->result_types.push_back(parse_type(rest.substr(c + 3)));
+    }
+    blk.ops.push_back(std::move(op));
+    return;
+  }
+  if (op->name == "tt.reduce" || op->name == "tt.scan") {
+    // (%x[, %y]) <{axis = 0 : i32}> ({
+    size_t close = rest.find(')');
+    collect_operands(rest.substr(0, close + 1), op->operands);
+    size_t a0 = rest.find("<{"), a1 = rest.find("}>");
+    if (a0 != std::string::npos && a1 != std::string::npos)
+      parse_attr_dict(rest.substr(a0 + 2, a1 - a0 - 2), op->attrs);
+    if (rest.size() < 2 || rest.substr(rest.size() - 2) != "({")
+      throw Unsupported("expected region after " + op->name);
+    op->regions.emplace_back();
+    Block &rb = op->regions.back();
+    // ^bb0(%a: f32, %b: f32):
+    std::string hdr = L.v[L.i++];
+    size_t o = hdr.find('('), c2 = hdr.rfind(')');
+    if (!starts_with(hdr, "^") || o == std::string::npos) throw Unsupported("expected block header: " + hdr);
+    for (auto &a : split_top(hdr.substr(o + 1, c2 - o - 1), {","})) {
+      size_t col = a.find(':');
+      rb.arg_names.push_back(trim(a.substr(0, col)));
+      rb.arg_types.push_back(parse_type(a.substr(col + 1)));
+    }
+    parse_block(L, rb);
+    std::string tail = L.v[L.i++];  // }) : (types) -> types
+    if (!starts_with(tail, "})")) throw Unsupported("region of " + op->name + " not closed: " + tail);
+    size_t col = tail.find(':');
+    size_t arrow = tail.find("->");
+    op->types = parse_type_list(tail.substr(col + 1, arrow - col - 1));
+    op->result_types = parse_type_list(tail.substr(arrow + 2));
+    blk.ops.push_back(std::move(op));
+    return;
+  }
+
+  // generic custom-assembly line: operands/words/attrs, then ':' types
+  size_t colon = top_colon(rest);
+  std::string head = colon == std::string::npos ? rest : rest.substr(0, colon);
+  std::string tail = colon == std::string::npos ? "" : rest.substr(colon + 1);
+  // attribute dictionary
+  {
+    int depth = 0;
+    size_t open = std::string::npos;
+    for (size_t i = 0; i < head.size(); i++) {
+      if (head[i] == '{') {
+        if (depth == 0) open = i;
+        depth++;
+      } else if (head[i] == '}') {
+        if (--depth == 0 && open != std::string::npos) {
+          parse_attr_dict(head.substr(open + 1, i - open - 1), op->attrs);
+          head = head.substr(0, open) + " " + head.substr(i + 1);
+          i = open;
+          open = std::string::npos;
+        }
+      }
+    }
+  }
+  collect_operands(head, op->operands);
+  {
+    std::string w;
+    auto flush = [&]() {
+      if (!w.empty() && w[0] != '%' && w != "=") op->words.push_back(w);
+      w.clear();
+    };
+    for (char ch : head) {
+      if (isspace((unsigned char)ch) || ch == ',') flush();
+      else w.push_back(ch);
+    }
+    flush();
+  }
+  if (!tail.empty()) op->types = parse_type_list(tail);
+  if (!rest.empty() && rest.back() == '{')
+    throw Unsupported("operation with an unexpected region: " + op->name);
+  blk.ops.push_back(std::move(op));
+}
+
+static void parse_block(Lines &L, Block &blk) {
+  while (L.i < L.v.size()) {
+    const std::string &line = L.v[L.i];
+    if (line == "}" || starts_with(line, "})")) return;
+    parse_op(L, blk);
+  }
+}
+
+Func parse_ttir(const std::string &text) {
+  std::string clean = strip_locations(text);
+  Lines L;
+  {
+    std::istringstream is(clean);
+    std::string ln;
+    while (std::getline(is, ln)) {
+      ln = trim(ln);
+      if (!ln.empty()) L.v.push_back(ln);
+    }
+  }
+  Func f;
+  bool found = false;
+  while (L.i < L.v.size()) {
+    const std::string &line = L.v[L.i];
+    if (starts_with(line, "module")) { L.i++; continue; }
+    if (line == "}") { L.i++; continue; }
+    if (starts_with(line, "tt.func")) {
+      if (found) throw Unsupported("more than one tt.func in the module (non-inlined call?)");
+      found = true;
+      size_t at = line.find('@');
+      size_t open = line.find('(', at);
+      f.name = line.substr(at + 1, open - at - 1);
+      int depth = 0;
+      size_t close = open;
+      for (; close < line.size(); close++) {
+        if (line[close] == '(') depth++;
+        if (line[close] == ')' && --depth == 0) break;
+      }
+      std::string args = line.substr(open + 1, close - open - 1);
+      if (!trim(args).empty())
+        for (auto &a : split_top(args, {","})) {
+          size_t col = a.find(':');
+          std::string ty = a.substr(col + 1);
+          size_t brace = ty.find('{');
+          if (brace != std::string::npos) ty = ty.substr(0, brace);
+          f.arg_names.push_back(trim(a.substr(0, col)));
+          f.arg_types.push_back(parse_type(ty));
+        }
+      if (line.find("->", close) != std::string::npos && line.find("->", close) < line.rfind('{'))
+        throw Unsupported("tt.func with results is not a kernel");
+      L.i++;
+      parse_block(L, f.body);
+      if (L.i >= L.v.size() || L.v[L.i] != "}") throw Unsupported("tt.func body not closed");
+      L.i++;
+      continue;
+    }
+    throw Unsupported("unexpected top-level line: " + line);
+  }
+  if (!found) throw Unsupported("no tt.func found");
+  return f;
+}
+
+}  // namespace tts

@@ -1,0 +1,124 @@
+"""The five Triton kernels of the hot path, written against the unchanged Triton
+frontend (`@triton.jit`, `tl.*`).  They are ordinary user code: nothing in them
+knows which driver is active.
+
+Provenance of the algorithms (reference, read as text):
+  * vector add      - python/examples/test_vec_add.py:8-34
+  * row softmax     - python/examples/test_softmax.py:8-29
+  * LayerNorm fwd   - python/examples/test_layernorm.py:29-76
+  * blocked matmul  - python/examples/test_matmul.py:33-108, with edge masks on
+                      M/N instead of the `% M` wraparound and a narrowing epilogue
+  * W8A16 matmul    - no counterpart in the reference; weight-only int8 with
+                      per-output-channel scales, dequantised inside the K loop
+"""
+import triton
+import triton.language as tl
+
+
+@triton.jit
+def vec_add(x_ptr, y_ptr, z_ptr, n, BLOCK: tl.constexpr):
+    first = tl.program_id(0) * BLOCK
+    idx = first + tl.arange(0, BLOCK)
+    live = idx < n
+    a = tl.load(x_ptr + idx, mask=live)
+    b = tl.load(y_ptr + idx, mask=live)
+    tl.store(z_ptr + idx, a + b, mask=live)
+
+
+@triton.jit
+def row_softmax(out_ptr, in_ptr, in_pitch, out_pitch, n_cols, BLOCK: tl.constexpr):
+    r = tl.program_id(0)
+    cols = tl.arange(0, BLOCK)
+    v = tl.load(in_ptr + r * in_pitch + cols, mask=cols < n_cols, other=-float("inf"))
+    e = tl.exp(v - tl.max(v, axis=0))
+    p = e / tl.sum(e, axis=0)
+    tl.store(out_ptr + r * out_pitch + cols, p, mask=cols < n_cols)
+
+
+@triton.jit
+def layer_norm_fwd(X, Y, W, B, Mean, Rstd, pitch, N, eps, BLOCK: tl.constexpr):
+    r = tl.program_id(0)
+    X += r * pitch
+    Y += r * pitch
+    acc = tl.zeros([BLOCK], dtype=tl.float32)
+    for base in range(0, N, BLOCK):
+        c = base + tl.arange(0, BLOCK)
+        acc += tl.load(X + c, mask=c < N, other=0.).to(tl.float32)
+    mean = tl.sum(acc, axis=0) / N
+    acc2 = tl.zeros([BLOCK], dtype=tl.float32)
+    for base in range(0, N, BLOCK):
+        c = base + tl.arange(0, BLOCK)
+        d = tl.load(X + c, mask=c < N, other=0.).to(tl.float32)
+        d = tl.where(c < N, d - mean, 0.)
+        acc2 += d * d
+    var = tl.sum(acc2, axis=0) / N
+    rstd = 1 / tl.sqrt(var + eps)
+    tl.store(Mean + r, mean)
+    tl.store(Rstd + r, rstd)
+    for base in range(0, N, BLOCK):
+        c = base + tl.arange(0, BLOCK)
+        ok = c < N
+        w = tl.load(W + c, mask=ok)
+        b = tl.load(B + c, mask=ok)
+        d = tl.load(X + c, mask=ok, other=0.).to(tl.float32)
+        y = (d - mean) * rstd * w + b
+        tl.store(Y + c, y, mask=ok)
+
+
+@triton.jit
+def matmul_tiles(a_ptr, b_ptr, c_ptr, M, N, K,
+                 s_am, s_ak, s_bk, s_bn, s_cm, s_cn,
+                 BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr, GROUP_M: tl.constexpr):
+    pid = tl.program_id(0)
+    tiles_m = tl.cdiv(M, BM)
+    tiles_n = tl.cdiv(N, BN)
+    per_group = GROUP_M * tiles_n
+    g = pid // per_group
+    m0 = g * GROUP_M
+    rows_in_group = min(tiles_m - m0, GROUP_M)
+    tm = m0 + (pid % rows_in_group)
+    tn = (pid % per_group) // rows_in_group
+
+    rm = tm * BM + tl.arange(0, BM)
+    rn = tn * BN + tl.arange(0, BN)
+    rk = tl.arange(0, BK)
+    pa = a_ptr + (rm[:, None] * s_am + rk[None, :] * s_ak)
+    pb = b_ptr + (rk[:, None] * s_bk + rn[None, :] * s_bn)
+
+    acc = tl.zeros((BM, BN), dtype=tl.float32)
+    for k in range(0, tl.cdiv(K, BK)):
+        left = K - k * BK
+        a = tl.load(pa, mask=(rm[:, None] < M) & (rk[None, :] < left), other=0.0)
+        b = tl.load(pb, mask=(rk[:, None] < left) & (rn[None, :] < N), other=0.0)
+        acc += tl.dot(a, b)
+        pa += BK * s_ak
+        pb += BK * s_bk
+    out = acc.to(c_ptr.dtype.element_ty)
+    pc = c_ptr + s_cm * rm[:, None] + s_cn * rn[None, :]
+    tl.store(pc, out, mask=(rm[:, None] < M) & (rn[None, :] < N))
+
+
+@triton.jit
+def w8a16_matmul(a_ptr, w_ptr, s_ptr, c_ptr, M, N, K,
+                 s_am, s_ak, s_wk, s_wn, s_cm, s_cn,
+                 BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr):
+    tm = tl.program_id(0)
+    tn = tl.program_id(1)
+    rm = tm * BM + tl.arange(0, BM)
+    rn = tn * BN + tl.arange(0, BN)
+    rk = tl.arange(0, BK)
+    pa = a_ptr + (rm[:, None] * s_am + rk[None, :] * s_ak)
+    pw = w_ptr + (rk[:, None] * s_wk + rn[None, :] * s_wn)
+    scale = tl.load(s_ptr + rn, mask=rn < N, other=0.0)
+
+    acc = tl.zeros((BM, BN), dtype=tl.float32)
+    for k in range(0, tl.cdiv(K, BK)):
+        left = K - k * BK
+        a = tl.load(pa, mask=(rm[:, None] < M) & (rk[None, :] < left), other=0.0)
+        q = tl.load(pw, mask=(rk[:, None] < left) & (rn[None, :] < N), other=0)
+        w = q.to(tl.float16) * scale[None, :]
+        acc += tl.dot(a, w)
+        pa += BK * s_ak
+        pw += BK * s_wk
+    pc = c_ptr + s_cm * rm[:, None] + s_cn * rn[None, :]
+    tl.store(pc, acc.to(tl.float16), mask=(rm[:, None] < M) & (rn[None, :] < N))
