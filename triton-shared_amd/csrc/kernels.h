@@ -1,0 +1,79 @@
+// Launch interface of the hand-written gfx950 kernels, one per kernel family.
+// Parameter blocks are plain data resolved by the launcher from the plan's
+// bindings; the kernels know nothing about Triton.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace tts {
+
+// value(pid) = c0 + cx*pid.x + cy*pid.y + cz*pid.z, in elements
+struct Affine {
+  int64_t c0 = 0;
+  int64_t c[3] = {0, 0, 0};
+};
+
+// z[off_z(p)+i] = x[off_x(p)+i] op y[off_y(p)+i],  0 <= i < extent(p)
+// extent(p) = masked ? clamp(bound - m_start(p), 0, block) : block
+struct Map1DParams {
+  const float *x, *y;
+  float *z;
+  Affine xo, yo, zo, m_start;
+  int64_t bound;
+  int block;
+  int masked;
+  int op;    // 0 add 1 sub 2 mul 3 div 4 maximum 5 minimum
+  int swap;  // operands of `op` are (y, x)
+};
+hipError_t launch_map1d(const Map1DParams &p, int gx, int gy, int gz, hipStream_t s, const char **kernel_name);
+
+// out[off_out(p)+i] = softmax(row)[i], i < d_out, where row[i] = i < d_in ? in[off_in(p)+i] : other, i < block
+struct SoftmaxParams {
+  const float *in;
+  float *out;
+  Affine in_off, out_off;
+  int64_t d_in, d_out;
+  int block;
+  float other;
+  int propagate_nan;  // the max reduction is arith.maximumf rather than arith.maxnumf
+};
+hipError_t launch_softmax(const SoftmaxParams &p, int gx, int gy, int gz, hipStream_t s, const char **kernel_name);
+
+// LayerNorm forward over rows of N elements (fp16 or bf16 I/O, fp32 statistics)
+struct LayerNormParams {
+  const void *x, *w, *b;
+  void *y;
+  float *mean, *rstd;
+  Affine x_off, y_off, w_off, b_off, mean_off, rstd_off;
+  int64_t N;
+  float eps;
+  int is_bf16;
+};
+hipError_t launch_layernorm(const LayerNormParams &p, int gx, int gy, int gz, hipStream_t s, const char **kernel_name);
+
+// C[M,N] = A[M,K] * B[K,N], 16-bit inputs, fp32 accumulate, 16-bit output (RTNE)
+struct GemmParams {
+  const void *a, *b;
+  void *c;
+  int64_t M, N, K;
+  int64_t lda, ldb, ldc;  // row pitches in elements; the inner strides are 1
+  int is_bf16;
+};
+hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **kernel_name);
+
+// C[M,N] = A[M,K] * (f16(W[K,N]) * scale[N]), A/scale/C fp16, W int8, fp32 accumulate, M <= 16
+struct GemmW8A16Params {
+  const void *a;
+  const int8_t *w;
+  const void *scale;
+  void *c;
+  int64_t M, N, K;
+  int64_t lda, ldw, ldc;
+  float *workspace;        // split-K partial sums, or null when split == 1
+  int split;
+};
+int gemm_w8a16_split(int64_t M, int64_t N, int64_t K);  // how many K slices the kernel wants
+hipError_t launch_gemm_w8a16(const GemmW8A16Params &p, hipStream_t s, const char **kernel_name);
+
+}  // namespace tts

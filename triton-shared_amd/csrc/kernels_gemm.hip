@@ -1,0 +1,387 @@
+// MFMA kernel families for gfx950: 16-bit GEMM with fp32 accumulate, and the
+// weight-only int8 GEMM at decode shapes (M <= 16).
+//
+// What they replace in the reference CPU path: per program and per K step, two
+// malloc'd operand tiles filled with 0 and partially copied
+// (StructuredToMemref.cpp:794-853), linalg.matmul on operands widened to f32 into
+// a zero tile, an elementwise add into the loop-carried accumulator
+// (ConversionPatterns.hpp:1171-1196), a truncf tile (RTNE) and a partial copy out
+// (StructuredToMemref.cpp:1163-1196); the int8 variant adds a sitofp tile and a
+// mulf tile per K step.  The launcher has proved that the grid of programs is a
+// dense C = A*B, so these kernels choose their own tiling.
+#include "kernels.h"
+
+namespace tts {
+
+namespace {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest even
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ uint16_t f32_to_f16(float f) {
+  _Float16 h = (_Float16)f;
+  uint16_t r;
+  __builtin_memcpy(&r, &h, 2);
+  return r;
+}
+
+template <bool BF16>
+__device__ __forceinline__ f32x16 mfma32(uint4 a, uint4 b, f32x16 c) {
+  if (BF16) return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+// 8 consecutive 16-bit elements starting at p[0], zero beyond `valid`
+__device__ __forceinline__ uint4 load8(const uint16_t *p, int valid, bool vec) {
+  if (valid >= 8 && vec) return *reinterpret_cast<const uint4 *>(p);
+  uint32_t w[4] = {0, 0, 0, 0};
+  for (int i = 0; i < 8 && i < valid; i++) w[i >> 1] |= (uint32_t)p[i] << (16 * (i & 1));
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// ------------------------------------------------------------- 16-bit GEMM
+// Workgroup: 256 threads = 2 x 2 wavefronts; each wavefront owns TM x TN MFMA
+// tiles of 32 x 32.  A and B tiles are staged through LDS, both stored with K
+// contiguous ([row][k] and [col][k], pitch BK + 8 elements so that 16-byte
+// fragment reads of 32 consecutive rows hit distinct banks).  B is row-major
+// [K][N] in memory; it is transposed on the way into LDS by packing the two
+// K-neighbours of every column into one 32-bit word.
+template <bool BF16, int TM, int TN, int BK>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmParams p, int tiles_m, int tiles_n) {
+  constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32, PITCH = BK + 8;
+  constexpr int CA = BM * BK / 8 / 256;          // 16-byte chunks of A per thread
+  constexpr int UB = (BK / 2) * (BN / 8) / 256;  // 2x8 units of B per thread
+  extern __shared__ __align__(16) uint16_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // workgroup -> output tile: consecutive ids share an XCD's L2 (ids are dealt
+  // round-robin to the 8 XCDs), and within an XCD walk 8-tile-tall column groups
+  int bid = blockIdx.x;
+  const int nwg = tiles_m * tiles_n;
+  if (nwg % 8 == 0) bid = (bid % 8) * (nwg / 8) + bid / 8;
+  const int group = 8 * tiles_n;
+  const int g0 = (bid / group) * 8;
+  const int gh = min(tiles_m - g0, 8);
+  const int tile_m = g0 + (bid % group) % gh, tile_n = (bid % group) / gh;
+  const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+
+  const uint16_t *__restrict__ A = (const uint16_t *)p.a;
+  const uint16_t *__restrict__ B = (const uint16_t *)p.b;
+  const bool a_vec = (p.lda % 8 == 0) && (((uintptr_t)A & 15) == 0);
+  const bool b_vec = (p.ldb % 8 == 0) && (((uintptr_t)B & 15) == 0);
+  const int K = (int)p.K;
+
+  uint4 ra[CA], rb[UB][2];
+  auto load_tiles = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < CA; j++) {
+      int c = tid + 256 * j, row = c / (BK / 8), kc = c % (BK / 8);
+      int64_t gr = m0 + row;
+      int gk = k0 + kc * 8;
+      ra[j] = gr < p.M ? load8(A + gr * p.lda + gk, K - gk, a_vec) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < UB; j++) {
+      int u = tid + 256 * j, kp = u / (BN / 8), nc = u % (BN / 8);
+      int gk = k0 + 2 * kp;
+      int64_t gn = n0 + nc * 8;
+      int valid = (int)min((int64_t)8, p.N - gn);
+#pragma unroll
+      for (int r = 0; r < 2; r++)
+        rb[j][r] = (gk + r < K && valid > 0) ? load8(B + (int64_t)(gk + r) * p.ldb + gn, valid, b_vec) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store_tiles = [&](int buf) {
+    uint16_t *As = smem + buf * (BM + BN) * PITCH, *Bs = As + BM * PITCH;
+#pragma unroll
+    for (int j = 0; j < CA; j++) {
+      int c = tid + 256 * j, row = c / (BK / 8), kc = c % (BK / 8);
+      *reinterpret_cast<uint4 *>(As + row * PITCH + kc * 8) = ra[j];
+    }
+#pragma unroll
+    for (int j = 0; j < UB; j++) {
+      int u = tid + 256 * j, kp = u / (BN / 8), nc = u % (BN / 8);
+      uint32_t r0[4] = {rb[j][0].x, rb[j][0].y, rb[j][0].z, rb[j][0].w};
+      uint32_t r1[4] = {rb[j][1].x, rb[j][1].y, rb[j][1].z, rb[j][1].w};
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        uint32_t lo = (r0[i] & 0xffffu) | (r1[i] << 16);          // column 2i:   k, k+1
+        uint32_t hi = (r0[i] >> 16) | (r1[i] & 0xffff0000u);      // column 2i+1: k, k+1
+        *reinterpret_cast<uint32_t *>(Bs + (nc * 8 + 2 * i) * PITCH + 2 * kp) = lo;
+        *reinterpret_cast<uint32_t *>(Bs + (nc * 8 + 2 * i + 1) * PITCH + 2 * kp) = hi;
+      }
+    }
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+  const int nk = (K + BK - 1) / BK;
+  if (nk > 0) {
+    load_tiles(0);
+    store_tiles(0);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < nk; kt++) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) load_tiles((kt + 1) * BK);
+    const uint16_t *As = smem + cur * (BM + BN) * PITCH, *Bs = As + BM * PITCH;
+    const uint16_t *a_base = As + (wm * TM * 32 + (lane & 31)) * PITCH + 8 * (lane >> 5);
+    const uint16_t *b_base = Bs + (wn * TN * 32 + (lane & 31)) * PITCH + 8 * (lane >> 5);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      uint4 af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) af[i] = *reinterpret_cast<const uint4 *>(a_base + i * 32 * PITCH + ks * 16);
+#pragma unroll
+      for (int j = 0; j < TN; j++) bf[j] = *reinterpret_cast<const uint4 *>(b_base + j * 32 * PITCH + ks * 16);
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = mfma32<BF16>(af[i], bf[j], acc[i][j]);
+    }
+    if (kt + 1 < nk) store_tiles(cur ^ 1);
+    __syncthreads();
+  }
+
+  // epilogue: lane holds column (lane % 32), rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile
+  uint16_t *__restrict__ C = (uint16_t *)p.c;
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      int64_t col = n0 + wn * TN * 32 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        int64_t row = m0 + wm * TM * 32 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        if (row < p.M && col < p.N) C[row * p.ldc + col] = BF16 ? f32_to_bf16(acc[i][j][v]) : f32_to_f16(acc[i][j][v]);
+      }
+    }
+}
+
+template <bool BF16, int TM, int TN, int BK>
+hipError_t launch_gemm_cfg(const GemmParams &p, hipStream_t s) {
+  constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32;
+  constexpr size_t lds = 2 * (size_t)(BM + BN) * (BK + 8) * 2;
+  static bool configured = false;
+  auto kern = gemm_mfma_kernel<BF16, TM, TN, BK>;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + BN - 1) / BN);
+  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds, s, p, tiles_m, tiles_n);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------ int8-weight GEMM
+// Workgroup: NW wavefronts share one 128-column slab of W and split its K range
+// in interleaved steps of 32 rows.  In a step, lane (j = lane % 16, g = lane / 16)
+// streams rows 8g..8g+7 of the step, 8 columns (8 bytes) each, so that a
+// 16-lane group reads 128 contiguous bytes of a row.  Bytes are widened to fp16
+// exactly (bit pattern 0x6400 | (b ^ 0x80) is 1152 + b), multiplied by the
+// column's fp16 scale in fp16 as the Triton source does, and fed to eight
+// 16x16x32 MFMAs, one per column of the lane's eight.
+constexpr int W8_COLS = 128;
+
+__device__ __forceinline__ uint32_t pk_sub_1152_mul(uint32_t biased, uint32_t scale2) {
+  f16x2 v = __builtin_bit_cast(f16x2, biased);
+  f16x2 s = __builtin_bit_cast(f16x2, scale2);
+  const f16x2 off = {(_Float16)1152.0f, (_Float16)1152.0f};
+  v = v - off;  // exact: integers in [-128, 127]
+  v = v * s;    // one fp16 rounding, as arith.mulf on f16
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, int steps_per_slice) {
+  constexpr int RW = NW > 4 ? 4 : NW;  // wavefronts combined per round
+  __shared__ float red[RW][16][W8_COLS + 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int j = lane & 15, g = lane >> 4;
+  const int64_t n0 = (int64_t)blockIdx.x * W8_COLS;
+  const int slice = blockIdx.y;
+  const uint16_t *__restrict__ A = (const uint16_t *)p.a;
+  const int8_t *__restrict__ W = p.w;
+  const uint16_t *__restrict__ S = (const uint16_t *)p.scale;
+  const int K = (int)p.K;
+  const bool a_vec = (p.lda % 8 == 0) && (((uintptr_t)A & 15) == 0);
+  const bool w_vec = (p.ldw % 8 == 0) && (((uintptr_t)W & 7) == 0);
+  const int64_t ncol = n0 + 8 * j;                       // first of this lane's 8 columns
+  const int ncols = (int)max((int64_t)0, min((int64_t)8, p.N - ncol));
+
+  uint32_t scale2[8];
+#pragma unroll
+  for (int c = 0; c < 8; c++) {
+    uint32_t s = c < ncols ? S[ncol + c] : 0;
+    scale2[c] = s | (s << 16);
+  }
+  f32x4 acc[8];
+#pragma unroll
+  for (int c = 0; c < 8; c++) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const int step_begin = slice * steps_per_slice;
+  const int step_end = min(step_begin + steps_per_slice, (K + 31) / 32);
+
+  auto load_w = [&](int step, uint2 (&q)[8]) {
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      int k = step * 32 + 8 * g + t;
+      if (k < K && ncols == 8 && w_vec) {
+        q[t] = *reinterpret_cast<const uint2 *>(W + (int64_t)k * p.ldw + ncol);
+      } else {
+        uint32_t lo = 0, hi = 0;
+        if (k < K)
+          for (int c = 0; c < ncols; c++) {
+            uint32_t b = (uint8_t)W[(int64_t)k * p.ldw + ncol + c];
+            if (c < 4) lo |= b << (8 * c);
+            else hi |= b << (8 * (c - 4));
+          }
+        q[t] = make_uint2(lo, hi);
+      }
+    }
+  };
+  auto load_a = [&](int step) {
+    int k = step * 32 + 8 * g;
+    return j < p.M ? load8(A + (int64_t)j * p.lda + k, K - k, a_vec) : make_uint4(0, 0, 0, 0);
+  };
+
+  uint2 q[8], qn[8];
+  uint4 af, afn;
+  int step = step_begin + wave;
+  if (step < step_end) {
+    load_w(step, q);
+    af = load_a(step);
+  }
+  for (; step < step_end; step += NW) {
+    const int next = step + NW;
+    if (next < step_end) {
+      load_w(next, qn);
+      afn = load_a(next);
+    }
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+      uint32_t frag[4];
+#pragma unroll
+      for (int tp = 0; tp < 4; tp++) {
+        uint32_t w0 = c < 4 ? q[2 * tp].x : q[2 * tp].y;
+        uint32_t w1 = c < 4 ? q[2 * tp + 1].x : q[2 * tp + 1].y;
+        // bytes [w0.b, 0, w1.b, 0], then flip the sign bit and set the exponent: 0x6400 | (b ^ 0x80)
+        uint32_t sel = 0x0c000c00u | (uint32_t)(c & 3) | ((uint32_t)(4 + (c & 3)) << 16);
+        uint32_t pair = __builtin_amdgcn_perm(w1, w0, sel) ^ 0x64806480u;
+        frag[tp] = pk_sub_1152_mul(pair, scale2[c]);
+      }
+      uint4 bfrag = make_uint4(frag[0], frag[1], frag[2], frag[3]);
+      acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af), __builtin_bit_cast(f16x8, bfrag), acc[c], 0, 0, 0);
+    }
+    if (next < step_end) {
+#pragma unroll
+      for (int t = 0; t < 8; t++) q[t] = qn[t];
+      af = afn;
+    }
+  }
+
+  // combine the wavefronts' partial tiles through LDS, RW wavefronts at a time;
+  // lane holds rows 4g+v (v = 0..3) of column n0 + 8j + c
+  constexpr int ROUNDS = (NW + RW - 1) / RW;
+  constexpr int PER_THREAD = (16 * W8_COLS + NW * 64 - 1) / (NW * 64);
+  float total[PER_THREAD];
+#pragma unroll
+  for (int e = 0; e < PER_THREAD; e++) total[e] = 0.f;
+  for (int r = 0; r < ROUNDS; r++) {
+    if (r) __syncthreads();
+    if (wave / RW == r) {
+#pragma unroll
+      for (int c = 0; c < 8; c++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) red[wave % RW][4 * g + v][8 * j + c] = acc[c][v];
+    }
+    __syncthreads();
+    const int live = min(RW, NW - RW * r);
+#pragma unroll
+    for (int e = 0; e < PER_THREAD; e++) {
+      int idx = tid + e * NW * 64;
+      if (idx < 16 * W8_COLS) {
+        int m = idx / W8_COLS, n = idx % W8_COLS;
+        for (int w = 0; w < live; w++) total[e] += red[w][m][n];
+      }
+    }
+  }
+  uint16_t *__restrict__ C = (uint16_t *)p.c;
+#pragma unroll
+  for (int e = 0; e < PER_THREAD; e++) {
+    int idx = tid + e * NW * 64;
+    if (idx >= 16 * W8_COLS) continue;
+    int m = idx / W8_COLS;
+    int64_t n = n0 + idx % W8_COLS;
+    if (m >= p.M || n >= p.N) continue;
+    if (p.split > 1) p.workspace[((int64_t)slice * 16 + m) * p.N + n] = total[e];
+    else C[(int64_t)m * p.ldc + n] = f32_to_f16(total[e]);
+  }
+}
+
+__global__ __launch_bounds__(256) void gemm_w8a16_reduce_kernel(GemmW8A16Params p) {
+  int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= p.M * p.N) return;
+  int64_t m = idx / p.N, n = idx % p.N;
+  float s = 0.f;
+  for (int k = 0; k < p.split; k++) s += p.workspace[((int64_t)k * 16 + m) * p.N + n];
+  ((uint16_t *)p.c)[m * p.ldc + n] = f32_to_f16(s);
+}
+
+constexpr int W8_WAVES = 16;
+
+}  // namespace
+
+hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
+  static const char *tile_env = getenv("TTS_GEMM_TILE");
+  bool big = p.M >= 2048 && p.N >= 2048;
+  if (tile_env) big = atoi(tile_env) >= 256;
+  if (big) {
+    *name = "gemm_mfma_kernel<256x256x32>";
+    return p.is_bf16 ? launch_gemm_cfg<true, 4, 4, 32>(p, s) : launch_gemm_cfg<false, 4, 4, 32>(p, s);
+  }
+  *name = "gemm_mfma_kernel<128x128x64>";
+  return p.is_bf16 ? launch_gemm_cfg<true, 2, 2, 64>(p, s) : launch_gemm_cfg<false, 2, 2, 64>(p, s);
+}
+
+int gemm_w8a16_split(int64_t M, int64_t N, int64_t K) {
+  (void)M;
+  int64_t slabs = (N + W8_COLS - 1) / W8_COLS;
+  int64_t steps = (K + 31) / 32;
+  if (slabs >= 192) return 1;
+  int64_t want = (256 + slabs - 1) / slabs;                 // about one workgroup per CU
+  int64_t most = std::max<int64_t>(1, steps / W8_WAVES);    // keep every wavefront busy
+  return (int)std::max<int64_t>(1, std::min<int64_t>(std::min(want, most), 64));
+}
+
+hipError_t launch_gemm_w8a16(const GemmW8A16Params &p, hipStream_t s, const char **name) {
+  *name = "gemm_w8a16_kernel";
+  int slabs = (int)((p.N + W8_COLS - 1) / W8_COLS);
+  int steps = (int)((p.K + 31) / 32);
+  int steps_per_slice = (steps + p.split - 1) / p.split;
+  hipLaunchKernelGGL((gemm_w8a16_kernel<W8_WAVES>), dim3(slabs, p.split), dim3(W8_WAVES * 64), 0, s, p, steps_per_slice);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || p.split == 1) return e;
+  int64_t outs = p.M * p.N;
+  hipLaunchKernelGGL(gemm_w8a16_reduce_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, s, p);
+  return hipGetLastError();
+}
+
+}  // namespace tts

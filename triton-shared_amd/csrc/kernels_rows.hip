@@ -1,0 +1,349 @@
+// Memory-bound kernel families for gfx950: masked 1-D elementwise map, row
+// softmax, LayerNorm forward.  One Triton program maps to one workgroup (map1d,
+// layernorm) or one wavefront (softmax); every kernel covers the whole grid in
+// one launch.
+//
+// What they replace in the reference CPU path, per program: a malloc'd tile per
+// masked load filled with `other` and a partial element-wise copy
+// (StructuredToMemref.cpp:794-853, CRunnerUtils.cpp:58-113), one scalar loop
+// nest per linalg op with a full-tile temporary in between, sequential
+// reductions (ConversionPatterns.hpp:1395-1407), and a partial copy back
+// (StructuredToMemref.cpp:1163-1196).  Here a tile lives in registers, masking is
+// a per-lane predicate derived from the same valid extent, and the elementwise
+// ops are fused.  Compiled with -ffp-contract=off: the reference requests no
+// FMA contraction and no fast-math (backend/compiler.py:127-129,172-173).
+#include "kernels.h"
+
+namespace tts {
+
+namespace {
+
+constexpr int WAVE = 64;
+
+__device__ __forceinline__ int64_t affine(const Affine &a, int px, int py, int pz) {
+  return a.c0 + a.c[0] * px + a.c[1] * py + a.c[2] * pz;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+template <bool NAN_PROP>
+__device__ __forceinline__ float fmax_sel(float a, float b) {
+  if (NAN_PROP) return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b);
+  return fmaxf(a, b);  // arith.maxnumf: a NaN operand loses
+}
+template <bool NAN_PROP>
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmax_sel<NAN_PROP>(v, __shfl_xor(v, o, WAVE));
+  return v;
+}
+
+// ------------------------------------------------------------------ map1d
+template <int OP>
+__device__ __forceinline__ float apply(float a, float b) {
+  if (OP == 0) return a + b;
+  if (OP == 1) return a - b;
+  if (OP == 2) return a * b;
+  if (OP == 3) return a / b;
+  if (OP == 4) return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b);
+  return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b);
+}
+
+template <int OP, bool SWAP>
+__global__ __launch_bounds__(256) void map1d_f32_kernel(Map1DParams p) {
+  const int px = blockIdx.x, py = blockIdx.y, pz = blockIdx.z;
+  const float *__restrict__ x = p.x + affine(p.xo, px, py, pz);
+  const float *__restrict__ y = p.y + affine(p.yo, px, py, pz);
+  float *__restrict__ z = p.z + affine(p.zo, px, py, pz);
+  int d = p.block;
+  if (p.masked) {
+    int64_t left = p.bound - affine(p.m_start, px, py, pz);
+    d = left < 0 ? 0 : left < p.block ? (int)left : p.block;
+  }
+  const bool vec = (((uintptr_t)x | (uintptr_t)y | (uintptr_t)z) & 15) == 0;
+  for (int i = threadIdx.x * 4; i < d; i += 256 * 4) {
+    if (vec && i + 4 <= d) {
+      float4 a = *reinterpret_cast<const float4 *>(x + i);
+      float4 b = *reinterpret_cast<const float4 *>(y + i);
+      float4 r;
+      if (SWAP) {
+        r.x = apply<OP>(b.x, a.x); r.y = apply<OP>(b.y, a.y); r.z = apply<OP>(b.z, a.z); r.w = apply<OP>(b.w, a.w);
+      } else {
+        r.x = apply<OP>(a.x, b.x); r.y = apply<OP>(a.y, b.y); r.z = apply<OP>(a.z, b.z); r.w = apply<OP>(a.w, b.w);
+      }
+      *reinterpret_cast<float4 *>(z + i) = r;
+    } else {
+      for (int j = i; j < i + 4 && j < d; j++) z[j] = SWAP ? apply<OP>(y[j], x[j]) : apply<OP>(x[j], y[j]);
+    }
+  }
+}
+
+template <int OP>
+hipError_t launch_map1d_op(const Map1DParams &p, dim3 grid, hipStream_t s) {
+  if (p.swap) hipLaunchKernelGGL((map1d_f32_kernel<OP, true>), grid, dim3(256), 0, s, p);
+  else hipLaunchKernelGGL((map1d_f32_kernel<OP, false>), grid, dim3(256), 0, s, p);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------- softmax
+// T threads share one row; thread t holds elements t, t+T, ... (NPL of them).
+template <int NPL, int WAVES, bool NAN_PROP>
+__global__ __launch_bounds__(256) void softmax_f32_kernel(SoftmaxParams p, int gx, int gy, int64_t programs) {
+  constexpr int T = WAVES * WAVE;
+  constexpr int ROWS_PER_WG = 256 / T;
+  __shared__ float red[4];
+  const int sub = threadIdx.x / T, t = threadIdx.x % T;
+  const int64_t prog = (int64_t)blockIdx.x * ROWS_PER_WG + sub;
+  const bool active = prog < programs;
+  const int px = active ? (int)(prog % gx) : 0, py = active ? (int)((prog / gx) % gy) : 0;
+  const int pz = active ? (int)(prog / ((int64_t)gx * gy)) : 0;
+  const float *__restrict__ in = p.in + affine(p.in_off, px, py, pz);
+  float *__restrict__ out = p.out + affine(p.out_off, px, py, pz);
+  const int d_in = active ? (int)p.d_in : 0, d_out = active ? (int)p.d_out : 0;
+  // lanes beyond d_in hold `other` and take part in the reductions, as a filled
+  // tile does; lanes beyond the block do not exist
+  float v[NPL];
+#pragma unroll
+  for (int j = 0; j < NPL; j++) {
+    int i = t + j * T;
+    v[j] = i < d_in ? in[i] : p.other;
+  }
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < NPL; j++)
+    if (t + j * T < p.block) m = fmax_sel<NAN_PROP>(m, v[j]);
+  m = wave_max<NAN_PROP>(m);
+  if (WAVES > 1) {
+    if (t % WAVE == 0) red[t / WAVE] = m;
+    __syncthreads();
+    m = red[0];
+#pragma unroll
+    for (int w = 1; w < WAVES; w++) m = fmax_sel<NAN_PROP>(m, red[w]);
+    __syncthreads();
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < NPL; j++) {
+    v[j] = expf(v[j] - m);
+    if (t + j * T < p.block) sum += v[j];
+  }
+  sum = wave_sum(sum);
+  if (WAVES > 1) {
+    if (t % WAVE == 0) red[t / WAVE] = sum;
+    __syncthreads();
+    sum = red[0];
+#pragma unroll
+    for (int w = 1; w < WAVES; w++) sum += red[w];
+  }
+#pragma unroll
+  for (int j = 0; j < NPL; j++) {
+    int i = t + j * T;
+    if (i < d_out) out[i] = v[j] / sum;
+  }
+}
+
+template <int NPL, int WAVES>
+hipError_t launch_softmax_cfg(const SoftmaxParams &p, int gx, int gy, int gz, hipStream_t s) {
+  int64_t programs = (int64_t)gx * gy * gz;
+  int rows_per_wg = 256 / (WAVES * WAVE);
+  dim3 grid((unsigned)((programs + rows_per_wg - 1) / rows_per_wg));
+  if (p.propagate_nan) hipLaunchKernelGGL((softmax_f32_kernel<NPL, WAVES, true>), grid, dim3(256), 0, s, p, gx, gy, programs);
+  else hipLaunchKernelGGL((softmax_f32_kernel<NPL, WAVES, false>), grid, dim3(256), 0, s, p, gx, gy, programs);
+  return hipGetLastError();
+}
+
+// -------------------------------------------------------------- layernorm
+template <bool BF16>
+struct Half;
+template <>
+struct Half<false> {
+  static __device__ __forceinline__ float up(uint16_t h) {
+    _Float16 f;
+    __builtin_memcpy(&f, &h, 2);
+    return (float)f;
+  }
+  static __device__ __forceinline__ uint16_t down(float f) {  // arith.truncf, round to nearest even
+    _Float16 h = (_Float16)f;
+    uint16_t r;
+    __builtin_memcpy(&r, &h, 2);
+    return r;
+  }
+};
+template <>
+struct Half<true> {
+  static __device__ __forceinline__ float up(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+  static __device__ __forceinline__ uint16_t down(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // NaN stays NaN
+    u += 0x7fffu + ((u >> 16) & 1);
+    return (uint16_t)(u >> 16);
+  }
+};
+
+__device__ __forceinline__ float block_sum_256(float v, float *red) {
+  v = wave_sum(v);
+  __syncthreads();  // red may still be read from the previous use
+  if (threadIdx.x % WAVE == 0) red[threadIdx.x / WAVE] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// One workgroup per row.  The row is read from HBM once and kept in registers
+// as fp32 (CPT chunks of 8 elements per thread); the Triton source's three
+// passes over the row all read these registers.
+template <bool BF16, int CPT>
+__global__ __launch_bounds__(256) void layernorm_fwd_kernel(LayerNormParams p) {
+  __shared__ float red[4];
+  const int px = blockIdx.x, py = blockIdx.y, pz = blockIdx.z;
+  const uint16_t *__restrict__ x = (const uint16_t *)p.x + affine(p.x_off, px, py, pz);
+  const uint16_t *__restrict__ w = (const uint16_t *)p.w + affine(p.w_off, px, py, pz);
+  const uint16_t *__restrict__ b = (const uint16_t *)p.b + affine(p.b_off, px, py, pz);
+  uint16_t *__restrict__ y = (uint16_t *)p.y + affine(p.y_off, px, py, pz);
+  const int N = (int)p.N;
+  const bool vec = (((uintptr_t)x | (uintptr_t)w | (uintptr_t)b | (uintptr_t)y) & 15) == 0;
+  float v[CPT][8];
+#pragma unroll
+  for (int c = 0; c < CPT; c++) {
+    int i0 = (threadIdx.x + c * 256) * 8;
+    if (vec && i0 + 8 <= N) {
+      uint4 raw = *reinterpret_cast<const uint4 *>(x + i0);
+      uint32_t q[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        v[c][2 * k] = Half<BF16>::up((uint16_t)(q[k] & 0xffff));
+        v[c][2 * k + 1] = Half<BF16>::up((uint16_t)(q[k] >> 16));
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; k++) v[c][k] = i0 + k < N ? Half<BF16>::up(x[i0 + k]) : 0.f;  // other = 0
+    }
+  }
+  const float n_f = (float)N;  // arith.sitofp
+  float s = 0.f;
+#pragma unroll
+  for (int c = 0; c < CPT; c++)
+#pragma unroll
+    for (int k = 0; k < 8; k++) s += v[c][k];
+  const float mean = block_sum_256(s, red) / n_f;
+  float s2 = 0.f;
+#pragma unroll
+  for (int c = 0; c < CPT; c++) {
+    int i0 = (threadIdx.x + c * 256) * 8;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+      float d = i0 + k < N ? v[c][k] - mean : 0.f;  // tl.where(cols < N, x - mean, 0)
+      s2 += d * d;
+    }
+  }
+  const float var = block_sum_256(s2, red) / n_f;
+  const float rstd = 1.0f / sqrtf(var + p.eps);
+  if (threadIdx.x == 0) {
+    p.mean[affine(p.mean_off, px, py, pz)] = mean;
+    p.rstd[affine(p.rstd_off, px, py, pz)] = rstd;
+  }
+#pragma unroll
+  for (int c = 0; c < CPT; c++) {
+    int i0 = (threadIdx.x + c * 256) * 8;
+    if (vec && i0 + 8 <= N) {
+      uint4 wr = *reinterpret_cast<const uint4 *>(w + i0);
+      uint4 br = *reinterpret_cast<const uint4 *>(b + i0);
+      uint32_t wq[4] = {wr.x, wr.y, wr.z, wr.w}, bq[4] = {br.x, br.y, br.z, br.w}, o[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        float y0 = (v[c][2 * k] - mean) * rstd * Half<BF16>::up((uint16_t)(wq[k] & 0xffff)) +
+                   Half<BF16>::up((uint16_t)(bq[k] & 0xffff));
+        float y1 = (v[c][2 * k + 1] - mean) * rstd * Half<BF16>::up((uint16_t)(wq[k] >> 16)) +
+                   Half<BF16>::up((uint16_t)(bq[k] >> 16));
+        o[k] = (uint32_t)Half<BF16>::down(y0) | ((uint32_t)Half<BF16>::down(y1) << 16);
+      }
+      *reinterpret_cast<uint4 *>(y + i0) = make_uint4(o[0], o[1], o[2], o[3]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; k++)
+        if (i0 + k < N)
+          y[i0 + k] = Half<BF16>::down((v[c][k] - mean) * rstd * Half<BF16>::up(w[i0 + k]) + Half<BF16>::up(b[i0 + k]));
+    }
+  }
+}
+
+// Rows too long for the register file: three passes over global memory, the
+// second and third served by L2.
+template <bool BF16>
+__global__ __launch_bounds__(256) void layernorm_fwd_long_kernel(LayerNormParams p) {
+  __shared__ float red[4];
+  const int px = blockIdx.x, py = blockIdx.y, pz = blockIdx.z;
+  const uint16_t *__restrict__ x = (const uint16_t *)p.x + affine(p.x_off, px, py, pz);
+  const uint16_t *__restrict__ w = (const uint16_t *)p.w + affine(p.w_off, px, py, pz);
+  const uint16_t *__restrict__ b = (const uint16_t *)p.b + affine(p.b_off, px, py, pz);
+  uint16_t *__restrict__ y = (uint16_t *)p.y + affine(p.y_off, px, py, pz);
+  const int64_t N = p.N;
+  const float n_f = (float)(int)N;
+  float s = 0.f;
+  for (int64_t i = threadIdx.x; i < N; i += 256) s += Half<BF16>::up(x[i]);
+  const float mean = block_sum_256(s, red) / n_f;
+  float s2 = 0.f;
+  for (int64_t i = threadIdx.x; i < N; i += 256) {
+    float d = Half<BF16>::up(x[i]) - mean;
+    s2 += d * d;
+  }
+  const float var = block_sum_256(s2, red) / n_f;
+  const float rstd = 1.0f / sqrtf(var + p.eps);
+  if (threadIdx.x == 0) {
+    p.mean[affine(p.mean_off, px, py, pz)] = mean;
+    p.rstd[affine(p.rstd_off, px, py, pz)] = rstd;
+  }
+  for (int64_t i = threadIdx.x; i < N; i += 256)
+    y[i] = Half<BF16>::down((Half<BF16>::up(x[i]) - mean) * rstd * Half<BF16>::up(w[i]) + Half<BF16>::up(b[i]));
+}
+
+template <bool BF16>
+hipError_t launch_layernorm_t(const LayerNormParams &p, dim3 grid, hipStream_t s, const char **name) {
+  int64_t chunks = (p.N + 7) / 8;
+  if (chunks <= 256) { hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, 1>), grid, dim3(256), 0, s, p); *name = "layernorm_fwd_kernel<1>"; }
+  else if (chunks <= 512) { hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, 2>), grid, dim3(256), 0, s, p); *name = "layernorm_fwd_kernel<2>"; }
+  else if (chunks <= 1024) { hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, 4>), grid, dim3(256), 0, s, p); *name = "layernorm_fwd_kernel<4>"; }
+  else if (chunks <= 2048) { hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, 8>), grid, dim3(256), 0, s, p); *name = "layernorm_fwd_kernel<8>"; }
+  else { hipLaunchKernelGGL((layernorm_fwd_long_kernel<BF16>), grid, dim3(256), 0, s, p); *name = "layernorm_fwd_long_kernel"; }
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_map1d(const Map1DParams &p, int gx, int gy, int gz, hipStream_t s, const char **name) {
+  dim3 grid(gx, gy, gz);
+  *name = "map1d_f32_kernel";
+  switch (p.op) {
+    case 0: return launch_map1d_op<0>(p, grid, s);
+    case 1: return launch_map1d_op<1>(p, grid, s);
+    case 2: return launch_map1d_op<2>(p, grid, s);
+    case 3: return launch_map1d_op<3>(p, grid, s);
+    case 4: return launch_map1d_op<4>(p, grid, s);
+    case 5: return launch_map1d_op<5>(p, grid, s);
+  }
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_softmax(const SoftmaxParams &p, int gx, int gy, int gz, hipStream_t s, const char **name) {
+  *name = "softmax_f32_kernel";
+  int b = p.block;
+  if (b <= 64) return launch_softmax_cfg<1, 1>(p, gx, gy, gz, s);
+  if (b <= 128) return launch_softmax_cfg<2, 1>(p, gx, gy, gz, s);
+  if (b <= 256) return launch_softmax_cfg<4, 1>(p, gx, gy, gz, s);
+  if (b <= 512) return launch_softmax_cfg<8, 1>(p, gx, gy, gz, s);
+  if (b <= 1024) return launch_softmax_cfg<16, 1>(p, gx, gy, gz, s);
+  if (b <= 2048) return launch_softmax_cfg<32, 1>(p, gx, gy, gz, s);
+  if (b <= 4096) return launch_softmax_cfg<16, 4>(p, gx, gy, gz, s);
+  if (b <= 8192) return launch_softmax_cfg<32, 4>(p, gx, gy, gz, s);
+  if (b <= 16384) return launch_softmax_cfg<64, 4>(p, gx, gy, gz, s);
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_layernorm(const LayerNormParams &p, int gx, int gy, int gz, hipStream_t s, const char **name) {
+  dim3 grid(gx, gy, gz);
+  return p.is_bf16 ? launch_layernorm_t<true>(p, grid, s, name) : launch_layernorm_t<false>(p, grid, s, name);
+}
+
+}  // namespace tts

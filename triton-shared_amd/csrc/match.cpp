@@ -241,7 +241,11 @@ void unit_stride(Matcher &m, const Access &a, const char *family) {
   if (!m.is_const(a.strides.back(), 1)) refuse(family, "its innermost stride is not 1");
 }
 
-Lin as_lin(const LinIv &l) { return (Lin)l; }
+Lin as_lin(const LinIv &l, int orig) {
+  Lin r = (Lin)l;
+  r.orig = orig;
+  return r;
+}
 
 // ------------------------------------------------------------------ map1d
 // load, load, one binary f32 op, store: z[i] = x[i] op y[i] over each program's block.
@@ -279,7 +283,7 @@ bool try_map1d(Plan &pl) {
   for (SOp *a : {l0, l1, st}) {
     LinIv l;
     if (!m.linear(a->acc.offsets[0], l)) refuse(F, "a block offset is not linear in the program id");
-    pl.lin[names[i++]] = as_lin(l);
+    pl.lin[names[i++]] = as_lin(l, a->acc.offsets[0]);
   }
   pl.k["masked"] = !st->acc.dims.empty();
   if (!st->acc.dims.empty()) {
@@ -288,7 +292,7 @@ bool try_map1d(Plan &pl) {
     LinIv l;
     if (!m.linear(start, l)) refuse(F, "its mask start is not linear in the program id");
     if (!m.pid_free(bound) || !m.loop_free(bound)) refuse(F, "its mask bound depends on the program id");
-    pl.lin["m_start"] = as_lin(l);
+    pl.lin["m_start"] = as_lin(l, start);
     pl.e["bound"] = bound;
   }
   return true;
@@ -321,8 +325,8 @@ bool try_softmax(Plan &pl) {
   LinIv li, lo;
   if (!m.linear(ld->acc.offsets[0], li) || !m.linear(st->acc.offsets[0], lo))
     refuse(F, "a row offset is not linear in the program id");
-  pl.lin["in_off"] = as_lin(li);
-  pl.lin["out_off"] = as_lin(lo);
+  pl.lin["in_off"] = as_lin(li, ld->acc.offsets[0]);
+  pl.lin["out_off"] = as_lin(lo, st->acc.offsets[0]);
   for (SOp *a : {ld, st})
     if (!m.pid_free(a->acc.dims[0]) || !m.loop_free(a->acc.dims[0])) refuse(F, "its column mask depends on the program id");
   pl.e["in_dims"] = ld->acc.dims[0];
@@ -375,7 +379,7 @@ bool try_layernorm(Plan &pl) {
     if (start != X.to_index(X.iv(loop, 32)) || bound != Nidx) refuse(F, "a column mask is not (loop offset + arange) < N");
     LinIv l;
     if (!m.linear(a->acc.offsets[0], l, loop) || !m.is_const(l.iv, 1)) refuse(F, "a block offset is not row offset + loop offset");
-    pl.lin[names[i]] = as_lin(l);
+    pl.lin[names[i]] = as_lin(l, a->acc.offsets[0]);
   }
   auto same = [&](const Lin &a, const Lin &c) {
     return a.c0 == c.c0 && a.coef[0] == c.coef[0] && a.coef[1] == c.coef[1] && a.coef[2] == c.coef[2];
@@ -401,7 +405,7 @@ bool try_layernorm(Plan &pl) {
   for (SOp *s : {mean_st, rstd_st}) {
     LinIv l;
     if (!m.linear(s->acc.offsets[0], l)) refuse(F, "a statistics offset is not linear in the program id");
-    pl.lin[s == mean_st ? "mean_off" : "rstd_off"] = as_lin(l);
+    pl.lin[s == mean_st ? "mean_off" : "rstd_off"] = as_lin(l, s->acc.offsets[0]);
   }
   pl.family = Family::LayerNormFwd;
   pl.k["block"] = B;

@@ -22,6 +22,7 @@ const char *family_name(Family f);
 struct Lin {
   int c0 = -1;
   int coef[3] = {-1, -1, -1};
+  int orig = -1;  // the expression the form was derived from (loop offsets taken as 0)
 };
 
 struct Plan {

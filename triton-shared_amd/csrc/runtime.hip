@@ -1,0 +1,458 @@
+// C ABI (include/tts_hip.h) and the launcher: resolves a plan's symbolic
+// bindings for the scalar arguments and grid of one launch, checks what the
+// whole-grid kernels assume, and enqueues one kernel for the whole grid.
+//
+// The reference runs `for x, for y, for z: kernel(args, grid, x, y, z)` on the
+// calling thread (backend/driver.py:116-133).  Here the per-program index
+// arithmetic the reference executes inside each program (offsets, valid
+// extents) is evaluated on the host once per distinct (scalars, grid) and
+// cached; the device kernels receive closed forms of it.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <set>
+#include <sstream>
+#include <unordered_map>
+
+#include "../../include/tts_hip.h"
+#include "kernels.h"
+#include "match.h"
+
+using namespace tts;
+
+namespace {
+
+thread_local std::string g_error;
+
+tts_status fail(tts_status st, const std::string &msg) {
+  g_error = msg;
+  return st;
+}
+
+char *dup_string(const std::string &s) {
+  char *p = (char *)malloc(s.size() + 1);
+  memcpy(p, s.c_str(), s.size() + 1);
+  return p;
+}
+
+struct Invalid : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+
+// Everything a launch needs besides the pointers, resolved for one (scalars, grid).
+struct Bound {
+  Family family;
+  Map1DParams map1d{};
+  SoftmaxParams softmax{};
+  LayerNormParams layernorm{};
+  GemmParams gemm{};
+  GemmW8A16Params w8{};
+  bool empty = false;  // nothing to do (e.g. zero trip count with nothing stored)
+  std::string describe;
+};
+
+}  // namespace
+
+struct tts_plan {
+  Plan plan;
+  std::string family;
+  std::vector<int> arg_kinds;
+  std::unordered_map<std::string, std::shared_ptr<Bound>> cache;
+  std::mutex mu;
+  const char *last_kernel = "";
+  float *workspace = nullptr;  // split-K partial sums (device), owned by the plan
+  size_t workspace_bytes = 0;
+  ~tts_plan() {
+    if (workspace) (void)hipFree(workspace);
+  }
+};
+
+namespace {
+
+struct Resolver {
+  const Plan &pl;
+  const ExprPool &X;
+  std::vector<int64_t> ints;
+  std::vector<double> floats;
+  int g[3];
+  Resolver(const Plan &p, const tts_arg *args, int n, int gx, int gy, int gz) : pl(p), X(p.prog.pool), g{gx, gy, gz} {
+    ints.assign(n, 0);
+    floats.assign(n, 0.0);
+    for (int i = 0; i < n; i++) {
+      if (args[i].kind == TTS_ARG_INT) ints[i] = args[i].v.i;
+      if (args[i].kind == TTS_ARG_FLOAT) floats[i] = args[i].v.f;
+    }
+  }
+  EvalEnv env(int px = 0, int py = 0, int pz = 0) const {
+    EvalEnv e;
+    e.args = ints.data();
+    e.pid[0] = px; e.pid[1] = py; e.pid[2] = pz;
+    e.nprog[0] = g[0]; e.nprog[1] = g[1]; e.nprog[2] = g[2];
+    e.iv.assign(pl.prog.num_loops, 0);
+    e.iter.assign(pl.prog.num_loops, {});
+    e.result.assign(pl.prog.num_loops, {});
+    return e;
+  }
+  int64_t ev(const std::string &name, const EvalEnv &e) const { return X.eval(pl.e.at(name), e); }
+  int64_t ev0(const std::string &name) const { return ev(name, env()); }
+  Affine affine(const std::string &name) const {
+    const Lin &l = pl.lin.at(name);
+    EvalEnv e = env();
+    Affine a;
+    a.c0 = X.eval(l.c0, e);
+    for (int k = 0; k < 3; k++) a.c[k] = X.eval(l.coef[k], e);
+    if (l.orig >= 0) {
+      // the linear form was derived looking through i32 -> index extensions;
+      // confirm on the last program that no 32-bit product wrapped
+      EvalEnv last = env(g[0] - 1, g[1] - 1, g[2] - 1);
+      int64_t want = X.eval(l.orig, last);
+      int64_t got = a.c0 + a.c[0] * (g[0] - 1) + a.c[1] * (g[1] - 1) + a.c[2] * (g[2] - 1);
+      if (want != got)
+        throw Invalid("32-bit overflow in the kernel's index arithmetic for '" + name + "' at the last program of the grid");
+    }
+    return a;
+  }
+};
+
+std::string show(const Affine &a) {
+  std::ostringstream os;
+  os << a.c0 << "+" << a.c[0] << "*x+" << a.c[1] << "*y+" << a.c[2] << "*z";
+  return os.str();
+}
+
+void bind_map1d(const Resolver &r, Bound &b) {
+  Map1DParams &p = b.map1d;
+  p.xo = r.affine("x_off");
+  p.yo = r.affine("y_off");
+  p.zo = r.affine("z_off");
+  p.block = (int)r.pl.k.at("block");
+  p.masked = (int)r.pl.k.at("masked");
+  p.op = (int)r.pl.k.at("op");
+  p.swap = (int)r.pl.k.at("swap");
+  if (p.masked) {
+    p.m_start = r.affine("m_start");
+    p.bound = r.ev0("bound");
+  }
+  std::ostringstream os;
+  os << "kernel=map1d_f32\nop=" << p.op << "\nswap=" << p.swap << "\nblock=" << p.block << "\nmasked=" << p.masked
+     << "\nx_off=" << show(p.xo) << "\ny_off=" << show(p.yo) << "\nz_off=" << show(p.zo) << "\nm_start=" << show(p.m_start)
+     << "\nbound=" << p.bound << "\n";
+  b.describe = os.str();
+}
+
+void bind_softmax(const Resolver &r, Bound &b) {
+  SoftmaxParams &p = b.softmax;
+  p.in_off = r.affine("in_off");
+  p.out_off = r.affine("out_off");
+  p.d_in = r.ev0("in_dims");
+  p.d_out = r.ev0("out_dims");
+  p.block = (int)r.pl.k.at("block");
+  p.other = (float)r.pl.f.at("other");
+  p.propagate_nan = r.pl.signature.find("maximumf") != std::string::npos;
+  if (p.block > 16384) throw Unsupported("row_softmax: block sizes above 16384 are not implemented");
+  std::ostringstream os;
+  os << "kernel=softmax_f32\nblock=" << p.block << "\nd_in=" << p.d_in << "\nd_out=" << p.d_out << "\nother=" << p.other
+     << "\nin_off=" << show(p.in_off) << "\nout_off=" << show(p.out_off) << "\n";
+  b.describe = os.str();
+}
+
+void bind_layernorm(const Resolver &r, Bound &b) {
+  LayerNormParams &p = b.layernorm;
+  p.x_off = r.affine("x_off");
+  p.y_off = r.affine("y_off");
+  p.w_off = r.affine("w_off");
+  p.b_off = r.affine("b_off");
+  p.mean_off = r.affine("mean_off");
+  p.rstd_off = r.affine("rstd_off");
+  p.N = r.ev0("N");
+  p.eps = (float)r.floats.at(r.pl.k.at("eps_arg"));
+  p.is_bf16 = (int)r.pl.k.at("half_is_bf16");
+  if (p.N > INT32_MAX) throw Invalid("layernorm_fwd: N does not fit 32 bits");
+  std::ostringstream os;
+  os << "kernel=layernorm_fwd\nN=" << p.N << "\neps=" << p.eps << "\nbf16=" << p.is_bf16 << "\nx_off=" << show(p.x_off)
+     << "\ny_off=" << show(p.y_off) << "\nw_off=" << show(p.w_off) << "\nb_off=" << show(p.b_off)
+     << "\nmean_off=" << show(p.mean_off) << "\nrstd_off=" << show(p.rstd_off) << "\n";
+  b.describe = os.str();
+}
+
+// Shared by both GEMM families: evaluates every program's tile origin and
+// operand offsets, and proves that the grid of programs is exactly a dense
+// C[M,N] = A[M,K] * B[K,N] tiled BM x BN, so that one kernel with its own
+// tiling may compute it.
+struct DenseGemm {
+  int64_t M, N, K, lda, ldb, ldc;
+};
+
+DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
+  const Plan &pl = r.pl;
+  const ExprPool &X = r.X;
+  const int64_t BM = pl.k.at("BM"), BN = pl.k.at("BN"), BK = pl.k.at("BK");
+  const int loop = (int)pl.k.at("loop");
+  DenseGemm d;
+  d.M = r.ev0("M");
+  d.N = r.ev0("N");
+  d.lda = r.ev0("sam");
+  d.ldb = r.ev0("sbk");
+  d.ldc = r.ev0("scm");
+  auto need = [&](bool ok, const std::string &why) {
+    if (!ok) throw Unsupported(std::string(F) + ": " + why);
+  };
+  need(r.ev0("sak") == 1 && r.ev0("sbn") == 1 && r.ev0("scn") == 1, "only unit inner strides (row-major operands) are implemented");
+  need(d.M > 0 && d.N > 0, "empty problem");
+  // K: the loop must sweep K in full blocks followed by at most one partial block
+  int64_t trip = r.ev0("trip");
+  need(trip >= 0 && trip < (1 << 24), "unreasonable K trip count");
+  d.K = 0;
+  {
+    EvalEnv e = r.env();
+    for (int64_t k = 0; k < trip; k++) {
+      e.iv[loop] = k;
+      int64_t kd = X.eval(pl.e.at("kdim"), e);
+      need(kd == BK || (k == trip - 1 && kd >= 0), "the K mask does not describe a contiguous sweep of K");
+      d.K += kd;
+    }
+  }
+  need(r.ev0("a_kstep") == BK && r.ev0("b_kstep") == BK * d.ldb, "operand pointers do not advance by one K block per iteration");
+  // tiles: every program's origin, offsets consistent with a dense layout, exact cover
+  const int64_t tm = (d.M + BM - 1) / BM, tn = (d.N + BN - 1) / BN;
+  need((int64_t)r.g[0] * r.g[1] * r.g[2] == tm * tn, "the grid does not have one program per output tile");
+  std::vector<char> seen(tm * tn, 0);
+  for (int z = 0; z < r.g[2]; z++)
+    for (int y = 0; y < r.g[1]; y++)
+      for (int x = 0; x < r.g[0]; x++) {
+        EvalEnv e = r.env(x, y, z);
+        int64_t r0 = r.ev("r0", e), c0 = r.ev("c0", e);
+        need(r0 >= 0 && c0 >= 0 && r0 % BM == 0 && c0 % BN == 0 && r0 / BM < tm && c0 / BN < tn, "a program's tile origin is off the tile grid");
+        char &s = seen[(r0 / BM) * tn + c0 / BN];
+        need(!s, "two programs compute the same output tile");
+        s = 1;
+        need(r.ev("a_base", e) == r0 * d.lda, "A tile offset is not row0 * lda");
+        need(r.ev("b_base", e) == c0, "B tile offset is not col0");
+        need(r.ev("c_base", e) == r0 * d.ldc + c0, "C tile offset is not row0 * ldc + col0");
+      }
+  return d;
+}
+
+void bind_gemm(const Resolver &r, Bound &b) {
+  DenseGemm d = prove_dense_gemm(r, "gemm");
+  GemmParams &p = b.gemm;
+  p.M = d.M; p.N = d.N; p.K = d.K; p.lda = d.lda; p.ldb = d.ldb; p.ldc = d.ldc;
+  p.is_bf16 = (int)r.pl.k.at("is_bf16");
+  std::ostringstream os;
+  os << "kernel=gemm_mfma\nM=" << p.M << "\nN=" << p.N << "\nK=" << p.K << "\nlda=" << p.lda << "\nldb=" << p.ldb
+     << "\nldc=" << p.ldc << "\nbf16=" << p.is_bf16 << "\n";
+  b.describe = os.str();
+}
+
+void bind_w8a16(const Resolver &r, Bound &b) {
+  DenseGemm d = prove_dense_gemm(r, "gemm_w8a16");
+  if (d.M > 16) throw Unsupported("gemm_w8a16: only the decode shape M <= 16 is implemented");
+  GemmW8A16Params &p = b.w8;
+  p.M = d.M; p.N = d.N; p.K = d.K; p.lda = d.lda; p.ldw = d.ldb; p.ldc = d.ldc;
+  p.split = gemm_w8a16_split(p.M, p.N, p.K);
+  std::ostringstream os;
+  os << "kernel=gemm_w8a16\nM=" << p.M << "\nN=" << p.N << "\nK=" << p.K << "\nlda=" << p.lda << "\nldw=" << p.ldw
+     << "\nldc=" << p.ldc << "\nsplit=" << p.split << "\n";
+  b.describe = os.str();
+}
+
+std::shared_ptr<Bound> resolve(tts_plan *h, int gx, int gy, int gz, const tts_arg *args, int n) {
+  if (n != (int)h->arg_kinds.size())
+    throw Invalid("expected " + std::to_string(h->arg_kinds.size()) + " kernel arguments, got " + std::to_string(n));
+  std::string key;
+  key.reserve(16 + 8 * n);
+  int g[3] = {gx, gy, gz};
+  key.append((const char *)g, sizeof g);
+  for (int i = 0; i < n; i++) {
+    if (args[i].kind != h->arg_kinds[i])
+      throw Invalid("kernel argument " + std::to_string(i) + " has the wrong kind (pointer/integer/float)");
+    if (args[i].kind != TTS_ARG_PTR) key.append((const char *)&args[i].v, 8);
+  }
+  std::lock_guard<std::mutex> lock(h->mu);
+  auto it = h->cache.find(key);
+  if (it != h->cache.end()) return it->second;
+  auto b = std::make_shared<Bound>();
+  b->family = h->plan.family;
+  Resolver r(h->plan, args, n, gx, gy, gz);
+  switch (b->family) {
+    case Family::Map1D: bind_map1d(r, *b); break;
+    case Family::RowSoftmax: bind_softmax(r, *b); break;
+    case Family::LayerNormFwd: bind_layernorm(r, *b); break;
+    case Family::Gemm: bind_gemm(r, *b); break;
+    case Family::GemmW8A16: bind_w8a16(r, *b); break;
+  }
+  if (h->cache.size() > 256) h->cache.clear();
+  h->cache[key] = b;
+  return b;
+}
+
+template <class T>
+T *ptr_arg(const tts_arg *args, const Plan &pl, const char *name) {
+  return (T *)args[pl.k.at(name)].v.ptr;
+}
+
+template <class F>
+tts_status guarded(F &&f) {
+  try {
+    return f();
+  } catch (const Unsupported &e) {
+    return fail(TTS_UNSUPPORTED, e.what());
+  } catch (const Invalid &e) {
+    return fail(TTS_INVALID, e.what());
+  } catch (const std::exception &e) {
+    return fail(TTS_INVALID, e.what());
+  }
+}
+
+const char *PLAN_MAGIC = "tts.plan 1";
+
+}  // namespace
+
+extern "C" {
+
+const char *tts_last_error(void) { return g_error.c_str(); }
+void tts_free(void *p) { free(p); }
+
+tts_status tts_ttir_to_structured(const char *ttir_text, char **out) {
+  if (!ttir_text || !out) return fail(TTS_INVALID, "null argument");
+  return guarded([&]() {
+    Func f = parse_ttir(ttir_text);
+    Program p = lower_ttir(f);
+    *out = dup_string(print_program(p));
+    return TTS_OK;
+  });
+}
+
+tts_status tts_structured_to_plan(const char *structured_text, char **out_plan, size_t *out_len, char **out_name) {
+  if (!structured_text || !out_plan || !out_len) return fail(TTS_INVALID, "null argument");
+  return guarded([&]() {
+    Program p = read_program(structured_text);
+    std::string name = p.name;
+    Plan pl = make_plan(std::move(p));  // refuses here, at compile time, if no family matches
+    std::string bytes = std::string(PLAN_MAGIC) + " family=" + family_name(pl.family) + "\n" + structured_text;
+    *out_plan = dup_string(bytes);
+    *out_len = bytes.size();
+    if (out_name) *out_name = dup_string(name);
+    return TTS_OK;
+  });
+}
+
+tts_status tts_plan_load(const char *plan_bytes, size_t len, tts_plan **out) {
+  if (!plan_bytes || !out) return fail(TTS_INVALID, "null argument");
+  return guarded([&]() {
+    std::string text(plan_bytes, len);
+    if (text.rfind(PLAN_MAGIC, 0) != 0) throw Invalid("not a tts launch plan");
+    size_t nl = text.find('\n');
+    std::string header = text.substr(0, nl);
+    auto h = std::make_unique<tts_plan>();
+    h->plan = make_plan(read_program(text.substr(nl + 1)));
+    h->family = family_name(h->plan.family);
+    if (header.find("family=" + h->family) == std::string::npos) throw Invalid("plan header and plan body disagree on the kernel family");
+    for (auto &t : h->plan.prog.arg_types)
+      h->arg_kinds.push_back(t.ptr ? TTS_ARG_PTR : t.is_float() ? TTS_ARG_FLOAT : TTS_ARG_INT);
+    *out = h.release();
+    return TTS_OK;
+  });
+}
+
+void tts_plan_destroy(tts_plan *plan) { delete plan; }
+const char *tts_plan_kernel_name(const tts_plan *plan) { return plan->plan.prog.name.c_str(); }
+const char *tts_plan_family(const tts_plan *plan) { return plan->family.c_str(); }
+const char *tts_plan_signature(const tts_plan *plan) { return plan->plan.signature.c_str(); }
+int tts_plan_num_args(const tts_plan *plan) { return (int)plan->arg_kinds.size(); }
+int tts_plan_arg_kind(const tts_plan *plan, int i) {
+  return i >= 0 && i < (int)plan->arg_kinds.size() ? plan->arg_kinds[i] : -1;
+}
+const char *tts_plan_last_kernel(const tts_plan *plan) { return plan->last_kernel; }
+
+tts_status tts_plan_describe_launch(tts_plan *plan, int gx, int gy, int gz, const tts_arg *args, int n, char **out) {
+  if (!plan || !out || (n > 0 && !args)) return fail(TTS_INVALID, "null argument");
+  return guarded([&]() {
+    if ((int64_t)gx * gy * gz <= 0) {
+      *out = dup_string("kernel=none\n");
+      return TTS_OK;
+    }
+    auto b = resolve(plan, gx, gy, gz, args, n);
+    *out = dup_string("family=" + plan->family + "\n" + b->describe);
+    return TTS_OK;
+  });
+}
+
+tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, const tts_arg *args, int n) {
+  if (!plan || (n > 0 && !args)) return fail(TTS_INVALID, "null argument");
+  return guarded([&]() {
+    if (gx < 0 || gy < 0 || gz < 0) throw Invalid("negative grid");
+    if ((int64_t)gx * gy * gz == 0) return TTS_OK;  // backend/driver.py:117
+    if (gy > 65535 || gz > 65535) throw Unsupported("grid y/z extents above 65535");
+    auto b = resolve(plan, gx, gy, gz, args, n);
+    const Plan &pl = plan->plan;
+    hipStream_t s = (hipStream_t)stream;
+    hipError_t err = hipSuccess;
+    const char *kname = "";
+    switch (b->family) {
+      case Family::Map1D: {
+        Map1DParams p = b->map1d;
+        p.x = ptr_arg<const float>(args, pl, "x_arg");
+        p.y = ptr_arg<const float>(args, pl, "y_arg");
+        p.z = ptr_arg<float>(args, pl, "z_arg");
+        err = launch_map1d(p, gx, gy, gz, s, &kname);
+        break;
+      }
+      case Family::RowSoftmax: {
+        SoftmaxParams p = b->softmax;
+        p.in = ptr_arg<const float>(args, pl, "in_arg");
+        p.out = ptr_arg<float>(args, pl, "out_arg");
+        err = launch_softmax(p, gx, gy, gz, s, &kname);
+        break;
+      }
+      case Family::LayerNormFwd: {
+        LayerNormParams p = b->layernorm;
+        p.x = ptr_arg<const void>(args, pl, "x_arg");
+        p.y = ptr_arg<void>(args, pl, "y_arg");
+        p.w = ptr_arg<const void>(args, pl, "w_arg");
+        p.b = ptr_arg<const void>(args, pl, "b_arg");
+        p.mean = ptr_arg<float>(args, pl, "mean_arg");
+        p.rstd = ptr_arg<float>(args, pl, "rstd_arg");
+        err = launch_layernorm(p, gx, gy, gz, s, &kname);
+        break;
+      }
+      case Family::Gemm: {
+        GemmParams p = b->gemm;
+        p.a = ptr_arg<const void>(args, pl, "a_arg");
+        p.b = ptr_arg<const void>(args, pl, "b_arg");
+        p.c = ptr_arg<void>(args, pl, "c_arg");
+        err = launch_gemm(p, s, &kname);
+        break;
+      }
+      case Family::GemmW8A16: {
+        GemmW8A16Params p = b->w8;
+        p.a = ptr_arg<const void>(args, pl, "a_arg");
+        p.w = ptr_arg<const int8_t>(args, pl, "b_arg");
+        p.scale = ptr_arg<const void>(args, pl, "s_arg");
+        p.c = ptr_arg<void>(args, pl, "c_arg");
+        if (p.split > 1) {
+          size_t need = (size_t)p.split * 16 * (size_t)p.N * sizeof(float);
+          std::lock_guard<std::mutex> lock(plan->mu);
+          if (plan->workspace_bytes < need) {
+            if (plan->workspace) (void)hipFree(plan->workspace);
+            plan->workspace = nullptr;
+            plan->workspace_bytes = 0;
+            hipError_t e = hipMalloc((void **)&plan->workspace, need);
+            if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(split-K workspace): ") + hipGetErrorString(e));
+            plan->workspace_bytes = need;
+          }
+          p.workspace = plan->workspace;
+        }
+        err = launch_gemm_w8a16(p, s, &kname);
+        break;
+      }
+    }
+    plan->last_kernel = kname;
+    if (err != hipSuccess) return fail(TTS_HIP_ERROR, std::string("kernel launch failed: ") + hipGetErrorString(err));
+    return TTS_OK;
+  });
+}
+
+}  // extern "C"
