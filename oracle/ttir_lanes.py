@@ -1,0 +1,443 @@
+"""TEST INFRASTRUCTURE - not part of the product.
+
+Lane-by-lane interpreter of TTIR text in numpy: it executes a Triton program the
+way the Triton language defines it - a tensor of pointers is an array of element
+addresses, a mask is an array of booleans evaluated per lane, tt.load gathers and
+tt.store scatters - without any notion of structured accesses.  It shares no
+code with the product's planner (own reader, own evaluation), which makes it the
+brute-force pin for what the reference derives symbolically:
+
+  * addresses: lib/AnalysisStructured/PtrAnalysis.cpp (offsets, strides, sizes)
+  * valid extents: lib/Analysis/MaskAnalysis.cpp:461-603 - for prefix-shaped masks
+    the number of true lanes per dimension must equal dims[i], including the
+    all-masked case the max() at :568-585 exists for
+  * per-program results of the CPU path (serial grid, backend/driver.py:116-133).
+
+Reductions fold sequentially in index order in f32 and tt.dot sums k innermost
+into a zero tile before adding the accumulator, as the reference's lowering does
+(ConversionPatterns.hpp:1171-1196,1395-1407).  bf16 tensors are held as float32
+arrays of exactly representable values.  Meant for small shapes: every program
+is a Python-level loop over numpy calls.
+"""
+import re
+
+import numpy as np
+
+_INT_BITS = {"i1": 1, "i8": 8, "i16": 16, "i32": 32, "i64": 64, "index": 64}
+_NP = {"i1": np.bool_, "i8": np.int8, "i16": np.int16, "i32": np.int32, "i64": np.int64, "index": np.int64,
+       "f16": np.float16, "bf16": np.float32, "f32": np.float32, "f64": np.float64}
+
+
+class Ty:
+    def __init__(self, shape, elem, ptr):
+        self.shape, self.elem, self.ptr = tuple(shape), elem, ptr
+
+    @property
+    def tensor(self):
+        return self.shape is not None and len(self.shape) > 0 or self._is_tensor
+
+    _is_tensor = False
+
+
+def parse_type(s):
+    s = s.strip()
+    if s.startswith("tensor<"):
+        inner = s[7:-1]
+        dims = []
+        while True:
+            m = re.match(r"(\d+)x", inner)
+            if not m:
+                break
+            dims.append(int(m.group(1)))
+            inner = inner[m.end():]
+        e = parse_type(inner)
+        t = Ty(dims, e.elem, e.ptr)
+        t._is_tensor = True
+        return t
+    if s.startswith("!tt.ptr<"):
+        return Ty((), s[8:-1].split(",")[0].strip(), True)
+    return Ty((), s, False)
+
+
+def _strip_loc(text):
+    out, i, n = [], 0, len(text)
+    while i < n:
+        if text.startswith(" loc(", i):
+            j, depth = i + 5, 1
+            while depth:
+                depth += {"(": 1, ")": -1}.get(text[j], 0)
+                j += 1
+            i = j
+        else:
+            out.append(text[i])
+            i += 1
+    return "\n".join(l for l in "".join(out).splitlines() if not l.lstrip().startswith("#loc"))
+
+
+def round_bf16(x):
+    """float32 array -> nearest-even bf16 value, returned as float32."""
+    u = np.asarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    nan = (u & 0x7fffffff) > 0x7f800000
+    r = ((u + 0x7fff + ((u >> 16) & 1)) >> 16) << 16
+    r = np.where(nan, (u | 0x400000) & 0xffff0000, r).astype(np.uint32)
+    return r.view(np.float32)
+
+
+class Val:
+    __slots__ = ("d", "elem", "base")
+
+    def __init__(self, d, elem, base=None):
+        self.d, self.elem, self.base = d, elem, base  # base: argument index for pointers
+
+
+def _wrap(v, bits):
+    v &= (1 << bits) - 1
+    return v - (1 << bits) if bits > 1 and v >> (bits - 1) else v
+
+
+class Interpreter:
+    def __init__(self, ttir_text):
+        lines = [l.strip() for l in _strip_loc(ttir_text).splitlines() if l.strip()]
+        self.lines = lines
+        hdr = next(l for l in lines if l.startswith("tt.func"))
+        self.name = re.search(r"@(\w+)", hdr).group(1)
+        args = hdr[hdr.index("(") + 1:hdr.index(") attributes") if ") attributes" in hdr else hdr.rindex(")")]
+        self.args = []
+        for a in re.split(r",\s*(?=%)", args):
+            if not a.strip():
+                continue
+            name, ty = a.split(":", 1)
+            self.args.append((name.strip(), parse_type(ty.split("{")[0])))
+        self.body_start = lines.index(hdr) + 1
+
+    # ---------------------------------------------------------------- running
+    def run(self, grid, arg_values, memory):
+        """arg_values: per kernel argument an int/float (scalars) or None (pointers);
+        memory: {arg index: flat numpy array} (uint16 storage for bf16).  Returns the
+        access log: one list of (kind, arg, offsets) per program, x outermost."""
+        self.mem = memory
+        log = []
+        gx, gy, gz = (list(grid) + [1, 1])[:3]
+        for x in range(gx):
+            for y in range(gy):
+                for z in range(gz):
+                    self.pid, self.nprog, self.acc = (x, y, z), (gx, gy, gz), []
+                    env = {}
+                    for i, (name, ty) in enumerate(self.args):
+                        if ty.ptr:
+                            env[name] = Val(0, ty.elem, base=i)
+                        elif ty.elem in _INT_BITS:
+                            env[name] = Val(_wrap(int(arg_values[i]), _INT_BITS[ty.elem]), ty.elem)
+                        else:
+                            env[name] = Val(_NP[ty.elem](arg_values[i]), ty.elem)
+                    self._block(self.body_start, env)
+                    log.append(self.acc)
+        return log
+
+    def _block(self, i, env):
+        """Executes lines from i until the closing '}' of the block; returns (next index, yielded values)."""
+        L = self.lines
+        while i < len(L):
+            line = L[i]
+            if line == "}" or line.startswith("})"):
+                return i, None
+            if line.startswith("scf.yield"):
+                names = re.findall(r"%[\w.#$]+", line.split(":")[0])
+                return i, [env[n] for n in names]
+            if line.startswith("tt.return"):
+                i += 1
+                continue
+            i = self._op(i, env)
+        return i, None
+
+    def _skip_block(self, i):
+        depth = 1
+        L = self.lines
+        while depth:
+            if L[i].endswith("{"):
+                depth += 1
+            if L[i] == "}" or L[i].startswith("})"):
+                depth -= 1
+            i += 1
+        return i  # index after the closing line
+
+    # -------------------------------------------------------------------- ops
+    def _op(self, i, env):
+        line = self.lines[i]
+        results = []
+        rest = line
+        if line.startswith("%"):
+            lhs, rest = line.split(" = ", 1)
+            for r in lhs.split(","):
+                r = r.strip()
+                if ":" in r:
+                    b, n = r.split(":")
+                    results += [f"{b}#{k}" for k in range(int(n))]
+                else:
+                    results.append(r)
+        m = re.match(r'"?([\w.]+)"?', rest)
+        name = m.group(1)
+        tail = rest[m.end():].lstrip('"').strip()
+
+        if name == "scf.for":
+            return self._for(i, results, tail, env)
+        if name == "tt.reduce":
+            return self._reduce(i, results, tail, env)
+        if name == "arith.constant":
+            lit, ty = (tail.rsplit(" : ", 1) + ["i1"])[:2] if " : " in tail else (tail, "i1")
+            env[results[0]] = self._constant(lit.strip(), parse_type(ty))
+            return i + 1
+        head, _, types = self._split_types(tail)
+        ops = [env[n] for n in re.findall(r"%[\w.#$]+", re.sub(r"\{[^}]*\}", "", head))]
+        attrs = dict(re.findall(r"(\w+) = (-?\w+)", " ".join(re.findall(r"\{([^}]*)\}", head))))
+        tys = [parse_type(t) for t in re.split(r"\s*(?:->|,| to | \* )\s*", types) if t.strip()] if types else []
+        words = [w for w in re.split(r"[\s,]+", re.sub(r"\{[^}]*\}", "", head)) if w and not w.startswith("%")]
+        out = self._eval(name, ops, attrs, tys, words)
+        if results:
+            env[results[0]] = out
+        return i + 1
+
+    @staticmethod
+    def _split_types(tail):
+        depth = 0
+        j = 0
+        while j < len(tail):
+            c = tail[j]
+            if tail.startswith("->", j):
+                j += 2
+                continue
+            if c in "({<[":
+                depth += 1
+            elif c in ")}>]":
+                depth -= 1
+            elif c == ":" and depth == 0:
+                return tail[:j], ":", tail[j + 1:]
+            j += 1
+        return tail, "", ""
+
+    def _constant(self, lit, ty):
+        if lit.startswith("dense<"):
+            lit = lit[6:-1]
+        if ty.elem in _INT_BITS:
+            v = {"true": 1, "false": 0}.get(lit)
+            v = int(lit) if v is None else v
+            if ty._is_tensor:
+                return Val(np.full(ty.shape, v, dtype=_NP[ty.elem]), ty.elem)
+            return Val(_wrap(v, _INT_BITS[ty.elem]), ty.elem)
+        if lit.lower().startswith("0x"):
+            bits = int(lit, 16)
+            if ty.elem == "f32":
+                f = np.array([bits], dtype=np.uint32).view(np.float32)[0]
+            elif ty.elem == "f16":
+                f = np.array([bits], dtype=np.uint16).view(np.float16)[0]
+            elif ty.elem == "bf16":
+                f = np.array([bits << 16], dtype=np.uint32).view(np.float32)[0]
+            else:
+                f = np.array([bits], dtype=np.uint64).view(np.float64)[0]
+        else:
+            f = float(lit)
+        if ty._is_tensor:
+            return Val(np.full(ty.shape, f, dtype=_NP[ty.elem]), ty.elem)
+        return Val(_NP[ty.elem](f), ty.elem)
+
+    def _eval(self, name, ops, attrs, tys, words):
+        if name == "tt.get_program_id":
+            return Val(self.pid["xyz".index(words[0])], "i32")
+        if name == "tt.get_num_programs":
+            return Val(self.nprog["xyz".index(words[0])], "i32")
+        if name == "tt.make_range":
+            return Val(np.arange(int(attrs["start"]), int(attrs["end"]), dtype=np.int32), "i32")
+        if name == "tt.splat":
+            a, shape = ops[0], tys[-1].shape
+            if a.base is not None:
+                return Val(np.full(shape, a.d, dtype=np.int64), a.elem, base=a.base)
+            return Val(np.full(shape, a.d, dtype=_NP[a.elem]), a.elem)
+        if name == "tt.expand_dims":
+            return Val(np.expand_dims(ops[0].d, int(attrs["axis"])), ops[0].elem, ops[0].base)
+        if name == "tt.broadcast":
+            return Val(np.broadcast_to(ops[0].d, tys[-1].shape).copy(), ops[0].elem, ops[0].base)
+        if name == "tt.addptr":
+            p, o = ops
+            if isinstance(p.d, np.ndarray):
+                return Val(p.d + o.d.astype(np.int64), p.elem, p.base)
+            return Val(int(p.d) + int(o.d), p.elem, p.base)
+        if name == "tt.load":
+            return self._load(ops)
+        if name == "tt.store":
+            return self._store(ops)
+        if name == "tt.dot":
+            a, b, c = ops
+            af, bf = a.d.astype(np.float32), b.d.astype(np.float32)
+            prod = np.zeros(c.d.shape, dtype=np.float32)
+            for k in range(af.shape[1]):  # k innermost per output element = this order for every (i, j)
+                prod = prod + af[:, k:k + 1] * bf[k:k + 1, :]
+            return Val(prod + c.d, "f32")
+        return self._arith(name, ops, tys, words)
+
+    def _storage(self, arg, elem):
+        return self.mem[arg]
+
+    def _load(self, ops):
+        p = ops[0]
+        store = self.mem[p.base]
+        if not isinstance(p.d, np.ndarray):
+            self.acc.append(("load", p.base, np.array([p.d], dtype=np.int64)))
+            return Val(self._widen(store[p.d:p.d + 1], p.elem)[0], p.elem)
+        mask = ops[1].d if len(ops) > 1 else np.ones(p.d.shape, dtype=bool)
+        other = ops[2].d if len(ops) > 2 else np.zeros(p.d.shape, dtype=_NP[p.elem])
+        out = np.array(np.broadcast_to(other, p.d.shape), dtype=_NP[p.elem])
+        idx = p.d[mask]
+        self.acc.append(("load", p.base, np.sort(idx.ravel())))
+        if idx.size:
+            if idx.min() < 0 or idx.max() >= store.size:
+                raise IndexError(f"load outside argument {p.base}: [{idx.min()}, {idx.max()}] of {store.size}")
+            out[mask] = self._widen(store[idx], p.elem)
+        return Val(out, p.elem)
+
+    def _store(self, ops):
+        p, v = ops[0], ops[1]
+        store = self.mem[p.base]
+        if not isinstance(p.d, np.ndarray):
+            self.acc.append(("store", p.base, np.array([p.d], dtype=np.int64)))
+            store[p.d] = self._narrow(np.array([v.d]), p.elem)[0]
+            return None
+        mask = ops[2].d if len(ops) > 2 else np.ones(p.d.shape, dtype=bool)
+        idx = p.d[mask]
+        self.acc.append(("store", p.base, np.sort(idx.ravel())))
+        if idx.size:
+            if idx.min() < 0 or idx.max() >= store.size:
+                raise IndexError(f"store outside argument {p.base}")
+            store[idx] = self._narrow(v.d[mask], p.elem)
+        return None
+
+    @staticmethod
+    def _widen(raw, elem):
+        if elem == "bf16":
+            return (raw.astype(np.uint32) << 16).view(np.float32)
+        return raw
+
+    @staticmethod
+    def _narrow(vals, elem):
+        if elem == "bf16":
+            return (np.asarray(vals, dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        return vals
+
+    def _arith(self, name, ops, tys, words):
+        a = ops[0]
+        b = ops[1] if len(ops) > 1 else None
+        scalar_int = a.elem in _INT_BITS and not isinstance(a.d, np.ndarray)
+        if name in ("arith.addi", "arith.subi", "arith.muli", "arith.divsi", "arith.remsi", "arith.minsi", "arith.maxsi",
+                    "arith.andi", "arith.ori", "arith.xori"):
+            if scalar_int:
+                x, y = int(a.d), int(b.d)
+                if name == "arith.divsi":
+                    r = abs(x) // abs(y) * (1 if (x < 0) == (y < 0) else -1)
+                elif name == "arith.remsi":
+                    r = abs(x) % abs(y) * (1 if x >= 0 else -1)
+                else:
+                    r = {"arith.addi": x + y, "arith.subi": x - y, "arith.muli": x * y, "arith.minsi": min(x, y),
+                         "arith.maxsi": max(x, y), "arith.andi": x & y, "arith.ori": x | y, "arith.xori": x ^ y}[name]
+                return Val(_wrap(r, _INT_BITS[a.elem]), a.elem)
+            f = {"arith.addi": np.add, "arith.subi": np.subtract, "arith.muli": np.multiply, "arith.minsi": np.minimum,
+                 "arith.maxsi": np.maximum, "arith.andi": np.bitwise_and, "arith.ori": np.bitwise_or,
+                 "arith.xori": np.bitwise_xor,
+                 "arith.divsi": lambda x, y: (np.trunc(x.astype(np.float64) / y)).astype(x.dtype),
+                 "arith.remsi": np.fmod}[name]
+            with np.errstate(over="ignore"):
+                return Val(f(a.d, b.d), a.elem)
+        if name == "arith.cmpi":
+            f = {"slt": np.less, "sle": np.less_equal, "sgt": np.greater, "sge": np.greater_equal, "eq": np.equal,
+                 "ne": np.not_equal, "ult": np.less}[words[0]]
+            r = f(a.d, b.d)
+            return Val(r if isinstance(r, np.ndarray) else int(bool(r)), "i1")
+        if name == "arith.select":
+            c, x, y = ops
+            if isinstance(c.d, np.ndarray) or isinstance(x.d, np.ndarray):
+                return Val(np.where(c.d, x.d, y.d).astype(_NP[x.elem]), x.elem)
+            return Val(x.d if c.d else y.d, x.elem)
+        if name in ("arith.extsi", "arith.trunci", "arith.index_cast"):
+            e = tys[-1].elem
+            if scalar_int:
+                return Val(_wrap(int(a.d), _INT_BITS[e]), e)
+            return Val(a.d.astype(_NP[e]), e)
+        e = tys[-1].elem if tys else a.elem
+        if name == "arith.sitofp":
+            v = np.asarray(a.d).astype(np.float32)
+            return self._as_float(v, e, isinstance(a.d, np.ndarray))
+        if name in ("arith.extf", "arith.truncf"):
+            v = np.asarray(a.d, dtype=np.float32) if a.elem != "f64" else np.asarray(a.d)
+            return self._as_float(v, e, isinstance(a.d, np.ndarray))
+        fl = {"arith.addf": np.add, "arith.subf": np.subtract, "arith.mulf": np.multiply, "arith.divf": np.divide,
+              "arith.maxnumf": np.fmax, "arith.minnumf": np.fmin, "arith.maximumf": np.maximum,
+              "arith.minimumf": np.minimum}
+        if name in fl:
+            with np.errstate(all="ignore"):
+                r = fl[name](a.d, b.d)
+            return self._as_float(r, a.elem, isinstance(r, np.ndarray), already=a.elem != "bf16")
+        un = {"math.exp": np.exp, "math.sqrt": np.sqrt, "math.log": np.log, "math.absf": np.abs, "arith.negf": np.negative}
+        if name in un:
+            with np.errstate(all="ignore"):
+                r = un[name](a.d)
+            return self._as_float(r, a.elem, isinstance(r, np.ndarray), already=a.elem != "bf16")
+        raise NotImplementedError(f"ttir_lanes: {name}")
+
+    @staticmethod
+    def _as_float(v, elem, tensor, already=False):
+        if elem == "bf16":
+            v = round_bf16(np.asarray(v, dtype=np.float32))
+        elif not already or np.asarray(v).dtype != _NP[elem]:
+            v = np.asarray(v).astype(_NP[elem])
+        return Val(v if tensor else _NP[elem if elem != "bf16" else "f32"](v), elem)
+
+    # ------------------------------------------------------------ structured
+    def _for(self, i, results, tail, env):
+        m = re.match(r"(%[\w.#$]+) = (%[\w.#$]+) to (%[\w.#$]+) step (%[\w.#$]+)(.*)", tail)
+        iv, lb, ub, st, rest = m.groups()
+        iters = re.search(r"iter_args\((.*?)\) -> ", rest)
+        names, inits = [], []
+        if iters:
+            for pair in re.split(r",\s*(?=%)", iters.group(1)):
+                n, v = pair.split("=")
+                names.append(n.strip())
+                inits.append(env[v.strip()])
+        cur = list(inits)
+        k = int(env[lb].d)
+        end = i + 1
+        while k < int(env[ub].d):
+            env[iv] = Val(_wrap(k, 32), "i32")
+            for n, v in zip(names, cur):
+                env[n] = v
+            end, yielded = self._block(i + 1, env)
+            if yielded is not None:
+                cur = yielded
+            k += int(env[st].d)
+        close = self._skip_block(i + 1) - 1  # index of the closing '}'
+        for r, v in zip(results, cur):
+            env[r] = v
+        return close + 1
+
+    def _reduce(self, i, results, tail, env):
+        operand = env[re.findall(r"%[\w.#$]+", tail)[0]]
+        axis = int(re.search(r"axis = (\d+)", tail).group(1))
+        comb = re.match(r'(%[\w.#$]+) = ([\w.]+)', self.lines[i + 2]).group(2)
+        x = np.moveaxis(operand.d, axis, 0)
+        if comb == "arith.addf" and x.ndim == 1:
+            out = np.add.accumulate(x.astype(np.float32), dtype=np.float32)[-1]  # sequential fold
+        elif comb == "arith.addf":
+            acc = np.zeros(x.shape[1:], dtype=np.float32)
+            for row in x.astype(np.float32):  # sequential, index order, f32 (f16/bf16 are promoted)
+                acc = acc + row
+            out = acc
+        elif comb in ("arith.maxnumf", "arith.maximumf"):
+            f = np.fmax if comb == "arith.maxnumf" else np.maximum
+            acc = np.full(x.shape[1:], -np.inf, dtype=np.float32)
+            for row in x.astype(np.float32):
+                acc = f(acc, row)
+            out = acc
+        elif comb == "arith.addi":
+            out = x.sum(axis=0, dtype=x.dtype)
+        else:
+            raise NotImplementedError(f"ttir_lanes: reduce with {comb}")
+        out = out.astype(_NP[operand.elem]) if operand.elem != "bf16" else round_bf16(out)
+        env[results[0]] = Val(out if out.ndim else out[()], operand.elem)
+        return self._skip_block(i + 1)

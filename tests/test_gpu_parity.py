@@ -1,0 +1,294 @@
+"""Parity of the HIP path against the oracle on a real MI355X.  Every launch goes
+through the C ABI (tts_launch): either from the unchanged Triton frontend with
+HIPDriver active, or directly on a plan handle.
+
+Bars (BASELINE.json): bit-exact for fp32 elementwise and all index/mask handling;
+max-abs <= 1e-5 for fp32 softmax; <= 1e-2 for fp16 LayerNorm; relative Frobenius
+error <= 1e-2 for the bf16 and int8-weight GEMMs."""
+import numpy as np
+import pytest
+import torch
+import triton
+
+from conftest import plan_for
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def hip_driver():
+    import triton_shared_amd as tsa
+    drv = tsa.activate()
+    yield drv
+
+
+@pytest.fixture(scope="module")
+def K():
+    from triton_shared_amd.examples import kernels
+    return kernels
+
+
+def relfro(got, ref):
+    return ((got.double() - ref.double()).norm() / ref.double().norm()).item()
+
+
+# ------------------------------------------------------------------ cfg1
+def test_cfg1_vec_add_bit_exact(K, oracle_cpu):
+    torch.manual_seed(0)
+    n = 98432
+    x, y = torch.rand(n), torch.rand(n)
+    xd, yd = x.to(DEV), y.to(DEV)
+    zd = torch.full((n + 64,), -7.0, device=DEV)           # sentinel after the end
+    k = K.vec_add[(triton.cdiv(n, 1024),)](xd, yd, zd, n, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "map1d" and k.function.last_kernel == "map1d_f32_kernel"
+    assert torch.equal(zd[:n].cpu(), oracle_cpu.vec_add(x, y))
+    assert torch.equal(zd[n:].cpu(), torch.full((64,), -7.0))  # the masked tail is not written
+
+
+@pytest.mark.parametrize("n", [1, 3, 1023, 1024, 1025, 5000, (1 << 22) + 5])
+def test_vec_add_sizes_and_unaligned_views(K, oracle_cpu, n):
+    torch.manual_seed(n)
+    x, y = torch.rand(n + 3), torch.rand(n + 3)
+    xd, yd, zd = x.to(DEV), y.to(DEV), torch.zeros(n + 3, device=DEV)
+    # views starting 1, 2 and 3 elements into the allocation: no 16-byte alignment
+    K.vec_add[(triton.cdiv(n, 1024) + 1,)](xd[1:], yd[2:], zd[3:], n, BLOCK=1024)  # one extra, all-masked program
+    torch.cuda.synchronize()
+    assert torch.equal(zd[3:3 + n].cpu(), x[1:1 + n] + y[2:2 + n])
+    assert zd[:3].abs().sum().item() == 0
+
+
+def test_map1d_other_ops_through_c_abi(native):
+    # the same plan family with other binary ops, launched directly on plan handles
+    import extra_kernels as X
+    from triton_shared_amd.examples import kernels  # noqa: F401
+    torch.manual_seed(1)
+    n = 3000
+    x, y = torch.randn(n), torch.randn(n) + 2.0
+    xd, yd, zd = x.to(DEV), y.to(DEV), torch.zeros(n, device=DEV)
+    X.vec_sub_swapped[(triton.cdiv(n, 128),)](xd, yd, zd, n, BLOCK=128)
+    torch.cuda.synchronize()
+    assert torch.equal(zd.cpu(), y - x)
+    plan, _ = plan_for(native, "vec_add.small")
+    stream = torch.cuda.current_stream().cuda_stream
+    plan.launch((triton.cdiv(n, 64), 1, 1), stream, [xd.data_ptr(), yd.data_ptr(), zd.data_ptr(), n])
+    torch.cuda.synchronize()
+    assert torch.equal(zd.cpu(), x + y)
+    plan.launch((0, 1, 1), stream, [0, 0, 0, n])  # empty grid: nothing is dereferenced
+
+
+# ------------------------------------------------------------------ cfg2
+def test_cfg2_softmax(K, oracle_cpu):
+    torch.manual_seed(0)
+    x = torch.randn(4096, 781)
+    xd = x.to(DEV)
+    od = torch.full((4096, 781), 3.0, device=DEV)
+    k = K.row_softmax[(4096,)](od, xd, xd.stride(0), od.stride(0), 781, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "row_softmax"
+    ref = oracle_cpu.row_softmax(x)
+    assert (od.cpu() - ref).abs().max().item() <= 1e-5
+    assert (od.cpu().double() - torch.softmax(x.double(), 1)).abs().max().item() <= 1e-5
+    assert torch.allclose(od.sum(1), torch.ones(4096, device=DEV), atol=1e-5)
+
+
+@pytest.mark.parametrize("rows,cols,block,pad", [(1823, 781, 1024, 0), (33, 1, 64, 5), (7, 64, 64, 3), (5, 4096, 4096, 0),
+                                                (3, 6000, 8192, 8), (9, 130, 256, 1)])
+def test_softmax_shapes_and_pitches(K, oracle_cpu, rows, cols, block, pad):
+    torch.manual_seed(rows)
+    xfull = torch.randn(rows, cols + pad)
+    x = xfull[:, :cols]
+    xd = xfull.to(DEV)[:, :cols]
+    ofull = torch.full((rows, cols + pad), -9.0, device=DEV)
+    od = ofull[:, :cols]
+    K.row_softmax[(rows,)](od, xd, xd.stride(0), od.stride(0), cols, BLOCK=block)
+    torch.cuda.synchronize()
+    assert torch.allclose(od.cpu(), torch.softmax(x, 1))   # the reference's assertion (test_softmax.py:65)
+    assert (od.cpu() - oracle_cpu.row_softmax(x.contiguous(), BLOCK=block)).abs().max().item() <= 1e-5
+    if pad:
+        assert torch.equal(ofull[:, cols:].cpu(), torch.full((rows, pad), -9.0))  # columns beyond the mask untouched
+
+
+# ------------------------------------------------------------------ cfg3
+def _ln_inputs(M, N, dtype, seed=0):
+    torch.manual_seed(seed)
+    x = torch.randn(M, N).to(dtype)
+    w = (1 + 0.1 * torch.randn(N)).to(dtype)
+    b = (0.1 * torch.randn(N)).to(dtype)
+    return x, w, b
+
+
+def _run_ln(K, x, w, b, eps, block=1024):
+    M, N = x.shape
+    xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
+    yd = torch.zeros_like(xd)
+    mean = torch.zeros(M, dtype=torch.float32, device=DEV)
+    rstd = torch.zeros(M, dtype=torch.float32, device=DEV)
+    k = K.layer_norm_fwd[(M,)](xd, yd, wd, bd, mean, rstd, xd.stride(0), N, eps, BLOCK=block)
+    torch.cuda.synchronize()
+    assert k.function.family == "layernorm_fwd"
+    return yd.cpu(), mean.cpu(), rstd.cpu()
+
+
+def test_cfg3_layernorm(K, oracle_cpu):
+    x, w, b = _ln_inputs(4096, 8192, torch.float16)
+    y, mean, rstd = _run_ln(K, x, w, b, 1e-5)
+    yr, mr, rr = oracle_cpu.layer_norm_fwd(x, w, b, 1e-5)
+    assert (y.float() - yr.float()).abs().max().item() <= 1e-2
+    assert (mean - mr).abs().max().item() <= 1e-5
+    assert ((rstd - rr) / rr).abs().max().item() <= 1e-5
+    # almost every output is the same fp16 value; the rest differ by one rounding
+    assert (y != yr).float().mean().item() < 0.02
+
+
+@pytest.mark.parametrize("M,N,dtype", [(1151, 8192, torch.float16), (17, 1000, torch.float16), (5, 8191, torch.float16),
+                                      (3, 64, torch.float16), (9, 16384, torch.float16), (2, 20000, torch.float16),
+                                      (33, 4096, torch.bfloat16), (4, 777, torch.bfloat16)])
+def test_layernorm_shapes(K, oracle_cpu, M, N, dtype):
+    x, w, b = _ln_inputs(M, N, dtype, seed=N)
+    y, mean, rstd = _run_ln(K, x, w, b, 1e-5)
+    yr, mr, rr = oracle_cpu.layer_norm_fwd(x, w, b, 1e-5)
+    tol = 1e-2 if dtype == torch.float16 else 4e-2      # one bf16 ulp at |y| ~ 4
+    assert (y.float() - yr.float()).abs().max().item() <= tol
+    assert (mean - mr).abs().max().item() <= 1e-5 and ((rstd - rr) / rr).abs().max().item() <= 1e-5
+
+
+# ------------------------------------------------------------------ cfg4
+def _run_mm(K, a, b, BM=128, BN=128, BK=64):
+    M, Kd = a.shape
+    N = b.shape[1]
+    ad, bd = a.to(DEV), b.to(DEV)
+    cd = torch.full((M, N), 5.0, dtype=a.dtype, device=DEV)
+    grid = (triton.cdiv(M, BM) * triton.cdiv(N, BN),)
+    k = K.matmul_tiles[grid](ad, bd, cd, M, N, Kd, ad.stride(0), ad.stride(1), bd.stride(0), bd.stride(1),
+                             cd.stride(0), cd.stride(1), BM=BM, BN=BN, BK=BK, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm"
+    return cd
+
+
+def test_cfg4_gemm_4096(K, oracle_cpu):
+    torch.manual_seed(0)
+    a = (torch.randn(4096, 4096) * 0.02).bfloat16()
+    b = (torch.randn(4096, 4096) * 0.02).bfloat16()
+    cd = _run_mm(K, a, b)
+    ref = torch.matmul(a.to(DEV).float(), b.to(DEV).float())     # fp32 on the GPU: the full-size check
+    assert relfro(cd.float(), ref) <= 1e-2
+    # the oracle on four programs of the grid (first, a group boundary, the middle, the last)
+    c = cd.cpu()
+    for pid in (0, 255, 517, 1023):
+        tile = torch.zeros(4096, 4096, dtype=torch.bfloat16)
+        oracle_cpu.matmul_tiles(a, b, pids=(pid, pid + 1), out=tile)
+        nz = tile.nonzero()
+        r0, c0 = nz[:, 0].min().item() // 128 * 128, nz[:, 1].min().item() // 128 * 128
+        assert relfro(c[r0:r0 + 128, c0:c0 + 128], tile[r0:r0 + 128, c0:c0 + 128]) <= 1e-2
+
+
+def test_gemm_exact_against_permutation(K):
+    # size-independent property at full size: A @ P for a permutation matrix P permutes columns exactly;
+    # a transposed operand, a wrong tile origin or a wrong lane mapping cannot pass
+    torch.manual_seed(1)
+    n = 4096
+    a = torch.randn(n, n).bfloat16()
+    perm = torch.randperm(n)
+    p = torch.zeros(n, n)
+    p[perm, torch.arange(n)] = 1.0
+    cd = _run_mm(K, a, p.bfloat16())
+    assert torch.equal(cd.cpu(), a[:, perm])
+
+
+@pytest.mark.parametrize("M,N,Kd,dtype", [(179, 321, 167, torch.bfloat16), (179, 321, 167, torch.float16),
+                                         (128, 128, 64, torch.bfloat16), (2, 3, 5, torch.bfloat16),
+                                         (130, 257, 72, torch.bfloat16), (256, 384, 200, torch.float16),
+                                         (2048, 2304, 96, torch.bfloat16)])
+def test_gemm_ragged_shapes(K, oracle_cpu, M, N, Kd, dtype):
+    torch.manual_seed(M + N)
+    a, b = (torch.randn(M, Kd) * 0.5).to(dtype), (torch.randn(Kd, N) * 0.5).to(dtype)
+    cd = _run_mm(K, a, b)
+    assert relfro(cd.cpu(), a.double() @ b.double()) <= 1e-2
+    if M * N * Kd <= 179 * 321 * 167:
+        assert relfro(cd.cpu(), oracle_cpu.matmul_tiles(a, b)) <= 1e-2
+
+
+def test_gemm_with_padded_pitches_and_untouched_border(K):
+    torch.manual_seed(3)
+    M, N, Kd = 200, 300, 150
+    A, B = (torch.randn(M, Kd + 8) * 0.5).bfloat16().to(DEV), (torch.randn(Kd, N + 16) * 0.5).bfloat16().to(DEV)
+    Cfull = torch.full((M, N + 8), 5.0, dtype=torch.bfloat16, device=DEV)
+    a, b, c = A[:, :Kd], B[:, :N], Cfull[:, :N]
+    K.matmul_tiles[(triton.cdiv(M, 128) * triton.cdiv(N, 128),)](a, b, c, M, N, Kd, a.stride(0), 1, b.stride(0), 1,
+                                                               c.stride(0), 1, BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert relfro(c.cpu(), a.cpu().double() @ b.cpu().double()) <= 1e-2
+    assert torch.equal(Cfull[:, N:].cpu(), torch.full((M, 8), 5.0, dtype=torch.bfloat16))
+
+
+# ------------------------------------------------------------------ cfg5
+def _run_w8(K, a, w, s, BN=128, BK=128):
+    M, Kd = a.shape
+    N = w.shape[1]
+    ad, wd, sd = a.to(DEV), w.to(DEV), s.to(DEV)
+    cd = torch.full((M, N), 5.0, dtype=torch.float16, device=DEV)
+    k = K.w8a16_matmul[(triton.cdiv(M, 16), triton.cdiv(N, BN))](ad, wd, sd, cd, M, N, Kd, ad.stride(0), 1, wd.stride(0), 1,
+                                                                cd.stride(0), 1, BM=16, BN=BN, BK=BK)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm_w8a16"
+    return cd
+
+
+def test_cfg5_w8a16(K, oracle_cpu):
+    torch.manual_seed(0)
+    M, N, Kd = 16, 28672, 8192
+    a = torch.randn(M, Kd).half()
+    w = torch.randint(-127, 128, (Kd, N), dtype=torch.int8)
+    s = (0.001 + 0.009 * torch.rand(N)).half()
+    cd = _run_w8(K, a, w, s)
+    ref = a.to(DEV).float() @ (w.to(DEV).half() * s.to(DEV)[None, :]).float()   # closed form, full size
+    assert relfro(cd.float(), ref) <= 1e-2
+    part = torch.zeros(M, N, dtype=torch.float16)
+    for y in (0, 100, 223):                                                      # oracle on three column blocks
+        oracle_cpu.w8a16_matmul(a, w, s, ys=(y, y + 1), out=part)
+        assert relfro(cd.cpu()[:, y * 128:(y + 1) * 128], part[:, y * 128:(y + 1) * 128]) <= 1e-2
+
+
+def test_w8a16_exact_selection(K):
+    # W picks and negates single rows, scales are powers of two: the result is exact in fp16
+    torch.manual_seed(2)
+    M, N, Kd = 16, 28672, 8192
+    a = torch.randn(M, Kd).half()
+    cols = torch.arange(N)
+    rows = (cols * 7) % Kd
+    w = torch.zeros(Kd, N, dtype=torch.int8)
+    sign = torch.where(cols % 2 == 0, 1, -1).to(torch.int8)
+    w[rows, cols] = sign * 3
+    s = torch.where(cols % 3 == 0, 0.5, 0.25).half()
+    cd = _run_w8(K, a, w, s)
+    want = (a[:, rows].float() * (sign.float() * 3 * s.float())[None, :]).half()
+    assert torch.equal(cd.cpu(), want)
+
+
+@pytest.mark.parametrize("M,N,Kd", [(13, 1000, 1000), (16, 256, 512), (1, 130, 70), (16, 4096, 4096), (5, 128, 8192)])
+def test_w8a16_ragged_shapes(K, oracle_cpu, M, N, Kd):
+    torch.manual_seed(N)
+    a = torch.randn(M, Kd).half()
+    w = torch.randint(-127, 128, (Kd, N), dtype=torch.int8)
+    s = (0.001 + 0.009 * torch.rand(N)).half()
+    cd = _run_w8(K, a, w, s)
+    ref = a.double() @ (w.half() * s[None, :]).double()
+    assert relfro(cd.cpu(), ref) <= 1e-2
+    if N * Kd <= 1000 * 1000:
+        assert relfro(cd.cpu(), oracle_cpu.w8a16_matmul(a, w, s)) <= 1e-2
+
+
+# ------------------------------------------------------------- error paths
+def test_errors_surface_as_python_exceptions(K):
+    import extra_kernels as X
+    x = torch.zeros(1024, device=DEV)
+    with pytest.raises(TypeError, match="device"):
+        K.vec_add[(1,)](torch.zeros(1024), x, x, 1024, BLOCK=1024)     # host tensor
+    with pytest.raises(NotImplementedError):
+        X.fused_mul_add[(1,)](x, x, x, 1024, BLOCK=256)                # matches no family: refused, no fallback
+    with pytest.raises(NotImplementedError, match="one program per output tile"):
+        a = torch.zeros(256, 256, dtype=torch.bfloat16, device=DEV)
+        K.matmul_tiles[(3,)](a, a, a, 256, 256, 256, 256, 1, 256, 1, 256, 1, BM=128, BN=128, BK=64, GROUP_M=8)

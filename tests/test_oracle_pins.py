@@ -1,0 +1,169 @@
+"""Pins the oracle (oracle/cpu_path.c and oracle/ttir_lanes.py) before anything
+is compared against it: closed forms, library routines, brute force on tiny
+inputs, and agreement of the two independent restatements.  No GPU."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import golden_ttir
+from oracle import ttir_lanes
+
+
+# ---------------------------------------------------------------- primitives
+def test_valid_extent_matches_counting_true_lanes(oracle_cpu):
+    # MaskAnalysis.cpp:568-585: dims = max(min(start+size, bound), start) - start.  A dropped max()
+    # (negative extent when bound < start) or a swapped min/max fails this.
+    L = oracle_cpu.lib()
+    for start in (-3, 0, 5, 64, 1000):
+        for size in (1, 16, 64):
+            for bound in (-10, 0, 3, 5, 6, 64, 70, 1000, 1063, 1064, 5000):
+                lanes = start + np.arange(size)
+                assert L.oracle_valid_extent(start, size, bound) == int((lanes < bound).sum())
+
+
+def test_half_conversions_match_torch(oracle_cpu):
+    L = oracle_cpu.lib()
+    rng = np.random.default_rng(0)
+    vals = np.concatenate([rng.standard_normal(4000).astype(np.float32) * 10.0 ** rng.integers(-9, 6, 4000),
+                           np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 65536.0, 1e-8, 2.0 ** -24, 2.0 ** -25,
+                                     2.0 ** -25 * 1.0001, 6.1e-5, 6.0e-8, np.inf, -np.inf], dtype=np.float32)])
+    t = torch.from_numpy(vals)
+    want16 = t.half().view(torch.int16).numpy().view(np.uint16)
+    wantbf = t.bfloat16().view(torch.int16).numpy().view(np.uint16)
+    for v, h, b in zip(vals, want16, wantbf):
+        assert L.oracle_f32_to_f16(float(v)) == h, v
+        assert L.oracle_f32_to_bf16(float(v)) == b, v
+    all16 = np.arange(65536, dtype=np.uint16)
+    back = torch.from_numpy(all16.view(np.int16)).view(torch.float16).float().numpy()
+    for h in list(range(0, 65536, 97)) + [0x7c00, 0xfc00, 0x0001, 0x03ff, 0x0400]:
+        got = L.oracle_f16_to_f32(int(h))
+        assert got == back[h] or (np.isnan(got) and np.isnan(back[h]))
+
+
+# -------------------------------------------------- C restatement vs closed forms
+def test_vec_add_is_ieee_addition(oracle_cpu):
+    torch.manual_seed(0)
+    for n in (1, 127, 1024, 98432):
+        x, y = torch.rand(n), torch.rand(n)
+        assert torch.equal(oracle_cpu.vec_add(x, y), x + y)  # bit-exact
+
+
+def test_softmax_matches_torch_and_float64(oracle_cpu):
+    torch.manual_seed(0)
+    x = torch.randn(1823, 781)  # the reference's own test shape (python/examples/test_softmax.py:60-65)
+    y = oracle_cpu.row_softmax(x)
+    assert torch.allclose(y, torch.softmax(x, 1))  # the reference's assertion
+    assert (y.double() - torch.softmax(x.double(), 1)).abs().max() <= 1e-6
+    assert torch.allclose(y.sum(1), torch.ones(1823), atol=1e-5)
+
+
+def _layernorm_f64(x, w, b, eps):
+    xf = x.double()
+    mu = xf.mean(1)
+    var = ((xf - mu[:, None]) ** 2).mean(1)  # biased
+    rs = 1 / torch.sqrt(var + eps)
+    return (xf - mu[:, None]) * rs[:, None] * w.double() + b.double(), mu, rs
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N", [8192, 1000, 64])
+def test_layernorm_matches_float64_formula(oracle_cpu, dtype, N):
+    torch.manual_seed(1)
+    x = (torch.randn(37, N) * 1.5 - 0.3).to(dtype)
+    w, b = (1 + 0.1 * torch.randn(N)).to(dtype), (0.1 * torch.randn(N)).to(dtype)
+    y, mean, rstd = oracle_cpu.layer_norm_fwd(x, w, b, 1e-5, BLOCK=1024 if N > 64 else 64)
+    yr, mu, rs = _layernorm_f64(x, w, b, 1e-5)
+    tol = 1e-2 if dtype == torch.float16 else 5e-2
+    assert (y.double() - yr).abs().max() <= tol
+    assert (mean.double() - mu).abs().max() <= 1e-5
+    assert ((rstd.double() - rs) / rs).abs().max() <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_matmul_matches_float64(oracle_cpu, dtype):
+    torch.manual_seed(2)
+    # ragged in every dimension, as python/examples/test_matmul.py:137-157 (179x167x321)
+    a, b = (torch.randn(179, 167) * 0.5).to(dtype), (torch.randn(167, 321) * 0.5).to(dtype)
+    c = oracle_cpu.matmul_tiles(a, b, BM=32, BN=64, BK=16, GROUP_M=8)
+    ref = a.double() @ b.double()
+    assert torch.allclose(c.double(), ref, atol=1e-2 * ref.abs().max().item(), rtol=0)
+    assert (c.double() - ref).norm() / ref.norm() <= 1e-2
+    # transposed operand would fail: the product is not symmetric
+    assert (c.double() - (b.double().T @ a.double().T).T).norm() / ref.norm() <= 1e-2
+
+
+def test_w8a16_matches_closed_form(oracle_cpu):
+    torch.manual_seed(3)
+    a = torch.randn(16, 300).half()
+    w = torch.randint(-127, 128, (300, 200), dtype=torch.int8)
+    s = (0.001 + 0.009 * torch.rand(200)).half()
+    c = oracle_cpu.w8a16_matmul(a, w, s, BN=64, BK=64)
+    ref = a.double() @ (w.half() * s[None, :]).double()  # dequantised weights rounded to fp16 first
+    assert (c.double() - ref).norm() / ref.norm() <= 2e-3
+    # scale per *output channel*: scaling rows instead would fail
+    wrong = a.double() @ (w.double() * s.double()[:200][None, :].flip(1))
+    assert (c.double() - wrong).norm() / ref.norm() > 0.1
+
+
+# ---------------------------------- lane interpreter vs C restatement (independent)
+def _u16(t):
+    return t.view(torch.int16).numpy().view(np.uint16).reshape(-1)
+
+
+def test_lanes_vs_c_vec_add(oracle_cpu):
+    torch.manual_seed(0)
+    n, B = 333, 64
+    x, y, z = torch.rand(n), torch.rand(n), torch.zeros(n)
+    it = ttir_lanes.Interpreter(golden_ttir("vec_add.small"))
+    grid = (n + B - 1) // B + 2  # two programs entirely past the end: all-masked
+    log = it.run((grid,), [None, None, None, n], {0: x.numpy(), 1: y.numpy(), 2: z.numpy()})
+    assert torch.equal(z, oracle_cpu.vec_add(x, y, BLOCK=B))
+    counts = [len(a[2]) for a in (prog[2] for prog in log)]
+    assert counts == [oracle_cpu.lib().oracle_valid_extent(p * B, B, n) for p in range(grid)]
+    assert counts[-1] == 0 and counts[-2] == 0 and counts[5] == 333 - 320
+
+
+def test_lanes_vs_c_softmax(oracle_cpu):
+    torch.manual_seed(0)
+    x, o = torch.randn(9, 50), torch.zeros(9, 50)
+    it = ttir_lanes.Interpreter(golden_ttir("row_softmax.small"))
+    it.run((9,), [None, None, 50, 50, 50], {0: o.numpy().reshape(-1), 1: x.numpy().reshape(-1)})
+    ref = oracle_cpu.row_softmax(x, BLOCK=64)
+    assert (o - ref).abs().max() <= 1e-7  # np.exp vs libm expf
+    assert torch.allclose(o, torch.softmax(x, 1))
+
+
+def test_lanes_vs_c_layernorm(oracle_cpu):
+    torch.manual_seed(0)
+    M, N = 5, 150
+    x, w, b = torch.randn(M, N).half(), torch.randn(N).half(), torch.randn(N).half()
+    y, mean, rstd = torch.zeros(M, N).half(), torch.zeros(M), torch.zeros(M)
+    it = ttir_lanes.Interpreter(golden_ttir("layer_norm_fwd.small"))
+    it.run((M,), [None] * 6 + [N, N, 1e-5], {0: x.numpy().reshape(-1), 1: y.numpy().reshape(-1), 2: w.numpy(),
+                                             3: b.numpy(), 4: mean.numpy(), 5: rstd.numpy()})
+    y2, m2, r2 = oracle_cpu.layer_norm_fwd(x, w, b, 1e-5, BLOCK=64)
+    assert torch.equal(y, y2) and torch.equal(mean, m2) and torch.equal(rstd, r2)
+
+
+def test_lanes_vs_c_matmul(oracle_cpu):
+    torch.manual_seed(0)
+    M, N, K = 70, 90, 40
+    a, b = (torch.randn(M, K) * 0.5).bfloat16(), (torch.randn(K, N) * 0.5).bfloat16()
+    c = torch.zeros(M, N).bfloat16()
+    it = ttir_lanes.Interpreter(golden_ttir("matmul_tiles.small"))
+    grid = ((M + 31) // 32) * ((N + 31) // 32)
+    it.run((grid,), [None, None, None, M, N, K, K, N, N], {0: _u16(a), 1: _u16(b), 2: _u16(c)})
+    assert torch.equal(c, oracle_cpu.matmul_tiles(a, b, BM=32, BN=32, BK=16, GROUP_M=2))
+
+
+def test_lanes_vs_c_w8a16(oracle_cpu):
+    torch.manual_seed(0)
+    M, N, K = 13, 70, 100
+    a = torch.randn(M, K).half()
+    w = torch.randint(-127, 128, (K, N), dtype=torch.int8)
+    s = (0.001 + 0.009 * torch.rand(N)).half()
+    c = torch.zeros(M, N).half()
+    it = ttir_lanes.Interpreter(golden_ttir("w8a16_matmul.small"))
+    it.run((1, (N + 31) // 32), [None] * 4 + [M, N, K, K, N, N],
+           {0: a.numpy().reshape(-1), 1: w.numpy().reshape(-1), 2: s.numpy(), 3: c.numpy().reshape(-1)})
+    assert torch.equal(c, oracle_cpu.w8a16_matmul(a, w, s, BM=16, BN=32, BK=32))

@@ -1,0 +1,283 @@
+"""Host-side tests of the native planner: TTIR text -> structured program ->
+kernel family + bindings.  The expectations are hand-encoded from the CHECK lines
+of the reference's lit tests (read, not copied) and pinned by brute force with
+the independent lane interpreter.  No GPU."""
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import golden_ttir, plan_for
+from oracle import ttir_lanes
+
+
+def accesses(structured):
+    """[(kind, readable comment)] of every load/store line, in program order."""
+    out = []
+    for line in structured.splitlines():
+        m = re.match(r"\s*(load|store|scalar_store|scalar_load)\b.*? ; (.*)$", line)
+        if m:
+            out.append((m.group(1), m.group(2)))
+    return out
+
+
+def compile_ttir(fn, sig, consts):
+    import os
+    import triton
+    from triton.backends.compiler import GPUTarget
+    from triton.compiler import ASTSource
+    import triton_shared_amd as tsa
+    tsa.register_backend()
+    os.environ.setdefault("TRITON_ALWAYS_COMPILE", "1")
+    # stop after the TTIR stage by asking for the asm of a kernel that may not match any family
+    from triton_shared_amd.backend.compiler import HIPBackend
+    src = ASTSource(fn, signature=sig, constexprs=consts)
+    target = GPUTarget(tsa.BACKEND_NAME, "gfx950", 64)
+    backend = HIPBackend(target)
+    from triton._C.libtriton import ir
+    ctx = ir.context()
+    ir.load_dialects(ctx)
+    options = backend.parse_options({})
+    mod = src.make_ir(target, options, backend.get_codegen_implementation(options), backend.get_module_map(), ctx)
+    return str(backend.make_ttir(mod, {}, options))
+
+
+# ------------------------------------------------- goldens from the lit tests
+def test_vec_add_structured_matches_reference_golden(native):
+    # test/Conversion/TritonToStructured/kernel-01-vector-add.mlir CHECK :27-65:
+    # sizes [1024], strides [1], offsets [index_cast(pid*1024)], dims = max(min(off+1024, n), off) - off,
+    # the same for both loads and the store; addf on the two loaded tiles.
+    s = native.ttir_to_structured(golden_ttir("vec_add"))
+    acc = accesses(s)
+    assert [k for k, _ in acc] == ["load", "load", "store"]
+    dims = "dims=[(max((1024 * pid.x), min(((1024 * pid.x) + 1024), arg3)) - (1024 * pid.x))]"
+    for (kind, text), arg in zip(acc, ("%x_ptr", "%y_ptr", "%z_ptr")):
+        assert text.startswith(arg + " offsets=[(1024 * pid.x)] strides=[1] " + dims), text
+    assert "sizes=[1024]" in s and s.count("name=arith.addf") == 1
+    assert " other" not in s  # tail lanes are left as they are: no fill
+
+
+def test_softmax_structured_matches_reference_golden(native):
+    # kernel-02-fused-softmax.mlir CHECK :46-75 (there with block 128): offsets [index_cast(pid*stride)],
+    # dims = max(min(n_cols, BLOCK), 0), other = -inf on the load, none on the store.
+    s = native.ttir_to_structured(golden_ttir("row_softmax"))
+    (k0, ld), (k1, st) = accesses(s)
+    assert (k0, k1) == ("load", "store")
+    assert ld == "%in_ptr offsets=[(arg2 * pid.x)] strides=[1] dims=[max(0, min(1024, arg4))] other=-inf"
+    assert st == "%out_ptr offsets=[(pid.x * arg3)] strides=[1] dims=[max(0, min(1024, arg4))]"
+    names = re.findall(r"name=([\w.]+)", s)
+    assert names == ["arith.maxnumf", "arith.subf", "math.exp", "arith.addf", "arith.divf"]
+
+
+def test_matmul_structured_matches_reference_golden(native):
+    # kernel-03-matrix-multiplication.mlir CHECK :155-190: loop-carried offsets, the K advance of both
+    # operands lands in dimension 0 (a splat constant is an offset of the outermost dimension,
+    # PtrAnalysis.cpp:1068-1100), strides [stride_am, 1] / [stride_bk, 1], 2-D store mask as a min per dim.
+    s = native.ttir_to_structured(golden_ttir("matmul_tiles"))
+    iters = re.findall(r"int_iter .*? ; (it0\.\d) = (.*) then (.*)$", s, re.M)
+    by = {n: (init, nxt) for n, init, nxt in iters}
+    assert by["it0.0"][1] == "(it0.0 + 64)" and by["it0.0"][0].startswith("(arg6 * (128 * ")   # A: row0*stride_am, += BK
+    assert by["it0.1"] == ("0", "it0.1")
+    assert by["it0.2"] == ("arg6", "it0.2") and by["it0.3"] == ("1", "it0.3")
+    assert by["it0.4"] == ("0", "(it0.4 + (arg7 * 64))")                                      # B: += BK*stride_bk
+    assert by["it0.5"][1] == "it0.5" and by["it0.6"] == ("arg7", "it0.6") and by["it0.7"] == ("1", "it0.7")
+    acc = accesses(s)
+    assert [k for k, _ in acc] == ["load", "load", "store"]
+    assert "strides=[arg8, 1]" in acc[2][1]
+    assert acc[2][1].count("min(128, ") == 2          # minsi(dim, 128) on both store dims (CHECK :188-189)
+    assert "for loop=0" in s and "0 to ((63 + arg5) / 64) step 1" in s
+    assert s.count(" dot ") == 1 and "name=arith.truncf" in s
+
+
+def test_layernorm_structured(native):
+    # kernel-05-layer-norm-fwd.mlir: three scf.for over column blocks, scalar stores of mean and rstd
+    # at offset pid, masked loads padding with 0.
+    s = native.ttir_to_structured(golden_ttir("layer_norm_fwd"))
+    acc = accesses(s)
+    assert [k for k, _ in acc] == ["load", "load", "scalar_store", "scalar_store", "load", "load", "load", "store"]
+    assert acc[2][1].startswith("%Mean offsets=[pid.x]") and acc[3][1].startswith("%Rstd offsets=[pid.x]")
+    assert acc[0][1] == "%X offsets=[((arg6 * pid.x) + iv0)] strides=[1] dims=[(max(iv0, min((iv0 + 1024), arg7)) - iv0)] other=0"
+    assert acc[4][1].startswith("%W offsets=[iv2] strides=[1]") and "other" not in acc[4][1]
+    assert s.count("for loop=") == 3 and s.count("0 to arg7 step 1024") == 3
+
+
+def test_masked_2d_window_matches_reference_golden(native):
+    # test/Conversion/TritonToStructured/masked_ldst_2d.mlir CHECK :75-98: sizes [128, 256],
+    # strides [1, 1024], offsets [2, 3072], dims [min(max(min(rows,130),2)-2,128), min(max(min(cols,259),3)-3,256)],
+    # other = -inf.
+    import extra_kernels as X
+    ttir = compile_ttir(X.masked_copy_2d, {"src": "*bf16", "dst": "*bf16", "rows": "i32", "cols": "i32"}, {})
+    s = native.ttir_to_structured(ttir)
+    (k0, ld), (k1, st) = accesses(s)
+    assert "sizes=[128,256]" in s
+    want = ("offsets=[2, 3072] strides=[1, 1024] "
+            "dims=[min(128, (max(2, min(130, arg2)) - 2)), min(256, (max(3, min(259, arg3)) - 3))]")
+    assert ld == "%src " + want + " other=-inf"
+    assert st == "%dst " + want
+    with pytest.raises(NotImplementedError, match="no hand-written kernel family"):
+        native.structured_to_plan(s)
+
+
+# ---------------------------------------------------------------- text form
+@pytest.mark.parametrize("name", ["vec_add", "row_softmax", "layer_norm_fwd", "matmul_tiles", "w8a16_matmul"])
+def test_family_and_signature(native, name):
+    plan, structured = plan_for(native, name)
+    want = {"vec_add": "map1d", "row_softmax": "row_softmax", "layer_norm_fwd": "layernorm_fwd",
+            "matmul_tiles": "gemm", "w8a16_matmul": "gemm_w8a16"}[name]
+    assert plan.family == want and plan.kernel_name == name
+    # the small-block variant has the same op structure, hence the same signature
+    small, _ = plan_for(native, name + ".small")
+    assert small.signature == plan.signature and small.family == want
+
+
+def test_plan_bytes_are_self_contained(native):
+    structured = native.ttir_to_structured(golden_ttir("row_softmax"))
+    plan_bytes, name = native.structured_to_plan(structured)
+    assert name == "row_softmax" and plan_bytes.startswith(b"tts.plan 1 family=row_softmax\n")
+    with pytest.raises(ValueError):
+        native.PlanHandle(b"garbage")
+    with pytest.raises(ValueError, match="disagree"):
+        native.PlanHandle(plan_bytes.replace(b"family=row_softmax", b"family=gemm", 1))
+
+
+# ------------------------------------------------------------------ refusals
+def test_unsupported_kernels_are_refused(native):
+    import extra_kernels as X
+    sig = {"src": "*fp32", "dst": "*fp32", "M": "i32", "BLOCK": "constexpr"}
+    with pytest.raises(NotImplementedError, match="modulo"):
+        native.ttir_to_structured(compile_ttir(X.wraparound_rows, sig, {"BLOCK": 64}))
+    sig = {"src": "*fp32", "idx": "*i32", "dst": "*fp32", "BLOCK": "constexpr"}
+    with pytest.raises(NotImplementedError, match="not a structured access"):
+        native.ttir_to_structured(compile_ttir(X.gather_rows, sig, {"BLOCK": 64}))
+    sig = {"x_ptr": "*fp32", "y_ptr": "*fp32", "z_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"}
+    s = native.ttir_to_structured(compile_ttir(X.fused_mul_add, sig, {"BLOCK": 256}))
+    with pytest.raises(NotImplementedError, match="no hand-written kernel family"):
+        native.structured_to_plan(s)
+    with pytest.raises(NotImplementedError):
+        native.ttir_to_structured("module {\n  tt.func public @k(%a: !tt.ptr<f32>) {\n    %0 = foo.bar %a : i32\n    tt.return\n  }\n}\n")
+
+
+def test_operand_order_is_kept(native):
+    import extra_kernels as X
+    sig = {"x_ptr": "*fp32", "y_ptr": "*fp32", "z_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"}
+    s = native.ttir_to_structured(compile_ttir(X.vec_sub_swapped, sig, {"BLOCK": 128}))
+    plan = native.PlanHandle(native.structured_to_plan(s)[0])
+    d = plan.describe_launch((4, 1, 1), [0, 0, 0, 500])
+    assert d["kernel"] == "map1d_f32" and d["op"] == "1" and d["swap"] == "1" and d["block"] == "128"
+
+
+# --------------------------------- bindings vs brute force (lane interpreter)
+def affine(text, x, y=0, z=0):
+    c0, cx, cy, cz = [int(v) for v in re.match(r"(-?\d+)\+(-?\d+)\*x\+(-?\d+)\*y\+(-?\d+)\*z", text).groups()]
+    return c0 + cx * x + cy * y + cz * z
+
+
+@pytest.mark.parametrize("n", [333, 64, 1, 640])
+def test_map1d_binding_matches_every_lane(native, n):
+    B = 64
+    grid = (n + B - 1) // B + 1  # one extra, fully masked program
+    plan, _ = plan_for(native, "vec_add.small")
+    d = plan.describe_launch((grid, 1, 1), [0, 0, 0, n])
+    x = np.zeros(n + 2 * B, np.float32)
+    log = ttir_lanes.Interpreter(golden_ttir("vec_add.small")).run((grid,), [None, None, None, n],
+                                                                     {0: x, 1: x.copy(), 2: x.copy()})
+    for p, prog in enumerate(log):
+        extent = int(np.clip(int(d["bound"]) - affine(d["m_start"], p), 0, int(d["block"])))
+        for (kind, arg, offs), key in zip(prog, ("x_off", "y_off", "z_off")):
+            start = affine(d[key], p)
+            assert np.array_equal(offs, np.arange(start, start + extent)), (p, kind, arg)
+
+
+def test_softmax_binding_matches_every_lane(native):
+    plan, _ = plan_for(native, "row_softmax.small")
+    rows, n_cols, pitch_in, pitch_out = 7, 50, 70, 60
+    d = plan.describe_launch((rows, 1, 1), [0, 0, pitch_in, pitch_out, n_cols])
+    o, x = np.zeros(rows * pitch_out, np.float32), np.ones(rows * pitch_in, np.float32)
+    log = ttir_lanes.Interpreter(golden_ttir("row_softmax.small")).run(
+        (rows,), [None, None, pitch_in, pitch_out, n_cols], {0: o, 1: x})
+    assert d["other"] == "-inf" and d["block"] == "64"
+    for p, ((k0, a0, ld), (k1, a1, st)) in enumerate(log):
+        assert (a0, a1) == (1, 0)
+        assert np.array_equal(ld, affine(d["in_off"], p) + np.arange(int(d["d_in"])))
+        assert np.array_equal(st, affine(d["out_off"], p) + np.arange(int(d["d_out"])))
+    # n_cols above the block is clamped, a negative one gives 0 (the max with start)
+    assert plan.describe_launch((1, 1, 1), [0, 0, 70, 60, 1000])["d_in"] == "64"
+    assert plan.describe_launch((1, 1, 1), [0, 0, 70, 60, -5])["d_in"] == "0"
+
+
+def test_layernorm_binding_matches_every_lane(native):
+    plan, _ = plan_for(native, "layer_norm_fwd.small")
+    M, N, pitch = 3, 150, 160
+    d = plan.describe_launch((M, 1, 1), [0] * 6 + [pitch, N, 1e-5])
+    assert d["N"] == str(N) and abs(float(d["eps"]) - 1e-5) < 1e-12
+    mem = {0: np.ones(M * pitch, np.float16), 1: np.zeros(M * pitch, np.float16), 2: np.ones(N, np.float16),
+           3: np.ones(N, np.float16), 4: np.zeros(M, np.float32), 5: np.zeros(M, np.float32)}
+    log = ttir_lanes.Interpreter(golden_ttir("layer_norm_fwd.small")).run((M,), [None] * 6 + [pitch, N, 1e-5], mem)
+    for p, prog in enumerate(log):
+        touched = {}
+        for kind, arg, offs in prog:
+            touched.setdefault((kind, arg), []).append(offs)
+        row = np.arange(N)
+        for (kind, arg), key in ((("load", 0), "x_off"), (("store", 1), "y_off"), (("load", 2), "w_off"),
+                                 (("load", 3), "b_off")):
+            got = np.unique(np.concatenate(touched[(kind, arg)]))
+            assert np.array_equal(got, affine(d[key], p) + row), (p, kind, arg)
+        assert touched[("store", 4)][0][0] == affine(d["mean_off"], p)
+        assert touched[("store", 5)][0][0] == affine(d["rstd_off"], p)
+
+
+@pytest.mark.parametrize("shape", [(70, 90, 40), (32, 32, 16), (33, 1, 17)])
+def test_gemm_binding_matches_every_lane(native, shape):
+    M, N, K = shape
+    plan, _ = plan_for(native, "matmul_tiles.small")
+    grid = ((M + 31) // 32) * ((N + 31) // 32)
+    lda, ldb, ldc = K + 3, N + 5, N + 1
+    d = plan.describe_launch((grid, 1, 1), [0, 0, 0, M, N, K, lda, ldb, ldc])
+    assert (d["M"], d["N"], d["K"], d["lda"], d["ldb"], d["ldc"]) == tuple(str(v) for v in (M, N, K, lda, ldb, ldc))
+    mem = {0: np.zeros(M * lda, np.uint16), 1: np.zeros(K * ldb, np.uint16), 2: np.zeros(M * ldc, np.uint16)}
+    log = ttir_lanes.Interpreter(golden_ttir("matmul_tiles.small")).run(
+        (grid,), [None, None, None, M, N, K, lda, ldb, ldc], mem)
+    loads = {0: [], 1: []}
+    stores = []
+    for prog in log:
+        for kind, arg, offs in prog:
+            (stores if kind == "store" else loads[arg]).append(offs)
+    dense = lambda r, c, ld: (np.arange(r)[:, None] * ld + np.arange(c)[None, :]).ravel()
+    assert np.array_equal(np.unique(np.concatenate(loads[0])), dense(M, K, lda))
+    assert np.array_equal(np.unique(np.concatenate(loads[1])), dense(K, N, ldb))
+    all_stores = np.concatenate(stores)
+    assert np.array_equal(np.sort(all_stores), dense(M, N, ldc))  # every element of C exactly once
+
+
+def test_gemm_refuses_grids_that_are_not_the_tile_grid(native):
+    plan, _ = plan_for(native, "matmul_tiles.small")
+    with pytest.raises(NotImplementedError, match="one program per output tile"):
+        plan.describe_launch((5, 1, 1), [0, 0, 0, 70, 90, 40, 40, 90, 90])
+    with pytest.raises(NotImplementedError, match="inner strides|advance"):
+        # K == 0 trips are fine, but a transposed B (stride_bn != 1) is specialised away at compile time;
+        # here the wrong ldb makes b_kstep disagree only if BK*ldb overflows - use a huge pitch
+        plan.describe_launch((12, 1, 1), [0, 0, 0, 70, 90, 40, 40, 2 ** 31 - 1, 90])
+
+
+def test_w8a16_binding(native):
+    plan, _ = plan_for(native, "w8a16_matmul.small")
+    M, N, K = 13, 70, 100
+    d = plan.describe_launch((1, 3, 1), [0, 0, 0, 0, M, N, K, K, N, N])
+    assert (d["M"], d["N"], d["K"], d["lda"], d["ldw"], d["ldc"]) == ("13", "70", "100", "100", "70", "70")
+    with pytest.raises(NotImplementedError, match="M <= 16"):
+        plan.describe_launch((2, 3, 1), [0, 0, 0, 0, 20, N, K, K, N, N])
+
+
+def test_index_overflow_is_detected(native):
+    plan, _ = plan_for(native, "row_softmax")
+    # pid * in_pitch overflows i32 at the last program: the reference would wrap, so must we not assume linearity
+    with pytest.raises(ValueError, match="overflow"):
+        plan.describe_launch((4096, 1, 1), [0, 0, 2 ** 20, 781, 781])
+
+
+def test_argument_checks(native):
+    plan, _ = plan_for(native, "vec_add")
+    with pytest.raises(ValueError, match="arguments"):
+        plan.describe_launch((1, 1, 1), [0, 0, 0])
+    assert plan.describe_launch((0, 1, 1), [0, 0, 0, 5]) == {"kernel": "none"}

@@ -714,8 +714,19 @@ class Lowerer {
     if (n == "arith.constant") return lower_constant(op);
     if (op.results.size() != 1) throw Unsupported("operation " + n + " (line " + std::to_string(op.line) + ")");
     Type rt = result_type(op);
-    if (rt.ptr) return;                          // address computation: PtrAnalysis reads it on demand
-    if (!rt.is_tensor && rt.is_int()) return;    // scalar integer: int_of reads it on demand
+    if (rt.ptr) {  // address computation: PtrAnalysis reads it on demand
+      static const std::set<std::string> ptr_ops = {"tt.addptr", "tt.splat", "tt.broadcast", "tt.expand_dims"};
+      if (!ptr_ops.count(n)) throw Unsupported("pointer-valued operation " + n + " (line " + std::to_string(op.line) + ")");
+      return;
+    }
+    if (!rt.is_tensor && rt.is_int()) {  // scalar integer: int_of reads it on demand
+      static const std::set<std::string> int_ops = {
+          "tt.get_program_id", "tt.get_num_programs", "arith.addi", "arith.subi", "arith.muli", "arith.divsi",
+          "arith.remsi", "arith.minsi", "arith.maxsi", "arith.extsi", "arith.index_cast", "arith.trunci",
+          "arith.select", "arith.cmpi"};
+      if (!int_ops.count(n)) throw Unsupported("scalar integer operation " + n + " (line " + std::to_string(op.line) + ")");
+      return;
+    }
     if (n == "tt.make_range") {
       SOp s;
       s.kind = SK::Iota;
