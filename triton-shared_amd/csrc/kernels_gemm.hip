@@ -190,6 +190,191 @@ hipError_t launch_gemm_cfg(const GemmParams &p, hipStream_t s) {
   return hipGetLastError();
 }
 
+
+// ------------------------------------------- 16-bit GEMM, full-tile fast path
+// For problems made of whole 256 x 256 x BK tiles with 16-byte aligned rows.
+// Workgroup: 512 threads = 8 wavefronts (two per SIMD, so that one computes
+// while the other waits on LDS or the barrier), wave grid 2 (M) x 4 (N), each
+// wavefront 128 x 64 of C = 4 x 2 MFMA tiles.  Wavefronts 0-3 stage A (BK/8
+// 16-byte chunks per thread); wavefronts 4-7 stage B: each thread loads a
+// (BK/8) (k) x 8 (n) block as 16-byte rows, transposes it in registers and writes
+// eight K-contiguous chunks, so that global loads are whole 128-byte row
+// segments and LDS accesses are conflict-free.  DIST tiles are in flight in
+// registers, so global/L2 latency is covered by DIST K steps of MFMA work.
+// LDS: [2 buffers][256 A rows + 256 B columns][BK + 8] 16-bit elements.
+constexpr int F_BM = 256, F_BN = 256;
+
+template <bool BF16, int BK, int DIST, bool EARLY, int DBG>
+__global__ __launch_bounds__(512) void gemm_fast_kernel(GemmParams p, int tiles_m, int tiles_n) {
+  constexpr int PITCH = BK + 8, NL = BK / 8;  // NL: 16-byte loads per thread and tile
+  constexpr int KS = BK / 16;
+  extern __shared__ __align__(16) uint16_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;
+
+  int bid = blockIdx.x;
+  const int nwg = tiles_m * tiles_n;
+  if (nwg % 8 == 0) bid = (bid % 8) * (nwg / 8) + bid / 8;  // consecutive ids on one XCD
+  const int group = 4 * tiles_n;                             // 4-tile-tall column groups
+  const int g0 = (bid / group) * 4;
+  const int gh = min(tiles_m - g0, 4);
+  const int tile_m = g0 + (bid % group) % gh, tile_n = (bid % group) / gh;
+  const int64_t m0 = (int64_t)tile_m * F_BM, n0 = (int64_t)tile_n * F_BN;
+
+  const uint16_t *__restrict__ A = (const uint16_t *)p.a;
+  const uint16_t *__restrict__ B = (const uint16_t *)p.b;
+  const bool loads_a = wave < 4;
+  const int lt = tid & 255;  // index among the 256 threads with the same role
+
+  // A role: chunk c = lt + 256 j -> row c / NL, 16-byte chunk c % NL
+  // B role: unit (kg = lt % 8, nc = lt / 8): rows NL kg .. NL kg + NL - 1, columns 8 nc .. 8 nc + 7
+  const uint16_t *gsrc;
+  int64_t gstep;  // elements between this thread's loads
+  if (loads_a) {
+    gsrc = A + (m0 + lt / NL) * p.lda + (lt % NL) * 8;
+    gstep = (256 / NL) * p.lda;
+  } else {
+    gsrc = B + (int64_t)((lt & 7) * NL) * p.ldb + n0 + (lt >> 3) * 8;
+    gstep = p.ldb;
+  }
+  auto gload = [&](int k0, uint4 (&r)[NL]) {
+    const uint16_t *src = loads_a ? gsrc + k0 : gsrc + (int64_t)k0 * p.ldb;
+#pragma unroll
+    for (int j = 0; j < NL; j++) r[j] = *reinterpret_cast<const uint4 *>(src + j * gstep);
+  };
+  auto lstore = [&](int buf, uint4 (&r)[NL]) {
+    uint16_t *As = smem + buf * (F_BM + F_BN) * PITCH, *Bs = As + F_BM * PITCH;
+    if (loads_a) {
+#pragma unroll
+      for (int j = 0; j < NL; j++)
+        *reinterpret_cast<uint4 *>(As + (lt / NL + (256 / NL) * j) * PITCH + (lt % NL) * 8) = r[j];
+    } else {
+      // r[t] = row k = NL kg + t, columns c = 0..7 (two per 32-bit word); the chunk written for
+      // column c holds k = 0..NL-1 of that column
+      uint32_t in[NL][4];
+#pragma unroll
+      for (int t = 0; t < NL; t++) { in[t][0] = r[t].x; in[t][1] = r[t].y; in[t][2] = r[t].z; in[t][3] = r[t].w; }
+      uint16_t *dst = Bs + ((lt >> 3) * 8) * PITCH + (lt & 7) * NL;
+#pragma unroll
+      for (int c2 = 0; c2 < 4; c2++) {
+        uint32_t even[NL / 2], odd[NL / 2];
+#pragma unroll
+        for (int tp = 0; tp < NL / 2; tp++) {
+          uint32_t x = in[2 * tp][c2], y = in[2 * tp + 1][c2];
+          even[tp] = __builtin_amdgcn_perm(y, x, 0x05040100u);  // [x.lo16, y.lo16]
+          odd[tp] = __builtin_amdgcn_perm(y, x, 0x07060302u);   // [x.hi16, y.hi16]
+        }
+        if (NL == 8) {
+          *reinterpret_cast<uint4 *>(dst + (2 * c2) * PITCH) = make_uint4(even[0], even[1], even[NL / 2 - 2], even[NL / 2 - 1]);
+          *reinterpret_cast<uint4 *>(dst + (2 * c2 + 1) * PITCH) = make_uint4(odd[0], odd[1], odd[NL / 2 - 2], odd[NL / 2 - 1]);
+        } else {
+          *reinterpret_cast<uint2 *>(dst + (2 * c2) * PITCH) = make_uint2(even[0], even[1]);
+          *reinterpret_cast<uint2 *>(dst + (2 * c2 + 1) * PITCH) = make_uint2(odd[0], odd[1]);
+        }
+      }
+    }
+  };
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+  const int nk = (int)(p.K / BK);
+  uint4 r0[NL], r1[NL];
+  // One K step.  Tile kt is in LDS buffer `cur`.  `rnew` is free and receives tile kt+DIST; `rsto`
+  // holds tile kt+1, which goes to the other LDS buffer (free since the barrier that ended step kt-1).
+  auto step = [&](int kt, int cur, uint4 (&rnew)[NL], uint4 (&rsto)[NL]) {
+    if (!(DBG & 4) && kt + DIST < nk) gload((kt + DIST) * BK, rnew);
+    if (EARLY && !(DBG & 4) && kt + 1 < nk) lstore(cur ^ 1, rsto);
+    const uint16_t *As = smem + cur * (F_BM + F_BN) * PITCH, *Bs = As + F_BM * PITCH;
+    const uint16_t *a_base = As + (wm * 128 + (lane & 31)) * PITCH + 8 * (lane >> 5);
+    const uint16_t *b_base = Bs + (wn * 64 + (lane & 31)) * PITCH + 8 * (lane >> 5);
+    uint4 af[2][4], bf[2][2];
+#pragma unroll
+    for (int i = 0; i < 4; i++) af[0][i] = *reinterpret_cast<const uint4 *>(a_base + i * 32 * PITCH);
+#pragma unroll
+    for (int j = 0; j < 2; j++) bf[0][j] = *reinterpret_cast<const uint4 *>(b_base + j * 32 * PITCH);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      const int c = ks & 1, n = c ^ 1;
+      if (!(DBG & 2) && ks + 1 < KS) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) af[n][i] = *reinterpret_cast<const uint4 *>(a_base + i * 32 * PITCH + (ks + 1) * 16);
+#pragma unroll
+        for (int j = 0; j < 2; j++) bf[n][j] = *reinterpret_cast<const uint4 *>(b_base + j * 32 * PITCH + (ks + 1) * 16);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+          if (DBG & 1) acc[i][j][0] += __uint_as_float(af[c][i].x ^ bf[c][j].x);
+          else acc[i][j] = mfma32<BF16>(af[c][i], bf[c][j], acc[i][j]);
+        }
+    }
+    // pin the software pipeline: the fragment reads of step ks+1 are issued before the MFMAs of step
+    // ks, so that LDS latency is covered by eight MFMAs instead of being waited for
+    __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+#pragma unroll
+    for (int ks = 0; ks + 1 < KS; ks++) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+    if (!EARLY && !(DBG & 4) && kt + 1 < nk) lstore(cur ^ 1, rsto);
+    __syncthreads();
+  };
+  gload(0, r0);
+  if (DIST == 2 && nk > 1) gload(BK, r1);
+  lstore(0, r0);
+  __syncthreads();
+  for (int kt = 0; kt < nk; kt += 2) {
+    if (DIST == 2) {
+      step(kt, 0, r0, r1);                        // tile kt was in r0, tile kt+1 is in r1
+      if (kt + 1 < nk) step(kt + 1, 1, r1, r0);
+    } else {
+      step(kt, 0, r0, r0);
+      if (kt + 1 < nk) step(kt + 1, 1, r0, r0);
+    }
+  }
+
+  uint16_t *__restrict__ C = (uint16_t *)p.c;
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      int64_t col = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        int64_t row = m0 + wm * 128 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        C[row * p.ldc + col] = BF16 ? f32_to_bf16(acc[i][j][v]) : f32_to_f16(acc[i][j][v]);
+      }
+    }
+}
+
+template <bool BF16, int BK, int DIST, bool EARLY, int DBG = 0>
+hipError_t launch_gemm_fast(const GemmParams &p, hipStream_t s) {
+  constexpr size_t lds = 2 * (size_t)(F_BM + F_BN) * (BK + 8) * 2;
+  static bool configured = false;
+  auto kern = gemm_fast_kernel<BF16, BK, DIST, EARLY, DBG>;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  int tiles_m = (int)(p.M / F_BM), tiles_n = (int)(p.N / F_BN);
+  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(512), lds, s, p, tiles_m, tiles_n);
+  return hipGetLastError();
+}
+
+bool gemm_fast_path_ok(const GemmParams &p) {
+  return p.M % F_BM == 0 && p.N % F_BN == 0 && p.K % 64 == 0 && p.K >= 64 && p.lda % 8 == 0 && p.ldb % 8 == 0 &&
+         ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0;
+}
+
 // ------------------------------------------------------ int8-weight GEMM
 // Workgroup: NW wavefronts share one 128-column slab of W and split its K range
 // in interleaved steps of 32 rows.  In a step, lane (j = lane % 16, g = lane / 16)
@@ -350,7 +535,13 @@ constexpr int W8_WAVES = 16;
 }  // namespace
 
 hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
-  static const char *tile_env = getenv("TTS_GEMM_TILE");
+  static const char *tile_env = getenv("TTS_GEMM_TILE");  // tuning aid: 128, 256 (general kernel) or unset
+  if (!tile_env && gemm_fast_path_ok(p)) {
+    // BK = 64, one tile in flight, LDS filled after the MFMAs: the fastest of the measured
+    // combinations of BK in {32, 64}, DIST in {1, 2} and EARLY in {false, true} at 4096^3
+    *name = "gemm_fast_kernel";
+    return p.is_bf16 ? launch_gemm_fast<true, 64, 1, false>(p, s) : launch_gemm_fast<false, 64, 1, false>(p, s);
+  }
   bool big = p.M >= 2048 && p.N >= 2048;
   if (tile_env) big = atoi(tile_env) >= 256;
   if (big) {
