@@ -394,7 +394,10 @@ __device__ __forceinline__ uint32_t pk_sub_1152_mul(uint32_t biased, uint32_t sc
   return __builtin_bit_cast(uint32_t, v);
 }
 
-template <int NW>
+// FAST: K is a multiple of 32, N of 128, rows are 8/16-byte aligned: every load is unconditional,
+// so that the compiler keeps all loads of a step (and of DEPTH steps) in flight.  Rows of A beyond
+// M are read from row M-1: they only reach rows of the MFMA result that are never stored.
+template <int NW, int DEPTH, bool FAST>
 __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, int steps_per_slice) {
   constexpr int RW = NW > 4 ? 4 : NW;  // wavefronts combined per round
   __shared__ float red[RW][16][W8_COLS + 4];
@@ -424,7 +427,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, 
   const int step_begin = slice * steps_per_slice;
   const int step_end = min(step_begin + steps_per_slice, (K + 31) / 32);
 
+  const int8_t *w_lane = W + (int64_t)(8 * g) * p.ldw + ncol;
+  const uint16_t *a_lane = A + (int64_t)min(j, (int)p.M - 1) * p.lda + 8 * g;
   auto load_w = [&](int step, uint2 (&q)[8]) {
+    if (FAST) {
+      const int8_t *src = w_lane + (int64_t)step * 32 * p.ldw;
+#pragma unroll
+      for (int t = 0; t < 8; t++) q[t] = *reinterpret_cast<const uint2 *>(src + (int64_t)t * p.ldw);
+      return;
+    }
 #pragma unroll
     for (int t = 0; t < 8; t++) {
       int k = step * 32 + 8 * g + t;
@@ -443,23 +454,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, 
     }
   };
   auto load_a = [&](int step) {
+    if (FAST) return *reinterpret_cast<const uint4 *>(a_lane + step * 32);
     int k = step * 32 + 8 * g;
     return j < p.M ? load8(A + (int64_t)j * p.lda + k, K - k, a_vec) : make_uint4(0, 0, 0, 0);
   };
 
-  uint2 q[8], qn[8];
-  uint4 af, afn;
-  int step = step_begin + wave;
-  if (step < step_end) {
-    load_w(step, q);
-    af = load_a(step);
-  }
-  for (; step < step_end; step += NW) {
-    const int next = step + NW;
-    if (next < step_end) {
-      load_w(next, qn);
-      afn = load_a(next);
-    }
+  auto consume = [&](const uint2 (&q)[8], const uint4 &af) {
 #pragma unroll
     for (int c = 0; c < 8; c++) {
       uint32_t frag[4];
@@ -475,10 +475,22 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, 
       uint4 bfrag = make_uint4(frag[0], frag[1], frag[2], frag[3]);
       acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af), __builtin_bit_cast(f16x8, bfrag), acc[c], 0, 0, 0);
     }
-    if (next < step_end) {
+  };
+  // DEPTH steps are in flight in DEPTH register sets (the loop is unrolled over them, so no
+  // copies), giving a step's loads the time of DEPTH steps' arithmetic to arrive
+  uint2 q[DEPTH][8];
+  uint4 a[DEPTH];
+  int step = step_begin + wave;
 #pragma unroll
-      for (int t = 0; t < 8; t++) q[t] = qn[t];
-      af = afn;
+  for (int d = 0; d < DEPTH; d++)
+    if (step + d * NW < step_end) { load_w(step + d * NW, q[d]); a[d] = load_a(step + d * NW); }
+  for (; step < step_end; step += DEPTH * NW) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) {
+      if (step + d * NW < step_end) {
+        consume(q[d], a[d]);
+        if (step + (d + DEPTH) * NW < step_end) { load_w(step + (d + DEPTH) * NW, q[d]); a[d] = load_a(step + (d + DEPTH) * NW); }
+      }
     }
   }
 
@@ -567,7 +579,12 @@ hipError_t launch_gemm_w8a16(const GemmW8A16Params &p, hipStream_t s, const char
   int slabs = (int)((p.N + W8_COLS - 1) / W8_COLS);
   int steps = (int)((p.K + 31) / 32);
   int steps_per_slice = (steps + p.split - 1) / p.split;
-  hipLaunchKernelGGL((gemm_w8a16_kernel<W8_WAVES>), dim3(slabs, p.split), dim3(W8_WAVES * 64), 0, s, p, steps_per_slice);
+  const bool fast = p.K % 32 == 0 && p.N % W8_COLS == 0 && p.lda % 8 == 0 && p.ldw % 8 == 0 &&
+                    ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.w & 7) == 0;
+  dim3 grid(slabs, p.split);
+  // 16 wavefronts x 2 steps in flight; 8 x 2..6 and 4 x 8 measured the same (HBM-bound) at the decode shape
+  if (fast) hipLaunchKernelGGL((gemm_w8a16_kernel<W8_WAVES, 2, true>), grid, dim3(W8_WAVES * 64), 0, s, p, steps_per_slice);
+  else hipLaunchKernelGGL((gemm_w8a16_kernel<W8_WAVES, 2, false>), grid, dim3(W8_WAVES * 64), 0, s, p, steps_per_slice);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || p.split == 1) return e;
   int64_t outs = p.M * p.N;
