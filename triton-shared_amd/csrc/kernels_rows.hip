@@ -98,8 +98,11 @@ __global__ __launch_bounds__(256) void softmax_f32_kernel(SoftmaxParams p, int g
   const int sub = threadIdx.x / T, t = threadIdx.x % T;
   const int64_t prog = (int64_t)blockIdx.x * ROWS_PER_WG + sub;
   const bool active = prog < programs;
-  const int px = active ? (int)(prog % gx) : 0, py = active ? (int)((prog / gx) % gy) : 0;
-  const int pz = active ? (int)(prog / ((int64_t)gx * gy)) : 0;
+  int px = 0, py = 0, pz = 0;
+  if (active) {
+    if (gy == 1 && programs == gx) px = (int)prog;  // 1-D grid: no divisions
+    else { px = (int)(prog % gx); py = (int)((prog / gx) % gy); pz = (int)(prog / ((int64_t)gx * gy)); }
+  }
   const float *__restrict__ in = p.in + affine(p.in_off, px, py, pz);
   float *__restrict__ out = p.out + affine(p.out_off, px, py, pz);
   const int d_in = active ? (int)p.d_in : 0, d_out = active ? (int)p.d_out : 0;
@@ -194,7 +197,10 @@ __device__ __forceinline__ float block_sum_256(float v, float *red) {
 // One workgroup per row.  The row is read from HBM once and kept in registers
 // as fp32 (CPT chunks of 8 elements per thread); the Triton source's three
 // passes over the row all read these registers.
-template <bool BF16, int CPT>
+// FAST: N is a multiple of 8 and every row of x, y, w, b starts 16-byte aligned, so a chunk is
+// either whole or absent and all loads are unconditional (an absent chunk re-reads chunk 0 and is
+// zeroed), which lets the compiler keep the CPT loads of a thread in flight together.
+template <bool BF16, int CPT, bool FAST>
 __global__ __launch_bounds__(256) void layernorm_fwd_kernel(LayerNormParams p) {
   __shared__ float red[4];
   const int px = blockIdx.x, py = blockIdx.y, pz = blockIdx.z;
@@ -208,7 +214,16 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(LayerNormParams p) {
 #pragma unroll
   for (int c = 0; c < CPT; c++) {
     int i0 = (threadIdx.x + c * 256) * 8;
-    if (vec && i0 + 8 <= N) {
+    if (FAST) {
+      const bool present = i0 < N;
+      uint4 raw = *reinterpret_cast<const uint4 *>(x + (present ? i0 : 0));
+      uint32_t q[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        v[c][2 * k] = present ? Half<BF16>::up((uint16_t)(q[k] & 0xffff)) : 0.f;
+        v[c][2 * k + 1] = present ? Half<BF16>::up((uint16_t)(q[k] >> 16)) : 0.f;
+      }
+    } else if (vec && i0 + 8 <= N) {
       uint4 raw = *reinterpret_cast<const uint4 *>(x + i0);
       uint32_t q[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -247,7 +262,7 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(LayerNormParams p) {
 #pragma unroll
   for (int c = 0; c < CPT; c++) {
     int i0 = (threadIdx.x + c * 256) * 8;
-    if (vec && i0 + 8 <= N) {
+    if (FAST ? i0 < N : (vec && i0 + 8 <= N)) {
       uint4 wr = *reinterpret_cast<const uint4 *>(w + i0);
       uint4 br = *reinterpret_cast<const uint4 *>(b + i0);
       uint32_t wq[4] = {wr.x, wr.y, wr.z, wr.w}, bq[4] = {br.x, br.y, br.z, br.w}, o[4];
@@ -302,11 +317,21 @@ __global__ __launch_bounds__(256) void layernorm_fwd_long_kernel(LayerNormParams
 template <bool BF16>
 hipError_t launch_layernorm_t(const LayerNormParams &p, dim3 grid, hipStream_t s, const char **name) {
   int64_t chunks = (p.N + 7) / 8;
-  if (chunks <= 256) { hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, 1>), grid, dim3(256), 0, s, p); *name = "layernorm_fwd_kernel<1>"; }
-  else if (chunks <= 512) { hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, 2>), grid, dim3(256), 0, s, p); *name = "layernorm_fwd_kernel<2>"; }
-  else if (chunks <= 1024) { hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, 4>), grid, dim3(256), 0, s, p); *name = "layernorm_fwd_kernel<4>"; }
-  else if (chunks <= 2048) { hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, 8>), grid, dim3(256), 0, s, p); *name = "layernorm_fwd_kernel<8>"; }
+  auto aligned = [](const Affine &a) { return (a.c0 | a.c[0] | a.c[1] | a.c[2]) % 8 == 0; };
+  const bool fast = p.N % 8 == 0 && aligned(p.x_off) && aligned(p.y_off) && aligned(p.w_off) && aligned(p.b_off) &&
+                    (((uintptr_t)p.x | (uintptr_t)p.y | (uintptr_t)p.w | (uintptr_t)p.b) & 15) == 0;
+#define TTS_LN(CPT)                                                                                          \
+  do {                                                                                                       \
+    if (fast) hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, CPT, true>), grid, dim3(256), 0, s, p);        \
+    else hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, CPT, false>), grid, dim3(256), 0, s, p);            \
+    *name = "layernorm_fwd_kernel<" #CPT ">";                                                                \
+  } while (0)
+  if (chunks <= 256) TTS_LN(1);
+  else if (chunks <= 512) TTS_LN(2);
+  else if (chunks <= 1024) TTS_LN(4);
+  else if (chunks <= 2048) TTS_LN(8);
   else { hipLaunchKernelGGL((layernorm_fwd_long_kernel<BF16>), grid, dim3(256), 0, s, p); *name = "layernorm_fwd_long_kernel"; }
+#undef TTS_LN
   return hipGetLastError();
 }
 
