@@ -201,7 +201,7 @@ __device__ __forceinline__ float block_sum_256(float v, float *red) {
 // either whole or absent and all loads are unconditional (an absent chunk re-reads chunk 0 and is
 // zeroed), which lets the compiler keep the CPT loads of a thread in flight together.
 template <bool BF16, int CPT, bool FAST>
-__global__ __launch_bounds__(256) void layernorm_fwd_kernel(LayerNormParams p) {
+__global__ __launch_bounds__(256, CPT <= 4 ? 8 : 4) void layernorm_fwd_kernel(LayerNormParams p) {
   __shared__ float red[4];
   const int px = blockIdx.x, py = blockIdx.y, pz = blockIdx.z;
   const uint16_t *__restrict__ x = (const uint16_t *)p.x + affine(p.x_off, px, py, pz);
