@@ -104,7 +104,7 @@ def test_load_binary_tuple(native):
     structured = native.ttir_to_structured(open(os.path.join(ROOT, "tests/golden/vec_add.ttir")).read())
     plan_bytes, _ = native.structured_to_plan(structured)
     mod, fn, n_regs, n_spills, n_max = tsa.HIPUtils.load_binary("vec_add", plan_bytes, 0, 0)
-    assert mod is None and fn.family == "map1d" and n_max == sys.maxsize and fn.arg_kinds == [0, 0, 0, 1]
+    assert mod is fn and fn.family == "map1d" and n_max == sys.maxsize and fn.arg_kinds == [0, 0, 0, 1]
 
 
 def test_missing_extension_fails_loudly(monkeypatch):

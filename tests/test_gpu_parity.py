@@ -292,3 +292,12 @@ def test_errors_surface_as_python_exceptions(K):
     with pytest.raises(NotImplementedError, match="one program per output tile"):
         a = torch.zeros(256, 256, dtype=torch.bfloat16, device=DEV)
         K.matmul_tiles[(3,)](a, a, a, 256, 256, 256, 256, 1, 256, 1, 256, 1, BM=128, BN=128, BK=64, GROUP_M=8)
+
+
+def test_plan_handle_is_loaded_once(K):
+    # the launcher must keep the native plan (and its binding cache) across launches
+    x = torch.zeros(2048, device=DEV)
+    k1 = K.vec_add[(2,)](x, x, x, 2048, BLOCK=1024)
+    h1 = k1.function
+    k2 = K.vec_add[(2,)](x, x, x, 2048, BLOCK=1024)
+    assert k2 is k1 and k2.function is h1

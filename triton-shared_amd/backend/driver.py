@@ -117,7 +117,10 @@ class HIPUtils(object):
     @staticmethod
     def load_binary(name, kernel_obj, shared, device):
         plan = _native.PlanHandle(kernel_obj)
-        return (None, plan, None, None, sys.maxsize)  # module, function, n_regs, n_spills, n_max_threads
+        # (module, function, n_regs, n_spills, n_max_threads).  The module slot must not be None:
+        # Triton treats a None module as "handles not initialised yet" and would reload the plan, and
+        # with it drop the plan's binding cache, on every launch.
+        return (plan, plan, None, None, sys.maxsize)
 
 
 class HIPDriver(DriverBase):
