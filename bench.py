@@ -184,14 +184,25 @@ def time_workload(torch, spy, wl, steps, warmup):
     return dict(us=us, hot_us=hot_us, wall_us=wall_us, kernel=plan.last_kernel, sets=sets, frontend_us=frontend_us)
 
 
-def roofline(wl, us):
+def measured_traffic(name):
+    """HBM bytes per launch from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE, scaled by
+    a copy-kernel calibration; see profiles/hbm_traffic.json), or None if no figure is on file."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            return json.load(f).get(name, {}).get("hbm_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
+def roofline(wl, us, name=None):
+    traffic = measured_traffic(name) if name else None
     if wl["bound"] == "hbm":
         achieved = wl["work"] / us / 1e3  # GB/s
         return dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None)
+                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=traffic)
     achieved = wl["work"] / us / 1e6  # TFLOP/s
     return dict(bound="mfma", achieved=round(achieved, 1), peak=BF16_PEAK_TFLOPS, unit="TFLOP/s",
-                frac=round(achieved / BF16_PEAK_TFLOPS, 4), traffic=None)
+                frac=round(achieved / BF16_PEAK_TFLOPS, 4), traffic=traffic)
 
 
 def cpu_baseline(torch, name, wl):
@@ -275,7 +286,7 @@ def main():
         t = time_workload(torch, spy, wl, steps, args.warmup)
         entry = dict(workload=wl["desc"], us=round(t["us"], 3), kernel=t["kernel"], steps=steps,
                      rotating_buffer_sets=t["sets"], frontend_us_per_launch=round(t["frontend_us"], 1),
-                     roofline=roofline(wl, t["us"]), dtype=wl["dtype"],
+                     roofline=roofline(wl, t["us"], name), dtype=wl["dtype"], algorithmic_work=wl["work"],
                      same_buffers=dict(us=round(t["hot_us"], 3), frac=roofline(wl, t["hot_us"])["frac"]))
         if not args.no_cpu and (name == args.workload or not name.endswith(("2p28", "1m"))):
             entry["cpu_baseline"] = cpu_baseline(torch, name, wl)
