@@ -24,10 +24,24 @@ __device__ __forceinline__ int64_t affine(const Affine &a, int px, int py, int p
   return a.c0 + a.c[0] * px + a.c[1] * py + a.c[2] * pz;
 }
 
+// Wavefront reductions with DPP cross-lane operands (no LDS round trips): quad swaps, half-row and
+// row mirrors leave every lane of a 16-lane row with the row's result; row_bcast15 / row_bcast31 fold
+// the four rows into lane 63, which is then broadcast.  Lanes a step does not write take the
+// reduction's identity.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float v, float identity) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(identity), __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float lane63(float v) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63)); }
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-  return v;
+  v += dpp_move<0xB1, 0xf>(v, 0.f);   // quad_perm [1,0,3,2]
+  v += dpp_move<0x4E, 0xf>(v, 0.f);   // quad_perm [2,3,0,1]
+  v += dpp_move<0x141, 0xf>(v, 0.f);  // row_half_mirror
+  v += dpp_move<0x140, 0xf>(v, 0.f);  // row_mirror
+  v += dpp_move<0x142, 0xa>(v, 0.f);  // row_bcast15 into rows 1 and 3
+  v += dpp_move<0x143, 0xc>(v, 0.f);  // row_bcast31 into rows 2 and 3
+  return lane63(v);
 }
 template <bool NAN_PROP>
 __device__ __forceinline__ float fmax_sel(float a, float b) {
@@ -36,9 +50,13 @@ __device__ __forceinline__ float fmax_sel(float a, float b) {
 }
 template <bool NAN_PROP>
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmax_sel<NAN_PROP>(v, __shfl_xor(v, o, WAVE));
-  return v;
+  v = fmax_sel<NAN_PROP>(v, dpp_move<0xB1, 0xf>(v, -INFINITY));
+  v = fmax_sel<NAN_PROP>(v, dpp_move<0x4E, 0xf>(v, -INFINITY));
+  v = fmax_sel<NAN_PROP>(v, dpp_move<0x141, 0xf>(v, -INFINITY));
+  v = fmax_sel<NAN_PROP>(v, dpp_move<0x140, 0xf>(v, -INFINITY));
+  v = fmax_sel<NAN_PROP>(v, dpp_move<0x142, 0xa>(v, -INFINITY));
+  v = fmax_sel<NAN_PROP>(v, dpp_move<0x143, 0xc>(v, -INFINITY));
+  return lane63(v);
 }
 
 // ------------------------------------------------------------------ map1d
