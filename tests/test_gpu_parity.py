@@ -268,7 +268,8 @@ def test_w8a16_exact_selection(K):
     assert torch.equal(cd.cpu(), want)
 
 
-@pytest.mark.parametrize("M,N,Kd", [(13, 1000, 1000), (16, 256, 512), (1, 130, 70), (16, 4096, 4096), (5, 128, 8192)])
+@pytest.mark.parametrize("M,N,Kd", [(13, 1000, 1000), (16, 256, 512), (1, 130, 70), (16, 4096, 4096), (5, 128, 8192),
+                                    (3, 512, 2048), (16, 768, 32)])
 def test_w8a16_ragged_shapes(K, oracle_cpu, M, N, Kd):
     torch.manual_seed(N)
     a = torch.randn(M, Kd).half()
@@ -279,6 +280,24 @@ def test_w8a16_ragged_shapes(K, oracle_cpu, M, N, Kd):
     assert relfro(cd.cpu(), ref) <= 1e-2
     if N * Kd <= 1000 * 1000:
         assert relfro(cd.cpu(), oracle_cpu.w8a16_matmul(a, w, s)) <= 1e-2
+
+
+def test_w8a16_split_k_repeated_launches(K):
+    # the K slices meet through a workspace whose arrival counters must be back at zero after every launch
+    M, N, Kd = 16, 1024, 4096
+    prev = None
+    for seed in range(4):
+        torch.manual_seed(seed)
+        a = torch.randn(M, Kd).half()
+        w = torch.randint(-127, 128, (Kd, N), dtype=torch.int8)
+        s = (0.001 + 0.009 * torch.rand(N)).half()
+        cd = _run_w8(K, a, w, s)
+        ref = a.double() @ (w.half() * s[None, :]).double()
+        assert relfro(cd.cpu(), ref) <= 1e-2
+        again = _run_w8(K, a, w, s)
+        assert torch.equal(cd, again)                     # slices are added in slice order: reproducible
+        assert prev is None or not torch.equal(prev, cd)
+        prev = cd
 
 
 # ------------------------------------------------------------- error paths

@@ -70,10 +70,13 @@ struct GemmW8A16Params {
   void *c;
   int64_t M, N, K;
   int64_t lda, ldw, ldc;
-  float *workspace;        // split-K partial sums, or null when split == 1
+  float *workspace;        // split-K partial sums, gemm_w8a16_workspace_bytes() large, or null when split == 1
+  int *counters;           // gemm_w8a16_counters() arrival counters, zero between launches (clear them once)
   int split;
 };
-int gemm_w8a16_split(int64_t M, int64_t N, int64_t K);  // how many K slices the kernel wants
+int gemm_w8a16_split(const GemmW8A16Params &p);  // how many K slices the kernel wants (from shapes and pitches)
+size_t gemm_w8a16_workspace_bytes(const GemmW8A16Params &p);
+size_t gemm_w8a16_counters(const GemmW8A16Params &p);
 hipError_t launch_gemm_w8a16(const GemmW8A16Params &p, hipStream_t s, const char **kernel_name);
 
 }  // namespace tts

@@ -383,7 +383,8 @@ bool gemm_fast_path_ok(const GemmParams &p) {
 // exactly (bit pattern 0x6400 | (b ^ 0x80) is 1152 + b), multiplied by the
 // column's fp16 scale in fp16 as the Triton source does, and fed to eight
 // 16x16x32 MFMAs, one per column of the lane's eight.
-constexpr int W8_COLS = 128;
+constexpr int W8_COLS = 128;       // slab width of the 8-byte-load kernel
+constexpr int W8_COLS_WIDE = 256;  // and of the 16-byte-load kernel
 
 __device__ __forceinline__ uint32_t pk_sub_1152_mul(uint32_t biased, uint32_t scale2) {
   f16x2 v = __builtin_bit_cast(f16x2, biased);
@@ -397,9 +398,14 @@ __device__ __forceinline__ uint32_t pk_sub_1152_mul(uint32_t biased, uint32_t sc
 // FAST: K is a multiple of 32, N of 128, rows are 8/16-byte aligned: every load is unconditional,
 // so that the compiler keeps all loads of a step (and of DEPTH steps) in flight.  Rows of A beyond
 // M are read from row M-1: they only reach rows of the MFMA result that are never stored.
-template <int NW, int DEPTH, bool FAST>
+// CW: columns per lane (8: 8-byte weight loads, 128-column slabs; 16: 16-byte loads, 256-column
+// slabs, FAST only).
+template <int NW, int DEPTH, bool FAST, int CW>
 __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, int steps_per_slice) {
-  constexpr int RW = NW > 4 ? 4 : NW;  // wavefronts combined per round
+  static_assert(CW == 8 || (CW == 16 && FAST), "wide slabs exist on the unconditional path only");
+  constexpr int W8_COLS = 16 * CW;
+  constexpr int RW = NW > (CW == 8 ? 4 : 2) ? (CW == 8 ? 4 : 2) : NW;  // wavefronts combined per round
+  using wvec = typename std::conditional<CW == 8, uint2, uint4>::type;
   __shared__ float red[RW][16][W8_COLS + 4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int j = lane & 15, g = lane >> 4;
@@ -411,31 +417,31 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, 
   const int K = (int)p.K;
   const bool a_vec = (p.lda % 8 == 0) && (((uintptr_t)A & 15) == 0);
   const bool w_vec = (p.ldw % 8 == 0) && (((uintptr_t)W & 7) == 0);
-  const int64_t ncol = n0 + 8 * j;                       // first of this lane's 8 columns
-  const int ncols = (int)max((int64_t)0, min((int64_t)8, p.N - ncol));
+  const int64_t ncol = n0 + CW * j;                      // first of this lane's CW columns
+  const int ncols = (int)max((int64_t)0, min((int64_t)CW, p.N - ncol));
 
-  uint32_t scale2[8];
+  uint32_t scale2[CW];
 #pragma unroll
-  for (int c = 0; c < 8; c++) {
+  for (int c = 0; c < CW; c++) {
     uint32_t s = c < ncols ? S[ncol + c] : 0;
     scale2[c] = s | (s << 16);
   }
-  f32x4 acc[8];
+  f32x4 acc[CW];
 #pragma unroll
-  for (int c = 0; c < 8; c++) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int c = 0; c < CW; c++) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
   const int step_begin = slice * steps_per_slice;
   const int step_end = min(step_begin + steps_per_slice, (K + 31) / 32);
 
   const int8_t *w_lane = W + (int64_t)(8 * g) * p.ldw + ncol;
   const uint16_t *a_lane = A + (int64_t)min(j, (int)p.M - 1) * p.lda + 8 * g;
-  auto load_w = [&](int step, uint2 (&q)[8]) {
-    if (FAST) {
+  auto load_w = [&](int step, wvec (&q)[8]) {
+    if constexpr (FAST) {
       const int8_t *src = w_lane + (int64_t)step * 32 * p.ldw;
 #pragma unroll
-      for (int t = 0; t < 8; t++) q[t] = *reinterpret_cast<const uint2 *>(src + (int64_t)t * p.ldw);
+      for (int t = 0; t < 8; t++) q[t] = *reinterpret_cast<const wvec *>(src + (int64_t)t * p.ldw);
       return;
-    }
+    } else {
 #pragma unroll
     for (int t = 0; t < 8; t++) {
       int k = step * 32 + 8 * g + t;
@@ -452,6 +458,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, 
         q[t] = make_uint2(lo, hi);
       }
     }
+    }
   };
   auto load_a = [&](int step) {
     if (FAST) return *reinterpret_cast<const uint4 *>(a_lane + step * 32);
@@ -459,14 +466,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, 
     return j < p.M ? load8(A + (int64_t)j * p.lda + k, K - k, a_vec) : make_uint4(0, 0, 0, 0);
   };
 
-  auto consume = [&](const uint2 (&q)[8], const uint4 &af) {
+  auto word = [](const wvec &v, int i) -> uint32_t {
+    if constexpr (CW == 8) return i == 0 ? v.x : v.y;
+    else return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w;
+  };
+  auto consume = [&](const wvec (&q)[8], const uint4 &af) {
 #pragma unroll
-    for (int c = 0; c < 8; c++) {
+    for (int c = 0; c < CW; c++) {
       uint32_t frag[4];
 #pragma unroll
       for (int tp = 0; tp < 4; tp++) {
-        uint32_t w0 = c < 4 ? q[2 * tp].x : q[2 * tp].y;
-        uint32_t w1 = c < 4 ? q[2 * tp + 1].x : q[2 * tp + 1].y;
+        uint32_t w0 = word(q[2 * tp], c / 4);
+        uint32_t w1 = word(q[2 * tp + 1], c / 4);
         // bytes [w0.b, 0, w1.b, 0], then flip the sign bit and set the exponent: 0x6400 | (b ^ 0x80)
         uint32_t sel = 0x0c000c00u | (uint32_t)(c & 3) | ((uint32_t)(4 + (c & 3)) << 16);
         uint32_t pair = __builtin_amdgcn_perm(w1, w0, sel) ^ 0x64806480u;
@@ -478,7 +489,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, 
   };
   // DEPTH steps are in flight in DEPTH register sets (the loop is unrolled over them, so no
   // copies), giving a step's loads the time of DEPTH steps' arithmetic to arrive
-  uint2 q[DEPTH][8];
+  wvec q[DEPTH][8];
   uint4 a[DEPTH];
   int step = step_begin + wave;
 #pragma unroll
@@ -495,7 +506,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, 
   }
 
   // combine the wavefronts' partial tiles through LDS, RW wavefronts at a time;
-  // lane holds rows 4g+v (v = 0..3) of column n0 + 8j + c
+  // lane holds rows 4g+v (v = 0..3) of column n0 + CW*j + c
   constexpr int ROUNDS = (NW + RW - 1) / RW;
   constexpr int PER_THREAD = (16 * W8_COLS + NW * 64 - 1) / (NW * 64);
   float total[PER_THREAD];
@@ -505,9 +516,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, 
     if (r) __syncthreads();
     if (wave / RW == r) {
 #pragma unroll
-      for (int c = 0; c < 8; c++)
+      for (int c = 0; c < CW; c++)
 #pragma unroll
-        for (int v = 0; v < 4; v++) red[wave % RW][4 * g + v][8 * j + c] = acc[c][v];
+        for (int v = 0; v < 4; v++) red[wave % RW][4 * g + v][CW * j + c] = acc[c][v];
     }
     __syncthreads();
     const int live = min(RW, NW - RW * r);
@@ -530,6 +541,166 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, 
     if (m >= p.M || n >= p.N) continue;
     if (p.split > 1) p.workspace[((int64_t)slice * 16 + m) * p.N + n] = total[e];
     else C[(int64_t)m * p.ldc + n] = f32_to_f16(total[e]);
+  }
+}
+
+// The decode shape's kernel: 256-column slabs, 16-byte weight loads (a lane holds 16 columns of
+// 8 rows per step), one workgroup per (slab, K slice).  Requires K % 32 == 0, N % 256 == 0,
+// 16-byte-aligned rows of W and A.
+//
+// Tail: the NW wavefronts' partial tiles are summed through LDS in one round (float4 per lane,
+// conflict-free).  With split > 1 every workgroup writes its slice's tile to its workspace slot and
+// bumps the slab's arrival counter; the workgroup that arrives last adds the slices in slice
+// order (so the sum does not depend on the order of arrival), writes C, and resets the counter
+// for the next launch.  The counters are zero between launches (whoever allocates them clears
+// them once).  Launches that share a workspace must not overlap.
+template <int NW, int DEPTH>
+__global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Params p, int steps_per_slice) {
+  extern __shared__ float4 w8_lds[];  // [NW][16][64]
+  __shared__ int is_last;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int j = lane & 15, g = lane >> 4;
+  const int slab = blockIdx.x, slice = blockIdx.y;
+  const int64_t n0 = (int64_t)slab * W8_COLS_WIDE;
+  const uint16_t *__restrict__ S = (const uint16_t *)p.scale;
+
+  uint32_t scale2[16];
+  {
+    const uint4 *sp = reinterpret_cast<const uint4 *>(S + n0 + 16 * j);
+    const bool s_vec = (((uintptr_t)S) & 15) == 0;
+    uint16_t sv[16];
+    if (s_vec) {
+      uint4 lo = sp[0], hi = sp[1];
+      uint32_t wds[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+      for (int c = 0; c < 16; c++) sv[c] = (uint16_t)(wds[c / 2] >> (16 * (c & 1)));
+    } else {
+#pragma unroll
+      for (int c = 0; c < 16; c++) sv[c] = S[n0 + 16 * j + c];
+    }
+#pragma unroll
+    for (int c = 0; c < 16; c++) scale2[c] = (uint32_t)sv[c] | ((uint32_t)sv[c] << 16);
+  }
+  f32x4 acc[16];
+#pragma unroll
+  for (int c = 0; c < 16; c++) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const int step_begin = slice * steps_per_slice;
+  const int step_end = min(step_begin + steps_per_slice, (int)(p.K / 32));
+  const int8_t *w_lane = p.w + (int64_t)(8 * g) * p.ldw + n0 + 16 * j;
+  const uint16_t *a_lane = (const uint16_t *)p.a + (int64_t)min(j, (int)p.M - 1) * p.lda + 8 * g;
+
+  auto load_w = [&](int step, uint4 (&q)[8]) {
+    const int8_t *src = w_lane + (int64_t)step * 32 * p.ldw;
+#pragma unroll
+    for (int t = 0; t < 8; t++) q[t] = *reinterpret_cast<const uint4 *>(src + (int64_t)t * p.ldw);
+  };
+  auto load_a = [&](int step) { return *reinterpret_cast<const uint4 *>(a_lane + step * 32); };
+  auto word = [](const uint4 &v, int i) -> uint32_t { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; };
+  auto consume = [&](const uint4 (&q)[8], const uint4 &af) {
+#pragma unroll
+    for (int c = 0; c < 16; c++) {
+      uint32_t frag[4];
+#pragma unroll
+      for (int tp = 0; tp < 4; tp++) {
+        // bytes [w0.b, 0, w1.b, 0], then flip the sign bit and set the exponent: 0x6400 | (b ^ 0x80)
+        uint32_t sel = 0x0c000c00u | (uint32_t)(c & 3) | ((uint32_t)(4 + (c & 3)) << 16);
+        uint32_t pair = __builtin_amdgcn_perm(word(q[2 * tp + 1], c / 4), word(q[2 * tp], c / 4), sel) ^ 0x64806480u;
+        frag[tp] = pk_sub_1152_mul(pair, scale2[c]);
+      }
+      uint4 bfrag = make_uint4(frag[0], frag[1], frag[2], frag[3]);
+      acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af), __builtin_bit_cast(f16x8, bfrag), acc[c], 0, 0, 0);
+    }
+  };
+  uint4 q[DEPTH][8];
+  uint4 a[DEPTH];
+  int step = step_begin + wave;
+#pragma unroll
+  for (int d = 0; d < DEPTH; d++)
+    if (step + d * NW < step_end) { load_w(step + d * NW, q[d]); a[d] = load_a(step + d * NW); }
+  for (; step < step_end; step += DEPTH * NW) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) {
+      if (step + d * NW < step_end) {
+        consume(q[d], a[d]);
+        if (step + (d + DEPTH) * NW < step_end) { load_w(step + (d + DEPTH) * NW, q[d]); a[d] = load_a(step + (d + DEPTH) * NW); }
+      }
+    }
+  }
+
+  // sum the wavefronts' tiles: entry (c, lane) is rows 4g..4g+3 of column n0 + 16j + c
+#pragma unroll
+  for (int c = 0; c < 16; c++) w8_lds[(wave * 16 + c) * 64 + lane] = __builtin_bit_cast(float4, acc[c]);
+  __syncthreads();
+  constexpr int PER = 1024 / (NW * 64);
+  float4 tot[PER];
+#pragma unroll
+  for (int e = 0; e < PER; e++) {
+    const int idx = tid + e * NW * 64;
+    float4 t = w8_lds[idx];
+#pragma unroll
+    for (int w = 1; w < NW; w++) {
+      float4 u = w8_lds[w * 1024 + idx];
+      t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+    }
+    tot[e] = t;
+  }
+  if (p.split > 1) {
+    float4 *slots = reinterpret_cast<float4 *>(p.workspace) + (int64_t)slab * p.split * 1024;
+#pragma unroll
+    for (int e = 0; e < PER; e++) slots[slice * 1024 + tid + e * NW * 64] = tot[e];
+    __syncthreads();  // every wavefront's stores have reached L2
+    if (tid == 0) {
+      // one lane publishes the whole workgroup's tile (the release writes L2 back) and, when it
+      // finds itself last, makes the others' tiles readable (the acquire drops stale lines)
+      int *counter = p.counters + slab;
+      int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      is_last = before == p.split - 1;
+      if (before == p.split - 1) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!is_last) return;
+#pragma unroll
+    for (int e = 0; e < PER; e++) {
+      const int idx = tid + e * NW * 64;
+      float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int sl = 0; sl < p.split; sl++) {
+        float4 u = sl == slice ? tot[e] : slots[sl * 1024 + idx];
+        if (sl == 0) t = u;
+        else { t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w; }
+      }
+      tot[e] = t;
+    }
+  }
+  // to row-major through LDS, then 16-byte stores of eight fp16 values
+  __syncthreads();
+  constexpr int PITCH = W8_COLS_WIDE + 4;
+  float *tile = reinterpret_cast<float *>(w8_lds);
+#pragma unroll
+  for (int e = 0; e < PER; e++) {
+    const int idx = tid + e * NW * 64;
+    const int c = idx >> 6, jj = idx & 15, gg = (idx >> 4) & 3;
+    float *dst = tile + (4 * gg) * PITCH + 16 * jj + c;
+    dst[0] = tot[e].x; dst[PITCH] = tot[e].y; dst[2 * PITCH] = tot[e].z; dst[3 * PITCH] = tot[e].w;
+  }
+  __syncthreads();
+  uint16_t *__restrict__ C = (uint16_t *)p.c;
+  const bool c_vec = (p.ldc % 8 == 0) && (((uintptr_t)C & 15) == 0);
+  for (int item = tid; item < 16 * (W8_COLS_WIDE / 8); item += NW * 64) {
+    const int m = item / (W8_COLS_WIDE / 8), n8 = (item % (W8_COLS_WIDE / 8)) * 8;
+    if (m >= p.M) continue;
+    const float *src = tile + m * PITCH + n8;
+    uint16_t h[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) h[i] = f32_to_f16(src[i]);
+    uint16_t *dst = C + (int64_t)m * p.ldc + n0 + n8;
+    if (c_vec) {
+      *reinterpret_cast<uint4 *>(dst) = make_uint4(h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16,
+                                                   h[4] | (uint32_t)h[5] << 16, h[6] | (uint32_t)h[7] << 16);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; i++) dst[i] = h[i];
+    }
   }
 }
 
@@ -564,27 +735,78 @@ hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
   return p.is_bf16 ? launch_gemm_cfg<true, 2, 2, 64>(p, s) : launch_gemm_cfg<false, 2, 2, 64>(p, s);
 }
 
-int gemm_w8a16_split(int64_t M, int64_t N, int64_t K) {
-  (void)M;
-  int64_t slabs = (N + W8_COLS - 1) / W8_COLS;
-  int64_t steps = (K + 31) / 32;
-  if (slabs >= 192) return 1;
-  int64_t want = (256 + slabs - 1) / slabs;                 // about one workgroup per CU
-  int64_t most = std::max<int64_t>(1, steps / W8_WAVES);    // keep every wavefront busy
-  return (int)std::max<int64_t>(1, std::min<int64_t>(std::min(want, most), 64));
+namespace {
+struct W8Config { int cw, nw, depth, split; };
+
+// The shape decides the kernel: 256-column slabs with 16-byte weight loads when N and the
+// weight pitch allow, split over K so that about one workgroup lands on each CU.
+// TTS_W8=cw,nw,depth,split overrides the choice (tuning aid).
+W8Config w8_config(const GemmW8A16Params &p) {
+  const int64_t steps = (p.K + 31) / 32;
+  W8Config c{8, 16, 2, 1};
+  const bool fast = p.K % 32 == 0 && p.N % W8_COLS == 0 && p.lda % 8 == 0 && p.ldw % 8 == 0;
+  if (fast && p.N % W8_COLS_WIDE == 0 && p.ldw % 16 == 0) c = W8Config{16, 8, 2, 1};
+  static const char *env = getenv("TTS_W8");
+  int want_split = 0;
+  if (env) {
+    int cw = 0, nw = 0, depth = 0;
+    if (sscanf(env, "%d,%d,%d,%d", &cw, &nw, &depth, &want_split) >= 3 && (cw == 8 || (cw == 16 && c.cw == 16))) {
+      c.cw = cw; c.nw = nw; c.depth = depth;
+    }
+  }
+  const int64_t slabs = (p.N + 16 * c.cw - 1) / (16 * c.cw);
+  if (want_split > 0) c.split = want_split;
+  else if (slabs < 192) {
+    int64_t want = (256 + slabs - 1) / slabs;                 // about one workgroup per CU
+    int64_t most = std::max<int64_t>(1, steps / c.nw);        // keep every wavefront busy
+    c.split = (int)std::max<int64_t>(1, std::min<int64_t>(std::min(want, most), 64));
+  }
+  return c;
 }
 
+template <int NW, int DEPTH, bool FAST>
+void w8_launch(const GemmW8A16Params &p, int steps_per_slice, hipStream_t s) {
+  dim3 grid((unsigned)((p.N + W8_COLS - 1) / W8_COLS), p.split);
+  hipLaunchKernelGGL((gemm_w8a16_kernel<NW, DEPTH, FAST, 8>), grid, dim3(NW * 64), 0, s, p, steps_per_slice);
+}
+
+template <int NW, int DEPTH>
+hipError_t w8_launch_wide(const GemmW8A16Params &p, int steps_per_slice, hipStream_t s) {
+  constexpr size_t lds = (size_t)NW * 16 * 64 * sizeof(float4);
+  static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_w8a16_wide_kernel<NW, DEPTH>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (attr != hipSuccess) return attr;
+  dim3 grid((unsigned)(p.N / W8_COLS_WIDE), p.split);
+  hipLaunchKernelGGL((gemm_w8a16_wide_kernel<NW, DEPTH>), grid, dim3(NW * 64), lds, s, p, steps_per_slice);
+  return hipGetLastError();
+}
+}  // namespace
+
+int gemm_w8a16_split(const GemmW8A16Params &p) { return w8_config(p).split; }
+
+size_t gemm_w8a16_workspace_bytes(const GemmW8A16Params &p) {
+  if (p.split <= 1) return 0;
+  return (size_t)p.split * 16 * (size_t)((p.N + 255) / 256 * 256) * sizeof(float);  // per-slice partial tiles, 16 rows of fp32
+}
+
+size_t gemm_w8a16_counters(const GemmW8A16Params &p) { return p.split <= 1 ? 0 : (size_t)((p.N + 255) / 256); }
+
 hipError_t launch_gemm_w8a16(const GemmW8A16Params &p, hipStream_t s, const char **name) {
-  *name = "gemm_w8a16_kernel";
-  int slabs = (int)((p.N + W8_COLS - 1) / W8_COLS);
-  int steps = (int)((p.K + 31) / 32);
-  int steps_per_slice = (steps + p.split - 1) / p.split;
+  W8Config c = w8_config(p);
+  const int steps = (int)((p.K + 31) / 32);
+  const int sps = (steps + p.split - 1) / p.split;
   const bool fast = p.K % 32 == 0 && p.N % W8_COLS == 0 && p.lda % 8 == 0 && p.ldw % 8 == 0 &&
                     ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.w & 7) == 0;
-  dim3 grid(slabs, p.split);
-  // 16 wavefronts x 2 steps in flight; 8 x 2..6 and 4 x 8 measured the same (HBM-bound) at the decode shape
-  if (fast) hipLaunchKernelGGL((gemm_w8a16_kernel<W8_WAVES, 2, true>), grid, dim3(W8_WAVES * 64), 0, s, p, steps_per_slice);
-  else hipLaunchKernelGGL((gemm_w8a16_kernel<W8_WAVES, 2, false>), grid, dim3(W8_WAVES * 64), 0, s, p, steps_per_slice);
+  const bool wide = fast && c.cw == 16 && ((uintptr_t)p.w & 15) == 0;
+  if (wide) {
+    *name = "gemm_w8a16_wide_kernel";
+    if (c.nw == 8 && c.depth == 1) return w8_launch_wide<8, 1>(p, sps, s);
+    if (c.nw == 4) return w8_launch_wide<4, 2>(p, sps, s);
+    return w8_launch_wide<8, 2>(p, sps, s);
+  }
+  *name = "gemm_w8a16_kernel";
+  if (!fast) w8_launch<W8_WAVES, 2, false>(p, sps, s);
+  else w8_launch<W8_WAVES, 2, true>(p, sps, s);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || p.split == 1) return e;
   int64_t outs = p.M * p.N;

@@ -64,8 +64,11 @@ struct tts_plan {
   const char *last_kernel = "";
   float *workspace = nullptr;  // split-K partial sums (device), owned by the plan
   size_t workspace_bytes = 0;
+  int *counters = nullptr;     // split-K arrival counters (device), zero between launches
+  size_t counters_count = 0;
   ~tts_plan() {
     if (workspace) (void)hipFree(workspace);
+    if (counters) (void)hipFree(counters);
   }
 };
 
@@ -251,7 +254,7 @@ void bind_w8a16(const Resolver &r, Bound &b) {
   if (d.M > 16) throw Unsupported("gemm_w8a16: only the decode shape M <= 16 is implemented");
   GemmW8A16Params &p = b.w8;
   p.M = d.M; p.N = d.N; p.K = d.K; p.lda = d.lda; p.ldw = d.ldb; p.ldc = d.ldc;
-  p.split = gemm_w8a16_split(p.M, p.N, p.K);
+  p.split = gemm_w8a16_split(p);
   std::ostringstream os;
   os << "kernel=gemm_w8a16\nM=" << p.M << "\nN=" << p.N << "\nK=" << p.K << "\nlda=" << p.lda << "\nldw=" << p.ldw
      << "\nldc=" << p.ldc << "\nsplit=" << p.split << "\n";
@@ -433,7 +436,7 @@ tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, cons
         p.scale = ptr_arg<const void>(args, pl, "s_arg");
         p.c = ptr_arg<void>(args, pl, "c_arg");
         if (p.split > 1) {
-          size_t need = (size_t)p.split * 16 * (size_t)p.N * sizeof(float);
+          size_t need = gemm_w8a16_workspace_bytes(p);
           std::lock_guard<std::mutex> lock(plan->mu);
           if (plan->workspace_bytes < need) {
             if (plan->workspace) (void)hipFree(plan->workspace);
@@ -443,7 +446,18 @@ tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, cons
             if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(split-K workspace): ") + hipGetErrorString(e));
             plan->workspace_bytes = need;
           }
+          size_t ncount = gemm_w8a16_counters(p);
+          if (plan->counters_count < ncount) {
+            if (plan->counters) (void)hipFree(plan->counters);
+            plan->counters = nullptr;
+            plan->counters_count = 0;
+            hipError_t e = hipMalloc((void **)&plan->counters, ncount * sizeof(int));
+            if (e == hipSuccess) e = hipMemset(plan->counters, 0, ncount * sizeof(int));
+            if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(split-K counters): ") + hipGetErrorString(e));
+            plan->counters_count = ncount;
+          }
           p.workspace = plan->workspace;
+          p.counters = plan->counters;
         }
         err = launch_gemm_w8a16(p, s, &kname);
         break;
