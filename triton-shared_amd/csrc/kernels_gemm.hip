@@ -544,16 +544,35 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_kernel(GemmW8A16Params p, 
   }
 }
 
+// Partial tiles cross between workgroups (and so between the XCDs' L2 caches) through agent-scope
+// relaxed atomic accesses: the stores are written through to memory and the loads bypass stale
+// lines, without the whole-cache write-back and invalidate that a release/acquire pair costs
+// (measured: 8 us per launch at the decode shape against 3 us this way).
+__device__ __forceinline__ void store_through(float4 *dst, float4 v) {
+  unsigned long long *d = reinterpret_cast<unsigned long long *>(dst);
+  ulonglong2 u = __builtin_bit_cast(ulonglong2, v);
+  __hip_atomic_store(d, u.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(d + 1, u.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float4 load_through(float4 *src) {
+  unsigned long long *d = reinterpret_cast<unsigned long long *>(src);
+  ulonglong2 u;
+  u.x = __hip_atomic_load(d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  u.y = __hip_atomic_load(d + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return __builtin_bit_cast(float4, u);
+}
+
 // The decode shape's kernel: 256-column slabs, 16-byte weight loads (a lane holds 16 columns of
 // 8 rows per step), one workgroup per (slab, K slice).  Requires K % 32 == 0, N % 256 == 0,
 // 16-byte-aligned rows of W and A.
 //
 // Tail: the NW wavefronts' partial tiles are summed through LDS in one round (float4 per lane,
-// conflict-free).  With split > 1 every workgroup writes its slice's tile to its workspace slot and
-// bumps the slab's arrival counter; the workgroup that arrives last adds the slices in slice
-// order (so the sum does not depend on the order of arrival), writes C, and resets the counter
-// for the next launch.  The counters are zero between launches (whoever allocates them clears
-// them once).  Launches that share a workspace must not overlap.
+// conflict-free).  With split > 1 every workgroup writes its slice's tile through to its workspace
+// slot, waits for the stores' acknowledgement, and bumps the slab's arrival counter; the workgroup
+// that arrives last adds the slices in slice order (so the sum does not depend on the order of
+// arrival), writes C, and resets the counter for the next launch.  No workgroup waits for another.
+// The counters are zero between launches (whoever allocates them clears them once).  Launches
+// that share a workspace must not overlap.
 template <int NW, int DEPTH>
 __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Params p, int steps_per_slice) {
   extern __shared__ float4 w8_lds[];  // [NW][16][64]
@@ -648,13 +667,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
   if (p.split > 1) {
     float4 *slots = reinterpret_cast<float4 *>(p.workspace) + (int64_t)slab * p.split * 1024;
 #pragma unroll
-    for (int e = 0; e < PER; e++) slots[slice * 1024 + tid + e * NW * 64] = tot[e];
-    __syncthreads();  // every wavefront's stores have reached L2
+    for (int e = 0; e < PER; e++) store_through(slots + slice * 1024 + tid + e * NW * 64, tot[e]);
+    __builtin_amdgcn_s_waitcnt(0);  // the stores have been acknowledged: the tile is in memory
+    __syncthreads();                // ... every wavefront's part of it
     if (tid == 0) {
-      // one lane publishes the whole workgroup's tile (the release writes L2 back) and, when it
-      // finds itself last, makes the others' tiles readable (the acquire drops stale lines)
       int *counter = p.counters + slab;
-      int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       is_last = before == p.split - 1;
       if (before == p.split - 1) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -665,7 +683,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
       const int idx = tid + e * NW * 64;
       float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
       for (int sl = 0; sl < p.split; sl++) {
-        float4 u = sl == slice ? tot[e] : slots[sl * 1024 + idx];
+        float4 u = sl == slice ? tot[e] : load_through(slots + sl * 1024 + idx);
         if (sl == 0) t = u;
         else { t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w; }
       }
@@ -745,7 +763,7 @@ W8Config w8_config(const GemmW8A16Params &p) {
   const int64_t steps = (p.K + 31) / 32;
   W8Config c{8, 16, 2, 1};
   const bool fast = p.K % 32 == 0 && p.N % W8_COLS == 0 && p.lda % 8 == 0 && p.ldw % 8 == 0;
-  if (fast && p.N % W8_COLS_WIDE == 0 && p.ldw % 16 == 0) c = W8Config{16, 8, 2, 1};
+  if (fast && p.N % W8_COLS_WIDE == 0 && p.ldw % 16 == 0) c = W8Config{16, 8, 1, 1};
   static const char *env = getenv("TTS_W8");
   int want_split = 0;
   if (env) {
@@ -757,7 +775,8 @@ W8Config w8_config(const GemmW8A16Params &p) {
   const int64_t slabs = (p.N + 16 * c.cw - 1) / (16 * c.cw);
   if (want_split > 0) c.split = want_split;
   else if (slabs < 192) {
-    int64_t want = (256 + slabs - 1) / slabs;                 // about one workgroup per CU
+    // about one workgroup per CU; the wide kernel's LDS tile admits only one, so never more than 256 of those
+    int64_t want = c.cw == 16 ? std::max<int64_t>(1, 256 / slabs) : (256 + slabs - 1) / slabs;
     int64_t most = std::max<int64_t>(1, steps / c.nw);        // keep every wavefront busy
     c.split = (int)std::max<int64_t>(1, std::min<int64_t>(std::min(want, most), 64));
   }
@@ -800,9 +819,9 @@ hipError_t launch_gemm_w8a16(const GemmW8A16Params &p, hipStream_t s, const char
   const bool wide = fast && c.cw == 16 && ((uintptr_t)p.w & 15) == 0;
   if (wide) {
     *name = "gemm_w8a16_wide_kernel";
-    if (c.nw == 8 && c.depth == 1) return w8_launch_wide<8, 1>(p, sps, s);
-    if (c.nw == 4) return w8_launch_wide<4, 2>(p, sps, s);
-    return w8_launch_wide<8, 2>(p, sps, s);
+    // one step in flight per wavefront; two measured 1.2 us slower at the decode shape
+    if (c.depth == 2) return w8_launch_wide<8, 2>(p, sps, s);
+    return w8_launch_wide<8, 1>(p, sps, s);
   }
   *name = "gemm_w8a16_kernel";
   if (!fast) w8_launch<W8_WAVES, 2, false>(p, sps, s);
