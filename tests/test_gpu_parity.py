@@ -211,6 +211,32 @@ def test_gemm_ragged_shapes(K, oracle_cpu, M, N, Kd, dtype):
         assert relfro(cd.cpu(), oracle_cpu.matmul_tiles(a, b)) <= 1e-2
 
 
+@pytest.mark.parametrize("M,N,Kd,dtype,pad", [(256, 256, 32, torch.bfloat16, 0), (256, 512, 64, torch.bfloat16, 0),
+                                             (512, 256, 96, torch.bfloat16, 8), (768, 256, 160, torch.float16, 16),
+                                             (256, 256, 4096, torch.bfloat16, 0), (1024, 1280, 352, torch.float16, 0)])
+def test_gemm_whole_tile_kernel(K, M, N, Kd, dtype, pad):
+    # whole 256 x 256 x 32 tiles: the direct-to-LDS kernel, from one K tile (fewer than its pipeline stages) upwards
+    torch.manual_seed(M + Kd)
+    A, B = (torch.randn(M, Kd + pad) * 0.5).to(dtype).to(DEV), (torch.randn(Kd, N + pad) * 0.5).to(dtype).to(DEV)
+    Cfull = torch.full((M, N + pad), 5.0, dtype=dtype, device=DEV)
+    a, b, c = A[:, :Kd], B[:, :N], Cfull[:, :N]
+    k = K.matmul_tiles[(triton.cdiv(M, 128) * triton.cdiv(N, 128),)](a, b, c, M, N, Kd, a.stride(0), 1, b.stride(0), 1,
+                                                                   c.stride(0), 1, BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert k.function.last_kernel == "gemm_dma_kernel"
+    assert relfro(c.cpu(), a.cpu().double() @ b.cpu().double()) <= 1e-2
+    assert torch.equal(Cfull[:, N:].cpu(), torch.full((M, pad), 5.0, dtype=dtype))
+    # exact: B selects and negates columns of A
+    perm = torch.randperm(Kd)[:N] if N <= Kd else torch.randint(0, Kd, (N,))
+    sel = torch.zeros(Kd, N)
+    sel[perm, torch.arange(N)] = -1.0
+    B[:, :N] = sel.to(dtype).to(DEV)
+    K.matmul_tiles[(triton.cdiv(M, 128) * triton.cdiv(N, 128),)](a, b, c, M, N, Kd, a.stride(0), 1, b.stride(0), 1,
+                                                               c.stride(0), 1, BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert torch.equal(c.cpu(), -a.cpu()[:, perm])
+
+
 def test_gemm_with_padded_pitches_and_untouched_border(K):
     torch.manual_seed(3)
     M, N, Kd = 200, 300, 150

@@ -192,25 +192,50 @@ hipError_t launch_gemm_cfg(const GemmParams &p, hipStream_t s) {
 
 
 // ------------------------------------------- 16-bit GEMM, full-tile fast path
-// For problems made of whole 256 x 256 x BK tiles with 16-byte aligned rows.
-// Workgroup: 512 threads = 8 wavefronts (two per SIMD, so that one computes
-// while the other waits on LDS or the barrier), wave grid 2 (M) x 4 (N), each
-// wavefront 128 x 64 of C = 4 x 2 MFMA tiles.  Wavefronts 0-3 stage A (BK/8
-// 16-byte chunks per thread); wavefronts 4-7 stage B: each thread loads a
-// (BK/8) (k) x 8 (n) block as 16-byte rows, transposes it in registers and writes
-// eight K-contiguous chunks, so that global loads are whole 128-byte row
-// segments and LDS accesses are conflict-free.  DIST tiles are in flight in
-// registers, so global/L2 latency is covered by DIST K steps of MFMA work.
-// LDS: [2 buffers][256 A rows + 256 B columns][BK + 8] 16-bit elements.
-constexpr int F_BM = 256, F_BN = 256;
+// For problems made of whole 256 x 256 x 32 tiles with 16-byte aligned rows.
+//
+// Workgroup: 256 threads = 4 wavefronts (one per SIMD), wave grid 2 x 2, each wavefront
+// 128 x 128 of C = 4 x 4 MFMA tiles of 32 x 32 (256 accumulator registers).
+//
+// Global -> LDS without passing through registers: `global_load_lds_dwordx4` writes the 64
+// lanes' 16-byte chunks to 1 KB of consecutive LDS, so the LDS layout is fixed by which global
+// chunk each lane fetches.
+//   A stage [256 rows][64 bytes]: position q of row r holds chunk q ^ ((r / 4) & 3) of the row's
+//     four; 16-byte fragment reads of 16 consecutive rows then fall into 16 distinct slots.
+//   B stage [32 k rows][512 bytes], as in memory (N contiguous): position q of row k holds chunk
+//     q ^ ((k & 3) << 2).  The MFMA operand wants K contiguous per lane; `ds_read_b64_tr_b16` does
+//     that transposition on the way out: within 16 lanes, lane i receives element i % 4 of the
+//     8-byte rows addressed by lanes i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12.  Lane r of a group
+//     therefore addresses k row r / 4, columns 4 (r % 4) .. +3 of the group's 16 columns, and
+//     two reads (k 0-3, k 4-7) make one 8-element operand.
+// Both layouts were checked on the device: no LDS bank conflicts (SQ_LDS_BANK_CONFLICT = 0).
+//
+// Pipeline: STAGES LDS stages of one K tile each.  An iteration has two phases of 16 MFMAs (the
+// tile's two K halves).  Every MFMA is followed by one LDS read or one direct-to-LDS load, which
+// the matrix pipe hides: phase A reads the operands of phase B, phase B those of the next
+// tile's phase A; a quarter of the way through each phase one load of tile t+STAGES-1 goes out,
+// into the stage of tile t-1, which every wavefront finished reading before the previous barrier.
+// One barrier per tile, between the phases: it follows the wait that tells this wavefront its
+// own loads of tile t+1 have landed.  Loads past the last tile fetch the last tile again, so the
+// wait count is the same in every iteration.
+//
+// The direct-to-LDS load is issued from inline assembly: the compiler orders every later LDS
+// read behind such a load with a full vmcnt wait (it cannot tell the stages apart), which
+// would serialise the pipeline.  Its own counting of ordinary loads stays conservative.
+constexpr int F_BM = 256, F_BN = 256, F_BK = 32, F_STAGES = 4;
+constexpr int F_A_BYTES = F_BM * F_BK * 2, F_STAGE_BYTES = F_A_BYTES + F_BK * F_BN * 2;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+#define TTS_LDS(p) ((__attribute__((address_space(3))) void *)(p))
 
-template <bool BF16, int BK, int DIST, bool EARLY, int DBG>
-__global__ __launch_bounds__(512) void gemm_fast_kernel(GemmParams p, int tiles_m, int tiles_n) {
-  constexpr int PITCH = BK + 8, NL = BK / 8;  // NL: 16-byte loads per thread and tile
-  constexpr int KS = BK / 16;
-  extern __shared__ __align__(16) uint16_t smem[];
+// s_waitcnt immediate: vmcnt in bits 3:0 and 15:14, expcnt (not waited for) in 6:4, lgkmcnt in 11:8
+constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | (lgkm << 8); }
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void gemm_dma_kernel(GemmParams p, int tiles_m, int tiles_n) {
+  extern __shared__ __align__(16) char dma_smem[];
+  char *smem = dma_smem;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 2, wn = wave & 3;
+  const int wm = wave >> 1, wn = wave & 1;
 
   int bid = blockIdx.x;
   const int nwg = tiles_m * tiles_n;
@@ -221,132 +246,110 @@ __global__ __launch_bounds__(512) void gemm_fast_kernel(GemmParams p, int tiles_
   const int tile_m = g0 + (bid % group) % gh, tile_n = (bid % group) / gh;
   const int64_t m0 = (int64_t)tile_m * F_BM, n0 = (int64_t)tile_n * F_BN;
 
-  const uint16_t *__restrict__ A = (const uint16_t *)p.a;
-  const uint16_t *__restrict__ B = (const uint16_t *)p.b;
-  const bool loads_a = wave < 4;
-  const int lt = tid & 255;  // index among the 256 threads with the same role
-
-  // A role: chunk c = lt + 256 j -> row c / NL, 16-byte chunk c % NL
-  // B role: unit (kg = lt % 8, nc = lt / 8): rows NL kg .. NL kg + NL - 1, columns 8 nc .. 8 nc + 7
-  const uint16_t *gsrc;
-  int64_t gstep;  // elements between this thread's loads
-  if (loads_a) {
-    gsrc = A + (m0 + lt / NL) * p.lda + (lt % NL) * 8;
-    gstep = (256 / NL) * p.lda;
-  } else {
-    gsrc = B + (int64_t)((lt & 7) * NL) * p.ldb + n0 + (lt >> 3) * 8;
-    gstep = p.ldb;
+  // Wavefront w issues A instructions 4w..4w+3 (rows 16 ia + lane / 4) and B instructions
+  // 4w..4w+3 (k rows 2 ib + lane / 32) of a tile.  Per-lane byte offsets are constant; the
+  // tile's base address moves in scalar registers.
+  uint32_t a_voff[4], b_voff[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+    a_voff[i] = (uint32_t)(((64 * wave + 16 * i + lane / 4) * p.lda + 8 * ((lane & 3) ^ ((lane >> 4) & 3))) * 2);
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int krow = 8 * wave + 2 * i + lane / 32;
+    b_voff[i] = (uint32_t)((krow * p.ldb + 8 * ((lane & 31) ^ ((krow & 3) << 2))) * 2);
   }
-  auto gload = [&](int k0, uint4 (&r)[NL]) {
-    const uint16_t *src = loads_a ? gsrc + k0 : gsrc + (int64_t)k0 * p.ldb;
-#pragma unroll
-    for (int j = 0; j < NL; j++) r[j] = *reinterpret_cast<const uint4 *>(src + j * gstep);
+  const char *a_base = (const char *)((const uint16_t *)p.a + m0 * p.lda);
+  const char *b_base = (const char *)((const uint16_t *)p.b + n0);
+  const uint32_t lds0 = (uint32_t)(uintptr_t)TTS_LDS(smem);
+  const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int nk = (int)(p.K / F_BK);
+  auto dma = [&](const char *sbase, uint32_t voff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(voff), "s"(sbase) : "memory", "m0");
   };
-  auto lstore = [&](int buf, uint4 (&r)[NL]) {
-    uint16_t *As = smem + buf * (F_BM + F_BN) * PITCH, *Bs = As + F_BM * PITCH;
-    if (loads_a) {
-#pragma unroll
-      for (int j = 0; j < NL; j++)
-        *reinterpret_cast<uint4 *>(As + (lt / NL + (256 / NL) * j) * PITCH + (lt % NL) * 8) = r[j];
-    } else {
-      // r[t] = row k = NL kg + t, columns c = 0..7 (two per 32-bit word); the chunk written for
-      // column c holds k = 0..NL-1 of that column
-      uint32_t in[NL][4];
-#pragma unroll
-      for (int t = 0; t < NL; t++) { in[t][0] = r[t].x; in[t][1] = r[t].y; in[t][2] = r[t].z; in[t][3] = r[t].w; }
-      uint16_t *dst = Bs + ((lt >> 3) * 8) * PITCH + (lt & 7) * NL;
-#pragma unroll
-      for (int c2 = 0; c2 < 4; c2++) {
-        uint32_t even[NL / 2], odd[NL / 2];
-#pragma unroll
-        for (int tp = 0; tp < NL / 2; tp++) {
-          uint32_t x = in[2 * tp][c2], y = in[2 * tp + 1][c2];
-          even[tp] = __builtin_amdgcn_perm(y, x, 0x05040100u);  // [x.lo16, y.lo16]
-          odd[tp] = __builtin_amdgcn_perm(y, x, 0x07060302u);   // [x.hi16, y.hi16]
-        }
-        if (NL == 8) {
-          *reinterpret_cast<uint4 *>(dst + (2 * c2) * PITCH) = make_uint4(even[0], even[1], even[NL / 2 - 2], even[NL / 2 - 1]);
-          *reinterpret_cast<uint4 *>(dst + (2 * c2 + 1) * PITCH) = make_uint4(odd[0], odd[1], odd[NL / 2 - 2], odd[NL / 2 - 1]);
-        } else {
-          *reinterpret_cast<uint2 *>(dst + (2 * c2) * PITCH) = make_uint2(even[0], even[1]);
-          *reinterpret_cast<uint2 *>(dst + (2 * c2 + 1) * PITCH) = make_uint2(odd[0], odd[1]);
-        }
-      }
-    }
+  auto dma_one = [&](int t, int n) {  // n = 0..3: A part, 4..7: B part of tile t, into stage t % F_STAGES
+    const int tc = min(t, nk - 1);
+    const uint32_t st = lds0 + (t % F_STAGES) * F_STAGE_BYTES + wave_u * 4096;
+    if (n < 4) dma(a_base + (int64_t)tc * F_BK * 2, a_voff[n], st + n * 1024);
+    else dma(b_base + (int64_t)tc * F_BK * p.ldb * 2, b_voff[n - 4], st + F_A_BYTES + (n - 4) * 1024);
   };
 
-  f32x16 acc[4][2];
+  // fragment read offsets (bytes, within a stage)
+  // A: row r = wm * 128 + i * 32 + lane % 32, chunk c = 2 ks + lane / 32 at position c ^ ((r / 4) & 3)
+  const int ar = wm * 128 + (lane & 31);
+  const int a_off = ar * 64, a_sw = (ar >> 2) & 3;
+  // B: 16-lane group q = lane / 16, r16 = lane % 16: k row ks * 16 + 8 (q / 2) + 4 h + r16 / 4,
+  // chunk wn * 16 + 4 j + 2 (q & 1) + (r16 % 4) / 2, byte 8 (r16 & 1) within the chunk
+  const int q = lane >> 4, r16 = lane & 15;
+  const int b_chunk = wn * 16 + 2 * (q & 1) + ((r16 & 3) >> 1), b_sw = (r16 >> 2) << 2;
+  const int b_off = F_A_BYTES + (8 * (q >> 1) + (r16 >> 2)) * 512 + 8 * (r16 & 1);
+
+  f32x16 acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; i++)
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < 4; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-  const int nk = (int)(p.K / BK);
-  uint4 r0[NL], r1[NL];
-  // One K step.  Tile kt is in LDS buffer `cur`.  `rnew` is free and receives tile kt+DIST; `rsto`
-  // holds tile kt+1, which goes to the other LDS buffer (free since the barrier that ended step kt-1).
-  auto step = [&](int kt, int cur, uint4 (&rnew)[NL], uint4 (&rsto)[NL]) {
-    if (!(DBG & 4) && kt + DIST < nk) gload((kt + DIST) * BK, rnew);
-    if (EARLY && !(DBG & 4) && kt + 1 < nk) lstore(cur ^ 1, rsto);
-    const uint16_t *As = smem + cur * (F_BM + F_BN) * PITCH, *Bs = As + F_BM * PITCH;
-    const uint16_t *a_base = As + (wm * 128 + (lane & 31)) * PITCH + 8 * (lane >> 5);
-    const uint16_t *b_base = Bs + (wn * 64 + (lane & 31)) * PITCH + 8 * (lane >> 5);
-    uint4 af[2][4], bf[2][2];
-#pragma unroll
-    for (int i = 0; i < 4; i++) af[0][i] = *reinterpret_cast<const uint4 *>(a_base + i * 32 * PITCH);
-#pragma unroll
-    for (int j = 0; j < 2; j++) bf[0][j] = *reinterpret_cast<const uint4 *>(b_base + j * 32 * PITCH);
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      const int c = ks & 1, n = c ^ 1;
-      if (!(DBG & 2) && ks + 1 < KS) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) af[n][i] = *reinterpret_cast<const uint4 *>(a_base + i * 32 * PITCH + (ks + 1) * 16);
-#pragma unroll
-        for (int j = 0; j < 2; j++) bf[n][j] = *reinterpret_cast<const uint4 *>(b_base + j * 32 * PITCH + (ks + 1) * 16);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-          if (DBG & 1) acc[i][j][0] += __uint_as_float(af[c][i].x ^ bf[c][j].x);
-          else acc[i][j] = mfma32<BF16>(af[c][i], bf[c][j], acc[i][j]);
-        }
-    }
-    // pin the software pipeline: the fragment reads of step ks+1 are issued before the MFMAs of step
-    // ks, so that LDS latency is covered by eight MFMAs instead of being waited for
-    __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
-#pragma unroll
-    for (int ks = 0; ks + 1 < KS; ks++) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
-    if (!EARLY && !(DBG & 4) && kt + 1 < nk) lstore(cur ^ 1, rsto);
-    __syncthreads();
-  };
-  gload(0, r0);
-  if (DIST == 2 && nk > 1) gload(BK, r1);
-  lstore(0, r0);
-  __syncthreads();
-  for (int kt = 0; kt < nk; kt += 2) {
-    if (DIST == 2) {
-      step(kt, 0, r0, r1);                        // tile kt was in r0, tile kt+1 is in r1
-      if (kt + 1 < nk) step(kt + 1, 1, r1, r0);
+  uint4 af[2][4], bf[2][4];
+  // one fragment read (n = 0..3: A row block n; n = 4..11: B column block (n - 4) / 2, k half (n - 4) % 2)
+  auto read_one = [&](int t, int ks, int n, uint4 (&a)[4], uint4 (&b)[4]) {
+    const char *st = smem + (t % F_STAGES) * F_STAGE_BYTES;
+    if (n < 4) {
+      a[n] = *reinterpret_cast<const uint4 *>(st + a_off + n * 2048 + (((2 * ks + (lane >> 5)) ^ a_sw) << 4));
     } else {
-      step(kt, 0, r0, r0);
-      if (kt + 1 < nk) step(kt + 1, 1, r0, r0);
+      const int j = (n - 4) >> 1, h = (n - 4) & 1;
+      const char *bp = st + b_off + ks * 16 * 512 + (((b_chunk + 4 * j) ^ b_sw) << 4) + h * 4 * 512;
+      s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)TTS_LDS(bp));
+      uint2 v2 = __builtin_bit_cast(uint2, v);
+      if (h == 0) { b[j].x = v2.x; b[j].y = v2.y; } else { b[j].z = v2.x; b[j].w = v2.y; }
     }
+  };
+  auto mfma_one = [&](int n, uint4 (&a)[4], uint4 (&b)[4]) {
+    acc[n >> 2][n & 3] = mfma32<BF16>(a[n >> 2], b[n & 3], acc[n >> 2][n & 3]);
+  };
+
+  // prologue: STAGES - 1 tiles in flight; tile 0 landed; its first operands read
+  for (int t = 0; t < F_STAGES - 1; t++)
+#pragma unroll
+    for (int n = 0; n < 8; n++) dma_one(t, n);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(8 * (F_STAGES - 2), 15));
+  __syncthreads();
+#pragma unroll
+  for (int n = 0; n < 12; n++) read_one(0, 0, n, af[0], bf[0]);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+  for (int t = 0; t < nk; t++) {
+    // phase A: MFMAs of (tile t, first half); read (tile t, second half); first half of the loads of tile t + STAGES - 1
+#pragma unroll
+    for (int n = 0; n < 16; n++) {
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_one(n, af[0], bf[0]);
+      if (n < 12) read_one(t, 1, n, af[1], bf[1]);
+      if ((n & 3) == 3) dma_one(t + F_STAGES - 1, n >> 2);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // own loads of tile t+1 have landed (later ones may be in flight); own reads of tile t are complete
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(8 * (F_STAGES - 3) + 4, 0));
+    __syncthreads();
+    // phase B: MFMAs of (tile t, second half); read (tile t+1, first half); the rest of the loads
+#pragma unroll
+    for (int n = 0; n < 16; n++) {
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_one(n, af[1], bf[1]);
+      if (n < 12) read_one(t + 1, 0, n, af[0], bf[0]);
+      if ((n & 3) == 3) dma_one(t + F_STAGES - 1, (n >> 2) + 4);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
   }
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));  // the surplus loads land before the LDS goes away
 
   uint16_t *__restrict__ C = (uint16_t *)p.c;
 #pragma unroll
   for (int i = 0; i < 4; i++)
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      int64_t col = n0 + wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < 4; j++) {
+      int64_t col = n0 + wn * 128 + j * 32 + (lane & 31);
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         int64_t row = m0 + wm * 128 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
@@ -355,24 +358,21 @@ __global__ __launch_bounds__(512) void gemm_fast_kernel(GemmParams p, int tiles_
     }
 }
 
-template <bool BF16, int BK, int DIST, bool EARLY, int DBG = 0>
-hipError_t launch_gemm_fast(const GemmParams &p, hipStream_t s) {
-  constexpr size_t lds = 2 * (size_t)(F_BM + F_BN) * (BK + 8) * 2;
-  static bool configured = false;
-  auto kern = gemm_fast_kernel<BF16, BK, DIST, EARLY, DBG>;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+template <bool BF16>
+hipError_t launch_gemm_dma(const GemmParams &p, hipStream_t s) {
+  constexpr size_t lds = (size_t)F_STAGES * F_STAGE_BYTES;
+  auto kern = gemm_dma_kernel<BF16>;
+  static const hipError_t attr = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (attr != hipSuccess) return attr;
   int tiles_m = (int)(p.M / F_BM), tiles_n = (int)(p.N / F_BN);
-  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(512), lds, s, p, tiles_m, tiles_n);
+  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds, s, p, tiles_m, tiles_n);
   return hipGetLastError();
 }
 
+// whole tiles, 16-byte aligned rows, and per-lane byte offsets that fit 32 bits
 bool gemm_fast_path_ok(const GemmParams &p) {
-  return p.M % F_BM == 0 && p.N % F_BN == 0 && p.K % 64 == 0 && p.K >= 64 && p.lda % 8 == 0 && p.ldb % 8 == 0 &&
-         ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0;
+  return p.M % F_BM == 0 && p.N % F_BN == 0 && p.K % F_BK == 0 && p.K >= F_BK && p.lda % 8 == 0 && p.ldb % 8 == 0 &&
+         ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0 && p.lda < (1 << 22) && p.ldb < (1 << 25);
 }
 
 // ------------------------------------------------------ int8-weight GEMM
@@ -738,10 +738,8 @@ constexpr int W8_WAVES = 16;
 hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
   static const char *tile_env = getenv("TTS_GEMM_TILE");  // tuning aid: 128, 256 (general kernel) or unset
   if (!tile_env && gemm_fast_path_ok(p)) {
-    // BK = 64, one tile in flight, LDS filled after the MFMAs: the fastest of the measured
-    // combinations of BK in {32, 64}, DIST in {1, 2} and EARLY in {false, true} at 4096^3
-    *name = "gemm_fast_kernel";
-    return p.is_bf16 ? launch_gemm_fast<true, 64, 1, false>(p, s) : launch_gemm_fast<false, 64, 1, false>(p, s);
+    *name = "gemm_dma_kernel";
+    return p.is_bf16 ? launch_gemm_dma<true>(p, s) : launch_gemm_dma<false>(p, s);
   }
   bool big = p.M >= 2048 && p.N >= 2048;
   if (tile_env) big = atoi(tile_env) >= 256;
