@@ -42,6 +42,10 @@ def parse():
     ap.add_argument("--workload", default="cfg2", help="headline workload: cfg1..cfg5, cfg1_2p28, cfg2_1m")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-headline", action="store_true", help="time only the headline workload")
+    ap.add_argument("--rotating-only", action="store_true",
+                    help="skip the same-buffer and frontend passes, so that a kernel trace of this run holds rotating-buffer launches only")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run a 256 MiB device-to-device copy three times and exit (the known-size kernel that scales FETCH_SIZE/WRITE_SIZE)")
     return ap.parse_args()
 
 
@@ -134,7 +138,7 @@ def make_workloads(torch, triton, K):
     return W
 
 
-def time_workload(torch, spy, wl, steps, warmup):
+def time_workload(torch, spy, wl, steps, warmup, rotating_only=False):
     """Returns dict(us, kernel, sets).  Rotates over `sets` independent buffer sets."""
     sets = max(1, min(32, math.ceil(ROTATE_BYTES / wl["set_bytes"])))
     if wl["set_bytes"] > 1e9:
@@ -169,6 +173,11 @@ def time_workload(torch, spy, wl, steps, warmup):
     torch.cuda.synchronize()
     wall_us = (time.perf_counter() - t0) * 1e6 / steps
     us = start.elapsed_time(stop) * 1e3 / steps
+    if rotating_only:
+        kernel = plan.last_kernel
+        del launches
+        torch.cuda.empty_cache()
+        return dict(us=us, hot_us=us, wall_us=wall_us, kernel=kernel, sets=sets, frontend_us=0.0, warmup_steps_run=done)
     # same measurement on one buffer set ("hot": inputs may sit in the Infinity Cache), for information
     g, arr, n, _ = launches[0]
     for _ in range(warmup):
@@ -279,6 +288,16 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
+    if args.calibrate_copy:
+        n = 256 * 1024 * 1024
+        src = torch.ones(n, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration_copy_bytes": n, "copies": 3}))
+        return
     tsa.activate()
     spy = Spy()
     torch.manual_seed(0)
@@ -291,7 +310,7 @@ def main():
     for name in names:
         wl = W[name]
         steps = args.steps if wl["set_bytes"] < 1e9 else max(10, args.steps // 10)
-        t = time_workload(torch, spy, wl, steps, args.warmup)
+        t = time_workload(torch, spy, wl, steps, args.warmup, args.rotating_only)
         entry = dict(workload=wl["desc"], us=round(t["us"], 3), kernel=t["kernel"], steps=steps,
                      rotating_buffer_sets=t["sets"], warmup_steps_run=t["warmup_steps_run"], frontend_us_per_launch=round(t["frontend_us"], 1),
                      roofline=roofline(wl, t["us"], name), dtype=wl["dtype"], algorithmic_work=wl["work"],
