@@ -70,6 +70,20 @@ __device__ __forceinline__ float apply(float a, float b) {
   return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b);
 }
 
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+// Outputs are written once and not read again by the kernel: nontemporal stores keep them from
+// displacing the inputs in L2 / Infinity Cache (LayerNorm [4096, 8192]: 29.2 -> 27.4 us from HBM,
+// 23.3 -> 21.3 us with the input cached; nontemporal loads gained nothing and lost the cached case).
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void ntstore(uint4 *p, uint4 v) {
+  u32x4_t w = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(w, reinterpret_cast<u32x4_t *>(p));
+}
+__device__ __forceinline__ void ntstore(float4 *p, float4 v) {
+  f32x4_t w = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(w, reinterpret_cast<f32x4_t *>(p));
+}
+
 template <int OP, bool SWAP>
 __global__ __launch_bounds__(256) void map1d_f32_kernel(Map1DParams p) {
   const int px = blockIdx.x, py = blockIdx.y, pz = blockIdx.z;
@@ -92,7 +106,7 @@ __global__ __launch_bounds__(256) void map1d_f32_kernel(Map1DParams p) {
       } else {
         r.x = apply<OP>(a.x, b.x); r.y = apply<OP>(a.y, b.y); r.z = apply<OP>(a.z, b.z); r.w = apply<OP>(a.w, b.w);
       }
-      *reinterpret_cast<float4 *>(z + i) = r;
+      ntstore(reinterpret_cast<float4 *>(z + i), r);
     } else {
       for (int j = i; j < i + 4 && j < d; j++) z[j] = SWAP ? apply<OP>(y[j], x[j]) : apply<OP>(x[j], y[j]);
     }
@@ -198,7 +212,7 @@ __global__ __launch_bounds__(256) void softmax_f32_kernel(SoftmaxParams p, int g
       f32x4_a4 w;
 #pragma unroll
       for (int c = 0; c < 4; c++) w[c] = v[4 * j + c] * rsum;
-      if (i0 + 4 <= d_out) *reinterpret_cast<f32x4_a4 *>(out + i0) = w;
+      if (i0 + 4 <= d_out) __builtin_nontemporal_store(w, reinterpret_cast<f32x4_a4 *>(out + i0));
       else
 #pragma unroll
         for (int c = 0; c < 4; c++)
@@ -345,7 +359,7 @@ __global__ __launch_bounds__(256, CPT <= 4 ? 8 : 4) void layernorm_fwd_kernel(La
                    Half<BF16>::up((uint16_t)(bq[k] >> 16));
         o[k] = (uint32_t)Half<BF16>::down(y0) | ((uint32_t)Half<BF16>::down(y1) << 16);
       }
-      *reinterpret_cast<uint4 *>(y + i0) = make_uint4(o[0], o[1], o[2], o[3]);
+      ntstore(reinterpret_cast<uint4 *>(y + i0), make_uint4(o[0], o[1], o[2], o[3]));
     } else {
 #pragma unroll
       for (int k = 0; k < 8; k++)
