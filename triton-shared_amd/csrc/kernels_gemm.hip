@@ -353,7 +353,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmParams p, int tiles_m
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         int64_t row = m0 + wm * 128 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        C[row * p.ldc + col] = BF16 ? f32_to_bf16(acc[i][j][v]) : f32_to_f16(acc[i][j][v]);
+        __builtin_nontemporal_store(BF16 ? f32_to_bf16(acc[i][j][v]) : f32_to_f16(acc[i][j][v]), &C[row * p.ldc + col]);
       }
     }
 }
