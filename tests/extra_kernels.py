@@ -18,7 +18,7 @@ def masked_copy_2d(src, dst, rows, cols):
 
 @triton.jit
 def wraparound_rows(src, dst, M, BLOCK: tl.constexpr):
-    # modulo addressing: refused by this backend (wraparound is out of scope)
+    # modulo addressing outside a matmul: lowered to a structured access with a period, refused at the plan stage
     i = (tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)) % M
     tl.store(dst + tl.arange(0, BLOCK), tl.load(src + i))
 

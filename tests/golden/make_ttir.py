@@ -33,6 +33,11 @@ SIGS = {
                                       "s_cm": "i32", "s_cn": "constexpr", "BM": "constexpr", "BN": "constexpr",
                                       "BK": "constexpr", "GROUP_M": "constexpr"},
                      {"s_ak": 1, "s_bn": 1, "s_cn": 1, "BM": 128, "BN": 128, "BK": 64, "GROUP_M": 8}),
+    "matmul_wrapped": (K.matmul_wrapped, {"a_ptr": "*bf16", "b_ptr": "*bf16", "c_ptr": "*bf16", "M": "i32", "N": "i32",
+                                          "K": "i32", "s_am": "i32", "s_ak": "constexpr", "s_bk": "i32", "s_bn": "constexpr",
+                                          "s_cm": "i32", "s_cn": "constexpr", "BM": "constexpr", "BN": "constexpr",
+                                          "BK": "constexpr", "GROUP_M": "constexpr"},
+                       {"s_ak": 1, "s_bn": 1, "s_cn": 1, "BM": 128, "BN": 128, "BK": 64, "GROUP_M": 8}),
     "w8a16_matmul": (K.w8a16_matmul, {"a_ptr": "*fp16", "w_ptr": "*i8", "s_ptr": "*fp16", "c_ptr": "*fp16", "M": "i32",
                                       "N": "i32", "K": "i32", "s_am": "i32", "s_ak": "constexpr", "s_wk": "i32",
                                       "s_wn": "constexpr", "s_cm": "i32", "s_cn": "constexpr", "BM": "constexpr",
@@ -45,6 +50,7 @@ SMALL = {
     "row_softmax.small": ("row_softmax", {"BLOCK": 64}),
     "layer_norm_fwd.small": ("layer_norm_fwd", {"BLOCK": 64}),
     "matmul_tiles.small": ("matmul_tiles", {"BM": 32, "BN": 32, "BK": 16, "GROUP_M": 2}),
+    "matmul_wrapped.small": ("matmul_wrapped", {"BM": 32, "BN": 32, "BK": 16, "GROUP_M": 2}),
     "w8a16_matmul.small": ("w8a16_matmul", {"BM": 16, "BN": 32, "BK": 32}),
 }
 

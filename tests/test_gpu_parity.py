@@ -237,6 +237,27 @@ def test_gemm_whole_tile_kernel(K, M, N, Kd, dtype, pad):
     assert torch.equal(c.cpu(), -a.cpu()[:, perm])
 
 
+@pytest.mark.parametrize("M,N,Kd,dtype", [(179, 321, 167, torch.bfloat16), (70, 90, 40, torch.float16), (512, 768, 96, torch.bfloat16),
+                                         (1000, 130, 264, torch.float16)])
+def test_matmul_with_wraparound_operands(K, oracle_cpu, M, N, Kd, dtype):
+    # the stock tutorial form: rows of A / columns of B beyond the problem are read modulo M / N, not masked
+    # (test_matmul.py:74-75 in the reference); the result must be the dense product, and bit-identical to
+    # the masked form of the same kernel, which runs the same device code
+    torch.manual_seed(M * 7 + N)
+    a, b = (torch.randn(M, Kd) * 0.5).to(dtype), (torch.randn(Kd, N) * 0.5).to(dtype)
+    ad, bd = a.to(DEV), b.to(DEV)
+    cd = torch.full((M, N), 5.0, dtype=dtype, device=DEV)
+    grid = (triton.cdiv(M, 128) * triton.cdiv(N, 128),)
+    k = K.matmul_wrapped[grid](ad, bd, cd, M, N, Kd, ad.stride(0), 1, bd.stride(0), 1, cd.stride(0), 1,
+                               BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm"
+    assert relfro(cd.cpu(), a.double() @ b.double()) <= 1e-2
+    assert torch.equal(cd, _run_mm(K, a, b))
+    if M * N * Kd <= 179 * 321 * 167:
+        assert relfro(cd.cpu(), oracle_cpu.matmul_tiles(a, b)) <= 1e-2
+
+
 def test_gemm_with_padded_pitches_and_untouched_border(K):
     torch.manual_seed(3)
     M, N, Kd = 200, 300, 150

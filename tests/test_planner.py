@@ -120,11 +120,11 @@ def test_masked_2d_window_matches_reference_golden(native):
 
 
 # ---------------------------------------------------------------- text form
-@pytest.mark.parametrize("name", ["vec_add", "row_softmax", "layer_norm_fwd", "matmul_tiles", "w8a16_matmul"])
+@pytest.mark.parametrize("name", ["vec_add", "row_softmax", "layer_norm_fwd", "matmul_tiles", "matmul_wrapped", "w8a16_matmul"])
 def test_family_and_signature(native, name):
     plan, structured = plan_for(native, name)
     want = {"vec_add": "map1d", "row_softmax": "row_softmax", "layer_norm_fwd": "layernorm_fwd",
-            "matmul_tiles": "gemm", "w8a16_matmul": "gemm_w8a16"}[name]
+            "matmul_tiles": "gemm", "matmul_wrapped": "gemm", "w8a16_matmul": "gemm_w8a16"}[name]
     assert plan.family == want and plan.kernel_name == name
     # the small-block variant has the same op structure, hence the same signature
     small, _ = plan_for(native, name + ".small")
@@ -145,8 +145,10 @@ def test_plan_bytes_are_self_contained(native):
 def test_unsupported_kernels_are_refused(native):
     import extra_kernels as X
     sig = {"src": "*fp32", "dst": "*fp32", "M": "i32", "BLOCK": "constexpr"}
-    with pytest.raises(NotImplementedError, match="modulo"):
-        native.ttir_to_structured(compile_ttir(X.wraparound_rows, sig, {"BLOCK": 64}))
+    wrapped = native.ttir_to_structured(compile_ttir(X.wraparound_rows, sig, {"BLOCK": 64}))
+    assert "wraps=[arg2]" in wrapped                       # the structured stage carries the period (tts.make_tptr shape)
+    with pytest.raises(NotImplementedError, match="no hand-written kernel family"):
+        native.structured_to_plan(wrapped)                 # ... but only the matmul family executes it
     sig = {"src": "*fp32", "idx": "*i32", "dst": "*fp32", "BLOCK": "constexpr"}
     with pytest.raises(NotImplementedError, match="not a structured access"):
         native.ttir_to_structured(compile_ttir(X.gather_rows, sig, {"BLOCK": 64}))
@@ -227,16 +229,19 @@ def test_layernorm_binding_matches_every_lane(native):
         assert touched[("store", 5)][0][0] == affine(d["rstd_off"], p)
 
 
+@pytest.mark.parametrize("kernel", ["matmul_tiles.small", "matmul_wrapped.small"])
 @pytest.mark.parametrize("shape", [(70, 90, 40), (32, 32, 16), (33, 1, 17)])
-def test_gemm_binding_matches_every_lane(native, shape):
+def test_gemm_binding_matches_every_lane(native, shape, kernel):
+    # matmul_wrapped reads rows of A / columns of B modulo M / N (the stock tutorial form): the lanes it
+    # touches are still exactly the dense operands, and the launcher binds it to the same dense problem
     M, N, K = shape
-    plan, _ = plan_for(native, "matmul_tiles.small")
+    plan, _ = plan_for(native, kernel)
     grid = ((M + 31) // 32) * ((N + 31) // 32)
     lda, ldb, ldc = K + 3, N + 5, N + 1
     d = plan.describe_launch((grid, 1, 1), [0, 0, 0, M, N, K, lda, ldb, ldc])
     assert (d["M"], d["N"], d["K"], d["lda"], d["ldb"], d["ldc"]) == tuple(str(v) for v in (M, N, K, lda, ldb, ldc))
     mem = {0: np.zeros(M * lda, np.uint16), 1: np.zeros(K * ldb, np.uint16), 2: np.zeros(M * ldc, np.uint16)}
-    log = ttir_lanes.Interpreter(golden_ttir("matmul_tiles.small")).run(
+    log = ttir_lanes.Interpreter(golden_ttir(kernel)).run(
         (grid,), [None, None, None, M, N, K, lda, ldb, ldc], mem)
     loads = {0: [], 1: []}
     stores = []

@@ -34,7 +34,17 @@ struct PtrState {   // PtrAnalysis.h:52-129, structured fields only
   int scalar = -1;  // index expr
   std::vector<int> offsets, strides;
   std::vector<int64_t> sizes;
+  // per-dim wraparound period in elements of the pointee, already multiplied by the stride
+  // (PtrState::shape, PtrAnalysis.h:52-129); -1 = the dimension does not wrap.  The address
+  // contribution of dim d at index j is (offsets[d] + j * strides[d]) mod mods[d].
+  std::vector<int> mods;
   size_t rank() const { return sizes.size(); }
+  bool has_mod() const {
+    for (int m : mods)
+      if (m >= 0) return true;
+    return false;
+  }
+  void pad_mods() { mods.resize(sizes.size(), -1); }
 };
 
 struct MaskState {  // MaskAnalysis.h:63-180
@@ -204,7 +214,33 @@ class Lowerer {
       s.strides.push_back(P.pool.bin(EK::Add, l.strides[i], r.strides[i]));
       s.sizes.push_back(l.sizes[i]);
     }
+    // wraparound (PtrAnalysis.cpp:440-500): a dimension that wraps keeps its period when the other
+    // side adds nothing to it.  A scalar added to every lane (a splat, whose value sits in dim 0)
+    // is added after the wrap, so it moves to a dimension that does not wrap.
+    s.pad_mods();
+    const PtrState *a = &l, *b = &r;
+    if (b->has_mod()) std::swap(a, b);
+    if (b->has_mod()) throw Unsupported("PtrAnalysis: adding two wraparound index expressions");
+    if (a->has_mod()) {
+      for (size_t i = 0; i < a->rank(); i++) {
+        if (a->mods[i] < 0) continue;
+        s.mods[i] = a->mods[i];
+        if (is_zero(b->offsets[i]) && is_zero(b->strides[i])) continue;
+        size_t other = a->rank();
+        for (size_t j = 0; j < a->rank(); j++)
+          if (j != i && a->mods[j] < 0) { other = j; break; }
+        if (!is_zero(b->strides[i]) || other == a->rank())
+          throw Unsupported("PtrAnalysis: adding an index tensor to a dimension that wraps around (line " + std::to_string(op.line) + ")");
+        s.offsets[i] = a->offsets[i];
+        s.offsets[other] = P.pool.bin(EK::Add, s.offsets[other], b->offsets[i]);
+      }
+    }
     return s;
+  }
+
+  bool is_zero(int e) {
+    const Expr x = P.pool.at(e);
+    return x.k == EK::Const && x.val == 0;
   }
 
   PtrState mul_state(const PtrState &lhs, const PtrState &rhs, const Op &op) {  // PtrAnalysis.cpp:539-625
@@ -215,10 +251,12 @@ class Lowerer {
     if (r->scalar < 0 && l->scalar >= 0) std::swap(l, r);
     PtrState s;
     if (lhs.scalar >= 0 && rhs.scalar >= 0) s.scalar = P.pool.bin(EK::Mul, lhs.scalar, rhs.scalar);
+    if (r->has_mod()) throw Unsupported("PtrAnalysis: multiplying by a wraparound index expression");
     for (size_t i = 0; i < l->rank(); i++) {
       s.offsets.push_back(P.pool.bin(EK::Mul, l->offsets[i], r->scalar));
       s.strides.push_back(P.pool.bin(EK::Mul, l->strides[i], r->scalar));
       s.sizes.push_back(l->sizes[i]);
+      s.mods.push_back(i < l->mods.size() && l->mods[i] >= 0 ? P.pool.bin(EK::Mul, l->mods[i], r->scalar) : -1);
     }
     return s;
   }
@@ -261,6 +299,9 @@ class Lowerer {
       s.offsets.insert(s.offsets.begin() + axis, c64(0));
       s.sizes.insert(s.sizes.begin() + axis, 1);
       s.strides.insert(s.strides.begin() + axis, c64(0));
+      s.pad_mods();
+      s.mods.insert(s.mods.begin() + axis, -1);
+      s.mods.resize(s.sizes.size());
       return s;
     }
     if (op.name == "tt.broadcast") {  // :954-989
@@ -291,8 +332,18 @@ class Lowerer {
       }
       return s;
     }
-    if (op.name == "arith.remsi")
-      throw Unsupported("PtrAnalysis: modulo (wraparound) addressing is not supported by this backend");
+    if (op.name == "arith.remsi") {  // :810-891
+      PtrState rhs = visit(op.operands[1]);
+      if (rhs.scalar < 0) throw Unsupported("PtrAnalysis: remainder by something that is not a scalar");
+      s = visit(op.operands[0]);
+      s.pad_mods();
+      if (s.has_mod()) throw Unsupported("PtrAnalysis: several modulo operations in one index expression");
+      if (s.rank() == 1) s.mods[0] = rhs.scalar;
+      else if (s.rank() == 2 && d.type.shape[0] == 1) s.mods[1] = rhs.scalar;
+      else if (s.rank() == 2 && d.type.shape[1] == 1) s.mods[0] = rhs.scalar;
+      else throw Unsupported("PtrAnalysis: modulo on a tensor of this shape");
+      return s;
+    }
     throw Unsupported("PtrAnalysis: address computed by " + op.name + " (line " + std::to_string(op.line) +
                       ") is not a structured access");
   }
@@ -449,6 +500,10 @@ class Lowerer {
     a.sizes = st.sizes;
     a.offsets = st.offsets;
     a.strides = st.strides;
+    if (st.has_mod()) {
+      a.mods = st.mods;
+      a.mods.resize(st.rank(), -1);
+    }
     if (st.rank() == 0) a.offsets.push_back(st.scalar >= 0 ? st.scalar : c64(0));
     return a;
   }
@@ -606,8 +661,9 @@ class Lowerer {
         const std::string &y = yield->operands[j];
         if (c.kind == 0) {
           PtrState ns = visit(y);
-          if (ns.source != c.st.source || ns.sizes != c.st.sizes)
-            throw Unsupported("loop-carried pointer changes its base or block shape");
+          ns.pad_mods();
+          if (ns.source != c.st.source || ns.sizes != c.st.sizes || ns.mods != c.st.mods)
+            throw Unsupported("loop-carried pointer changes its base, block shape or wraparound");
           size_t slot = c.first_slot;
           if (ns.rank() == 0) {
             s.int_iters[slot].next = ns.scalar;

@@ -237,6 +237,12 @@ struct Matcher {
   throw Unsupported(std::string("the program has the op structure of family '") + family + "' but " + why);
 }
 
+void no_wrap(Matcher &m, const char *family) {
+  for (SOp *a : m.accesses)
+    for (int e : a->acc.mods)
+      if (e >= 0) refuse(family, "it addresses memory modulo a size (wraparound), which only the matmul family implements");
+}
+
 void unit_stride(Matcher &m, const Access &a, const char *family) {
   if (!m.is_const(a.strides.back(), 1)) refuse(family, "its innermost stride is not 1");
 }
@@ -263,6 +269,7 @@ bool try_map1d(Plan &pl) {
   if (!direct && !swapped) return false;
   if (st->operands[0] != op->result) return false;
   const char *F = "map1d";
+  no_wrap(m, F);
   for (SOp *a : {l0, l1, st}) {
     if (a->acc.sizes.size() != 1) return false;
     if (a->acc.elem != "f32") refuse(F, "its element type is " + a->acc.elem + " (only f32 is implemented)");
@@ -314,6 +321,7 @@ bool try_softmax(Plan &pl) {
   const char *F = "row_softmax";
   Matcher m(pl.prog);
   SOp *ld = m.accesses.at(0), *st = m.accesses.at(1);
+  no_wrap(m, F);
   unit_stride(m, ld->acc, F);
   unit_stride(m, st->acc, F);
   if (ld->acc.sizes != st->acc.sizes) refuse(F, "its load and store blocks differ in size");
@@ -353,6 +361,7 @@ bool try_layernorm(Plan &pl) {
   const char *F = "layernorm_fwd";
   Matcher m(pl.prog);
   if (m.loops.size() != 3 || m.accesses.size() != 8) return false;
+  no_wrap(m, F);
   SOp *x0 = m.accesses[0], *x1 = m.accesses[1], *mean_st = m.accesses[2], *rstd_st = m.accesses[3];
   SOp *w = m.accesses[4], *b = m.accesses[5], *x2 = m.accesses[6], *y = m.accesses[7];
   int64_t B = x0->acc.sizes[0];
@@ -436,6 +445,7 @@ struct Carried2D {
   int base = -1;   // sum of the offsets at iteration 0
   int kstep = -1;  // sum of the per-iteration advances
   int stride[2] = {-1, -1};
+  int init[2] = {-1, -1};  // per-dim offset at iteration 0
 };
 
 bool carried_state(Matcher &m, SOp *loop, const Access &a, Carried2D &out) {
@@ -473,6 +483,7 @@ bool carried_state(Matcher &m, SOp *loop, const Access &a, Carried2D &out) {
   }
   out.base = m.sum(inits);
   out.kstep = m.sum(steps);
+  for (size_t d = 0; d < 2 && d < inits.size(); d++) out.init[d] = inits[d];
   return true;
 }
 
@@ -505,11 +516,25 @@ bool try_gemm(Plan &pl, bool w8a16) {
   for (int e : C->acc.strides)
     if (!m.pid_free(e) || !m.loop_free(e)) refuse(F, "its output strides depend on the program id");
   // masks: rows against M, columns against N, K against what is left
+  // Rows of A / columns of B beyond the problem are either masked off (other = 0) or, as in the
+  // stock tutorial kernel, read modulo M / N (test_matmul.py:74-75): those lanes only reach
+  // outputs that the store masks off, so both forms are the same dense product.  The launcher
+  // checks that the period is M * lda (N) and that the tile origin itself does not wrap.
+  auto wraps = [&](const Access &a, size_t dim) { return a.mods.size() == 2 && a.mods[dim] >= 0; };
+  const bool a_wraps = wraps(A->acc, 0), b_wraps = wraps(Bm->acc, 1);
+  if (wraps(A->acc, 1) || wraps(Bm->acc, 0) || !C->acc.mods.empty()) refuse(F, "it wraps an address around in K or in the output");
   int r0, Mb, c0, Nb, r0c, Mc, c0c, Nc;
-  if (A->acc.dims.size() != 2 || !m.extent(A->acc.dims[0], BM, r0, Mb)) refuse(F, "its A rows are not masked as row0+arange < M");
-  if (Bm->acc.dims.size() != 2 || !m.extent(Bm->acc.dims[1], BN, c0, Nb)) refuse(F, "its B columns are not masked as col0+arange < N");
   if (C->acc.dims.size() != 2 || !m.extent(C->acc.dims[0], BM, r0c, Mc) || !m.extent(C->acc.dims[1], BN, c0c, Nc))
     refuse(F, "its output is not masked as (row0+arange < M) & (col0+arange < N)");
+  if (A->acc.dims.size() != 2 || Bm->acc.dims.size() != 2) refuse(F, "its operand loads carry no K mask");
+  if (a_wraps) {
+    if (!m.is_const(A->acc.dims[0], BM)) refuse(F, "its A rows are both wrapped and masked");
+    r0 = r0c; Mb = Mc;
+  } else if (!m.extent(A->acc.dims[0], BM, r0, Mb)) refuse(F, "its A rows are not masked as row0+arange < M");
+  if (b_wraps) {
+    if (!m.is_const(Bm->acc.dims[1], BN)) refuse(F, "its B columns are both wrapped and masked");
+    c0 = c0c; Nb = Nc;
+  } else if (!m.extent(Bm->acc.dims[1], BN, c0, Nb)) refuse(F, "its B columns are not masked as col0+arange < N");
   if (r0 != r0c || c0 != c0c || Mb != Mc || Nb != Nc) refuse(F, "its operand masks and its output mask disagree");
   if (A->acc.dims[1] != Bm->acc.dims[0]) refuse(F, "A and B mask the K dimension differently");
   if (!m.pid_free(A->acc.dims[1])) refuse(F, "its K mask depends on the program id");
@@ -554,6 +579,8 @@ bool try_gemm(Plan &pl, bool w8a16) {
   pl.e["N"] = Nb;
   pl.e["kdim"] = A->acc.dims[1];
   pl.e["trip"] = loop->ub;
+  if (a_wraps) { pl.e["a_mod"] = A->acc.mods[0]; pl.e["a_wrapped"] = ca.init[0]; }
+  if (b_wraps) { pl.e["b_mod"] = Bm->acc.mods[1]; pl.e["b_wrapped"] = cb.init[1]; }
   return true;
 }
 

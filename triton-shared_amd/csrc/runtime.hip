@@ -218,6 +218,10 @@ DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
     }
   }
   need(r.ev0("a_kstep") == BK && r.ev0("b_kstep") == BK * d.ldb, "operand pointers do not advance by one K block per iteration");
+  // wraparound operands: the period is the whole matrix, so rows (columns) inside the problem are not affected
+  const bool a_wraps = pl.e.count("a_mod"), b_wraps = pl.e.count("b_mod");
+  if (a_wraps) need(r.ev0("a_mod") == d.M * d.lda, "A rows wrap around with a period other than M");
+  if (b_wraps) need(r.ev0("b_mod") == d.N, "B columns wrap around with a period other than N");
   // tiles: every program's origin, offsets consistent with a dense layout, exact cover
   const int64_t tm = (d.M + BM - 1) / BM, tn = (d.N + BN - 1) / BN;
   need((int64_t)r.g[0] * r.g[1] * r.g[2] == tm * tn, "the grid does not have one program per output tile");
@@ -233,6 +237,8 @@ DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
         s = 1;
         need(r.ev("a_base", e) == r0 * d.lda, "A tile offset is not row0 * lda");
         need(r.ev("b_base", e) == c0, "B tile offset is not col0");
+        if (a_wraps) need(r.ev("a_wrapped", e) == r0 * d.lda, "the wrapped part of A's offset is not row0 * lda");
+        if (b_wraps) need(r.ev("b_wrapped", e) == c0, "the wrapped part of B's offset is not col0");
         need(r.ev("c_base", e) == r0 * d.ldc + c0, "C tile offset is not row0 * ldc + col0");
       }
   return d;

@@ -54,6 +54,9 @@ struct Access {          // the tts.make_tptr + mask part of a load/store
   std::vector<int> offsets;          // per-dim, already multiplied by the stride (index exprs)
   std::vector<int> strides;          // per-dim (index exprs)
   std::vector<int> dims;             // per-dim valid extent (index exprs); empty = unmasked
+  std::vector<int> mods;             // per-dim wraparound period (index exprs, in elements, -1 = none); empty = no wraparound:
+                                     // dim d at index j contributes (offsets[d] + j * strides[d]) mod mods[d] to the address
+                                     // (tts.make_tptr `shape`, TritonStructuredDialect.td:33-121; StructuredToMemref.cpp:263-487)
   bool has_other = false;
   double other_f = 0;                // value of `other` when the element type is a float
   int64_t other_i = 0;               // ... when it is an integer

@@ -86,6 +86,7 @@ std::string print_program(const Program &p) {
       for (int e : s.acc.offsets) reach(e);
       for (int e : s.acc.strides) reach(e);
       for (int e : s.acc.dims) reach(e);
+      for (int e : s.acc.mods) reach(e);
       reach(s.expr);
       if (s.kind == SK::For) {
         reach(s.lb); reach(s.ub); reach(s.step);
@@ -138,10 +139,16 @@ std::string print_program(const Program &p) {
         case SK::Load: case SK::Store: case SK::ScalarLoad: case SK::ScalarStore:
           os << " base=" << s.acc.base_arg << " elem=" << s.acc.elem << " sizes=" << list(s.acc.sizes)
              << " offsets=" << list(s.acc.offsets) << " strides=" << list(s.acc.strides) << " dims=" << list(s.acc.dims);
+          if (!s.acc.mods.empty()) os << " mods=" << list(s.acc.mods);
           if (s.acc.has_other) os << " other_f=" << dbl_bits(s.acc.other_f) << " other_i=" << s.acc.other_i;
           os << " ; " << p.arg_names[s.acc.base_arg] << " offsets=" << exprs(s.acc.offsets)
              << " strides=" << exprs(s.acc.strides);
           if (!s.acc.dims.empty()) os << " dims=" << exprs(s.acc.dims);
+          if (!s.acc.mods.empty()) {
+            os << " wraps=[";
+            for (size_t i = 0; i < s.acc.mods.size(); i++) os << (i ? ", " : "") << (s.acc.mods[i] < 0 ? std::string("-") : p.pool.str(s.acc.mods[i]));
+            os << "]";
+          }
           if (s.acc.has_other) os << " other=" << (s.acc.elem[0] == 'i' ? (double)s.acc.other_i : s.acc.other_f);
           break;
         case SK::Const: os << " fval=" << dbl_bits(s.fval) << " ival=" << s.ival << " ; " << (p.values[s.result].dtype[0] == 'i' ? (double)s.ival : s.fval); break;
@@ -331,6 +338,7 @@ Program read_program(const std::string &text) {
       s.acc.offsets = Es(f.get("offsets"));
       s.acc.strides = Es(f.get("strides"));
       s.acc.dims = Es(f.get("dims"));
+      if (f.has("mods")) s.acc.mods = Es(f.get("mods"));
       if (f.has("other_f")) {
         s.acc.has_other = true;
         s.acc.other_f = bits_dbl(f.get("other_f"));

@@ -99,6 +99,43 @@ def matmul_tiles(a_ptr, b_ptr, c_ptr, M, N, K,
 
 
 @triton.jit
+def matmul_wrapped(a_ptr, b_ptr, c_ptr, M, N, K,
+                   s_am, s_ak, s_bk, s_bn, s_cm, s_cn,
+                   BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr, GROUP_M: tl.constexpr):
+    """The stock tutorial form of the tiled matmul: rows of A and columns of B beyond the problem are read
+    modulo M and N instead of being masked; only K and the output carry masks."""
+    pid = tl.program_id(0)
+    tiles_m = tl.cdiv(M, BM)
+    tiles_n = tl.cdiv(N, BN)
+    per_group = GROUP_M * tiles_n
+    g = pid // per_group
+    m0 = g * GROUP_M
+    rows_in_group = min(tiles_m - m0, GROUP_M)
+    tm = m0 + (pid % rows_in_group)
+    tn = (pid % per_group) // rows_in_group
+
+    ra = (tm * BM + tl.arange(0, BM)) % M
+    rb = (tn * BN + tl.arange(0, BN)) % N
+    rk = tl.arange(0, BK)
+    pa = a_ptr + (ra[:, None] * s_am + rk[None, :] * s_ak)
+    pb = b_ptr + (rk[:, None] * s_bk + rb[None, :] * s_bn)
+
+    acc = tl.zeros((BM, BN), dtype=tl.float32)
+    for k in range(0, tl.cdiv(K, BK)):
+        left = K - k * BK
+        a = tl.load(pa, mask=rk[None, :] < left, other=0.0)
+        b = tl.load(pb, mask=rk[:, None] < left, other=0.0)
+        acc += tl.dot(a, b)
+        pa += BK * s_ak
+        pb += BK * s_bk
+    out = acc.to(c_ptr.dtype.element_ty)
+    rm = tm * BM + tl.arange(0, BM)
+    rn = tn * BN + tl.arange(0, BN)
+    pc = c_ptr + s_cm * rm[:, None] + s_cn * rn[None, :]
+    tl.store(pc, out, mask=(rm[:, None] < M) & (rn[None, :] < N))
+
+
+@triton.jit
 def w8a16_matmul(a_ptr, w_ptr, s_ptr, c_ptr, M, N, K,
                  s_am, s_ak, s_wk, s_wn, s_cm, s_cn,
                  BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr):
