@@ -128,6 +128,22 @@ def make_workloads(torch, triton, K):
         return dict(desc="W8A16 matmul A fp16 [16, 8192] x W int8 [8192, 28672], fp16 scales, fp32 acc", work=work,
                     bound="hbm", dtype="f16", make=make, set_bytes=work)
 
+    def fused_gelu(n):
+        def make():
+            x, b = torch.randn(n, device=dev), torch.randn(n, device=dev)
+            y = torch.empty(n, device=dev)
+            return lambda: K.gelu_tanh_bias[(triton.cdiv(n, 1024),)](x, b, y, n, BLOCK=1024)
+        return dict(desc=f"fused map y = gelu_tanh(x + b) fp32 N={n}, BLOCK=1024 (19 elementwise ops on the interpreter kernel)",
+                    work=3 * n * 4, bound="hbm", dtype="f32", make=make, set_bytes=3 * n * 4)
+
+    def fused_silu(n):
+        def make():
+            g, u = torch.randn(n, device=dev).half(), torch.randn(n, device=dev).half()
+            o = torch.empty(n, dtype=torch.float16, device=dev)
+            return lambda: K.silu_mul_f16[(triton.cdiv(n, 1024),)](g, u, o, n, BLOCK=1024)
+        return dict(desc=f"fused map out = silu(g) * u fp16 N={n}, BLOCK=1024 (10 elementwise ops on the interpreter kernel)",
+                    work=3 * n * 2, bound="hbm", dtype="f16", make=make, set_bytes=3 * n * 2)
+
     W["cfg1"] = vec_add(98432)
     W["cfg2"] = softmax(4096)
     W["cfg3"] = layernorm()
@@ -135,6 +151,8 @@ def make_workloads(torch, triton, K):
     W["cfg5"] = w8a16()
     W["cfg1_2p28"] = vec_add(1 << 28)
     W["cfg2_1m"] = softmax(1 << 20)
+    W["next_fused_gelu_2p26"] = fused_gelu(1 << 26)
+    W["next_fused_silu_2p26"] = fused_silu(1 << 26)
     return W
 
 
@@ -315,7 +333,7 @@ def main():
                      rotating_buffer_sets=t["sets"], warmup_steps_run=t["warmup_steps_run"], frontend_us_per_launch=round(t["frontend_us"], 1),
                      roofline=roofline(wl, t["us"], name), dtype=wl["dtype"], algorithmic_work=wl["work"],
                      same_buffers=dict(us=round(t["hot_us"], 3), frac=roofline(wl, t["hot_us"])["frac"]))
-        if not args.no_cpu and (name == args.workload or not name.endswith(("2p28", "1m"))):
+        if not args.no_cpu and (name == args.workload or not name.endswith(("2p28", "1m", "2p26"))):
             entry["cpu_baseline"] = cpu_baseline(torch, name, wl)
         kernels[name] = entry
     head = kernels[args.workload]

@@ -95,6 +95,11 @@ def _wrap(v, bits):
     return v - (1 << bits) if bits > 1 and v >> (bits - 1) else v
 
 
+def _erf(v):
+    from scipy.special import erf
+    return erf(v).astype(np.asarray(v).dtype)
+
+
 class Interpreter:
     def __init__(self, ttir_text):
         lines = [l.strip() for l in _strip_loc(ttir_text).splitlines() if l.strip()]
@@ -350,6 +355,16 @@ class Interpreter:
                  "ne": np.not_equal, "ult": np.less}[words[0]]
             r = f(a.d, b.d)
             return Val(r if isinstance(r, np.ndarray) else int(bool(r)), "i1")
+        if name == "arith.cmpf":
+            lt, gt, eq = np.less(a.d, b.d), np.greater(a.d, b.d), np.equal(a.d, b.d)
+            uno = np.isnan(a.d) | np.isnan(b.d)
+            r = {"oeq": eq, "one": lt | gt, "olt": lt, "ole": lt | eq, "ogt": gt, "oge": gt | eq, "ord": ~uno, "uno": uno,
+                 "ueq": uno | eq, "une": ~eq, "ult": uno | lt, "ule": uno | lt | eq, "ugt": uno | gt, "uge": uno | gt | eq}[words[0]]
+            return Val(r if isinstance(r, np.ndarray) else int(bool(r)), "i1")
+        if name == "math.fma":
+            with np.errstate(all="ignore"):
+                r = (np.asarray(ops[0].d, np.float64) * np.asarray(ops[1].d, np.float64) + np.asarray(ops[2].d, np.float64))
+            return self._as_float(r.astype(np.float32), a.elem, isinstance(a.d, np.ndarray), already=False)
         if name == "arith.select":
             c, x, y = ops
             if isinstance(c.d, np.ndarray) or isinstance(x.d, np.ndarray):
@@ -374,7 +389,9 @@ class Interpreter:
             with np.errstate(all="ignore"):
                 r = fl[name](a.d, b.d)
             return self._as_float(r, a.elem, isinstance(r, np.ndarray), already=a.elem != "bf16")
-        un = {"math.exp": np.exp, "math.sqrt": np.sqrt, "math.log": np.log, "math.absf": np.abs, "arith.negf": np.negative}
+        un = {"math.exp": np.exp, "math.sqrt": np.sqrt, "math.log": np.log, "math.absf": np.abs, "arith.negf": np.negative,
+              "math.exp2": np.exp2, "math.log2": np.log2, "math.rsqrt": lambda v: 1 / np.sqrt(v), "math.sin": np.sin,
+              "math.cos": np.cos, "math.tanh": np.tanh, "math.floor": np.floor, "math.ceil": np.ceil, "math.erf": _erf}
         if name in un:
             with np.errstate(all="ignore"):
                 r = un[name](a.d)

@@ -32,7 +32,7 @@ def gather_rows(src, idx, dst, BLOCK: tl.constexpr):
 
 @triton.jit
 def fused_mul_add(x_ptr, y_ptr, z_ptr, n, BLOCK: tl.constexpr):
-    # structured, but matches no hand-written kernel family (two ops in the map)
+    # two ops in the map: runs on the fused-map interpreter kernel
     i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
     m = i < n
     a = tl.load(x_ptr + i, mask=m)
@@ -47,3 +47,11 @@ def vec_sub_swapped(x_ptr, y_ptr, z_ptr, n, BLOCK: tl.constexpr):
     a = tl.load(x_ptr + i, mask=m)
     b = tl.load(y_ptr + i, mask=m)
     tl.store(z_ptr + i, b - a, mask=m)
+
+
+@triton.jit
+def block_sum(x_ptr, out_ptr, n, BLOCK: tl.constexpr):
+    # structured, but matches no hand-written kernel family (a reduction to one value per program)
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    v = tl.load(x_ptr + i, mask=i < n, other=0.0)
+    tl.store(out_ptr + tl.program_id(0), tl.sum(v, axis=0))

@@ -43,6 +43,12 @@ SIGS = {
                                       "s_wn": "constexpr", "s_cm": "i32", "s_cn": "constexpr", "BM": "constexpr",
                                       "BN": "constexpr", "BK": "constexpr"},
                      {"s_ak": 1, "s_wn": 1, "s_cn": 1, "BM": 16, "BN": 128, "BK": 128}),
+    "gelu_tanh_bias": (K.gelu_tanh_bias, {"x_ptr": "*fp32", "b_ptr": "*fp32", "y_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"},
+                       {"BLOCK": 1024}),
+    "clamp_scale_where": (K.clamp_scale_where, {"x_ptr": "*fp32", "y_ptr": "*fp32", "out_ptr": "*fp32", "n": "i32", "lo": "fp32",
+                                                "hi": "fp32", "alpha": "fp32", "BLOCK": "constexpr"}, {"BLOCK": 1024}),
+    "silu_mul_f16": (K.silu_mul_f16, {"g_ptr": "*fp16", "u_ptr": "*fp16", "out_ptr": "*fp16", "n": "i32", "BLOCK": "constexpr"},
+                     {"BLOCK": 1024}),
 }
 # small-block variants for the brute-force tests
 SMALL = {
@@ -71,10 +77,19 @@ def strip_loc(text):
 
 
 def ttir_of(fn, sig, consts):
+    """TTIR only: the frontend plus the reference's TTIR pass list, without the later stages (a kernel
+    need not belong to a kernel family to have a fixture)."""
+    from triton._C.libtriton import ir
+    from triton_shared_amd.backend.compiler import HIPBackend
     tsa.register_backend()
-    os.environ.setdefault("TRITON_ALWAYS_COMPILE", "1")
-    k = triton.compile(ASTSource(fn, signature=sig, constexprs=consts), target=GPUTarget(tsa.BACKEND_NAME, "gfx950", 64))
-    return k.asm["ttir"]
+    src = ASTSource(fn, signature=sig, constexprs=consts)
+    target = GPUTarget(tsa.BACKEND_NAME, "gfx950", 64)
+    backend = HIPBackend(target)
+    ctx = ir.context()
+    ir.load_dialects(ctx)
+    options = backend.parse_options({})
+    mod = src.make_ir(target, options, backend.get_codegen_implementation(options), backend.get_module_map(), ctx)
+    return str(backend.make_ttir(mod, {}, options))
 
 
 def main():

@@ -347,6 +347,111 @@ def test_w8a16_split_k_repeated_launches(K):
         prev = cd
 
 
+# ------------------------------------------------------------- fused maps
+def _lanes(name, n, scalars, inputs, out_dtype, block=1024):
+    from conftest import golden_ttir
+    from oracle import ttir_lanes
+    mem = {i: a for i, a in enumerate(inputs)}
+    out = np.zeros(n, dtype=out_dtype)
+    mem[len(inputs)] = out
+    ttir_lanes.Interpreter(golden_ttir(name)).run(((n + block - 1) // block,), [None] * (len(inputs) + 1) + [n] + list(scalars), mem)
+    return out
+
+
+@pytest.mark.parametrize("n", [1, 1023, 5000, (1 << 20) + 3])
+def test_fused_map_gelu(K, n):
+    torch.manual_seed(n)
+    x, b = torch.randn(n) * 2, torch.randn(n)
+    xd, bd, yd = x.to(DEV), b.to(DEV), torch.full((n + 8,), 5.0, device=DEV)
+    k = K.gelu_tanh_bias[(triton.cdiv(n, 1024),)](xd, bd, yd, n, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "fused_map" and k.function.last_kernel == "fused_map (hipRTC)"
+    v = (x + b).double()
+    want = 0.5 * v * (1 + torch.tanh(0.7978845608028654 * (v + 0.044715 * v ** 3)))
+    assert (yd[:n].cpu().double() - want).abs().max().item() <= 2e-6
+    assert torch.equal(yd[n:].cpu(), torch.full((8,), 5.0))               # nothing past the mask is written
+    if n <= 5000:                                                          # the oracle: every op as the lanes do it
+        ref = _lanes("gelu_tanh_bias", n, [], [x.numpy().copy(), b.numpy().copy()], np.float32)
+        assert np.abs(yd[:n].cpu().numpy() - ref).max() <= 1e-6
+
+
+def test_fused_map_scalars_compare_select(K):
+    n = 4099
+    torch.manual_seed(5)
+    x, y = torch.randn(n), torch.randn(n)
+    x[:4] = torch.tensor([float("nan"), 1.0, float("-inf"), 0.5])
+    y[:4] = torch.tensor([0.0, float("nan"), 2.0, 0.5])
+    xd, yd, od = x.to(DEV), y.to(DEV), torch.zeros(n, device=DEV)
+    k = K.clamp_scale_where[(triton.cdiv(n, 1024),)](xd, yd, od, n, -0.5, 1.25, 3.0, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "fused_map"
+    ref = _lanes("clamp_scale_where", n, [-0.5, 1.25, 3.0], [x.numpy().copy(), y.numpy().copy()], np.float32)
+    got = od.cpu().numpy()
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    assert np.array_equal(got[~np.isnan(ref)], ref[~np.isnan(ref)])      # one IEEE op per value and exact selects: bit-exact
+    # other scalar arguments reuse the plan with new immediates
+    K.clamp_scale_where[(triton.cdiv(n, 1024),)](xd, yd, od, n, 0.0, 0.25, -2.0, BLOCK=1024)
+    ref = _lanes("clamp_scale_where", n, [0.0, 0.25, -2.0], [x.numpy().copy(), y.numpy().copy()], np.float32)
+    got = od.cpu().numpy()
+    assert np.array_equal(got[~np.isnan(ref)], ref[~np.isnan(ref)])
+
+
+@pytest.mark.parametrize("n", [7, 4096, 100003])
+def test_fused_map_fp16_io(K, n):
+    torch.manual_seed(n)
+    g, u = (torch.randn(n) * 3).half(), torch.randn(n).half()
+    gd, ud, od = g.to(DEV), u.to(DEV), torch.zeros(n, dtype=torch.float16, device=DEV)
+    k = K.silu_mul_f16[(triton.cdiv(n, 1024),)](gd, ud, od, n, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "fused_map"
+    want = (g.double() / (1 + torch.exp(-g.double())) * u.double())
+    assert ((od.cpu().double() - want).abs() <= 1e-3 * want.abs() + 1e-4).all()     # half an fp16 ulp is 4.9e-4 relative
+    if n <= 4096:
+        ref = _lanes("silu_mul_f16", n, [], [g.numpy().copy(), u.numpy().copy()], np.float16)
+        # fp32 exp differs in the last bit between libm and the device: at most one fp16 ulp after the final rounding
+        assert np.abs(od.cpu().numpy().astype(np.float32) - ref.astype(np.float32)).max() <= 2e-3 * max(1.0, np.abs(ref.astype(np.float32)).max())
+
+
+@pytest.mark.parametrize("kernel", ["gelu", "where", "silu"])
+def test_fused_map_interpreter_and_compiled_kernel_agree(K, kernel, monkeypatch):
+    # the register program runs either on the interpreter kernel or as a kernel compiled from the same program:
+    # every instruction is the same expression in both, so the outputs are the same bits
+    n = 70001
+    torch.manual_seed(11)
+    x, y = (torch.randn(n) * 3).to(DEV), torch.randn(n).to(DEV)
+    outs = []
+    for mode in ("interpreter", "compiled"):
+        if mode == "interpreter":
+            monkeypatch.setenv("TTS_FUSED_MAP", "interpreter")
+        else:
+            monkeypatch.delenv("TTS_FUSED_MAP", raising=False)
+        if kernel == "gelu":
+            o = torch.zeros(n, device=DEV)
+            k = K.gelu_tanh_bias[(triton.cdiv(n, 1024),)](x, y, o, n, BLOCK=1024)
+        elif kernel == "where":
+            o = torch.zeros(n, device=DEV)
+            k = K.clamp_scale_where[(triton.cdiv(n, 1024),)](x, y, o, n, -0.75, 0.5, 1.5, BLOCK=1024)
+        else:
+            o = torch.zeros(n, dtype=torch.float16, device=DEV)
+            k = K.silu_mul_f16[(triton.cdiv(n, 1024),)](x.half(), y.half(), o, n, BLOCK=1024)
+        torch.cuda.synchronize()
+        assert k.function.last_kernel == ("mapn_kernel" if mode == "interpreter" else "fused_map (hipRTC)")
+        outs.append(o)
+    assert torch.equal(outs[0], outs[1])
+
+
+def test_fused_map_two_ops(K):
+    import extra_kernels as X
+    n = 3000
+    torch.manual_seed(1)
+    a, b = torch.randn(n), torch.randn(n)
+    zd = torch.zeros(n, device=DEV)
+    k = X.fused_mul_add[(triton.cdiv(n, 256),)](a.to(DEV), b.to(DEV), zd, n, BLOCK=256)
+    torch.cuda.synchronize()
+    assert k.function.family == "fused_map"
+    assert torch.equal(zd.cpu(), a * b + a)                              # two roundings, no contraction into an fma
+
+
 # ------------------------------------------------------------- error paths
 def test_errors_surface_as_python_exceptions(K):
     import extra_kernels as X
@@ -354,7 +459,7 @@ def test_errors_surface_as_python_exceptions(K):
     with pytest.raises(TypeError, match="device"):
         K.vec_add[(1,)](torch.zeros(1024), x, x, 1024, BLOCK=1024)     # host tensor
     with pytest.raises(NotImplementedError):
-        X.fused_mul_add[(1,)](x, x, x, 1024, BLOCK=256)                # matches no family: refused, no fallback
+        X.block_sum[(4,)](x, x, 1024, BLOCK=256)                       # matches no family: refused, no fallback
     with pytest.raises(NotImplementedError, match="one program per output tile"):
         a = torch.zeros(256, 256, dtype=torch.bfloat16, device=DEV)
         K.matmul_tiles[(3,)](a, a, a, 256, 256, 256, 256, 1, 256, 1, 256, 1, BM=128, BN=128, BK=64, GROUP_M=8)

@@ -167,3 +167,36 @@ def test_lanes_vs_c_w8a16(oracle_cpu):
     it.run((1, (N + 31) // 32), [None] * 4 + [M, N, K, K, N, N],
            {0: a.numpy().reshape(-1), 1: w.numpy().reshape(-1), 2: s.numpy(), 3: c.numpy().reshape(-1)})
     assert torch.equal(c, oracle_cpu.w8a16_matmul(a, w, s, BM=16, BN=32, BK=32))
+
+
+# ---- fused elementwise maps: the lane interpreter is the oracle; pin its ops by closed forms in float64
+def _run_lanes(name, n, scalars, inputs, out_dtype, block=1024):
+    it = ttir_lanes.Interpreter(golden_ttir(name))
+    mem = {i: a for i, a in enumerate(inputs)}
+    out = np.zeros(n, dtype=out_dtype)
+    mem[len(inputs)] = out
+    it.run(((n + block - 1) // block,), [None] * (len(inputs) + 1) + [n] + list(scalars), mem)
+    return out
+
+
+def test_lanes_fused_maps_against_closed_forms():
+    rng = np.random.default_rng(0)
+    n = 3000
+    x, y = rng.standard_normal(n).astype(np.float32) * 2, rng.standard_normal(n).astype(np.float32)
+    got = _run_lanes("gelu_tanh_bias", n, [], [x.copy(), y.copy()], np.float32)
+    v = x.astype(np.float64) + y
+    want = 0.5 * v * (1 + np.tanh(0.7978845608028654 * (v + 0.044715 * v ** 3)))
+    assert np.abs(got - want).max() <= 2e-6
+    got = _run_lanes("clamp_scale_where", n, [-0.5, 1.25, 3.0], [x.copy(), y.copy()], np.float32)
+    want = np.where(x > y, 3.0 * np.clip(x, -0.5, 1.25), np.sqrt(np.abs(y.astype(np.float64))))
+    assert np.abs(got - want).max() <= 1e-6
+    g, u = x.astype(np.float16), y.astype(np.float16)
+    got = _run_lanes("silu_mul_f16", n, [], [g.copy(), u.copy()], np.float16)
+    g64, u64 = g.astype(np.float64), u.astype(np.float64)
+    want = g64 / (1 + np.exp(-g64)) * u64
+    assert np.abs(got.astype(np.float64) - want).max() <= 2e-3 * np.abs(want).max()
+    # special values through the comparison and min/max ops: NaN compares false, maxnumf/minnumf drop it
+    xs = np.array([np.nan, 1.0, -np.inf, 0.5], np.float32)
+    ys = np.array([0.0, np.nan, 2.0, 0.5], np.float32)
+    got = _run_lanes("clamp_scale_where", 4, [-0.5, 1.25, 3.0], [xs.copy(), ys.copy()], np.float32)
+    assert got[0] == 0.0 and np.isnan(got[1]) and got[2] == np.float32(np.sqrt(2.0)) and got[3] == np.float32(np.sqrt(0.5))

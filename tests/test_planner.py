@@ -147,13 +147,13 @@ def test_unsupported_kernels_are_refused(native):
     sig = {"src": "*fp32", "dst": "*fp32", "M": "i32", "BLOCK": "constexpr"}
     wrapped = native.ttir_to_structured(compile_ttir(X.wraparound_rows, sig, {"BLOCK": 64}))
     assert "wraps=[arg2]" in wrapped                       # the structured stage carries the period (tts.make_tptr shape)
-    with pytest.raises(NotImplementedError, match="no hand-written kernel family"):
+    with pytest.raises(NotImplementedError, match="wraparound"):
         native.structured_to_plan(wrapped)                 # ... but only the matmul family executes it
     sig = {"src": "*fp32", "idx": "*i32", "dst": "*fp32", "BLOCK": "constexpr"}
     with pytest.raises(NotImplementedError, match="not a structured access"):
         native.ttir_to_structured(compile_ttir(X.gather_rows, sig, {"BLOCK": 64}))
-    sig = {"x_ptr": "*fp32", "y_ptr": "*fp32", "z_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"}
-    s = native.ttir_to_structured(compile_ttir(X.fused_mul_add, sig, {"BLOCK": 256}))
+    sig = {"x_ptr": "*fp32", "out_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"}
+    s = native.ttir_to_structured(compile_ttir(X.block_sum, sig, {"BLOCK": 256}))
     with pytest.raises(NotImplementedError, match="no hand-written kernel family"):
         native.structured_to_plan(s)
     with pytest.raises(NotImplementedError):

@@ -1,0 +1,267 @@
+// Run-time specialisation of a fused elementwise map: the register program that the planner
+// assembled for the interpreter kernel (mapn_isa.h) is printed as straight-line HIP source inside
+// a fixed mover (the load / predicate / store code of the hand-written map kernels) and compiled
+// once per plan with hipRTC, at the first launch -- the point at which the reference compiles
+// its launcher with g++ (backend/driver.py:274-345).  Every instruction becomes the same C
+// expression the interpreter evaluates, with contraction off, so both paths give identical bits.
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <sstream>
+#include <string>
+
+#include "kernels.h"
+
+namespace tts {
+
+namespace {
+
+// the argument block of the generated kernel; its text below must describe the same layout
+struct RtcArgs {
+  const void *in[MAPN_MAX_IN];
+  void *out[MAPN_MAX_OUT];
+  long long in_off[MAPN_MAX_IN][4], out_off[MAPN_MAX_OUT][4], m_start[4];
+  long long bound;
+  int block, masked;
+  float other[MAPN_MAX_IN];
+  float imm[MAPN_MAX_IMM];
+};
+
+const char *PRELUDE = R"SRC(
+struct Args {
+  const void *in[%IN%];
+  void *out[%OUT%];
+  long long in_off[%IN%][4], out_off[%OUT%][4], m_start[4];
+  long long bound;
+  int block, masked;
+  float other[%IN%];
+  float imm[%IMM%];
+};
+static_assert(sizeof(Args) == %SIZE%, "argument block layout");
+constexpr int W = %W%;  // elements per thread and pass: 4, or 8 when every tensor is 16 bits wide (16-byte accesses either way)
+typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef unsigned short hw __attribute__((ext_vector_type(W)));
+__device__ inline long long affine(const long long (&a)[4]) { return a[0] + a[1] * blockIdx.x + a[2] * blockIdx.y + a[3] * blockIdx.z; }
+__device__ inline float up_f16(unsigned short h) { _Float16 f; __builtin_memcpy(&f, &h, 2); return (float)f; }
+__device__ inline unsigned short down_f16(float f) { _Float16 h = (_Float16)f; unsigned short r; __builtin_memcpy(&r, &h, 2); return r; }
+__device__ inline float up_bf16(unsigned short h) { return __uint_as_float((unsigned)h << 16); }
+__device__ inline unsigned short down_bf16(float f) {
+  unsigned u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1);
+  return (unsigned short)(u >> 16);
+}
+__device__ inline float maximum_f(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
+__device__ inline float minimum_f(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
+__device__ inline float as_bool(bool b) { return b ? 1.0f : 0.0f; }
+__device__ inline void load_f32(float (&v)[W], const void *base, int i, int valid, float other) {
+  const float *p = (const float *)base + i;
+  if (valid >= 4) { f4 w = *(const f4 *)p; v[0] = w[0]; v[1] = w[1]; v[2] = w[2]; v[3] = w[3]; return; }
+  for (int e = 0; e < 4; e++) v[e] = e < valid ? p[e] : other;
+}
+template <bool BF16>
+__device__ inline void load_h(float (&v)[W], const void *base, int i, int valid, float other) {
+  const unsigned short *p = (const unsigned short *)base + i;
+  unsigned short h[W];
+  for (int e = 0; e < W; e++) h[e] = 0;
+  if (valid >= W && (((unsigned long long)p) & (2 * W - 1)) == 0) { hw w = *(const hw *)p; for (int e = 0; e < W; e++) h[e] = w[e]; }
+  else for (int e = 0; e < W && e < valid; e++) h[e] = p[e];
+  for (int e = 0; e < W; e++) v[e] = e < valid ? (BF16 ? up_bf16(h[e]) : up_f16(h[e])) : other;
+}
+__device__ inline void store_f32(void *base, int i, int valid, const float (&v)[W]) {
+  float *p = (float *)base + i;
+  if (valid >= 4) { f4 w = {v[0], v[1], v[2], v[3]}; __builtin_nontemporal_store(w, (f4 *)p); return; }
+  for (int e = 0; e < valid; e++) p[e] = v[e];
+}
+template <bool BF16>
+__device__ inline void store_h(void *base, int i, int valid, const float (&v)[W]) {
+  unsigned short *p = (unsigned short *)base + i;
+  hw w;
+  for (int e = 0; e < W; e++) w[e] = BF16 ? down_bf16(v[e]) : down_f16(v[e]);
+  if (valid >= W && (((unsigned long long)p) & (2 * W - 1)) == 0) { __builtin_nontemporal_store(w, (hw *)p); return; }
+  for (int e = 0; e < W && e < valid; e++) p[e] = w[e];
+}
+)SRC";
+
+std::string replace_all(std::string s, const std::string &from, const std::string &to) {
+  for (size_t pos = 0; (pos = s.find(from, pos)) != std::string::npos; pos += to.size()) s.replace(pos, from.size(), to);
+  return s;
+}
+
+std::string expression(int op, const std::string &a, const std::string &b, const std::string &c) {
+  switch (op) {
+    case MO_MOV: return a;
+    case MO_ADD: return a + " + " + b;
+    case MO_SUB: return a + " - " + b;
+    case MO_MUL: return a + " * " + b;
+    case MO_DIV: return a + " / " + b;
+    case MO_MAXNUM: return "fmaxf(" + a + ", " + b + ")";
+    case MO_MINNUM: return "fminf(" + a + ", " + b + ")";
+    case MO_MAXIMUM: return "maximum_f(" + a + ", " + b + ")";
+    case MO_MINIMUM: return "minimum_f(" + a + ", " + b + ")";
+    case MO_NEG: return "-" + a;
+    case MO_ABS: return "fabsf(" + a + ")";
+    case MO_EXP: return "expf(" + a + ")";
+    case MO_EXP2: return "exp2f(" + a + ")";
+    case MO_LOG: return "logf(" + a + ")";
+    case MO_LOG2: return "log2f(" + a + ")";
+    case MO_SQRT: return "sqrtf(" + a + ")";
+    case MO_RSQRT: return "1.0f / sqrtf(" + a + ")";
+    case MO_SIN: return "sinf(" + a + ")";
+    case MO_COS: return "cosf(" + a + ")";
+    case MO_TANH: return "tanhf(" + a + ")";
+    case MO_ERF: return "erff(" + a + ")";
+    case MO_FLOOR: return "floorf(" + a + ")";
+    case MO_CEIL: return "ceilf(" + a + ")";
+    case MO_FMA: return "fmaf(" + a + ", " + b + ", " + c + ")";
+    case MO_SELECT: return a + " != 0.f ? " + b + " : " + c;
+    case MO_AND: return "as_bool(" + a + " != 0.f && " + b + " != 0.f)";
+    case MO_OR: return "as_bool(" + a + " != 0.f || " + b + " != 0.f)";
+    case MO_XOR: return "as_bool((" + a + " != 0.f) != (" + b + " != 0.f))";
+    case MO_CMP_OEQ: return "as_bool(" + a + " == " + b + ")";
+    case MO_CMP_ONE: return "as_bool(" + a + " < " + b + " || " + a + " > " + b + ")";
+    case MO_CMP_OLT: return "as_bool(" + a + " < " + b + ")";
+    case MO_CMP_OLE: return "as_bool(" + a + " <= " + b + ")";
+    case MO_CMP_OGT: return "as_bool(" + a + " > " + b + ")";
+    case MO_CMP_OGE: return "as_bool(" + a + " >= " + b + ")";
+    case MO_CMP_UNE: return "as_bool(!(" + a + " == " + b + "))";
+    case MO_CMP_UEQ: return "as_bool(!(" + a + " < " + b + " || " + a + " > " + b + "))";
+    case MO_CMP_ULT: return "as_bool(!(" + a + " >= " + b + "))";
+    case MO_CMP_ULE: return "as_bool(!(" + a + " > " + b + "))";
+    case MO_CMP_UGT: return "as_bool(!(" + a + " <= " + b + "))";
+    case MO_CMP_UGE: return "as_bool(!(" + a + " < " + b + "))";
+    case MO_CMP_ORD: return "as_bool(" + a + " == " + a + " && " + b + " == " + b + ")";
+    case MO_CMP_UNO: return "as_bool(" + a + " != " + a + " || " + b + " != " + b + ")";
+  }
+  return "0.f";
+}
+
+std::string source_of(const MapNParams &p) {
+  std::string src = PRELUDE;
+  src = replace_all(src, "%IN%", std::to_string(MAPN_MAX_IN));
+  src = replace_all(src, "%OUT%", std::to_string(MAPN_MAX_OUT));
+  src = replace_all(src, "%IMM%", std::to_string(MAPN_MAX_IMM));
+  src = replace_all(src, "%SIZE%", std::to_string(sizeof(RtcArgs)));
+  bool narrow = true;
+  for (int k = 0; k < p.n_in; k++) narrow = narrow && p.in_type[k] != 0;
+  for (int j = 0; j < p.n_out; j++) narrow = narrow && p.out_type[j] != 0;
+  src = replace_all(src, "%W%", narrow ? "8" : "4");
+  std::ostringstream os;
+  os << src;
+  os << "extern \"C\" __global__ __launch_bounds__(256) void fused_map(const Args p) {\n"
+     << "  int d = p.block;\n"
+     << "  if (p.masked) { long long left = p.bound - affine(p.m_start); d = left < 0 ? 0 : left < p.block ? (int)left : p.block; }\n";
+  for (int k = 0; k < p.n_in; k++)
+    os << "  const char *in" << k << " = (const char *)p.in[" << k << "] + affine(p.in_off[" << k << "]) * " << (p.in_type[k] == 0 ? 4 : 2) << ";\n";
+  for (int j = 0; j < p.n_out; j++)
+    os << "  char *out" << j << " = (char *)p.out[" << j << "] + affine(p.out_off[" << j << "]) * " << (p.out_type[j] == 0 ? 4 : 2) << ";\n";
+  os << "  for (int i = W * threadIdx.x; i < d; i += 256 * W) {\n    const int valid = d - i;\n";
+  for (int r = 0; r < p.n_regs; r++) os << "    float r" << r << "[W];\n";
+  os << "    float prev[W];\n    for (int e = 0; e < W; e++) prev[e] = 0.f;\n";
+  for (int k = 0; k < p.n_in; k++) {
+    const char *fn = p.in_type[k] == 0 ? "load_f32" : p.in_type[k] == 1 ? "load_h<false>" : "load_h<true>";
+    os << "    " << fn << "(r" << (int)p.in_reg[k] << ", in" << k << ", i, valid, p.other[" << k << "]);\n";
+  }
+  for (int t = 0; t < p.n_ins; t++) {
+    const MapIns &ins = p.ins[t];
+    auto operand = [&](int kind, int idx) {
+      if (kind == MS_PREV) return std::string("prev[e]");
+      if (kind == MS_IMM) return "p.imm[" + std::to_string(idx) + "]";
+      return "r" + std::to_string(idx) + "[e]";
+    };
+    std::string e = expression(ins.op, operand(ins.kinds & 3, ins.a), operand((ins.kinds >> 2) & 3, ins.b), operand((ins.kinds >> 4) & 3, ins.c));
+    os << "    { float t[W];\n      for (int e = 0; e < W; e++) { float v = " << e << ";";
+    if (ins.round == 1) os << " v = up_f16(down_f16(v));";
+    if (ins.round == 2) os << " v = up_bf16(down_bf16(v));";
+    os << " t[e] = v; }\n      for (int e = 0; e < W; e++) { prev[e] = t[e];";
+    if (!(ins.kinds & 64)) os << " r" << (int)ins.dst << "[e] = t[e];";
+    os << " } }\n";
+  }
+  for (int j = 0; j < p.n_out; j++) {
+    const char *fn = p.out_type[j] == 0 ? "store_f32" : p.out_type[j] == 1 ? "store_h<false>" : "store_h<true>";
+    os << "    " << fn << "(out" << j << ", i, valid, r" << (int)p.out_reg[j] << ");\n";
+  }
+  os << "  }\n}\n";
+  return os.str();
+}
+
+}  // namespace
+
+struct FusedMapModule {
+  hipModule_t module = nullptr;
+  hipFunction_t fn = nullptr;
+  std::string source;
+};
+
+std::string fused_map_source(const MapNParams &p) { return source_of(p); }
+
+hipError_t fused_map_compile(const MapNParams &p, FusedMapModule **out, std::string *err) {
+  auto *m = new FusedMapModule;
+  m->source = source_of(p);
+  hiprtcProgram prog;
+  if (hiprtcCreateProgram(&prog, m->source.c_str(), "fused_map.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
+    *err = "hiprtcCreateProgram failed";
+    delete m;
+    return hipErrorUnknown;
+  }
+  const char *opts[] = {"--offload-arch=gfx950", "-O3", "-ffp-contract=off"};
+  hiprtcResult r = hiprtcCompileProgram(prog, 3, opts);
+  if (r != HIPRTC_SUCCESS) {
+    size_t n = 0;
+    hiprtcGetProgramLogSize(prog, &n);
+    std::string log(n, '\0');
+    if (n) hiprtcGetProgramLog(prog, &log[0]);
+    *err = std::string("hipRTC: ") + hiprtcGetErrorString(r) + "\n" + log;
+    hiprtcDestroyProgram(&prog);
+    delete m;
+    return hipErrorUnknown;
+  }
+  size_t size = 0;
+  hiprtcGetCodeSize(prog, &size);
+  std::string code(size, '\0');
+  hiprtcGetCode(prog, &code[0]);
+  hiprtcDestroyProgram(&prog);
+  hipError_t e = hipModuleLoadData(&m->module, code.data());
+  if (e == hipSuccess) e = hipModuleGetFunction(&m->fn, m->module, "fused_map");
+  if (e != hipSuccess) {
+    *err = std::string("loading the compiled fused map: ") + hipGetErrorString(e);
+    if (m->module) (void)hipModuleUnload(m->module);
+    delete m;
+    return e;
+  }
+  *out = m;
+  return hipSuccess;
+}
+
+void fused_map_release(FusedMapModule *m) {
+  if (!m) return;
+  if (m->module) (void)hipModuleUnload(m->module);
+  delete m;
+}
+
+hipError_t fused_map_launch(FusedMapModule *m, const MapNParams &p, int gx, int gy, int gz, hipStream_t s) {
+  RtcArgs a{};
+  auto put = [](long long (&dst)[4], const Affine &src) {
+    dst[0] = src.c0;
+    for (int i = 0; i < 3; i++) dst[1 + i] = src.c[i];
+  };
+  for (int k = 0; k < p.n_in; k++) {
+    a.in[k] = p.in[k];
+    put(a.in_off[k], p.in_off[k]);
+    a.other[k] = p.in_other[k];
+  }
+  for (int j = 0; j < p.n_out; j++) {
+    a.out[j] = p.out[j];
+    put(a.out_off[j], p.out_off[j]);
+  }
+  put(a.m_start, p.m_start);
+  a.bound = p.bound;
+  a.block = p.block;
+  a.masked = p.masked;
+  for (int q = 0; q < MAPN_MAX_IMM; q++) a.imm[q] = p.imm[q];
+  size_t size = sizeof a;
+  void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &a, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+  return hipModuleLaunchKernel(m->fn, gx, gy, gz, 256, 1, 1, 0, s, nullptr, config);
+}
+
+}  // namespace tts

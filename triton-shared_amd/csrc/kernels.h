@@ -5,6 +5,9 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <string>
+
+#include "mapn_isa.h"
 
 namespace tts {
 
@@ -27,6 +30,34 @@ struct Map1DParams {
   int swap;  // operands of `op` are (y, x)
 };
 hipError_t launch_map1d(const Map1DParams &p, int gx, int gy, int gz, hipStream_t s, const char **kernel_name);
+
+// Fused elementwise map over one-dimensional blocks: out_j[off(p)+i] = f_j(in_0[..+i], ..., scalars), 0 <= i < extent(p).
+// f is a straight-line program over 32-bit registers, one instruction per elementwise op of the
+// Triton kernel (linalg.generic bodies in the reference, TritonArithToLinalg.cpp:104), run by an
+// interpreter inside the kernel.  Narrow float types live in registers as fp32 and are rounded
+// (RTNE) after every op whose Triton result type is narrow, which gives the same values as
+// computing in the narrow type.  i1 values are 0.0f / 1.0f.
+struct MapNParams {
+  const void *in[MAPN_MAX_IN];
+  void *out[MAPN_MAX_OUT];
+  Affine in_off[MAPN_MAX_IN], out_off[MAPN_MAX_OUT], m_start;
+  int64_t bound;
+  int block, masked;
+  int n_in, n_out, n_ins, n_regs;
+  uint8_t in_type[MAPN_MAX_IN], out_type[MAPN_MAX_OUT];  // 0 fp32, 1 fp16, 2 bf16
+  uint8_t in_reg[MAPN_MAX_IN], out_reg[MAPN_MAX_OUT];
+  float in_other[MAPN_MAX_IN];
+  float imm[MAPN_MAX_IMM];
+  MapIns ins[MAPN_MAX_INS];
+};
+hipError_t launch_mapn(const MapNParams &p, int gx, int gy, int gz, hipStream_t s, const char **kernel_name);
+
+// The same register program printed as HIP source and compiled once with hipRTC (fused_rtc.hip).
+struct FusedMapModule;
+hipError_t fused_map_compile(const MapNParams &p, FusedMapModule **out, std::string *err);
+hipError_t fused_map_launch(FusedMapModule *m, const MapNParams &p, int gx, int gy, int gz, hipStream_t s);
+void fused_map_release(FusedMapModule *m);
+std::string fused_map_source(const MapNParams &p);
 
 // out[off_out(p)+i] = softmax(row)[i], i < d_out, where row[i] = i < d_in ? in[off_in(p)+i] : other, i < block
 struct SoftmaxParams {

@@ -420,6 +420,224 @@ hipError_t launch_layernorm_t(const LayerNormParams &p, dim3 grid, hipStream_t s
   return hipGetLastError();
 }
 
+// -------------------------------------------------------------- fused map
+// The interpreter's registers are float4 slots in LDS, one column per lane (a lane only ever
+// touches its own column: no bank conflicts, no barriers), because registers indexed by a
+// run-time number would live in scratch memory.  Fetch and dispatch are scalar: all lanes run
+// the same instruction.
+typedef uint16_t u16x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+
+template <class F>
+__device__ __forceinline__ float4 map4(float4 a, F f) { return make_float4(f(a.x), f(a.y), f(a.z), f(a.w)); }
+template <class F>
+__device__ __forceinline__ float4 map4(float4 a, float4 b, F f) { return make_float4(f(a.x, b.x), f(a.y, b.y), f(a.z, b.z), f(a.w, b.w)); }
+template <class F>
+__device__ __forceinline__ float4 map4(float4 a, float4 b, float4 c, F f) {
+  return make_float4(f(a.x, b.x, c.x), f(a.y, b.y, c.y), f(a.z, b.z, c.z), f(a.w, b.w, c.w));
+}
+__device__ __forceinline__ float as_bool(bool b) { return b ? 1.0f : 0.0f; }
+
+__device__ __forceinline__ float4 mapn_load(const void *base, int type, int i, int valid, float other) {
+  float v[4] = {other, other, other, other};
+  if (type == 0) {
+    const float *p = (const float *)base + i;
+    if (valid >= 4) {
+      f32x4_a4 w = *reinterpret_cast<const f32x4_a4 *>(p);
+      return make_float4(w[0], w[1], w[2], w[3]);
+    }
+    for (int e = 0; e < valid; e++) v[e] = p[e];
+  } else {
+    const uint16_t *p = (const uint16_t *)base + i;
+    uint16_t h[4] = {0, 0, 0, 0};
+    if (valid >= 4) {
+      u16x4_a2 w = *reinterpret_cast<const u16x4_a2 *>(p);
+      h[0] = w[0]; h[1] = w[1]; h[2] = w[2]; h[3] = w[3];
+    } else {
+      for (int e = 0; e < valid; e++) h[e] = p[e];
+    }
+    for (int e = 0; e < 4; e++)
+      if (e < valid) v[e] = type == 1 ? Half<false>::up(h[e]) : Half<true>::up(h[e]);
+  }
+  return make_float4(v[0], v[1], v[2], v[3]);
+}
+
+__device__ __forceinline__ void mapn_store(void *base, int type, int i, int valid, float4 r) {
+  float v[4] = {r.x, r.y, r.z, r.w};
+  if (type == 0) {
+    float *p = (float *)base + i;
+    if (valid >= 4) {
+      f32x4_a4 w = {v[0], v[1], v[2], v[3]};
+      __builtin_nontemporal_store(w, reinterpret_cast<f32x4_a4 *>(p));
+    } else {
+      for (int e = 0; e < valid; e++) p[e] = v[e];
+    }
+  } else {
+    uint16_t *p = (uint16_t *)base + i;
+    uint16_t h[4];
+    for (int e = 0; e < 4; e++) h[e] = type == 1 ? Half<false>::down(v[e]) : Half<true>::down(v[e]);
+    if (valid >= 4) {
+      u16x4_a2 w = {h[0], h[1], h[2], h[3]};
+      __builtin_nontemporal_store(w, reinterpret_cast<u16x4_a2 *>(p));
+    } else {
+      for (int e = 0; e < valid; e++) p[e] = h[e];
+    }
+  }
+}
+
+// One wavefront per program.  A lane owns MAPN_CHUNKS four-element chunks per pass over the block (chunk j
+// starts at element 4 * (lane + 64 j)), so that fetching and dispatching an instruction (a lane read and a
+// tree of scalar compares, about a hundred cycles) is paid once per 1024 elements.
+constexpr int MAPN_CHUNKS = 4, MAPN_PASS = 64 * 4 * MAPN_CHUNKS;
+
+template <class F>
+__device__ __forceinline__ void mapn_apply1(float4 (&r)[MAPN_CHUNKS], const float4 (&a)[MAPN_CHUNKS], F f) {
+#pragma unroll
+  for (int j = 0; j < MAPN_CHUNKS; j++) r[j] = map4(a[j], f);
+}
+template <class F>
+__device__ __forceinline__ void mapn_apply2(float4 (&r)[MAPN_CHUNKS], const float4 (&a)[MAPN_CHUNKS], const float4 (&b)[MAPN_CHUNKS], F f) {
+#pragma unroll
+  for (int j = 0; j < MAPN_CHUNKS; j++) r[j] = map4(a[j], b[j], f);
+}
+template <class F>
+__device__ __forceinline__ void mapn_apply3(float4 (&r)[MAPN_CHUNKS], const float4 (&a)[MAPN_CHUNKS], const float4 (&b)[MAPN_CHUNKS],
+                                            const float4 (&c)[MAPN_CHUNKS], F f) {
+#pragma unroll
+  for (int j = 0; j < MAPN_CHUNKS; j++) r[j] = map4(a[j], b[j], c[j], f);
+}
+
+template <int N_IN>
+__global__ __launch_bounds__(64) void mapn_kernel(MapNParams p) {
+  extern __shared__ float4 mapn_regs[];  // [n_regs][MAPN_CHUNKS][64]
+  const int lane = threadIdx.x;
+  const int px = blockIdx.x, py = blockIdx.y, pz = blockIdx.z;
+  int d = p.block;
+  if (p.masked) {
+    int64_t left = p.bound - affine(p.m_start, px, py, pz);
+    d = left < 0 ? 0 : left < p.block ? (int)left : p.block;
+  }
+  const uint2 my_ins = lane < MAPN_MAX_INS ? reinterpret_cast<const uint2 *>(p.ins)[lane] : make_uint2(0, 0);
+  const uint32_t my_imm = lane < MAPN_MAX_IMM ? __float_as_uint(p.imm[lane]) : 0u;
+  const char *in[N_IN];
+#pragma unroll
+  for (int k = 0; k < N_IN; k++) in[k] = (const char *)p.in[k] + affine(p.in_off[k], px, py, pz) * (p.in_type[k] == 0 ? 4 : 2);
+  auto reg = [&](int r, int j) -> float4 & { return mapn_regs[(r * MAPN_CHUNKS + j) * 64 + lane]; };
+  for (int i0 = 0; i0 < d; i0 += MAPN_PASS) {
+    float4 v[N_IN][MAPN_CHUNKS];
+#pragma unroll
+    for (int k = 0; k < N_IN; k++)
+#pragma unroll
+      for (int j = 0; j < MAPN_CHUNKS; j++) {
+        const int i = i0 + 4 * (lane + 64 * j);
+        v[k][j] = mapn_load(in[k], p.in_type[k], i, d - i, p.in_other[k]);
+      }
+#pragma unroll
+    for (int k = 0; k < N_IN; k++)
+#pragma unroll
+      for (int j = 0; j < MAPN_CHUNKS; j++) reg(p.in_reg[k], j) = v[k][j];
+    float4 prev[MAPN_CHUNKS];
+#pragma unroll
+    for (int j = 0; j < MAPN_CHUNKS; j++) prev[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int t = 0; t < p.n_ins; t++) {
+      // instruction words and immediates sit one per lane in two registers; a lane read makes them scalar
+      const uint32_t w0 = __builtin_amdgcn_readlane(my_ins.x, t), w1 = __builtin_amdgcn_readlane(my_ins.y, t);
+      const int op = w0 & 255, dst = (w0 >> 8) & 255, ia = (w0 >> 16) & 255, ib = w0 >> 24;
+      const int ic = w1 & 255, kinds = (w1 >> 8) & 255, round = (w1 >> 16) & 255;
+      auto fetch = [&](float4 (&o)[MAPN_CHUNKS], int kind, int idx) {
+        if (kind == MS_PREV) {
+#pragma unroll
+          for (int j = 0; j < MAPN_CHUNKS; j++) o[j] = prev[j];
+        } else if (kind == MS_IMM) {
+          float c = __uint_as_float(__builtin_amdgcn_readlane(my_imm, idx));
+#pragma unroll
+          for (int j = 0; j < MAPN_CHUNKS; j++) o[j] = make_float4(c, c, c, c);
+        } else {
+#pragma unroll
+          for (int j = 0; j < MAPN_CHUNKS; j++) o[j] = reg(idx, j);
+        }
+      };
+      float4 a[MAPN_CHUNKS], b[MAPN_CHUNKS], c[MAPN_CHUNKS], r[MAPN_CHUNKS];
+      fetch(a, kinds & 3, ia);
+      const bool unary = op == MO_MOV || (op >= MO_NEG && op <= MO_CEIL);
+      if (!unary) fetch(b, (kinds >> 2) & 3, ib);
+      else
+#pragma unroll
+        for (int j = 0; j < MAPN_CHUNKS; j++) b[j] = a[j];
+      if (op == MO_FMA || op == MO_SELECT) fetch(c, (kinds >> 4) & 3, ic);
+      else
+#pragma unroll
+        for (int j = 0; j < MAPN_CHUNKS; j++) c[j] = a[j];
+#pragma unroll
+      for (int j = 0; j < MAPN_CHUNKS; j++) r[j] = a[j];
+      switch (op) {
+        case MO_MOV: break;
+        case MO_ADD: mapn_apply2(r, a, b, [](float x, float y) { return x + y; }); break;
+        case MO_SUB: mapn_apply2(r, a, b, [](float x, float y) { return x - y; }); break;
+        case MO_MUL: mapn_apply2(r, a, b, [](float x, float y) { return x * y; }); break;
+        case MO_DIV: mapn_apply2(r, a, b, [](float x, float y) { return x / y; }); break;
+        case MO_MAXNUM: mapn_apply2(r, a, b, [](float x, float y) { return fmaxf(x, y); }); break;
+        case MO_MINNUM: mapn_apply2(r, a, b, [](float x, float y) { return fminf(x, y); }); break;
+        case MO_MAXIMUM: mapn_apply2(r, a, b, [](float x, float y) { return apply<4>(x, y); }); break;
+        case MO_MINIMUM: mapn_apply2(r, a, b, [](float x, float y) { return apply<5>(x, y); }); break;
+        case MO_NEG: mapn_apply1(r, a, [](float x) { return -x; }); break;
+        case MO_ABS: mapn_apply1(r, a, [](float x) { return fabsf(x); }); break;
+        case MO_EXP: mapn_apply1(r, a, [](float x) { return expf(x); }); break;
+        case MO_EXP2: mapn_apply1(r, a, [](float x) { return exp2f(x); }); break;
+        case MO_LOG: mapn_apply1(r, a, [](float x) { return logf(x); }); break;
+        case MO_LOG2: mapn_apply1(r, a, [](float x) { return log2f(x); }); break;
+        case MO_SQRT: mapn_apply1(r, a, [](float x) { return sqrtf(x); }); break;
+        case MO_RSQRT: mapn_apply1(r, a, [](float x) { return 1.0f / sqrtf(x); }); break;
+        case MO_SIN: mapn_apply1(r, a, [](float x) { return sinf(x); }); break;
+        case MO_COS: mapn_apply1(r, a, [](float x) { return cosf(x); }); break;
+        case MO_TANH: mapn_apply1(r, a, [](float x) { return tanhf(x); }); break;
+        case MO_ERF: mapn_apply1(r, a, [](float x) { return erff(x); }); break;
+        case MO_FLOOR: mapn_apply1(r, a, [](float x) { return floorf(x); }); break;
+        case MO_CEIL: mapn_apply1(r, a, [](float x) { return ceilf(x); }); break;
+        case MO_FMA: mapn_apply3(r, a, b, c, [](float x, float y, float z) { return fmaf(x, y, z); }); break;
+        case MO_SELECT: mapn_apply3(r, a, b, c, [](float s, float x, float y) { return s != 0.f ? x : y; }); break;
+        case MO_AND: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(x != 0.f && y != 0.f); }); break;
+        case MO_OR: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(x != 0.f || y != 0.f); }); break;
+        case MO_XOR: mapn_apply2(r, a, b, [](float x, float y) { return as_bool((x != 0.f) != (y != 0.f)); }); break;
+        case MO_CMP_OEQ: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(x == y); }); break;
+        case MO_CMP_ONE: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(x < y || x > y); }); break;
+        case MO_CMP_OLT: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(x < y); }); break;
+        case MO_CMP_OLE: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(x <= y); }); break;
+        case MO_CMP_OGT: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(x > y); }); break;
+        case MO_CMP_OGE: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(x >= y); }); break;
+        case MO_CMP_UNE: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(!(x == y)); }); break;
+        case MO_CMP_UEQ: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(!(x < y || x > y)); }); break;
+        case MO_CMP_ULT: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(!(x >= y)); }); break;
+        case MO_CMP_ULE: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(!(x > y)); }); break;
+        case MO_CMP_UGT: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(!(x <= y)); }); break;
+        case MO_CMP_UGE: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(!(x < y)); }); break;
+        case MO_CMP_ORD: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(x == x && y == y); }); break;
+        case MO_CMP_UNO: mapn_apply2(r, a, b, [](float x, float y) { return as_bool(x != x || y != y); }); break;
+      }
+      if (round == 1) mapn_apply1(r, r, [](float x) { return Half<false>::up(Half<false>::down(x)); });
+      else if (round == 2) mapn_apply1(r, r, [](float x) { return Half<true>::up(Half<true>::down(x)); });
+#pragma unroll
+      for (int j = 0; j < MAPN_CHUNKS; j++) prev[j] = r[j];
+      if (!(kinds & 64))
+#pragma unroll
+        for (int j = 0; j < MAPN_CHUNKS; j++) reg(dst, j) = r[j];
+    }
+    for (int o = 0; o < p.n_out; o++) {
+      char *out = (char *)p.out[o] + affine(p.out_off[o], px, py, pz) * (p.out_type[o] == 0 ? 4 : 2);
+#pragma unroll
+      for (int j = 0; j < MAPN_CHUNKS; j++) {
+        const int i = i0 + 4 * (lane + 64 * j);
+        mapn_store(out, p.out_type[o], i, d - i, reg(p.out_reg[o], j));
+      }
+    }
+  }
+}
+
+template <int N_IN>
+hipError_t launch_mapn_n(const MapNParams &p, dim3 grid, hipStream_t s) {
+  hipLaunchKernelGGL((mapn_kernel<N_IN>), grid, dim3(64), (size_t)p.n_regs * MAPN_CHUNKS * 64 * sizeof(float4), s, p);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t launch_map1d(const Map1DParams &p, int gx, int gy, int gz, hipStream_t s, const char **name) {
@@ -432,6 +650,20 @@ hipError_t launch_map1d(const Map1DParams &p, int gx, int gy, int gz, hipStream_
     case 3: return launch_map1d_op<3>(p, grid, s);
     case 4: return launch_map1d_op<4>(p, grid, s);
     case 5: return launch_map1d_op<5>(p, grid, s);
+  }
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_mapn(const MapNParams &p, int gx, int gy, int gz, hipStream_t s, const char **name) {
+  dim3 grid(gx, gy, gz);
+  *name = "mapn_kernel";
+  switch (p.n_in) {
+    case 1: return launch_mapn_n<1>(p, grid, s);
+    case 2: return launch_mapn_n<2>(p, grid, s);
+    case 3: return launch_mapn_n<3>(p, grid, s);
+    case 4: return launch_mapn_n<4>(p, grid, s);
+    case 5: return launch_mapn_n<5>(p, grid, s);
+    case 6: return launch_mapn_n<6>(p, grid, s);
   }
   return hipErrorInvalidValue;
 }

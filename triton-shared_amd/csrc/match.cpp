@@ -1,6 +1,8 @@
 // Family recognition and binding extraction: see match.h.
 #include "match.h"
 
+#include "mapn_isa.h"
+
 #include <functional>
 #include <sstream>
 
@@ -13,6 +15,7 @@ const char *family_name(Family f) {
     case Family::LayerNormFwd: return "layernorm_fwd";
     case Family::Gemm: return "gemm";
     case Family::GemmW8A16: return "gemm_w8a16";
+    case Family::FusedMap: return "fused_map";
   }
   return "?";
 }
@@ -586,11 +589,217 @@ bool try_gemm(Plan &pl, bool w8a16) {
 
 }  // namespace
 
+// ------------------------------------------------------------- fused map
+// Any straight-line program of one-dimensional loads, elementwise ops, constants, splatted scalar
+// arguments and stores over blocks of one size becomes a register program for the interpreter
+// kernel: one instruction per elementwise op (the reference runs one linalg.generic loop per op,
+// TritonArithToLinalg.cpp:104; here they run back to back on values that stay on chip).
+bool try_fused_map(Plan &pl) {
+  Matcher m(pl.prog);
+  const char *F = "fused_map";
+  if (!m.loops.empty() || m.accesses.empty()) return false;
+  std::vector<SOp *> loads, stores;
+  int64_t B = -1;
+  for (SOp *s : m.all) {
+    switch (s->kind) {
+      case SK::Load: loads.push_back(s); break;
+      case SK::Store: stores.push_back(s); break;
+      case SK::Map: case SK::Splat: case SK::Const: case SK::ScalarArg: break;
+      default: return false;
+    }
+    if (s->kind == SK::Load || s->kind == SK::Store) {
+      if (s->acc.sizes.size() != 1) return false;
+      if (B < 0) B = s->acc.sizes[0];
+      if (s->acc.sizes[0] != B) return false;
+    }
+  }
+  if (stores.empty() || B <= 0) return false;
+  for (SOp *s : m.all)
+    if (s->result >= 0) {
+      const Value &v = pl.prog.values[s->result];
+      if (!(v.shape.empty() || (v.shape.size() == 1 && v.shape[0] == B))) return false;
+    }
+  no_wrap(m, F);
+  if ((int)loads.size() > MAPN_MAX_IN) refuse(F, "it has more than " + std::to_string(MAPN_MAX_IN) + " block loads");
+  if (loads.empty()) refuse(F, "it loads nothing");
+  if ((int)stores.size() > MAPN_MAX_OUT) refuse(F, "it has more than " + std::to_string(MAPN_MAX_OUT) + " block stores");
+  auto type_code = [&](const std::string &t) -> int {
+    if (t == "f32") return 0;
+    if (t == "f16") return 1;
+    if (t == "bf16") return 2;
+    refuse(F, "element type " + t + " (fp32, fp16 and bf16 are implemented)");
+  };
+  const std::vector<int> &dims = stores[0]->acc.dims;
+  for (SOp *a : m.accesses) {
+    unit_stride(m, a->acc, F);
+    if (a->acc.dims != dims) refuse(F, "its loads and stores are masked differently");
+  }
+  // liveness: position of the last use of every value
+  std::map<int, size_t> last_use;
+  for (size_t i = 0; i < m.all.size(); i++)
+    for (int v : m.all[i]->operands) last_use[v] = m.all[i]->kind == SK::Store ? SIZE_MAX : std::max(last_use[v], i);
+  // (the kernel stores after the whole program has run, so a stored value keeps its register to the end)
+  static const std::map<std::string, int> ops = {
+      {"arith.addf", MO_ADD}, {"arith.subf", MO_SUB}, {"arith.mulf", MO_MUL}, {"arith.divf", MO_DIV},
+      {"arith.maxnumf", MO_MAXNUM}, {"arith.minnumf", MO_MINNUM}, {"arith.maximumf", MO_MAXIMUM}, {"arith.minimumf", MO_MINIMUM},
+      {"arith.negf", MO_NEG}, {"math.absf", MO_ABS}, {"math.exp", MO_EXP}, {"math.exp2", MO_EXP2}, {"math.log", MO_LOG},
+      {"math.log2", MO_LOG2}, {"math.sqrt", MO_SQRT}, {"math.rsqrt", MO_RSQRT}, {"math.sin", MO_SIN}, {"math.cos", MO_COS},
+      {"math.tanh", MO_TANH}, {"math.erf", MO_ERF}, {"math.floor", MO_FLOOR}, {"math.ceil", MO_CEIL}, {"math.fma", MO_FMA},
+      {"arith.select", MO_SELECT}, {"arith.andi", MO_AND}, {"arith.ori", MO_OR}, {"arith.xori", MO_XOR},
+      {"arith.cmpf.oeq", MO_CMP_OEQ}, {"arith.cmpf.one", MO_CMP_ONE}, {"arith.cmpf.olt", MO_CMP_OLT}, {"arith.cmpf.ole", MO_CMP_OLE},
+      {"arith.cmpf.ogt", MO_CMP_OGT}, {"arith.cmpf.oge", MO_CMP_OGE}, {"arith.cmpf.une", MO_CMP_UNE}, {"arith.cmpf.ueq", MO_CMP_UEQ},
+      {"arith.cmpf.ult", MO_CMP_ULT}, {"arith.cmpf.ule", MO_CMP_ULE}, {"arith.cmpf.ugt", MO_CMP_UGT}, {"arith.cmpf.uge", MO_CMP_UGE},
+      {"arith.cmpf.ord", MO_CMP_ORD}, {"arith.cmpf.uno", MO_CMP_UNO}, {"arith.extf", MO_MOV}, {"arith.truncf", MO_MOV}};
+  // operands: a value lives in a register, is the result of the instruction before, or is an immediate
+  struct Where { int kind = -1, idx = 0; };
+  std::map<int, int> reg_of;          // value -> register
+  std::map<int, int> imm_of;          // value -> immediate index
+  std::map<int, int> scalar_arg_of;   // scalar value -> kernel argument index
+  std::vector<char> busy(MAPN_MAX_REGS, 0);
+  auto alloc = [&]() {
+    for (int r = 0; r < MAPN_MAX_REGS; r++)
+      if (!busy[r]) { busy[r] = 1; return r; }
+    refuse(F, "it keeps more than " + std::to_string(MAPN_MAX_REGS) + " block values alive at once");
+  };
+  // the kernel performs every load before the first instruction, so loaded values get their
+  // registers first; such a register is reused only after its loaded value has died
+  for (SOp *s : loads) reg_of[s->result] = alloc();
+  // positions of the ops that become instructions, and per value the positions that read it
+  std::vector<size_t> map_pos;
+  std::map<int, std::vector<size_t>> readers;
+  for (size_t i = 0; i < m.all.size(); i++) {
+    if (m.all[i]->kind == SK::Map) map_pos.push_back(i);
+    for (int v : m.all[i]->operands) readers[v].push_back(i);
+  }
+  auto next_map_after = [&](size_t pos) -> size_t {
+    for (size_t q : map_pos)
+      if (q > pos) return q;
+    return SIZE_MAX;
+  };
+  int n_ins = 0, n_imm = 0, n_in = 0, n_out = 0, n_regs = (int)loads.size();
+  int prev_value = -1;
+  auto new_imm = [&](double value, int arg) {
+    if (n_imm >= MAPN_MAX_IMM) refuse(F, "it has more than " + std::to_string(MAPN_MAX_IMM) + " constants and scalar arguments");
+    pl.f["imm" + std::to_string(n_imm)] = value;
+    pl.k["imm" + std::to_string(n_imm) + "_arg"] = arg;
+    return n_imm++;
+  };
+  auto round_of = [&](int value) {
+    const std::string &t = pl.prog.values[value].dtype;
+    return t == "f16" ? 1 : t == "bf16" ? 2 : 0;
+  };
+  auto release_dead = [&](size_t pos, const std::vector<int> &operands) {
+    for (int v : operands) {
+      auto it = reg_of.find(v);
+      if (it != reg_of.end() && last_use[v] == pos) busy[it->second] = 0;
+    }
+  };
+  for (size_t i = 0; i < m.all.size(); i++) {
+    SOp *s = m.all[i];
+    switch (s->kind) {
+      case SK::ScalarArg: scalar_arg_of[s->result] = (int)s->ival; break;
+      case SK::Load: {
+        LinIv l;
+        if (!m.linear(s->acc.offsets[0], l)) refuse(F, "a block offset is not linear in the program id");
+        std::string n = "in" + std::to_string(n_in++);
+        pl.lin[n + "_off"] = as_lin(l, s->acc.offsets[0]);
+        pl.k[n + "_arg"] = s->acc.base_arg;
+        pl.k[n + "_type"] = type_code(s->acc.elem);
+        pl.f[n + "_other"] = s->acc.has_other ? s->acc.other_f : 0.0;
+        pl.k[n + "_reg"] = reg_of.at(s->result);
+        if (!last_use.count(s->result)) busy[reg_of.at(s->result)] = 0;
+        break;
+      }
+      case SK::Const: {
+        const Value &v = pl.prog.values[s->result];
+        if (v.dtype[0] == 'i' && v.dtype != "i1") refuse(F, "integer block constants are not implemented");
+        imm_of[s->result] = new_imm(v.dtype == "i1" ? (double)(s->ival != 0) : s->fval, -1);
+        break;
+      }
+      case SK::Splat: {
+        auto it = scalar_arg_of.find(s->operands.at(0));
+        if (it == scalar_arg_of.end()) refuse(F, "it splats something other than a floating-point kernel argument");
+        if (round_of(s->result)) refuse(F, "it splats a scalar argument into a narrow float type");
+        imm_of[s->result] = new_imm(0.0, it->second);
+        break;
+      }
+      case SK::Map: {
+        auto it = ops.find(s->name);
+        if (it == ops.end()) refuse(F, "elementwise op " + s->name + " is not implemented");
+        const Value &rv = pl.prog.values[s->result];
+        if (rv.dtype != "f32" && rv.dtype != "f16" && rv.dtype != "bf16" && rv.dtype != "i1")
+          refuse(F, "elementwise op " + s->name + " on " + rv.dtype + " is not implemented");
+        if (s->operands.size() > 3) refuse(F, "elementwise op " + s->name + " has more than three operands");
+        int src[3] = {0, 0, 0}, kind[3] = {MS_REG, MS_REG, MS_REG};
+        for (size_t q = 0; q < s->operands.size(); q++) {
+          const int v = s->operands[q];
+          const std::string &ot = pl.prog.values[v].dtype;
+          if (ot != "f32" && ot != "f16" && ot != "bf16" && ot != "i1") refuse(F, "elementwise op " + s->name + " on " + ot + " is not implemented");
+          if (imm_of.count(v)) { kind[q] = MS_IMM; src[q] = imm_of[v]; }
+          else if (v == prev_value) { kind[q] = MS_PREV; }
+          else if (reg_of.count(v)) { kind[q] = MS_REG; src[q] = reg_of[v]; }
+          else refuse(F, "an operand of " + s->name + " is not a block value");
+        }
+        release_dead(i, s->operands);  // the result may take the register of an operand that dies here
+        // the result goes to the register file unless its only reader is the next instruction
+        const auto &rd = readers[s->result];
+        const size_t nxt = next_map_after(i);
+        bool only_next = !rd.empty();
+        for (size_t q : rd) only_next = only_next && q == nxt && m.all[q]->kind == SK::Map;
+        int dst = 0;
+        if (!only_next && !rd.empty()) {
+          dst = alloc();
+          reg_of[s->result] = dst;
+          n_regs = std::max(n_regs, dst + 1);
+        }
+        if (n_ins >= MAPN_MAX_INS) refuse(F, "it has more than " + std::to_string(MAPN_MAX_INS) + " elementwise ops");
+        const int kinds = kind[0] | (kind[1] << 2) | (kind[2] << 4) | ((only_next || rd.empty()) ? 64 : 0);
+        pl.k["ins" + std::to_string(n_ins++)] = (int64_t)it->second | ((int64_t)dst << 8) | ((int64_t)src[0] << 16) | ((int64_t)src[1] << 24) |
+                                                ((int64_t)src[2] << 32) | ((int64_t)kinds << 40) | ((int64_t)round_of(s->result) << 48);
+        prev_value = s->result;
+        break;
+      }
+      case SK::Store: {
+        LinIv l;
+        if (!m.linear(s->acc.offsets[0], l)) refuse(F, "a block offset is not linear in the program id");
+        const int v = s->operands.at(0);
+        if (!reg_of.count(v)) refuse(F, "it stores something that is not a computed or loaded block value");
+        if (pl.prog.values[v].dtype != s->acc.elem) refuse(F, "a stored value and its destination differ in type");
+        std::string n = "out" + std::to_string(n_out++);
+        pl.lin[n + "_off"] = as_lin(l, s->acc.offsets[0]);
+        pl.k[n + "_arg"] = s->acc.base_arg;
+        pl.k[n + "_type"] = type_code(s->acc.elem);
+        pl.k[n + "_reg"] = reg_of[v];
+        break;
+      }
+      default: return false;
+    }
+  }
+  pl.family = Family::FusedMap;
+  pl.k["block"] = B;
+  pl.k["n_in"] = n_in;
+  pl.k["n_out"] = n_out;
+  pl.k["n_ins"] = n_ins;
+  pl.k["n_imm"] = n_imm;
+  pl.k["n_regs"] = n_regs;
+  pl.k["masked"] = !dims.empty();
+  if (!dims.empty()) {
+    int start, bound;
+    if (!m.extent(dims[0], B, start, bound)) refuse(F, "its mask is not of the form start+arange < bound");
+    LinIv l;
+    if (!m.linear(start, l)) refuse(F, "its mask start is not linear in the program id");
+    if (!m.pid_free(bound) || !m.loop_free(bound)) refuse(F, "its mask bound depends on the program id");
+    pl.lin["m_start"] = as_lin(l, start);
+    pl.e["bound"] = bound;
+  }
+  return true;
+}
+
 Plan make_plan(Program &&p) {
   Plan pl;
   pl.prog = std::move(p);
   pl.signature = signature(pl.prog);
-  if (try_map1d(pl) || try_softmax(pl) || try_layernorm(pl) || try_gemm(pl, false) || try_gemm(pl, true)) return pl;
+  if (try_map1d(pl) || try_softmax(pl) || try_layernorm(pl) || try_gemm(pl, false) || try_gemm(pl, true) || try_fused_map(pl)) return pl;
   throw Unsupported("no hand-written kernel family matches this structured program; signature: " + pl.signature);
 }
 

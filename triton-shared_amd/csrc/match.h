@@ -14,7 +14,7 @@
 
 namespace tts {
 
-enum class Family { Map1D, RowSoftmax, LayerNormFwd, Gemm, GemmW8A16 };
+enum class Family { Map1D, RowSoftmax, LayerNormFwd, Gemm, GemmW8A16, FusedMap };
 const char *family_name(Family f);
 
 // value(pid) = c0 + cx*pid.x + cy*pid.y + cz*pid.z ; all four are index

@@ -49,6 +49,7 @@ struct Bound {
   LayerNormParams layernorm{};
   GemmParams gemm{};
   GemmW8A16Params w8{};
+  MapNParams mapn{};
   bool empty = false;  // nothing to do (e.g. zero trip count with nothing stored)
   std::string describe;
 };
@@ -66,9 +67,11 @@ struct tts_plan {
   size_t workspace_bytes = 0;
   int *counters = nullptr;     // split-K arrival counters (device), zero between launches
   size_t counters_count = 0;
+  FusedMapModule *fused = nullptr;  // the fused map compiled for this plan (first launch)
   ~tts_plan() {
     if (workspace) (void)hipFree(workspace);
     if (counters) (void)hipFree(counters);
+    fused_map_release(fused);
   }
 };
 
@@ -142,6 +145,56 @@ void bind_map1d(const Resolver &r, Bound &b) {
   os << "kernel=map1d_f32\nop=" << p.op << "\nswap=" << p.swap << "\nblock=" << p.block << "\nmasked=" << p.masked
      << "\nx_off=" << show(p.xo) << "\ny_off=" << show(p.yo) << "\nz_off=" << show(p.zo) << "\nm_start=" << show(p.m_start)
      << "\nbound=" << p.bound << "\n";
+  b.describe = os.str();
+}
+
+void bind_fused_map(const Resolver &r, Bound &b) {
+  MapNParams &p = b.mapn;
+  const auto &k = r.pl.k;
+  p.block = (int)k.at("block");
+  p.masked = (int)k.at("masked");
+  p.n_in = (int)k.at("n_in");
+  p.n_out = (int)k.at("n_out");
+  p.n_ins = (int)k.at("n_ins");
+  p.n_regs = (int)k.at("n_regs");
+  if (p.masked) {
+    p.m_start = r.affine("m_start");
+    p.bound = r.ev0("bound");
+  }
+  std::ostringstream os;
+  os << "kernel=mapn\nblock=" << p.block << "\nmasked=" << p.masked << "\nbound=" << p.bound << "\nm_start=" << show(p.m_start)
+     << "\nregs=" << p.n_regs << "\n";
+  for (int i = 0; i < p.n_in; i++) {
+    std::string n = "in" + std::to_string(i);
+    p.in_off[i] = r.affine(n + "_off");
+    p.in_type[i] = (uint8_t)k.at(n + "_type");
+    p.in_reg[i] = (uint8_t)k.at(n + "_reg");
+    p.in_other[i] = (float)r.pl.f.at(n + "_other");
+    os << n << "_off=" << show(p.in_off[i]) << "\n";
+  }
+  for (int j = 0; j < p.n_out; j++) {
+    std::string n = "out" + std::to_string(j);
+    p.out_off[j] = r.affine(n + "_off");
+    p.out_type[j] = (uint8_t)k.at(n + "_type");
+    p.out_reg[j] = (uint8_t)k.at(n + "_reg");
+    os << n << "_off=" << show(p.out_off[j]) << "\n";
+  }
+  for (int q = 0; q < (int)k.at("n_imm"); q++) {
+    int64_t arg = k.at("imm" + std::to_string(q) + "_arg");
+    p.imm[q] = arg >= 0 ? (float)r.floats.at(arg) : (float)r.pl.f.at("imm" + std::to_string(q));
+  }
+  for (int t = 0; t < p.n_ins; t++) {
+    uint64_t w = (uint64_t)k.at("ins" + std::to_string(t));
+    MapIns &ins = p.ins[t];
+    ins.op = w & 255; ins.dst = (w >> 8) & 255; ins.a = (w >> 16) & 255; ins.b = (w >> 24) & 255;
+    ins.c = (w >> 32) & 255; ins.kinds = (w >> 40) & 255; ins.round = (w >> 48) & 255; ins.pad = 0;
+    auto src = [&](int kind, int idx) {
+      return kind == MS_PREV ? std::string("prev") : kind == MS_IMM ? "#" + std::to_string(p.imm[idx]) : "r" + std::to_string(idx);
+    };
+    os << "ins" << t << "=op" << (int)ins.op << " " << ((ins.kinds & 64) ? std::string("prev") : "r" + std::to_string(ins.dst)) << " <- "
+       << src(ins.kinds & 3, ins.a) << ", " << src((ins.kinds >> 2) & 3, ins.b) << ", " << src((ins.kinds >> 4) & 3, ins.c)
+       << (ins.round ? (ins.round == 1 ? " ->f16" : " ->bf16") : "") << "\n";
+  }
   b.describe = os.str();
 }
 
@@ -291,6 +344,7 @@ std::shared_ptr<Bound> resolve(tts_plan *h, int gx, int gy, int gz, const tts_ar
     case Family::LayerNormFwd: bind_layernorm(r, *b); break;
     case Family::Gemm: bind_gemm(r, *b); break;
     case Family::GemmW8A16: bind_w8a16(r, *b); break;
+    case Family::FusedMap: bind_fused_map(r, *b); break;
   }
   if (h->cache.size() > 256) h->cache.clear();
   h->cache[key] = b;
@@ -407,6 +461,29 @@ tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, cons
         p.y = ptr_arg<const float>(args, pl, "y_arg");
         p.z = ptr_arg<float>(args, pl, "z_arg");
         err = launch_map1d(p, gx, gy, gz, s, &kname);
+        break;
+      }
+      case Family::FusedMap: {
+        MapNParams p = b->mapn;
+        for (int i = 0; i < p.n_in; i++) p.in[i] = ptr_arg<const void>(args, pl, ("in" + std::to_string(i) + "_arg").c_str());
+        for (int j = 0; j < p.n_out; j++) p.out[j] = ptr_arg<void>(args, pl, ("out" + std::to_string(j) + "_arg").c_str());
+        // TTS_FUSED_MAP=interpreter keeps the program on the interpreter kernel; otherwise it is compiled
+        // into a kernel of its own at the plan's first launch (scalar arguments stay arguments: one compile per plan)
+        const char *mode = getenv("TTS_FUSED_MAP");
+        if (mode && std::string(mode) == "interpreter") {
+          err = launch_mapn(p, gx, gy, gz, s, &kname);
+          break;
+        }
+        {
+          std::lock_guard<std::mutex> lock(plan->mu);
+          if (!plan->fused) {
+            std::string why;
+            hipError_t ce = fused_map_compile(p, &plan->fused, &why);
+            if (ce != hipSuccess) return fail(TTS_HIP_ERROR, "fused_map: " + why);
+          }
+        }
+        kname = "fused_map (hipRTC)";
+        err = fused_map_launch(plan->fused, p, gx, gy, gz, s);
         break;
       }
       case Family::RowSoftmax: {

@@ -159,3 +159,36 @@ def w8a16_matmul(a_ptr, w_ptr, s_ptr, c_ptr, M, N, K,
         pw += BK * s_wk
     pc = c_ptr + s_cm * rm[:, None] + s_cn * rn[None, :]
     tl.store(pc, acc.to(tl.float16), mask=(rm[:, None] < M) & (rn[None, :] < N))
+
+
+# ---- fused elementwise maps (one-dimensional blocks; any number of inputs, constants and scalar arguments)
+@triton.jit
+def gelu_tanh_bias(x_ptr, b_ptr, y_ptr, n, BLOCK: tl.constexpr):
+    """y = gelu(x + b), tanh approximation written with exp, on fp32."""
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = i < n
+    x = tl.load(x_ptr + i, mask=m, other=0.0) + tl.load(b_ptr + i, mask=m, other=0.0)
+    u = 0.7978845608028654 * (x + 0.044715 * x * x * x)
+    t = 1.0 - 2.0 / (tl.exp(2.0 * u) + 1.0)
+    tl.store(y_ptr + i, 0.5 * x * (1.0 + t), mask=m)
+
+
+@triton.jit
+def clamp_scale_where(x_ptr, y_ptr, out_ptr, n, lo, hi, alpha, BLOCK: tl.constexpr):
+    """out = where(x > y, alpha * clamp(x, lo, hi), sqrt(|y|)), fp32 with scalar arguments."""
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = i < n
+    x = tl.load(x_ptr + i, mask=m, other=0.0)
+    y = tl.load(y_ptr + i, mask=m, other=0.0)
+    c = tl.minimum(tl.maximum(x, lo), hi)
+    tl.store(out_ptr + i, tl.where(x > y, alpha * c, tl.sqrt(tl.abs(y))), mask=m)
+
+
+@triton.jit
+def silu_mul_f16(g_ptr, u_ptr, out_ptr, n, BLOCK: tl.constexpr):
+    """out = silu(g) * u on fp16 tensors, computed in fp32 (the SwiGLU gate)."""
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = i < n
+    g = tl.load(g_ptr + i, mask=m, other=0.0).to(tl.float32)
+    u = tl.load(u_ptr + i, mask=m, other=0.0).to(tl.float32)
+    tl.store(out_ptr + i, (g / (1.0 + tl.exp(-g)) * u).to(tl.float16), mask=m)
