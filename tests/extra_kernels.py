@@ -18,7 +18,7 @@ def masked_copy_2d(src, dst, rows, cols):
 
 @triton.jit
 def wraparound_rows(src, dst, M, BLOCK: tl.constexpr):
-    # modulo addressing outside a matmul: lowered to a structured access with a period, refused at the plan stage
+    # modulo addressing outside a matmul: a structured access with a period, run by the generic tile-program family
     i = (tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)) % M
     tl.store(dst + tl.arange(0, BLOCK), tl.load(src + i))
 
@@ -55,3 +55,110 @@ def block_sum(x_ptr, out_ptr, n, BLOCK: tl.constexpr):
     i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
     v = tl.load(x_ptr + i, mask=i < n, other=0.0)
     tl.store(out_ptr + tl.program_id(0), tl.sum(v, axis=0))
+
+
+# ---- small tile programs (the shapes of the reference's functional tests in python/examples; the code is ours)
+@triton.jit
+def wrap_rows_loop(a_ptr, c_ptr, M, N, s_am, s_an, s_cm, s_cn, BK: tl.constexpr):
+    # rows 2..5 of A modulo M, two steps of BK columns (test_modulo.py: stacked wraparound)
+    ra = (2 + tl.arange(0, 4)) % M
+    pa = a_ptr + (ra[:, None] * s_am + tl.arange(0, 4)[None, :] * s_an)
+    pc = c_ptr + s_cm * tl.arange(0, 4)[:, None] + s_cn * tl.arange(0, 4)[None, :]
+    for k in range(0, 2):
+        tl.store(pc, tl.load(pa))
+        pa += BK * s_an
+        pc += BK * s_an
+
+
+@triton.jit
+def wrap_cols_row(a_ptr, c_ptr, M, N, s_am, s_an, s_cm, s_cn):
+    # row 7, columns 6..9 modulo N (test_modulo.py: 1-D)
+    ca = (6 + tl.arange(0, 4)) % N
+    tl.store(c_ptr + s_cn * tl.arange(0, 4)[None, :], tl.load(a_ptr + 7 * s_am + ca[None, :] * s_an))
+
+
+@triton.jit
+def wrap_cols_tile(a_ptr, c_ptr, M, N, s_am, s_an, s_cm, s_cn):
+    # rows 2..5, columns 6..9 modulo N (test_modulo.py: side by side)
+    ra = 2 + tl.arange(0, 4)
+    ca = (6 + tl.arange(0, 4)) % N
+    pa = a_ptr + (ra[:, None] * s_am + ca[None, :] * s_an)
+    pc = c_ptr + s_cm * tl.arange(0, 4)[:, None] + s_cn * tl.arange(0, 4)[None, :]
+    tl.store(pc, tl.load(pa))
+
+
+@triton.jit
+def wrap_cols_masked_loop(a_ptr, c_ptr, M, N, s_am, s_an, s_cm, s_cn, BK: tl.constexpr):
+    # as above with a row mask (other = -99) and two steps down the rows (test_modulo.py: masked loop)
+    ra = 2 + tl.arange(0, BK)
+    ca = (6 + tl.arange(0, BK)) % N
+    pa = a_ptr + (ra[:, None] * s_am + ca[None, :] * s_an)
+    rk = tl.arange(0, BK)
+    pc = c_ptr + s_cm * tl.arange(0, BK)[:, None] + s_cn * tl.arange(0, BK)[None, :]
+    for k in range(0, 2):
+        tl.store(pc, tl.load(pa, mask=rk[:, None] < 2, other=-99))
+        pa += BK * s_am
+        pc += BK * s_an
+
+
+@triton.jit
+def masked_gather_const(in0, out0):
+    # every lane masked off: the store writes `other` (test_mask.py)
+    offs = 100 + tl.arange(0, 4)
+    tl.store(out0 + tl.arange(0, 4), tl.load(in0 + offs, mask=offs < 4, other=-1))
+
+
+@triton.jit
+def mask_with_scalar(in0, out0, bound, value):
+    # a scalar condition in conjunction with a lane mask (test_mask.py)
+    offs = tl.arange(0, 8)
+    tl.store(out0 + offs, tl.load(in0 + offs, mask=(value < 5) & (offs < bound), other=-1))
+
+
+@triton.jit
+def swap_blocks(x_ptr, y_ptr, BLOCK: tl.constexpr):
+    # in-place exchange: both loads must complete before either store (test_swap.py)
+    o = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    x = tl.load(x_ptr + o)
+    y = tl.load(y_ptr + o)
+    tl.store(x_ptr + o, y)
+    tl.store(y_ptr + o, x)
+
+
+@triton.jit
+def fill_rows(val, out, s_row, s_col, BC: tl.constexpr):
+    # a splatted scalar argument stored as a 2-row tile (test_splat.py)
+    x = tl.full((2, BC), val, dtype=tl.float32)
+    r = 2 * tl.program_id(0) + tl.arange(0, 2)
+    tl.store(out + (r[:, None] * s_row + tl.arange(0, BC)[None, :] * s_col), x)
+
+
+@triton.jit
+def scalar_walk(in0, out0):
+    # scalar loads and stores through pointers advanced in a loop (test_addptr.py)
+    for i in range(0, 10, 2):
+        p = in0 + 1 + i
+        q = out0 + 1 + i
+        a = tl.load(p)
+        b = tl.load(p + 1)
+        tl.store(q, a)
+        tl.store(q + 1, b)
+
+
+@triton.jit
+def affine_tile_2d(x_ptr, y_ptr, n_rows, n_cols, s0, s1, BR: tl.constexpr, BC: tl.constexpr):
+    # y = 2 x + 1 on a 2-D grid of tiles (test_load_2d_tensor_block.py, with ordinary pointers)
+    r = tl.program_id(0) * BR + tl.arange(0, BR)
+    c = tl.program_id(1) * BC + tl.arange(0, BC)
+    m = (r[:, None] < n_rows) & (c[None, :] < n_cols)
+    x = tl.load(x_ptr + r[:, None] * s0 + c[None, :] * s1, mask=m, other=0.0)
+    tl.store(y_ptr + r[:, None] * s0 + c[None, :] * s1, 2 * x + 1, mask=m)
+
+
+@triton.jit
+def copy_tile_strided(x_ptr, y_ptr, n_rows, n_cols, sx0, sx1, sy0, sy1, BR: tl.constexpr, BC: tl.constexpr):
+    # masked 2-D copy between tensors of unrelated strides (a transposing read when sx1 != 1)
+    r = tl.program_id(0) * BR + tl.arange(0, BR)
+    c = tl.program_id(1) * BC + tl.arange(0, BC)
+    m = (r[:, None] < n_rows) & (c[None, :] < n_cols)
+    tl.store(y_ptr + r[:, None] * sy0 + c[None, :] * sy1, tl.load(x_ptr + r[:, None] * sx0 + c[None, :] * sx1, mask=m), mask=m)

@@ -452,6 +452,97 @@ def test_fused_map_two_ops(K):
     assert torch.equal(zd.cpu(), a * b + a)                              # two roundings, no contraction into an fma
 
 
+# ------------------------------------------------------------- tile programs (generic family)
+# Expected values marked "reference golden" are the literal tensors the reference's own functional tests assert
+# (python/examples/test_modulo.py, test_mask.py); the kernels are ours, written to the same access patterns.
+def _run_wrap(kernel, M, N, *consts, **kw):
+    a = torch.arange(0, M * N, dtype=torch.float32, device=DEV).reshape(M, N)
+    out = torch.full((M, N), 88888.0, device=DEV)
+    k = kernel[(1,)](a, out, M, N, a.stride(0), a.stride(1), out.stride(0), out.stride(1), **kw)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    return out.cpu().int()
+
+
+def test_tile_program_wraparound_reference_goldens():
+    import extra_kernels as X
+    F = 88888
+    got = _run_wrap(X.wrap_rows_loop, 4, 8, BK=4)            # test_modulo.py:53-57 (stacked)
+    assert got.tolist() == [list(range(16, 24)), list(range(24, 32)), list(range(0, 8)), list(range(8, 16))]
+    got = _run_wrap(X.wrap_cols_row, 8, 8)                   # test_modulo.py:91-100 (one row)
+    assert got.tolist() == [[62, 63, 56, 57, F, F, F, F]] + [[F] * 8] * 7
+    got = _run_wrap(X.wrap_cols_tile, 8, 8)                  # test_modulo.py:136-145 (side by side)
+    assert got.tolist() == [[22, 23, 16, 17, F, F, F, F], [30, 31, 24, 25, F, F, F, F], [38, 39, 32, 33, F, F, F, F],
+                            [46, 47, 40, 41, F, F, F, F]] + [[F] * 8] * 4
+    got = _run_wrap(X.wrap_cols_masked_loop, 12, 8, BK=4)    # test_modulo.py:193-206 (mask, other=-99, loop down the rows)
+    assert got.tolist() == [[22, 23, 16, 17, 54, 55, 48, 49], [30, 31, 24, 25, 62, 63, 56, 57], [-99] * 8, [-99] * 8] + [[F] * 8] * 8
+
+
+def test_tile_program_all_masked_load_reference_golden():
+    import extra_kernels as X
+    inp = torch.arange(0, 8, dtype=torch.int32, device=DEV)
+    out = torch.full((8,), -2, dtype=torch.int32, device=DEV)
+    k = X.masked_gather_const[(1,)](inp, out)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program" and k.function.last_kernel == "tile_program (hipRTC)"
+    assert out.cpu().tolist() == [-1, -1, -1, -1, -2, -2, -2, -2]  # test_mask.py:38
+
+
+def test_tile_program_in_place_swap():
+    import extra_kernels as X
+    torch.manual_seed(0)
+    x, y = torch.rand(10240, device=DEV), torch.rand(10240, device=DEV)
+    x0, y0 = x.clone(), y.clone()
+    X.swap_blocks[(10,)](x, y, BLOCK=1024)                    # test_swap.py: both loads before either store
+    torch.cuda.synchronize()
+    assert torch.equal(x, y0) and torch.equal(y, x0)
+
+
+def test_tile_program_splat_scalar_walk_and_2d_tiles():
+    import extra_kernels as X
+    out = torch.empty(256, 512, device=DEV)
+    X.fill_rows[(128,)](123.456, out, out.stride(0), out.stride(1), BC=512)        # test_splat.py
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), torch.full((256, 512), 123.456))
+    inp, o = torch.arange(0, 11, dtype=torch.float32, device=DEV), torch.zeros(11, device=DEV)
+    X.scalar_walk[(1,)](inp, o)                                                    # test_addptr.py
+    torch.cuda.synchronize()
+    assert torch.equal(inp, o)
+    for rows, cols, BR, BC in [(512, 256, 4, 2), (100, 70, 32, 64), (33, 1000, 16, 256)]:
+        x = torch.randn(rows, cols, device=DEV)
+        y = torch.full((rows, cols), -1.0, device=DEV)
+        k = X.affine_tile_2d[(triton.cdiv(rows, BR), triton.cdiv(cols, BC))](x, y, rows, cols, x.stride(0), 1, BR=BR, BC=BC)
+        torch.cuda.synchronize()
+        assert k.function.family == "tile_program"
+        assert torch.equal(y, 2 * x + 1)
+    # different row pitches for input and output are different strides: transposed read
+    x = torch.randn(64, 48, device=DEV)
+    xt = x.t().contiguous().t()                                  # same values, column-major storage
+    y = torch.zeros(64, 48, device=DEV)
+    X.copy_tile_strided[(2, 3)](xt, y, 64, 48, xt.stride(0), xt.stride(1), y.stride(0), y.stride(1), BR=32, BC=16)
+    torch.cuda.synchronize()
+    assert torch.equal(y, x)
+
+
+def test_tile_program_against_lane_interpreter():
+    # random wraparound windows, checked element by element against the lane-level oracle
+    import extra_kernels as X
+    from test_planner import compile_ttir
+    from oracle import ttir_lanes
+    sig = {"a_ptr": "*fp32", "c_ptr": "*fp32", "M": "i32", "N": "i32", "s_am": "i32", "s_an": "i32", "s_cm": "i32", "s_cn": "i32",
+           "BK": "constexpr"}
+    ttir = compile_ttir(X.wrap_cols_masked_loop, sig, {"BK": 4})
+    rng = np.random.default_rng(3)
+    for M, N in [(12, 8), (10, 7), (16, 9)]:
+        a = rng.standard_normal((M, N)).astype(np.float32)
+        ref = np.full((M, 8), 88888.0, np.float32)
+        ttir_lanes.Interpreter(ttir).run((1,), [None, None, M, N, N, 1, 8, 1], {0: a.reshape(-1).copy(), 1: ref.reshape(-1)})
+        ad, od = torch.from_numpy(a).to(DEV), torch.full((M, 8), 88888.0, device=DEV)
+        X.wrap_cols_masked_loop[(1,)](ad, od, M, N, N, 1, 8, 1, BK=4)
+        torch.cuda.synchronize()
+        assert np.array_equal(od.cpu().numpy(), ref.reshape(M, 8))
+
+
 # ------------------------------------------------------------- error paths
 def test_errors_surface_as_python_exceptions(K):
     import extra_kernels as X

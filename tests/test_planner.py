@@ -115,8 +115,8 @@ def test_masked_2d_window_matches_reference_golden(native):
             "dims=[min(128, (max(2, min(130, arg2)) - 2)), min(256, (max(3, min(259, arg3)) - 3))]")
     assert ld == "%src " + want + " other=-inf"
     assert st == "%dst " + want
-    with pytest.raises(NotImplementedError, match="no hand-written kernel family"):
-        native.structured_to_plan(s)
+    plan = native.PlanHandle(native.structured_to_plan(s)[0])
+    assert plan.family == "tile_program"                   # a masked 2-D copy runs on the generic family
 
 
 # ---------------------------------------------------------------- text form
@@ -147,8 +147,7 @@ def test_unsupported_kernels_are_refused(native):
     sig = {"src": "*fp32", "dst": "*fp32", "M": "i32", "BLOCK": "constexpr"}
     wrapped = native.ttir_to_structured(compile_ttir(X.wraparound_rows, sig, {"BLOCK": 64}))
     assert "wraps=[arg2]" in wrapped                       # the structured stage carries the period (tts.make_tptr shape)
-    with pytest.raises(NotImplementedError, match="wraparound"):
-        native.structured_to_plan(wrapped)                 # ... but only the matmul family executes it
+    assert native.PlanHandle(native.structured_to_plan(wrapped)[0]).family == "tile_program"   # ... and the generic family runs it
     sig = {"src": "*fp32", "idx": "*i32", "dst": "*fp32", "BLOCK": "constexpr"}
     with pytest.raises(NotImplementedError, match="not a structured access"):
         native.ttir_to_structured(compile_ttir(X.gather_rows, sig, {"BLOCK": 64}))

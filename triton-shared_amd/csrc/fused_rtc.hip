@@ -187,19 +187,17 @@ std::string source_of(const MapNParams &p) {
 
 }  // namespace
 
-struct FusedMapModule {
+struct RtcModule {
   hipModule_t module = nullptr;
   hipFunction_t fn = nullptr;
-  std::string source;
 };
 
 std::string fused_map_source(const MapNParams &p) { return source_of(p); }
 
-hipError_t fused_map_compile(const MapNParams &p, FusedMapModule **out, std::string *err) {
-  auto *m = new FusedMapModule;
-  m->source = source_of(p);
+hipError_t rtc_compile(const std::string &source, const char *entry, RtcModule **out, std::string *err) {
+  auto *m = new RtcModule;
   hiprtcProgram prog;
-  if (hiprtcCreateProgram(&prog, m->source.c_str(), "fused_map.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
+  if (hiprtcCreateProgram(&prog, source.c_str(), "kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
     *err = "hiprtcCreateProgram failed";
     delete m;
     return hipErrorUnknown;
@@ -222,9 +220,9 @@ hipError_t fused_map_compile(const MapNParams &p, FusedMapModule **out, std::str
   hiprtcGetCode(prog, &code[0]);
   hiprtcDestroyProgram(&prog);
   hipError_t e = hipModuleLoadData(&m->module, code.data());
-  if (e == hipSuccess) e = hipModuleGetFunction(&m->fn, m->module, "fused_map");
+  if (e == hipSuccess) e = hipModuleGetFunction(&m->fn, m->module, entry);
   if (e != hipSuccess) {
-    *err = std::string("loading the compiled fused map: ") + hipGetErrorString(e);
+    *err = std::string("loading the compiled kernel: ") + hipGetErrorString(e);
     if (m->module) (void)hipModuleUnload(m->module);
     delete m;
     return e;
@@ -233,13 +231,20 @@ hipError_t fused_map_compile(const MapNParams &p, FusedMapModule **out, std::str
   return hipSuccess;
 }
 
-void fused_map_release(FusedMapModule *m) {
+void rtc_release(RtcModule *m) {
   if (!m) return;
   if (m->module) (void)hipModuleUnload(m->module);
   delete m;
 }
 
-hipError_t fused_map_launch(FusedMapModule *m, const MapNParams &p, int gx, int gy, int gz, hipStream_t s) {
+hipError_t rtc_launch(RtcModule *m, int gx, int gy, int gz, int block, void *args, size_t size, hipStream_t s) {
+  void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+  return hipModuleLaunchKernel(m->fn, gx, gy, gz, block, 1, 1, 0, s, nullptr, config);
+}
+
+hipError_t fused_map_compile(const MapNParams &p, RtcModule **out, std::string *err) { return rtc_compile(source_of(p), "fused_map", out, err); }
+
+hipError_t fused_map_launch(RtcModule *m, const MapNParams &p, int gx, int gy, int gz, hipStream_t s) {
   RtcArgs a{};
   auto put = [](long long (&dst)[4], const Affine &src) {
     dst[0] = src.c0;
@@ -259,9 +264,7 @@ hipError_t fused_map_launch(FusedMapModule *m, const MapNParams &p, int gx, int 
   a.block = p.block;
   a.masked = p.masked;
   for (int q = 0; q < MAPN_MAX_IMM; q++) a.imm[q] = p.imm[q];
-  size_t size = sizeof a;
-  void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &a, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
-  return hipModuleLaunchKernel(m->fn, gx, gy, gz, 256, 1, 1, 0, s, nullptr, config);
+  return rtc_launch(m, gx, gy, gz, 256, &a, sizeof a, s);
 }
 
 }  // namespace tts

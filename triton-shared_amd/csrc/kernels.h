@@ -52,11 +52,14 @@ struct MapNParams {
 };
 hipError_t launch_mapn(const MapNParams &p, int gx, int gy, int gz, hipStream_t s, const char **kernel_name);
 
-// The same register program printed as HIP source and compiled once with hipRTC (fused_rtc.hip).
-struct FusedMapModule;
-hipError_t fused_map_compile(const MapNParams &p, FusedMapModule **out, std::string *err);
-hipError_t fused_map_launch(FusedMapModule *m, const MapNParams &p, int gx, int gy, int gz, hipStream_t s);
-void fused_map_release(FusedMapModule *m);
+// Kernels compiled at run time with hipRTC (fused_rtc.hip): a compiled module with one entry point.
+struct RtcModule;
+hipError_t rtc_compile(const std::string &source, const char *entry, RtcModule **out, std::string *err);
+hipError_t rtc_launch(RtcModule *m, int gx, int gy, int gz, int block, void *args, size_t size, hipStream_t s);
+void rtc_release(RtcModule *m);
+// The fused map's register program printed as HIP source and compiled once.
+hipError_t fused_map_compile(const MapNParams &p, RtcModule **out, std::string *err);
+hipError_t fused_map_launch(RtcModule *m, const MapNParams &p, int gx, int gy, int gz, hipStream_t s);
 std::string fused_map_source(const MapNParams &p);
 
 // out[off_out(p)+i] = softmax(row)[i], i < d_out, where row[i] = i < d_in ? in[off_in(p)+i] : other, i < block

@@ -16,6 +16,7 @@ const char *family_name(Family f) {
     case Family::Gemm: return "gemm";
     case Family::GemmW8A16: return "gemm_w8a16";
     case Family::FusedMap: return "fused_map";
+    case Family::TileProgram: return "tile_program";
   }
   return "?";
 }
@@ -795,11 +796,30 @@ bool try_fused_map(Plan &pl) {
   return true;
 }
 
+// Anything made of structured loads, elementwise ops and stores that no hand-written family took.
+bool try_tile_program(Plan &pl) {
+  Matcher m(pl.prog);
+  for (SOp *s : m.all)
+    if (s->kind == SK::Reduce || s->kind == SK::Dot) return false;
+  if (m.accesses.empty()) return false;
+  pl.source = tile_program_source(pl.prog);  // throws Unsupported with the reason
+  pl.family = Family::TileProgram;
+  return true;
+}
+
 Plan make_plan(Program &&p) {
   Plan pl;
   pl.prog = std::move(p);
   pl.signature = signature(pl.prog);
-  if (try_map1d(pl) || try_softmax(pl) || try_layernorm(pl) || try_gemm(pl, false) || try_gemm(pl, true) || try_fused_map(pl)) return pl;
+  if (try_map1d(pl) || try_softmax(pl) || try_layernorm(pl) || try_gemm(pl, false) || try_gemm(pl, true)) return pl;
+  try {
+    if (try_fused_map(pl)) return pl;
+  } catch (const Unsupported &) {
+    // what the vectorised one-dimensional map declines (integer data, loads and stores masked differently, ...) the
+    // generic family may still take
+    pl.k.clear(); pl.e.clear(); pl.lin.clear(); pl.f.clear();
+  }
+  if (try_tile_program(pl)) return pl;
   throw Unsupported("no hand-written kernel family matches this structured program; signature: " + pl.signature);
 }
 

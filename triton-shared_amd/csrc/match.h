@@ -14,7 +14,7 @@
 
 namespace tts {
 
-enum class Family { Map1D, RowSoftmax, LayerNormFwd, Gemm, GemmW8A16, FusedMap };
+enum class Family { Map1D, RowSoftmax, LayerNormFwd, Gemm, GemmW8A16, FusedMap, TileProgram };
 const char *family_name(Family f);
 
 // value(pid) = c0 + cx*pid.x + cy*pid.y + cz*pid.z ; all four are index
@@ -33,7 +33,14 @@ struct Plan {
   std::map<std::string, Lin> lin;   // named pid-linear forms
   std::map<std::string, int64_t> k; // named compile-time constants (block sizes, arg indices)
   std::map<std::string, double> f;  // named float constants
+  std::string source;               // TileProgram: the HIP source of the program's kernel
 };
+
+// Generic family: HIP source for a program of structured loads, elementwise ops and stores
+// (tile_codegen.cpp).  Throws Unsupported for anything else.  The kernel's argument block holds
+// every kernel argument by index: { void *ptr[N]; long long ival[N]; float fval[N]; }, N = TILE_MAX_ARGS.
+constexpr int TILE_MAX_ARGS = 32;
+std::string tile_program_source(const Program &p);
 
 // Normalised listing of a program's ops (no shapes, no expression ids).
 std::string signature(const Program &p);

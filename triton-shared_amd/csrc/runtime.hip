@@ -67,11 +67,11 @@ struct tts_plan {
   size_t workspace_bytes = 0;
   int *counters = nullptr;     // split-K arrival counters (device), zero between launches
   size_t counters_count = 0;
-  FusedMapModule *fused = nullptr;  // the fused map compiled for this plan (first launch)
+  RtcModule *fused = nullptr;  // the kernel compiled for this plan at its first launch (fused maps, tile programs)
   ~tts_plan() {
     if (workspace) (void)hipFree(workspace);
     if (counters) (void)hipFree(counters);
-    fused_map_release(fused);
+    rtc_release(fused);
   }
 };
 
@@ -345,6 +345,7 @@ std::shared_ptr<Bound> resolve(tts_plan *h, int gx, int gy, int gz, const tts_ar
     case Family::Gemm: bind_gemm(r, *b); break;
     case Family::GemmW8A16: bind_w8a16(r, *b); break;
     case Family::FusedMap: bind_fused_map(r, *b); break;
+    case Family::TileProgram: b->describe = "kernel=tile_program\n"; break;
   }
   if (h->cache.size() > 256) h->cache.clear();
   h->cache[key] = b;
@@ -484,6 +485,25 @@ tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, cons
         }
         kname = "fused_map (hipRTC)";
         err = fused_map_launch(plan->fused, p, gx, gy, gz, s);
+        break;
+      }
+      case Family::TileProgram: {
+        struct { void *ptr[TILE_MAX_ARGS]; long long ival[TILE_MAX_ARGS]; float fval[TILE_MAX_ARGS]; } a{};
+        for (int i = 0; i < n; i++) {
+          if (args[i].kind == TTS_ARG_PTR) a.ptr[i] = args[i].v.ptr;
+          else if (args[i].kind == TTS_ARG_INT) a.ival[i] = args[i].v.i;
+          else a.fval[i] = (float)args[i].v.f;
+        }
+        {
+          std::lock_guard<std::mutex> lock(plan->mu);
+          if (!plan->fused) {
+            std::string why;
+            hipError_t ce = rtc_compile(pl.source, "tile_program", &plan->fused, &why);
+            if (ce != hipSuccess) return fail(TTS_HIP_ERROR, "tile_program: " + why + "\n--- source ---\n" + pl.source);
+          }
+        }
+        kname = "tile_program (hipRTC)";
+        err = rtc_launch(plan->fused, gx, gy, gz, 256, &a, sizeof a, s);
         break;
       }
       case Family::RowSoftmax: {

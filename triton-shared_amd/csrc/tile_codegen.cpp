@@ -1,0 +1,433 @@
+// Structured program -> HIP source, for programs made of structured loads, elementwise ops and
+// stores (no reductions, no dots): the generic family behind the hand-tuned ones.
+//
+// What the reference does with such a program: one memref copy per load/store
+// (StructuredToMemref.cpp:748-853,1163-1196, wraparound as two chunks :263-487), one
+// linalg.generic loop per elementwise op (TritonArithToLinalg.cpp:104), scf.for around them.
+// Here one workgroup runs one program; a body's tile ops are fused into one loop over the
+// tile's elements (thread t takes elements t, t + 256, ...), index expressions are printed from
+// the expression pool with their i32 / index widths, and the source is compiled with hipRTC at
+// the plan's first launch.
+//
+// Order of memory effects.  The reference finishes every load of a body before the op after it
+// starts.  A fused element loop keeps that order per element only, which differs when a store
+// writes what another element's load reads (an in-place shift).  Tiles of up to 4096 elements are
+// therefore run in two phases -- every load of the body into per-thread registers, a barrier,
+// then ops and stores; larger tiles are fused in one loop and accepted only when no store's base
+// argument is also a load's.
+#include <functional>
+#include <map>
+#include <set>
+#include <sstream>
+
+#include "match.h"
+
+namespace tts {
+
+namespace {
+
+constexpr int64_t TWO_PHASE_MAX = 4096;  // elements; 16 per thread
+
+struct Gen {
+  const Program &P;
+  std::ostringstream os;
+  std::map<int, const SOp *> def;          // value id -> defining op
+  std::map<int, std::string> var;          // value id -> C variable holding it at the current element
+  std::map<int, std::pair<int, int>> tile_arg;  // region value -> (loop, index) : refused
+  int indent = 1;
+
+  explicit Gen(const Program &p) : P(p) {}
+
+  [[noreturn]] void no(const std::string &why) { throw Unsupported("tile_program: " + why); }
+  std::string pad() const { return std::string(2 * indent, ' '); }
+
+  static std::string ctype(const std::string &t) {
+    if (t == "f32" || t == "f16" || t == "bf16") return "float";
+    if (t == "i1") return "bool";
+    if (t == "i8") return "signed char";
+    if (t == "i16") return "short";
+    if (t == "i32") return "int";
+    if (t == "i64") return "long long";
+    throw Unsupported("tile_program: element type " + t);
+  }
+  static std::string memtype(const std::string &t) {
+    if (t == "f32") return "float";
+    if (t == "f16" || t == "bf16") return "unsigned short";
+    return ctype(t);
+  }
+  static bool is_float(const std::string &t) { return t[0] == 'f' || t[0] == 'b'; }
+
+  // ---- index expressions -------------------------------------------------
+  std::string ex(int id) {
+    const Expr &e = P.pool.at(id);
+    auto w = [&](const std::string &s) { return e.bits == 32 ? "(long long)(int)(" + s + ")" : "(" + s + ")"; };
+    auto u = [&](const char *op) {  // wrapping arithmetic through unsigned
+      return e.bits == 32 ? "(long long)(int)((unsigned)" + ex(e.a) + " " + op + " (unsigned)" + ex(e.b) + ")"
+                          : "(long long)((unsigned long long)" + ex(e.a) + " " + op + " (unsigned long long)" + ex(e.b) + ")";
+    };
+    switch (e.k) {
+      case EK::Const: return "(" + std::to_string(e.val) + "LL)";
+      case EK::Arg: return w("p.ival[" + std::to_string(e.a) + "]");
+      case EK::Pid: return std::string("pid") + "xyz"[e.a];
+      case EK::NProg: return std::string("np") + "xyz"[e.a];
+      case EK::IV: return "iv" + std::to_string(e.a);
+      case EK::Iter: return "it" + std::to_string(e.a) + "_" + std::to_string(e.b);
+      case EK::Result: return "res" + std::to_string(e.a) + "_" + std::to_string(e.b);
+      case EK::Add: return u("+");
+      case EK::Sub: return u("-");
+      case EK::Mul: return u("*");
+      case EK::DivS: return w("sdiv(" + ex(e.a) + ", " + ex(e.b) + ")");
+      case EK::RemS: return w("srem(" + ex(e.a) + ", " + ex(e.b) + ")");
+      case EK::MinS: return "smin(" + ex(e.a) + ", " + ex(e.b) + ")";
+      case EK::MaxS: return "smax(" + ex(e.a) + ", " + ex(e.b) + ")";
+      case EK::Sext: return ex(e.a);
+      case EK::Trunc: return "(long long)(int)" + ex(e.a);
+      case EK::CmpSel: {
+        static const char *ps[] = {"<", "<=", ">", ">=", "==", "!="};
+        return "(" + ex(e.a) + " " + ps[e.val] + " " + ex(e.b) + " ? " + ex(e.c) + " : " + ex(e.d) + ")";
+      }
+    }
+    return "0";
+  }
+
+  // ---- shapes ------------------------------------------------------------
+  const Value &val(int v) const { return P.values.at(v); }
+  static int64_t count(const std::vector<int64_t> &s) {
+    int64_t n = 1;
+    for (auto d : s) n *= d;
+    return n;
+  }
+
+  // C expression for element (i0, i1) of value v; rank-1 values use i0, scalars neither
+  std::string at(int v, const std::string &i0, const std::string &i1) {
+    auto it = var.find(v);
+    if (it != var.end()) return it->second;
+    auto d = def.find(v);
+    if (d == def.end()) no("a value that is carried around a loop (only pointers and integers may be)");
+    const SOp &s = *d->second;
+    const Value &V = val(v);
+    auto idx = [&](const std::vector<int64_t> &shape, size_t dim) -> std::string {
+      // index along `dim` of a value of this shape, seen from the enclosing element
+      if (shape[dim] == 1) return "0";
+      return shape.size() == 1 ? i0 : dim == 0 ? i0 : i1;
+    };
+    switch (s.kind) {
+      case SK::ScalarArg: return "p.fval[" + std::to_string(s.ival) + "]";
+      case SK::FromIndex: return "(" + ctype(V.dtype) + ")" + ex(s.expr);
+      case SK::Const:
+        if (is_float(V.dtype)) {
+          std::ostringstream c;
+          c.precision(9);
+          if (s.fval != s.fval) return "__builtin_nanf(\"\")";
+          if (s.fval == 1.0 / 0.0) return "__builtin_inff()";
+          if (s.fval == -1.0 / 0.0) return "(-__builtin_inff())";
+          c << std::hexfloat << (float)s.fval << "f";
+          return "(" + c.str() + ")";
+        }
+        return "(" + ctype(V.dtype) + ")(" + std::to_string(s.ival) + "LL)";
+      case SK::Splat: return at(s.operands.at(0), "0", "0");
+      case SK::Iota: return "(int)(" + std::to_string(s.ival) + " + " + i0 + ")";
+      case SK::ExpandDims: {
+        // operand has one dimension fewer; element (i0, i1) reads the operand at the index of the kept dimension
+        const Value &O = val(s.operands.at(0));
+        if (O.shape.size() != 1 || V.shape.size() != 2) no("expand_dims beyond rank 2");
+        return at(s.operands[0], s.axis == 0 ? i1 : i0, "0");
+      }
+      case SK::Broadcast: {
+        const Value &O = val(s.operands.at(0));
+        if (O.shape.size() != V.shape.size()) no("broadcast that changes the rank");
+        if (O.shape.size() == 1) return at(s.operands[0], O.shape[0] == 1 ? "0" : i0, "0");
+        return at(s.operands[0], O.shape[0] == 1 ? "0" : i0, O.shape[1] == 1 ? "0" : i1);
+      }
+      case SK::Map: {
+        std::vector<std::string> a;
+        for (int o : s.operands) {
+          const Value &O = val(o);
+          if (O.shape.size() == V.shape.size()) {
+            a.push_back(O.shape.size() == 2   ? at(o, idx(O.shape, 0), idx(O.shape, 1))
+                        : O.shape.size() == 1 ? at(o, idx(O.shape, 0), "0")
+                                              : at(o, "0", "0"));
+          } else if (O.shape.empty()) a.push_back(at(o, "0", "0"));
+          else no("an elementwise op whose operands differ in rank");
+        }
+        return "(" + map_expr(s, a) + ")";
+      }
+      default: no("internal: value without an inline form");
+    }
+  }
+
+  std::string rounded(const std::string &dtype, const std::string &e) {
+    if (dtype == "f16") return "up_f16(down_f16(" + e + "))";
+    if (dtype == "bf16") return "up_bf16(down_bf16(" + e + "))";
+    return e;
+  }
+
+  std::string map_expr(const SOp &s, const std::vector<std::string> &a) {
+    const std::string &n = s.name;
+    const std::string &rt = val(s.result).dtype;
+    const std::string ot = s.operands.empty() ? rt : val(s.operands[0]).dtype;
+    auto need = [&](size_t k) { if (a.size() != k) no("elementwise op " + n + " with " + std::to_string(a.size()) + " operands"); };
+    auto fl = [&](const std::string &e) { return rounded(rt, e); };
+    auto wrapi = [&](const char *op) {  // wrapping integer arithmetic in the result type
+      const std::string T = ctype(rt), U = rt == "i64" ? "unsigned long long" : "unsigned";
+      return "(" + T + ")((" + U + ")" + a[0] + " " + op + " (" + U + ")" + a[1] + ")";
+    };
+    static const std::map<std::string, const char *> bin_f = {{"arith.addf", "+"}, {"arith.subf", "-"}, {"arith.mulf", "*"}, {"arith.divf", "/"}};
+    static const std::map<std::string, const char *> fn2 = {{"arith.maxnumf", "fmaxf"}, {"arith.minnumf", "fminf"},
+                                                            {"arith.maximumf", "maximum_f"}, {"arith.minimumf", "minimum_f"}};
+    static const std::map<std::string, const char *> fn1 = {
+        {"math.absf", "fabsf"}, {"math.exp", "expf"}, {"math.exp2", "exp2f"}, {"math.log", "logf"}, {"math.log2", "log2f"},
+        {"math.sqrt", "sqrtf"}, {"math.sin", "sinf"}, {"math.cos", "cosf"}, {"math.tanh", "tanhf"}, {"math.erf", "erff"},
+        {"math.floor", "floorf"}, {"math.ceil", "ceilf"}};
+    static const std::map<std::string, const char *> cmpf = {
+        {"oeq", "A == B"}, {"one", "A < B || A > B"}, {"olt", "A < B"}, {"ole", "A <= B"}, {"ogt", "A > B"}, {"oge", "A >= B"},
+        {"une", "!(A == B)"}, {"ueq", "!(A < B || A > B)"}, {"ult", "!(A >= B)"}, {"ule", "!(A > B)"}, {"ugt", "!(A <= B)"},
+        {"uge", "!(A < B)"}, {"ord", "A == A && B == B"}, {"uno", "A != A || B != B"}};
+    static const std::map<std::string, const char *> cmpi = {{"slt", "<"}, {"sle", "<="}, {"sgt", ">"}, {"sge", ">="}, {"eq", "=="}, {"ne", "!="}};
+    if (bin_f.count(n)) { need(2); return fl(a[0] + " " + bin_f.at(n) + " " + a[1]); }
+    if (fn2.count(n)) { need(2); return fl(std::string(fn2.at(n)) + "(" + a[0] + ", " + a[1] + ")"); }
+    if (fn1.count(n)) { need(1); return fl(std::string(fn1.at(n)) + "(" + a[0] + ")"); }
+    if (n == "arith.negf") { need(1); return "-" + a[0]; }
+    if (n == "math.rsqrt") { need(1); return fl("1.0f / sqrtf(" + a[0] + ")"); }
+    if (n == "math.fma") { need(3); return fl("fmaf(" + a[0] + ", " + a[1] + ", " + a[2] + ")"); }
+    if (n == "arith.select") { need(3); return a[0] + " ? " + a[1] + " : " + a[2]; }
+    if (n == "arith.extf") { need(1); return a[0]; }
+    if (n == "arith.truncf") { need(1); return fl(a[0]); }
+    if (n == "arith.sitofp") { need(1); return fl("(float)" + a[0]); }
+    if (n == "arith.fptosi") { need(1); return "(" + ctype(rt) + ")" + a[0]; }
+    if (n == "arith.extsi" || n == "arith.trunci") { need(1); return "(" + ctype(rt) + ")" + a[0]; }
+    if (n == "arith.extui") { need(1); return ot == "i1" ? "(" + ctype(rt) + ")(" + a[0] + " ? 1 : 0)" : "(" + ctype(rt) + ")(unsigned " + ctype(ot) + ")" + a[0]; }
+    if (n == "arith.addi") { need(2); return rt == "i1" ? a[0] + " != " + a[1] : wrapi("+"); }
+    if (n == "arith.subi") { need(2); return rt == "i1" ? a[0] + " != " + a[1] : wrapi("-"); }
+    if (n == "arith.muli") { need(2); return rt == "i1" ? a[0] + " && " + a[1] : wrapi("*"); }
+    if (n == "arith.divsi") { need(2); return "(" + ctype(rt) + ")sdiv(" + a[0] + ", " + a[1] + ")"; }
+    if (n == "arith.remsi") { need(2); return "(" + ctype(rt) + ")srem(" + a[0] + ", " + a[1] + ")"; }
+    if (n == "arith.minsi") { need(2); return "(" + ctype(rt) + ")smin(" + a[0] + ", " + a[1] + ")"; }
+    if (n == "arith.maxsi") { need(2); return "(" + ctype(rt) + ")smax(" + a[0] + ", " + a[1] + ")"; }
+    if (n == "arith.andi") { need(2); return rt == "i1" ? a[0] + " && " + a[1] : "(" + ctype(rt) + ")(" + a[0] + " & " + a[1] + ")"; }
+    if (n == "arith.ori") { need(2); return rt == "i1" ? a[0] + " || " + a[1] : "(" + ctype(rt) + ")(" + a[0] + " | " + a[1] + ")"; }
+    if (n == "arith.xori") { need(2); return rt == "i1" ? a[0] + " != " + a[1] : "(" + ctype(rt) + ")(" + a[0] + " ^ " + a[1] + ")"; }
+    if (n.rfind("arith.cmpf.", 0) == 0 && cmpf.count(n.substr(11))) {
+      need(2);
+      std::string t = cmpf.at(n.substr(11)), out;
+      for (char c : t) out += c == 'A' ? "(" + a[0] + ")" : c == 'B' ? "(" + a[1] + ")" : std::string(1, c);
+      return out;
+    }
+    if (n.rfind("arith.cmpi.", 0) == 0 && cmpi.count(n.substr(11))) { need(2); return a[0] + " " + cmpi.at(n.substr(11)) + " " + a[1]; }
+    no("elementwise op " + n + " is not implemented");
+  }
+
+  // ---- accesses ----------------------------------------------------------
+  // element offset and validity of an access at (i0, i1); fills `pred` ("" = always)
+  std::string address(const Access &a, const std::string &i0, const std::string &i1, std::string &pred) {
+    std::string sum;
+    pred.clear();
+    for (size_t d = 0; d < a.sizes.size(); d++) {
+      const std::string i = a.sizes.size() == 1 ? i0 : d == 0 ? i0 : i1;
+      std::string term = "(" + ex(a.offsets[d]) + " + " + i + " * " + ex(a.strides[d]) + ")";
+      if (!a.mods.empty() && a.mods[d] >= 0) term = "wrap(" + term + ", " + ex(a.mods[d]) + ")";
+      sum += (d ? " + " : "") + term;
+      if (!a.dims.empty()) pred += std::string(pred.empty() ? "" : " && ") + i + " < " + ex(a.dims[d]);
+    }
+    if (a.sizes.empty()) sum = ex(a.offsets.at(0));
+    return sum;
+  }
+
+  std::string mem_read(const Access &a, const std::string &addr) {
+    const std::string ptr = "((const " + memtype(a.elem) + " *)p.ptr[" + std::to_string(a.base_arg) + "])[" + addr + "]";
+    if (a.elem == "f16") return "up_f16(" + ptr + ")";
+    if (a.elem == "bf16") return "up_bf16(" + ptr + ")";
+    return ptr;
+  }
+  std::string other_of(const Access &a) {
+    if (!a.has_other) return is_float(a.elem) ? "0.f" : "(" + ctype(a.elem) + ")0";
+    if (is_float(a.elem)) {
+      if (a.other_f != a.other_f) return "__builtin_nanf(\"\")";
+      if (a.other_f == 1.0 / 0.0) return "__builtin_inff()";
+      if (a.other_f == -1.0 / 0.0) return "(-__builtin_inff())";
+      std::ostringstream c;
+      c << std::hexfloat << (float)a.other_f << "f";
+      return "(" + c.str() + ")";
+    }
+    return "(" + ctype(a.elem) + ")(" + std::to_string(a.other_i) + "LL)";
+  }
+  void mem_write(const Access &a, const std::string &addr, const std::string &pred, const std::string &value) {
+    std::string v = value;
+    if (a.elem == "f16") v = "down_f16(" + v + ")";
+    if (a.elem == "bf16") v = "down_bf16(" + v + ")";
+    os << pad() << (pred.empty() ? "" : "if (" + pred + ") ") << "((" << memtype(a.elem) << " *)p.ptr[" << a.base_arg << "])[" << addr
+       << "] = " << v << ";\n";
+  }
+
+  // ---- bodies ------------------------------------------------------------
+  void body(const std::vector<SOp> &ops) {
+    for (auto &s : ops)
+      if (s.result >= 0) def[s.result] = &s;
+    // the tile shape of this body: every load, store and stored value must have it
+    std::vector<int64_t> shape;
+    bool have = false;
+    std::set<int> load_bases, store_bases;
+    for (auto &s : ops) {
+      if (s.kind == SK::Load || s.kind == SK::Store) {
+        if (s.acc.sizes.size() > 2 || s.acc.sizes.empty()) no("block accesses of rank " + std::to_string(s.acc.sizes.size()));
+        if (!have) { shape = s.acc.sizes; have = true; }
+        if (s.acc.sizes != shape) no("block accesses of different shapes in one body");
+        (s.kind == SK::Load ? load_bases : store_bases).insert(s.acc.base_arg);
+      }
+    }
+    const int64_t T = have ? count(shape) : 0;
+    bool aliasing = false;
+    for (int b : store_bases) aliasing = aliasing || load_bases.count(b);
+    const bool two_phase = have && T <= TWO_PHASE_MAX;
+    if (have && !two_phase && aliasing)
+      no("a block of more than " + std::to_string(TWO_PHASE_MAX) + " elements is stored to an argument that the same body loads from");
+    const int64_t per_thread = (T + 255) / 256;
+    const std::string i0 = shape.size() == 2 ? "(t / " + std::to_string(shape[1]) + ")" : "t";
+    const std::string i1 = shape.size() == 2 ? "(t % " + std::to_string(shape[1]) + ")" : "0";
+
+    auto emit_load = [&](const SOp &s, const std::string &target) {
+      std::string pred, addr = address(s.acc, i0, i1, pred);
+      os << pad() << target << " = " << (pred.empty() ? mem_read(s.acc, addr) : "(" + pred + ") ? " + mem_read(s.acc, addr) + " : " + other_of(s.acc))
+         << ";\n";
+    };
+
+    // uniform part first in program order is not possible in general (scalars may depend on tiles only through
+    // reductions, which this family does not have), so: scalar loads and stores run where they stand, outside the
+    // element loop; tile ops between them are gathered into element loops.
+    size_t k = 0;
+    while (k < ops.size()) {
+      const SOp &s = ops[k];
+      if (s.kind == SK::For) { loop(s); k++; continue; }
+      if (s.kind == SK::ScalarLoad) {
+        std::string pred, addr = address(s.acc, "0", "0", pred);
+        std::string name = "s" + std::to_string(s.result);
+        os << pad() << "const " << ctype(val(s.result).dtype) << " " << name << " = " << mem_read(s.acc, addr) << ";\n";
+        var[s.result] = name;
+        k++;
+        continue;
+      }
+      if (s.kind == SK::ScalarStore) {
+        std::string pred, addr = address(s.acc, "0", "0", pred);
+        os << pad() << "if (threadIdx.x == 0) {\n";
+        indent++;
+        mem_write(s.acc, addr, "", at(s.operands.at(0), "0", "0"));
+        indent--;
+        os << pad() << "}\n";
+        k++;
+        continue;
+      }
+      if (s.kind == SK::Reduce || s.kind == SK::Dot) no("reductions and dots belong to the hand-written families");
+      // a run of tile ops up to the next loop or scalar access
+      size_t end = k;
+      while (end < ops.size() && ops[end].kind != SK::For && ops[end].kind != SK::ScalarLoad && ops[end].kind != SK::ScalarStore) end++;
+      bool any_access = false;
+      for (size_t q = k; q < end; q++) any_access = any_access || ops[q].kind == SK::Load || ops[q].kind == SK::Store;
+      if (any_access) {
+        if (two_phase) {
+          for (size_t q = k; q < end; q++)
+            if (ops[q].kind == SK::Load)
+              os << pad() << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << per_thread << "];\n";
+          os << pad() << "for (int n = 0; n < " << per_thread << "; n++) {\n";
+          indent++;
+          os << pad() << "const int t = threadIdx.x + 256 * n;\n" << pad() << "if (t >= " << T << ") break;\n";
+          for (size_t q = k; q < end; q++)
+            if (ops[q].kind == SK::Load) emit_load(ops[q], "ld" + std::to_string(ops[q].result) + "[n]");
+          indent--;
+          os << pad() << "}\n" << pad() << "__syncthreads();\n";
+          os << pad() << "for (int n = 0; n < " << per_thread << "; n++) {\n";
+          indent++;
+          os << pad() << "const int t = threadIdx.x + 256 * n;\n" << pad() << "if (t >= " << T << ") break;\n";
+          for (size_t q = k; q < end; q++)
+            if (ops[q].kind == SK::Load) var[ops[q].result] = "ld" + std::to_string(ops[q].result) + "[n]";
+        } else {
+          os << pad() << "for (int t = threadIdx.x; t < " << T << "; t += 256) {\n";
+          indent++;
+          for (size_t q = k; q < end; q++)
+            if (ops[q].kind == SK::Load) {
+              std::string name = "v" + std::to_string(ops[q].result);
+              emit_load(ops[q], "const " + ctype(val(ops[q].result).dtype) + " " + name);
+              var[ops[q].result] = name;
+            }
+        }
+        for (size_t q = k; q < end; q++) {
+          const SOp &o = ops[q];
+          if (o.kind == SK::Map && val(o.result).shape == shape) {  // a full-tile op: name it, later ops reuse it
+            std::string name = "v" + std::to_string(o.result);
+            std::string e = at(o.result, i0, i1);
+            os << pad() << "const " << ctype(val(o.result).dtype) << " " << name << " = " << e << ";\n";
+            var[o.result] = name;
+          } else if (o.kind == SK::Store) {
+            const Value &sv = val(o.operands.at(0));
+            if (sv.shape != shape) no("a stored value whose shape is not the block's");
+            std::string pred, addr = address(o.acc, i0, i1, pred);
+            mem_write(o.acc, addr, pred, at(o.operands[0], i0, i1));
+          }
+        }
+        indent--;
+        os << pad() << "}\n";
+        for (size_t q = k; q < end; q++)
+          if (ops[q].result >= 0 && (ops[q].kind == SK::Load || ops[q].kind == SK::Map)) var.erase(ops[q].result);
+        os << pad() << "__syncthreads();\n";
+      }
+      k = end;
+    }
+  }
+
+  void loop(const SOp &s) {
+    if (!s.tile_args.empty()) no("a loop that carries block values (only pointers and integers may be carried)");
+    const std::string L = std::to_string(s.loop);
+    for (size_t q = 0; q < s.int_iters.size(); q++)
+      os << pad() << "long long it" << L << "_" << q << " = " << ex(s.int_iters[q].init) << ";\n";
+    os << pad() << "for (long long iv" << L << " = " << ex(s.lb) << "; iv" << L << " < " << ex(s.ub) << "; iv" << L << " = (long long)(int)(iv" << L
+       << " + " << ex(s.step) << ")) {\n";
+    indent++;
+    body(s.body);
+    for (size_t q = 0; q < s.int_iters.size(); q++)
+      os << pad() << "const long long nx" << L << "_" << q << " = " << ex(s.int_iters[q].next) << ";\n";
+    for (size_t q = 0; q < s.int_iters.size(); q++) os << pad() << "it" << L << "_" << q << " = nx" << L << "_" << q << ";\n";
+    indent--;
+    os << pad() << "}\n";
+    for (size_t q = 0; q < s.int_iters.size(); q++)
+      os << pad() << "const long long res" << L << "_" << q << " = it" << L << "_" << q << ";\n";
+  }
+};
+
+const char *TILE_PRELUDE = R"SRC(
+struct Args { void *ptr[%N%]; long long ival[%N%]; float fval[%N%]; };
+__device__ inline float up_f16(unsigned short h) { _Float16 f; __builtin_memcpy(&f, &h, 2); return (float)f; }
+__device__ inline unsigned short down_f16(float f) { _Float16 h = (_Float16)f; unsigned short r; __builtin_memcpy(&r, &h, 2); return r; }
+__device__ inline float up_bf16(unsigned short h) { return __uint_as_float((unsigned)h << 16); }
+__device__ inline unsigned short down_bf16(float f) {
+  unsigned u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1);
+  return (unsigned short)(u >> 16);
+}
+__device__ inline float maximum_f(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
+__device__ inline float minimum_f(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
+__device__ inline long long smin(long long a, long long b) { return a < b ? a : b; }
+__device__ inline long long smax(long long a, long long b) { return a > b ? a : b; }
+__device__ inline long long sdiv(long long a, long long b) { return b == 0 ? 0 : a / b; }
+__device__ inline long long srem(long long a, long long b) { return b == 0 ? 0 : a % b; }
+__device__ inline long long wrap(long long x, long long m) { return m > 0 ? ((x % m) + m) % m : x; }
+)SRC";
+
+}  // namespace
+
+std::string tile_program_source(const Program &p) {
+  if ((int)p.arg_names.size() > TILE_MAX_ARGS) throw Unsupported("tile_program: more than " + std::to_string(TILE_MAX_ARGS) + " kernel arguments");
+  Gen g(p);
+  std::string pre = TILE_PRELUDE;
+  const std::string n = std::to_string(TILE_MAX_ARGS);
+  for (size_t pos = 0; (pos = pre.find("%N%", pos)) != std::string::npos;) pre.replace(pos, 3, n);
+  g.os << pre;
+  g.os << "extern \"C\" __global__ __launch_bounds__(256) void tile_program(const Args p) {\n"
+       << "  const long long pidx = blockIdx.x, pidy = blockIdx.y, pidz = blockIdx.z;\n"
+       << "  const long long npx = gridDim.x, npy = gridDim.y, npz = gridDim.z;\n"
+       << "  (void)pidx; (void)pidy; (void)pidz; (void)npx; (void)npy; (void)npz;\n";
+  g.body(p.body);
+  g.os << "}\n";
+  return g.os.str();
+}
+
+}  // namespace tts

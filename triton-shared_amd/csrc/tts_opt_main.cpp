@@ -4,6 +4,7 @@
 //   tts-opt --roundtrip file     -> read the structured text back and print it again
 //   tts-opt --signature file     -> normalised op listing used by the family matcher
 //   tts-opt --plan file          -> matched kernel family and its bindings
+//   tts-opt --source file        -> HIP source of a program of the generic tile_program family
 #include <fstream>
 #include <iostream>
 #include <sstream>
@@ -11,12 +12,13 @@
 #include "match.h"
 
 int main(int argc, char **argv) {
-  bool roundtrip = false, sig = false, plan = false;
+  bool roundtrip = false, sig = false, plan = false, source = false;
   const char *path = nullptr;
   for (int i = 1; i < argc; i++) {
     if (std::string(argv[i]) == "--roundtrip") roundtrip = true;
     else if (std::string(argv[i]) == "--signature") sig = true;
     else if (std::string(argv[i]) == "--plan") plan = true;
+    else if (std::string(argv[i]) == "--source") source = true;
     else path = argv[i];
   }
   if (!path) {
@@ -31,6 +33,10 @@ int main(int argc, char **argv) {
     tts::Program p = tts::lower_ttir(f);
     if (sig) {
       std::cout << tts::signature(p) << "\n";
+      return 0;
+    }
+    if (source) {
+      std::cout << tts::tile_program_source(p);
       return 0;
     }
     if (plan) {
