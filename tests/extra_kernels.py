@@ -162,3 +162,27 @@ def copy_tile_strided(x_ptr, y_ptr, n_rows, n_cols, sx0, sx1, sy0, sy1, BR: tl.c
     c = tl.program_id(1) * BC + tl.arange(0, BC)
     m = (r[:, None] < n_rows) & (c[None, :] < n_cols)
     tl.store(y_ptr + r[:, None] * sy0 + c[None, :] * sy1, tl.load(x_ptr + r[:, None] * sx0 + c[None, :] * sx1, mask=m), mask=m)
+
+
+@triton.jit
+def block_ptr_affine(x_ptr, y_ptr, n_rows, n_cols, s0, s1, BR: tl.constexpr, BC: tl.constexpr):
+    # y = 2 x + 1 through block pointers, boundary-checked on both dimensions (test_load_2d_tensor_block.py)
+    px = tl.make_block_ptr(base=x_ptr, shape=[n_rows, n_cols], strides=[s0, s1],
+                           offsets=[tl.program_id(0) * BR, tl.program_id(1) * BC], block_shape=[BR, BC], order=[1, 0])
+    py = tl.make_block_ptr(base=y_ptr, shape=[n_rows, n_cols], strides=[s0, s1],
+                           offsets=[tl.program_id(0) * BR, tl.program_id(1) * BC], block_shape=[BR, BC], order=[1, 0])
+    x = tl.load(px, boundary_check=(0, 1), padding_option="zero")
+    tl.store(py, 2 * x + 1, boundary_check=(0, 1))
+
+
+@triton.jit
+def block_ptr_row_walk(x_ptr, y_ptr, n_rows, n_cols, s0, BR: tl.constexpr, BC: tl.constexpr):
+    # one program per row block walks the columns with tl.advance
+    px = tl.make_block_ptr(base=x_ptr, shape=[n_rows, n_cols], strides=[s0, 1], offsets=[tl.program_id(0) * BR, 0],
+                           block_shape=[BR, BC], order=[1, 0])
+    py = tl.make_block_ptr(base=y_ptr, shape=[n_rows, n_cols], strides=[s0, 1], offsets=[tl.program_id(0) * BR, 0],
+                           block_shape=[BR, BC], order=[1, 0])
+    for _ in range(0, tl.cdiv(n_cols, BC)):
+        tl.store(py, tl.load(px, boundary_check=(0, 1)) * 0.5, boundary_check=(0, 1))
+        px = tl.advance(px, [0, BC])
+        py = tl.advance(py, [0, BC])

@@ -488,6 +488,35 @@ def test_tile_program_all_masked_load_reference_golden():
     assert out.cpu().tolist() == [-1, -1, -1, -1, -2, -2, -2, -2]  # test_mask.py:38
 
 
+def test_tile_program_scalar_condition_in_mask_reference_goldens():
+    import extra_kernels as X
+    inp = torch.arange(0, 8, dtype=torch.int32, device=DEV)
+    for bound, value, want in [(4, 3, [0, 1, 2, 3, -1, -1, -1, -1]),      # test_mask.py:57-58: the scalar condition holds
+                               (4, 8, [-1] * 8)]:                          # test_mask.py:64-65: it does not
+        out = torch.full((8,), -2, dtype=torch.int32, device=DEV)
+        X.mask_with_scalar[(1,)](inp, out, bound, value)
+        torch.cuda.synchronize()
+        assert out.cpu().tolist() == want
+
+
+def test_tile_program_block_pointers():
+    # tl.make_block_ptr / tl.advance arrive as ordinary pointer arithmetic on i64 tensors with `0 <= i < shape` masks
+    # (the frontend's rewrite_tensor_pointer pass); boundary checks become the per-dimension extents
+    import extra_kernels as X
+    for rows, cols, BR, BC in [(512, 256, 4, 2), (37, 50, 16, 32)]:
+        x = torch.arange(0, rows * cols, dtype=torch.float32, device=DEV).reshape(rows, cols)
+        y = torch.full((rows, cols), -1.0, device=DEV)
+        k = X.block_ptr_affine[(triton.cdiv(rows, BR), triton.cdiv(cols, BC))](x, y, rows, cols, x.stride(0), x.stride(1), BR=BR, BC=BC)
+        torch.cuda.synchronize()
+        assert k.function.family == "tile_program"
+        assert torch.equal(y, 2 * x + 1)                                    # test_load_2d_tensor_block.py's expectation
+    x = torch.randn(21, 100, device=DEV)
+    y = torch.zeros(21, 100, device=DEV)
+    X.block_ptr_row_walk[(triton.cdiv(21, 8),)](x, y, 21, 100, x.stride(0), BR=8, BC=32)
+    torch.cuda.synchronize()
+    assert torch.equal(y, x * 0.5)
+
+
 def test_tile_program_in_place_swap():
     import extra_kernels as X
     torch.manual_seed(0)

@@ -193,6 +193,13 @@ class Lowerer {
         auto pit = preds.find(c.op->words.at(0));
         if (pit == preds.end()) throw Unsupported("scalar cmpi predicate " + c.op->words[0]);
         e = P.pool.cmpsel(pit->second, int_of(c.op->operands[0]), int_of(c.op->operands[1]), opnd(1), opnd(2));
+      } else if (op.name == "arith.cmpi") {  // a scalar condition: 1 or 0
+        static const std::map<std::string, int> preds = {{"slt", 0}, {"sle", 1}, {"sgt", 2}, {"sge", 3}, {"eq", 4}, {"ne", 5}};
+        auto pit = preds.find(op.words.at(0));
+        if (pit == preds.end()) throw Unsupported("scalar cmpi predicate " + op.words[0]);
+        e = P.pool.cmpsel(pit->second, opnd(0), opnd(1), P.pool.constant(1, 32), P.pool.constant(0, 32));
+      } else if (op.name == "arith.andi" && d.type.elem == "i1") {
+        e = P.pool.bin(EK::Mul, opnd(0), opnd(1));
       } else {
         throw Unsupported("scalar integer op " + op.name + " (line " + std::to_string(op.line) + ")");
       }
@@ -374,8 +381,7 @@ class Lowerer {
       return m;
     }
     if (!d.type.is_tensor && d.type.is_int()) {  // :312-324
-      if (d.type.elem == "i1") throw Unsupported("MaskAnalysis: scalar boolean in a mask is not supported");
-      m.scalar = P.pool.to_index(int_of(name));
+      m.scalar = P.pool.to_index(int_of(name));  // an i1 scalar is 1 or 0: see the conjunction below
       return m;
     }
     if (!d.op) throw Unsupported("MaskAnalysis: loop-carried mask operand");
@@ -393,7 +399,15 @@ class Lowerer {
     }
     if (op.name == "arith.andi") {  // :355-453, :269-286
       MaskState l = mask_parse(op.operands[0]), r = mask_parse(op.operands[1]);
-      if (l.scalar >= 0 || r.scalar >= 0) throw Unsupported("MaskAnalysis: conjunction with a scalar condition");
+      if (l.scalar >= 0 && r.scalar >= 0) throw Unsupported("MaskAnalysis: conjunction of two scalar conditions");
+      if (l.scalar >= 0 || r.scalar >= 0) {
+        // a splatted scalar condition keeps the other side's extents when it holds and empties them otherwise
+        // (MaskAnalysis.cpp:269-286, exercised by test_mask.py's scalar-conjunction cases)
+        const MaskState &t = l.scalar >= 0 ? r : l;
+        const int c = l.scalar >= 0 ? l.scalar : r.scalar;
+        for (size_t i = 0; i < t.rank(); i++) m.dims.push_back(P.pool.cmpsel(5, c, c64(0), t.dims[i], c64(0)));
+        return m;
+      }
       if (l.rank() != r.rank()) throw Unsupported("MaskAnalysis: conjunction of different ranks");
       for (size_t i = 0; i < l.rank(); i++) m.dims.push_back(P.pool.bin(EK::MinS, l.dims[i], r.dims[i]));
       return m;
