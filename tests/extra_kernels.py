@@ -186,3 +186,86 @@ def block_ptr_row_walk(x_ptr, y_ptr, n_rows, n_cols, s0, BR: tl.constexpr, BC: t
         tl.store(py, tl.load(px, boundary_check=(0, 1)) * 0.5, boundary_check=(0, 1))
         px = tl.advance(px, [0, BC])
         py = tl.advance(py, [0, BC])
+
+
+# ---- unstructured (gather / scatter) accesses --------------------------------------------
+# The four kernels below compute what python/examples/test_gather_scatter.py's kernels compute
+# (same index arithmetic, written our way), so that the literal tensors that test asserts are
+# the expected outputs.
+@triton.jit
+def gather_div10(src, dst):
+    lane = tl.arange(0, 64)
+    where = lane
+    for step in range(0, 2):
+        where = where // 10 + (step + 5)
+        tl.store(dst + lane + 64 * step, tl.load(src + where))
+        where += 64
+
+
+@triton.jit
+def gather_quarter_masked(src, dst):
+    lane = tl.arange(0, 64)
+    for step in range(0, 2):
+        pick = (lane + 64 * step) // 4
+        got = tl.load(src + pick, mask=pick < 8 + 16 * step)
+        tl.store(dst + lane + 64 * step, got)
+
+
+@triton.jit
+def gather_quarter_masked_other(src, dst):
+    lane = tl.arange(0, 64)
+    limit = 8
+    for step in range(0, 2):
+        pick = (lane + 64 * step) // 4
+        got = tl.load(src + pick, mask=pick < limit, other=-1)
+        tl.store(dst + lane + 64 * step, got)
+        limit += 16
+
+
+@triton.jit
+def gather_div12_masked_store(src, dst):
+    where = tl.arange(0, 64)
+    to = tl.arange(0, 64)
+    for step in range(0, 2):
+        where = where // 12
+        got = tl.load(src + where, mask=where < 64, other=99)
+        tl.store(dst + to, got, mask=to < 77)
+        where += 64
+        to += 64
+
+
+@triton.jit
+def scatter_by_index(src, idx, dst, n, BLOCK: tl.constexpr):
+    # dst[idx[i]] = src[i]
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = i < n
+    tl.store(dst + tl.load(idx + i, mask=m), tl.load(src + i, mask=m), mask=m)
+
+
+@triton.jit
+def select_rows(src, dst, rows, pitch_rows, pitch_src, pitch_dst, period, R: tl.constexpr, C: tl.constexpr):
+    # dst[r, :] = src[rows[r] + r % period, :]  (python/examples/test_index_select.py checks this against
+    # torch.index_select)
+    r = tl.arange(0, R)
+    c = tl.arange(0, C)
+    which = tl.load(rows + r * pitch_rows)
+    tile = tl.load(src + (which[:, None] + r[:, None] % period) * pitch_src + c[None, :])
+    tl.store(dst + r[:, None] * pitch_dst + c[None, :], tile)
+
+
+@triton.jit
+def _move_masked(src, dst, where):
+    # dst[where] = src[where] where where < 32, else 0 (the store is not masked); returns the next offsets
+    tl.store(dst + where, tl.load(src + where, mask=where < 32))
+    return where + 32
+
+
+@triton.jit
+def gather_scatter_nested(src, dst):
+    # python/examples/test_gather_scatter.py's nested-loop case: offsets carried through two loop levels
+    where = tl.arange(0, 32)
+    for i in range(0, 2):
+        where = _move_masked(src, dst, where // 3 + i)
+        for j in range(0, 2):
+            where = _move_masked(src, dst, where // ((i + 1) * (j + 1)) + i)
+        where = _move_masked(src, dst, where // 3 + i)

@@ -592,3 +592,78 @@ def test_plan_handle_is_loaded_once(K):
     h1 = k1.function
     k2 = K.vec_add[(2,)](x, x, x, 2048, BLOCK=1024)
     assert k2 is k1 and k2.function is h1
+
+
+# ------------------------------------------------------------- gathers and scatters (generic family)
+def _gather_case(kernel):
+    # python/examples/test_gather_scatter.py:91-105: 128 int32 inputs 2..129, output preset to -1, one program
+    src = torch.arange(2, 130, dtype=torch.int32, device=DEV)
+    dst = torch.full((128,), -1, dtype=torch.int32, device=DEV)
+    k = kernel[(1,)](src, dst)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    return dst.cpu().tolist()
+
+
+def _runs(*pairs):
+    out = []
+    for value, times in pairs:
+        out += [value] * times
+    return out
+
+
+def test_gather_scatter_reference_goldens():
+    """Expected values are the literal tensors python/examples/test_gather_scatter.py asserts (written here as runs)."""
+    import extra_kernels as X
+    assert _gather_case(X.gather_div10) == _runs(*[(v, 10) for v in range(7, 13)], (13, 4), (14, 10), (15, 54))     # :108-117
+    quarter = lambda fill: _runs(*[(v, 4) for v in range(2, 10)], (fill, 32), *[(v, 4) for v in range(18, 26)], (fill, 32))
+    assert _gather_case(X.gather_quarter_masked) == quarter(0)                                                      # :119-128
+    assert _gather_case(X.gather_quarter_masked_other) == quarter(-1)                                               # :131-140
+    assert _gather_case(X.gather_div12_masked_store) == _runs(*[(v, 12) for v in range(2, 7)], (7, 17), (-1, 51))   # :143-152
+    assert _gather_case(X.gather_scatter_nested) == (                                                               # :155-164
+        list(range(2, 13)) + [-1] * 4 + [17, 18, -1, 20, 21, -1, 23, 24, 25, -1, -1, 28] + [-1] * 5 + [0] * 11 + [-1] * 85)
+
+
+def test_index_select_against_torch():
+    # python/examples/test_index_select.py:67-81: rows picked through an index vector plus a modulo of the row number
+    import extra_kernels as X
+    torch.manual_seed(5)
+    src = torch.randn(16, 16, device=DEV)
+    rows = torch.tensor([1, 3, 5, 7], dtype=torch.int32, device=DEV)
+    for period in (2, 3):
+        dst = torch.empty(4, 16, device=DEV)
+        k = X.select_rows[(1,)](src, dst, rows, rows.stride(0), src.stride(0), dst.stride(0), period, R=4, C=16)
+        torch.cuda.synchronize()
+        assert k.function.family == "tile_program"
+        want = torch.index_select(src, 0, (rows + torch.arange(0, 4, device=DEV, dtype=torch.int32) % period).long())
+        assert torch.equal(dst, want)
+
+
+def test_gather_and_scatter_through_an_index_vector():
+    import extra_kernels as X
+    from oracle import ttir_lanes
+    from test_planner import compile_ttir
+    torch.manual_seed(6)
+    n = 3000
+    src = torch.randn(n, device=DEV)
+    perm = torch.randperm(n, device=DEV).int()
+    # scatter: dst[perm[i]] = src[i]
+    dst = torch.zeros(n, device=DEV)
+    k = X.scatter_by_index[(triton.cdiv(n, 256),)](src, perm, dst, n, BLOCK=256)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    want = torch.zeros(n, device=DEV)
+    want[perm.long()] = src
+    assert torch.equal(dst, want)
+    # ... and the lane-level oracle agrees
+    ttir = compile_ttir(X.scatter_by_index, {"src": "*fp32", "idx": "*i32", "dst": "*fp32", "n": "i32", "BLOCK": "constexpr"}, {"BLOCK": 256})
+    ref = np.zeros(n, dtype=np.float32)
+    ttir_lanes.Interpreter(ttir).run((triton.cdiv(n, 256),), [None, None, None, n], {0: src.cpu().numpy(), 1: perm.cpu().numpy(), 2: ref})
+    assert np.array_equal(ref, dst.cpu().numpy())
+    # gather: dst[i] = src[idx[i]], whole blocks
+    idx = torch.randint(0, n, (1024,), device=DEV, dtype=torch.int32)
+    out = torch.zeros(1024, device=DEV)
+    for b in range(4):
+        X.gather_rows[(1,)](src, idx[b * 256:], out[b * 256:], BLOCK=256)
+    torch.cuda.synchronize()
+    assert torch.equal(out, src[idx.long()])

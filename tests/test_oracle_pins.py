@@ -200,3 +200,32 @@ def test_lanes_fused_maps_against_closed_forms():
     ys = np.array([0.0, np.nan, 2.0, 0.5], np.float32)
     got = _run_lanes("clamp_scale_where", 4, [-0.5, 1.25, 3.0], [xs.copy(), ys.copy()], np.float32)
     assert got[0] == 0.0 and np.isnan(got[1]) and got[2] == np.float32(np.sqrt(2.0)) and got[3] == np.float32(np.sqrt(0.5))
+
+
+def test_lanes_gathers_and_scatters_against_reference_goldens():
+    """The lane interpreter on data-dependent addresses, carried offset blocks and nested loops: the expected outputs are
+    the literal tensors python/examples/test_gather_scatter.py:108-164 asserts (written as runs)."""
+    import extra_kernels as X
+    from test_planner import compile_ttir
+
+    def runs(*pairs):
+        out = []
+        for value, times in pairs:
+            out += [value] * times
+        return out
+
+    quarter = lambda fill: runs(*[(v, 4) for v in range(2, 10)], (fill, 32), *[(v, 4) for v in range(18, 26)], (fill, 32))
+    want = {
+        "gather_div10": runs(*[(v, 10) for v in range(7, 13)], (13, 4), (14, 10), (15, 54)),
+        "gather_quarter_masked": quarter(0),
+        "gather_quarter_masked_other": quarter(-1),
+        "gather_div12_masked_store": runs(*[(v, 12) for v in range(2, 7)], (7, 17), (-1, 51)),
+        "gather_scatter_nested": list(range(2, 13)) + [-1] * 4 + [17, 18, -1, 20, 21, -1, 23, 24, 25, -1, -1, 28] + [-1] * 5 + [0] * 11 + [-1] * 85,
+    }
+    for name, expected in want.items():
+        assert len(expected) == 128
+        ttir = compile_ttir(getattr(X, name), {"src": "*i32", "dst": "*i32"}, {})
+        src = np.arange(2, 130, dtype=np.int32)
+        dst = np.full(128, -1, dtype=np.int32)
+        ttir_lanes.Interpreter(ttir).run((1,), [None, None], {0: src, 1: dst})
+        assert dst.tolist() == expected, name

@@ -149,8 +149,9 @@ def test_unsupported_kernels_are_refused(native):
     assert "wraps=[arg2]" in wrapped                       # the structured stage carries the period (tts.make_tptr shape)
     assert native.PlanHandle(native.structured_to_plan(wrapped)[0]).family == "tile_program"   # ... and the generic family runs it
     sig = {"src": "*fp32", "idx": "*i32", "dst": "*fp32", "BLOCK": "constexpr"}
-    with pytest.raises(NotImplementedError, match="not a structured access"):
-        native.ttir_to_structured(compile_ttir(X.gather_rows, sig, {"BLOCK": 64}))
+    gathered = native.ttir_to_structured(compile_ttir(X.gather_rows, sig, {"BLOCK": 64}))
+    assert "gather=" in gathered                           # data-dependent addresses: an unstructured access
+    assert native.PlanHandle(native.structured_to_plan(gathered)[0]).family == "tile_program"
     sig = {"x_ptr": "*fp32", "out_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"}
     s = native.ttir_to_structured(compile_ttir(X.block_sum, sig, {"BLOCK": 256}))
     with pytest.raises(NotImplementedError, match="no hand-written kernel family"):
@@ -285,3 +286,28 @@ def test_argument_checks(native):
     with pytest.raises(ValueError, match="arguments"):
         plan.describe_launch((1, 1, 1), [0, 0, 0])
     assert plan.describe_launch((0, 1, 1), [0, 0, 0, 5]) == {"kernel": "none"}
+
+
+# ------------------------------------------------------------------ gathers and scatters
+def test_unstructured_accesses_keep_offsets_and_masks_as_data(native):
+    """What PtrAnalysis cannot express stays a tensor of offsets (and a tensor mask) on the access; block values carried
+    around loops, integer ones included, become loop-carried block arguments (StructuredToMemref.cpp:855-993,1034-1157)."""
+    import extra_kernels as X
+    s = native.ttir_to_structured(compile_ttir(X.gather_div12_masked_store, {"src": "*i32", "dst": "*i32"}, {}))
+    loads = [l for l in s.splitlines() if l.strip().startswith("load ")]
+    stores = [l for l in s.splitlines() if l.strip().startswith("store ")]
+    assert len(loads) == 1 and len(stores) == 1
+    assert "gather=" in loads[0] and "maskv=-1" not in loads[0] and "other_i=99" in loads[0]
+    assert "gather=" in stores[0] and "maskv=-1" not in stores[0]
+    assert s.count("tile_iter") == 2
+    plan = native.PlanHandle(native.structured_to_plan(s)[0])
+    assert plan.family == "tile_program"
+    # a structured store next to a gathered load stays structured
+    s = native.ttir_to_structured(compile_ttir(X.gather_div10, {"src": "*i32", "dst": "*i32"}, {}))
+    store = [l for l in s.splitlines() if l.strip().startswith("store ")][0]
+    assert "gather=" not in store and "strides=[1]" in store
+    # a rank-1 index vector feeding a rank-2 gather
+    sig = {"src": "*fp32", "dst": "*fp32", "rows": "*i32", "pitch_rows": "i32", "pitch_src": "i32", "pitch_dst": "i32", "period": "i32",
+           "R": "constexpr", "C": "constexpr"}
+    s = native.ttir_to_structured(compile_ttir(X.select_rows, sig, {"R": 4, "C": 16}))
+    assert native.PlanHandle(native.structured_to_plan(s)[0]).family == "tile_program"

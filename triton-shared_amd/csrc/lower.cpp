@@ -534,10 +534,126 @@ class Lowerer {
     else a.other_i = lit == "true" ? 1 : lit == "false" ? 0 : std::stoll(lit);
   }
 
+  // ---- unstructured addresses: base pointer + scalar offset + a tile of per-element integer offsets
+  struct Scattered { int base = -1, scalar = -1, value = -1; };
+  int widen_to_i64(int v) {
+    if (P.values[v].dtype == "i64") return v;
+    SOp s;
+    s.kind = SK::Map;
+    s.name = "arith.extsi";
+    s.operands = {v};
+    Type t;
+    t.is_tensor = true;
+    t.shape = P.values[v].shape;
+    t.elem = "i64";
+    s.result = new_value(t);
+    cur_->push_back(s);
+    return s.result;
+  }
+  Scattered scattered(const std::string &name) {
+    const Def &d = def(name);
+    Scattered u;
+    if (!d.type.is_tensor) {
+      PtrState st = visit(name);
+      if (st.source < 0) throw Unsupported("pointer without a base argument");
+      u.base = st.source;
+      u.scalar = st.scalar >= 0 ? st.scalar : c64(0);
+      return u;
+    }
+    if (!d.op) throw Unsupported("a tensor of pointers carried around a loop is not a structured access");
+    const Op &op = *d.op;
+    if (op.name == "tt.splat") return scattered(op.operands[0]);
+    if (op.name == "tt.broadcast" || op.name == "tt.expand_dims") {
+      u = scattered(op.operands[0]);
+      if (u.value >= 0) {
+        SOp s;
+        s.kind = op.name == "tt.broadcast" ? SK::Broadcast : SK::ExpandDims;
+        if (s.kind == SK::ExpandDims) s.axis = std::stoi(op.attrs.at("axis"));
+        s.operands = {u.value};
+        Type t;
+        t.is_tensor = true;
+        t.shape = d.type.shape;
+        t.elem = P.values[u.value].dtype;
+        s.result = new_value(t);
+        cur_->push_back(s);
+        u.value = s.result;
+      }
+      return u;
+    }
+    if (op.name == "tt.addptr") {
+      u = scattered(op.operands[0]);
+      const Def &o = def(op.operands[1]);
+      if (!o.type.is_tensor) {
+        u.scalar = P.pool.add_index(u.scalar, int_of(op.operands[1]));
+        return u;
+      }
+      int v = widen_to_i64(data_of(op.operands[1]));
+      if (u.value < 0) {
+        u.value = v;
+      } else {
+        SOp s;
+        s.kind = SK::Map;
+        s.name = "arith.addi";
+        s.operands = {widen_to_i64(u.value), v};
+        Type t;
+        t.is_tensor = true;
+        t.shape = d.type.shape;
+        t.elem = "i64";
+        s.result = new_value(t);
+        cur_->push_back(s);
+        u.value = s.result;
+      }
+      return u;
+    }
+    throw Unsupported("address computed by " + op.name + " (line " + std::to_string(op.line) + ")");
+  }
+  // the access of a load / store whose pointer PtrAnalysis or whose mask MaskAnalysis cannot describe
+  void scattered_access(const Op &op, size_t mask_operand, const Type &elem_type, SOp &s) {
+    Scattered u = scattered(op.operands[0]);
+    if (u.value < 0) throw Unsupported("unstructured access without per-element offsets");
+    s.acc = Access();
+    s.acc.base_arg = u.base;
+    s.acc.elem = elem_type.elem;
+    s.acc.sizes = def(op.operands[0]).type.shape;
+    s.acc.offsets = {u.scalar};
+    s.acc.gather = u.value;
+    s.operands.push_back(u.value);
+    if (op.operands.size() > mask_operand) {
+      s.acc.mask_value = data_of(op.operands[mask_operand]);
+      s.operands.push_back(s.acc.mask_value);
+    }
+  }
+
   void lower_load(const Op &op) {
     const Def &p = def(op.operands[0]);
     Type rt = result_type(op);
     SOp s;
+    if (p.type.is_tensor) {
+      // structured when PtrAnalysis and MaskAnalysis succeed, otherwise a gather (PtrAnalysis.cpp:200-275 marks
+      // such dimensions unstructured and TritonToStructured falls back to make_gather_scatter_tptr)
+      bool structured = true;
+      try {
+        PtrState st = visit(op.operands[0]);
+        s.acc = make_access(st, rt);
+        if (op.operands.size() >= 2) {
+          MaskState m = mask_parse(op.operands[1]);
+          if (m.rank() != st.rank()) throw Unsupported("mask rank differs from pointer rank");
+          s.acc.dims = m.dims;
+        }
+      } catch (const Unsupported &) {
+        structured = false;
+      }
+      if (!structured) {
+        s.kind = SK::Load;
+        scattered_access(op, 1, rt, s);
+        if (op.operands.size() >= 3) scalar_other(op.operands[2], s.acc);
+        s.result = new_value(rt);
+        data_[op.results[0]] = s.result;
+        cur_->push_back(s);
+        return;
+      }
+      s = SOp();
+    }
     PtrState st = visit(op.operands[0]);
     s.acc = make_access(st, rt);
     if (!p.type.is_tensor) {
@@ -560,8 +676,24 @@ class Lowerer {
   void lower_store(const Op &op) {
     const Def &p = def(op.operands[0]);
     SOp s;
-    PtrState st = visit(op.operands[0]);
     Type vt = def(op.operands[1]).type;
+    if (p.type.is_tensor) {
+      bool structured = true;
+      try {
+        PtrState st = visit(op.operands[0]);
+        if (op.operands.size() >= 3 && mask_parse(op.operands[2]).rank() != st.rank()) throw Unsupported("mask rank differs from pointer rank");
+      } catch (const Unsupported &) {
+        structured = false;
+      }
+      if (!structured) {  // a scatter
+        s.kind = SK::Store;
+        s.operands.push_back(data_of(op.operands[1]));
+        scattered_access(op, 2, vt, s);
+        cur_->push_back(s);
+        return;
+      }
+    }
+    PtrState st = visit(op.operands[0]);
     s.acc = make_access(st, vt);
     s.operands.push_back(data_of(op.operands[1]));
     if (!p.type.is_tensor) {
@@ -643,9 +775,10 @@ class Lowerer {
         it.result_expr = P.pool.result(s.loop, (int)c.first_slot, bits);
         s.int_iters.push_back(it);
         int_memo_[op.iter_names[j]] = it.iter_expr;
-      } else if (t.is_tensor && t.is_int()) {
-        throw Unsupported("loop-carried integer tensors are not supported");
       } else {
+        // block values, integer ones included: an address built from a carried integer block is then not a
+        // structured access and is lowered as a gather / scatter
+
         c.kind = 2;
         c.tile_index = (int)s.tile_args.size();
         s.tile_inits.push_back(data_of(op.iter_inits[j]));

@@ -811,6 +811,17 @@ Plan make_plan(Program &&p) {
   Plan pl;
   pl.prog = std::move(p);
   pl.signature = signature(pl.prog);
+  // the hand-written families read their operands through structured accesses only: a program with a gather or a
+  // scatter goes to the generic family
+  bool unstructured = false;
+  {
+    Matcher m(pl.prog);
+    for (SOp *a : m.accesses) unstructured = unstructured || a->acc.gather >= 0;
+  }
+  if (unstructured) {
+    if (try_tile_program(pl)) return pl;
+    throw Unsupported("a program with gathers or scatters that also reduces or multiplies matrices; signature: " + pl.signature);
+  }
   if (try_map1d(pl) || try_softmax(pl) || try_layernorm(pl) || try_gemm(pl, false) || try_gemm(pl, true)) return pl;
   try {
     if (try_fused_map(pl)) return pl;

@@ -57,6 +57,11 @@ struct Access {          // the tts.make_tptr + mask part of a load/store
   std::vector<int> mods;             // per-dim wraparound period (index exprs, in elements, -1 = none); empty = no wraparound:
                                      // dim d at index j contributes (offsets[d] + j * strides[d]) mod mods[d] to the address
                                      // (tts.make_tptr `shape`, TritonStructuredDialect.td:33-121; StructuredToMemref.cpp:263-487)
+  // Unstructured (gather / scatter) access, used when the address is not an affine block: element e is at
+  // base[offsets[0] + value(gather)[e]] and is valid iff value(mask_value)[e] (tts.make_gather_scatter_tptr,
+  // StructuredToMemref.cpp:855-993,1034-1157, restated per element).  sizes is the block shape; strides/dims unused.
+  int gather = -1;                   // value id of the integer offset tile, or -1 for a structured access
+  int mask_value = -1;               // value id of the i1 mask tile, or -1
   bool has_other = false;
   double other_f = 0;                // value of `other` when the element type is a float
   int64_t other_i = 0;               // ... when it is an integer

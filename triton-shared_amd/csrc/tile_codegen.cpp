@@ -35,6 +35,8 @@ struct Gen {
   std::map<int, std::string> var;          // value id -> C variable holding it at the current element
   std::map<int, std::pair<int, int>> tile_arg;  // region value -> (loop, index) : refused
   int indent = 1;
+  std::set<int> all_inline_bases, all_store_bases;  // checked against each other at the end
+  std::map<int, std::string> carried;               // region value of a loop-carried tile -> its per-thread array
 
   explicit Gen(const Program &p) : P(p) {}
 
@@ -103,7 +105,7 @@ struct Gen {
     auto it = var.find(v);
     if (it != var.end()) return it->second;
     auto d = def.find(v);
-    if (d == def.end()) no("a value that is carried around a loop (only pointers and integers may be)");
+    if (d == def.end()) no("internal: use of an undefined value");
     const SOp &s = *d->second;
     const Value &V = val(v);
     auto idx = [&](const std::vector<int64_t> &shape, size_t dim) -> std::string {
@@ -139,6 +141,15 @@ struct Gen {
         if (O.shape.size() == 1) return at(s.operands[0], O.shape[0] == 1 ? "0" : i0, "0");
         return at(s.operands[0], O.shape[0] == 1 ? "0" : i0, O.shape[1] == 1 ? "0" : i1);
       }
+      case SK::Load: {
+        // a load that is not of the body's block shape (an index vector, a row of scales) is read where it is used;
+        // body() has checked that nothing in the program stores to its base
+        all_inline_bases.insert(s.acc.base_arg);
+        std::string pred, addr = address(s.acc, i0, i1, pred);
+        const std::string rd = mem_read(s.acc, addr);
+        return "(" + (pred.empty() ? rd : "(" + pred + ") ? " + rd + " : " + other_of(s.acc)) + ")";
+      }
+      case SK::ScalarLoad: no("internal: scalar load without a variable");
       case SK::Map: {
         std::vector<std::string> a;
         for (int o : s.operands) {
@@ -222,6 +233,10 @@ struct Gen {
   std::string address(const Access &a, const std::string &i0, const std::string &i1, std::string &pred) {
     std::string sum;
     pred.clear();
+    if (a.gather >= 0) {  // per-element offsets and mask are data
+      if (a.mask_value >= 0) pred = at(a.mask_value, i0, i1);
+      return ex(a.offsets.at(0)) + " + (long long)" + at(a.gather, i0, i1);
+    }
     for (size_t d = 0; d < a.sizes.size(); d++) {
       const std::string i = a.sizes.size() == 1 ? i0 : d == 0 ? i0 : i1;
       std::string term = "(" + ex(a.offsets[d]) + " + " + i + " * " + ex(a.strides[d]) + ")";
@@ -263,18 +278,33 @@ struct Gen {
   void body(const std::vector<SOp> &ops) {
     for (auto &s : ops)
       if (s.result >= 0) def[s.result] = &s;
-    // the tile shape of this body: every load, store and stored value must have it
+    // the block shape of this body: that of its stores (or, without stores, of its largest load); loads of other
+    // shapes are read where they are used
     std::vector<int64_t> shape;
     bool have = false;
     std::set<int> load_bases, store_bases;
-    for (auto &s : ops) {
-      if (s.kind == SK::Load || s.kind == SK::Store) {
+    for (auto &s : ops)
+      if (s.kind == SK::Store) {
         if (s.acc.sizes.size() > 2 || s.acc.sizes.empty()) no("block accesses of rank " + std::to_string(s.acc.sizes.size()));
         if (!have) { shape = s.acc.sizes; have = true; }
-        if (s.acc.sizes != shape) no("block accesses of different shapes in one body");
-        (s.kind == SK::Load ? load_bases : store_bases).insert(s.acc.base_arg);
+        if (s.acc.sizes != shape) no("block stores of different shapes in one body");
+        store_bases.insert(s.acc.base_arg);
       }
-    }
+    for (auto &s : ops)
+      if (s.kind == SK::Load) {
+        if (s.acc.sizes.size() > 2 || s.acc.sizes.empty()) no("block accesses of rank " + std::to_string(s.acc.sizes.size()));
+        if (!have || (store_bases.empty() && count(s.acc.sizes) > count(shape))) { shape = s.acc.sizes; have = true; }
+      }
+    auto inlined = [&](const SOp &s) { return s.kind == SK::Load && s.acc.sizes != shape; };
+    for (auto &s : ops)
+      if (s.kind == SK::Load) {
+        if (inlined(s)) all_inline_bases.insert(s.acc.base_arg);
+        else load_bases.insert(s.acc.base_arg);
+      }
+    for (int b : store_bases) all_store_bases.insert(b);
+    if (have)  // a carried value is held by the thread that owns the element: only right when the shapes agree
+      for (auto &cv : carried)
+        if (val(cv.first).shape != shape) no("a loop-carried block value used in a body of another block shape");
     const int64_t T = have ? count(shape) : 0;
     bool aliasing = false;
     for (int b : store_bases) aliasing = aliasing || load_bases.count(b);
@@ -325,25 +355,31 @@ struct Gen {
       if (any_access) {
         if (two_phase) {
           for (size_t q = k; q < end; q++)
-            if (ops[q].kind == SK::Load)
+            if (ops[q].kind == SK::Load && !inlined(ops[q]))
               os << pad() << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << per_thread << "];\n";
           os << pad() << "for (int n = 0; n < " << per_thread << "; n++) {\n";
           indent++;
           os << pad() << "const int t = threadIdx.x + 256 * n;\n" << pad() << "if (t >= " << T << ") break;\n";
+          for (auto &cv : carried) var[cv.first] = cv.second + "[n]";
           for (size_t q = k; q < end; q++)
-            if (ops[q].kind == SK::Load) emit_load(ops[q], "ld" + std::to_string(ops[q].result) + "[n]");
+            if (ops[q].kind == SK::Load && !inlined(ops[q])) {
+              emit_load(ops[q], "ld" + std::to_string(ops[q].result) + "[n]");
+              var[ops[q].result] = "ld" + std::to_string(ops[q].result) + "[n]";  // a later load may be indexed by it
+            }
           indent--;
           os << pad() << "}\n" << pad() << "__syncthreads();\n";
           os << pad() << "for (int n = 0; n < " << per_thread << "; n++) {\n";
           indent++;
           os << pad() << "const int t = threadIdx.x + 256 * n;\n" << pad() << "if (t >= " << T << ") break;\n";
           for (size_t q = k; q < end; q++)
-            if (ops[q].kind == SK::Load) var[ops[q].result] = "ld" + std::to_string(ops[q].result) + "[n]";
+            if (ops[q].kind == SK::Load && !inlined(ops[q])) var[ops[q].result] = "ld" + std::to_string(ops[q].result) + "[n]";
+          for (auto &cv : carried) var[cv.first] = cv.second + "[n]";
         } else {
           os << pad() << "for (int t = threadIdx.x; t < " << T << "; t += 256) {\n";
           indent++;
+          if (!carried.empty()) no("a loop that carries block values over blocks of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
           for (size_t q = k; q < end; q++)
-            if (ops[q].kind == SK::Load) {
+            if (ops[q].kind == SK::Load && !inlined(ops[q])) {
               std::string name = "v" + std::to_string(ops[q].result);
               emit_load(ops[q], "const " + ctype(val(ops[q].result).dtype) + " " + name);
               var[ops[q].result] = name;
@@ -374,14 +410,53 @@ struct Gen {
   }
 
   void loop(const SOp &s) {
-    if (!s.tile_args.empty()) no("a loop that carries block values (only pointers and integers may be carried)");
     const std::string L = std::to_string(s.loop);
+    // loop-carried block values live in per-thread arrays (element-wise programs never move a value between
+    // elements, so each thread carries the elements it owns); all of them must have one shape of <= 4096 elements
+    std::vector<int64_t> cshape;
+    for (size_t q = 0; q < s.tile_args.size(); q++) {
+      const Value &V = val(s.tile_args[q]);
+      if (V.shape.empty() || V.shape.size() > 2) no("a loop-carried value of rank " + std::to_string(V.shape.size()));
+      if (q == 0) cshape = V.shape;
+      if (V.shape != cshape) no("loop-carried block values of different shapes");
+    }
+    const int64_t CT = s.tile_args.empty() ? 0 : count(cshape);
+    if (CT > TWO_PHASE_MAX) no("a loop-carried block value of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
+    const int64_t cper = (CT + 255) / 256;
+    const std::string ci0 = cshape.size() == 2 ? "(t / " + std::to_string(cshape[1]) + ")" : "t";
+    const std::string ci1 = cshape.size() == 2 ? "(t % " + std::to_string(cshape[1]) + ")" : "0";
+    auto element_loop = [&](const std::function<void()> &inside) {
+      os << pad() << "for (int n = 0; n < " << cper << "; n++) {\n";
+      indent++;
+      os << pad() << "const int t = threadIdx.x + 256 * n;\n" << pad() << "if (t >= " << CT << ") break;\n";
+      inside();
+      indent--;
+      os << pad() << "}\n";
+    };
+    for (size_t q = 0; q < s.tile_args.size(); q++)
+      os << pad() << ctype(val(s.tile_args[q]).dtype) << " car" << L << "_" << q << "[" << cper << "];\n";
+    if (!s.tile_args.empty())
+      element_loop([&] {
+        for (auto &cv : carried) var[cv.first] = cv.second + "[n]";
+        for (size_t q = 0; q < s.tile_args.size(); q++) os << pad() << "car" << L << "_" << q << "[n] = " << at(s.tile_inits[q], ci0, ci1) << ";\n";
+        for (auto &cv : carried) var.erase(cv.first);
+      });
+    std::map<int, std::string> saved_carried = carried;
+    for (size_t q = 0; q < s.tile_args.size(); q++) carried[s.tile_args[q]] = "car" + L + "_" + std::to_string(q);
     for (size_t q = 0; q < s.int_iters.size(); q++)
       os << pad() << "long long it" << L << "_" << q << " = " << ex(s.int_iters[q].init) << ";\n";
     os << pad() << "for (long long iv" << L << " = " << ex(s.lb) << "; iv" << L << " < " << ex(s.ub) << "; iv" << L << " = (long long)(int)(iv" << L
        << " + " << ex(s.step) << ")) {\n";
     indent++;
     body(s.body);
+    if (!s.tile_args.empty())
+      element_loop([&] {
+        for (auto &cv : carried) var[cv.first] = cv.second + "[n]";
+        for (size_t q = 0; q < s.tile_args.size(); q++)
+          os << pad() << "const " << ctype(val(s.tile_args[q]).dtype) << " ny" << q << " = " << at(s.tile_yields[q], ci0, ci1) << ";\n";
+        for (size_t q = 0; q < s.tile_args.size(); q++) os << pad() << "car" << L << "_" << q << "[n] = ny" << q << ";\n";
+        for (auto &cv : carried) var.erase(cv.first);
+      });
     for (size_t q = 0; q < s.int_iters.size(); q++)
       os << pad() << "const long long nx" << L << "_" << q << " = " << ex(s.int_iters[q].next) << ";\n";
     for (size_t q = 0; q < s.int_iters.size(); q++) os << pad() << "it" << L << "_" << q << " = nx" << L << "_" << q << ";\n";
@@ -389,6 +464,10 @@ struct Gen {
     os << pad() << "}\n";
     for (size_t q = 0; q < s.int_iters.size(); q++)
       os << pad() << "const long long res" << L << "_" << q << " = it" << L << "_" << q << ";\n";
+    // after the loop the carried arrays hold the results
+    carried = saved_carried;
+    for (size_t q = 0; q < s.results.size(); q++)
+      if (s.results[q] >= 0) carried[s.results[q]] = "car" + L + "_" + std::to_string(q);
   }
 };
 
@@ -427,6 +506,9 @@ std::string tile_program_source(const Program &p) {
        << "  (void)pidx; (void)pidy; (void)pidz; (void)npx; (void)npy; (void)npz;\n";
   g.body(p.body);
   g.os << "}\n";
+  for (int b : g.all_inline_bases)
+    if (g.all_store_bases.count(b))
+      throw Unsupported("tile_program: an argument is both stored to and read by a load that is not of its body's block shape");
   return g.os.str();
 }
 
