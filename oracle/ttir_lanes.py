@@ -188,6 +188,8 @@ class Interpreter:
             return self._for(i, results, tail, env)
         if name == "tt.reduce":
             return self._reduce(i, results, tail, env)
+        if name == "tt.scan":
+            return self._scan(i, results, tail, env)
         if name == "arith.constant":
             lit, ty = (tail.rsplit(" : ", 1) + ["i1"])[:2] if " : " in tail else (tail, "i1")
             env[results[0]] = self._constant(lit.strip(), parse_type(ty))
@@ -433,7 +435,50 @@ class Interpreter:
             env[r] = v
         return close + 1
 
+    def _fold(self, i, results, tail, env, scan):
+        """tt.reduce / tt.scan with any combiner region (argmin / argmax take two operands and a region of compares and
+        selects, ConversionPatterns.hpp:1443-1769): a sequential left fold along `axis` in index order, the region
+        evaluated by this interpreter on whole lines at once."""
+        names = re.findall(r"%[\w.#$]+", tail[:tail.index(")")])
+        operands = [env[n] for n in names]
+        axis = int(re.search(r"axis = (\d+)", tail).group(1))
+        reverse = re.search(r"reverse = true", tail) is not None
+        args = re.findall(r"(%[\w.#$]+)\s*:", self.lines[i + 1])
+        lo = hi = i + 2
+        while not self.lines[hi].startswith(("tt.reduce.return", "tt.scan.return")):
+            hi += 1
+        rets = re.findall(r"%[\w.#$]+", self.lines[hi].split(" : ")[0])
+        xs = [np.moveaxis(o.d, axis, 0) for o in operands]
+        order = range(xs[0].shape[0] - 1, -1, -1) if reverse else range(xs[0].shape[0])
+        outs = [np.empty_like(x) for x in xs]
+        acc = None
+        for l in order:
+            cur = [Val(x[l], o.elem) for x, o in zip(xs, operands)]
+            if acc is None:
+                acc = cur
+            else:
+                local = dict(env)
+                local.update(zip(args, acc + cur))
+                j = lo
+                while j < hi:
+                    j = self._op(j, local)
+                acc = [local[r] for r in rets]
+            for out, a in zip(outs, acc):
+                out[l] = a.d
+        for k, (r, o) in enumerate(zip(results, operands)):
+            if scan:
+                env[r] = Val(np.moveaxis(outs[k], 0, axis), o.elem)
+            else:
+                d = np.asarray(acc[k].d)
+                env[r] = Val(d if d.ndim else d[()], o.elem)
+        return self._skip_block(i + 1)
+
+    def _scan(self, i, results, tail, env):
+        return self._fold(i, results, tail, env, scan=True)
+
     def _reduce(self, i, results, tail, env):
+        if tail[:tail.index(")")].count("%") > 1:
+            return self._fold(i, results, tail, env, scan=False)
         operand = env[re.findall(r"%[\w.#$]+", tail)[0]]
         axis = int(re.search(r"axis = (\d+)", tail).group(1))
         comb = re.match(r'(%[\w.#$]+) = ([\w.]+)', self.lines[i + 2]).group(2)
@@ -454,7 +499,7 @@ class Interpreter:
         elif comb == "arith.addi":
             out = x.sum(axis=0, dtype=x.dtype)
         else:
-            raise NotImplementedError(f"ttir_lanes: reduce with {comb}")
+            return self._fold(i, results, tail, env, scan=False)
         out = out.astype(_NP[operand.elem]) if operand.elem != "bf16" else round_bf16(out)
         env[results[0]] = Val(out if out.ndim else out[()], operand.elem)
         return self._skip_block(i + 1)

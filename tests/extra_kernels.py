@@ -51,10 +51,25 @@ def vec_sub_swapped(x_ptr, y_ptr, z_ptr, n, BLOCK: tl.constexpr):
 
 @triton.jit
 def block_sum(x_ptr, out_ptr, n, BLOCK: tl.constexpr):
-    # structured, but matches no hand-written kernel family (a reduction to one value per program)
+    # a reduction to one value per program: no hand-written family, run by the generic one
     i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
     v = tl.load(x_ptr + i, mask=i < n, other=0.0)
     tl.store(out_ptr + tl.program_id(0), tl.sum(v, axis=0))
+
+
+@triton.jit
+def atomic_accumulate(x_ptr, out_ptr, n, BLOCK: tl.constexpr):
+    # read-modify-write memory ops have no structured lowering: refused
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    tl.atomic_add(out_ptr + i, tl.load(x_ptr + i, mask=i < n, other=0.0), mask=i < n)
+
+
+@triton.jit
+def small_dot(a_ptr, b_ptr, c_ptr, B: tl.constexpr):
+    # a matrix product that is not shaped like the tiled matmul kernels (no K loop): no family takes it
+    i = tl.arange(0, B)
+    at = i[:, None] * B + i[None, :]
+    tl.store(c_ptr + at, tl.dot(tl.load(a_ptr + at), tl.load(b_ptr + at)))
 
 
 # ---- small tile programs (the shapes of the reference's functional tests in python/examples; the code is ours)
@@ -269,3 +284,82 @@ def gather_scatter_nested(src, dst):
         for j in range(0, 2):
             where = _move_masked(src, dst, where // ((i + 1) * (j + 1)) + i)
         where = _move_masked(src, dst, where // 3 + i)
+
+
+# ---- reductions and scans in the generic family ---------------------------------------------
+@triton.jit
+def reduce_rows_2d(x_ptr, out_ptr, n_rows, n_cols, pitch, BR: tl.constexpr, BC: tl.constexpr, KIND: tl.constexpr):
+    # out[r] = sum / max / min over the columns of row r (one program per BR rows)
+    r = tl.program_id(0) * BR + tl.arange(0, BR)
+    c = tl.arange(0, BC)
+    m = (r[:, None] < n_rows) & (c[None, :] < n_cols)
+    if KIND == 0:
+        x = tl.load(x_ptr + r[:, None] * pitch + c[None, :], mask=m, other=0.0)
+        v = tl.sum(x, axis=1)
+    elif KIND == 1:
+        x = tl.load(x_ptr + r[:, None] * pitch + c[None, :], mask=m, other=float("-inf"))
+        v = tl.max(x, axis=1)
+    else:
+        x = tl.load(x_ptr + r[:, None] * pitch + c[None, :], mask=m, other=float("inf"))
+        v = tl.min(x, axis=1)
+    tl.store(out_ptr + r, v, mask=r < n_rows)
+
+
+@triton.jit
+def reduce_cols_2d(x_ptr, out_ptr, n_rows, n_cols, pitch, BR: tl.constexpr, BC: tl.constexpr):
+    # out[c] = sum over the rows of column c (one program per BC columns)
+    r = tl.arange(0, BR)
+    c = tl.program_id(0) * BC + tl.arange(0, BC)
+    m = (r[:, None] < n_rows) & (c[None, :] < n_cols)
+    x = tl.load(x_ptr + r[:, None] * pitch + c[None, :], mask=m, other=0.0)
+    tl.store(out_ptr + c, tl.sum(x, axis=0), mask=c < n_cols)
+
+
+@triton.jit
+def centre_rows(x_ptr, y_ptr, n_cols, pitch, BC: tl.constexpr):
+    # y[row, :] = x[row, :] - mean(x[row, :]): a reduction whose result feeds an elementwise op of the block
+    row = tl.program_id(0)
+    c = tl.arange(0, BC)
+    m = c < n_cols
+    x = tl.load(x_ptr + row * pitch + c, mask=m, other=0.0)
+    mean = tl.sum(x, axis=0) / n_cols
+    tl.store(y_ptr + row * pitch + c, x - mean, mask=m)
+
+
+@triton.jit
+def int_reductions(x_ptr, out_ptr, n, BLOCK: tl.constexpr):
+    # integer sum, max, min and xor of one block
+    i = tl.arange(0, BLOCK)
+    x = tl.load(x_ptr + i, mask=i < n, other=0)
+    tl.store(out_ptr + 0, tl.sum(x, axis=0))
+    tl.store(out_ptr + 1, tl.max(x, axis=0))
+    tl.store(out_ptr + 2, tl.min(x, axis=0))
+    tl.store(out_ptr + 3, tl.xor_sum(x, axis=0))
+
+
+@triton.jit
+def arg_extremes_rows(x_ptr, max_ptr, min_ptr, n_cols, pitch, BC: tl.constexpr):
+    # index of the first maximum and of the first minimum of each row
+    row = tl.program_id(0)
+    c = tl.arange(0, BC)
+    m = c < n_cols
+    hi = tl.load(x_ptr + row * pitch + c, mask=m, other=float("-inf"))
+    lo = tl.load(x_ptr + row * pitch + c, mask=m, other=float("inf"))
+    tl.store(max_ptr + row, tl.argmax(hi, axis=0))
+    tl.store(min_ptr + row, tl.argmin(lo, axis=0))
+
+
+@triton.jit
+def running_sum(x_ptr, y_ptr, n, BLOCK: tl.constexpr):
+    # inclusive prefix sum of each program's block
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = i < n
+    tl.store(y_ptr + i, tl.cumsum(tl.load(x_ptr + i, mask=m, other=0.0), axis=0), mask=m)
+
+
+@triton.jit
+def running_sum_2d(x_ptr, y_ptr, pitch, BR: tl.constexpr, BC: tl.constexpr, AXIS: tl.constexpr):
+    r = tl.arange(0, BR)
+    c = tl.arange(0, BC)
+    at = r[:, None] * pitch + c[None, :]
+    tl.store(y_ptr + at, tl.cumsum(tl.load(x_ptr + at), axis=AXIS))

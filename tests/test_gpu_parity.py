@@ -579,7 +579,9 @@ def test_errors_surface_as_python_exceptions(K):
     with pytest.raises(TypeError, match="device"):
         K.vec_add[(1,)](torch.zeros(1024), x, x, 1024, BLOCK=1024)     # host tensor
     with pytest.raises(NotImplementedError):
-        X.block_sum[(4,)](x, x, 1024, BLOCK=256)                       # matches no family: refused, no fallback
+        X.atomic_accumulate[(4,)](x, x, 1024, BLOCK=256)               # no structured lowering: refused, no fallback
+    with pytest.raises(NotImplementedError, match="no hand-written kernel family"):
+        X.small_dot[(1,)](x, x, x, B=32)                               # a product no family is shaped for
     with pytest.raises(NotImplementedError, match="one program per output tile"):
         a = torch.zeros(256, 256, dtype=torch.bfloat16, device=DEV)
         K.matmul_tiles[(3,)](a, a, a, 256, 256, 256, 256, 1, 256, 1, 256, 1, BM=128, BN=128, BK=64, GROUP_M=8)
@@ -667,3 +669,104 @@ def test_gather_and_scatter_through_an_index_vector():
         X.gather_rows[(1,)](src, idx[b * 256:], out[b * 256:], BLOCK=256)
     torch.cuda.synchronize()
     assert torch.equal(out, src[idx.long()])
+
+
+# ------------------------------------------------------------- reductions and scans (generic family)
+def test_tile_program_axis_reductions():
+    """2-D reductions along either axis (ConversionPatterns.hpp:1343-1364), checked against torch; float sums to 1e-5
+    relative (the order of a sum differs from the reference's sequential one when a line is cut into pieces), max / min
+    exactly."""
+    import extra_kernels as X
+    torch.manual_seed(7)
+    rows, cols = 37, 100
+    x = torch.randn(rows, cols, device=DEV)
+    for kind, want in [(0, x.sum(1)), (1, x.max(1).values), (2, x.min(1).values)]:
+        out = torch.full((rows,), 7.0, device=DEV)
+        k = X.reduce_rows_2d[(triton.cdiv(rows, 8),)](x, out, rows, cols, x.stride(0), BR=8, BC=128, KIND=kind)
+        torch.cuda.synchronize()
+        assert k.function.family == "tile_program"
+        if kind == 0:
+            torch.testing.assert_close(out, want, rtol=1e-5, atol=1e-5)
+        else:
+            assert torch.equal(out, want)
+    out = torch.zeros(cols, device=DEV)
+    X.reduce_cols_2d[(triton.cdiv(cols, 64),)](x[:16], out, 16, cols, x.stride(0), BR=16, BC=64)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out, x[:16].sum(0), rtol=1e-5, atol=1e-5)
+
+
+def test_tile_program_reduction_feeding_the_block():
+    import extra_kernels as X
+    from oracle import ttir_lanes
+    from test_planner import compile_ttir
+    torch.manual_seed(8)
+    x = torch.randn(9, 1000, device=DEV)
+    y = torch.zeros_like(x)
+    k = X.centre_rows[(9,)](x, y, 1000, x.stride(0), BC=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    torch.testing.assert_close(y, x - x.mean(1, keepdim=True), rtol=1e-5, atol=1e-5)
+    ttir = compile_ttir(X.centre_rows, {"x_ptr": "*fp32", "y_ptr": "*fp32", "n_cols": "i32", "pitch": "i32", "BC": "constexpr"}, {"BC": 1024})
+    ref = np.zeros(9 * 1000, dtype=np.float32)
+    ttir_lanes.Interpreter(ttir).run((9,), [None, None, 1000, 1000], {0: x.cpu().numpy().reshape(-1).copy(), 1: ref})
+    assert np.abs(ref.reshape(9, 1000) - y.cpu().numpy()).max() <= 1e-5
+
+
+def test_tile_program_integer_reductions_are_exact():
+    import extra_kernels as X
+    g = torch.Generator().manual_seed(9)
+    x = torch.randint(-2**31, 2**31 - 1, (300,), generator=g, dtype=torch.int64).to(torch.int32)
+    out = torch.zeros(4, dtype=torch.int32, device=DEV)
+    X.int_reductions[(1,)](x.to(DEV), out, 300, BLOCK=512)
+    torch.cuda.synchronize()
+    v = np.concatenate([x.numpy(), np.zeros(212, np.int32)])
+    assert out.cpu().tolist() == [int(v.sum(dtype=np.int32)), int(v.max()), int(v.min()), int(np.bitwise_xor.reduce(v))]
+
+
+def test_tile_program_argmax_argmin_first_index_wins():
+    # ConversionPatterns.hpp:1443-1769: the two-operand reduction with the tie-breaking combiner
+    import extra_kernels as X
+    g = torch.Generator().manual_seed(10)
+    x = torch.randint(0, 6, (33, 200), generator=g).float()          # many ties
+    hi = torch.zeros(33, dtype=torch.int32, device=DEV)
+    lo = torch.zeros(33, dtype=torch.int32, device=DEV)
+    xd = x.to(DEV)
+    k = X.arg_extremes_rows[(33,)](xd, hi, lo, 200, xd.stride(0), BC=256)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    assert hi.cpu().tolist() == x.numpy().argmax(1).tolist()
+    assert lo.cpu().tolist() == x.numpy().argmin(1).tolist()
+
+
+def test_tile_program_cumsum():
+    import extra_kernels as X
+    torch.manual_seed(11)
+    n = 5000
+    x = torch.randn(n, device=DEV)
+    y = torch.zeros(n, device=DEV)
+    k = X.running_sum[(triton.cdiv(n, 1024),)](x, y, n, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    want = torch.cat([c.double().cumsum(0) for c in x.split(1024)]).float()
+    torch.testing.assert_close(y, want, rtol=1e-5, atol=1e-4)
+    xi = torch.arange(1, 1025, dtype=torch.float32, device=DEV)        # exact in f32: any order gives the same sums
+    yi = torch.zeros(1024, device=DEV)
+    X.running_sum[(1,)](xi, yi, 1024, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert torch.equal(yi, xi.cumsum(0))
+    for axis, (BR, BC) in [(1, (4, 8)), (0, (64, 32)), (1, (16, 256))]:
+        x2 = torch.randn(BR, BC, device=DEV)
+        y2 = torch.zeros_like(x2)
+        X.running_sum_2d[(1,)](x2, y2, x2.stride(0), BR=BR, BC=BC, AXIS=axis)
+        torch.cuda.synchronize()
+        torch.testing.assert_close(y2, x2.double().cumsum(axis).float(), rtol=1e-5, atol=1e-5)
+
+
+def test_block_sum_runs_in_the_generic_family():
+    import extra_kernels as X
+    x = torch.arange(0, 1000, dtype=torch.float32, device=DEV)
+    out = torch.zeros(4, device=DEV)
+    k = X.block_sum[(4,)](x, out, 1000, BLOCK=256)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    assert out.cpu().tolist() == [float(sum(range(b * 256, min(1000, (b + 1) * 256)))) for b in range(4)]

@@ -229,3 +229,30 @@ def test_lanes_gathers_and_scatters_against_reference_goldens():
         dst = np.full(128, -1, dtype=np.int32)
         ttir_lanes.Interpreter(ttir).run((1,), [None, None], {0: src, 1: dst})
         assert dst.tolist() == expected, name
+
+
+def test_lanes_reductions_with_regions_and_scans_against_numpy():
+    """Combiner regions (argmax / argmin with ties, first index wins), integer reductions with wraparound, and scans along
+    either axis, against numpy's closed forms."""
+    import extra_kernels as X
+    from test_planner import compile_ttir
+    P, I = "*fp32", "*i32"
+    rng = np.random.default_rng(0)
+    x = rng.integers(0, 6, (5, 200)).astype(np.float32)          # many ties
+    t = compile_ttir(X.arg_extremes_rows, {"x_ptr": P, "max_ptr": I, "min_ptr": I, "n_cols": "i32", "pitch": "i32", "BC": "constexpr"}, {"BC": 256})
+    hi, lo = np.zeros(5, np.int32), np.zeros(5, np.int32)
+    ttir_lanes.Interpreter(t).run((5,), [None, None, None, 200, 200], {0: x.reshape(-1).copy(), 1: hi, 2: lo})
+    assert hi.tolist() == x.argmax(1).tolist() and lo.tolist() == x.argmin(1).tolist()
+    for axis, (BR, BC) in [(1, (4, 8)), (0, (64, 32))]:
+        sig = {"x_ptr": P, "y_ptr": P, "pitch": "i32", "BR": "constexpr", "BC": "constexpr", "AXIS": "constexpr"}
+        t = compile_ttir(X.running_sum_2d, sig, {"BR": BR, "BC": BC, "AXIS": axis})
+        x = rng.standard_normal((BR, BC)).astype(np.float32)
+        y = np.zeros(BR * BC, np.float32)
+        ttir_lanes.Interpreter(t).run((1,), [None, None, BC], {0: x.reshape(-1).copy(), 1: y})
+        assert np.abs(y.reshape(BR, BC) - np.cumsum(x.astype(np.float64), axis=axis)).max() < 1e-5
+    t = compile_ttir(X.int_reductions, {"x_ptr": I, "out_ptr": I, "n": "i32", "BLOCK": "constexpr"}, {"BLOCK": 512})
+    xi = rng.integers(-2**31, 2**31, 300).astype(np.int32)
+    out = np.zeros(4, np.int32)
+    ttir_lanes.Interpreter(t).run((1,), [None, None, 300], {0: xi.copy(), 1: out})
+    pad = np.concatenate([xi, np.zeros(212, np.int32)])
+    assert out.tolist() == [int(pad.sum(dtype=np.int32)), int(pad.max()), int(pad.min()), int(np.bitwise_xor.reduce(pad))]

@@ -154,6 +154,10 @@ def test_unsupported_kernels_are_refused(native):
     assert native.PlanHandle(native.structured_to_plan(gathered)[0]).family == "tile_program"
     sig = {"x_ptr": "*fp32", "out_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"}
     s = native.ttir_to_structured(compile_ttir(X.block_sum, sig, {"BLOCK": 256}))
+    assert native.PlanHandle(native.structured_to_plan(s)[0]).family == "tile_program"      # a reduction outside softmax / LayerNorm
+    with pytest.raises(NotImplementedError, match="tt.atomic_rmw"):
+        native.ttir_to_structured(compile_ttir(X.atomic_accumulate, sig, {"BLOCK": 256}))
+    s = native.ttir_to_structured(compile_ttir(X.small_dot, {"a_ptr": "*fp32", "b_ptr": "*fp32", "c_ptr": "*fp32", "B": "constexpr"}, {"B": 32}))
     with pytest.raises(NotImplementedError, match="no hand-written kernel family"):
         native.structured_to_plan(s)
     with pytest.raises(NotImplementedError):
@@ -311,3 +315,28 @@ def test_unstructured_accesses_keep_offsets_and_masks_as_data(native):
            "R": "constexpr", "C": "constexpr"}
     s = native.ttir_to_structured(compile_ttir(X.select_rows, sig, {"R": 4, "C": 16}))
     assert native.PlanHandle(native.structured_to_plan(s)[0]).family == "tile_program"
+
+
+# ------------------------------------------------------------------ reductions and scans outside the hand-written families
+def test_reductions_and_scans_lower_to_the_generic_family(native):
+    import extra_kernels as X
+    P, I = "*fp32", "*i32"
+    sig = {"x_ptr": P, "max_ptr": I, "min_ptr": I, "n_cols": "i32", "pitch": "i32", "BC": "constexpr"}
+    s = native.ttir_to_structured(compile_ttir(X.arg_extremes_rows, sig, {"BC": 256}))
+    reduces = [l for l in s.splitlines() if l.strip().startswith("reduce ")]
+    assert len(reduces) == 2 and all("name=region" in l and "region=1" in l for l in reduces)   # two operands, a combiner region
+    assert s.count("region_arg") == 8 and s.count("region_result") == 4
+    plan_bytes, _ = native.structured_to_plan(s)
+    assert native.PlanHandle(plan_bytes).family == "tile_program"
+    assert native.structured_to_plan(s)[0] == plan_bytes                                         # the text form round-trips
+    sig = {"x_ptr": P, "y_ptr": P, "n": "i32", "BLOCK": "constexpr"}
+    s = native.ttir_to_structured(compile_ttir(X.running_sum, sig, {"BLOCK": 1024}))
+    assert "scan " in s and "name=arith.addf" in s
+    assert native.PlanHandle(native.structured_to_plan(s)[0]).family == "tile_program"
+    sig = {"x_ptr": P, "out_ptr": P, "n_rows": "i32", "n_cols": "i32", "pitch": "i32", "BR": "constexpr", "BC": "constexpr", "KIND": "constexpr"}
+    s = native.ttir_to_structured(compile_ttir(X.reduce_rows_2d, sig, {"BR": 8, "BC": 128, "KIND": 0}))
+    assert "reduce " in s and "axis=1" in s
+    assert native.PlanHandle(native.structured_to_plan(s)[0]).family == "tile_program"
+    # a block too large for the staged reduction is refused with the reason
+    with pytest.raises(NotImplementedError, match="more than 4096 elements"):
+        native.structured_to_plan(native.ttir_to_structured(compile_ttir(X.reduce_rows_2d, sig, {"BR": 64, "BC": 128, "KIND": 0})))

@@ -117,6 +117,7 @@ class Lowerer {
   Program P;
   std::map<std::string, Def> defs_;
   std::map<std::string, int> int_memo_;       // scalar integer SSA name -> expr
+  int in_region_ = 0;                         // inside a combiner region: scalar integers are data, not index expressions
   std::map<std::string, PtrState> known_ptr_; // loop-carried / loop-result pointer states
   std::map<std::string, int> data_;           // SSA name -> value id
   std::vector<SOp> *cur_ = nullptr;
@@ -857,32 +858,66 @@ class Lowerer {
     cur_->push_back(std::move(s));
   }
 
-  void lower_reduce(const Op &op) {  // ConversionPatterns.hpp:1203-1440
-    if (op.operands.size() != 1 || op.regions.size() != 1) throw Unsupported("tt.reduce with several operands (argmin/argmax)");
+  void lower_reduce(const Op &op) {  // ConversionPatterns.hpp:1203-1440 (one combiner op), :1443-1769 (argmin / argmax)
+    const bool scan = op.name == "tt.scan";
+    const size_t k = op.operands.size();
+    if (op.regions.size() != 1 || k == 0) throw Unsupported(op.name + " without operands or combiner");
     const Block &rb = op.regions[0];
-    if (rb.ops.size() != 2 || rb.ops[1]->name != "tt.reduce.return") throw Unsupported("tt.reduce with a compound combiner");
-    const Op &comb = *rb.ops[0];
+    if (rb.arg_names.size() != 2 * k || op.result_types.size() != k) throw Unsupported(op.name + " whose combiner does not take two values per operand");
+    if (rb.ops.empty() || rb.ops.back()->name != (scan ? "tt.scan.return" : "tt.reduce.return") || rb.ops.back()->operands.size() != k)
+      throw Unsupported(op.name + " whose combiner does not end in a return of one value per operand");
+    SOp s;
+    s.kind = scan ? SK::Scan : SK::Reduce;
+    s.axis = std::stoi(op.attrs.at("axis"));
+    if (scan) s.ival = op.attrs.count("reverse") && op.attrs.at("reverse") == "true";
+    for (auto &o : op.operands) s.operands.push_back(data_of(o));
+    // the common case: one op that combines the two block arguments
     static const std::set<std::string> ok = {"arith.addf", "arith.addi", "arith.maxnumf", "arith.maximumf",
                                              "arith.minnumf", "arith.minimumf", "arith.mulf", "arith.maxsi",
                                              "arith.minsi", "arith.maxui", "arith.minui", "arith.ori",
                                              "arith.andi", "arith.xori", "arith.muli"};
-    if (!ok.count(comb.name)) throw Unsupported("tt.reduce combiner " + comb.name);
-    std::set<std::string> ins(comb.operands.begin(), comb.operands.end());
-    if (comb.operands.size() != 2 || !ins.count(rb.arg_names.at(0)) || !ins.count(rb.arg_names.at(1)))
-      throw Unsupported("tt.reduce combiner does not combine the two block arguments");
-    SOp s;
-    s.kind = SK::Reduce;
-    s.name = comb.name;
-    s.axis = std::stoi(op.attrs.at("axis"));
-    s.operands.push_back(data_of(op.operands[0]));
-    s.result = new_value(result_type(op));
-    data_[op.results[0]] = s.result;
-    cur_->push_back(s);
+    if (k == 1 && rb.ops.size() == 2) {
+      const Op &comb = *rb.ops[0];
+      std::set<std::string> ins(comb.operands.begin(), comb.operands.end());
+      if (ok.count(comb.name) && comb.operands.size() == 2 && ins.count(rb.arg_names[0]) && ins.count(rb.arg_names[1]) &&
+          rb.ops[1]->operands[0] == comb.results.at(0))
+        s.name = comb.name;
+    }
+    if (!s.name.empty() && !scan) {
+      s.result = new_value(result_type(op));
+      data_[op.results[0]] = s.result;
+      cur_->push_back(s);
+      return;
+    }
+    // the combiner as a region of scalar ops
+    if (s.name.empty()) s.name = "region";
+    std::vector<SOp> *saved = cur_;
+    cur_ = &s.body;
+    in_region_++;
+    for (size_t i = 0; i < rb.arg_names.size(); i++) {
+      Def d;
+      d.type = rb.arg_types.at(i);
+      defs_[rb.arg_names[i]] = d;
+      int v = new_value(d.type);
+      data_[rb.arg_names[i]] = v;
+      s.tile_args.push_back(v);
+    }
+    for (size_t i = 0; i + 1 < rb.ops.size(); i++) lower_op(*rb.ops[i]);
+    for (auto &r : rb.ops.back()->operands) s.tile_yields.push_back(data_of(r));
+    in_region_--;
+    cur_ = saved;
+    for (size_t j = 0; j < k; j++) {
+      int v = new_value(op.result_types[j]);
+      data_[op.results.at(j)] = v;
+      s.results.push_back(v);
+    }
+    s.result = s.results[0];
+    cur_->push_back(std::move(s));
   }
 
   void lower_constant(const Op &op) {
     Type t = result_type(op);
-    if (!t.is_tensor && t.is_int()) return;  // reached through int_of on demand
+    if (!t.is_tensor && t.is_int() && !in_region_) return;  // reached through int_of on demand
     SOp s;
     s.kind = SK::Const;
     std::string lit = op.literal;
@@ -905,7 +940,7 @@ class Lowerer {
         Def d;
         d.op = &op;
         d.index = (int)i;
-        d.type = result_type(op);
+        d.type = i < op.result_types.size() ? op.result_types[i] : result_type(op);
         defs_[op.results[i]] = d;
       }
     const std::string &n = op.name;
@@ -913,7 +948,7 @@ class Lowerer {
     if (n == "scf.for") return lower_for(op);
     if (n == "tt.load") return lower_load(op);
     if (n == "tt.store") return lower_store(op);
-    if (n == "tt.reduce") return lower_reduce(op);
+    if (n == "tt.reduce" || n == "tt.scan") return lower_reduce(op);
     if (n == "arith.constant") return lower_constant(op);
     if (op.results.size() != 1) throw Unsupported("operation " + n + " (line " + std::to_string(op.line) + ")");
     Type rt = result_type(op);
@@ -922,7 +957,7 @@ class Lowerer {
       if (!ptr_ops.count(n)) throw Unsupported("pointer-valued operation " + n + " (line " + std::to_string(op.line) + ")");
       return;
     }
-    if (!rt.is_tensor && rt.is_int()) {  // scalar integer: int_of reads it on demand
+    if (!rt.is_tensor && rt.is_int() && !in_region_) {  // scalar integer: int_of reads it on demand
       static const std::set<std::string> int_ops = {
           "tt.get_program_id", "tt.get_num_programs", "arith.addi", "arith.subi", "arith.muli", "arith.divsi",
           "arith.remsi", "arith.minsi", "arith.maxsi", "arith.extsi", "arith.index_cast", "arith.trunci",
@@ -995,6 +1030,13 @@ class Lowerer {
             }
             mark(s.body);
           }
+        } else if (!s.results.empty()) {  // a reduction or scan with a combiner region: all of it or nothing
+          bool res_live = false;
+          for (int r : s.results) res_live |= live[r];
+          if (res_live) {
+            for (int v : s.operands) use(v);
+            for (int r : s.results) use(r);
+          }
         } else if (s.result >= 0 && live[s.result]) {
           for (int v : s.operands) use(v);
         }
@@ -1031,7 +1073,8 @@ class Lowerer {
             s.tile_yields = y;
             s.results = r;
           }
-        } else keep = s.result >= 0 && live[s.result];
+        } else if (!s.results.empty()) keep = live[s.results[0]];
+        else keep = s.result >= 0 && live[s.result];
         if (keep) {
           out.push_back(std::move(s));
           keep_any = true;

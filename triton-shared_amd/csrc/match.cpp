@@ -64,7 +64,19 @@ std::string signature(const Program &p) {
         case SK::Iota: os << def(s.result) << "=iota;"; break;
         case SK::FromIndex: os << def(s.result) << "=index;"; break;
         case SK::ScalarArg: os << def(s.result) << "=farg;"; break;
-        case SK::Reduce: { std::string o = operands(); os << def(s.result) << "=reduce." << s.name << "." << s.axis << o << ";"; break; }
+        case SK::Reduce: {
+          std::string o = operands();
+          if (s.results.empty()) os << def(s.result);
+          for (size_t j = 0; j < s.results.size(); j++) os << (j ? "," : "") << def(s.results[j]);
+          os << "=reduce." << s.name << "." << s.axis << o << ";";
+          break;
+        }
+        case SK::Scan: {
+          std::string o = operands();
+          for (size_t j = 0; j < s.results.size(); j++) os << (j ? "," : "") << def(s.results[j]);
+          os << "=scan." << s.name << "." << s.axis << o << ";";
+          break;
+        }
         case SK::Dot: { std::string o = operands(); os << def(s.result) << "=dot" << o << ";"; break; }
         case SK::ExpandDims: { std::string o = operands(); os << def(s.result) << "=expand." << s.axis << o << ";"; break; }
         case SK::Broadcast: { std::string o = operands(); os << def(s.result) << "=bcast" << o << ";"; break; }
@@ -800,7 +812,7 @@ bool try_fused_map(Plan &pl) {
 bool try_tile_program(Plan &pl) {
   Matcher m(pl.prog);
   for (SOp *s : m.all)
-    if (s->kind == SK::Reduce || s->kind == SK::Dot) return false;
+    if (s->kind == SK::Dot) return false;
   if (m.accesses.empty()) return false;
   pl.source = tile_program_source(pl.prog);  // throws Unsupported with the reason
   pl.family = Family::TileProgram;

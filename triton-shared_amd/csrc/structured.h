@@ -41,6 +41,7 @@ enum class SK {
   FromIndex,   // integer expression -> i32/i64 scalar data value
   ScalarArg,   // floating-point kernel argument as a scalar data value; ival = argument index
   Reduce,      // linalg.reduce over `axis` with combiner `name`
+  Scan,        // inclusive scan along `axis` (tt.scan, ttx.cumsum for addf); ival = 1 when reversed
   Dot,         // linalg.matmul(a,b) then + c
   ExpandDims,  // tensor.expand_shape
   Broadcast,   // linalg.generic broadcast
@@ -93,6 +94,10 @@ struct SOp {
   std::vector<int> tile_yields;      // value ids (inside body)
   std::vector<int> results;          // value ids after the loop (parallel to tile_args)
   std::vector<SOp> body;
+  // Reduce / Scan whose combiner is more than one op of the two block arguments (argmin / argmax, ConversionPatterns.hpp:
+  // 1443-1769), or that take several operands: name = "region"; operands = the k input blocks; results = the k results
+  // (result = results[0]); tile_args = the 2k scalar region arguments (k left, then k right); body = the combiner's
+  // scalar ops; tile_yields = the k values it returns.  Every Scan has this form.
 };
 
 struct Program {

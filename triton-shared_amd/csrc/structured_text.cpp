@@ -25,6 +25,7 @@ static const char *kind_name(SK k) {
     case SK::FromIndex: return "from_index";
     case SK::ScalarArg: return "scalar_arg";
     case SK::Reduce: return "reduce";
+    case SK::Scan: return "scan";
     case SK::Dot: return "dot";
     case SK::ExpandDims: return "expand_dims";
     case SK::Broadcast: return "broadcast";
@@ -35,7 +36,7 @@ static const char *kind_name(SK k) {
 
 static SK kind_from(const std::string &s) {
   static const SK all[] = {SK::Load, SK::Store, SK::ScalarLoad, SK::ScalarStore, SK::Map, SK::Splat, SK::Const,
-                           SK::Iota, SK::FromIndex, SK::ScalarArg, SK::Reduce, SK::Dot, SK::ExpandDims,
+                           SK::Iota, SK::FromIndex, SK::ScalarArg, SK::Reduce, SK::Scan, SK::Dot, SK::ExpandDims,
                            SK::Broadcast, SK::For};
   for (SK k : all)
     if (s == kind_name(k)) return k;
@@ -157,7 +158,18 @@ std::string print_program(const Program &p) {
         case SK::ScalarArg: os << " ival=" << s.ival << " ; " << p.arg_names[s.ival]; break;
         case SK::FromIndex: os << " expr=" << s.expr << " ; " << p.pool.str(s.expr); break;
         case SK::Reduce: case SK::ExpandDims: os << " axis=" << s.axis; break;
+        case SK::Scan: os << " axis=" << s.axis << " ival=" << s.ival; break;
         default: break;
+      }
+      if ((s.kind == SK::Reduce || s.kind == SK::Scan) && !s.tile_args.empty()) {
+        os << " region=1\n";
+        for (int a : s.tile_args) os << ind << "  region_arg arg=" << a << ":" << vty(a) << "\n";
+        for (size_t j = 0; j < s.results.size(); j++)
+          os << ind << "  region_result value=" << s.results[j] << ":" << vty(s.results[j]) << " yield=" << s.tile_yields[j] << "\n";
+        os << ind << "  {\n";
+        emit(s.body, depth + 2);
+        os << ind << "  }\n";
+        continue;
       }
       os << "\n";
     }
@@ -314,6 +326,15 @@ Program read_program(const std::string &text) {
       if (r >= 0) p.values[r] = p.values[fo->tile_args.back()];
       continue;
     }
+    if (f.head == "region_arg") {
+      open_fors.back()->tile_args.push_back(value_ref(f.get("arg"), true));
+      continue;
+    }
+    if (f.head == "region_result") {
+      open_fors.back()->results.push_back(value_ref(f.get("value"), true));
+      open_fors.back()->tile_yields.push_back(std::stoi(f.get("yield")));
+      continue;
+    }
     SOp s;
     s.kind = kind_from(f.head);
     if (s.kind == SK::For) {
@@ -354,7 +375,13 @@ Program read_program(const std::string &text) {
     if (f.has("ival")) s.ival = std::stoll(f.get("ival"));
     if (f.has("expr")) s.expr = E(std::stoll(f.get("expr")));
     if (f.has("axis")) s.axis = std::stoi(f.get("axis"));
+    const bool region = f.has("region");
     stack.back()->push_back(std::move(s));
+    if (region) {  // the combiner's ops follow in a block of their own
+      SOp *ro = &stack.back()->back();
+      open_fors.push_back(ro);
+      stack.push_back(&ro->body);
+    }
   }
   if (p.name.empty()) throw Unsupported("structured text: missing tts.program header");
   return p;

@@ -33,10 +33,11 @@ struct Gen {
   std::ostringstream os;
   std::map<int, const SOp *> def;          // value id -> defining op
   std::map<int, std::string> var;          // value id -> C variable holding it at the current element
-  std::map<int, std::pair<int, int>> tile_arg;  // region value -> (loop, index) : refused
   int indent = 1;
   std::set<int> all_inline_bases, all_store_bases;  // checked against each other at the end
-  std::map<int, std::string> carried;               // region value of a loop-carried tile -> its per-thread array
+  std::ostringstream fns;                           // combiner functions of reductions and scans (before the kernel)
+  std::ostringstream decl;                          // LDS arrays holding their results (top of the kernel)
+  size_t pool_bytes = 0, out_bytes = 0;             // staging pool shared by all reductions; result arrays
 
   explicit Gen(const Program &p) : P(p) {}
 
@@ -105,7 +106,7 @@ struct Gen {
     auto it = var.find(v);
     if (it != var.end()) return it->second;
     auto d = def.find(v);
-    if (d == def.end()) no("internal: use of an undefined value");
+    if (d == def.end()) no("a loop-carried block value used in a loop over another block shape");
     const SOp &s = *d->second;
     const Value &V = val(v);
     auto idx = [&](const std::vector<int64_t> &shape, size_t dim) -> std::string {
@@ -150,6 +151,15 @@ struct Gen {
         return "(" + (pred.empty() ? rd : "(" + pred + ") ? " + rd + " : " + other_of(s.acc)) + ")";
       }
       case SK::ScalarLoad: no("internal: scalar load without a variable");
+      case SK::Reduce: case SK::Scan: {
+        size_t j = 0;
+        for (size_t q = 0; q < s.results.size(); q++)
+          if (s.results[q] == v) j = q;
+        const std::string arr = "out" + std::to_string(s.result) + "_" + std::to_string(j);
+        if (V.shape.empty()) return arr + "[0]";
+        if (V.shape.size() == 1) return arr + "[" + i0 + "]";
+        return arr + "[" + i0 + " * " + std::to_string(V.shape[1]) + " + " + i1 + "]";
+      }
       case SK::Map: {
         std::vector<std::string> a;
         for (int o : s.operands) {
@@ -215,6 +225,11 @@ struct Gen {
     if (n == "arith.remsi") { need(2); return "(" + ctype(rt) + ")srem(" + a[0] + ", " + a[1] + ")"; }
     if (n == "arith.minsi") { need(2); return "(" + ctype(rt) + ")smin(" + a[0] + ", " + a[1] + ")"; }
     if (n == "arith.maxsi") { need(2); return "(" + ctype(rt) + ")smax(" + a[0] + ", " + a[1] + ")"; }
+    if (n == "arith.maxui" || n == "arith.minui") {
+      need(2);
+      const std::string U = rt == "i64" ? "unsigned long long" : "unsigned";
+      return "(" + ctype(rt) + ")((" + U + ")" + a[0] + (n == "arith.maxui" ? " > (" : " < (") + U + ")" + a[1] + " ? " + a[0] + " : " + a[1] + ")";
+    }
     if (n == "arith.andi") { need(2); return rt == "i1" ? a[0] + " && " + a[1] : "(" + ctype(rt) + ")(" + a[0] + " & " + a[1] + ")"; }
     if (n == "arith.ori") { need(2); return rt == "i1" ? a[0] + " || " + a[1] : "(" + ctype(rt) + ")(" + a[0] + " | " + a[1] + ")"; }
     if (n == "arith.xori") { need(2); return rt == "i1" ? a[0] + " != " + a[1] : "(" + ctype(rt) + ")(" + a[0] + " ^ " + a[1] + ")"; }
@@ -275,60 +290,48 @@ struct Gen {
   }
 
   // ---- bodies ------------------------------------------------------------
+  // Values that a thread keeps for the elements it owns (element t + 256 n of the value's shape in slot n): the loads of
+  // two-phase runs and loop-carried blocks.  They can be named only inside an element loop over the same shape;
+  // elsewhere a load is read again in place and a carried block is refused.
+  struct Held { std::string name; std::vector<int64_t> shape; };
+  std::map<int, Held> held;
+  void map_vars(const std::vector<int64_t> &shape) {
+    for (auto &h : held) {
+      if (h.second.shape == shape) var[h.first] = h.second.name + "[n]";
+      else var.erase(h.first);
+    }
+  }
+  static std::string idx0(const std::vector<int64_t> &shape) { return shape.size() == 2 ? "(t / " + std::to_string(shape[1]) + ")" : "t"; }
+  static std::string idx1(const std::vector<int64_t> &shape) { return shape.size() == 2 ? "(t % " + std::to_string(shape[1]) + ")" : "0"; }
+  void open_element_loop(const std::vector<int64_t> &shape) {
+    const int64_t T = count(shape);
+    os << pad() << "for (int n = 0; n < " << (T + 255) / 256 << "; n++) {\n";
+    indent++;
+    os << pad() << "const int t = threadIdx.x + 256 * n;\n" << pad() << "if (t >= " << T << ") break;\n";
+    map_vars(shape);
+  }
+  void close_loop() {
+    indent--;
+    os << pad() << "}\n";
+  }
+
   void body(const std::vector<SOp> &ops) {
-    for (auto &s : ops)
+    for (auto &s : ops) {
       if (s.result >= 0) def[s.result] = &s;
-    // the block shape of this body: that of its stores (or, without stores, of its largest load); loads of other
-    // shapes are read where they are used
-    std::vector<int64_t> shape;
-    bool have = false;
-    std::set<int> load_bases, store_bases;
-    for (auto &s : ops)
-      if (s.kind == SK::Store) {
-        if (s.acc.sizes.size() > 2 || s.acc.sizes.empty()) no("block accesses of rank " + std::to_string(s.acc.sizes.size()));
-        if (!have) { shape = s.acc.sizes; have = true; }
-        if (s.acc.sizes != shape) no("block stores of different shapes in one body");
-        store_bases.insert(s.acc.base_arg);
-      }
-    for (auto &s : ops)
-      if (s.kind == SK::Load) {
-        if (s.acc.sizes.size() > 2 || s.acc.sizes.empty()) no("block accesses of rank " + std::to_string(s.acc.sizes.size()));
-        if (!have || (store_bases.empty() && count(s.acc.sizes) > count(shape))) { shape = s.acc.sizes; have = true; }
-      }
-    auto inlined = [&](const SOp &s) { return s.kind == SK::Load && s.acc.sizes != shape; };
-    for (auto &s : ops)
-      if (s.kind == SK::Load) {
-        if (inlined(s)) all_inline_bases.insert(s.acc.base_arg);
-        else load_bases.insert(s.acc.base_arg);
-      }
-    for (int b : store_bases) all_store_bases.insert(b);
-    if (have)  // a carried value is held by the thread that owns the element: only right when the shapes agree
-      for (auto &cv : carried)
-        if (val(cv.first).shape != shape) no("a loop-carried block value used in a body of another block shape");
-    const int64_t T = have ? count(shape) : 0;
-    bool aliasing = false;
-    for (int b : store_bases) aliasing = aliasing || load_bases.count(b);
-    const bool two_phase = have && T <= TWO_PHASE_MAX;
-    if (have && !two_phase && aliasing)
-      no("a block of more than " + std::to_string(TWO_PHASE_MAX) + " elements is stored to an argument that the same body loads from");
-    const int64_t per_thread = (T + 255) / 256;
-    const std::string i0 = shape.size() == 2 ? "(t / " + std::to_string(shape[1]) + ")" : "t";
-    const std::string i1 = shape.size() == 2 ? "(t % " + std::to_string(shape[1]) + ")" : "0";
-
-    auto emit_load = [&](const SOp &s, const std::string &target) {
-      std::string pred, addr = address(s.acc, i0, i1, pred);
-      os << pad() << target << " = " << (pred.empty() ? mem_read(s.acc, addr) : "(" + pred + ") ? " + mem_read(s.acc, addr) + " : " + other_of(s.acc))
-         << ";\n";
+      if (s.kind != SK::For)
+        for (int r : s.results) def[r] = &s;
+    }
+    auto is_break = [](const SOp &s) {
+      return s.kind == SK::For || s.kind == SK::ScalarLoad || s.kind == SK::ScalarStore || s.kind == SK::Reduce || s.kind == SK::Scan ||
+             s.kind == SK::Dot;
     };
-
-    // uniform part first in program order is not possible in general (scalars may depend on tiles only through
-    // reductions, which this family does not have), so: scalar loads and stores run where they stand, outside the
-    // element loop; tile ops between them are gathered into element loops.
+    std::vector<int> mine;  // loads this body holds in registers
     size_t k = 0;
     while (k < ops.size()) {
       const SOp &s = ops[k];
       if (s.kind == SK::For) { loop(s); k++; continue; }
       if (s.kind == SK::ScalarLoad) {
+        map_vars({-1});
         std::string pred, addr = address(s.acc, "0", "0", pred);
         std::string name = "s" + std::to_string(s.result);
         os << pad() << "const " << ctype(val(s.result).dtype) << " " << name << " = " << mem_read(s.acc, addr) << ";\n";
@@ -337,6 +340,7 @@ struct Gen {
         continue;
       }
       if (s.kind == SK::ScalarStore) {
+        map_vars({-1});
         std::string pred, addr = address(s.acc, "0", "0", pred);
         os << pad() << "if (threadIdx.x == 0) {\n";
         indent++;
@@ -346,66 +350,111 @@ struct Gen {
         k++;
         continue;
       }
-      if (s.kind == SK::Reduce || s.kind == SK::Dot) no("reductions and dots belong to the hand-written families");
-      // a run of tile ops up to the next loop or scalar access
+      if (s.kind == SK::Dot) no("matrix products belong to the hand-written families");
+      if (s.kind == SK::Reduce || s.kind == SK::Scan) {
+        const std::vector<int64_t> shape = val(s.operands.at(0)).shape;
+        if (shape.empty() || shape.size() > 2) no("a reduction over a block of rank " + std::to_string(shape.size()));
+        if (count(shape) > TWO_PHASE_MAX) no("a reduction or scan over a block of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
+        reduce(s, shape);
+        k++;
+        continue;
+      }
+      // a run of block ops up to the next loop, scalar access or reduction.  Its block shape is that of its stores (else
+      // of its largest load); loads of other shapes are read where they are used.
       size_t end = k;
-      while (end < ops.size() && ops[end].kind != SK::For && ops[end].kind != SK::ScalarLoad && ops[end].kind != SK::ScalarStore) end++;
-      bool any_access = false;
-      for (size_t q = k; q < end; q++) any_access = any_access || ops[q].kind == SK::Load || ops[q].kind == SK::Store;
-      if (any_access) {
-        if (two_phase) {
+      while (end < ops.size() && !is_break(ops[end])) end++;
+      std::vector<int64_t> shape;
+      bool have = false, stores = false;
+      for (size_t q = k; q < end; q++)
+        if (ops[q].kind == SK::Store) {
+          const auto &sz = ops[q].acc.sizes;
+          if (sz.size() > 2 || sz.empty()) no("block accesses of rank " + std::to_string(sz.size()));
+          if (!have) { shape = sz; have = stores = true; }
+          if (sz != shape) no("block stores of different shapes next to each other");
+        }
+      for (size_t q = k; q < end; q++)
+        if (ops[q].kind == SK::Load) {
+          const auto &sz = ops[q].acc.sizes;
+          if (sz.size() > 2 || sz.empty()) no("block accesses of rank " + std::to_string(sz.size()));
+          if (!have || (!stores && count(sz) > count(shape))) { shape = sz; have = true; }
+        }
+      if (!have) { k = end; continue; }  // only elementwise ops: they are written out where their results are used
+      auto own = [&](const SOp &o) { return o.kind == SK::Load && o.acc.sizes == shape; };
+      const int64_t T = count(shape);
+      const bool two_phase = T <= TWO_PHASE_MAX;
+      const std::string i0 = idx0(shape), i1 = idx1(shape);
+      auto emit_load = [&](const SOp &o, const std::string &target) {
+        std::string pred, addr = address(o.acc, i0, i1, pred);
+        os << pad() << target << " = " << (pred.empty() ? mem_read(o.acc, addr) : "(" + pred + ") ? " + mem_read(o.acc, addr) + " : " + other_of(o.acc))
+           << ";\n";
+      };
+      if (two_phase) {
+        bool any_load = false;
+        for (size_t q = k; q < end; q++)
+          if (own(ops[q])) {
+            os << pad() << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << (T + 255) / 256 << "];\n";
+            any_load = true;
+          }
+        if (any_load) {
+          open_element_loop(shape);
           for (size_t q = k; q < end; q++)
-            if (ops[q].kind == SK::Load && !inlined(ops[q]))
-              os << pad() << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << per_thread << "];\n";
-          os << pad() << "for (int n = 0; n < " << per_thread << "; n++) {\n";
-          indent++;
-          os << pad() << "const int t = threadIdx.x + 256 * n;\n" << pad() << "if (t >= " << T << ") break;\n";
-          for (auto &cv : carried) var[cv.first] = cv.second + "[n]";
-          for (size_t q = k; q < end; q++)
-            if (ops[q].kind == SK::Load && !inlined(ops[q])) {
-              emit_load(ops[q], "ld" + std::to_string(ops[q].result) + "[n]");
-              var[ops[q].result] = "ld" + std::to_string(ops[q].result) + "[n]";  // a later load may be indexed by it
+            if (own(ops[q])) {
+              const std::string name = "ld" + std::to_string(ops[q].result);
+              emit_load(ops[q], name + "[n]");
+              held[ops[q].result] = {name, shape};  // a later load of this run may be indexed by it
+              var[ops[q].result] = name + "[n]";
+              mine.push_back(ops[q].result);
             }
-          indent--;
-          os << pad() << "}\n" << pad() << "__syncthreads();\n";
-          os << pad() << "for (int n = 0; n < " << per_thread << "; n++) {\n";
-          indent++;
-          os << pad() << "const int t = threadIdx.x + 256 * n;\n" << pad() << "if (t >= " << T << ") break;\n";
-          for (size_t q = k; q < end; q++)
-            if (ops[q].kind == SK::Load && !inlined(ops[q])) var[ops[q].result] = "ld" + std::to_string(ops[q].result) + "[n]";
-          for (auto &cv : carried) var[cv.first] = cv.second + "[n]";
-        } else {
+          close_loop();
+          os << pad() << "__syncthreads();\n";
+        }
+        if (stores) open_element_loop(shape);
+      } else {
+        std::set<int> load_bases;
+        for (size_t q = k; q < end; q++)
+          if (ops[q].kind == SK::Load) load_bases.insert(ops[q].acc.base_arg);
+        for (size_t q = k; q < end; q++)
+          if (ops[q].kind == SK::Store && load_bases.count(ops[q].acc.base_arg))
+            no("a block of more than " + std::to_string(TWO_PHASE_MAX) + " elements is stored to an argument that is loaded next to the store");
+        if (stores) {
           os << pad() << "for (int t = threadIdx.x; t < " << T << "; t += 256) {\n";
           indent++;
-          if (!carried.empty()) no("a loop that carries block values over blocks of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
+          map_vars({-1});
           for (size_t q = k; q < end; q++)
-            if (ops[q].kind == SK::Load && !inlined(ops[q])) {
+            if (own(ops[q])) {
               std::string name = "v" + std::to_string(ops[q].result);
               emit_load(ops[q], "const " + ctype(val(ops[q].result).dtype) + " " + name);
               var[ops[q].result] = name;
             }
         }
+      }
+      if (stores) {
         for (size_t q = k; q < end; q++) {
           const SOp &o = ops[q];
-          if (o.kind == SK::Map && val(o.result).shape == shape) {  // a full-tile op: name it, later ops reuse it
+          if (o.kind == SK::Map && val(o.result).shape == shape) {  // a whole-block op: name it, later ops reuse it
             std::string name = "v" + std::to_string(o.result);
             std::string e = at(o.result, i0, i1);
             os << pad() << "const " << ctype(val(o.result).dtype) << " " << name << " = " << e << ";\n";
             var[o.result] = name;
           } else if (o.kind == SK::Store) {
+            all_store_bases.insert(o.acc.base_arg);
             const Value &sv = val(o.operands.at(0));
             if (sv.shape != shape) no("a stored value whose shape is not the block's");
             std::string pred, addr = address(o.acc, i0, i1, pred);
             mem_write(o.acc, addr, pred, at(o.operands[0], i0, i1));
           }
         }
-        indent--;
-        os << pad() << "}\n";
-        for (size_t q = k; q < end; q++)
-          if (ops[q].result >= 0 && (ops[q].kind == SK::Load || ops[q].kind == SK::Map)) var.erase(ops[q].result);
+        close_loop();
         os << pad() << "__syncthreads();\n";
       }
+      // values named inside the loop end with it (a load of a two-phase run stays in its registers)
+      for (size_t q = k; q < end; q++)
+        if (ops[q].result >= 0 && (ops[q].kind == SK::Map || (ops[q].kind == SK::Load && !held.count(ops[q].result)))) var.erase(ops[q].result);
       k = end;
+    }
+    for (int v : mine) {
+      held.erase(v);
+      var.erase(v);
     }
   }
 
@@ -422,41 +471,28 @@ struct Gen {
     }
     const int64_t CT = s.tile_args.empty() ? 0 : count(cshape);
     if (CT > TWO_PHASE_MAX) no("a loop-carried block value of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
-    const int64_t cper = (CT + 255) / 256;
-    const std::string ci0 = cshape.size() == 2 ? "(t / " + std::to_string(cshape[1]) + ")" : "t";
-    const std::string ci1 = cshape.size() == 2 ? "(t % " + std::to_string(cshape[1]) + ")" : "0";
-    auto element_loop = [&](const std::function<void()> &inside) {
-      os << pad() << "for (int n = 0; n < " << cper << "; n++) {\n";
-      indent++;
-      os << pad() << "const int t = threadIdx.x + 256 * n;\n" << pad() << "if (t >= " << CT << ") break;\n";
-      inside();
-      indent--;
-      os << pad() << "}\n";
-    };
+    const std::string ci0 = idx0(cshape), ci1 = idx1(cshape);
     for (size_t q = 0; q < s.tile_args.size(); q++)
-      os << pad() << ctype(val(s.tile_args[q]).dtype) << " car" << L << "_" << q << "[" << cper << "];\n";
-    if (!s.tile_args.empty())
-      element_loop([&] {
-        for (auto &cv : carried) var[cv.first] = cv.second + "[n]";
-        for (size_t q = 0; q < s.tile_args.size(); q++) os << pad() << "car" << L << "_" << q << "[n] = " << at(s.tile_inits[q], ci0, ci1) << ";\n";
-        for (auto &cv : carried) var.erase(cv.first);
-      });
-    std::map<int, std::string> saved_carried = carried;
-    for (size_t q = 0; q < s.tile_args.size(); q++) carried[s.tile_args[q]] = "car" + L + "_" + std::to_string(q);
+      os << pad() << ctype(val(s.tile_args[q]).dtype) << " car" << L << "_" << q << "[" << (CT + 255) / 256 << "];\n";
+    if (!s.tile_args.empty()) {
+      open_element_loop(cshape);
+      for (size_t q = 0; q < s.tile_args.size(); q++) os << pad() << "car" << L << "_" << q << "[n] = " << at(s.tile_inits[q], ci0, ci1) << ";\n";
+      close_loop();
+    }
+    for (size_t q = 0; q < s.tile_args.size(); q++) held[s.tile_args[q]] = {"car" + L + "_" + std::to_string(q), cshape};
     for (size_t q = 0; q < s.int_iters.size(); q++)
       os << pad() << "long long it" << L << "_" << q << " = " << ex(s.int_iters[q].init) << ";\n";
     os << pad() << "for (long long iv" << L << " = " << ex(s.lb) << "; iv" << L << " < " << ex(s.ub) << "; iv" << L << " = (long long)(int)(iv" << L
        << " + " << ex(s.step) << ")) {\n";
     indent++;
     body(s.body);
-    if (!s.tile_args.empty())
-      element_loop([&] {
-        for (auto &cv : carried) var[cv.first] = cv.second + "[n]";
-        for (size_t q = 0; q < s.tile_args.size(); q++)
-          os << pad() << "const " << ctype(val(s.tile_args[q]).dtype) << " ny" << q << " = " << at(s.tile_yields[q], ci0, ci1) << ";\n";
-        for (size_t q = 0; q < s.tile_args.size(); q++) os << pad() << "car" << L << "_" << q << "[n] = ny" << q << ";\n";
-        for (auto &cv : carried) var.erase(cv.first);
-      });
+    if (!s.tile_args.empty()) {
+      open_element_loop(cshape);
+      for (size_t q = 0; q < s.tile_args.size(); q++)
+        os << pad() << "const " << ctype(val(s.tile_args[q]).dtype) << " ny" << q << " = " << at(s.tile_yields[q], ci0, ci1) << ";\n";
+      for (size_t q = 0; q < s.tile_args.size(); q++) os << pad() << "car" << L << "_" << q << "[n] = ny" << q << ";\n";
+      close_loop();
+    }
     for (size_t q = 0; q < s.int_iters.size(); q++)
       os << pad() << "const long long nx" << L << "_" << q << " = " << ex(s.int_iters[q].next) << ";\n";
     for (size_t q = 0; q < s.int_iters.size(); q++) os << pad() << "it" << L << "_" << q << " = nx" << L << "_" << q << ";\n";
@@ -465,10 +501,181 @@ struct Gen {
     for (size_t q = 0; q < s.int_iters.size(); q++)
       os << pad() << "const long long res" << L << "_" << q << " = it" << L << "_" << q << ";\n";
     // after the loop the carried arrays hold the results
-    carried = saved_carried;
-    for (size_t q = 0; q < s.results.size(); q++)
-      if (s.results[q] >= 0) carried[s.results[q]] = "car" + L + "_" + std::to_string(q);
+    for (size_t q = 0; q < s.tile_args.size(); q++) {
+      held.erase(s.tile_args[q]);
+      var.erase(s.tile_args[q]);
+      if (s.results[q] >= 0) held[s.results[q]] = {"car" + L + "_" + std::to_string(q), cshape};
+    }
   }
+
+  // ---- reductions and scans ----------------------------------------------
+  static size_t held_bytes(const std::string &t) { return t == "i64" ? 8 : (t == "i1" || t == "i8") ? 1 : t == "i16" ? 2 : 4; }
+
+  // `void <fname>(a0.., b0.., &r0..)`: r = combine(a, b)
+  void combiner(const SOp &s, const std::string &fname) {
+    const size_t k = s.operands.size();
+    std::ostringstream f;
+    f << "__device__ inline void " << fname << "(";
+    for (size_t j = 0; j < k; j++) f << "const " << ctype(val(s.operands[j]).dtype) << " a" << j << ", ";
+    for (size_t j = 0; j < k; j++) f << "const " << ctype(val(s.operands[j]).dtype) << " b" << j << ", ";
+    for (size_t j = 0; j < k; j++) f << (j ? ", " : "") << ctype(val(s.operands[j]).dtype) << " &r" << j;
+    f << ") {\n";
+    if (s.body.empty()) {
+      const std::string &dt = val(s.operands[0]).dtype;
+      if (s.name == "arith.addf" && (dt == "f16" || dt == "bf16")) {
+        f << "  r0 = a0 + b0;\n";  // 16-bit sums accumulate in f32 and round once (ConversionPatterns.hpp:1280-1286)
+      } else {
+        SOp m;
+        m.kind = SK::Map;
+        m.name = s.name;
+        m.result = s.operands[0];  // the element type of the result is the operand's
+        m.operands = {s.operands[0], s.operands[0]};
+        f << "  r0 = " << map_expr(m, {"a0", "b0"}) << ";\n";
+      }
+    } else {
+      std::map<int, std::string> saved = var;
+      for (size_t j = 0; j < k; j++) {
+        var[s.tile_args.at(j)] = "a" + std::to_string(j);
+        var[s.tile_args.at(k + j)] = "b" + std::to_string(j);
+      }
+      for (auto &o : s.body) {
+        if (o.kind != SK::Map && o.kind != SK::Const) no("a combiner with an op that is not scalar arithmetic");
+        def[o.result] = &o;
+      }
+      for (auto &o : s.body) {
+        const std::string name = "c" + std::to_string(o.result);
+        f << "  const " << ctype(val(o.result).dtype) << " " << name << " = " << at(o.result, "0", "0") << ";\n";
+        var[o.result] = name;
+      }
+      for (size_t j = 0; j < k; j++) f << "  r" << j << " = " << at(s.tile_yields.at(j), "0", "0") << ";\n";
+      var = saved;
+    }
+    f << "}\n";
+    fns << f.str();
+  }
+
+  // The operand blocks are staged in LDS; each output line is cut into SEG pieces combined by SEG threads and then in
+  // piece order by one (lines of >= 256 outputs: one thread per line, in element order, as the reference's loop does).
+  void reduce(const SOp &s, const std::vector<int64_t> &shape) {
+    const std::string i0 = idx0(shape), i1 = idx1(shape);
+    const size_t k = s.operands.size();
+    const bool scan = s.kind == SK::Scan;
+    const std::string id = std::to_string(s.result);
+    for (int o : s.operands)
+      if (val(o).shape != shape) no("a reduction or scan over a block whose shape is not the body's");
+    const int rank = (int)shape.size();
+    if (s.axis < 0 || s.axis >= rank) no("a reduction axis outside the block's rank");
+    const int64_t T = count(shape), L = shape[s.axis], O = T / L;
+    const int64_t OS = rank == 1 ? 0 : s.axis == 1 ? shape[1] : 1, LS = rank == 1 ? 1 : s.axis == 1 ? 1 : shape[1];
+    int64_t SEG = 1;
+    while (SEG * 2 * O <= 256 && (SEG * 2) * (SEG * 2) <= 2 * L) SEG *= 2;  // about sqrt(L) pieces: L / SEG + SEG steps
+    const int64_t CH = (L + SEG - 1) / SEG, NSEG = scan ? (L + CH - 1) / CH : SEG, PS = O * NSEG;
+    const std::string fname = "comb" + id;
+    combiner(s, fname);
+    // LDS: staging and partials in the shared pool, results in arrays of their own
+    std::vector<std::string> Tn(k);
+    size_t off = 0;
+    os << pad() << "__syncthreads();\n";
+    for (size_t j = 0; j < k; j++) {
+      Tn[j] = ctype(val(s.operands[j]).dtype);
+      const size_t sz = held_bytes(val(s.operands[j]).dtype);
+      os << pad() << Tn[j] << " *const st" << id << "_" << j << " = (" << Tn[j] << " *)(pool + " << off << ");\n";
+      off = (off + T * sz + 15) / 16 * 16;
+      os << pad() << Tn[j] << " *const pt" << id << "_" << j << " = (" << Tn[j] << " *)(pool + " << off << ");\n";
+      off = (off + PS * sz + 15) / 16 * 16;
+      const int64_t n_out = scan ? T : O;
+      decl << "  __shared__ " << Tn[j] << " out" << id << "_" << j << "[" << n_out << "];\n";
+      out_bytes += (n_out * sz + 15) / 16 * 16;
+    }
+    pool_bytes = std::max(pool_bytes, off);
+    auto list = [&](const std::string &pre, const std::string &post) {
+      std::string r;
+      for (size_t j = 0; j < k; j++) r += (j ? ", " : "") + pre + std::to_string(j) + post;
+      return r;
+    };
+    const std::string S = "st" + id + "_", Pt = "pt" + id + "_", Out = "out" + id + "_";
+    // stage
+    open_element_loop(shape);
+    for (size_t j = 0; j < k; j++) os << pad() << S << j << "[t] = " << at(s.operands[j], i0, i1) << ";\n";
+    close_loop();
+    os << pad() << "__syncthreads();\n";
+    auto final_value = [&](size_t j, const std::string &e) {  // a 16-bit sum is rounded once, here
+      const std::string &dt = val(s.operands[j]).dtype;
+      return s.body.empty() && s.name == "arith.addf" ? rounded(dt, e) : e;
+    };
+    if (!scan) {
+      os << pad() << "for (int q = threadIdx.x; q < " << PS << "; q += 256) {\n";
+      indent++;
+      os << pad() << "const int o = q / " << SEG << ", sg = q % " << SEG << ";\n";
+      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << " = " << S << j << "[o * " << OS << " + sg * " << LS << "];\n";
+      os << pad() << "for (int l = sg + " << SEG << "; l < " << L << "; l += " << SEG << ") " << fname << "(" << list("acc", "") << ", "
+         << list(S, "[o * " + std::to_string(OS) + " + l * " + std::to_string(LS) + "]") << ", " << list("acc", "") << ");\n";
+      for (size_t j = 0; j < k; j++) {
+        if (SEG == 1) os << pad() << Out << j << "[o] = " << final_value(j, "acc" + std::to_string(j)) << ";\n";
+        else os << pad() << Pt << j << "[q] = acc" << j << ";\n";
+      }
+      indent--;
+      os << pad() << "}\n" << pad() << "__syncthreads();\n";
+      if (SEG > 1) {
+        os << pad() << "for (int o = threadIdx.x; o < " << O << "; o += 256) {\n";
+        indent++;
+        for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << " = " << Pt << j << "[o * " << SEG << "];\n";
+        os << pad() << "for (int sg = 1; sg < " << SEG << "; sg++) " << fname << "(" << list("acc", "") << ", "
+           << list(Pt, "[o * " + std::to_string(SEG) + " + sg]") << ", " << list("acc", "") << ");\n";
+        for (size_t j = 0; j < k; j++) os << pad() << Out << j << "[o] = " << final_value(j, "acc" + std::to_string(j)) << ";\n";
+        indent--;
+        os << pad() << "}\n" << pad() << "__syncthreads();\n";
+      }
+      return;
+    }
+    // scan: each piece on its own, then the pieces' totals in order, then the carry into every later piece
+    const std::string at_l = "[o * " + std::to_string(OS) + " + " + (s.ival ? "(" + std::to_string(L - 1) + " - l)" : std::string("l")) + " * " +
+                             std::to_string(LS) + "]";
+    os << pad() << "for (int q = threadIdx.x; q < " << PS << "; q += 256) {\n";
+    indent++;
+    os << pad() << "const int o = q / " << NSEG << ", sg = q % " << NSEG << ";\n";
+    os << pad() << "int l = sg * " << CH << ";\n" << pad() << "const int l1 = l + " << CH << " < " << L << " ? l + " << CH << " : " << L << ";\n";
+    for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << " = " << S << j << at_l << ";\n";
+    for (size_t j = 0; j < k; j++) os << pad() << Out << j << at_l << " = acc" << j << ";\n";
+    os << pad() << "for (l++; l < l1; l++) {\n";
+    indent++;
+    os << pad() << fname << "(" << list("acc", "") << ", " << list(S, at_l) << ", " << list("acc", "") << ");\n";
+    for (size_t j = 0; j < k; j++) os << pad() << Out << j << at_l << " = acc" << j << ";\n";
+    indent--;
+    os << pad() << "}\n";
+    for (size_t j = 0; j < k; j++) os << pad() << Pt << j << "[q] = acc" << j << ";\n";
+    indent--;
+    os << pad() << "}\n" << pad() << "__syncthreads();\n";
+    if (NSEG > 1) {
+      os << pad() << "for (int o = threadIdx.x; o < " << O << "; o += 256) {\n";
+      indent++;
+      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << " = " << Pt << j << "[o * " << NSEG << "];\n";
+      os << pad() << "for (int sg = 1; sg < " << NSEG << "; sg++) {\n";
+      indent++;
+      for (size_t j = 0; j < k; j++) os << pad() << "const " << Tn[j] << " tot" << j << " = " << Pt << j << "[o * " << NSEG << " + sg];\n";
+      for (size_t j = 0; j < k; j++) os << pad() << Pt << j << "[o * " << NSEG << " + sg] = acc" << j << ";\n";
+      os << pad() << fname << "(" << list("acc", "") << ", " << list("tot", "") << ", " << list("acc", "") << ");\n";
+      indent--;
+      os << pad() << "}\n";
+      indent--;
+      os << pad() << "}\n" << pad() << "__syncthreads();\n";
+      os << pad() << "for (int q = threadIdx.x; q < " << PS << "; q += 256) {\n";
+      indent++;
+      os << pad() << "const int o = q / " << NSEG << ", sg = q % " << NSEG << ";\n" << pad() << "if (sg == 0) continue;\n";
+      os << pad() << "const int l1 = (sg + 1) * " << CH << " < " << L << " ? (sg + 1) * " << CH << " : " << L << ";\n";
+      for (size_t j = 0; j < k; j++) os << pad() << "const " << Tn[j] << " carry" << j << " = " << Pt << j << "[q];\n";
+      os << pad() << "for (int l = sg * " << CH << "; l < l1; l++) {\n";
+      indent++;
+      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " upd" << j << ";\n";
+      os << pad() << fname << "(" << list("carry", "") << ", " << list(Out, at_l) << ", " << list("upd", "") << ");\n";
+      for (size_t j = 0; j < k; j++) os << pad() << Out << j << at_l << " = upd" << j << ";\n";
+      indent--;
+      os << pad() << "}\n";
+      indent--;
+      os << pad() << "}\n" << pad() << "__syncthreads();\n";
+    }
+  }
+
 };
 
 const char *TILE_PRELUDE = R"SRC(
@@ -499,17 +706,21 @@ std::string tile_program_source(const Program &p) {
   std::string pre = TILE_PRELUDE;
   const std::string n = std::to_string(TILE_MAX_ARGS);
   for (size_t pos = 0; (pos = pre.find("%N%", pos)) != std::string::npos;) pre.replace(pos, 3, n);
-  g.os << pre;
-  g.os << "extern \"C\" __global__ __launch_bounds__(256) void tile_program(const Args p) {\n"
-       << "  const long long pidx = blockIdx.x, pidy = blockIdx.y, pidz = blockIdx.z;\n"
-       << "  const long long npx = gridDim.x, npy = gridDim.y, npz = gridDim.z;\n"
-       << "  (void)pidx; (void)pidy; (void)pidz; (void)npx; (void)npy; (void)npz;\n";
   g.body(p.body);
-  g.os << "}\n";
+  if (g.pool_bytes + g.out_bytes > 64 * 1024)
+    throw Unsupported("tile_program: the reductions of this program need " + std::to_string(g.pool_bytes + g.out_bytes) + " bytes of LDS (limit 65536)");
+  std::ostringstream all;
+  all << pre << g.fns.str();
+  all << "extern \"C\" __global__ __launch_bounds__(256) void tile_program(const Args p) {\n"
+      << "  const long long pidx = blockIdx.x, pidy = blockIdx.y, pidz = blockIdx.z;\n"
+      << "  const long long npx = gridDim.x, npy = gridDim.y, npz = gridDim.z;\n"
+      << "  (void)pidx; (void)pidy; (void)pidz; (void)npx; (void)npy; (void)npz;\n";
+  if (g.pool_bytes) all << "  __shared__ __attribute__((aligned(16))) unsigned char pool[" << g.pool_bytes << "];\n";
+  all << g.decl.str() << g.os.str() << "}\n";
   for (int b : g.all_inline_bases)
     if (g.all_store_bases.count(b))
       throw Unsupported("tile_program: an argument is both stored to and read by a load that is not of its body's block shape");
-  return g.os.str();
+  return all.str();
 }
 
 }  // namespace tts
