@@ -133,16 +133,71 @@ def make_workloads(torch, triton, K):
             x, b = torch.randn(n, device=dev), torch.randn(n, device=dev)
             y = torch.empty(n, device=dev)
             return lambda: K.gelu_tanh_bias[(triton.cdiv(n, 1024),)](x, b, y, n, BLOCK=1024)
-        return dict(desc=f"fused map y = gelu_tanh(x + b) fp32 N={n}, BLOCK=1024 (19 elementwise ops on the interpreter kernel)",
-                    work=3 * n * 4, bound="hbm", dtype="f32", make=make, set_bytes=3 * n * 4)
+        m = 1 << 16
+        cpu = lanes((m // 1024,), [m], lambda: [np.random.rand(m).astype(np.float32), np.random.rand(m).astype(np.float32),
+                                                np.zeros(m, np.float32)], m / n, f"N={m}")
+        return dict(desc=f"fused map y = gelu_tanh(x + b) fp32 N={n}, BLOCK=1024 (19 elementwise ops, compiled with hipRTC)",
+                    work=3 * n * 4, bound="hbm", dtype="f32", make=make, set_bytes=3 * n * 4, lanes=cpu)
 
     def fused_silu(n):
         def make():
             g, u = torch.randn(n, device=dev).half(), torch.randn(n, device=dev).half()
             o = torch.empty(n, dtype=torch.float16, device=dev)
             return lambda: K.silu_mul_f16[(triton.cdiv(n, 1024),)](g, u, o, n, BLOCK=1024)
-        return dict(desc=f"fused map out = silu(g) * u fp16 N={n}, BLOCK=1024 (10 elementwise ops on the interpreter kernel)",
-                    work=3 * n * 2, bound="hbm", dtype="f16", make=make, set_bytes=3 * n * 2)
+        m = 1 << 16
+        cpu = lanes((m // 1024,), [m], lambda: [np.random.rand(m).astype(np.float16), np.random.rand(m).astype(np.float16),
+                                                np.zeros(m, np.float16)], m / n, f"N={m}")
+        return dict(desc=f"fused map out = silu(g) * u fp16 N={n}, BLOCK=1024 (10 elementwise ops, compiled with hipRTC)",
+                    work=3 * n * 2, bound="hbm", dtype="f16", make=make, set_bytes=3 * n * 2, lanes=cpu)
+
+    def lanes(grid, scalars, arrays, frac, sample):
+        """CPU baseline of a workload outside the five configurations: the lane-level oracle on a smaller problem
+        made of the same programs.  arrays() -> numpy buffers in pointer-argument order."""
+        def run(ttir):
+            from oracle import ttir_lanes
+            bufs = arrays()
+            t0 = time.perf_counter()
+            ttir_lanes.Interpreter(ttir).run(grid, [None] * len(bufs) + list(scalars), dict(enumerate(bufs)))
+            return time.perf_counter() - t0, frac, sample
+        return run
+
+    import numpy as np
+
+    def take_rows(rows, cols):
+        def make():
+            src = torch.randn(rows, cols, device=dev)
+            idx = torch.randint(0, rows, (rows,), device=dev, dtype=torch.int32)
+            dst = torch.empty_like(src)
+            return lambda: K.take_rows[(triton.cdiv(rows, 4),)](src, idx, dst, rows, cols, src.stride(0), dst.stride(0), BR=4, BC=1024)
+        work = 2 * rows * cols * 4 + rows * 4
+        r = 256
+        cpu = lanes((r // 4,), [r, cols, cols, cols],
+                    lambda: [np.random.rand(r, cols).astype(np.float32).reshape(-1), np.random.randint(0, r, r).astype(np.int32),
+                             np.zeros(r * cols, np.float32)], r / rows, f"{r} of {rows} rows")
+        return dict(desc=f"gather of rows dst[r, :] = src[idx[r], :] fp32 [{rows}, {cols}], 4 rows per program (generic family)",
+                    work=work, bound="hbm", dtype="f32", make=make, set_bytes=work, lanes=cpu)
+
+    def row_sums(rows, cols):
+        def make():
+            x = torch.randn(rows, cols, device=dev)
+            out = torch.empty(rows, device=dev)
+            return lambda: K.row_sums[(triton.cdiv(rows, 4),)](x, out, rows, cols, x.stride(0), BR=4, BC=1024)
+        work = rows * cols * 4 + rows * 4
+        r = 256
+        cpu = lanes((r // 4,), [r, cols, cols],
+                    lambda: [np.random.rand(r, cols).astype(np.float32).reshape(-1), np.zeros(r, np.float32)], r / rows, f"{r} of {rows} rows")
+        return dict(desc=f"row sums of fp32 [{rows}, {cols}], 4 rows per program (generic family, axis reduction)", work=work, bound="hbm",
+                    dtype="f32", make=make, set_bytes=work, lanes=cpu)
+
+    def block_cumsum(n):
+        def make():
+            x = torch.randn(n, device=dev)
+            y = torch.empty_like(x)
+            return lambda: K.block_cumsum[(triton.cdiv(n, 1024),)](x, y, n, BLOCK=1024)
+        m = 1 << 16
+        cpu = lanes((m // 1024,), [m], lambda: [np.random.rand(m).astype(np.float32), np.zeros(m, np.float32)], m / n, f"N={m}")
+        return dict(desc=f"inclusive prefix sums inside blocks of 1024, fp32 N={n} (generic family, scan)", work=8 * n, bound="hbm",
+                    dtype="f32", make=make, set_bytes=8 * n, lanes=cpu)
 
     W["cfg1"] = vec_add(98432)
     W["cfg2"] = softmax(4096)
@@ -153,6 +208,9 @@ def make_workloads(torch, triton, K):
     W["cfg2_1m"] = softmax(1 << 20)
     W["next_fused_gelu_2p26"] = fused_gelu(1 << 26)
     W["next_fused_silu_2p26"] = fused_silu(1 << 26)
+    W["next_take_rows_2p26"] = take_rows(1 << 16, 1024)
+    W["next_row_sums_2p26"] = row_sums(1 << 16, 1024)
+    W["next_block_cumsum_2p26"] = block_cumsum(1 << 26)
     return W
 
 
@@ -167,6 +225,7 @@ def time_workload(torch, spy, wl, steps, warmup, rotating_only=False):
         fn = wl["make"]()
         k = fn()  # compiles on first use, launches once through the full frontend
         plan = k.function
+        ttir = k.asm.get("ttir") if hasattr(k, "asm") else None
         grid, vals = spy.last
         launches.append((grid, plan.pack(vals), len(vals), fn))
     torch.cuda.synchronize()
@@ -195,7 +254,7 @@ def time_workload(torch, spy, wl, steps, warmup, rotating_only=False):
         kernel = plan.last_kernel
         del launches
         torch.cuda.empty_cache()
-        return dict(us=us, hot_us=us, wall_us=wall_us, kernel=kernel, sets=sets, frontend_us=0.0, warmup_steps_run=done)
+        return dict(us=us, hot_us=us, wall_us=wall_us, kernel=kernel, sets=sets, frontend_us=0.0, warmup_steps_run=done, ttir=ttir)
     # same measurement on one buffer set ("hot": inputs may sit in the Infinity Cache), for information
     g, arr, n, _ = launches[0]
     for _ in range(warmup):
@@ -215,7 +274,7 @@ def time_workload(torch, spy, wl, steps, warmup, rotating_only=False):
     frontend_us = (time.perf_counter() - t0) * 1e6 / 20
     del launches
     torch.cuda.empty_cache()
-    return dict(us=us, hot_us=hot_us, wall_us=wall_us, kernel=plan.last_kernel, sets=sets, frontend_us=frontend_us,
+    return dict(us=us, hot_us=hot_us, wall_us=wall_us, kernel=plan.last_kernel, sets=sets, frontend_us=frontend_us, ttir=ttir,
                 warmup_steps_run=done)
 
 
@@ -240,10 +299,16 @@ def roofline(wl, us, name=None):
                 frac=round(achieved / BF16_PEAK_TFLOPS, 4), traffic=traffic)
 
 
-def cpu_baseline(torch, name, wl):
+def cpu_baseline(torch, name, wl, ttir=None):
     """Times the CPU restatement (1 thread) on a bounded sample of the workload."""
     from oracle import cpu
     torch.manual_seed(0)
+    if "lanes" in wl:
+        seconds, frac, sample = wl["lanes"](ttir)
+        full_seconds = seconds / frac
+        return dict(value=float(f"{wl['work'] / full_seconds / 1e9:.4g}"), unit="GB/s", cores=1, kind="port",
+                    sample=sample + " (lane-level interpreter of the kernel's TTIR)", seconds_full_workload=float(f"{full_seconds:.4g}"),
+                    host_cores_available=os.cpu_count())
 
     def timed(fn, repeats):
         ts = []
@@ -333,8 +398,8 @@ def main():
                      rotating_buffer_sets=t["sets"], warmup_steps_run=t["warmup_steps_run"], frontend_us_per_launch=round(t["frontend_us"], 1),
                      roofline=roofline(wl, t["us"], name), dtype=wl["dtype"], algorithmic_work=wl["work"],
                      same_buffers=dict(us=round(t["hot_us"], 3), frac=roofline(wl, t["hot_us"])["frac"]))
-        if not args.no_cpu and (name == args.workload or not name.endswith(("2p28", "1m", "2p26"))):
-            entry["cpu_baseline"] = cpu_baseline(torch, name, wl)
+        if not args.no_cpu and (name == args.workload or "lanes" in wl or not name.endswith(("2p28", "1m", "2p26"))):
+            entry["cpu_baseline"] = cpu_baseline(torch, name, wl, t.get("ttir"))
         kernels[name] = entry
     head = kernels[args.workload]
     wl = W[args.workload]

@@ -192,3 +192,33 @@ def silu_mul_f16(g_ptr, u_ptr, out_ptr, n, BLOCK: tl.constexpr):
     g = tl.load(g_ptr + i, mask=m, other=0.0).to(tl.float32)
     u = tl.load(u_ptr + i, mask=m, other=0.0).to(tl.float32)
     tl.store(out_ptr + i, (g / (1.0 + tl.exp(-g)) * u).to(tl.float16), mask=m)
+
+
+# ---- generic family: gathers, reductions along an axis, scans
+@triton.jit
+def take_rows(src_ptr, rows_ptr, dst_ptr, n_rows, n_cols, pitch_src, pitch_dst, BR: tl.constexpr, BC: tl.constexpr):
+    """dst[r, :] = src[rows[r], :]: a gather of whole rows through an index vector (torch.index_select along dim 0)."""
+    r = tl.program_id(0) * BR + tl.arange(0, BR)
+    c = tl.arange(0, BC)
+    which = tl.load(rows_ptr + r, mask=r < n_rows, other=0)
+    m = (r[:, None] < n_rows) & (c[None, :] < n_cols)
+    tile = tl.load(src_ptr + which[:, None].to(tl.int64) * pitch_src + c[None, :], mask=m, other=0.0)
+    tl.store(dst_ptr + r[:, None].to(tl.int64) * pitch_dst + c[None, :], tile, mask=m)
+
+
+@triton.jit
+def row_sums(x_ptr, out_ptr, n_rows, n_cols, pitch, BR: tl.constexpr, BC: tl.constexpr):
+    """out[r] = sum of row r, BR rows per program."""
+    r = tl.program_id(0) * BR + tl.arange(0, BR)
+    c = tl.arange(0, BC)
+    m = (r[:, None] < n_rows) & (c[None, :] < n_cols)
+    x = tl.load(x_ptr + r[:, None].to(tl.int64) * pitch + c[None, :], mask=m, other=0.0)
+    tl.store(out_ptr + r, tl.sum(x, axis=1), mask=r < n_rows)
+
+
+@triton.jit
+def block_cumsum(x_ptr, y_ptr, n, BLOCK: tl.constexpr):
+    """Inclusive prefix sum inside each block of BLOCK elements."""
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = i < n
+    tl.store(y_ptr + i, tl.cumsum(tl.load(x_ptr + i, mask=m, other=0.0), axis=0), mask=m)
