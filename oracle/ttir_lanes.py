@@ -147,10 +147,62 @@ class Interpreter:
             if line == "}" or line.startswith("})"):
                 return i, None
             if line.startswith("scf.yield"):
-                names = re.findall(r"%[\w.#$]+", line.split(":")[0])
+                names = re.findall(r"%[\w.#$-]+", line.split(":")[0])
                 return i, [env[n] for n in names]
             if line.startswith("tt.return"):
+                return len(L), None          # the program ends here (an early return sits in a block of its own)
+            if line.startswith("^"):         # a block label reached by falling through: cannot happen in valid IR
                 i += 1
+                continue
+            if line.startswith("cf.cond_br"):
+                c, then, other = re.match(r"cf\.cond_br (%[\w.#$-]+), (\^\w+), (\^\w+)$", line).groups()
+                label = then if bool(env[c].d) else other
+                i = next(k for k, l in enumerate(L) if l.startswith(label + ":")) + 1
+                continue
+            if line.startswith("cf.br"):
+                label = re.match(r"cf\.br (\^\w+)$", line).group(1)
+                i = next(k for k, l in enumerate(L) if l.startswith(label + ":")) + 1
+                continue
+            if line.startswith("scf.if"):
+                i = self._if(i, env)
+                continue
+            i = self._op(i, env)
+        return i, None
+
+    def _if(self, i, env):
+        """scf.if without results: `scf.if %c {` ... [`} else {` ...] `}`."""
+        L = self.lines
+        m = re.match(r"scf\.if (%[\w.#$-]+) \{$", L[i])
+        if not m:
+            raise NotImplementedError("ttir_lanes: scf.if with results")
+        take = bool(env[m.group(1)].d)
+        # find the matching else / end at this nesting depth
+        depth, j, els = 1, i + 1, None
+        while depth:
+            l = L[j]
+            if l == "} else {" and depth == 1:
+                els = j
+            elif l.endswith("{") and not l.startswith("}"):
+                depth += 1
+            elif l == "}" or l.startswith("})"):
+                depth -= 1
+            j += 1
+        end = j - 1
+        if take:
+            k, _ = self._block(i + 1, env) if els is None else self._run_until(i + 1, els, env)
+        elif els is not None:
+            k, _ = self._block(els + 1, env)
+        else:
+            k = end
+        return len(L) if k >= len(L) else end + 1
+
+    def _run_until(self, i, stop, env):
+        L = self.lines
+        while i < stop:
+            if L[i].startswith("tt.return"):
+                return len(L), None
+            if L[i].startswith("scf.if"):
+                i = self._if(i, env)
                 continue
             i = self._op(i, env)
         return i, None
@@ -195,7 +247,7 @@ class Interpreter:
             env[results[0]] = self._constant(lit.strip(), parse_type(ty))
             return i + 1
         head, _, types = self._split_types(tail)
-        ops = [env[n] for n in re.findall(r"%[\w.#$]+", re.sub(r"\{[^}]*\}", "", head))]
+        ops = [env[n] for n in re.findall(r"%[\w.#$-]+", re.sub(r"\{[^}]*\}", "", head))]
         attrs = dict(re.findall(r"(\w+) = (-?\w+)", " ".join(re.findall(r"\{([^}]*)\}", head))))
         tys = [parse_type(t) for t in re.split(r"\s*(?:->|,| to | \* )\s*", types) if t.strip()] if types else []
         words = [w for w in re.split(r"[\s,]+", re.sub(r"\{[^}]*\}", "", head)) if w and not w.startswith("%")]
@@ -410,7 +462,7 @@ class Interpreter:
 
     # ------------------------------------------------------------ structured
     def _for(self, i, results, tail, env):
-        m = re.match(r"(%[\w.#$]+) = (%[\w.#$]+) to (%[\w.#$]+) step (%[\w.#$]+)(.*)", tail)
+        m = re.match(r"(%[\w.#$-]+) = (%[\w.#$-]+) to (%[\w.#$-]+) step (%[\w.#$-]+)(.*)", tail)
         iv, lb, ub, st, rest = m.groups()
         iters = re.search(r"iter_args\((.*?)\) -> ", rest)
         names, inits = [], []
@@ -439,15 +491,15 @@ class Interpreter:
         """tt.reduce / tt.scan with any combiner region (argmin / argmax take two operands and a region of compares and
         selects, ConversionPatterns.hpp:1443-1769): a sequential left fold along `axis` in index order, the region
         evaluated by this interpreter on whole lines at once."""
-        names = re.findall(r"%[\w.#$]+", tail[:tail.index(")")])
+        names = re.findall(r"%[\w.#$-]+", tail[:tail.index(")")])
         operands = [env[n] for n in names]
         axis = int(re.search(r"axis = (\d+)", tail).group(1))
         reverse = re.search(r"reverse = true", tail) is not None
-        args = re.findall(r"(%[\w.#$]+)\s*:", self.lines[i + 1])
+        args = re.findall(r"(%[\w.#$-]+)\s*:", self.lines[i + 1])
         lo = hi = i + 2
         while not self.lines[hi].startswith(("tt.reduce.return", "tt.scan.return")):
             hi += 1
-        rets = re.findall(r"%[\w.#$]+", self.lines[hi].split(" : ")[0])
+        rets = re.findall(r"%[\w.#$-]+", self.lines[hi].split(" : ")[0])
         xs = [np.moveaxis(o.d, axis, 0) for o in operands]
         order = range(xs[0].shape[0] - 1, -1, -1) if reverse else range(xs[0].shape[0])
         outs = [np.empty_like(x) for x in xs]
@@ -479,9 +531,9 @@ class Interpreter:
     def _reduce(self, i, results, tail, env):
         if tail[:tail.index(")")].count("%") > 1:
             return self._fold(i, results, tail, env, scan=False)
-        operand = env[re.findall(r"%[\w.#$]+", tail)[0]]
+        operand = env[re.findall(r"%[\w.#$-]+", tail)[0]]
         axis = int(re.search(r"axis = (\d+)", tail).group(1))
-        comb = re.match(r'(%[\w.#$]+) = ([\w.]+)', self.lines[i + 2]).group(2)
+        comb = re.match(r'(%[\w.#$-]+) = ([\w.]+)', self.lines[i + 2]).group(2)
         x = np.moveaxis(operand.d, axis, 0)
         if comb == "arith.addf" and x.ndim == 1:
             out = np.add.accumulate(x.astype(np.float32), dtype=np.float32)[-1]  # sequential fold

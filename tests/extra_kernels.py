@@ -363,3 +363,195 @@ def running_sum_2d(x_ptr, y_ptr, pitch, BR: tl.constexpr, BC: tl.constexpr, AXIS
     c = tl.arange(0, BC)
     at = r[:, None] * pitch + c[None, :]
     tl.store(y_ptr + at, tl.cumsum(tl.load(x_ptr + at), axis=AXIS))
+
+
+# ---- control flow and data-dependent scalars (semantics of python/examples/test_early_return.py,
+# test_scalar_store.py, test_sign_extend.py; the code is ours)
+@triton.jit
+def stop_on_flag(flags, dst):
+    # a program whose flag is -1 writes nothing
+    flag = tl.load(flags + tl.program_id(0))
+    if flag == -1:
+        return
+    i = tl.arange(0, 4)
+    tl.store(dst + i, i + 1)
+
+
+@triton.jit
+def count_up_scalars(dst, N: tl.constexpr):
+    # dst[0 .. N) = 0, 1, 2, ... written one scalar at a time from two nested loops
+    at = dst + tl.program_id(0)
+    for a in range(0, N // 2):
+        v = 2 * a
+        for b in range(0, N // 4):
+            v += b
+            tl.store(at, v)
+            at += 1
+
+
+@triton.jit
+def window_at_loaded_offset(start_ptr, src, dst, n):
+    # the window's start is read from memory and widened to 64 bits
+    first = tl.load(start_ptr).to(tl.int64)
+    i = first + tl.arange(0, 4)
+    tl.store(dst + tl.arange(0, 4), tl.load(src + i, mask=i < n, other=11))
+
+
+# ---- more access patterns of the reference's functional tests (python/examples/test_blockptr_complex_offset.py,
+# test_gather_scatter_continuous.py, test_load_2d_tensor_col.py, test_mask_loop_iter_arg.py, test_nested_loops.py,
+# test_reduce.py, test_tensor_index_iterargs.py, test_unstructured_mask.py, test_einsum_qhmd_hmpd_to_qhmp.py);
+# the kernels are ours, written to the same semantics so that those tests' expectations apply
+@triton.jit
+def block_ptr_shifted_base(src, dst):
+    # a 2x2 block pointer whose base is 8 elements into the buffer
+    a = tl.make_block_ptr(base=src + 8, shape=(2, 2), strides=(2, 1), offsets=(0, 0), block_shape=(2, 2), order=(1, 0))
+    b = tl.make_block_ptr(base=dst, shape=(2, 2), strides=(2, 1), offsets=(0, 0), block_shape=(2, 2), order=(1, 0))
+    tl.store(b, tl.load(a, boundary_check=(0,)), boundary_check=(0,))
+
+
+@triton.jit
+def copy_as_3d(src, dst, X: tl.constexpr, Y: tl.constexpr, Z: tl.constexpr, MASK: tl.constexpr):
+    # a contiguous [X, Y, Z] buffer addressed as [(X*Y), Z] with the row index split by // and %;
+    # MASK 1 masks the load to z < 4 (other = 0), MASK 2 masks the store
+    row = tl.arange(0, X * Y)[:, None]
+    z = tl.arange(0, Z)[None, :]
+    at = (row // Y) * (Y * Z) + (row % Y) * Z + z
+    if MASK == 1:
+        v = tl.load(src + at, mask=z < 4, other=0)
+    else:
+        v = tl.load(src + at)
+    if MASK == 2:
+        tl.store(dst + at, v, mask=z < 4)
+    else:
+        tl.store(dst + at, v)
+
+
+@triton.jit
+def block_ptr_column(src, dst, n_rows, n_cols, BR: tl.constexpr, PITCH: tl.constexpr):
+    # each program copies one whole column through a [BR, 1] block pointer
+    col = tl.program_id(0)
+    a = tl.make_block_ptr(base=src, shape=[n_rows, n_cols], strides=[PITCH, 1], offsets=[0, col], block_shape=[BR, 1], order=[1, 0])
+    b = tl.make_block_ptr(base=dst, shape=[n_rows, n_cols], strides=[PITCH, 1], offsets=[0, col], block_shape=[BR, 1], order=[1, 0])
+    tl.store(b, tl.load(a))
+
+
+@triton.jit
+def grid_stride_copy(dst, src, total, BLOCK: tl.constexpr):
+    # a grid-stride loop whose offsets are a loop-carried block and whose bound is a 64-bit argument
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    hop = tl.num_programs(0) * BLOCK
+    for _ in range(tl.cdiv(total, 4)):
+        m = i < total
+        tl.store(dst + i, tl.load(src + i, mask=m).to(tl.float32), mask=m)
+        i += hop
+
+
+@triton.jit
+def nested_walk(src, dst, pitch_m, pitch_n):
+    # 2x2 blocks walked by pointers carried through three loop levels; three loads interleaved with three stores
+    r = tl.arange(0, 2)
+    a = src + (r[:, None] * pitch_m + r[None, :] * pitch_n)
+    c = dst + (r[:, None] * pitch_m + r[None, :] * pitch_n)
+    for i in range(0, 2):
+        v1 = tl.load(a)
+        for j in range(0, 2):
+            a += 2 * pitch_n
+            v2 = tl.load(a)
+            for k in range(0, 2):
+                a += 2 * pitch_n
+                v3 = tl.load(a)
+                tl.store(c, v1)
+                c += 2 * pitch_n
+                tl.store(c, v2)
+                c += 2 * pitch_n
+                tl.store(c, v3)
+                c += 2 * pitch_n
+        a += 2 * pitch_n
+
+
+@triton.jit
+def block_ptr_row_sum(x_ptr, out_ptr, pitch, n, BLOCK: tl.constexpr):
+    # one row per program through a rank-1 block pointer with a boundary check, summed
+    row = tl.program_id(0)
+    p = tl.make_block_ptr(base=x_ptr, shape=[n * tl.num_programs(0)], strides=[1], offsets=[pitch * row], block_shape=[BLOCK], order=[0])
+    x = tl.load(p, boundary_check=[0])
+    tl.store(out_ptr + row, tl.sum(x, axis=0).to(x.dtype))
+
+
+@triton.jit
+def carried_offsets_masked(src, dst, bound):
+    # 4 blocks of 4; the mask on the carried offsets only bites in the last block (other = -11)
+    i = tl.arange(0, 4)
+    o = tl.arange(0, 4)
+    for _ in range(0, 4):
+        tl.store(dst + o, tl.load(src + i, mask=i < bound, other=-11))
+        i += 4
+        o += 4
+
+
+@triton.jit
+def carried_offsets_nested(src, dst):
+    i = tl.arange(0, 4)
+    o = tl.arange(0, 4)
+    for a in range(0, 2):
+        i += a * 2
+        tl.store(dst + o, tl.load(src + i))
+        i += 4
+        o += 4
+        for b in range(0, 3):
+            i += b * 3
+            tl.store(dst + o, tl.load(src + i))
+            i += 4
+            o += 4
+
+
+@triton.jit
+def store_carried_block(dst):
+    v = tl.arange(0, 4)
+    o = tl.arange(0, 4)
+    for _ in range(0, 2):
+        tl.store(dst + o, v)
+        o += 4
+        v += 4
+
+
+@triton.jit
+def masks_from_memory_2d(src, dst, keep_rows, keep_cols, m, n, M: tl.constexpr, N: tl.constexpr):
+    # rows are loaded where keep_rows says so (other = -2), columns stored where keep_cols says so
+    r = tl.arange(0, M)
+    c = tl.arange(0, N)
+    kr = tl.load(keep_rows + r, mask=r < m, other=0) != 0
+    kc = tl.load(keep_cols + c, mask=c < n, other=0) != 0
+    at = r[:, None] * N + c[None, :]
+    v = tl.load(src + at, mask=kr[:, None] & (c[None, :] < n), other=-2)
+    tl.store(dst + at, v, mask=(r[:, None] < m) & kc[None, :])
+
+
+@triton.jit
+def rows_by_index_masked(src, dst, idx, n_idx, m, n, pitch_m, pitch_n, IM: tl.constexpr, N: tl.constexpr):
+    # dst[k, :] = src[idx[k], :] for idx[k] < m (else -2)
+    k = tl.arange(0, IM)
+    c = tl.arange(0, N)
+    which = tl.load(idx + k, mask=k < n_idx, other=0)
+    ok = (which < m) & (k < n_idx)
+    v = tl.load(src + which[:, None] * pitch_m + c[None, :] * pitch_n, mask=ok[:, None] & (c[None, :] < n), other=-2)
+    tl.store(dst + k[:, None] * pitch_m + c[None, :] * pitch_n, v, mask=(k[:, None] < n_idx) & (c[None, :] < n))
+
+
+@triton.jit
+def einsum_qhmd_hmpd(a_ptr, b_ptr, c_ptr, Q, H, M, P, D, a_q, a_h, a_m, a_d, b_h, b_m, b_p, b_d, c_q, c_h, c_m, c_p,
+                     BQ: tl.constexpr, BP: tl.constexpr):
+    # C[q,h,m,p] = sum_d A[q,h,m,d] * B[h,m,p,d]; (q,h,m) flattened into one block dimension and split again by // and %
+    f = tl.program_id(0) * BQ + tl.arange(0, BQ)
+    p = tl.program_id(1) * BP + tl.arange(0, BP)
+    okf = f < Q * H * M
+    okp = p < P
+    q = f // (H * M)
+    h = (f % (H * M)) // M
+    m = (f % (H * M)) % M
+    acc = tl.zeros((BQ, BP), dtype=tl.float32)
+    for d in range(D):
+        av = tl.load(a_ptr + q * a_q + h * a_h + m * a_m + d * a_d, mask=okf, other=0.0)
+        bv = tl.load(b_ptr + (h * b_h + m * b_m + d * b_d)[:, None] + p[None, :] * b_p, mask=okf[:, None] & okp[None, :], other=0.0)
+        acc += av[:, None] * bv
+    tl.store(c_ptr + (q * c_q + h * c_h + m * c_m)[:, None] + p[None, :] * c_p, acc, mask=okf[:, None] & okp[None, :])

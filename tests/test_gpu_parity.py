@@ -770,3 +770,39 @@ def test_block_sum_runs_in_the_generic_family():
     torch.cuda.synchronize()
     assert k.function.family == "tile_program"
     assert out.cpu().tolist() == [float(sum(range(b * 256, min(1000, (b + 1) * 256)))) for b in range(4)]
+
+
+# ------------------------------------------------------------- the reference's functional tests, case by case
+def _reference_case_ids():
+    import reference_cases
+    return [c["name"] for c in reference_cases.cases()]
+
+
+@pytest.mark.parametrize("name", _reference_case_ids())
+def test_reference_functional_case(name):
+    """tests/reference_cases.py: inputs and expectations of python/examples/*.py; the same cases pin the lane oracle."""
+    import extra_kernels as X
+    import reference_cases
+    case = next(c for c in reference_cases.cases() if c["name"] == name)
+    args = case["args"]()
+    dev = [torch.from_numpy(a).to(DEV) if isinstance(a, np.ndarray) else a for a in args]
+    k = getattr(X, case["kernel"])[case["grid"]](*dev, **case["consts"])
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    case["check"]([d.cpu().numpy() for d in dev if isinstance(d, torch.Tensor)])
+
+
+def test_tile_program_nested_pointer_walk_against_lane_interpreter():
+    # python/examples/test_nested_loops.py is a template without expectations: the oracle provides them
+    import extra_kernels as X
+    from oracle import ttir_lanes
+    from test_planner import compile_ttir
+    src = torch.arange(0, 2 * 64, dtype=torch.float32, device=DEV)
+    dst = torch.full((2 * 64,), -1.0, device=DEV)
+    k = X.nested_walk[(1,)](src, dst, 64, 1)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    ttir = compile_ttir(X.nested_walk, {"src": "*fp32", "dst": "*fp32", "pitch_m": "i32", "pitch_n": "i32"}, {})
+    ref = np.full(128, -1.0, dtype=np.float32)
+    ttir_lanes.Interpreter(ttir).run((1,), [None, None, 64, 1], {0: src.cpu().numpy(), 1: ref})
+    assert np.array_equal(ref, dst.cpu().numpy()) and (ref != -1).sum() > 40

@@ -256,3 +256,23 @@ def test_lanes_reductions_with_regions_and_scans_against_numpy():
     ttir_lanes.Interpreter(t).run((1,), [None, None, 300], {0: xi.copy(), 1: out})
     pad = np.concatenate([xi, np.zeros(212, np.int32)])
     assert out.tolist() == [int(pad.sum(dtype=np.int32)), int(pad.max()), int(pad.min()), int(np.bitwise_xor.reduce(pad))]
+
+
+def test_lanes_on_the_reference_functional_cases():
+    """The lane interpreter against the expectations of the reference's functional tests (tests/reference_cases.py):
+    early return, scalar stores from nested loops, a loaded 64-bit offset, block pointers, index arithmetic with // and %,
+    grid-stride loops, loop-carried offset blocks, masks read from memory, an einsum with carried accumulators."""
+    import extra_kernels as X
+    import reference_cases
+    from test_planner import compile_ttir
+    for case in reference_cases.cases():
+        ttir = compile_ttir(getattr(X, case["kernel"]), case["sig"], case["consts"])
+        args = case["args"]()
+        arrays = [a for a in args if isinstance(a, np.ndarray)]
+        values = [None if isinstance(a, np.ndarray) else a for a in args]
+        log = ttir_lanes.Interpreter(ttir).run(case["grid"], values, dict(enumerate(arrays)))
+        case["check"](arrays)
+        for program in log:                      # and no lane of any program leaves its buffer
+            for _kind, arg, offsets in program:
+                o = np.asarray(offsets)
+                assert o.size == 0 or (o.min() >= 0 and o.max() < arrays[arg].size), (case["name"], arg)

@@ -487,9 +487,25 @@ class Lowerer {
     if (it != data_.end()) return it->second;
     const Def &d = def(name);
     if (!d.type.is_tensor && d.type.is_int()) {  // integer scalar used as data
+      int expr = -1;
+      try {
+        expr = int_of(name);
+      } catch (const Unsupported &) {
+        // not an index expression (it depends on a value read from memory): computed as data, op by op
+        if (!d.op || (d.op->name.rfind("arith.", 0) != 0)) throw;
+        const Op &op = *d.op;
+        SOp s;
+        s.kind = SK::Map;
+        s.name = op.name;
+        if (op.name == "arith.cmpi" || op.name == "arith.cmpf") s.name += "." + op.words.at(0);
+        for (auto &o : op.operands) s.operands.push_back(data_of(o));
+        s.result = new_value(d.type);
+        cur_->push_back(s);
+        return s.result;
+      }
       SOp s;
       s.kind = SK::FromIndex;
-      s.expr = int_of(name);
+      s.expr = expr;
       s.result = new_value(d.type);
       cur_->push_back(s);
       // not memoised across scopes: an expression may depend on a loop's state
@@ -946,6 +962,7 @@ class Lowerer {
     const std::string &n = op.name;
     if (n == "tt.return") return;
     if (n == "scf.for") return lower_for(op);
+    if (n == "cf.if" || n == "scf.if") return lower_if(op);
     if (n == "tt.load") return lower_load(op);
     if (n == "tt.store") return lower_store(op);
     if (n == "tt.reduce" || n == "tt.scan") return lower_reduce(op);
@@ -993,6 +1010,25 @@ class Lowerer {
     throw Unsupported("operation " + n + " (line " + std::to_string(op.line) + ") has no structured lowering");
   }
 
+  // A branch on a scalar condition, without results: an early `return` (cf.cond_br to a block that only returns) or an
+  // `if` around memory effects.  Each non-empty side becomes one If op on the same condition value.
+  void lower_if(const Op &op) {
+    if (!op.results.empty()) throw Unsupported("scf.if with results (line " + std::to_string(op.line) + ")");
+    const int cond = data_of(op.operands.at(0));
+    for (int side = 0; side < 2 && side < (int)op.regions.size(); side++) {
+      if (op.regions[side].ops.empty()) continue;
+      SOp s;
+      s.kind = SK::If;
+      s.operands.push_back(cond);
+      s.ival = side;
+      std::vector<SOp> *saved = cur_;
+      cur_ = &s.body;
+      lower_block(op.regions[side]);
+      cur_ = saved;
+      if (!s.body.empty()) cur_->push_back(std::move(s));
+    }
+  }
+
   void lower_block(const Block &b) {
     for (auto &op : b.ops) lower_op(*op);
   }
@@ -1029,6 +1065,11 @@ class Lowerer {
               }
             }
             mark(s.body);
+          }
+        } else if (s.kind == SK::If) {
+          if (mark(s.body)) {
+            any_effect = true;
+            for (int v : s.operands) use(v);
           }
         } else if (!s.results.empty()) {  // a reduction or scan with a combiner region: all of it or nothing
           bool res_live = false;
@@ -1073,7 +1114,8 @@ class Lowerer {
             s.tile_yields = y;
             s.results = r;
           }
-        } else if (!s.results.empty()) keep = live[s.results[0]];
+        } else if (s.kind == SK::If) keep = sweep(s.body);
+        else if (!s.results.empty()) keep = live[s.results[0]];
         else keep = s.result >= 0 && live[s.result];
         if (keep) {
           out.push_back(std::move(s));

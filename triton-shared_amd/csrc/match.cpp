@@ -80,6 +80,12 @@ std::string signature(const Program &p) {
         case SK::Dot: { std::string o = operands(); os << def(s.result) << "=dot" << o << ";"; break; }
         case SK::ExpandDims: { std::string o = operands(); os << def(s.result) << "=expand." << s.axis << o << ";"; break; }
         case SK::Broadcast: { std::string o = operands(); os << def(s.result) << "=bcast" << o << ";"; break; }
+        case SK::If: {
+          os << (s.ival ? "unless" : "if") << operands() << "{";
+          walk(s.body);
+          os << "};";
+          break;
+        }
         case SK::For: {
           os << "for[";
           for (size_t j = 0; j < s.tile_args.size(); j++) {
@@ -239,6 +245,7 @@ struct Matcher {
         loops.push_back(&s);
         index_ops(s.body);
       }
+      if (s.kind == SK::If) index_ops(s.body);
     }
   }
   std::vector<SOp *> of_kind(SK k) {

@@ -46,6 +46,7 @@ enum class SK {
   ExpandDims,  // tensor.expand_shape
   Broadcast,   // linalg.generic broadcast
   For,         // scf.for
+  If,          // body runs iff the scalar i1 operand is true (false when ival = 1); no results (cf.cond_br trees, scf.if)
 };
 
 struct Access {          // the tts.make_tptr + mask part of a load/store

@@ -30,13 +30,14 @@ static const char *kind_name(SK k) {
     case SK::ExpandDims: return "expand_dims";
     case SK::Broadcast: return "broadcast";
     case SK::For: return "for";
+    case SK::If: return "if";
   }
   return "?";
 }
 
 static SK kind_from(const std::string &s) {
   static const SK all[] = {SK::Load, SK::Store, SK::ScalarLoad, SK::ScalarStore, SK::Map, SK::Splat, SK::Const,
-                           SK::Iota, SK::FromIndex, SK::ScalarArg, SK::Reduce, SK::Scan, SK::Dot, SK::ExpandDims,
+                           SK::Iota, SK::FromIndex, SK::ScalarArg, SK::Reduce, SK::Scan, SK::Dot, SK::ExpandDims, SK::If,
                            SK::Broadcast, SK::For};
   for (SK k : all)
     if (s == kind_name(k)) return k;
@@ -92,6 +93,8 @@ std::string print_program(const Program &p) {
       if (s.kind == SK::For) {
         reach(s.lb); reach(s.ub); reach(s.step);
         for (auto &it : s.int_iters) { reach(it.iter_expr); reach(it.init); reach(it.next); reach(it.result_expr); }
+        scan(s.body);
+      } else if (!s.body.empty()) {
         scan(s.body);
       }
     }
@@ -159,9 +162,10 @@ std::string print_program(const Program &p) {
         case SK::FromIndex: os << " expr=" << s.expr << " ; " << p.pool.str(s.expr); break;
         case SK::Reduce: case SK::ExpandDims: os << " axis=" << s.axis; break;
         case SK::Scan: os << " axis=" << s.axis << " ival=" << s.ival; break;
+        case SK::If: os << " ival=" << s.ival; break;
         default: break;
       }
-      if ((s.kind == SK::Reduce || s.kind == SK::Scan) && !s.tile_args.empty()) {
+      if (((s.kind == SK::Reduce || s.kind == SK::Scan) && !s.tile_args.empty()) || s.kind == SK::If) {
         os << " region=1\n";
         for (int a : s.tile_args) os << ind << "  region_arg arg=" << a << ":" << vty(a) << "\n";
         for (size_t j = 0; j < s.results.size(); j++)

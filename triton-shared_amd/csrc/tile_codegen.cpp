@@ -322,7 +322,7 @@ struct Gen {
         for (int r : s.results) def[r] = &s;
     }
     auto is_break = [](const SOp &s) {
-      return s.kind == SK::For || s.kind == SK::ScalarLoad || s.kind == SK::ScalarStore || s.kind == SK::Reduce || s.kind == SK::Scan ||
+      return s.kind == SK::For || s.kind == SK::If || s.kind == SK::ScalarLoad || s.kind == SK::ScalarStore || s.kind == SK::Reduce || s.kind == SK::Scan ||
              s.kind == SK::Dot;
     };
     std::vector<int> mine;  // loads this body holds in registers
@@ -330,6 +330,16 @@ struct Gen {
     while (k < ops.size()) {
       const SOp &s = ops[k];
       if (s.kind == SK::For) { loop(s); k++; continue; }
+      if (s.kind == SK::If) {  // the condition is a scalar, the same for every thread: barriers inside are safe
+        map_vars({-1});
+        os << pad() << "if (" << (s.ival ? "!" : "") << "(" << at(s.operands.at(0), "0", "0") << ")) {\n";
+        indent++;
+        body(s.body);
+        indent--;
+        os << pad() << "}\n";
+        k++;
+        continue;
+      }
       if (s.kind == SK::ScalarLoad) {
         map_vars({-1});
         std::string pred, addr = address(s.acc, "0", "0", pred);

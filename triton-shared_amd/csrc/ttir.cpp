@@ -3,6 +3,8 @@
 #include "ttir.h"
 
 #include <cctype>
+#include <functional>
+#include <map>
 #include <sstream>
 
 namespace tts {
@@ -95,7 +97,7 @@ static std::string strip_locations(const std::string &text) {
 }
 
 static bool ssa_char(char c) {
-  return isalnum((unsigned char)c) || c == '_' || c == '.' || c == '$' || c == '#';
+  return isalnum((unsigned char)c) || c == '_' || c == '.' || c == '$' || c == '#' || c == '-';
 }
 
 // Splits at top-level occurrences of any separator in seps (each a literal).
@@ -294,6 +296,22 @@ static void parse_op(Lines &L, Block &blk) {
     blk.ops.push_back(std::move(op));
     return;
   }
+  if (op->name == "scf.if") {
+    // scf.if %c {  ...  [} else {  ...]  }   (without results)
+    if (!op->results.empty()) throw Unsupported("scf.if with results");
+    size_t brace = rest.rfind('{');
+    collect_operands(rest.substr(0, brace), op->operands);
+    op->regions.resize(2);
+    parse_block(L, op->regions[0]);
+    if (L.i < L.v.size() && L.v[L.i] == "} else {") {
+      L.i++;
+      parse_block(L, op->regions[1]);
+    }
+    if (L.i >= L.v.size() || L.v[L.i] != "}") throw Unsupported("scf.if region not closed");
+    L.i++;
+    blk.ops.push_back(std::move(op));
+    return;
+  }
   if (op->name == "tt.reduce" || op->name == "tt.scan") {
     // (%x[, %y]) <{axis = 0 : i32}> ({
     size_t close = rest.find(')');
@@ -369,9 +387,84 @@ static void parse_op(Lines &L, Block &blk) {
 static void parse_block(Lines &L, Block &blk) {
   while (L.i < L.v.size()) {
     const std::string &line = L.v[L.i];
-    if (line == "}" || starts_with(line, "})")) return;
+    if (line == "}" || starts_with(line, "})") || starts_with(line, "} else")) return;
     parse_op(L, blk);
   }
+}
+
+// The body of the function may be a tree of basic blocks (an early `return` under an `if` becomes
+// cf.cond_br to a block that only returns).  It is rebuilt as nested "cf.if" ops with a then and an else
+// region; control flow that merges again, loops or passes block arguments is refused.
+static void parse_func_body(Lines &L, Block &out) {
+  struct Cfg {
+    Block ops;
+    std::string term = "return", cond, a, b;
+    bool used = false;
+  };
+  std::map<std::string, Cfg> blocks;
+  std::string cur = "^entry";
+  blocks[cur];
+  auto label_of = [](const std::string &t) {
+    std::string l = trim(t);
+    if (l.find('(') != std::string::npos) throw Unsupported("branch with block arguments: " + l);
+    return l;
+  };
+  while (L.i < L.v.size()) {
+    const std::string line = L.v[L.i];
+    if (line == "}") break;
+    if (line[0] == '^') {
+      size_t e = line.find_first_of(":(");
+      if (e == std::string::npos || line[e] == '(') throw Unsupported("block with arguments: " + line);
+      cur = line.substr(0, e);
+      blocks[cur];
+      L.i++;
+      continue;
+    }
+    if (starts_with(line, "cf.cond_br")) {
+      auto parts = split_top(line.substr(10), {","});
+      if (parts.size() != 3) throw Unsupported("cannot parse: " + line);
+      Cfg &c = blocks[cur];
+      c.term = "cond_br";
+      c.cond = trim(parts[0]);
+      c.a = label_of(parts[1]);
+      c.b = label_of(parts[2]);
+      L.i++;
+      continue;
+    }
+    if (starts_with(line, "cf.br")) {
+      Cfg &c = blocks[cur];
+      c.term = "br";
+      c.a = label_of(line.substr(5));
+      L.i++;
+      continue;
+    }
+    if (starts_with(line, "tt.return")) {
+      blocks[cur].term = "return";
+      L.i++;
+      continue;
+    }
+    parse_op(L, blocks[cur].ops);
+  }
+  std::function<void(const std::string &, Block &)> emit = [&](const std::string &label, Block &dst) {
+    auto it = blocks.find(label);
+    if (it == blocks.end()) throw Unsupported("branch to an unknown block " + label);
+    Cfg &c = it->second;
+    if (c.used) throw Unsupported("control flow that merges or loops (block " + label + " is reached twice)");
+    c.used = true;
+    for (auto &o : c.ops.ops) dst.ops.push_back(std::move(o));
+    if (c.term == "br") return emit(c.a, dst);
+    if (c.term == "cond_br") {
+      auto op = std::make_unique<Op>();
+      op->name = "cf.if";
+      op->operands.push_back(c.cond);
+      op->regions.resize(2);
+      Op *raw = op.get();
+      dst.ops.push_back(std::move(op));
+      emit(c.a, raw->regions[0]);
+      emit(c.b, raw->regions[1]);
+    }
+  };
+  emit("^entry", out);
 }
 
 Func parse_ttir(const std::string &text) {
@@ -416,7 +509,7 @@ Func parse_ttir(const std::string &text) {
       if (line.find("->", close) != std::string::npos && line.find("->", close) < line.rfind('{'))
         throw Unsupported("tt.func with results is not a kernel");
       L.i++;
-      parse_block(L, f.body);
+      parse_func_body(L, f.body);
       if (L.i >= L.v.size() || L.v[L.i] != "}") throw Unsupported("tt.func body not closed");
       L.i++;
       continue;
