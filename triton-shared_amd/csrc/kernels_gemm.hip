@@ -344,16 +344,30 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmParams p, int tiles_m
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));  // the surplus loads land before the LDS goes away
 
+  // Epilogue.  A lane holds one column of each 32x32 block (rows 8 (v/4) + 4 (lane/32) + v%4 in element v).  Two rows
+  // are narrowed at once (v_cvt_pk_bf16_f32 for bf16: round to nearest even, NaNs quieted), the pair is exchanged with
+  // the neighbouring lane, and the even lane stores row r at columns (n, n+1), the odd lane row r+1 at (n-1, n):
+  // half as many store instructions as one 2-byte store per element, and a handful of VALU ops per pair.
   uint16_t *__restrict__ C = (uint16_t *)p.c;
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  const bool odd = lane & 1;
+  const uint32_t sel = odd ? 0x03020706u : 0x05040100u;  // odd: high halves of (neighbour, mine); even: low halves of (mine, neighbour)
 #pragma unroll
   for (int i = 0; i < 4; i++)
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      int64_t col = n0 + wn * 128 + j * 32 + (lane & 31);
+      const int64_t col = n0 + wn * 128 + j * 32 + (lane & 31) - (odd ? 1 : 0);
 #pragma unroll
-      for (int v = 0; v < 16; v++) {
-        int64_t row = m0 + wm * 128 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        __builtin_nontemporal_store(BF16 ? f32_to_bf16(acc[i][j][v]) : f32_to_f16(acc[i][j][v]), &C[row * p.ldc + col]);
+      for (int v = 0; v < 16; v += 2) {
+        const f32x2_t pr = {acc[i][j][v], acc[i][j][v + 1]};
+        const uint32_t pk = BF16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, bf16x2_t))
+                                 : __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, f16x2_t));
+        const uint32_t nb = __builtin_amdgcn_mov_dpp(pk, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]: the neighbour's pair
+        const uint32_t w = __builtin_amdgcn_perm(nb, pk, sel);
+        const int64_t row = m0 + wm * 128 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3) + (odd ? 1 : 0);
+        __builtin_nontemporal_store(w, reinterpret_cast<uint32_t *>(&C[row * p.ldc + col]));
       }
     }
 }
@@ -372,7 +386,8 @@ hipError_t launch_gemm_dma(const GemmParams &p, hipStream_t s) {
 // whole tiles, 16-byte aligned rows, and per-lane byte offsets that fit 32 bits
 bool gemm_fast_path_ok(const GemmParams &p) {
   return p.M % F_BM == 0 && p.N % F_BN == 0 && p.K % F_BK == 0 && p.K >= F_BK && p.lda % 8 == 0 && p.ldb % 8 == 0 &&
-         ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0 && p.lda < (1 << 22) && p.ldb < (1 << 25);
+         ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0 && p.lda < (1 << 22) && p.ldb < (1 << 25) &&
+         p.ldc % 2 == 0 && ((uintptr_t)p.c & 3) == 0;  // C is written in 4-byte pairs
 }
 
 // ------------------------------------------------------ int8-weight GEMM
