@@ -555,3 +555,29 @@ def einsum_qhmd_hmpd(a_ptr, b_ptr, c_ptr, Q, H, M, P, D, a_q, a_h, a_m, a_d, b_h
         bv = tl.load(b_ptr + (h * b_h + m * b_m + d * b_d)[:, None] + p[None, :] * b_p, mask=okf[:, None] & okp[None, :], other=0.0)
         acc += av[:, None] * bv
     tl.store(c_ptr + (q * c_q + h * c_h + m * c_m)[:, None] + p[None, :] * c_p, acc, mask=okf[:, None] & okp[None, :])
+
+
+@triton.jit
+def mm_peeled(a_ptr, b_ptr, c_ptr, M, N, K, s_am, s_ak, s_bk, s_bn, s_cm, s_cn,
+              BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr):
+    # the shape of python/examples/test_mm.py: whole K blocks without masks, then one masked remainder block; operand
+    # rows and columns wrap (% M, % N) instead of being masked; 32x32x32 blocks, so the generic family's small products
+    tn_count = tl.cdiv(N, BN)
+    tm = tl.program_id(0) // tn_count
+    tn = tl.program_id(0) % tn_count
+    rm = tm * BM + tl.arange(0, BM)
+    rn = tn * BN + tl.arange(0, BN)
+    am = rm % M
+    bn = rn % N
+    whole = (tl.cdiv(K, BK) - 1) * BK
+    acc = tl.zeros((BM, BN), dtype=tl.float32)
+    for k0 in range(0, whole, BK):
+        rk = k0 + tl.arange(0, BK)
+        a = tl.load(a_ptr + am[:, None] * s_am + rk[None, :] * s_ak)
+        b = tl.load(b_ptr + rk[:, None] * s_bk + bn[None, :] * s_bn)
+        acc += tl.dot(a, b)
+    rk = whole + tl.arange(0, BK)
+    a = tl.load(a_ptr + am[:, None] * s_am + rk[None, :] * s_ak, mask=(rk < K)[None, :], other=0.0)
+    b = tl.load(b_ptr + rk[:, None] * s_bk + bn[None, :] * s_bn, mask=(rk < K)[:, None], other=0.0)
+    acc += tl.dot(a, b)
+    tl.store(c_ptr + rm[:, None] * s_cm + rn[None, :] * s_cn, acc.to(c_ptr.dtype.element_ty), mask=(rm < M)[:, None] & (rn < N)[None, :])

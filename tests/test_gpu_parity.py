@@ -580,8 +580,9 @@ def test_errors_surface_as_python_exceptions(K):
         K.vec_add[(1,)](torch.zeros(1024), x, x, 1024, BLOCK=1024)     # host tensor
     with pytest.raises(NotImplementedError):
         X.atomic_accumulate[(4,)](x, x, 1024, BLOCK=256)               # no structured lowering: refused, no fallback
-    with pytest.raises(NotImplementedError, match="no hand-written kernel family"):
-        X.small_dot[(1,)](x, x, x, B=32)                               # a product no family is shaped for
+    with pytest.raises(NotImplementedError, match="more than 4096 outputs"):
+        big = torch.zeros(128 * 128, device=DEV)
+        X.small_dot[(1,)](big, big, big, B=128)                        # a large product outside the tiled matmul shapes
     with pytest.raises(NotImplementedError, match="one program per output tile"):
         a = torch.zeros(256, 256, dtype=torch.bfloat16, device=DEV)
         K.matmul_tiles[(3,)](a, a, a, 256, 256, 256, 256, 1, 256, 1, 256, 1, BM=128, BN=128, BK=64, GROUP_M=8)
@@ -806,3 +807,31 @@ def test_tile_program_nested_pointer_walk_against_lane_interpreter():
     ref = np.full(128, -1.0, dtype=np.float32)
     ttir_lanes.Interpreter(ttir).run((1,), [None, None, 64, 1], {0: src.cpu().numpy(), 1: ref})
     assert np.array_equal(ref, dst.cpu().numpy()) and (ref != -1).sum() > 40
+
+
+# ------------------------------------------------------------- small matrix products (generic family)
+def test_tile_program_small_dot_and_loop_peeled_matmul():
+    """tt.dot outside the tiled matmul kernels: a one-shot 32x32 product, and the structure of python/examples/test_mm.py
+    (whole K blocks unmasked, a masked remainder block, wrapped operand rows / columns), against torch.matmul; products
+    are folded in k order in fp32, so the tolerance only covers torch's own summation order."""
+    import extra_kernels as X
+    torch.manual_seed(12)
+    a = torch.randn(32, 32, device=DEV)
+    b = torch.randn(32, 32, device=DEV)
+    c = torch.zeros(32, 32, device=DEV)
+    k = X.small_dot[(1,)](a, b, c, B=32)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    torch.testing.assert_close(c, (a.double() @ b.double()).float(), rtol=1e-5, atol=1e-5)
+    for dtype, tol in [(torch.float32, 1e-5), (torch.float16, 2e-3), (torch.bfloat16, 2e-2)]:
+        for M, N, K in [(37, 53, 70), (64, 32, 32), (5, 100, 33)]:
+            a = torch.randn(M, K, device=DEV).to(dtype)
+            b = torch.randn(K, N, device=DEV).to(dtype)
+            c = torch.full((M, N), 7.0, device=DEV, dtype=dtype)
+            grid = (triton.cdiv(M, 32) * triton.cdiv(N, 32),)
+            k = X.mm_peeled[grid](a, b, c, M, N, K, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1), BM=32, BN=32, BK=32)
+            torch.cuda.synchronize()
+            assert k.function.family == "tile_program"
+            want = a.double() @ b.double()
+            err = (c.double() - want).norm() / want.norm()
+            assert err <= tol, (dtype, M, N, K, float(err))

@@ -157,8 +157,11 @@ def test_unsupported_kernels_are_refused(native):
     assert native.PlanHandle(native.structured_to_plan(s)[0]).family == "tile_program"      # a reduction outside softmax / LayerNorm
     with pytest.raises(NotImplementedError, match="tt.atomic_rmw"):
         native.ttir_to_structured(compile_ttir(X.atomic_accumulate, sig, {"BLOCK": 256}))
-    s = native.ttir_to_structured(compile_ttir(X.small_dot, {"a_ptr": "*fp32", "b_ptr": "*fp32", "c_ptr": "*fp32", "B": "constexpr"}, {"B": 32}))
-    with pytest.raises(NotImplementedError, match="no hand-written kernel family"):
+    dot_sig = {"a_ptr": "*fp32", "b_ptr": "*fp32", "c_ptr": "*fp32", "B": "constexpr"}
+    s = native.ttir_to_structured(compile_ttir(X.small_dot, dot_sig, {"B": 32}))
+    assert native.PlanHandle(native.structured_to_plan(s)[0]).family == "tile_program"      # a small product: generic family
+    s = native.ttir_to_structured(compile_ttir(X.small_dot, dot_sig, {"B": 128}))
+    with pytest.raises(NotImplementedError, match="more than 4096 outputs"):                 # a large one outside the matmul shapes
         native.structured_to_plan(s)
     with pytest.raises(NotImplementedError):
         native.ttir_to_structured("module {\n  tt.func public @k(%a: !tt.ptr<f32>) {\n    %0 = foo.bar %a : i32\n    tt.return\n  }\n}\n")

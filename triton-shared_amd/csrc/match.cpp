@@ -818,8 +818,6 @@ bool try_fused_map(Plan &pl) {
 // Anything made of structured loads, elementwise ops and stores that no hand-written family took.
 bool try_tile_program(Plan &pl) {
   Matcher m(pl.prog);
-  for (SOp *s : m.all)
-    if (s->kind == SK::Dot) return false;
   if (m.accesses.empty()) return false;
   pl.source = tile_program_source(pl.prog);  // throws Unsupported with the reason
   pl.family = Family::TileProgram;
@@ -841,7 +839,23 @@ Plan make_plan(Program &&p) {
     if (try_tile_program(pl)) return pl;
     throw Unsupported("a program with gathers or scatters that also reduces or multiplies matrices; signature: " + pl.signature);
   }
-  if (try_map1d(pl) || try_softmax(pl) || try_layernorm(pl) || try_gemm(pl, false) || try_gemm(pl, true)) return pl;
+  if (try_map1d(pl) || try_softmax(pl) || try_layernorm(pl)) return pl;
+  std::string gemm_refusal;
+  try {
+    if (try_gemm(pl, false) || try_gemm(pl, true)) return pl;
+  } catch (const Unsupported &e) {
+    // shaped like a tiled matmul but outside what those kernels take: the generic family may run it (small tiles);
+    // if not, the matmul family's reason is the one to report
+    gemm_refusal = e.what();
+    pl.k.clear(); pl.e.clear(); pl.lin.clear(); pl.f.clear();
+  }
+  if (!gemm_refusal.empty()) {
+    try {
+      if (try_tile_program(pl)) return pl;
+    } catch (const Unsupported &) {
+    }
+    throw Unsupported(gemm_refusal);
+  }
   try {
     if (try_fused_map(pl)) return pl;
   } catch (const Unsupported &) {

@@ -315,7 +315,9 @@ struct Gen {
     os << pad() << "}\n";
   }
 
-  void body(const std::vector<SOp> &ops) {
+  // `defer`: the caller releases the values this body holds in registers (a loop does, after it has computed the
+  // values it carries to the next iteration from them)
+  void body(const std::vector<SOp> &ops, std::vector<int> *defer = nullptr) {
     for (auto &s : ops) {
       if (s.result >= 0) def[s.result] = &s;
       if (s.kind != SK::For)
@@ -360,7 +362,11 @@ struct Gen {
         k++;
         continue;
       }
-      if (s.kind == SK::Dot) no("matrix products belong to the hand-written families");
+      if (s.kind == SK::Dot) {
+        dot(s, mine);
+        k++;
+        continue;
+      }
       if (s.kind == SK::Reduce || s.kind == SK::Scan) {
         const std::vector<int64_t> shape = val(s.operands.at(0)).shape;
         if (shape.empty() || shape.size() > 2) no("a reduction over a block of rank " + std::to_string(shape.size()));
@@ -462,6 +468,10 @@ struct Gen {
         if (ops[q].result >= 0 && (ops[q].kind == SK::Map || (ops[q].kind == SK::Load && !held.count(ops[q].result)))) var.erase(ops[q].result);
       k = end;
     }
+    if (defer) {
+      defer->insert(defer->end(), mine.begin(), mine.end());
+      return;
+    }
     for (int v : mine) {
       held.erase(v);
       var.erase(v);
@@ -495,13 +505,18 @@ struct Gen {
     os << pad() << "for (long long iv" << L << " = " << ex(s.lb) << "; iv" << L << " < " << ex(s.ub) << "; iv" << L << " = (long long)(int)(iv" << L
        << " + " << ex(s.step) << ")) {\n";
     indent++;
-    body(s.body);
+    std::vector<int> body_held;
+    body(s.body, &body_held);
     if (!s.tile_args.empty()) {
       open_element_loop(cshape);
       for (size_t q = 0; q < s.tile_args.size(); q++)
         os << pad() << "const " << ctype(val(s.tile_args[q]).dtype) << " ny" << q << " = " << at(s.tile_yields[q], ci0, ci1) << ";\n";
       for (size_t q = 0; q < s.tile_args.size(); q++) os << pad() << "car" << L << "_" << q << "[n] = ny" << q << ";\n";
       close_loop();
+    }
+    for (int v : body_held) {
+      held.erase(v);
+      var.erase(v);
     }
     for (size_t q = 0; q < s.int_iters.size(); q++)
       os << pad() << "const long long nx" << L << "_" << q << " = " << ex(s.int_iters[q].next) << ";\n";
@@ -516,6 +531,44 @@ struct Gen {
       var.erase(s.tile_args[q]);
       if (s.results[q] >= 0) held[s.results[q]] = {"car" + L + "_" + std::to_string(q), cshape};
     }
+  }
+
+  // ---- small matrix products ----------------------------------------------
+  // result = a x b + c (ConversionPatterns.hpp:1128-1201: linalg.matmul into zeros, then + c), for products that are not
+  // shaped like the tiled kernels of the GEMM families: a and b are staged in LDS as fp32, every thread folds k in
+  // index order for the outputs it owns (the reference's loop order) and keeps them in registers.
+  void dot(const SOp &s, std::vector<int> &mine) {
+    const Value &A = val(s.operands.at(0)), &B = val(s.operands.at(1)), &R = val(s.result);
+    if (A.shape.size() != 2 || B.shape.size() != 2 || R.shape.size() != 2 || A.shape[1] != B.shape[0] || R.shape[0] != A.shape[0] ||
+        R.shape[1] != B.shape[1])
+      no("a matrix product whose operands are not [M, K] x [K, N]");
+    const int64_t M = A.shape[0], K = A.shape[1], N = B.shape[1];
+    if (M * N > TWO_PHASE_MAX) no("a matrix product with more than " + std::to_string(TWO_PHASE_MAX) + " outputs outside the tiled matmul kernels");
+    const size_t bytes = (size_t)(M * K + K * N) * 4;
+    if (bytes > 48 * 1024) no("a matrix product whose operands need " + std::to_string(bytes) + " bytes of LDS (limit 49152)");
+    if (!is_float(A.dtype) || !is_float(B.dtype) || !is_float(R.dtype)) no("an integer matrix product");
+    pool_bytes = std::max(pool_bytes, bytes);
+    const std::string id = std::to_string(s.result);
+    os << pad() << "__syncthreads();\n";
+    os << pad() << "float *const da" << id << " = (float *)pool, *const db" << id << " = (float *)pool + " << M * K << ";\n";
+    open_element_loop(A.shape);
+    os << pad() << "da" << id << "[t] = " << at(s.operands[0], idx0(A.shape), idx1(A.shape)) << ";\n";
+    close_loop();
+    open_element_loop(B.shape);
+    os << pad() << "db" << id << "[t] = " << at(s.operands[1], idx0(B.shape), idx1(B.shape)) << ";\n";
+    close_loop();
+    os << pad() << "__syncthreads();\n";
+    const std::string name = "dot" + id;
+    os << pad() << "float " << name << "[" << (M * N + 255) / 256 << "];\n";
+    open_element_loop(R.shape);
+    os << pad() << "float sum = 0.f;\n";
+    os << pad() << "for (int k = 0; k < " << K << "; k++) sum += da" << id << "[" << idx0(R.shape) << " * " << K << " + k] * db" << id << "[k * " << N
+       << " + " << idx1(R.shape) << "];\n";
+    os << pad() << name << "[n] = " << rounded(R.dtype, "sum + " + at(s.operands.at(2), idx0(R.shape), idx1(R.shape))) << ";\n";
+    close_loop();
+    os << pad() << "__syncthreads();\n";
+    held[s.result] = {name, R.shape};
+    mine.push_back(s.result);
   }
 
   // ---- reductions and scans ----------------------------------------------
