@@ -404,11 +404,35 @@ class Interpreter:
                  "arith.remsi": np.fmod}[name]
             with np.errstate(over="ignore"):
                 return Val(f(a.d, b.d), a.elem)
+        if name in ("arith.divui", "arith.remui", "arith.shli", "arith.shrsi", "arith.shrui", "arith.minui", "arith.maxui",
+                    "tt.mulhiui", "math.absi"):
+            bits = _INT_BITS[a.elem]
+            mask = (1 << bits) - 1
+            one = lambda x, y: {  # exact integers in, the result wrapped to the type on the way out
+                "arith.divui": lambda: (x & mask) // (y & mask) if (y & mask) else 0,
+                "arith.remui": lambda: (x & mask) % (y & mask) if (y & mask) else 0,
+                "arith.shli": lambda: x << (y & (bits - 1)),
+                "arith.shrsi": lambda: x >> (y & (bits - 1)),
+                "arith.shrui": lambda: (x & mask) >> (y & (bits - 1)),
+                "arith.minui": lambda: min(x & mask, y & mask),
+                "arith.maxui": lambda: max(x & mask, y & mask),
+                "tt.mulhiui": lambda: ((x & mask) * (y & mask)) >> bits,
+                "math.absi": lambda: abs(x)}[name]()
+            if scalar_int:
+                return Val(_wrap(one(int(a.d), int(b.d) if b is not None else 0), bits), a.elem)
+            xs = np.asarray(a.d).ravel().tolist()
+            ys = np.asarray(b.d).ravel().tolist() if b is not None else [0] * len(xs)
+            out = np.array([_wrap(one(x, y), bits) for x, y in zip(xs, ys)], dtype=_NP[a.elem]).reshape(np.asarray(a.d).shape)
+            return Val(out, a.elem)
         if name == "arith.cmpi":
+            x, y = a.d, b.d
+            if words[0] in ("ult", "ule", "ugt", "uge"):  # compare the unsigned readings
+                u = {8: np.uint8, 16: np.uint16, 32: np.uint32, 64: np.uint64}[_INT_BITS[a.elem] if a.elem != "i1" else 8]
+                x, y = np.asarray(x).astype(u), np.asarray(y).astype(u)
             f = {"slt": np.less, "sle": np.less_equal, "sgt": np.greater, "sge": np.greater_equal, "eq": np.equal,
-                 "ne": np.not_equal, "ult": np.less}[words[0]]
-            r = f(a.d, b.d)
-            return Val(r if isinstance(r, np.ndarray) else int(bool(r)), "i1")
+                 "ne": np.not_equal, "ult": np.less, "ule": np.less_equal, "ugt": np.greater, "uge": np.greater_equal}[words[0]]
+            r = f(x, y)
+            return Val(r if isinstance(a.d, np.ndarray) or isinstance(b.d, np.ndarray) else int(bool(r)), "i1")
         if name == "arith.cmpf":
             lt, gt, eq = np.less(a.d, b.d), np.greater(a.d, b.d), np.equal(a.d, b.d)
             uno = np.isnan(a.d) | np.isnan(b.d)
@@ -430,6 +454,32 @@ class Interpreter:
                 return Val(_wrap(int(a.d), _INT_BITS[e]), e)
             return Val(a.d.astype(_NP[e]), e)
         e = tys[-1].elem if tys else a.elem
+        if name in ("tt.bitcast", "arith.bitcast"):
+            if (a.elem in _INT_BITS) == (e in _INT_BITS):
+                return Val(a.d, e)                     # signedness only
+            return Val(np.asarray(a.d).view(_NP[e]) if isinstance(a.d, np.ndarray) else np.asarray([a.d]).view(_NP[e])[0], e)
+        if name == "arith.fptosi":
+            with np.errstate(all="ignore"):
+                return Val(np.trunc(np.asarray(a.d, dtype=np.float64)).astype(_NP[e]), e)
+        if name == "arith.fptoui":
+            with np.errstate(all="ignore"):
+                u = {8: np.uint8, 16: np.uint16, 32: np.uint32, 64: np.uint64}[_INT_BITS[e]]
+                return Val(np.trunc(np.asarray(a.d, dtype=np.float64)).astype(u).astype(_NP[e]), e)
+        if name == "arith.uitofp":
+            u = {8: np.uint8, 16: np.uint16, 32: np.uint32, 64: np.uint64}[_INT_BITS[a.elem]]
+            return self._as_float(np.asarray(a.d).astype(u).astype(np.float32), e, isinstance(a.d, np.ndarray))
+        if name in ("tt.clampf",):
+            f_max, f_min = (np.maximum, np.minimum) if "all" in words else (np.fmax, np.fmin)
+            with np.errstate(all="ignore"):
+                r = f_min(f_max(a.d, ops[1].d), ops[2].d)
+            return self._as_float(r, a.elem, isinstance(r, np.ndarray), already=a.elem != "bf16")
+        if name == "tt.precise_sqrt":
+            with np.errstate(all="ignore"):
+                return self._as_float(np.sqrt(a.d), a.elem, isinstance(a.d, np.ndarray), already=a.elem != "bf16")
+        if name == "tt.precise_divf":
+            with np.errstate(all="ignore"):
+                r = np.divide(a.d, b.d)
+            return self._as_float(r, a.elem, isinstance(r, np.ndarray), already=a.elem != "bf16")
         if name == "arith.sitofp":
             v = np.asarray(a.d).astype(np.float32)
             return self._as_float(v, e, isinstance(a.d, np.ndarray))

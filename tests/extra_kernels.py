@@ -581,3 +581,46 @@ def mm_peeled(a_ptr, b_ptr, c_ptr, M, N, K, s_am, s_ak, s_bk, s_bn, s_cm, s_cn,
     b = tl.load(b_ptr + rk[:, None] * s_bk + bn[None, :] * s_bn, mask=(rk < K)[:, None], other=0.0)
     acc += tl.dot(a, b)
     tl.store(c_ptr + rm[:, None] * s_cm + rn[None, :] * s_cn, acc.to(c_ptr.dtype.element_ty), mask=(rm < M)[:, None] & (rn < N)[None, :])
+
+
+# ---- integer, bit and conversion ops (the op classes of test_core's test_bin_op / test_bitwise_op / test_shift_op /
+# test_umulhi / test_abs / test_clamp / test_floordiv / test_precise_math, which the reference's conftest whitelists)
+@triton.jit
+def int_ops(x_ptr, y_ptr, out_ptr, n, BLOCK: tl.constexpr):
+    # 12 results per element, stored as 12 planes of n
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = i < n
+    x = tl.load(x_ptr + i, mask=m, other=1)
+    y = tl.load(y_ptr + i, mask=m, other=1)
+    ux = x.to(tl.uint32, bitcast=True)
+    uy = y.to(tl.uint32, bitcast=True)
+    sh = y & 31
+    tl.store(out_ptr + 0 * n + i, x // y, mask=m)                                   # signed division (truncating in the IR)
+    tl.store(out_ptr + 1 * n + i, x % y, mask=m)
+    tl.store(out_ptr + 2 * n + i, (ux // uy).to(tl.int32, bitcast=True), mask=m)    # unsigned division
+    tl.store(out_ptr + 3 * n + i, (ux % uy).to(tl.int32, bitcast=True), mask=m)
+    tl.store(out_ptr + 4 * n + i, x << sh, mask=m)
+    tl.store(out_ptr + 5 * n + i, x >> sh, mask=m)                                  # arithmetic shift
+    tl.store(out_ptr + 6 * n + i, (ux >> sh.to(tl.uint32)).to(tl.int32, bitcast=True), mask=m)   # logical shift
+    tl.store(out_ptr + 7 * n + i, tl.umulhi(ux, uy).to(tl.int32, bitcast=True), mask=m)
+    tl.store(out_ptr + 8 * n + i, tl.abs(x), mask=m)
+    tl.store(out_ptr + 9 * n + i, tl.where(ux < uy, x, y), mask=m)                  # unsigned compare
+    tl.store(out_ptr + 10 * n + i, (x ^ y) | (x & ~y), mask=m)
+    tl.store(out_ptr + 11 * n + i, tl.maximum(ux, uy).to(tl.int32, bitcast=True), mask=m)
+
+
+@triton.jit
+def float_ops(x_ptr, y_ptr, out_ptr, n, lo, hi, BLOCK: tl.constexpr):
+    # 8 results per element, stored as 8 planes of n
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = i < n
+    x = tl.load(x_ptr + i, mask=m, other=1.0)
+    y = tl.load(y_ptr + i, mask=m, other=1.0)
+    tl.store(out_ptr + 0 * n + i, tl.clamp(x, lo, hi), mask=m)
+    tl.store(out_ptr + 1 * n + i, tl.sqrt_rn(tl.abs(x)), mask=m)
+    tl.store(out_ptr + 2 * n + i, tl.div_rn(x, y), mask=m)
+    tl.store(out_ptr + 3 * n + i, x.to(tl.int32).to(tl.float32), mask=m)             # fptosi then sitofp
+    tl.store(out_ptr + 4 * n + i, tl.abs(x).to(tl.uint32).to(tl.float32), mask=m)    # fptoui then uitofp
+    tl.store(out_ptr + 5 * n + i, x.to(tl.int32, bitcast=True).to(tl.float32), mask=m)   # the bits as an integer
+    tl.store(out_ptr + 6 * n + i, tl.floor(x) + tl.ceil(y), mask=m)
+    tl.store(out_ptr + 7 * n + i, tl.fma(x, y, x), mask=m)

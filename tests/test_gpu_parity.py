@@ -835,3 +835,26 @@ def test_tile_program_small_dot_and_loop_peeled_matmul():
             want = a.double() @ b.double()
             err = (c.double() - want).norm() / want.norm()
             assert err <= tol, (dtype, M, N, K, float(err))
+
+
+def test_tile_program_integer_bit_and_conversion_ops_are_exact():
+    """The op classes of test_core's whitelisted test_bin_op / test_bitwise_op / test_shift_op / test_umulhi / test_abs /
+    test_clamp / test_floordiv / test_precise_math (python/examples/conftest.py:48-91), bit for bit against numpy."""
+    import extra_kernels as X
+    import op_zoo
+    n = 1000
+    x, y = op_zoo.int_inputs(n)
+    out = torch.zeros(12 * n, dtype=torch.int32, device=DEV)
+    k = X.int_ops[(4,)](torch.from_numpy(x).to(DEV), torch.from_numpy(y).to(DEV), out, n, BLOCK=256)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    got, want = out.cpu().numpy().reshape(12, n), op_zoo.int_expected(x, y)
+    for plane in range(12):
+        assert np.array_equal(got[plane], want[plane]), plane
+    xf, yf = op_zoo.float_inputs(n)
+    outf = torch.zeros(8 * n, device=DEV)
+    X.float_ops[(4,)](torch.from_numpy(xf).to(DEV), torch.from_numpy(yf).to(DEV), outf, n, -50.0, 75.5, BLOCK=256)
+    torch.cuda.synchronize()
+    gotf, wantf = outf.cpu().numpy().reshape(8, n), op_zoo.float_expected(xf, yf, -50.0, 75.5)
+    for plane in range(8):
+        assert np.array_equal(gotf[plane], wantf[plane]), plane

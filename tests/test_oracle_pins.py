@@ -276,3 +276,23 @@ def test_lanes_on_the_reference_functional_cases():
             for _kind, arg, offsets in program:
                 o = np.asarray(offsets)
                 assert o.size == 0 or (o.min() >= 0 and o.max() < arrays[arg].size), (case["name"], arg)
+
+
+def test_lanes_integer_bit_and_conversion_ops_against_numpy():
+    """Unsigned division / remainder / compare / max, shifts, umulhi, abs, bit casts, float <-> integer conversions, clamp,
+    correctly rounded sqrt / divide and fma: every plane bit for bit against tests/op_zoo.py."""
+    import extra_kernels as X
+    import op_zoo
+    from test_planner import compile_ttir
+    n = 1000
+    x, y = op_zoo.int_inputs(n)
+    t = compile_ttir(X.int_ops, {"x_ptr": "*i32", "y_ptr": "*i32", "out_ptr": "*i32", "n": "i32", "BLOCK": "constexpr"}, {"BLOCK": 256})
+    out = np.zeros(12 * n, np.int32)
+    ttir_lanes.Interpreter(t).run((4,), [None, None, None, n], {0: x, 1: y, 2: out})
+    assert np.array_equal(out.reshape(12, n), op_zoo.int_expected(x, y))
+    xf, yf = op_zoo.float_inputs(n)
+    sig = {"x_ptr": "*fp32", "y_ptr": "*fp32", "out_ptr": "*fp32", "n": "i32", "lo": "fp32", "hi": "fp32", "BLOCK": "constexpr"}
+    t = compile_ttir(X.float_ops, sig, {"BLOCK": 256})
+    outf = np.zeros(8 * n, np.float32)
+    ttir_lanes.Interpreter(t).run((4,), [None, None, None, n, -50.0, 75.5], {0: xf, 1: yf, 2: outf})
+    assert np.array_equal(outf.reshape(8, n), op_zoo.float_expected(xf, yf, -50.0, 75.5))

@@ -202,8 +202,9 @@ hipError_t rtc_compile(const std::string &source, const char *entry, RtcModule *
     delete m;
     return hipErrorUnknown;
   }
-  const char *opts[] = {"--offload-arch=gfx950", "-O3", "-ffp-contract=off"};
-  hiprtcResult r = hiprtcCompileProgram(prog, 3, opts);
+  // no contraction into fmas, IEEE division and square root: the reference's loops are plain scalar C semantics
+  const char *opts[] = {"--offload-arch=gfx950", "-O3", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt"};
+  hiprtcResult r = hiprtcCompileProgram(prog, 4, opts);
   if (r != HIPRTC_SUCCESS) {
     size_t n = 0;
     hiprtcGetProgramLogSize(prog, &n);

@@ -1002,9 +1002,17 @@ class Lowerer {
       if (op.operands.size() != 3) throw Unsupported("tt.dot without an accumulator operand");
       return emit_simple(op, SK::Dot, "", op.operands);
     }
-    if (n.rfind("arith.", 0) == 0 || n.rfind("math.", 0) == 0) {
+    static const std::set<std::string> tt_elementwise = {"tt.bitcast", "tt.clampf", "tt.mulhiui", "tt.precise_sqrt", "tt.precise_divf"};
+    if (n.rfind("arith.", 0) == 0 || n.rfind("math.", 0) == 0 || tt_elementwise.count(n)) {
       std::string name = n;
       if (n == "arith.cmpi" || n == "arith.cmpf") name += "." + op.words.at(0);
+      if (n == "tt.clampf") {  // propagateNan = none | all
+        bool all = false;
+        for (auto &w : op.words) all = all || w == "all";
+        auto it = op.attrs.find("propagateNan");
+        if (it != op.attrs.end() && it->second.find("all") != std::string::npos) all = true;
+        name += all ? ".all" : ".none";
+      }
       return emit_simple(op, SK::Map, name, op.operands);
     }
     throw Unsupported("operation " + n + " (line " + std::to_string(op.line) + ") has no structured lowering");

@@ -230,6 +230,42 @@ struct Gen {
       const std::string U = rt == "i64" ? "unsigned long long" : "unsigned";
       return "(" + ctype(rt) + ")((" + U + ")" + a[0] + (n == "arith.maxui" ? " > (" : " < (") + U + ")" + a[1] + " ? " + a[0] + " : " + a[1] + ")";
     }
+    {
+      const std::string U = (rt == "i64" || ot == "i64") ? "unsigned long long" : ot == "i8" ? "unsigned char" : ot == "i16" ? "unsigned short" : "unsigned";
+      const int bits = ot == "i64" ? 64 : ot == "i8" ? 8 : ot == "i16" ? 16 : 32;
+      if (n == "arith.divui") { need(2); return "(" + ctype(rt) + ")((" + U + ")" + a[1] + " == 0 ? 0 : (" + U + ")" + a[0] + " / (" + U + ")" + a[1] + ")"; }
+      if (n == "arith.remui") { need(2); return "(" + ctype(rt) + ")((" + U + ")" + a[1] + " == 0 ? 0 : (" + U + ")" + a[0] + " % (" + U + ")" + a[1] + ")"; }
+      // shifts by the width or more are undefined in the source dialect; the amount is taken modulo the width here
+      const std::string amount = "((" + U + ")" + (a.size() > 1 ? a[1] : std::string("0")) + " & " + std::to_string(bits - 1) + ")";
+      if (n == "arith.shli") { need(2); return "(" + ctype(rt) + ")((" + U + ")" + a[0] + " << " + amount + ")"; }
+      if (n == "arith.shrui") { need(2); return "(" + ctype(rt) + ")((" + U + ")" + a[0] + " >> " + amount + ")"; }
+      if (n == "arith.shrsi") { need(2); return "(" + ctype(rt) + ")(" + a[0] + " >> " + amount + ")"; }
+      static const std::map<std::string, const char *> cmpu = {{"ult", "<"}, {"ule", "<="}, {"ugt", ">"}, {"uge", ">="}};
+      if (n.rfind("arith.cmpi.", 0) == 0 && cmpu.count(n.substr(11))) {
+        need(2);
+        return "(" + U + ")" + a[0] + " " + cmpu.at(n.substr(11)) + " (" + U + ")" + a[1];
+      }
+      if (n == "arith.uitofp") { need(1); return fl("(float)(" + U + ")" + a[0]); }
+      if (n == "arith.fptoui") { need(1); return "(" + ctype(rt) + ")(" + (rt == "i64" ? std::string("unsigned long long") : std::string("unsigned")) + ")" + a[0]; }
+      if (n == "tt.mulhiui") {
+        need(2);
+        if (rt == "i64") return "(long long)__umul64hi((unsigned long long)" + a[0] + ", (unsigned long long)" + a[1] + ")";
+        return "(int)(((unsigned long long)(unsigned)" + a[0] + " * (unsigned long long)(unsigned)" + a[1] + ") >> 32)";
+      }
+      if (n == "math.absi") { need(1); return "(" + ctype(rt) + ")(" + a[0] + " < 0 ? (" + U + ")0 - (" + U + ")" + a[0] + " : (" + U + ")" + a[0] + ")"; }
+    }
+    if (n == "tt.bitcast" || n == "arith.bitcast") {
+      need(1);
+      if (is_float(ot) == is_float(rt)) return a[0];                           // same class (signedness only): the bits are the value
+      if (ot != "f32" && rt != "f32") no("a bitcast between 16-bit floats and integers");
+      return is_float(rt) ? "__int_as_float(" + a[0] + ")" : "__float_as_int(" + a[0] + ")";
+    }
+    // correctly rounded whatever the compiler's defaults: the fp64 result rounds to the fp32 one (53 >= 2 * 24 + 2 bits)
+    if (n == "tt.precise_sqrt") { need(1); return fl("(float)sqrt((double)" + a[0] + ")"); }
+    if (n == "tt.precise_divf") { need(2); return fl("(float)((double)" + a[0] + " / (double)" + a[1] + ")"); }
+    if (n == "arith.remf") { need(2); return fl("fmodf(" + a[0] + ", " + a[1] + ")"); }
+    if (n == "tt.clampf.none") { need(3); return fl("fminf(fmaxf(" + a[0] + ", " + a[1] + "), " + a[2] + ")"); }
+    if (n == "tt.clampf.all") { need(3); return fl("minimum_f(maximum_f(" + a[0] + ", " + a[1] + "), " + a[2] + ")"); }
     if (n == "arith.andi") { need(2); return rt == "i1" ? a[0] + " && " + a[1] : "(" + ctype(rt) + ")(" + a[0] + " & " + a[1] + ")"; }
     if (n == "arith.ori") { need(2); return rt == "i1" ? a[0] + " || " + a[1] : "(" + ctype(rt) + ")(" + a[0] + " | " + a[1] + ")"; }
     if (n == "arith.xori") { need(2); return rt == "i1" ? a[0] + " != " + a[1] : "(" + ctype(rt) + ")(" + a[0] + " ^ " + a[1] + ")"; }
