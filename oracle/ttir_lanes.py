@@ -311,6 +311,13 @@ class Interpreter:
             if a.base is not None:
                 return Val(np.full(shape, a.d, dtype=np.int64), a.elem, base=a.base)
             return Val(np.full(shape, a.d, dtype=_NP[a.elem]), a.elem)
+        if name == "tt.trans":
+            order = [int(x) for x in re.findall(r"\d+", attrs.get("order", "") or "")]
+            a = ops[0]
+            return Val(np.transpose(a.d, order[-a.d.ndim:] if order else None).copy(), a.elem, base=a.base)
+        if name == "tt.reshape":
+            a = ops[0]
+            return Val(np.reshape(a.d, tys[-1].shape).copy(), a.elem, base=a.base)
         if name == "tt.expand_dims":
             return Val(np.expand_dims(ops[0].d, int(attrs["axis"])), ops[0].elem, ops[0].base)
         if name == "tt.broadcast":

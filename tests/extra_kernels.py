@@ -624,3 +624,25 @@ def float_ops(x_ptr, y_ptr, out_ptr, n, lo, hi, BLOCK: tl.constexpr):
     tl.store(out_ptr + 5 * n + i, x.to(tl.int32, bitcast=True).to(tl.float32), mask=m)   # the bits as an integer
     tl.store(out_ptr + 6 * n + i, tl.floor(x) + tl.ceil(y), mask=m)
     tl.store(out_ptr + 7 * n + i, tl.fma(x, y, x), mask=m)
+
+
+# ---- shape ops (test_core's whitelisted test_trans_2d / test_transpose and reshapes between ranks 1 and 2)
+@triton.jit
+def transpose_tile(src, dst, R: tl.constexpr, C: tl.constexpr):
+    # dst[C, R] = src[R, C]^T with a bias that depends on the destination column, so a wrong index order shows
+    r = tl.arange(0, R)
+    c = tl.arange(0, C)
+    x = tl.load(src + r[:, None] * C + c[None, :])
+    y = tl.trans(x) + r[None, :].to(tl.float32)
+    tl.store(dst + c[:, None] * R + r[None, :], y)
+
+
+@triton.jit
+def fold_and_sum(src, dst, R: tl.constexpr, C: tl.constexpr):
+    # a flat block of R*C elements viewed as [R, C], summed along the columns, and written back flat after scaling
+    i = tl.arange(0, R * C)
+    x = tl.load(src + i)
+    m = tl.reshape(x, (R, C))
+    s = tl.sum(m, axis=1)
+    tl.store(dst + tl.arange(0, R), s)
+    tl.store(dst + R + i, tl.reshape(m * 2.0, (R * C,)))

@@ -858,3 +858,21 @@ def test_tile_program_integer_bit_and_conversion_ops_are_exact():
     gotf, wantf = outf.cpu().numpy().reshape(8, n), op_zoo.float_expected(xf, yf, -50.0, 75.5)
     for plane in range(8):
         assert np.array_equal(gotf[plane], wantf[plane]), plane
+
+
+def test_tile_program_transpose_and_reshape():
+    import extra_kernels as X
+    torch.manual_seed(13)
+    for R, C in [(16, 32), (32, 32)]:                     # the square case: same block shape on both sides of the transpose
+        x = torch.randn(R, C, device=DEV)
+        y = torch.zeros(C, R, device=DEV)
+        k = X.transpose_tile[(1,)](x, y, R=R, C=C)
+        torch.cuda.synchronize()
+        assert k.function.family == "tile_program"
+        assert torch.equal(y, x.t() + torch.arange(R, device=DEV, dtype=torch.float32)[None, :])
+    x = torch.randn(512, device=DEV)
+    y = torch.zeros(8 + 512, device=DEV)
+    X.fold_and_sum[(1,)](x, y, R=8, C=64)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(y[:8], x.reshape(8, 64).double().sum(1).float(), rtol=1e-5, atol=1e-5)
+    assert torch.equal(y[8:], x * 2)

@@ -296,3 +296,20 @@ def test_lanes_integer_bit_and_conversion_ops_against_numpy():
     outf = np.zeros(8 * n, np.float32)
     ttir_lanes.Interpreter(t).run((4,), [None, None, None, n, -50.0, 75.5], {0: xf, 1: yf, 2: outf})
     assert np.array_equal(outf.reshape(8, n), op_zoo.float_expected(xf, yf, -50.0, 75.5))
+
+
+def test_lanes_transpose_and_reshape_against_numpy():
+    import extra_kernels as X
+    from test_planner import compile_ttir
+    P = "*fp32"
+    for R, C in [(16, 32), (32, 32)]:
+        t = compile_ttir(X.transpose_tile, {"src": P, "dst": P, "R": "constexpr", "C": "constexpr"}, {"R": R, "C": C})
+        x = np.random.default_rng(0).standard_normal((R, C)).astype(np.float32)
+        y = np.zeros(R * C, np.float32)
+        ttir_lanes.Interpreter(t).run((1,), [None, None], {0: x.reshape(-1).copy(), 1: y})
+        assert np.array_equal(y.reshape(C, R), x.T + np.arange(R, dtype=np.float32)[None, :])
+    t = compile_ttir(X.fold_and_sum, {"src": P, "dst": P, "R": "constexpr", "C": "constexpr"}, {"R": 8, "C": 64})
+    x = np.random.default_rng(1).standard_normal(512).astype(np.float32)
+    y = np.zeros(8 + 512, np.float32)
+    ttir_lanes.Interpreter(t).run((1,), [None, None], {0: x.copy(), 1: y})
+    assert np.abs(y[:8] - x.reshape(8, 64).astype(np.float64).sum(1)).max() < 1e-5 and np.array_equal(y[8:], x * 2)

@@ -1002,6 +1002,22 @@ class Lowerer {
       if (op.operands.size() != 3) throw Unsupported("tt.dot without an accumulator operand");
       return emit_simple(op, SK::Dot, "", op.operands);
     }
+    if (n == "tt.trans" || n == "tt.reshape") {  // index shuffles: a Map whose element (i, j) reads another element of its operand
+      if (n == "tt.trans") {
+        auto it = op.attrs.find("order");
+        std::string order = it == op.attrs.end() ? "" : it->second;
+        std::string digits;
+        for (char ch : order.substr(order.find(':') == std::string::npos ? 0 : order.find(':')))
+          if (isdigit((unsigned char)ch)) digits += ch;
+        if (rt.shape.size() != 2 || (digits != "10" && digits != "3210")) {
+          // "array<i32: 1, 0>" -> "3210" when the type's digits are kept, "10" otherwise
+          if (rt.shape.size() != 2) throw Unsupported("tt.trans of a block of rank " + std::to_string(rt.shape.size()));
+        }
+      } else if (rt.shape.size() > 2 || def(op.operands.at(0)).type.shape.size() > 2) {
+        throw Unsupported("tt.reshape beyond rank 2 (line " + std::to_string(op.line) + ")");
+      }
+      return emit_simple(op, SK::Map, n, {op.operands.at(0)});
+    }
     static const std::set<std::string> tt_elementwise = {"tt.bitcast", "tt.clampf", "tt.mulhiui", "tt.precise_sqrt", "tt.precise_divf"};
     if (n.rfind("arith.", 0) == 0 || n.rfind("math.", 0) == 0 || tt_elementwise.count(n)) {
       std::string name = n;

@@ -104,7 +104,12 @@ struct Gen {
   // C expression for element (i0, i1) of value v; rank-1 values use i0, scalars neither
   std::string at(int v, const std::string &i0, const std::string &i1) {
     auto it = var.find(v);
-    if (it != var.end()) return it->second;
+    if (it != var.end()) {
+      // a named value is the element the thread owns in the current loop; any other element (behind a transpose or a
+      // reshape) is computed again from its definition
+      const auto &sh = val(v).shape;
+      if (sh.empty() || (i0 == cur_i0 && (sh.size() < 2 || i1 == cur_i1))) return it->second;
+    }
     auto d = def.find(v);
     if (d == def.end()) no("a loop-carried block value used in a loop over another block shape");
     const SOp &s = *d->second;
@@ -161,6 +166,17 @@ struct Gen {
         return arr + "[" + i0 + " * " + std::to_string(V.shape[1]) + " + " + i1 + "]";
       }
       case SK::Map: {
+        if (s.name == "tt.trans") {  // rank 2, order (1, 0)
+          const Value &O = val(s.operands.at(0));
+          if (O.shape.size() != 2 || V.shape.size() != 2) no("tt.trans of a block that is not of rank 2");
+          return at(s.operands[0], i1, i0);
+        }
+        if (s.name == "tt.reshape") {  // row-major element order is kept
+          const Value &O = val(s.operands.at(0));
+          const std::string lin = V.shape.size() == 2 ? "(" + i0 + " * " + std::to_string(V.shape[1]) + " + " + i1 + ")" : V.shape.size() == 1 ? i0 : "0";
+          if (O.shape.size() == 2) return at(s.operands[0], "(" + lin + " / " + std::to_string(O.shape[1]) + ")", "(" + lin + " % " + std::to_string(O.shape[1]) + ")");
+          return at(s.operands[0], O.shape.empty() ? "0" : lin, "0");
+        }
         std::vector<std::string> a;
         for (int o : s.operands) {
           const Value &O = val(o);
@@ -339,8 +355,11 @@ struct Gen {
   }
   static std::string idx0(const std::vector<int64_t> &shape) { return shape.size() == 2 ? "(t / " + std::to_string(shape[1]) + ")" : "t"; }
   static std::string idx1(const std::vector<int64_t> &shape) { return shape.size() == 2 ? "(t % " + std::to_string(shape[1]) + ")" : "0"; }
+  std::string cur_i0, cur_i1;  // the index expressions of the element loop being written
   void open_element_loop(const std::vector<int64_t> &shape) {
     const int64_t T = count(shape);
+    cur_i0 = idx0(shape);
+    cur_i1 = idx1(shape);
     os << pad() << "for (int n = 0; n < " << (T + 255) / 256 << "; n++) {\n";
     indent++;
     os << pad() << "const int t = threadIdx.x + 256 * n;\n" << pad() << "if (t >= " << T << ") break;\n";
@@ -414,7 +433,14 @@ struct Gen {
       // a run of block ops up to the next loop, scalar access or reduction.  Its block shape is that of its stores (else
       // of its largest load); loads of other shapes are read where they are used.
       size_t end = k;
-      while (end < ops.size() && !is_break(ops[end])) end++;
+      {
+        const std::vector<int64_t> *first_store = nullptr;  // stores of another block shape start a run of their own
+        for (; end < ops.size() && !is_break(ops[end]); end++)
+          if (ops[end].kind == SK::Store) {
+            if (first_store && ops[end].acc.sizes != *first_store) break;
+            first_store = &ops[end].acc.sizes;
+          }
+      }
       std::vector<int64_t> shape;
       bool have = false, stores = false;
       for (size_t q = k; q < end; q++)
@@ -472,6 +498,8 @@ struct Gen {
           os << pad() << "for (int t = threadIdx.x; t < " << T << "; t += 256) {\n";
           indent++;
           map_vars({-1});
+          cur_i0 = i0;
+          cur_i1 = i1;
           for (size_t q = k; q < end; q++)
             if (own(ops[q])) {
               std::string name = "v" + std::to_string(ops[q].result);
