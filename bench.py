@@ -8,8 +8,8 @@ through the C ABI (tts_launch) on torch's current stream, on a plan compiled by
 the unchanged Triton frontend.  Inputs live in HBM before the timed region; the
 buffers of consecutive steps rotate over enough copies (> 600 MB) that a step
 does not find its input in the 256 MB Infinity Cache left by the previous one.
-Prints ONE JSON line.  The headline workload is BASELINE.json's configs[1]
-(row softmax, fp32 [4096, 781]); the other four configs and two steady-state
+Prints ONE JSON line.  The headline workload is the row softmax, fp32 [4096, 781]
+(the second of the five configurations); the other four configs and two steady-state
 sizes are reported in "kernels".
 
 Per kernel: `us` = mean kernel duration from HIP events around the timed

@@ -2,7 +2,7 @@
 through the C ABI (tts_launch): either from the unchanged Triton frontend with
 HIPDriver active, or directly on a plan handle.
 
-Bars (BASELINE.json): bit-exact for fp32 elementwise and all index/mask handling;
+Bars: bit-exact for fp32 elementwise and all index/mask handling;
 max-abs <= 1e-5 for fp32 softmax; <= 1e-2 for fp16 LayerNorm; relative Frobenius
 error <= 1e-2 for the bf16 and int8-weight GEMMs."""
 import numpy as np
