@@ -148,8 +148,13 @@ struct Gen {
         return at(s.operands[0], O.shape[0] == 1 ? "0" : i0, O.shape[1] == 1 ? "0" : i1);
       }
       case SK::Load: {
-        // a load that is not of the body's block shape (an index vector, a row of scales) is read where it is used;
-        // body() has checked that nothing in the program stores to its base
+        // a load that is not of the run's block shape (an index vector, a row of scales): from its copy in LDS when the
+        // run staged one, else read where it is used (the program is then refused if anything stores to its base)
+        auto st = staged.find(v);
+        if (st != staged.end()) {
+          if (V.shape.size() == 2) return st->second + "[" + i0 + " * " + std::to_string(V.shape[1]) + " + " + i1 + "]";
+          return st->second + "[" + i0 + "]";
+        }
         all_inline_bases.insert(s.acc.base_arg);
         std::string pred, addr = address(s.acc, i0, i1, pred);
         const std::string rd = mem_read(s.acc, addr);
@@ -345,6 +350,7 @@ struct Gen {
   // Values that a thread keeps for the elements it owns (element t + 256 n of the value's shape in slot n): the loads of
   // two-phase runs and loop-carried blocks.  They can be named only inside an element loop over the same shape;
   // elsewhere a load is read again in place and a carried block is refused.
+  std::map<int, std::string> staged;  // load of another shape than its run's -> LDS array holding the whole block
   struct Held { std::string name; std::vector<int64_t> shape; };
   std::map<int, Held> held;
   void map_vars(const std::vector<int64_t> &shape) {
@@ -360,7 +366,7 @@ struct Gen {
     const int64_t T = count(shape);
     cur_i0 = idx0(shape);
     cur_i1 = idx1(shape);
-    os << pad() << "for (int n = 0; n < " << (T + 255) / 256 << "; n++) {\n";
+    os << pad() << "#pragma unroll\n" << pad() << "for (int n = 0; n < " << (T + 255) / 256 << "; n++) {\n";
     indent++;
     os << pad() << "const int t = threadIdx.x + 256 * n;\n" << pad() << "if (t >= " << T << ") break;\n";
     map_vars(shape);
@@ -466,6 +472,27 @@ struct Gen {
         os << pad() << target << " = " << (pred.empty() ? mem_read(o.acc, addr) : "(" + pred + ") ? " + mem_read(o.acc, addr) + " : " + other_of(o.acc))
            << ";\n";
       };
+      // Loads of another shape are small blocks used through broadcasts (an index vector, a row of scales).  Read in
+      // place they would sit in the address computation of the run's own loads, and every one of those would wait for
+      // the one before it (loads complete in order): copy them to LDS first, at the place in the program where they stand.
+      for (size_t q = k; q < end; q++) {
+        const SOp &o = ops[q];
+        if (o.kind != SK::Load || own(o) || staged.count(o.result)) continue;
+        const size_t bytes = (size_t)count(o.acc.sizes) * held_bytes(val(o.result).dtype);
+        if (count(o.acc.sizes) > TWO_PHASE_MAX || pool_bytes + out_bytes + bytes > 48 * 1024) continue;
+        const std::string name = "blk" + std::to_string(o.result);
+        decl << "  __shared__ " << ctype(val(o.result).dtype) << " " << name << "[" << count(o.acc.sizes) << "];\n";
+        out_bytes += (bytes + 15) / 16 * 16;
+        open_element_loop(o.acc.sizes);
+        {
+          std::string pred, addr = address(o.acc, idx0(o.acc.sizes), idx1(o.acc.sizes), pred);
+          os << pad() << name << "[t] = " << (pred.empty() ? mem_read(o.acc, addr) : "(" + pred + ") ? " + mem_read(o.acc, addr) + " : " + other_of(o.acc))
+             << ";\n";
+        }
+        close_loop();
+        os << pad() << "__syncthreads();\n";
+        staged[o.result] = name;
+      }
       if (two_phase) {
         bool any_load = false;
         for (size_t q = k; q < end; q++)
@@ -699,6 +726,74 @@ struct Gen {
     const int64_t CH = (L + SEG - 1) / SEG, NSEG = scan ? (L + CH - 1) / CH : SEG, PS = O * NSEG;
     const std::string fname = "comb" + id;
     combiner(s, fname);
+    // Lines along the contiguous dimension whose length is a multiple of the workgroup size: every thread owns
+    // L / 256 elements of each line.  It folds those in registers, the wavefront folds its 64 partials with a butterfly
+    // of lane exchanges, and one LDS round trip folds the four wavefronts: no staging of the block.
+    if (!scan && L % 256 == 0 && (rank == 1 || s.axis == 1)) {
+      std::vector<std::string> Tn(k);
+      size_t off = 0;
+      os << pad() << "__syncthreads();\n";
+      for (size_t j = 0; j < k; j++) {
+        Tn[j] = ctype(val(s.operands[j]).dtype);
+        const size_t sz = held_bytes(val(s.operands[j]).dtype);
+        os << pad() << Tn[j] << " *const wp" << id << "_" << j << " = (" << Tn[j] << " *)(pool + " << off << ");\n";
+        off = (off + O * 4 * sz + 15) / 16 * 16;
+        decl << "  __shared__ " << Tn[j] << " out" << id << "_" << j << "[" << O << "];\n";
+        out_bytes += (O * sz + 15) / 16 * 16;
+      }
+      pool_bytes = std::max(pool_bytes, off);
+      auto list = [&](const std::string &pre, const std::string &post) {
+        std::string r;
+        for (size_t j = 0; j < k; j++) r += (j ? ", " : "") + pre + std::to_string(j) + post;
+        return r;
+      };
+      auto final_value = [&](size_t j, const std::string &e) {
+        const std::string &dt = val(s.operands[j]).dtype;
+        return s.body.empty() && s.name == "arith.addf" ? rounded(dt, e) : e;
+      };
+      const int64_t LQ = L / 256;
+      map_vars(shape);
+      cur_i0 = i0;
+      cur_i1 = i1;
+      os << pad() << "#pragma unroll\n" << pad() << "for (int o = 0; o < " << O << "; o++) {\n";
+      indent++;
+      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << ";\n";
+      os << pad() << "#pragma unroll\n" << pad() << "for (int q = 0; q < " << LQ << "; q++) {\n";
+      indent++;
+      os << pad() << "const int n = o * " << LQ << " + q;\n" << pad() << "const int t = threadIdx.x + 256 * n;\n";
+      for (size_t j = 0; j < k; j++) os << pad() << "const " << Tn[j] << " el" << j << " = " << at(s.operands[j], i0, i1) << ";\n";
+      os << pad() << "if (q == 0) { ";
+      for (size_t j = 0; j < k; j++) os << "acc" << j << " = el" << j << "; ";
+      os << "} else " << fname << "(" << list("acc", "") << ", " << list("el", "") << ", " << list("acc", "") << ");\n";
+      indent--;
+      os << pad() << "}\n";
+      os << pad() << "#pragma unroll\n" << pad() << "for (int m = 32; m >= 1; m >>= 1) {\n";
+      indent++;
+      for (size_t j = 0; j < k; j++) {
+        const std::string &dt = val(s.operands[j]).dtype;
+        const bool narrow = dt == "i1" || dt == "i8" || dt == "i16";
+        os << pad() << "const " << Tn[j] << " ot" << j << " = " << (narrow ? "(" + Tn[j] + ")__shfl_xor((int)acc" + std::to_string(j) + ", m)"
+                                                                          : "__shfl_xor(acc" + std::to_string(j) + ", m)") << ";\n";
+      }
+      os << pad() << fname << "(" << list("acc", "") << ", " << list("ot", "") << ", " << list("acc", "") << ");\n";
+      indent--;
+      os << pad() << "}\n";
+      os << pad() << "if ((threadIdx.x & 63) == 0) { ";
+      for (size_t j = 0; j < k; j++) os << "wp" << id << "_" << j << "[o * 4 + (threadIdx.x >> 6)] = acc" << j << "; ";
+      os << "}\n";
+      indent--;
+      os << pad() << "}\n" << pad() << "__syncthreads();\n";
+      os << pad() << "for (int o = threadIdx.x; o < " << O << "; o += 256) {\n";
+      indent++;
+      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << " = wp" << id << "_" << j << "[o * 4];\n";
+      os << pad() << "for (int w = 1; w < 4; w++) " << fname << "(" << list("acc", "") << ", " << list("wp" + id + "_", "[o * 4 + w]") << ", " << list("acc", "") << ");\n";
+      for (size_t j = 0; j < k; j++) os << pad() << "out" << id << "_" << j << "[o] = " << final_value(j, "acc" + std::to_string(j)) << ";\n";
+      indent--;
+      os << pad() << "}\n" << pad() << "__syncthreads();\n";
+      cur_i0.clear();
+      cur_i1.clear();
+      return;
+    }
     // LDS: staging and partials in the shared pool, results in arrays of their own
     std::vector<std::string> Tn(k);
     size_t off = 0;
