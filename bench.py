@@ -181,7 +181,8 @@ def make_workloads(torch, triton, K):
         def make():
             x = torch.randn(rows, cols, device=dev)
             out = torch.empty(rows, device=dev)
-            return lambda: K.row_sums[(triton.cdiv(rows, 4),)](x, out, rows, cols, x.stride(0), BR=4, BC=1024)
+            br = int(os.environ.get("TTS_BENCH_BR", "4"))
+            return lambda: K.row_sums[(triton.cdiv(rows, br),)](x, out, rows, cols, x.stride(0), BR=br, BC=1024)
         work = rows * cols * 4 + rows * 4
         r = 256
         cpu = lanes((r // 4,), [r, cols, cols],

@@ -501,16 +501,43 @@ struct Gen {
             any_load = true;
           }
         if (any_load) {
+          // A masked load is written as `if (valid) x = *p;` here and gets its `other` in a second loop: selecting
+          // between the loaded value and `other` on the spot would need the value, and with it a wait for every load
+          // before the next one is issued.
+          std::vector<std::pair<const SOp *, std::string>> fill;  // masked loads whose `other` is still to be filled in
+          auto fill_others = [&]() {
+            if (fill.empty()) return;
+            open_element_loop(shape);
+            for (auto &f : fill) {
+              std::string pred, addr = address(f.first->acc, i0, i1, pred);
+              os << pad() << "if (!(" << pred << ")) " << f.second << "[n] = " << other_of(f.first->acc) << ";\n";
+            }
+            close_loop();
+            fill.clear();
+          };
           open_element_loop(shape);
           for (size_t q = k; q < end; q++)
             if (own(ops[q])) {
               const std::string name = "ld" + std::to_string(ops[q].result);
-              emit_load(ops[q], name + "[n]");
+              std::string pred, addr = address(ops[q].acc, i0, i1, pred);
+              bool needs_filled = false;  // indexed or masked by a load that still lacks its `other`
+              for (auto &f : fill) needs_filled = needs_filled || addr.find(f.second + "[") != std::string::npos || pred.find(f.second + "[") != std::string::npos;
+              if (needs_filled) {
+                close_loop();
+                fill_others();
+                open_element_loop(shape);
+              }
+              if (pred.empty()) os << pad() << name << "[n] = " << mem_read(ops[q].acc, addr) << ";\n";
+              else {
+                os << pad() << "if (" << pred << ") " << name << "[n] = " << mem_read(ops[q].acc, addr) << ";\n";
+                fill.push_back({&ops[q], name});
+              }
               held[ops[q].result] = {name, shape};  // a later load of this run may be indexed by it
               var[ops[q].result] = name + "[n]";
               mine.push_back(ops[q].result);
             }
           close_loop();
+          fill_others();
           os << pad() << "__syncthreads();\n";
         }
         if (stores) open_element_loop(shape);
@@ -788,6 +815,72 @@ struct Gen {
       for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << " = wp" << id << "_" << j << "[o * 4];\n";
       os << pad() << "for (int w = 1; w < 4; w++) " << fname << "(" << list("acc", "") << ", " << list("wp" + id + "_", "[o * 4 + w]") << ", " << list("acc", "") << ");\n";
       for (size_t j = 0; j < k; j++) os << pad() << "out" << id << "_" << j << "[o] = " << final_value(j, "acc" + std::to_string(j)) << ";\n";
+      indent--;
+      os << pad() << "}\n" << pad() << "__syncthreads();\n";
+      cur_i0.clear();
+      cur_i1.clear();
+      return;
+    }
+    // The same lines, scanned: the 64 elements a wavefront owns in one slot are consecutive, so it scans them with lane
+    // exchanges (Hillis-Steele, earlier elements always on the left of the combiner); the totals of the 4 L / 256
+    // pieces of a line meet in LDS, and every piece folds the totals before it into its elements.
+    if (scan && !s.ival && L % 256 == 0 && (rank == 1 || s.axis == 1)) {
+      std::vector<std::string> Tn(k);
+      const int64_t LQ = L / 256, slots = O * LQ;
+      size_t off = 0;
+      os << pad() << "__syncthreads();\n";
+      for (size_t j = 0; j < k; j++) {
+        Tn[j] = ctype(val(s.operands[j]).dtype);
+        const size_t sz = held_bytes(val(s.operands[j]).dtype);
+        os << pad() << Tn[j] << " *const wp" << id << "_" << j << " = (" << Tn[j] << " *)(pool + " << off << ");\n";
+        off = (off + slots * 4 * sz + 15) / 16 * 16;
+        decl << "  __shared__ " << Tn[j] << " out" << id << "_" << j << "[" << T << "];\n";
+        out_bytes += (T * sz + 15) / 16 * 16;
+      }
+      pool_bytes = std::max(pool_bytes, off);
+      auto list = [&](const std::string &pre, const std::string &post) {
+        std::string r;
+        for (size_t j = 0; j < k; j++) r += (j ? ", " : "") + pre + std::to_string(j) + post;
+        return r;
+      };
+      auto shfl = [&](size_t j, const std::string &what) {
+        const std::string &dt = val(s.operands[j]).dtype;
+        const bool narrow = dt == "i1" || dt == "i8" || dt == "i16";
+        return narrow ? "(" + Tn[j] + ")__shfl_up((int)" + what + ", d)" : "__shfl_up(" + what + ", d)";
+      };
+      map_vars(shape);
+      cur_i0 = i0;
+      cur_i1 = i1;
+      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " sc" << id << "_" << j << "[" << slots << "];\n";
+      os << pad() << "#pragma unroll\n" << pad() << "for (int n = 0; n < " << slots << "; n++) {\n";
+      indent++;
+      os << pad() << "const int t = threadIdx.x + 256 * n;\n";
+      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << " = " << at(s.operands[j], i0, i1) << ";\n";
+      os << pad() << "#pragma unroll\n" << pad() << "for (int d = 1; d < 64; d <<= 1) {\n";
+      indent++;
+      for (size_t j = 0; j < k; j++) os << pad() << "const " << Tn[j] << " ot" << j << " = " << shfl(j, "acc" + std::to_string(j)) << ";\n";
+      os << pad() << "if ((threadIdx.x & 63) >= d) " << fname << "(" << list("ot", "") << ", " << list("acc", "") << ", " << list("acc", "") << ");\n";
+      indent--;
+      os << pad() << "}\n";
+      for (size_t j = 0; j < k; j++) os << pad() << "sc" << id << "_" << j << "[n] = acc" << j << ";\n";
+      os << pad() << "if ((threadIdx.x & 63) == 63) { ";
+      for (size_t j = 0; j < k; j++) os << "wp" << id << "_" << j << "[n * 4 + (threadIdx.x >> 6)] = acc" << j << "; ";
+      os << "}\n";
+      indent--;
+      os << pad() << "}\n" << pad() << "__syncthreads();\n";
+      os << pad() << "#pragma unroll\n" << pad() << "for (int n = 0; n < " << slots << "; n++) {\n";
+      indent++;
+      os << pad() << "const int t = threadIdx.x + 256 * n;\n";
+      os << pad() << "const int first = (n / " << LQ << ") * " << LQ * 4 << ", pieces = (n % " << LQ << ") * 4 + (threadIdx.x >> 6);\n";
+      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " res" << j << " = sc" << id << "_" << j << "[n];\n";
+      os << pad() << "if (pieces > 0) {\n";
+      indent++;
+      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " carry" << j << " = wp" << id << "_" << j << "[first];\n";
+      os << pad() << "for (int i = 1; i < pieces; i++) " << fname << "(" << list("carry", "") << ", " << list("wp" + id + "_", "[first + i]") << ", " << list("carry", "") << ");\n";
+      os << pad() << fname << "(" << list("carry", "") << ", " << list("sc" + id + "_", "[n]") << ", " << list("res", "") << ");\n";
+      indent--;
+      os << pad() << "}\n";
+      for (size_t j = 0; j < k; j++) os << pad() << "out" << id << "_" << j << "[t] = res" << j << ";\n";
       indent--;
       os << pad() << "}\n" << pad() << "__syncthreads();\n";
       cur_i0.clear();
