@@ -646,3 +646,23 @@ def fold_and_sum(src, dst, R: tl.constexpr, C: tl.constexpr):
     s = tl.sum(m, axis=1)
     tl.store(dst + tl.arange(0, R), s)
     tl.store(dst + R + i, tl.reshape(m * 2.0, (R * C,)))
+
+
+# ---- extern elementwise functions (the libdevice symbols test/Conversion/TritonToLinalg/convert_extern_elementwise.mlir lists)
+from triton.language.extra.cuda import libdevice as _libdevice  # noqa: E402  (only the symbol names matter: "__nv_powf" ...)
+
+
+@triton.jit
+def extern_math(x_ptr, y_ptr, out_ptr, n, BLOCK: tl.constexpr):
+    # 6 planes: pow, atan2, log1p, tanh via sinh / cosh, trunc, asin of a clamped value
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = i < n
+    x = tl.load(x_ptr + i, mask=m, other=1.0)
+    y = tl.load(y_ptr + i, mask=m, other=1.0)
+    tl.store(out_ptr + 0 * n + i, _libdevice.pow(tl.abs(x), y), mask=m)
+    tl.store(out_ptr + 1 * n + i, _libdevice.atan2(x, y), mask=m)
+    tl.store(out_ptr + 2 * n + i, _libdevice.log1p(tl.abs(x)), mask=m)
+    tl.store(out_ptr + 3 * n + i, _libdevice.sinh(y) / _libdevice.cosh(y), mask=m)
+    tl.store(out_ptr + 4 * n + i, _libdevice.trunc(x), mask=m)
+    tl.store(out_ptr + 5 * n + i, _libdevice.asin(tl.minimum(tl.maximum(y, -1.0), 1.0)), mask=m)
+    tl.device_assert(n > 0, "n must be positive")

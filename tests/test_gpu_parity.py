@@ -876,3 +876,21 @@ def test_tile_program_transpose_and_reshape():
     torch.cuda.synchronize()
     torch.testing.assert_close(y[:8], x.reshape(8, 64).double().sum(1).float(), rtol=1e-5, atol=1e-5)
     assert torch.equal(y[8:], x * 2)
+
+
+def test_tile_program_extern_functions():
+    # libdevice-style functions by symbol name run on the device math library: a few ulp from the float64 values
+    import extra_kernels as X
+    torch.manual_seed(14)
+    n = 500
+    x = torch.randn(n, device=DEV) * 3
+    y = torch.randn(n, device=DEV)
+    out = torch.zeros(6 * n, device=DEV)
+    k = X.extern_math[(2,)](x, y, out, n, BLOCK=256)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    xd, yd = x.double().cpu(), y.double().cpu()
+    want = torch.stack([xd.abs() ** yd, torch.atan2(xd, yd), torch.log1p(xd.abs()), torch.tanh(yd), torch.trunc(xd), torch.asin(yd.clamp(-1, 1))])
+    got = out.cpu().double().reshape(6, n)
+    err = (got - want).abs().amax(1) / want.abs().amax(1)
+    assert (err <= 1e-6).all(), err

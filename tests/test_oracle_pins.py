@@ -313,3 +313,20 @@ def test_lanes_transpose_and_reshape_against_numpy():
     y = np.zeros(8 + 512, np.float32)
     ttir_lanes.Interpreter(t).run((1,), [None, None], {0: x.copy(), 1: y})
     assert np.abs(y[:8] - x.reshape(8, 64).astype(np.float64).sum(1)).max() < 1e-5 and np.array_equal(y[8:], x * 2)
+
+
+def test_lanes_extern_functions_against_float64():
+    """tt.extern_elementwise by symbol name (test/Conversion/TritonToLinalg/convert_extern_elementwise.mlir): each plane
+    within 2e-7 relative of the float64 value."""
+    import extra_kernels as X
+    from test_planner import compile_ttir
+    t = compile_ttir(X.extern_math, {"x_ptr": "*fp32", "y_ptr": "*fp32", "out_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"}, {"BLOCK": 256})
+    rng = np.random.default_rng(0)
+    n = 500
+    x = (rng.standard_normal(n) * 3).astype(np.float32)
+    y = rng.standard_normal(n).astype(np.float32)
+    out = np.zeros(6 * n, np.float32)
+    ttir_lanes.Interpreter(t).run((2,), [None, None, None, n], {0: x, 1: y, 2: out})
+    x64, y64 = x.astype(np.float64), y.astype(np.float64)
+    want = np.stack([np.abs(x64) ** y64, np.arctan2(x64, y64), np.log1p(np.abs(x64)), np.tanh(y64), np.trunc(x64), np.arcsin(np.clip(y64, -1, 1))])
+    assert (np.abs(out.reshape(6, n) - want).max(axis=1) <= 2e-7 * np.abs(want).max(axis=1)).all()

@@ -960,7 +960,7 @@ class Lowerer {
         defs_[op.results[i]] = d;
       }
     const std::string &n = op.name;
-    if (n == "tt.return") return;
+    if (n == "tt.return" || n == "tt.assert") return;  // assertions are dropped, as the reference does (triton_assert.mlir)
     if (n == "scf.for") return lower_for(op);
     if (n == "cf.if" || n == "scf.if") return lower_if(op);
     if (n == "tt.load") return lower_load(op);
@@ -1001,6 +1001,14 @@ class Lowerer {
     if (n == "tt.dot") {  // ConversionPatterns.hpp:1128-1201
       if (op.operands.size() != 3) throw Unsupported("tt.dot without an accumulator operand");
       return emit_simple(op, SK::Dot, "", op.operands);
+    }
+    if (n == "tt.extern_elementwise") {  // a libdevice-style function by name (convert_extern_elementwise.mlir)
+      auto it = op.attrs.find("symbol");
+      if (it == op.attrs.end()) throw Unsupported("tt.extern_elementwise without a symbol (line " + std::to_string(op.line) + ")");
+      std::string sym;
+      for (char ch : it->second)
+        if (isalnum((unsigned char)ch) || ch == '_') sym += ch;
+      return emit_simple(op, SK::Map, "extern." + sym, op.operands);
     }
     if (n == "tt.trans" || n == "tt.reshape") {  // index shuffles: a Map whose element (i, j) reads another element of its operand
       if (n == "tt.trans") {

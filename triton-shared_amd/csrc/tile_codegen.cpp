@@ -275,6 +275,16 @@ struct Gen {
       }
       if (n == "math.absi") { need(1); return "(" + ctype(rt) + ")(" + a[0] + " < 0 ? (" + U + ")0 - (" + U + ")" + a[0] + " : (" + U + ")" + a[0] + ")"; }
     }
+    if (n.rfind("extern.__nv_", 0) == 0) {  // the fp32 libdevice names: the device math library's function of the same name
+      static const std::set<std::string> fns = {"acosf", "acoshf", "asinf", "asinhf", "atan2f", "atanf", "atanhf", "ceilf", "cosf", "coshf",
+                                                "erff", "exp2f", "expf", "fabsf", "floorf", "log10f", "log1pf", "logf", "log2f", "powf",
+                                                "rsqrtf", "sinf", "sinhf", "sqrtf", "tanf", "tanhf", "truncf", "fmodf", "expm1f", "cbrtf"};
+      const std::string fn = n.substr(12);
+      if (!fns.count(fn) || rt != "f32") no("extern function " + n.substr(7));
+      std::string call = fn + "(";
+      for (size_t q = 0; q < a.size(); q++) call += (q ? ", " : "") + a[q];
+      return call + ")";
+    }
     if (n == "tt.bitcast" || n == "arith.bitcast") {
       need(1);
       if (is_float(ot) == is_float(rt)) return a[0];                           // same class (signedness only): the bits are the value
