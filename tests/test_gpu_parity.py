@@ -580,7 +580,7 @@ def test_errors_surface_as_python_exceptions(K):
         K.vec_add[(1,)](torch.zeros(1024), x, x, 1024, BLOCK=1024)     # host tensor
     with pytest.raises(NotImplementedError):
         X.atomic_accumulate[(4,)](x, x, 1024, BLOCK=256)               # no structured lowering: refused, no fallback
-    with pytest.raises(NotImplementedError, match="more than 4096 outputs"):
+    with pytest.raises(NotImplementedError, match="bytes of LDS"):
         big = torch.zeros(128 * 128, device=DEV)
         X.small_dot[(1,)](big, big, big, B=128)                        # a large product outside the tiled matmul shapes
     with pytest.raises(NotImplementedError, match="one program per output tile"):
@@ -894,3 +894,21 @@ def test_tile_program_extern_functions():
     got = out.cpu().double().reshape(6, n)
     err = (got - want).abs().amax(1) / want.abs().amax(1)
     assert (err <= 1e-6).all(), err
+
+
+def test_tile_program_large_blocks():
+    """Blocks of up to 16384 elements are held in registers (64 per thread): a one-dimensional block of 8192 reduced and
+    rescaled, and a 64 x 128 block reduced along its rows through the LDS-staged path."""
+    import extra_kernels as X
+    torch.manual_seed(15)
+    x = torch.randn(3, 8000, device=DEV)
+    y = torch.zeros_like(x)
+    k = X.centre_rows[(3,)](x, y, 8000, x.stride(0), BC=8192)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    torch.testing.assert_close(y, x - x.mean(1, keepdim=True), rtol=1e-5, atol=2e-5)
+    x = torch.randn(100, 100, device=DEV)
+    out = torch.zeros(100, device=DEV)
+    X.reduce_rows_2d[(2,)](x, out, 100, 100, x.stride(0), BR=64, BC=128, KIND=0)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out, x.sum(1), rtol=1e-5, atol=2e-5)

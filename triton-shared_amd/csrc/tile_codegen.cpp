@@ -11,7 +11,7 @@
 //
 // Order of memory effects.  The reference finishes every load of a body before the op after it
 // starts.  A fused element loop keeps that order per element only, which differs when a store
-// writes what another element's load reads (an in-place shift).  Tiles of up to 4096 elements are
+// writes what another element's load reads (an in-place shift).  Tiles of up to 16384 elements are
 // therefore run in two phases -- every load of the body into per-thread registers, a barrier,
 // then ops and stores; larger tiles are fused in one loop and accepted only when no store's base
 // argument is also a load's.
@@ -26,7 +26,7 @@ namespace tts {
 
 namespace {
 
-constexpr int64_t TWO_PHASE_MAX = 4096;  // elements; 16 per thread
+constexpr int64_t TWO_PHASE_MAX = 16384;  // elements; 64 registers per thread and held block value
 
 struct Gen {
   const Program &P;
@@ -609,7 +609,7 @@ struct Gen {
   void loop(const SOp &s) {
     const std::string L = std::to_string(s.loop);
     // loop-carried block values live in per-thread arrays (element-wise programs never move a value between
-    // elements, so each thread carries the elements it owns); all of them must have one shape of <= 4096 elements
+    // elements, so each thread carries the elements it owns); all of them must have one shape of <= 16384 elements
     std::vector<int64_t> cshape;
     for (size_t q = 0; q < s.tile_args.size(); q++) {
       const Value &V = val(s.tile_args[q]);
