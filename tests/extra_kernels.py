@@ -666,3 +666,47 @@ def extern_math(x_ptr, y_ptr, out_ptr, n, BLOCK: tl.constexpr):
     tl.store(out_ptr + 4 * n + i, _libdevice.trunc(x), mask=m)
     tl.store(out_ptr + 5 * n + i, _libdevice.asin(tl.minimum(tl.maximum(y, -1.0), 1.0)), mask=m)
     tl.device_assert(n > 0, "n must be positive")
+
+
+# ---- kernels in the style of the Triton tutorials, run by the generic family
+@triton.jit
+def seeded_dropout(x_ptr, out_ptr, n, p, seed, BLOCK: tl.constexpr):
+    # tutorial 04: a Philox random number per element (umulhi, xor, shifts), compare, select, scale
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = i < n
+    x = tl.load(x_ptr + i, mask=m)
+    keep = tl.rand(seed, i) > p
+    tl.store(out_ptr + i, tl.where(keep, x / (1 - p), 0.0), mask=m)
+
+
+@triton.jit
+def rms_norm_rows(x_ptr, w_ptr, y_ptr, pitch, n_cols, eps, BLOCK: tl.constexpr):
+    # y = x / sqrt(mean(x^2) + eps) * w, one row per program, fp16 in and out, fp32 arithmetic
+    row = tl.program_id(0)
+    c = tl.arange(0, BLOCK)
+    m = c < n_cols
+    x = tl.load(x_ptr + row * pitch + c, mask=m, other=0.0).to(tl.float32)
+    w = tl.load(w_ptr + c, mask=m, other=0.0).to(tl.float32)
+    r = 1.0 / tl.sqrt(tl.sum(x * x, axis=0) / n_cols + eps)
+    tl.store(y_ptr + row * pitch + c, (x * r * w).to(tl.float16), mask=m)
+
+
+@triton.jit
+def column_sums_looped(x_ptr, out_ptr, n_rows, n_cols, pitch, BR: tl.constexpr, BC: tl.constexpr):
+    # the shape of the tutorial's LayerNorm backward dw/db kernel: a [BR, BC] accumulator carried down the rows, summed at the end
+    c = tl.program_id(0) * BC + tl.arange(0, BC)
+    acc = tl.zeros((BR, BC), dtype=tl.float32)
+    for r0 in range(0, n_rows, BR):
+        r = r0 + tl.arange(0, BR)
+        m = (r[:, None] < n_rows) & (c[None, :] < n_cols)
+        acc += tl.load(x_ptr + r[:, None] * pitch + c[None, :], mask=m, other=0.0)
+    tl.store(out_ptr + c, tl.sum(acc, axis=0), mask=c < n_cols)
+
+
+@triton.jit
+def log_sum_exp_rows(x_ptr, out_ptr, pitch, n_cols, BLOCK: tl.constexpr):
+    row = tl.program_id(0)
+    c = tl.arange(0, BLOCK)
+    x = tl.load(x_ptr + row * pitch + c, mask=c < n_cols, other=-float("inf"))
+    top = tl.max(x, axis=0)
+    tl.store(out_ptr + row, top + tl.log(tl.sum(tl.exp(x - top), axis=0)))

@@ -912,3 +912,46 @@ def test_tile_program_large_blocks():
     X.reduce_rows_2d[(2,)](x, out, 100, 100, x.stride(0), BR=64, BC=128, KIND=0)
     torch.cuda.synchronize()
     torch.testing.assert_close(out, x.sum(1), rtol=1e-5, atol=2e-5)
+
+
+# ------------------------------------------------------------- tutorial-style kernels on the generic family
+def test_tile_program_seeded_dropout_is_exact():
+    import extra_kernels as X
+    import op_zoo
+    n = 100_000
+    x = torch.randn(n, device=DEV)
+    out = torch.zeros(n, device=DEV)
+    k = X.seeded_dropout[(triton.cdiv(n, 1024),)](x, out, n, 0.3, 1234, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    u = op_zoo.philox_uniform(1234, np.arange(n))
+    xs = x.cpu().numpy()
+    want = np.where(u > np.float32(0.3), xs / (np.float32(1) - np.float32(0.3)), np.float32(0))
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
+def test_tile_program_norms_and_reductions_of_the_tutorials():
+    import extra_kernels as X
+    torch.manual_seed(16)
+    # RMSNorm, fp16 rows of 4000 in blocks of 4096
+    x = torch.randn(7, 4000, device=DEV).half()
+    w = (1 + 0.1 * torch.randn(4000, device=DEV)).half()
+    y = torch.zeros_like(x)
+    k = X.rms_norm_rows[(7,)](x, w, y, x.stride(0), 4000, 1e-6, BLOCK=4096)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    xf = x.float()
+    want = xf / torch.sqrt((xf * xf).mean(1, keepdim=True) + 1e-6) * w.float()
+    assert (y.float() - want).abs().max() <= 1e-2
+    # column sums with a [32, 128] accumulator carried down the rows (the dw / db kernel of the LayerNorm tutorial)
+    a = torch.randn(1000, 300, device=DEV)
+    out = torch.zeros(300, device=DEV)
+    X.column_sums_looped[(triton.cdiv(300, 128),)](a, out, 1000, 300, a.stride(0), BR=32, BC=128)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out, a.double().sum(0).float(), rtol=1e-5, atol=1e-4)
+    # log-sum-exp of rows
+    b = torch.randn(50, 2000, device=DEV) * 5
+    lse = torch.zeros(50, device=DEV)
+    X.log_sum_exp_rows[(50,)](b, lse, b.stride(0), 2000, BLOCK=2048)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(lse, torch.logsumexp(b.double(), 1).float(), rtol=1e-6, atol=1e-5)

@@ -330,3 +330,19 @@ def test_lanes_extern_functions_against_float64():
     x64, y64 = x.astype(np.float64), y.astype(np.float64)
     want = np.stack([np.abs(x64) ** y64, np.arctan2(x64, y64), np.log1p(np.abs(x64)), np.tanh(y64), np.trunc(x64), np.arcsin(np.clip(y64, -1, 1))])
     assert (np.abs(out.reshape(6, n) - want).max(axis=1) <= 2e-7 * np.abs(want).max(axis=1)).all()
+
+
+def test_lanes_philox_dropout_against_an_independent_philox():
+    """tl.rand expands into ~60 integer ops per element (umulhi, xor, shifts, wrapping adds); the oracle's result equals
+    tests/op_zoo.philox_uniform, written from the published algorithm, bit for bit."""
+    import extra_kernels as X
+    import op_zoo
+    from test_planner import compile_ttir
+    sig = {"x_ptr": "*fp32", "out_ptr": "*fp32", "n": "i32", "p": "fp32", "seed": "i32", "BLOCK": "constexpr"}
+    t = compile_ttir(X.seeded_dropout, sig, {"BLOCK": 1024})
+    n = 3000
+    x = np.random.default_rng(0).standard_normal(n).astype(np.float32)
+    out = np.zeros(n, np.float32)
+    ttir_lanes.Interpreter(t).run((3,), [None, None, n, 0.3, 1234], {0: x, 1: out})
+    u = op_zoo.philox_uniform(1234, np.arange(n))
+    assert np.array_equal(out, np.where(u > np.float32(0.3), x / (np.float32(1) - np.float32(0.3)), np.float32(0)))

@@ -492,12 +492,11 @@ class Lowerer {
         expr = int_of(name);
       } catch (const Unsupported &) {
         // not an index expression (it depends on a value read from memory): computed as data, op by op
-        if (!d.op || (d.op->name.rfind("arith.", 0) != 0)) throw;
+        if (!d.op || !is_elementwise(d.op->name)) throw;
         const Op &op = *d.op;
         SOp s;
         s.kind = SK::Map;
-        s.name = op.name;
-        if (op.name == "arith.cmpi" || op.name == "arith.cmpf") s.name += "." + op.words.at(0);
+        s.name = map_name(op);
         for (auto &o : op.operands) s.operands.push_back(data_of(o));
         s.result = new_value(d.type);
         cur_->push_back(s);
@@ -725,6 +724,24 @@ class Lowerer {
       }
     }
     cur_->push_back(s);
+  }
+
+  // Elementwise ops (one result element per operand element) and the name their Map op carries.
+  static bool is_elementwise(const std::string &n) {
+    static const std::set<std::string> tt_ops = {"tt.bitcast", "tt.clampf", "tt.mulhiui", "tt.precise_sqrt", "tt.precise_divf"};
+    return n.rfind("arith.", 0) == 0 || n.rfind("math.", 0) == 0 || tt_ops.count(n) > 0;
+  }
+  static std::string map_name(const Op &op) {
+    std::string name = op.name;
+    if (op.name == "arith.cmpi" || op.name == "arith.cmpf") name += "." + op.words.at(0);
+    if (op.name == "tt.clampf") {  // propagateNan = none | all
+      bool all = false;
+      for (auto &w : op.words) all = all || w == "all";
+      auto it = op.attrs.find("propagateNan");
+      if (it != op.attrs.end() && it->second.find("all") != std::string::npos) all = true;
+      name += all ? ".all" : ".none";
+    }
+    return name;
   }
 
   void emit_simple(const Op &op, SK kind, const std::string &name, std::vector<std::string> operand_names) {
@@ -979,7 +996,8 @@ class Lowerer {
           "tt.get_program_id", "tt.get_num_programs", "arith.addi", "arith.subi", "arith.muli", "arith.divsi",
           "arith.remsi", "arith.minsi", "arith.maxsi", "arith.extsi", "arith.index_cast", "arith.trunci",
           "arith.select", "arith.cmpi"};
-      if (!int_ops.count(n)) throw Unsupported("scalar integer operation " + n + " (line " + std::to_string(op.line) + ")");
+      // the index expressions know the ops above; any other elementwise op on scalars is computed as data when used
+      if (!int_ops.count(n) && !is_elementwise(n)) throw Unsupported("scalar integer operation " + n + " (line " + std::to_string(op.line) + ")");
       return;
     }
     if (n == "tt.make_range") {
@@ -1026,19 +1044,7 @@ class Lowerer {
       }
       return emit_simple(op, SK::Map, n, {op.operands.at(0)});
     }
-    static const std::set<std::string> tt_elementwise = {"tt.bitcast", "tt.clampf", "tt.mulhiui", "tt.precise_sqrt", "tt.precise_divf"};
-    if (n.rfind("arith.", 0) == 0 || n.rfind("math.", 0) == 0 || tt_elementwise.count(n)) {
-      std::string name = n;
-      if (n == "arith.cmpi" || n == "arith.cmpf") name += "." + op.words.at(0);
-      if (n == "tt.clampf") {  // propagateNan = none | all
-        bool all = false;
-        for (auto &w : op.words) all = all || w == "all";
-        auto it = op.attrs.find("propagateNan");
-        if (it != op.attrs.end() && it->second.find("all") != std::string::npos) all = true;
-        name += all ? ".all" : ".none";
-      }
-      return emit_simple(op, SK::Map, name, op.operands);
-    }
+    if (is_elementwise(n)) return emit_simple(op, SK::Map, map_name(op), op.operands);
     throw Unsupported("operation " + n + " (line " + std::to_string(op.line) + ") has no structured lowering");
   }
 
