@@ -1030,15 +1030,13 @@ class Lowerer {
     }
     if (n == "tt.trans" || n == "tt.reshape") {  // index shuffles: a Map whose element (i, j) reads another element of its operand
       if (n == "tt.trans") {
+        // {order = array<i32: 1, 0>}: the digits after the element type
         auto it = op.attrs.find("order");
-        std::string order = it == op.attrs.end() ? "" : it->second;
-        std::string digits;
-        for (char ch : order.substr(order.find(':') == std::string::npos ? 0 : order.find(':')))
+        std::string order = it == op.attrs.end() ? "" : it->second, digits;
+        const size_t colon = order.find(':');
+        for (char ch : order.substr(colon == std::string::npos ? 0 : colon))
           if (isdigit((unsigned char)ch)) digits += ch;
-        if (rt.shape.size() != 2 || (digits != "10" && digits != "3210")) {
-          // "array<i32: 1, 0>" -> "3210" when the type's digits are kept, "10" otherwise
-          if (rt.shape.size() != 2) throw Unsupported("tt.trans of a block of rank " + std::to_string(rt.shape.size()));
-        }
+        if (rt.shape.size() != 2 || digits != "10") throw Unsupported("tt.trans other than the transpose of a rank-2 block (line " + std::to_string(op.line) + ")");
       } else if (rt.shape.size() > 2 || def(op.operands.at(0)).type.shape.size() > 2) {
         throw Unsupported("tt.reshape beyond rank 2 (line " + std::to_string(op.line) + ")");
       }
