@@ -955,3 +955,29 @@ def test_tile_program_norms_and_reductions_of_the_tutorials():
     X.log_sum_exp_rows[(50,)](b, lse, b.stride(0), 2000, BLOCK=2048)
     torch.cuda.synchronize()
     torch.testing.assert_close(lse, torch.logsumexp(b.double(), 1).float(), rtol=1e-6, atol=1e-5)
+
+
+def test_compiled_kernels_are_cached_on_disk(tmp_path, monkeypatch):
+    """The code object of a run-time compiled kernel is written to the cache directory at the first launch and loaded
+    from there by the next plan of the same source (the reference caches its compiled launchers the same way,
+    backend/driver.py:274-282)."""
+    import extra_kernels as X
+    from triton_shared_amd import _native as native
+    from test_planner import compile_ttir
+    monkeypatch.setenv("TTS_RTC_CACHE", str(tmp_path))
+    sig = {"x_ptr": "*fp32", "out_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"}
+    plan_bytes, _ = native.structured_to_plan(native.ttir_to_structured(compile_ttir(X.block_sum, sig, {"BLOCK": 512})))
+    x = torch.arange(0, 1024, dtype=torch.float32, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    for attempt in range(2):
+        out = torch.zeros(2, device=DEV)
+        plan = native.PlanHandle(plan_bytes)                      # a fresh plan: compiles (or loads) at its first launch
+        plan.launch((2, 1, 1), stream, [x.data_ptr(), out.data_ptr(), 1024])
+        torch.cuda.synchronize()
+        assert out.tolist() == [float(sum(range(512))), float(sum(range(512, 1024)))]
+        files = sorted(p.name for p in tmp_path.iterdir())
+        assert len(files) == 1 and files[0].endswith(".hsaco"), files
+        if attempt == 0:
+            stamp = (tmp_path / files[0]).stat().st_mtime_ns
+        else:
+            assert (tmp_path / files[0]).stat().st_mtime_ns == stamp   # loaded, not rewritten

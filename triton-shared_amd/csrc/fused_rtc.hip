@@ -6,6 +6,10 @@
 // expression the interpreter evaluates, with contraction off, so both paths give identical bits.
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
+#include <sys/stat.h>
+#include <unistd.h>
+#include <cstdio>
+#include <cstdlib>
 
 #include <sstream>
 #include <string>
@@ -194,42 +198,111 @@ struct RtcModule {
 
 std::string fused_map_source(const MapNParams &p) { return source_of(p); }
 
-hipError_t rtc_compile(const std::string &source, const char *entry, RtcModule **out, std::string *err) {
+namespace {
+// Compiled code objects are kept on disk, as the reference keeps its compiled launchers in Triton's cache
+// (backend/driver.py:274-282,344-345): <dir>/<hash of source, options and hipRTC version>.hsaco, with <dir> =
+// $TTS_RTC_CACHE, else $TRITON_CACHE_DIR/tts_rtc, else $HOME/.triton/cache/tts_rtc.  TTS_RTC_CACHE=off disables it.
+const char *const RTC_OPTS[] = {"--offload-arch=gfx950", "-O3", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt"};
+
+std::string cache_dir() {
+  const char *own = getenv("TTS_RTC_CACHE");
+  if (own) return std::string(own) == "off" ? "" : own;
+  if (const char *t = getenv("TRITON_CACHE_DIR")) return std::string(t) + "/tts_rtc";
+  if (const char *h = getenv("HOME")) return std::string(h) + "/.triton/cache/tts_rtc";
+  return "";
+}
+
+std::string cache_key(const std::string &source) {
+  int major = 0, minor = 0;
+  hiprtcVersion(&major, &minor);
+  std::string all = source + "\n" + std::to_string(major) + "." + std::to_string(minor);
+  for (const char *o : RTC_OPTS) all += std::string("\n") + o;
+  uint64_t h1 = 1469598103934665603ull, h2 = 0x9E3779B97F4A7C15ull;  // two FNV-1a style passes: 128 bits of name
+  for (unsigned char c : all) {
+    h1 = (h1 ^ c) * 1099511628211ull;
+    h2 = (h2 + c) * 0x100000001B3ull ^ (h2 >> 29);
+  }
+  char buf[40];
+  snprintf(buf, sizeof buf, "%016llx%016llx", (unsigned long long)h1, (unsigned long long)h2);
+  return buf;
+}
+
+bool read_file(const std::string &path, std::string *out) {
+  FILE *f = fopen(path.c_str(), "rb");
+  if (!f) return false;
+  std::string data;
+  char chunk[65536];
+  size_t n;
+  while ((n = fread(chunk, 1, sizeof chunk, f)) > 0) data.append(chunk, n);
+  fclose(f);
+  if (data.empty()) return false;
+  *out = std::move(data);
+  return true;
+}
+
+void write_file(const std::string &dir, const std::string &name, const std::string &data) {
+  // best effort: mkdir -p, write to a temporary name, rename (so that a concurrent reader never sees half a file)
+  for (size_t i = 1; i <= dir.size(); i++)
+    if (i == dir.size() || dir[i] == '/') mkdir(dir.substr(0, i).c_str(), 0777);
+  const std::string tmp = dir + "/" + name + ".tmp" + std::to_string((long)getpid());
+  FILE *f = fopen(tmp.c_str(), "wb");
+  if (!f) return;
+  const bool ok = fwrite(data.data(), 1, data.size(), f) == data.size();
+  if (fclose(f) != 0 || !ok || rename(tmp.c_str(), (dir + "/" + name).c_str()) != 0) remove(tmp.c_str());
+}
+}  // namespace
+
+static hipError_t rtc_compile_with(const std::string &source, const char *entry, RtcModule **out, std::string *err, bool use_cache) {
   auto *m = new RtcModule;
-  hiprtcProgram prog;
-  if (hiprtcCreateProgram(&prog, source.c_str(), "kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
-    *err = "hiprtcCreateProgram failed";
-    delete m;
-    return hipErrorUnknown;
-  }
-  // no contraction into fmas, IEEE division and square root: the reference's loops are plain scalar C semantics
-  const char *opts[] = {"--offload-arch=gfx950", "-O3", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt"};
-  hiprtcResult r = hiprtcCompileProgram(prog, 4, opts);
-  if (r != HIPRTC_SUCCESS) {
-    size_t n = 0;
-    hiprtcGetProgramLogSize(prog, &n);
-    std::string log(n, '\0');
-    if (n) hiprtcGetProgramLog(prog, &log[0]);
-    *err = std::string("hipRTC: ") + hiprtcGetErrorString(r) + "\n" + log;
+  const std::string dir = use_cache ? cache_dir() : "", name = dir.empty() ? "" : cache_key(source) + ".hsaco";
+  std::string code;
+  const bool cached = !dir.empty() && read_file(dir + "/" + name, &code);
+  if (!cached) {
+    hiprtcProgram prog;
+    if (hiprtcCreateProgram(&prog, source.c_str(), "kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
+      *err = "hiprtcCreateProgram failed";
+      delete m;
+      return hipErrorUnknown;
+    }
+    // no contraction into fmas, IEEE division and square root: the reference's loops are plain scalar C semantics
+    hiprtcResult r = hiprtcCompileProgram(prog, (int)(sizeof RTC_OPTS / sizeof RTC_OPTS[0]), RTC_OPTS);
+    if (r != HIPRTC_SUCCESS) {
+      size_t n = 0;
+      hiprtcGetProgramLogSize(prog, &n);
+      std::string log(n, '\0');
+      if (n) hiprtcGetProgramLog(prog, &log[0]);
+      *err = std::string("hipRTC: ") + hiprtcGetErrorString(r) + "\n" + log;
+      hiprtcDestroyProgram(&prog);
+      delete m;
+      return hipErrorUnknown;
+    }
+    size_t size = 0;
+    hiprtcGetCodeSize(prog, &size);
+    code.assign(size, '\0');
+    hiprtcGetCode(prog, &code[0]);
     hiprtcDestroyProgram(&prog);
-    delete m;
-    return hipErrorUnknown;
   }
-  size_t size = 0;
-  hiprtcGetCodeSize(prog, &size);
-  std::string code(size, '\0');
-  hiprtcGetCode(prog, &code[0]);
-  hiprtcDestroyProgram(&prog);
   hipError_t e = hipModuleLoadData(&m->module, code.data());
   if (e == hipSuccess) e = hipModuleGetFunction(&m->fn, m->module, entry);
+  if (e != hipSuccess && cached) {  // a damaged cache file: forget it and compile
+    if (m->module) (void)hipModuleUnload(m->module);
+    delete m;
+    remove((dir + "/" + name).c_str());
+    return rtc_compile_with(source, entry, out, err, false);
+  }
   if (e != hipSuccess) {
     *err = std::string("loading the compiled kernel: ") + hipGetErrorString(e);
     if (m->module) (void)hipModuleUnload(m->module);
     delete m;
     return e;
   }
+  if (!cached && !dir.empty()) write_file(dir, name, code);
   *out = m;
   return hipSuccess;
+}
+
+hipError_t rtc_compile(const std::string &source, const char *entry, RtcModule **out, std::string *err) {
+  return rtc_compile_with(source, entry, out, err, true);
 }
 
 void rtc_release(RtcModule *m) {
