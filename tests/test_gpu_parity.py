@@ -981,3 +981,26 @@ def test_compiled_kernels_are_cached_on_disk(tmp_path, monkeypatch):
             stamp = (tmp_path / files[0]).stat().st_mtime_ns
         else:
             assert (tmp_path / files[0]).stat().st_mtime_ns == stamp   # loaded, not rewritten
+
+
+def test_reference_matmul_test_in_fp32():
+    """python/examples/test_matmul.py:137-157 as it stands: fp32 operands, 179 x 167 @ 167 x 321, blocks 32 x 64 x 16,
+    GROUP_M 8, operand rows / columns wrapped, and the reference's own assertion (atol 1e-2, rtol 0).  fp32 products run
+    on the generic family (the MFMA kernels take bf16 / fp16)."""
+    torch.manual_seed(0)
+    a = torch.randn(179, 167, device=DEV)
+    b = torch.randn(167, 321, device=DEV)
+    for kernel in (K_mod().matmul_wrapped, K_mod().matmul_tiles):
+        c = torch.empty(179, 321, device=DEV)
+        grid = (triton.cdiv(179, 32) * triton.cdiv(321, 64),)
+        k = kernel[grid](a, b, c, 179, 321, 167, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+                         BM=32, BN=64, BK=16, GROUP_M=8)
+        torch.cuda.synchronize()
+        assert k.function.family == "tile_program"
+        torch.testing.assert_close(c, torch.matmul(a, b), atol=1e-2, rtol=0)
+        assert ((c.double() - a.double() @ b.double()).norm() / (a.double() @ b.double()).norm()) < 1e-6
+
+
+def K_mod():
+    from triton_shared_amd.examples import kernels
+    return kernels
