@@ -262,6 +262,10 @@ class Interpreter:
         attrs = dict(re.findall(r"(\w+) = (-?\w+)", " ".join(re.findall(r"\{([^}]*)\}", head))))
         tys = [parse_type(t) for t in re.split(r"\s*(?:->|,| to | \* )\s*", types) if t.strip()] if types else []
         words = [w for w in re.split(r"[\s,]+", re.sub(r"\{[^}]*\}", "", head)) if w and not w.startswith("%")]
+        if name == "tt.split":
+            env[results[0]] = Val(ops[0].d[..., 0].copy(), ops[0].elem)
+            env[results[1]] = Val(ops[0].d[..., 1].copy(), ops[0].elem)
+            return i + 1
         out = self._eval(name, ops, attrs, tys, words)
         if results:
             env[results[0]] = out
@@ -326,6 +330,12 @@ class Interpreter:
             order = [int(x) for x in re.findall(r"\d+", attrs.get("order", "") or "")]
             a = ops[0]
             return Val(np.transpose(a.d, order[-a.d.ndim:] if order else None).copy(), a.elem, base=a.base)
+        if name == "tt.cat":
+            return Val(np.concatenate([ops[0].d, ops[1].d]), ops[0].elem)
+        if name == "tt.join":
+            return Val(np.stack([ops[0].d, ops[1].d], axis=-1), ops[0].elem)
+        if name == "tt.unsplat":
+            return Val(np.asarray(ops[0].d).reshape(-1)[0], ops[0].elem)
         if name == "tt.reshape":
             a = ops[0]
             return Val(np.reshape(a.d, tys[-1].shape).copy(), a.elem, base=a.base)

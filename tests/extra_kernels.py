@@ -710,3 +710,17 @@ def log_sum_exp_rows(x_ptr, out_ptr, pitch, n_cols, BLOCK: tl.constexpr):
     x = tl.load(x_ptr + row * pitch + c, mask=c < n_cols, other=-float("inf"))
     top = tl.max(x, axis=0)
     tl.store(out_ptr + row, top + tl.log(tl.sum(tl.exp(x - top), axis=0)))
+
+
+@triton.jit
+def join_split_cat(a_ptr, b_ptr, out_ptr, N: tl.constexpr):
+    # out[0 : 2N] = interleave(a, b) (join + reshape); out[2N : 4N] = cat(a + 1, b + 1); out[4N : 5N], out[5N : 6N] = the two
+    # halves split out of the joined block again, swapped
+    i = tl.arange(0, N)
+    a = tl.load(a_ptr + i)
+    b = tl.load(b_ptr + i)
+    tl.store(out_ptr + tl.arange(0, 2 * N), tl.interleave(a, b))
+    tl.store(out_ptr + 2 * N + tl.arange(0, 2 * N), tl.cat(a + 1, b + 1, can_reorder=True))
+    first, second = tl.split(tl.join(a, b))
+    tl.store(out_ptr + 4 * N + i, second)
+    tl.store(out_ptr + 5 * N + i, first)

@@ -1004,3 +1004,15 @@ def test_reference_matmul_test_in_fp32():
 def K_mod():
     from triton_shared_amd.examples import kernels
     return kernels
+
+
+def test_tile_program_join_split_cat():
+    # TritonArithToLinalg/join.mlir, split.mlir and tl.cat: index shuffles of rank-1 blocks
+    import extra_kernels as X
+    a = torch.arange(0, 64, dtype=torch.float32, device=DEV)
+    b = 100 + torch.arange(0, 64, dtype=torch.float32, device=DEV)
+    out = torch.zeros(6 * 64, device=DEV)
+    k = X.join_split_cat[(1,)](a, b, out, N=64)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    assert torch.equal(out, torch.cat([torch.stack([a, b], 1).reshape(-1), a + 1, b + 1, b, a]))

@@ -346,3 +346,14 @@ def test_lanes_philox_dropout_against_an_independent_philox():
     ttir_lanes.Interpreter(t).run((3,), [None, None, n, 0.3, 1234], {0: x, 1: out})
     u = op_zoo.philox_uniform(1234, np.arange(n))
     assert np.array_equal(out, np.where(u > np.float32(0.3), x / (np.float32(1) - np.float32(0.3)), np.float32(0)))
+
+
+def test_lanes_join_split_cat_against_numpy():
+    import extra_kernels as X
+    from test_planner import compile_ttir
+    t = compile_ttir(X.join_split_cat, {"a_ptr": "*fp32", "b_ptr": "*fp32", "out_ptr": "*fp32", "N": "constexpr"}, {"N": 64})
+    a = np.arange(64, dtype=np.float32)
+    b = 100 + np.arange(64, dtype=np.float32)
+    out = np.zeros(6 * 64, np.float32)
+    ttir_lanes.Interpreter(t).run((1,), [None, None, None], {0: a, 1: b, 2: out})
+    assert np.array_equal(out, np.concatenate([np.stack([a, b], 1).reshape(-1), a + 1, b + 1, b, a]))

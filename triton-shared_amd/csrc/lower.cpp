@@ -984,6 +984,22 @@ class Lowerer {
     if (n == "tt.store") return lower_store(op);
     if (n == "tt.reduce" || n == "tt.scan") return lower_reduce(op);
     if (n == "arith.constant") return lower_constant(op);
+    if (n == "tt.split") {  // [.., 2] -> two blocks: one Map per half, "tt.split.0" and "tt.split.1"
+      if (op.results.size() != 2) throw Unsupported("tt.split without two results (line " + std::to_string(op.line) + ")");
+      const int x = data_of(op.operands.at(0));
+      if (P.values[x].shape.size() != 2 || P.values[x].shape[1] != 2) throw Unsupported("tt.split of a block that is not [N, 2]");
+      Type t = result_type(op);
+      for (int half = 0; half < 2; half++) {
+        SOp s;
+        s.kind = SK::Map;
+        s.name = "tt.split." + std::to_string(half);
+        s.operands.push_back(x);
+        s.result = new_value(t);
+        data_[op.results[half]] = s.result;
+        cur_->push_back(s);
+      }
+      return;
+    }
     if (op.results.size() != 1) throw Unsupported("operation " + n + " (line " + std::to_string(op.line) + ")");
     Type rt = result_type(op);
     if (rt.ptr) {  // address computation: PtrAnalysis reads it on demand
@@ -1027,6 +1043,11 @@ class Lowerer {
       for (char ch : it->second)
         if (isalnum((unsigned char)ch) || ch == '_') sym += ch;
       return emit_simple(op, SK::Map, "extern." + sym, op.operands);
+    }
+    if (n == "tt.cat" || n == "tt.join" || n == "tt.unsplat") {  // index shuffles of rank-1 blocks
+      for (auto &o : op.operands)
+        if (def(o).type.shape.size() > 1) throw Unsupported(n + " of blocks of rank > 1 (line " + std::to_string(op.line) + ")");
+      return emit_simple(op, SK::Map, n, op.operands);
     }
     if (n == "tt.trans" || n == "tt.reshape") {  // index shuffles: a Map whose element (i, j) reads another element of its operand
       if (n == "tt.trans") {

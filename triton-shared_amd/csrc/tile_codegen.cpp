@@ -176,6 +176,15 @@ struct Gen {
           if (O.shape.size() != 2 || V.shape.size() != 2) no("tt.trans of a block that is not of rank 2");
           return at(s.operands[0], i1, i0);
         }
+        if (s.name == "tt.cat") {  // two rank-1 blocks end to end
+          const int64_t na = val(s.operands.at(0)).shape.at(0);
+          return "(" + i0 + " < " + std::to_string(na) + " ? " + at(s.operands[0], i0, "0") + " : " +
+                 at(s.operands.at(1), "(" + i0 + " - " + std::to_string(na) + ")", "0") + ")";
+        }
+        if (s.name == "tt.join")  // [N] and [N] -> [N, 2]
+          return "(" + i1 + " == 0 ? " + at(s.operands.at(0), i0, "0") + " : " + at(s.operands.at(1), i0, "0") + ")";
+        if (s.name == "tt.split.0" || s.name == "tt.split.1") return at(s.operands.at(0), i0, s.name.substr(9));
+        if (s.name == "tt.unsplat") return at(s.operands.at(0), "0", "0");
         if (s.name == "tt.reshape") {  // row-major element order is kept
           const Value &O = val(s.operands.at(0));
           const std::string lin = V.shape.size() == 2 ? "(" + i0 + " * " + std::to_string(V.shape[1]) + " + " + i1 + ")" : V.shape.size() == 1 ? i0 : "0";
