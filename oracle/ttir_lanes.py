@@ -173,7 +173,7 @@ class Interpreter:
                 label = re.match(r"cf\.br (\^\w+)$", line).group(1)
                 i = next(k for k, l in enumerate(L) if l.startswith(label + ":")) + 1
                 continue
-            if line.startswith("scf.if"):
+            if line.startswith("scf.if") or re.match(r"%[\w.#$:-]+(, %[\w.#$:-]+)* = scf\.if ", line):
                 i = self._if(i, env)
                 continue
             i = self._op(i, env)
@@ -182,9 +182,14 @@ class Interpreter:
     def _if(self, i, env):
         """scf.if without results: `scf.if %c {` ... [`} else {` ...] `}`."""
         L = self.lines
-        m = re.match(r"scf\.if (%[\w.#$-]+) \{$", L[i])
-        if not m:
-            raise NotImplementedError("ttir_lanes: scf.if with results")
+        results = []
+        head = L[i]
+        if head.startswith("%"):                     # %r:2 = scf.if %c -> (types) {
+            lhs, head = head.split(" = ", 1)
+            for r in lhs.split(","):
+                r = r.strip()
+                results += [f"{r.split(':')[0]}#{k}" for k in range(int(r.split(":")[1]))] if ":" in r else [r]
+        m = re.match(r"scf\.if (%[\w.#$-]+)( -> .*)? \{$", head)
         take = bool(env[m.group(1)].d)
         # find the matching else / end at this nesting depth
         depth, j, els = 1, i + 1, None
@@ -199,19 +204,24 @@ class Interpreter:
             j += 1
         end = j - 1
         if take:
-            k, _ = self._block(i + 1, env) if els is None else self._run_until(i + 1, els, env)
+            k, ys = self._block(i + 1, env) if els is None else self._run_until(i + 1, els, env)
         elif els is not None:
-            k, _ = self._block(els + 1, env)
+            k, ys = self._block(els + 1, env)
         else:
-            k = end
+            k, ys = end, None
+        if results:
+            for r, y in zip(results, ys):
+                env[r] = y
         return len(L) if k >= len(L) else end + 1
 
     def _run_until(self, i, stop, env):
         L = self.lines
         while i < stop:
+            if L[i].startswith("scf.yield"):
+                return i, [env[n] for n in re.findall(r"%[\w.#$-]+", L[i].split(" : ")[0])]
             if L[i].startswith("tt.return"):
                 return len(L), None
-            if L[i].startswith("scf.if"):
+            if L[i].startswith("scf.if") or re.match(r"%[\w.#$:-]+(, %[\w.#$:-]+)* = scf\.if ", L[i]):
                 i = self._if(i, env)
                 continue
             i = self._op(i, env)

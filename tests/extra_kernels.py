@@ -724,3 +724,21 @@ def join_split_cat(a_ptr, b_ptr, out_ptr, N: tl.constexpr):
     first, second = tl.split(tl.join(a, b))
     tl.store(out_ptr + 4 * N + i, second)
     tl.store(out_ptr + 5 * N + i, first)
+
+
+@triton.jit
+def branch_with_results(x_ptr, flag_ptr, out_ptr, N: tl.constexpr):
+    # an if / else on a value read from memory that produces a block, a float scalar and an integer scalar
+    pid = tl.program_id(0)
+    i = tl.arange(0, N)
+    x = tl.load(x_ptr + i)
+    f = tl.load(flag_ptr + pid)
+    if f > 0:
+        y = x * 2.0
+        s = 1.0
+        k = f * 3
+    else:
+        y = x - 1.0
+        s = -1.0
+        k = 7 - f
+    tl.store(out_ptr + pid * N + i, y + s + k.to(tl.float32))

@@ -1016,3 +1016,17 @@ def test_tile_program_join_split_cat():
     torch.cuda.synchronize()
     assert k.function.family == "tile_program"
     assert torch.equal(out, torch.cat([torch.stack([a, b], 1).reshape(-1), a + 1, b + 1, b, a]))
+
+
+def test_tile_program_if_with_results():
+    # an if / else on a loaded scalar that yields a block, and an integer scalar that later feeds float arithmetic
+    import extra_kernels as X
+    torch.manual_seed(17)
+    x = torch.randn(128, device=DEV)
+    flags = torch.tensor([3, -2, 0, 5], dtype=torch.int32, device=DEV)
+    out = torch.zeros(4, 128, device=DEV)
+    k = X.branch_with_results[(4,)](x, flags, out, N=128)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    want = torch.stack([(x * 2 + 1 + float(3 * f)) if f > 0 else (x - 1 - 1 + float(7 - f)) for f in flags.tolist()])
+    assert torch.equal(out, want)

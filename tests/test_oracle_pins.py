@@ -357,3 +357,15 @@ def test_lanes_join_split_cat_against_numpy():
     out = np.zeros(6 * 64, np.float32)
     ttir_lanes.Interpreter(t).run((1,), [None, None, None], {0: a, 1: b, 2: out})
     assert np.array_equal(out, np.concatenate([np.stack([a, b], 1).reshape(-1), a + 1, b + 1, b, a]))
+
+
+def test_lanes_if_with_results_against_numpy():
+    import extra_kernels as X
+    from test_planner import compile_ttir
+    t = compile_ttir(X.branch_with_results, {"x_ptr": "*fp32", "flag_ptr": "*i32", "out_ptr": "*fp32", "N": "constexpr"}, {"N": 128})
+    x = np.random.default_rng(2).standard_normal(128).astype(np.float32)
+    flags = np.array([3, -2, 0, 5], dtype=np.int32)
+    out = np.zeros(4 * 128, np.float32)
+    ttir_lanes.Interpreter(t).run((4,), [None, None, None], {0: x, 1: flags, 2: out})
+    want = np.stack([(x * 2 + 1 + np.float32(3 * f)) if f > 0 else (x - 1 - 1 + np.float32(7 - f)) for f in flags])
+    assert np.array_equal(out.reshape(4, 128), want.astype(np.float32))

@@ -1067,23 +1067,43 @@ class Lowerer {
     throw Unsupported("operation " + n + " (line " + std::to_string(op.line) + ") has no structured lowering");
   }
 
-  // A branch on a scalar condition, without results: an early `return` (cf.cond_br to a block that only returns) or an
-  // `if` around memory effects.  Each non-empty side becomes one If op on the same condition value.
+  // A branch on a scalar condition: an early `return` (cf.cond_br to a block that only returns), an `if` around memory
+  // effects, or an `if` / `else` that yields values.  Each side becomes one If op on the same condition value; with
+  // results, both sides name the same result values and give their own yields.
   void lower_if(const Op &op) {
-    if (!op.results.empty()) throw Unsupported("scf.if with results (line " + std::to_string(op.line) + ")");
     const int cond = data_of(op.operands.at(0));
+    const size_t nres = op.results.size();
+    if (nres && op.regions.size() != 2) throw Unsupported("scf.if with results but without an else region");
+    std::vector<int> results;
+    for (size_t j = 0; j < nres; j++) {
+      const Type &t = op.result_types.at(j);
+      if (t.ptr) throw Unsupported("scf.if that yields pointers (line " + std::to_string(op.line) + ")");
+      results.push_back(new_value(t));
+    }
     for (int side = 0; side < 2 && side < (int)op.regions.size(); side++) {
-      if (op.regions[side].ops.empty()) continue;
+      const Block &region = op.regions[side];
+      if (region.ops.empty() && !nres) continue;
       SOp s;
       s.kind = SK::If;
       s.operands.push_back(cond);
       s.ival = side;
+      s.results = results;
       std::vector<SOp> *saved = cur_;
       cur_ = &s.body;
-      lower_block(op.regions[side]);
+      size_t count = region.ops.size();
+      if (nres) {
+        if (region.ops.empty() || region.ops.back()->name != "scf.yield" || region.ops.back()->operands.size() != nres)
+          throw Unsupported("scf.if region that does not end in a yield of its results (line " + std::to_string(op.line) + ")");
+        count--;
+      }
+      for (size_t i = 0; i < count; i++) lower_op(*region.ops[i]);
+      if (nres)
+        for (auto &y : region.ops.back()->operands) s.tile_yields.push_back(data_of(y));
       cur_ = saved;
-      if (!s.body.empty()) cur_->push_back(std::move(s));
+      if (!s.body.empty() || nres) cur_->push_back(std::move(s));
     }
+    // the results are data from here on (an integer result is not an index expression: what is computed from it is data too)
+    for (size_t j = 0; j < nres; j++) data_[op.results[j]] = results[j];
   }
 
   void lower_block(const Block &b) {
@@ -1124,9 +1144,17 @@ class Lowerer {
             mark(s.body);
           }
         } else if (s.kind == SK::If) {
-          if (mark(s.body)) {
-            any_effect = true;
+          bool res_live = false;
+          for (int r : s.results) res_live |= live[r];
+          const bool eff = mark(s.body);
+          if (eff || res_live) {
+            any_effect |= eff;
             for (int v : s.operands) use(v);
+            if (res_live) {
+              for (int r : s.results) use(r);          // both sides of the branch keep all of them
+              for (int y : s.tile_yields) use(y);
+              mark(s.body);
+            }
           }
         } else if (!s.results.empty()) {  // a reduction or scan with a combiner region: all of it or nothing
           bool res_live = false;
@@ -1171,7 +1199,15 @@ class Lowerer {
             s.tile_yields = y;
             s.results = r;
           }
-        } else if (s.kind == SK::If) keep = sweep(s.body);
+        } else if (s.kind == SK::If) {
+          bool res_live = false;
+          for (int r : s.results) res_live = res_live || live[r];
+          if (!res_live) {  // nobody reads what the branch yields
+            s.results.clear();
+            s.tile_yields.clear();
+          }
+          keep = sweep(s.body) || res_live;
+        }
         else if (!s.results.empty()) keep = live[s.results[0]];
         else keep = s.result >= 0 && live[s.result];
         if (keep) {

@@ -414,9 +414,47 @@ struct Gen {
       if (s.kind == SK::For) { loop(s); k++; continue; }
       if (s.kind == SK::If) {  // the condition is a scalar, the same for every thread: barriers inside are safe
         map_vars({-1});
-        os << pad() << "if (" << (s.ival ? "!" : "") << "(" << at(s.operands.at(0), "0", "0") << ")) {\n";
+        // results: a variable per scalar, a per-thread array per block, declared once (the `then` side comes first)
+        // and assigned at the end of whichever side runs
+        for (size_t j = 0; j < s.results.size(); j++) {
+          const int r = s.results[j];
+          const Value &R = val(r);
+          const std::string name = "ifr" + std::to_string(r);
+          if (R.shape.size() > 2) no("an if that yields a block of rank " + std::to_string(R.shape.size()));
+          if (R.shape.empty()) {
+            if (!var.count(r)) os << pad() << ctype(R.dtype) << " " << name << ";\n";
+            var[r] = name;
+          } else {
+            if (count(R.shape) > TWO_PHASE_MAX) no("an if that yields a block of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
+            if (!held.count(r)) {
+              os << pad() << ctype(R.dtype) << " " << name << "[" << (count(R.shape) + 255) / 256 << "];\n";
+              mine.push_back(r);
+            }
+            held[r] = {name, R.shape};
+          }
+        }
+        const std::string cond = at(s.operands.at(0), "0", "0");
+        os << pad() << "if (" << (s.ival ? "!" : "") << "(" << cond << ")) {\n";
         indent++;
-        body(s.body);
+        std::vector<int> side_held;
+        body(s.body, &side_held);
+        for (size_t j = 0; j < s.results.size(); j++) {
+          const Value &R = val(s.results[j]);
+          const std::string name = "ifr" + std::to_string(s.results[j]);
+          if (R.shape.empty()) {
+            map_vars({-1});
+            os << pad() << name << " = " << at(s.tile_yields.at(j), "0", "0") << ";\n";
+          } else {
+            open_element_loop(R.shape);
+            var.erase(s.results[j]);  // the result itself is not readable while it is being written
+            os << pad() << name << "[n] = " << at(s.tile_yields.at(j), idx0(R.shape), idx1(R.shape)) << ";\n";
+            close_loop();
+          }
+        }
+        for (int v : side_held) {
+          held.erase(v);
+          var.erase(v);
+        }
         indent--;
         os << pad() << "}\n";
         k++;

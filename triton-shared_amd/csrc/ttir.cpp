@@ -297,10 +297,12 @@ static void parse_op(Lines &L, Block &blk) {
     return;
   }
   if (op->name == "scf.if") {
-    // scf.if %c {  ...  [} else {  ...]  }   (without results)
-    if (!op->results.empty()) throw Unsupported("scf.if with results");
+    // scf.if %c [-> (types)] {  ...  [} else {  ...]  }   ; with results both regions end in scf.yield
     size_t brace = rest.rfind('{');
-    collect_operands(rest.substr(0, brace), op->operands);
+    size_t arrow = rest.find("->");
+    collect_operands(rest.substr(0, arrow == std::string::npos ? brace : arrow), op->operands);
+    if (arrow != std::string::npos) op->result_types = parse_type_list(rest.substr(arrow + 2, brace - arrow - 2));
+    if (op->result_types.size() != op->results.size()) throw Unsupported("scf.if: results and result types differ in number");
     op->regions.resize(2);
     parse_block(L, op->regions[0]);
     if (L.i < L.v.size() && L.v[L.i] == "} else {") {
