@@ -15,7 +15,7 @@ brute-force pin for what the reference derives symbolically:
 
 Beyond the five hot-path kernels it also runs what the generic kernel family takes: tt.reduce / tt.scan with any
 combiner region (argmin / argmax, ConversionPatterns.hpp:1443-1769), integer, bit and conversion ops, extern functions
-by symbol name, tt.trans / tt.reshape, cf.cond_br trees (early return) and result-less scf.if.  Pins, all in
+by symbol name, tt.trans / tt.reshape / tt.cat / tt.join / tt.split, cf.cond_br trees (early return) and scf.if.  Pins, all in
 tests/test_oracle_pins.py: the reference's golden tensors (python/examples/test_modulo.py, test_mask.py,
 test_gather_scatter.py and the 21 cases of tests/reference_cases.py), numpy closed forms per op class
 (tests/op_zoo.py, including an independent Philox for tl.rand), float64 formulas for the float kernels.

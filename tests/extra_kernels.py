@@ -742,3 +742,16 @@ def branch_with_results(x_ptr, flag_ptr, out_ptr, N: tl.constexpr):
         s = -1.0
         k = 7 - f
     tl.store(out_ptr + pid * N + i, y + s + k.to(tl.float32))
+
+
+@triton.jit
+def softmax_persistent(out_ptr, in_ptr, in_pitch, out_pitch, n_rows, n_cols, BLOCK: tl.constexpr):
+    # the current fused-softmax tutorial: each program walks rows pid, pid + num_programs, ...
+    first = tl.program_id(0)
+    hop = tl.num_programs(0)
+    for row in tl.range(first, n_rows, hop):
+        c = tl.arange(0, BLOCK)
+        m = c < n_cols
+        x = tl.load(in_ptr + row * in_pitch + c, mask=m, other=-float("inf"))
+        e = tl.exp(x - tl.max(x, axis=0))
+        tl.store(out_ptr + row * out_pitch + c, e / tl.sum(e, axis=0), mask=m)

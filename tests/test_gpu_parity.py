@@ -1030,3 +1030,17 @@ def test_tile_program_if_with_results():
     assert k.function.family == "tile_program"
     want = torch.stack([(x * 2 + 1 + float(3 * f)) if f > 0 else (x - 1 - 1 + float(7 - f)) for f in flags.tolist()])
     assert torch.equal(out, want)
+
+
+def test_tile_program_persistent_softmax():
+    """The grid-stride softmax of the current tutorial on the generic family, with the reference's own shape and assertion
+    (python/examples/test_softmax.py:60-65) and the 1e-5 max-abs bar against float64."""
+    import extra_kernels as X
+    torch.manual_seed(0)
+    x = torch.randn(1823, 781, device=DEV)
+    y = torch.empty_like(x)
+    k = X.softmax_persistent[(256,)](y, x, x.stride(0), y.stride(0), 1823, 781, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    assert torch.allclose(y, torch.softmax(x, 1))
+    assert (y.double() - torch.softmax(x.double(), 1)).abs().max() <= 1e-5
