@@ -755,3 +755,26 @@ def softmax_persistent(out_ptr, in_ptr, in_pitch, out_pitch, n_rows, n_cols, BLO
         x = tl.load(in_ptr + row * in_pitch + c, mask=m, other=-float("inf"))
         e = tl.exp(x - tl.max(x, axis=0))
         tl.store(out_ptr + row * out_pitch + c, e / tl.sum(e, axis=0), mask=m)
+
+
+@triton.jit
+def matmul_leaky(a_ptr, b_ptr, c_ptr, M, N, K, s_am, s_bk, s_cm, slope, BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr):
+    # a tiled matmul with an activation fused before the narrowing store (the tutorial's ACTIVATION hook): not the shape
+    # the MFMA kernels take, so the generic family runs it
+    tm = tl.program_id(0)
+    tn = tl.program_id(1)
+    rm = tm * BM + tl.arange(0, BM)
+    rn = tn * BN + tl.arange(0, BN)
+    rk = tl.arange(0, BK)
+    pa = a_ptr + rm[:, None] * s_am + rk[None, :]
+    pb = b_ptr + rk[:, None] * s_bk + rn[None, :]
+    acc = tl.zeros((BM, BN), dtype=tl.float32)
+    for k in range(0, tl.cdiv(K, BK)):
+        left = K - k * BK
+        a = tl.load(pa, mask=(rm[:, None] < M) & (rk[None, :] < left), other=0.0)
+        b = tl.load(pb, mask=(rk[:, None] < left) & (rn[None, :] < N), other=0.0)
+        acc = tl.dot(a, b, acc)
+        pa += BK
+        pb += BK * s_bk
+    acc = tl.where(acc >= 0, acc, slope * acc)
+    tl.store(c_ptr + rm[:, None] * s_cm + rn[None, :], acc.to(c_ptr.dtype.element_ty), mask=(rm[:, None] < M) & (rn[None, :] < N))

@@ -1044,3 +1044,19 @@ def test_tile_program_persistent_softmax():
     assert k.function.family == "tile_program"
     assert torch.allclose(y, torch.softmax(x, 1))
     assert (y.double() - torch.softmax(x.double(), 1)).abs().max() <= 1e-5
+
+
+def test_tile_program_matmul_with_fused_activation():
+    """A 128 x 128 x 64 bf16 tile matmul with a leaky-relu before the store: outside the MFMA kernels' shape, so it runs as
+    small-product code (operands staged in LDS in their 16-bit type)."""
+    import extra_kernels as X
+    torch.manual_seed(18)
+    M, N, K = 200, 300, 150
+    a = torch.randn(M, K, device=DEV).bfloat16()
+    b = torch.randn(K, N, device=DEV).bfloat16()
+    c = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+    k = X.matmul_leaky[(triton.cdiv(M, 128), triton.cdiv(N, 128))](a, b, c, M, N, K, a.stride(0), b.stride(0), c.stride(0), 0.01, BM=128, BN=128, BK=64)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    want = torch.nn.functional.leaky_relu(a.double() @ b.double(), 0.01)
+    assert ((c.double() - want).norm() / want.norm()) <= 1e-2

@@ -719,26 +719,33 @@ struct Gen {
       no("a matrix product whose operands are not [M, K] x [K, N]");
     const int64_t M = A.shape[0], K = A.shape[1], N = B.shape[1];
     if (M * N > TWO_PHASE_MAX) no("a matrix product with more than " + std::to_string(TWO_PHASE_MAX) + " outputs outside the tiled matmul kernels");
-    const size_t bytes = (size_t)(M * K + K * N) * 4;
+    // operands of a 16-bit type are staged in that type (their values are exactly representable), others as fp32
+    auto narrow = [](const std::string &t) { return t == "f16" || t == "bf16"; };
+    const size_t a_size = narrow(A.dtype) ? 2 : 4, b_size = narrow(B.dtype) ? 2 : 4;
+    const size_t a_bytes = ((size_t)(M * K) * a_size + 15) / 16 * 16, bytes = a_bytes + (size_t)(K * N) * b_size;
     if (bytes > 48 * 1024) no("a matrix product whose operands need " + std::to_string(bytes) + " bytes of LDS (limit 49152)");
     if (!is_float(A.dtype) || !is_float(B.dtype) || !is_float(R.dtype)) no("an integer matrix product");
     pool_bytes = std::max(pool_bytes, bytes);
     const std::string id = std::to_string(s.result);
+    auto staged_type = [&](const std::string &t) { return narrow(t) ? std::string("unsigned short") : std::string("float"); };
+    auto put = [&](const std::string &t, const std::string &e) { return t == "f16" ? "down_f16(" + e + ")" : t == "bf16" ? "down_bf16(" + e + ")" : e; };
+    auto get = [&](const std::string &t, const std::string &e) { return t == "f16" ? "up_f16(" + e + ")" : t == "bf16" ? "up_bf16(" + e + ")" : e; };
     os << pad() << "__syncthreads();\n";
-    os << pad() << "float *const da" << id << " = (float *)pool, *const db" << id << " = (float *)pool + " << M * K << ";\n";
+    os << pad() << staged_type(A.dtype) << " *const da" << id << " = (" << staged_type(A.dtype) << " *)pool;\n";
+    os << pad() << staged_type(B.dtype) << " *const db" << id << " = (" << staged_type(B.dtype) << " *)(pool + " << a_bytes << ");\n";
     open_element_loop(A.shape);
-    os << pad() << "da" << id << "[t] = " << at(s.operands[0], idx0(A.shape), idx1(A.shape)) << ";\n";
+    os << pad() << "da" << id << "[t] = " << put(A.dtype, at(s.operands[0], idx0(A.shape), idx1(A.shape))) << ";\n";
     close_loop();
     open_element_loop(B.shape);
-    os << pad() << "db" << id << "[t] = " << at(s.operands[1], idx0(B.shape), idx1(B.shape)) << ";\n";
+    os << pad() << "db" << id << "[t] = " << put(B.dtype, at(s.operands[1], idx0(B.shape), idx1(B.shape))) << ";\n";
     close_loop();
     os << pad() << "__syncthreads();\n";
     const std::string name = "dot" + id;
     os << pad() << "float " << name << "[" << (M * N + 255) / 256 << "];\n";
     open_element_loop(R.shape);
     os << pad() << "float sum = 0.f;\n";
-    os << pad() << "for (int k = 0; k < " << K << "; k++) sum += da" << id << "[" << idx0(R.shape) << " * " << K << " + k] * db" << id << "[k * " << N
-       << " + " << idx1(R.shape) << "];\n";
+    os << pad() << "for (int k = 0; k < " << K << "; k++) sum += " << get(A.dtype, "da" + id + "[" + idx0(R.shape) + " * " + std::to_string(K) + " + k]") << " * "
+       << get(B.dtype, "db" + id + "[k * " + std::to_string(N) + " + " + idx1(R.shape) + "]") << ";\n";
     os << pad() << name << "[n] = " << rounded(R.dtype, "sum + " + at(s.operands.at(2), idx0(R.shape), idx1(R.shape))) << ";\n";
     close_loop();
     os << pad() << "__syncthreads();\n";
