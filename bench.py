@@ -200,6 +200,15 @@ def make_workloads(torch, triton, K):
         return dict(desc=f"inclusive prefix sums inside blocks of 1024, fp32 N={n} (generic family, scan)", work=8 * n, bound="hbm",
                     dtype="f32", make=make, set_bytes=8 * n, lanes=cpu)
 
+    def matmul_act(n):
+        def make():
+            a = (torch.randn(n, n, device=dev) * 0.02).bfloat16()
+            b = (torch.randn(n, n, device=dev) * 0.02).bfloat16()
+            c = torch.empty(n, n, dtype=torch.bfloat16, device=dev)
+            return lambda: K.matmul_leaky_relu[(n // 128, n // 128)](a, b, c, n, n, n, n, n, n, 0.01, BM=128, BN=128, BK=64)
+        return dict(desc=f"C = leaky_relu(A @ B) bf16 {n}^3, BM=BN=128 BK=64 (generic family: LDS-staged operands, 32x32 MFMA blocks)",
+                    work=2 * n ** 3, bound="mfma", dtype="bf16", make=make, set_bytes=3 * n * n * 2)
+
     W["cfg1"] = vec_add(98432)
     W["cfg2"] = softmax(4096)
     W["cfg3"] = layernorm()
@@ -209,6 +218,7 @@ def make_workloads(torch, triton, K):
     W["cfg2_1m"] = softmax(1 << 20)
     W["next_fused_gelu_2p26"] = fused_gelu(1 << 26)
     W["next_fused_silu_2p26"] = fused_silu(1 << 26)
+    W["next_matmul_act_2048"] = matmul_act(2048)
     W["next_take_rows_2p26"] = take_rows(1 << 16, 1024)
     W["next_row_sums_2p26"] = row_sums(1 << 16, 1024)
     W["next_block_cumsum_2p26"] = block_cumsum(1 << 26)
@@ -399,7 +409,7 @@ def main():
                      rotating_buffer_sets=t["sets"], warmup_steps_run=t["warmup_steps_run"], frontend_us_per_launch=round(t["frontend_us"], 1),
                      roofline=roofline(wl, t["us"], name), dtype=wl["dtype"], algorithmic_work=wl["work"],
                      same_buffers=dict(us=round(t["hot_us"], 3), frac=roofline(wl, t["hot_us"])["frac"]))
-        if not args.no_cpu and (name == args.workload or "lanes" in wl or not name.endswith(("2p28", "1m", "2p26"))):
+        if not args.no_cpu and (name == args.workload or "lanes" in wl or not name.endswith(("2p28", "1m", "2p26", "2048"))):
             entry["cpu_baseline"] = cpu_baseline(torch, name, wl, t.get("ttir"))
         kernels[name] = entry
     head = kernels[args.workload]

@@ -15,6 +15,7 @@
 // therefore run in two phases -- every load of the body into per-thread registers, a barrier,
 // then ops and stores; larger tiles are fused in one loop and accepted only when no store's base
 // argument is also a load's.
+#include <algorithm>
 #include <functional>
 #include <map>
 #include <set>
@@ -38,6 +39,7 @@ struct Gen {
   std::ostringstream fns;                           // combiner functions of reductions and scans (before the kernel)
   std::ostringstream decl;                          // LDS arrays holding their results (top of the kernel)
   size_t pool_bytes = 0, out_bytes = 0;             // staging pool shared by all reductions; result arrays
+  bool uses_mfma = false;
 
   explicit Gen(const Program &p) : P(p) {}
 
@@ -521,6 +523,10 @@ struct Gen {
         }
       if (!have) { k = end; continue; }  // only elementwise ops: they are written out where their results are used
       auto own = [&](const SOp &o) { return o.kind == SK::Load && o.acc.sizes == shape; };
+      const bool two_phase_run = count(shape) <= TWO_PHASE_MAX;
+      auto big_other = [&](const SOp &o) {
+        return two_phase_run && o.kind == SK::Load && o.acc.sizes != shape && count(o.acc.sizes) >= 2048 && count(o.acc.sizes) <= TWO_PHASE_MAX;
+      };
       const int64_t T = count(shape);
       const bool two_phase = T <= TWO_PHASE_MAX;
       const std::string i0 = idx0(shape), i1 = idx1(shape);
@@ -534,7 +540,7 @@ struct Gen {
       // the one before it (loads complete in order): copy them to LDS first, at the place in the program where they stand.
       for (size_t q = k; q < end; q++) {
         const SOp &o = ops[q];
-        if (o.kind != SK::Load || own(o) || staged.count(o.result)) continue;
+        if (o.kind != SK::Load || own(o) || big_other(o) || staged.count(o.result)) continue;
         const size_t bytes = (size_t)count(o.acc.sizes) * held_bytes(val(o.result).dtype);
         if (count(o.acc.sizes) > TWO_PHASE_MAX || pool_bytes + out_bytes + bytes > 48 * 1024) continue;
         const std::string name = "blk" + std::to_string(o.result);
@@ -551,52 +557,62 @@ struct Gen {
         staged[o.result] = name;
       }
       if (two_phase) {
-        bool any_load = false;
+        // Registers for the run's own loads, and for large blocks of another shape (a [K, N] operand next to an [M, K]
+        // one): those are held by the threads that own their elements and can be named in loops over their own shape.
+        std::vector<std::vector<int64_t>> shapes = {shape};
         for (size_t q = k; q < end; q++)
-          if (own(ops[q])) {
-            os << pad() << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << (T + 255) / 256 << "];\n";
-            any_load = true;
-          }
-        if (any_load) {
+          if (big_other(ops[q]) && std::find(shapes.begin(), shapes.end(), ops[q].acc.sizes) == shapes.end()) shapes.push_back(ops[q].acc.sizes);
+        bool any_load = false;
+        for (const auto &ls : shapes) {
+          auto mine_here = [&](const SOp &o) { return o.kind == SK::Load && o.acc.sizes == ls && (own(o) || big_other(o)); };
+          bool any = false;
+          for (size_t q = k; q < end; q++)
+            if (mine_here(ops[q])) {
+              os << pad() << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << (count(ls) + 255) / 256 << "];\n";
+              any = true;
+            }
+          if (!any) continue;
+          any_load = true;
+          const std::string l0 = idx0(ls), l1 = idx1(ls);
           // A masked load is written as `if (valid) x = *p;` here and gets its `other` in a second loop: selecting
           // between the loaded value and `other` on the spot would need the value, and with it a wait for every load
           // before the next one is issued.
           std::vector<std::pair<const SOp *, std::string>> fill;  // masked loads whose `other` is still to be filled in
           auto fill_others = [&]() {
             if (fill.empty()) return;
-            open_element_loop(shape);
+            open_element_loop(ls);
             for (auto &f : fill) {
-              std::string pred, addr = address(f.first->acc, i0, i1, pred);
+              std::string pred, addr = address(f.first->acc, l0, l1, pred);
               os << pad() << "if (!(" << pred << ")) " << f.second << "[n] = " << other_of(f.first->acc) << ";\n";
             }
             close_loop();
             fill.clear();
           };
-          open_element_loop(shape);
+          open_element_loop(ls);
           for (size_t q = k; q < end; q++)
-            if (own(ops[q])) {
+            if (mine_here(ops[q])) {
               const std::string name = "ld" + std::to_string(ops[q].result);
-              std::string pred, addr = address(ops[q].acc, i0, i1, pred);
+              std::string pred, addr = address(ops[q].acc, l0, l1, pred);
               bool needs_filled = false;  // indexed or masked by a load that still lacks its `other`
               for (auto &f : fill) needs_filled = needs_filled || addr.find(f.second + "[") != std::string::npos || pred.find(f.second + "[") != std::string::npos;
               if (needs_filled) {
                 close_loop();
                 fill_others();
-                open_element_loop(shape);
+                open_element_loop(ls);
               }
               if (pred.empty()) os << pad() << name << "[n] = " << mem_read(ops[q].acc, addr) << ";\n";
               else {
                 os << pad() << "if (" << pred << ") " << name << "[n] = " << mem_read(ops[q].acc, addr) << ";\n";
                 fill.push_back({&ops[q], name});
               }
-              held[ops[q].result] = {name, shape};  // a later load of this run may be indexed by it
+              held[ops[q].result] = {name, ls};  // a later load of this run may be indexed by it
               var[ops[q].result] = name + "[n]";
               mine.push_back(ops[q].result);
             }
           close_loop();
           fill_others();
-          os << pad() << "__syncthreads();\n";
         }
+        if (any_load) os << pad() << "__syncthreads();\n";
         if (stores) open_element_loop(shape);
       } else {
         std::set<int> load_bases;
@@ -736,12 +752,66 @@ struct Gen {
     open_element_loop(A.shape);
     os << pad() << "da" << id << "[t] = " << put(A.dtype, at(s.operands[0], idx0(A.shape), idx1(A.shape))) << ";\n";
     close_loop();
+    // for the 16-bit matrix-core path B is staged transposed ([N][K], K contiguous), so that a lane's eight consecutive k
+    // of a column are one 16-byte LDS read, as they are for A
+    const bool both16 = A.dtype == B.dtype && narrow(A.dtype);
+    const bool both32 = A.dtype == "f32" && B.dtype == "f32";
+    const size_t band_bytes = (size_t)32 * N * 4;
+    const bool mfma = M % 32 == 0 && N % 32 == 0 && ((both16 && K % 16 == 0) || (both32 && K % 2 == 0)) && band_bytes <= 32 * 1024 &&
+                      bytes + band_bytes <= 60 * 1024;
     open_element_loop(B.shape);
-    os << pad() << "db" << id << "[t] = " << put(B.dtype, at(s.operands[1], idx0(B.shape), idx1(B.shape))) << ";\n";
+    if (mfma && both16)
+      os << pad() << "db" << id << "[" << idx1(B.shape) << " * " << K << " + " << idx0(B.shape) << "] = " << put(B.dtype, at(s.operands[1], idx0(B.shape), idx1(B.shape))) << ";\n";
+    else
+      os << pad() << "db" << id << "[t] = " << put(B.dtype, at(s.operands[1], idx0(B.shape), idx1(B.shape))) << ";\n";
     close_loop();
     os << pad() << "__syncthreads();\n";
     const std::string name = "dot" + id;
     os << pad() << "float " << name << "[" << (M * N + 255) / 256 << "];\n";
+    // Matrix cores when the shapes allow: 32 x 32 output blocks, one 32-row band of the result at a time.  The four
+    // wavefronts take the band's column blocks in turn, accumulate over K with v_mfma_f32_32x32x16 (16-bit operands) or
+    // 32x32x2 (fp32), and leave the band in LDS, from where every thread picks up the elements it owns.
+    if (mfma) {
+      const size_t band_off = (bytes + 15) / 16 * 16;
+      pool_bytes = std::max(pool_bytes, band_off + band_bytes);
+      uses_mfma = true;
+      os << pad() << "float *const dc" << id << " = (float *)(pool + " << band_off << ");\n";
+      os << pad() << "for (int br = 0; br < " << M / 32 << "; br++) {\n";
+      indent++;
+      os << pad() << "for (int bc = threadIdx.x >> 6; bc < " << N / 32 << "; bc += 4) {\n";
+      indent++;
+      os << pad() << "const int ln = threadIdx.x & 63, row = br * 32 + (ln & 31), col = bc * 32 + (ln & 31), kg = ln >> 5;\n";
+      os << pad() << "f32x16_t acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};\n";
+      if (both16) {
+        os << pad() << "for (int k0 = 0; k0 < " << K << "; k0 += 16) {\n";
+        indent++;
+        os << pad() << "const u16x8_t fa = *(const u16x8_t *)&da" << id << "[row * " << K << " + k0 + 8 * kg], fb = *(const u16x8_t *)&db" << id << "[col * " << K
+           << " + k0 + 8 * kg];\n";
+        os << pad() << "acc = " << (A.dtype == "bf16" ? "__builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fa), __builtin_bit_cast(bf16x8_t, fb)"
+                                                      : "__builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, fa), __builtin_bit_cast(f16x8_t, fb)")
+           << ", acc, 0, 0, 0);\n";
+        indent--;
+        os << pad() << "}\n";
+      } else {
+        os << pad() << "for (int k0 = 0; k0 < " << K << "; k0 += 2) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(da" << id << "[row * " << K << " + k0 + kg], db" << id
+           << "[(k0 + kg) * " << N << " + col], acc, 0, 0, 0);\n";
+      }
+      os << pad() << "#pragma unroll\n" << pad() << "for (int v = 0; v < 16; v++) dc" << id << "[(8 * (v >> 2) + 4 * kg + (v & 3)) * " << N << " + col] = acc[v];\n";
+      indent--;
+      os << pad() << "}\n" << pad() << "__syncthreads();\n";
+      open_element_loop(R.shape);
+      os << pad() << "if (" << idx0(R.shape) << " / 32 == br) " << name << "[n] = "
+         << rounded(R.dtype, "dc" + id + "[(" + idx0(R.shape) + " % 32) * " + std::to_string(N) + " + " + idx1(R.shape) + "] + " +
+                                 at(s.operands.at(2), idx0(R.shape), idx1(R.shape)))
+         << ";\n";
+      close_loop();
+      os << pad() << "__syncthreads();\n";
+      indent--;
+      os << pad() << "}\n";
+      held[s.result] = {name, R.shape};
+      mine.push_back(s.result);
+      return;
+    }
     open_element_loop(R.shape);
     os << pad() << "float sum = 0.f;\n";
     os << pad() << "for (int k = 0; k < " << K << "; k++) sum += " << get(A.dtype, "da" + id + "[" + idx0(R.shape) + " * " + std::to_string(K) + " + k]") << " * "
@@ -1075,6 +1145,10 @@ __device__ inline long long smax(long long a, long long b) { return a > b ? a : 
 __device__ inline long long sdiv(long long a, long long b) { return b == 0 ? 0 : a / b; }
 __device__ inline long long srem(long long a, long long b) { return b == 0 ? 0 : a % b; }
 __device__ inline long long wrap(long long x, long long m) { return m > 0 ? ((x % m) + m) % m : x; }
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef unsigned short u16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 )SRC";
 
 }  // namespace

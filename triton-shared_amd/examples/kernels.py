@@ -222,3 +222,26 @@ def block_cumsum(x_ptr, y_ptr, n, BLOCK: tl.constexpr):
     i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
     m = i < n
     tl.store(y_ptr + i, tl.cumsum(tl.load(x_ptr + i, mask=m, other=0.0), axis=0), mask=m)
+
+
+@triton.jit
+def matmul_leaky_relu(a_ptr, b_ptr, c_ptr, M, N, K, s_am, s_bk, s_cm, slope, BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr):
+    """C = leaky_relu(A @ B): a tiled matmul with an activation fused before the narrowing store.  Not the shape the
+    hand-written MFMA kernels take: it runs on the generic family (operands staged in LDS, 32x32 MFMA blocks)."""
+    tm = tl.program_id(0)
+    tn = tl.program_id(1)
+    rm = tm * BM + tl.arange(0, BM)
+    rn = tn * BN + tl.arange(0, BN)
+    rk = tl.arange(0, BK)
+    pa = a_ptr + rm[:, None] * s_am + rk[None, :]
+    pb = b_ptr + rk[:, None] * s_bk + rn[None, :]
+    acc = tl.zeros((BM, BN), dtype=tl.float32)
+    for k in range(0, tl.cdiv(K, BK)):
+        left = K - k * BK
+        a = tl.load(pa, mask=(rm[:, None] < M) & (rk[None, :] < left), other=0.0)
+        b = tl.load(pb, mask=(rk[:, None] < left) & (rn[None, :] < N), other=0.0)
+        acc = tl.dot(a, b, acc)
+        pa += BK
+        pb += BK * s_bk
+    acc = tl.where(acc >= 0, acc, slope * acc)
+    tl.store(c_ptr + rm[:, None] * s_cm + rn[None, :], acc.to(c_ptr.dtype.element_ty), mask=(rm[:, None] < M) & (rn[None, :] < N))
