@@ -627,7 +627,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
   auto load_w = [&](int step, uint4 (&q)[8]) {
     const int8_t *src = w_lane + (int64_t)step * 32 * p.ldw;
 #pragma unroll
-    for (int t = 0; t < 8; t++) q[t] = *reinterpret_cast<const uint4 *>(src + (int64_t)t * p.ldw);
+    for (int t = 0; t < 8; t++) {
+      // the weights are read once per launch: nontemporal, so that they do not displace A, the scales and the partial
+      // tiles from the caches (46.2 -> 43.1 us at the decode shape with the weights coming from HBM)
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + (int64_t)t * p.ldw));
+      q[t] = make_uint4(v[0], v[1], v[2], v[3]);
+    }
   };
   auto load_a = [&](int step) { return *reinterpret_cast<const uint4 *>(a_lane + step * 32); };
   auto word = [](const uint4 &v, int i) -> uint32_t { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; };
