@@ -1,20 +1,34 @@
-// Structured program -> HIP source, for programs made of structured loads, elementwise ops and
-// stores (no reductions, no dots): the generic family behind the hand-tuned ones.
+// Structured program -> HIP source: the generic family behind the hand-tuned ones.  It takes whatever
+// program of block loads and stores (structured, wrapped, gathered / scattered), elementwise ops,
+// reductions, scans, index shuffles, small matrix products, loops and branches no other family took.
 //
 // What the reference does with such a program: one memref copy per load/store
-// (StructuredToMemref.cpp:748-853,1163-1196, wraparound as two chunks :263-487), one
-// linalg.generic loop per elementwise op (TritonArithToLinalg.cpp:104), scf.for around them.
-// Here one workgroup runs one program; a body's tile ops are fused into one loop over the
-// tile's elements (thread t takes elements t, t + 256, ...), index expressions are printed from
-// the expression pool with their i32 / index widths, and the source is compiled with hipRTC at
-// the plan's first launch.
+// (StructuredToMemref.cpp:748-853,1163-1196, wraparound as two chunks :263-487, gathers and scatters as
+// loops over rows :855-993,1034-1157), one linalg.generic loop per elementwise op
+// (TritonArithToLinalg.cpp:104), linalg.reduce / linalg.matmul (ConversionPatterns.hpp:1128-1440),
+// scf.for / scf.if around them.
+// Here one workgroup of 256 threads runs one program.  Thread t owns elements t, t + 256, ... of every
+// block (row-major); the ops of a body are fused into loops over the elements, index expressions are
+// printed from the expression pool with their i32 / index widths, and the source is compiled with
+// hipRTC at the plan's first launch.
 //
 // Order of memory effects.  The reference finishes every load of a body before the op after it
 // starts.  A fused element loop keeps that order per element only, which differs when a store
-// writes what another element's load reads (an in-place shift).  Tiles of up to 16384 elements are
-// therefore run in two phases -- every load of the body into per-thread registers, a barrier,
-// then ops and stores; larger tiles are fused in one loop and accepted only when no store's base
+// writes what another element's load reads (an in-place shift).  Blocks of up to 16384 elements are
+// therefore run in two phases -- every load of a run of ops into per-thread registers, a barrier,
+// then ops and stores; larger blocks are fused in one loop and accepted only when no store's base
 // argument is also a load's.
+//
+// Values.  A block value lives in one of four places: nowhere (an elementwise op is written out where
+// its result is used), the owning threads' registers (loads of a two-phase run, loop-carried blocks,
+// results of matrix products and of `if`), LDS (results of reductions and scans, small blocks of another
+// shape than the run's), or memory (a load of another shape that found no room in LDS is read again
+// where it is used; the program is refused if its base is also stored to).  Registers can only be named
+// for the element the thread owns: any other element, behind a transpose say, is computed again.
+//
+// Loads are written so that they issue back to back: a wavefront's loads complete in order, so a load
+// whose address waits for another load's result, or a select between a loaded value and `other` right
+// after the load, serialises the whole run (see the notes at the two places).
 #include <algorithm>
 #include <functional>
 #include <map>
