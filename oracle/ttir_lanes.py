@@ -111,16 +111,27 @@ class Interpreter:
     def __init__(self, ttir_text):
         lines = [l.strip() for l in _strip_loc(ttir_text).splitlines() if l.strip()]
         self.lines = lines
-        hdr = next(l for l in lines if l.startswith("tt.func"))
-        self.name = re.search(r"@(\w+)", hdr).group(1)
-        args = hdr[hdr.index("(") + 1:hdr.index(") attributes") if ") attributes" in hdr else hdr.rindex(")")]
-        self.args = []
-        for a in re.split(r",\s*(?=%)", args):
-            if not a.strip():
+        # every tt.func of the module: the public one is the kernel, the private ones are reached by tt.call
+        self.funcs = {}
+        for k, l in enumerate(lines):
+            if not l.startswith("tt.func"):
                 continue
-            name, ty = a.split(":", 1)
-            self.args.append((name.strip(), parse_type(ty.split("{")[0])))
-        self.body_start = lines.index(hdr) + 1
+            name = re.search(r"@([\w.$]+)", l).group(1)
+            depth, close = 0, l.index("(")
+            for close in range(l.index("("), len(l)):
+                depth += {"(": 1, ")": -1}.get(l[close], 0)
+                if depth == 0:
+                    break
+            args = []
+            for a in re.split(r",\s*(?=%)", l[l.index("(") + 1:close]):
+                if a.strip():
+                    arg, ty = a.split(":", 1)
+                    args.append((arg.strip(), parse_type(ty.split("{")[0])))
+            self.funcs[name] = (args, k + 1, self._skip_block(k + 1) - 1)
+            if "private" not in l[:l.index("@")]:
+                self.name, self.args, self.body_start = name, args, k + 1
+        self._range = self.funcs[self.name][1:]
+        self._returned = []
 
     # ---------------------------------------------------------------- running
     def run(self, grid, arg_values, memory):
@@ -160,24 +171,42 @@ class Interpreter:
                 i += 1
                 continue
             if line.startswith("tt.return"):
-                return len(L), None          # the program ends here (an early return sits in a block of its own)
+                # the function ends here (an early return sits in a block of its own); a callee leaves its values behind
+                self._returned = [env[n] for n in re.findall(r"%[\w.#$-]+", line.split(" : ")[0])]
+                return len(L), None
             if line.startswith("^"):         # a block label reached by falling through: cannot happen in valid IR
                 i += 1
                 continue
             if line.startswith("cf.cond_br"):
-                c, then, other = re.match(r"cf\.cond_br (%[\w.#$-]+), (\^\w+), (\^\w+)$", line).groups()
-                label = then if bool(env[c].d) else other
-                i = next(k for k, l in enumerate(L) if l.startswith(label + ":")) + 1
+                c, then, then_args, other, other_args = re.match(
+                    r"cf\.cond_br (%[\w.#$-]+), (\^\w+)(\([^)]*\))?, (\^\w+)(\([^)]*\))?$", line).groups()
+                i = self._jump(*((then, then_args) if bool(env[c].d) else (other, other_args)), env)
                 continue
             if line.startswith("cf.br"):
-                label = re.match(r"cf\.br (\^\w+)$", line).group(1)
-                i = next(k for k, l in enumerate(L) if l.startswith(label + ":")) + 1
+                i = self._jump(*re.match(r"cf\.br (\^\w+)(\([^)]*\))?$", line).groups(), env)
                 continue
             if line.startswith("scf.if") or re.match(r"%[\w.#$:-]+(, %[\w.#$:-]+)* = scf\.if ", line):
                 i = self._if(i, env)
                 continue
             i = self._op(i, env)
         return i, None
+
+    def _jump(self, label, passed, env):
+        """Branch to a block of the current function; the values in `passed` ("(%a, %b : i32, i32)") become its arguments."""
+        L = self.lines
+        k = next(k for k in range(*self._range) if L[k].startswith((label + ":", label + "(")))
+        if passed:
+            values = [env[n] for n in re.findall(r"%[\w.#$-]+", passed.split(" : ")[0])]
+            for n, v in zip(re.findall(r"(%[\w.#$-]+)\s*:", L[k]), values):
+                env[n] = v
+        return k + 1
+
+    def _call(self, callee, values):
+        args, start, end = self.funcs[callee]
+        saved, self._range, self._returned = self._range, (start, end), []
+        self._block(start, {name: v for (name, _ty), v in zip(args, values)})
+        self._range = saved
+        return self._returned
 
     def _if(self, i, env):
         """scf.if without results: `scf.if %c {` ... [`} else {` ...] `}`."""
@@ -231,7 +260,7 @@ class Interpreter:
         depth = 1
         L = self.lines
         while depth:
-            if L[i].endswith("{"):
+            if L[i].endswith("{") and not L[i].startswith("}"):
                 depth += 1
             if L[i] == "}" or L[i].startswith("})"):
                 depth -= 1
@@ -265,6 +294,11 @@ class Interpreter:
         if name == "arith.constant":
             lit, ty = (tail.rsplit(" : ", 1) + ["i1"])[:2] if " : " in tail else (tail, "i1")
             env[results[0]] = self._constant(lit.strip(), parse_type(ty))
+            return i + 1
+        if name == "tt.call":                        # @callee(%a, %b) : (types) -> types
+            callee, passed = re.match(r"@([\w.$]+)\((.*?)\)", tail).groups()
+            for r, v in zip(results, self._call(callee, [env[n] for n in re.findall(r"%[\w.#$-]+", passed)])):
+                env[r] = v
             return i + 1
         self._last_line = line
         head, _, types = self._split_types(tail)
@@ -337,9 +371,9 @@ class Interpreter:
                 return Val(np.full(shape, a.d, dtype=np.int64), a.elem, base=a.base)
             return Val(np.full(shape, a.d, dtype=_NP[a.elem]), a.elem)
         if name == "tt.trans":
-            order = [int(x) for x in re.findall(r"\d+", attrs.get("order", "") or "")]
+            order = [int(x) for x in re.search(r"order = array<i32: ([\d, ]+)>", self._last_line).group(1).split(",")]
             a = ops[0]
-            return Val(np.transpose(a.d, order[-a.d.ndim:] if order else None).copy(), a.elem, base=a.base)
+            return Val(np.transpose(a.d, order).copy(), a.elem, base=a.base)
         if name == "tt.cat":
             return Val(np.concatenate([ops[0].d, ops[1].d]), ops[0].elem)
         if name == "tt.join":
@@ -378,6 +412,8 @@ class Interpreter:
         p = ops[0]
         store = self.mem[p.base]
         if not isinstance(p.d, np.ndarray):
+            if len(ops) > 1 and not bool(ops[1].d):      # a scalar load under a false mask reads nothing
+                return Val(ops[2].d if len(ops) > 2 else _NP[p.elem](0), p.elem)
             self.acc.append(("load", p.base, np.array([p.d], dtype=np.int64)))
             return Val(self._widen(store[p.d:p.d + 1], p.elem)[0], p.elem)
         mask = ops[1].d if len(ops) > 1 else np.ones(p.d.shape, dtype=bool)
@@ -491,6 +527,12 @@ class Interpreter:
             if scalar_int:
                 return Val(_wrap(int(a.d), _INT_BITS[e]), e)
             return Val(a.d.astype(_NP[e]), e)
+        if name == "arith.extui":
+            bits = _INT_BITS[a.elem]
+            e = tys[-1].elem
+            if scalar_int:
+                return Val(int(a.d) & ((1 << bits) - 1), e)
+            return Val((a.d.astype(np.int64) & ((1 << bits) - 1)).astype(_NP[e]), e)
         e = tys[-1].elem if tys else a.elem
         if name == "tt.extern_elementwise":
             fn = re.search(r"__nv_(\w+?)f\b", " ".join(words) + " " + str(self._last_line)).group(1)
@@ -573,7 +615,7 @@ class Interpreter:
         k = int(env[lb].d)
         end = i + 1
         while k < int(env[ub].d):
-            env[iv] = Val(_wrap(k, 32), "i32")
+            env[iv] = Val(_wrap(k, _INT_BITS[env[lb].elem]), env[lb].elem)
             for n, v in zip(names, cur):
                 env[n] = v
             end, yielded = self._block(i + 1, env)
@@ -633,6 +675,8 @@ class Interpreter:
         axis = int(re.search(r"axis = (\d+)", tail).group(1))
         comb = re.match(r'(%[\w.#$-]+) = ([\w.]+)', self.lines[i + 2]).group(2)
         x = np.moveaxis(operand.d, axis, 0)
+        if operand.elem == "f64":                # the fast paths below accumulate in f32
+            return self._fold(i, results, tail, env, scan=False)
         if comb == "arith.addf" and x.ndim == 1:
             out = np.add.accumulate(x.astype(np.float32), dtype=np.float32)[-1]  # sequential fold
         elif comb == "arith.addf":

@@ -793,6 +793,29 @@ def test_reference_functional_case(name):
     case["check"]([d.cpu().numpy() for d in dev if isinstance(d, torch.Tensor)])
 
 
+def _core_case_ids():
+    import core_cases
+    return [c["name"] for c in core_cases.cases()]
+
+
+@pytest.mark.parametrize("name", _core_case_ids())
+def test_core_language_case(name):
+    """tests/core_cases.py: one kernel per language feature the reference enables from Triton's core tests
+    (python/examples/conftest.py:52-92), closed-form expectations; the same cases pin the lane oracle."""
+    import core_cases
+    import core_kernels
+    case = next(c for c in core_cases.cases() if c["name"] == name)
+    dev = []
+    for a, ty in zip(case["args"](), [t for t in case["sig"].values() if t != "constexpr"]):
+        if isinstance(a, np.ndarray):
+            a = torch.from_numpy(a).to(DEV)
+            a = a.view(torch.bfloat16) if ty == "*bf16" else a
+        dev.append(a)
+    getattr(core_kernels, case["kernel"])[case["grid"]](*dev, **case["consts"])
+    torch.cuda.synchronize()
+    case["check"]([(d.view(torch.uint16) if d.dtype == torch.bfloat16 else d).cpu().numpy() for d in dev if isinstance(d, torch.Tensor)])
+
+
 def test_tile_program_nested_pointer_walk_against_lane_interpreter():
     # python/examples/test_nested_loops.py is a template without expectations: the oracle provides them
     import extra_kernels as X

@@ -278,6 +278,28 @@ def test_lanes_on_the_reference_functional_cases():
                 assert o.size == 0 or (o.min() >= 0 and o.max() < arrays[arg].size), (case["name"], arg)
 
 
+def test_lanes_on_the_core_language_cases():
+    """The lane interpreter against closed forms for the language features the reference enables from Triton's core tests
+    (tests/core_cases.py): umulhi, 64-bit loop indices, calls of functions kept out of line, new axes, tl.full in every
+    type, double precision, early returns through merged blocks, NaN rules of min / max / clamp, permutes up to rank 4,
+    broadcasts, products of constants, masked scalar loads, fma, const pointers, arange, every fp16 value widened, abs,
+    cache hints, unary ops, // and %, argument specialisation, unary math, fp16 products."""
+    import core_cases
+    import core_kernels
+    from test_planner import compile_ttir
+    for case in core_cases.cases():
+        ttir = compile_ttir(getattr(core_kernels, case["kernel"]), case["sig"], case["consts"])
+        args = case["args"]()
+        arrays = [a for a in args if isinstance(a, np.ndarray)]
+        values = [None if isinstance(a, np.ndarray) else a for a in args]
+        log = ttir_lanes.Interpreter(ttir).run(case["grid"], values, dict(enumerate(arrays)))
+        case["check"](arrays)
+        for program in log:
+            for _kind, arg, offsets in program:
+                o = np.asarray(offsets)
+                assert o.size == 0 or (o.min() >= 0 and o.max() < arrays[arg].size), (case["name"], arg)
+
+
 def test_lanes_integer_bit_and_conversion_ops_against_numpy():
     """Unsigned division / remainder / compare / max, shifts, umulhi, abs, bit casts, float <-> integer conversions, clamp,
     correctly rounded sqrt / divide and fma: every plane bit for bit against tests/op_zoo.py."""

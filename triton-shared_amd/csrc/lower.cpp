@@ -673,8 +673,12 @@ class Lowerer {
     PtrState st = visit(op.operands[0]);
     s.acc = make_access(st, rt);
     if (!p.type.is_tensor) {
-      if (op.operands.size() > 1) throw Unsupported("masked scalar load");
       s.kind = SK::ScalarLoad;
+      if (op.operands.size() > 1) {  // a scalar condition: the value is `other` (or zero) when it is false
+        s.acc.mask_value = data_of(op.operands[1]);
+        s.operands.push_back(s.acc.mask_value);
+        if (op.operands.size() >= 3) scalar_other(op.operands[2], s.acc);
+      }
     } else {
       s.kind = SK::Load;
       if (op.operands.size() >= 2) {
@@ -713,8 +717,11 @@ class Lowerer {
     s.acc = make_access(st, vt);
     s.operands.push_back(data_of(op.operands[1]));
     if (!p.type.is_tensor) {
-      if (op.operands.size() > 2) throw Unsupported("masked scalar store");
       s.kind = SK::ScalarStore;
+      if (op.operands.size() > 2) {
+        s.acc.mask_value = data_of(op.operands[2]);
+        s.operands.push_back(s.acc.mask_value);
+      }
     } else {
       s.kind = SK::Store;
       if (op.operands.size() >= 3) {
@@ -1049,20 +1056,21 @@ class Lowerer {
         if (def(o).type.shape.size() > 1) throw Unsupported(n + " of blocks of rank > 1 (line " + std::to_string(op.line) + ")");
       return emit_simple(op, SK::Map, n, op.operands);
     }
-    if (n == "tt.trans" || n == "tt.reshape") {  // index shuffles: a Map whose element (i, j) reads another element of its operand
-      if (n == "tt.trans") {
-        // {order = array<i32: 1, 0>}: the digits after the element type
-        auto it = op.attrs.find("order");
-        std::string order = it == op.attrs.end() ? "" : it->second, digits;
-        const size_t colon = order.find(':');
-        for (char ch : order.substr(colon == std::string::npos ? 0 : colon))
-          if (isdigit((unsigned char)ch)) digits += ch;
-        if (rt.shape.size() != 2 || digits != "10") throw Unsupported("tt.trans other than the transpose of a rank-2 block (line " + std::to_string(op.line) + ")");
-      } else if (rt.shape.size() > 2 || def(op.operands.at(0)).type.shape.size() > 2) {
-        throw Unsupported("tt.reshape beyond rank 2 (line " + std::to_string(op.line) + ")");
-      }
-      return emit_simple(op, SK::Map, n, {op.operands.at(0)});
+    if (n == "tt.trans") {  // an index shuffle: a Map whose element reads another element of its operand; result dim d is operand dim order[d]
+      // {order = array<i32: 1, 0>}: the numbers after the element type
+      auto it = op.attrs.find("order");
+      std::string order = it == op.attrs.end() ? "" : it->second, name = "tt.trans";
+      const size_t colon = order.find(':');
+      size_t dims = 0;
+      for (char ch : order.substr(colon == std::string::npos ? 0 : colon))
+        if (isdigit((unsigned char)ch)) {
+          name += std::string(".") + ch;
+          dims++;
+        }
+      if (dims != rt.shape.size() || dims > 4) throw Unsupported("tt.trans whose order does not fit its block (line " + std::to_string(op.line) + ")");
+      return emit_simple(op, SK::Map, name == "tt.trans.1.0" ? "tt.trans" : name, {op.operands.at(0)});
     }
+    if (n == "tt.reshape") return emit_simple(op, SK::Map, n, {op.operands.at(0)});  // row-major element order is kept
     if (is_elementwise(n)) return emit_simple(op, SK::Map, map_name(op), op.operands);
     throw Unsupported("operation " + n + " (line " + std::to_string(op.line) + ") has no structured lowering");
   }
@@ -1173,6 +1181,52 @@ class Lowerer {
       changed = false;
       mark(P.body);
     }
+    // Loops whose carried integers are read after them (EK::Result nodes in the index expressions of what is kept) stay
+    // too, even with no block result and no effect inside: found as a fixed point over the expressions of the kept ops.
+    std::set<int> need_loop;
+    {
+      std::vector<char> seen(P.pool.size(), 0);
+      bool grew = true;
+      std::function<void(int)> note = [&](int e) {
+        if (e < 0 || seen[e]) return;
+        seen[e] = 1;
+        const Expr &x = P.pool.at(e);
+        switch (x.k) {
+          case EK::Const: case EK::Arg: case EK::Pid: case EK::NProg: case EK::IV: case EK::Iter: return;
+          case EK::Result:
+            if (need_loop.insert(x.a).second) grew = true;
+            return;
+          default:
+            note(x.a); note(x.b); note(x.c); note(x.d);
+        }
+      };
+      std::function<bool(const std::vector<SOp> &)> scan = [&](const std::vector<SOp> &ops) {
+        bool keep_any = false;
+        for (auto &s : ops) {
+          bool keep;
+          if (s.kind == SK::Store || s.kind == SK::ScalarStore) keep = true;
+          else if (s.kind == SK::For) {
+            keep = scan(s.body) || need_loop.count(s.loop);
+            for (int r : s.results) keep = keep || (r >= 0 && live[r]);
+          } else if (s.kind == SK::If) {
+            keep = scan(s.body);
+            for (int r : s.results) keep = keep || live[r];
+          } else if (!s.results.empty()) keep = live[s.results[0]];
+          else keep = s.result >= 0 && live[s.result];
+          if (!keep) continue;
+          keep_any = true;
+          for (auto *list : {&s.acc.offsets, &s.acc.strides, &s.acc.dims, &s.acc.mods})
+            for (int e : *list) note(e);
+          note(s.expr); note(s.lb); note(s.ub); note(s.step);
+          for (auto &it : s.int_iters) { note(it.init); note(it.next); }
+        }
+        return keep_any;
+      };
+      while (grew) {
+        grew = false;
+        scan(P.body);
+      }
+    }
     std::function<bool(std::vector<SOp> &)> sweep = [&](std::vector<SOp> &ops) {
       bool keep_any = false;
       std::vector<SOp> out;
@@ -1181,7 +1235,7 @@ class Lowerer {
         if (s.kind == SK::Store || s.kind == SK::ScalarStore) keep = true;
         else if (s.kind == SK::For) {
           bool eff = sweep(s.body);
-          bool res_live = false;
+          bool res_live = need_loop.count(s.loop) > 0;
           for (int r : s.results) res_live |= (r >= 0 && live[r]);
           keep = eff || res_live;
           if (keep) {

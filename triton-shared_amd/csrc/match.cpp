@@ -830,6 +830,11 @@ Plan make_plan(Program &&p) {
   pl.signature = signature(pl.prog);
   // the hand-written families read their operands through structured accesses only: a program with a gather or a
   // scatter goes to the generic family
+  if (pl.prog.body.empty()) {  // nothing with an effect on memory is left: an empty kernel keeps the launch's place in the stream
+    pl.source = tile_program_source(pl.prog);
+    pl.family = Family::TileProgram;
+    return pl;
+  }
   bool unstructured = false;
   {
     Matcher m(pl.prog);

@@ -38,7 +38,7 @@ struct Plan {
 
 // Generic family: HIP source for a program of structured loads, elementwise ops and stores
 // (tile_codegen.cpp).  Throws Unsupported for anything else.  The kernel's argument block holds
-// every kernel argument by index: { void *ptr[N]; long long ival[N]; float fval[N]; }, N = TILE_MAX_ARGS.
+// every kernel argument by index: { void *ptr[N]; long long ival[N]; double fval[N]; }, N = TILE_MAX_ARGS.
 constexpr int TILE_MAX_ARGS = 32;
 std::string tile_program_source(const Program &p);
 

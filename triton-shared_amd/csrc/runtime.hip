@@ -488,11 +488,11 @@ tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, cons
         break;
       }
       case Family::TileProgram: {
-        struct { void *ptr[TILE_MAX_ARGS]; long long ival[TILE_MAX_ARGS]; float fval[TILE_MAX_ARGS]; } a{};
+        struct { void *ptr[TILE_MAX_ARGS]; long long ival[TILE_MAX_ARGS]; double fval[TILE_MAX_ARGS]; } a{};
         for (int i = 0; i < n; i++) {
           if (args[i].kind == TTS_ARG_PTR) a.ptr[i] = args[i].v.ptr;
           else if (args[i].kind == TTS_ARG_INT) a.ival[i] = args[i].v.i;
-          else a.fval[i] = (float)args[i].v.f;
+          else a.fval[i] = args[i].v.f;
         }
         {
           std::lock_guard<std::mutex> lock(plan->mu);

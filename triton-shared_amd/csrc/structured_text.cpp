@@ -144,7 +144,8 @@ std::string print_program(const Program &p) {
           os << " base=" << s.acc.base_arg << " elem=" << s.acc.elem << " sizes=" << list(s.acc.sizes)
              << " offsets=" << list(s.acc.offsets) << " strides=" << list(s.acc.strides) << " dims=" << list(s.acc.dims);
           if (!s.acc.mods.empty()) os << " mods=" << list(s.acc.mods);
-          if (s.acc.gather >= 0) os << " gather=" << s.acc.gather << " maskv=" << s.acc.mask_value;
+          if (s.acc.gather >= 0) os << " gather=" << s.acc.gather;
+          if (s.acc.gather >= 0 || s.acc.mask_value >= 0) os << " maskv=" << s.acc.mask_value;
           if (s.acc.has_other) os << " other_f=" << dbl_bits(s.acc.other_f) << " other_i=" << s.acc.other_i;
           os << " ; " << p.arg_names[s.acc.base_arg] << " offsets=" << exprs(s.acc.offsets)
              << " strides=" << exprs(s.acc.strides);
@@ -365,10 +366,8 @@ Program read_program(const std::string &text) {
       s.acc.strides = Es(f.get("strides"));
       s.acc.dims = Es(f.get("dims"));
       if (f.has("mods")) s.acc.mods = Es(f.get("mods"));
-      if (f.has("gather")) {
-        s.acc.gather = std::stoi(f.get("gather"));
-        s.acc.mask_value = std::stoi(f.get("maskv"));
-      }
+      if (f.has("gather")) s.acc.gather = std::stoi(f.get("gather"));
+      if (f.has("maskv")) s.acc.mask_value = std::stoi(f.get("maskv"));
       if (f.has("other_f")) {
         s.acc.has_other = true;
         s.acc.other_f = bits_dbl(f.get("other_f"));

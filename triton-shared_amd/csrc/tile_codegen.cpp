@@ -67,6 +67,7 @@ struct Gen {
     if (t == "i16") return "short";
     if (t == "i32") return "int";
     if (t == "i64") return "long long";
+    if (t == "f64") return "double";
     throw Unsupported("tile_program: element type " + t);
   }
   static std::string memtype(const std::string &t) {
@@ -117,6 +118,46 @@ struct Gen {
     return n;
   }
 
+  // Blocks of rank above 2 are addressed like rank-2 blocks: i1 is the index along the last dimension and i0 the
+  // row-major index over all the others.  Where an op needs the index along one dimension, i0 is taken apart with
+  // divisions by constants, and put together again for the operand.
+  using Idx = std::vector<std::string>;
+  static Idx split_index(const std::vector<int64_t> &shape, const std::string &i0, const std::string &i1) {
+    const size_t r = shape.size();
+    if (r == 0) return {};
+    if (r == 1) return {i0};
+    if (r == 2) return {i0, i1};
+    Idx ix(r);
+    ix[r - 1] = i1;
+    int64_t below = 1;  // product of the leading dimensions after d
+    for (size_t d = r - 1; d-- > 0;) {
+      std::string e = below == 1 ? i0 : "(" + i0 + " / " + std::to_string(below) + ")";
+      ix[d] = shape[d] == 1 ? "0" : d == 0 ? e : "(" + e + " % " + std::to_string(shape[d]) + ")";
+      below *= shape[d];
+    }
+    return ix;
+  }
+  static std::pair<std::string, std::string> join_index(const std::vector<int64_t> &shape, const Idx &ix) {
+    const size_t r = shape.size();
+    if (r == 0) return {"0", "0"};
+    if (r == 1) return {ix[0], "0"};
+    if (r == 2) return {ix[0], ix[1]};
+    std::string lead;
+    int64_t below = 1;
+    for (size_t d = r - 1; d-- > 0;) {
+      if (ix[d] != "0") lead = (below == 1 ? ix[d] : ix[d] + " * " + std::to_string(below)) + (lead.empty() ? "" : " + " + lead);
+      below *= shape[d];
+    }
+    return {lead.empty() ? "0" : "(" + lead + ")", ix[r - 1]};
+  }
+  std::string at_index(int v, const Idx &ix) {
+    auto ij = join_index(val(v).shape, ix);
+    return at(v, ij.first, ij.second);
+  }
+  static std::string linear(const std::vector<int64_t> &shape, const std::string &i0, const std::string &i1) {
+    return shape.empty() ? "0" : shape.size() == 1 ? i0 : "(" + i0 + " * " + std::to_string(shape.back()) + " + " + i1 + ")";
+  }
+
   // C expression for element (i0, i1) of value v; rank-1 values use i0, scalars neither
   std::string at(int v, const std::string &i0, const std::string &i1) {
     auto it = var.find(v);
@@ -136,9 +177,17 @@ struct Gen {
       return shape.size() == 1 ? i0 : dim == 0 ? i0 : i1;
     };
     switch (s.kind) {
-      case SK::ScalarArg: return "p.fval[" + std::to_string(s.ival) + "]";
+      case SK::ScalarArg: return (V.dtype == "f64" ? "p.fval[" : "(float)p.fval[") + std::to_string(s.ival) + "]";
       case SK::FromIndex: return "(" + ctype(V.dtype) + ")" + ex(s.expr);
       case SK::Const:
+        if (V.dtype == "f64") {
+          std::ostringstream c;
+          if (s.fval != s.fval) return "__builtin_nan(\"\")";
+          if (s.fval == 1.0 / 0.0) return "__builtin_inf()";
+          if (s.fval == -1.0 / 0.0) return "(-__builtin_inf())";
+          c << std::hexfloat << s.fval;
+          return "(" + c.str() + ")";
+        }
         if (is_float(V.dtype)) {
           std::ostringstream c;
           c.precision(9);
@@ -154,22 +203,29 @@ struct Gen {
       case SK::ExpandDims: {
         // operand has one dimension fewer; element (i0, i1) reads the operand at the index of the kept dimension
         const Value &O = val(s.operands.at(0));
-        if (O.shape.size() != 1 || V.shape.size() != 2) no("expand_dims beyond rank 2");
-        return at(s.operands[0], s.axis == 0 ? i1 : i0, "0");
+        if (O.shape.size() + 1 != V.shape.size()) no("expand_dims that adds more than one dimension");
+        if (V.shape.size() == 2) return at(s.operands[0], s.axis == 0 ? i1 : i0, "0");
+        Idx ix = split_index(V.shape, i0, i1);
+        ix.erase(ix.begin() + s.axis);
+        return at_index(s.operands[0], ix);
       }
       case SK::Broadcast: {
         const Value &O = val(s.operands.at(0));
         if (O.shape.size() != V.shape.size()) no("broadcast that changes the rank");
         if (O.shape.size() == 1) return at(s.operands[0], O.shape[0] == 1 ? "0" : i0, "0");
-        return at(s.operands[0], O.shape[0] == 1 ? "0" : i0, O.shape[1] == 1 ? "0" : i1);
+        if (O.shape.size() == 2) return at(s.operands[0], O.shape[0] == 1 ? "0" : i0, O.shape[1] == 1 ? "0" : i1);
+        if (O.shape == V.shape) return at(s.operands[0], i0, i1);
+        Idx ix = split_index(V.shape, i0, i1);
+        for (size_t d = 0; d < ix.size(); d++)
+          if (O.shape[d] == 1) ix[d] = "0";
+        return at_index(s.operands[0], ix);
       }
       case SK::Load: {
         // a load that is not of the run's block shape (an index vector, a row of scales): from its copy in LDS when the
         // run staged one, else read where it is used (the program is then refused if anything stores to its base)
         auto st = staged.find(v);
         if (st != staged.end()) {
-          if (V.shape.size() == 2) return st->second + "[" + i0 + " * " + std::to_string(V.shape[1]) + " + " + i1 + "]";
-          return st->second + "[" + i0 + "]";
+          return st->second + "[" + linear(V.shape, i0, i1) + "]";
         }
         all_inline_bases.insert(s.acc.base_arg);
         std::string pred, addr = address(s.acc, i0, i1, pred);
@@ -182,15 +238,27 @@ struct Gen {
         for (size_t q = 0; q < s.results.size(); q++)
           if (s.results[q] == v) j = q;
         const std::string arr = "out" + std::to_string(s.result) + "_" + std::to_string(j);
-        if (V.shape.empty()) return arr + "[0]";
-        if (V.shape.size() == 1) return arr + "[" + i0 + "]";
-        return arr + "[" + i0 + " * " + std::to_string(V.shape[1]) + " + " + i1 + "]";
+        return arr + "[" + linear(V.shape, i0, i1) + "]";
       }
       case SK::Map: {
-        if (s.name == "tt.trans") {  // rank 2, order (1, 0)
+        if (s.name.rfind("tt.trans", 0) == 0) {  // "tt.trans" (rank 2, order (1, 0)) or "tt.trans.<order>": result dim d is operand dim order[d]
           const Value &O = val(s.operands.at(0));
-          if (O.shape.size() != 2 || V.shape.size() != 2) no("tt.trans of a block that is not of rank 2");
-          return at(s.operands[0], i1, i0);
+          if (O.shape.size() != V.shape.size()) no("tt.trans that changes the rank");
+          if (s.name == "tt.trans") {
+            if (V.shape.size() != 2) no("tt.trans of a block of rank above 2 without an order");
+            return at(s.operands[0], i1, i0);
+          }
+          std::vector<size_t> order;
+          for (size_t q = 8; q < s.name.size(); q++)
+            if (isdigit((unsigned char)s.name[q])) order.push_back((size_t)(s.name[q] - '0'));
+          if (order.size() != V.shape.size()) no("tt.trans with an order of another rank than the block");
+          const Idx ix = split_index(V.shape, i0, i1);
+          Idx ox(order.size());
+          for (size_t d = 0; d < order.size(); d++) {
+            if (order[d] >= order.size() || O.shape[order[d]] != V.shape[d]) no("tt.trans whose order does not fit the shapes");
+            ox[order[d]] = ix[d];
+          }
+          return at_index(s.operands[0], ox);
         }
         if (s.name == "tt.cat") {  // two rank-1 blocks end to end
           const int64_t na = val(s.operands.at(0)).shape.at(0);
@@ -203,15 +271,16 @@ struct Gen {
         if (s.name == "tt.unsplat") return at(s.operands.at(0), "0", "0");
         if (s.name == "tt.reshape") {  // row-major element order is kept
           const Value &O = val(s.operands.at(0));
-          const std::string lin = V.shape.size() == 2 ? "(" + i0 + " * " + std::to_string(V.shape[1]) + " + " + i1 + ")" : V.shape.size() == 1 ? i0 : "0";
-          if (O.shape.size() == 2) return at(s.operands[0], "(" + lin + " / " + std::to_string(O.shape[1]) + ")", "(" + lin + " % " + std::to_string(O.shape[1]) + ")");
+          const std::string lin = linear(V.shape, i0, i1);
+          if (O.shape.size() >= 2) return at(s.operands[0], "(" + lin + " / " + std::to_string(O.shape.back()) + ")", "(" + lin + " % " + std::to_string(O.shape.back()) + ")");
           return at(s.operands[0], O.shape.empty() ? "0" : lin, "0");
         }
         std::vector<std::string> a;
         for (int o : s.operands) {
           const Value &O = val(o);
           if (O.shape.size() == V.shape.size()) {
-            a.push_back(O.shape.size() == 2   ? at(o, idx(O.shape, 0), idx(O.shape, 1))
+            a.push_back(O.shape.size() > 2    ? at(o, i0, i1)
+                        : O.shape.size() == 2 ? at(o, idx(O.shape, 0), idx(O.shape, 1))
                         : O.shape.size() == 1 ? at(o, idx(O.shape, 0), "0")
                                               : at(o, "0", "0"));
           } else if (O.shape.empty()) a.push_back(at(o, "0", "0"));
@@ -251,6 +320,32 @@ struct Gen {
         {"une", "!(A == B)"}, {"ueq", "!(A < B || A > B)"}, {"ult", "!(A >= B)"}, {"ule", "!(A > B)"}, {"ugt", "!(A <= B)"},
         {"uge", "!(A < B)"}, {"ord", "A == A && B == B"}, {"uno", "A != A || B != B"}};
     static const std::map<std::string, const char *> cmpi = {{"slt", "<"}, {"sle", "<="}, {"sgt", ">"}, {"sge", ">="}, {"eq", "=="}, {"ne", "!="}};
+    if (rt == "f64" || ot == "f64") {  // double precision: the same ops through the double-precision library names
+      auto plain = [](std::string f) { f.pop_back(); return f; };  // "sqrtf" -> "sqrt"
+      if (bin_f.count(n)) { need(2); return a[0] + " " + bin_f.at(n) + " " + a[1]; }
+      if (n == "arith.maxnumf" || n == "arith.minnumf") { need(2); return std::string(n == "arith.maxnumf" ? "fmax(" : "fmin(") + a[0] + ", " + a[1] + ")"; }
+      if (n == "arith.maximumf" || n == "arith.minimumf") { need(2); return std::string(n == "arith.maximumf" ? "maximum_d(" : "minimum_d(") + a[0] + ", " + a[1] + ")"; }
+      if (fn1.count(n)) { need(1); return plain(fn1.at(n)) + "(" + a[0] + ")"; }
+      if (n == "math.rsqrt") { need(1); return "1.0 / sqrt(" + a[0] + ")"; }
+      if (n == "math.fma") { need(3); return "fma(" + a[0] + ", " + a[1] + ", " + a[2] + ")"; }
+      if (n == "arith.extf" || n == "arith.sitofp") { need(1); return "(double)" + a[0]; }
+      if (n == "arith.uitofp") { need(1); return "(double)(" + std::string(ot == "i64" ? "unsigned long long" : ot == "i8" ? "unsigned char" : ot == "i16" ? "unsigned short" : "unsigned") + ")" + a[0]; }
+      if (n == "arith.truncf") { need(1); return fl("(float)" + a[0]); }
+      if (n == "tt.precise_sqrt") { need(1); return "sqrt(" + a[0] + ")"; }
+      if (n == "tt.precise_divf") { need(2); return a[0] + " / " + a[1]; }
+      if (n == "arith.remf") { need(2); return "fmod(" + a[0] + ", " + a[1] + ")"; }
+      if (n == "tt.clampf.none") { need(3); return "fmin(fmax(" + a[0] + ", " + a[1] + "), " + a[2] + ")"; }
+      if (n == "tt.clampf.all") { need(3); return "minimum_d(maximum_d(" + a[0] + ", " + a[1] + "), " + a[2] + ")"; }
+      if (n == "tt.bitcast" || n == "arith.bitcast") {
+        need(1);
+        if (rt == ot) return a[0];
+        if (rt == "f64" && ot == "i64") return "__longlong_as_double(" + a[0] + ")";
+        if (rt == "i64" && ot == "f64") return "__double_as_longlong(" + a[0] + ")";
+        no("a bitcast between f64 and " + (rt == "f64" ? ot : rt));
+      }
+      if (n.rfind("extern.", 0) == 0) no("double-precision function " + n.substr(7));
+      // negation, select, comparisons and conversions to integers read the same for every width: below
+    }
     if (bin_f.count(n)) { need(2); return fl(a[0] + " " + bin_f.at(n) + " " + a[1]); }
     if (fn2.count(n)) { need(2); return fl(std::string(fn2.at(n)) + "(" + a[0] + ", " + a[1] + ")"); }
     if (fn1.count(n)) { need(1); return fl(std::string(fn1.at(n)) + "(" + a[0] + ")"); }
@@ -344,8 +439,9 @@ struct Gen {
       if (a.mask_value >= 0) pred = at(a.mask_value, i0, i1);
       return ex(a.offsets.at(0)) + " + (long long)" + at(a.gather, i0, i1);
     }
+    const Idx ix = split_index(a.sizes, i0, i1);
     for (size_t d = 0; d < a.sizes.size(); d++) {
-      const std::string i = a.sizes.size() == 1 ? i0 : d == 0 ? i0 : i1;
+      const std::string &i = ix[d];
       std::string term = "(" + ex(a.offsets[d]) + " + " + i + " * " + ex(a.strides[d]) + ")";
       if (!a.mods.empty() && a.mods[d] >= 0) term = "wrap(" + term + ", " + ex(a.mods[d]) + ")";
       sum += (d ? " + " : "") + term;
@@ -362,7 +458,15 @@ struct Gen {
     return ptr;
   }
   std::string other_of(const Access &a) {
-    if (!a.has_other) return is_float(a.elem) ? "0.f" : "(" + ctype(a.elem) + ")0";
+    if (!a.has_other) return a.elem == "f64" ? "0.0" : is_float(a.elem) ? "0.f" : "(" + ctype(a.elem) + ")0";
+    if (a.elem == "f64") {
+      if (a.other_f != a.other_f) return "__builtin_nan(\"\")";
+      if (a.other_f == 1.0 / 0.0) return "__builtin_inf()";
+      if (a.other_f == -1.0 / 0.0) return "(-__builtin_inf())";
+      std::ostringstream c;
+      c << std::hexfloat << a.other_f;
+      return "(" + c.str() + ")";
+    }
     if (is_float(a.elem)) {
       if (a.other_f != a.other_f) return "__builtin_nanf(\"\")";
       if (a.other_f == 1.0 / 0.0) return "__builtin_inff()";
@@ -394,8 +498,8 @@ struct Gen {
       else var.erase(h.first);
     }
   }
-  static std::string idx0(const std::vector<int64_t> &shape) { return shape.size() == 2 ? "(t / " + std::to_string(shape[1]) + ")" : "t"; }
-  static std::string idx1(const std::vector<int64_t> &shape) { return shape.size() == 2 ? "(t % " + std::to_string(shape[1]) + ")" : "0"; }
+  static std::string idx0(const std::vector<int64_t> &shape) { return shape.size() >= 2 ? "(t / " + std::to_string(shape.back()) + ")" : "t"; }
+  static std::string idx1(const std::vector<int64_t> &shape) { return shape.size() >= 2 ? "(t % " + std::to_string(shape.back()) + ")" : "0"; }
   std::string cur_i0, cur_i1;  // the index expressions of the element loop being written
   void open_element_loop(const std::vector<int64_t> &shape) {
     const int64_t T = count(shape);
@@ -480,7 +584,8 @@ struct Gen {
         map_vars({-1});
         std::string pred, addr = address(s.acc, "0", "0", pred);
         std::string name = "s" + std::to_string(s.result);
-        os << pad() << "const " << ctype(val(s.result).dtype) << " " << name << " = " << mem_read(s.acc, addr) << ";\n";
+        os << pad() << "const " << ctype(val(s.result).dtype) << " " << name << " = "
+           << (s.acc.mask_value >= 0 ? "(" + at(s.acc.mask_value, "0", "0") + ") ? " + mem_read(s.acc, addr) + " : " + other_of(s.acc) : mem_read(s.acc, addr)) << ";\n";
         var[s.result] = name;
         k++;
         continue;
@@ -488,7 +593,7 @@ struct Gen {
       if (s.kind == SK::ScalarStore) {
         map_vars({-1});
         std::string pred, addr = address(s.acc, "0", "0", pred);
-        os << pad() << "if (threadIdx.x == 0) {\n";
+        os << pad() << "if (threadIdx.x == 0" << (s.acc.mask_value >= 0 ? " && (" + at(s.acc.mask_value, "0", "0") + ")" : "") << ") {\n";
         indent++;
         mem_write(s.acc, addr, "", at(s.operands.at(0), "0", "0"));
         indent--;
@@ -525,14 +630,14 @@ struct Gen {
       for (size_t q = k; q < end; q++)
         if (ops[q].kind == SK::Store) {
           const auto &sz = ops[q].acc.sizes;
-          if (sz.size() > 2 || sz.empty()) no("block accesses of rank " + std::to_string(sz.size()));
+          if (sz.size() > 4 || sz.empty()) no("block accesses of rank " + std::to_string(sz.size()));
           if (!have) { shape = sz; have = stores = true; }
           if (sz != shape) no("block stores of different shapes next to each other");
         }
       for (size_t q = k; q < end; q++)
         if (ops[q].kind == SK::Load) {
           const auto &sz = ops[q].acc.sizes;
-          if (sz.size() > 2 || sz.empty()) no("block accesses of rank " + std::to_string(sz.size()));
+          if (sz.size() > 4 || sz.empty()) no("block accesses of rank " + std::to_string(sz.size()));
           if (!have || (!stores && count(sz) > count(shape))) { shape = sz; have = true; }
         }
       if (!have) { k = end; continue; }  // only elementwise ops: they are written out where their results are used
@@ -707,8 +812,9 @@ struct Gen {
     for (size_t q = 0; q < s.tile_args.size(); q++) held[s.tile_args[q]] = {"car" + L + "_" + std::to_string(q), cshape};
     for (size_t q = 0; q < s.int_iters.size(); q++)
       os << pad() << "long long it" << L << "_" << q << " = " << ex(s.int_iters[q].init) << ";\n";
-    os << pad() << "for (long long iv" << L << " = " << ex(s.lb) << "; iv" << L << " < " << ex(s.ub) << "; iv" << L << " = (long long)(int)(iv" << L
-       << " + " << ex(s.step) << ")) {\n";
+    // the induction variable wraps at the width of the loop's bounds
+    os << pad() << "for (long long iv" << L << " = " << ex(s.lb) << "; iv" << L << " < " << ex(s.ub) << "; iv" << L << " = "
+       << (P.pool.at(s.lb).bits == 32 ? "(long long)(int)" : "") << "(iv" << L << " + " << ex(s.step) << ")) {\n";
     indent++;
     std::vector<int> body_held;
     body(s.body, &body_held);
@@ -838,7 +944,7 @@ struct Gen {
   }
 
   // ---- reductions and scans ----------------------------------------------
-  static size_t held_bytes(const std::string &t) { return t == "i64" ? 8 : (t == "i1" || t == "i8") ? 1 : t == "i16" ? 2 : 4; }
+  static size_t held_bytes(const std::string &t) { return (t == "i64" || t == "f64") ? 8 : (t == "i1" || t == "i8") ? 1 : t == "i16" ? 2 : 4; }
 
   // `void <fname>(a0.., b0.., &r0..)`: r = combine(a, b)
   void combiner(const SOp &s, const std::string &fname) {
@@ -1142,7 +1248,7 @@ struct Gen {
 };
 
 const char *TILE_PRELUDE = R"SRC(
-struct Args { void *ptr[%N%]; long long ival[%N%]; float fval[%N%]; };
+struct Args { void *ptr[%N%]; long long ival[%N%]; double fval[%N%]; };
 __device__ inline float up_f16(unsigned short h) { _Float16 f; __builtin_memcpy(&f, &h, 2); return (float)f; }
 __device__ inline unsigned short down_f16(float f) { _Float16 h = (_Float16)f; unsigned short r; __builtin_memcpy(&r, &h, 2); return r; }
 __device__ inline float up_bf16(unsigned short h) { return __uint_as_float((unsigned)h << 16); }
@@ -1154,6 +1260,8 @@ __device__ inline unsigned short down_bf16(float f) {
 }
 __device__ inline float maximum_f(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
 __device__ inline float minimum_f(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
+__device__ inline double maximum_d(double a, double b) { return (a != a || b != b) ? __builtin_nan("") : fmax(a, b); }
+__device__ inline double minimum_d(double a, double b) { return (a != a || b != b) ? __builtin_nan("") : fmin(a, b); }
 __device__ inline long long smin(long long a, long long b) { return a < b ? a : b; }
 __device__ inline long long smax(long long a, long long b) { return a > b ? a : b; }
 __device__ inline long long sdiv(long long a, long long b) { return b == 0 ? 0 : a / b; }

@@ -345,6 +345,20 @@ static void parse_op(Lines &L, Block &blk) {
     return;
   }
 
+  if (op->name == "tt.call") {  // @callee(%a, %b) : (i32, i32) -> i32
+    const size_t at = rest.find('@'), open = rest.find('('), close = rest.find(')');
+    if (at == std::string::npos || open == std::string::npos || close == std::string::npos) throw Unsupported("cannot parse: " + line);
+    op->words.push_back(trim(rest.substr(at, open - at)));
+    collect_operands(rest.substr(open, close - open + 1), op->operands);
+    const size_t arrow = rest.find("->", close);
+    if (arrow != std::string::npos) {
+      std::string tys = trim(rest.substr(arrow + 2));
+      if (tys != "()") op->result_types = parse_type_list(tys);
+    }
+    if (op->result_types.size() != op->results.size()) throw Unsupported("tt.call: results and result types differ in number");
+    blk.ops.push_back(std::move(op));
+    return;
+  }
   // generic custom-assembly line: operands/words/attrs, then ':' types
   size_t colon = top_colon(rest);
   std::string head = colon == std::string::npos ? rest : rest.substr(0, colon);
@@ -394,79 +408,235 @@ static void parse_block(Lines &L, Block &blk) {
   }
 }
 
-// The body of the function may be a tree of basic blocks (an early `return` under an `if` becomes
-// cf.cond_br to a block that only returns).  It is rebuilt as nested "cf.if" ops with a then and an else
-// region; control flow that merges again, loops or passes block arguments is refused.
+// ---------------------------------------------------------------- copies of ops under new names
+// Tail duplication (a block reached from two branches) and the inlining of calls both copy ops; every copy gets
+// its own SSA names, so that nothing keyed by name downstream sees two definitions of one value.
+using Renames = std::map<std::string, std::string>;
+
+static std::string renamed(const std::string &name, const Renames &m) {
+  auto whole = m.find(name);  // one result of a pack ("%r#1") replaced by itself
+  if (whole != m.end()) return whole->second;
+  const size_t hash = name.find('#');
+  auto it = m.find(hash == std::string::npos ? name : name.substr(0, hash));
+  if (it == m.end()) return name;
+  return hash == std::string::npos ? it->second : it->second + name.substr(hash);
+}
+
+static void collect_defs(const Block &b, std::vector<std::string> &out) {
+  for (auto &a : b.arg_names) out.push_back(a);
+  for (auto &op : b.ops) {
+    for (auto &r : op->results) {
+      const size_t hash = r.find('#');
+      out.push_back(hash == std::string::npos ? r : r.substr(0, hash));
+    }
+    if (!op->iv.empty()) out.push_back(op->iv);
+    for (auto &n : op->iter_names) out.push_back(n);
+    for (auto &r : op->regions) collect_defs(r, out);
+  }
+}
+
+static void copy_block(const Block &src, Block &dst, const Renames &m);
+
+static std::unique_ptr<Op> copy_op(const Op &o, const Renames &m) {
+  auto c = std::make_unique<Op>();
+  c->name = o.name;
+  c->result_types = o.result_types;
+  c->words = o.words;
+  c->attrs = o.attrs;
+  c->types = o.types;
+  c->literal = o.literal;
+  c->line = o.line;
+  for (auto &r : o.results) c->results.push_back(renamed(r, m));
+  for (auto &r : o.operands) c->operands.push_back(renamed(r, m));
+  c->iv = o.iv.empty() ? o.iv : renamed(o.iv, m);
+  for (auto &r : o.iter_names) c->iter_names.push_back(renamed(r, m));
+  for (auto &r : o.iter_inits) c->iter_inits.push_back(renamed(r, m));
+  c->regions.resize(o.regions.size());
+  for (size_t i = 0; i < o.regions.size(); i++) copy_block(o.regions[i], c->regions[i], m);
+  return c;
+}
+
+static void copy_block(const Block &src, Block &dst, const Renames &m) {
+  for (auto &a : src.arg_names) dst.arg_names.push_back(renamed(a, m));
+  dst.arg_types = src.arg_types;
+  for (auto &op : src.ops) dst.ops.push_back(copy_op(*op, m));
+}
+
+// "^bb1(%a, %b : i32, i32)" -> label and the values passed
+static void parse_successor(const std::string &text, std::string &label, std::vector<std::string> &passed) {
+  std::string t = trim(text);
+  const size_t open = t.find('(');
+  label = trim(t.substr(0, open));
+  if (open == std::string::npos) return;
+  const size_t colon = t.find(':', open);
+  collect_operands(t.substr(open + 1, (colon == std::string::npos ? t.rfind(')') : colon) - open - 1), passed);
+}
+
+// The body of a function may be a graph of basic blocks (an early `return` under an `if` becomes cf.cond_br to a
+// block that only returns; blocks that end alike are merged and take arguments).  It is rebuilt as nested "cf.if"
+// ops with a then and an else region: a block reached from several places is copied to each of them, with the values
+// passed to it in place of its arguments; control flow that loops is refused.  A `tt.return` with operands stays in
+// the tree as an op (the body of a callee); one without ends its path.
 static void parse_func_body(Lines &L, Block &out) {
   struct Cfg {
     Block ops;
+    std::vector<std::string> arg_names;
     std::string term = "return", cond, a, b;
-    bool used = false;
+    std::vector<std::string> a_args, b_args, returned;
+    int copies = 0;
+    bool open = false;
   };
   std::map<std::string, Cfg> blocks;
   std::string cur = "^entry";
   blocks[cur];
-  auto label_of = [](const std::string &t) {
-    std::string l = trim(t);
-    if (l.find('(') != std::string::npos) throw Unsupported("branch with block arguments: " + l);
-    return l;
-  };
   while (L.i < L.v.size()) {
     const std::string line = L.v[L.i];
     if (line == "}") break;
-    if (line[0] == '^') {
+    if (line[0] == '^') {  // ^bb1:  or  ^bb1(%x: i32, %y: f32):
       size_t e = line.find_first_of(":(");
-      if (e == std::string::npos || line[e] == '(') throw Unsupported("block with arguments: " + line);
+      if (e == std::string::npos) throw Unsupported("cannot parse: " + line);
       cur = line.substr(0, e);
-      blocks[cur];
+      Cfg &c = blocks[cur];
+      if (line[e] == '(') {
+        const size_t close = line.rfind(')');
+        for (auto &a : split_top(line.substr(e + 1, close - e - 1), {","})) c.arg_names.push_back(trim(a.substr(0, a.find(':'))));
+      }
       L.i++;
       continue;
     }
     if (starts_with(line, "cf.cond_br")) {
       auto parts = split_top(line.substr(10), {","});
-      if (parts.size() != 3) throw Unsupported("cannot parse: " + line);
+      // the values passed to a successor are separated by commas too: glue the pieces of one parenthesis together again
+      std::vector<std::string> glued;
+      int depth = 0;
+      for (auto &piece : parts) {
+        if (depth > 0) glued.back() += "," + piece;
+        else glued.push_back(piece);
+        for (char ch : piece) depth += ch == '(' ? 1 : ch == ')' ? -1 : 0;
+      }
+      if (glued.size() != 3) throw Unsupported("cannot parse: " + line);
       Cfg &c = blocks[cur];
       c.term = "cond_br";
-      c.cond = trim(parts[0]);
-      c.a = label_of(parts[1]);
-      c.b = label_of(parts[2]);
+      c.cond = trim(glued[0]);
+      parse_successor(glued[1], c.a, c.a_args);
+      parse_successor(glued[2], c.b, c.b_args);
       L.i++;
       continue;
     }
     if (starts_with(line, "cf.br")) {
       Cfg &c = blocks[cur];
       c.term = "br";
-      c.a = label_of(line.substr(5));
+      parse_successor(line.substr(5), c.a, c.a_args);
       L.i++;
       continue;
     }
     if (starts_with(line, "tt.return")) {
-      blocks[cur].term = "return";
+      Cfg &c = blocks[cur];
+      c.term = "return";
+      const size_t colon = line.find(" : ");
+      collect_operands(line.substr(9, colon == std::string::npos ? std::string::npos : colon - 9), c.returned);
       L.i++;
       continue;
     }
     parse_op(L, blocks[cur].ops);
   }
-  std::function<void(const std::string &, Block &)> emit = [&](const std::string &label, Block &dst) {
-    auto it = blocks.find(label);
-    if (it == blocks.end()) throw Unsupported("branch to an unknown block " + label);
-    Cfg &c = it->second;
-    if (c.used) throw Unsupported("control flow that merges or loops (block " + label + " is reached twice)");
-    c.used = true;
-    for (auto &o : c.ops.ops) dst.ops.push_back(std::move(o));
-    if (c.term == "br") return emit(c.a, dst);
-    if (c.term == "cond_br") {
-      auto op = std::make_unique<Op>();
-      op->name = "cf.if";
-      op->operands.push_back(c.cond);
-      op->regions.resize(2);
-      Op *raw = op.get();
-      dst.ops.push_back(std::move(op));
-      emit(c.a, raw->regions[0]);
-      emit(c.b, raw->regions[1]);
+  int emitted = 0;
+  std::function<void(const std::string &, const std::vector<std::string> &, const Renames &, Block &)> emit =
+      [&](const std::string &label, const std::vector<std::string> &passed, const Renames &outer, Block &dst) {
+        auto it = blocks.find(label);
+        if (it == blocks.end()) throw Unsupported("branch to an unknown block " + label);
+        Cfg &c = it->second;
+        if (c.open) throw Unsupported("control flow that loops (block " + label + " reaches itself)");
+        if (passed.size() != c.arg_names.size()) throw Unsupported("branch to " + label + " with the wrong number of values");
+        // names visible in this copy: what the path so far renamed, this block's arguments, and (from the second copy
+        // on) fresh names for everything the block defines
+        Renames m = outer;
+        for (size_t i = 0; i < passed.size(); i++) m[c.arg_names[i]] = passed[i];
+        if (c.copies++) {
+          std::vector<std::string> defs;
+          collect_defs(c.ops, defs);
+          for (auto &d : defs) m[d] = d + "__c" + std::to_string(c.copies);
+        }
+        if ((emitted += (int)c.ops.ops.size() + 1) > 20000) throw Unsupported("control flow too tangled to unfold");
+        c.open = true;
+        for (auto &o : c.ops.ops) dst.ops.push_back(copy_op(*o, m));
+        auto values = [&](const std::vector<std::string> &v) {
+          std::vector<std::string> out;
+          for (auto &x : v) out.push_back(renamed(x, m));
+          return out;
+        };
+        if (c.term == "br") {
+          emit(c.a, values(c.a_args), m, dst);
+        } else if (c.term == "cond_br") {
+          auto op = std::make_unique<Op>();
+          op->name = "cf.if";
+          op->operands.push_back(renamed(c.cond, m));
+          op->regions.resize(2);
+          Op *raw = op.get();
+          dst.ops.push_back(std::move(op));
+          emit(c.a, values(c.a_args), m, raw->regions[0]);
+          emit(c.b, values(c.b_args), m, raw->regions[1]);
+        } else if (!c.returned.empty()) {
+          auto op = std::make_unique<Op>();
+          op->name = "tt.return";
+          op->operands = values(c.returned);
+          dst.ops.push_back(std::move(op));
+        }
+        c.open = false;
+      };
+  emit("^entry", {}, {}, out);
+}
+
+// ---------------------------------------------------------------- calls
+// A function kept out of line (`noinline`) arrives as its own tt.func and a tt.call.  The reference's pipeline inlines
+// it on the way down (triton-shared-opt runs the inliner before the conversion); here the callee's ops are copied to
+// the call site under fresh names, arguments replaced by the call's operands and the call's results by what the callee
+// returns.  A callee that returns values from inside a branch is refused.
+struct Callee {
+  Func f;
+  bool busy = false;
+};
+
+static void inline_calls(Block &b, std::map<std::string, Callee> &callees, Renames &subst, int &serial) {
+  std::vector<std::unique_ptr<Op>> out;
+  for (auto &a : b.arg_names) (void)a;
+  for (auto &held : b.ops) {
+    Op &op = *held;
+    for (auto &o : op.operands) o = renamed(o, subst);
+    for (auto &o : op.iter_inits) o = renamed(o, subst);
+    if (op.name != "tt.call") {
+      for (auto &r : op.regions) inline_calls(r, callees, subst, serial);
+      out.push_back(std::move(held));
+      continue;
     }
-  };
-  emit("^entry", out);
+    auto it = callees.find(op.words.at(0));
+    if (it == callees.end()) throw Unsupported("call of an unknown function " + op.words.at(0));
+    Callee &c = it->second;
+    if (c.busy) throw Unsupported("recursive call of " + op.words.at(0));
+    if (op.operands.size() != c.f.arg_names.size()) throw Unsupported("call of " + op.words.at(0) + " with the wrong number of arguments");
+    Renames m;
+    std::vector<std::string> defs;
+    collect_defs(c.f.body, defs);
+    const std::string tag = "__i" + std::to_string(++serial);
+    for (auto &d : defs) m[d] = d + tag;
+    for (size_t i = 0; i < op.operands.size(); i++) m[c.f.arg_names[i]] = op.operands[i];
+    Block body;
+    copy_block(c.f.body, body, m);
+    c.busy = true;
+    Renames inner;  // the callee's own calls
+    inline_calls(body, callees, inner, serial);
+    c.busy = false;
+    std::vector<std::string> returned;
+    if (!body.ops.empty() && body.ops.back()->name == "tt.return") {
+      returned = body.ops.back()->operands;
+      body.ops.pop_back();
+    }
+    if (returned.size() != op.results.size())
+      throw Unsupported("call of " + op.words.at(0) + ": the callee returns its values from inside a branch");
+    for (size_t i = 0; i < returned.size(); i++) subst[op.results[i]] = returned[i];
+    for (auto &o : body.ops) out.push_back(std::move(o));
+  }
+  b.ops = std::move(out);
 }
 
 Func parse_ttir(const std::string &text) {
@@ -480,18 +650,19 @@ Func parse_ttir(const std::string &text) {
       if (!ln.empty()) L.v.push_back(ln);
     }
   }
-  Func f;
+  Func kernel;
+  std::map<std::string, Callee> callees;
   bool found = false;
   while (L.i < L.v.size()) {
     const std::string &line = L.v[L.i];
     if (starts_with(line, "module")) { L.i++; continue; }
     if (line == "}") { L.i++; continue; }
     if (starts_with(line, "tt.func")) {
-      if (found) throw Unsupported("more than one tt.func in the module (non-inlined call?)");
-      found = true;
+      Func f;
       size_t at = line.find('@');
       size_t open = line.find('(', at);
       f.name = line.substr(at + 1, open - at - 1);
+      const bool is_private = line.substr(0, at).find("private") != std::string::npos;
       int depth = 0;
       size_t close = open;
       for (; close < line.size(); close++) {
@@ -508,18 +679,28 @@ Func parse_ttir(const std::string &text) {
           f.arg_names.push_back(trim(a.substr(0, col)));
           f.arg_types.push_back(parse_type(ty));
         }
-      if (line.find("->", close) != std::string::npos && line.find("->", close) < line.rfind('{'))
-        throw Unsupported("tt.func with results is not a kernel");
+      const bool has_results = line.find("->", close) != std::string::npos && line.find("->", close) < line.rfind('{');
+      if (has_results && !is_private) throw Unsupported("tt.func with results is not a kernel");
       L.i++;
       parse_func_body(L, f.body);
       if (L.i >= L.v.size() || L.v[L.i] != "}") throw Unsupported("tt.func body not closed");
       L.i++;
+      if (is_private) {
+        callees["@" + f.name].f = std::move(f);
+      } else {
+        if (found) throw Unsupported("more than one public tt.func in the module");
+        found = true;
+        kernel = std::move(f);
+      }
       continue;
     }
     throw Unsupported("unexpected top-level line: " + line);
   }
   if (!found) throw Unsupported("no tt.func found");
-  return f;
+  Renames subst;
+  int serial = 0;
+  inline_calls(kernel.body, callees, subst, serial);
+  return kernel;
 }
 
 }  // namespace tts
