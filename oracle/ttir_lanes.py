@@ -398,6 +398,9 @@ class Interpreter:
             return self._store(ops)
         if name == "tt.dot":
             a, b, c = ops
+            if a.elem in _INT_BITS:              # integer product: exact, wrapped to the accumulator's width
+                wide = a.d.astype(np.int64) @ b.d.astype(np.int64) + c.d.astype(np.int64)
+                return Val(wide.astype(_NP[c.elem]), c.elem)
             af, bf = a.d.astype(np.float32), b.d.astype(np.float32)
             prod = np.zeros(c.d.shape, dtype=np.float32)
             for k in range(af.shape[1]):  # k innermost per output element = this order for every (i, j)

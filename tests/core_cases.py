@@ -230,4 +230,61 @@ def cases():
         add(f"dot_fp16_acc{acc}", "dot_in_half_precision", {"a_ptr": H, "b_ptr": H, "c_ptr": P, "M": C, "N": C, "K": C, "ACC_IN": C}, {"M": 32, "N": 32, "K": 64, "ACC_IN": acc}, (1,),
             lambda: [ha.reshape(-1).copy(), hb.reshape(-1).copy(), hc.reshape(-1).copy()],
             lambda a, acc=acc: _eq(a[2].reshape(32, 32), ha.astype(np.float32) @ hb.astype(np.float32) + (hc if acc else 0)))
+    # tile products with the epilogues of the core dot test; small integers so that every order of summation is exact
+    for dt, name in [(np.float32, "fp32"), (np.float16, "fp16"), (np.int8, "i8")]:
+        M, N, K = 32, 32, 64
+        dx_ = rng.integers(-3, 4, (M, K)).astype(dt)
+        dy_ = rng.integers(-3, 4, (K, N)).astype(dt)
+        dw_ = rng.integers(-2, 3, (N, N)).astype(dt)
+        acc_t = np.int32 if dt == np.int8 else np.float32
+        dz_ = rng.integers(-9, 10, (M, N)).astype(acc_t)
+        prod = dx_.astype(np.int64) @ dy_.astype(np.int64)
+        sig = {"x_ptr": "*" + name, "y_ptr": "*" + name, "w_ptr": "*" + name, "z_ptr": "*i32" if dt == np.int8 else P, "M": C, "N": C, "K": C, "EPI": C}
+        for epi in range(7):
+            if epi == 4 and dt == np.int8:
+                continue
+            if epi == 5 and dt == np.float16:       # the first product is narrowed to fp16 before the second: keep it exact
+                prod5 = np.clip(prod, -2048, 2048)
+                assert np.array_equal(prod5, prod)
+
+            def check(a, epi=epi, prod=prod, dz_=dz_, dw_=dw_, acc_t=acc_t, M=M, N=N):
+                got = a[3].reshape(N, M).T if epi == 6 else a[3].reshape(M, N)
+                if epi == 4:
+                    e = np.exp((prod - prod.max(1, keepdims=True)).astype(np.float64))
+                    return _close(got, e / e.sum(1, keepdims=True), 1e-6)
+                want = [prod, prod + dz_, prod + dz_[:, :1], prod + dz_[:1, :], None, prod @ dw_.astype(np.int64), prod][epi]
+                _eq(got, want.astype(acc_t))
+            add(f"dot_{name}_epilogue{epi}", "dot_with_epilogue", sig, {"M": M, "N": N, "K": K, "EPI": epi}, (1,),
+                lambda dx_=dx_, dy_=dy_, dw_=dw_, dz_=dz_: [dx_.reshape(-1).copy(), dy_.reshape(-1).copy(), dw_.reshape(-1).copy(), dz_.reshape(-1).copy()], check)
+
+    # integer arithmetic, bit operations, shifts and comparisons in every width and signedness
+    for dt, name in [(np.int8, "i8"), (np.int16, "i16"), (np.int32, "i32"), (np.int64, "i64"), (np.uint8, "u8"), (np.uint16, "u16"), (np.uint32, "u32"), (np.uint64, "u64")]:
+        info = np.iinfo(dt)
+        n = 600
+        ix = rng.integers(info.min, info.max, n, dtype=dt, endpoint=True)
+        iy = rng.integers(info.min, info.max, n, dtype=dt, endpoint=True)
+        iy[iy == 0] = 3
+        if info.min < 0:
+            iy[iy == -1] = 5                                        # min // -1 overflows: undefined in the source language
+        ix[:3] = [info.min, info.max, 0]
+
+        def check_int(a, dt=dt, ix=ix, iy=iy, n=n, info=info):
+            o = a[2].reshape(13, n)
+            X, Y = [int(v) for v in ix], [int(v) for v in iy]
+            bits = info.bits
+
+            def wrap(v):
+                v &= (1 << bits) - 1
+                return v - (1 << bits) if info.min < 0 and v >> (bits - 1) else v
+            tdiv = lambda p, q: abs(p) // abs(q) * (1 if (p < 0) == (q < 0) else -1)       # C division: towards zero
+            planes = [[wrap(p + q) for p, q in zip(X, Y)], [wrap(p - q) for p, q in zip(X, Y)], [wrap(p * q) for p, q in zip(X, Y)],
+                      [wrap(tdiv(p, q)) for p, q in zip(X, Y)], [wrap(p - tdiv(p, q) * q) for p, q in zip(X, Y)],
+                      [wrap(p & q) for p, q in zip(X, Y)], [wrap(p | q) for p, q in zip(X, Y)], [wrap(p ^ q) for p, q in zip(X, Y)],
+                      [wrap(p << (q & 3)) for p, q in zip(X, Y)], [wrap(p >> (q & 3)) for p, q in zip(X, Y)],
+                      [(p < q) + 2 * (p <= q) + 4 * (p == q) for p, q in zip(X, Y)], [wrap(max(p, q) - min(p, q)) for p, q in zip(X, Y)],
+                      [max(p, q) for p, q in zip(X, Y)]]
+            for k, (got, want) in enumerate(zip(o, planes)):
+                assert [int(v) for v in got] == want, (k, [int(v) for v in got][:8], want[:8])
+        add(f"int_ops_{name}", "integer_ops_any_width", {"x_ptr": "*" + name, "y_ptr": "*" + name, "out_ptr": "*" + name, "n": "i32", "BLOCK": C}, {"BLOCK": 256}, (3,),
+            lambda ix=ix, iy=iy, dt=dt, n=n: [ix.copy(), iy.copy(), np.zeros(13 * n, dt), n], check_int)
     return out

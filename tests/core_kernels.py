@@ -337,3 +337,56 @@ def dot_in_half_precision(a_ptr, b_ptr, c_ptr, M: tl.constexpr, N: tl.constexpr,
     else:
         c = tl.dot(a, b)
     tl.store(c_ptr + i[:, None] * N + j[None, :], c)
+
+
+@triton.jit
+def dot_with_epilogue(x_ptr, y_ptr, w_ptr, z_ptr, M: tl.constexpr, N: tl.constexpr, K: tl.constexpr, EPI: tl.constexpr):
+    # one tile product, then: 0 nothing, 1 + matrix, 2 + a value per row, 3 + a value per column, 4 row softmax,
+    # 5 a second product with w[N, N], 6 the result stored transposed
+    i = tl.arange(0, M)
+    j = tl.arange(0, N)
+    k = tl.arange(0, K)
+    x = tl.load(x_ptr + i[:, None] * K + k[None, :])
+    y = tl.load(y_ptr + k[:, None] * N + j[None, :])
+    z = tl.dot(x, y)
+    at = z_ptr + i[:, None] * N + j[None, :]
+    if EPI == 1:
+        z += tl.load(at)
+    if EPI == 2:
+        z += tl.load(z_ptr + i * N)[:, None]
+    if EPI == 3:
+        z += tl.load(z_ptr + j)[None, :]
+    if EPI == 4:
+        z = z - tl.max(z, 1)[:, None]
+        num = tl.exp(z)
+        z = num / tl.sum(num, 1)[:, None]
+    if EPI == 5:
+        w = tl.load(w_ptr + j[:, None] * N + j[None, :])
+        z = tl.dot(z.to(w.dtype), w)
+    if EPI == 6:
+        tl.store(z_ptr + i[:, None] + j[None, :] * M, z)
+    else:
+        tl.store(at, z)
+
+
+@triton.jit
+def integer_ops_any_width(x_ptr, y_ptr, out_ptr, n, BLOCK: tl.constexpr):
+    # the planes of test_bin_op / test_bitwise_op / test_shift_op / comparisons for whatever integer type the pointers have
+    o = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = o < n
+    x = tl.load(x_ptr + o, mask=m, other=1)
+    y = tl.load(y_ptr + o, mask=m, other=1)
+    s = (y & 3).to(x.dtype)
+    tl.store(out_ptr + 0 * n + o, x + y, mask=m)
+    tl.store(out_ptr + 1 * n + o, x - y, mask=m)
+    tl.store(out_ptr + 2 * n + o, x * y, mask=m)
+    tl.store(out_ptr + 3 * n + o, x // y, mask=m)
+    tl.store(out_ptr + 4 * n + o, x % y, mask=m)
+    tl.store(out_ptr + 5 * n + o, x & y, mask=m)
+    tl.store(out_ptr + 6 * n + o, x | y, mask=m)
+    tl.store(out_ptr + 7 * n + o, x ^ y, mask=m)
+    tl.store(out_ptr + 8 * n + o, x << s, mask=m)
+    tl.store(out_ptr + 9 * n + o, x >> s, mask=m)
+    tl.store(out_ptr + 10 * n + o, (x < y).to(x.dtype) + (x <= y).to(x.dtype) * 2 + (x == y).to(x.dtype) * 4, mask=m)
+    tl.store(out_ptr + 11 * n + o, tl.maximum(x, y) - tl.minimum(x, y), mask=m)
+    tl.store(out_ptr + 12 * n + o, tl.where(x > y, x, y), mask=m)

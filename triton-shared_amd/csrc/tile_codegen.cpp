@@ -860,10 +860,14 @@ struct Gen {
     const size_t a_size = narrow(A.dtype) ? 2 : 4, b_size = narrow(B.dtype) ? 2 : 4;
     const size_t a_bytes = ((size_t)(M * K) * a_size + 15) / 16 * 16, bytes = a_bytes + (size_t)(K * N) * b_size;
     if (bytes > 48 * 1024) no("a matrix product whose operands need " + std::to_string(bytes) + " bytes of LDS (limit 49152)");
-    if (!is_float(A.dtype) || !is_float(B.dtype) || !is_float(R.dtype)) no("an integer matrix product");
+    // integers (i8 x i8 -> i32 and the like): staged as 32-bit integers, multiplied and added with wrap-around
+    const bool integer = !is_float(A.dtype) && !is_float(B.dtype) && !is_float(R.dtype);
+    if (!integer && (!is_float(A.dtype) || !is_float(B.dtype) || !is_float(R.dtype))) no("a matrix product that mixes integers and floats");
+    if (A.dtype == "f64" || B.dtype == "f64" || R.dtype == "f64" || A.dtype == "i64" || B.dtype == "i64" || R.dtype == "i64")
+      no("a matrix product of 64-bit elements");
     pool_bytes = std::max(pool_bytes, bytes);
     const std::string id = std::to_string(s.result);
-    auto staged_type = [&](const std::string &t) { return narrow(t) ? std::string("unsigned short") : std::string("float"); };
+    auto staged_type = [&](const std::string &t) { return integer ? std::string("int") : narrow(t) ? std::string("unsigned short") : std::string("float"); };
     auto put = [&](const std::string &t, const std::string &e) { return t == "f16" ? "down_f16(" + e + ")" : t == "bf16" ? "down_bf16(" + e + ")" : e; };
     auto get = [&](const std::string &t, const std::string &e) { return t == "f16" ? "up_f16(" + e + ")" : t == "bf16" ? "up_bf16(" + e + ")" : e; };
     os << pad() << "__syncthreads();\n";
@@ -877,7 +881,7 @@ struct Gen {
     const bool both16 = A.dtype == B.dtype && narrow(A.dtype);
     const bool both32 = A.dtype == "f32" && B.dtype == "f32";
     const size_t band_bytes = (size_t)32 * N * 4;
-    const bool mfma = M % 32 == 0 && N % 32 == 0 && ((both16 && K % 16 == 0) || (both32 && K % 2 == 0)) && band_bytes <= 32 * 1024 &&
+    const bool mfma = !integer && M % 32 == 0 && N % 32 == 0 && ((both16 && K % 16 == 0) || (both32 && K % 2 == 0)) && band_bytes <= 32 * 1024 &&
                       bytes + band_bytes <= 60 * 1024;
     open_element_loop(B.shape);
     if (mfma && both16)
@@ -887,7 +891,7 @@ struct Gen {
     close_loop();
     os << pad() << "__syncthreads();\n";
     const std::string name = "dot" + id;
-    os << pad() << "float " << name << "[" << (M * N + 255) / 256 << "];\n";
+    os << pad() << (integer ? "int " : "float ") << name << "[" << (M * N + 255) / 256 << "];\n";
     // Matrix cores when the shapes allow: 32 x 32 output blocks, one 32-row band of the result at a time.  The four
     // wavefronts take the band's column blocks in turn, accumulate over K with v_mfma_f32_32x32x16 (16-bit operands) or
     // 32x32x2 (fp32), and leave the band in LDS, from where every thread picks up the elements it owns.
@@ -928,6 +932,18 @@ struct Gen {
       os << pad() << "__syncthreads();\n";
       indent--;
       os << pad() << "}\n";
+      held[s.result] = {name, R.shape};
+      mine.push_back(s.result);
+      return;
+    }
+    if (integer) {
+      open_element_loop(R.shape);
+      os << pad() << "unsigned sum = 0u;\n";
+      os << pad() << "for (int k = 0; k < " << K << "; k++) sum += (unsigned)da" << id << "[" << idx0(R.shape) << " * " << K << " + k] * (unsigned)db" << id << "[k * "
+         << N << " + " << idx1(R.shape) << "];\n";
+      os << pad() << name << "[n] = (int)(sum + (unsigned)" << at(s.operands.at(2), idx0(R.shape), idx1(R.shape)) << ");\n";
+      close_loop();
+      os << pad() << "__syncthreads();\n";
       held[s.result] = {name, R.shape};
       mine.push_back(s.result);
       return;
