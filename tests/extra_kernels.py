@@ -778,3 +778,119 @@ def matmul_leaky(a_ptr, b_ptr, c_ptr, M, N, K, s_am, s_bk, s_cm, slope, BM: tl.c
         pb += BK * s_bk
     acc = tl.where(acc >= 0, acc, slope * acc)
     tl.store(c_ptr + rm[:, None] * s_cm + rn[None, :], acc.to(c_ptr.dtype.element_ty), mask=(rm[:, None] < M) & (rn[None, :] < N))
+
+
+@triton.jit
+def masks_from_memory_3d(src, dst, keep_rows, keep_cols, b, m, n, B: tl.constexpr, M: tl.constexpr, N: tl.constexpr):
+    # masks_from_memory_2d for every matrix of a batch: the middle index masked by data on the load, the last one on the store
+    q = tl.arange(0, B)
+    r = tl.arange(0, M)
+    c = tl.arange(0, N)
+    kr = tl.load(keep_rows + r, mask=r < m, other=0) != 0
+    kc = tl.load(keep_cols + c, mask=c < n, other=0) != 0
+    at = q[:, None, None] * (m * n) + r[None, :, None] * n + c[None, None, :]
+    v = tl.load(src + at, mask=(q[:, None, None] < b) & kr[None, :, None] & (c[None, None, :] < n), other=-2)
+    tl.store(dst + at, v, mask=(q[:, None, None] < b) & (r[None, :, None] < m) & kc[None, None, :])
+
+
+@triton.jit
+def columns_by_index_masked(src, dst, idx, n_idx, m, n, pitch_m, pitch_n, M: tl.constexpr, IN: tl.constexpr):
+    # dst[:, idx[k]] = src[:, k] for idx[k] < n
+    r = tl.arange(0, M)
+    k = tl.arange(0, IN)
+    which = tl.load(idx + k, mask=k < n_idx, other=0)
+    ok = (which < n) & (k < n_idx)
+    v = tl.load(src + r[:, None] * pitch_m + k[None, :] * pitch_n, mask=(r[:, None] < m) & (k[None, :] < n_idx), other=-2)
+    tl.store(dst + r[:, None] * pitch_m + which[None, :] * pitch_n, v, mask=(r[:, None] < m) & ok[None, :])
+
+
+@triton.jit
+def rows_by_index_masked_3d(src, dst, idx, n_idx, b, m, n, s_b, s_m, s_n, d_b, d_m, d_n, B: tl.constexpr, IM: tl.constexpr, N: tl.constexpr):
+    # dst[q, k, :] = src[q, idx[k], :] for idx[k] < m (else -2)
+    q = tl.arange(0, B)
+    k = tl.arange(0, IM)
+    c = tl.arange(0, N)
+    which = tl.load(idx + k, mask=k < n_idx, other=0)
+    ok = (which < m) & (k < n_idx)
+    v = tl.load(src + q[:, None, None] * s_b + which[None, :, None] * s_m + c[None, None, :] * s_n,
+                mask=(q[:, None, None] < b) & ok[None, :, None] & (c[None, None, :] < n), other=-2)
+    tl.store(dst + q[:, None, None] * d_b + k[None, :, None] * d_m + c[None, None, :] * d_n, v,
+             mask=(q[:, None, None] < b) & (k[None, :, None] < n_idx) & (c[None, None, :] < n))
+
+
+@triton.jit
+def columns_by_index_masked_3d(src, dst, idx, n_idx, b, m, n, s_b, s_m, s_n, B: tl.constexpr, M: tl.constexpr, IN: tl.constexpr):
+    # dst[q, :, idx[k]] = src[q, :, k] for idx[k] < n
+    q = tl.arange(0, B)
+    r = tl.arange(0, M)
+    k = tl.arange(0, IN)
+    which = tl.load(idx + k, mask=k < n_idx, other=0)
+    ok = (which < n) & (k < n_idx)
+    v = tl.load(src + q[:, None, None] * s_b + r[None, :, None] * s_m + k[None, None, :] * s_n,
+                mask=(q[:, None, None] < b) & (r[None, :, None] < m) & (k[None, None, :] < n_idx), other=-2)
+    tl.store(dst + q[:, None, None] * s_b + r[None, :, None] * s_m + which[None, None, :] * s_n, v,
+             mask=(q[:, None, None] < b) & (r[None, :, None] < m) & ok[None, None, :])
+
+
+@triton.jit
+def masks_above_program_id(src, dst, m, n, s_pid, s_m, s_n, M: tl.constexpr, N: tl.constexpr):
+    # rows beyond the program id are loaded (other = -2), columns beyond it stored: comparisons against a value that is
+    # not a bound of the block, together with the ordinary bounds
+    pid = tl.program_id(0)
+    r = tl.arange(0, M)
+    c = tl.arange(0, N)
+    at = pid * s_pid + r[:, None] * s_m + c[None, :] * s_n
+    v = tl.load(src + at, mask=(r[:, None] < m) & (c[None, :] < n) & (r > pid)[:, None], other=-2)
+    tl.store(dst + at, v, mask=(r[:, None] < m) & (c[None, :] < n) & (c > pid)[None, :])
+
+
+# ---- blocks past the register budget, reductions of rank-3 blocks -----------------------------
+@triton.jit
+def reduce_big_block_2d(x_ptr, out_ptr, R: tl.constexpr, C: tl.constexpr, AXIS: tl.constexpr, KIND: tl.constexpr):
+    # one program reduces a whole [R, C] block (test/Conversion/TritonToLinalg/reducesum_512_256_*_axis{0,1}.mlir do this at 512 x 256)
+    r = tl.arange(0, R)
+    c = tl.arange(0, C)
+    x = tl.load(x_ptr + r[:, None] * C + c[None, :])
+    if KIND == 0:
+        v = tl.sum(x, axis=AXIS)
+    else:
+        v = tl.max(x, axis=AXIS)
+    if AXIS == 0:
+        tl.store(out_ptr + c, v)
+    else:
+        tl.store(out_ptr + r, v)
+
+
+@triton.jit
+def block_total_and_extremes(x_ptr, out_ptr, n, BLOCK: tl.constexpr):
+    i = tl.arange(0, BLOCK)
+    x = tl.load(x_ptr + i, mask=i < n, other=0)
+    tl.store(out_ptr, tl.sum(x, axis=0))
+    tl.store(out_ptr + 1, tl.max(x, axis=0))
+    tl.store(out_ptr + 2, tl.min(x, axis=0))
+
+
+@triton.jit
+def reduce_3d(x_ptr, out_ptr, A: tl.constexpr, B: tl.constexpr, C: tl.constexpr, AXIS: tl.constexpr, KIND: tl.constexpr):
+    # test/Conversion/StructuredToMemref/reducesum_middle_dim.mlir reduces the middle index of a rank-3 block
+    a = tl.arange(0, A)
+    b = tl.arange(0, B)
+    c = tl.arange(0, C)
+    x = tl.load(x_ptr + a[:, None, None] * (B * C) + b[None, :, None] * C + c[None, None, :])
+    if KIND == 0:
+        v = tl.sum(x, axis=AXIS)
+    else:
+        v = tl.max(x, axis=AXIS)
+    if AXIS == 0:
+        tl.store(out_ptr + b[:, None] * C + c[None, :], v)
+    elif AXIS == 1:
+        tl.store(out_ptr + a[:, None] * C + c[None, :], v)
+    else:
+        tl.store(out_ptr + a[:, None] * B + b[None, :], v)
+
+
+@triton.jit
+def shift_left_in_place(x_ptr, R: tl.constexpr, C: tl.constexpr):
+    # every element takes its right neighbour's old value: all loads come before any store, whatever the block's size
+    at = tl.arange(0, R)[:, None] * C + tl.arange(0, C)[None, :]
+    tl.store(x_ptr + at, tl.load(x_ptr + at + 1))

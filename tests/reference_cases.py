@@ -94,6 +94,58 @@ def cases():
         {"src": P, "dst": P, "idx": I, "n_idx": "i32", "m": "i32", "n": "i32", "pitch_m": "i32", "pitch_n": "i32", "IM": "constexpr", "N": "constexpr"},
         {"IM": 4, "N": 16}, (1,), lambda: [xin.reshape(-1).copy(), np.full(3 * n, -1, np.float32), idx.copy(), 3, m, n, n, 1],
         lambda a: _eq(a[1], want_rows()))
+    # test_unstructured_mask.py:69-110 (the batched form), 167-211 (columns through an index), 215-325 (both in three
+    # dimensions), 328-375 (masks from comparisons with the program id)
+    b3 = 4
+    x3 = np.arange(2, 2 + b3 * m * n, dtype=np.float32).reshape(b3, m, n)
+
+    def want_masks_3d():
+        v = np.full_like(x3, -2)
+        v[:, keep_r != 0, :] = x3[:, keep_r != 0, :]
+        w = np.full_like(x3, -1)
+        w[:, :, keep_c != 0] = v[:, :, keep_c != 0]
+        return w.reshape(-1)
+    add("masks_from_memory_3d", "masks_from_memory_3d",
+        {"src": P, "dst": P, "keep_rows": "*i8", "keep_cols": "*i8", "b": "i32", "m": "i32", "n": "i32", "B": "constexpr", "M": "constexpr", "N": "constexpr"},
+        {"B": 4, "M": M, "N": N}, (1,),
+        lambda: [x3.reshape(-1).copy(), np.full(x3.size, -1, np.float32), keep_r.copy(), keep_c.copy(), b3, m, n], lambda a: _eq(a[1], want_masks_3d()))
+    idx_n = np.array([10, 20, 15, 1, 3, 5, 7, 0, 2, 4, 6, 8], dtype=np.int32)
+
+    def want_columns(src):
+        w = np.full_like(src, -1)
+        ok = idx_n < n
+        w[..., idx_n[ok]] = src[..., :len(idx_n)][..., ok]
+        return w.reshape(-1)
+    add("columns_by_index_masked", "columns_by_index_masked",
+        {"src": P, "dst": P, "idx": I, "n_idx": "i32", "m": "i32", "n": "i32", "pitch_m": "i32", "pitch_n": "i32", "M": "constexpr", "IN": "constexpr"},
+        {"M": 8, "IN": 16}, (1,), lambda: [xin.reshape(-1).copy(), np.full(m * n, -1, np.float32), idx_n.copy(), len(idx_n), m, n, n, 1],
+        lambda a: _eq(a[1], want_columns(xin)))
+
+    def want_rows_3d():
+        w = np.full((b3, 3, n), -2, dtype=np.float32)
+        ok = idx[idx < m]
+        w[:, :len(ok), :] = x3[:, ok, :]
+        return w.reshape(-1)
+    add("rows_by_index_masked_3d", "rows_by_index_masked_3d",
+        dict([("src", P), ("dst", P), ("idx", I)] + [(k, "i32") for k in "n_idx b m n s_b s_m s_n d_b d_m d_n".split()] + [(k, "constexpr") for k in ("B", "IM", "N")]),
+        {"B": 4, "IM": 4, "N": 16}, (1,),
+        lambda: [x3.reshape(-1).copy(), np.full(b3 * 3 * n, -1, np.float32), idx.copy(), 3, b3, m, n, m * n, n, 1, 3 * n, n, 1], lambda a: _eq(a[1], want_rows_3d()))
+    add("columns_by_index_masked_3d", "columns_by_index_masked_3d",
+        dict([("src", P), ("dst", P), ("idx", I)] + [(k, "i32") for k in "n_idx b m n s_b s_m s_n".split()] + [(k, "constexpr") for k in ("B", "M", "IN")]),
+        {"B": 4, "M": 8, "IN": 16}, (1,),
+        lambda: [x3.reshape(-1).copy(), np.full(x3.size, -1, np.float32), idx_n.copy(), len(idx_n), b3, m, n, m * n, n, 1], lambda a: _eq(a[1], want_columns(x3)))
+    xp = np.arange(2, 2 + 3 * m * n, dtype=np.float32).reshape(3, m, n)
+
+    def want_above_pid():
+        w = np.full_like(xp, -1)
+        for pid in range(3):
+            t = np.full((m, n), -2, np.float32)
+            t[np.arange(m) > pid, :] = xp[pid][np.arange(m) > pid, :]
+            w[pid][:, np.arange(n) > pid] = t[:, np.arange(n) > pid]
+        return w.reshape(-1)
+    add("masks_above_program_id", "masks_above_program_id",
+        dict([("src", P), ("dst", P)] + [(k, "i32") for k in "m n s_pid s_m s_n".split()] + [("M", "constexpr"), ("N", "constexpr")]), {"M": 8, "N": 16}, (3,),
+        lambda: [xp.reshape(-1).copy(), np.full(xp.size, -1, np.float32), m, n, m * n, n, 1], lambda a: _eq(a[1], want_above_pid()))
     # test_einsum_qhmd_hmpd_to_qhmp.py:150-165
     Q, H, Mm, D, Pp = 1, 2, 2, 2, 4
     rng = np.random.default_rng(4)

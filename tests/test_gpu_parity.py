@@ -793,6 +793,46 @@ def test_reference_functional_case(name):
     case["check"]([d.cpu().numpy() for d in dev if isinstance(d, torch.Tensor)])
 
 
+def test_tile_program_blocks_past_the_register_budget():
+    """Reductions of blocks too large to stage (one thread per line, in index order), in-place blocks of more than 16384
+    elements (still two phases: every load before any store), a tile product with 32768 outputs."""
+    import core_kernels
+    import extra_kernels as X
+    rng = np.random.default_rng(21)
+    x = rng.integers(-8, 9, (512, 256)).astype(np.float32)           # small integers: every order of summation is exact
+    for axis in (0, 1):
+        for kind, want in ((0, x.sum(axis)), (1, x.max(axis))):
+            out = torch.zeros(x.shape[1 - axis], device=DEV)
+            k = X.reduce_big_block_2d[(1,)](torch.from_numpy(x).to(DEV), out, R=512, C=256, AXIS=axis, KIND=kind)
+            torch.cuda.synchronize()
+            assert k.function.family == "tile_program"
+            assert np.array_equal(out.cpu().numpy(), want), (axis, kind)
+    xi = rng.integers(-1000, 1000, 50000).astype(np.int32)
+    out = torch.zeros(3, dtype=torch.int32, device=DEV)
+    X.block_total_and_extremes[(1,)](torch.from_numpy(xi).to(DEV), out, 50000, BLOCK=65536)
+    torch.cuda.synchronize()
+    assert out.cpu().tolist() == [int(xi.sum()), max(int(xi.max()), 0), min(int(xi.min()), 0)]
+    x3 = rng.integers(-8, 9, (8, 16, 32)).astype(np.float32)
+    for axis in (0, 1, 2):
+        for kind, want in ((0, x3.sum(axis)), (1, x3.max(axis))):
+            out = torch.zeros(want.size, device=DEV)
+            X.reduce_3d[(1,)](torch.from_numpy(x3).to(DEV), out, A=8, B=16, C=32, AXIS=axis, KIND=kind)
+            torch.cuda.synchronize()
+            assert np.array_equal(out.cpu().numpy().reshape(want.shape), want), (axis, kind)
+    for R, C in ((64, 128), (256, 128), (512, 128)):                 # 8192 (registers), 32768 and 65536 (two phases all the same)
+        v = rng.standard_normal(R * C + 1).astype(np.float32)
+        d = torch.from_numpy(v).to(DEV)
+        X.shift_left_in_place[(1,)](d, R=R, C=C)
+        torch.cuda.synchronize()
+        assert np.array_equal(d.cpu().numpy(), np.concatenate([v[1:], v[-1:]])), (R, C)
+    a = rng.integers(-3, 4, (128, 64)).astype(np.float16)
+    b = rng.integers(-3, 4, (64, 256)).astype(np.float16)
+    c = torch.zeros(128 * 256, device=DEV)
+    core_kernels.dot_in_half_precision[(1,)](torch.from_numpy(a).to(DEV), torch.from_numpy(b).to(DEV), c, M=128, N=256, K=64, ACC_IN=0)
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy().reshape(128, 256), a.astype(np.float32) @ b.astype(np.float32))
+
+
 def _core_case_ids():
     import core_cases
     return [c["name"] for c in core_cases.cases()]

@@ -340,6 +340,9 @@ def test_reductions_and_scans_lower_to_the_generic_family(native):
     s = native.ttir_to_structured(compile_ttir(X.reduce_rows_2d, sig, {"BR": 8, "BC": 128, "KIND": 0}))
     assert "reduce " in s and "axis=1" in s
     assert native.PlanHandle(native.structured_to_plan(s)[0]).family == "tile_program"
-    # a block too large for the staged reduction is refused with the reason
-    with pytest.raises(NotImplementedError, match="more than 16384 elements"):
-        native.structured_to_plan(native.ttir_to_structured(compile_ttir(X.reduce_rows_2d, sig, {"BR": 256, "BC": 128, "KIND": 0})))
+    # a block too large to stage is reduced by one thread per line; a scan of that size is refused with the reason
+    big = native.structured_to_plan(native.ttir_to_structured(compile_ttir(X.reduce_rows_2d, sig, {"BR": 256, "BC": 128, "KIND": 0})))
+    assert native.PlanHandle(big[0]).family == "tile_program"
+    sig = {"x_ptr": P, "y_ptr": P, "n": "i32", "BLOCK": "constexpr"}
+    with pytest.raises(NotImplementedError, match="a scan over a block of more than 16384 elements"):
+        native.structured_to_plan(native.ttir_to_structured(compile_ttir(X.running_sum, sig, {"BLOCK": 32768})))

@@ -41,6 +41,7 @@ namespace tts {
 
 namespace {
 
+constexpr int64_t HAZARD_MAX = 65536;     // elements; the limit for blocks that must run in two phases
 constexpr int64_t TWO_PHASE_MAX = 16384;  // elements; 64 registers per thread and held block value
 
 struct Gen {
@@ -608,8 +609,9 @@ struct Gen {
       }
       if (s.kind == SK::Reduce || s.kind == SK::Scan) {
         const std::vector<int64_t> shape = val(s.operands.at(0)).shape;
-        if (shape.empty() || shape.size() > 2) no("a reduction over a block of rank " + std::to_string(shape.size()));
-        if (count(shape) > TWO_PHASE_MAX) no("a reduction or scan over a block of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
+        if (shape.empty() || shape.size() > 4) no("a reduction over a block of rank " + std::to_string(shape.size()));
+        if (s.kind == SK::Scan && shape.size() > 2) no("a scan over a block of rank " + std::to_string(shape.size()));
+        if (s.kind == SK::Scan && count(shape) > TWO_PHASE_MAX) no("a scan over a block of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
         reduce(s, shape);
         k++;
         continue;
@@ -642,12 +644,21 @@ struct Gen {
         }
       if (!have) { k = end; continue; }  // only elementwise ops: they are written out where their results are used
       auto own = [&](const SOp &o) { return o.kind == SK::Load && o.acc.sizes == shape; };
-      const bool two_phase_run = count(shape) <= TWO_PHASE_MAX;
+      // a larger block that is stored to an argument it is also loaded from still runs in two phases, whatever that
+      // costs in registers (up to 256 values per thread, spilled if need be): the order of its memory effects is kept
+      bool hazard = false;
+      {
+        std::set<int> load_bases;
+        for (size_t q = k; q < end; q++)
+          if (ops[q].kind == SK::Load) load_bases.insert(ops[q].acc.base_arg);
+        for (size_t q = k; q < end; q++) hazard = hazard || (ops[q].kind == SK::Store && load_bases.count(ops[q].acc.base_arg));
+      }
+      const bool two_phase_run = count(shape) <= (hazard ? HAZARD_MAX : TWO_PHASE_MAX);
       auto big_other = [&](const SOp &o) {
         return two_phase_run && o.kind == SK::Load && o.acc.sizes != shape && count(o.acc.sizes) >= 2048 && count(o.acc.sizes) <= TWO_PHASE_MAX;
       };
       const int64_t T = count(shape);
-      const bool two_phase = T <= TWO_PHASE_MAX;
+      const bool two_phase = two_phase_run;
       const std::string i0 = idx0(shape), i1 = idx1(shape);
       auto emit_load = [&](const SOp &o, const std::string &target) {
         std::string pred, addr = address(o.acc, i0, i1, pred);
@@ -739,13 +750,19 @@ struct Gen {
           if (ops[q].kind == SK::Load) load_bases.insert(ops[q].acc.base_arg);
         for (size_t q = k; q < end; q++)
           if (ops[q].kind == SK::Store && load_bases.count(ops[q].acc.base_arg))
-            no("a block of more than " + std::to_string(TWO_PHASE_MAX) + " elements is stored to an argument that is loaded next to the store");
+            no("a block of more than " + std::to_string(HAZARD_MAX) + " elements is stored to an argument that is loaded next to the store");
         if (stores) {
-          os << pad() << "for (int t = threadIdx.x; t < " << T << "; t += 256) {\n";
-          indent++;
-          map_vars({-1});
-          cur_i0 = i0;
-          cur_i1 = i1;
+          bool reads_held = false;  // a value of this shape that threads keep in registers (the result of a matrix product)
+          for (auto &h : held) reads_held = reads_held || h.second.shape == shape;
+          if (reads_held) {
+            open_element_loop(shape);
+          } else {
+            os << pad() << "for (int t = threadIdx.x; t < " << T << "; t += 256) {\n";
+            indent++;
+            map_vars({-1});
+            cur_i0 = i0;
+            cur_i1 = i1;
+          }
           for (size_t q = k; q < end; q++)
             if (own(ops[q])) {
               std::string name = "v" + std::to_string(ops[q].result);
@@ -854,7 +871,7 @@ struct Gen {
         R.shape[1] != B.shape[1])
       no("a matrix product whose operands are not [M, K] x [K, N]");
     const int64_t M = A.shape[0], K = A.shape[1], N = B.shape[1];
-    if (M * N > TWO_PHASE_MAX) no("a matrix product with more than " + std::to_string(TWO_PHASE_MAX) + " outputs outside the tiled matmul kernels");
+    if (M * N > 2 * TWO_PHASE_MAX) no("a matrix product with more than " + std::to_string(2 * TWO_PHASE_MAX) + " outputs outside the tiled matmul kernels");
     // operands of a 16-bit type are staged in that type (their values are exactly representable), others as fp32
     auto narrow = [](const std::string &t) { return t == "f16" || t == "bf16"; };
     const size_t a_size = narrow(A.dtype) ? 2 : 4, b_size = narrow(B.dtype) ? 2 : 4;
@@ -1017,6 +1034,58 @@ struct Gen {
     const int rank = (int)shape.size();
     if (s.axis < 0 || s.axis >= rank) no("a reduction axis outside the block's rank");
     const int64_t T = count(shape), L = shape[s.axis], O = T / L;
+    const bool big = T > TWO_PHASE_MAX;  // nothing of this shape is held in registers: loops need not be unrolled
+    const std::string unroll = big ? std::string() : "#pragma unroll\n" + pad();
+    const bool lines_of_256 = !scan && L % 256 == 0 && (rank == 1 || (rank == 2 && s.axis == 1));
+    // Blocks too large to stage, and blocks of rank above 2: one thread per line.  It walks its line in index order (the
+    // order of the reference's sequential loop) and reads every element from its definition, so the operands must be
+    // computable in place (loads read where they are used); neighbouring threads read neighbouring lines.
+    if (!scan && !lines_of_256 && (big || rank > 2)) {
+      const std::string fname = "comb" + id;
+      combiner(s, fname);
+      std::vector<int64_t> rshape = shape;
+      rshape.erase(rshape.begin() + s.axis);
+      Idx full = split_index(rshape, rshape.size() >= 2 ? "(o / " + std::to_string(rshape.back()) + ")" : "o",
+                             rshape.size() >= 2 ? "(o % " + std::to_string(rshape.back()) + ")" : "0");
+      full.insert(full.begin() + s.axis, "l");
+      const auto ij = join_index(shape, full);
+      std::vector<std::string> Tn(k);
+      for (size_t j = 0; j < k; j++) {
+        Tn[j] = ctype(val(s.operands[j]).dtype);
+        const size_t sz = held_bytes(val(s.operands[j]).dtype);
+        decl << "  __shared__ " << Tn[j] << " out" << id << "_" << j << "[" << O << "];\n";
+        out_bytes += (O * sz + 15) / 16 * 16;
+      }
+      if (out_bytes + pool_bytes > 60 * 1024) no("a reduction whose results need more than 60 KB of LDS");
+      auto list = [&](const std::string &pre) {
+        std::string r;
+        for (size_t j = 0; j < k; j++) r += (j ? ", " : "") + pre + std::to_string(j);
+        return r;
+      };
+      map_vars({-1});
+      cur_i0.clear();
+      cur_i1.clear();
+      os << pad() << "__syncthreads();\n";
+      os << pad() << "for (int o = threadIdx.x; o < " << O << "; o += 256) {\n";
+      indent++;
+      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << ";\n";
+      os << pad() << "for (int l = 0; l < " << L << "; l++) {\n";
+      indent++;
+      for (size_t j = 0; j < k; j++) os << pad() << "const " << Tn[j] << " el" << j << " = " << at(s.operands[j], ij.first, ij.second) << ";\n";
+      os << pad() << "if (l == 0) { ";
+      for (size_t j = 0; j < k; j++) os << "acc" << j << " = el" << j << "; ";
+      os << "} else " << fname << "(" << list("acc") << ", " << list("el") << ", " << list("acc") << ");\n";
+      indent--;
+      os << pad() << "}\n";
+      for (size_t j = 0; j < k; j++) {
+        const std::string &dt = val(s.operands[j]).dtype;
+        os << pad() << "out" << id << "_" << j << "[o] = " << (s.body.empty() && s.name == "arith.addf" ? rounded(dt, "acc" + std::to_string(j)) : "acc" + std::to_string(j)) << ";\n";
+      }
+      indent--;
+      os << pad() << "}\n" << pad() << "__syncthreads();\n";
+      return;
+    }
+    if (big && !lines_of_256) no("a scan over a block of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
     const int64_t OS = rank == 1 ? 0 : s.axis == 1 ? shape[1] : 1, LS = rank == 1 ? 1 : s.axis == 1 ? 1 : shape[1];
     int64_t SEG = 1;
     while (SEG * 2 * O <= 256 && (SEG * 2) * (SEG * 2) <= 2 * L) SEG *= 2;  // about sqrt(L) pieces: L / SEG + SEG steps
@@ -1026,7 +1095,7 @@ struct Gen {
     // Lines along the contiguous dimension whose length is a multiple of the workgroup size: every thread owns
     // L / 256 elements of each line.  It folds those in registers, the wavefront folds its 64 partials with a butterfly
     // of lane exchanges, and one LDS round trip folds the four wavefronts: no staging of the block.
-    if (!scan && L % 256 == 0 && (rank == 1 || s.axis == 1)) {
+    if (lines_of_256) {
       std::vector<std::string> Tn(k);
       size_t off = 0;
       os << pad() << "__syncthreads();\n";
@@ -1052,10 +1121,10 @@ struct Gen {
       map_vars(shape);
       cur_i0 = i0;
       cur_i1 = i1;
-      os << pad() << "#pragma unroll\n" << pad() << "for (int o = 0; o < " << O << "; o++) {\n";
+      os << pad() << unroll << "for (int o = 0; o < " << O << "; o++) {\n";
       indent++;
       for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << ";\n";
-      os << pad() << "#pragma unroll\n" << pad() << "for (int q = 0; q < " << LQ << "; q++) {\n";
+      os << pad() << unroll << "for (int q = 0; q < " << LQ << "; q++) {\n";
       indent++;
       os << pad() << "const int n = o * " << LQ << " + q;\n" << pad() << "const int t = threadIdx.x + 256 * n;\n";
       for (size_t j = 0; j < k; j++) os << pad() << "const " << Tn[j] << " el" << j << " = " << at(s.operands[j], i0, i1) << ";\n";

@@ -230,7 +230,8 @@ static void parse_for(const std::string &rest, Op &op, Lines &L) {
       op.iter_inits.push_back(trim(pair.substr(q + 1)));
     }
     size_t arrow = rest.find("->", close);
-    size_t tcolon = rest.rfind(" : ");
+    size_t tcolon = rest.rfind(" : ");  // the induction variable's type, printed when it is not `index`
+    if (tcolon == std::string::npos || tcolon < arrow) tcolon = rest.rfind('{');
     std::string tys = trim(rest.substr(arrow + 2, tcolon - arrow - 2));
     op.result_types = parse_type_list(tys);
     if (op.result_types.size() != op.iter_names.size())
@@ -337,6 +338,13 @@ static void parse_op(Lines &L, Block &blk) {
     parse_block(L, rb);
     std::string tail = L.v[L.i++];  // }) : (types) -> types
     if (!starts_with(tail, "})")) throw Unsupported("region of " + op->name + " not closed: " + tail);
+    {  // the generic form carries the attributes here: }) {axis = 0 : i32} : (types) -> types
+      const size_t b0 = tail.find('{'), b1 = tail.find('}', 2);
+      if (b0 != std::string::npos && b1 != std::string::npos && b0 < tail.find("(", 2)) {
+        parse_attr_dict(tail.substr(b0 + 1, b1 - b0 - 1), op->attrs);
+        tail = "})" + tail.substr(b1 + 1);
+      }
+    }
     size_t col = tail.find(':');
     size_t arrow = tail.find("->");
     op->types = parse_type_list(tail.substr(col + 1, arrow - col - 1));
@@ -385,6 +393,7 @@ static void parse_op(Lines &L, Block &blk) {
   {
     std::string w;
     auto flush = [&]() {
+      if (w.size() > 2 && w.front() == '"' && w.back() == '"') w = w.substr(1, w.size() - 2);  // generic form: "oeq"
       if (!w.empty() && w[0] != '%' && w != "=") op->words.push_back(w);
       w.clear();
     };
@@ -643,12 +652,28 @@ Func parse_ttir(const std::string &text) {
   std::string clean = strip_locations(text);
   Lines L;
   {
+    // one op per entry: a line whose parentheses are still open and that does not open a region (hand-written IR breaks
+    // long signatures over several lines) is continued by the next one; `//` comments go
     std::istringstream is(clean);
-    std::string ln;
+    std::string ln, pending;
+    int depth = 0;
     while (std::getline(is, ln)) {
+      const size_t comment = ln.find("//");
+      if (comment != std::string::npos) ln = ln.substr(0, comment);
       ln = trim(ln);
-      if (!ln.empty()) L.v.push_back(ln);
+      if (ln.empty()) continue;
+      if (ln == "{" && pending.empty() && !L.v.empty()) {  // a region's brace on a line of its own
+        L.v.back() += " {";
+        continue;
+      }
+      pending = pending.empty() ? ln : pending + " " + ln;
+      depth = 0;
+      for (char ch : pending) depth += ch == '(' ? 1 : ch == ')' ? -1 : 0;
+      if (depth > 0 && pending.back() != '{') continue;
+      L.v.push_back(pending);
+      pending.clear();
     }
+    if (!pending.empty()) L.v.push_back(pending);
   }
   Func kernel;
   std::map<std::string, Callee> callees;
@@ -679,7 +704,16 @@ Func parse_ttir(const std::string &text) {
           f.arg_names.push_back(trim(a.substr(0, col)));
           f.arg_types.push_back(parse_type(ty));
         }
-      const bool has_results = line.find("->", close) != std::string::npos && line.find("->", close) < line.rfind('{');
+      bool has_results = false;
+      {
+        const size_t arrow = line.find("->", close), brace = line.rfind('{');
+        if (arrow != std::string::npos && arrow < brace) {
+          std::string res = trim(line.substr(arrow + 2, brace - arrow - 2));
+          const size_t attr = res.find("attributes");
+          if (attr != std::string::npos) res = trim(res.substr(0, attr));
+          has_results = res != "()";
+        }
+      }
       if (has_results && !is_private) throw Unsupported("tt.func with results is not a kernel");
       L.i++;
       parse_func_body(L, f.body);
