@@ -230,6 +230,12 @@ def cases():
         add(f"dot_fp16_acc{acc}", "dot_in_half_precision", {"a_ptr": H, "b_ptr": H, "c_ptr": P, "M": C, "N": C, "K": C, "ACC_IN": C}, {"M": 32, "N": 32, "K": 64, "ACC_IN": acc}, (1,),
             lambda: [ha.reshape(-1).copy(), hb.reshape(-1).copy(), hc.reshape(-1).copy()],
             lambda a, acc=acc: _eq(a[2].reshape(32, 32), ha.astype(np.float32) @ hb.astype(np.float32) + (hc if acc else 0)))
+    fx_ = rng.standard_normal(1024).astype(np.float32)
+    falt = rng.standard_normal(1024).astype(np.float32)
+    add("other_is_data", "fill_values_that_are_data", {"x_ptr": P, "alt_ptr": P, "out_ptr": P, "n": "i32", "fill": "i32", "BLOCK": C}, {"BLOCK": 256}, (4,),
+        lambda: [fx_.copy(), falt.copy(), np.zeros(2048, np.float32), 700, -7],
+        lambda a: _eq(a[2], np.concatenate([np.where(np.arange(1024) < 700, fx_, np.float32(-7)), np.where(np.arange(1024) < 700, fx_, falt)])))
+
     # tile products with the epilogues of the core dot test; small integers so that every order of summation is exact
     for dt, name in [(np.float32, "fp32"), (np.float16, "fp16"), (np.int8, "i8")]:
         M, N, K = 32, 32, 64

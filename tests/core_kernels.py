@@ -390,3 +390,14 @@ def integer_ops_any_width(x_ptr, y_ptr, out_ptr, n, BLOCK: tl.constexpr):
     tl.store(out_ptr + 10 * n + o, (x < y).to(x.dtype) + (x <= y).to(x.dtype) * 2 + (x == y).to(x.dtype) * 4, mask=m)
     tl.store(out_ptr + 11 * n + o, tl.maximum(x, y) - tl.minimum(x, y), mask=m)
     tl.store(out_ptr + 12 * n + o, tl.where(x > y, x, y), mask=m)
+
+
+@triton.jit
+def fill_values_that_are_data(x_ptr, alt_ptr, out_ptr, n, fill, BLOCK: tl.constexpr):
+    # `other` of a masked load as a kernel argument (test/Conversion/TritonToStructured/masked_ldst_sitofp_other.mlir
+    # converts an integer argument for it), then as a block loaded from elsewhere
+    o = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    a = tl.load(x_ptr + o, mask=o < n, other=fill.to(tl.float32))
+    b = tl.load(x_ptr + o, mask=o < n, other=tl.load(alt_ptr + o))
+    tl.store(out_ptr + o, a)
+    tl.store(out_ptr + tl.num_programs(0) * BLOCK + o, b)

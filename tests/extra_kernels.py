@@ -894,3 +894,32 @@ def shift_left_in_place(x_ptr, R: tl.constexpr, C: tl.constexpr):
     # every element takes its right neighbour's old value: all loads come before any store, whatever the block's size
     at = tl.arange(0, R)[:, None] * C + tl.arange(0, C)[None, :]
     tl.store(x_ptr + at, tl.load(x_ptr + at + 1))
+
+
+@triton.jit
+def grouped_rows_matmul(a_ptr, b_ptr, c_ptr, rows_ptr, expert_ptr, n_rows, K, N, s_am, s_be, s_bk, s_cm,
+                        BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr):
+    # C[i, :] = A[rows[i], :] @ B[expert of i's block] -- the shape of a mixture-of-experts layer
+    # (test/Conversion/TritonToLinalgExperimental/unstructured_ptr_used_in_loop.mlir is such a kernel): a scalar read
+    # from memory picks the weight matrix and may end the program early, the rows of A come through loaded indices,
+    # and both blocks of pointers are carried along K by the loop
+    pid_m = tl.program_id(0)
+    pid_n = tl.program_id(1)
+    expert = tl.load(expert_ptr + pid_m)
+    if expert < 0:
+        return
+    i = pid_m * BM + tl.arange(0, BM)
+    ok = i < n_rows
+    which = tl.load(rows_ptr + i, mask=ok, other=0)
+    j = pid_n * BN + tl.arange(0, BN)
+    k = tl.arange(0, BK)
+    a_ptrs = a_ptr + which[:, None] * s_am + k[None, :]
+    b_ptrs = b_ptr + expert * s_be + k[:, None] * s_bk + j[None, :]
+    acc = tl.zeros((BM, BN), tl.float32)
+    for k0 in range(0, K, BK):
+        a = tl.load(a_ptrs, mask=ok[:, None] & (k[None, :] < K - k0), other=0.0)
+        b = tl.load(b_ptrs, mask=(k[:, None] < K - k0) & (j[None, :] < N), other=0.0)
+        acc = tl.dot(a, b, acc)
+        a_ptrs += BK
+        b_ptrs += BK * s_bk
+    tl.store(c_ptr + i[:, None] * s_cm + j[None, :], acc, mask=ok[:, None] & (j[None, :] < N))

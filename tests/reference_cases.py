@@ -146,6 +146,27 @@ def cases():
     add("masks_above_program_id", "masks_above_program_id",
         dict([("src", P), ("dst", P)] + [(k, "i32") for k in "m n s_pid s_m s_n".split()] + [("M", "constexpr"), ("N", "constexpr")]), {"M": 8, "N": 16}, (3,),
         lambda: [xp.reshape(-1).copy(), np.full(xp.size, -1, np.float32), m, n, m * n, n, 1], lambda a: _eq(a[1], want_above_pid()))
+    # a mixture-of-experts product (the kernel of test/Conversion/TritonToLinalgExperimental/unstructured_ptr_used_in_loop.mlir,
+    # which has no runtime test in the reference): small integers, so every summation order gives the same bits
+    rng = np.random.default_rng(6)
+    n_tok, Kd, Nd, E = 40, 48, 24, 3
+    Am = rng.integers(-3, 4, (64, Kd)).astype(np.float32)
+    Bm = rng.integers(-3, 4, (E, Kd, Nd)).astype(np.float32)
+    rows = rng.integers(0, 64, n_tok).astype(np.int32)
+    experts = np.array([2, -1, 0], dtype=np.int32)                      # per block of 16 rows; -1: nothing to do
+
+    def want_moe():
+        w = np.full((n_tok, Nd), -1, np.float32)
+        for blk, e in enumerate(experts):
+            if e >= 0:
+                r = slice(blk * 16, min(n_tok, blk * 16 + 16))
+                w[r] = Am[rows[r]] @ Bm[e]
+        return w.reshape(-1)
+    add("grouped_rows_matmul", "grouped_rows_matmul",
+        dict([("a_ptr", P), ("b_ptr", P), ("c_ptr", P), ("rows_ptr", I), ("expert_ptr", I)] + [(k, "i32") for k in "n_rows K N s_am s_be s_bk s_cm".split()]
+             + [(k, "constexpr") for k in ("BM", "BN", "BK")]), {"BM": 16, "BN": 16, "BK": 32}, (3, 2),
+        lambda: [Am.reshape(-1).copy(), Bm.reshape(-1).copy(), np.full(n_tok * Nd, -1, np.float32), rows.copy(), experts.copy(), n_tok, Kd, Nd, Kd, Kd * Nd, Nd, Nd],
+        lambda a: _eq(a[2], want_moe()))
     # test_einsum_qhmd_hmpd_to_qhmp.py:150-165
     Q, H, Mm, D, Pp = 1, 2, 2, 2, 4
     rng = np.random.default_rng(4)

@@ -346,3 +346,67 @@ def test_reductions_and_scans_lower_to_the_generic_family(native):
     sig = {"x_ptr": P, "y_ptr": P, "n": "i32", "BLOCK": "constexpr"}
     with pytest.raises(NotImplementedError, match="a scan over a block of more than 16384 elements"):
         native.structured_to_plan(native.ttir_to_structured(compile_ttir(X.running_sum, sig, {"BLOCK": 32768})))
+
+
+# ------------------------------------------------- the reference's lit inputs, all of them
+_LIT = "/root/reference/test/Conversion"
+
+
+def _lit_functions(text):
+    """One module per public tt.func of a lit file (private functions go with every piece); comment lines dropped."""
+    lines = [l for l in text.splitlines() if not l.lstrip().startswith("//")]
+    funcs, i = [], 0
+    while i < len(lines):
+        if not lines[i].lstrip().startswith("tt.func"):
+            i += 1
+            continue
+        j, depth, seen = i, 0, False
+        while True:
+            depth += lines[j].count("{") - lines[j].count("}")
+            seen = seen or "{" in lines[j]
+            if seen and depth <= 0:
+                break
+            j += 1
+        funcs.append("\n".join(lines[i:j + 1]))
+        i = j + 1
+    private = [f for f in funcs if "private" in f.split("@")[0]]
+    return ["module {\n" + "\n".join([f] + private) + "\n}" for f in funcs if "private" not in f.split("@")[0]]
+
+
+@pytest.mark.skipif(not __import__("os").path.isdir(_LIT), reason="the reference tree is not here")
+def test_reference_lit_inputs_plan_or_are_refused_for_a_known_reason(native):
+    """Every tt.func in the reference's conversion tests (test/Conversion/*/*.mlir, hand-written IR included) goes through
+    the reader, the analyses and the planner.  What is refused is refused for one of the reasons listed here, each with
+    the number of functions it may account for; anything else, or more of the same, fails."""
+    import collections
+    import glob
+    known = {  # reason (prefix) -> functions
+        "tensor-typed kernel argument": 18,                       # blocks of pointers as arguments: no launcher can pass them
+        "operation tensor.empty": 9,                              # tensor dialect ops written by hand into triton_assert.mlir
+        "tt.func with results is not a kernel": 6,
+        "tile_program: a loop-carried block value of more than 16384 elements": 6,   # dot + separate add of an older front end, 128 x 256 accumulators
+        "unsupported type '<tensor<": 8,                          # block pointers: the front end pass list rewrites them before this stage
+        "tile_program: the reductions of this program need": 4,
+        "tile_program: elementwise op extern.some_symbol": 3,     # the reference refuses it too (unsupported_extern_elementwise.mlir)
+        "pointer-valued operation": 10,                           # int_to_ptr / bitcast / cat / select on pointers (the reference's TritonToPtr fallback)
+        "scf.if that yields pointers": 4,
+        "unsupported type 'f8E4M3FN'": 1,
+        "unsupported type '[": 3,                                 # tts / memref dialect inputs of later stages
+        "unsupported type '}'": 1,
+    }
+    planned, refused = 0, collections.Counter()
+    for path in sorted(glob.glob(_LIT + "/*/*.mlir")):
+        text = open(path).read()
+        if "tt.func" not in text:
+            continue
+        for module in _lit_functions(text):
+            try:
+                native.PlanHandle(native.structured_to_plan(native.ttir_to_structured(module))[0])
+                planned += 1
+            except NotImplementedError as e:
+                why = next((k for k in known if k in str(e)), None)
+                assert why is not None, (path, str(e)[:300])
+                refused[why] += 1
+    for why, n in refused.items():
+        assert n <= known[why], (why, n)
+    assert planned >= 330, (planned, dict(refused))

@@ -158,9 +158,22 @@ int ExprPool::cmpsel(int pred, int a, int b, int c, int d) {
   return intern(e);
 }
 
+int ExprPool::data(int value, int bits) {
+  Expr e{EK::Data, (uint8_t)bits};
+  e.a = value;
+  return intern(e);
+}
+
+bool ExprPool::has_data() const {
+  for (auto &e : nodes_)
+    if (e.k == EK::Data) return true;
+  return false;
+}
+
 int64_t ExprPool::eval(int id, const EvalEnv &env) const {
   const Expr &e = nodes_[id];
   switch (e.k) {
+    case EK::Data: throw std::runtime_error("an index expression that depends on data has no value on the host");
     case EK::Const: return e.val;
     case EK::Arg: return wrap(env.args[e.a], e.bits);
     case EK::Pid: return env.pid[e.a];
@@ -179,7 +192,7 @@ bool ExprPool::depends_on(int id, EK kind, int a) const {
   const Expr &e = nodes_[id];
   if (e.k == kind && (a < 0 || e.a == a)) return true;
   switch (e.k) {
-    case EK::Const: case EK::Arg: case EK::Pid: case EK::NProg: case EK::IV: case EK::Iter: case EK::Result:
+    case EK::Const: case EK::Arg: case EK::Pid: case EK::NProg: case EK::IV: case EK::Iter: case EK::Result: case EK::Data:
       return false;
     case EK::Sext: case EK::Trunc: return depends_on(e.a, kind, a);
     case EK::CmpSel:
@@ -201,6 +214,7 @@ std::string ExprPool::str(int id) const {
     case EK::IV: return "iv" + std::to_string(e.a);
     case EK::Iter: return "it" + std::to_string(e.a) + "." + std::to_string(e.b);
     case EK::Result: return "res" + std::to_string(e.a) + "." + std::to_string(e.b);
+    case EK::Data: return "value" + std::to_string(e.a);
     case EK::Add: return two("+");
     case EK::Sub: return two("-");
     case EK::Mul: return two("*");

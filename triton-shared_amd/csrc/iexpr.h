@@ -27,6 +27,8 @@ enum class EK : uint8_t {
   Sext,    // i32 -> index
   Trunc,   // index/i64 -> i32
   CmpSel,  // (a pred b) ? c : d ; pred in val: 0 slt, 1 sle, 2 sgt, 3 sge, 4 eq, 5 ne
+  Data,    // a = id of a scalar integer value the program computes from memory (a loaded offset, a reduced count):
+           // known only on the device, so no host-side evaluation of an expression that holds one
 };
 
 struct Expr {
@@ -58,6 +60,8 @@ class ExprPool {
   int sext(int a);
   int trunc(int a);
   int cmpsel(int pred, int a, int b, int c, int d);
+  int data(int value, int bits);
+  bool has_data() const;  // any Data leaf in the pool
   // index-typed helpers (operands are widened when needed)
   int to_index(int a) { return at(a).bits == 64 ? a : sext(a); }
   int add_index(int a, int b) { return bin(EK::Add, to_index(a), to_index(b)); }

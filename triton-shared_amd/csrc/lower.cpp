@@ -119,6 +119,9 @@ class Lowerer {
   std::map<std::string, int> int_memo_;       // scalar integer SSA name -> expr
   int in_region_ = 0;                         // inside a combiner region: scalar integers are data, not index expressions
   std::map<std::string, PtrState> known_ptr_; // loop-carried / loop-result pointer states
+  // an unstructured address: base pointer + scalar offset + a block of per-element integer offsets
+  struct Scattered { int base = -1, scalar = -1, value = -1; };
+  std::map<std::string, Scattered> carried_scatter_;  // loop-carried / loop-result blocks of pointers that are gathers
   std::map<std::string, int> data_;           // SSA name -> value id
   std::vector<SOp> *cur_ = nullptr;
 
@@ -202,7 +205,24 @@ class Lowerer {
       } else if (op.name == "arith.andi" && d.type.elem == "i1") {
         e = P.pool.bin(EK::Mul, opnd(0), opnd(1));
       } else {
-        throw Unsupported("scalar integer op " + op.name + " (line " + std::to_string(op.line) + ")");
+        // a value read from memory, reduced, yielded by a branch, or computed from one by an op the expressions do not
+        // know: a leaf that names the data value (the device knows it, the host does not)
+        int v = -1;
+        auto dit = data_.find(name);
+        if (dit != data_.end()) {
+          v = dit->second;
+        } else if (is_elementwise(op.name) && !in_region_) {
+          SOp s;
+          s.kind = SK::Map;
+          s.name = map_name(op);
+          for (auto &o : op.operands) s.operands.push_back(data_of(o));
+          s.result = new_value(d.type);
+          cur_->push_back(s);
+          data_[name] = v = s.result;
+        } else {
+          throw Unsupported("scalar integer op " + op.name + " (line " + std::to_string(op.line) + ")");
+        }
+        e = P.pool.data(v, bits);
       }
     }
     int_memo_[name] = e;
@@ -538,11 +558,17 @@ class Lowerer {
     return a;
   }
 
-  void scalar_other(const std::string &name, Access &a) {  // TritonStructuredOps.cpp:38-98
+  void scalar_other(const std::string &name, SOp &s) {  // TritonStructuredOps.cpp:38-98
+    Access &a = s.acc;
     const Def &d = def(name);
     const Op *op = d.op;
     if (op && op->name == "tt.splat") op = def(op->operands[0]).op;
-    if (!op || op->name != "arith.constant") throw Unsupported("masked load whose `other` is not a constant");
+    if (!op || op->name != "arith.constant") {  // a value computed by the program: read as data where the mask is false
+      a.has_other = true;
+      a.other_value = data_of(name);
+      s.operands.push_back(a.other_value);
+      return;
+    }
     std::string lit = op->literal;
     if (lit.rfind("dense<", 0) == 0) lit = lit.substr(6, lit.size() - 7);
     a.has_other = true;
@@ -551,7 +577,6 @@ class Lowerer {
   }
 
   // ---- unstructured addresses: base pointer + scalar offset + a tile of per-element integer offsets
-  struct Scattered { int base = -1, scalar = -1, value = -1; };
   int widen_to_i64(int v) {
     if (P.values[v].dtype == "i64") return v;
     SOp s;
@@ -576,7 +601,11 @@ class Lowerer {
       u.scalar = st.scalar >= 0 ? st.scalar : c64(0);
       return u;
     }
-    if (!d.op) throw Unsupported("a tensor of pointers carried around a loop is not a structured access");
+    {
+      auto it = carried_scatter_.find(name);
+      if (it != carried_scatter_.end()) return it->second;
+    }
+    if (!d.op || d.op->name == "scf.for") throw Unsupported("a tensor of pointers carried around a loop is not a structured access");
     const Op &op = *d.op;
     if (op.name == "tt.splat") return scattered(op.operands[0]);
     if (op.name == "tt.broadcast" || op.name == "tt.expand_dims") {
@@ -623,6 +652,35 @@ class Lowerer {
     }
     throw Unsupported("address computed by " + op.name + " (line " + std::to_string(op.line) + ")");
   }
+  // the per-element offsets of an unstructured address as one block of 64-bit integers, its scalar part added in
+  int offsets_block(const Scattered &u, const std::vector<int64_t> &shape) {
+    int v = u.value >= 0 ? widen_to_i64(u.value) : -1;
+    int64_t c = 0;
+    if (v >= 0 && P.pool.is_const(u.scalar, &c) && c == 0) return v;
+    Type st;
+    st.elem = "i64";
+    SOp f;
+    f.kind = SK::FromIndex;
+    f.expr = P.pool.to_index(u.scalar);
+    f.result = new_value(st);
+    cur_->push_back(f);
+    Type bt = st;
+    bt.is_tensor = true;
+    bt.shape = shape;
+    SOp sp;
+    sp.kind = SK::Splat;
+    sp.operands = {f.result};
+    sp.result = new_value(bt);
+    cur_->push_back(sp);
+    if (v < 0) return sp.result;
+    SOp a;
+    a.kind = SK::Map;
+    a.name = "arith.addi";
+    a.operands = {v, sp.result};
+    a.result = new_value(bt);
+    cur_->push_back(a);
+    return a.result;
+  }
   // the access of a load / store whose pointer PtrAnalysis or whose mask MaskAnalysis cannot describe
   void scattered_access(const Op &op, size_t mask_operand, const Type &elem_type, SOp &s) {
     Scattered u = scattered(op.operands[0]);
@@ -662,7 +720,7 @@ class Lowerer {
       if (!structured) {
         s.kind = SK::Load;
         scattered_access(op, 1, rt, s);
-        if (op.operands.size() >= 3) scalar_other(op.operands[2], s.acc);
+        if (op.operands.size() >= 3) scalar_other(op.operands[2], s);
         s.result = new_value(rt);
         data_[op.results[0]] = s.result;
         cur_->push_back(s);
@@ -677,7 +735,7 @@ class Lowerer {
       if (op.operands.size() > 1) {  // a scalar condition: the value is `other` (or zero) when it is false
         s.acc.mask_value = data_of(op.operands[1]);
         s.operands.push_back(s.acc.mask_value);
-        if (op.operands.size() >= 3) scalar_other(op.operands[2], s.acc);
+        if (op.operands.size() >= 3) scalar_other(op.operands[2], s);
       }
     } else {
       s.kind = SK::Load;
@@ -686,7 +744,7 @@ class Lowerer {
         if (m.rank() != st.rank()) throw Unsupported("mask rank differs from pointer rank");
         s.acc.dims = m.dims;
       }
-      if (op.operands.size() >= 3) scalar_other(op.operands[2], s.acc);
+      if (op.operands.size() >= 3) scalar_other(op.operands[2], s);
     }
     s.result = new_value(rt);
     data_[op.results[0]] = s.result;
@@ -776,7 +834,7 @@ class Lowerer {
       defs_[op.iv] = d;
       int_memo_[op.iv] = P.pool.iv(s.loop, iv_bits);
     }
-    struct Carried { int kind; PtrState st; size_t first_slot; int tile_index; };  // 0 ptr, 1 int, 2 tile
+    struct Carried { int kind; PtrState st; size_t first_slot; int tile_index; int base; };  // 0 ptr, 1 int, 2 tile, 3 gathered ptrs
     std::vector<Carried> carried;
     for (size_t j = 0; j < op.iter_names.size(); j++) {
       const Type &t = op.result_types[j];
@@ -784,9 +842,37 @@ class Lowerer {
       d.type = t;
       defs_[op.iter_names[j]] = d;
       Carried c{};
+      bool gathered = false;
+      PtrState init;
       if (t.ptr) {
+        try {
+          init = visit(op.iter_inits[j]);
+        } catch (const Unsupported &) {
+          if (!t.is_tensor) throw;
+          gathered = true;
+        }
+      }
+      if (gathered) {
+        // a block of pointers that PtrAnalysis cannot describe (rows picked by loaded indices, walked along K): carried
+        // as its base argument and a block of 64-bit element offsets
+        Scattered u = scattered(op.iter_inits[j]);
+        c.kind = 3;
+        c.base = u.base;
+        c.tile_index = (int)s.tile_args.size();
+        s.tile_inits.push_back(offsets_block(u, t.shape));
+        Type ot;
+        ot.is_tensor = true;
+        ot.shape = t.shape;
+        ot.elem = "i64";
+        int v = new_value(ot);
+        s.tile_args.push_back(v);
+        Scattered inside;
+        inside.base = u.base;
+        inside.scalar = c64(0);
+        inside.value = v;
+        carried_scatter_[op.iter_names[j]] = inside;
+      } else if (t.ptr) {
         c.kind = 0;
-        PtrState init = visit(op.iter_inits[j]);
         c.first_slot = s.int_iters.size();
         PtrState inside = init;
         auto carry = [&](int init_expr) {
@@ -861,6 +947,10 @@ class Lowerer {
           }
         } else if (c.kind == 1) {
           s.int_iters[c.first_slot].next = int_of(y);
+        } else if (c.kind == 3) {
+          Scattered ny = scattered(y);
+          if (ny.base != c.base) throw Unsupported("loop-carried pointer changes its base");
+          s.tile_yields[c.tile_index] = offsets_block(ny, op.result_types[j].shape);
         } else {
           s.tile_yields[c.tile_index] = data_of(y);
         }
@@ -889,6 +979,17 @@ class Lowerer {
         known_ptr_[rname] = after;
       } else if (c.kind == 1) {
         int_memo_[rname] = s.int_iters[c.first_slot].result_expr;
+      } else if (c.kind == 3) {
+        Type ot = d.type;
+        ot.ptr = false;
+        ot.elem = "i64";
+        int v = new_value(ot);
+        s.results[c.tile_index] = v;
+        Scattered after;
+        after.base = c.base;
+        after.scalar = c64(0);
+        after.value = v;
+        carried_scatter_[rname] = after;
       } else {
         int v = new_value(d.type);
         s.results[c.tile_index] = v;
@@ -982,6 +1083,9 @@ class Lowerer {
         d.index = (int)i;
         d.type = i < op.result_types.size() ? op.result_types[i] : result_type(op);
         defs_[op.results[i]] = d;
+        // sibling regions may use one SSA name for different values: nothing remembered under it survives a new definition
+        int_memo_.erase(op.results[i]);
+        data_.erase(op.results[i]);
       }
     const std::string &n = op.name;
     if (n == "tt.return" || n == "tt.assert") return;  // assertions are dropped, as the reference does (triton_assert.mlir)
@@ -1121,6 +1225,8 @@ class Lowerer {
   // ------------------------------------------------------------------ DCE
   void dce() {
     std::vector<char> live(P.values.size(), 0);
+    for (int e = 0; e < P.pool.size(); e++)  // what an index expression reads stays
+      if (P.pool.at(e).k == EK::Data) live[P.pool.at(e).a] = 1;
     bool changed = true;
     std::function<bool(std::vector<SOp> &)> mark = [&](std::vector<SOp> &ops) {
       bool any_effect = false;
@@ -1192,7 +1298,7 @@ class Lowerer {
         seen[e] = 1;
         const Expr &x = P.pool.at(e);
         switch (x.k) {
-          case EK::Const: case EK::Arg: case EK::Pid: case EK::NProg: case EK::IV: case EK::Iter: return;
+          case EK::Const: case EK::Arg: case EK::Pid: case EK::NProg: case EK::IV: case EK::Iter: case EK::Data: return;
           case EK::Result:
             if (need_loop.insert(x.a).second) grew = true;
             return;

@@ -835,14 +835,14 @@ Plan make_plan(Program &&p) {
     pl.family = Family::TileProgram;
     return pl;
   }
-  bool unstructured = false;
+  bool unstructured = pl.prog.pool.has_data();  // addresses that depend on loaded values: nothing the host could check or bind
   {
     Matcher m(pl.prog);
-    for (SOp *a : m.accesses) unstructured = unstructured || a->acc.gather >= 0;
+    for (SOp *a : m.accesses) unstructured = unstructured || a->acc.gather >= 0 || a->acc.other_value >= 0 || a->acc.mask_value >= 0;
   }
   if (unstructured) {
     if (try_tile_program(pl)) return pl;
-    throw Unsupported("a program with gathers or scatters that also reduces or multiplies matrices; signature: " + pl.signature);
+    throw Unsupported("a program with gathers, scatters or masks and fill values that are data is outside the hand-written families; signature: " + pl.signature);
   }
   if (try_map1d(pl) || try_softmax(pl) || try_layernorm(pl)) return pl;
   std::string gemm_refusal;

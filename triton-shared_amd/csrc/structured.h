@@ -67,6 +67,7 @@ struct Access {          // the tts.make_tptr + mask part of a load/store
   bool has_other = false;
   double other_f = 0;                // value of `other` when the element type is a float
   int64_t other_i = 0;               // ... when it is an integer
+  int other_value = -1;              // value id (a scalar, or a block of the access's shape) when `other` is not a constant
 };
 
 struct IntIter {         // loop-carried integer (offset or stride of a carried pointer, or an i32)

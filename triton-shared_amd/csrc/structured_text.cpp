@@ -77,7 +77,7 @@ std::string print_program(const Program &p) {
     need[e] = 1;
     const Expr &x = p.pool.at(e);
     switch (x.k) {
-      case EK::Const: case EK::Arg: case EK::Pid: case EK::NProg: case EK::IV: case EK::Iter: case EK::Result: break;
+      case EK::Const: case EK::Arg: case EK::Pid: case EK::NProg: case EK::IV: case EK::Iter: case EK::Result: case EK::Data: break;
       case EK::Sext: case EK::Trunc: reach(x.a); break;
       case EK::CmpSel: reach(x.a); reach(x.b); reach(x.c); reach(x.d); break;
       default: reach(x.a); reach(x.b);
@@ -147,6 +147,7 @@ std::string print_program(const Program &p) {
           if (s.acc.gather >= 0) os << " gather=" << s.acc.gather;
           if (s.acc.gather >= 0 || s.acc.mask_value >= 0) os << " maskv=" << s.acc.mask_value;
           if (s.acc.has_other) os << " other_f=" << dbl_bits(s.acc.other_f) << " other_i=" << s.acc.other_i;
+          if (s.acc.other_value >= 0) os << " otherv=" << s.acc.other_value;
           os << " ; " << p.arg_names[s.acc.base_arg] << " offsets=" << exprs(s.acc.offsets)
              << " strides=" << exprs(s.acc.strides);
           if (!s.acc.dims.empty()) os << " dims=" << exprs(s.acc.dims);
@@ -285,7 +286,7 @@ Program read_program(const std::string &text) {
         x.k = (EK)k;
         x.bits = (uint8_t)bits;
         switch (x.k) {
-          case EK::Const: case EK::Arg: case EK::Pid: case EK::NProg: case EK::IV: case EK::Iter: case EK::Result: break;
+          case EK::Const: case EK::Arg: case EK::Pid: case EK::NProg: case EK::IV: case EK::Iter: case EK::Result: case EK::Data: break;
           case EK::Sext: case EK::Trunc: x.a = E(x.a); break;
           case EK::CmpSel: x.a = E(x.a); x.b = E(x.b); x.c = E(x.c); x.d = E(x.d); break;
           default: x.a = E(x.a); x.b = E(x.b);
@@ -368,6 +369,7 @@ Program read_program(const std::string &text) {
       if (f.has("mods")) s.acc.mods = Es(f.get("mods"));
       if (f.has("gather")) s.acc.gather = std::stoi(f.get("gather"));
       if (f.has("maskv")) s.acc.mask_value = std::stoi(f.get("maskv"));
+      if (f.has("otherv")) s.acc.other_value = std::stoi(f.get("otherv"));
       if (f.has("other_f")) {
         s.acc.has_other = true;
         s.acc.other_f = bits_dbl(f.get("other_f"));

@@ -94,6 +94,7 @@ struct Gen {
       case EK::IV: return "iv" + std::to_string(e.a);
       case EK::Iter: return "it" + std::to_string(e.a) + "_" + std::to_string(e.b);
       case EK::Result: return "res" + std::to_string(e.a) + "_" + std::to_string(e.b);
+      case EK::Data: return w("(long long)" + at(e.a, "0", "0"));
       case EK::Add: return u("+");
       case EK::Sub: return u("-");
       case EK::Mul: return u("*");
@@ -231,7 +232,7 @@ struct Gen {
         all_inline_bases.insert(s.acc.base_arg);
         std::string pred, addr = address(s.acc, i0, i1, pred);
         const std::string rd = mem_read(s.acc, addr);
-        return "(" + (pred.empty() ? rd : "(" + pred + ") ? " + rd + " : " + other_of(s.acc)) + ")";
+        return "(" + (pred.empty() ? rd : "(" + pred + ") ? " + rd + " : " + other_of(s.acc, i0, i1)) + ")";
       }
       case SK::ScalarLoad: no("internal: scalar load without a variable");
       case SK::Reduce: case SK::Scan: {
@@ -458,7 +459,8 @@ struct Gen {
     if (a.elem == "bf16") return "up_bf16(" + ptr + ")";
     return ptr;
   }
-  std::string other_of(const Access &a) {
+  std::string other_of(const Access &a, const std::string &i0 = "0", const std::string &i1 = "0") {
+    if (a.other_value >= 0) return at(a.other_value, i0, i1);
     if (!a.has_other) return a.elem == "f64" ? "0.0" : is_float(a.elem) ? "0.f" : "(" + ctype(a.elem) + ")0";
     if (a.elem == "f64") {
       if (a.other_f != a.other_f) return "__builtin_nan(\"\")";
@@ -662,7 +664,7 @@ struct Gen {
       const std::string i0 = idx0(shape), i1 = idx1(shape);
       auto emit_load = [&](const SOp &o, const std::string &target) {
         std::string pred, addr = address(o.acc, i0, i1, pred);
-        os << pad() << target << " = " << (pred.empty() ? mem_read(o.acc, addr) : "(" + pred + ") ? " + mem_read(o.acc, addr) + " : " + other_of(o.acc))
+        os << pad() << target << " = " << (pred.empty() ? mem_read(o.acc, addr) : "(" + pred + ") ? " + mem_read(o.acc, addr) + " : " + other_of(o.acc, i0, i1))
            << ";\n";
       };
       // Loads of another shape are small blocks used through broadcasts (an index vector, a row of scales).  Read in
@@ -679,7 +681,8 @@ struct Gen {
         open_element_loop(o.acc.sizes);
         {
           std::string pred, addr = address(o.acc, idx0(o.acc.sizes), idx1(o.acc.sizes), pred);
-          os << pad() << name << "[t] = " << (pred.empty() ? mem_read(o.acc, addr) : "(" + pred + ") ? " + mem_read(o.acc, addr) + " : " + other_of(o.acc))
+          os << pad() << name << "[t] = "
+             << (pred.empty() ? mem_read(o.acc, addr) : "(" + pred + ") ? " + mem_read(o.acc, addr) + " : " + other_of(o.acc, idx0(o.acc.sizes), idx1(o.acc.sizes)))
              << ";\n";
         }
         close_loop();
@@ -713,7 +716,7 @@ struct Gen {
             open_element_loop(ls);
             for (auto &f : fill) {
               std::string pred, addr = address(f.first->acc, l0, l1, pred);
-              os << pad() << "if (!(" << pred << ")) " << f.second << "[n] = " << other_of(f.first->acc) << ";\n";
+              os << pad() << "if (!(" << pred << ")) " << f.second << "[n] = " << other_of(f.first->acc, l0, l1) << ";\n";
             }
             close_loop();
             fill.clear();
@@ -808,25 +811,23 @@ struct Gen {
   void loop(const SOp &s) {
     const std::string L = std::to_string(s.loop);
     // loop-carried block values live in per-thread arrays (element-wise programs never move a value between
-    // elements, so each thread carries the elements it owns); all of them must have one shape of <= 16384 elements
-    std::vector<int64_t> cshape;
+    // elements, so each thread carries the elements it owns), each of <= 16384 elements; values of one shape are
+    // initialised and stepped together
+    std::vector<std::vector<int64_t>> cshapes;
     for (size_t q = 0; q < s.tile_args.size(); q++) {
       const Value &V = val(s.tile_args[q]);
-      if (V.shape.empty() || V.shape.size() > 2) no("a loop-carried value of rank " + std::to_string(V.shape.size()));
-      if (q == 0) cshape = V.shape;
-      if (V.shape != cshape) no("loop-carried block values of different shapes");
+      if (V.shape.empty() || V.shape.size() > 4) no("a loop-carried value of rank " + std::to_string(V.shape.size()));
+      if (count(V.shape) > TWO_PHASE_MAX) no("a loop-carried block value of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
+      if (std::find(cshapes.begin(), cshapes.end(), V.shape) == cshapes.end()) cshapes.push_back(V.shape);
+      os << pad() << ctype(V.dtype) << " car" << L << "_" << q << "[" << (count(V.shape) + 255) / 256 << "];\n";
     }
-    const int64_t CT = s.tile_args.empty() ? 0 : count(cshape);
-    if (CT > TWO_PHASE_MAX) no("a loop-carried block value of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
-    const std::string ci0 = idx0(cshape), ci1 = idx1(cshape);
-    for (size_t q = 0; q < s.tile_args.size(); q++)
-      os << pad() << ctype(val(s.tile_args[q]).dtype) << " car" << L << "_" << q << "[" << (CT + 255) / 256 << "];\n";
-    if (!s.tile_args.empty()) {
+    for (const auto &cshape : cshapes) {
       open_element_loop(cshape);
-      for (size_t q = 0; q < s.tile_args.size(); q++) os << pad() << "car" << L << "_" << q << "[n] = " << at(s.tile_inits[q], ci0, ci1) << ";\n";
+      for (size_t q = 0; q < s.tile_args.size(); q++)
+        if (val(s.tile_args[q]).shape == cshape) os << pad() << "car" << L << "_" << q << "[n] = " << at(s.tile_inits[q], idx0(cshape), idx1(cshape)) << ";\n";
       close_loop();
     }
-    for (size_t q = 0; q < s.tile_args.size(); q++) held[s.tile_args[q]] = {"car" + L + "_" + std::to_string(q), cshape};
+    for (size_t q = 0; q < s.tile_args.size(); q++) held[s.tile_args[q]] = {"car" + L + "_" + std::to_string(q), val(s.tile_args[q]).shape};
     for (size_t q = 0; q < s.int_iters.size(); q++)
       os << pad() << "long long it" << L << "_" << q << " = " << ex(s.int_iters[q].init) << ";\n";
     // the induction variable wraps at the width of the loop's bounds
@@ -835,11 +836,13 @@ struct Gen {
     indent++;
     std::vector<int> body_held;
     body(s.body, &body_held);
-    if (!s.tile_args.empty()) {
+    for (const auto &cshape : cshapes) {  // all new values of a shape first, then the assignments: a yield may read another carried value
       open_element_loop(cshape);
       for (size_t q = 0; q < s.tile_args.size(); q++)
-        os << pad() << "const " << ctype(val(s.tile_args[q]).dtype) << " ny" << q << " = " << at(s.tile_yields[q], ci0, ci1) << ";\n";
-      for (size_t q = 0; q < s.tile_args.size(); q++) os << pad() << "car" << L << "_" << q << "[n] = ny" << q << ";\n";
+        if (val(s.tile_args[q]).shape == cshape)
+          os << pad() << "const " << ctype(val(s.tile_args[q]).dtype) << " ny" << q << " = " << at(s.tile_yields[q], idx0(cshape), idx1(cshape)) << ";\n";
+      for (size_t q = 0; q < s.tile_args.size(); q++)
+        if (val(s.tile_args[q]).shape == cshape) os << pad() << "car" << L << "_" << q << "[n] = ny" << q << ";\n";
       close_loop();
     }
     for (int v : body_held) {
@@ -857,7 +860,7 @@ struct Gen {
     for (size_t q = 0; q < s.tile_args.size(); q++) {
       held.erase(s.tile_args[q]);
       var.erase(s.tile_args[q]);
-      if (s.results[q] >= 0) held[s.results[q]] = {"car" + L + "_" + std::to_string(q), cshape};
+      if (s.results[q] >= 0) held[s.results[q]] = {"car" + L + "_" + std::to_string(q), val(s.tile_args[q]).shape};
     }
   }
 

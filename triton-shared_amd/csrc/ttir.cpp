@@ -600,11 +600,32 @@ static void parse_func_body(Lines &L, Block &out) {
 // A function kept out of line (`noinline`) arrives as its own tt.func and a tt.call.  The reference's pipeline inlines
 // it on the way down (triton-shared-opt runs the inliner before the conversion); here the callee's ops are copied to
 // the call site under fresh names, arguments replaced by the call's operands and the call's results by what the callee
-// returns.  A callee that returns values from inside a branch is refused.
+// returns.
 struct Callee {
   Func f;
   bool busy = false;
 };
+
+// A callee that returns from both sides of a branch (`if c: return a` ... `return b`): the branch becomes an `if` that
+// yields the returned values, followed by a single return of its results.  True when the block ends in one return.
+static bool single_return(Block &b, const std::vector<Type> &types, int &serial) {
+  if (b.ops.empty()) return false;
+  Op &last = *b.ops.back();
+  if (last.name == "tt.return") return true;
+  if (last.name != "cf.if" || last.regions.size() != 2) return false;
+  if (!single_return(last.regions[0], types, serial) || !single_return(last.regions[1], types, serial)) return false;
+  for (auto &r : last.regions) r.ops.back()->name = "scf.yield";
+  last.name = "scf.if";
+  last.result_types = types;
+  auto ret = std::make_unique<Op>();
+  ret->name = "tt.return";
+  for (size_t i = 0; i < types.size(); i++) {
+    last.results.push_back("%ret__" + std::to_string(++serial) + "_" + std::to_string(i));
+    ret->operands.push_back(last.results.back());
+  }
+  b.ops.push_back(std::move(ret));
+  return true;
+}
 
 static void inline_calls(Block &b, std::map<std::string, Callee> &callees, Renames &subst, int &serial) {
   std::vector<std::unique_ptr<Op>> out;
@@ -636,12 +657,13 @@ static void inline_calls(Block &b, std::map<std::string, Callee> &callees, Renam
     inline_calls(body, callees, inner, serial);
     c.busy = false;
     std::vector<std::string> returned;
+    if (!op.results.empty()) single_return(body, c.f.result_types, serial);
     if (!body.ops.empty() && body.ops.back()->name == "tt.return") {
       returned = body.ops.back()->operands;
       body.ops.pop_back();
     }
     if (returned.size() != op.results.size())
-      throw Unsupported("call of " + op.words.at(0) + ": the callee returns its values from inside a branch");
+      throw Unsupported("call of " + op.words.at(0) + ": the callee returns its values from inside a loop or a nested region");
     for (size_t i = 0; i < returned.size(); i++) subst[op.results[i]] = returned[i];
     for (auto &o : body.ops) out.push_back(std::move(o));
   }
@@ -712,6 +734,7 @@ Func parse_ttir(const std::string &text) {
           const size_t attr = res.find("attributes");
           if (attr != std::string::npos) res = trim(res.substr(0, attr));
           has_results = res != "()";
+          if (has_results) f.result_types = parse_type_list(res);
         }
       }
       if (has_results && !is_private) throw Unsupported("tt.func with results is not a kernel");

@@ -68,6 +68,7 @@ struct Func {
   std::string name;
   std::vector<std::string> arg_names;
   std::vector<Type> arg_types;
+  std::vector<Type> result_types;  // of a callee; a kernel has none
   Block body;
 };
 
