@@ -923,3 +923,14 @@ def grouped_rows_matmul(a_ptr, b_ptr, c_ptr, rows_ptr, expert_ptr, n_rows, K, N,
         a_ptrs += BK
         b_ptrs += BK * s_bk
     tl.store(c_ptr + i[:, None] * s_cm + j[None, :], acc, mask=ok[:, None] & (j[None, :] < N))
+
+
+@triton.jit
+def pointer_picked_by_branch(src, dst, which):
+    # both sides of a branch produce a pointer into the same argument (test/Conversion/TritonToStructured/conditional_ptr_as_src.mlir)
+    if which == 5:
+        p = src + which * 2
+    else:
+        p = src + which
+    i = tl.arange(0, 4)
+    tl.store(dst + i, tl.load(p + 6 + i))

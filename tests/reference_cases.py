@@ -167,6 +167,11 @@ def cases():
              + [(k, "constexpr") for k in ("BM", "BN", "BK")]), {"BM": 16, "BN": 16, "BK": 32}, (3, 2),
         lambda: [Am.reshape(-1).copy(), Bm.reshape(-1).copy(), np.full(n_tok * Nd, -1, np.float32), rows.copy(), experts.copy(), n_tok, Kd, Nd, Kd, Kd * Nd, Nd, Nd],
         lambda a: _eq(a[2], want_moe()))
+    # test/Conversion/TritonToStructured/conditional_ptr_as_src.mlir (a lit input without a runtime test in the reference)
+    for which, first in [(5, 16), (3, 9)]:
+        add(f"pointer_picked_by_branch_{which}", "pointer_picked_by_branch", {"src": P, "dst": P, "which": "i32"}, {}, (1,),
+            lambda which=which: [np.arange(32, dtype=np.float32), np.full(4, -1, np.float32), which],
+            lambda a, first=first: _eq(a[1], np.arange(first, first + 4, dtype=np.float32)))
     # test_einsum_qhmd_hmpd_to_qhmp.py:150-165
     Q, H, Mm, D, Pp = 1, 2, 2, 2, 4
     rng = np.random.default_rng(4)

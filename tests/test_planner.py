@@ -384,12 +384,12 @@ def test_reference_lit_inputs_plan_or_are_refused_for_a_known_reason(native):
         "tensor-typed kernel argument": 18,                       # blocks of pointers as arguments: no launcher can pass them
         "operation tensor.empty": 9,                              # tensor dialect ops written by hand into triton_assert.mlir
         "tt.func with results is not a kernel": 6,
-        "tile_program: a loop-carried block value of more than 16384 elements": 6,   # dot + separate add of an older front end, 128 x 256 accumulators
+        "tile_program: a loop-carried block value of more than 32768 elements": 3,   # 256 x 256 accumulators in one program (kernel-05-layer-norm-dwdb.mlir)
         "unsupported type '<tensor<": 8,                          # block pointers: the front end pass list rewrites them before this stage
         "tile_program: the reductions of this program need": 4,
         "tile_program: elementwise op extern.some_symbol": 3,     # the reference refuses it too (unsupported_extern_elementwise.mlir)
         "pointer-valued operation": 10,                           # int_to_ptr / bitcast / cat / select on pointers (the reference's TritonToPtr fallback)
-        "scf.if that yields pointers": 4,
+        "scf.if that yields blocks of pointers": 2,
         "unsupported type 'f8E4M3FN'": 1,
         "unsupported type '[": 3,                                 # tts / memref dialect inputs of later stages
         "unsupported type '}'": 1,
@@ -409,4 +409,4 @@ def test_reference_lit_inputs_plan_or_are_refused_for_a_known_reason(native):
                 refused[why] += 1
     for why, n in refused.items():
         assert n <= known[why], (why, n)
-    assert planned >= 330, (planned, dict(refused))
+    assert planned >= 335, (planned, dict(refused))

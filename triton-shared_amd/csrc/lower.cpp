@@ -1187,9 +1187,17 @@ class Lowerer {
     const size_t nres = op.results.size();
     if (nres && op.regions.size() != 2) throw Unsupported("scf.if with results but without an else region");
     std::vector<int> results;
+    // A scalar pointer that both sides derive from one argument is yielded as its offset from that argument, a 64-bit
+    // integer like any other result; after the branch the pointer is the argument plus that value.
+    std::vector<int> ptr_base(nres, -1);
     for (size_t j = 0; j < nres; j++) {
-      const Type &t = op.result_types.at(j);
-      if (t.ptr) throw Unsupported("scf.if that yields pointers (line " + std::to_string(op.line) + ")");
+      Type t = op.result_types.at(j);
+      if (t.ptr) {
+        if (t.is_tensor) throw Unsupported("scf.if that yields blocks of pointers (line " + std::to_string(op.line) + ")");
+        ptr_base[j] = -2;  // the sides fill it in
+        t.ptr = false;
+        t.elem = "i64";
+      }
       results.push_back(new_value(t));
     }
     for (int side = 0; side < 2 && side < (int)op.regions.size(); side++) {
@@ -1210,12 +1218,40 @@ class Lowerer {
       }
       for (size_t i = 0; i < count; i++) lower_op(*region.ops[i]);
       if (nres)
-        for (auto &y : region.ops.back()->operands) s.tile_yields.push_back(data_of(y));
+        for (size_t j = 0; j < nres; j++) {
+          const std::string &y = region.ops.back()->operands[j];
+          if (ptr_base[j] == -1) {
+            s.tile_yields.push_back(data_of(y));
+            continue;
+          }
+          PtrState st = visit(y);
+          if (st.rank() != 0 || st.source < 0) throw Unsupported("scf.if that yields a pointer without a base argument (line " + std::to_string(op.line) + ")");
+          if (ptr_base[j] >= 0 && ptr_base[j] != st.source)
+            throw Unsupported("scf.if whose sides yield pointers into different arguments (line " + std::to_string(op.line) + ")");
+          ptr_base[j] = st.source;
+          SOp f;
+          f.kind = SK::FromIndex;
+          f.expr = P.pool.to_index(st.scalar >= 0 ? st.scalar : c64(0));
+          Type it;
+          it.elem = "i64";
+          f.result = new_value(it);
+          cur_->push_back(f);
+          s.tile_yields.push_back(f.result);
+        }
       cur_ = saved;
       if (!s.body.empty() || nres) cur_->push_back(std::move(s));
     }
     // the results are data from here on (an integer result is not an index expression: what is computed from it is data too)
-    for (size_t j = 0; j < nres; j++) data_[op.results[j]] = results[j];
+    for (size_t j = 0; j < nres; j++) {
+      if (ptr_base[j] == -1) {
+        data_[op.results[j]] = results[j];
+        continue;
+      }
+      PtrState after;
+      after.source = ptr_base[j];
+      after.scalar = P.pool.data(results[j], 64);
+      known_ptr_[op.results[j]] = after;
+    }
   }
 
   void lower_block(const Block &b) {

@@ -817,7 +817,7 @@ struct Gen {
     for (size_t q = 0; q < s.tile_args.size(); q++) {
       const Value &V = val(s.tile_args[q]);
       if (V.shape.empty() || V.shape.size() > 4) no("a loop-carried value of rank " + std::to_string(V.shape.size()));
-      if (count(V.shape) > TWO_PHASE_MAX) no("a loop-carried block value of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
+      if (count(V.shape) > 2 * TWO_PHASE_MAX) no("a loop-carried block value of more than " + std::to_string(2 * TWO_PHASE_MAX) + " elements");
       if (std::find(cshapes.begin(), cshapes.end(), V.shape) == cshapes.end()) cshapes.push_back(V.shape);
       os << pad() << ctype(V.dtype) << " car" << L << "_" << q << "[" << (count(V.shape) + 255) / 256 << "];\n";
     }
