@@ -209,6 +209,18 @@ def make_workloads(torch, triton, K):
         return dict(desc=f"C = leaky_relu(A @ B) bf16 {n}^3, BM=BN=128 BK=64 (generic family: LDS-staged operands, 32x32 MFMA blocks)",
                     work=2 * n ** 3, bound="mfma", dtype="bf16", make=make, set_bytes=3 * n * n * 2)
 
+    def expert_rows(tokens, kd, nd, experts):
+        def make():
+            a = (torch.randn(tokens, kd, device=dev) * 0.02).bfloat16()
+            b = (torch.randn(experts, kd, nd, device=dev) * 0.02).bfloat16()
+            c = torch.empty(tokens, nd, dtype=torch.bfloat16, device=dev)
+            rows = torch.randperm(tokens, device=dev).int()
+            ids = (torch.arange(tokens // 128, device=dev) % experts).int()
+            return lambda: K.expert_rows_matmul[(tokens // 128, nd // 128)](a, b, c, rows, ids, tokens, kd, nd, kd, kd * nd, nd, nd, BM=128, BN=128, BK=64)
+        return dict(desc=f"mixture-of-experts product bf16: {tokens} rows gathered through an index vector, x [{experts}, {kd}, {nd}] weights picked by a "
+                         "loaded expert id per 128 rows (generic family: carried gather offsets, LDS-staged operands, 32x32 MFMA blocks)",
+                    work=2 * tokens * kd * nd, bound="mfma", dtype="bf16", make=make, set_bytes=(tokens * kd + experts * kd * nd + tokens * nd) * 2)
+
     W["cfg1"] = vec_add(98432)
     W["cfg2"] = softmax(4096)
     W["cfg3"] = layernorm()
@@ -219,6 +231,7 @@ def make_workloads(torch, triton, K):
     W["next_fused_gelu_2p26"] = fused_gelu(1 << 26)
     W["next_fused_silu_2p26"] = fused_silu(1 << 26)
     W["next_matmul_act_2048"] = matmul_act(2048)
+    W["next_expert_rows_4096"] = expert_rows(4096, 2048, 2048, 8)
     W["next_take_rows_2p26"] = take_rows(1 << 16, 1024)
     W["next_row_sums_2p26"] = row_sums(1 << 16, 1024)
     W["next_block_cumsum_2p26"] = block_cumsum(1 << 26)

@@ -758,9 +758,11 @@ def softmax_persistent(out_ptr, in_ptr, in_pitch, out_pitch, n_rows, n_cols, BLO
 
 
 @triton.jit
-def matmul_leaky(a_ptr, b_ptr, c_ptr, M, N, K, s_am, s_bk, s_cm, slope, BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr):
-    # a tiled matmul with an activation fused before the narrowing store (the tutorial's ACTIVATION hook): not the shape
-    # the MFMA kernels take, so the generic family runs it
+def matmul_leaky(a_ptr, b_ptr, c_ptr, M, N, K, s_am, s_bk, s_cm, slope, BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr,
+                 ACT: tl.constexpr = 0, bias_ptr=None):
+    # a tiled matmul with elementwise ops fused before the narrowing store (the tutorial's ACTIVATION hook).  ACT 0: leaky
+    # relu, 1: x * sigmoid(slope * x) -- functions of the accumulator alone, which the matmul kernels take as an epilogue;
+    # 2: a bias per column before the leaky relu -- depends on the element's position, so the generic family runs it
     tm = tl.program_id(0)
     tn = tl.program_id(1)
     rm = tm * BM + tl.arange(0, BM)
@@ -776,7 +778,12 @@ def matmul_leaky(a_ptr, b_ptr, c_ptr, M, N, K, s_am, s_bk, s_cm, slope, BM: tl.c
         acc = tl.dot(a, b, acc)
         pa += BK
         pb += BK * s_bk
-    acc = tl.where(acc >= 0, acc, slope * acc)
+    if ACT == 1:
+        acc = acc * tl.sigmoid(acc * slope)
+    else:
+        if ACT == 2:
+            acc += tl.load(bias_ptr + rn, mask=rn < N, other=0.0)[None, :]
+        acc = tl.where(acc >= 0, acc, slope * acc)
     tl.store(c_ptr + rm[:, None] * s_cm + rn[None, :], acc.to(c_ptr.dtype.element_ty), mask=(rm[:, None] < M) & (rn[None, :] < N))
 
 

@@ -1110,16 +1110,45 @@ def test_tile_program_persistent_softmax():
 
 
 def test_tile_program_matmul_with_fused_activation():
-    """A 128 x 128 x 64 bf16 tile matmul with a leaky-relu before the store: outside the MFMA kernels' shape, so it runs as
-    small-product code (operands staged in LDS in their 16-bit type)."""
+    """A 128 x 128 x 64 bf16 tile matmul with a bias per column and a leaky-relu before the store: the epilogue depends on
+    the element's position, so it runs as small-product code (operands staged in LDS in their 16-bit type)."""
     import extra_kernels as X
     torch.manual_seed(18)
     M, N, K = 200, 300, 150
     a = torch.randn(M, K, device=DEV).bfloat16()
     b = torch.randn(K, N, device=DEV).bfloat16()
+    bias = torch.randn(N, device=DEV)
     c = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
-    k = X.matmul_leaky[(triton.cdiv(M, 128), triton.cdiv(N, 128))](a, b, c, M, N, K, a.stride(0), b.stride(0), c.stride(0), 0.01, BM=128, BN=128, BK=64)
+    k = X.matmul_leaky[(triton.cdiv(M, 128), triton.cdiv(N, 128))](a, b, c, M, N, K, a.stride(0), b.stride(0), c.stride(0), 0.01, BM=128, BN=128, BK=64,
+                                                                    ACT=2, bias_ptr=bias)
     torch.cuda.synchronize()
     assert k.function.family == "tile_program"
-    want = torch.nn.functional.leaky_relu(a.double() @ b.double(), 0.01)
+    want = torch.nn.functional.leaky_relu(a.double() @ b.double() + bias.double(), 0.01)
+    assert ((c.double() - want).norm() / want.norm()) <= 1e-2
+
+
+@pytest.mark.parametrize("M,N,K,kernel", [(512, 768, 96, "gemm_dma_kernel + epilogue"), (200, 300, 150, "gemm_mfma_kernel<128x128x64> + epilogue"),
+                                          (2100, 2060, 72, "gemm_mfma_kernel<256x256x32> + epilogue")])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gemm_with_fused_epilogue(M, N, K, kernel, dtype):
+    """The tutorial matmul's fused activation (test_matmul.py:98-99, 112-117): ops on the accumulator alone are compiled into
+    the epilogue of the matmul kernels.  Operands of -1 / 0 / 1 and a slope of 1/2 make every value exact in 16 bits, so
+    the result must equal leaky_relu(A @ B) bit for bit, on each of the three kernels the launcher chooses from."""
+    import extra_kernels as X
+    g = torch.Generator(device="cpu").manual_seed(M + K)
+    a = torch.randint(-1, 2, (M, K), generator=g).to(dtype).to(DEV)
+    b = torch.randint(-1, 2, (K, N), generator=g).to(dtype).to(DEV)
+    c = torch.full((M, N), 7, device=DEV, dtype=dtype)
+    k = X.matmul_leaky[(triton.cdiv(M, 128), triton.cdiv(N, 128))](a, b, c, M, N, K, a.stride(0), b.stride(0), c.stride(0), 0.5, BM=128, BN=128, BK=64)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and k.function.last_kernel.startswith(kernel), k.function.last_kernel
+    want = torch.nn.functional.leaky_relu(a.float() @ b.float(), 0.5)
+    assert torch.equal(c.float(), want)
+    # a smooth activation: within the tolerance of the family
+    a = torch.randn(M, K, device=DEV).to(dtype)
+    b = torch.randn(K, N, device=DEV).to(dtype)
+    X.matmul_leaky[(triton.cdiv(M, 128), triton.cdiv(N, 128))](a, b, c, M, N, K, a.stride(0), b.stride(0), c.stride(0), 0.25, BM=128, BN=128, BK=64, ACT=1)
+    torch.cuda.synchronize()
+    z = a.double() @ b.double()
+    want = z * torch.sigmoid(z * 0.25)
     assert ((c.double() - want).norm() / want.norm()) <= 1e-2

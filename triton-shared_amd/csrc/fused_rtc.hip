@@ -317,6 +317,13 @@ hipError_t rtc_launch(RtcModule *m, int gx, int gy, int gz, int block, void *arg
   return hipModuleLaunchKernel(m->fn, gx, gy, gz, block, 1, 1, 0, s, nullptr, config);
 }
 
+const char *gemm_device_source() {
+  static const char *text =
+#include "gemm_device.inc"
+      ;
+  return text;
+}
+
 hipError_t fused_map_compile(const MapNParams &p, RtcModule **out, std::string *err) { return rtc_compile(source_of(p), "fused_map", out, err); }
 
 hipError_t fused_map_launch(RtcModule *m, const MapNParams &p, int gx, int gy, int gz, hipStream_t s) {

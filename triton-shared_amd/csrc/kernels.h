@@ -7,6 +7,7 @@
 #include <cstdint>
 #include <string>
 
+#include "gemm_device.h"
 #include "mapn_isa.h"
 
 namespace tts {
@@ -56,6 +57,7 @@ hipError_t launch_mapn(const MapNParams &p, int gx, int gy, int gz, hipStream_t 
 struct RtcModule;
 hipError_t rtc_compile(const std::string &source, const char *entry, RtcModule **out, std::string *err);
 hipError_t rtc_launch(RtcModule *m, int gx, int gy, int gz, int block, void *args, size_t size, hipStream_t s);
+const char *gemm_device_source();  // the text of gemm_device.h
 void rtc_release(RtcModule *m);
 // The fused map's register program printed as HIP source and compiled once.
 hipError_t fused_map_compile(const MapNParams &p, RtcModule **out, std::string *err);
@@ -87,14 +89,14 @@ struct LayerNormParams {
 hipError_t launch_layernorm(const LayerNormParams &p, int gx, int gy, int gz, hipStream_t s, const char **kernel_name);
 
 // C[M,N] = A[M,K] * B[K,N], 16-bit inputs, fp32 accumulate, 16-bit output (RTNE)
-struct GemmParams {
-  const void *a, *b;
-  void *c;
-  int64_t M, N, K;
-  int64_t lda, ldb, ldc;  // row pitches in elements; the inner strides are 1
-  int is_bf16;
-};
+using GemmParams = ::TtsGemmParams;  // gemm_device.h
 hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **kernel_name);
+// The same product with elementwise ops fused into the epilogue: `epilogue` is the source of the functor (match.h:
+// gemm_epilogue_source), `modules` the plan's three slots for the kernels compiled from it (one per tiling, filled at
+// the first launch that needs it), `args` / `args_size` the generic families' argument block.
+struct RtcModule;
+hipError_t launch_gemm_epilogue(const GemmParams &p, const std::string &epilogue, RtcModule **modules, void *args, size_t args_size,
+                                hipStream_t s, const char **kernel_name, std::string *err);
 
 // C[M,N] = A[M,K] * (f16(W[K,N]) * scale[N]), A/scale/C fp16, W int8, fp32 accumulate, M <= 16
 struct GemmW8A16Params {

@@ -4,6 +4,7 @@
 #include "mapn_isa.h"
 
 #include <functional>
+#include <set>
 #include <sstream>
 
 namespace tts {
@@ -824,6 +825,82 @@ bool try_tile_program(Plan &pl) {
   return true;
 }
 
+// A tiled matmul whose accumulator goes through elementwise ops before the store (the tutorial kernel's fused
+// activation, test_matmul.py:98-99): the ops between the K loop and the store are taken out as an epilogue functor, and
+// what is left -- the loop, a narrowing cast, the store -- is matched as the plain product.
+static bool try_gemm_with_epilogue(Plan &pl) {
+  const Program &P = pl.prog;
+  int loop_at = -1, store_at = -1;
+  for (size_t i = 0; i < P.body.size(); i++) {
+    const SK k = P.body[i].kind;
+    if (k == SK::For) {
+      if (loop_at >= 0) return false;
+      loop_at = (int)i;
+    } else if (k == SK::Store) {
+      if (store_at >= 0) return false;
+      store_at = (int)i;
+    } else if (k != SK::Map && k != SK::Const && k != SK::Splat && k != SK::ScalarArg && k != SK::FromIndex) {
+      return false;
+    }
+  }
+  if (loop_at < 0 || store_at != (int)P.body.size() - 1 || store_at < loop_at) return false;
+  const SOp &loop = P.body[loop_at], &st = P.body[store_at];
+  if (loop.results.size() != 1 || loop.results[0] < 0 || st.operands.empty()) return false;
+  const int acc = loop.results[0], out = st.operands[0];
+  const std::string T = st.acc.elem;
+  if ((T != "bf16" && T != "f16") || P.values[acc].dtype != "f32" || P.values[out].shape != P.values[acc].shape) return false;
+  if (store_at == loop_at + 2 && P.body[loop_at + 1].kind == SK::Map && P.body[loop_at + 1].name == "arith.truncf" &&
+      P.body[loop_at + 1].operands.at(0) == acc)
+    return false;  // the plain product: nothing to take out
+  // the product without the epilogue
+  Program Q = P;
+  Value narrowed = P.values[acc];
+  narrowed.dtype = T;
+  Q.values.push_back(narrowed);
+  SOp cast;
+  cast.kind = SK::Map;
+  cast.name = "arith.truncf";
+  cast.operands = {acc};
+  cast.result = (int)Q.values.size() - 1;
+  SOp store = st;
+  store.operands[0] = cast.result;
+  // values the loop reads keep their definitions; what only the epilogue read goes
+  std::set<int> used;
+  std::function<void(const SOp &)> reads = [&](const SOp &s) {
+    for (int v : s.operands) used.insert(v);
+    for (int v : s.tile_inits) used.insert(v);
+    for (int v : {s.acc.gather, s.acc.mask_value, s.acc.other_value})
+      if (v >= 0) used.insert(v);
+    for (auto &b : s.body) reads(b);
+  };
+  reads(loop);
+  std::vector<SOp> kept;
+  for (int i = loop_at - 1; i >= 0; i--) {
+    const SOp &s = P.body[i];
+    if (s.result >= 0 && !used.count(s.result)) continue;
+    reads(s);
+    kept.insert(kept.begin(), s);
+  }
+  Q.body = kept;
+  Q.body.push_back(loop);
+  Q.body.push_back(cast);
+  Q.body.push_back(store);
+  Plan q;
+  q.prog = std::move(Q);
+  q.signature = signature(q.prog);
+  try {
+    if (!try_gemm(q, false)) return false;
+    std::vector<const SOp *> ops;
+    for (auto &s : P.body)
+      if (s.kind != SK::For && s.kind != SK::Store) ops.push_back(&s);
+    q.source = gemm_epilogue_source(P, ops, acc, out);
+  } catch (const Unsupported &) {
+    return false;  // not this shape of program: the other families get their turn
+  }
+  pl = std::move(q);
+  return true;
+}
+
 Plan make_plan(Program &&p) {
   Plan pl;
   pl.prog = std::move(p);
@@ -845,6 +922,7 @@ Plan make_plan(Program &&p) {
     throw Unsupported("a program with gathers, scatters or masks and fill values that are data is outside the hand-written families; signature: " + pl.signature);
   }
   if (try_map1d(pl) || try_softmax(pl) || try_layernorm(pl)) return pl;
+  if (try_gemm_with_epilogue(pl)) return pl;
   std::string gemm_refusal;
   try {
     if (try_gemm(pl, false) || try_gemm(pl, true)) return pl;

@@ -33,7 +33,7 @@ struct Plan {
   std::map<std::string, Lin> lin;   // named pid-linear forms
   std::map<std::string, int64_t> k; // named compile-time constants (block sizes, arg indices)
   std::map<std::string, double> f;  // named float constants
-  std::string source;               // TileProgram: the HIP source of the program's kernel
+  std::string source;               // TileProgram: the HIP source of the program's kernel; Gemm: of its epilogue functor, if any
 };
 
 // Generic family: HIP source for a program of structured loads, elementwise ops and stores
@@ -41,6 +41,9 @@ struct Plan {
 // every kernel argument by index: { void *ptr[N]; long long ival[N]; double fval[N]; }, N = TILE_MAX_ARGS.
 constexpr int TILE_MAX_ARGS = 32;
 std::string tile_program_source(const Program &p);
+// Matmul family with ops between the K loop and the store: the source of the functor that applies them to one
+// accumulator value (tile_codegen.cpp), compiled at run time together with the kernels of gemm_device.h.
+std::string gemm_epilogue_source(const Program &p, const std::vector<const SOp *> &ops, int acc, int out);
 
 // Normalised listing of a program's ops (no shapes, no expression ids).
 std::string signature(const Program &p);

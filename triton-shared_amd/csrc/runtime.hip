@@ -68,10 +68,12 @@ struct tts_plan {
   int *counters = nullptr;     // split-K arrival counters (device), zero between launches
   size_t counters_count = 0;
   RtcModule *fused = nullptr;  // the kernel compiled for this plan at its first launch (fused maps, tile programs)
+  RtcModule *gemm_rtc[3] = {nullptr, nullptr, nullptr};  // matrix products with a fused epilogue: one kernel per tiling
   ~tts_plan() {
     if (workspace) (void)hipFree(workspace);
     if (counters) (void)hipFree(counters);
     rtc_release(fused);
+    for (RtcModule *m : gemm_rtc) rtc_release(m);
   }
 };
 
@@ -529,7 +531,22 @@ tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, cons
         p.a = ptr_arg<const void>(args, pl, "a_arg");
         p.b = ptr_arg<const void>(args, pl, "b_arg");
         p.c = ptr_arg<void>(args, pl, "c_arg");
-        err = launch_gemm(p, s, &kname);
+        if (pl.source.empty()) {
+          err = launch_gemm(p, s, &kname);
+          break;
+        }
+        struct { void *ptr[TILE_MAX_ARGS]; long long ival[TILE_MAX_ARGS]; double fval[TILE_MAX_ARGS]; } a{};
+        for (int i = 0; i < n; i++) {
+          if (args[i].kind == TTS_ARG_PTR) a.ptr[i] = args[i].v.ptr;
+          else if (args[i].kind == TTS_ARG_INT) a.ival[i] = args[i].v.i;
+          else a.fval[i] = args[i].v.f;
+        }
+        std::string why;
+        {
+          std::lock_guard<std::mutex> lock(plan->mu);
+          err = launch_gemm_epilogue(p, pl.source, plan->gemm_rtc, &a, sizeof a, s, &kname, &why);
+        }
+        if (err != hipSuccess && !why.empty()) return fail(TTS_HIP_ERROR, "gemm epilogue: " + why);
         break;
       }
       case Family::GemmW8A16: {

@@ -1386,4 +1386,34 @@ std::string tile_program_source(const Program &p) {
   return all.str();
 }
 
+// The elementwise ops a matmul kernel applies to its accumulator before the store (an activation, a scale, the
+// narrowing cast), as the functor the matrix-product kernels of gemm_device.h call on every accumulator value: `ops` are
+// the program's ops after the K loop, `acc` the loop's result, `out` the value that is stored.  The ops may read the
+// accumulator, constants and scalar kernel arguments only (nothing that depends on the element's position or the program
+// id): the kernels use a tiling of their own.  Throws Unsupported otherwise.
+std::string gemm_epilogue_source(const Program &p, const std::vector<const SOp *> &ops, int acc, int out) {
+  if ((int)p.arg_names.size() > TILE_MAX_ARGS) throw Unsupported("more than " + std::to_string(TILE_MAX_ARGS) + " kernel arguments");
+  Gen g(p);
+  for (const SOp *s : ops) {
+    if (s->kind != SK::Map && s->kind != SK::Const && s->kind != SK::Splat && s->kind != SK::ScalarArg && s->kind != SK::FromIndex)
+      throw Unsupported("an epilogue op that is not elementwise arithmetic on the accumulator");
+    if (s->kind == SK::Map && (s->name.rfind("tt.", 0) == 0 && s->name.rfind("tt.clampf", 0) != 0 && s->name.rfind("tt.precise", 0) != 0))
+      throw Unsupported("an epilogue op that moves elements (" + s->name + ")");
+    if (s->kind == SK::FromIndex)
+      for (EK k : {EK::Pid, EK::NProg, EK::IV, EK::Iter, EK::Result, EK::Data})
+        if (p.pool.depends_on(s->expr, k)) throw Unsupported("an epilogue value that depends on the program id or on data");
+    g.def[s->result] = s;
+  }
+  g.var[acc] = "acc";
+  g.cur_i0 = g.cur_i1 = "e";  // one element: whatever is named is the element's own value
+  const std::string expr = g.at(out, "e", "e");
+  std::string pre = TILE_PRELUDE;
+  const std::string n = std::to_string(TILE_MAX_ARGS);
+  for (size_t pos = 0; (pos = pre.find("%N%", pos)) != std::string::npos;) pre.replace(pos, 3, n);
+  std::ostringstream all;
+  all << pre << "typedef Args TtsEpArgs;\n"
+      << "struct TtsEp {\n  TtsEpArgs p;\n  __device__ __forceinline__ float operator()(float acc) const { return " << expr << "; }\n};\n";
+  return all.str();
+}
+
 }  // namespace tts

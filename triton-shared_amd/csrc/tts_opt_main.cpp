@@ -4,7 +4,7 @@
 //   tts-opt --roundtrip file     -> read the structured text back and print it again
 //   tts-opt --signature file     -> normalised op listing used by the family matcher
 //   tts-opt --plan file          -> matched kernel family and its bindings
-//   tts-opt --source file        -> HIP source of a program of the generic tile_program family
+//   tts-opt --source file        -> HIP source of a program of the generic tile_program family (or of a fused matmul epilogue)
 #include <fstream>
 #include <iostream>
 #include <sstream>
@@ -35,8 +35,9 @@ int main(int argc, char **argv) {
       std::cout << tts::signature(p) << "\n";
       return 0;
     }
-    if (source) {
-      std::cout << tts::tile_program_source(p);
+    if (source) {  // the generic family's kernel, or the epilogue functor of a matrix product that fuses one
+      tts::Plan pl = tts::make_plan(tts::Program(p));
+      std::cout << (pl.source.empty() ? tts::tile_program_source(p) : pl.source);
       return 0;
     }
     if (plan) {

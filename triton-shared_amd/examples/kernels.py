@@ -245,3 +245,31 @@ def matmul_leaky_relu(a_ptr, b_ptr, c_ptr, M, N, K, s_am, s_bk, s_cm, slope, BM:
         pb += BK * s_bk
     acc = tl.where(acc >= 0, acc, slope * acc)
     tl.store(c_ptr + rm[:, None] * s_cm + rn[None, :], acc.to(c_ptr.dtype.element_ty), mask=(rm[:, None] < M) & (rn[None, :] < N))
+
+
+@triton.jit
+def expert_rows_matmul(a_ptr, b_ptr, c_ptr, rows_ptr, expert_ptr, n_rows, K, N, s_am, s_be, s_bk, s_cm,
+                       BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr):
+    """C[i, :] = A[rows[i], :] @ B[expert of i's block of BM rows]: the product of a mixture-of-experts layer.  The
+    expert id is read from memory (negative: nothing to do for this block), the rows of A come through loaded indices,
+    and both blocks of pointers are carried along K.  Runs on the generic family."""
+    pid_m = tl.program_id(0)
+    pid_n = tl.program_id(1)
+    expert = tl.load(expert_ptr + pid_m)
+    if expert < 0:
+        return
+    i = pid_m * BM + tl.arange(0, BM)
+    ok = i < n_rows
+    which = tl.load(rows_ptr + i, mask=ok, other=0)
+    j = pid_n * BN + tl.arange(0, BN)
+    k = tl.arange(0, BK)
+    a_ptrs = a_ptr + which[:, None] * s_am + k[None, :]
+    b_ptrs = b_ptr + expert * s_be + k[:, None] * s_bk + j[None, :]
+    acc = tl.zeros((BM, BN), tl.float32)
+    for k0 in range(0, K, BK):
+        a = tl.load(a_ptrs, mask=ok[:, None] & (k[None, :] < K - k0), other=0.0)
+        b = tl.load(b_ptrs, mask=(k[:, None] < K - k0) & (j[None, :] < N), other=0.0)
+        acc = tl.dot(a, b, acc)
+        a_ptrs += BK
+        b_ptrs += BK * s_bk
+    tl.store(c_ptr + i[:, None] * s_cm + j[None, :], acc.to(c_ptr.dtype.element_ty), mask=ok[:, None] & (j[None, :] < N))
