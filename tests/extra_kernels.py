@@ -762,7 +762,8 @@ def matmul_leaky(a_ptr, b_ptr, c_ptr, M, N, K, s_am, s_bk, s_cm, slope, BM: tl.c
                  ACT: tl.constexpr = 0, bias_ptr=None):
     # a tiled matmul with elementwise ops fused before the narrowing store (the tutorial's ACTIVATION hook).  ACT 0: leaky
     # relu, 1: x * sigmoid(slope * x) -- functions of the accumulator alone, which the matmul kernels take as an epilogue;
-    # 2: a bias per column before the leaky relu -- depends on the element's position, so the generic family runs it
+    # 2: a bias per column before the leaky relu, 3: slope * acc + what the output held -- these depend on the element's
+    # position, which the epilogue finds through the table of tile owners
     tm = tl.program_id(0)
     tn = tl.program_id(1)
     rm = tm * BM + tl.arange(0, BM)
@@ -780,6 +781,9 @@ def matmul_leaky(a_ptr, b_ptr, c_ptr, M, N, K, s_am, s_bk, s_cm, slope, BM: tl.c
         pb += BK * s_bk
     if ACT == 1:
         acc = acc * tl.sigmoid(acc * slope)
+    elif ACT == 3:
+        at = c_ptr + rm[:, None] * s_cm + rn[None, :]
+        acc = acc * slope + tl.load(at, mask=(rm[:, None] < M) & (rn[None, :] < N), other=0.0).to(tl.float32)
     else:
         if ACT == 2:
             acc += tl.load(bias_ptr + rn, mask=rn < N, other=0.0)[None, :]
@@ -941,3 +945,33 @@ def pointer_picked_by_branch(src, dst, which):
         p = src + which
     i = tl.arange(0, 4)
     tl.store(dst + i, tl.load(p + 6 + i))
+
+
+@triton.jit
+def matmul_grouped_order_plus_bias(a_ptr, b_ptr, c_ptr, bias_ptr, M, N, K, s_am, s_bk, s_cm, BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr,
+                                   GROUP_M: tl.constexpr):
+    # the tutorial's one-dimensional grid (tiles walked in groups of GROUP_M rows) with a bias per row and per column added
+    # before the cast: the epilogue has to find the program that owns an element through that tile order
+    pid = tl.program_id(0)
+    tiles_m = tl.cdiv(M, BM)
+    tiles_n = tl.cdiv(N, BN)
+    per_group = GROUP_M * tiles_n
+    m0 = (pid // per_group) * GROUP_M
+    rows_in_group = min(tiles_m - m0, GROUP_M)
+    tm = m0 + (pid % rows_in_group)
+    tn = (pid % per_group) // rows_in_group
+    rm = tm * BM + tl.arange(0, BM)
+    rn = tn * BN + tl.arange(0, BN)
+    rk = tl.arange(0, BK)
+    pa = a_ptr + rm[:, None] * s_am + rk[None, :]
+    pb = b_ptr + rk[:, None] * s_bk + rn[None, :]
+    acc = tl.zeros((BM, BN), dtype=tl.float32)
+    for k in range(0, tl.cdiv(K, BK)):
+        left = K - k * BK
+        a = tl.load(pa, mask=(rm[:, None] < M) & (rk[None, :] < left), other=0.0)
+        b = tl.load(pb, mask=(rk[:, None] < left) & (rn[None, :] < N), other=0.0)
+        acc = tl.dot(a, b, acc)
+        pa += BK
+        pb += BK * s_bk
+    acc += tl.load(bias_ptr + rn, mask=rn < N, other=0.0)[None, :] + 16.0 * tl.load(bias_ptr + N + rm, mask=rm < M, other=0.0)[:, None]
+    tl.store(c_ptr + rm[:, None] * s_cm + rn[None, :], acc.to(c_ptr.dtype.element_ty), mask=(rm[:, None] < M) & (rn[None, :] < N))

@@ -1109,22 +1109,50 @@ def test_tile_program_persistent_softmax():
     assert (y.double() - torch.softmax(x.double(), 1)).abs().max() <= 1e-5
 
 
-def test_tile_program_matmul_with_fused_activation():
-    """A 128 x 128 x 64 bf16 tile matmul with a bias per column and a leaky-relu before the store: the epilogue depends on
-    the element's position, so it runs as small-product code (operands staged in LDS in their 16-bit type)."""
+def test_gemm_epilogue_in_the_grouped_tile_order(K):
+    """The stock tutorial kernel with its activation (one-dimensional grid, tiles in groups of 8 rows, wrapped operands), and
+    a kernel in the same tile order whose epilogue adds a value per row and per column: exact on small integers."""
     import extra_kernels as X
+    g = torch.Generator(device="cpu").manual_seed(5)
+    M, N, Kd = 700, 520, 96
+    a = torch.randint(-1, 2, (M, Kd), generator=g).to(torch.bfloat16).to(DEV)
+    b = torch.randint(-1, 2, (Kd, N), generator=g).to(torch.bfloat16).to(DEV)
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+    grid = (triton.cdiv(M, 64) * triton.cdiv(N, 128),)
+    k = K.matmul_wrapped[grid](a, b, c, M, N, Kd, a.stride(0), 1, b.stride(0), 1, c.stride(0), 1, BM=64, BN=128, BK=32, GROUP_M=8, ACTIVATION="leaky_relu")
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and "epilogue" in k.function.last_kernel
+    z = a.float() @ b.float()
+    assert torch.equal(c.float(), torch.where(z >= 0, z, (z * 0.01).bfloat16().float()))
+    bias = torch.cat([torch.randint(-4, 5, (N,), generator=g), torch.randint(-2, 3, (M,), generator=g)]).float().to(DEV)
+    k = X.matmul_grouped_order_plus_bias[grid](a, b, c, bias, M, N, Kd, a.stride(0), b.stride(0), c.stride(0), BM=64, BN=128, BK=32, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and "epilogue" in k.function.last_kernel
+    assert torch.equal(c.float(), z + bias[:N][None, :] + 16.0 * bias[N:][:, None])
+
+
+def test_tile_program_matmul_with_gathered_rows_in_bf16():
+    """128 x 128 x 64 bf16 tile products whose A rows come through an index vector and whose weights are picked by a loaded
+    expert id (examples/kernels.py:expert_rows_matmul): not a dense product, so it runs as small-product code of the
+    generic family (operands staged in LDS in their 16-bit type, 32 x 32 MFMA blocks)."""
+    from triton_shared_amd.examples import kernels
     torch.manual_seed(18)
-    M, N, K = 200, 300, 150
-    a = torch.randn(M, K, device=DEV).bfloat16()
-    b = torch.randn(K, N, device=DEV).bfloat16()
-    bias = torch.randn(N, device=DEV)
-    c = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
-    k = X.matmul_leaky[(triton.cdiv(M, 128), triton.cdiv(N, 128))](a, b, c, M, N, K, a.stride(0), b.stride(0), c.stride(0), 0.01, BM=128, BN=128, BK=64,
-                                                                    ACT=2, bias_ptr=bias)
+    tokens, kd, nd, experts = 300, 150, 256, 3
+    a = torch.randn(512, kd, device=DEV).bfloat16()
+    b = torch.randn(experts, kd, nd, device=DEV).bfloat16()
+    rows = torch.randint(0, 512, (tokens,), device=DEV, dtype=torch.int32)
+    ids = torch.tensor([2, -1, 0], device=DEV, dtype=torch.int32)
+    c = torch.zeros(tokens, nd, device=DEV, dtype=torch.bfloat16)
+    k = kernels.expert_rows_matmul[(3, 2)](a, b, c, rows, ids, tokens, kd, nd, kd, kd * nd, nd, nd, BM=128, BN=128, BK=64)
     torch.cuda.synchronize()
     assert k.function.family == "tile_program"
-    want = torch.nn.functional.leaky_relu(a.double() @ b.double() + bias.double(), 0.01)
+    want = torch.zeros(tokens, nd, dtype=torch.float64, device=DEV)
+    for blk, e in enumerate(ids.tolist()):
+        if e >= 0:
+            r = slice(blk * 128, min(tokens, blk * 128 + 128))
+            want[r] = a[rows[r].long()].double() @ b[e].double()
     assert ((c.double() - want).norm() / want.norm()) <= 1e-2
+    assert torch.equal(c[128:256], torch.zeros_like(c[128:256]))          # the block whose expert id is negative is left alone
 
 
 @pytest.mark.parametrize("M,N,K,kernel", [(512, 768, 96, "gemm_dma_kernel + epilogue"), (200, 300, 150, "gemm_mfma_kernel<128x128x64> + epilogue"),
@@ -1144,6 +1172,19 @@ def test_gemm_with_fused_epilogue(M, N, K, kernel, dtype):
     assert k.function.family == "gemm" and k.function.last_kernel.startswith(kernel), k.function.last_kernel
     want = torch.nn.functional.leaky_relu(a.float() @ b.float(), 0.5)
     assert torch.equal(c.float(), want)
+    # epilogues that depend on the element's position: a bias per column before the activation, then slope * acc + what
+    # the output held (the kernels find the Triton program that owns an element through the table of tile owners)
+    bias = torch.randint(-4, 5, (N,), generator=g).float().to(DEV)
+    X.matmul_leaky[(triton.cdiv(M, 128), triton.cdiv(N, 128))](a, b, c, M, N, K, a.stride(0), b.stride(0), c.stride(0), 0.5, BM=128, BN=128, BK=64,
+                                                               ACT=2, bias_ptr=bias)
+    torch.cuda.synchronize()
+    assert torch.equal(c.float(), torch.nn.functional.leaky_relu(a.float() @ b.float() + bias, 0.5))
+    held = torch.randint(-8, 9, (M, N), generator=g).to(dtype).to(DEV)
+    c.copy_(held)
+    k = X.matmul_leaky[(triton.cdiv(M, 128), triton.cdiv(N, 128))](a, b, c, M, N, K, a.stride(0), b.stride(0), c.stride(0), 0.5, BM=128, BN=128, BK=64, ACT=3)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and k.function.last_kernel.startswith(kernel)
+    assert torch.equal(c.float(), (a.float() @ b.float()) * 0.5 + held.float())
     # a smooth activation: within the tolerance of the family
     a = torch.randn(M, K, device=DEV).to(dtype)
     b = torch.randn(K, N, device=DEV).to(dtype)

@@ -410,3 +410,19 @@ def test_reference_lit_inputs_plan_or_are_refused_for_a_known_reason(native):
     for why, n in refused.items():
         assert n <= known[why], (why, n)
     assert planned >= 335, (planned, dict(refused))
+
+
+def test_every_functional_case_plans(native):
+    """The kernels of tests/reference_cases.py and tests/core_cases.py (run on the GPU by the gpu tests, on the lane oracle by
+    test_oracle_pins.py) all get a plan here, without a GPU; the structured text survives a round trip through its reader."""
+    import core_cases
+    import core_kernels
+    import extra_kernels
+    import reference_cases
+    families = set()
+    for cases, kernels in ((reference_cases.cases(), extra_kernels), (core_cases.cases(), core_kernels)):
+        for case in cases:
+            text = native.ttir_to_structured(compile_ttir(getattr(kernels, case["kernel"]), case["sig"], case["consts"]))
+            plan_bytes, _names = native.structured_to_plan(text)
+            families.add(native.PlanHandle(plan_bytes).family)
+    assert families == {"tile_program", "fused_map"}, families

@@ -2,8 +2,8 @@
 // time into the library (kernels_gemm.hip, results stored as they are), and at run time with hipRTC when the Triton
 // kernel applies elementwise ops to the accumulator before the store (a fused activation): the generated source
 // defines TTS_GEMM_RTC (which kernel: 0 whole 256 x 256 x 32 tiles, 1 any shape in 256 x 256 tiles, 2 any shape in
-// 128 x 128 tiles), TTS_GEMM_BF16, the argument block TtsEpArgs and the functor TtsEp that maps an accumulator value to
-// the value stored, then this file's text.  Nothing here may need a host header.
+// 128 x 128 tiles), TTS_GEMM_BF16 and the functor TtsEp (a plain struct, passed as the kernel's last argument) that maps
+// an accumulator value and its position to the value stored, then this file's text.  Nothing here may need a host header.
 #pragma once
 #ifdef __HIPCC_RTC__
 typedef __INT64_TYPE__ int64_t;
@@ -69,7 +69,8 @@ __device__ __forceinline__ uint4 load8(const uint16_t *p, int valid, bool vec) {
 // fragment reads of 32 consecutive rows hit distinct banks).  B is row-major
 // [K][N] in memory; it is transposed on the way into LDS by packing the two
 // K-neighbours of every column into one 32-bit word.
-// `ep` maps an accumulator value to the value that is stored (the identity for a plain product).
+// `ep(acc, row, col)` maps an accumulator value to the value that is stored at (row, col) of C (the identity for a plain
+// product); it is only called for elements inside the problem.
 template <bool BF16, int TM, int TN, int BK, class Ep>
 __device__ __forceinline__ void gemm_mfma_body(const GemmParams &p, int tiles_m, int tiles_n, const Ep &ep) {
   constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32, PITCH = BK + 8;
@@ -188,7 +189,7 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams &p, int tiles_m,
 #pragma unroll
       for (int v = 0; v < 16; v++) {
         int64_t row = m0 + wm * TM * 32 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        if (row < p.M && col < p.N) C[row * p.ldc + col] = BF16 ? f32_to_bf16(ep(acc[i][j][v])) : f32_to_f16(ep(acc[i][j][v]));
+        if (row < p.M && col < p.N) C[row * p.ldc + col] = BF16 ? f32_to_bf16(ep(acc[i][j][v], row, col)) : f32_to_f16(ep(acc[i][j][v], row, col));
       }
     }
 }
@@ -375,7 +376,8 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
       const int64_t col = n0 + wn * 128 + j * 32 + (lane & 31) - (odd ? 1 : 0);
 #pragma unroll
       for (int v = 0; v < 16; v += 2) {
-        const f32x2_t pr = {ep(acc[i][j][v]), ep(acc[i][j][v + 1])};
+        const int64_t er = m0 + wm * 128 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), ec = n0 + wn * 128 + j * 32 + (lane & 31);
+        const f32x2_t pr = {ep(acc[i][j][v], er, ec), ep(acc[i][j][v + 1], er + 1, ec)};
         const uint32_t pk = BF16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, bf16x2_t))
                                  : __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, f16x2_t));
         const uint32_t nb = __builtin_amdgcn_mov_dpp(pk, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]: the neighbour's pair
@@ -389,8 +391,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
 }  // namespace tts_gemm_device
 
 #ifdef TTS_GEMM_RTC
-extern "C" __global__ __launch_bounds__(256) void gemm_rtc(TtsGemmParams p, int tiles_m, int tiles_n, TtsEpArgs args) {
-  const TtsEp ep{args};
+extern "C" __global__ __launch_bounds__(256) void gemm_rtc(TtsGemmParams p, int tiles_m, int tiles_n, TtsEp ep) {
 #if TTS_GEMM_RTC == 0
   tts_gemm_device::gemm_dma_body<TTS_GEMM_BF16 != 0>(p, tiles_m, tiles_n, ep);
 #elif TTS_GEMM_RTC == 1

@@ -95,7 +95,17 @@ hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **kernel_n
 // gemm_epilogue_source), `modules` the plan's three slots for the kernels compiled from it (one per tiling, filled at
 // the first launch that needs it), `args` / `args_size` the generic families' argument block.
 struct RtcModule;
-hipError_t launch_gemm_epilogue(const GemmParams &p, const std::string &epilogue, RtcModule **modules, void *args, size_t args_size,
+// The epilogue functor as the kernel receives it (the generated `struct TtsEp` has this layout): every kernel argument
+// by index, then what it takes to find the Triton program that owns an element -- tile_pid[(row / BM) * tiles_n +
+// col / BN] is that program's linear id x + gx * (y + gy * z) in the Triton launch grid (device memory).
+struct GemmEpilogueArgs {
+  void *ptr[32];
+  long long ival[32];
+  double fval[32];
+  const int *tile_pid;
+  int tiles_n, gx, gy, gz;
+};
+hipError_t launch_gemm_epilogue(const GemmParams &p, const std::string &epilogue, RtcModule **modules, const GemmEpilogueArgs &ep,
                                 hipStream_t s, const char **kernel_name, std::string *err);
 
 // C[M,N] = A[M,K] * (f16(W[K,N]) * scale[N]), A/scale/C fp16, W int8, fp32 accumulate, M <= 16

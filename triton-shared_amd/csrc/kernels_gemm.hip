@@ -20,7 +20,7 @@ namespace {
 using namespace tts_gemm_device;
 
 struct IdentityEp {
-  __device__ __forceinline__ float operator()(float x) const { return x; }
+  __device__ __forceinline__ float operator()(float x, int64_t, int64_t) const { return x; }
 };
 
 // the kernels' device code is in gemm_device.h (it is also compiled at run time, with a fused epilogue)
@@ -453,7 +453,7 @@ hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
 
 // Kernel 0: whole 256 x 256 x 32 tiles; 1: any shape in 256 x 256 tiles; 2: any shape in 128 x 128 tiles -- the choice
 // launch_gemm makes, with the kernels compiled from gemm_device.h plus the epilogue functor at the first launch.
-hipError_t launch_gemm_epilogue(const GemmParams &p, const std::string &epilogue, RtcModule **modules, void *args, size_t args_size,
+hipError_t launch_gemm_epilogue(const GemmParams &p, const std::string &epilogue, RtcModule **modules, const GemmEpilogueArgs &ep,
                                 hipStream_t s, const char **name, std::string *err) {
   static const char *names[3] = {"gemm_dma_kernel + epilogue (hipRTC)", "gemm_mfma_kernel<256x256x32> + epilogue (hipRTC)",
                                  "gemm_mfma_kernel<128x128x64> + epilogue (hipRTC)"};
@@ -472,16 +472,12 @@ hipError_t launch_gemm_epilogue(const GemmParams &p, const std::string &epilogue
   struct {
     GemmParams p;
     int tiles_m, tiles_n;
-    alignas(8) unsigned char ep[3 * 8 * 32];  // the generic families' argument block (ptr, ival, fval of 32 arguments)
+    GemmEpilogueArgs ep;  // the functor: same layout as the generated struct TtsEp
   } a;
-  if (args_size != sizeof a.ep) {
-    *err = "argument block of unexpected size";
-    return hipErrorInvalidValue;
-  }
   a.p = p;
   a.tiles_m = (int)((p.M + tile - 1) / tile);
   a.tiles_n = (int)((p.N + tile - 1) / tile);
-  std::memcpy(a.ep, args, args_size);
+  a.ep = ep;
   return rtc_launch(modules[which], a.tiles_m * a.tiles_n, 1, 1, 256, &a, sizeof a, s);
 }
 

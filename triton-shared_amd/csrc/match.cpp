@@ -826,8 +826,8 @@ bool try_tile_program(Plan &pl) {
 }
 
 // A tiled matmul whose accumulator goes through elementwise ops before the store (the tutorial kernel's fused
-// activation, test_matmul.py:98-99): the ops between the K loop and the store are taken out as an epilogue functor, and
-// what is left -- the loop, a narrowing cast, the store -- is matched as the plain product.
+// activation, test_matmul.py:98-99; a bias, a residual): what stands between the K loop and the store is taken out as an
+// epilogue functor, and what is left -- the loop, a narrowing cast, the store -- is matched as the plain product.
 static bool try_gemm_with_epilogue(Plan &pl) {
   const Program &P = pl.prog;
   int loop_at = -1, store_at = -1;
@@ -839,7 +839,8 @@ static bool try_gemm_with_epilogue(Plan &pl) {
     } else if (k == SK::Store) {
       if (store_at >= 0) return false;
       store_at = (int)i;
-    } else if (k != SK::Map && k != SK::Const && k != SK::Splat && k != SK::ScalarArg && k != SK::FromIndex) {
+    } else if (k != SK::Map && k != SK::Const && k != SK::Splat && k != SK::ScalarArg && k != SK::FromIndex && k != SK::Load && k != SK::Iota &&
+               k != SK::ExpandDims && k != SK::Broadcast) {
       return false;
     }
   }
@@ -893,7 +894,7 @@ static bool try_gemm_with_epilogue(Plan &pl) {
     std::vector<const SOp *> ops;
     for (auto &s : P.body)
       if (s.kind != SK::For && s.kind != SK::Store) ops.push_back(&s);
-    q.source = gemm_epilogue_source(P, ops, acc, out);
+    q.source = gemm_epilogue_source(P, ops, acc, out, q.k.at("BM"), q.k.at("BN"));
   } catch (const Unsupported &) {
     return false;  // not this shape of program: the other families get their turn
   }

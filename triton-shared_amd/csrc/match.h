@@ -43,7 +43,7 @@ constexpr int TILE_MAX_ARGS = 32;
 std::string tile_program_source(const Program &p);
 // Matmul family with ops between the K loop and the store: the source of the functor that applies them to one
 // accumulator value (tile_codegen.cpp), compiled at run time together with the kernels of gemm_device.h.
-std::string gemm_epilogue_source(const Program &p, const std::vector<const SOp *> &ops, int acc, int out);
+std::string gemm_epilogue_source(const Program &p, const std::vector<const SOp *> &ops, int acc, int out, int64_t BM, int64_t BN);
 
 // Normalised listing of a program's ops (no shapes, no expression ids).
 std::string signature(const Program &p);

@@ -52,6 +52,15 @@ struct Bound {
   MapNParams mapn{};
   bool empty = false;  // nothing to do (e.g. zero trip count with nothing stored)
   std::string describe;
+  // matrix products with a fused epilogue: which program owns which BM x BN tile (device memory, owned by the binding)
+  int *tile_pid = nullptr;
+  int tiles_n = 0;
+  Bound() = default;
+  Bound(const Bound &) = delete;
+  Bound &operator=(const Bound &) = delete;
+  ~Bound() {
+    if (tile_pid) (void)hipFree(tile_pid);
+  }
 };
 
 }  // namespace
@@ -241,6 +250,8 @@ void bind_layernorm(const Resolver &r, Bound &b) {
 // tiling may compute it.
 struct DenseGemm {
   int64_t M, N, K, lda, ldb, ldc;
+  std::vector<int> tile_pid;  // per BM x BN tile (row-major over the tile grid): linear id of the program that computes it
+  int tiles_n = 0;
 };
 
 DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
@@ -281,6 +292,8 @@ DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
   const int64_t tm = (d.M + BM - 1) / BM, tn = (d.N + BN - 1) / BN;
   need((int64_t)r.g[0] * r.g[1] * r.g[2] == tm * tn, "the grid does not have one program per output tile");
   std::vector<char> seen(tm * tn, 0);
+  d.tile_pid.assign(tm * tn, 0);
+  d.tiles_n = (int)tn;
   for (int z = 0; z < r.g[2]; z++)
     for (int y = 0; y < r.g[1]; y++)
       for (int x = 0; x < r.g[0]; x++) {
@@ -290,6 +303,7 @@ DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
         char &s = seen[(r0 / BM) * tn + c0 / BN];
         need(!s, "two programs compute the same output tile");
         s = 1;
+        d.tile_pid[(r0 / BM) * tn + c0 / BN] = x + r.g[0] * (y + r.g[1] * z);
         need(r.ev("a_base", e) == r0 * d.lda, "A tile offset is not row0 * lda");
         need(r.ev("b_base", e) == c0, "B tile offset is not col0");
         if (a_wraps) need(r.ev("a_wrapped", e) == r0 * d.lda, "the wrapped part of A's offset is not row0 * lda");
@@ -304,6 +318,12 @@ void bind_gemm(const Resolver &r, Bound &b) {
   GemmParams &p = b.gemm;
   p.M = d.M; p.N = d.N; p.K = d.K; p.lda = d.lda; p.ldb = d.ldb; p.ldc = d.ldc;
   p.is_bf16 = (int)r.pl.k.at("is_bf16");
+  if (!r.pl.source.empty()) {  // a fused epilogue looks up the program that owns an element
+    hipError_t e = hipMalloc((void **)&b.tile_pid, d.tile_pid.size() * sizeof(int));
+    if (e == hipSuccess) e = hipMemcpy(b.tile_pid, d.tile_pid.data(), d.tile_pid.size() * sizeof(int), hipMemcpyHostToDevice);
+    if (e != hipSuccess) throw std::runtime_error(std::string("gemm: tile table: ") + hipGetErrorString(e));
+    b.tiles_n = d.tiles_n;
+  }
   std::ostringstream os;
   os << "kernel=gemm_mfma\nM=" << p.M << "\nN=" << p.N << "\nK=" << p.K << "\nlda=" << p.lda << "\nldb=" << p.ldb
      << "\nldc=" << p.ldc << "\nbf16=" << p.is_bf16 << "\n";
@@ -535,16 +555,22 @@ tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, cons
           err = launch_gemm(p, s, &kname);
           break;
         }
-        struct { void *ptr[TILE_MAX_ARGS]; long long ival[TILE_MAX_ARGS]; double fval[TILE_MAX_ARGS]; } a{};
+        static_assert(TILE_MAX_ARGS == 32, "GemmEpilogueArgs holds 32 arguments");
+        GemmEpilogueArgs a{};
         for (int i = 0; i < n; i++) {
           if (args[i].kind == TTS_ARG_PTR) a.ptr[i] = args[i].v.ptr;
           else if (args[i].kind == TTS_ARG_INT) a.ival[i] = args[i].v.i;
           else a.fval[i] = args[i].v.f;
         }
+        a.tile_pid = b->tile_pid;
+        a.tiles_n = b->tiles_n;
+        a.gx = gx;
+        a.gy = gy;
+        a.gz = gz;
         std::string why;
         {
           std::lock_guard<std::mutex> lock(plan->mu);
-          err = launch_gemm_epilogue(p, pl.source, plan->gemm_rtc, &a, sizeof a, s, &kname, &why);
+          err = launch_gemm_epilogue(p, pl.source, plan->gemm_rtc, a, s, &kname, &why);
         }
         if (err != hipSuccess && !why.empty()) return fail(TTS_HIP_ERROR, "gemm epilogue: " + why);
         break;

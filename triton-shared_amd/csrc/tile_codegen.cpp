@@ -1386,33 +1386,43 @@ std::string tile_program_source(const Program &p) {
   return all.str();
 }
 
-// The elementwise ops a matmul kernel applies to its accumulator before the store (an activation, a scale, the
+// What a matmul kernel does to its accumulator between the K loop and the store (an activation, a bias, a residual, the
 // narrowing cast), as the functor the matrix-product kernels of gemm_device.h call on every accumulator value: `ops` are
-// the program's ops after the K loop, `acc` the loop's result, `out` the value that is stored.  The ops may read the
-// accumulator, constants and scalar kernel arguments only (nothing that depends on the element's position or the program
-// id): the kernels use a tiling of their own.  Throws Unsupported otherwise.
-std::string gemm_epilogue_source(const Program &p, const std::vector<const SOp *> &ops, int acc, int out) {
+// the program's top-level ops outside the loop, `acc` the loop's result, `out` the value that is stored, BM x BN the
+// Triton kernel's block.  Those kernels use a tiling of their own, so the functor finds the program that owns the element
+// (its ids through a table the launcher fills) and the element's indices inside that program's block, and evaluates the
+// stored value for that one element: whatever can be written out per element goes (loads of a bias row or a residual
+// block included); anything that needs other elements of the accumulator throws Unsupported.
+std::string gemm_epilogue_source(const Program &p, const std::vector<const SOp *> &ops, int acc, int out, int64_t BM, int64_t BN) {
   if ((int)p.arg_names.size() > TILE_MAX_ARGS) throw Unsupported("more than " + std::to_string(TILE_MAX_ARGS) + " kernel arguments");
   Gen g(p);
   for (const SOp *s : ops) {
-    if (s->kind != SK::Map && s->kind != SK::Const && s->kind != SK::Splat && s->kind != SK::ScalarArg && s->kind != SK::FromIndex)
-      throw Unsupported("an epilogue op that is not elementwise arithmetic on the accumulator");
-    if (s->kind == SK::Map && (s->name.rfind("tt.", 0) == 0 && s->name.rfind("tt.clampf", 0) != 0 && s->name.rfind("tt.precise", 0) != 0))
-      throw Unsupported("an epilogue op that moves elements (" + s->name + ")");
-    if (s->kind == SK::FromIndex)
-      for (EK k : {EK::Pid, EK::NProg, EK::IV, EK::Iter, EK::Result, EK::Data})
-        if (p.pool.depends_on(s->expr, k)) throw Unsupported("an epilogue value that depends on the program id or on data");
-    g.def[s->result] = s;
+    if (s->result >= 0) g.def[s->result] = s;
+    std::vector<int> es = s->acc.offsets;
+    es.insert(es.end(), s->acc.strides.begin(), s->acc.strides.end());
+    es.insert(es.end(), s->acc.dims.begin(), s->acc.dims.end());
+    es.insert(es.end(), s->acc.mods.begin(), s->acc.mods.end());
+    if (s->expr >= 0) es.push_back(s->expr);
+    for (EK k : {EK::IV, EK::Iter, EK::Result, EK::Data})
+      for (int e : es)
+        if (e >= 0 && p.pool.depends_on(e, k)) throw Unsupported("an epilogue value that depends on the K loop or on data");
   }
   g.var[acc] = "acc";
-  g.cur_i0 = g.cur_i1 = "e";  // one element: whatever is named is the element's own value
-  const std::string expr = g.at(out, "e", "e");
+  g.cur_i0 = "i0";
+  g.cur_i1 = "i1";
+  const std::string expr = g.at(out, "i0", "i1");
+  if (!g.fns.str().empty() || g.pool_bytes || g.out_bytes) throw Unsupported("an epilogue that needs more than one element at a time");
   std::string pre = TILE_PRELUDE;
   const std::string n = std::to_string(TILE_MAX_ARGS);
   for (size_t pos = 0; (pos = pre.find("%N%", pos)) != std::string::npos;) pre.replace(pos, 3, n);
   std::ostringstream all;
-  all << pre << "typedef Args TtsEpArgs;\n"
-      << "struct TtsEp {\n  TtsEpArgs p;\n  __device__ __forceinline__ float operator()(float acc) const { return " << expr << "; }\n};\n";
+  all << pre << "struct TtsEp {\n  Args p;\n  const int *tile_pid;\n  int tiles_n, gx, gy, gz;\n"
+      << "  __device__ __forceinline__ float operator()(float acc, long long row, long long col) const {\n"
+      << "    const int i0 = (int)(row % " << BM << "), i1 = (int)(col % " << BN << ");\n"
+      << "    const int q = tile_pid[(row / " << BM << ") * tiles_n + col / " << BN << "];\n"
+      << "    const long long pidx = q % gx, pidy = (q / gx) % gy, pidz = q / (gx * gy), npx = gx, npy = gy, npz = gz;\n"
+      << "    (void)i0; (void)i1; (void)pidx; (void)pidy; (void)pidz; (void)npx; (void)npy; (void)npz;\n"
+      << "    return " << expr << ";\n  }\n};\n";
   return all.str();
 }
 

@@ -101,9 +101,10 @@ def matmul_tiles(a_ptr, b_ptr, c_ptr, M, N, K,
 @triton.jit
 def matmul_wrapped(a_ptr, b_ptr, c_ptr, M, N, K,
                    s_am, s_ak, s_bk, s_bn, s_cm, s_cn,
-                   BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr, GROUP_M: tl.constexpr):
+                   BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr, GROUP_M: tl.constexpr, ACTIVATION: tl.constexpr = ""):
     """The stock tutorial form of the tiled matmul: rows of A and columns of B beyond the problem are read
-    modulo M and N instead of being masked; only K and the output carry masks."""
+    modulo M and N instead of being masked; only K and the output carry masks.  ACTIVATION="leaky_relu" fuses the
+    tutorial's activation before the cast (python/examples/test_matmul.py:98-99 in the reference)."""
     pid = tl.program_id(0)
     tiles_m = tl.cdiv(M, BM)
     tiles_n = tl.cdiv(N, BN)
@@ -128,6 +129,8 @@ def matmul_wrapped(a_ptr, b_ptr, c_ptr, M, N, K,
         acc += tl.dot(a, b)
         pa += BK * s_ak
         pb += BK * s_bk
+    if ACTIVATION == "leaky_relu":
+        acc = tl.where(acc >= 0, acc, 0.01 * acc)
     out = acc.to(c_ptr.dtype.element_ty)
     rm = tm * BM + tl.arange(0, BM)
     rn = tn * BN + tl.arange(0, BN)
