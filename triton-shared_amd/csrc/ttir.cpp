@@ -629,7 +629,6 @@ static bool single_return(Block &b, const std::vector<Type> &types, int &serial)
 
 static void inline_calls(Block &b, std::map<std::string, Callee> &callees, Renames &subst, int &serial) {
   std::vector<std::unique_ptr<Op>> out;
-  for (auto &a : b.arg_names) (void)a;
   for (auto &held : b.ops) {
     Op &op = *held;
     for (auto &o : op.operands) o = renamed(o, subst);

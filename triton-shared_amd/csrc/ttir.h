@@ -2,10 +2,11 @@
 //
 // The reference hands the Triton IR to its middle layer as text
 // (backend/compiler.py:48-67: str(mod) -> tt.mlir -> subprocess).  This backend
-// consumes the same text.  Only the subset of the MLIR custom assembly that the
-// TTIR pass list of backend/compiler.py:244-260 produces for structured kernels
-// is understood; anything else raises tts::Unsupported so the caller can refuse
-// the kernel instead of guessing.
+// consumes the same text.  What is understood: the MLIR custom assembly that the
+// TTIR pass list of backend/compiler.py:244-260 prints, and the hand-written forms
+// of the reference's conversion tests (signatures over several lines, generic-form
+// tt.reduce, loops without a type suffix); anything else raises tts::Unsupported so
+// the caller can refuse the kernel instead of guessing.
 #pragma once
 #include <cstdint>
 #include <map>
@@ -72,7 +73,9 @@ struct Func {
   Block body;
 };
 
-// Parses one module holding exactly one public tt.func.
+// Parses one module: exactly one public tt.func (the kernel) and any number of private ones, whose calls (tt.call, from
+// functions the front end kept out of line) are inlined into the kernel.  A function body that is a graph of basic
+// blocks (early returns) comes back as a tree of "cf.if" ops.
 Func parse_ttir(const std::string &text);
 
 }  // namespace tts
