@@ -434,6 +434,8 @@ class Interpreter:
         p, v = ops[0], ops[1]
         store = self.mem[p.base]
         if not isinstance(p.d, np.ndarray):
+            if len(ops) > 2 and not bool(ops[2].d):      # a scalar store under a false mask writes nothing
+                return None
             self.acc.append(("store", p.base, np.array([p.d], dtype=np.int64)))
             store[p.d] = self._narrow(np.array([v.d]), p.elem)[0]
             return None

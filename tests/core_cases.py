@@ -152,6 +152,10 @@ def cases():
         add(f"masked_load_scalar_{index}", "scalar_load_under_mask", {"src_ptr": P, "dst_ptr": P, "index": "i32", "n": "i32", "OTHER": C}, {"OTHER": -5.0}, (1,),
             lambda index=index: [sv.copy(), np.zeros(1, np.float32), index, 8], lambda a, want=want: _eq(a[1], [want]))
 
+    for flag, want in [(3, [7, -1]), (-3, [-1, 8])]:
+        add(f"masked_store_scalar_{flag}", "scalar_store_under_mask", {"dst_ptr": I, "flag": "i32", "value": "i32"}, {}, (1,),
+            lambda flag=flag: [np.full(2, -1, np.int32), flag, 7], lambda a, want=want: _eq(a[0], want))
+
     fx, fy, fz = (rng.standard_normal(256).astype(np.float32) for _ in range(3))
     fx[0], fy[0], fz[0] = np.float32(1 + 2 ** -12), np.float32(1 + 2 ** -12), np.float32(-1)     # the product's low bits survive only when fused
     add("fma", "fused_multiply_add", {"x_ptr": P, "y_ptr": P, "z_ptr": P, "out_ptr": P, "BLOCK": C}, {"BLOCK": 256}, (1,),

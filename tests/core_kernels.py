@@ -401,3 +401,9 @@ def fill_values_that_are_data(x_ptr, alt_ptr, out_ptr, n, fill, BLOCK: tl.conste
     b = tl.load(x_ptr + o, mask=o < n, other=tl.load(alt_ptr + o))
     tl.store(out_ptr + o, a)
     tl.store(out_ptr + tl.num_programs(0) * BLOCK + o, b)
+
+
+@triton.jit
+def scalar_store_under_mask(dst_ptr, flag, value):
+    tl.store(dst_ptr, value, mask=flag > 0)
+    tl.store(dst_ptr + 1, value + 1, mask=flag <= 0)
