@@ -152,6 +152,12 @@ def cases():
         add(f"masked_load_scalar_{index}", "scalar_load_under_mask", {"src_ptr": P, "dst_ptr": P, "index": "i32", "n": "i32", "OTHER": C}, {"OTHER": -5.0}, (1,),
             lambda index=index: [sv.copy(), np.zeros(1, np.float32), index, 8], lambda a, want=want: _eq(a[1], [want]))
 
+    for order in (0, 1):
+        for size in (1, 128):
+            ap = rng.standard_normal(size).astype(np.float32)
+            add(f"addptr_order{order}_size{size}", "copy_with_offsets_first", {"x_ptr": P, "y_ptr": P, "ORDER": C, "SIZE": C}, {"ORDER": order, "SIZE": size}, (1,),
+                lambda ap=ap: [ap.copy(), np.zeros(ap.size, np.float32)], lambda a, ap=ap: _eq(a[1], ap))
+
     for flag, want in [(3, [7, -1]), (-3, [-1, 8])]:
         add(f"masked_store_scalar_{flag}", "scalar_store_under_mask", {"dst_ptr": I, "flag": "i32", "value": "i32"}, {}, (1,),
             lambda flag=flag: [np.full(2, -1, np.int32), flag, 7], lambda a, want=want: _eq(a[0], want))
@@ -234,6 +240,10 @@ def cases():
         add(f"dot_fp16_acc{acc}", "dot_in_half_precision", {"a_ptr": H, "b_ptr": H, "c_ptr": P, "M": C, "N": C, "K": C, "ACC_IN": C}, {"M": 32, "N": 32, "K": 64, "ACC_IN": acc}, (1,),
             lambda: [ha.reshape(-1).copy(), hb.reshape(-1).copy(), hc.reshape(-1).copy()],
             lambda a, acc=acc: _eq(a[2].reshape(32, 32), ha.astype(np.float32) @ hb.astype(np.float32) + (hc if acc else 0)))
+    add("dot_fp16_out_fp16", "dot_accumulating_in_half", {"a_ptr": H, "b_ptr": H, "c_ptr": H, "M": C, "N": C, "K": C}, {"M": 32, "N": 32, "K": 64}, (1,),
+        lambda: [ha.reshape(-1).copy(), hb.reshape(-1).copy(), np.zeros(32 * 32, np.float16)],
+        lambda a: _eq(a[2].reshape(32, 32), (ha.astype(np.float32) @ hb.astype(np.float32)).astype(np.float16)))
+
     fx_ = rng.standard_normal(1024).astype(np.float32)
     falt = rng.standard_normal(1024).astype(np.float32)
     add("other_is_data", "fill_values_that_are_data", {"x_ptr": P, "alt_ptr": P, "out_ptr": P, "n": "i32", "fill": "i32", "BLOCK": C}, {"BLOCK": 256}, (4,),

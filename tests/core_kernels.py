@@ -407,3 +407,23 @@ def fill_values_that_are_data(x_ptr, alt_ptr, out_ptr, n, fill, BLOCK: tl.conste
 def scalar_store_under_mask(dst_ptr, flag, value):
     tl.store(dst_ptr, value, mask=flag > 0)
     tl.store(dst_ptr + 1, value + 1, mask=flag <= 0)
+
+
+@triton.jit
+def copy_with_offsets_first(x_ptr, y_ptr, ORDER: tl.constexpr, SIZE: tl.constexpr):
+    # pointer + offsets in either order; SIZE = 1 is a block of one element
+    o = tl.arange(0, SIZE)
+    if ORDER == 0:
+        tl.store(y_ptr + o, tl.load(x_ptr + o))
+    else:
+        tl.store(o + y_ptr, tl.load(o + x_ptr))
+
+
+@triton.jit
+def dot_accumulating_in_half(a_ptr, b_ptr, c_ptr, M: tl.constexpr, N: tl.constexpr, K: tl.constexpr):
+    i = tl.arange(0, M)
+    j = tl.arange(0, N)
+    k = tl.arange(0, K)
+    a = tl.load(a_ptr + i[:, None] * K + k[None, :])
+    b = tl.load(b_ptr + k[:, None] * N + j[None, :])
+    tl.store(c_ptr + i[:, None] * N + j[None, :], tl.dot(a, b, out_dtype=tl.float16))
