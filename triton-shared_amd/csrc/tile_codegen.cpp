@@ -459,6 +459,9 @@ struct Gen {
     if (a.elem == "bf16") return "up_bf16(" + ptr + ")";
     return ptr;
   }
+  static bool raw16(const SOp &o) {  // a masked load of f16 / bf16 (see the two-phase loads)
+    return (o.acc.elem == "f16" || o.acc.elem == "bf16") && (!o.acc.dims.empty() || o.acc.mask_value >= 0);
+  }
   std::string other_of(const Access &a, const std::string &i0 = "0", const std::string &i1 = "0") {
     if (a.other_value >= 0) return at(a.other_value, i0, i1);
     if (!a.has_other) return a.elem == "f64" ? "0.0" : is_float(a.elem) ? "0.f" : "(" + ctype(a.elem) + ")0";
@@ -702,6 +705,9 @@ struct Gen {
           for (size_t q = k; q < end; q++)
             if (mine_here(ops[q])) {
               os << pad() << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << (count(ls) + 255) / 256 << "];\n";
+              // a masked load of a 16-bit float keeps its raw bits until the fill loop: widening it next to the load
+              // would need the value, and with it a wait for every load before the next one is issued
+              if (raw16(ops[q])) os << pad() << "unsigned short ldr" << ops[q].result << "[" << (count(ls) + 255) / 256 << "];\n";
               any = true;
             }
           if (!any) continue;
@@ -716,7 +722,11 @@ struct Gen {
             open_element_loop(ls);
             for (auto &f : fill) {
               std::string pred, addr = address(f.first->acc, l0, l1, pred);
-              os << pad() << "if (!(" << pred << ")) " << f.second << "[n] = " << other_of(f.first->acc, l0, l1) << ";\n";
+              if (raw16(*f.first))
+                os << pad() << f.second << "[n] = (" << pred << ") ? " << (f.first->acc.elem == "f16" ? "up_f16(" : "up_bf16(") << "ldr" << f.first->result
+                   << "[n]) : " << other_of(f.first->acc, l0, l1) << ";\n";
+              else
+                os << pad() << "if (!(" << pred << ")) " << f.second << "[n] = " << other_of(f.first->acc, l0, l1) << ";\n";
             }
             close_loop();
             fill.clear();
@@ -735,7 +745,10 @@ struct Gen {
               }
               if (pred.empty()) os << pad() << name << "[n] = " << mem_read(ops[q].acc, addr) << ";\n";
               else {
-                os << pad() << "if (" << pred << ") " << name << "[n] = " << mem_read(ops[q].acc, addr) << ";\n";
+                if (raw16(ops[q]))
+                  os << pad() << "if (" << pred << ") ldr" << ops[q].result << "[n] = ((const unsigned short *)p.ptr[" << ops[q].acc.base_arg << "])[" << addr << "];\n";
+                else
+                  os << pad() << "if (" << pred << ") " << name << "[n] = " << mem_read(ops[q].acc, addr) << ";\n";
                 fill.push_back({&ops[q], name});
               }
               held[ops[q].result] = {name, ls};  // a later load of this run may be indexed by it
@@ -878,8 +891,19 @@ struct Gen {
     // operands of a 16-bit type are staged in that type (their values are exactly representable), others as fp32
     auto narrow = [](const std::string &t) { return t == "f16" || t == "bf16"; };
     const size_t a_size = narrow(A.dtype) ? 2 : 4, b_size = narrow(B.dtype) ? 2 : 4;
-    const size_t a_bytes = ((size_t)(M * K) * a_size + 15) / 16 * 16, bytes = a_bytes + (size_t)(K * N) * b_size;
-    if (bytes > 48 * 1024) no("a matrix product whose operands need " + std::to_string(bytes) + " bytes of LDS (limit 49152)");
+    if (((size_t)(M * K) * a_size + 15) / 16 * 16 + (size_t)(K * N) * b_size > 48 * 1024)
+      no("a matrix product whose operands need " + std::to_string(((size_t)(M * K) * a_size + 15) / 16 * 16 + (size_t)(K * N) * b_size) +
+         " bytes of LDS (limit 49152)");
+    // The 16-bit matrix-core path reads 16-byte fragments of 32 consecutive rows at once: rows K elements apart would
+    // fall into the same few banks (measured: more cycles of bank conflict than of anything else), so its rows are K + 8
+    // elements apart when that still fits.
+    const bool both16 = A.dtype == B.dtype && narrow(A.dtype);
+    const bool both32 = A.dtype == "f32" && B.dtype == "f32";
+    const size_t band_bytes = (size_t)32 * N * 4;
+    const bool shaped = !(!is_float(A.dtype) && !is_float(B.dtype)) && M % 32 == 0 && N % 32 == 0 && ((both16 && K % 16 == 0) || (both32 && K % 2 == 0)) &&
+                        band_bytes <= 32 * 1024;
+    const int64_t KP = (shaped && both16 && (size_t)(M + N) * (K + 8) * 2 + band_bytes <= 60 * 1024) ? K + 8 : K;  // row pitch of the staged operands
+    const size_t a_bytes = ((size_t)(M * KP) * a_size + 15) / 16 * 16, bytes = a_bytes + (size_t)(KP * N) * b_size;
     // integers (i8 x i8 -> i32 and the like): staged as 32-bit integers, multiplied and added with wrap-around
     const bool integer = !is_float(A.dtype) && !is_float(B.dtype) && !is_float(R.dtype);
     if (!integer && (!is_float(A.dtype) || !is_float(B.dtype) || !is_float(R.dtype))) no("a matrix product that mixes integers and floats");
@@ -894,18 +918,15 @@ struct Gen {
     os << pad() << staged_type(A.dtype) << " *const da" << id << " = (" << staged_type(A.dtype) << " *)pool;\n";
     os << pad() << staged_type(B.dtype) << " *const db" << id << " = (" << staged_type(B.dtype) << " *)(pool + " << a_bytes << ");\n";
     open_element_loop(A.shape);
-    os << pad() << "da" << id << "[t] = " << put(A.dtype, at(s.operands[0], idx0(A.shape), idx1(A.shape))) << ";\n";
+    os << pad() << "da" << id << "[" << (KP == K ? std::string("t") : idx0(A.shape) + " * " + std::to_string(KP) + " + " + idx1(A.shape)) << "] = "
+       << put(A.dtype, at(s.operands[0], idx0(A.shape), idx1(A.shape))) << ";\n";
     close_loop();
     // for the 16-bit matrix-core path B is staged transposed ([N][K], K contiguous), so that a lane's eight consecutive k
     // of a column are one 16-byte LDS read, as they are for A
-    const bool both16 = A.dtype == B.dtype && narrow(A.dtype);
-    const bool both32 = A.dtype == "f32" && B.dtype == "f32";
-    const size_t band_bytes = (size_t)32 * N * 4;
-    const bool mfma = !integer && M % 32 == 0 && N % 32 == 0 && ((both16 && K % 16 == 0) || (both32 && K % 2 == 0)) && band_bytes <= 32 * 1024 &&
-                      bytes + band_bytes <= 60 * 1024;
+    const bool mfma = !integer && shaped && bytes + band_bytes <= 60 * 1024;
     open_element_loop(B.shape);
     if (mfma && both16)
-      os << pad() << "db" << id << "[" << idx1(B.shape) << " * " << K << " + " << idx0(B.shape) << "] = " << put(B.dtype, at(s.operands[1], idx0(B.shape), idx1(B.shape))) << ";\n";
+      os << pad() << "db" << id << "[" << idx1(B.shape) << " * " << KP << " + " << idx0(B.shape) << "] = " << put(B.dtype, at(s.operands[1], idx0(B.shape), idx1(B.shape))) << ";\n";
     else
       os << pad() << "db" << id << "[t] = " << put(B.dtype, at(s.operands[1], idx0(B.shape), idx1(B.shape))) << ";\n";
     close_loop();
@@ -920,6 +941,10 @@ struct Gen {
       pool_bytes = std::max(pool_bytes, band_off + band_bytes);
       uses_mfma = true;
       os << pad() << "float *const dc" << id << " = (float *)(pool + " << band_off << ");\n";
+      // With few bands the band loop is unrolled, so that the slots of the result a thread fills from a band (N / 8 of
+      // them, consecutive) are known at compile time and the result stays in registers.
+      const bool unrolled_bands = M / 32 <= 8;
+      if (unrolled_bands) os << pad() << "#pragma unroll\n";
       os << pad() << "for (int br = 0; br < " << M / 32 << "; br++) {\n";
       indent++;
       os << pad() << "for (int bc = threadIdx.x >> 6; bc < " << N / 32 << "; bc += 4) {\n";
@@ -929,7 +954,7 @@ struct Gen {
       if (both16) {
         os << pad() << "for (int k0 = 0; k0 < " << K << "; k0 += 16) {\n";
         indent++;
-        os << pad() << "const u16x8_t fa = *(const u16x8_t *)&da" << id << "[row * " << K << " + k0 + 8 * kg], fb = *(const u16x8_t *)&db" << id << "[col * " << K
+        os << pad() << "const u16x8_t fa = *(const u16x8_t *)&da" << id << "[row * " << KP << " + k0 + 8 * kg], fb = *(const u16x8_t *)&db" << id << "[col * " << KP
            << " + k0 + 8 * kg];\n";
         os << pad() << "acc = " << (A.dtype == "bf16" ? "__builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fa), __builtin_bit_cast(bf16x8_t, fb)"
                                                       : "__builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, fa), __builtin_bit_cast(f16x8_t, fb)")
@@ -943,12 +968,26 @@ struct Gen {
       os << pad() << "#pragma unroll\n" << pad() << "for (int v = 0; v < 16; v++) dc" << id << "[(8 * (v >> 2) + 4 * kg + (v & 3)) * " << N << " + col] = acc[v];\n";
       indent--;
       os << pad() << "}\n" << pad() << "__syncthreads();\n";
-      open_element_loop(R.shape);
-      os << pad() << "if (" << idx0(R.shape) << " / 32 == br) " << name << "[n] = "
-         << rounded(R.dtype, "dc" + id + "[(" + idx0(R.shape) + " % 32) * " + std::to_string(N) + " + " + idx1(R.shape) + "] + " +
-                                 at(s.operands.at(2), idx0(R.shape), idx1(R.shape)))
-         << ";\n";
-      close_loop();
+      if (unrolled_bands) {
+        os << pad() << "#pragma unroll\n" << pad() << "for (int q = 0; q < " << N / 8 << "; q++) {\n";
+        indent++;
+        os << pad() << "const int n = br * " << N / 8 << " + q;\n" << pad() << "const int t = threadIdx.x + 256 * n;\n";
+        cur_i0 = idx0(R.shape);
+        cur_i1 = idx1(R.shape);
+        map_vars(R.shape);
+        os << pad() << name << "[n] = "
+           << rounded(R.dtype, "dc" + id + "[(" + idx0(R.shape) + " % 32) * " + std::to_string(N) + " + " + idx1(R.shape) + "] + " +
+                                   at(s.operands.at(2), idx0(R.shape), idx1(R.shape)))
+           << ";\n";
+        close_loop();
+      } else {
+        open_element_loop(R.shape);
+        os << pad() << "if (" << idx0(R.shape) << " / 32 == br) " << name << "[n] = "
+           << rounded(R.dtype, "dc" + id + "[(" + idx0(R.shape) + " % 32) * " + std::to_string(N) + " + " + idx1(R.shape) + "] + " +
+                                   at(s.operands.at(2), idx0(R.shape), idx1(R.shape)))
+           << ";\n";
+        close_loop();
+      }
       os << pad() << "__syncthreads();\n";
       indent--;
       os << pad() << "}\n";
