@@ -459,7 +459,7 @@ struct Gen {
     if (a.elem == "bf16") return "up_bf16(" + ptr + ")";
     return ptr;
   }
-  static bool raw16(const SOp &o) {  // a masked load of f16 / bf16 (see the two-phase loads)
+  static bool raw16(const SOp &o) {  // a masked load of f16 / bf16: widened in the fill loop (see the two-phase loads)
     return (o.acc.elem == "f16" || o.acc.elem == "bf16") && (!o.acc.dims.empty() || o.acc.mask_value >= 0);
   }
   std::string other_of(const Access &a, const std::string &i0 = "0", const std::string &i1 = "0") {
@@ -705,9 +705,6 @@ struct Gen {
           for (size_t q = k; q < end; q++)
             if (mine_here(ops[q])) {
               os << pad() << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << (count(ls) + 255) / 256 << "];\n";
-              // a masked load of a 16-bit float keeps its raw bits until the fill loop: widening it next to the load
-              // would need the value, and with it a wait for every load before the next one is issued
-              if (raw16(ops[q])) os << pad() << "unsigned short ldr" << ops[q].result << "[" << (count(ls) + 255) / 256 << "];\n";
               any = true;
             }
           if (!any) continue;
@@ -723,8 +720,8 @@ struct Gen {
             for (auto &f : fill) {
               std::string pred, addr = address(f.first->acc, l0, l1, pred);
               if (raw16(*f.first))
-                os << pad() << f.second << "[n] = (" << pred << ") ? " << (f.first->acc.elem == "f16" ? "up_f16(" : "up_bf16(") << "ldr" << f.first->result
-                   << "[n]) : " << other_of(f.first->acc, l0, l1) << ";\n";
+                os << pad() << f.second << "[n] = (" << pred << ") ? " << (f.first->acc.elem == "f16" ? "up_f16(" : "up_bf16(") << "(unsigned short)__float_as_uint("
+                   << f.second << "[n])) : " << other_of(f.first->acc, l0, l1) << ";\n";
               else
                 os << pad() << "if (!(" << pred << ")) " << f.second << "[n] = " << other_of(f.first->acc, l0, l1) << ";\n";
             }
@@ -745,8 +742,10 @@ struct Gen {
               }
               if (pred.empty()) os << pad() << name << "[n] = " << mem_read(ops[q].acc, addr) << ";\n";
               else {
-                if (raw16(ops[q]))
-                  os << pad() << "if (" << pred << ") ldr" << ops[q].result << "[n] = ((const unsigned short *)p.ptr[" << ops[q].acc.base_arg << "])[" << addr << "];\n";
+                if (raw16(ops[q]))  // the raw bits, in the register that will hold the value: widening them here would need the
+                                    // loaded value, and with it a wait for every load before the next one is issued
+                  os << pad() << "if (" << pred << ") " << name << "[n] = __uint_as_float(((const unsigned short *)p.ptr[" << ops[q].acc.base_arg << "])[" << addr
+                     << "]);\n";
                 else
                   os << pad() << "if (" << pred << ") " << name << "[n] = " << mem_read(ops[q].acc, addr) << ";\n";
                 fill.push_back({&ops[q], name});
