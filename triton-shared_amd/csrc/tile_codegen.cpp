@@ -1214,6 +1214,8 @@ struct Gen {
         const size_t sz = held_bytes(val(s.operands[j]).dtype);
         os << pad() << Tn[j] << " *const wp" << id << "_" << j << " = (" << Tn[j] << " *)(pool + " << off << ");\n";
         off = (off + slots * 4 * sz + 15) / 16 * 16;
+        os << pad() << Tn[j] << " *const wq" << id << "_" << j << " = (" << Tn[j] << " *)(pool + " << off << ");\n";  // what precedes each piece in its line
+        off = (off + slots * 4 * sz + 15) / 16 * 16;
         decl << "  __shared__ " << Tn[j] << " out" << id << "_" << j << "[" << T << "];\n";
         out_bytes += (T * sz + 15) / 16 * 16;
       }
@@ -1236,16 +1238,48 @@ struct Gen {
       indent++;
       os << pad() << "const int t = threadIdx.x + 256 * n;\n";
       for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << " = " << at(s.operands[j], i0, i1) << ";\n";
-      os << pad() << "#pragma unroll\n" << pad() << "for (int d = 1; d < 64; d <<= 1) {\n";
-      indent++;
-      for (size_t j = 0; j < k; j++) os << pad() << "const " << Tn[j] << " ot" << j << " = " << shfl(j, "acc" + std::to_string(j)) << ";\n";
-      os << pad() << "if ((threadIdx.x & 63) >= d) " << fname << "(" << list("ot", "") << ", " << list("acc", "") << ", " << list("acc", "") << ");\n";
-      indent--;
-      os << pad() << "}\n";
+      bool all32 = true;  // 32-bit values move between lanes inside the ALU (DPP); others go through the LDS crossbar
+      for (size_t j = 0; j < k; j++) all32 = all32 && (Tn[j] == "float" || Tn[j] == "int");
+      if (all32) {
+        // rows of 16 lanes: shifts by 1, 2, 4, 8 inside a row; then lane 15 of a row to the next row (rows 1 and 3), then
+        // lane 31 to the upper half -- the wavefront's inclusive scan in six steps, the earlier element always on the left
+        static const struct { const char *ctrl, *rows, *cond; } steps[6] = {
+            {"0x111", "0xF", "(threadIdx.x & 15) >= 1"}, {"0x112", "0xF", "(threadIdx.x & 15) >= 2"}, {"0x114", "0xF", "(threadIdx.x & 15) >= 4"},
+            {"0x118", "0xF", "(threadIdx.x & 15) >= 8"}, {"0x142", "0xA", "(threadIdx.x & 16) != 0"},   {"0x143", "0xC", "(threadIdx.x & 32) != 0"}};
+        for (const auto &st : steps) {
+          os << pad() << "{\n";
+          indent++;
+          for (size_t j = 0; j < k; j++)
+            os << pad() << "const " << Tn[j] << " ot" << j << " = " << (Tn[j] == "float" ? "TTS_DPP_F(acc" : "TTS_DPP_I(acc") << j << ", " << st.ctrl << ", " << st.rows << ");\n";
+          os << pad() << "if (" << st.cond << ") " << fname << "(" << list("ot", "") << ", " << list("acc", "") << ", " << list("acc", "") << ");\n";
+          indent--;
+          os << pad() << "}\n";
+        }
+      } else {
+        os << pad() << "#pragma unroll\n" << pad() << "for (int d = 1; d < 64; d <<= 1) {\n";
+        indent++;
+        for (size_t j = 0; j < k; j++) os << pad() << "const " << Tn[j] << " ot" << j << " = " << shfl(j, "acc" + std::to_string(j)) << ";\n";
+        os << pad() << "if ((threadIdx.x & 63) >= d) " << fname << "(" << list("ot", "") << ", " << list("acc", "") << ", " << list("acc", "") << ");\n";
+        indent--;
+        os << pad() << "}\n";
+      }
       for (size_t j = 0; j < k; j++) os << pad() << "sc" << id << "_" << j << "[n] = acc" << j << ";\n";
       os << pad() << "if ((threadIdx.x & 63) == 63) { ";
       for (size_t j = 0; j < k; j++) os << "wp" << id << "_" << j << "[n * 4 + (threadIdx.x >> 6)] = acc" << j << "; ";
       os << "}\n";
+      indent--;
+      os << pad() << "}\n" << pad() << "__syncthreads();\n";
+      // one thread per piece folds the totals of the pieces before it in its line (in piece order), once for the workgroup
+      os << pad() << "for (int q = threadIdx.x; q < " << slots * 4 << "; q += 256) {\n";
+      indent++;
+      os << pad() << "const int first = (q / " << LQ * 4 << ") * " << LQ * 4 << ";\n";
+      os << pad() << "if (q > first) {\n";
+      indent++;
+      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " carry" << j << " = wp" << id << "_" << j << "[first];\n";
+      os << pad() << "for (int i = first + 1; i < q; i++) " << fname << "(" << list("carry", "") << ", " << list("wp" + id + "_", "[i]") << ", " << list("carry", "") << ");\n";
+      for (size_t j = 0; j < k; j++) os << pad() << "wq" << id << "_" << j << "[q] = carry" << j << ";\n";
+      indent--;
+      os << pad() << "}\n";
       indent--;
       os << pad() << "}\n" << pad() << "__syncthreads();\n";
       os << pad() << "#pragma unroll\n" << pad() << "for (int n = 0; n < " << slots << "; n++) {\n";
@@ -1253,13 +1287,7 @@ struct Gen {
       os << pad() << "const int t = threadIdx.x + 256 * n;\n";
       os << pad() << "const int first = (n / " << LQ << ") * " << LQ * 4 << ", pieces = (n % " << LQ << ") * 4 + (threadIdx.x >> 6);\n";
       for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " res" << j << " = sc" << id << "_" << j << "[n];\n";
-      os << pad() << "if (pieces > 0) {\n";
-      indent++;
-      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " carry" << j << " = wp" << id << "_" << j << "[first];\n";
-      os << pad() << "for (int i = 1; i < pieces; i++) " << fname << "(" << list("carry", "") << ", " << list("wp" + id + "_", "[first + i]") << ", " << list("carry", "") << ");\n";
-      os << pad() << fname << "(" << list("carry", "") << ", " << list("sc" + id + "_", "[n]") << ", " << list("res", "") << ");\n";
-      indent--;
-      os << pad() << "}\n";
+      os << pad() << "if (pieces > 0) " << fname << "(" << list("wq" + id + "_", "[first + pieces]") << ", " << list("sc" + id + "_", "[n]") << ", " << list("res", "") << ");\n";
       for (size_t j = 0; j < k; j++) os << pad() << "out" << id << "_" << j << "[t] = res" << j << ";\n";
       indent--;
       os << pad() << "}\n" << pad() << "__syncthreads();\n";
@@ -1386,6 +1414,8 @@ __device__ inline unsigned short down_bf16(float f) {
 }
 __device__ inline float maximum_f(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
 __device__ inline float minimum_f(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
+#define TTS_DPP_I(v, ctrl, rows) __builtin_amdgcn_update_dpp((int)(v), (int)(v), ctrl, rows, 0xF, false)
+#define TTS_DPP_F(v, ctrl, rows) __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), ctrl, rows, 0xF, false))
 __device__ inline double maximum_d(double a, double b) { return (a != a || b != b) ? __builtin_nan("") : fmax(a, b); }
 __device__ inline double minimum_d(double a, double b) { return (a != a || b != b) ? __builtin_nan("") : fmin(a, b); }
 __device__ inline long long smin(long long a, long long b) { return a < b ? a : b; }
