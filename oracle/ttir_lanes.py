@@ -15,7 +15,9 @@ brute-force pin for what the reference derives symbolically:
 
 Beyond the five hot-path kernels it also runs what the generic kernel family takes: tt.reduce / tt.scan with any
 combiner region (argmin / argmax, ConversionPatterns.hpp:1443-1769), integer, bit and conversion ops, extern functions
-by symbol name, tt.trans / tt.reshape / tt.cat / tt.join / tt.split, cf.cond_br trees (early return) and scf.if.  Pins, all in
+by symbol name, tt.trans / tt.reshape / tt.cat / tt.join / tt.split, cf.cond_br trees (early return), scf.if, and block
+pointers as ops (tt.make_tensor_ptr / tt.advance / boundaryCheck + padding, with the language's `0 <= index < shape` per
+checked dimension; pinned by running the same kernels with the frontend's rewrite to plain pointers).  Pins, all in
 tests/test_oracle_pins.py: the reference's golden tensors (python/examples/test_modulo.py, test_mask.py,
 test_gather_scatter.py and the 21 cases of tests/reference_cases.py), numpy closed forms per op class
 (tests/op_zoo.py, including an independent Philox for tl.rand), float64 formulas for the float kernels.
@@ -61,6 +63,13 @@ def parse_type(s):
         t = Ty(dims, e.elem, e.ptr)
         t._is_tensor = True
         return t
+    if s.startswith("<tensor<"):                     # short form of a block pointer type in the custom assembly
+        s = "!tt.ptr" + s
+    if s.startswith("!tt.ptr<tensor<"):
+        inner = parse_type(s[8:-1])
+        t = Ty(inner.shape, inner.elem, True)
+        t._is_tensor = True
+        return t
     if s.startswith("!tt.ptr<"):
         return Ty((), s[8:-1].split(",")[0].strip(), True)
     return Ty((), s, False)
@@ -88,6 +97,24 @@ def round_bf16(x):
     r = ((u + 0x7fff + ((u >> 16) & 1)) >> 16) << 16
     r = np.where(nan, (u | 0x400000) & 0xffff0000, r).astype(np.uint32)
     return r.view(np.float32)
+
+
+class BlockPtr:
+    """What tt.make_tensor_ptr makes: element (i0, i1, ...) of the block is the parent's element offs[d] + i_d per dimension."""
+    __slots__ = ("origin", "shape", "strides", "offs", "block")
+
+    def __init__(self, origin, shape, strides, offs, block):
+        self.origin, self.shape, self.strides, self.offs, self.block = origin, shape, strides, offs, block
+
+    def lanes(self, checked):
+        idx = np.full(self.block, self.origin, dtype=np.int64)
+        mask = np.ones(self.block, dtype=bool)
+        for d, (n, o, s, ext) in enumerate(zip(self.block, self.offs, self.strides, self.shape)):
+            i = (o + np.arange(n, dtype=np.int64)).reshape([-1 if k == d else 1 for k in range(len(self.block))])
+            idx = idx + i * s
+            if d in checked:
+                mask = mask & (i >= 0) & (i < ext)
+        return idx, mask
 
 
 class Val:
@@ -392,6 +419,15 @@ class Interpreter:
             if isinstance(p.d, np.ndarray):
                 return Val(p.d + o.d.astype(np.int64), p.elem, p.base)
             return Val(int(p.d) + int(o.d), p.elem, p.base)
+        if name == "tt.make_tensor_ptr":
+            t = tys[-1]
+            r = len(t.shape)
+            ints = [int(o.d) for o in ops[1:]]
+            return Val(BlockPtr(int(ops[0].d), ints[:r], ints[r:2 * r], ints[2 * r:], tuple(t.shape)), t.elem, ops[0].base)
+        if name == "tt.advance":
+            b = ops[0].d
+            moved = [o + int(d.d) for o, d in zip(b.offs, ops[1:])]
+            return Val(BlockPtr(b.origin, b.shape, b.strides, moved, b.block), ops[0].elem, ops[0].base)
         if name == "tt.load":
             return self._load(ops)
         if name == "tt.store":
@@ -411,9 +447,25 @@ class Interpreter:
     def _storage(self, arg, elem):
         return self.mem[arg]
 
+    def _checked_dims(self):
+        m = re.search(r"boundaryCheck = array<i32(?:: ([\d, ]*))?>", self._last_line)
+        return [int(x) for x in m.group(1).split(",")] if m and m.group(1) else []
+
     def _load(self, ops):
         p = ops[0]
         store = self.mem[p.base]
+        if isinstance(p.d, BlockPtr):
+            idx, mask = p.d.lanes(self._checked_dims())
+            pad = re.search(r"padding = (\d)", self._last_line)
+            fill = np.nan if pad and pad.group(1) == "2" else 0
+            out = np.full(idx.shape, fill, dtype=_NP[p.elem])
+            sel = idx[mask]
+            self.acc.append(("load", p.base, np.sort(sel.ravel())))
+            if sel.size:
+                if sel.min() < 0 or sel.max() >= store.size:
+                    raise IndexError(f"block load outside argument {p.base}: [{sel.min()}, {sel.max()}] of {store.size}")
+                out[mask] = self._widen(store[sel], p.elem)
+            return Val(out, p.elem)
         if not isinstance(p.d, np.ndarray):
             if len(ops) > 1 and not bool(ops[1].d):      # a scalar load under a false mask reads nothing
                 return Val(ops[2].d if len(ops) > 2 else _NP[p.elem](0), p.elem)
@@ -433,6 +485,15 @@ class Interpreter:
     def _store(self, ops):
         p, v = ops[0], ops[1]
         store = self.mem[p.base]
+        if isinstance(p.d, BlockPtr):
+            idx, mask = p.d.lanes(self._checked_dims())
+            sel = idx[mask]
+            self.acc.append(("store", p.base, np.sort(sel.ravel())))
+            if sel.size:
+                if sel.min() < 0 or sel.max() >= store.size:
+                    raise IndexError(f"block store outside argument {p.base}")
+                store[sel] = self._narrow(np.asarray(v.d)[mask], p.elem)
+            return None
         if not isinstance(p.d, np.ndarray):
             if len(ops) > 2 and not bool(ops[2].d):      # a scalar store under a false mask writes nothing
                 return None

@@ -191,6 +191,23 @@ def block_ptr_affine(x_ptr, y_ptr, n_rows, n_cols, s0, s1, BR: tl.constexpr, BC:
 
 
 @triton.jit
+def block_ptr_matmul(a_ptr, b_ptr, c_ptr, M, N, K, sam, sbk, scm, BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr, PAD: tl.constexpr):
+    # C = A @ B with both operands and the result behind block pointers that advance along K (the tutorial's block-pointer
+    # product, test/Conversion/TritonToStructured/block_ptr_advance.mlir's shape); PAD picks the padding of the A tiles
+    pa = tl.make_block_ptr(base=a_ptr, shape=[M, K], strides=[sam, 1], offsets=[tl.program_id(0) * BM, 0], block_shape=[BM, BK], order=[1, 0])
+    pb = tl.make_block_ptr(base=b_ptr, shape=[K, N], strides=[sbk, 1], offsets=[0, tl.program_id(1) * BN], block_shape=[BK, BN], order=[1, 0])
+    acc = tl.zeros([BM, BN], dtype=tl.float32)
+    for _ in range(0, tl.cdiv(K, BK)):
+        a = tl.load(pa, boundary_check=(0, 1), padding_option=PAD)
+        b = tl.load(pb, boundary_check=(0, 1), padding_option="zero")
+        acc = tl.dot(a, b, acc)
+        pa = tl.advance(pa, [0, BK])
+        pb = tl.advance(pb, [BK, 0])
+    pc = tl.make_block_ptr(base=c_ptr, shape=[M, N], strides=[scm, 1], offsets=[tl.program_id(0) * BM, tl.program_id(1) * BN], block_shape=[BM, BN], order=[1, 0])
+    tl.store(pc, acc, boundary_check=(0, 1))
+
+
+@triton.jit
 def block_ptr_row_walk(x_ptr, y_ptr, n_rows, n_cols, s0, BR: tl.constexpr, BC: tl.constexpr):
     # one program per row block walks the columns with tl.advance
     px = tl.make_block_ptr(base=x_ptr, shape=[n_rows, n_cols], strides=[s0, 1], offsets=[tl.program_id(0) * BR, 0],

@@ -517,6 +517,48 @@ def test_tile_program_block_pointers():
     assert torch.equal(y, x * 0.5)
 
 
+def test_tile_program_block_pointer_ops():
+    """The same kernels with tt.make_tensor_ptr / tt.advance kept as ops (raw_block_pointers=True): a block pointer is a
+    structured access whose boundaryCheck dimensions are cut at the parent tensor's extent, loop-carried ones carry their
+    position.  Checked on test_load_2d_tensor_block.py's expectation, exact integer-valued products and the lane interpreter."""
+    import extra_kernels as X
+    from test_planner import compile_ttir
+    from oracle import ttir_lanes
+    for rows, cols, BR, BC in [(512, 256, 4, 2), (37, 50, 16, 32)]:
+        x = torch.arange(0, rows * cols, dtype=torch.float32, device=DEV).reshape(rows, cols)
+        y = torch.full((rows, cols), -1.0, device=DEV)
+        k = X.block_ptr_affine[(triton.cdiv(rows, BR), triton.cdiv(cols, BC))](x, y, rows, cols, x.stride(0), x.stride(1), BR=BR, BC=BC, raw_block_pointers=True)
+        torch.cuda.synchronize()
+        assert k.function.family == "tile_program" and "tt.make_tensor_ptr" in k.asm["ttir"]
+        assert torch.equal(y, 2 * x + 1)
+    x = torch.randn(21, 100, device=DEV)
+    y = torch.zeros(21, 100, device=DEV)
+    k = X.block_ptr_row_walk[(triton.cdiv(21, 8),)](x, y, 21, 100, x.stride(0), BR=8, BC=32, raw_block_pointers=True)
+    torch.cuda.synchronize()
+    assert "tt.advance" in k.asm["ttir"] and torch.equal(y, x * 0.5)
+    g = torch.Generator(device="cpu").manual_seed(3)
+    sig = {"a_ptr": "*bf16", "b_ptr": "*bf16", "c_ptr": "*fp32", "M": "i32", "N": "i32", "K": "i32", "sam": "i32", "sbk": "i32",
+           "scm": "i32", "BM": "constexpr", "BN": "constexpr", "BK": "constexpr", "PAD": "constexpr"}
+    for pad, (M, N, Kd), (BM, BN, BK) in [("zero", (200, 150, 72), (64, 64, 32)), ("nan", (130, 70, 64), (64, 64, 32)), ("nan", (40, 50, 24), (32, 32, 16))]:
+        a = torch.randint(-2, 3, (M, Kd), generator=g).to(torch.bfloat16).to(DEV)
+        b = torch.randint(-2, 3, (Kd, N), generator=g).to(torch.bfloat16).to(DEV)
+        c = torch.full((M, N), -7.0, device=DEV)
+        grid = (triton.cdiv(M, BM), triton.cdiv(N, BN))
+        k = X.block_ptr_matmul[grid](a, b, c, M, N, Kd, a.stride(0), b.stride(0), c.stride(0), BM=BM, BN=BN, BK=BK, PAD=pad, raw_block_pointers=True)
+        torch.cuda.synchronize()
+        assert k.function.family == "tile_program" and "tt.make_tensor_ptr" in k.asm["ttir"]
+        if Kd % BK == 0 or pad == "zero":
+            assert torch.equal(c, a.float() @ b.float())
+        else:
+            assert torch.isnan(c).all()
+        if M * N <= 4096:
+            ttir = compile_ttir(X.block_ptr_matmul, sig, {"BM": BM, "BN": BN, "BK": BK, "PAD": pad}, raw_block_pointers=True)
+            mem = {0: a.view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1).copy(), 1: b.view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1).copy(),
+                   2: np.full(M * N, -7, np.float32)}
+            ttir_lanes.Interpreter(ttir).run(grid, [None, None, None, M, N, Kd, Kd, N, N], mem)
+            assert np.array_equal(mem[2].reshape(M, N), c.cpu().numpy(), equal_nan=True)
+
+
 def test_tile_program_in_place_swap():
     import extra_kernels as X
     torch.manual_seed(0)

@@ -22,7 +22,7 @@ def accesses(structured):
     return out
 
 
-def compile_ttir(fn, sig, consts):
+def compile_ttir(fn, sig, consts, **opts):
     import os
     import triton
     from triton.backends.compiler import GPUTarget
@@ -38,7 +38,7 @@ def compile_ttir(fn, sig, consts):
     from triton._C.libtriton import ir
     ctx = ir.context()
     ir.load_dialects(ctx)
-    options = backend.parse_options({})
+    options = backend.parse_options(opts)
     mod = src.make_ir(target, options, backend.get_codegen_implementation(options), backend.get_module_map(), ctx)
     return str(backend.make_ttir(mod, {}, options))
 
@@ -385,7 +385,6 @@ def test_reference_lit_inputs_plan_or_are_refused_for_a_known_reason(native):
         "operation tensor.empty": 9,                              # tensor dialect ops written by hand into triton_assert.mlir
         "tt.func with results is not a kernel": 6,
         "tile_program: a loop-carried block value of more than 32768 elements": 3,   # 256 x 256 accumulators in one program (kernel-05-layer-norm-dwdb.mlir)
-        "unsupported type '<tensor<": 8,                          # block pointers: the front end pass list rewrites them before this stage
         "tile_program: the reductions of this program need": 4,
         "tile_program: elementwise op extern.some_symbol": 3,     # the reference refuses it too (unsupported_extern_elementwise.mlir)
         "pointer-valued operation": 10,                           # int_to_ptr / bitcast / cat / select on pointers (the reference's TritonToPtr fallback)
@@ -409,7 +408,38 @@ def test_reference_lit_inputs_plan_or_are_refused_for_a_known_reason(native):
                 refused[why] += 1
     for why, n in refused.items():
         assert n <= known[why], (why, n)
-    assert planned >= 335, (planned, dict(refused))
+    assert planned >= 343, (planned, dict(refused))
+
+
+def test_block_pointer_ops_plan_and_agree_with_the_frontend_rewrite(native):
+    """tt.make_tensor_ptr / tt.advance / boundaryCheck + padding as ops (raw_block_pointers=True keeps them; the lit inputs
+    block_ptr_advance.mlir, block_ptr_complex_offset.mlir, make_tensor_ptr*.mlir hold the same forms): the program plans,
+    and the lane interpreter gives the same memory image for the raw ops as for what the frontend's rewrite to plain
+    pointer arithmetic makes of the same kernel - which pins the interpreter's reading of the ops on the frontend's."""
+    import numpy as np
+    import extra_kernels as X
+    from oracle import ttir_lanes
+    sig = {"a_ptr": "*bf16", "b_ptr": "*bf16", "c_ptr": "*fp32", "M": "i32", "N": "i32", "K": "i32", "sam": "i32", "sbk": "i32",
+           "scm": "i32", "BM": "constexpr", "BN": "constexpr", "BK": "constexpr", "PAD": "constexpr"}
+    rng = np.random.default_rng(1)
+    for pad, (M, N, K) in [("zero", (40, 50, 24)), ("nan", (40, 50, 32)), ("nan", (33, 20, 24))]:
+        a = (rng.integers(-2, 3, M * K).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        b = (rng.integers(-2, 3, K * N).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        images = []
+        for raw in (False, True):
+            ttir = compile_ttir(X.block_ptr_matmul, sig, {"BM": 32, "BN": 32, "BK": 16, "PAD": pad}, raw_block_pointers=raw)
+            assert ("tt.make_tensor_ptr" in ttir) == raw and ("tt.advance" in ttir) == raw
+            plan = native.structured_to_plan(native.ttir_to_structured(ttir))[0]
+            assert plan.startswith(b"tts.plan 1 family=tile_program")
+            c = np.full(M * N, -7, np.float32)
+            ttir_lanes.Interpreter(ttir).run((2, 2), [None, None, None, M, N, K, K, N, N], {0: a.copy(), 1: b.copy(), 2: c})
+            images.append(c)
+        assert np.array_equal(images[0], images[1], equal_nan=True)
+        if K % 16 == 0:          # no padding inside the products: the plain product, NaN padding or not
+            want = (a.astype(np.uint32) << 16).view(np.float32).reshape(M, K) @ (b.astype(np.uint32) << 16).view(np.float32).reshape(K, N)
+            assert np.array_equal(images[1].reshape(M, N), want)
+        elif pad == "nan":       # K tiles stick out of A: NaN-padded columns meet zero-padded rows of B, NaN everywhere
+            assert np.isnan(images[1]).all()
 
 
 def test_every_functional_case_plans(native):

@@ -77,6 +77,9 @@ class HIPOptions:
     launch_cooperative_grid: bool = False
     instrumentation_mode: str = ""
     backend_name: str = BACKEND_NAME
+    # True: tl.make_block_ptr / tl.advance reach the planner as tt.make_tensor_ptr / tt.advance ops instead of being
+    # rewritten to plain pointer arithmetic first (the default, and what the reference's pass list does)
+    raw_block_pointers: bool = os.environ.get("TTS_RAW_BLOCK_POINTERS", "0") == "1"
 
     def hash(self):
         key = "_".join(f"{k}-{v}" for k, v in sorted(self.__dict__.items()))
@@ -113,7 +116,8 @@ class HIPBackend(BaseBackend):
         pm = ir.pass_manager(mod.context)
         pm.enable_debug()
         passes.common.add_inliner(pm)
-        passes.ttir.add_rewrite_tensor_pointer(pm)
+        if not options.raw_block_pointers:
+            passes.ttir.add_rewrite_tensor_pointer(pm)
         passes.ttir.add_rewrite_tensor_descriptor_to_pointer(pm)
         passes.common.add_canonicalizer(pm)
         passes.ttir.add_combine(pm)

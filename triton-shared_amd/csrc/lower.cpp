@@ -38,6 +38,9 @@ struct PtrState {   // PtrAnalysis.h:52-129, structured fields only
   // (PtrState::shape, PtrAnalysis.h:52-129); -1 = the dimension does not wrap.  The address
   // contribution of dim d at index j is (offsets[d] + j * strides[d]) mod mods[d].
   std::vector<int> mods;
+  // block pointers (tt.make_tensor_ptr) only: the extent of the parent tensor and the block's current position in
+  // it, per dimension, in elements; a load or store with boundaryCheck on a dimension keeps indices below the extent
+  std::vector<int> bshape, boff;
   size_t rank() const { return sizes.size(); }
   bool has_mod() const {
     for (int m : mods)
@@ -357,6 +360,37 @@ class Lowerer {
         s.offsets.push_back(i == 0 ? s.scalar : c64(0));
         s.sizes.push_back(d.type.shape[i]);
         s.strides.push_back(c64(0));
+      }
+      return s;
+    }
+    if (op.name == "tt.make_tensor_ptr") {  // :1105-1160 (base, shape, strides, offsets; the order attribute is a layout hint)
+      size_t r = d.type.shape.size();
+      if (!d.type.block || op.operands.size() != 1 + 3 * r)
+        throw Unsupported("tt.make_tensor_ptr with " + std::to_string(op.operands.size()) + " operands for rank " + std::to_string(r));
+      PtrState b = visit(op.operands[0]);
+      if (b.source < 0 || b.rank() != 0) throw Unsupported("tt.make_tensor_ptr whose base is not a scalar pointer");
+      s.source = b.source;
+      for (size_t i = 0; i < r; i++) {
+        int shape = P.pool.to_index(int_of(op.operands[1 + i]));
+        int stride = P.pool.to_index(int_of(op.operands[1 + r + i]));
+        int off = P.pool.to_index(int_of(op.operands[1 + 2 * r + i]));
+        s.sizes.push_back(d.type.shape[i]);
+        s.strides.push_back(stride);
+        s.offsets.push_back(P.pool.bin(EK::Mul, off, stride));
+        s.bshape.push_back(shape);
+        s.boff.push_back(off);
+      }
+      if (b.scalar >= 0) s.offsets[0] = P.pool.bin(EK::Add, s.offsets[0], P.pool.to_index(b.scalar));
+      s.pad_mods();
+      return s;
+    }
+    if (op.name == "tt.advance") {  // :1162-1198
+      s = visit(op.operands[0]);
+      if (s.boff.size() != s.rank() || op.operands.size() != 1 + s.rank()) throw Unsupported("tt.advance on something that is not a block pointer");
+      for (size_t i = 0; i < s.rank(); i++) {
+        int delta = P.pool.to_index(int_of(op.operands[1 + i]));
+        s.boff[i] = P.pool.bin(EK::Add, s.boff[i], delta);
+        s.offsets[i] = P.pool.bin(EK::Add, s.offsets[i], P.pool.bin(EK::Mul, delta, s.strides[i]));
       }
       return s;
     }
@@ -698,8 +732,74 @@ class Lowerer {
     }
   }
 
+  // boundaryCheck = array<i32: d, ...> of a block-pointer access: per checked dimension, the count of indices that stay
+  // below the parent tensor's extent (the upper bound only, a count from the block's first index as for every mask)
+  void boundary_dims(const Op &op, const PtrState &st, Access &a) {
+    auto it = op.attrs.find("boundaryCheck");
+    if (it == op.attrs.end()) return;
+    std::string in = it->second;
+    size_t colon = in.find(':');
+    if (colon == std::string::npos) return;  // array<i32>: nothing checked
+    std::vector<bool> checked(st.rank(), false);
+    bool any = false;
+    for (size_t p = colon + 1; p < in.size();) {
+      if (!isdigit((unsigned char)in[p])) { p++; continue; }
+      size_t q = p;
+      while (q < in.size() && isdigit((unsigned char)in[q])) q++;
+      size_t dim = std::stoul(in.substr(p, q - p));
+      if (dim >= st.rank()) throw Unsupported("boundaryCheck names dimension " + std::to_string(dim));
+      checked[dim] = any = true;
+      p = q;
+    }
+    if (!any) return;
+    for (size_t i = 0; i < st.rank(); i++) {
+      int n = c64(st.sizes[i]);
+      if (checked[i]) {
+        int left = P.pool.bin(EK::MaxS, P.pool.bin(EK::Sub, st.bshape[i], st.boff[i]), c64(0));
+        n = P.pool.bin(EK::MinS, left, n);
+      }
+      a.dims.push_back(n);
+    }
+  }
+  void lower_block_load(const Op &op) {  // tt.load of a !tt.ptr<tensor<...>>: no mask operands, boundaryCheck + padding
+    Type rt = def(op.operands[0]).type;
+    rt.ptr = rt.block = false;
+    PtrState st = visit(op.operands[0]);
+    if (st.boff.size() != st.rank()) throw Unsupported("block-pointer load without a block position");
+    SOp s;
+    s.kind = SK::Load;
+    s.acc = make_access(st, rt);
+    boundary_dims(op, st, s.acc);
+    auto pad = op.attrs.find("padding");
+    if (!s.acc.dims.empty() && pad != op.attrs.end()) {  // 1 = zero, 2 = NaN (PaddingOption)
+      int kind = std::stoi(pad->second);
+      s.acc.has_other = true;
+      if (kind == 2) {
+        if (!rt.is_float()) throw Unsupported("NaN padding of an integer block");
+        s.acc.other_f = std::numeric_limits<double>::quiet_NaN();
+      } else if (kind != 1) {
+        throw Unsupported("padding option " + pad->second);
+      }
+    }
+    s.result = new_value(rt);
+    data_[op.results[0]] = s.result;
+    cur_->push_back(s);
+  }
+  void lower_block_store(const Op &op) {
+    Type vt = def(op.operands[1]).type;
+    PtrState st = visit(op.operands[0]);
+    if (st.boff.size() != st.rank()) throw Unsupported("block-pointer store without a block position");
+    SOp s;
+    s.kind = SK::Store;
+    s.acc = make_access(st, vt);
+    s.operands.push_back(data_of(op.operands[1]));
+    boundary_dims(op, st, s.acc);
+    cur_->push_back(s);
+  }
+
   void lower_load(const Op &op) {
     const Def &p = def(op.operands[0]);
+    if (p.type.block) return lower_block_load(op);
     Type rt = result_type(op);
     SOp s;
     if (p.type.is_tensor) {
@@ -753,6 +853,7 @@ class Lowerer {
 
   void lower_store(const Op &op) {
     const Def &p = def(op.operands[0]);
+    if (p.type.block) return lower_block_store(op);
     SOp s;
     Type vt = def(op.operands[1]).type;
     if (p.type.is_tensor) {
@@ -889,6 +990,7 @@ class Lowerer {
         } else {
           for (auto &o : inside.offsets) o = carry(o);
           for (auto &st : inside.strides) st = carry(st);
+          for (auto &o : inside.boff) o = carry(o);
         }
         c.st = inside;
         known_ptr_[op.iter_names[j]] = inside;
@@ -936,14 +1038,15 @@ class Lowerer {
         if (c.kind == 0) {
           PtrState ns = visit(y);
           ns.pad_mods();
-          if (ns.source != c.st.source || ns.sizes != c.st.sizes || ns.mods != c.st.mods)
-            throw Unsupported("loop-carried pointer changes its base, block shape or wraparound");
+          if (ns.source != c.st.source || ns.sizes != c.st.sizes || ns.mods != c.st.mods || ns.bshape != c.st.bshape)
+            throw Unsupported("loop-carried pointer changes its base, block shape, parent extent or wraparound");
           size_t slot = c.first_slot;
           if (ns.rank() == 0) {
             s.int_iters[slot].next = ns.scalar;
           } else {
             for (auto o : ns.offsets) s.int_iters[slot++].next = o;
             for (auto st : ns.strides) s.int_iters[slot++].next = st;
+            for (auto o : ns.boff) s.int_iters[slot++].next = o;
           }
         } else if (c.kind == 1) {
           s.int_iters[c.first_slot].next = int_of(y);
@@ -975,6 +1078,7 @@ class Lowerer {
         } else {
           for (auto &o : after.offsets) o = s.int_iters[slot++].result_expr;
           for (auto &st : after.strides) st = s.int_iters[slot++].result_expr;
+          for (auto &o : after.boff) o = s.int_iters[slot++].result_expr;
         }
         known_ptr_[rname] = after;
       } else if (c.kind == 1) {
@@ -1114,7 +1218,7 @@ class Lowerer {
     if (op.results.size() != 1) throw Unsupported("operation " + n + " (line " + std::to_string(op.line) + ")");
     Type rt = result_type(op);
     if (rt.ptr) {  // address computation: PtrAnalysis reads it on demand
-      static const std::set<std::string> ptr_ops = {"tt.addptr", "tt.splat", "tt.broadcast", "tt.expand_dims"};
+      static const std::set<std::string> ptr_ops = {"tt.addptr", "tt.splat", "tt.broadcast", "tt.expand_dims", "tt.make_tensor_ptr", "tt.advance"};
       if (!ptr_ops.count(n)) throw Unsupported("pointer-valued operation " + n + " (line " + std::to_string(op.line) + ")");
       return;
     }

@@ -10,11 +10,12 @@
 namespace tts {
 
 std::string Type::str() const {
-  std::string e = ptr ? "!tt.ptr<" + elem + ">" : elem;
+  std::string e = ptr && !block ? "!tt.ptr<" + elem + ">" : elem;
   if (!is_tensor) return e;
   std::string s = "tensor<";
   for (auto d : shape) s += std::to_string(d) + "x";
-  return s + e + ">";
+  s += e + ">";
+  return block ? "!tt.ptr<" + s + ">" : s;
 }
 
 static std::string trim(const std::string &s) {
@@ -52,10 +53,16 @@ Type parse_type(const std::string &raw) {
     size_t comma = in.find(',');  // address space suffix, if printed
     if (comma != std::string::npos) in = in.substr(0, comma);
     t.elem = trim(in);
-    if (starts_with(t.elem, "tensor<") || starts_with(t.elem, "!tt.ptr"))
-      throw Unsupported("block pointers / pointer-to-pointer are not supported: " + s);
+    if (starts_with(t.elem, "tensor<")) {  // a block pointer: the block's shape and element type, flagged
+      t = parse_type(t.elem);
+      if (t.ptr) throw Unsupported("pointer to a block of pointers: " + s);
+      t.ptr = t.block = true;
+      return t;
+    }
+    if (starts_with(t.elem, "!tt.ptr")) throw Unsupported("pointer-to-pointer is not supported: " + s);
     return t;
   }
+  if (starts_with(s, "<tensor<")) return parse_type("!tt.ptr" + s);  // the short form the custom assembly prints
   static const char *known[] = {"i1", "i8", "i16", "i32", "i64", "f16", "bf16", "f32", "f64", "index"};
   for (auto k : known)
     if (s == k) {

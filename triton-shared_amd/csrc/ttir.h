@@ -28,6 +28,7 @@ struct Type {
   std::vector<int64_t> shape;
   bool is_tensor = false;
   bool ptr = false;
+  bool block = false;  // !tt.ptr<tensor<...>>: one pointer to a block (tt.make_tensor_ptr), not a block of pointers
   std::string elem;
   bool is_int() const { return !ptr && (elem[0] == 'i'); }
   bool is_float() const { return !ptr && (elem[0] == 'f' || elem[0] == 'b'); }
