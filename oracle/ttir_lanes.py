@@ -585,6 +585,10 @@ class Interpreter:
             return self._as_float(r.astype(np.float32), a.elem, isinstance(a.d, np.ndarray), already=False)
         if name == "arith.select":
             c, x, y = ops
+            if x.base is not None:               # pointers: element addresses, both sides inside one argument
+                if x.base != y.base:
+                    raise NotImplementedError("select between pointers into different arguments")
+                return Val(np.where(c.d, x.d, y.d).astype(np.int64) if isinstance(c.d, np.ndarray) else (x.d if c.d else y.d), x.elem, x.base)
             if isinstance(c.d, np.ndarray) or isinstance(x.d, np.ndarray):
                 return Val(np.where(c.d, x.d, y.d).astype(_NP[x.elem]), x.elem)
             return Val(x.d if c.d else y.d, x.elem)

@@ -992,3 +992,17 @@ def matmul_grouped_order_plus_bias(a_ptr, b_ptr, c_ptr, bias_ptr, M, N, K, s_am,
         pb += BK * s_bk
     acc += tl.load(bias_ptr + rn, mask=rn < N, other=0.0)[None, :] + 16.0 * tl.load(bias_ptr + N + rm, mask=rm < M, other=0.0)[:, None]
     tl.store(c_ptr + rm[:, None] * s_cm + rn[None, :], acc.to(c_ptr.dtype.element_ty), mask=(rm[:, None] < M) & (rn[None, :] < N))
+
+
+@triton.jit
+def pointer_blocks_by_branch(src, idx, dst, flag, pitch, BLOCK: tl.constexpr):
+    # a block of pointers chosen by an if / else (one side gathered through loaded row numbers, the other strided) and then
+    # by tl.where between two blocks of pointers (TritonToStructured/conditional_ptr_as_src_for_yield_input.mlir's shape)
+    offs = tl.arange(0, BLOCK)
+    rows = tl.load(idx + offs)
+    if flag == 0:
+        p = src + rows * pitch + offs
+    else:
+        p = src + offs * 2
+    q = tl.where((offs % 2) == 0, p, src + offs + tl.program_id(0))
+    tl.store(dst + tl.program_id(0) * BLOCK + offs, tl.load(q))

@@ -559,6 +559,32 @@ def test_tile_program_block_pointer_ops():
             assert np.array_equal(mem[2].reshape(M, N), c.cpu().numpy(), equal_nan=True)
 
 
+def test_tile_program_pointer_blocks_chosen_by_branch_and_where():
+    """A block of pointers yielded by an if / else (gathered on one side, strided on the other) and tl.where between two
+    blocks of pointers: both become blocks of 64-bit offsets from the one argument.  Exact against the index arithmetic
+    in numpy and against the lane interpreter."""
+    import extra_kernels as X
+    from test_planner import compile_ttir
+    from oracle import ttir_lanes
+    g = torch.Generator(device="cpu").manual_seed(11)
+    src = torch.randn(64 * 80, generator=g).to(DEV)
+    idx = torch.randint(0, 64, (64,), generator=g, dtype=torch.int32).to(DEV)
+    sig = {"src": "*fp32", "idx": "*i32", "dst": "*fp32", "flag": "i32", "pitch": "i32", "BLOCK": "constexpr"}
+    ttir = compile_ttir(X.pointer_blocks_by_branch, sig, {"BLOCK": 64})
+    for flag in (0, 1, 7):
+        dst = torch.zeros(3 * 64, device=DEV)
+        k = X.pointer_blocks_by_branch[(3,)](src, idx, dst, flag, 80, BLOCK=64)
+        torch.cuda.synchronize()
+        assert k.function.family == "tile_program"
+        offs = np.arange(64)
+        p = idx.cpu().numpy() * 80 + offs if flag == 0 else offs * 2
+        want = np.concatenate([src.cpu().numpy()[np.where(offs % 2 == 0, p, offs + pid)] for pid in range(3)])
+        assert np.array_equal(dst.cpu().numpy(), want)
+        mem = {0: src.cpu().numpy().copy(), 1: idx.cpu().numpy().copy(), 2: np.zeros(3 * 64, np.float32)}
+        ttir_lanes.Interpreter(ttir).run((3,), [None, None, None, flag, 80], mem)
+        assert np.array_equal(mem[2], want)
+
+
 def test_tile_program_in_place_swap():
     import extra_kernels as X
     torch.manual_seed(0)

@@ -684,6 +684,26 @@ class Lowerer {
       }
       return u;
     }
+    if (op.name == "arith.select") {  // tl.where between two blocks of pointers into one argument: a choice of offsets
+      Scattered a = scattered(op.operands[1]), b = scattered(op.operands[2]);
+      if (a.base != b.base) throw Unsupported("select between pointers into different arguments (line " + std::to_string(op.line) + ")");
+      const Def &c = def(op.operands[0]);
+      if (!c.type.is_tensor) throw Unsupported("select between blocks of pointers on a scalar condition (line " + std::to_string(op.line) + ")");
+      SOp s;
+      s.kind = SK::Map;
+      s.name = "arith.select";
+      s.operands = {data_of(op.operands[0]), offsets_block(a, d.type.shape), offsets_block(b, d.type.shape)};
+      Type t;
+      t.is_tensor = true;
+      t.shape = d.type.shape;
+      t.elem = "i64";
+      s.result = new_value(t);
+      cur_->push_back(s);
+      u.base = a.base;
+      u.scalar = c64(0);
+      u.value = s.result;
+      return u;
+    }
     throw Unsupported("address computed by " + op.name + " (line " + std::to_string(op.line) + ")");
   }
   // the per-element offsets of an unstructured address as one block of 64-bit integers, its scalar part added in
@@ -1218,7 +1238,7 @@ class Lowerer {
     if (op.results.size() != 1) throw Unsupported("operation " + n + " (line " + std::to_string(op.line) + ")");
     Type rt = result_type(op);
     if (rt.ptr) {  // address computation: PtrAnalysis reads it on demand
-      static const std::set<std::string> ptr_ops = {"tt.addptr", "tt.splat", "tt.broadcast", "tt.expand_dims", "tt.make_tensor_ptr", "tt.advance"};
+      static const std::set<std::string> ptr_ops = {"tt.addptr", "tt.splat", "tt.broadcast", "tt.expand_dims", "tt.make_tensor_ptr", "tt.advance", "arith.select"};
       if (!ptr_ops.count(n)) throw Unsupported("pointer-valued operation " + n + " (line " + std::to_string(op.line) + ")");
       return;
     }
@@ -1292,12 +1312,13 @@ class Lowerer {
     if (nres && op.regions.size() != 2) throw Unsupported("scf.if with results but without an else region");
     std::vector<int> results;
     // A scalar pointer that both sides derive from one argument is yielded as its offset from that argument, a 64-bit
-    // integer like any other result; after the branch the pointer is the argument plus that value.
+    // integer like any other result; after the branch the pointer is the argument plus that value.  A block of pointers
+    // is yielded the same way, as a block of 64-bit offsets, and is an unstructured address from there on.
     std::vector<int> ptr_base(nres, -1);
     for (size_t j = 0; j < nres; j++) {
       Type t = op.result_types.at(j);
       if (t.ptr) {
-        if (t.is_tensor) throw Unsupported("scf.if that yields blocks of pointers (line " + std::to_string(op.line) + ")");
+        if (t.block) throw Unsupported("scf.if that yields a block pointer (line " + std::to_string(op.line) + ")");
         ptr_base[j] = -2;  // the sides fill it in
         t.ptr = false;
         t.elem = "i64";
@@ -1328,6 +1349,14 @@ class Lowerer {
             s.tile_yields.push_back(data_of(y));
             continue;
           }
+          if (op.result_types[j].is_tensor) {
+            Scattered u = scattered(y);
+            if (ptr_base[j] >= 0 && ptr_base[j] != u.base)
+              throw Unsupported("scf.if whose sides yield pointers into different arguments (line " + std::to_string(op.line) + ")");
+            ptr_base[j] = u.base;
+            s.tile_yields.push_back(offsets_block(u, op.result_types[j].shape));
+            continue;
+          }
           PtrState st = visit(y);
           if (st.rank() != 0 || st.source < 0) throw Unsupported("scf.if that yields a pointer without a base argument (line " + std::to_string(op.line) + ")");
           if (ptr_base[j] >= 0 && ptr_base[j] != st.source)
@@ -1349,6 +1378,14 @@ class Lowerer {
     for (size_t j = 0; j < nres; j++) {
       if (ptr_base[j] == -1) {
         data_[op.results[j]] = results[j];
+        continue;
+      }
+      if (op.result_types[j].is_tensor) {
+        Scattered after;
+        after.base = ptr_base[j];
+        after.scalar = c64(0);
+        after.value = results[j];
+        carried_scatter_[op.results[j]] = after;
         continue;
       }
       PtrState after;
