@@ -453,7 +453,7 @@ class Interpreter:
 
     def _load(self, ops):
         p = ops[0]
-        store = self.mem[p.base]
+        store = self._seen_as(self.mem[p.base], p.elem)
         if isinstance(p.d, BlockPtr):
             idx, mask = p.d.lanes(self._checked_dims())
             pad = re.search(r"padding = (\d)", self._last_line)
@@ -484,7 +484,7 @@ class Interpreter:
 
     def _store(self, ops):
         p, v = ops[0], ops[1]
-        store = self.mem[p.base]
+        store = self._seen_as(self.mem[p.base], p.elem)
         if isinstance(p.d, BlockPtr):
             idx, mask = p.d.lanes(self._checked_dims())
             sel = idx[mask]
@@ -508,6 +508,14 @@ class Interpreter:
                 raise IndexError(f"store outside argument {p.base}")
             store[idx] = self._narrow(v.d[mask], p.elem)
         return None
+
+    @staticmethod
+    def _seen_as(store, elem):
+        """An argument's memory under a pointer cast to another type of the same width: the same bytes (a numpy view)."""
+        want = np.dtype(_NP[elem]) if elem != "bf16" else np.dtype(np.uint16)
+        if store.dtype != want and store.dtype.itemsize == want.itemsize and elem != "i1":
+            return store.view(want)
+        return store
 
     @staticmethod
     def _widen(raw, elem):
@@ -614,6 +622,8 @@ class Interpreter:
             with np.errstate(all="ignore"):
                 r = table[fn](*[np.asarray(o.d, dtype=np.float64) for o in ops])
             return self._as_float(np.asarray(r).astype(np.float32), a.elem, isinstance(a.d, np.ndarray), already=False)
+        if name == "tt.bitcast" and ops[0].base is not None:      # a pointer cast: same addresses, another element type
+            return Val(ops[0].d, tys[-1].elem, ops[0].base)
         if name in ("tt.bitcast", "arith.bitcast"):
             if (a.elem in _INT_BITS) == (e in _INT_BITS):
                 return Val(a.d, e)                     # signedness only

@@ -1006,3 +1006,16 @@ def pointer_blocks_by_branch(src, idx, dst, flag, pitch, BLOCK: tl.constexpr):
         p = src + offs * 2
     q = tl.where((offs % 2) == 0, p, src + offs + tl.program_id(0))
     tl.store(dst + tl.program_id(0) * BLOCK + offs, tl.load(q))
+
+
+@triton.jit
+def float_bits_through_pointer_cast(x_ptr, bits_ptr, y_ptr, n, BLOCK: tl.constexpr):
+    # the same buffer read as fp32 and, through a pointer cast, as its bit patterns; the sign bit is cleared in the integer
+    # view and the result written back through a float buffer seen as integers
+    offs = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = offs < n
+    xi = x_ptr.to(tl.pointer_type(tl.int32))
+    b = tl.load(xi + offs, mask=m, other=0)
+    tl.store(bits_ptr + offs, b, mask=m)
+    yi = (y_ptr + 0).to(tl.pointer_type(tl.int32))
+    tl.store(yi + offs, b & 0x7FFFFFFF, mask=m)

@@ -585,6 +585,26 @@ def test_tile_program_pointer_blocks_chosen_by_branch_and_where():
         assert np.array_equal(mem[2], want)
 
 
+def test_tile_program_same_width_pointer_cast():
+    """`ptr.to(tl.pointer_type(tl.int32))` on a float buffer (tt.bitcast of a scalar pointer to a type of the same width):
+    the same addresses, read and written as bit patterns.  Exact against numpy views and against the lane interpreter."""
+    import extra_kernels as X
+    from test_planner import compile_ttir
+    from oracle import ttir_lanes
+    n = 1000
+    x = torch.randn(n, generator=torch.Generator(device="cpu").manual_seed(2)).to(DEV)
+    bits = torch.zeros(n, dtype=torch.int32, device=DEV)
+    y = torch.zeros(n, device=DEV)
+    k = X.float_bits_through_pointer_cast[(4,)](x, bits, y, n, BLOCK=256)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program" and "tt.bitcast" in k.asm["ttir"]
+    assert torch.equal(bits, x.view(torch.int32)) and torch.equal(y, x.abs())
+    sig = {"x_ptr": "*fp32", "bits_ptr": "*i32", "y_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"}
+    mem = {0: x.cpu().numpy().copy(), 1: np.zeros(n, np.int32), 2: np.zeros(n, np.float32)}
+    ttir_lanes.Interpreter(compile_ttir(X.float_bits_through_pointer_cast, sig, {"BLOCK": 256})).run((4,), [None, None, None, n], mem)
+    assert np.array_equal(mem[1], bits.cpu().numpy()) and np.array_equal(mem[2], y.cpu().numpy())
+
+
 def test_tile_program_in_place_swap():
     import extra_kernels as X
     torch.manual_seed(0)

@@ -387,7 +387,9 @@ def test_reference_lit_inputs_plan_or_are_refused_for_a_known_reason(native):
         "tile_program: a loop-carried block value of more than 32768 elements": 3,   # 256 x 256 accumulators in one program (kernel-05-layer-norm-dwdb.mlir)
         "tile_program: the reductions of this program need": 4,
         "tile_program: elementwise op extern.some_symbol": 3,     # the reference refuses it too (unsupported_extern_elementwise.mlir)
-        "pointer-valued operation": 9,                            # int_to_ptr / bitcast / cat on pointers (the reference's TritonToPtr fallback)
+        "pointer-valued operation": 7,                            # int_to_ptr / cat on pointers (the reference's TritonToPtr fallback)
+        "scalar integer operation tt.ptr_to_int": 1,              # cast_with_int_ptr.mlir: addresses as integers
+        "pointer cast that changes the element width": 2,         # i32 <-> i64 / i8 views of one buffer: every offset would be rescaled
         "scalar pointer produced by arith.select": 1,             # a choice between two arguments (mixed_structured_unstructured.mlir)
         "unsupported type 'f8E4M3FN'": 1,
         "unsupported type '[": 3,                                 # tts / memref dialect inputs of later stages

@@ -307,6 +307,15 @@ class Lowerer {
         return s;
       }
       if (d.op && d.op->name == "tt.addptr") return visit_addptr(*d.op);
+      if (d.op && d.op->name == "tt.bitcast") {
+        // the same memory read as another type of the same width (float bits as integers): offsets count elements, so
+        // they stay what they are; a cast that changes the element width would rescale every offset and is refused
+        static const std::map<std::string, int> width = {{"i1", 1}, {"i8", 1}, {"i16", 2}, {"f16", 2}, {"bf16", 2}, {"i32", 4}, {"f32", 4}, {"i64", 8}, {"f64", 8}};
+        auto from = width.find(def(d.op->operands.at(0)).type.elem), to = width.find(d.type.elem);
+        if (from == width.end() || to == width.end() || from->second != to->second)
+          throw Unsupported("pointer cast that changes the element width (line " + std::to_string(d.op->line) + ")");
+        return visit(d.op->operands[0]);
+      }
       throw Unsupported("scalar pointer produced by " + (d.op ? d.op->name : std::string("a region argument")));
     }
     if (!d.op) throw Unsupported("PtrAnalysis: tensor region argument " + name + " without a known state");
@@ -1239,7 +1248,8 @@ class Lowerer {
     Type rt = result_type(op);
     if (rt.ptr) {  // address computation: PtrAnalysis reads it on demand
       static const std::set<std::string> ptr_ops = {"tt.addptr", "tt.splat", "tt.broadcast", "tt.expand_dims", "tt.make_tensor_ptr", "tt.advance", "arith.select"};
-      if (!ptr_ops.count(n)) throw Unsupported("pointer-valued operation " + n + " (line " + std::to_string(op.line) + ")");
+      if (!ptr_ops.count(n) && !(n == "tt.bitcast" && !rt.is_tensor))
+        throw Unsupported("pointer-valued operation " + n + " (line " + std::to_string(op.line) + ")");
       return;
     }
     if (!rt.is_tensor && rt.is_int() && !in_region_) {  // scalar integer: int_of reads it on demand
