@@ -1,0 +1,72 @@
+"""tts_launch_noalloc (the launch for callers that cannot allocate device memory) against tts_launch, through the C ABI.
+
+Both run the same kernels and add the K slices in slice order, so the int8-weight product must come out bit for bit
+the same whether its partial tiles sit in the plan's own workspace (tts_launch) or in the library's static scratch
+array (tts_launch_noalloc).  Two calls in a row share that array; the second is a smaller problem."""
+import pytest
+import torch
+
+from conftest import plan_for
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _inputs(M, N, Kd, seed):
+    torch.manual_seed(seed)
+    a = torch.randn(M, Kd).half().to(DEV)
+    w = torch.randint(-127, 128, (Kd, N), dtype=torch.int8).to(DEV)
+    s = (0.001 + 0.009 * torch.rand(N)).half().to(DEV)
+    return a, w, s
+
+
+def _values(a, w, s, c, M, N, Kd):
+    # w8a16_matmul(a, w, scale, c, M, N, K, stride_am, stride_wk, stride_cm): the unit inner strides are constants
+    return [a.data_ptr(), w.data_ptr(), s.data_ptr(), c.data_ptr(), M, N, Kd, a.stride(0), w.stride(0), c.stride(0)]
+
+
+def test_noalloc_launch_matches_the_allocating_launch(native):
+    plan, _ = plan_for(native, "w8a16_matmul")
+    assert plan.family == "gemm_w8a16"
+    stream = torch.cuda.current_stream().cuda_stream
+    # a split-K shape on the wide kernel (counters and partial tiles), then a smaller one on the same scratch array,
+    # then a shape that the narrow kernel and its separate reduce kernel take
+    for seed, (M, N, Kd) in enumerate([(16, 2048, 8192), (16, 1024, 4096), (13, 384, 4096)]):
+        a, w, s = _inputs(M, N, Kd, seed)
+        grid = (1, (N + 127) // 128, 1)
+        want = torch.full((M, N), 5.0, dtype=torch.float16, device=DEV)
+        got = torch.full((M, N), 7.0, dtype=torch.float16, device=DEV)
+        vals = _values(a, w, s, want, M, N, Kd)
+        d = plan.describe_launch(grid, vals)
+        assert int(d["split"]) > 1, d            # the case that needs scratch memory
+        plan.launch(grid, stream, vals)
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        plan.launch_noalloc(grid, stream, _values(a, w, s, got, M, N, Kd))
+        torch.cuda.synchronize()
+        if seed > 0:                             # the first call on a device looks up the scratch array's address
+            assert torch.cuda.mem_get_info()[0] >= free_before
+        assert torch.equal(got, want), (M, N, Kd)
+        ref = a.double() @ (w.half() * s[None, :]).double()
+        assert ((got.double() - ref).norm() / ref.norm()).item() <= 1e-2
+
+
+def test_noalloc_launch_refuses_a_plan_that_still_has_to_compile(native):
+    # a fused map is compiled into a kernel of its own at its first launch, which allocates: the no-allocation launch
+    # says so instead of compiling (nothing is dereferenced before the refusal)
+    plan, _ = plan_for(native, "gelu_tanh_bias")
+    assert plan.family == "fused_map"
+    n = 4096
+    x = torch.randn(n, device=DEV)
+    b = torch.randn(n, device=DEV)
+    y = torch.zeros(n, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    vals = [x.data_ptr(), b.data_ptr(), y.data_ptr(), n]
+    with pytest.raises(NotImplementedError, match="allocates"):
+        plan.launch_noalloc((4, 1, 1), stream, vals)
+    plan.launch((4, 1, 1), stream, vals)         # compiles
+    want = y.clone()
+    y.zero_()
+    plan.launch_noalloc((4, 1, 1), stream, vals)  # now there is nothing left to allocate
+    torch.cuda.synchronize()
+    assert torch.equal(y, want) and want.abs().sum().item() > 0

@@ -59,6 +59,7 @@ def lib():
                                            ctypes.POINTER(TtsArg), ctypes.c_int, ctypes.POINTER(ctypes.c_void_p)]
     L.tts_launch.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                              ctypes.POINTER(TtsArg), ctypes.c_int]
+    L.tts_launch_noalloc.argtypes = L.tts_launch.argtypes
     _lib = L
     return L
 
@@ -148,6 +149,13 @@ class PlanHandle:
 
     def launch_packed(self, grid, stream, arr, n):
         st = lib().tts_launch(self._h, grid[0], grid[1], grid[2], stream, arr, n)
+        if st != TTS_OK:
+            _raise(st)
+
+    def launch_noalloc(self, grid, stream, values):
+        """tts_launch_noalloc: the launch for callers that cannot allocate device memory."""
+        arr = self.pack(values)
+        st = lib().tts_launch_noalloc(self._h, grid[0], grid[1], grid[2], stream, arr, len(values))
         if st != TTS_OK:
             _raise(st)
 

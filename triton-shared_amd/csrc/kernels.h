@@ -105,6 +105,7 @@ struct GemmEpilogueArgs {
   const int *tile_pid;
   int tiles_n, gx, gy, gz;
 };
+int gemm_epilogue_kernel_index(const GemmParams &p);  // which of `modules` a launch of this shape uses
 hipError_t launch_gemm_epilogue(const GemmParams &p, const std::string &epilogue, RtcModule **modules, const GemmEpilogueArgs &ep,
                                 hipStream_t s, const char **kernel_name, std::string *err);
 

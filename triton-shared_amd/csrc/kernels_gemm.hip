@@ -451,13 +451,15 @@ hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
   return p.is_bf16 ? launch_gemm_cfg<true, 2, 2, 64>(p, s) : launch_gemm_cfg<false, 2, 2, 64>(p, s);
 }
 
+int gemm_epilogue_kernel_index(const GemmParams &p) { return gemm_fast_path_ok(p) ? 0 : (p.M >= 2048 && p.N >= 2048) ? 1 : 2; }
+
 // Kernel 0: whole 256 x 256 x 32 tiles; 1: any shape in 256 x 256 tiles; 2: any shape in 128 x 128 tiles -- the choice
 // launch_gemm makes, with the kernels compiled from gemm_device.h plus the epilogue functor at the first launch.
 hipError_t launch_gemm_epilogue(const GemmParams &p, const std::string &epilogue, RtcModule **modules, const GemmEpilogueArgs &ep,
                                 hipStream_t s, const char **name, std::string *err) {
   static const char *names[3] = {"gemm_dma_kernel + epilogue (hipRTC)", "gemm_mfma_kernel<256x256x32> + epilogue (hipRTC)",
                                  "gemm_mfma_kernel<128x128x64> + epilogue (hipRTC)"};
-  const int which = gemm_fast_path_ok(p) ? 0 : (p.M >= 2048 && p.N >= 2048) ? 1 : 2;
+  const int which = gemm_epilogue_kernel_index(p);
   const int64_t tile = which == 2 ? 128 : 256;
   *name = names[which];
   if (!modules[which]) {

@@ -41,6 +41,12 @@ struct Invalid : std::runtime_error {
   using std::runtime_error::runtime_error;
 };
 
+thread_local bool g_no_alloc = false;  // set while tts_launch_noalloc runs on this thread
+void may_allocate(const char *what) {
+  if (g_no_alloc)
+    throw Unsupported(std::string("tts_launch_noalloc: this launch needs ") + what + ", which allocates; run it once through tts_launch first");
+}
+
 // Everything a launch needs besides the pointers, resolved for one (scalars, grid).
 struct Bound {
   Family family;
@@ -319,6 +325,7 @@ void bind_gemm(const Resolver &r, Bound &b) {
   p.M = d.M; p.N = d.N; p.K = d.K; p.lda = d.lda; p.ldb = d.ldb; p.ldc = d.ldc;
   p.is_bf16 = (int)r.pl.k.at("is_bf16");
   if (!r.pl.source.empty()) {  // a fused epilogue looks up the program that owns an element
+    may_allocate("a table of tile owners on the device");
     hipError_t e = hipMalloc((void **)&b.tile_pid, d.tile_pid.size() * sizeof(int));
     if (e == hipSuccess) e = hipMemcpy(b.tile_pid, d.tile_pid.data(), d.tile_pid.size() * sizeof(int), hipMemcpyHostToDevice);
     if (e != hipSuccess) throw std::runtime_error(std::string("gemm: tile table: ") + hipGetErrorString(e));
@@ -394,6 +401,43 @@ tts_status guarded(F &&f) {
 
 const char *PLAN_MAGIC = "tts.plan 1";
 
+// ---- tts_launch_noalloc: the split-K scratch memory of callers that cannot allocate
+// Partial tiles first, arrival counters behind them.  One copy of the array per GPU, held until the process ends.
+constexpr size_t NOALLOC_WORKSPACE_BYTES = (size_t)8 << 20;
+constexpr size_t NOALLOC_COUNTERS = 4096;
+constexpr int NOALLOC_MAX_DEVICES = 64;
+
+}  // namespace
+
+// In host code this name is only a handle for hipGetSymbolAddress: the device address is looked up once per device
+// (noalloc_scratch) and that pointer is what kernels and copies receive.
+static __device__ __align__(256) unsigned char scratch[NOALLOC_WORKSPACE_BYTES + NOALLOC_COUNTERS * sizeof(int)];
+
+namespace {
+
+__global__ void clear_ints_kernel(int *p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// the current device's copy of `scratch`
+unsigned char *noalloc_scratch() {
+  static std::mutex mu;
+  static unsigned char *ptrs[NOALLOC_MAX_DEVICES] = {};
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) throw std::runtime_error(std::string("hipGetDevice: ") + hipGetErrorString(e));
+  if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) throw Invalid("tts_launch_noalloc: device ordinal out of range");
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) throw std::runtime_error(std::string("hipGetSymbolAddress(scratch): ") + hipGetErrorString(e));
+    ptrs[dev] = (unsigned char *)p;
+  }
+  return ptrs[dev];
+}
+
 }  // namespace
 
 extern "C" {
@@ -466,8 +510,18 @@ tts_status tts_plan_describe_launch(tts_plan *plan, int gx, int gy, int gz, cons
   });
 }
 
-tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, const tts_arg *args, int n) {
+}  // extern "C"
+
+namespace {
+
+// tts_launch and tts_launch_noalloc (no_alloc: nothing below may allocate device memory or compile)
+tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, const tts_arg *args, int n, bool no_alloc) {
   if (!plan || (n > 0 && !args)) return fail(TTS_INVALID, "null argument");
+  struct Flag {
+    bool saved;
+    explicit Flag(bool v) : saved(g_no_alloc) { g_no_alloc = v; }
+    ~Flag() { g_no_alloc = saved; }
+  } flag(no_alloc);
   return guarded([&]() {
     if (gx < 0 || gy < 0 || gz < 0) throw Invalid("negative grid");
     if ((int64_t)gx * gy * gz == 0) return TTS_OK;  // backend/driver.py:117
@@ -500,6 +554,7 @@ tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, cons
         {
           std::lock_guard<std::mutex> lock(plan->mu);
           if (!plan->fused) {
+            may_allocate("to compile the fused map's kernel");
             std::string why;
             hipError_t ce = fused_map_compile(p, &plan->fused, &why);
             if (ce != hipSuccess) return fail(TTS_HIP_ERROR, "fused_map: " + why);
@@ -519,6 +574,7 @@ tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, cons
         {
           std::lock_guard<std::mutex> lock(plan->mu);
           if (!plan->fused) {
+            may_allocate("to compile the program's kernel");
             std::string why;
             hipError_t ce = rtc_compile(pl.source, "tile_program", &plan->fused, &why);
             if (ce != hipSuccess) return fail(TTS_HIP_ERROR, "tile_program: " + why + "\n--- source ---\n" + pl.source);
@@ -568,6 +624,12 @@ tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, cons
         a.gy = gy;
         a.gz = gz;
         std::string why;
+        if (no_alloc) {
+          const GemmParams &gp = p;
+          const int which = gemm_epilogue_kernel_index(gp);
+          std::lock_guard<std::mutex> lock(plan->mu);
+          if (!plan->gemm_rtc[which]) may_allocate("to compile the matrix product with its fused epilogue");
+        }
         {
           std::lock_guard<std::mutex> lock(plan->mu);
           err = launch_gemm_epilogue(p, pl.source, plan->gemm_rtc, a, s, &kname, &why);
@@ -581,7 +643,23 @@ tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, cons
         p.w = ptr_arg<const int8_t>(args, pl, "b_arg");
         p.scale = ptr_arg<const void>(args, pl, "s_arg");
         p.c = ptr_arg<void>(args, pl, "c_arg");
-        if (p.split > 1) {
+        if (p.split > 1 && no_alloc) {
+          const size_t need = gemm_w8a16_workspace_bytes(p), ncount = gemm_w8a16_counters(p);
+          if (need > NOALLOC_WORKSPACE_BYTES || ncount > NOALLOC_COUNTERS)
+            throw Unsupported("tts_launch_noalloc: the split-K partial tiles of this shape need " + std::to_string(need) + " bytes and " +
+                              std::to_string(ncount) + " counters; the static scratch array holds " +
+                              std::to_string(NOALLOC_WORKSPACE_BYTES) + " bytes and " + std::to_string(NOALLOC_COUNTERS) + " counters");
+          unsigned char *base = noalloc_scratch();
+          p.workspace = reinterpret_cast<float *>(base);
+          p.counters = reinterpret_cast<int *>(base + NOALLOC_WORKSPACE_BYTES);
+          // every call on this GPU shares the array: the counters start at zero whatever the last call left there
+          // (a fill kernel rather than hipMemsetAsync, so that the call may be captured into a graph)
+          if (ncount) {
+            hipLaunchKernelGGL(clear_ints_kernel, dim3((unsigned)((ncount + 255) / 256)), dim3(256), 0, s, p.counters, (int)ncount);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("clearing the split-K counters: ") + hipGetErrorString(e));
+          }
+        } else if (p.split > 1) {
           size_t need = gemm_w8a16_workspace_bytes(p);
           std::lock_guard<std::mutex> lock(plan->mu);
           if (plan->workspace_bytes < need) {
@@ -613,6 +691,18 @@ tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, cons
     if (err != hipSuccess) return fail(TTS_HIP_ERROR, std::string("kernel launch failed: ") + hipGetErrorString(err));
     return TTS_OK;
   });
+}
+
+}  // namespace
+
+extern "C" {
+
+tts_status tts_launch(tts_plan *plan, int gx, int gy, int gz, void *stream, const tts_arg *args, int n) {
+  return launch_impl(plan, gx, gy, gz, stream, args, n, false);
+}
+
+tts_status tts_launch_noalloc(tts_plan *plan, int gx, int gy, int gz, void *stream, const tts_arg *args, int n) {
+  return launch_impl(plan, gx, gy, gz, stream, args, n, true);
 }
 
 }  // extern "C"
