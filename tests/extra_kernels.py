@@ -1019,3 +1019,37 @@ def float_bits_through_pointer_cast(x_ptr, bits_ptr, y_ptr, n, BLOCK: tl.constex
     tl.store(bits_ptr + offs, b, mask=m)
     yi = (y_ptr + 0).to(tl.pointer_type(tl.int32))
     tl.store(yi + offs, b & 0x7FFFFFFF, mask=m)
+
+
+@triton.jit
+def double_in_place_then_square(p_ptr, q_ptr, n, BLOCK: tl.constexpr):
+    # a load that follows a store to the same buffer inside one program has to see the store: q = (2 p)^2, not p^2
+    offs = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = offs < n
+    x = tl.load(p_ptr + offs, mask=m)
+    tl.store(p_ptr + offs, x + x, mask=m)
+    y = tl.load(p_ptr + offs, mask=m)
+    tl.store(q_ptr + offs, y * y, mask=m)
+
+
+@triton.jit
+def bump_counter_and_report(acc_ptr, out_ptr, BLOCK: tl.constexpr):
+    # a scalar read, then a scalar write of the same address, then the value read goes out as a block: every element of
+    # `out` is the old value; and a second read after the write sees the new one
+    old = tl.load(acc_ptr)
+    tl.store(acc_ptr, old + 1)
+    offs = tl.arange(0, BLOCK)
+    tl.store(out_ptr + offs, tl.zeros((BLOCK,), tl.int32) + old)
+    new = tl.load(acc_ptr)
+    tl.store(out_ptr + BLOCK + offs, tl.zeros((BLOCK,), tl.int32) + new)
+
+
+@triton.jit
+def strided_row_softmax(out_ptr, in_ptr, in_pitch, out_pitch, col_stride, n_cols, BLOCK: tl.constexpr):
+    # the row softmax over every col_stride-th element of the input row
+    r = tl.program_id(0)
+    cols = tl.arange(0, BLOCK)
+    v = tl.load(in_ptr + r * in_pitch + cols * col_stride, mask=cols < n_cols, other=-float("inf"))
+    e = tl.exp(v - tl.max(v, axis=0))
+    p = e / tl.sum(e, axis=0)
+    tl.store(out_ptr + r * out_pitch + cols, p, mask=cols < n_cols)

@@ -347,6 +347,137 @@ def test_w8a16_split_k_repeated_launches(K):
         prev = cd
 
 
+# ----------------------------------------- launches and details the hand-written families decline
+@pytest.mark.parametrize("M,N,Kd,dtype", [(4096, 4096, 4096, torch.bfloat16), (200, 333, 150, torch.bfloat16), (512, 384, 200, torch.float16)])
+def test_gemm_with_column_major_b(K, M, N, Kd, dtype):
+    # the tutorial's b.T (python/examples/test_matmul.py:129-136 passes b.stride(0), b.stride(1) whatever they are;
+    # StructuredToMemref.cpp:105-138 takes any strides): B is stored [N, K], the kernel reads it through strides (1, K)
+    torch.manual_seed(M + 1)
+    a = (torch.randn(M, Kd) * 0.1).to(dtype).to(DEV)
+    bt = (torch.randn(N, Kd) * 0.1).to(dtype).to(DEV)
+    b = bt.t()
+    c = torch.full((M, N), 5.0, dtype=dtype, device=DEV)
+    grid = (triton.cdiv(M, 128) * triton.cdiv(N, 128),)
+    k = K.matmul_tiles[grid](a, b, c, M, N, Kd, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+                             BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and k.function.last_kernel.startswith("gemm_mfma_kernel")
+    assert relfro(c.float(), a.float() @ b.float()) <= 1e-2
+    # exact: B^T holds one -1 per column of B, so C is a signed selection of A's columns
+    perm = torch.randint(0, Kd, (N,))
+    bt.zero_()
+    bt[torch.arange(N), perm.to(DEV)] = -1.0
+    K.matmul_tiles[grid](a, b, c, M, N, Kd, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+                         BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert torch.equal(c.cpu(), -a.cpu()[:, perm])
+
+
+def test_gemm_with_column_major_a_and_with_strides_no_kernel_takes(K):
+    torch.manual_seed(11)
+    M, N, Kd = 300, 260, 136
+    at = (torch.randn(Kd, M) * 0.1).bfloat16().to(DEV)
+    a = at.t()                                                            # strides (1, M)
+    b = (torch.randn(Kd, N) * 0.1).bfloat16().to(DEV)
+    c = torch.full((M, N), 5.0, dtype=torch.bfloat16, device=DEV)
+    grid = (triton.cdiv(M, 128) * triton.cdiv(N, 128),)
+    k = K.matmul_tiles[grid](a, b, c, M, N, Kd, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+                             BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert k.function.last_kernel.startswith("gemm_mfma_kernel")
+    assert relfro(c.float(), a.float() @ b.float()) <= 1e-2
+    # every second column of a wider B: neither stride of B is 1, which none of the matrix-product kernels reads; the
+    # launch goes to the generic family's kernel for the same program instead of failing
+    wide = (torch.randn(Kd, 2 * N) * 0.1).bfloat16().to(DEV)
+    b2 = wide[:, ::2]
+    c.fill_(5.0)
+    k = K.matmul_tiles[grid](a, b2, c, M, N, Kd, a.stride(0), a.stride(1), b2.stride(0), b2.stride(1), c.stride(0), c.stride(1),
+                             BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and k.function.last_kernel == "tile_program (hipRTC)"
+    assert relfro(c.float(), a.float() @ b2.float()) <= 1e-2
+
+
+@pytest.mark.parametrize("M", [17, 64])
+def test_w8a16_beyond_the_decode_shape(K, oracle_cpu, M):
+    # the reference's matmul lowering has no shape limit (ConversionPatterns.hpp:1128-1201); the decode kernels stop at
+    # 16 rows, more rows run on the generic family's kernel for the same program
+    torch.manual_seed(M)
+    N, Kd = 384, 512
+    a = torch.randn(M, Kd).half()
+    w = torch.randint(-127, 128, (Kd, N), dtype=torch.int8)
+    s = (0.001 + 0.009 * torch.rand(N)).half()
+    ad, wd, sd = a.to(DEV), w.to(DEV), s.to(DEV)
+    cd = torch.full((M, N), 5.0, dtype=torch.float16, device=DEV)
+    k = K.w8a16_matmul[(triton.cdiv(M, 16), triton.cdiv(N, 128))](ad, wd, sd, cd, M, N, Kd, ad.stride(0), 1, wd.stride(0), 1,
+                                                                  cd.stride(0), 1, BM=16, BN=128, BK=128)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm_w8a16" and k.function.last_kernel == "tile_program (hipRTC)"
+    assert relfro(cd.cpu(), oracle_cpu.w8a16_matmul(a, w, s)) <= 1e-2
+    assert relfro(cd.cpu(), a.double() @ (w.half() * s[None, :]).double()) <= 1e-2
+
+
+def test_softmax_rows_the_row_kernel_declines(K, oracle_cpu):
+    import extra_kernels as X
+    torch.manual_seed(5)
+    # rows of 32768 columns: more than the row kernel keeps in registers
+    x = torch.randn(6, 30000)
+    xd = x.to(DEV)
+    od = torch.full((6, 30000), -9.0, device=DEV)
+    k = K.row_softmax[(6,)](od, xd, xd.stride(0), od.stride(0), 30000, BLOCK=32768)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    assert torch.allclose(od.cpu(), torch.softmax(x, 1))
+    assert (od.cpu() - oracle_cpu.row_softmax(x, BLOCK=32768)).abs().max().item() <= 1e-5
+    # every third element of the input row
+    x = torch.randn(40, 3 * 700)
+    xd = x.to(DEV)
+    od = torch.full((40, 700), -9.0, device=DEV)
+    k = X.strided_row_softmax[(40,)](od, xd, xd.stride(0), od.stride(0), 3, 700, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    assert torch.allclose(od.cpu(), torch.softmax(x[:, ::3], 1))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_vec_add_in_16_bit_floats(K, dtype):
+    torch.manual_seed(7)
+    n = 70000
+    x, y = torch.randn(n).to(dtype).to(DEV), torch.randn(n).to(dtype).to(DEV)
+    z = torch.zeros(n + 8, dtype=dtype, device=DEV)
+    k = K.vec_add[(triton.cdiv(n, 1024),)](x, y, z, n, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "fused_map"
+    assert torch.equal(z[:n], x + y) and z[n:].abs().sum().item() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.int32])
+def test_tile_program_load_after_store_sees_the_store(dtype):
+    # the serial reference finishes the store before the next load of the same buffer starts
+    import extra_kernels as X
+    torch.manual_seed(9)
+    n = 5000
+    p = (torch.randn(n) * 8).to(dtype).to(DEV)
+    p0 = p.clone()
+    q = torch.zeros(n, dtype=dtype, device=DEV)
+    k = X.double_in_place_then_square[(triton.cdiv(n, 1024),)](p, q, n, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    assert torch.equal(p, p0 + p0) and torch.equal(q, (p0 + p0) * (p0 + p0))
+
+
+def test_tile_program_scalar_read_modify_write():
+    import extra_kernels as X
+    acc = torch.tensor([41], dtype=torch.int32, device=DEV)
+    out = torch.zeros(2048, dtype=torch.int32, device=DEV)
+    for step in range(3):
+        X.bump_counter_and_report[(1,)](acc, out, BLOCK=1024)
+        torch.cuda.synchronize()
+        assert acc.item() == 42 + step
+        assert torch.equal(out[:1024], torch.full((1024,), 41 + step, dtype=torch.int32, device=DEV))   # the value read before the write
+        assert torch.equal(out[1024:], torch.full((1024,), 42 + step, dtype=torch.int32, device=DEV))   # and the one read after it
+
+
 # ------------------------------------------------------------- fused maps
 def _lanes(name, n, scalars, inputs, out_dtype, block=1024):
     from conftest import golden_ttir

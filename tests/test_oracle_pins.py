@@ -88,8 +88,14 @@ def test_matmul_matches_float64(oracle_cpu, dtype):
     ref = a.double() @ b.double()
     assert torch.allclose(c.double(), ref, atol=1e-2 * ref.abs().max().item(), rtol=0)
     assert (c.double() - ref).norm() / ref.norm() <= 1e-2
-    # transposed operand would fail: the product is not symmetric
-    assert (c.double() - (b.double().T @ a.double().T).T).norm() / ref.norm() <= 1e-2
+    # negative check: an oracle that read an operand transposed would compute another product; on a square problem
+    # (where such a mistake still has matching shapes) the oracle's result is far from both wrong products
+    a, b = (torch.randn(96, 96) * 0.5).to(dtype), (torch.randn(96, 96) * 0.5).to(dtype)
+    c = oracle_cpu.matmul_tiles(a, b, BM=32, BN=64, BK=16, GROUP_M=8).double()
+    ref = a.double() @ b.double()
+    assert (c - ref).norm() / ref.norm() <= 1e-2
+    for wrong in (a.double().T @ b.double(), a.double() @ b.double().T, b.double() @ a.double()):
+        assert (c - wrong).norm() / ref.norm() > 0.5
 
 
 def test_w8a16_matches_closed_form(oracle_cpu):

@@ -262,14 +262,18 @@ def test_gemm_binding_matches_every_lane(native, shape, kernel):
     assert np.array_equal(np.sort(all_stores), dense(M, N, ldc))  # every element of C exactly once
 
 
-def test_gemm_refuses_grids_that_are_not_the_tile_grid(native):
+def test_gemm_launches_the_product_kernels_decline_go_to_the_generic_family(native):
+    # what the matrix-product family can only check at launch (the grid's shape, strides) does not end the launch:
+    # the same program runs on the generic family's kernel, and the launch description says why
     plan, _ = plan_for(native, "matmul_tiles.small")
-    with pytest.raises(NotImplementedError, match="one program per output tile"):
-        plan.describe_launch((5, 1, 1), [0, 0, 0, 70, 90, 40, 40, 90, 90])
-    with pytest.raises(NotImplementedError, match="inner strides|advance"):
-        # K == 0 trips are fine, but a transposed B (stride_bn != 1) is specialised away at compile time;
-        # here the wrong ldb makes b_kstep disagree only if BK*ldb overflows - use a huge pitch
-        plan.describe_launch((12, 1, 1), [0, 0, 0, 70, 90, 40, 40, 2 ** 31 - 1, 90])
+    d = plan.describe_launch((5, 1, 1), [0, 0, 0, 70, 90, 40, 40, 90, 90])
+    assert d["kernel"] == "tile_program" and "one program per output tile" in d["fallback_reason"]
+    # a pitch so large that BK * ldb wraps in 32 bits: the pointer advance is no longer one K block
+    d = plan.describe_launch((9, 1, 1), [0, 0, 0, 70, 90, 40, 40, 2 ** 31 - 1, 90])
+    assert d["kernel"] == "tile_program" and "advance" in d["fallback_reason"]
+    # the ordinary launch stays on the product kernels
+    d = plan.describe_launch((9, 1, 1), [0, 0, 0, 70, 90, 40, 40, 90, 90])
+    assert d["kernel"] == "gemm_mfma" and d["a_trans"] == "0" and d["b_trans"] == "0"
 
 
 def test_w8a16_binding(native):
@@ -277,8 +281,8 @@ def test_w8a16_binding(native):
     M, N, K = 13, 70, 100
     d = plan.describe_launch((1, 3, 1), [0, 0, 0, 0, M, N, K, K, N, N])
     assert (d["M"], d["N"], d["K"], d["lda"], d["ldw"], d["ldc"]) == ("13", "70", "100", "100", "70", "70")
-    with pytest.raises(NotImplementedError, match="M <= 16"):
-        plan.describe_launch((2, 3, 1), [0, 0, 0, 0, 20, N, K, K, N, N])
+    d = plan.describe_launch((2, 3, 1), [0, 0, 0, 0, 20, N, K, K, N, N])   # beyond the decode shape: the generic family
+    assert d["kernel"] == "tile_program" and "M <= 16" in d["fallback_reason"]
 
 
 def test_index_overflow_is_detected(native):
@@ -458,3 +462,79 @@ def test_every_functional_case_plans(native):
             plan_bytes, _names = native.structured_to_plan(text)
             families.add(native.PlanHandle(plan_bytes).family)
     assert families == {"tile_program", "fused_map"}, families
+
+
+def _generic_source(tmp_path, ttir):
+    """HIP source of the generic family's kernel for a program, from the tts-opt tool."""
+    import os
+    import subprocess
+    from conftest import ROOT
+    f = tmp_path / "k.ttir"
+    f.write_text(ttir)
+    res = subprocess.run([os.path.join(ROOT, "triton-shared_amd", "csrc", "tts-opt"), "--source", str(f)], text=True, capture_output=True)
+    assert res.returncode == 0, res.stderr
+    return res.stdout
+
+
+def test_memory_effects_keep_their_order_inside_a_program(native, tmp_path):
+    import extra_kernels as X
+    # a load after a store to the same argument: the vectorised map (all loads first) must decline, and the generic
+    # family must start a new phase at that load, behind a barrier
+    sig = {"p_ptr": "*fp32", "q_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"}
+    ttir = compile_ttir(X.double_in_place_then_square, sig, {"BLOCK": 1024})
+    plan = native.PlanHandle(native.structured_to_plan(native.ttir_to_structured(ttir))[0])
+    assert plan.family == "tile_program"
+    body = _generic_source(tmp_path, ttir)
+    stores = [m.start() for m in re.finditer(r"\(\(float \*\)p\.ptr\[\d\]\)\[[^;]*\] = ", body)]
+    loads = [m.start() for m in re.finditer(r"ld\d+\[n\] = \(\(const float \*\)p\.ptr\[0\]\)", body)]
+    assert len(stores) == 2 and len(loads) == 2, body
+    assert loads[0] < stores[0] < loads[1] < stores[1]                      # program order
+    assert "__syncthreads();" in body[stores[0]:loads[1]]                   # and a barrier between the store and the re-load
+    # scalar read-modify-write of one address: barriers keep thread 0's store apart from the other threads' reads
+    sig = {"acc_ptr": "*i32", "out_ptr": "*i32", "BLOCK": "constexpr"}
+    ttir = compile_ttir(X.bump_counter_and_report, sig, {"BLOCK": 1024})
+    assert native.PlanHandle(native.structured_to_plan(native.ttir_to_structured(ttir))[0]).family == "tile_program"
+    body = _generic_source(tmp_path, ttir)
+    first_read = body.index("const int s")
+    write = body.index("if (threadIdx.x == 0")
+    second_read = body.index("const int s", write)
+    assert first_read < write < second_read
+    assert "__syncthreads();" in body[first_read:write] and "__syncthreads();" in body[write:second_read]
+
+
+def test_declined_details_of_a_handwritten_family_fall_through(native):
+    import extra_kernels as X
+    from triton_shared_amd.examples import kernels as K
+    # the op structure of the two-input map in fp16 / bf16: the fused map takes it
+    for t in ("fp16", "bf16"):
+        sig = {"x_ptr": "*" + t, "y_ptr": "*" + t, "z_ptr": "*" + t, "n": "i32", "BLOCK": "constexpr"}
+        text = native.ttir_to_structured(compile_ttir(K.vec_add, sig, {"BLOCK": 1024}))
+        assert native.PlanHandle(native.structured_to_plan(text)[0]).family == "fused_map"
+    # a softmax whose input row is strided, and one whose rows are longer than the row kernel holds: the generic family
+    sig = {"out_ptr": "*fp32", "in_ptr": "*fp32", "in_pitch": "i32", "out_pitch": "i32", "col_stride": "i32", "n_cols": "i32", "BLOCK": "constexpr"}
+    text = native.ttir_to_structured(compile_ttir(X.strided_row_softmax, sig, {"BLOCK": 1024}))
+    assert native.PlanHandle(native.structured_to_plan(text)[0]).family == "tile_program"
+    sig = {"out_ptr": "*fp32", "in_ptr": "*fp32", "in_pitch": "i32", "out_pitch": "i32", "n_cols": "i32", "BLOCK": "constexpr"}
+    text = native.ttir_to_structured(compile_ttir(K.row_softmax, sig, {"BLOCK": 32768}))
+    assert native.PlanHandle(native.structured_to_plan(text)[0]).family == "tile_program"
+    text = native.ttir_to_structured(compile_ttir(K.row_softmax, sig, {"BLOCK": 16384}))
+    assert native.PlanHandle(native.structured_to_plan(text)[0]).family == "row_softmax"
+
+
+def test_gemm_binds_column_major_operands(native):
+    from triton_shared_amd.examples import kernels as K
+    # the tutorial's b.T: stride_bk == 1 is specialised to a constant and stride_bn is the pitch
+    sig = {"a_ptr": "*bf16", "b_ptr": "*bf16", "c_ptr": "*bf16", "M": "i32", "N": "i32", "K": "i32", "s_am": "i32", "s_ak": "constexpr",
+           "s_bk": "constexpr", "s_bn": "i32", "s_cm": "i32", "s_cn": "constexpr", "BM": "constexpr", "BN": "constexpr", "BK": "constexpr",
+           "GROUP_M": "constexpr"}
+    text = native.ttir_to_structured(compile_ttir(K.matmul_tiles, sig, {"s_ak": 1, "s_bk": 1, "s_cn": 1, "BM": 128, "BN": 128, "BK": 64, "GROUP_M": 8}))
+    plan = native.PlanHandle(native.structured_to_plan(text)[0])
+    assert plan.family == "gemm"
+    d = plan.describe_launch((4 * 3, 1, 1), [0, 0, 0, 512, 384, 200, 208, 216, 392])
+    assert (d["kernel"], d["a_trans"], d["b_trans"], d["lda"], d["ldb"], d["ldc"]) == ("gemm_mfma", "0", "1", "208", "216", "392")
+    # both strides of B run-time values, neither of them 1: the generic family
+    sig["s_bk"] = "i32"
+    text = native.ttir_to_structured(compile_ttir(K.matmul_tiles, sig, {"s_ak": 1, "s_cn": 1, "BM": 128, "BN": 128, "BK": 64, "GROUP_M": 8}))
+    plan = native.PlanHandle(native.structured_to_plan(text)[0])
+    d = plan.describe_launch((4 * 3, 1, 1), [0, 0, 0, 512, 384, 200, 208, 2, 432, 392])
+    assert d["kernel"] == "tile_program" and "neither stride of B is 1" in d["fallback_reason"]

@@ -17,13 +17,14 @@ typedef __UINTPTR_TYPE__ uintptr_t;
 #include <cstdint>
 #endif
 
-// C[M,N] = A[M,K] * B[K,N], 16-bit operands, fp32 accumulate
+// C[M,N] = A[M,K] * B[K,N], 16-bit operands, fp32 accumulate; C is row-major, A and B row- or column-major
 struct TtsGemmParams {
   const void *a, *b;
   void *c;
   int64_t M, N, K;
-  int64_t lda, ldb, ldc;  // row pitches in elements; the inner strides are 1
+  int64_t lda, ldb, ldc;  // pitches in elements; the other stride of each matrix is 1
   int is_bf16;
+  int a_trans, b_trans;   // A / B is column-major: element (m, k) of A is a[m + k * lda], (k, n) of B is b[k + n * ldb]
 };
 
 namespace tts_gemm_device {
@@ -100,47 +101,68 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams &p, int tiles_m,
   const bool a_vec = (p.lda % 8 == 0) && (((uintptr_t)A & 15) == 0);
   const bool b_vec = (p.ldb % 8 == 0) && (((uintptr_t)B & 15) == 0);
   const int K = (int)p.K;
+  static_assert(BM == BN && CA == 2 * UB, "both operands are staged by the same two routines");
 
-  uint4 ra[CA], rb[UB][2];
-  auto load_tiles = [&](int k0) {
+  // An operand tile is R = BM = BN rows (rows of A, columns of B) by BK values of k.  In memory either k is the
+  // contiguous index (A row-major, B column-major: element (r, k) at P[r * ld + k]) or r is (A column-major, B
+  // row-major: P[k * ld + r]).  Either way the tile lands in LDS as [r][k]; in the second form the two K-neighbours of
+  // eight consecutive r are packed into 32-bit words on the way.
+  auto load_k_contiguous = [&](uint4 (&reg)[CA], const uint16_t *P, int64_t ld, int64_t r0, int64_t rows, bool vec, int k0) {
 #pragma unroll
     for (int j = 0; j < CA; j++) {
       int c = tid + 256 * j, row = c / (BK / 8), kc = c % (BK / 8);
-      int64_t gr = m0 + row;
+      int64_t gr = r0 + row;
       int gk = k0 + kc * 8;
-      ra[j] = gr < p.M ? load8(A + gr * p.lda + gk, K - gk, a_vec) : make_uint4(0, 0, 0, 0);
+      reg[j] = gr < rows ? load8(P + gr * ld + gk, K - gk, vec) : make_uint4(0, 0, 0, 0);
     }
+  };
+  auto store_k_contiguous = [&](const uint4 (&reg)[CA], uint16_t *S) {
+#pragma unroll
+    for (int j = 0; j < CA; j++) {
+      int c = tid + 256 * j, row = c / (BK / 8), kc = c % (BK / 8);
+      *reinterpret_cast<uint4 *>(S + row * PITCH + kc * 8) = reg[j];
+    }
+  };
+  auto load_r_contiguous = [&](uint4 (&reg)[CA], const uint16_t *P, int64_t ld, int64_t r0, int64_t rows, bool vec, int k0) {
 #pragma unroll
     for (int j = 0; j < UB; j++) {
       int u = tid + 256 * j, kp = u / (BN / 8), nc = u % (BN / 8);
       int gk = k0 + 2 * kp;
-      int64_t gn = n0 + nc * 8;
-      int valid = (int)min((int64_t)8, p.N - gn);
+      int64_t gn = r0 + nc * 8;
+      int valid = (int)min((int64_t)8, rows - gn);
 #pragma unroll
       for (int r = 0; r < 2; r++)
-        rb[j][r] = (gk + r < K && valid > 0) ? load8(B + (int64_t)(gk + r) * p.ldb + gn, valid, b_vec) : make_uint4(0, 0, 0, 0);
+        reg[2 * j + r] = (gk + r < K && valid > 0) ? load8(P + (int64_t)(gk + r) * ld + gn, valid, vec) : make_uint4(0, 0, 0, 0);
     }
   };
-  auto store_tiles = [&](int buf) {
-    uint16_t *As = smem + buf * (BM + BN) * PITCH, *Bs = As + BM * PITCH;
-#pragma unroll
-    for (int j = 0; j < CA; j++) {
-      int c = tid + 256 * j, row = c / (BK / 8), kc = c % (BK / 8);
-      *reinterpret_cast<uint4 *>(As + row * PITCH + kc * 8) = ra[j];
-    }
+  auto store_r_contiguous = [&](const uint4 (&reg)[CA], uint16_t *S) {
 #pragma unroll
     for (int j = 0; j < UB; j++) {
       int u = tid + 256 * j, kp = u / (BN / 8), nc = u % (BN / 8);
-      uint32_t r0[4] = {rb[j][0].x, rb[j][0].y, rb[j][0].z, rb[j][0].w};
-      uint32_t r1[4] = {rb[j][1].x, rb[j][1].y, rb[j][1].z, rb[j][1].w};
+      uint32_t r0[4] = {reg[2 * j].x, reg[2 * j].y, reg[2 * j].z, reg[2 * j].w};
+      uint32_t r1[4] = {reg[2 * j + 1].x, reg[2 * j + 1].y, reg[2 * j + 1].z, reg[2 * j + 1].w};
 #pragma unroll
       for (int i = 0; i < 4; i++) {
-        uint32_t lo = (r0[i] & 0xffffu) | (r1[i] << 16);          // column 2i:   k, k+1
-        uint32_t hi = (r0[i] >> 16) | (r1[i] & 0xffff0000u);      // column 2i+1: k, k+1
-        *reinterpret_cast<uint32_t *>(Bs + (nc * 8 + 2 * i) * PITCH + 2 * kp) = lo;
-        *reinterpret_cast<uint32_t *>(Bs + (nc * 8 + 2 * i + 1) * PITCH + 2 * kp) = hi;
+        uint32_t lo = (r0[i] & 0xffffu) | (r1[i] << 16);          // row 2i:   k, k+1
+        uint32_t hi = (r0[i] >> 16) | (r1[i] & 0xffff0000u);      // row 2i+1: k, k+1
+        *reinterpret_cast<uint32_t *>(S + (nc * 8 + 2 * i) * PITCH + 2 * kp) = lo;
+        *reinterpret_cast<uint32_t *>(S + (nc * 8 + 2 * i + 1) * PITCH + 2 * kp) = hi;
       }
     }
+  };
+  uint4 ra[CA], rb[CA];
+  auto load_tiles = [&](int k0) {
+    if (p.a_trans) load_r_contiguous(ra, A, p.lda, m0, p.M, a_vec, k0);
+    else load_k_contiguous(ra, A, p.lda, m0, p.M, a_vec, k0);
+    if (p.b_trans) load_k_contiguous(rb, B, p.ldb, n0, p.N, b_vec, k0);
+    else load_r_contiguous(rb, B, p.ldb, n0, p.N, b_vec, k0);
+  };
+  auto store_tiles = [&](int buf) {
+    uint16_t *As = smem + buf * (BM + BN) * PITCH, *Bs = As + BM * PITCH;
+    if (p.a_trans) store_r_contiguous(ra, As);
+    else store_k_contiguous(ra, As);
+    if (p.b_trans) store_k_contiguous(rb, Bs);
+    else store_r_contiguous(rb, Bs);
   };
 
   f32x16 acc[TM][TN];

@@ -64,7 +64,7 @@ hipError_t launch_gemm_dma(const GemmParams &p, hipStream_t s) {
 
 // whole tiles, 16-byte aligned rows, and per-lane byte offsets that fit 32 bits
 bool gemm_fast_path_ok(const GemmParams &p) {
-  return p.M % F_BM == 0 && p.N % F_BN == 0 && p.K % F_BK == 0 && p.K >= F_BK && p.lda % 8 == 0 && p.ldb % 8 == 0 &&
+  return !p.a_trans && !p.b_trans && p.M % F_BM == 0 && p.N % F_BN == 0 && p.K % F_BK == 0 && p.K >= F_BK && p.lda % 8 == 0 && p.ldb % 8 == 0 &&
          ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0 && p.lda < (1 << 22) && p.ldb < (1 << 25) &&
          p.ldc % 2 == 0 && ((uintptr_t)p.c & 3) == 0;  // C is written in 4-byte pairs
 }

@@ -349,6 +349,7 @@ bool try_softmax(Plan &pl) {
   unit_stride(m, ld->acc, F);
   unit_stride(m, st->acc, F);
   if (ld->acc.sizes != st->acc.sizes) refuse(F, "its load and store blocks differ in size");
+  if (ld->acc.sizes[0] > 16384) refuse(F, "its rows are longer than the 16384 elements the row kernel keeps in registers");
   pl.family = Family::RowSoftmax;
   pl.k["block"] = ld->acc.sizes[0];
   pl.k["in_arg"] = ld->acc.base_arg;
@@ -635,6 +636,15 @@ bool try_fused_map(Plan &pl) {
     }
   }
   if (stores.empty() || B <= 0) return false;
+  {
+    // the kernel performs every load before the first store: a load from an argument that an earlier store wrote has
+    // to see that store, which only the generic family's phases arrange
+    std::set<int> stored;
+    for (SOp *s : m.all) {
+      if (s->kind == SK::Load && stored.count(s->acc.base_arg)) return false;
+      if (s->kind == SK::Store) stored.insert(s->acc.base_arg);
+    }
+  }
   for (SOp *s : m.all)
     if (s->result >= 0) {
       const Value &v = pl.prog.values[s->result];
@@ -828,6 +838,16 @@ bool try_tile_program(Plan &pl) {
 // A tiled matmul whose accumulator goes through elementwise ops before the store (the tutorial kernel's fused
 // activation, test_matmul.py:98-99; a bias, a residual): what stands between the K loop and the store is taken out as an
 // epilogue functor, and what is left -- the loop, a narrowing cast, the store -- is matched as the plain product.
+// What the matrix-product families check only at launch (strides, M, the grid) may fail for a launch that the
+// generic family runs all the same: its kernel for the same program, if it takes the program.
+static std::string generic_fallback(const Program &p) {
+  try {
+    return tile_program_source(p);
+  } catch (const Unsupported &) {
+    return std::string();
+  }
+}
+
 static bool try_gemm_with_epilogue(Plan &pl) {
   const Program &P = pl.prog;
   int loop_at = -1, store_at = -1;
@@ -898,6 +918,7 @@ static bool try_gemm_with_epilogue(Plan &pl) {
   } catch (const Unsupported &) {
     return false;  // not this shape of program: the other families get their turn
   }
+  q.fallback_source = generic_fallback(P);
   pl = std::move(q);
   return true;
 }
@@ -922,11 +943,38 @@ Plan make_plan(Program &&p) {
     if (try_tile_program(pl)) return pl;
     throw Unsupported("a program with gathers, scatters or masks and fill values that are data is outside the hand-written families; signature: " + pl.signature);
   }
-  if (try_map1d(pl) || try_softmax(pl) || try_layernorm(pl)) return pl;
+  // A program with the op structure of a hand-written family but a detail that family declines (another element
+  // type, a strided load, a block too long) goes on to the families after it; the first refusal is the one reported
+  // if none of them takes it.
+  std::string first_refusal;
+  auto reset = [&]() { pl.k.clear(); pl.e.clear(); pl.lin.clear(); pl.f.clear(); };
+  for (bool (*attempt)(Plan &) : {try_map1d, try_softmax, try_layernorm}) {
+    try {
+      if (attempt(pl)) return pl;
+    } catch (const Unsupported &e) {
+      if (first_refusal.empty()) first_refusal = e.what();
+      reset();
+    }
+  }
+  if (!first_refusal.empty()) {
+    try {
+      if (try_fused_map(pl)) return pl;
+    } catch (const Unsupported &) {
+      reset();
+    }
+    try {
+      if (try_tile_program(pl)) return pl;
+    } catch (const Unsupported &) {
+    }
+    throw Unsupported(first_refusal);
+  }
   if (try_gemm_with_epilogue(pl)) return pl;
   std::string gemm_refusal;
   try {
-    if (try_gemm(pl, false) || try_gemm(pl, true)) return pl;
+    if (try_gemm(pl, false) || try_gemm(pl, true)) {
+      pl.fallback_source = generic_fallback(pl.prog);
+      return pl;
+    }
   } catch (const Unsupported &e) {
     // shaped like a tiled matmul but outside what those kernels take: the generic family may run it (small tiles);
     // if not, the matmul family's reason is the one to report

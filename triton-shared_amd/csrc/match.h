@@ -5,7 +5,7 @@
 // (backend/driver.py:116-133).  This backend instead recognises the shape of
 // the whole structured program and hands the whole grid to one hand-written
 // gfx950 kernel of the matching family.  A program that matches no family is
-// refused (tts::Unsupported); nothing falls back to a slower path.
+// refused (tts::Unsupported); nothing falls back to the CPU.
 #pragma once
 #include <map>
 #include <string>
@@ -34,6 +34,8 @@ struct Plan {
   std::map<std::string, int64_t> k; // named compile-time constants (block sizes, arg indices)
   std::map<std::string, double> f;  // named float constants
   std::string source;               // TileProgram: the HIP source of the program's kernel; Gemm: of its epilogue functor, if any
+  std::string fallback_source;      // Gemm, GemmW8A16: the same program as a TileProgram kernel (empty if that family declines it),
+                                    // for launches whose strides, sizes or grid the matrix-product kernels do not take
 };
 
 // Generic family: HIP source for a program of structured loads, elementwise ops and stores

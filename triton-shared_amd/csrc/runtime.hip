@@ -10,6 +10,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+#include <list>
 #include <memory>
 #include <mutex>
 #include <set>
@@ -57,6 +58,7 @@ struct Bound {
   GemmW8A16Params w8{};
   MapNParams mapn{};
   bool empty = false;  // nothing to do (e.g. zero trip count with nothing stored)
+  bool fallback = false;  // the family's kernels do not take this launch; the generic family's kernel for the same program runs it
   std::string describe;
   // matrix products with a fused epilogue: which program owns which BM x BN tile (device memory, owned by the binding)
   int *tile_pid = nullptr;
@@ -75,7 +77,13 @@ struct tts_plan {
   Plan plan;
   std::string family;
   std::vector<int> arg_kinds;
-  std::unordered_map<std::string, std::shared_ptr<Bound>> cache;
+  // bindings per (grid, scalar arguments), least recently used last; the oldest goes when there are more than 256
+  struct CacheEntry {
+    std::shared_ptr<Bound> bound;
+    std::list<std::string>::iterator pos;
+  };
+  std::unordered_map<std::string, CacheEntry> cache;
+  std::list<std::string> lru;
   std::mutex mu;
   const char *last_kernel = "";
   float *workspace = nullptr;  // split-K partial sums (device), owned by the plan
@@ -84,10 +92,12 @@ struct tts_plan {
   size_t counters_count = 0;
   RtcModule *fused = nullptr;  // the kernel compiled for this plan at its first launch (fused maps, tile programs)
   RtcModule *gemm_rtc[3] = {nullptr, nullptr, nullptr};  // matrix products with a fused epilogue: one kernel per tiling
+  RtcModule *fallback = nullptr;  // the generic family's kernel for a matrix-product plan (launches the product kernels decline)
   ~tts_plan() {
     if (workspace) (void)hipFree(workspace);
     if (counters) (void)hipFree(counters);
     rtc_release(fused);
+    rtc_release(fallback);
     for (RtcModule *m : gemm_rtc) rtc_release(m);
   }
 };
@@ -127,13 +137,18 @@ struct Resolver {
     a.c0 = X.eval(l.c0, e);
     for (int k = 0; k < 3; k++) a.c[k] = X.eval(l.coef[k], e);
     if (l.orig >= 0) {
-      // the linear form was derived looking through i32 -> index extensions;
-      // confirm on the last program that no 32-bit product wrapped
-      EvalEnv last = env(g[0] - 1, g[1] - 1, g[2] - 1);
-      int64_t want = X.eval(l.orig, last);
-      int64_t got = a.c0 + a.c[0] * (g[0] - 1) + a.c[1] * (g[1] - 1) + a.c[2] * (g[2] - 1);
-      if (want != got)
-        throw Invalid("32-bit overflow in the kernel's index arithmetic for '" + name + "' at the last program of the grid");
+      // the linear form was derived looking through i32 -> index extensions; confirm at every corner of the grid
+      // (a coefficient may be negative, so the extreme offset can sit at any of them) that no 32-bit product wrapped
+      for (int corner = 0; corner < 8; corner++) {
+        const int px = (corner & 1) ? g[0] - 1 : 0, py = (corner & 2) ? g[1] - 1 : 0, pz = (corner & 4) ? g[2] - 1 : 0;
+        if (((corner & 1) && g[0] == 1) || ((corner & 2) && g[1] == 1) || ((corner & 4) && g[2] == 1)) continue;  // same program as another corner
+        EvalEnv at = env(px, py, pz);
+        int64_t want = X.eval(l.orig, at);
+        int64_t got = a.c0 + a.c[0] * px + a.c[1] * py + a.c[2] * pz;
+        if (want != got)
+          throw Invalid("32-bit overflow in the kernel's index arithmetic for '" + name + "' at program (" + std::to_string(px) + ", " +
+                        std::to_string(py) + ", " + std::to_string(pz) + ") of the grid");
+      }
     }
     return a;
   }
@@ -256,6 +271,7 @@ void bind_layernorm(const Resolver &r, Bound &b) {
 // tiling may compute it.
 struct DenseGemm {
   int64_t M, N, K, lda, ldb, ldc;
+  bool a_trans = false, b_trans = false;  // column-major operands (the tutorial's `b.T`): the pitch is the other stride
   std::vector<int> tile_pid;  // per BM x BN tile (row-major over the tile grid): linear id of the program that computes it
   int tiles_n = 0;
 };
@@ -268,13 +284,20 @@ DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
   DenseGemm d;
   d.M = r.ev0("M");
   d.N = r.ev0("N");
-  d.lda = r.ev0("sam");
-  d.ldb = r.ev0("sbk");
+  const int64_t sam = r.ev0("sam"), sak = r.ev0("sak"), sbk = r.ev0("sbk"), sbn = r.ev0("sbn"), scn = r.ev0("scn");
   d.ldc = r.ev0("scm");
   auto need = [&](bool ok, const std::string &why) {
     if (!ok) throw Unsupported(std::string(F) + ": " + why);
   };
-  need(r.ev0("sak") == 1 && r.ev0("sbn") == 1 && r.ev0("scn") == 1, "only unit inner strides (row-major operands) are implemented");
+  // the reference's lowering takes any strides (StructuredToMemref.cpp:105-138); these kernels want one stride of each
+  // operand to be 1 and C row-major
+  need(sak == 1 || sam == 1, "neither stride of A is 1");
+  need(sbn == 1 || sbk == 1, "neither stride of B is 1");
+  need(scn == 1, "the inner stride of C is not 1");
+  d.a_trans = sak != 1;
+  d.b_trans = sbn != 1;
+  d.lda = d.a_trans ? sak : sam;
+  d.ldb = d.b_trans ? sbn : sbk;
   need(d.M > 0 && d.N > 0, "empty problem");
   // K: the loop must sweep K in full blocks followed by at most one partial block
   int64_t trip = r.ev0("trip");
@@ -289,11 +312,11 @@ DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
       d.K += kd;
     }
   }
-  need(r.ev0("a_kstep") == BK && r.ev0("b_kstep") == BK * d.ldb, "operand pointers do not advance by one K block per iteration");
+  need(r.ev0("a_kstep") == BK * sak && r.ev0("b_kstep") == BK * sbk, "operand pointers do not advance by one K block per iteration");
   // wraparound operands: the period is the whole matrix, so rows (columns) inside the problem are not affected
   const bool a_wraps = pl.e.count("a_mod"), b_wraps = pl.e.count("b_mod");
-  if (a_wraps) need(r.ev0("a_mod") == d.M * d.lda, "A rows wrap around with a period other than M");
-  if (b_wraps) need(r.ev0("b_mod") == d.N, "B columns wrap around with a period other than N");
+  if (a_wraps) need(r.ev0("a_mod") == d.M * sam, "A rows wrap around with a period other than M");
+  if (b_wraps) need(r.ev0("b_mod") == d.N * sbn, "B columns wrap around with a period other than N");
   // tiles: every program's origin, offsets consistent with a dense layout, exact cover
   const int64_t tm = (d.M + BM - 1) / BM, tn = (d.N + BN - 1) / BN;
   need((int64_t)r.g[0] * r.g[1] * r.g[2] == tm * tn, "the grid does not have one program per output tile");
@@ -310,10 +333,10 @@ DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
         need(!s, "two programs compute the same output tile");
         s = 1;
         d.tile_pid[(r0 / BM) * tn + c0 / BN] = x + r.g[0] * (y + r.g[1] * z);
-        need(r.ev("a_base", e) == r0 * d.lda, "A tile offset is not row0 * lda");
-        need(r.ev("b_base", e) == c0, "B tile offset is not col0");
-        if (a_wraps) need(r.ev("a_wrapped", e) == r0 * d.lda, "the wrapped part of A's offset is not row0 * lda");
-        if (b_wraps) need(r.ev("b_wrapped", e) == c0, "the wrapped part of B's offset is not col0");
+        need(r.ev("a_base", e) == r0 * sam, "A tile offset is not row0 * its row stride");
+        need(r.ev("b_base", e) == c0 * sbn, "B tile offset is not col0 * its column stride");
+        if (a_wraps) need(r.ev("a_wrapped", e) == r0 * sam, "the wrapped part of A's offset is not row0 * its row stride");
+        if (b_wraps) need(r.ev("b_wrapped", e) == c0 * sbn, "the wrapped part of B's offset is not col0 * its column stride");
         need(r.ev("c_base", e) == r0 * d.ldc + c0, "C tile offset is not row0 * ldc + col0");
       }
   return d;
@@ -323,6 +346,7 @@ void bind_gemm(const Resolver &r, Bound &b) {
   DenseGemm d = prove_dense_gemm(r, "gemm");
   GemmParams &p = b.gemm;
   p.M = d.M; p.N = d.N; p.K = d.K; p.lda = d.lda; p.ldb = d.ldb; p.ldc = d.ldc;
+  p.a_trans = d.a_trans; p.b_trans = d.b_trans;
   p.is_bf16 = (int)r.pl.k.at("is_bf16");
   if (!r.pl.source.empty()) {  // a fused epilogue looks up the program that owns an element
     may_allocate("a table of tile owners on the device");
@@ -333,13 +357,14 @@ void bind_gemm(const Resolver &r, Bound &b) {
   }
   std::ostringstream os;
   os << "kernel=gemm_mfma\nM=" << p.M << "\nN=" << p.N << "\nK=" << p.K << "\nlda=" << p.lda << "\nldb=" << p.ldb
-     << "\nldc=" << p.ldc << "\nbf16=" << p.is_bf16 << "\n";
+     << "\nldc=" << p.ldc << "\nbf16=" << p.is_bf16 << "\na_trans=" << p.a_trans << "\nb_trans=" << p.b_trans << "\n";
   b.describe = os.str();
 }
 
 void bind_w8a16(const Resolver &r, Bound &b) {
   DenseGemm d = prove_dense_gemm(r, "gemm_w8a16");
   if (d.M > 16) throw Unsupported("gemm_w8a16: only the decode shape M <= 16 is implemented");
+  if (d.a_trans || d.b_trans) throw Unsupported("gemm_w8a16: only row-major operands are implemented");
   GemmW8A16Params &p = b.w8;
   p.M = d.M; p.N = d.N; p.K = d.K; p.lda = d.lda; p.ldw = d.ldb; p.ldc = d.ldc;
   p.split = gemm_w8a16_split(p);
@@ -363,7 +388,10 @@ std::shared_ptr<Bound> resolve(tts_plan *h, int gx, int gy, int gz, const tts_ar
   }
   std::lock_guard<std::mutex> lock(h->mu);
   auto it = h->cache.find(key);
-  if (it != h->cache.end()) return it->second;
+  if (it != h->cache.end()) {
+    h->lru.splice(h->lru.begin(), h->lru, it->second.pos);
+    return it->second.bound;
+  }
   auto b = std::make_shared<Bound>();
   b->family = h->plan.family;
   Resolver r(h->plan, args, n, gx, gy, gz);
@@ -371,13 +399,28 @@ std::shared_ptr<Bound> resolve(tts_plan *h, int gx, int gy, int gz, const tts_ar
     case Family::Map1D: bind_map1d(r, *b); break;
     case Family::RowSoftmax: bind_softmax(r, *b); break;
     case Family::LayerNormFwd: bind_layernorm(r, *b); break;
-    case Family::Gemm: bind_gemm(r, *b); break;
-    case Family::GemmW8A16: bind_w8a16(r, *b); break;
+    case Family::Gemm:
+    case Family::GemmW8A16:
+      // what these families can only check now (strides, M, the grid's shape) may fail for a launch that is a valid
+      // Triton program all the same: the generic family's kernel for the same program runs it
+      try {
+        if (b->family == Family::Gemm) bind_gemm(r, *b);
+        else bind_w8a16(r, *b);
+      } catch (const Unsupported &e) {
+        if (h->plan.fallback_source.empty()) throw;
+        b->fallback = true;
+        b->describe = std::string("kernel=tile_program\nfallback_reason=") + e.what() + "\n";
+      }
+      break;
     case Family::FusedMap: bind_fused_map(r, *b); break;
     case Family::TileProgram: b->describe = "kernel=tile_program\n"; break;
   }
-  if (h->cache.size() > 256) h->cache.clear();
-  h->cache[key] = b;
+  h->lru.push_front(key);
+  h->cache[key] = {b, h->lru.begin()};
+  if (h->cache.size() > 256) {  // launches in flight hold their own reference to the binding they use
+    h->cache.erase(h->lru.back());
+    h->lru.pop_back();
+  }
   return b;
 }
 
@@ -531,6 +574,34 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
     hipStream_t s = (hipStream_t)stream;
     hipError_t err = hipSuccess;
     const char *kname = "";
+    // one workgroup of 256 threads per Triton program, on the kernel generated for the program (compiled at its first use)
+    auto run_tile_program = [&](RtcModule **slot, const std::string &source) -> tts_status {
+      struct { void *ptr[TILE_MAX_ARGS]; long long ival[TILE_MAX_ARGS]; double fval[TILE_MAX_ARGS]; } a{};
+      for (int i = 0; i < n; i++) {
+        if (args[i].kind == TTS_ARG_PTR) a.ptr[i] = args[i].v.ptr;
+        else if (args[i].kind == TTS_ARG_INT) a.ival[i] = args[i].v.i;
+        else a.fval[i] = args[i].v.f;
+      }
+      {
+        std::lock_guard<std::mutex> lock(plan->mu);
+        if (!*slot) {
+          may_allocate("to compile the program's kernel");
+          std::string why;
+          hipError_t ce = rtc_compile(source, "tile_program", slot, &why);
+          if (ce != hipSuccess) return fail(TTS_HIP_ERROR, "tile_program: " + why + "\n--- source ---\n" + source);
+        }
+      }
+      kname = "tile_program (hipRTC)";
+      err = rtc_launch(*slot, gx, gy, gz, 256, &a, sizeof a, s);
+      return TTS_OK;
+    };
+    if (b->fallback) {
+      tts_status st = run_tile_program(&plan->fallback, pl.fallback_source);
+      if (st != TTS_OK) return st;
+      plan->last_kernel = kname;
+      if (err != hipSuccess) return fail(TTS_HIP_ERROR, std::string("kernel launch failed: ") + hipGetErrorString(err));
+      return TTS_OK;
+    }
     switch (b->family) {
       case Family::Map1D: {
         Map1DParams p = b->map1d;
@@ -565,23 +636,8 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
         break;
       }
       case Family::TileProgram: {
-        struct { void *ptr[TILE_MAX_ARGS]; long long ival[TILE_MAX_ARGS]; double fval[TILE_MAX_ARGS]; } a{};
-        for (int i = 0; i < n; i++) {
-          if (args[i].kind == TTS_ARG_PTR) a.ptr[i] = args[i].v.ptr;
-          else if (args[i].kind == TTS_ARG_INT) a.ival[i] = args[i].v.i;
-          else a.fval[i] = args[i].v.f;
-        }
-        {
-          std::lock_guard<std::mutex> lock(plan->mu);
-          if (!plan->fused) {
-            may_allocate("to compile the program's kernel");
-            std::string why;
-            hipError_t ce = rtc_compile(pl.source, "tile_program", &plan->fused, &why);
-            if (ce != hipSuccess) return fail(TTS_HIP_ERROR, "tile_program: " + why + "\n--- source ---\n" + pl.source);
-          }
-        }
-        kname = "tile_program (hipRTC)";
-        err = rtc_launch(plan->fused, gx, gy, gz, 256, &a, sizeof a, s);
+        tts_status st = run_tile_program(&plan->fused, pl.source);
+        if (st != TTS_OK) return st;
         break;
       }
       case Family::RowSoftmax: {

@@ -51,6 +51,17 @@ struct Gen {
   std::map<int, std::string> var;          // value id -> C variable holding it at the current element
   int indent = 1;
   std::set<int> all_inline_bases, all_store_bases;  // checked against each other at the end
+  // Arguments the program reads anywhere, and arguments a scalar store writes anywhere (collected before the body is
+  // written, so that an access in a later iteration of a loop counts): a scalar store is one thread's, every read is
+  // all threads', so the two are kept apart by barriers wherever they may touch the same argument.
+  std::set<int> read_bases_anywhere, scalar_store_bases_anywhere;
+  void collect_bases(const std::vector<SOp> &ops) {
+    for (const SOp &s : ops) {
+      if (s.kind == SK::Load || s.kind == SK::ScalarLoad) read_bases_anywhere.insert(s.acc.base_arg);
+      if (s.kind == SK::ScalarStore) scalar_store_bases_anywhere.insert(s.acc.base_arg);
+      if (s.kind == SK::For || s.kind == SK::If) collect_bases(s.body);
+    }
+  }
   std::ostringstream fns;                           // combiner functions of reductions and scans (before the kernel)
   std::ostringstream decl;                          // LDS arrays holding their results (top of the kernel)
   size_t pool_bytes = 0, out_bytes = 0;             // staging pool shared by all reductions; result arrays
@@ -588,6 +599,8 @@ struct Gen {
       }
       if (s.kind == SK::ScalarLoad) {
         map_vars({-1});
+        // thread 0's scalar store to this argument (earlier in the program, or in the previous iteration) is visible
+        if (scalar_store_bases_anywhere.count(s.acc.base_arg)) os << pad() << "__syncthreads();\n";
         std::string pred, addr = address(s.acc, "0", "0", pred);
         std::string name = "s" + std::to_string(s.result);
         os << pad() << "const " << ctype(val(s.result).dtype) << " " << name << " = "
@@ -598,6 +611,8 @@ struct Gen {
       }
       if (s.kind == SK::ScalarStore) {
         map_vars({-1});
+        // every thread has read what it reads from this argument before thread 0 overwrites it
+        if (read_bases_anywhere.count(s.acc.base_arg)) os << pad() << "__syncthreads();\n";
         std::string pred, addr = address(s.acc, "0", "0", pred);
         os << pad() << "if (threadIdx.x == 0" << (s.acc.mask_value >= 0 ? " && (" + at(s.acc.mask_value, "0", "0") + ")" : "") << ") {\n";
         indent++;
@@ -626,12 +641,22 @@ struct Gen {
       size_t end = k;
       {
         const std::vector<int64_t> *first_store = nullptr;  // stores of another block shape start a run of their own
-        for (; end < ops.size() && !is_break(ops[end]); end++)
+        std::set<int> stored;  // a load from an argument that the run has stored to starts a run of its own as well: every
+                               // load of a run is issued before the run's first store, and this one has to see that store
+        for (; end < ops.size() && !is_break(ops[end]); end++) {
+          if (ops[end].kind == SK::Load && stored.count(ops[end].acc.base_arg)) break;
           if (ops[end].kind == SK::Store) {
             if (first_store && ops[end].acc.sizes != *first_store) break;
             first_store = &ops[end].acc.sizes;
+            stored.insert(ops[end].acc.base_arg);
           }
+        }
       }
+      for (size_t q = k; q < end; q++)
+        if (ops[q].kind == SK::Load && scalar_store_bases_anywhere.count(ops[q].acc.base_arg)) {
+          os << pad() << "__syncthreads();\n";  // thread 0's scalar store to an argument this run loads from is visible
+          break;
+        }
       std::vector<int64_t> shape;
       bool have = false, stores = false;
       for (size_t q = k; q < end; q++)
@@ -1437,6 +1462,7 @@ std::string tile_program_source(const Program &p) {
   std::string pre = TILE_PRELUDE;
   const std::string n = std::to_string(TILE_MAX_ARGS);
   for (size_t pos = 0; (pos = pre.find("%N%", pos)) != std::string::npos;) pre.replace(pos, 3, n);
+  g.collect_bases(p.body);
   g.body(p.body);
   if (g.pool_bytes + g.out_bytes > 64 * 1024)
     throw Unsupported("tile_program: the reductions of this program need " + std::to_string(g.pool_bytes + g.out_bytes) + " bytes of LDS (limit 65536)");
