@@ -1,22 +1,29 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2] [--no-cpu] [--only-headline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3] [--no-cpu] [--only-headline]
 
 A step is one pass of one workload's kernel over its synthetic input, enqueued
 through the C ABI (tts_launch) on torch's current stream, on a plan compiled by
 the unchanged Triton frontend.  Inputs live in HBM before the timed region; the
 buffers of consecutive steps rotate over enough copies (> 600 MB) that a step
 does not find its input in the 256 MB Infinity Cache left by the previous one.
-Prints ONE JSON line.  The headline workload is the row softmax, fp32 [4096, 781]
-(the second of the five configurations); the other four configs and two steady-state
-sizes are reported in "kernels".
+Prints ONE JSON line.  The headline workload is the LayerNorm forward, fp16
+[4096, 8192] (the third of the five configurations: HBM-bound at a size that
+neither fits the caches nor is dominated by the launch); the other four
+configurations, two steady-state sizes, the two stream ceilings of the machine
+(a copy and a read-only reduction, through this backend) and the workloads of
+the generic families are reported in "kernels".
 
-Per kernel: `us` = mean kernel duration from HIP events around the timed
-launches; `achieved` = algorithmic bytes (or flops) / that duration; `frac` =
-achieved / MI355X peak (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s).  The CPU
-baseline is the restatement of the reference's CPU path (oracle/cpu_path.c, one
-thread as the reference launcher is single-threaded) on a bounded sample.
+Per kernel: `us` = mean kernel duration from HIP events around the K timed
+launches (the line's ms_per_step); `launch_us` = median / min / std of the
+durations of single launches, each between its own pair of events;
+`achieved` = algorithmic bytes (or flops) / `us`; `frac` = achieved / MI355X
+peak (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s).  The CPU baseline is the
+restatement of the reference's CPU path (oracle/cpu_path.c, one thread as the
+reference launcher is single-threaded) on a bounded sample, timed as the
+reference's own harness does (python/examples/benchmark.py:15-65: wall and
+process time, mean / min / std over the repeats).
 """
 import argparse
 import json
@@ -39,7 +46,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg2", help="headline workload: cfg1..cfg5, cfg1_2p28, cfg2_1m")
+    ap.add_argument("--workload", default="cfg3", help="headline workload: cfg1..cfg5, cfg1_2p28, cfg2_1m, stream_*, next_*")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-headline", action="store_true", help="time only the headline workload")
     ap.add_argument("--rotating-only", action="store_true",
@@ -133,35 +140,16 @@ def make_workloads(torch, triton, K):
             x, b = torch.randn(n, device=dev), torch.randn(n, device=dev)
             y = torch.empty(n, device=dev)
             return lambda: K.gelu_tanh_bias[(triton.cdiv(n, 1024),)](x, b, y, n, BLOCK=1024)
-        m = 1 << 16
-        cpu = lanes((m // 1024,), [m], lambda: [np.random.rand(m).astype(np.float32), np.random.rand(m).astype(np.float32),
-                                                np.zeros(m, np.float32)], m / n, f"N={m}")
         return dict(desc=f"fused map y = gelu_tanh(x + b) fp32 N={n}, BLOCK=1024 (19 elementwise ops, compiled with hipRTC)",
-                    work=3 * n * 4, bound="hbm", dtype="f32", make=make, set_bytes=3 * n * 4, lanes=cpu)
+                    work=3 * n * 4, bound="hbm", dtype="f32", make=make, set_bytes=3 * n * 4)
 
     def fused_silu(n):
         def make():
             g, u = torch.randn(n, device=dev).half(), torch.randn(n, device=dev).half()
             o = torch.empty(n, dtype=torch.float16, device=dev)
             return lambda: K.silu_mul_f16[(triton.cdiv(n, 1024),)](g, u, o, n, BLOCK=1024)
-        m = 1 << 16
-        cpu = lanes((m // 1024,), [m], lambda: [np.random.rand(m).astype(np.float16), np.random.rand(m).astype(np.float16),
-                                                np.zeros(m, np.float16)], m / n, f"N={m}")
         return dict(desc=f"fused map out = silu(g) * u fp16 N={n}, BLOCK=1024 (10 elementwise ops, compiled with hipRTC)",
-                    work=3 * n * 2, bound="hbm", dtype="f16", make=make, set_bytes=3 * n * 2, lanes=cpu)
-
-    def lanes(grid, scalars, arrays, frac, sample):
-        """CPU baseline of a workload outside the five configurations: the lane-level oracle on a smaller problem
-        made of the same programs.  arrays() -> numpy buffers in pointer-argument order."""
-        def run(ttir):
-            from oracle import ttir_lanes
-            bufs = arrays()
-            t0 = time.perf_counter()
-            ttir_lanes.Interpreter(ttir).run(grid, [None] * len(bufs) + list(scalars), dict(enumerate(bufs)))
-            return time.perf_counter() - t0, frac, sample
-        return run
-
-    import numpy as np
+                    work=3 * n * 2, bound="hbm", dtype="f16", make=make, set_bytes=3 * n * 2)
 
     def take_rows(rows, cols):
         def make():
@@ -170,12 +158,8 @@ def make_workloads(torch, triton, K):
             dst = torch.empty_like(src)
             return lambda: K.take_rows[(triton.cdiv(rows, 4),)](src, idx, dst, rows, cols, src.stride(0), dst.stride(0), BR=4, BC=1024)
         work = 2 * rows * cols * 4 + rows * 4
-        r = 256
-        cpu = lanes((r // 4,), [r, cols, cols, cols],
-                    lambda: [np.random.rand(r, cols).astype(np.float32).reshape(-1), np.random.randint(0, r, r).astype(np.int32),
-                             np.zeros(r * cols, np.float32)], r / rows, f"{r} of {rows} rows")
         return dict(desc=f"gather of rows dst[r, :] = src[idx[r], :] fp32 [{rows}, {cols}], 4 rows per program (generic family)",
-                    work=work, bound="hbm", dtype="f32", make=make, set_bytes=work, lanes=cpu)
+                    work=work, bound="hbm", dtype="f32", make=make, set_bytes=work)
 
     def row_sums(rows, cols):
         def make():
@@ -184,21 +168,16 @@ def make_workloads(torch, triton, K):
             br = int(os.environ.get("TTS_BENCH_BR", "4"))
             return lambda: K.row_sums[(triton.cdiv(rows, br),)](x, out, rows, cols, x.stride(0), BR=br, BC=1024)
         work = rows * cols * 4 + rows * 4
-        r = 256
-        cpu = lanes((r // 4,), [r, cols, cols],
-                    lambda: [np.random.rand(r, cols).astype(np.float32).reshape(-1), np.zeros(r, np.float32)], r / rows, f"{r} of {rows} rows")
         return dict(desc=f"row sums of fp32 [{rows}, {cols}], 4 rows per program (generic family, axis reduction)", work=work, bound="hbm",
-                    dtype="f32", make=make, set_bytes=work, lanes=cpu)
+                    dtype="f32", make=make, set_bytes=work)
 
     def block_cumsum(n):
         def make():
             x = torch.randn(n, device=dev)
             y = torch.empty_like(x)
             return lambda: K.block_cumsum[(triton.cdiv(n, 1024),)](x, y, n, BLOCK=1024)
-        m = 1 << 16
-        cpu = lanes((m // 1024,), [m], lambda: [np.random.rand(m).astype(np.float32), np.zeros(m, np.float32)], m / n, f"N={m}")
         return dict(desc=f"inclusive prefix sums inside blocks of 1024, fp32 N={n} (generic family, scan)", work=8 * n, bound="hbm",
-                    dtype="f32", make=make, set_bytes=8 * n, lanes=cpu)
+                    dtype="f32", make=make, set_bytes=8 * n)
 
     def matmul_act(n):
         def make():
@@ -221,6 +200,22 @@ def make_workloads(torch, triton, K):
                          "loaded expert id per 128 rows (generic family: carried gather offsets, LDS-staged operands, 32x32 MFMA blocks)",
                     work=2 * tokens * kd * nd, bound="mfma", dtype="bf16", make=make, set_bytes=(tokens * kd + experts * kd * nd + tokens * nd) * 2)
 
+    def stream_copy(n):
+        def make():
+            x = torch.rand(n, device=dev)
+            z = torch.empty_like(x)
+            return lambda: K.copy_blocks[(triton.cdiv(n, 4096),)](x, z, n, BLOCK=4096)
+        return dict(desc=f"stream ceiling, 1:1 read/write: z = x fp32 N={n}, BLOCK=4096 (fused map with no ops)", work=8 * n, bound="hbm",
+                    dtype="f32", make=make, set_bytes=8 * n)
+
+    def stream_read(n):
+        def make():
+            x = torch.rand(n, device=dev)
+            out = torch.empty(triton.cdiv(n, 4096), device=dev)
+            return lambda: K.block_sums[(triton.cdiv(n, 4096),)](x, out, n, BLOCK=4096)
+        return dict(desc=f"stream ceiling, read only: out[p] = sum of block p of x, fp32 N={n}, BLOCK=4096 (generic family)",
+                    work=4 * n + 4 * triton.cdiv(n, 4096), bound="hbm", dtype="f32", make=make, set_bytes=4 * n)
+
     W["cfg1"] = vec_add(98432)
     W["cfg2"] = softmax(4096)
     W["cfg3"] = layernorm()
@@ -228,6 +223,8 @@ def make_workloads(torch, triton, K):
     W["cfg5"] = w8a16()
     W["cfg1_2p28"] = vec_add(1 << 28)
     W["cfg2_1m"] = softmax(1 << 20)
+    W["stream_copy_2p28"] = stream_copy(1 << 28)
+    W["stream_read_2p28"] = stream_read(1 << 28)
     W["next_fused_gelu_2p26"] = fused_gelu(1 << 26)
     W["next_fused_silu_2p26"] = fused_silu(1 << 26)
     W["next_matmul_act_4096"] = matmul_act(4096)
@@ -274,11 +271,26 @@ def time_workload(torch, spy, wl, steps, warmup, rotating_only=False):
     torch.cuda.synchronize()
     wall_us = (time.perf_counter() - t0) * 1e6 / steps
     us = start.elapsed_time(stop) * 1e3 / steps
+    # single launches, each between its own pair of events: median / min / std (the events add a little to every launch,
+    # so these sit slightly above `us`; they show the spread, `us` is the figure the fractions use)
+    singles = max(steps, 100) if wl["set_bytes"] < 1e9 else steps
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(singles)]
+    for i, (e0, e1) in enumerate(pairs):
+        g, arr, n, _ = launches[i % sets]
+        e0.record()
+        plan.launch_packed(g, stream, arr, n)
+        e1.record()
+    torch.cuda.synchronize()
+    per = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in pairs)
+    mean = sum(per) / len(per)
+    launch_us = dict(median=round(per[len(per) // 2], 3), min=round(per[0], 3),
+                     std=round((sum((v - mean) ** 2 for v in per) / len(per)) ** 0.5, 3), n=len(per))
     if rotating_only:
         kernel = plan.last_kernel
         del launches
         torch.cuda.empty_cache()
-        return dict(us=us, hot_us=us, wall_us=wall_us, kernel=kernel, sets=sets, frontend_us=0.0, warmup_steps_run=done, ttir=ttir)
+        return dict(us=us, hot_us=us, wall_us=wall_us, kernel=kernel, sets=sets, frontend_us=0.0, warmup_steps_run=done, ttir=ttir,
+                    launch_us=launch_us)
     # same measurement on one buffer set ("hot": inputs may sit in the Infinity Cache), for information
     g, arr, n, _ = launches[0]
     for _ in range(warmup):
@@ -299,7 +311,7 @@ def time_workload(torch, spy, wl, steps, warmup, rotating_only=False):
     del launches
     torch.cuda.empty_cache()
     return dict(us=us, hot_us=hot_us, wall_us=wall_us, kernel=plan.last_kernel, sets=sets, frontend_us=frontend_us, ttir=ttir,
-                warmup_steps_run=done)
+                warmup_steps_run=done, launch_us=launch_us)
 
 
 def measured_traffic(name):
@@ -323,63 +335,81 @@ def roofline(wl, us, name=None):
                 frac=round(achieved / BF16_PEAK_TFLOPS, 4), traffic=traffic)
 
 
-def cpu_baseline(torch, name, wl, ttir=None):
-    """Times the CPU restatement (1 thread) on a bounded sample of the workload."""
+def host_cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(torch, name, wl, headline):
+    """Times the CPU restatement (one thread) on a bounded sample of a workload of the five configurations, the way the
+    reference's own harness does (python/examples/benchmark.py:15-65): wall and process time per repeat, mean / min / std.
+    The headline's sample is sized for 10-30 s of CPU work, the others for about a second.  None for other workloads
+    (there is no restatement of theirs to time)."""
     from oracle import cpu
     torch.manual_seed(0)
-    if "lanes" in wl:
-        seconds, frac, sample = wl["lanes"](ttir)
-        full_seconds = seconds / frac
-        return dict(value=float(f"{wl['work'] / full_seconds / 1e9:.4g}"), unit="GB/s", cores=1, kind="port",
-                    sample=sample + " (lane-level interpreter of the kernel's TTIR)", seconds_full_workload=float(f"{full_seconds:.4g}"),
-                    host_cores_available=os.cpu_count())
+    small = not headline
 
     def timed(fn, repeats):
-        ts = []
+        wall, proc = [], []
         for _ in range(repeats):
-            t0 = time.perf_counter()
+            w0, p0 = time.perf_counter(), time.process_time()
             fn()
-            ts.append(time.perf_counter() - t0)
-        return sum(ts) / len(ts), min(ts)
+            wall.append(time.perf_counter() - w0)
+            proc.append(time.process_time() - p0)
+        stat = lambda v: dict(mean=float(f"{sum(v) / len(v):.4g}"), min=float(f"{min(v):.4g}"),
+                              std=float(f"{(sum((t - sum(v) / len(v)) ** 2 for t in v) / len(v)) ** 0.5:.3g}"))
+        return sum(wall) / len(wall), stat(wall), stat(proc)
 
     if name.startswith("cfg1"):
         n = 98432 if name == "cfg1" else 1 << 24
         x, y = torch.rand(n), torch.rand(n)
-        mean, best = timed(lambda: cpu.vec_add(x, y), 20)
-        frac, sample = n * 12 / wl["work"], f"N={n}, 20 repeats"
+        repeats = 20 if small else (2000 if name == "cfg1" else 100)
+        mean, wall, proc = timed(lambda: cpu.vec_add(x, y), repeats)
+        frac, sample = n * 12 / wl["work"], f"N={n}, {repeats} repeats"
     elif name.startswith("cfg2"):
         rows = 4096
         x = torch.randn(rows, 781)
-        mean, best = timed(lambda: cpu.row_softmax(x), 10)
-        frac, sample = rows * 781 * 8 / wl["work"], f"{rows} rows, 10 repeats"
+        repeats = 10 if small else 500
+        mean, wall, proc = timed(lambda: cpu.row_softmax(x), repeats)
+        frac, sample = rows * 781 * 8 / wl["work"], f"{rows} rows, {repeats} repeats"
     elif name == "cfg3":
-        rows = 1024
+        rows = 1024 if small else 4096
         x = torch.randn(rows, 8192).half()
         w, b = torch.randn(8192).half(), torch.randn(8192).half()
-        mean, best = timed(lambda: cpu.layer_norm_fwd(x, w, b, 1e-5), 5)
-        frac, sample = rows / 4096, f"{rows} of 4096 rows, 5 repeats"
+        repeats = 3 if small else 30
+        mean, wall, proc = timed(lambda: cpu.layer_norm_fwd(x, w, b, 1e-5), repeats)
+        frac, sample = rows / 4096, f"{rows} of 4096 rows, {repeats} repeats"
     elif name == "cfg4":
         a = (torch.randn(4096, 4096) * 0.02).bfloat16()
         b = (torch.randn(4096, 4096) * 0.02).bfloat16()
         out = torch.zeros(4096, 4096, dtype=torch.bfloat16)
-        progs = 8
-        mean, best = timed(lambda: cpu.matmul_tiles(a, b, pids=(0, progs), out=out), 1)
-        frac, sample = progs / 1024, f"{progs} of 1024 programs (identical work each), 1 run"
-    else:
+        progs, repeats = (8, 1) if small else (32, 3)
+        mean, wall, proc = timed(lambda: cpu.matmul_tiles(a, b, pids=(0, progs), out=out), repeats)
+        frac, sample = progs / 1024, f"{progs} of 1024 programs (identical work each), {repeats} repeats"
+    elif name == "cfg5":
         a = torch.randn(16, 8192).half()
         w = torch.randint(-127, 128, (8192, 28672), dtype=torch.int8)
         s = (0.001 + 0.009 * torch.rand(28672)).half()
         out = torch.zeros(16, 28672, dtype=torch.float16)
-        ys = 16
-        mean, best = timed(lambda: cpu.w8a16_matmul(a, w, s, ys=(0, ys), out=out), 1)
-        frac, sample = ys / 224, f"{ys} of 224 column blocks, 1 run"
+        ys, repeats = (16, 1) if small else (112, 3)
+        mean, wall, proc = timed(lambda: cpu.w8a16_matmul(a, w, s, ys=(0, ys), out=out), repeats)
+        frac, sample = ys / 224, f"{ys} of 224 column blocks, {repeats} repeats"
+    else:
+        return None
     full_seconds = mean / frac
     if wl["bound"] == "hbm":
         value, unit = wl["work"] / full_seconds / 1e9, "GB/s"
     else:
         value, unit = wl["work"] / full_seconds / 1e12, "TFLOP/s"
     return dict(value=float(f"{value:.4g}"), unit=unit, cores=1, kind="port", sample=sample,
-                seconds_full_workload=float(f"{full_seconds:.4g}"), host_cores_available=os.cpu_count())
+                seconds_full_workload=float(f"{full_seconds:.4g}"), wall_seconds_per_repeat=wall, process_seconds_per_repeat=proc,
+                host_cpu=host_cpu_model(), host_cores_available=os.cpu_count())
 
 
 def main():
@@ -418,12 +448,14 @@ def main():
         wl = W[name]
         steps = args.steps if wl["set_bytes"] < 1e9 else max(10, args.steps // 10)
         t = time_workload(torch, spy, wl, steps, args.warmup, args.rotating_only)
-        entry = dict(workload=wl["desc"], us=round(t["us"], 3), kernel=t["kernel"], steps=steps,
+        entry = dict(workload=wl["desc"], us=round(t["us"], 3), launch_us=t["launch_us"], kernel=t["kernel"], steps=steps,
                      rotating_buffer_sets=t["sets"], warmup_steps_run=t["warmup_steps_run"], frontend_us_per_launch=round(t["frontend_us"], 1),
                      roofline=roofline(wl, t["us"], name), dtype=wl["dtype"], algorithmic_work=wl["work"],
                      same_buffers=dict(us=round(t["hot_us"], 3), frac=roofline(wl, t["hot_us"])["frac"]))
-        if not args.no_cpu and (name == args.workload or "lanes" in wl or not name.endswith(("2p28", "1m", "2p26", "2048"))):
-            entry["cpu_baseline"] = cpu_baseline(torch, name, wl, t.get("ttir"))
+        if not args.no_cpu and (name == args.workload or name in ("cfg1", "cfg2", "cfg3", "cfg4", "cfg5")):
+            base = cpu_baseline(torch, name, wl, headline=name == args.workload)
+            if base is not None:
+                entry["cpu_baseline"] = base
         kernels[name] = entry
     head = kernels[args.workload]
     wl = W[args.workload]

@@ -144,7 +144,9 @@ def test_cfg3_layernorm(K, oracle_cpu):
 
 @pytest.mark.parametrize("M,N,dtype", [(1151, 8192, torch.float16), (17, 1000, torch.float16), (5, 8191, torch.float16),
                                       (3, 64, torch.float16), (9, 16384, torch.float16), (2, 20000, torch.float16),
-                                      (33, 4096, torch.bfloat16), (4, 777, torch.bfloat16)])
+                                      (33, 4096, torch.bfloat16), (4, 777, torch.bfloat16),
+                                      # enough whole rows for workgroups that walk several rows each, in uneven numbers
+                                      (4100, 8192, torch.bfloat16), (8200, 4096, torch.float16), (16390, 2048, torch.float16)])
 def test_layernorm_shapes(K, oracle_cpu, M, N, dtype):
     x, w, b = _ln_inputs(M, N, dtype, seed=N)
     y, mean, rstd = _run_ln(K, x, w, b, 1e-5)
@@ -802,9 +804,23 @@ def test_errors_surface_as_python_exceptions(K):
     with pytest.raises(NotImplementedError, match="bytes of LDS"):
         big = torch.zeros(128 * 128, device=DEV)
         X.small_dot[(1,)](big, big, big, B=128)                        # a large product outside the tiled matmul shapes
-    with pytest.raises(NotImplementedError, match="one program per output tile"):
-        a = torch.zeros(256, 256, dtype=torch.bfloat16, device=DEV)
-        K.matmul_tiles[(3,)](a, a, a, 256, 256, 256, 256, 1, 256, 1, 256, 1, BM=128, BN=128, BK=64, GROUP_M=8)
+
+
+def test_gemm_with_a_grid_that_is_not_the_tile_grid_runs_program_by_program(K):
+    # three programs for four output tiles: not a dense product, so the matrix-product kernels decline at launch and
+    # the generic family runs the three programs, as the reference's serial loop would; the fourth tile stays untouched
+    torch.manual_seed(4)
+    a = (torch.randn(256, 256) * 0.1).bfloat16().to(DEV)
+    b = (torch.randn(256, 256) * 0.1).bfloat16().to(DEV)
+    c = torch.full((256, 256), 5.0, dtype=torch.bfloat16, device=DEV)
+    k = K.matmul_tiles[(3,)](a, b, c, 256, 256, 256, 256, 1, 256, 1, 256, 1, BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and k.function.last_kernel == "tile_program (hipRTC)"
+    ref = a.float() @ b.float()
+    for tm, tn in [(0, 0), (1, 0), (0, 1)]:      # programs 0, 1, 2 in the kernel's grouped order
+        blk = (slice(128 * tm, 128 * tm + 128), slice(128 * tn, 128 * tn + 128))
+        assert relfro(c[blk].float(), ref[blk]) <= 1e-2
+    assert torch.equal(c[128:, 128:].cpu(), torch.full((128, 128), 5.0, dtype=torch.bfloat16))
 
 
 def test_plan_handle_is_loaded_once(K):

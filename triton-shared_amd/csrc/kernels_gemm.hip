@@ -268,7 +268,7 @@ __device__ __forceinline__ float4 load_through(float4 *src) {
 // The counters are zero between launches (whoever allocates them clears them once).  Launches
 // that share a workspace must not overlap.
 template <int NW, int DEPTH>
-__global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Params p, int steps_per_slice) {
+__global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Params p, int first_steps, int other_steps) {
   extern __shared__ float4 w8_lds[];  // [NW][16][64]
   __shared__ int is_last;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -298,8 +298,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
 #pragma unroll
   for (int c = 0; c < 16; c++) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  const int step_begin = slice * steps_per_slice;
-  const int step_end = min(step_begin + steps_per_slice, (int)(p.K / 32));
+  // slice 0 takes first_steps steps of 32 rows, every other slice other_steps
+  const int step_begin = slice == 0 ? 0 : first_steps + (slice - 1) * other_steps;
+  const int step_end = min(step_begin + (slice == 0 ? first_steps : other_steps), (int)(p.K / 32));
   const int8_t *w_lane = p.w + (int64_t)(8 * g) * p.ldw + n0 + 16 * j;
   const uint16_t *a_lane = (const uint16_t *)p.a + (int64_t)min(j, (int)p.M - 1) * p.lda + 8 * g;
 
@@ -366,12 +367,35 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
   }
   if (p.split > 1) {
     float4 *slots = reinterpret_cast<float4 *>(p.workspace) + (int64_t)slab * p.split * 1024;
+    int *counter = p.counters + slab;
+    bool others_done = false;
+    if (slice == 0) {
+      // Slice 0 is given slightly more of K than the others, so it usually ends last: if every other slice has arrived
+      // already, nobody needs this slice's tile in memory, and the write, its acknowledgement and the counter update
+      // drop out of the kernel's tail.  (If not, slice 0 goes the way of the others below.)
+      if (tid == 0) is_last = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.split - 1;
+      __syncthreads();
+      others_done = is_last;
+      __syncthreads();  // is_last is written again below
+    }
+    if (others_done) {
+      if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int e = 0; e < PER; e++) {
+        const int idx = tid + e * NW * 64;
+        float4 t = tot[e];
+        for (int sl = 1; sl < p.split; sl++) {  // slice order, as in the general case: the sum does not depend on who arrived when
+          float4 u = load_through(slots + sl * 1024 + idx);
+          t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+        }
+        tot[e] = t;
+      }
+    } else {
 #pragma unroll
     for (int e = 0; e < PER; e++) store_through(slots + slice * 1024 + tid + e * NW * 64, tot[e]);
     __builtin_amdgcn_s_waitcnt(0);  // the stores have been acknowledged: the tile is in memory
     __syncthreads();                // ... every wavefront's part of it
     if (tid == 0) {
-      int *counter = p.counters + slab;
       int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       is_last = before == p.split - 1;
       if (before == p.split - 1) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -388,6 +412,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
         else { t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w; }
       }
       tot[e] = t;
+    }
     }
   }
   // to row-major through LDS, then 16-byte stores of eight fp16 values
@@ -520,13 +545,13 @@ void w8_launch(const GemmW8A16Params &p, int steps_per_slice, hipStream_t s) {
 }
 
 template <int NW, int DEPTH>
-hipError_t w8_launch_wide(const GemmW8A16Params &p, int steps_per_slice, hipStream_t s) {
+hipError_t w8_launch_wide(const GemmW8A16Params &p, int first_steps, int other_steps, hipStream_t s) {
   constexpr size_t lds = (size_t)NW * 16 * 64 * sizeof(float4);
   static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_w8a16_wide_kernel<NW, DEPTH>),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return attr;
   dim3 grid((unsigned)(p.N / W8_COLS_WIDE), p.split);
-  hipLaunchKernelGGL((gemm_w8a16_wide_kernel<NW, DEPTH>), grid, dim3(NW * 64), lds, s, p, steps_per_slice);
+  hipLaunchKernelGGL((gemm_w8a16_wide_kernel<NW, DEPTH>), grid, dim3(NW * 64), lds, s, p, first_steps, other_steps);
   return hipGetLastError();
 }
 }  // namespace
@@ -549,9 +574,17 @@ hipError_t launch_gemm_w8a16(const GemmW8A16Params &p, hipStream_t s, const char
   const bool wide = fast && c.cw == 16 && ((uintptr_t)p.w & 15) == 0;
   if (wide) {
     *name = "gemm_w8a16_wide_kernel";
+    // slice 0 gets `bias` steps more than an even share (see the kernel's tail), taken evenly from the others
+    int first = sps, other = sps;
+    if (p.split > 1) {
+      static const char *bias_env = getenv("TTS_W8_BIAS");  // tuning aid
+      const int bias = bias_env ? atoi(bias_env) : 4;
+      const int take = (bias + p.split - 2) / (p.split - 1);  // per other slice
+      if (sps - take >= 8 && sps * p.split == steps) { first = sps + take * (p.split - 1); other = sps - take; }
+    }
     // one step in flight per wavefront; two measured 1.2 us slower at the decode shape
-    if (c.depth == 2) return w8_launch_wide<8, 2>(p, sps, s);
-    return w8_launch_wide<8, 1>(p, sps, s);
+    if (c.depth == 2) return w8_launch_wide<8, 2>(p, first, other, s);
+    return w8_launch_wide<8, 1>(p, first, other, s);
   }
   *name = "gemm_w8a16_kernel";
   if (!fast) w8_launch<W8_WAVES, 2, false>(p, sps, s);

@@ -14,6 +14,8 @@
 // FMA contraction and no fast-math (backend/compiler.py:127-129,172-173).
 #include "kernels.h"
 
+#include <type_traits>
+
 namespace tts {
 
 namespace {
@@ -372,6 +374,135 @@ __global__ __launch_bounds__(256, CPT <= 4 ? 8 : 4) void layernorm_fwd_kernel(La
   }
 }
 
+// The same row arithmetic in a workgroup that walks rows blockIdx.x, blockIdx.x + gridDim.x, ...: the weight and bias
+// chunks a thread needs are read once and stay in registers (packed), and the loads of the next row are issued before
+// the current row is reduced, so a workgroup always has a row in flight while it computes and stores another.
+// Measured on fp16 [4096, 8192] with the rows coming from HBM: one workgroup per row 27.4 us; 1024 / 512 / 256
+// workgroups walking rows 26.3 / 25.0 / 24.4 us (a plain copy of the same bytes: 23.4 us).  What the row-per-workgroup
+// kernel loses is the 32 KB of w and b that every row fetches again through L2: taking those loads out of it, and
+// nothing else, gives 23.8 us.  512 or 1024 threads per workgroup, a third row in flight and nontemporal row loads
+// gain nothing or lose.  [8192, 8192]: 51.7 -> 44.8 us (6.0 TB/s).
+// For one-dimensional grids, rows of exactly CPT * 2048 elements starting 16-byte aligned, w and b the same for every row.
+template <bool BF16, int CPT>
+__global__ __launch_bounds__(256) void layernorm_fwd_persistent_kernel(LayerNormParams p, int rows) {
+  __shared__ float red[2][2][4];  // [which reduction][row parity][wavefront]: one barrier per reduction
+  const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+  const int N = (int)p.N;
+  const uint16_t *__restrict__ xb = (const uint16_t *)p.x + p.x_off.c0;
+  uint16_t *__restrict__ yb = (uint16_t *)p.y + p.y_off.c0;
+  const uint16_t *__restrict__ w = (const uint16_t *)p.w + p.w_off.c0;
+  const uint16_t *__restrict__ b = (const uint16_t *)p.b + p.b_off.c0;
+  uint4 wq[CPT], bq[CPT];
+#pragma unroll
+  for (int c = 0; c < CPT; c++) {
+    wq[c] = *reinterpret_cast<const uint4 *>(w + (tid + c * 256) * 8);
+    bq[c] = *reinterpret_cast<const uint4 *>(b + (tid + c * 256) * 8);
+  }
+  // A row's loads are issued from inline assembly and waited for by hand (row_landed): left to the compiler, the wait
+  // for a row also waits for the next row's loads, issued just before (it does not count memory operations across the
+  // loop's back edge), and the rows do not overlap.
+  auto load_row = [&](u32x4_t (&q)[CPT], int r) {
+    const uint16_t *x = xb + (int64_t)r * p.x_off.c[0];
+#pragma unroll
+    for (int c = 0; c < CPT; c++) {
+      const uint16_t *src = x + (tid + c * 256) * 8;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(q[c]) : "v"(src) : "memory");
+    }
+  };
+  // Waits until at most `newer` vector memory operations issued after the row's loads are outstanding (they complete in
+  // order, so the row has landed), and ties the row's registers to the wait so that no use moves above it.
+  auto row_landed = [&](u32x4_t (&q)[CPT], int newer) {
+    switch (newer) {  // a constant after inlining; the instruction takes an immediate
+      case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+      case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+      case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+      case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+#pragma unroll
+    for (int c = 0; c < CPT; c++) asm volatile("" : "+v"(q[c]) : : "memory");
+  };
+  auto block_sum = [&](float v, int which, int parity) {
+    v = wave_sum(v);
+    if (lane == 0) red[which][parity][wave] = v;
+    __syncthreads();
+    return (red[which][parity][0] + red[which][parity][1]) + (red[which][parity][2] + red[which][parity][3]);
+  };
+  const float n_f = (float)N;  // arith.sitofp
+  auto process = [&](const u32x4_t (&raw)[CPT], int r, int parity) {
+    float v[CPT][8];
+#pragma unroll
+    for (int c = 0; c < CPT; c++)
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        v[c][2 * k] = Half<BF16>::up((uint16_t)(raw[c][k] & 0xffff));
+        v[c][2 * k + 1] = Half<BF16>::up((uint16_t)(raw[c][k] >> 16));
+      }
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < CPT; c++)
+#pragma unroll
+      for (int k = 0; k < 8; k++) s += v[c][k];
+    const float mean = block_sum(s, 0, parity) / n_f;
+    float s2 = 0.f;
+#pragma unroll
+    for (int c = 0; c < CPT; c++)
+#pragma unroll
+      for (int k = 0; k < 8; k++) {
+        const float d = v[c][k] - mean;
+        s2 += d * d;
+      }
+    const float var = block_sum(s2, 1, parity) / n_f;
+    const float rstd = 1.0f / sqrtf(var + p.eps);
+    uint16_t *y = yb + (int64_t)r * p.y_off.c[0];
+#pragma unroll
+    for (int c = 0; c < CPT; c++) {
+      // opaque to the optimiser: it would otherwise widen w and b to fp32 once, outside the row loop, and keep 16 more
+      // registers per chunk alive for it
+      asm volatile("" : "+v"(wq[c].x), "+v"(wq[c].y), "+v"(wq[c].z), "+v"(wq[c].w), "+v"(bq[c].x), "+v"(bq[c].y), "+v"(bq[c].z), "+v"(bq[c].w));
+      const uint32_t wv[4] = {wq[c].x, wq[c].y, wq[c].z, wq[c].w}, bv[4] = {bq[c].x, bq[c].y, bq[c].z, bq[c].w};
+      uint32_t o[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        const float y0 = (v[c][2 * k] - mean) * rstd * Half<BF16>::up((uint16_t)(wv[k] & 0xffff)) + Half<BF16>::up((uint16_t)(bv[k] & 0xffff));
+        const float y1 = (v[c][2 * k + 1] - mean) * rstd * Half<BF16>::up((uint16_t)(wv[k] >> 16)) + Half<BF16>::up((uint16_t)(bv[k] >> 16));
+        o[k] = (uint32_t)Half<BF16>::down(y0) | ((uint32_t)Half<BF16>::down(y1) << 16);
+      }
+      ntstore(reinterpret_cast<uint4 *>(y + (tid + c * 256) * 8), make_uint4(o[0], o[1], o[2], o[3]));
+    }
+    if (tid == 0) {
+      p.mean[p.mean_off.c0 + (int64_t)r * p.mean_off.c[0]] = mean;
+      p.rstd[p.rstd_off.c0 + (int64_t)r * p.rstd_off.c[0]] = rstd;
+    }
+  };
+  // Two register sets take turns, so that no row is copied from one to the other (a copy would wait for the loads).
+  // Past the last row a workgroup loads the last row again: the loads are unconditional, hence countable.  Between a
+  // row's loads and its use lie the next row's CPT loads and, from the second row on, the previous row's CPT stores
+  // (every wavefront issues all of them: the rows are whole) -- plus the two statistics stores of the first wavefront,
+  // which only make its wait stricter than necessary.
+  int r = blockIdx.x;
+  if (r >= rows) return;
+  const int step = gridDim.x, last = rows - 1;
+  u32x4_t even[CPT], odd[CPT];
+  load_row(even, r);
+  load_row(odd, min(r + step, last));
+  row_landed(even, CPT);
+  process(even, r, 0);
+  r += step;
+  while (r < rows) {
+    load_row(even, min(r + step, last));
+    row_landed(odd, 2 * CPT);
+    process(odd, r, 1);
+    r += step;
+    if (r >= rows) break;
+    load_row(odd, min(r + step, last));
+    row_landed(even, 2 * CPT);
+    process(even, r, 0);
+    r += step;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the surplus loads of the last row land before the registers go away
+}
+
 // Rows too long for the register file: three passes over global memory, the
 // second and third served by L2.
 template <bool BF16>
@@ -408,6 +539,35 @@ hipError_t launch_layernorm_t(const LayerNormParams &p, dim3 grid, hipStream_t s
   auto aligned = [](const Affine &a) { return (a.c0 | a.c[0] | a.c[1] | a.c[2]) % 8 == 0; };
   const bool fast = p.N % 8 == 0 && aligned(p.x_off) && aligned(p.y_off) && aligned(p.w_off) && aligned(p.b_off) &&
                     (((uintptr_t)p.x | (uintptr_t)p.y | (uintptr_t)p.w | (uintptr_t)p.b) & 15) == 0;
+  // Rows walked by persistent workgroups (see layernorm_fwd_persistent_kernel): whole rows of 2048, 4096 or 8192
+  // elements in one-dimensional grids with enough rows to amortise the walk (fewer, and the workgroup-per-row kernel
+  // measured faster), w and b the same for every row.  About 32 KB of row loads in flight per CU: one workgroup per CU
+  // for rows of 8192 elements, four for 4096, eight for 2048 (measured best of 1, 2, 4 and 8 per CU on [8192, 4096] and
+  // [16384, 2048]: 25.5 us against 26.3 and 26.5 us against 31.1 for a workgroup per row).
+  static const char *ln_env = getenv("TTS_LN");  // tuning aid: "0" = always one workgroup per row; "G" = G persistent workgroups
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    return n;
+  }();
+  const int cpt = chunks == 256 ? 1 : chunks == 512 ? 2 : chunks == 1024 ? 4 : 0;
+  int persistent_grid = cus * (cpt == 1 ? 8 : cpt == 2 ? 4 : 1);
+  int64_t min_rows = (int64_t)persistent_grid * (cpt == 4 ? 16 : 8);
+  if (ln_env) {
+    persistent_grid = atoi(ln_env);
+    min_rows = 2 * (int64_t)persistent_grid;
+  }
+  auto row_invariant = [](const Affine &a) { return (a.c[0] | a.c[1] | a.c[2]) == 0; };
+  if (fast && cpt && persistent_grid > 0 && grid.y == 1 && grid.z == 1 && (int64_t)grid.x >= min_rows && row_invariant(p.w_off) &&
+      row_invariant(p.b_off)) {
+    const int rows = (int)grid.x;
+    const dim3 pg((unsigned)persistent_grid);
+    if (cpt == 1) hipLaunchKernelGGL((layernorm_fwd_persistent_kernel<BF16, 1>), pg, dim3(256), 0, s, p, rows);
+    else if (cpt == 2) hipLaunchKernelGGL((layernorm_fwd_persistent_kernel<BF16, 2>), pg, dim3(256), 0, s, p, rows);
+    else hipLaunchKernelGGL((layernorm_fwd_persistent_kernel<BF16, 4>), pg, dim3(256), 0, s, p, rows);
+    *name = "layernorm_fwd_persistent_kernel";
+    return hipGetLastError();
+  }
 #define TTS_LN(CPT)                                                                                          \
   do {                                                                                                       \
     if (fast) hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, CPT, true>), grid, dim3(256), 0, s, p);        \

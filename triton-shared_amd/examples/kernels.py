@@ -276,3 +276,19 @@ def expert_rows_matmul(a_ptr, b_ptr, c_ptr, rows_ptr, expert_ptr, n_rows, K, N, 
         a_ptrs += BK
         b_ptrs += BK * s_bk
     tl.store(c_ptr + i[:, None] * s_cm + j[None, :], acc.to(c_ptr.dtype.element_ty), mask=ok[:, None] & (j[None, :] < N))
+
+
+# ---- the machine's stream ceilings, measured through this backend: a 1:1 read/write stream and a read-only stream
+@triton.jit
+def copy_blocks(x_ptr, z_ptr, n, BLOCK: tl.constexpr):
+    """z = x: one byte written for every byte read."""
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = i < n
+    tl.store(z_ptr + i, tl.load(x_ptr + i, mask=m), mask=m)
+
+
+@triton.jit
+def block_sums(x_ptr, out_ptr, n, BLOCK: tl.constexpr):
+    """out[p] = sum of block p of x: BLOCK elements read for one written."""
+    i = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    tl.store(out_ptr + tl.program_id(0), tl.sum(tl.load(x_ptr + i, mask=i < n, other=0.0), axis=0))
