@@ -111,16 +111,22 @@ def make_workloads(torch, triton, K):
         return dict(desc="LayerNorm fwd fp16 [4096, 8192], BLOCK=1024 looped, fp32 stats", work=work, bound="hbm",
                     dtype="f16", make=make, set_bytes=work)
 
-    def gemm():
+    def gemm(zeros=False):
         n = 4096
 
         def make():
-            a = (torch.randn(n, n, device=dev) * 0.02).bfloat16()
-            b = (torch.randn(n, n, device=dev) * 0.02).bfloat16()
+            if zeros:
+                a, b = torch.zeros(n, n, dtype=torch.bfloat16, device=dev), torch.zeros(n, n, dtype=torch.bfloat16, device=dev)
+            else:
+                a = (torch.randn(n, n, device=dev) * 0.02).bfloat16()
+                b = (torch.randn(n, n, device=dev) * 0.02).bfloat16()
             c = torch.empty(n, n, dtype=torch.bfloat16, device=dev)
             return lambda: K.matmul_tiles[(32 * 32,)](a, b, c, n, n, n, n, 1, n, 1, n, 1, BM=128, BN=128, BK=64, GROUP_M=8)
-        return dict(desc="matmul bf16 4096x4096x4096, BM=BN=128 BK=64, fp32 acc, bf16 out", work=2 * n ** 3,
-                    bound="mfma", dtype="bf16", make=make, set_bytes=3 * n * n * 2)
+        desc = "matmul bf16 4096x4096x4096, BM=BN=128 BK=64, fp32 acc, bf16 out"
+        if zeros:
+            desc = ("diagnostic, not a configuration: the cfg4 launch on all-zero operands (same kernel, same instruction stream; what is left of "
+                    "the difference to cfg4 is the power the data path draws when its bits toggle, which sets the clock)")
+        return dict(desc=desc, work=2 * n ** 3, bound="mfma", dtype="bf16", make=make, set_bytes=3 * n * n * 2)
 
     def w8a16():
         M, N, Kd = 16, 28672, 8192
@@ -223,6 +229,7 @@ def make_workloads(torch, triton, K):
     W["cfg5"] = w8a16()
     W["cfg1_2p28"] = vec_add(1 << 28)
     W["cfg2_1m"] = softmax(1 << 20)
+    W["diag_cfg4_zero_operands"] = gemm(zeros=True)
     W["stream_copy_2p28"] = stream_copy(1 << 28)
     W["stream_read_2p28"] = stream_read(1 << 28)
     W["next_fused_gelu_2p26"] = fused_gelu(1 << 26)

@@ -349,6 +349,34 @@ def test_w8a16_split_k_repeated_launches(K):
         prev = cd
 
 
+def test_w8a16_split_k_on_two_streams(K):
+    # one plan launched alternately on two streams: each stream has partial tiles and arrival counters of its own, so
+    # launches that overlap in time do not mix their K slices; every result equals the single-stream one bit for bit
+    M, N, Kd = 16, 1024, 8192
+    cases = []
+    for seed in range(6):
+        torch.manual_seed(100 + seed)
+        a = torch.randn(M, Kd).half().to(DEV)
+        w = torch.randint(-127, 128, (Kd, N), dtype=torch.int8).to(DEV)
+        s = (0.001 + 0.009 * torch.rand(N)).half().to(DEV)
+        cases.append((a, w, s, torch.zeros(M, N, dtype=torch.float16, device=DEV), torch.zeros(M, N, dtype=torch.float16, device=DEV)))
+
+    def run(a, w, s, c):
+        return K.w8a16_matmul[(1, N // 128)](a, w, s, c, M, N, Kd, a.stride(0), 1, w.stride(0), 1, c.stride(0), 1, BM=16, BN=128, BK=128)
+    for a, w, s, want, _ in cases:
+        k = run(a, w, s, want)
+    torch.cuda.synchronize()
+    assert int(k.function.describe_launch((1, N // 128, 1), [a.data_ptr(), w.data_ptr(), s.data_ptr(), want.data_ptr(), M, N, Kd, Kd, N, N])["split"]) > 1
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for rep in range(20):
+        for i, (a, w, s, _, got) in enumerate(cases):
+            with torch.cuda.stream(streams[i % 2]):
+                run(a, w, s, got)
+    torch.cuda.synchronize()
+    for a, w, s, want, got in cases:
+        assert torch.equal(got, want)
+
+
 # ----------------------------------------- launches and details the hand-written families decline
 @pytest.mark.parametrize("M,N,Kd,dtype", [(4096, 4096, 4096, torch.bfloat16), (200, 333, 150, torch.bfloat16), (512, 384, 200, torch.float16)])
 def test_gemm_with_column_major_b(K, M, N, Kd, dtype):

@@ -5,6 +5,8 @@
 // its launcher with g++ (backend/driver.py:274-345).  Every instruction becomes the same C
 // expression the interpreter evaluates, with contraction off, so both paths give identical bits.
 #include <hip/hip_runtime.h>
+
+#include <algorithm>
 #include <hip/hiprtc.h>
 #include <sys/stat.h>
 #include <unistd.h>
@@ -160,7 +162,7 @@ std::string source_of(const MapNParams &p) {
     os << "  const char *in" << k << " = (const char *)p.in[" << k << "] + affine(p.in_off[" << k << "]) * " << (p.in_type[k] == 0 ? 4 : 2) << ";\n";
   for (int j = 0; j < p.n_out; j++)
     os << "  char *out" << j << " = (char *)p.out[" << j << "] + affine(p.out_off[" << j << "]) * " << (p.out_type[j] == 0 ? 4 : 2) << ";\n";
-  os << "  for (int i = W * threadIdx.x; i < d; i += 256 * W) {\n    const int valid = d - i;\n";
+  os << "  for (int i = W * threadIdx.x; i < d; i += blockDim.x * W) {\n    const int valid = d - i;\n";
   for (int r = 0; r < p.n_regs; r++) os << "    float r" << r << "[W];\n";
   os << "    float prev[W];\n    for (int e = 0; e < W; e++) prev[e] = 0.f;\n";
   for (int k = 0; k < p.n_in; k++) {
@@ -346,7 +348,14 @@ hipError_t fused_map_launch(RtcModule *m, const MapNParams &p, int gx, int gy, i
   a.block = p.block;
   a.masked = p.masked;
   for (int q = 0; q < MAPN_MAX_IMM; q++) a.imm[q] = p.imm[q];
-  return rtc_launch(m, gx, gy, gz, 256, &a, sizeof a, s);
+  // as many threads as the block has chunks (8 elements of a 16-bit type, 4 of fp32 per thread and pass), in whole
+  // wavefronts: a block of 1024 fp16 values is 128 threads' worth, and idle wavefronts would only take up room
+  bool narrow = true;
+  for (int k = 0; k < p.n_in; k++) narrow = narrow && p.in_type[k] != 0;
+  for (int j = 0; j < p.n_out; j++) narrow = narrow && p.out_type[j] != 0;
+  const int chunks = (p.block + (narrow ? 8 : 4) - 1) / (narrow ? 8 : 4);
+  const int threads = std::min(256, std::max(64, (chunks + 63) / 64 * 64));
+  return rtc_launch(m, gx, gy, gz, threads, &a, sizeof a, s);
 }
 
 }  // namespace tts

@@ -86,16 +86,24 @@ struct tts_plan {
   std::list<std::string> lru;
   std::mutex mu;
   const char *last_kernel = "";
-  float *workspace = nullptr;  // split-K partial sums (device), owned by the plan
-  size_t workspace_bytes = 0;
-  int *counters = nullptr;     // split-K arrival counters (device), zero between launches
-  size_t counters_count = 0;
+  // Split-K partial sums and arrival counters (device memory, owned by the plan), one set per stream the plan has been
+  // launched on: launches on one stream run one after the other, launches on different streams may overlap and must
+  // not share them.  Counters are zero between launches.
+  struct SplitK {
+    float *workspace = nullptr;
+    size_t workspace_bytes = 0;
+    int *counters = nullptr;
+    size_t counters_count = 0;
+  };
+  std::unordered_map<void *, SplitK> split_k;
   RtcModule *fused = nullptr;  // the kernel compiled for this plan at its first launch (fused maps, tile programs)
   RtcModule *gemm_rtc[3] = {nullptr, nullptr, nullptr};  // matrix products with a fused epilogue: one kernel per tiling
   RtcModule *fallback = nullptr;  // the generic family's kernel for a matrix-product plan (launches the product kernels decline)
   ~tts_plan() {
-    if (workspace) (void)hipFree(workspace);
-    if (counters) (void)hipFree(counters);
+    for (auto &kv : split_k) {
+      if (kv.second.workspace) (void)hipFree(kv.second.workspace);
+      if (kv.second.counters) (void)hipFree(kv.second.counters);
+    }
     rtc_release(fused);
     rtc_release(fallback);
     for (RtcModule *m : gemm_rtc) rtc_release(m);
@@ -716,28 +724,30 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
             if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("clearing the split-K counters: ") + hipGetErrorString(e));
           }
         } else if (p.split > 1) {
-          size_t need = gemm_w8a16_workspace_bytes(p);
+          const size_t need = gemm_w8a16_workspace_bytes(p), ncount = gemm_w8a16_counters(p);
           std::lock_guard<std::mutex> lock(plan->mu);
-          if (plan->workspace_bytes < need) {
-            if (plan->workspace) (void)hipFree(plan->workspace);
-            plan->workspace = nullptr;
-            plan->workspace_bytes = 0;
-            hipError_t e = hipMalloc((void **)&plan->workspace, need);
+          tts_plan::SplitK &sk = plan->split_k[stream];
+          if (sk.workspace_bytes < need) {
+            // the stream's earlier launches may still be using the old buffer: hipFree waits for the device
+            if (sk.workspace) (void)hipFree(sk.workspace);
+            sk.workspace = nullptr;
+            sk.workspace_bytes = 0;
+            hipError_t e = hipMalloc((void **)&sk.workspace, need);
             if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(split-K workspace): ") + hipGetErrorString(e));
-            plan->workspace_bytes = need;
+            sk.workspace_bytes = need;
           }
-          size_t ncount = gemm_w8a16_counters(p);
-          if (plan->counters_count < ncount) {
-            if (plan->counters) (void)hipFree(plan->counters);
-            plan->counters = nullptr;
-            plan->counters_count = 0;
-            hipError_t e = hipMalloc((void **)&plan->counters, ncount * sizeof(int));
-            if (e == hipSuccess) e = hipMemset(plan->counters, 0, ncount * sizeof(int));
+          if (sk.counters_count < ncount) {
+            if (sk.counters) (void)hipFree(sk.counters);
+            sk.counters = nullptr;
+            sk.counters_count = 0;
+            hipError_t e = hipMalloc((void **)&sk.counters, ncount * sizeof(int));
+            if (e == hipSuccess) e = hipMemset(sk.counters, 0, ncount * sizeof(int));
+            if (e == hipSuccess) e = hipDeviceSynchronize();  // the fill has landed before a launch on any stream reads the counters
             if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(split-K counters): ") + hipGetErrorString(e));
-            plan->counters_count = ncount;
+            sk.counters_count = ncount;
           }
-          p.workspace = plan->workspace;
-          p.counters = plan->counters;
+          p.workspace = sk.workspace;
+          p.counters = sk.counters;
         }
         err = launch_gemm_w8a16(p, s, &kname);
         break;
