@@ -1394,32 +1394,64 @@ def test_gemm_epilogue_in_the_grouped_tile_order(K):
     assert torch.equal(c.float(), z + bias[:N][None, :] + 16.0 * bias[N:][:, None])
 
 
-def test_tile_program_matmul_with_gathered_rows_in_bf16():
-    """128 x 128 x 64 bf16 tile products whose A rows come through an index vector and whose weights are picked by a loaded
-    expert id (examples/kernels.py:expert_rows_matmul): not a dense product, so it runs as small-product code of the
-    generic family (operands staged in LDS in their 16-bit type, 32 x 32 MFMA blocks)."""
+@pytest.mark.parametrize("dtype,BM,family", [(torch.bfloat16, 128, "gemm"), (torch.float16, 128, "gemm"), (torch.bfloat16, 64, "tile_program")])
+def test_matmul_with_gathered_rows(dtype, BM, family):
+    """Tile products whose A rows come through an index vector and whose weights are picked by a loaded expert id
+    (examples/kernels.py:expert_rows_matmul, the shape of unstructured_ptr_used_in_loop.mlir): with blocks of 128 rows
+    the matrix-product kernel takes the index vector and the ids as they are; with smaller blocks the program runs as
+    small-product code of the generic family."""
     from triton_shared_amd.examples import kernels
     torch.manual_seed(18)
     tokens, kd, nd, experts = 300, 150, 256, 3
-    a = torch.randn(512, kd, device=DEV).bfloat16()
-    b = torch.randn(experts, kd, nd, device=DEV).bfloat16()
+    a = torch.randn(512, kd, device=DEV).to(dtype)
+    b = torch.randn(experts, kd, nd, device=DEV).to(dtype)
     rows = torch.randint(0, 512, (tokens,), device=DEV, dtype=torch.int32)
-    ids = torch.tensor([2, -1, 0], device=DEV, dtype=torch.int32)
-    c = torch.zeros(tokens, nd, device=DEV, dtype=torch.bfloat16)
-    k = kernels.expert_rows_matmul[(3, 2)](a, b, c, rows, ids, tokens, kd, nd, kd, kd * nd, nd, nd, BM=128, BN=128, BK=64)
+    blocks = triton.cdiv(tokens, BM)
+    ids = torch.tensor([2, -1, 0, 1, -1][:blocks], device=DEV, dtype=torch.int32)
+    c = torch.zeros(tokens, nd, device=DEV, dtype=dtype)
+    k = kernels.expert_rows_matmul[(blocks, 2)](a, b, c, rows, ids, tokens, kd, nd, kd, kd * nd, nd, nd, BM=BM, BN=128, BK=64)
     torch.cuda.synchronize()
-    assert k.function.family == "tile_program"
+    assert k.function.family == family
+    if family == "gemm":
+        assert k.function.last_kernel.startswith("gemm_mfma_kernel")
     want = torch.zeros(tokens, nd, dtype=torch.float64, device=DEV)
     for blk, e in enumerate(ids.tolist()):
+        r = slice(blk * BM, min(tokens, blk * BM + BM))
         if e >= 0:
-            r = slice(blk * 128, min(tokens, blk * 128 + 128))
             want[r] = a[rows[r].long()].double() @ b[e].double()
+        else:
+            assert torch.equal(c[r], torch.zeros_like(c[r]))          # a block whose expert id is negative is left alone
     assert ((c.double() - want).norm() / want.norm()) <= 1e-2
-    assert torch.equal(c[128:256], torch.zeros_like(c[128:256]))          # the block whose expert id is negative is left alone
+
+
+def test_matmul_with_gathered_rows_is_exact_on_selections():
+    # every expert's matrix selects and negates columns of its input rows: the result is exact, so a wrong row index, a
+    # wrong expert, a wrong pitch or a transposed operand cannot pass; 16-byte aligned pitches (the vector path) and
+    # rows picked more than once
+    import extra_kernels as X
+    torch.manual_seed(19)
+    tokens, kd, nd, experts = 1000, 256, 384, 4
+    a = torch.randint(-8, 9, (700, kd), device=DEV).bfloat16()
+    pick = torch.randint(0, kd, (experts, nd), device=DEV)
+    b = torch.zeros(experts, kd, nd, device=DEV, dtype=torch.bfloat16)
+    for e in range(experts):
+        b[e, pick[e], torch.arange(nd, device=DEV)] = -1.0
+    rows = torch.randint(0, 700, (tokens,), device=DEV, dtype=torch.int32)
+    ids = torch.randint(-1, experts, (triton.cdiv(tokens, 128),), device=DEV, dtype=torch.int32)
+    c = torch.full((tokens, nd), 5.0, device=DEV, dtype=torch.bfloat16)
+    k = X.grouped_rows_matmul[(triton.cdiv(tokens, 128), triton.cdiv(nd, 128))](a, b, c, rows, ids, tokens, kd, nd, kd, kd * nd, nd, nd, BM=128, BN=128, BK=64)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and k.function.last_kernel.startswith("gemm_mfma_kernel")
+    want = torch.full((tokens, nd), 5.0, device=DEV, dtype=torch.bfloat16)
+    for blk, e in enumerate(ids.tolist()):
+        r = slice(blk * 128, min(tokens, blk * 128 + 128))
+        if e >= 0:
+            want[r] = -a[rows[r].long()][:, pick[e]]
+    assert torch.equal(c, want)
 
 
 @pytest.mark.parametrize("M,N,K,kernel", [(512, 768, 96, "gemm_dma_kernel + epilogue"), (200, 300, 150, "gemm_mfma_kernel<128x128x64> + epilogue"),
-                                          (2100, 2060, 72, "gemm_mfma_kernel<256x256x32> + epilogue")])
+                                          (2100, 2060, 72, "gemm_mfma_kernel<128x128x64> + epilogue")])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_gemm_with_fused_epilogue(M, N, K, kernel, dtype):
     """The tutorial matmul's fused activation (test_matmul.py:98-99, 112-117): ops on the accumulator alone are compiled into

@@ -25,6 +25,14 @@ struct TtsGemmParams {
   int64_t lda, ldb, ldc;  // pitches in elements; the other stride of each matrix is 1
   int is_bf16;
   int a_trans, b_trans;   // A / B is column-major: element (m, k) of A is a[m + k * lda], (k, n) of B is b[k + n * ldb]
+  // Gathered operands (null / 0 for a plain product): row m of A is row a_rows[m] of the matrix at `a` (row-major A only);
+  // the rows of block m / b_block_rows multiply the matrix at b + b_block[m / b_block_rows] * b_block_stride elements,
+  // or nothing at all when that id is negative (their part of C is not written).
+  const int *a_rows;
+  const int *b_block;
+  int64_t b_block_stride;
+  int b_block_rows;
+  int gather_mul32;       // bit 0: a_rows[m] * lda, bit 1: id * b_block_stride is a 32-bit product that wraps, as the source computes it
 };
 
 namespace tts_gemm_device {
@@ -64,21 +72,43 @@ __device__ __forceinline__ uint4 load8(const uint16_t *p, int valid, bool vec) {
 }
 
 // ------------------------------------------------------------- 16-bit GEMM
-// Workgroup: 256 threads = 2 x 2 wavefronts; each wavefront owns TM x TN MFMA
-// tiles of 32 x 32.  A and B tiles are staged through LDS, both stored with K
-// contiguous ([row][k] and [col][k], pitch BK + 8 elements so that 16-byte
-// fragment reads of 32 consecutive rows hit distinct banks).  B is row-major
-// [K][N] in memory; it is transposed on the way into LDS by packing the two
-// K-neighbours of every column into one 32-bit word.
+// The kernel for any shape, any alignment, and operands that are row- or column-major.
+// Workgroup: 256 threads = 2 x 2 wavefronts; each wavefront owns TM x TN MFMA tiles of 32 x 32.  An operand tile is
+// R = BM = BN rows (rows of A, columns of B) by BK values of k and is staged through LDS (two buffers) in the form it
+// has in memory, with 16-byte loads and stores where alignment allows:
+//   k contiguous (A row-major, B column-major): LDS [r][k], pitch BK + 8 elements; a lane's MFMA operand (8 consecutive
+//     k of row lane % 32) is one 16-byte read, and 32 consecutive rows hit distinct banks;
+//   r contiguous (B row-major, A column-major): LDS [k][r], pitch R + 16 elements; `ds_read_b64_tr_b16` transposes on
+//     the way out -- within 16 lanes, lane i receives element i % 4 of the 8-byte rows addressed by lanes i / 4,
+//     i / 4 + 4, i / 4 + 8, i / 4 + 12, so lane j of a group addresses k row j / 4, elements 4 (j % 4) .. +3 of the
+//     group's 16, and two reads (k 0-3, k 4-7) make one operand.
+// Rows of A may be taken through an index vector (p.a_rows) and the base of B may depend on the block of rows
+// (p.b_block): a mixture-of-experts product is this kernel with both set.
 // `ep(acc, row, col)` maps an accumulator value to the value that is stored at (row, col) of C (the identity for a plain
 // product); it is only called for elements inside the problem.
+template <bool V>
+struct BoolConstant {
+  static constexpr bool value = V;
+};
+
+template <int BM, int BN, int BK>
+struct GemmStageLds {
+  static constexpr int A_ELEMS = (BM * (BK + 8) > BK * (BM + 16)) ? BM * (BK + 8) : BK * (BM + 16);
+  static constexpr int B_ELEMS = (BN * (BK + 8) > BK * (BN + 16)) ? BN * (BK + 8) : BK * (BN + 16);
+  static constexpr int BUFFER_ELEMS = A_ELEMS + B_ELEMS;
+  static constexpr int BYTES = 2 * BUFFER_ELEMS * 2;
+};
+
 template <bool BF16, int TM, int TN, int BK, class Ep>
 __device__ __forceinline__ void gemm_mfma_body(const GemmParams &p, int tiles_m, int tiles_n, const Ep &ep) {
-  constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32, PITCH = BK + 8;
-  constexpr int CA = BM * BK / 8 / 256;          // 16-byte chunks of A per thread
-  constexpr int UB = (BK / 2) * (BN / 8) / 256;  // 2x8 units of B per thread
-  #ifdef TTS_GEMM_RTC
-  __shared__ __align__(16) uint16_t smem[2 * (BM + BN) * PITCH];
+  constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32;
+  constexpr int PK = BK + 8;   // pitch of a k-contiguous tile
+  constexpr int PR = BM + 16;  // pitch of an r-contiguous tile
+  constexpr int CA = BM * BK / 8 / 256;  // 16-byte chunks of an operand tile per thread
+  static_assert(BM == BN, "both operands are staged by the same routines");
+  using Lds = GemmStageLds<BM, BN, BK>;
+#ifdef TTS_GEMM_RTC
+  __shared__ __align__(16) uint16_t smem[2 * Lds::BUFFER_ELEMS];
 #else
   extern __shared__ __align__(16) uint16_t smem[];
 #endif
@@ -98,71 +128,69 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams &p, int tiles_m,
 
   const uint16_t *__restrict__ A = (const uint16_t *)p.a;
   const uint16_t *__restrict__ B = (const uint16_t *)p.b;
+  if (p.b_block) {  // the rows of this tile multiply a matrix of their own; a negative id: nothing to do for them
+    const int which = p.b_block[m0 / p.b_block_rows];
+    if (which < 0) return;
+    B += (p.gather_mul32 & 2) ? (int64_t)(int)((uint32_t)which * (uint32_t)p.b_block_stride) : (int64_t)which * p.b_block_stride;
+  }
   const bool a_vec = (p.lda % 8 == 0) && (((uintptr_t)A & 15) == 0);
   const bool b_vec = (p.ldb % 8 == 0) && (((uintptr_t)B & 15) == 0);
   const int K = (int)p.K;
-  static_assert(BM == BN && CA == 2 * UB, "both operands are staged by the same two routines");
 
-  // An operand tile is R = BM = BN rows (rows of A, columns of B) by BK values of k.  In memory either k is the
-  // contiguous index (A row-major, B column-major: element (r, k) at P[r * ld + k]) or r is (A column-major, B
-  // row-major: P[k * ld + r]).  Either way the tile lands in LDS as [r][k]; in the second form the two K-neighbours of
-  // eight consecutive r are packed into 32-bit words on the way.
-  auto load_k_contiguous = [&](uint4 (&reg)[CA], const uint16_t *P, int64_t ld, int64_t r0, int64_t rows, bool vec, int k0) {
+  // where this thread's chunks of the tiles are: (row, k chunk) of a k-contiguous tile, (k, row chunk) of an
+  // r-contiguous one; element offsets of the chunks' rows in memory (-1: outside the problem)
+  int64_t a_at[CA], b_at[CA];
+#pragma unroll
+  for (int j = 0; j < CA; j++) {
+    const int c = tid + 256 * j;
+    if (p.a_trans) {
+      a_at[j] = m0 + (c % (BM / 8)) * 8;  // first of 8 rows; the k row moves with the loop
+    } else {
+      const int64_t gr = m0 + c / (BK / 8);
+      if (gr >= p.M) a_at[j] = -1;
+      else if (!p.a_rows) a_at[j] = gr * p.lda;
+      else a_at[j] = (p.gather_mul32 & 1) ? (int64_t)(int)((uint32_t)p.a_rows[gr] * (uint32_t)p.lda) : (int64_t)p.a_rows[gr] * p.lda;
+    }
+    if (p.b_trans) {
+      const int64_t gn = n0 + c / (BK / 8);
+      b_at[j] = gn < p.N ? gn * p.ldb : -1;
+    } else {
+      b_at[j] = n0 + (c % (BN / 8)) * 8;
+    }
+  }
+  uint4 ra[CA], rb[CA];
+  auto load_operand = [&](uint4 (&reg)[CA], const uint16_t *P, bool r_contiguous, const int64_t (&at)[CA], int64_t ld, int64_t rows, bool vec, int k0) {
 #pragma unroll
     for (int j = 0; j < CA; j++) {
-      int c = tid + 256 * j, row = c / (BK / 8), kc = c % (BK / 8);
-      int64_t gr = r0 + row;
-      int gk = k0 + kc * 8;
-      reg[j] = gr < rows ? load8(P + gr * ld + gk, K - gk, vec) : make_uint4(0, 0, 0, 0);
-    }
-  };
-  auto store_k_contiguous = [&](const uint4 (&reg)[CA], uint16_t *S) {
-#pragma unroll
-    for (int j = 0; j < CA; j++) {
-      int c = tid + 256 * j, row = c / (BK / 8), kc = c % (BK / 8);
-      *reinterpret_cast<uint4 *>(S + row * PITCH + kc * 8) = reg[j];
-    }
-  };
-  auto load_r_contiguous = [&](uint4 (&reg)[CA], const uint16_t *P, int64_t ld, int64_t r0, int64_t rows, bool vec, int k0) {
-#pragma unroll
-    for (int j = 0; j < UB; j++) {
-      int u = tid + 256 * j, kp = u / (BN / 8), nc = u % (BN / 8);
-      int gk = k0 + 2 * kp;
-      int64_t gn = r0 + nc * 8;
-      int valid = (int)min((int64_t)8, rows - gn);
-#pragma unroll
-      for (int r = 0; r < 2; r++)
-        reg[2 * j + r] = (gk + r < K && valid > 0) ? load8(P + (int64_t)(gk + r) * ld + gn, valid, vec) : make_uint4(0, 0, 0, 0);
-    }
-  };
-  auto store_r_contiguous = [&](const uint4 (&reg)[CA], uint16_t *S) {
-#pragma unroll
-    for (int j = 0; j < UB; j++) {
-      int u = tid + 256 * j, kp = u / (BN / 8), nc = u % (BN / 8);
-      uint32_t r0[4] = {reg[2 * j].x, reg[2 * j].y, reg[2 * j].z, reg[2 * j].w};
-      uint32_t r1[4] = {reg[2 * j + 1].x, reg[2 * j + 1].y, reg[2 * j + 1].z, reg[2 * j + 1].w};
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        uint32_t lo = (r0[i] & 0xffffu) | (r1[i] << 16);          // row 2i:   k, k+1
-        uint32_t hi = (r0[i] >> 16) | (r1[i] & 0xffff0000u);      // row 2i+1: k, k+1
-        *reinterpret_cast<uint32_t *>(S + (nc * 8 + 2 * i) * PITCH + 2 * kp) = lo;
-        *reinterpret_cast<uint32_t *>(S + (nc * 8 + 2 * i + 1) * PITCH + 2 * kp) = hi;
+      const int c = tid + 256 * j;
+      if (r_contiguous) {
+        const int gk = k0 + c / (BM / 8);
+        const int valid = (int)min((int64_t)8, rows - at[j]);
+        reg[j] = (gk < K && valid > 0) ? load8(P + (int64_t)gk * ld + at[j], valid, vec) : make_uint4(0, 0, 0, 0);
+      } else {
+        const int gk = k0 + (c % (BK / 8)) * 8;
+        reg[j] = at[j] >= 0 ? load8(P + at[j] + gk, K - gk, vec) : make_uint4(0, 0, 0, 0);
       }
     }
   };
-  uint4 ra[CA], rb[CA];
-  auto load_tiles = [&](int k0) {
-    if (p.a_trans) load_r_contiguous(ra, A, p.lda, m0, p.M, a_vec, k0);
-    else load_k_contiguous(ra, A, p.lda, m0, p.M, a_vec, k0);
-    if (p.b_trans) load_k_contiguous(rb, B, p.ldb, n0, p.N, b_vec, k0);
-    else load_r_contiguous(rb, B, p.ldb, n0, p.N, b_vec, k0);
+  auto store_operand = [&](const uint4 (&reg)[CA], uint16_t *S, bool r_contiguous) {
+#pragma unroll
+    for (int j = 0; j < CA; j++) {
+      const int c = tid + 256 * j;
+      if (r_contiguous) *reinterpret_cast<uint4 *>(S + (c / (BM / 8)) * PR + (c % (BM / 8)) * 8) = reg[j];
+      else *reinterpret_cast<uint4 *>(S + (c / (BK / 8)) * PK + (c % (BK / 8)) * 8) = reg[j];
+    }
   };
-  auto store_tiles = [&](int buf) {
-    uint16_t *As = smem + buf * (BM + BN) * PITCH, *Bs = As + BM * PITCH;
-    if (p.a_trans) store_r_contiguous(ra, As);
-    else store_k_contiguous(ra, As);
-    if (p.b_trans) store_k_contiguous(rb, Bs);
-    else store_r_contiguous(rb, Bs);
+  // a lane's MFMA operand for the 32 rows starting at `row0` of a staged tile, k = ks * 16 + 8 (lane / 32) .. +7
+  auto fragment = [&](const uint16_t *S, bool r_contiguous, int row0, int ks) -> uint4 {
+    if (!r_contiguous) return *reinterpret_cast<const uint4 *>(S + (row0 + (lane & 31)) * PK + ks * 16 + 8 * (lane >> 5));
+    const int g = lane >> 4, j = lane & 15;
+    const uint16_t *at = S + (ks * 16 + 8 * (g >> 1) + (j >> 2)) * PR + row0 + 16 * (g & 1) + 4 * (j & 3);
+    typedef short s16x4_t __attribute__((ext_vector_type(4)));
+    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3))) *)((__attribute__((address_space(3))) void *)at));
+    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4_t __attribute__((address_space(3))) *)((__attribute__((address_space(3))) void *)(at + 4 * PR)));
+    const uint2 l2 = __builtin_bit_cast(uint2, lo), h2 = __builtin_bit_cast(uint2, hi);
+    return make_uint4(l2.x, l2.y, h2.x, h2.y);
   };
 
   f32x16 acc[TM][TN];
@@ -173,32 +201,51 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams &p, int tiles_m,
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
+  // The forms of the two operands are fixed for the launch: the loop is compiled once per combination, so that inside
+  // it the loads, the LDS traffic and the MFMAs are straight-line code the compiler can overlap.
   const int nk = (K + BK - 1) / BK;
-  if (nk > 0) {
-    load_tiles(0);
-    store_tiles(0);
-  }
-  __syncthreads();
-  for (int kt = 0; kt < nk; kt++) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) load_tiles((kt + 1) * BK);
-    const uint16_t *As = smem + cur * (BM + BN) * PITCH, *Bs = As + BM * PITCH;
-    const uint16_t *a_base = As + (wm * TM * 32 + (lane & 31)) * PITCH + 8 * (lane >> 5);
-    const uint16_t *b_base = Bs + (wn * TN * 32 + (lane & 31)) * PITCH + 8 * (lane >> 5);
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ks++) {
-      uint4 af[TM], bf[TN];
-#pragma unroll
-      for (int i = 0; i < TM; i++) af[i] = *reinterpret_cast<const uint4 *>(a_base + i * 32 * PITCH + ks * 16);
-#pragma unroll
-      for (int j = 0; j < TN; j++) bf[j] = *reinterpret_cast<const uint4 *>(b_base + j * 32 * PITCH + ks * 16);
-#pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++) acc[i][j] = mfma32<BF16>(af[i], bf[j], acc[i][j]);
+  auto sweep_k = [&](auto a_form, auto b_form) {
+    constexpr bool a_r = decltype(a_form)::value, b_r = decltype(b_form)::value;  // r-contiguous in memory and in LDS
+    auto load_tiles = [&](int k0) {
+      load_operand(ra, A, a_r, a_at, p.lda, p.M, a_vec, k0);
+      load_operand(rb, B, b_r, b_at, p.ldb, p.N, b_vec, k0);
+    };
+    auto store_tiles = [&](int buf) {
+      uint16_t *As = smem + buf * Lds::BUFFER_ELEMS, *Bs = As + Lds::A_ELEMS;
+      store_operand(ra, As, a_r);
+      store_operand(rb, Bs, b_r);
+    };
+    if (nk > 0) {
+      load_tiles(0);
+      store_tiles(0);
     }
-    if (kt + 1 < nk) store_tiles(cur ^ 1);
     __syncthreads();
+    for (int kt = 0; kt < nk; kt++) {
+      const int cur = kt & 1;
+      if (kt + 1 < nk) load_tiles((kt + 1) * BK);
+      const uint16_t *As = smem + cur * Lds::BUFFER_ELEMS, *Bs = As + Lds::A_ELEMS;
+#pragma unroll
+      for (int ks = 0; ks < BK / 16; ks++) {
+        uint4 af[TM], bf[TN];
+#pragma unroll
+        for (int i = 0; i < TM; i++) af[i] = fragment(As, a_r, wm * TM * 32 + i * 32, ks);
+#pragma unroll
+        for (int j = 0; j < TN; j++) bf[j] = fragment(Bs, b_r, wn * TN * 32 + j * 32, ks);
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+          for (int j = 0; j < TN; j++) acc[i][j] = mfma32<BF16>(af[i], bf[j], acc[i][j]);
+      }
+      if (kt + 1 < nk) store_tiles(cur ^ 1);
+      __syncthreads();
+    }
+  };
+  if (p.a_trans) {
+    if (p.b_trans) sweep_k(BoolConstant<true>(), BoolConstant<false>());
+    else sweep_k(BoolConstant<true>(), BoolConstant<true>());
+  } else {
+    if (p.b_trans) sweep_k(BoolConstant<false>(), BoolConstant<false>());
+    else sweep_k(BoolConstant<false>(), BoolConstant<true>());
   }
 
   // epilogue: lane holds column (lane % 32), rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile

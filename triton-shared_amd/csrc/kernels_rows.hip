@@ -457,9 +457,8 @@ __global__ __launch_bounds__(256) void layernorm_fwd_persistent_kernel(LayerNorm
     uint16_t *y = yb + (int64_t)r * p.y_off.c[0];
 #pragma unroll
     for (int c = 0; c < CPT; c++) {
-      // opaque to the optimiser: it would otherwise widen w and b to fp32 once, outside the row loop, and keep 16 more
-      // registers per chunk alive for it
-      asm volatile("" : "+v"(wq[c].x), "+v"(wq[c].y), "+v"(wq[c].z), "+v"(wq[c].w), "+v"(bq[c].x), "+v"(bq[c].y), "+v"(bq[c].z), "+v"(bq[c].w));
+      // (the optimiser widens w and b to fp32 once, outside the row loop: 16 registers per chunk, which a workgroup
+      // that has a CU's register file nearly to itself can afford, and four operations per element and row saved)
       const uint32_t wv[4] = {wq[c].x, wq[c].y, wq[c].z, wq[c].w}, bv[4] = {bq[c].x, bq[c].y, bq[c].z, bq[c].w};
       uint32_t o[4];
 #pragma unroll

@@ -9,6 +9,8 @@
 
 namespace tts {
 
+static std::string generic_fallback(const Program &p);
+
 const char *family_name(Family f) {
   switch (f) {
     case Family::Map1D: return "map1d";
@@ -609,6 +611,126 @@ bool try_gemm(Plan &pl, bool w8a16) {
   return true;
 }
 
+// ----------------------------------------------------- gemm, gathered operands
+// The product of a mixture-of-experts layer (test/Conversion/TritonToUnstructured/unstructured_ptr_used_in_loop.mlir
+// has its shape): program (pm, pn) reads an id from memory -- negative: return at once --, takes BM rows of A through an
+// index vector, multiplies them with the matrix b + id * stride, and stores a BM x BN tile of C.  The reference lowers
+// the row gather to a loop of per-row copies (StructuredToMemref.cpp:855-993) and runs the rest as any other tiled
+// product; here the matrix-product kernel takes the index vector and the table of ids as they are.
+// The op structure is pinned by the signature; what the ops' leaves must be is checked here.
+const char *SIG_GEMM_GATHERED =
+    "v0=const:f32;v1=const:i32;v2=sload:i32.r0;v3=index;unless(v3){v4=iota;v5=index;v6=splat(v5);v7=arith.addi:i32(v6,v4);v8=index;"
+    "v9=splat(v8);v10=arith.cmpi.slt:i1(v7,v9);v11=load:i32.r1.m.o;v12=iota;v13=expand.1(v11);v14=index;v15=splat(v14);v16=arith.mu"
+    "li:i32(v13,v15);v17=expand.0(v12);v18=bcast(v17);v19=expand.1(v10);v20=bcast(v19);v21=arith.extsi:i64(v16);v22=bcast(v21);v23="
+    "arith.extsi:i64(v18);v24=arith.addi:i64(v22,v23);for[v25<-v24,v26<-v0]{v27=index;v28=splat(v27);v29=arith.cmpi.slt:i1(v17,v28)"
+    ";v30=bcast(v29);v31=arith.andi:i1(v20,v30);v32=load:{T}.r2.o;v33=load:{T}.r2.m.o;v34=dot(v32,v33,v26);v35=arith.extsi:i64(v1);"
+    "v36=arith.addi:i64(v25,v35);yield(v36,v34)}->v37,v38;v39=arith.truncf:{T}(v38);store:{T}.r2.m(v39);};";
+
+bool try_gemm_gathered(Plan &pl) {
+  std::string T;
+  if (pl.signature == subst(SIG_GEMM_GATHERED, "{T}", "bf16")) T = "bf16";
+  else if (pl.signature == subst(SIG_GEMM_GATHERED, "{T}", "f16")) T = "f16";
+  else return false;
+  const char *F = "gemm (gathered rows)";
+  Matcher m(pl.prog);
+  ExprPool &X = m.X;
+  if (m.all.size() != 39 || m.loops.size() != 1) return false;
+  SOp *acc0 = m.all[0], *step = m.all[1], *id = m.all[2], *cond = m.all[3], *unless = m.all[4], *lane_m = m.all[5], *row0 = m.all[6],
+      *n_rows = m.all[9], *rows = m.all[12], *lane_k = m.all[13], *pitch = m.all[15], *loop = m.all[26], *k_left = m.all[27],
+      *k_ok = m.all[31], *A = m.all[32], *Bm = m.all[33], *C = m.all[38];
+  if (A->acc.sizes.size() != 2 || Bm->acc.sizes.size() != 2 || C->acc.sizes.size() != 2) return false;
+  const int64_t BM = A->acc.sizes[0], BK = A->acc.sizes[1], BN = Bm->acc.sizes[1];
+  if (Bm->acc.sizes[0] != BK || C->acc.sizes[0] != BM || C->acc.sizes[1] != BN) refuse(F, "its block shapes do not compose");
+  if (acc0->fval != 0.0) refuse(F, "its accumulator does not start at 0");
+  if (BM % 128 != 0) refuse(F, "its blocks of rows are not whole 128-row kernel tiles");
+  if (step->ival != BK) refuse(F, "its row pointers do not advance by one K block per iteration");
+  if (unless->kind != SK::If || unless->ival != 1) return false;
+  // the id and the early return
+  if (id->acc.offsets.size() != 1 || id->acc.gather >= 0 || id->acc.mask_value >= 0) refuse(F, "its matrix id is not read from a plain address");
+  {
+    const Expr c = X.at(cond->expr);
+    if (c.k != EK::CmpSel || c.val != 0 || X.at(c.a).k != EK::Data || X.at(c.a).a != id->result || !m.is_const(c.b, 0) || !m.is_const(c.c, 1) ||
+        !m.is_const(c.d, 0))
+      refuse(F, "its early return is not `id < 0`");
+  }
+  // rows: which = rows_ptr[row0 + arange(BM)], masked against n_rows
+  if (lane_m->ival != 0 || lane_k->ival != 0) refuse(F, "its lane indices do not start at 0");
+  const int r0 = X.to_index(row0->expr), Mb = X.to_index(n_rows->expr);
+  {
+    int start, bound;
+    if (rows->acc.gather >= 0 || rows->acc.mask_value >= 0 || rows->acc.sizes.size() != 1 || rows->acc.sizes[0] != BM || !m.is_const(rows->acc.strides[0], 1) ||
+        X.to_index(rows->acc.offsets[0]) != r0 || rows->acc.dims.size() != 1 || !m.extent(rows->acc.dims[0], BM, start, bound) || start != r0 || bound != Mb ||
+        rows->acc.other_i != 0 || !rows->acc.mods.empty())
+      refuse(F, "its index vector is not rows_ptr[row0 + arange] masked against the row count");
+  }
+  if (!m.pid_free(Mb) || !m.loop_free(Mb) || !m.pid_free(pitch->expr) || !m.loop_free(pitch->expr)) refuse(F, "its row count or row pitch depends on the program id");
+  // the K loop: k0 = 0, BK, ... < K; the K mask is arange(BK) < K - k0
+  if (!m.is_const(loop->lb, 0) || !m.is_const(loop->step, BK) || !m.pid_free(loop->ub)) refuse(F, "its K loop is not range(0, K, BK)");
+  {
+    const Expr l = X.at(k_left->expr);
+    if (l.k != EK::Sub || l.a != loop->ub || X.at(l.b).k != EK::IV || X.at(l.b).a != loop->loop) refuse(F, "its K mask is not arange < K - k0");
+  }
+  // A: gathered through the carried block of offsets, masked by (row ok) & (k ok), padded with 0
+  if (A->acc.gather != loop->tile_args.at(0) || A->acc.mask_value != k_ok->result || !A->acc.has_other || A->acc.other_f != 0.0 || A->acc.other_value >= 0 ||
+      A->acc.offsets.size() != 1 || !m.is_const(A->acc.offsets[0], 0))
+    refuse(F, "its A rows are not read through the carried offsets with the row and K masks, padded with 0");
+  // B: a structured block below the matrix the id picks
+  if (Bm->acc.gather >= 0 || Bm->acc.mask_value >= 0 || !Bm->acc.mods.empty() || !C->acc.mods.empty()) refuse(F, "its B or C block is not structured");
+  Carried2D cb;
+  if (!carried_state(m, loop, Bm->acc, cb)) refuse(F, "its B pointer does not advance by a constant per K step");
+  int block_stride = -1;
+  bool mul32 = false;
+  {
+    int e = cb.init[0];
+    if (X.at(e).k == EK::Sext) { e = X.at(e).a; mul32 = true; }
+    const Expr mu = X.at(e);
+    if (mu.k != EK::Mul) refuse(F, "its B base is not id * stride");
+    auto is_id = [&](int x) { return X.at(x).k == EK::Data && X.at(x).a == id->result; };
+    if (is_id(mu.a)) block_stride = mu.b;
+    else if (is_id(mu.b)) block_stride = mu.a;
+    else refuse(F, "its B base is not id * stride");
+    if (mu.bits != 32) mul32 = false;
+    if (!m.pid_free(block_stride) || !m.loop_free(block_stride) || X.depends_on(block_stride, EK::Data)) refuse(F, "its matrix stride is not a launch constant");
+  }
+  const int c0 = X.to_index(cb.init[1]);
+  if (X.depends_on(c0, EK::Data) || !m.loop_free(c0)) refuse(F, "its column origin depends on data");
+  if (!m.is_const(cb.stride[1], 1)) refuse(F, "B's inner stride is not 1");
+  int c0b, Nb, r0c, Mc, c0c, Nc;
+  if (Bm->acc.dims.size() != 2 || !m.pid_free(Bm->acc.dims[0]) || !m.extent(Bm->acc.dims[1], BN, c0b, Nb) || c0b != c0)
+    refuse(F, "its B block is not masked as (K left) x (col0 + arange < N)");
+  if (C->acc.dims.size() != 2 || !m.extent(C->acc.dims[0], BM, r0c, Mc) || !m.extent(C->acc.dims[1], BN, c0c, Nc) || r0c != r0 || Mc != Mb || c0c != c0 || Nc != Nb)
+    refuse(F, "its output is not masked as (row0 + arange < rows) & (col0 + arange < N)");
+  if (!m.pid_free(Nb) || !m.loop_free(Nb)) refuse(F, "its column count depends on the program id");
+  if (!m.is_const(C->acc.strides[1], 1)) refuse(F, "C's inner stride is not 1");
+  if (!Bm->acc.has_other || Bm->acc.other_f != 0.0) refuse(F, "its B block does not pad with 0");
+  if (A->acc.elem != T || Bm->acc.elem != T || C->acc.elem != T) return false;
+  LinIv lid;
+  if (!m.linear(id->acc.offsets[0], lid)) refuse(F, "the address of its matrix id is not linear in the program id");
+  pl.family = Family::Gemm;
+  pl.k["gathered"] = 1;
+  pl.k["BM"] = BM; pl.k["BN"] = BN; pl.k["BK"] = BK;
+  pl.k["a_arg"] = A->acc.base_arg;
+  pl.k["b_arg"] = Bm->acc.base_arg;
+  pl.k["c_arg"] = C->acc.base_arg;
+  pl.k["rows_arg"] = rows->acc.base_arg;
+  pl.k["block_arg"] = id->acc.base_arg;
+  pl.k["is_bf16"] = T == "bf16";
+  pl.k["mul32"] = mul32;
+  pl.e["r0"] = r0;
+  pl.e["c0"] = c0;
+  pl.e["M"] = Mb;
+  pl.e["N"] = Nb;
+  pl.e["K"] = loop->ub;
+  pl.e["sam"] = pitch->expr;
+  pl.e["sbk"] = cb.stride[0];
+  pl.e["b_kstep"] = cb.kstep;
+  pl.e["scm"] = C->acc.strides[0];
+  pl.e["c_base"] = m.sum(C->acc.offsets);
+  pl.e["block_off"] = X.to_index(id->acc.offsets[0]);
+  pl.e["block_stride"] = block_stride;
+  return true;
+}
+
 }  // namespace
 
 // ------------------------------------------------------------- fused map
@@ -933,6 +1055,21 @@ Plan make_plan(Program &&p) {
     pl.source = tile_program_source(pl.prog);
     pl.family = Family::TileProgram;
     return pl;
+  }
+  {
+    // one unstructured shape the matrix-product kernels take: a product whose A rows come through an index vector and
+    // whose B matrix is picked by an id read from memory (the generic family's kernel stays behind it for launches
+    // those kernels decline)
+    bool taken = false;
+    try {
+      taken = try_gemm_gathered(pl);
+    } catch (const Unsupported &) {
+      pl.k.clear(); pl.e.clear(); pl.lin.clear(); pl.f.clear();
+    }
+    if (taken) {
+      pl.fallback_source = generic_fallback(pl.prog);
+      return pl;
+    }
   }
   bool unstructured = pl.prog.pool.has_data();  // addresses that depend on loaded values: nothing the host could check or bind
   {

@@ -350,7 +350,49 @@ DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
   return d;
 }
 
+// The product with gathered rows (match.cpp: try_gemm_gathered): one program per BM x BN tile of C, rows of A through an
+// index vector at rows_ptr + row0, the matrix of a block of BM rows picked by the id at block_ptr + row0 / BM.
+void bind_gemm_gathered(const Resolver &r, Bound &b) {
+  const Plan &pl = r.pl;
+  const char *F = "gemm (gathered rows)";
+  auto need = [&](bool ok, const std::string &why) {
+    if (!ok) throw Unsupported(std::string(F) + ": " + why);
+  };
+  const int64_t BM = pl.k.at("BM"), BN = pl.k.at("BN"), BK = pl.k.at("BK");
+  GemmParams &p = b.gemm;
+  p.M = r.ev0("M"); p.N = r.ev0("N"); p.K = r.ev0("K");
+  p.lda = r.ev0("sam"); p.ldb = r.ev0("sbk"); p.ldc = r.ev0("scm");
+  p.is_bf16 = (int)pl.k.at("is_bf16");
+  need(p.M > 0 && p.N > 0 && p.K >= 0, "empty problem");
+  need(BM % 128 == 0, "blocks of rows that are not whole 128-row kernel tiles");
+  need(r.ev0("b_kstep") == BK * p.ldb, "the B pointer does not advance by one K block per iteration");
+  need(p.lda >= 0 && p.lda <= INT32_MAX && p.ldb >= 0, "negative or oversized pitches");
+  const int64_t tm = (p.M + BM - 1) / BM, tn = (p.N + BN - 1) / BN;
+  need((int64_t)r.g[0] * r.g[1] * r.g[2] == tm * tn, "the grid does not have one program per output tile");
+  std::vector<char> seen(tm * tn, 0);
+  for (int z = 0; z < r.g[2]; z++)
+    for (int y = 0; y < r.g[1]; y++)
+      for (int x = 0; x < r.g[0]; x++) {
+        EvalEnv e = r.env(x, y, z);
+        const int64_t r0 = r.ev("r0", e), c0 = r.ev("c0", e);
+        need(r0 >= 0 && c0 >= 0 && r0 % BM == 0 && c0 % BN == 0 && r0 / BM < tm && c0 / BN < tn, "a program's tile origin is off the tile grid");
+        char &s = seen[(r0 / BM) * tn + c0 / BN];
+        need(!s, "two programs compute the same output tile");
+        s = 1;
+        need(r.ev("block_off", e) == r0 / BM, "the matrix id of a block of rows is not read from ids[row0 / BM]");
+        need(r.ev("c_base", e) == r0 * p.ldc + c0, "C tile offset is not row0 * ldc + col0");
+      }
+  p.b_block_rows = (int)BM;
+  p.b_block_stride = r.ev0("block_stride");
+  p.gather_mul32 = 1 | (pl.k.at("mul32") ? 2 : 0);
+  std::ostringstream os;
+  os << "kernel=gemm_mfma\ngathered=1\nM=" << p.M << "\nN=" << p.N << "\nK=" << p.K << "\nlda=" << p.lda << "\nldb=" << p.ldb << "\nldc=" << p.ldc
+     << "\nbf16=" << p.is_bf16 << "\nblock_rows=" << p.b_block_rows << "\nblock_stride=" << p.b_block_stride << "\n";
+  b.describe = os.str();
+}
+
 void bind_gemm(const Resolver &r, Bound &b) {
+  if (r.pl.k.count("gathered")) return bind_gemm_gathered(r, b);
   DenseGemm d = prove_dense_gemm(r, "gemm");
   GemmParams &p = b.gemm;
   p.M = d.M; p.N = d.N; p.K = d.K; p.lda = d.lda; p.ldb = d.ldb; p.ldc = d.ldc;
@@ -671,6 +713,10 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
         p.a = ptr_arg<const void>(args, pl, "a_arg");
         p.b = ptr_arg<const void>(args, pl, "b_arg");
         p.c = ptr_arg<void>(args, pl, "c_arg");
+        if (pl.k.count("gathered")) {
+          p.a_rows = ptr_arg<const int>(args, pl, "rows_arg");
+          p.b_block = ptr_arg<const int>(args, pl, "block_arg");
+        }
         if (pl.source.empty()) {
           err = launch_gemm(p, s, &kname);
           break;
