@@ -215,9 +215,12 @@ def test_gemm_ragged_shapes(K, oracle_cpu, M, N, Kd, dtype):
 
 @pytest.mark.parametrize("M,N,Kd,dtype,pad", [(256, 256, 32, torch.bfloat16, 0), (256, 512, 64, torch.bfloat16, 0),
                                              (512, 256, 96, torch.bfloat16, 8), (768, 256, 160, torch.float16, 16),
-                                             (256, 256, 4096, torch.bfloat16, 0), (1024, 1280, 352, torch.float16, 0)])
+                                             (256, 256, 4096, torch.bfloat16, 0), (1024, 1280, 352, torch.float16, 0),
+                                             # enough tiles for the 128 x 256 and the 256 x 128 variants, and for 256 x 256
+                                             (4096, 2048, 96, torch.bfloat16, 0), (4096, 2176, 64, torch.float16, 8), (4096, 4096, 32, torch.bfloat16, 0)])
 def test_gemm_whole_tile_kernel(K, M, N, Kd, dtype, pad):
-    # whole 256 x 256 x 32 tiles: the direct-to-LDS kernel, from one K tile (fewer than its pipeline stages) upwards
+    # whole tiles: the direct-to-LDS kernels (256 x 256, 128 x 256, 256 x 128 or 128 x 128 tiles by the number of tiles the
+    # problem gives), from one K tile (fewer than the pipeline's stages) upwards
     torch.manual_seed(M + Kd)
     A, B = (torch.randn(M, Kd + pad) * 0.5).to(dtype).to(DEV), (torch.randn(Kd, N + pad) * 0.5).to(dtype).to(DEV)
     Cfull = torch.full((M, N + pad), 5.0, dtype=dtype, device=DEV)
@@ -225,7 +228,8 @@ def test_gemm_whole_tile_kernel(K, M, N, Kd, dtype, pad):
     k = K.matmul_tiles[(triton.cdiv(M, 128) * triton.cdiv(N, 128),)](a, b, c, M, N, Kd, a.stride(0), 1, b.stride(0), 1,
                                                                    c.stride(0), 1, BM=128, BN=128, BK=64, GROUP_M=8)
     torch.cuda.synchronize()
-    assert k.function.last_kernel == "gemm_dma_kernel"
+    want_kernel = {(4096, 2048): "gemm_dma_kernel<128x256>", (4096, 2176): "gemm_dma_kernel<256x128>", (4096, 4096): "gemm_dma_kernel"}.get((M, N), "gemm_dma_kernel<128x128>")
+    assert k.function.last_kernel == want_kernel
     assert relfro(c.cpu(), a.cpu().double() @ b.cpu().double()) <= 1e-2
     assert torch.equal(Cfull[:, N:].cpu(), torch.full((M, pad), 5.0, dtype=dtype))
     # exact: B selects and negates columns of A

@@ -294,18 +294,43 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmParams &p, int tiles_m,
 // The direct-to-LDS load is issued from inline assembly: the compiler orders every later LDS
 // read behind such a load with a full vmcnt wait (it cannot tell the stages apart), which
 // would serialise the pipeline.  Its own counting of ordinary loads stays conservative.
-constexpr int F_BM = 256, F_BN = 256, F_BK = 32, F_STAGES = 4;
-constexpr int F_A_BYTES = F_BM * F_BK * 2, F_STAGE_BYTES = F_A_BYTES + F_BK * F_BN * 2;
+constexpr int F_BK = 32;
+// Tile geometry of the direct-to-LDS kernel: 2 x 2 wavefronts of TM x TN MFMA tiles each.
+template <int TM, int TN>
+struct DmaTile {
+  static constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32;
+  static constexpr int A_BYTES = BM * F_BK * 2, B_ROW_BYTES = BN * 2, STAGE_BYTES = A_BYTES + F_BK * B_ROW_BYTES;
+  static constexpr int A_DMA = BM / 64, B_DMA = BN / 64;  // direct-to-LDS instructions per wavefront and K tile
+  static constexpr int DMA = A_DMA + B_DMA;
+  // whole 256 x 256 tiles keep one workgroup per CU busy (256 accumulator registers per wavefront); the smaller tiles
+  // are sized so that two workgroups fit a CU's 160 KB of LDS
+  static constexpr int STAGES = (TM * TN == 8) ? 3 : 4;  // 64 KB (128 x 128), 72 KB (128 x 256, 256 x 128), 128 KB (256 x 256)
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+};
+constexpr int F_BM = DmaTile<4, 4>::BM, F_BN = DmaTile<4, 4>::BN, F_STAGES = DmaTile<4, 4>::STAGES;
+constexpr int F_A_BYTES = DmaTile<4, 4>::A_BYTES, F_STAGE_BYTES = DmaTile<4, 4>::STAGE_BYTES;
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 #define TTS_LDS(p) ((__attribute__((address_space(3))) void *)(p))
 
 // s_waitcnt immediate: vmcnt in bits 3:0 and 15:14, expcnt (not waited for) in 6:4, lgkmcnt in 11:8
 constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 14) | (7 << 4) | (lgkm << 8); }
 
-template <bool BF16, class Ep>
+// TM x TN = 4 x 4: the 256 x 256 tile described above.  Smaller tiles (2 x 2: 128 x 128, 2 x 4: 128 x 256, 4 x 2:
+// 256 x 128) use the same stages, swizzles and phases with fewer rows and columns: an A instruction still covers 16
+// rows of 64 bytes, a B instruction 1024 / (2 BN) k rows of 2 BN bytes (position q of k row k holds chunk
+// q ^ ((k & 3) << 2) of the row's BN / 8).  They take A rows through an index vector and a matrix id per block of rows
+// (p.a_rows, p.b_block): the A addresses are then 64-bit per lane.
+template <bool BF16, int TM, int TN, class Ep>
 __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, int tiles_n, const Ep &ep) {
-  #ifdef TTS_GEMM_RTC
-  __shared__ __align__(16) char dma_smem[F_STAGES * F_STAGE_BYTES];
+  using T = DmaTile<TM, TN>;
+  constexpr int BM = T::BM, BN = T::BN, STAGES = T::STAGES, A_BYTES = T::A_BYTES, STAGE_BYTES = T::STAGE_BYTES, ROWB = T::B_ROW_BYTES;
+  constexpr int A_DMA = T::A_DMA, B_DMA = T::B_DMA, DMA = T::DMA;
+  constexpr int B_KROWS = 1024 / ROWB;       // k rows one B instruction covers
+  constexpr int B_CHUNKS = ROWB / 16;        // 16-byte chunks per k row
+  constexpr bool GATHER = !(TM == 4 && TN == 4);
+  static_assert(DMA % 2 == 0, "half of a tile's loads go out in each phase");
+#ifdef TTS_GEMM_RTC
+  __shared__ __align__(16) char dma_smem[T::LDS_BYTES];
 #else
   extern __shared__ __align__(16) char dma_smem[];
 #endif
@@ -320,22 +345,38 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   const int g0 = (bid / group) * 4;
   const int gh = min(tiles_m - g0, 4);
   const int tile_m = g0 + (bid % group) % gh, tile_n = (bid % group) / gh;
-  const int64_t m0 = (int64_t)tile_m * F_BM, n0 = (int64_t)tile_n * F_BN;
+  const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
 
-  // Wavefront w issues A instructions 4w..4w+3 (rows 16 ia + lane / 4) and B instructions
-  // 4w..4w+3 (k rows 2 ib + lane / 32) of a tile.  Per-lane byte offsets are constant; the
-  // tile's base address moves in scalar registers.
-  uint32_t a_voff[4], b_voff[4];
+  const char *b_base = (const char *)((const uint16_t *)p.b + n0);
+  if (GATHER && p.b_block) {  // the rows of this tile multiply a matrix of their own; a negative id: nothing to do for them
+    const int which = p.b_block[m0 / p.b_block_rows];
+    if (which < 0) return;
+    b_base += 2 * ((p.gather_mul32 & 2) ? (int64_t)(int)((uint32_t)which * (uint32_t)p.b_block_stride) : (int64_t)which * p.b_block_stride);
+  }
+
+  // Wavefront w issues A instructions A_DMA w .. (rows 16 ia + lane / 4) and B instructions B_DMA w .. (k rows
+  // B_KROWS ib + lane / B_CHUNKS) of a tile.  Per-lane byte offsets are constant; the tile's base address moves in
+  // scalar registers (with gathered rows: per-lane 64-bit addresses that move by one K tile).
+  uint32_t a_voff[A_DMA], b_voff[B_DMA];
+  const char *a_lane[A_DMA];
 #pragma unroll
-  for (int i = 0; i < 4; i++)
-    a_voff[i] = (uint32_t)(((64 * wave + 16 * i + lane / 4) * p.lda + 8 * ((lane & 3) ^ ((lane >> 4) & 3))) * 2);
+  for (int i = 0; i < A_DMA; i++) {
+    const int row = 16 * (A_DMA * wave + i) + lane / 4;
+    const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
+    a_voff[i] = (uint32_t)((row * p.lda + 8 * chunk) * 2);
+    if (GATHER) {
+      int64_t r = m0 + row;
+      if (p.a_rows) r = (p.gather_mul32 & 1) ? (int64_t)(int)((uint32_t)p.a_rows[r] * (uint32_t)p.lda) : (int64_t)p.a_rows[r] * p.lda;
+      else r *= p.lda;
+      a_lane[i] = (const char *)((const uint16_t *)p.a + r + 8 * chunk);
+    }
+  }
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int krow = 8 * wave + 2 * i + lane / 32;
-    b_voff[i] = (uint32_t)((krow * p.ldb + 8 * ((lane & 31) ^ ((krow & 3) << 2))) * 2);
+  for (int i = 0; i < B_DMA; i++) {
+    const int krow = B_KROWS * (B_DMA * wave + i) + lane / B_CHUNKS;
+    b_voff[i] = (uint32_t)((krow * p.ldb + 8 * ((lane & (B_CHUNKS - 1)) ^ ((krow & 3) << 2))) * 2);
   }
   const char *a_base = (const char *)((const uint16_t *)p.a + m0 * p.lda);
-  const char *b_base = (const char *)((const uint16_t *)p.b + n0);
   const uint32_t lds0 = (uint32_t)(uintptr_t)TTS_LDS(smem);
   const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int nk = (int)(p.K / F_BK);
@@ -350,80 +391,89 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
 #endif
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(voff), "s"(sbase) : "memory", "m0");
   };
-  auto dma_one = [&](int t, int n) {  // n = 0..3: A part, 4..7: B part of tile t, into stage t % F_STAGES
+  auto dma_lane = [&](const char *addr, uint32_t lds) {  // every lane its own 64-bit address
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds), "v"(addr) : "memory", "m0");
+  };
+  auto dma_one = [&](int t, int n) {  // n < A_DMA: A part, else B part of tile t, into stage t % STAGES
     const int tc = min(t, nk - 1);
-    const uint32_t st = lds0 + (t % F_STAGES) * F_STAGE_BYTES + wave_u * 4096;
-    if (n < 4) dma(a_base + (int64_t)tc * F_BK * 2, a_voff[n], st + n * 1024);
-    else dma(b_base + (int64_t)tc * F_BK * p.ldb * 2, b_voff[n - 4], st + F_A_BYTES + (n - 4) * 1024);
+    const uint32_t st = lds0 + (t % STAGES) * STAGE_BYTES;
+    if (n < A_DMA) {
+      const uint32_t at = st + (A_DMA * wave_u + n) * 1024;
+      if (GATHER) dma_lane(a_lane[n] + (int64_t)tc * F_BK * 2, at);
+      else dma(a_base + (int64_t)tc * F_BK * 2, a_voff[n], at);
+    } else {
+      dma(b_base + (int64_t)tc * F_BK * p.ldb * 2, b_voff[n - A_DMA], st + A_BYTES + (B_DMA * wave_u + n - A_DMA) * 1024);
+    }
   };
 
   // fragment read offsets (bytes, within a stage)
-  // A: row r = wm * 128 + i * 32 + lane % 32, chunk c = 2 ks + lane / 32 at position c ^ ((r / 4) & 3)
-  const int ar = wm * 128 + (lane & 31);
+  // A: row r = wm * TM * 32 + i * 32 + lane % 32, chunk c = 2 ks + lane / 32 at position c ^ ((r / 4) & 3)
+  const int ar = wm * TM * 32 + (lane & 31);
   const int a_off = ar * 64, a_sw = (ar >> 2) & 3;
   // B: 16-lane group q = lane / 16, r16 = lane % 16: k row ks * 16 + 8 (q / 2) + 4 h + r16 / 4,
-  // chunk wn * 16 + 4 j + 2 (q & 1) + (r16 % 4) / 2, byte 8 (r16 & 1) within the chunk
+  // chunk wn * TN * 4 + 4 j + 2 (q & 1) + (r16 % 4) / 2, byte 8 (r16 & 1) within the chunk
   const int q = lane >> 4, r16 = lane & 15;
-  const int b_chunk = wn * 16 + 2 * (q & 1) + ((r16 & 3) >> 1), b_sw = (r16 >> 2) << 2;
-  const int b_off = F_A_BYTES + (8 * (q >> 1) + (r16 >> 2)) * 512 + 8 * (r16 & 1);
+  const int b_chunk = wn * TN * 4 + 2 * (q & 1) + ((r16 & 3) >> 1), b_sw = (r16 >> 2) << 2;
+  const int b_off = A_BYTES + (8 * (q >> 1) + (r16 >> 2)) * ROWB + 8 * (r16 & 1);
 
-  f32x16 acc[4][4];
+  f32x16 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < TN; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-  uint4 af[2][4], bf[2][4];
-  // one fragment read (n = 0..3: A row block n; n = 4..11: B column block (n - 4) / 2, k half (n - 4) % 2)
-  auto read_one = [&](int t, int ks, int n, uint4 (&a)[4], uint4 (&b)[4]) {
-    const char *st = smem + (t % F_STAGES) * F_STAGE_BYTES;
-    if (n < 4) {
+  constexpr int READS = TM + 2 * TN, MFMAS = TM * TN;
+  uint4 af[2][TM], bf[2][TN];
+  // one fragment read (n < TM: A row block n; else B column block (n - TM) / 2, k half (n - TM) % 2)
+  auto read_one = [&](int t, int ks, int n, uint4 (&a)[TM], uint4 (&b)[TN]) {
+    const char *st = smem + (t % STAGES) * STAGE_BYTES;
+    if (n < TM) {
       a[n] = *reinterpret_cast<const uint4 *>(st + a_off + n * 2048 + (((2 * ks + (lane >> 5)) ^ a_sw) << 4));
     } else {
-      const int j = (n - 4) >> 1, h = (n - 4) & 1;
-      const char *bp = st + b_off + ks * 16 * 512 + (((b_chunk + 4 * j) ^ b_sw) << 4) + h * 4 * 512;
+      const int j = (n - TM) >> 1, h = (n - TM) & 1;
+      const char *bp = st + b_off + ks * 16 * ROWB + (((b_chunk + 4 * j) ^ b_sw) << 4) + h * 4 * ROWB;
       s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)TTS_LDS(bp));
       uint2 v2 = __builtin_bit_cast(uint2, v);
       if (h == 0) { b[j].x = v2.x; b[j].y = v2.y; } else { b[j].z = v2.x; b[j].w = v2.y; }
     }
   };
-  auto mfma_one = [&](int n, uint4 (&a)[4], uint4 (&b)[4]) {
-    acc[n >> 2][n & 3] = mfma32<BF16>(a[n >> 2], b[n & 3], acc[n >> 2][n & 3]);
+  auto mfma_one = [&](int n, uint4 (&a)[TM], uint4 (&b)[TN]) {
+    acc[n / TN][n % TN] = mfma32<BF16>(a[n / TN], b[n % TN], acc[n / TN][n % TN]);
+  };
+  // A phase: MFMAS matrix instructions, READS fragment reads for the next phase, DMA / 2 loads; they are dealt out
+  // behind the matrix instructions as evenly as their numbers allow.
+  constexpr int SLOTS = MFMAS > READS ? MFMAS : READS;
+  auto phase = [&](uint4 (&a_use)[TM], uint4 (&b_use)[TN], uint4 (&a_next)[TM], uint4 (&b_next)[TN], int t_read, int ks_read, int t_load, int first_load) {
+#pragma unroll
+    for (int n = 0; n < SLOTS; n++) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (n < MFMAS) mfma_one(n, a_use, b_use);
+      if (n < READS) read_one(t_read, ks_read, n, a_next, b_next);
+      constexpr int every = SLOTS / (DMA / 2);
+      if (n % every == every - 1 && n / every < DMA / 2) dma_one(t_load, first_load + n / every);
+    }
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   // prologue: STAGES - 1 tiles in flight; tile 0 landed; its first operands read
-  for (int t = 0; t < F_STAGES - 1; t++)
+  for (int t = 0; t < STAGES - 1; t++)
 #pragma unroll
-    for (int n = 0; n < 8; n++) dma_one(t, n);
-  __builtin_amdgcn_s_waitcnt(waitcnt_imm(8 * (F_STAGES - 2), 15));
+    for (int n = 0; n < DMA; n++) dma_one(t, n);
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(DMA * (STAGES - 2), 15));
   __syncthreads();
 #pragma unroll
-  for (int n = 0; n < 12; n++) read_one(0, 0, n, af[0], bf[0]);
+  for (int n = 0; n < READS; n++) read_one(0, 0, n, af[0], bf[0]);
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
   for (int t = 0; t < nk; t++) {
     // phase A: MFMAs of (tile t, first half); read (tile t, second half); first half of the loads of tile t + STAGES - 1
-#pragma unroll
-    for (int n = 0; n < 16; n++) {
-      __builtin_amdgcn_sched_barrier(0);
-      mfma_one(n, af[0], bf[0]);
-      if (n < 12) read_one(t, 1, n, af[1], bf[1]);
-      if ((n & 3) == 3) dma_one(t + F_STAGES - 1, n >> 2);
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    phase(af[0], bf[0], af[1], bf[1], t, 1, t + STAGES - 1, 0);
     // own loads of tile t+1 have landed (later ones may be in flight); own reads of tile t are complete
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(8 * (F_STAGES - 3) + 4, 0));
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(DMA * (STAGES - 3) + DMA / 2, 0));
     __syncthreads();
     // phase B: MFMAs of (tile t, second half); read (tile t+1, first half); the rest of the loads
-#pragma unroll
-    for (int n = 0; n < 16; n++) {
-      __builtin_amdgcn_sched_barrier(0);
-      mfma_one(n, af[1], bf[1]);
-      if (n < 12) read_one(t + 1, 0, n, af[0], bf[0]);
-      if ((n & 3) == 3) dma_one(t + F_STAGES - 1, (n >> 2) + 4);
-    }
-    __builtin_amdgcn_sched_barrier(0);
+    phase(af[1], bf[1], af[0], bf[0], t + 1, 0, t + STAGES - 1, DMA / 2);
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));  // the surplus loads land before the LDS goes away
@@ -439,19 +489,19 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   const bool odd = lane & 1;
   const uint32_t sel = odd ? 0x03020706u : 0x05040100u;  // odd: high halves of (neighbour, mine); even: low halves of (mine, neighbour)
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const int64_t col = n0 + wn * 128 + j * 32 + (lane & 31) - (odd ? 1 : 0);
+    for (int j = 0; j < TN; j++) {
+      const int64_t col = n0 + wn * TN * 32 + j * 32 + (lane & 31) - (odd ? 1 : 0);
 #pragma unroll
       for (int v = 0; v < 16; v += 2) {
-        const int64_t er = m0 + wm * 128 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), ec = n0 + wn * 128 + j * 32 + (lane & 31);
+        const int64_t er = m0 + wm * TM * 32 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), ec = n0 + wn * TN * 32 + j * 32 + (lane & 31);
         const f32x2_t pr = {ep(acc[i][j][v], er, ec), ep(acc[i][j][v + 1], er + 1, ec)};
         const uint32_t pk = BF16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, bf16x2_t))
                                  : __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, f16x2_t));
         const uint32_t nb = __builtin_amdgcn_mov_dpp(pk, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]: the neighbour's pair
         const uint32_t w = __builtin_amdgcn_perm(nb, pk, sel);
-        const int64_t row = m0 + wm * 128 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3) + (odd ? 1 : 0);
+        const int64_t row = m0 + wm * TM * 32 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3) + (odd ? 1 : 0);
         __builtin_nontemporal_store(w, reinterpret_cast<uint32_t *>(&C[row * p.ldc + col]));
       }
     }
@@ -462,7 +512,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
 #ifdef TTS_GEMM_RTC
 extern "C" __global__ __launch_bounds__(256) void gemm_rtc(TtsGemmParams p, int tiles_m, int tiles_n, TtsEp ep) {
 #if TTS_GEMM_RTC == 0
-  tts_gemm_device::gemm_dma_body<TTS_GEMM_BF16 != 0>(p, tiles_m, tiles_n, ep);
+  tts_gemm_device::gemm_dma_body<TTS_GEMM_BF16 != 0, 4, 4>(p, tiles_m, tiles_n, ep);
 #elif TTS_GEMM_RTC == 1
   tts_gemm_device::gemm_mfma_body<TTS_GEMM_BF16 != 0, 4, 4, 32>(p, tiles_m, tiles_n, ep);
 #else

@@ -46,28 +46,33 @@ hipError_t launch_gemm_cfg(const GemmParams &p, hipStream_t s) {
 }
 
 
-template <bool BF16>
+template <bool BF16, int TM, int TN>
 __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmParams p, int tiles_m, int tiles_n) {
-  gemm_dma_body<BF16>(p, tiles_m, tiles_n, IdentityEp());
+  gemm_dma_body<BF16, TM, TN>(p, tiles_m, tiles_n, IdentityEp());
 }
 
-template <bool BF16>
+template <bool BF16, int TM, int TN>
 hipError_t launch_gemm_dma(const GemmParams &p, hipStream_t s) {
-  constexpr size_t lds = (size_t)F_STAGES * F_STAGE_BYTES;
-  auto kern = gemm_dma_kernel<BF16>;
+  using T = DmaTile<TM, TN>;
+  constexpr size_t lds = T::LDS_BYTES;
+  auto kern = gemm_dma_kernel<BF16, TM, TN>;
   static const hipError_t attr = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return attr;
-  int tiles_m = (int)(p.M / F_BM), tiles_n = (int)(p.N / F_BN);
+  int tiles_m = (int)(p.M / T::BM), tiles_n = (int)(p.N / T::BN);
   hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds, s, p, tiles_m, tiles_n);
   return hipGetLastError();
 }
 
-// whole tiles, 16-byte aligned rows, and per-lane byte offsets that fit 32 bits
-bool gemm_fast_path_ok(const GemmParams &p) {
-  return !p.a_trans && !p.b_trans && !p.a_rows && !p.b_block && p.M % F_BM == 0 && p.N % F_BN == 0 && p.K % F_BK == 0 && p.K >= F_BK && p.lda % 8 == 0 && p.ldb % 8 == 0 &&
+// whole bm x bn x 32 tiles, 16-byte aligned rows, and per-lane byte offsets that fit 32 bits
+bool gemm_dma_ok(const GemmParams &p, int64_t bm, int64_t bn) {
+  if (p.a_trans || p.b_trans) return false;
+  if ((p.a_rows || p.b_block) && bm != 128) return false;  // gathered rows: 128-row tiles (64-bit A addresses per lane)
+  if (p.b_block && p.b_block_rows % bm != 0) return false;
+  return p.M % bm == 0 && p.N % bn == 0 && p.K % F_BK == 0 && p.K >= F_BK && p.lda % 8 == 0 && p.ldb % 8 == 0 &&
          ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0 && p.lda < (1 << 22) && p.ldb < (1 << 25) &&
-         p.ldc % 2 == 0 && ((uintptr_t)p.c & 3) == 0;  // C is written in 4-byte pairs
+         (!p.b_block || p.b_block_stride % 8 == 0) && p.ldc % 2 == 0 && ((uintptr_t)p.c & 3) == 0;  // C is written in 4-byte pairs
 }
+bool gemm_fast_path_ok(const GemmParams &p) { return gemm_dma_ok(p, F_BM, F_BN); }
 
 // ------------------------------------------------------ int8-weight GEMM
 // Workgroup: NW wavefronts share one 128-column slab of W and split its K range
@@ -462,9 +467,30 @@ constexpr int W8_WAVES = 16;
 
 hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
   static const char *tile_env = getenv("TTS_GEMM_TILE");  // tuning aid: 128, 256 (general kernel) or unset
-  if (!tile_env && gemm_fast_path_ok(p)) {
-    *name = "gemm_dma_kernel";
-    return p.is_bf16 ? launch_gemm_dma<true>(p, s) : launch_gemm_dma<false>(p, s);
+  static const char *dma_env = getenv("TTS_GEMM_DMA");    // tuning aid: "256x256", "128x256", "256x128", "128x128" or unset
+  if (!tile_env) {
+    // Whole tiles go to the direct-to-LDS kernels: the largest tile that still gives every CU a workgroup.
+    static const int cus = [] {
+      int dev = 0, n = 0;
+      if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+      return n;
+    }();
+    auto tiles = [&](int64_t bm, int64_t bn) { return (p.M / bm) * (p.N / bn); };
+    auto want = [&](const char *tag, int64_t bm, int64_t bn, int64_t enough) {
+      if (dma_env) return std::string(dma_env) == tag && gemm_dma_ok(p, bm, bn);
+      return gemm_dma_ok(p, bm, bn) && tiles(bm, bn) >= enough;
+    };
+#define TTS_DMA(TM, TN, TAG)                                                                                  \
+  do {                                                                                                        \
+    *name = TAG;                                                                                              \
+    return p.is_bf16 ? launch_gemm_dma<true, TM, TN>(p, s) : launch_gemm_dma<false, TM, TN>(p, s);            \
+  } while (0)
+    if (want("256x256", 256, 256, cus)) TTS_DMA(4, 4, "gemm_dma_kernel");
+    if (want("128x256", 128, 256, cus)) TTS_DMA(2, 4, "gemm_dma_kernel<128x256>");
+    if (want("256x128", 256, 128, cus)) TTS_DMA(4, 2, "gemm_dma_kernel<256x128>");
+    if (want("128x128", 128, 128, 1)) TTS_DMA(2, 2, "gemm_dma_kernel<128x128>");
+    if (!dma_env && gemm_dma_ok(p, 256, 256)) TTS_DMA(4, 4, "gemm_dma_kernel");
+#undef TTS_DMA
   }
   // 128 x 128 x 64 tiles, two workgroups per CU, measured ahead of 256 x 256 x 32 at every size tried (4096^3: 197 against
   // 202 us; 4096 x 2048 x 2048: 56 against 112 us); the larger tile stays selectable for experiments
