@@ -538,3 +538,30 @@ def test_gemm_binds_column_major_operands(native):
     plan = native.PlanHandle(native.structured_to_plan(text)[0])
     d = plan.describe_launch((4 * 3, 1, 1), [0, 0, 0, 512, 384, 200, 208, 2, 432, 392])
     assert d["kernel"] == "tile_program" and "neither stride of B is 1" in d["fallback_reason"]
+
+
+def test_gathered_rows_matmul_binds_to_the_matrix_product_family(native):
+    # the mixture-of-experts product (rows of A through an index vector, the weight matrix of a block of rows picked by an
+    # id read from memory; test/Conversion/TritonToUnstructured/unstructured_ptr_used_in_loop.mlir has this shape)
+    import extra_kernels as X
+    from triton_shared_amd.examples import kernels as K
+    sig = {"a_ptr": "*bf16", "b_ptr": "*bf16", "c_ptr": "*bf16", "rows_ptr": "*i32", "expert_ptr": "*i32", "n_rows": "i32", "K": "i32", "N": "i32",
+           "s_am": "i32", "s_be": "i32", "s_bk": "i32", "s_cm": "i32", "BM": "constexpr", "BN": "constexpr", "BK": "constexpr"}
+    for fn in (K.expert_rows_matmul, X.grouped_rows_matmul):
+        text = native.ttir_to_structured(compile_ttir(fn, sig, {"BM": 128, "BN": 128, "BK": 64}))
+        plan = native.PlanHandle(native.structured_to_plan(text)[0])
+        assert plan.family == "gemm"
+        tokens, kd, nd = 300, 150, 256
+        vals = [0, 0, 0, 0, 0, tokens, kd, nd, kd + 2, kd * nd, nd + 8, nd + 16]
+        d = plan.describe_launch((3, 2, 1), vals)
+        assert (d["kernel"], d["gathered"], d["M"], d["N"], d["K"], d["lda"], d["ldb"], d["ldc"], d["block_rows"], d["block_stride"]) == \
+               ("gemm_mfma", "1", "300", "256", "150", str(kd + 2), str(nd + 8), str(nd + 16), "128", str(kd * nd))
+        # a grid that is not one program per tile: the generic family's kernel for the same program
+        d = plan.describe_launch((2, 2, 1), vals)
+        assert d["kernel"] == "tile_program" and "one program per output tile" in d["fallback_reason"]
+    # blocks of rows smaller than the kernel's tile, and fp32 data: the generic family from the start
+    text = native.ttir_to_structured(compile_ttir(K.expert_rows_matmul, sig, {"BM": 64, "BN": 128, "BK": 64}))
+    assert native.PlanHandle(native.structured_to_plan(text)[0]).family == "tile_program"
+    sig32 = {k: (v.replace("bf16", "fp32")) for k, v in sig.items()}
+    text = native.ttir_to_structured(compile_ttir(K.expert_rows_matmul, sig32, {"BM": 32, "BN": 32, "BK": 32}))
+    assert native.PlanHandle(native.structured_to_plan(text)[0]).family == "tile_program"
