@@ -1,8 +1,7 @@
 // Device code of the 16-bit matrix-product kernels, in a header of its own because it is compiled twice: ahead of
 // time into the library (kernels_gemm.hip, results stored as they are), and at run time with hipRTC when the Triton
 // kernel applies elementwise ops to the accumulator before the store (a fused activation): the generated source
-// defines TTS_GEMM_RTC (which kernel: 0 whole 256 x 256 x 32 tiles, 1 any shape in 256 x 256 tiles, 2 any shape in
-// 128 x 128 tiles), TTS_GEMM_BF16 and the functor TtsEp (a plain struct, passed as the kernel's last argument) that maps
+// defines TTS_GEMM_RTC (which kernel: 0 whole 256 x 256 x 32 tiles, 1 any shape in 128 x 128 x 64 tiles), TTS_GEMM_BF16 and the functor TtsEp (a plain struct, passed as the kernel's last argument) that maps
 // an accumulator value and its position to the value stored, then this file's text.  Nothing here may need a host header.
 #pragma once
 #ifdef __HIPCC_RTC__
@@ -513,8 +512,6 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
 extern "C" __global__ __launch_bounds__(256) void gemm_rtc(TtsGemmParams p, int tiles_m, int tiles_n, TtsEp ep) {
 #if TTS_GEMM_RTC == 0
   tts_gemm_device::gemm_dma_body<TTS_GEMM_BF16 != 0, 4, 4>(p, tiles_m, tiles_n, ep);
-#elif TTS_GEMM_RTC == 1
-  tts_gemm_device::gemm_mfma_body<TTS_GEMM_BF16 != 0, 4, 4, 32>(p, tiles_m, tiles_n, ep);
 #else
   tts_gemm_device::gemm_mfma_body<TTS_GEMM_BF16 != 0, 2, 2, 64>(p, tiles_m, tiles_n, ep);
 #endif

@@ -92,7 +92,7 @@ hipError_t launch_layernorm(const LayerNormParams &p, int gx, int gy, int gz, hi
 using GemmParams = ::TtsGemmParams;  // gemm_device.h
 hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **kernel_name);
 // The same product with elementwise ops fused into the epilogue: `epilogue` is the source of the functor (match.h:
-// gemm_epilogue_source), `modules` the plan's three slots for the kernels compiled from it (one per tiling, filled at
+// gemm_epilogue_source), `modules` the plan's two slots for the kernels compiled from it (one per tiling, filled at
 // the first launch that needs it), `args` / `args_size` the generic families' argument block.
 struct RtcModule;
 // The epilogue functor as the kernel receives it (the generated `struct TtsEp` has this layout): every kernel argument

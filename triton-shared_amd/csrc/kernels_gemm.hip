@@ -466,7 +466,7 @@ constexpr int W8_WAVES = 16;
 }  // namespace
 
 hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
-  static const char *tile_env = getenv("TTS_GEMM_TILE");  // tuning aid: 128, 256 (general kernel) or unset
+  static const char *tile_env = getenv("TTS_GEMM_TILE");  // tuning aid: set = the any-shape kernel even for whole tiles
   static const char *dma_env = getenv("TTS_GEMM_DMA");    // tuning aid: "256x256", "128x256", "256x128", "128x128" or unset
   if (!tile_env) {
     // Whole tiles go to the direct-to-LDS kernels: the largest tile that still gives every CU a workgroup.
@@ -492,28 +492,21 @@ hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
     if (!dma_env && gemm_dma_ok(p, 256, 256)) TTS_DMA(4, 4, "gemm_dma_kernel");
 #undef TTS_DMA
   }
-  // 128 x 128 x 64 tiles, two workgroups per CU, measured ahead of 256 x 256 x 32 at every size tried (4096^3: 197 against
-  // 202 us; 4096 x 2048 x 2048: 56 against 112 us); the larger tile stays selectable for experiments
-  bool big = false;
-  if (tile_env) big = atoi(tile_env) >= 256;
-  if (big) {
-    *name = "gemm_mfma_kernel<256x256x32>";
-    return p.is_bf16 ? launch_gemm_cfg<true, 4, 4, 32>(p, s) : launch_gemm_cfg<false, 4, 4, 32>(p, s);
-  }
+  // anything else: 128 x 128 x 64 tiles, two workgroups per CU (a 256 x 256 x 32 form of the same kernel measured behind it
+  // at every size tried: 4096^3: 202 against 197 us; 4096 x 2048 x 2048: 112 against 56 us)
   *name = "gemm_mfma_kernel<128x128x64>";
   return p.is_bf16 ? launch_gemm_cfg<true, 2, 2, 64>(p, s) : launch_gemm_cfg<false, 2, 2, 64>(p, s);
 }
 
-int gemm_epilogue_kernel_index(const GemmParams &p) { return gemm_fast_path_ok(p) ? 0 : 2; }
+int gemm_epilogue_kernel_index(const GemmParams &p) { return gemm_fast_path_ok(p) ? 0 : 1; }
 
-// Kernel 0: whole 256 x 256 x 32 tiles; 1: any shape in 256 x 256 tiles; 2: any shape in 128 x 128 tiles -- the choice
-// launch_gemm makes, with the kernels compiled from gemm_device.h plus the epilogue functor at the first launch.
+// Kernel 0: whole 256 x 256 x 32 tiles; 1: any shape in 128 x 128 x 64 tiles -- compiled from gemm_device.h plus the
+// epilogue functor at the first launch that needs it.
 hipError_t launch_gemm_epilogue(const GemmParams &p, const std::string &epilogue, RtcModule **modules, const GemmEpilogueArgs &ep,
                                 hipStream_t s, const char **name, std::string *err) {
-  static const char *names[3] = {"gemm_dma_kernel + epilogue (hipRTC)", "gemm_mfma_kernel<256x256x32> + epilogue (hipRTC)",
-                                 "gemm_mfma_kernel<128x128x64> + epilogue (hipRTC)"};
+  static const char *names[2] = {"gemm_dma_kernel + epilogue (hipRTC)", "gemm_mfma_kernel<128x128x64> + epilogue (hipRTC)"};
   const int which = gemm_epilogue_kernel_index(p);
-  const int64_t tile = which == 2 ? 128 : 256;
+  const int64_t tile = which == 1 ? 128 : 256;
   *name = names[which];
   if (!modules[which]) {
     const std::string source = epilogue + "#define TTS_GEMM_RTC " + std::to_string(which) + "\n#define TTS_GEMM_BF16 " + std::to_string(p.is_bf16 ? 1 : 0) +

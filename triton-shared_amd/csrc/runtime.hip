@@ -97,7 +97,7 @@ struct tts_plan {
   };
   std::unordered_map<void *, SplitK> split_k;
   RtcModule *fused = nullptr;  // the kernel compiled for this plan at its first launch (fused maps, tile programs)
-  RtcModule *gemm_rtc[3] = {nullptr, nullptr, nullptr};  // matrix products with a fused epilogue: one kernel per tiling
+  RtcModule *gemm_rtc[2] = {nullptr, nullptr};  // matrix products with a fused epilogue: one kernel per tiling
   RtcModule *fallback = nullptr;  // the generic family's kernel for a matrix-product plan (launches the product kernels decline)
   ~tts_plan() {
     for (auto &kv : split_k) {
