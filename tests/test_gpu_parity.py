@@ -1454,6 +1454,35 @@ def test_matmul_with_gathered_rows_is_exact_on_selections():
     assert torch.equal(c, want)
 
 
+@pytest.mark.parametrize("tokens,kd,nd,experts,kernel", [(1024, 256, 512, 4, "gemm_dma_kernel<128x128>"), (4096, 64, 2048, 8, "gemm_dma_kernel<128x256>"),
+                                                         (384, 96, 128, 5, "gemm_dma_kernel<128x128>")])
+def test_matmul_with_gathered_rows_on_whole_tiles(tokens, kd, nd, experts, kernel):
+    # whole 128-row tiles go to the direct-to-LDS kernel, which walks the row tiles in the order of their matrix ids (so
+    # that the tiles of one matrix share an L2): ids dealt out of order, repeated and negative; exact as above
+    import extra_kernels as X
+    g = torch.Generator(device="cpu").manual_seed(tokens + nd)
+    a = torch.randint(-8, 9, (tokens + 77, kd), generator=g).bfloat16().to(DEV)
+    pick = torch.randint(0, kd, (experts, nd), generator=g)
+    b = torch.zeros(experts, kd, nd, dtype=torch.bfloat16)
+    for e in range(experts):
+        b[e, pick[e], torch.arange(nd)] = -1.0
+    b = b.to(DEV)
+    rows = torch.randint(0, tokens + 77, (tokens,), generator=g, dtype=torch.int32).to(DEV)
+    ids = torch.randint(-1, experts, (tokens // 128,), generator=g, dtype=torch.int32)
+    ids[0] = experts - 1
+    ids = ids.to(DEV)
+    c = torch.full((tokens, nd), 5.0, device=DEV, dtype=torch.bfloat16)
+    k = X.grouped_rows_matmul[(tokens // 128, nd // 128)](a, b, c, rows, ids, tokens, kd, nd, kd, kd * nd, nd, nd, BM=128, BN=128, BK=64)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and k.function.last_kernel == kernel
+    want = torch.full((tokens, nd), 5.0, device=DEV, dtype=torch.bfloat16)
+    for blk, e in enumerate(ids.tolist()):
+        r = slice(blk * 128, blk * 128 + 128)
+        if e >= 0:
+            want[r] = -a[rows[r].long()][:, pick[e].to(DEV)]
+    assert torch.equal(c, want)
+
+
 @pytest.mark.parametrize("M,N,K,kernel", [(512, 768, 96, "gemm_dma_kernel + epilogue"), (200, 300, 150, "gemm_mfma_kernel<128x128x64> + epilogue"),
                                           (2100, 2060, 72, "gemm_mfma_kernel<128x128x64> + epilogue")])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

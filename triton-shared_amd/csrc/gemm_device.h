@@ -301,9 +301,10 @@ struct DmaTile {
   static constexpr int A_BYTES = BM * F_BK * 2, B_ROW_BYTES = BN * 2, STAGE_BYTES = A_BYTES + F_BK * B_ROW_BYTES;
   static constexpr int A_DMA = BM / 64, B_DMA = BN / 64;  // direct-to-LDS instructions per wavefront and K tile
   static constexpr int DMA = A_DMA + B_DMA;
-  // whole 256 x 256 tiles keep one workgroup per CU busy (256 accumulator registers per wavefront); the smaller tiles
-  // are sized so that two workgroups fit a CU's 160 KB of LDS
-  static constexpr int STAGES = (TM * TN == 8) ? 3 : 4;  // 64 KB (128 x 128), 72 KB (128 x 256, 256 x 128), 128 KB (256 x 256)
+  // Four stages everywhere: 128 KB (256 x 256), 96 KB (128 x 256, 256 x 128: one workgroup per CU, which is what a
+  // problem that gives fewer than one 256 x 256 tile per CU gets anyway), 64 KB (128 x 128: two per CU).  With three
+  // stages the 128 x 256 tile measured 46.3 us on 4096 x 2048 x 2048 against 40.4 with four (five and six: no better).
+  static constexpr int STAGES = 4;
   static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
 };
 constexpr int F_BM = DmaTile<4, 4>::BM, F_BN = DmaTile<4, 4>::BN, F_STAGES = DmaTile<4, 4>::STAGES;
@@ -343,7 +344,25 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   const int group = 4 * tiles_n;                             // 4-tile-tall column groups
   const int g0 = (bid / group) * 4;
   const int gh = min(tiles_m - g0, 4);
-  const int tile_m = g0 + (bid % group) % gh, tile_n = (bid % group) / gh;
+  int tile_m = g0 + (bid % group) % gh;
+  const int tile_n = (bid % group) / gh;
+  if (GATHER && p.b_block && tiles_m <= 256) {
+    // Row tiles that multiply the same matrix should sit behind one L2: the workgroup takes the row tile whose place in
+    // the order by matrix id (ties by position) is the one the tile order above gave it.  With ids 0..7 dealt round-robin
+    // to 32 blocks of 128 rows, every XCD otherwise streams four of the eight matrices (measured past L2: 319 MB per
+    // launch for 100 MB of operands).
+    __shared__ int block_key[256], sorted_tile;
+    if (tid < tiles_m) block_key[tid] = p.b_block[((int64_t)tid * BM) / p.b_block_rows];
+    __syncthreads();
+    if (tid < tiles_m) {
+      const int mine = block_key[tid];
+      int place = 0;
+      for (int o = 0; o < tiles_m; o++) place += (block_key[o] < mine || (block_key[o] == mine && o < tid)) ? 1 : 0;
+      if (place == tile_m) sorted_tile = tid;
+    }
+    __syncthreads();
+    tile_m = sorted_tile;
+  }
   const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
 
   const char *b_base = (const char *)((const uint16_t *)p.b + n0);

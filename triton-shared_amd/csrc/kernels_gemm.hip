@@ -373,6 +373,44 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
   if (p.split > 1) {
     float4 *slots = reinterpret_cast<float4 *>(p.workspace) + (int64_t)slab * p.split * 1024;
     int *counter = p.counters + slab;
+    // tot = the slices' tiles added in slice order, whoever adds them (so the sum does not depend on who arrived when);
+    // `self` is this workgroup's slice, whose tile is tot.  Up to four slices, every load is issued before the first add
+    // (one round trip to memory instead of one per slice).
+    auto add_slices = [&](int self) {
+      constexpr int EAGER = 4;
+      if (p.split <= EAGER) {
+        float4 u[EAGER][PER];
+#pragma unroll
+        for (int sl = 0; sl < EAGER; sl++)
+          if (sl < p.split && sl != self) {
+#pragma unroll
+            for (int e = 0; e < PER; e++) u[sl][e] = load_through(slots + sl * 1024 + tid + e * NW * 64);
+          }
+#pragma unroll
+        for (int e = 0; e < PER; e++) {
+          float4 t = self == 0 ? tot[e] : u[0][e];
+#pragma unroll
+          for (int sl = 1; sl < EAGER; sl++)
+            if (sl < p.split) {
+              const float4 v = sl == self ? tot[e] : u[sl][e];
+              t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+            }
+          tot[e] = t;
+        }
+        return;
+      }
+#pragma unroll
+      for (int e = 0; e < PER; e++) {
+        const int idx = tid + e * NW * 64;
+        float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int sl = 0; sl < p.split; sl++) {
+          float4 u = sl == self ? tot[e] : load_through(slots + sl * 1024 + idx);
+          if (sl == 0) t = u;
+          else { t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w; }
+        }
+        tot[e] = t;
+      }
+    };
     bool others_done = false;
     if (slice == 0) {
       // Slice 0 is given slightly more of K than the others, so it usually ends last: if every other slice has arrived
@@ -385,16 +423,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
     }
     if (others_done) {
       if (tid == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-      for (int e = 0; e < PER; e++) {
-        const int idx = tid + e * NW * 64;
-        float4 t = tot[e];
-        for (int sl = 1; sl < p.split; sl++) {  // slice order, as in the general case: the sum does not depend on who arrived when
-          float4 u = load_through(slots + sl * 1024 + idx);
-          t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
-        }
-        tot[e] = t;
-      }
+      add_slices(0);
     } else {
 #pragma unroll
     for (int e = 0; e < PER; e++) store_through(slots + slice * 1024 + tid + e * NW * 64, tot[e]);
@@ -407,17 +436,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
     }
     __syncthreads();
     if (!is_last) return;
-#pragma unroll
-    for (int e = 0; e < PER; e++) {
-      const int idx = tid + e * NW * 64;
-      float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-      for (int sl = 0; sl < p.split; sl++) {
-        float4 u = sl == slice ? tot[e] : load_through(slots + sl * 1024 + idx);
-        if (sl == 0) t = u;
-        else { t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w; }
-      }
-      tot[e] = t;
-    }
+    add_slices(slice);
     }
   }
   // to row-major through LDS, then 16-byte stores of eight fp16 values
