@@ -243,6 +243,33 @@ def test_gemm_whole_tile_kernel(K, M, N, Kd, dtype, pad):
     assert torch.equal(c.cpu(), -a.cpu()[:, perm])
 
 
+@pytest.mark.parametrize("M,N,Kd,dtype,kernel", [(4000, 2048, 96, torch.bfloat16, "gemm_dma_kernel<128x256>"), (1000, 1032, 64, torch.float16, "gemm_dma_kernel<128x128>"),
+                                                (130, 264, 96, torch.bfloat16, "gemm_dma_kernel<128x128>"), (4100, 4104, 64, torch.bfloat16, "gemm_dma_kernel"),
+                                                (4090, 2056, 32, torch.float16, "gemm_dma_kernel<256x128>"), (1, 8, 32, torch.bfloat16, "gemm_dma_kernel<128x128>")])
+def test_gemm_ragged_rows_and_columns_on_the_whole_k_tile_kernel(K, M, N, Kd, dtype, kernel):
+    # any M and any N that is a multiple of 8 (K in whole tiles of 32): the direct-to-LDS kernels clamp the addresses of the
+    # tiles that stick out of C and mask their stores; columns next to C in the same buffer stay as they were
+    torch.manual_seed(M + N)
+    pad = 8
+    A, B = (torch.randn(M, Kd) * 0.5).to(dtype).to(DEV), (torch.randn(Kd, N + pad) * 0.5).to(dtype).to(DEV)
+    Cfull = torch.full((M + 3, N + pad), 5.0, dtype=dtype, device=DEV)
+    a, b, c = A, B[:, :N], Cfull[:M, :N]
+    grid = (triton.cdiv(M, 128) * triton.cdiv(N, 128),)
+    k = K.matmul_tiles[grid](a, b, c, M, N, Kd, a.stride(0), 1, b.stride(0), 1, c.stride(0), 1, BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert k.function.last_kernel == kernel
+    assert relfro(c.cpu(), a.cpu().double() @ b.cpu().double()) <= 1e-2
+    assert torch.equal(Cfull[:, N:].cpu(), torch.full((M + 3, pad), 5.0, dtype=dtype)) and torch.equal(Cfull[M:].cpu(), torch.full((3, N + pad), 5.0, dtype=dtype))
+    perm = torch.randint(0, Kd, (N,))
+    sel = torch.zeros(Kd, N)
+    sel[perm, torch.arange(N)] = -1.0
+    B[:, :N] = sel.to(dtype).to(DEV)
+    K.matmul_tiles[grid](a, b, c, M, N, Kd, a.stride(0), 1, b.stride(0), 1, c.stride(0), 1, BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert torch.equal(c.cpu(), -a.cpu()[:, perm])
+    assert torch.equal(Cfull[:, N:].cpu(), torch.full((M + 3, pad), 5.0, dtype=dtype)) and torch.equal(Cfull[M:].cpu(), torch.full((3, N + pad), 5.0, dtype=dtype))
+
+
 @pytest.mark.parametrize("M,N,Kd,dtype", [(179, 321, 167, torch.bfloat16), (70, 90, 40, torch.float16), (512, 768, 96, torch.bfloat16),
                                          (1000, 130, 264, torch.float16)])
 def test_matmul_with_wraparound_operands(K, oracle_cpu, M, N, Kd, dtype):
@@ -1445,7 +1472,7 @@ def test_matmul_with_gathered_rows_is_exact_on_selections():
     c = torch.full((tokens, nd), 5.0, device=DEV, dtype=torch.bfloat16)
     k = X.grouped_rows_matmul[(triton.cdiv(tokens, 128), triton.cdiv(nd, 128))](a, b, c, rows, ids, tokens, kd, nd, kd, kd * nd, nd, nd, BM=128, BN=128, BK=64)
     torch.cuda.synchronize()
-    assert k.function.family == "gemm" and k.function.last_kernel.startswith("gemm_mfma_kernel")
+    assert k.function.family == "gemm" and k.function.last_kernel == "gemm_dma_kernel<128x128>"   # a ragged last row tile
     want = torch.full((tokens, nd), 5.0, device=DEV, dtype=torch.bfloat16)
     for blk, e in enumerate(ids.tolist()):
         r = slice(blk * 128, min(tokens, blk * 128 + 128))
@@ -1484,6 +1511,7 @@ def test_matmul_with_gathered_rows_on_whole_tiles(tokens, kd, nd, experts, kerne
 
 
 @pytest.mark.parametrize("M,N,K,kernel", [(512, 768, 96, "gemm_dma_kernel + epilogue"), (200, 300, 150, "gemm_mfma_kernel<128x128x64> + epilogue"),
+                                          (521, 776, 96, "gemm_dma_kernel + epilogue"),
                                           (2100, 2060, 72, "gemm_mfma_kernel<128x128x64> + epilogue")])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_gemm_with_fused_epilogue(M, N, K, kernel, dtype):

@@ -320,6 +320,7 @@ constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 1
 // rows of 64 bytes, a B instruction 1024 / (2 BN) k rows of 2 BN bytes (position q of k row k holds chunk
 // q ^ ((k & 3) << 2) of the row's BN / 8).  They take A rows through an index vector and a matrix id per block of rows
 // (p.a_rows, p.b_block): the A addresses are then 64-bit per lane.
+template <bool E> struct EdgeTile { static constexpr bool value = E; };
 template <bool BF16, int TM, int TN, class Ep>
 __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, int tiles_n, const Ep &ep) {
   using T = DmaTile<TM, TN>;
@@ -379,7 +380,8 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   const char *a_lane[A_DMA];
 #pragma unroll
   for (int i = 0; i < A_DMA; i++) {
-    const int row = 16 * (A_DMA * wave + i) + lane / 4;
+    // rows past M (the last row tile of a ragged problem) fetch row M - 1 again: they only reach outputs nobody stores
+    const int row = min(16 * (A_DMA * wave + i) + lane / 4, (int)(p.M - 1 - m0));
     const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
     a_voff[i] = (uint32_t)((row * p.lda + 8 * chunk) * 2);
     if (GATHER) {
@@ -392,7 +394,9 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
 #pragma unroll
   for (int i = 0; i < B_DMA; i++) {
     const int krow = B_KROWS * (B_DMA * wave + i) + lane / B_CHUNKS;
-    b_voff[i] = (uint32_t)((krow * p.ldb + 8 * ((lane & (B_CHUNKS - 1)) ^ ((krow & 3) << 2))) * 2);
+    // likewise, chunks of columns past N fetch the last whole chunk of the row (N is a multiple of 8)
+    const int chunk = min((lane & (B_CHUNKS - 1)) ^ ((krow & 3) << 2), (int)((p.N - n0) / 8 - 1));
+    b_voff[i] = (uint32_t)((krow * p.ldb + 8 * chunk) * 2);
   }
   const char *a_base = (const char *)((const uint16_t *)p.a + m0 * p.lda);
   const uint32_t lds0 = (uint32_t)(uintptr_t)TTS_LDS(smem);
@@ -506,23 +510,31 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   typedef float f32x2_t __attribute__((ext_vector_type(2)));
   const bool odd = lane & 1;
   const uint32_t sel = odd ? 0x03020706u : 0x05040100u;  // odd: high halves of (neighbour, mine); even: low halves of (mine, neighbour)
+  // EDGE: the tile sticks out of C (ragged M, or N that is not a multiple of the tile): elements outside are neither
+  // evaluated (the functor may read a bias or a residual at the element's position) nor stored.
+  auto store_tile = [&](auto edge) {
+    constexpr bool EDGE = decltype(edge)::value;
 #pragma unroll
-  for (int i = 0; i < TM; i++)
+    for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
-      const int64_t col = n0 + wn * TN * 32 + j * 32 + (lane & 31) - (odd ? 1 : 0);
+      for (int j = 0; j < TN; j++) {
+        const int64_t col = n0 + wn * TN * 32 + j * 32 + (lane & 31) - (odd ? 1 : 0);
 #pragma unroll
-      for (int v = 0; v < 16; v += 2) {
-        const int64_t er = m0 + wm * TM * 32 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), ec = n0 + wn * TN * 32 + j * 32 + (lane & 31);
-        const f32x2_t pr = {ep(acc[i][j][v], er, ec), ep(acc[i][j][v + 1], er + 1, ec)};
-        const uint32_t pk = BF16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, bf16x2_t))
-                                 : __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, f16x2_t));
-        const uint32_t nb = __builtin_amdgcn_mov_dpp(pk, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]: the neighbour's pair
-        const uint32_t w = __builtin_amdgcn_perm(nb, pk, sel);
-        const int64_t row = m0 + wm * TM * 32 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3) + (odd ? 1 : 0);
-        __builtin_nontemporal_store(w, reinterpret_cast<uint32_t *>(&C[row * p.ldc + col]));
+        for (int v = 0; v < 16; v += 2) {
+          const int64_t er = m0 + wm * TM * 32 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3), ec = n0 + wn * TN * 32 + j * 32 + (lane & 31);
+          const bool in0 = !EDGE || (er < p.M && ec < p.N), in1 = !EDGE || (er + 1 < p.M && ec < p.N);
+          const f32x2_t pr = {in0 ? ep(acc[i][j][v], er, ec) : 0.f, in1 ? ep(acc[i][j][v + 1], er + 1, ec) : 0.f};
+          const uint32_t pk = BF16 ? __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, bf16x2_t))
+                                   : __builtin_bit_cast(uint32_t, __builtin_convertvector(pr, f16x2_t));
+          const uint32_t nb = __builtin_amdgcn_mov_dpp(pk, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]: the neighbour's pair
+          const uint32_t w = __builtin_amdgcn_perm(nb, pk, sel);
+          const int64_t row = m0 + wm * TM * 32 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3) + (odd ? 1 : 0);
+          if (!EDGE || (row < p.M && col < p.N)) __builtin_nontemporal_store(w, reinterpret_cast<uint32_t *>(&C[row * p.ldc + col]));
+        }
       }
-    }
+  };
+  if (m0 + BM > p.M || n0 + BN > p.N) store_tile(EdgeTile<true>());
+  else store_tile(EdgeTile<false>());
 }
 
 }  // namespace tts_gemm_device

@@ -58,17 +58,18 @@ hipError_t launch_gemm_dma(const GemmParams &p, hipStream_t s) {
   auto kern = gemm_dma_kernel<BF16, TM, TN>;
   static const hipError_t attr = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return attr;
-  int tiles_m = (int)(p.M / T::BM), tiles_n = (int)(p.N / T::BN);
+  int tiles_m = (int)((p.M + T::BM - 1) / T::BM), tiles_n = (int)((p.N + T::BN - 1) / T::BN);
   hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds, s, p, tiles_m, tiles_n);
   return hipGetLastError();
 }
 
-// whole bm x bn x 32 tiles, 16-byte aligned rows, and per-lane byte offsets that fit 32 bits
+// Whole K tiles of 32, N a multiple of 8 (whole 16-byte chunks of B rows), any M; 16-byte aligned rows, and per-lane
+// byte offsets that fit 32 bits.  Tiles that stick out of C clamp their addresses and mask their stores.
 bool gemm_dma_ok(const GemmParams &p, int64_t bm, int64_t bn) {
   if (p.a_trans || p.b_trans) return false;
   if ((p.a_rows || p.b_block) && bm != 128) return false;  // gathered rows: 128-row tiles (64-bit A addresses per lane)
   if (p.b_block && p.b_block_rows % bm != 0) return false;
-  return p.M % bm == 0 && p.N % bn == 0 && p.K % F_BK == 0 && p.K >= F_BK && p.lda % 8 == 0 && p.ldb % 8 == 0 &&
+  return p.M >= 1 && p.N >= 8 && p.N % 8 == 0 && p.K % F_BK == 0 && p.K >= F_BK && p.lda % 8 == 0 && p.ldb % 8 == 0 &&
          ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0 && p.lda < (1 << 22) && p.ldb < (1 << 25) &&
          (!p.b_block || p.b_block_stride % 8 == 0) && p.ldc % 2 == 0 && ((uintptr_t)p.c & 3) == 0;  // C is written in 4-byte pairs
 }
@@ -488,27 +489,35 @@ hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
   static const char *tile_env = getenv("TTS_GEMM_TILE");  // tuning aid: set = the any-shape kernel even for whole tiles
   static const char *dma_env = getenv("TTS_GEMM_DMA");    // tuning aid: "256x256", "128x256", "256x128", "128x128" or unset
   if (!tile_env) {
-    // Whole tiles go to the direct-to-LDS kernels: the largest tile that still gives every CU a workgroup.
+    // Whole K tiles go to the direct-to-LDS kernels.
     static const int cus = [] {
       int dev = 0, n = 0;
       if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
       return n;
     }();
-    auto tiles = [&](int64_t bm, int64_t bn) { return (p.M / bm) * (p.N / bn); };
-    auto want = [&](const char *tag, int64_t bm, int64_t bn, int64_t enough) {
-      if (dma_env) return std::string(dma_env) == tag && gemm_dma_ok(p, bm, bn);
-      return gemm_dma_ok(p, bm, bn) && tiles(bm, bn) >= enough;
-    };
+    auto tiles = [&](int64_t bm, int64_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
+    // Among the tiles that give every CU a workgroup (128 x 128: always), the one with the least padded work per unit
+    // of the tile's measured efficiency at 4096^3 (105 / 136 / 144 / 179 us): a ragged edge counts against a tile that
+    // overshoots it by more.
+    struct Cand { const char *tag; int64_t bm, bn, enough; double eff; };
+    static const Cand cands[4] = {{"256x256", 256, 256, cus, 1.0}, {"128x256", 128, 256, cus, 0.77}, {"256x128", 256, 128, cus, 0.73}, {"128x128", 128, 128, 1, 0.59}};
+    const Cand *best = nullptr;
+    double best_cost = 0;
+    for (const Cand &c : cands) {
+      if (!gemm_dma_ok(p, c.bm, c.bn)) continue;
+      if (dma_env ? std::string(dma_env) != c.tag : tiles(c.bm, c.bn) < c.enough) continue;
+      const double cost = (double)(tiles(c.bm, c.bn) * c.bm * c.bn) / c.eff;
+      if (!best || cost < best_cost) { best = &c; best_cost = cost; }
+    }
 #define TTS_DMA(TM, TN, TAG)                                                                                  \
   do {                                                                                                        \
     *name = TAG;                                                                                              \
     return p.is_bf16 ? launch_gemm_dma<true, TM, TN>(p, s) : launch_gemm_dma<false, TM, TN>(p, s);            \
   } while (0)
-    if (want("256x256", 256, 256, cus)) TTS_DMA(4, 4, "gemm_dma_kernel");
-    if (want("128x256", 128, 256, cus)) TTS_DMA(2, 4, "gemm_dma_kernel<128x256>");
-    if (want("256x128", 256, 128, cus)) TTS_DMA(4, 2, "gemm_dma_kernel<256x128>");
-    if (want("128x128", 128, 128, 1)) TTS_DMA(2, 2, "gemm_dma_kernel<128x128>");
-    if (!dma_env && gemm_dma_ok(p, 256, 256)) TTS_DMA(4, 4, "gemm_dma_kernel");
+    if (best && best->bm == 256 && best->bn == 256) TTS_DMA(4, 4, "gemm_dma_kernel");
+    if (best && best->bm == 128 && best->bn == 256) TTS_DMA(2, 4, "gemm_dma_kernel<128x256>");
+    if (best && best->bm == 256 && best->bn == 128) TTS_DMA(4, 2, "gemm_dma_kernel<256x128>");
+    if (best) TTS_DMA(2, 2, "gemm_dma_kernel<128x128>");
 #undef TTS_DMA
   }
   // anything else: 128 x 128 x 64 tiles, two workgroups per CU (a 256 x 256 x 32 form of the same kernel measured behind it
