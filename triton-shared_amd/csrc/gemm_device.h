@@ -320,8 +320,11 @@ constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 1
 // rows of 64 bytes, a B instruction 1024 / (2 BN) k rows of 2 BN bytes (position q of k row k holds chunk
 // q ^ ((k & 3) << 2) of the row's BN / 8).  They take A rows through an index vector and a matrix id per block of rows
 // (p.a_rows, p.b_block): the A addresses are then 64-bit per lane.
+// BT: B is column-major (p.b_trans: element (k, n) at b[k + n * ldb], the tutorial's `b.T` and the weight layout of a
+// linear layer).  Its stage is then laid out like A's, [BN columns][64 bytes] with the same swizzle, and an operand is
+// one 16-byte read; nothing needs transposing.
 template <bool E> struct EdgeTile { static constexpr bool value = E; };
-template <bool BF16, int TM, int TN, class Ep>
+template <bool BF16, int TM, int TN, class Ep, bool BT = false>
 __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, int tiles_n, const Ep &ep) {
   using T = DmaTile<TM, TN>;
   constexpr int BM = T::BM, BN = T::BN, STAGES = T::STAGES, A_BYTES = T::A_BYTES, STAGE_BYTES = T::STAGE_BYTES, ROWB = T::B_ROW_BYTES;
@@ -366,7 +369,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   }
   const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
 
-  const char *b_base = (const char *)((const uint16_t *)p.b + n0);
+  const char *b_base = (const char *)((const uint16_t *)p.b + (BT ? n0 * p.ldb : n0));
   if (GATHER && p.b_block) {  // the rows of this tile multiply a matrix of their own; a negative id: nothing to do for them
     const int which = p.b_block[m0 / p.b_block_rows];
     if (which < 0) return;
@@ -393,6 +396,11 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   }
 #pragma unroll
   for (int i = 0; i < B_DMA; i++) {
+    if (BT) {  // as A: columns 16 (B_DMA w + i) + lane / 4 of the tile, those past N fetch column N - 1
+      const int col = min(16 * (B_DMA * wave + i) + lane / 4, (int)(p.N - 1 - n0));
+      b_voff[i] = (uint32_t)((col * p.ldb + 8 * ((lane & 3) ^ ((lane >> 4) & 3))) * 2);
+      continue;
+    }
     const int krow = B_KROWS * (B_DMA * wave + i) + lane / B_CHUNKS;
     // likewise, chunks of columns past N fetch the last whole chunk of the row (N is a multiple of 8)
     const int chunk = min((lane & (B_CHUNKS - 1)) ^ ((krow & 3) << 2), (int)((p.N - n0) / 8 - 1));
@@ -424,7 +432,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
       if (GATHER) dma_lane(a_lane[n] + (int64_t)tc * F_BK * 2, at);
       else dma(a_base + (int64_t)tc * F_BK * 2, a_voff[n], at);
     } else {
-      dma(b_base + (int64_t)tc * F_BK * p.ldb * 2, b_voff[n - A_DMA], st + A_BYTES + (B_DMA * wave_u + n - A_DMA) * 1024);
+      dma(b_base + (BT ? (int64_t)tc * F_BK * 2 : (int64_t)tc * F_BK * p.ldb * 2), b_voff[n - A_DMA], st + A_BYTES + (B_DMA * wave_u + n - A_DMA) * 1024);
     }
   };
 
@@ -446,13 +454,18 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
-  constexpr int READS = TM + 2 * TN, MFMAS = TM * TN;
+  // BT: column c = wn * TN * 32 + j * 32 + lane % 32 of the tile, chunk 2 ks + lane / 32 at position chunk ^ ((c / 4) & 3)
+  const int bc = wn * TN * 32 + (lane & 31);
+  const int bt_off = A_BYTES + bc * 64, bt_sw = (bc >> 2) & 3;
+  constexpr int READS = BT ? TM + TN : TM + 2 * TN, MFMAS = TM * TN;
   uint4 af[2][TM], bf[2][TN];
   // one fragment read (n < TM: A row block n; else B column block (n - TM) / 2, k half (n - TM) % 2)
   auto read_one = [&](int t, int ks, int n, uint4 (&a)[TM], uint4 (&b)[TN]) {
     const char *st = smem + (t % STAGES) * STAGE_BYTES;
     if (n < TM) {
       a[n] = *reinterpret_cast<const uint4 *>(st + a_off + n * 2048 + (((2 * ks + (lane >> 5)) ^ a_sw) << 4));
+    } else if (BT) {
+      b[n - TM] = *reinterpret_cast<const uint4 *>(st + bt_off + (n - TM) * 2048 + (((2 * ks + (lane >> 5)) ^ bt_sw) << 4));
     } else {
       const int j = (n - TM) >> 1, h = (n - TM) & 1;
       const char *bp = st + b_off + ks * 16 * ROWB + (((b_chunk + 4 * j) ^ b_sw) << 4) + h * 4 * ROWB;
