@@ -205,7 +205,9 @@ namespace {
 // Compiled code objects are kept on disk, as the reference keeps its compiled launchers in Triton's cache
 // (backend/driver.py:274-282,344-345): <dir>/<hash of source, options and hipRTC version>.hsaco, with <dir> =
 // $TTS_RTC_CACHE, else $TRITON_CACHE_DIR/tts_rtc, else $HOME/.triton/cache/tts_rtc.  TTS_RTC_CACHE=off disables it.
-const char *const RTC_OPTS[] = {"--offload-arch=gfx950", "-O3", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt"};
+// (no packed fp32 instructions, as in the library's own build: the compiler forms them from ordinary float code otherwise)
+const char *const RTC_OPTS[] = {"--offload-arch=gfx950", "-O3", "-ffp-contract=off", "-fhip-fp32-correctly-rounded-divide-sqrt",
+                                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
 
 std::string cache_dir() {
   const char *own = getenv("TTS_RTC_CACHE");
