@@ -437,6 +437,37 @@ def test_gemm_with_column_major_b(K, M, N, Kd, dtype, kernel):
     assert torch.equal(c.cpu(), -a.cpu()[:, perm])
 
 
+@pytest.mark.parametrize("M,N,Kd,dtype,b_too,kernel", [(1024, 512, 96, torch.bfloat16, False, "gemm_dma_kernel<128x128>"), (4096, 4096, 64, torch.bfloat16, False, "gemm_dma_kernel"),
+                                                      (1000, 264, 64, torch.float16, True, "gemm_dma_kernel<128x128>"), (4096, 2048, 32, torch.float16, True, "gemm_dma_kernel<128x256>"),
+                                                      (4088, 2176, 96, torch.bfloat16, False, "gemm_dma_kernel<256x128>"), (1004, 256, 64, torch.bfloat16, False, "gemm_mfma_kernel<128x128x64>")])
+def test_gemm_with_column_major_a_on_whole_k_tiles(K, M, N, Kd, dtype, b_too, kernel):
+    # A stored [K, M] (the product A^T B of a weight gradient), alone or with a column-major B: whole K tiles of 32 and M a
+    # multiple of 8 run on the direct-to-LDS kernels (A's stage laid out like a row-major B's); exact on a selection
+    torch.manual_seed(M + N + Kd)
+    at = torch.randint(-8, 9, (Kd, M)).to(dtype).to(DEV)
+    a = at.t()
+    perm = torch.randint(0, Kd, (N,))
+    sel = torch.zeros(Kd, N)
+    sel[perm, torch.arange(N)] = -1.0
+    b = sel.t().contiguous().to(dtype).to(DEV).t() if b_too else sel.to(dtype).to(DEV)
+    Cfull = torch.full((M + 2, N + 8), 5.0, dtype=dtype, device=DEV)
+    c = Cfull[:M, :N]
+    grid = (triton.cdiv(M, 128) * triton.cdiv(N, 128),)
+    k = K.matmul_tiles[grid](a, b, c, M, N, Kd, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+                             BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and k.function.last_kernel == kernel
+    assert torch.equal(c.cpu(), -a.cpu()[:, perm])
+    assert torch.equal(Cfull[:, N:].cpu(), torch.full((M + 2, 8), 5.0, dtype=dtype)) and torch.equal(Cfull[M:].cpu(), torch.full((2, N + 8), 5.0, dtype=dtype))
+    # and a random product within the family's tolerance
+    at.copy_((torch.randn(Kd, M) * 0.5).to(dtype))
+    bb = (torch.randn(N, Kd) * 0.5).to(dtype).to(DEV).t() if b_too else (torch.randn(Kd, N) * 0.5).to(dtype).to(DEV)
+    K.matmul_tiles[grid](a, bb, c, M, N, Kd, a.stride(0), a.stride(1), bb.stride(0), bb.stride(1), c.stride(0), c.stride(1),
+                         BM=128, BN=128, BK=64, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert relfro(c.float(), a.float() @ bb.float()) <= 1e-2
+
+
 def test_gemm_with_column_major_a_and_with_strides_no_kernel_takes(K):
     torch.manual_seed(11)
     M, N, Kd = 300, 260, 136

@@ -324,14 +324,17 @@ constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 1
 // linear layer).  Its stage is then laid out like A's, [BN columns][64 bytes] with the same swizzle, and an operand is
 // one 16-byte read; nothing needs transposing.
 template <bool E> struct EdgeTile { static constexpr bool value = E; };
-template <bool BF16, int TM, int TN, class Ep, bool BT = false>
+// AT: A is column-major (p.a_trans: element (m, k) at a[m + k * lda]).  Its stage is laid out like a row-major B's,
+// [32 k rows][2 BM bytes], and read through the same transposing LDS read.
+template <bool BF16, int TM, int TN, class Ep, bool BT = false, bool AT = false>
 __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, int tiles_n, const Ep &ep) {
   using T = DmaTile<TM, TN>;
   constexpr int BM = T::BM, BN = T::BN, STAGES = T::STAGES, A_BYTES = T::A_BYTES, STAGE_BYTES = T::STAGE_BYTES, ROWB = T::B_ROW_BYTES;
   constexpr int A_DMA = T::A_DMA, B_DMA = T::B_DMA, DMA = T::DMA;
   constexpr int B_KROWS = 1024 / ROWB;       // k rows one B instruction covers
   constexpr int B_CHUNKS = ROWB / 16;        // 16-byte chunks per k row
-  constexpr bool GATHER = !(TM == 4 && TN == 4);
+  constexpr bool GATHER = !(TM == 4 && TN == 4) && !AT;
+  constexpr int A_ROWB = BM * 2, A_KROWS = 1024 / A_ROWB, A_CHUNKS = A_ROWB / 16;  // AT: bytes per k row, k rows per instruction, chunks per k row
   static_assert(DMA % 2 == 0, "half of a tile's loads go out in each phase");
 #ifdef TTS_GEMM_RTC
   __shared__ __align__(16) char dma_smem[T::LDS_BYTES];
@@ -383,6 +386,12 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   const char *a_lane[A_DMA];
 #pragma unroll
   for (int i = 0; i < A_DMA; i++) {
+    if (AT) {  // as a row-major B: k rows A_KROWS (A_DMA w + i) + lane / A_CHUNKS, chunks of rows past M fetch the last whole chunk (M % 8 == 0)
+      const int krow = A_KROWS * (A_DMA * wave + i) + lane / A_CHUNKS;
+      const int chunk = min((lane & (A_CHUNKS - 1)) ^ ((krow & 3) << 2), (int)((p.M - m0) / 8 - 1));
+      a_voff[i] = (uint32_t)((krow * p.lda + 8 * chunk) * 2);
+      continue;
+    }
     // rows past M (the last row tile of a ragged problem) fetch row M - 1 again: they only reach outputs nobody stores
     const int row = min(16 * (A_DMA * wave + i) + lane / 4, (int)(p.M - 1 - m0));
     const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
@@ -406,7 +415,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
     const int chunk = min((lane & (B_CHUNKS - 1)) ^ ((krow & 3) << 2), (int)((p.N - n0) / 8 - 1));
     b_voff[i] = (uint32_t)((krow * p.ldb + 8 * chunk) * 2);
   }
-  const char *a_base = (const char *)((const uint16_t *)p.a + m0 * p.lda);
+  const char *a_base = (const char *)((const uint16_t *)p.a + (AT ? m0 : m0 * p.lda));
   const uint32_t lds0 = (uint32_t)(uintptr_t)TTS_LDS(smem);
   const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int nk = (int)(p.K / F_BK);
@@ -430,7 +439,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
     if (n < A_DMA) {
       const uint32_t at = st + (A_DMA * wave_u + n) * 1024;
       if (GATHER) dma_lane(a_lane[n] + (int64_t)tc * F_BK * 2, at);
-      else dma(a_base + (int64_t)tc * F_BK * 2, a_voff[n], at);
+      else dma(a_base + (AT ? (int64_t)tc * F_BK * p.lda * 2 : (int64_t)tc * F_BK * 2), a_voff[n], at);
     } else {
       dma(b_base + (BT ? (int64_t)tc * F_BK * 2 : (int64_t)tc * F_BK * p.ldb * 2), b_voff[n - A_DMA], st + A_BYTES + (B_DMA * wave_u + n - A_DMA) * 1024);
     }
@@ -457,17 +466,26 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   // BT: column c = wn * TN * 32 + j * 32 + lane % 32 of the tile, chunk 2 ks + lane / 32 at position chunk ^ ((c / 4) & 3)
   const int bc = wn * TN * 32 + (lane & 31);
   const int bt_off = A_BYTES + bc * 64, bt_sw = (bc >> 2) & 3;
-  constexpr int READS = BT ? TM + TN : TM + 2 * TN, MFMAS = TM * TN;
+  // AT: as the row-major B below, with the wavefront's rows in place of its columns
+  const int at_chunk = wm * TM * 4 + 2 * (q & 1) + ((r16 & 3) >> 1);
+  const int at_off = (8 * (q >> 1) + (r16 >> 2)) * A_ROWB + 8 * (r16 & 1);
+  constexpr int A_READS = AT ? 2 * TM : TM, READS = A_READS + (BT ? TN : 2 * TN), MFMAS = TM * TN;
   uint4 af[2][TM], bf[2][TN];
   // one fragment read (n < TM: A row block n; else B column block (n - TM) / 2, k half (n - TM) % 2)
   auto read_one = [&](int t, int ks, int n, uint4 (&a)[TM], uint4 (&b)[TN]) {
     const char *st = smem + (t % STAGES) * STAGE_BYTES;
-    if (n < TM) {
+    if (n < A_READS && AT) {
+      const int i = n >> 1, h = n & 1;
+      const char *ap = st + at_off + ks * 16 * A_ROWB + (((at_chunk + 4 * i) ^ b_sw) << 4) + h * 4 * A_ROWB;
+      s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)TTS_LDS(ap));
+      uint2 v2 = __builtin_bit_cast(uint2, v);
+      if (h == 0) { a[i].x = v2.x; a[i].y = v2.y; } else { a[i].z = v2.x; a[i].w = v2.y; }
+    } else if (n < A_READS) {
       a[n] = *reinterpret_cast<const uint4 *>(st + a_off + n * 2048 + (((2 * ks + (lane >> 5)) ^ a_sw) << 4));
     } else if (BT) {
-      b[n - TM] = *reinterpret_cast<const uint4 *>(st + bt_off + (n - TM) * 2048 + (((2 * ks + (lane >> 5)) ^ bt_sw) << 4));
+      b[n - A_READS] = *reinterpret_cast<const uint4 *>(st + bt_off + (n - A_READS) * 2048 + (((2 * ks + (lane >> 5)) ^ bt_sw) << 4));
     } else {
-      const int j = (n - TM) >> 1, h = (n - TM) & 1;
+      const int j = (n - A_READS) >> 1, h = (n - A_READS) & 1;
       const char *bp = st + b_off + ks * 16 * ROWB + (((b_chunk + 4 * j) ^ b_sw) << 4) + h * 4 * ROWB;
       s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)TTS_LDS(bp));
       uint2 v2 = __builtin_bit_cast(uint2, v);

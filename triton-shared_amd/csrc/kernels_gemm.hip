@@ -46,16 +46,16 @@ hipError_t launch_gemm_cfg(const GemmParams &p, hipStream_t s) {
 }
 
 
-template <bool BF16, int TM, int TN, bool BT>
+template <bool BF16, int TM, int TN, bool BT, bool AT>
 __global__ __launch_bounds__(256) void gemm_dma_kernel(GemmParams p, int tiles_m, int tiles_n) {
-  gemm_dma_body<BF16, TM, TN, IdentityEp, BT>(p, tiles_m, tiles_n, IdentityEp());
+  gemm_dma_body<BF16, TM, TN, IdentityEp, BT, AT>(p, tiles_m, tiles_n, IdentityEp());
 }
 
-template <bool BF16, int TM, int TN, bool BT>
+template <bool BF16, int TM, int TN, bool BT, bool AT>
 hipError_t launch_gemm_dma_t(const GemmParams &p, hipStream_t s) {
   using T = DmaTile<TM, TN>;
   constexpr size_t lds = T::LDS_BYTES;
-  auto kern = gemm_dma_kernel<BF16, TM, TN, BT>;
+  auto kern = gemm_dma_kernel<BF16, TM, TN, BT, AT>;
   static const hipError_t attr = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return attr;
   int tiles_m = (int)((p.M + T::BM - 1) / T::BM), tiles_n = (int)((p.N + T::BN - 1) / T::BN);
@@ -63,22 +63,25 @@ hipError_t launch_gemm_dma_t(const GemmParams &p, hipStream_t s) {
   return hipGetLastError();
 }
 
+// one instantiation per layout of the operands in memory
 template <bool BF16, int TM, int TN>
 hipError_t launch_gemm_dma(const GemmParams &p, hipStream_t s) {
-  return p.b_trans ? launch_gemm_dma_t<BF16, TM, TN, true>(p, s) : launch_gemm_dma_t<BF16, TM, TN, false>(p, s);
+  if (p.a_trans) return p.b_trans ? launch_gemm_dma_t<BF16, TM, TN, true, true>(p, s) : launch_gemm_dma_t<BF16, TM, TN, false, true>(p, s);
+  return p.b_trans ? launch_gemm_dma_t<BF16, TM, TN, true, false>(p, s) : launch_gemm_dma_t<BF16, TM, TN, false, false>(p, s);
 }
 
-// Whole K tiles of 32, N a multiple of 8 (whole 16-byte chunks of B rows), any M; 16-byte aligned rows, and per-lane
-// byte offsets that fit 32 bits.  Tiles that stick out of C clamp their addresses and mask their stores.
+// Whole K tiles of 32, N a multiple of 8 (whole 16-byte chunks of B rows), any M (a multiple of 8 when A is column-major);
+// 16-byte aligned rows, and per-lane byte offsets that fit 32 bits.  Either operand may be column-major.  Tiles that
+// stick out of C clamp their addresses and mask their stores.
 bool gemm_dma_ok(const GemmParams &p, int64_t bm, int64_t bn) {
-  if (p.a_trans) return false;  // (a column-major B is taken: its stage is laid out like A's)
+  if (p.a_trans && (p.M % 8 != 0 || p.a_rows || p.b_block)) return false;
   if ((p.a_rows || p.b_block) && bm != 128) return false;  // gathered rows: 128-row tiles (64-bit A addresses per lane)
   if (p.b_block && p.b_block_rows % bm != 0) return false;
   return p.M >= 1 && p.N >= 8 && p.N % 8 == 0 && p.K % F_BK == 0 && p.K >= F_BK && p.lda % 8 == 0 && p.ldb % 8 == 0 &&
-         ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0 && p.lda < (1 << 22) && p.ldb < (p.b_trans ? (1 << 22) : (1 << 25)) &&
+         ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0 && p.lda < (p.a_trans ? (1 << 25) : (1 << 22)) && p.ldb < (p.b_trans ? (1 << 22) : (1 << 25)) &&
          (!p.b_block || p.b_block_stride % 8 == 0) && p.ldc % 2 == 0 && ((uintptr_t)p.c & 3) == 0;  // C is written in 4-byte pairs
 }
-bool gemm_fast_path_ok(const GemmParams &p) { return !p.b_trans && gemm_dma_ok(p, F_BM, F_BN); }  // (the kernel compiled with an epilogue)
+bool gemm_fast_path_ok(const GemmParams &p) { return !p.a_trans && !p.b_trans && gemm_dma_ok(p, F_BM, F_BN); }  // (the kernel compiled with an epilogue)
 
 // ------------------------------------------------------ int8-weight GEMM
 // Workgroup: NW wavefronts share one 128-column slab of W and split its K range
