@@ -515,15 +515,17 @@ def test_w8a16_beyond_the_decode_shape(K, oracle_cpu, M):
 def test_softmax_rows_the_row_kernel_declines(K, oracle_cpu):
     import extra_kernels as X
     torch.manual_seed(5)
-    # rows of 32768 columns: more than the row kernel keeps in registers
-    x = torch.randn(6, 30000)
-    xd = x.to(DEV)
-    od = torch.full((6, 30000), -9.0, device=DEV)
-    k = K.row_softmax[(6,)](od, xd, xd.stride(0), od.stride(0), 30000, BLOCK=32768)
-    torch.cuda.synchronize()
-    assert k.function.family == "tile_program"
-    assert torch.allclose(od.cpu(), torch.softmax(x, 1))
-    assert (od.cpu() - oracle_cpu.row_softmax(x, BLOCK=32768)).abs().max().item() <= 1e-5
+    # rows of 32768 and 65536 columns: 8 and 16 wavefronts per row on the row kernel; 131072: more than it keeps in registers
+    for cols, block, family in [(30000, 32768, "row_softmax"), (40001, 65536, "row_softmax"), (70000, 131072, "tile_program")]:
+        x = torch.randn(6, cols)
+        xd = x.to(DEV)
+        od = torch.full((7, cols), -9.0, device=DEV)
+        k = K.row_softmax[(6,)](od, xd, xd.stride(0), od.stride(0), cols, BLOCK=block)
+        torch.cuda.synchronize()
+        assert k.function.family == family
+        assert torch.allclose(od[:6].cpu(), torch.softmax(x, 1))
+        assert (od[:6].cpu() - oracle_cpu.row_softmax(x, BLOCK=block)).abs().max().item() <= 1e-5
+        assert torch.equal(od[6].cpu(), torch.full((cols,), -9.0))
     # every third element of the input row
     x = torch.randn(40, 3 * 700)
     xd = x.to(DEV)

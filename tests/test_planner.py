@@ -515,9 +515,9 @@ def test_declined_details_of_a_handwritten_family_fall_through(native):
     text = native.ttir_to_structured(compile_ttir(X.strided_row_softmax, sig, {"BLOCK": 1024}))
     assert native.PlanHandle(native.structured_to_plan(text)[0]).family == "tile_program"
     sig = {"out_ptr": "*fp32", "in_ptr": "*fp32", "in_pitch": "i32", "out_pitch": "i32", "n_cols": "i32", "BLOCK": "constexpr"}
-    text = native.ttir_to_structured(compile_ttir(K.row_softmax, sig, {"BLOCK": 32768}))
+    text = native.ttir_to_structured(compile_ttir(K.row_softmax, sig, {"BLOCK": 131072}))
     assert native.PlanHandle(native.structured_to_plan(text)[0]).family == "tile_program"
-    text = native.ttir_to_structured(compile_ttir(K.row_softmax, sig, {"BLOCK": 16384}))
+    text = native.ttir_to_structured(compile_ttir(K.row_softmax, sig, {"BLOCK": 65536}))
     assert native.PlanHandle(native.structured_to_plan(text)[0]).family == "row_softmax"
 
 

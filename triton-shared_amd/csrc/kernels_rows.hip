@@ -134,10 +134,10 @@ typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
 template <int NPL, int WAVES, bool NAN_PROP, bool VEC, int WG = 256>
 __global__ __launch_bounds__(WG) void softmax_f32_kernel(SoftmaxParams p, int gx, int gy, int64_t programs) {
-  static_assert(WAVES == 1 || WG == 256, "rows that span wavefronts meet in red[], one row per workgroup");
+  static_assert(WAVES == 1 || WG == WAVES * WAVE, "rows that span wavefronts meet in red[], one row per workgroup");
   constexpr int T = WAVES * WAVE;
   constexpr int ROWS_PER_WG = WG / T;
-  __shared__ float red[4];
+  __shared__ float red[WAVES];
   const int sub = threadIdx.x / T, t = threadIdx.x % T;
   const int64_t prog = (int64_t)blockIdx.x * ROWS_PER_WG + sub;
   const bool active = prog < programs;
@@ -842,6 +842,9 @@ hipError_t launch_softmax(const SoftmaxParams &p, int gx, int gy, int gz, hipStr
   if (b <= 4096) return launch_softmax_cfg<16, 4>(p, gx, gy, gz, s);
   if (b <= 8192) return launch_softmax_cfg<32, 4>(p, gx, gy, gz, s);
   if (b <= 16384) return launch_softmax_cfg<64, 4>(p, gx, gy, gz, s);
+  // longer rows: more wavefronts per row, still one pass over memory with the row in registers
+  if (b <= 32768) return launch_softmax_cfg<64, 8, 512>(p, gx, gy, gz, s);
+  if (b <= 65536) return launch_softmax_cfg<64, 16, 1024>(p, gx, gy, gz, s);
   return hipErrorInvalidValue;
 }
 

@@ -351,7 +351,7 @@ bool try_softmax(Plan &pl) {
   unit_stride(m, ld->acc, F);
   unit_stride(m, st->acc, F);
   if (ld->acc.sizes != st->acc.sizes) refuse(F, "its load and store blocks differ in size");
-  if (ld->acc.sizes[0] > 16384) refuse(F, "its rows are longer than the 16384 elements the row kernel keeps in registers");
+  if (ld->acc.sizes[0] > 65536) refuse(F, "its rows are longer than the 65536 elements the row kernel keeps in registers");
   pl.family = Family::RowSoftmax;
   pl.k["block"] = ld->acc.sizes[0];
   pl.k["in_arg"] = ld->acc.base_arg;

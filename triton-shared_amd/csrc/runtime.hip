@@ -247,7 +247,7 @@ void bind_softmax(const Resolver &r, Bound &b) {
   p.block = (int)r.pl.k.at("block");
   p.other = (float)r.pl.f.at("other");
   p.propagate_nan = r.pl.signature.find("maximumf") != std::string::npos;
-  if (p.block > 16384) throw Unsupported("row_softmax: block sizes above 16384 are not implemented");
+  if (p.block > 65536) throw Unsupported("row_softmax: block sizes above 65536 are not implemented");
   std::ostringstream os;
   os << "kernel=softmax_f32\nblock=" << p.block << "\nd_in=" << p.d_in << "\nd_out=" << p.d_out << "\nother=" << p.other
      << "\nin_off=" << show(p.in_off) << "\nout_off=" << show(p.out_off) << "\n";
