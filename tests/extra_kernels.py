@@ -1053,3 +1053,15 @@ def strided_row_softmax(out_ptr, in_ptr, in_pitch, out_pitch, col_stride, n_cols
     e = tl.exp(v - tl.max(v, axis=0))
     p = e / tl.sum(e, axis=0)
     tl.store(out_ptr + r * out_pitch + cols, p, mask=cols < n_cols)
+
+
+@triton.jit
+def transpose_tiles(src, dst, R, C, BR: tl.constexpr, BC: tl.constexpr):
+    # dst[C, R] = src[R, C]^T in tiles of [BR, BC]: the transposed tile is read coalesced, turned in LDS and written coalesced
+    pr = tl.program_id(0)
+    pc = tl.program_id(1)
+    r = pr * BR + tl.arange(0, BR)
+    c = pc * BC + tl.arange(0, BC)
+    m = (r[:, None] < R) & (c[None, :] < C)
+    x = tl.load(src + r[:, None] * C + c[None, :], mask=m, other=0.0)
+    tl.store(dst + c[:, None] * R + r[None, :], tl.trans(x * 2.0), mask=tl.trans(m))

@@ -512,6 +512,21 @@ def test_w8a16_beyond_the_decode_shape(K, oracle_cpu, M):
     assert relfro(cd.cpu(), a.double() @ (w.half() * s[None, :]).double()) <= 1e-2
 
 
+@pytest.mark.parametrize("R,C,BR,BC", [(200, 300, 64, 64), (513, 130, 32, 128), (64, 64, 64, 64), (1000, 77, 128, 32)])
+def test_tiled_transpose_goes_through_lds(R, C, BR, BC):
+    # tl.trans of a loaded tile: the load is copied to LDS (pitch = columns + 1) and read back transposed, so that both
+    # the loads and the stores of a wavefront are contiguous; ragged edges in both dimensions, square and oblong tiles
+    import extra_kernels as X
+    torch.manual_seed(R + C)
+    x = torch.randn(R, C, device=DEV)
+    out = torch.full((C + 1, R), -7.0, device=DEV)
+    k = X.transpose_tiles[(triton.cdiv(R, BR), triton.cdiv(C, BC))](x, out, R, C, BR=BR, BC=BC)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    assert torch.equal(out[:C], (x * 2.0).t())
+    assert torch.equal(out[C], torch.full((R,), -7.0, device=DEV))
+
+
 def test_softmax_rows_the_row_kernel_declines(K, oracle_cpu):
     import extra_kernels as X
     torch.manual_seed(5)

@@ -236,10 +236,7 @@ struct Gen {
       case SK::Load: {
         // a load that is not of the run's block shape (an index vector, a row of scales): from its copy in LDS when the
         // run staged one, else read where it is used (the program is then refused if anything stores to its base)
-        auto st = staged.find(v);
-        if (st != staged.end()) {
-          return st->second + "[" + linear(V.shape, i0, i1) + "]";
-        }
+        if (staged.count(v)) return staged_at(v, i0, i1);
         all_inline_bases.insert(s.acc.base_arg);
         std::string pred, addr = address(s.acc, i0, i1, pred);
         const std::string rd = mem_read(s.acc, addr);
@@ -506,7 +503,33 @@ struct Gen {
   // Values that a thread keeps for the elements it owns (element t + 256 n of the value's shape in slot n): the loads of
   // two-phase runs and loop-carried blocks.  They can be named only inside an element loop over the same shape;
   // elsewhere a load is read again in place and a carried block is refused.
-  std::map<int, std::string> staged;  // load of another shape than its run's -> LDS array holding the whole block
+  // A load that a run copied to LDS whole: loads of another shape than the run's, and loads read through a transpose
+  // (coalesced into LDS where they stand, read back in any order).  pitch: elements between rows of a rank-2 block (one
+  // more than its columns under a transpose, so that a column's elements fall into different banks).
+  struct Staged { std::string name; int64_t pitch; };
+  std::map<int, Staged> staged;
+  std::string staged_at(int v, const std::string &i0, const std::string &i1) {
+    const Staged &st = staged.at(v);
+    const auto &sh = val(v).shape;
+    if (sh.size() == 2 && st.pitch != sh.back()) return st.name + "[(" + i0 + " * " + std::to_string(st.pitch) + " + " + i1 + ")]";
+    return st.name + "[" + linear(sh, i0, i1) + "]";
+  }
+  // loads of ops[k, end) that some tt.trans of the run reads, directly or through elementwise ops
+  std::set<int> loads_behind_transposes(const std::vector<SOp> &ops, size_t k, size_t end) {
+    std::set<int> found;
+    std::function<void(int, int)> walk = [&](int v, int depth) {
+      auto d = def.find(v);
+      if (d == def.end() || depth > 16) return;
+      const SOp &o = *d->second;
+      if (o.kind == SK::Load) { found.insert(v); return; }
+      if (o.kind == SK::Map || o.kind == SK::Broadcast || o.kind == SK::ExpandDims)
+        for (int x : o.operands) walk(x, depth + 1);
+    };
+    for (size_t q = k; q < end; q++)
+      if (ops[q].kind == SK::Map && ops[q].name.rfind("tt.trans", 0) == 0 && val(ops[q].result).shape.size() == 2)
+        for (int x : ops[q].operands) walk(x, 0);
+    return found;
+  }
   struct Held { std::string name; std::vector<int64_t> shape; };
   std::map<int, Held> held;
   void map_vars(const std::vector<int64_t> &shape) {
@@ -698,24 +721,31 @@ struct Gen {
       // Loads of another shape are small blocks used through broadcasts (an index vector, a row of scales).  Read in
       // place they would sit in the address computation of the run's own loads, and every one of those would wait for
       // the one before it (loads complete in order): copy them to LDS first, at the place in the program where they stand.
+      // A load that the run reads through a transpose is copied as well, whatever its shape: read where the transposed
+      // element is used, a wavefront's addresses would be a row pitch apart (a [64, 64] fp32 tile transposed that way
+      // moved 2.1 TB/s).
+      const std::set<int> transposed = loads_behind_transposes(ops, k, end);
       for (size_t q = k; q < end; q++) {
         const SOp &o = ops[q];
-        if (o.kind != SK::Load || own(o) || big_other(o) || staged.count(o.result)) continue;
-        const size_t bytes = (size_t)count(o.acc.sizes) * held_bytes(val(o.result).dtype);
+        const bool behind_transpose = transposed.count(o.result) && o.acc.sizes.size() == 2;
+        if (o.kind != SK::Load || ((own(o) || big_other(o)) && !behind_transpose) || staged.count(o.result)) continue;
+        const int64_t pitch = behind_transpose ? o.acc.sizes.back() + 1 : (o.acc.sizes.empty() ? 1 : o.acc.sizes.back());
+        const int64_t elems = behind_transpose ? o.acc.sizes[0] * pitch : count(o.acc.sizes);
+        const size_t bytes = (size_t)elems * held_bytes(val(o.result).dtype);
         if (count(o.acc.sizes) > TWO_PHASE_MAX || pool_bytes + out_bytes + bytes > 48 * 1024) continue;
         const std::string name = "blk" + std::to_string(o.result);
-        decl << "  __shared__ " << ctype(val(o.result).dtype) << " " << name << "[" << count(o.acc.sizes) << "];\n";
+        decl << "  __shared__ " << ctype(val(o.result).dtype) << " " << name << "[" << elems << "];\n";
         out_bytes += (bytes + 15) / 16 * 16;
+        staged[o.result] = {name, pitch};
         open_element_loop(o.acc.sizes);
         {
           std::string pred, addr = address(o.acc, idx0(o.acc.sizes), idx1(o.acc.sizes), pred);
-          os << pad() << name << "[t] = "
+          os << pad() << staged_at(o.result, idx0(o.acc.sizes), idx1(o.acc.sizes)) << " = "
              << (pred.empty() ? mem_read(o.acc, addr) : "(" + pred + ") ? " + mem_read(o.acc, addr) + " : " + other_of(o.acc, idx0(o.acc.sizes), idx1(o.acc.sizes)))
              << ";\n";
         }
         close_loop();
         os << pad() << "__syncthreads();\n";
-        staged[o.result] = name;
       }
       if (two_phase) {
         // Registers for the run's own loads, and for large blocks of another shape (a [K, N] operand next to an [M, K]
@@ -725,7 +755,7 @@ struct Gen {
           if (big_other(ops[q]) && std::find(shapes.begin(), shapes.end(), ops[q].acc.sizes) == shapes.end()) shapes.push_back(ops[q].acc.sizes);
         bool any_load = false;
         for (const auto &ls : shapes) {
-          auto mine_here = [&](const SOp &o) { return o.kind == SK::Load && o.acc.sizes == ls && (own(o) || big_other(o)); };
+          auto mine_here = [&](const SOp &o) { return o.kind == SK::Load && o.acc.sizes == ls && (own(o) || big_other(o)) && !staged.count(o.result); };
           bool any = false;
           for (size_t q = k; q < end; q++)
             if (mine_here(ops[q])) {
@@ -804,7 +834,7 @@ struct Gen {
             cur_i1 = i1;
           }
           for (size_t q = k; q < end; q++)
-            if (own(ops[q])) {
+            if (own(ops[q]) && !staged.count(ops[q].result)) {
               std::string name = "v" + std::to_string(ops[q].result);
               emit_load(ops[q], "const " + ctype(val(ops[q].result).dtype) + " " + name);
               var[ops[q].result] = name;
