@@ -156,6 +156,30 @@ def test_layernorm_shapes(K, oracle_cpu, M, N, dtype):
     assert (mean - mr).abs().max().item() <= 1e-5 and ((rstd - rr) / rr).abs().max().item() <= 1e-5
 
 
+@pytest.mark.parametrize("M,N,kernel", [(4100, 8192, "layernorm_fwd_persistent_kernel"), (8200, 2048, "layernorm_fwd_persistent_kernel"), (300, 4096, "layernorm_fwd_kernel<4>"),
+                                       (7, 1001, "layernorm_fwd_kernel<1>"), (5, 8191, "layernorm_fwd_kernel<8>"), (3, 20000, "layernorm_fwd_long_kernel")])
+def test_layernorm_on_fp32_tensors(K, M, N, kernel):
+    # the same Triton source on fp32 x, y, w, b (no widening or narrowing casts in its TTIR) runs on the same kernels with
+    # 16-byte chunks of four elements; pinned by the float64 formula (biased variance) and torch's layer_norm
+    x, w, b = _ln_inputs(M, N, torch.float32, seed=N + 1)
+    xd, wd, bd = x.to(DEV), w.to(DEV), b.to(DEV)
+    yd = torch.full((M + 1, N), -3.0, device=DEV)
+    mean = torch.zeros(M, dtype=torch.float32, device=DEV)
+    rstd = torch.zeros(M, dtype=torch.float32, device=DEV)
+    k = K.layer_norm_fwd[(M,)](xd, yd, wd, bd, mean, rstd, xd.stride(0), N, 1e-5, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "layernorm_fwd" and k.function.last_kernel == kernel
+    xx = x.double()
+    m64 = xx.mean(1)
+    v64 = ((xx - m64[:, None]) ** 2).mean(1)
+    r64 = 1.0 / torch.sqrt(v64 + 1e-5)
+    y64 = (xx - m64[:, None]) * r64[:, None] * w.double() + b.double()
+    assert (yd[:M].cpu().double() - y64).abs().max().item() <= 1e-5
+    assert (mean.cpu().double() - m64).abs().max().item() <= 1e-6 and ((rstd.cpu().double() - r64) / r64).abs().max().item() <= 1e-5
+    assert torch.allclose(yd[:M].cpu(), torch.nn.functional.layer_norm(x, (N,), w, b, 1e-5), atol=1e-5)
+    assert torch.equal(yd[M].cpu(), torch.full((N,), -3.0))
+
+
 # ------------------------------------------------------------------ cfg4
 def _run_mm(K, a, b, BM=128, BN=128, BK=64):
     M, Kd = a.shape

@@ -76,7 +76,7 @@ struct SoftmaxParams {
 };
 hipError_t launch_softmax(const SoftmaxParams &p, int gx, int gy, int gz, hipStream_t s, const char **kernel_name);
 
-// LayerNorm forward over rows of N elements (fp16 or bf16 I/O, fp32 statistics)
+// LayerNorm forward over rows of N elements (fp16, bf16 or fp32 I/O, fp32 statistics)
 struct LayerNormParams {
   const void *x, *w, *b;
   void *y;
@@ -84,7 +84,7 @@ struct LayerNormParams {
   Affine x_off, y_off, w_off, b_off, mean_off, rstd_off;
   int64_t N;
   float eps;
-  int is_bf16;
+  int elem_kind;  // the element type of x, y, w and b: 0 fp16, 1 bf16, 2 fp32
 };
 hipError_t launch_layernorm(const LayerNormParams &p, int gx, int gy, int gz, hipStream_t s, const char **kernel_name);
 

@@ -284,46 +284,79 @@ __device__ __forceinline__ float block_sum_256(float v, float *red) {
   return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
+// The element type of x, y, w and b: 0 fp16, 1 bf16, 2 fp32.  A chunk is the 16 bytes a thread moves at once: EPC elements.
+template <int KIND>
+struct LnType {
+  using elem = uint16_t;
+  static constexpr int EPC = 8;
+  static __device__ __forceinline__ float up(uint16_t h) { return Half<KIND == 1>::up(h); }
+  static __device__ __forceinline__ uint16_t down(float f) { return Half<KIND == 1>::down(f); }
+  static __device__ __forceinline__ void unpack(const uint32_t (&q)[4], float (&v)[8]) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      v[2 * k] = up((uint16_t)(q[k] & 0xffff));
+      v[2 * k + 1] = up((uint16_t)(q[k] >> 16));
+    }
+  }
+  static __device__ __forceinline__ uint4 pack(const float (&y)[8]) {
+    uint32_t o[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) o[k] = (uint32_t)down(y[2 * k]) | ((uint32_t)down(y[2 * k + 1]) << 16);
+    return make_uint4(o[0], o[1], o[2], o[3]);
+  }
+};
+template <>
+struct LnType<2> {
+  using elem = float;
+  static constexpr int EPC = 4;
+  static __device__ __forceinline__ float up(float x) { return x; }
+  static __device__ __forceinline__ float down(float f) { return f; }
+  static __device__ __forceinline__ void unpack(const uint32_t (&q)[4], float (&v)[4]) {
+#pragma unroll
+    for (int k = 0; k < 4; k++) v[k] = __uint_as_float(q[k]);
+  }
+  static __device__ __forceinline__ uint4 pack(const float (&y)[4]) {
+    return make_uint4(__float_as_uint(y[0]), __float_as_uint(y[1]), __float_as_uint(y[2]), __float_as_uint(y[3]));
+  }
+};
+
 // One workgroup per row.  The row is read from HBM once and kept in registers
-// as fp32 (CPT chunks of 8 elements per thread); the Triton source's three
+// as fp32 (CPT chunks of EPC elements per thread); the Triton source's three
 // passes over the row all read these registers.
-// FAST: N is a multiple of 8 and every row of x, y, w, b starts 16-byte aligned, so a chunk is
+// FAST: N is a multiple of EPC and every row of x, y, w, b starts 16-byte aligned, so a chunk is
 // either whole or absent and all loads are unconditional (an absent chunk re-reads chunk 0 and is
 // zeroed), which lets the compiler keep the CPT loads of a thread in flight together.
-template <bool BF16, int CPT, bool FAST>
+template <int KIND, int CPT, bool FAST>
 __global__ __launch_bounds__(256, CPT <= 4 ? 8 : 4) void layernorm_fwd_kernel(LayerNormParams p) {
+  using T = LnType<KIND>;
+  using E = typename T::elem;
+  constexpr int EPC = T::EPC;
   __shared__ float red[4];
   const int px = blockIdx.x, py = blockIdx.y, pz = blockIdx.z;
-  const uint16_t *__restrict__ x = (const uint16_t *)p.x + affine(p.x_off, px, py, pz);
-  const uint16_t *__restrict__ w = (const uint16_t *)p.w + affine(p.w_off, px, py, pz);
-  const uint16_t *__restrict__ b = (const uint16_t *)p.b + affine(p.b_off, px, py, pz);
-  uint16_t *__restrict__ y = (uint16_t *)p.y + affine(p.y_off, px, py, pz);
+  const E *__restrict__ x = (const E *)p.x + affine(p.x_off, px, py, pz);
+  const E *__restrict__ w = (const E *)p.w + affine(p.w_off, px, py, pz);
+  const E *__restrict__ b = (const E *)p.b + affine(p.b_off, px, py, pz);
+  E *__restrict__ y = (E *)p.y + affine(p.y_off, px, py, pz);
   const int N = (int)p.N;
   const bool vec = (((uintptr_t)x | (uintptr_t)w | (uintptr_t)b | (uintptr_t)y) & 15) == 0;
-  float v[CPT][8];
+  float v[CPT][EPC];
 #pragma unroll
   for (int c = 0; c < CPT; c++) {
-    int i0 = (threadIdx.x + c * 256) * 8;
+    int i0 = (threadIdx.x + c * 256) * EPC;
     if (FAST) {
       const bool present = i0 < N;
       uint4 raw = *reinterpret_cast<const uint4 *>(x + (present ? i0 : 0));
-      uint32_t q[4] = {raw.x, raw.y, raw.z, raw.w};
+      const uint32_t q[4] = {raw.x, raw.y, raw.z, raw.w};
+      T::unpack(q, v[c]);
 #pragma unroll
-      for (int k = 0; k < 4; k++) {
-        v[c][2 * k] = present ? Half<BF16>::up((uint16_t)(q[k] & 0xffff)) : 0.f;
-        v[c][2 * k + 1] = present ? Half<BF16>::up((uint16_t)(q[k] >> 16)) : 0.f;
-      }
-    } else if (vec && i0 + 8 <= N) {
+      for (int k = 0; k < EPC; k++) v[c][k] = present ? v[c][k] : 0.f;
+    } else if (vec && i0 + EPC <= N) {
       uint4 raw = *reinterpret_cast<const uint4 *>(x + i0);
-      uint32_t q[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-      for (int k = 0; k < 4; k++) {
-        v[c][2 * k] = Half<BF16>::up((uint16_t)(q[k] & 0xffff));
-        v[c][2 * k + 1] = Half<BF16>::up((uint16_t)(q[k] >> 16));
-      }
+      const uint32_t q[4] = {raw.x, raw.y, raw.z, raw.w};
+      T::unpack(q, v[c]);
     } else {
 #pragma unroll
-      for (int k = 0; k < 8; k++) v[c][k] = i0 + k < N ? Half<BF16>::up(x[i0 + k]) : 0.f;  // other = 0
+      for (int k = 0; k < EPC; k++) v[c][k] = i0 + k < N ? T::up(x[i0 + k]) : 0.f;  // other = 0
     }
   }
   const float n_f = (float)N;  // arith.sitofp
@@ -331,14 +364,14 @@ __global__ __launch_bounds__(256, CPT <= 4 ? 8 : 4) void layernorm_fwd_kernel(La
 #pragma unroll
   for (int c = 0; c < CPT; c++)
 #pragma unroll
-    for (int k = 0; k < 8; k++) s += v[c][k];
+    for (int k = 0; k < EPC; k++) s += v[c][k];
   const float mean = block_sum_256(s, red) / n_f;
   float s2 = 0.f;
 #pragma unroll
   for (int c = 0; c < CPT; c++) {
-    int i0 = (threadIdx.x + c * 256) * 8;
+    int i0 = (threadIdx.x + c * 256) * EPC;
 #pragma unroll
-    for (int k = 0; k < 8; k++) {
+    for (int k = 0; k < EPC; k++) {
       float d = i0 + k < N ? v[c][k] - mean : 0.f;  // tl.where(cols < N, x - mean, 0)
       s2 += d * d;
     }
@@ -351,25 +384,21 @@ __global__ __launch_bounds__(256, CPT <= 4 ? 8 : 4) void layernorm_fwd_kernel(La
   }
 #pragma unroll
   for (int c = 0; c < CPT; c++) {
-    int i0 = (threadIdx.x + c * 256) * 8;
-    if (FAST ? i0 < N : (vec && i0 + 8 <= N)) {
+    int i0 = (threadIdx.x + c * 256) * EPC;
+    if (FAST ? i0 < N : (vec && i0 + EPC <= N)) {
       uint4 wr = *reinterpret_cast<const uint4 *>(w + i0);
       uint4 br = *reinterpret_cast<const uint4 *>(b + i0);
-      uint32_t wq[4] = {wr.x, wr.y, wr.z, wr.w}, bq[4] = {br.x, br.y, br.z, br.w}, o[4];
+      const uint32_t wq[4] = {wr.x, wr.y, wr.z, wr.w}, bq[4] = {br.x, br.y, br.z, br.w};
+      float wv[EPC], bv[EPC], o[EPC];
+      T::unpack(wq, wv);
+      T::unpack(bq, bv);
 #pragma unroll
-      for (int k = 0; k < 4; k++) {
-        float y0 = (v[c][2 * k] - mean) * rstd * Half<BF16>::up((uint16_t)(wq[k] & 0xffff)) +
-                   Half<BF16>::up((uint16_t)(bq[k] & 0xffff));
-        float y1 = (v[c][2 * k + 1] - mean) * rstd * Half<BF16>::up((uint16_t)(wq[k] >> 16)) +
-                   Half<BF16>::up((uint16_t)(bq[k] >> 16));
-        o[k] = (uint32_t)Half<BF16>::down(y0) | ((uint32_t)Half<BF16>::down(y1) << 16);
-      }
-      ntstore(reinterpret_cast<uint4 *>(y + i0), make_uint4(o[0], o[1], o[2], o[3]));
+      for (int k = 0; k < EPC; k++) o[k] = (v[c][k] - mean) * rstd * wv[k] + bv[k];
+      ntstore(reinterpret_cast<uint4 *>(y + i0), T::pack(o));
     } else {
 #pragma unroll
-      for (int k = 0; k < 8; k++)
-        if (i0 + k < N)
-          y[i0 + k] = Half<BF16>::down((v[c][k] - mean) * rstd * Half<BF16>::up(w[i0 + k]) + Half<BF16>::up(b[i0 + k]));
+      for (int k = 0; k < EPC; k++)
+        if (i0 + k < N) y[i0 + k] = T::down((v[c][k] - mean) * rstd * T::up(w[i0 + k]) + T::up(b[i0 + k]));
     }
   }
 }
@@ -382,30 +411,33 @@ __global__ __launch_bounds__(256, CPT <= 4 ? 8 : 4) void layernorm_fwd_kernel(La
 // kernel loses is the 32 KB of w and b that every row fetches again through L2: taking those loads out of it, and
 // nothing else, gives 23.8 us.  512 or 1024 threads per workgroup, a third row in flight and nontemporal row loads
 // gain nothing or lose.  [8192, 8192]: 51.7 -> 44.8 us (6.0 TB/s).
-// For one-dimensional grids, rows of exactly CPT * 2048 elements starting 16-byte aligned, w and b the same for every row.
-template <bool BF16, int CPT>
+// For one-dimensional grids, rows of exactly CPT * 256 chunks starting 16-byte aligned, w and b the same for every row.
+template <int KIND, int CPT>
 __global__ __launch_bounds__(256) void layernorm_fwd_persistent_kernel(LayerNormParams p, int rows) {
+  using T = LnType<KIND>;
+  using E = typename T::elem;
+  constexpr int EPC = T::EPC;
   __shared__ float red[2][2][4];  // [which reduction][row parity][wavefront]: one barrier per reduction
   const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
   const int N = (int)p.N;
-  const uint16_t *__restrict__ xb = (const uint16_t *)p.x + p.x_off.c0;
-  uint16_t *__restrict__ yb = (uint16_t *)p.y + p.y_off.c0;
-  const uint16_t *__restrict__ w = (const uint16_t *)p.w + p.w_off.c0;
-  const uint16_t *__restrict__ b = (const uint16_t *)p.b + p.b_off.c0;
+  const E *__restrict__ xb = (const E *)p.x + p.x_off.c0;
+  E *__restrict__ yb = (E *)p.y + p.y_off.c0;
+  const E *__restrict__ w = (const E *)p.w + p.w_off.c0;
+  const E *__restrict__ b = (const E *)p.b + p.b_off.c0;
   uint4 wq[CPT], bq[CPT];
 #pragma unroll
   for (int c = 0; c < CPT; c++) {
-    wq[c] = *reinterpret_cast<const uint4 *>(w + (tid + c * 256) * 8);
-    bq[c] = *reinterpret_cast<const uint4 *>(b + (tid + c * 256) * 8);
+    wq[c] = *reinterpret_cast<const uint4 *>(w + (tid + c * 256) * EPC);
+    bq[c] = *reinterpret_cast<const uint4 *>(b + (tid + c * 256) * EPC);
   }
   // A row's loads are issued from inline assembly and waited for by hand (row_landed): left to the compiler, the wait
   // for a row also waits for the next row's loads, issued just before (it does not count memory operations across the
   // loop's back edge), and the rows do not overlap.
   auto load_row = [&](u32x4_t (&q)[CPT], int r) {
-    const uint16_t *x = xb + (int64_t)r * p.x_off.c[0];
+    const E *x = xb + (int64_t)r * p.x_off.c[0];
 #pragma unroll
     for (int c = 0; c < CPT; c++) {
-      const uint16_t *src = x + (tid + c * 256) * 8;
+      const E *src = x + (tid + c * 256) * EPC;
       asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(q[c]) : "v"(src) : "memory");
     }
   };
@@ -417,6 +449,7 @@ __global__ __launch_bounds__(256) void layernorm_fwd_persistent_kernel(LayerNorm
       case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
       case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
       case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+      case 16: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
       default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
     }
 #pragma unroll
@@ -430,44 +463,40 @@ __global__ __launch_bounds__(256) void layernorm_fwd_persistent_kernel(LayerNorm
   };
   const float n_f = (float)N;  // arith.sitofp
   auto process = [&](const u32x4_t (&raw)[CPT], int r, int parity) {
-    float v[CPT][8];
+    float v[CPT][EPC];
 #pragma unroll
-    for (int c = 0; c < CPT; c++)
-#pragma unroll
-      for (int k = 0; k < 4; k++) {
-        v[c][2 * k] = Half<BF16>::up((uint16_t)(raw[c][k] & 0xffff));
-        v[c][2 * k + 1] = Half<BF16>::up((uint16_t)(raw[c][k] >> 16));
-      }
+    for (int c = 0; c < CPT; c++) {
+      const uint32_t q[4] = {raw[c][0], raw[c][1], raw[c][2], raw[c][3]};
+      T::unpack(q, v[c]);
+    }
     float s = 0.f;
 #pragma unroll
     for (int c = 0; c < CPT; c++)
 #pragma unroll
-      for (int k = 0; k < 8; k++) s += v[c][k];
+      for (int k = 0; k < EPC; k++) s += v[c][k];
     const float mean = block_sum(s, 0, parity) / n_f;
     float s2 = 0.f;
 #pragma unroll
     for (int c = 0; c < CPT; c++)
 #pragma unroll
-      for (int k = 0; k < 8; k++) {
+      for (int k = 0; k < EPC; k++) {
         const float d = v[c][k] - mean;
         s2 += d * d;
       }
     const float var = block_sum(s2, 1, parity) / n_f;
     const float rstd = 1.0f / sqrtf(var + p.eps);
-    uint16_t *y = yb + (int64_t)r * p.y_off.c[0];
+    E *y = yb + (int64_t)r * p.y_off.c[0];
 #pragma unroll
     for (int c = 0; c < CPT; c++) {
       // (the optimiser widens w and b to fp32 once, outside the row loop: 16 registers per chunk, which a workgroup
       // that has a CU's register file nearly to itself can afford, and four operations per element and row saved)
-      const uint32_t wv[4] = {wq[c].x, wq[c].y, wq[c].z, wq[c].w}, bv[4] = {bq[c].x, bq[c].y, bq[c].z, bq[c].w};
-      uint32_t o[4];
+      const uint32_t wr[4] = {wq[c].x, wq[c].y, wq[c].z, wq[c].w}, br[4] = {bq[c].x, bq[c].y, bq[c].z, bq[c].w};
+      float wv[EPC], bv[EPC], o[EPC];
+      T::unpack(wr, wv);
+      T::unpack(br, bv);
 #pragma unroll
-      for (int k = 0; k < 4; k++) {
-        const float y0 = (v[c][2 * k] - mean) * rstd * Half<BF16>::up((uint16_t)(wv[k] & 0xffff)) + Half<BF16>::up((uint16_t)(bv[k] & 0xffff));
-        const float y1 = (v[c][2 * k + 1] - mean) * rstd * Half<BF16>::up((uint16_t)(wv[k] >> 16)) + Half<BF16>::up((uint16_t)(bv[k] >> 16));
-        o[k] = (uint32_t)Half<BF16>::down(y0) | ((uint32_t)Half<BF16>::down(y1) << 16);
-      }
-      ntstore(reinterpret_cast<uint4 *>(y + (tid + c * 256) * 8), make_uint4(o[0], o[1], o[2], o[3]));
+      for (int k = 0; k < EPC; k++) o[k] = (v[c][k] - mean) * rstd * wv[k] + bv[k];
+      ntstore(reinterpret_cast<uint4 *>(y + (tid + c * 256) * EPC), T::pack(o));
     }
     if (tid == 0) {
       p.mean[p.mean_off.c0 + (int64_t)r * p.mean_off.c[0]] = mean;
@@ -504,22 +533,24 @@ __global__ __launch_bounds__(256) void layernorm_fwd_persistent_kernel(LayerNorm
 
 // Rows too long for the register file: three passes over global memory, the
 // second and third served by L2.
-template <bool BF16>
+template <int KIND>
 __global__ __launch_bounds__(256) void layernorm_fwd_long_kernel(LayerNormParams p) {
+  using T = LnType<KIND>;
+  using E = typename T::elem;
   __shared__ float red[4];
   const int px = blockIdx.x, py = blockIdx.y, pz = blockIdx.z;
-  const uint16_t *__restrict__ x = (const uint16_t *)p.x + affine(p.x_off, px, py, pz);
-  const uint16_t *__restrict__ w = (const uint16_t *)p.w + affine(p.w_off, px, py, pz);
-  const uint16_t *__restrict__ b = (const uint16_t *)p.b + affine(p.b_off, px, py, pz);
-  uint16_t *__restrict__ y = (uint16_t *)p.y + affine(p.y_off, px, py, pz);
+  const E *__restrict__ x = (const E *)p.x + affine(p.x_off, px, py, pz);
+  const E *__restrict__ w = (const E *)p.w + affine(p.w_off, px, py, pz);
+  const E *__restrict__ b = (const E *)p.b + affine(p.b_off, px, py, pz);
+  E *__restrict__ y = (E *)p.y + affine(p.y_off, px, py, pz);
   const int64_t N = p.N;
   const float n_f = (float)(int)N;
   float s = 0.f;
-  for (int64_t i = threadIdx.x; i < N; i += 256) s += Half<BF16>::up(x[i]);
+  for (int64_t i = threadIdx.x; i < N; i += 256) s += T::up(x[i]);
   const float mean = block_sum_256(s, red) / n_f;
   float s2 = 0.f;
   for (int64_t i = threadIdx.x; i < N; i += 256) {
-    float d = Half<BF16>::up(x[i]) - mean;
+    float d = T::up(x[i]) - mean;
     s2 += d * d;
   }
   const float var = block_sum_256(s2, red) / n_f;
@@ -529,29 +560,30 @@ __global__ __launch_bounds__(256) void layernorm_fwd_long_kernel(LayerNormParams
     p.rstd[affine(p.rstd_off, px, py, pz)] = rstd;
   }
   for (int64_t i = threadIdx.x; i < N; i += 256)
-    y[i] = Half<BF16>::down((Half<BF16>::up(x[i]) - mean) * rstd * Half<BF16>::up(w[i]) + Half<BF16>::up(b[i]));
+    y[i] = T::down((T::up(x[i]) - mean) * rstd * T::up(w[i]) + T::up(b[i]));
 }
 
-template <bool BF16>
+template <int KIND>
 hipError_t launch_layernorm_t(const LayerNormParams &p, dim3 grid, hipStream_t s, const char **name) {
-  int64_t chunks = (p.N + 7) / 8;
-  auto aligned = [](const Affine &a) { return (a.c0 | a.c[0] | a.c[1] | a.c[2]) % 8 == 0; };
-  const bool fast = p.N % 8 == 0 && aligned(p.x_off) && aligned(p.y_off) && aligned(p.w_off) && aligned(p.b_off) &&
+  constexpr int EPC = LnType<KIND>::EPC;
+  int64_t chunks = (p.N + EPC - 1) / EPC;
+  auto aligned = [](const Affine &a) { return (a.c0 | a.c[0] | a.c[1] | a.c[2]) % EPC == 0; };
+  const bool fast = p.N % EPC == 0 && aligned(p.x_off) && aligned(p.y_off) && aligned(p.w_off) && aligned(p.b_off) &&
                     (((uintptr_t)p.x | (uintptr_t)p.y | (uintptr_t)p.w | (uintptr_t)p.b) & 15) == 0;
-  // Rows walked by persistent workgroups (see layernorm_fwd_persistent_kernel): whole rows of 2048, 4096 or 8192
-  // elements in one-dimensional grids with enough rows to amortise the walk (fewer, and the workgroup-per-row kernel
+  // Rows walked by persistent workgroups (see layernorm_fwd_persistent_kernel): whole rows of 256, 512, 1024 or (fp32)
+  // 2048 chunks in one-dimensional grids with enough rows to amortise the walk (fewer, and the workgroup-per-row kernel
   // measured faster), w and b the same for every row.  About 32 KB of row loads in flight per CU: one workgroup per CU
-  // for rows of 8192 elements, four for 4096, eight for 2048 (measured best of 1, 2, 4 and 8 per CU on [8192, 4096] and
-  // [16384, 2048]: 25.5 us against 26.3 and 26.5 us against 31.1 for a workgroup per row).
+  // for rows of 16 KB and more, four for 8 KB, eight for 4 KB (measured best of 1, 2, 4 and 8 per CU on fp16 [8192, 4096]
+  // and [16384, 2048]: 25.5 us against 26.3 and 26.5 us against 31.1 for a workgroup per row).
   static const char *ln_env = getenv("TTS_LN");  // tuning aid: "0" = always one workgroup per row; "G" = G persistent workgroups
   static const int cus = [] {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
     return n;
   }();
-  const int cpt = chunks == 256 ? 1 : chunks == 512 ? 2 : chunks == 1024 ? 4 : 0;
+  const int cpt = chunks == 256 ? 1 : chunks == 512 ? 2 : chunks == 1024 ? 4 : (chunks == 2048 && KIND == 2) ? 8 : 0;
   int persistent_grid = cus * (cpt == 1 ? 8 : cpt == 2 ? 4 : 1);
-  int64_t min_rows = (int64_t)persistent_grid * (cpt == 4 ? 16 : 8);
+  int64_t min_rows = (int64_t)persistent_grid * (cpt >= 4 ? 16 : 8);
   if (ln_env) {
     persistent_grid = atoi(ln_env);
     min_rows = 2 * (int64_t)persistent_grid;
@@ -561,23 +593,24 @@ hipError_t launch_layernorm_t(const LayerNormParams &p, dim3 grid, hipStream_t s
       row_invariant(p.b_off)) {
     const int rows = (int)grid.x;
     const dim3 pg((unsigned)persistent_grid);
-    if (cpt == 1) hipLaunchKernelGGL((layernorm_fwd_persistent_kernel<BF16, 1>), pg, dim3(256), 0, s, p, rows);
-    else if (cpt == 2) hipLaunchKernelGGL((layernorm_fwd_persistent_kernel<BF16, 2>), pg, dim3(256), 0, s, p, rows);
-    else hipLaunchKernelGGL((layernorm_fwd_persistent_kernel<BF16, 4>), pg, dim3(256), 0, s, p, rows);
+    if (cpt == 1) hipLaunchKernelGGL((layernorm_fwd_persistent_kernel<KIND, 1>), pg, dim3(256), 0, s, p, rows);
+    else if (cpt == 2) hipLaunchKernelGGL((layernorm_fwd_persistent_kernel<KIND, 2>), pg, dim3(256), 0, s, p, rows);
+    else if (cpt == 4) hipLaunchKernelGGL((layernorm_fwd_persistent_kernel<KIND, 4>), pg, dim3(256), 0, s, p, rows);
+    else if constexpr (KIND == 2) hipLaunchKernelGGL((layernorm_fwd_persistent_kernel<KIND, 8>), pg, dim3(256), 0, s, p, rows);
     *name = "layernorm_fwd_persistent_kernel";
     return hipGetLastError();
   }
 #define TTS_LN(CPT)                                                                                          \
   do {                                                                                                       \
-    if (fast) hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, CPT, true>), grid, dim3(256), 0, s, p);        \
-    else hipLaunchKernelGGL((layernorm_fwd_kernel<BF16, CPT, false>), grid, dim3(256), 0, s, p);            \
+    if (fast) hipLaunchKernelGGL((layernorm_fwd_kernel<KIND, CPT, true>), grid, dim3(256), 0, s, p);        \
+    else hipLaunchKernelGGL((layernorm_fwd_kernel<KIND, CPT, false>), grid, dim3(256), 0, s, p);            \
     *name = "layernorm_fwd_kernel<" #CPT ">";                                                                \
   } while (0)
   if (chunks <= 256) TTS_LN(1);
   else if (chunks <= 512) TTS_LN(2);
   else if (chunks <= 1024) TTS_LN(4);
   else if (chunks <= 2048) TTS_LN(8);
-  else { hipLaunchKernelGGL((layernorm_fwd_long_kernel<BF16>), grid, dim3(256), 0, s, p); *name = "layernorm_fwd_long_kernel"; }
+  else { hipLaunchKernelGGL((layernorm_fwd_long_kernel<KIND>), grid, dim3(256), 0, s, p); *name = "layernorm_fwd_long_kernel"; }
 #undef TTS_LN
   return hipGetLastError();
 }
@@ -850,7 +883,7 @@ hipError_t launch_softmax(const SoftmaxParams &p, int gx, int gy, int gz, hipStr
 
 hipError_t launch_layernorm(const LayerNormParams &p, int gx, int gy, int gz, hipStream_t s, const char **name) {
   dim3 grid(gx, gy, gz);
-  return p.is_bf16 ? launch_layernorm_t<true>(p, grid, s, name) : launch_layernorm_t<false>(p, grid, s, name);
+  return p.elem_kind == 2 ? launch_layernorm_t<2>(p, grid, s, name) : p.elem_kind == 1 ? launch_layernorm_t<1>(p, grid, s, name) : launch_layernorm_t<0>(p, grid, s, name);
 }
 
 }  // namespace tts

@@ -383,8 +383,20 @@ const char *SIG_LAYERNORM =
     "h.mulf:f32(v39,v40);v42=arith.extf:f32(v35);v43=arith.addf:f32(v41,v42);v44=arith.truncf:{T}(v43);st"
     "ore:{T}.r1.m(v44);yield()};";
 
+// the same program on fp32 tensors: no widening or narrowing casts
+const char *SIG_LAYERNORM_F32 =
+    "v0=const:f32;v1=const:f32;v2=iota;v3=index;v4=splat(v3);for[v5<-v1]{v6=load:f32.r1.m.o;v7=arith.addf:f32(v5,v6);yield(v7)}->v8;"
+    "v9=reduce.arith.addf.0(v8);v10=index;v11=arith.sitofp:f32(v10);v12=arith.divf:f32(v9,v11);v13=splat(v12);for[v14<-v1]{v15=index;"
+    "v16=splat(v15);v17=arith.addi:i32(v16,v2);v18=arith.cmpi.slt:i1(v17,v4);v19=load:f32.r1.m.o;v20=arith.subf:f32(v19,v13);"
+    "v21=arith.select:f32(v18,v20,v1);v22=arith.mulf:f32(v21,v21);v23=arith.addf:f32(v14,v22);yield(v23)}->v24;"
+    "v25=reduce.arith.addf.0(v24);v26=arith.divf:f32(v25,v11);v27=farg;v28=arith.addf:f32(v26,v27);v29=math.sqrt:f32(v28);"
+    "v30=arith.divf:f32(v0,v29);sstore:f32.r0(v12);sstore:f32.r0(v30);v31=splat(v30);for[]{v32=load:f32.r1.m;v33=load:f32.r1.m;"
+    "v34=load:f32.r1.m.o;v35=arith.subf:f32(v34,v13);v36=arith.mulf:f32(v35,v31);v37=arith.mulf:f32(v36,v32);v38=arith.addf:f32(v37,v33);"
+    "store:f32.r1.m(v38);yield()};";
+
 bool try_layernorm(Plan &pl) {
-  if (pl.signature != subst(SIG_LAYERNORM, "{T}", "f16") && pl.signature != subst(SIG_LAYERNORM, "{T}", "bf16")) return false;
+  if (pl.signature != subst(SIG_LAYERNORM, "{T}", "f16") && pl.signature != subst(SIG_LAYERNORM, "{T}", "bf16") && pl.signature != SIG_LAYERNORM_F32)
+    return false;
   const char *F = "layernorm_fwd";
   Matcher m(pl.prog);
   if (m.loops.size() != 3 || m.accesses.size() != 8) return false;
@@ -452,7 +464,9 @@ bool try_layernorm(Plan &pl) {
   pl.k["mean_arg"] = mean_st->acc.base_arg;
   pl.k["rstd_arg"] = rstd_st->acc.base_arg;
   pl.k["eps_arg"] = m.of_kind(SK::ScalarArg).at(0)->ival;
-  pl.k["half_is_bf16"] = x0->acc.elem == "bf16";
+  pl.k["elem_kind"] = x0->acc.elem == "f32" ? 2 : x0->acc.elem == "bf16" ? 1 : 0;
+  for (SOp *a : {x1, x2, w, b, y})
+    if (a->acc.elem != x0->acc.elem) refuse(F, "its tensors differ in element type");
   pl.e["N"] = N;
   return true;
 }

@@ -264,10 +264,10 @@ void bind_layernorm(const Resolver &r, Bound &b) {
   p.rstd_off = r.affine("rstd_off");
   p.N = r.ev0("N");
   p.eps = (float)r.floats.at(r.pl.k.at("eps_arg"));
-  p.is_bf16 = (int)r.pl.k.at("half_is_bf16");
+  p.elem_kind = (int)r.pl.k.at("elem_kind");
   if (p.N > INT32_MAX) throw Invalid("layernorm_fwd: N does not fit 32 bits");
   std::ostringstream os;
-  os << "kernel=layernorm_fwd\nN=" << p.N << "\neps=" << p.eps << "\nbf16=" << p.is_bf16 << "\nx_off=" << show(p.x_off)
+  os << "kernel=layernorm_fwd\nN=" << p.N << "\neps=" << p.eps << "\nelem=" << (p.elem_kind == 2 ? "f32" : p.elem_kind == 1 ? "bf16" : "f16") << "\nx_off=" << show(p.x_off)
      << "\ny_off=" << show(p.y_off) << "\nw_off=" << show(p.w_off) << "\nb_off=" << show(p.b_off)
      << "\nmean_off=" << show(p.mean_off) << "\nrstd_off=" << show(p.rstd_off) << "\n";
   b.describe = os.str();
