@@ -551,6 +551,26 @@ def test_tiled_transpose_goes_through_lds(R, C, BR, BC):
     assert torch.equal(out[C], torch.full((R,), -7.0, device=DEV))
 
 
+@pytest.mark.parametrize("rows,cols,pitch,block,dtype", [(64, 4096, 4096, 4096, torch.float16), (33, 781, 781, 1024, torch.float16), (5, 40000, 40000, 65536, torch.bfloat16),
+                                                        (40, 784, 790, 1024, torch.bfloat16), (300, 1024, 1024, 1024, torch.float16), (7, 8, 8, 64, torch.float16)])
+def test_row_softmax_on_16_bit_rows(K, rows, cols, pitch, block, dtype):
+    # the same source on fp16 / bf16 tensors (widened after the load, narrowed before the store; the arithmetic is the fp32
+    # kernel's): whole 16-byte chunks where rows are multiples of 8 elements and 16-byte aligned, element by element elsewhere
+    torch.manual_seed(rows + cols)
+    x = torch.randn(rows, pitch).to(dtype)[:, :cols]
+    xd = x.to(DEV)
+    full = torch.full((rows + 1, pitch), -9.0, dtype=dtype, device=DEV)
+    od = full[:, :cols]
+    k = K.row_softmax[(rows,)](od, xd, xd.stride(0), od.stride(0), cols, BLOCK=block)
+    torch.cuda.synchronize()
+    assert k.function.family == "row_softmax"
+    want = torch.softmax(x.float(), 1)
+    ulp = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+    assert (od[:rows].cpu().float() - want).abs().max().item() <= ulp        # results lie in [0, 1]: one rounding to 16 bits
+    assert (od[:rows].cpu() != want.to(dtype)).float().mean().item() < 0.01   # and nearly all are the correctly rounded value
+    assert torch.equal(full[rows].cpu(), torch.full((pitch,), -9.0, dtype=dtype)) and torch.equal(full[:, cols:].cpu(), torch.full((rows + 1, pitch - cols), -9.0, dtype=dtype))
+
+
 def test_softmax_rows_the_row_kernel_declines(K, oracle_cpu):
     import extra_kernels as X
     torch.manual_seed(5)

@@ -66,13 +66,14 @@ std::string fused_map_source(const MapNParams &p);
 
 // out[off_out(p)+i] = softmax(row)[i], i < d_out, where row[i] = i < d_in ? in[off_in(p)+i] : other, i < block
 struct SoftmaxParams {
-  const float *in;
-  float *out;
+  const void *in;
+  void *out;
   Affine in_off, out_off;
   int64_t d_in, d_out;
   int block;
   float other;
   int propagate_nan;  // the max reduction is arith.maximumf rather than arith.maxnumf
+  int elem_kind;      // the element type of in and out: 0 fp16, 1 bf16, 2 fp32 (the arithmetic is fp32 either way)
 };
 hipError_t launch_softmax(const SoftmaxParams &p, int gx, int gy, int gz, hipStream_t s, const char **kernel_name);
 

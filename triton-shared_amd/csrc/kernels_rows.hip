@@ -124,131 +124,7 @@ hipError_t launch_map1d_op(const Map1DParams &p, dim3 grid, hipStream_t s) {
   return hipGetLastError();
 }
 
-// ---------------------------------------------------------------- softmax
-// T threads share one row; thread t holds elements t, t+T, ... (NPL of them).
-// VEC (block == NPL * T, NPL % 4 == 0, d_in >= 4): thread t holds the four-element chunks t, t+T, ...
-// instead and moves each with one 16-byte access.  Rows need no 16-byte alignment for that (global
-// accesses of several dwords only need dword alignment).  Every load is unconditional: a chunk that
-// sticks out of the row is read from the row's last four elements and shifted into place.
-typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
-
-template <int NPL, int WAVES, bool NAN_PROP, bool VEC, int WG = 256>
-__global__ __launch_bounds__(WG) void softmax_f32_kernel(SoftmaxParams p, int gx, int gy, int64_t programs) {
-  static_assert(WAVES == 1 || WG == WAVES * WAVE, "rows that span wavefronts meet in red[], one row per workgroup");
-  constexpr int T = WAVES * WAVE;
-  constexpr int ROWS_PER_WG = WG / T;
-  __shared__ float red[WAVES];
-  const int sub = threadIdx.x / T, t = threadIdx.x % T;
-  const int64_t prog = (int64_t)blockIdx.x * ROWS_PER_WG + sub;
-  const bool active = prog < programs;
-  int px = 0, py = 0, pz = 0;
-  if (active) {
-    if (gy == 1 && programs == gx) px = (int)prog;  // 1-D grid: no divisions
-    else { px = (int)(prog % gx); py = (int)((prog / gx) % gy); pz = (int)(prog / ((int64_t)gx * gy)); }
-  }
-  const float *__restrict__ in = p.in + affine(p.in_off, px, py, pz);
-  float *__restrict__ out = p.out + affine(p.out_off, px, py, pz);
-  const int d_in = active ? (int)p.d_in : 0, d_out = active ? (int)p.d_out : 0;
-  // lanes beyond d_in hold `other` and take part in the reductions, as a filled
-  // tile does; lanes beyond the block do not exist
-  float v[NPL];
-  if constexpr (VEC) {
-    const int last = max(d_in - 4, 0);  // inactive rows (d_in == 0) read the first row's start and store nothing
-    f32x4_a4 win[NPL / 4];
-#pragma unroll
-    for (int j = 0; j < NPL / 4; j++) win[j] = *reinterpret_cast<const f32x4_a4 *>(in + min(4 * (t + j * T), last));
-#pragma unroll
-    for (int j = 0; j < NPL / 4; j++) {
-      const int i0 = 4 * (t + j * T);
-      const int shift = i0 - min(i0, last);  // chunk element c is window[c + shift]
-      const f32x4_a4 w = win[j];
-#pragma unroll
-      for (int c = 0; c < 4; c++) {
-        float x = p.other;
-        if (shift == 0) x = w[c];
-#pragma unroll
-        for (int sft = 1; sft < 4; sft++)
-          if (c + sft < 4 && shift == sft) x = w[c + sft];
-        v[4 * j + c] = i0 + c < d_in ? x : p.other;
-      }
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < NPL; j++) {
-      int i = t + j * T;
-      v[j] = i < d_in ? in[i] : p.other;
-    }
-  }
-  float m = -INFINITY;
-#pragma unroll
-  for (int j = 0; j < NPL; j++)
-    if (VEC || t + j * T < p.block) m = fmax_sel<NAN_PROP>(m, v[j]);
-  m = wave_max<NAN_PROP>(m);
-  if (WAVES > 1) {
-    if (t % WAVE == 0) red[t / WAVE] = m;
-    __syncthreads();
-    m = red[0];
-#pragma unroll
-    for (int w = 1; w < WAVES; w++) m = fmax_sel<NAN_PROP>(m, red[w]);
-    __syncthreads();
-  }
-  float sum = 0.f;
-#pragma unroll
-  for (int j = 0; j < NPL; j++) {
-    // exp through the hardware exp2 (1 ulp) of a product rounded once: relative error below 1e-5
-    // even at the smallest normal result; a row of 781 elements costs 40 instructions per lane
-    // this way against some 300 through libm's expf, which made the kernel ALU-bound
-    v[j] = __builtin_amdgcn_exp2f((v[j] - m) * 1.44269504088896341f);
-    if (VEC || t + j * T < p.block) sum += v[j];
-  }
-  sum = wave_sum(sum);
-  if (WAVES > 1) {
-    if (t % WAVE == 0) red[t / WAVE] = sum;
-    __syncthreads();
-    sum = red[0];
-#pragma unroll
-    for (int w = 1; w < WAVES; w++) sum += red[w];
-  }
-  const float rsum = 1.0f / sum;  // one division per lane; the products are within 1.5 ulp of the quotients
-  if constexpr (VEC) {
-#pragma unroll
-    for (int j = 0; j < NPL / 4; j++) {
-      const int i0 = 4 * (t + j * T);
-      f32x4_a4 w;
-#pragma unroll
-      for (int c = 0; c < 4; c++) w[c] = v[4 * j + c] * rsum;
-      if (i0 + 4 <= d_out) __builtin_nontemporal_store(w, reinterpret_cast<f32x4_a4 *>(out + i0));
-      else
-#pragma unroll
-        for (int c = 0; c < 4; c++)
-          if (i0 + c < d_out) out[i0 + c] = w[c];
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < NPL; j++) {
-      int i = t + j * T;
-      if (i < d_out) out[i] = v[j] * rsum;
-    }
-  }
-}
-
-template <int NPL, int WAVES, int WG = 256>
-hipError_t launch_softmax_cfg(const SoftmaxParams &p, int gx, int gy, int gz, hipStream_t s) {
-  int64_t programs = (int64_t)gx * gy * gz;
-  int rows_per_wg = WG / (WAVES * WAVE);
-  dim3 grid((unsigned)((programs + rows_per_wg - 1) / rows_per_wg));
-  constexpr bool CAN_VEC = NPL % 4 == 0;
-  if (CAN_VEC && p.block == NPL * WAVES * WAVE && p.d_in >= 4) {
-    if (p.propagate_nan) hipLaunchKernelGGL((softmax_f32_kernel<NPL, WAVES, true, CAN_VEC, WG>), grid, dim3(WG), 0, s, p, gx, gy, programs);
-    else hipLaunchKernelGGL((softmax_f32_kernel<NPL, WAVES, false, CAN_VEC, WG>), grid, dim3(WG), 0, s, p, gx, gy, programs);
-    return hipGetLastError();
-  }
-  if (p.propagate_nan) hipLaunchKernelGGL((softmax_f32_kernel<NPL, WAVES, true, false, WG>), grid, dim3(WG), 0, s, p, gx, gy, programs);
-  else hipLaunchKernelGGL((softmax_f32_kernel<NPL, WAVES, false, false, WG>), grid, dim3(WG), 0, s, p, gx, gy, programs);
-  return hipGetLastError();
-}
-
-// -------------------------------------------------------------- layernorm
+// fp16 / bf16 <-> fp32 (narrowing rounds to nearest even, as arith.truncf)
 template <bool BF16>
 struct Half;
 template <>
@@ -284,6 +160,180 @@ __device__ __forceinline__ float block_sum_256(float v, float *red) {
   return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
+// ---------------------------------------------------------------- softmax
+// T threads share one row; thread t holds elements t, t+T, ... (NPL of them).
+// VEC (block == NPL * T, NPL % 4 == 0, d_in >= 4): thread t holds the four-element chunks t, t+T, ...
+// instead and moves each with one 16-byte access.  Rows need no 16-byte alignment for that (global
+// accesses of several dwords only need dword alignment).  Every load is unconditional: a chunk that
+// sticks out of the row is read from the row's last four elements and shifted into place.
+typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+// IO: the element type of the rows in memory (0 fp16, 1 bf16, 2 fp32); a 16-bit row is widened after the load and narrowed
+// before the store, as its Triton source does, and its VEC path moves whole 16-byte chunks of eight elements (the
+// launcher picks it for rows that are multiples of 8 elements long and start 16-byte aligned).
+template <int NPL, int WAVES, bool NAN_PROP, bool VEC, int WG = 256, int IO = 2>
+__global__ __launch_bounds__(WG) void softmax_f32_kernel(SoftmaxParams p, int gx, int gy, int64_t programs) {
+  using E = typename std::conditional<IO == 2, float, uint16_t>::type;
+  auto up = [](E e) -> float {
+    if constexpr (IO == 2) return e;
+    else return Half<IO == 1>::up(e);
+  };
+  auto down = [](float f) -> E {
+    if constexpr (IO == 2) return f;
+    else return Half<IO == 1>::down(f);
+  };
+  static_assert(WAVES == 1 || WG == WAVES * WAVE, "rows that span wavefronts meet in red[], one row per workgroup");
+  constexpr int T = WAVES * WAVE;
+  constexpr int ROWS_PER_WG = WG / T;
+  __shared__ float red[WAVES];
+  const int sub = threadIdx.x / T, t = threadIdx.x % T;
+  const int64_t prog = (int64_t)blockIdx.x * ROWS_PER_WG + sub;
+  const bool active = prog < programs;
+  int px = 0, py = 0, pz = 0;
+  if (active) {
+    if (gy == 1 && programs == gx) px = (int)prog;  // 1-D grid: no divisions
+    else { px = (int)(prog % gx); py = (int)((prog / gx) % gy); pz = (int)(prog / ((int64_t)gx * gy)); }
+  }
+  const E *__restrict__ in = (const E *)p.in + affine(p.in_off, px, py, pz);
+  E *__restrict__ out = (E *)p.out + affine(p.out_off, px, py, pz);
+  const int d_in = active ? (int)p.d_in : 0, d_out = active ? (int)p.d_out : 0;
+  // lanes beyond d_in hold `other` and take part in the reductions, as a filled
+  // tile does; lanes beyond the block do not exist
+  float v[NPL];
+  if constexpr (VEC && IO != 2) {
+    // thread t holds the eight-element chunks t, t+T, ...; a chunk is whole or absent (an absent one reads the row's start)
+#pragma unroll
+    for (int j = 0; j < NPL / 8; j++) {
+      const int i0 = 8 * (t + j * T);
+      const bool present = i0 < d_in;
+      const uint4 raw = *reinterpret_cast<const uint4 *>(in + (present ? i0 : 0));
+      const uint32_t q[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        v[8 * j + 2 * k] = present ? up((uint16_t)(q[k] & 0xffff)) : p.other;
+        v[8 * j + 2 * k + 1] = present ? up((uint16_t)(q[k] >> 16)) : p.other;
+      }
+    }
+  } else if constexpr (VEC) {
+    const int last = max(d_in - 4, 0);  // inactive rows (d_in == 0) read the first row's start and store nothing
+    f32x4_a4 win[NPL / 4];
+#pragma unroll
+    for (int j = 0; j < NPL / 4; j++) win[j] = *reinterpret_cast<const f32x4_a4 *>(in + min(4 * (t + j * T), last));
+#pragma unroll
+    for (int j = 0; j < NPL / 4; j++) {
+      const int i0 = 4 * (t + j * T);
+      const int shift = i0 - min(i0, last);  // chunk element c is window[c + shift]
+      const f32x4_a4 w = win[j];
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        float x = p.other;
+        if (shift == 0) x = w[c];
+#pragma unroll
+        for (int sft = 1; sft < 4; sft++)
+          if (c + sft < 4 && shift == sft) x = w[c + sft];
+        v[4 * j + c] = i0 + c < d_in ? x : p.other;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < NPL; j++) {
+      int i = t + j * T;
+      v[j] = i < d_in ? up(in[i]) : p.other;
+    }
+  }
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < NPL; j++)
+    if (VEC || t + j * T < p.block) m = fmax_sel<NAN_PROP>(m, v[j]);
+  m = wave_max<NAN_PROP>(m);
+  if (WAVES > 1) {
+    if (t % WAVE == 0) red[t / WAVE] = m;
+    __syncthreads();
+    m = red[0];
+#pragma unroll
+    for (int w = 1; w < WAVES; w++) m = fmax_sel<NAN_PROP>(m, red[w]);
+    __syncthreads();
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < NPL; j++) {
+    // exp through the hardware exp2 (1 ulp) of a product rounded once: relative error below 1e-5
+    // even at the smallest normal result; a row of 781 elements costs 40 instructions per lane
+    // this way against some 300 through libm's expf, which made the kernel ALU-bound
+    v[j] = __builtin_amdgcn_exp2f((v[j] - m) * 1.44269504088896341f);
+    if (VEC || t + j * T < p.block) sum += v[j];
+  }
+  sum = wave_sum(sum);
+  if (WAVES > 1) {
+    if (t % WAVE == 0) red[t / WAVE] = sum;
+    __syncthreads();
+    sum = red[0];
+#pragma unroll
+    for (int w = 1; w < WAVES; w++) sum += red[w];
+  }
+  const float rsum = 1.0f / sum;  // one division per lane; the products are within 1.5 ulp of the quotients
+  if constexpr (VEC && IO != 2) {
+#pragma unroll
+    for (int j = 0; j < NPL / 8; j++) {
+      const int i0 = 8 * (t + j * T);
+      uint32_t o[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++)
+        o[k] = (uint32_t)down(v[8 * j + 2 * k] * rsum) | ((uint32_t)down(v[8 * j + 2 * k + 1] * rsum) << 16);
+      if (i0 < d_out) ntstore(reinterpret_cast<uint4 *>(out + i0), make_uint4(o[0], o[1], o[2], o[3]));
+    }
+  } else if constexpr (VEC) {
+#pragma unroll
+    for (int j = 0; j < NPL / 4; j++) {
+      const int i0 = 4 * (t + j * T);
+      f32x4_a4 w;
+#pragma unroll
+      for (int c = 0; c < 4; c++) w[c] = v[4 * j + c] * rsum;
+      if (i0 + 4 <= d_out) __builtin_nontemporal_store(w, reinterpret_cast<f32x4_a4 *>(out + i0));
+      else
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+          if (i0 + c < d_out) out[i0 + c] = w[c];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < NPL; j++) {
+      int i = t + j * T;
+      if (i < d_out) out[i] = down(v[j] * rsum);
+    }
+  }
+}
+
+template <int NPL, int WAVES, int WG, int IO>
+hipError_t launch_softmax_io(const SoftmaxParams &p, int gx, int gy, int gz, hipStream_t s) {
+  int64_t programs = (int64_t)gx * gy * gz;
+  int rows_per_wg = WG / (WAVES * WAVE);
+  dim3 grid((unsigned)((programs + rows_per_wg - 1) / rows_per_wg));
+  constexpr int EPC = IO == 2 ? 4 : 8;  // elements per 16-byte chunk
+  constexpr bool CAN_VEC = NPL % EPC == 0;
+  bool vec = CAN_VEC && p.block == NPL * WAVES * WAVE && p.d_in >= 4;
+  if (IO != 2) {  // whole chunks of aligned rows only
+    auto aligned = [](const Affine &a) { return (a.c0 | a.c[0] | a.c[1] | a.c[2]) % 8 == 0; };
+    vec = vec && p.d_in % 8 == 0 && p.d_out % 8 == 0 && aligned(p.in_off) && aligned(p.out_off) && (((uintptr_t)p.in | (uintptr_t)p.out) & 15) == 0;
+  }
+  if (vec) {
+    if (p.propagate_nan) hipLaunchKernelGGL((softmax_f32_kernel<NPL, WAVES, true, CAN_VEC, WG, IO>), grid, dim3(WG), 0, s, p, gx, gy, programs);
+    else hipLaunchKernelGGL((softmax_f32_kernel<NPL, WAVES, false, CAN_VEC, WG, IO>), grid, dim3(WG), 0, s, p, gx, gy, programs);
+    return hipGetLastError();
+  }
+  if (p.propagate_nan) hipLaunchKernelGGL((softmax_f32_kernel<NPL, WAVES, true, false, WG, IO>), grid, dim3(WG), 0, s, p, gx, gy, programs);
+  else hipLaunchKernelGGL((softmax_f32_kernel<NPL, WAVES, false, false, WG, IO>), grid, dim3(WG), 0, s, p, gx, gy, programs);
+  return hipGetLastError();
+}
+
+template <int NPL, int WAVES, int WG = 256>
+hipError_t launch_softmax_cfg(const SoftmaxParams &p, int gx, int gy, int gz, hipStream_t s) {
+  if (p.elem_kind == 2) return launch_softmax_io<NPL, WAVES, WG, 2>(p, gx, gy, gz, s);
+  if (p.elem_kind == 1) return launch_softmax_io<NPL, WAVES, WG, 1>(p, gx, gy, gz, s);
+  return launch_softmax_io<NPL, WAVES, WG, 0>(p, gx, gy, gz, s);
+}
+
+// -------------------------------------------------------------- layernorm
 // The element type of x, y, w and b: 0 fp16, 1 bf16, 2 fp32.  A chunk is the 16 bytes a thread moves at once: EPC elements.
 template <int KIND>
 struct LnType {

@@ -341,9 +341,18 @@ std::string subst(std::string s, const std::string &key, const std::string &val)
   return s;
 }
 
+// the same arithmetic on rows of fp16 / bf16: widened after the load, narrowed before the store
+const char *SIG_SOFTMAX_16 =
+    "v0=load:{T}.r1.m.o;v1=arith.extf:f32(v0);v2=reduce.arith.{MAX}.0(v1);v3=splat(v2);v4=arith.subf:f32(v1,v3);v5=math.exp:f32(v4);"
+    "v6=reduce.arith.addf.0(v5);v7=splat(v6);v8=arith.divf:f32(v5,v7);v9=arith.truncf:{T}(v8);store:{T}.r1.m(v9);";
+
 bool try_softmax(Plan &pl) {
-  if (pl.signature != subst(SIG_SOFTMAX, "{MAX}", "maxnumf") && pl.signature != subst(SIG_SOFTMAX, "{MAX}", "maximumf"))
-    return false;
+  bool known = false;
+  for (const char *mx : {"maxnumf", "maximumf"}) {
+    known = known || pl.signature == subst(SIG_SOFTMAX, "{MAX}", mx);
+    for (const char *t : {"f16", "bf16"}) known = known || pl.signature == subst(subst(SIG_SOFTMAX_16, "{MAX}", mx), "{T}", t);
+  }
+  if (!known) return false;
   const char *F = "row_softmax";
   Matcher m(pl.prog);
   SOp *ld = m.accesses.at(0), *st = m.accesses.at(1);
@@ -357,6 +366,8 @@ bool try_softmax(Plan &pl) {
   pl.k["in_arg"] = ld->acc.base_arg;
   pl.k["out_arg"] = st->acc.base_arg;
   pl.f["other"] = ld->acc.other_f;
+  if (ld->acc.elem != st->acc.elem) refuse(F, "its input and output differ in element type");
+  pl.k["elem_kind"] = ld->acc.elem == "f32" ? 2 : ld->acc.elem == "bf16" ? 1 : 0;
   LinIv li, lo;
   if (!m.linear(ld->acc.offsets[0], li) || !m.linear(st->acc.offsets[0], lo))
     refuse(F, "a row offset is not linear in the program id");

@@ -247,9 +247,10 @@ void bind_softmax(const Resolver &r, Bound &b) {
   p.block = (int)r.pl.k.at("block");
   p.other = (float)r.pl.f.at("other");
   p.propagate_nan = r.pl.signature.find("maximumf") != std::string::npos;
+  p.elem_kind = (int)r.pl.k.at("elem_kind");
   if (p.block > 65536) throw Unsupported("row_softmax: block sizes above 65536 are not implemented");
   std::ostringstream os;
-  os << "kernel=softmax_f32\nblock=" << p.block << "\nd_in=" << p.d_in << "\nd_out=" << p.d_out << "\nother=" << p.other
+  os << "kernel=softmax_f32\nelem=" << (p.elem_kind == 2 ? "f32" : p.elem_kind == 1 ? "bf16" : "f16") << "\nblock=" << p.block << "\nd_in=" << p.d_in << "\nd_out=" << p.d_out << "\nother=" << p.other
      << "\nin_off=" << show(p.in_off) << "\nout_off=" << show(p.out_off) << "\n";
   b.describe = os.str();
 }
@@ -692,8 +693,8 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
       }
       case Family::RowSoftmax: {
         SoftmaxParams p = b->softmax;
-        p.in = ptr_arg<const float>(args, pl, "in_arg");
-        p.out = ptr_arg<float>(args, pl, "out_arg");
+        p.in = ptr_arg<const void>(args, pl, "in_arg");
+        p.out = ptr_arg<void>(args, pl, "out_arg");
         err = launch_softmax(p, gx, gy, gz, s, &kname);
         break;
       }
