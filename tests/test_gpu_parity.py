@@ -492,6 +492,33 @@ def test_gemm_with_column_major_a_on_whole_k_tiles(K, M, N, Kd, dtype, b_too, ke
     assert relfro(c.float(), a.float() @ bb.float()) <= 1e-2
 
 
+@pytest.mark.parametrize("M,N,Kd,at,bt,BM,BN,BK", [(179, 321, 167, False, False, 32, 64, 16), (512, 384, 256, False, False, 128, 128, 32), (300, 260, 136, True, False, 64, 64, 32),
+                                                  (1000, 1031, 77, False, True, 128, 128, 32), (130, 200, 64, True, True, 64, 128, 16), (1, 5, 3, False, False, 32, 32, 16),
+                                                  (2048, 2048, 512, False, False, 128, 128, 32)])
+def test_gemm_on_fp32_blocks(K, M, N, Kd, at, bt, BM, BN, BK):
+    # tl.dot on fp32 blocks (the dtype of python/examples/test_matmul.py:137-157, whose first shape and blocks these are): the
+    # reference multiplies in fp32, and so does the fp32 matrix-core kernel; any shape, any alignment, either layout of A and B
+    torch.manual_seed(M + N + Kd)
+    A = torch.randint(-8, 9, (Kd, M) if at else (M, Kd)).float().to(DEV)
+    B = torch.randint(-8, 9, (N, Kd) if bt else (Kd, N)).float().to(DEV)
+    a, b = (A.t() if at else A), (B.t() if bt else B)
+    Cf = torch.full((M + 1, N + 3), 5.0, device=DEV)
+    c = Cf[:M, :N]
+    grid = (triton.cdiv(M, BM) * triton.cdiv(N, BN),)
+    k = K.matmul_tiles[grid](a, b, c, M, N, Kd, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1), BM=BM, BN=BN, BK=BK, GROUP_M=8)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and k.function.last_kernel == "gemm_f32_kernel"
+    assert torch.equal(c.cpu(), (a.cpu().double() @ b.cpu().double()).float())      # integers: every partial sum is exact in fp32
+    assert torch.equal(Cf[M].cpu(), torch.full((N + 3,), 5.0)) and torch.equal(Cf[:, N:].cpu(), torch.full((M + 1, 3), 5.0))
+    # random data: fp32 products and sums, so far inside the reference's own atol=1e-2 (test_matmul.py:157)
+    A.copy_(torch.randn_like(A))
+    B.copy_(torch.randn_like(B))
+    K.matmul_tiles[grid](a, b, c, M, N, Kd, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1), BM=BM, BN=BN, BK=BK, GROUP_M=8)
+    torch.cuda.synchronize()
+    want = a.cpu().double() @ b.cpu().double()
+    assert (c.cpu().double() - want).abs().max().item() <= 1e-3 and relfro(c.cpu(), want) <= 1e-5
+
+
 def test_gemm_with_column_major_a_and_with_strides_no_kernel_takes(K):
     torch.manual_seed(11)
     M, N, Kd = 300, 260, 136
@@ -1438,7 +1465,7 @@ def test_compiled_kernels_are_cached_on_disk(tmp_path, monkeypatch):
 def test_reference_matmul_test_in_fp32():
     """python/examples/test_matmul.py:137-157 as it stands: fp32 operands, 179 x 167 @ 167 x 321, blocks 32 x 64 x 16,
     GROUP_M 8, operand rows / columns wrapped, and the reference's own assertion (atol 1e-2, rtol 0).  fp32 products run
-    on the generic family (the MFMA kernels take bf16 / fp16)."""
+    on the fp32 matrix-core kernel of the matmul family."""
     torch.manual_seed(0)
     a = torch.randn(179, 167, device=DEV)
     b = torch.randn(167, 321, device=DEV)
@@ -1448,7 +1475,7 @@ def test_reference_matmul_test_in_fp32():
         k = kernel[grid](a, b, c, 179, 321, 167, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
                          BM=32, BN=64, BK=16, GROUP_M=8)
         torch.cuda.synchronize()
-        assert k.function.family == "tile_program"
+        assert k.function.family == "gemm" and k.function.last_kernel == "gemm_f32_kernel"
         torch.testing.assert_close(c, torch.matmul(a, b), atol=1e-2, rtol=0)
         assert ((c.double() - a.double() @ b.double()).norm() / (a.double() @ b.double()).norm()) < 1e-6
 

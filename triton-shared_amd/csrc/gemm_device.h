@@ -16,7 +16,7 @@ typedef __UINTPTR_TYPE__ uintptr_t;
 #include <cstdint>
 #endif
 
-// C[M,N] = A[M,K] * B[K,N], 16-bit operands, fp32 accumulate; C is row-major, A and B row- or column-major
+// C[M,N] = A[M,K] * B[K,N], 16-bit (or fp32) operands, fp32 accumulate; C is row-major, A and B row- or column-major
 struct TtsGemmParams {
   const void *a, *b;
   void *c;
@@ -32,6 +32,7 @@ struct TtsGemmParams {
   int64_t b_block_stride;
   int b_block_rows;
   int gather_mul32;       // bit 0: a_rows[m] * lda, bit 1: id * b_block_stride is a 32-bit product that wraps, as the source computes it
+  int is_f32;             // fp32 operands and result (kernels_gemm.hip: gemm_f32_kernel); is_bf16 is then 0
 };
 
 namespace tts_gemm_device {

@@ -83,6 +83,134 @@ bool gemm_dma_ok(const GemmParams &p, int64_t bm, int64_t bn) {
 }
 bool gemm_fast_path_ok(const GemmParams &p) { return !p.a_trans && !p.b_trans && gemm_dma_ok(p, F_BM, F_BN); }  // (the kernel compiled with an epilogue)
 
+// ------------------------------------------------------------- fp32 GEMM
+// tl.dot on fp32 blocks: the reference multiplies in fp32 (linalg.matmul on f32, ConversionPatterns.hpp:1128-1201; it
+// ignores the dot's inputPrecision), so this kernel uses the fp32 matrix instruction (v_mfma_f32_32x32x2_f32), not a
+// reduced-precision one.  Any shape and alignment, A and B row- or column-major.
+// Workgroup: 128 x 128 of C, 2 x 2 wavefronts of 64 x 64 (2 x 2 MFMA tiles of 32 x 32, 64 accumulator registers), K in
+// steps of 16.  Both operand tiles sit in LDS as [k][r] (r = row of A / column of B, pitch 132 floats): a lane's MFMA
+// operand is element (k0 + lane / 32, r0 + lane % 32), so a wavefront reads two runs of 32 consecutive floats.
+// Tiles go global -> registers -> LDS with the next tile's loads in flight during the current tile's arithmetic (two
+// LDS buffers, one barrier per tile); 16-byte global loads along whichever dimension is contiguous in memory.
+constexpr int F32_BM = 128, F32_BN = 128, F32_BK = 16, F32_PITCH = 132;
+
+__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p, int tiles_m, int tiles_n) {
+  __shared__ __align__(16) float smem[2][2][F32_BK * F32_PITCH];  // [buffer][A, B][k][r]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  int bid = blockIdx.x;
+  const int nwg = tiles_m * tiles_n;
+  if (nwg % 8 == 0) bid = (bid % 8) * (nwg / 8) + bid / 8;  // consecutive ids on one XCD
+  const int group = 8 * tiles_n;
+  const int g0 = (bid / group) * 8;
+  const int gh = min(tiles_m - g0, 8);
+  const int tile_m = g0 + (bid % group) % gh, tile_n = (bid % group) / gh;
+  const int64_t m0 = (int64_t)tile_m * F32_BM, n0 = (int64_t)tile_n * F32_BN;
+  const float *__restrict__ A = (const float *)p.a;
+  const float *__restrict__ B = (const float *)p.b;
+  const int64_t K = p.K;
+  const bool a_vec = p.lda % 4 == 0 && ((uintptr_t)A & 15) == 0, b_vec = p.ldb % 4 == 0 && ((uintptr_t)B & 15) == 0;
+
+  // An operand tile is 128 r x 16 k = 512 chunks of 4 floats, two per thread.  k contiguous in memory (A row-major, B
+  // column-major): chunk c = (r = c / 4, k = 4 (c % 4)); r contiguous (A column-major, B row-major): (k = c / 32, r = 4 (c % 32)).
+  auto load_tile = [&](float4 (&reg)[2], const float *P, bool r_contig, int64_t ld, int64_t r_base, int64_t rows, bool vec, int64_t k0) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int c = tid + 256 * j;
+      float v[4] = {0.f, 0.f, 0.f, 0.f};
+      if (r_contig) {
+        const int64_t k = k0 + c / 32, r = r_base + 4 * (c % 32);
+        if (k < K) {
+          const float *src = P + k * ld + r;
+          if (vec && r + 4 <= rows) { const float4 q = *reinterpret_cast<const float4 *>(src); v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w; }
+          else
+            for (int i = 0; i < 4; i++) if (r + i < rows) v[i] = src[i];
+        }
+      } else {
+        const int64_t r = r_base + c / 4, k = k0 + 4 * (c % 4);
+        if (r < rows) {
+          const float *src = P + r * ld + k;
+          if (vec && k + 4 <= K) { const float4 q = *reinterpret_cast<const float4 *>(src); v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w; }
+          else
+            for (int i = 0; i < 4; i++) if (k + i < K) v[i] = src[i];
+        }
+      }
+      reg[j] = make_float4(v[0], v[1], v[2], v[3]);
+    }
+  };
+  auto store_tile = [&](const float4 (&reg)[2], float *S, bool r_contig) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int c = tid + 256 * j;
+      if (r_contig) {
+        *reinterpret_cast<float4 *>(S + (c / 32) * F32_PITCH + 4 * (c % 32)) = reg[j];
+      } else {  // four k of one r: one float into each of four k rows
+        float *dst = S + (4 * (c % 4)) * F32_PITCH + c / 4;
+        dst[0] = reg[j].x; dst[F32_PITCH] = reg[j].y; dst[2 * F32_PITCH] = reg[j].z; dst[3 * F32_PITCH] = reg[j].w;
+      }
+    }
+  };
+  const bool a_r = p.a_trans != 0, b_r = p.b_trans == 0;  // r contiguous in memory
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+  float4 ra[2], rb[2];
+  const int64_t nk = (K + F32_BK - 1) / F32_BK;
+  if (nk > 0) {
+    load_tile(ra, A, a_r, p.lda, m0, p.M, a_vec, 0);
+    load_tile(rb, B, b_r, p.ldb, n0, p.N, b_vec, 0);
+    store_tile(ra, smem[0][0], a_r);
+    store_tile(rb, smem[0][1], b_r);
+  }
+  __syncthreads();
+  for (int64_t kt = 0; kt < nk; kt++) {
+    const int cur = (int)(kt & 1);
+    if (kt + 1 < nk) {
+      load_tile(ra, A, a_r, p.lda, m0, p.M, a_vec, (kt + 1) * F32_BK);
+      load_tile(rb, B, b_r, p.ldb, n0, p.N, b_vec, (kt + 1) * F32_BK);
+    }
+    const float *As = smem[cur][0] + (lane >> 5) * F32_PITCH + wm * 64 + (lane & 31);
+    const float *Bs = smem[cur][1] + (lane >> 5) * F32_PITCH + wn * 64 + (lane & 31);
+#pragma unroll
+    for (int ks = 0; ks < F32_BK; ks += 2) {
+      const float a0 = As[ks * F32_PITCH], a1 = As[ks * F32_PITCH + 32];
+      const float b0 = Bs[ks * F32_PITCH], b1 = Bs[ks * F32_PITCH + 32];
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+    }
+    if (kt + 1 < nk) {
+      store_tile(ra, smem[cur ^ 1][0], a_r);
+      store_tile(rb, smem[cur ^ 1][1], b_r);
+    }
+    __syncthreads();
+  }
+  // lane holds column (lane % 32), rows 8 (v / 4) + 4 (lane / 32) + v % 4 of each 32 x 32 tile
+  float *__restrict__ C = (float *)p.c;
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int64_t col = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int64_t row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        if (row < p.M && col < p.N) C[row * p.ldc + col] = acc[i][j][v];
+      }
+    }
+}
+
+hipError_t launch_gemm_f32(const GemmParams &p, hipStream_t s) {
+  const int tiles_m = (int)((p.M + F32_BM - 1) / F32_BM), tiles_n = (int)((p.N + F32_BN - 1) / F32_BN);
+  hipLaunchKernelGGL(gemm_f32_kernel, dim3(tiles_m * tiles_n), dim3(256), 0, s, p, tiles_m, tiles_n);
+  return hipGetLastError();
+}
+
 // ------------------------------------------------------ int8-weight GEMM
 // Workgroup: NW wavefronts share one 128-column slab of W and split its K range
 // in interleaved steps of 32 rows.  In a step, lane (j = lane % 16, g = lane / 16)
@@ -494,6 +622,11 @@ constexpr int W8_WAVES = 16;
 }  // namespace
 
 hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
+  if (p.is_f32) {
+    if (p.a_rows || p.b_block) return hipErrorInvalidValue;  // (the matcher takes gathered rows on 16-bit operands only)
+    *name = "gemm_f32_kernel";
+    return launch_gemm_f32(p, s);
+  }
   static const char *tile_env = getenv("TTS_GEMM_TILE");  // tuning aid: set = the any-shape kernel even for whole tiles
   static const char *dma_env = getenv("TTS_GEMM_DMA");    // tuning aid: "256x256", "128x256", "256x128", "128x128" or unset
   if (!tile_env) {

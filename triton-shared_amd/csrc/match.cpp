@@ -539,12 +539,16 @@ bool carried_state(Matcher &m, SOp *loop, const Access &a, Carried2D &out) {
   return true;
 }
 
+// the same program on fp32 blocks: the accumulator is stored as it is
+const char *SIG_GEMM_F32 = "v0=const:f32;for[v1<-v0]{v2=load:f32.r2.m.o;v3=load:f32.r2.m.o;v4=dot(v2,v3,v1);yield(v4)}->v5;store:f32.r2.m(v5);";
+
 bool try_gemm(Plan &pl, bool w8a16) {
   std::string sig = pl.signature;
   std::string T;
   if (!w8a16) {
     if (sig == subst(SIG_GEMM, "{T}", "bf16")) T = "bf16";
     else if (sig == subst(SIG_GEMM, "{T}", "f16")) T = "f16";
+    else if (sig == SIG_GEMM_F32) T = "f32";
     else return false;
   } else {
     if (sig != SIG_W8A16) return false;
@@ -613,6 +617,7 @@ bool try_gemm(Plan &pl, bool w8a16) {
   pl.k["b_arg"] = Bm->acc.base_arg;
   pl.k["c_arg"] = C->acc.base_arg;
   pl.k["is_bf16"] = T == "bf16";
+  pl.k["is_f32"] = T == "f32";
   pl.k["loop"] = loop->loop;
   pl.e["a_base"] = ca.base;
   pl.e["a_kstep"] = ca.kstep;

@@ -399,6 +399,8 @@ void bind_gemm(const Resolver &r, Bound &b) {
   p.M = d.M; p.N = d.N; p.K = d.K; p.lda = d.lda; p.ldb = d.ldb; p.ldc = d.ldc;
   p.a_trans = d.a_trans; p.b_trans = d.b_trans;
   p.is_bf16 = (int)r.pl.k.at("is_bf16");
+  p.is_f32 = r.pl.k.count("is_f32") ? (int)r.pl.k.at("is_f32") : 0;
+  if (p.is_f32 && !r.pl.source.empty()) throw Unsupported("gemm: a fused epilogue on fp32 operands");
   if (!r.pl.source.empty()) {  // a fused epilogue looks up the program that owns an element
     may_allocate("a table of tile owners on the device");
     hipError_t e = hipMalloc((void **)&b.tile_pid, d.tile_pid.size() * sizeof(int));
@@ -408,7 +410,7 @@ void bind_gemm(const Resolver &r, Bound &b) {
   }
   std::ostringstream os;
   os << "kernel=gemm_mfma\nM=" << p.M << "\nN=" << p.N << "\nK=" << p.K << "\nlda=" << p.lda << "\nldb=" << p.ldb
-     << "\nldc=" << p.ldc << "\nbf16=" << p.is_bf16 << "\na_trans=" << p.a_trans << "\nb_trans=" << p.b_trans << "\n";
+     << "\nldc=" << p.ldc << "\nbf16=" << p.is_bf16 << "\nf32=" << p.is_f32 << "\na_trans=" << p.a_trans << "\nb_trans=" << p.b_trans << "\n";
   b.describe = os.str();
 }
 
