@@ -88,14 +88,20 @@ bool gemm_fast_path_ok(const GemmParams &p) { return !p.a_trans && !p.b_trans &&
 // ignores the dot's inputPrecision), so this kernel uses the fp32 matrix instruction (v_mfma_f32_32x32x2_f32), not a
 // reduced-precision one.  Any shape and alignment, A and B row- or column-major.
 // Workgroup: 128 x 128 of C, 2 x 2 wavefronts of 64 x 64 (2 x 2 MFMA tiles of 32 x 32, 64 accumulator registers), K in
-// steps of 16.  Both operand tiles sit in LDS as [k][r] (r = row of A / column of B, pitch 132 floats): a lane's MFMA
+// steps of 16.  Both operand tiles sit in LDS as [k][r] (r = row of A / column of B, pitch = tile + 4 floats): a lane's MFMA
 // operand is element (k0 + lane / 32, r0 + lane % 32), so a wavefront reads two runs of 32 consecutive floats.
 // Tiles go global -> registers -> LDS with the next tile's loads in flight during the current tile's arithmetic (two
 // LDS buffers, one barrier per tile); 16-byte global loads along whichever dimension is contiguous in memory.
-constexpr int F32_BM = 128, F32_BN = 128, F32_BK = 16, F32_PITCH = 132;
+// T: MFMA tiles per wavefront and dimension: 2 = 128 x 128 per workgroup, 1 = 64 x 64 (for problems that give fewer than
+// two of the large tiles per CU: 2048^3 ran at 57 TFLOP/s on 256 large tiles, one wavefront per SIMD).
+constexpr int F32_BK = 16;
 
+template <int T>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p, int tiles_m, int tiles_n) {
-  __shared__ __align__(16) float smem[2][2][F32_BK * F32_PITCH];  // [buffer][A, B][k][r]
+  constexpr int BT = 64 * T;          // rows of A / columns of B per workgroup
+  constexpr int PITCH = BT + 4;       // floats between k rows in LDS
+  constexpr int CH = BT / 64;         // chunks of 4 floats per thread and operand tile (BT x 16 floats = 4 BT chunks)
+  __shared__ __align__(16) float smem[2][2][F32_BK * PITCH];  // [buffer][A, B][k][r]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   int bid = blockIdx.x;
@@ -105,21 +111,21 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p, int tiles_m
   const int g0 = (bid / group) * 8;
   const int gh = min(tiles_m - g0, 8);
   const int tile_m = g0 + (bid % group) % gh, tile_n = (bid % group) / gh;
-  const int64_t m0 = (int64_t)tile_m * F32_BM, n0 = (int64_t)tile_n * F32_BN;
+  const int64_t m0 = (int64_t)tile_m * BT, n0 = (int64_t)tile_n * BT;
   const float *__restrict__ A = (const float *)p.a;
   const float *__restrict__ B = (const float *)p.b;
   const int64_t K = p.K;
   const bool a_vec = p.lda % 4 == 0 && ((uintptr_t)A & 15) == 0, b_vec = p.ldb % 4 == 0 && ((uintptr_t)B & 15) == 0;
 
-  // An operand tile is 128 r x 16 k = 512 chunks of 4 floats, two per thread.  k contiguous in memory (A row-major, B
-  // column-major): chunk c = (r = c / 4, k = 4 (c % 4)); r contiguous (A column-major, B row-major): (k = c / 32, r = 4 (c % 32)).
-  auto load_tile = [&](float4 (&reg)[2], const float *P, bool r_contig, int64_t ld, int64_t r_base, int64_t rows, bool vec, int64_t k0) {
+  // An operand tile is BT r x 16 k = 4 BT chunks of 4 floats, CH per thread.  k contiguous in memory (A row-major, B
+  // column-major): chunk c = (r = c / 4, k = 4 (c % 4)); r contiguous (A column-major, B row-major): (k = c / (BT / 4), r = 4 (c % (BT / 4))).
+  auto load_tile = [&](float4 (&reg)[CH], const float *P, bool r_contig, int64_t ld, int64_t r_base, int64_t rows, bool vec, int64_t k0) {
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
+    for (int j = 0; j < CH; j++) {
       const int c = tid + 256 * j;
       float v[4] = {0.f, 0.f, 0.f, 0.f};
       if (r_contig) {
-        const int64_t k = k0 + c / 32, r = r_base + 4 * (c % 32);
+        const int64_t k = k0 + c / (BT / 4), r = r_base + 4 * (c % (BT / 4));
         if (k < K) {
           const float *src = P + k * ld + r;
           if (vec && r + 4 <= rows) { const float4 q = *reinterpret_cast<const float4 *>(src); v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w; }
@@ -138,27 +144,27 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p, int tiles_m
       reg[j] = make_float4(v[0], v[1], v[2], v[3]);
     }
   };
-  auto store_tile = [&](const float4 (&reg)[2], float *S, bool r_contig) {
+  auto store_tile = [&](const float4 (&reg)[CH], float *S, bool r_contig) {
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
+    for (int j = 0; j < CH; j++) {
       const int c = tid + 256 * j;
       if (r_contig) {
-        *reinterpret_cast<float4 *>(S + (c / 32) * F32_PITCH + 4 * (c % 32)) = reg[j];
+        *reinterpret_cast<float4 *>(S + (c / (BT / 4)) * PITCH + 4 * (c % (BT / 4))) = reg[j];
       } else {  // four k of one r: one float into each of four k rows
-        float *dst = S + (4 * (c % 4)) * F32_PITCH + c / 4;
-        dst[0] = reg[j].x; dst[F32_PITCH] = reg[j].y; dst[2 * F32_PITCH] = reg[j].z; dst[3 * F32_PITCH] = reg[j].w;
+        float *dst = S + (4 * (c % 4)) * PITCH + c / 4;
+        dst[0] = reg[j].x; dst[PITCH] = reg[j].y; dst[2 * PITCH] = reg[j].z; dst[3 * PITCH] = reg[j].w;
       }
     }
   };
   const bool a_r = p.a_trans != 0, b_r = p.b_trans == 0;  // r contiguous in memory
-  f32x16 acc[2][2];
+  f32x16 acc[T][T];
 #pragma unroll
-  for (int i = 0; i < 2; i++)
+  for (int i = 0; i < T; i++)
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < T; j++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
-  float4 ra[2], rb[2];
+  float4 ra[CH], rb[CH];
   const int64_t nk = (K + F32_BK - 1) / F32_BK;
   if (nk > 0) {
     load_tile(ra, A, a_r, p.lda, m0, p.M, a_vec, 0);
@@ -173,16 +179,19 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p, int tiles_m
       load_tile(ra, A, a_r, p.lda, m0, p.M, a_vec, (kt + 1) * F32_BK);
       load_tile(rb, B, b_r, p.ldb, n0, p.N, b_vec, (kt + 1) * F32_BK);
     }
-    const float *As = smem[cur][0] + (lane >> 5) * F32_PITCH + wm * 64 + (lane & 31);
-    const float *Bs = smem[cur][1] + (lane >> 5) * F32_PITCH + wn * 64 + (lane & 31);
+    const float *As = smem[cur][0] + (lane >> 5) * PITCH + wm * (32 * T) + (lane & 31);
+    const float *Bs = smem[cur][1] + (lane >> 5) * PITCH + wn * (32 * T) + (lane & 31);
 #pragma unroll
     for (int ks = 0; ks < F32_BK; ks += 2) {
-      const float a0 = As[ks * F32_PITCH], a1 = As[ks * F32_PITCH + 32];
-      const float b0 = Bs[ks * F32_PITCH], b1 = Bs[ks * F32_PITCH + 32];
-      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+      float af[T], bf[T];
+#pragma unroll
+      for (int i = 0; i < T; i++) af[i] = As[ks * PITCH + 32 * i];
+#pragma unroll
+      for (int j = 0; j < T; j++) bf[j] = Bs[ks * PITCH + 32 * j];
+#pragma unroll
+      for (int i = 0; i < T; i++)
+#pragma unroll
+        for (int j = 0; j < T; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
     }
     if (kt + 1 < nk) {
       store_tile(ra, smem[cur ^ 1][0], a_r);
@@ -193,21 +202,32 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p, int tiles_m
   // lane holds column (lane % 32), rows 8 (v / 4) + 4 (lane / 32) + v % 4 of each 32 x 32 tile
   float *__restrict__ C = (float *)p.c;
 #pragma unroll
-  for (int i = 0; i < 2; i++)
+  for (int i = 0; i < T; i++)
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const int64_t col = n0 + wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < T; j++) {
+      const int64_t col = n0 + wn * (32 * T) + j * 32 + (lane & 31);
 #pragma unroll
       for (int v = 0; v < 16; v++) {
-        const int64_t row = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+        const int64_t row = m0 + wm * (32 * T) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
         if (row < p.M && col < p.N) C[row * p.ldc + col] = acc[i][j][v];
       }
     }
 }
 
 hipError_t launch_gemm_f32(const GemmParams &p, hipStream_t s) {
-  const int tiles_m = (int)((p.M + F32_BM - 1) / F32_BM), tiles_n = (int)((p.N + F32_BN - 1) / F32_BN);
-  hipLaunchKernelGGL(gemm_f32_kernel, dim3(tiles_m * tiles_n), dim3(256), 0, s, p, tiles_m, tiles_n);
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    return n;
+  }();
+  const int64_t big = ((p.M + 127) / 128) * ((p.N + 127) / 128);
+  if (big >= 2 * cus) {
+    const int tiles_m = (int)((p.M + 127) / 128), tiles_n = (int)((p.N + 127) / 128);
+    hipLaunchKernelGGL(gemm_f32_kernel<2>, dim3(tiles_m * tiles_n), dim3(256), 0, s, p, tiles_m, tiles_n);
+  } else {
+    const int tiles_m = (int)((p.M + 63) / 64), tiles_n = (int)((p.N + 63) / 64);
+    hipLaunchKernelGGL(gemm_f32_kernel<1>, dim3(tiles_m * tiles_n), dim3(256), 0, s, p, tiles_m, tiles_n);
+  }
   return hipGetLastError();
 }
 
