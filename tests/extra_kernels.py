@@ -1065,3 +1065,31 @@ def transpose_tiles(src, dst, R, C, BR: tl.constexpr, BC: tl.constexpr):
     m = (r[:, None] < R) & (c[None, :] < C)
     x = tl.load(src + r[:, None] * C + c[None, :], mask=m, other=0.0)
     tl.store(dst + c[:, None] * R + r[None, :], tl.trans(x * 2.0), mask=tl.trans(m))
+
+
+@triton.jit
+def attention_fwd(Q, K, V, O, sm_scale, seq, stride_h, stride_s, BM: tl.constexpr, BN: tl.constexpr, D: tl.constexpr):
+    # flash-attention forward, one (query block, head) per program, plain pointer arithmetic on fp16 tensors: two tile products
+    # per step, an online softmax whose running maximum and sum (vectors of BM) are carried next to the [BM, D] accumulator
+    pm = tl.program_id(0)
+    ph = tl.program_id(1)
+    rm = pm * BM + tl.arange(0, BM)
+    rd = tl.arange(0, D)
+    q = tl.load(Q + ph * stride_h + rm[:, None] * stride_s + rd[None, :], mask=rm[:, None] < seq, other=0.0)
+    m_i = tl.zeros([BM], dtype=tl.float32) - float("inf")
+    l_i = tl.zeros([BM], dtype=tl.float32)
+    acc = tl.zeros([BM, D], dtype=tl.float32)
+    for start in range(0, seq, BN):
+        rn = start + tl.arange(0, BN)
+        k = tl.load(K + ph * stride_h + rn[:, None] * stride_s + rd[None, :], mask=rn[:, None] < seq, other=0.0)
+        v = tl.load(V + ph * stride_h + rn[:, None] * stride_s + rd[None, :], mask=rn[:, None] < seq, other=0.0)
+        qk = tl.dot(q, tl.trans(k)) * sm_scale
+        qk = tl.where(rn[None, :] < seq, qk, -float("inf"))
+        m_new = tl.maximum(m_i, tl.max(qk, axis=1))
+        p = tl.exp(qk - m_new[:, None])
+        alpha = tl.exp(m_i - m_new)
+        l_i = l_i * alpha + tl.sum(p, axis=1)
+        acc = acc * alpha[:, None] + tl.dot(p.to(tl.float16), v)
+        m_i = m_new
+    acc = acc / l_i[:, None]
+    tl.store(O + ph * stride_h + rm[:, None] * stride_s + rd[None, :], acc.to(tl.float16), mask=rm[:, None] < seq)

@@ -598,6 +598,23 @@ def test_row_softmax_on_16_bit_rows(K, rows, cols, pitch, block, dtype):
     assert torch.equal(full[rows].cpu(), torch.full((pitch,), -9.0, dtype=dtype)) and torch.equal(full[:, cols:].cpu(), torch.full((rows + 1, pitch - cols), -9.0, dtype=dtype))
 
 
+@pytest.mark.parametrize("H,seq,D,BM,BN", [(3, 200, 64, 64, 64), (2, 80, 32, 32, 32), (4, 1024, 64, 64, 32), (1, 33, 64, 32, 64)])
+def test_flash_attention_forward(H, seq, D, BM, BN):
+    # two tile products per step and an online softmax: the running maximum and sum are loop-carried vectors that the
+    # [BM, BN] scores and the [BM, D] accumulator read as columns, so they are kept in LDS next to their owners' registers
+    import extra_kernels as X
+    torch.manual_seed(seq + D)
+    q, k, v = (torch.randn(H, seq, D, device=DEV).half() for _ in range(3))
+    o = torch.full((H + 1, seq, D), 3.0, device=DEV, dtype=torch.float16)
+    kern = X.attention_fwd[(triton.cdiv(seq, BM), H)](q, k, v, o, D ** -0.5, seq, seq * D, D, BM=BM, BN=BN, D=D)
+    torch.cuda.synchronize()
+    assert kern.function.family == "tile_program"
+    s = torch.einsum("hqd,hkd->hqk", q.double(), k.double()) * D ** -0.5
+    want = torch.einsum("hqk,hkd->hqd", torch.softmax(s, -1), v.double())
+    assert (o[:H].double() - want).abs().max().item() <= 4e-3          # fp16 probabilities and output
+    assert torch.equal(o[H], torch.full((seq, D), 3.0, device=DEV, dtype=torch.float16))
+
+
 def test_softmax_rows_the_row_kernel_declines(K, oracle_cpu):
     import extra_kernels as X
     torch.manual_seed(5)

@@ -397,3 +397,23 @@ def test_lanes_if_with_results_against_numpy():
     ttir_lanes.Interpreter(t).run((4,), [None, None, None], {0: x, 1: flags, 2: out})
     want = np.stack([(x * 2 + 1 + np.float32(3 * f)) if f > 0 else (x - 1 - 1 + np.float32(7 - f)) for f in flags])
     assert np.array_equal(out.reshape(4, 128), want.astype(np.float32))
+
+
+def test_lanes_flash_attention_forward_matches_the_closed_form():
+    """The lane interpreter on a flash-attention forward (two tile products per step, online softmax with carried vectors):
+    softmax(Q K^T / sqrt(D)) V in float64, on a sequence that is not a multiple of the blocks."""
+    import extra_kernels as X
+    from test_planner import compile_ttir
+    sig = {"Q": "*fp16", "K": "*fp16", "V": "*fp16", "O": "*fp16", "sm_scale": "fp32", "seq": "i32", "stride_h": "i32", "stride_s": "i32",
+           "BM": "constexpr", "BN": "constexpr", "D": "constexpr"}
+    t = compile_ttir(X.attention_fwd, sig, {"BM": 32, "BN": 32, "D": 32})
+    rng = np.random.default_rng(0)
+    H, seq, D = 2, 80, 32
+    q, k, v = (rng.standard_normal((H, seq, D)).astype(np.float16) for _ in range(3))
+    bufs = {0: q.reshape(-1).copy(), 1: k.reshape(-1).copy(), 2: v.reshape(-1).copy(), 3: np.zeros(H * seq * D, np.float16)}
+    ttir_lanes.Interpreter(t).run(((seq + 31) // 32, H), [None, None, None, None, np.float32(D ** -0.5), seq, seq * D, D], bufs)
+    s = np.einsum("hqd,hkd->hqk", q.astype(np.float64), k.astype(np.float64)) * D ** -0.5
+    p = np.exp(s - s.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    want = np.einsum("hqk,hkd->hqd", p, v.astype(np.float64))
+    assert np.abs(bufs[3].reshape(H, seq, D).astype(np.float64) - want).max() <= 2e-3

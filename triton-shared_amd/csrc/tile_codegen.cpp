@@ -181,7 +181,11 @@ struct Gen {
       if (sh.empty() || (i0 == cur_i0 && (sh.size() < 2 || i1 == cur_i1))) return it->second;
     }
     auto d = def.find(v);
-    if (d == def.end()) no("a loop-carried block value used in a loop over another block shape");
+    if (d == def.end()) {
+      auto mi = mirror.find(v);
+      if (mi != mirror.end()) return mi->second + "[" + linear(val(v).shape, i0, i1) + "]";
+      no("a loop-carried block value used in a loop over another block shape");
+    }
     const SOp &s = *d->second;
     const Value &V = val(v);
     auto idx = [&](const std::vector<int64_t> &shape, size_t dim) -> std::string {
@@ -532,6 +536,10 @@ struct Gen {
   }
   struct Held { std::string name; std::vector<int64_t> shape; };
   std::map<int, Held> held;
+  // Loop-carried vectors that a loop also reads from blocks of another shape (the running maximum and sum of an online
+  // softmax next to its [BM, BN] scores): besides the owning threads' registers they are kept in an LDS array, written
+  // where the registers are, which any thread may read.  value id -> array
+  std::map<int, std::string> mirror;
   void map_vars(const std::vector<int64_t> &shape) {
     for (auto &h : held) {
       if (h.second.shape == shape) var[h.first] = h.second.name + "[n]";
@@ -888,13 +896,41 @@ struct Gen {
       if (std::find(cshapes.begin(), cshapes.end(), V.shape) == cshapes.end()) cshapes.push_back(V.shape);
       os << pad() << ctype(V.dtype) << " car" << L << "_" << q << "[" << (count(V.shape) + 255) / 256 << "];\n";
     }
+    // carried vectors of a loop that also works on blocks of another shape get an LDS copy (see `mirror`)
+    std::vector<std::string> mirrored(s.tile_args.size());
+    {
+      std::function<bool(const std::vector<SOp> &, const std::vector<int64_t> &)> other_shape = [&](const std::vector<SOp> &ops, const std::vector<int64_t> &sh) {
+        for (const SOp &o : ops) {
+          if (o.result >= 0 && !val(o.result).shape.empty() && val(o.result).shape != sh) return true;
+          if (other_shape(o.body, sh)) return true;
+        }
+        return false;
+      };
+      for (size_t q = 0; q < s.tile_args.size(); q++) {
+        const Value &V = val(s.tile_args[q]);
+        const size_t bytes = (size_t)count(V.shape) * held_bytes(V.dtype);
+        if (V.shape.size() != 1 || count(V.shape) > 4096 || !other_shape(s.body, V.shape) || pool_bytes + out_bytes + bytes > 56 * 1024) continue;
+        mirrored[q] = "carm" + L + "_" + std::to_string(q);
+        decl << "  __shared__ " << ctype(V.dtype) << " " << mirrored[q] << "[" << count(V.shape) << "];\n";
+        out_bytes += (bytes + 15) / 16 * 16;
+      }
+    }
+    bool any_mirror = false;
+    for (const auto &m : mirrored) any_mirror = any_mirror || !m.empty();
     for (const auto &cshape : cshapes) {
       open_element_loop(cshape);
       for (size_t q = 0; q < s.tile_args.size(); q++)
-        if (val(s.tile_args[q]).shape == cshape) os << pad() << "car" << L << "_" << q << "[n] = " << at(s.tile_inits[q], idx0(cshape), idx1(cshape)) << ";\n";
+        if (val(s.tile_args[q]).shape == cshape) {
+          os << pad() << "car" << L << "_" << q << "[n] = " << at(s.tile_inits[q], idx0(cshape), idx1(cshape)) << ";\n";
+          if (!mirrored[q].empty()) os << pad() << mirrored[q] << "[t] = car" << L << "_" << q << "[n];\n";
+        }
       close_loop();
     }
-    for (size_t q = 0; q < s.tile_args.size(); q++) held[s.tile_args[q]] = {"car" + L + "_" + std::to_string(q), val(s.tile_args[q]).shape};
+    if (any_mirror) os << pad() << "__syncthreads();\n";
+    for (size_t q = 0; q < s.tile_args.size(); q++) {
+      held[s.tile_args[q]] = {"car" + L + "_" + std::to_string(q), val(s.tile_args[q]).shape};
+      if (!mirrored[q].empty()) mirror[s.tile_args[q]] = mirrored[q];
+    }
     for (size_t q = 0; q < s.int_iters.size(); q++)
       os << pad() << "long long it" << L << "_" << q << " = " << ex(s.int_iters[q].init) << ";\n";
     // the induction variable wraps at the width of the loop's bounds
@@ -903,6 +939,28 @@ struct Gen {
     indent++;
     std::vector<int> body_held;
     body(s.body, &body_held);
+    // With LDS copies: every new value is computed (and every reader of the old copies is done) before a copy changes, and
+    // the new copies are complete before the next iteration reads them.
+    if (any_mirror) {
+      for (size_t q = 0; q < s.tile_args.size(); q++) os << pad() << ctype(val(s.tile_args[q]).dtype) << " nyv" << L << "_" << q << "[" << (count(val(s.tile_args[q]).shape) + 255) / 256 << "];\n";
+      for (const auto &cshape : cshapes) {
+        open_element_loop(cshape);
+        for (size_t q = 0; q < s.tile_args.size(); q++)
+          if (val(s.tile_args[q]).shape == cshape) os << pad() << "nyv" << L << "_" << q << "[n] = " << at(s.tile_yields[q], idx0(cshape), idx1(cshape)) << ";\n";
+        close_loop();
+      }
+      os << pad() << "__syncthreads();\n";
+      for (const auto &cshape : cshapes) {
+        open_element_loop(cshape);
+        for (size_t q = 0; q < s.tile_args.size(); q++)
+          if (val(s.tile_args[q]).shape == cshape) {
+            os << pad() << "car" << L << "_" << q << "[n] = nyv" << L << "_" << q << "[n];\n";
+            if (!mirrored[q].empty()) os << pad() << mirrored[q] << "[t] = nyv" << L << "_" << q << "[n];\n";
+          }
+        close_loop();
+      }
+      os << pad() << "__syncthreads();\n";
+    } else
     for (const auto &cshape : cshapes) {  // all new values of a shape first, then the assignments: a yield may read another carried value
       open_element_loop(cshape);
       for (size_t q = 0; q < s.tile_args.size(); q++)
@@ -927,7 +985,11 @@ struct Gen {
     for (size_t q = 0; q < s.tile_args.size(); q++) {
       held.erase(s.tile_args[q]);
       var.erase(s.tile_args[q]);
-      if (s.results[q] >= 0) held[s.results[q]] = {"car" + L + "_" + std::to_string(q), val(s.tile_args[q]).shape};
+      mirror.erase(s.tile_args[q]);
+      if (s.results[q] >= 0) {
+        held[s.results[q]] = {"car" + L + "_" + std::to_string(q), val(s.tile_args[q]).shape};
+        if (!mirrored[q].empty()) mirror[s.results[q]] = mirrored[q];  // (a result read from another shape after the loop)
+      }
     }
   }
 
