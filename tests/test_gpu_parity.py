@@ -598,7 +598,7 @@ def test_row_softmax_on_16_bit_rows(K, rows, cols, pitch, block, dtype):
     assert torch.equal(full[rows].cpu(), torch.full((pitch,), -9.0, dtype=dtype)) and torch.equal(full[:, cols:].cpu(), torch.full((rows + 1, pitch - cols), -9.0, dtype=dtype))
 
 
-@pytest.mark.parametrize("H,seq,D,BM,BN", [(3, 200, 64, 64, 64), (2, 80, 32, 32, 32), (4, 1024, 64, 64, 32), (1, 33, 64, 32, 64)])
+@pytest.mark.parametrize("H,seq,D,BM,BN", [(3, 200, 64, 64, 64), (2, 80, 32, 32, 32), (4, 1024, 64, 64, 32), (1, 33, 64, 32, 64), (2, 300, 128, 32, 64)])
 def test_flash_attention_forward(H, seq, D, BM, BN):
     # two tile products per step and an online softmax: the running maximum and sum are loop-carried vectors that the
     # [BM, BN] scores and the [BM, D] accumulator read as columns, so they are kept in LDS next to their owners' registers
