@@ -1621,7 +1621,9 @@ def test_matmul_with_gathered_rows_is_exact_on_selections():
 
 
 @pytest.mark.parametrize("tokens,kd,nd,experts,kernel", [(1024, 256, 512, 4, "gemm_dma_kernel<128x128>"), (4096, 64, 2048, 8, "gemm_dma_kernel<128x256>"),
-                                                         (384, 96, 128, 5, "gemm_dma_kernel<128x128>")])
+                                                         (384, 96, 128, 5, "gemm_dma_kernel<128x128>"),
+                                                         # more row tiles than the kernel sorts (256): taken in memory order
+                                                         (128 * 300, 32, 128, 6, "gemm_dma_kernel<128x128>")])
 def test_matmul_with_gathered_rows_on_whole_tiles(tokens, kd, nd, experts, kernel):
     # whole 128-row tiles go to the direct-to-LDS kernel, which walks the row tiles in the order of their matrix ids (so
     # that the tiles of one matrix share an L2): ids dealt out of order, repeated and negative; exact as above
