@@ -1620,18 +1620,26 @@ def test_matmul_with_gathered_rows_is_exact_on_selections():
     assert torch.equal(c, want)
 
 
-@pytest.mark.parametrize("tokens,kd,nd,experts,kernel", [(1024, 256, 512, 4, "gemm_dma_kernel<128x128>"), (4096, 64, 2048, 8, "gemm_dma_kernel<128x256>"),
+@pytest.mark.parametrize("case", [(1024, 256, 512, 4, "gemm_dma_kernel<128x128>"), (4096, 64, 2048, 8, "gemm_dma_kernel<128x256>"),
                                                          (384, 96, 128, 5, "gemm_dma_kernel<128x128>"),
                                                          # more row tiles than the kernel sorts (256): taken in memory order
-                                                         (128 * 300, 32, 128, 6, "gemm_dma_kernel<128x128>")])
-def test_matmul_with_gathered_rows_on_whole_tiles(tokens, kd, nd, experts, kernel):
+                                                         (128 * 300, 32, 128, 6, "gemm_dma_kernel<128x128>"),
+                                                         # enough K tiles for the wavefront that touches B's lines ahead of the others
+                                                         # (uneven numbers of row tiles per matrix: uneven shares of the lines); fewer K
+                                                         # tiles than matrix ids (the K walk starts at id % tiles); a ragged last column
+                                                         # tile; fp16
+                                                         (4096, 640, 2048, 8, "gemm_dma_kernel<128x256>"), (4096, 96, 2048, 8, "gemm_dma_kernel<128x256>"),
+                                                         (4096, 416, 2040, 7, "gemm_dma_kernel<128x256>"), (4224, 320, 2048, 3, "gemm_dma_kernel<128x256>", torch.float16)])
+def test_matmul_with_gathered_rows_on_whole_tiles(case):
+    tokens, kd, nd, experts, kernel = case[:5]
+    dtype = case[5] if len(case) > 5 else torch.bfloat16
     # whole 128-row tiles go to the direct-to-LDS kernel, which walks the row tiles in the order of their matrix ids (so
     # that the tiles of one matrix share an L2): ids dealt out of order, repeated and negative; exact as above
     import extra_kernels as X
     g = torch.Generator(device="cpu").manual_seed(tokens + nd)
-    a = torch.randint(-8, 9, (tokens + 77, kd), generator=g).bfloat16().to(DEV)
+    a = torch.randint(-8, 9, (tokens + 77, kd), generator=g).to(dtype).to(DEV)
     pick = torch.randint(0, kd, (experts, nd), generator=g)
-    b = torch.zeros(experts, kd, nd, dtype=torch.bfloat16)
+    b = torch.zeros(experts, kd, nd, dtype=dtype)
     for e in range(experts):
         b[e, pick[e], torch.arange(nd)] = -1.0
     b = b.to(DEV)
@@ -1639,11 +1647,11 @@ def test_matmul_with_gathered_rows_on_whole_tiles(tokens, kd, nd, experts, kerne
     ids = torch.randint(-1, experts, (tokens // 128,), generator=g, dtype=torch.int32)
     ids[0] = experts - 1
     ids = ids.to(DEV)
-    c = torch.full((tokens, nd), 5.0, device=DEV, dtype=torch.bfloat16)
-    k = X.grouped_rows_matmul[(tokens // 128, nd // 128)](a, b, c, rows, ids, tokens, kd, nd, kd, kd * nd, nd, nd, BM=128, BN=128, BK=64)
+    c = torch.full((tokens, nd), 5.0, device=DEV, dtype=dtype)
+    k = X.grouped_rows_matmul[(tokens // 128, triton.cdiv(nd, 128))](a, b, c, rows, ids, tokens, kd, nd, kd, kd * nd, nd, nd, BM=128, BN=128, BK=64)
     torch.cuda.synchronize()
     assert k.function.family == "gemm" and k.function.last_kernel == kernel
-    want = torch.full((tokens, nd), 5.0, device=DEV, dtype=torch.bfloat16)
+    want = torch.full((tokens, nd), 5.0, device=DEV, dtype=dtype)
     for blk, e in enumerate(ids.tolist()):
         r = slice(blk * 128, blk * 128 + 128)
         if e >= 0:

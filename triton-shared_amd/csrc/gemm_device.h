@@ -327,7 +327,10 @@ constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 15) | ((vm >> 4) << 1
 template <bool E> struct EdgeTile { static constexpr bool value = E; };
 // AT: A is column-major (p.a_trans: element (m, k) at a[m + k * lda]).  Its stage is laid out like a row-major B's,
 // [32 k rows][2 BM bytes], and read through the same transposing LDS read.
-template <bool BF16, int TM, int TN, class Ep, bool BT = false, bool AT = false>
+// PF: the workgroup has a fifth wavefront that fetches nothing into the stages; it touches lines of B some K tiles ahead
+// of the four that work (below).
+constexpr int F_PF_AHEAD = 8;
+template <bool BF16, int TM, int TN, class Ep, bool BT = false, bool AT = false, bool PF = false>
 __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, int tiles_n, const Ep &ep) {
   using T = DmaTile<TM, TN>;
   constexpr int BM = T::BM, BN = T::BN, STAGES = T::STAGES, A_BYTES = T::A_BYTES, STAGE_BYTES = T::STAGE_BYTES, ROWB = T::B_ROW_BYTES;
@@ -354,12 +357,13 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   const int gh = min(tiles_m - g0, 4);
   int tile_m = g0 + (bid % group) % gh;
   const int tile_n = (bid % group) / gh;
+  int pf_share = tile_m - g0, pf_shares = gh;  // PF: this workgroup's part of the B lines its column group reads
   if (GATHER && p.b_block && tiles_m <= 256) {
     // Row tiles that multiply the same matrix should sit behind one L2: the workgroup takes the row tile whose place in
     // the order by matrix id (ties by position) is the one the tile order above gave it.  With ids 0..7 dealt round-robin
     // to 32 blocks of 128 rows, every XCD otherwise streams four of the eight matrices (measured past L2: 319 MB per
     // launch for 100 MB of operands).
-    __shared__ int block_key[256], sorted_tile;
+    __shared__ int block_key[256], place_key[256], sorted_tile;
     if (tid < tiles_m) block_key[tid] = p.b_block[((int64_t)tid * BM) / p.b_block_rows];
     __syncthreads();
     if (tid < tiles_m) {
@@ -367,17 +371,73 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
       int place = 0;
       for (int o = 0; o < tiles_m; o++) place += (block_key[o] < mine || (block_key[o] == mine && o < tid)) ? 1 : 0;
       if (place == tile_m) sorted_tile = tid;
+      place_key[place] = mine;
     }
     __syncthreads();
+    if (PF) {  // the row tiles of this column group that multiply the same matrix split its lines between them
+      const int mine = place_key[tile_m];
+      pf_share = 0, pf_shares = 0;
+      for (int q = g0; q < g0 + gh; q++)
+        if (place_key[q] == mine) {
+          if (q < tile_m) pf_share++;
+          pf_shares++;
+        }
+    }
     tile_m = sorted_tile;
   }
   const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
 
   const char *b_base = (const char *)((const uint16_t *)p.b + (BT ? n0 * p.ldb : n0));
+  int which = 0;
   if (GATHER && p.b_block) {  // the rows of this tile multiply a matrix of their own; a negative id: nothing to do for them
-    const int which = p.b_block[m0 / p.b_block_rows];
+    which = p.b_block[m0 / p.b_block_rows];
     if (which < 0) return;
     b_base += 2 * ((p.gather_mul32 & 2) ? (int64_t)(int)((uint32_t)which * (uint32_t)p.b_block_stride) : (int64_t)which * p.b_block_stride);
+  }
+
+  const int nk = (int)(p.K / F_BK);
+  // Row tiles with matrices of their own walk K from different starting tiles (matrix id tiles in, wrapping round): the
+  // workgroups of a launch start together, and matrices that lie a power of two apart in memory would otherwise be read
+  // at the same offsets at the same time.  (The sum over K is taken in that order; 1.5 us of 45 on the measured case.)
+  const int k_first = (GATHER && p.b_block) ? (int)((uint32_t)which % (uint32_t)nk) : 0;
+  if (PF && wave == 4) {
+    // The working wavefronts' loads wait in the memory pipeline for as long as their lines take to arrive, and lines that
+    // come from HBM (several weight matrices: nothing of B is read twice out of the Infinity Cache) take long enough that
+    // more LDS stages do not help (five and six measured like four).  This wavefront asks for the lines first: a
+    // 4-byte load per 128-byte line of its share of the B tile F_PF_AHEAD tiles ahead, into a patch of LDS nobody reads (a
+    // load into a register would come back long after the compiler has given the register to something else).  It keeps
+    // step with the others through the same barriers.  Measured on 4096 gathered rows x [8, 2048, 2048]: 50.0 -> 43.8 us
+    // with operands from HBM; touching A's lines as well cost 1 us, touching every other line gained nothing.
+    static_assert(!PF || (!BT && !AT), "the prefetching wavefront walks a row-major B");
+    __shared__ int touched[64];
+    const uint32_t sink = (uint32_t)(uintptr_t)TTS_LDS(touched);
+    constexpr int LPR = ROWB / 128, LINES = F_BK * LPR;  // 128-byte lines per k row and per tile
+    const int per = (LINES + pf_shares - 1) / pf_shares;
+    const char *line_at[2];
+    bool on[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {  // at most 128 lines per tile
+      const int l = lane + 64 * h, line = pf_share * per + l;
+      on[h] = l < per && line < LINES && n0 + (line % LPR) * 64 < p.N;
+      line_at[h] = b_base + ((int64_t)(line / LPR) * p.ldb + (line % LPR) * 64) * 2;
+    }
+    auto touch = [&](int t) {
+      if (t >= nk) return;
+      t += k_first;
+      if (t >= nk) t -= nk;
+#pragma unroll
+      for (int h = 0; h < 2; h++)
+        if (on[h])
+          asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" : : "s"(sink), "v"(line_at[h] + (int64_t)t * F_BK * p.ldb * 2) : "memory", "m0");
+    };
+    for (int t = STAGES - 1; t < F_PF_AHEAD; t++) touch(t);
+    __syncthreads();  // the others' barrier after the prologue ...
+    for (int t = 0; t < nk; t++) {
+      touch(t + F_PF_AHEAD);
+      __syncthreads();  // ... and the one of every K tile
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));  // the patch of LDS goes away with the workgroup
+    return;
   }
 
   // Wavefront w issues A instructions A_DMA w .. (rows 16 ia + lane / 4) and B instructions B_DMA w .. (k rows
@@ -419,7 +479,6 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   const char *a_base = (const char *)((const uint16_t *)p.a + (AT ? m0 : m0 * p.lda));
   const uint32_t lds0 = (uint32_t)(uintptr_t)TTS_LDS(smem);
   const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
-  const int nk = (int)(p.K / F_BK);
   auto dma = [&](const char *sbase, uint32_t voff, uint32_t lds) {
 #ifdef TTS_GEMM_RTC
     // the run-time compiler may be an older one than the library's (a process that loaded PyTorch first gets PyTorch's
@@ -435,7 +494,8 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds), "v"(addr) : "memory", "m0");
   };
   auto dma_one = [&](int t, int n) {  // n < A_DMA: A part, else B part of tile t, into stage t % STAGES
-    const int tc = min(t, nk - 1);
+    int tc = min(t, nk - 1) + k_first;
+    if (tc >= nk) tc -= nk;
     const uint32_t st = lds0 + (t % STAGES) * STAGE_BYTES;
     if (n < A_DMA) {
       const uint32_t at = st + (A_DMA * wave_u + n) * 1024;

@@ -46,20 +46,27 @@ hipError_t launch_gemm_cfg(const GemmParams &p, hipStream_t s) {
 }
 
 
-template <bool BF16, int TM, int TN, bool BT, bool AT>
-__global__ __launch_bounds__(256) void gemm_dma_kernel(GemmParams p, int tiles_m, int tiles_n) {
-  gemm_dma_body<BF16, TM, TN, IdentityEp, BT, AT>(p, tiles_m, tiles_n, IdentityEp());
+// PF: a fifth wavefront that touches B's lines ahead of the four that work (gemm_device.h); the accumulators then sit in
+// the 256 registers two wavefronts of a SIMD can have each, which the 128 x 256 tile fits without spilling.
+template <bool BF16, int TM, int TN, bool BT, bool AT, bool PF>
+__global__ __launch_bounds__(PF ? 320 : 256) void gemm_dma_kernel(GemmParams p, int tiles_m, int tiles_n) {
+  gemm_dma_body<BF16, TM, TN, IdentityEp, BT, AT, PF>(p, tiles_m, tiles_n, IdentityEp());
 }
 
-template <bool BF16, int TM, int TN, bool BT, bool AT>
+template <bool BF16, int TM, int TN, bool BT, bool AT, bool PF = false>
 hipError_t launch_gemm_dma_t(const GemmParams &p, hipStream_t s) {
   using T = DmaTile<TM, TN>;
   constexpr size_t lds = T::LDS_BYTES;
-  auto kern = gemm_dma_kernel<BF16, TM, TN, BT, AT>;
+  // Row tiles with weight matrices of their own (p.b_block) stream B from HBM: they get the prefetching wavefront.
+  if constexpr (!PF && TM == 2 && TN == 4 && !BT && !AT) {
+    static const char *off = getenv("TTS_GEMM_PREFETCH");  // tuning aid: "0" = without
+    if (p.b_block && !(off && off[0] == '0')) return launch_gemm_dma_t<BF16, TM, TN, BT, AT, true>(p, s);
+  }
+  auto kern = gemm_dma_kernel<BF16, TM, TN, BT, AT, PF>;
   static const hipError_t attr = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return attr;
   int tiles_m = (int)((p.M + T::BM - 1) / T::BM), tiles_n = (int)((p.N + T::BN - 1) / T::BN);
-  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds, s, p, tiles_m, tiles_n);
+  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(PF ? 320 : 256), lds, s, p, tiles_m, tiles_n);
   return hipGetLastError();
 }
 
