@@ -203,7 +203,7 @@ def make_workloads(torch, triton, K):
             ids = (torch.arange(tokens // 128, device=dev) % experts).int()
             return lambda: K.expert_rows_matmul[(tokens // 128, nd // 128)](a, b, c, rows, ids, tokens, kd, nd, kd, kd * nd, nd, nd, BM=128, BN=128, BK=64)
         return dict(desc=f"mixture-of-experts product bf16: {tokens} rows gathered through an index vector, x [{experts}, {kd}, {nd}] weights picked by a "
-                         "loaded expert id per 128 rows (matmul family: the direct-to-LDS kernel takes the index vector and the id table)",
+                         "loaded expert id per 128 rows (matmul family: the direct-to-LDS kernel takes the index vector and the id table; a fifth wavefront touches B's lines ahead)",
                     work=2 * tokens * kd * nd, bound="mfma", dtype="bf16", make=make, set_bytes=(tokens * kd + experts * kd * nd + tokens * nd) * 2)
 
     def stream_copy(n):
