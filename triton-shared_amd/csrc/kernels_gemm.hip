@@ -59,8 +59,8 @@ hipError_t launch_gemm_dma_t(const GemmParams &p, hipStream_t s) {
   constexpr size_t lds = T::LDS_BYTES;
   // Row tiles with weight matrices of their own (p.b_block) stream B from HBM: they get the prefetching wavefront.
   if constexpr (!PF && TM == 2 && TN == 4 && !BT && !AT) {
-    static const char *off = getenv("TTS_GEMM_PREFETCH");  // tuning aid: "0" = without
-    if (p.b_block && !(off && off[0] == '0')) return launch_gemm_dma_t<BF16, TM, TN, BT, AT, true>(p, s);
+    static const char *pf = getenv("TTS_GEMM_PREFETCH");  // tuning aid: "0" = never, "2" = for every launch of this tile
+    if (pf ? pf[0] == '2' || (pf[0] != '0' && p.b_block) : p.b_block != nullptr) return launch_gemm_dma_t<BF16, TM, TN, BT, AT, true>(p, s);
   }
   auto kern = gemm_dma_kernel<BF16, TM, TN, BT, AT, PF>;
   static const hipError_t attr = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
