@@ -1093,3 +1093,21 @@ def attention_fwd(Q, K, V, O, sm_scale, seq, stride_h, stride_s, BM: tl.constexp
         m_i = m_new
     acc = acc / l_i[:, None]
     tl.store(O + ph * stride_h + rm[:, None] * stride_s + rd[None, :], acc.to(tl.float16), mask=rm[:, None] < seq)
+
+
+@triton.jit
+def narrow_scaled(x_ptr, y_ptr, n, scale, BLOCK: tl.constexpr):
+    # y = (x * scale) narrowed to y's element type: one elementwise pass
+    o = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    x = tl.load(x_ptr + o, mask=o < n, other=0.0)
+    tl.store(y_ptr + o, (x * scale).to(y_ptr.dtype.element_ty), mask=o < n)
+
+
+@triton.jit
+def narrow_scaled_with_row_max(x_ptr, y_ptr, m_ptr, n_cols, scale, BLOCK: tl.constexpr):
+    # the same narrowing next to a reduction (a row per program): the generic family
+    r = tl.program_id(0)
+    c = tl.arange(0, BLOCK)
+    x = tl.load(x_ptr + r * n_cols + c, mask=c < n_cols, other=0.0)
+    tl.store(m_ptr + r, tl.max(tl.abs(x), axis=0))
+    tl.store(y_ptr + r * n_cols + c, (x * scale).to(y_ptr.dtype.element_ty), mask=c < n_cols)

@@ -651,6 +651,39 @@ def test_vec_add_in_16_bit_floats(K, dtype):
     assert torch.equal(z[:n], x + y) and z[n:].abs().sum().item() == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_narrowing_rounds_to_nearest_even_in_both_generated_families(dtype):
+    """arith.truncf f32 -> bf16 / f16 rounds to nearest even (the reference lowers it to LLVM's fptrunc): ties, values a
+    bit above and below them, denormal results, overflow to infinity, signed zeros and NaNs, through an elementwise pass and
+    through a program with a reduction.  Every float32 whose low 16 bits are a tie or next to one, over all exponents."""
+    import extra_kernels as X
+    hi = torch.arange(0, 1 << 16, dtype=torch.int64)                         # every sign / exponent / high mantissa pattern
+    lows = torch.tensor([0x0000, 0x0001, 0x7FFF, 0x8000, 0x8001, 0xFFFF, 0x1000, 0x9000, 0x0FFF, 0xEFFF], dtype=torch.int64)
+    bits = ((hi[:, None] << 16) | lows[None, :]).reshape(-1)
+    x = torch.from_numpy(bits.numpy().astype("uint32").view("float32").copy())
+    n = x.numel()
+    want = x.to(dtype)
+    nan = torch.isnan(x)
+    xd = x.to(DEV)
+    y = torch.zeros(n + 8, dtype=dtype, device=DEV)
+    k = X.narrow_scaled[(triton.cdiv(n, 1024),)](xd, y, n, 1.0, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "fused_map"
+    got = y[:n].cpu()
+    assert torch.equal(got.view(torch.int16)[~nan], want.view(torch.int16)[~nan]) and torch.isnan(got[nan]).all()
+    assert y[n:].abs().sum().item() == 0
+    cols = 1000
+    rows = n // cols
+    y2 = torch.zeros(rows * cols, dtype=dtype, device=DEV)
+    m = torch.zeros(rows, device=DEV)
+    k = X.narrow_scaled_with_row_max[(rows,)](xd, y2, m, cols, 1.0, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    got = y2.cpu()
+    sel = ~nan[:rows * cols]
+    assert torch.equal(got.view(torch.int16)[sel], want[:rows * cols].view(torch.int16)[sel]) and torch.isnan(got[~sel]).all()
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.int32])
 def test_tile_program_load_after_store_sees_the_store(dtype):
     # the serial reference finishes the store before the next load of the same buffer starts

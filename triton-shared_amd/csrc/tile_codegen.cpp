@@ -1526,13 +1526,14 @@ struct Gen {
 const char *TILE_PRELUDE = R"SRC(
 struct Args { void *ptr[%N%]; long long ival[%N%]; double fval[%N%]; };
 __device__ inline float up_f16(unsigned short h) { _Float16 f; __builtin_memcpy(&f, &h, 2); return (float)f; }
-__device__ inline unsigned short down_f16(float f) { _Float16 h = (_Float16)f; unsigned short r; __builtin_memcpy(&r, &h, 2); return r; }
-__device__ inline float up_bf16(unsigned short h) { return __uint_as_float((unsigned)h << 16); }
+// The empty asm hides where f comes from: the compiler otherwise folds a multiplication into the narrowing (v_fma_mixlo_f16
+// with an addend of +0), which rounds once instead of twice and turns a product of -0 into +0.
+__device__ inline unsigned short down_f16(float f) { asm("" : "+v"(f)); _Float16 h = (_Float16)f; unsigned short r; __builtin_memcpy(&r, &h, 2); return r; }
+__device__ inline float up_bf16(unsigned short h) { __bf16 b; __builtin_memcpy(&b, &h, 2); return (float)b; }
+// the hardware conversion (v_cvt_pk_bf16_f32: round to nearest even); NaNs keep their sign and high payload bits
 __device__ inline unsigned short down_bf16(float f) {
-  unsigned u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1);
-  return (unsigned short)(u >> 16);
+  if (f != f) return (unsigned short)((__float_as_uint(f) >> 16) | 0x40);
+  __bf16 h = (__bf16)f; unsigned short r; __builtin_memcpy(&r, &h, 2); return r;
 }
 __device__ inline float maximum_f(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
 __device__ inline float minimum_f(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
