@@ -544,23 +544,26 @@ def test_gemm_with_column_major_a_and_with_strides_no_kernel_takes(K):
     assert relfro(c.float(), a.float() @ b2.float()) <= 1e-2
 
 
-@pytest.mark.parametrize("M", [17, 64])
-def test_w8a16_beyond_the_decode_shape(K, oracle_cpu, M):
-    # the reference's matmul lowering has no shape limit (ConversionPatterns.hpp:1128-1201); the decode kernels stop at
-    # 16 rows, more rows run on the generic family's kernel for the same program
+@pytest.mark.parametrize("M,N,Kd,BM,kernel", [(17, 384, 512, 16, "gemm_w8a16_kernel"), (64, 384, 512, 16, "gemm_w8a16_kernel"),
+                                             (40, 512, 1024, 16, "gemm_w8a16_wide_kernel"), (100, 1024, 2048, 64, "gemm_w8a16_wide_kernel"),
+                                             (33, 200, 100, 32, "gemm_w8a16_kernel")])
+def test_w8a16_beyond_the_decode_shape(K, oracle_cpu, M, N, Kd, BM, kernel):
+    # the reference's matmul lowering has no shape limit (ConversionPatterns.hpp:1128-1201); the decode kernels take 16
+    # rows, more rows run as one launch of them per group of 16 (the last group ragged), whatever the program's BM
     torch.manual_seed(M)
-    N, Kd = 384, 512
     a = torch.randn(M, Kd).half()
     w = torch.randint(-127, 128, (Kd, N), dtype=torch.int8)
     s = (0.001 + 0.009 * torch.rand(N)).half()
     ad, wd, sd = a.to(DEV), w.to(DEV), s.to(DEV)
-    cd = torch.full((M, N), 5.0, dtype=torch.float16, device=DEV)
-    k = K.w8a16_matmul[(triton.cdiv(M, 16), triton.cdiv(N, 128))](ad, wd, sd, cd, M, N, Kd, ad.stride(0), 1, wd.stride(0), 1,
-                                                                  cd.stride(0), 1, BM=16, BN=128, BK=128)
+    cd = torch.full((M + 3, N), 5.0, dtype=torch.float16, device=DEV)
+    for _ in range(2):   # twice: every launch leaves the split-K counters ready for the next
+        k = K.w8a16_matmul[(triton.cdiv(M, BM), triton.cdiv(N, 128))](ad, wd, sd, cd, M, N, Kd, ad.stride(0), 1, wd.stride(0), 1,
+                                                                      cd.stride(0), 1, BM=BM, BN=128, BK=128)
     torch.cuda.synchronize()
-    assert k.function.family == "gemm_w8a16" and k.function.last_kernel == "tile_program (hipRTC)"
-    assert relfro(cd.cpu(), oracle_cpu.w8a16_matmul(a, w, s)) <= 1e-2
-    assert relfro(cd.cpu(), a.double() @ (w.half() * s[None, :]).double()) <= 1e-2
+    assert k.function.family == "gemm_w8a16" and k.function.last_kernel == kernel
+    assert relfro(cd[:M].cpu(), oracle_cpu.w8a16_matmul(a, w, s)) <= 1e-2
+    assert relfro(cd[:M].cpu(), a.double() @ (w.half() * s[None, :]).double()) <= 1e-2
+    assert torch.equal(cd[M:].cpu(), torch.full((3, N), 5.0, dtype=torch.float16))
 
 
 @pytest.mark.parametrize("R,C,BR,BC", [(200, 300, 64, 64), (513, 130, 32, 128), (64, 64, 64, 64), (1000, 77, 128, 32)])

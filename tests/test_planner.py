@@ -281,8 +281,11 @@ def test_w8a16_binding(native):
     M, N, K = 13, 70, 100
     d = plan.describe_launch((1, 3, 1), [0, 0, 0, 0, M, N, K, K, N, N])
     assert (d["M"], d["N"], d["K"], d["lda"], d["ldw"], d["ldc"]) == ("13", "70", "100", "100", "70", "70")
-    d = plan.describe_launch((2, 3, 1), [0, 0, 0, 0, 20, N, K, K, N, N])   # beyond the decode shape: the generic family
-    assert d["kernel"] == "tile_program" and "M <= 16" in d["fallback_reason"]
+    d = plan.describe_launch((2, 3, 1), [0, 0, 0, 0, 20, N, K, K, N, N])   # beyond the decode shape: the same kernels, a launch per 16 rows
+    assert d["kernel"] == "gemm_w8a16" and d["M"] == "20"
+    # what the family can only decline at launch goes to the generic family's kernel: a pitch so large that BK * ldw wraps
+    d = plan.describe_launch((1, 3, 1), [0, 0, 0, 0, M, N, K, K, 2 ** 31 - 1, N])
+    assert d["kernel"] == "tile_program" and "fallback_reason" in d
 
 
 def test_index_overflow_is_detected(native):

@@ -782,7 +782,26 @@ size_t gemm_w8a16_workspace_bytes(const GemmW8A16Params &p) {
 
 size_t gemm_w8a16_counters(const GemmW8A16Params &p) { return p.split <= 1 ? 0 : (size_t)((p.N + 255) / 256); }
 
+static hipError_t launch_gemm_w8a16_rows(const GemmW8A16Params &p, hipStream_t s, const char **name);
+
+// More than 16 rows of A: the decode kernels once per group of 16 rows, one launch after the other on the stream (they
+// share the split-K workspace, which every launch leaves ready for the next).  W is read once per group, so this is
+// for the handful of rows beside the decode shape (M = 64 at [8192, 28672]: four passes over W, against 13 ms on the
+// generic family's kernel); a prefill-sized M wants the tiled matmul kernels on dequantised weights instead.
 hipError_t launch_gemm_w8a16(const GemmW8A16Params &p, hipStream_t s, const char **name) {
+  if (p.M <= 16) return launch_gemm_w8a16_rows(p, s, name);
+  for (int64_t m0 = 0; m0 < p.M; m0 += 16) {
+    GemmW8A16Params q = p;
+    q.M = std::min<int64_t>(16, p.M - m0);
+    q.a = (const uint16_t *)p.a + m0 * p.lda;
+    q.c = (uint16_t *)p.c + m0 * p.ldc;
+    hipError_t e = launch_gemm_w8a16_rows(q, s, name);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
+static hipError_t launch_gemm_w8a16_rows(const GemmW8A16Params &p, hipStream_t s, const char **name) {
   W8Config c = w8_config(p);
   const int steps = (int)((p.K + 31) / 32);
   const int sps = (steps + p.split - 1) / p.split;

@@ -416,7 +416,6 @@ void bind_gemm(const Resolver &r, Bound &b) {
 
 void bind_w8a16(const Resolver &r, Bound &b) {
   DenseGemm d = prove_dense_gemm(r, "gemm_w8a16");
-  if (d.M > 16) throw Unsupported("gemm_w8a16: only the decode shape M <= 16 is implemented");
   if (d.a_trans || d.b_trans) throw Unsupported("gemm_w8a16: only row-major operands are implemented");
   GemmW8A16Params &p = b.w8;
   p.M = d.M; p.N = d.N; p.K = d.K; p.lda = d.lda; p.ldw = d.ldb; p.ldc = d.ldc;
