@@ -356,10 +356,12 @@ def test_cfg5_w8a16(K, oracle_cpu):
         assert relfro(cd.cpu()[:, y * 128:(y + 1) * 128], part[:, y * 128:(y + 1) * 128]) <= 1e-2
 
 
-def test_w8a16_exact_selection(K):
-    # W picks and negates single rows, scales are powers of two: the result is exact in fp16
+@pytest.mark.parametrize("M", [16, 32, 41])
+def test_w8a16_exact_selection(K, M):
+    # W picks and negates single rows, scales are powers of two: the result is exact in fp16.  At the full size of the
+    # weight matrix: 16 rows (the decode shape), 32 (one launch with two groups of rows), 41 (two launches, the last ragged)
     torch.manual_seed(2)
-    M, N, Kd = 16, 28672, 8192
+    N, Kd = 28672, 8192
     a = torch.randn(M, Kd).half()
     cols = torch.arange(N)
     rows = (cols * 7) % Kd

@@ -436,7 +436,9 @@ __device__ __forceinline__ float4 load_through(float4 *src) {
 // arrival), writes C, and resets the counter for the next launch.  No workgroup waits for another.
 // The counters are zero between launches (whoever allocates them clears them once).  Launches
 // that share a workspace must not overlap.
-template <int NW, int DEPTH>
+// MT: groups of 16 rows of A a launch takes (1 or 2).  The weights are widened once per step and multiplied with every
+// group's rows; the tails below (the sum over the wavefronts, the hand-over between K slices, the stores) run once per group.
+template <int NW, int DEPTH, int MT>
 __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Params p, int first_steps, int other_steps) {
   extern __shared__ float4 w8_lds[];  // [NW][16][64]
   __shared__ int is_last;
@@ -463,15 +465,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
 #pragma unroll
     for (int c = 0; c < 16; c++) scale2[c] = (uint32_t)sv[c] | ((uint32_t)sv[c] << 16);
   }
-  f32x4 acc[16];
+  f32x4 acc[MT][16];
 #pragma unroll
-  for (int c = 0; c < 16; c++) acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int m = 0; m < MT; m++)
+#pragma unroll
+    for (int c = 0; c < 16; c++) acc[m][c] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
   // slice 0 takes first_steps steps of 32 rows, every other slice other_steps
   const int step_begin = slice == 0 ? 0 : first_steps + (slice - 1) * other_steps;
   const int step_end = min(step_begin + (slice == 0 ? first_steps : other_steps), (int)(p.K / 32));
   const int8_t *w_lane = p.w + (int64_t)(8 * g) * p.ldw + n0 + 16 * j;
-  const uint16_t *a_lane = (const uint16_t *)p.a + (int64_t)min(j, (int)p.M - 1) * p.lda + 8 * g;
+  const uint16_t *a_lane[MT];
+#pragma unroll
+  for (int m = 0; m < MT; m++) a_lane[m] = (const uint16_t *)p.a + (int64_t)min(16 * m + j, (int)p.M - 1) * p.lda + 8 * g;
 
   auto load_w = [&](int step, uint4 (&q)[8]) {
     const int8_t *src = w_lane + (int64_t)step * 32 * p.ldw;
@@ -484,9 +490,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
       q[t] = make_uint4(v[0], v[1], v[2], v[3]);
     }
   };
-  auto load_a = [&](int step) { return *reinterpret_cast<const uint4 *>(a_lane + step * 32); };
+  auto load_a = [&](int step, uint4 (&af)[MT]) {
+#pragma unroll
+    for (int m = 0; m < MT; m++) af[m] = *reinterpret_cast<const uint4 *>(a_lane[m] + step * 32);
+  };
   auto word = [](const uint4 &v, int i) -> uint32_t { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; };
-  auto consume = [&](const uint4 (&q)[8], const uint4 &af) {
+  auto consume = [&](const uint4 (&q)[8], const uint4 (&af)[MT]) {
 #pragma unroll
     for (int c = 0; c < 16; c++) {
       uint32_t frag[4];
@@ -498,44 +507,51 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
         frag[tp] = pk_sub_1152_mul(pair, scale2[c]);
       }
       uint4 bfrag = make_uint4(frag[0], frag[1], frag[2], frag[3]);
-      acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af), __builtin_bit_cast(f16x8, bfrag), acc[c], 0, 0, 0);
+#pragma unroll
+      for (int m = 0; m < MT; m++)
+        acc[m][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[m]), __builtin_bit_cast(f16x8, bfrag), acc[m][c], 0, 0, 0);
     }
   };
   uint4 q[DEPTH][8];
-  uint4 a[DEPTH];
+  uint4 a[DEPTH][MT];
   int step = step_begin + wave;
 #pragma unroll
   for (int d = 0; d < DEPTH; d++)
-    if (step + d * NW < step_end) { load_w(step + d * NW, q[d]); a[d] = load_a(step + d * NW); }
+    if (step + d * NW < step_end) { load_w(step + d * NW, q[d]); load_a(step + d * NW, a[d]); }
   for (; step < step_end; step += DEPTH * NW) {
 #pragma unroll
     for (int d = 0; d < DEPTH; d++) {
       if (step + d * NW < step_end) {
         consume(q[d], a[d]);
-        if (step + (d + DEPTH) * NW < step_end) { load_w(step + (d + DEPTH) * NW, q[d]); a[d] = load_a(step + (d + DEPTH) * NW); }
+        if (step + (d + DEPTH) * NW < step_end) { load_w(step + (d + DEPTH) * NW, q[d]); load_a(step + (d + DEPTH) * NW, a[d]); }
       }
     }
   }
 
-  // sum the wavefronts' tiles: entry (c, lane) is rows 4g..4g+3 of column n0 + 16j + c
-#pragma unroll
-  for (int c = 0; c < 16; c++) w8_lds[(wave * 16 + c) * 64 + lane] = __builtin_bit_cast(float4, acc[c]);
-  __syncthreads();
+  // sum the wavefronts' tiles: entry (c, lane) is rows 4g..4g+3 (of the group) of column n0 + 16j + c
   constexpr int PER = 1024 / (NW * 64);
-  float4 tot[PER];
+  float4 tot[MT][PER];
 #pragma unroll
-  for (int e = 0; e < PER; e++) {
-    const int idx = tid + e * NW * 64;
-    float4 t = w8_lds[idx];
+  for (int m = 0; m < MT; m++) {
+    if (m) __syncthreads();  // the previous group's tiles have been read
 #pragma unroll
-    for (int w = 1; w < NW; w++) {
-      float4 u = w8_lds[w * 1024 + idx];
-      t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+    for (int c = 0; c < 16; c++) w8_lds[(wave * 16 + c) * 64 + lane] = __builtin_bit_cast(float4, acc[m][c]);
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < PER; e++) {
+      const int idx = tid + e * NW * 64;
+      float4 t = w8_lds[idx];
+#pragma unroll
+      for (int w = 1; w < NW; w++) {
+        float4 u = w8_lds[w * 1024 + idx];
+        t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+      }
+      tot[m][e] = t;
     }
-    tot[e] = t;
   }
   if (p.split > 1) {
-    float4 *slots = reinterpret_cast<float4 *>(p.workspace) + (int64_t)slab * p.split * 1024;
+    // a slab's slots: [slice][group][1024 float4]
+    float4 *slots = reinterpret_cast<float4 *>(p.workspace) + (int64_t)slab * p.split * MT * 1024;
     int *counter = p.counters + slab;
     // tot = the slices' tiles added in slice order, whoever adds them (so the sum does not depend on who arrived when);
     // `self` is this workgroup's slice, whose tile is tot.  Up to four slices, every load is issued before the first add
@@ -543,37 +559,43 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
     auto add_slices = [&](int self) {
       constexpr int EAGER = 4;
       if (p.split <= EAGER) {
-        float4 u[EAGER][PER];
+        float4 u[EAGER][MT][PER];
 #pragma unroll
         for (int sl = 0; sl < EAGER; sl++)
           if (sl < p.split && sl != self) {
 #pragma unroll
-            for (int e = 0; e < PER; e++) u[sl][e] = load_through(slots + sl * 1024 + tid + e * NW * 64);
+            for (int m = 0; m < MT; m++)
+#pragma unroll
+              for (int e = 0; e < PER; e++) u[sl][m][e] = load_through(slots + (sl * MT + m) * 1024 + tid + e * NW * 64);
           }
 #pragma unroll
-        for (int e = 0; e < PER; e++) {
-          float4 t = self == 0 ? tot[e] : u[0][e];
+        for (int m = 0; m < MT; m++)
 #pragma unroll
-          for (int sl = 1; sl < EAGER; sl++)
-            if (sl < p.split) {
-              const float4 v = sl == self ? tot[e] : u[sl][e];
-              t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
-            }
-          tot[e] = t;
-        }
+          for (int e = 0; e < PER; e++) {
+            float4 t = self == 0 ? tot[m][e] : u[0][m][e];
+#pragma unroll
+            for (int sl = 1; sl < EAGER; sl++)
+              if (sl < p.split) {
+                const float4 v = sl == self ? tot[m][e] : u[sl][m][e];
+                t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+              }
+            tot[m][e] = t;
+          }
         return;
       }
 #pragma unroll
-      for (int e = 0; e < PER; e++) {
-        const int idx = tid + e * NW * 64;
-        float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int sl = 0; sl < p.split; sl++) {
-          float4 u = sl == self ? tot[e] : load_through(slots + sl * 1024 + idx);
-          if (sl == 0) t = u;
-          else { t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w; }
+      for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int e = 0; e < PER; e++) {
+          const int idx = tid + e * NW * 64;
+          float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+          for (int sl = 0; sl < p.split; sl++) {
+            float4 u = sl == self ? tot[m][e] : load_through(slots + (sl * MT + m) * 1024 + idx);
+            if (sl == 0) t = u;
+            else { t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w; }
+          }
+          tot[m][e] = t;
         }
-        tot[e] = t;
-      }
     };
     bool others_done = false;
     if (slice == 0) {
@@ -590,7 +612,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
       add_slices(0);
     } else {
 #pragma unroll
-    for (int e = 0; e < PER; e++) store_through(slots + slice * 1024 + tid + e * NW * 64, tot[e]);
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+      for (int e = 0; e < PER; e++) store_through(slots + (slice * MT + m) * 1024 + tid + e * NW * 64, tot[m][e]);
     __builtin_amdgcn_s_waitcnt(0);  // the stores have been acknowledged: the tile is in memory
     __syncthreads();                // ... every wavefront's part of it
     if (tid == 0) {
@@ -604,33 +628,36 @@ __global__ __launch_bounds__(NW * 64) void gemm_w8a16_wide_kernel(GemmW8A16Param
     }
   }
   // to row-major through LDS, then 16-byte stores of eight fp16 values
-  __syncthreads();
   constexpr int PITCH = W8_COLS_WIDE + 4;
   float *tile = reinterpret_cast<float *>(w8_lds);
-#pragma unroll
-  for (int e = 0; e < PER; e++) {
-    const int idx = tid + e * NW * 64;
-    const int c = idx >> 6, jj = idx & 15, gg = (idx >> 4) & 3;
-    float *dst = tile + (4 * gg) * PITCH + 16 * jj + c;
-    dst[0] = tot[e].x; dst[PITCH] = tot[e].y; dst[2 * PITCH] = tot[e].z; dst[3 * PITCH] = tot[e].w;
-  }
-  __syncthreads();
   uint16_t *__restrict__ C = (uint16_t *)p.c;
   const bool c_vec = (p.ldc % 8 == 0) && (((uintptr_t)C & 15) == 0);
-  for (int item = tid; item < 16 * (W8_COLS_WIDE / 8); item += NW * 64) {
-    const int m = item / (W8_COLS_WIDE / 8), n8 = (item % (W8_COLS_WIDE / 8)) * 8;
-    if (m >= p.M) continue;
-    const float *src = tile + m * PITCH + n8;
-    uint16_t h[8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) h[i] = f32_to_f16(src[i]);
-    uint16_t *dst = C + (int64_t)m * p.ldc + n0 + n8;
-    if (c_vec) {
-      *reinterpret_cast<uint4 *>(dst) = make_uint4(h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16,
-                                                   h[4] | (uint32_t)h[5] << 16, h[6] | (uint32_t)h[7] << 16);
-    } else {
+  for (int grp = 0; grp < MT; grp++) {
+    __syncthreads();
 #pragma unroll
-      for (int i = 0; i < 8; i++) dst[i] = h[i];
+    for (int e = 0; e < PER; e++) {
+      const int idx = tid + e * NW * 64;
+      const int c = idx >> 6, jj = idx & 15, gg = (idx >> 4) & 3;
+      float *dst = tile + (4 * gg) * PITCH + 16 * jj + c;
+      dst[0] = tot[grp][e].x; dst[PITCH] = tot[grp][e].y; dst[2 * PITCH] = tot[grp][e].z; dst[3 * PITCH] = tot[grp][e].w;
+    }
+    __syncthreads();
+    for (int item = tid; item < 16 * (W8_COLS_WIDE / 8); item += NW * 64) {
+      const int m = item / (W8_COLS_WIDE / 8), n8 = (item % (W8_COLS_WIDE / 8)) * 8;
+      if (16 * grp + m >= p.M) continue;
+      const float *src = tile + m * PITCH + n8;
+      uint16_t h[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) h[i] = f32_to_f16(src[i]);
+      uint16_t *dst = C + (int64_t)(16 * grp + m) * p.ldc + n0 + n8;
+      if (c_vec) {
+        *reinterpret_cast<uint4 *>(dst) = make_uint4(h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16,
+                                                     h[4] | (uint32_t)h[5] << 16, h[6] | (uint32_t)h[7] << 16);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) dst[i] = h[i];
+      }
     }
   }
 }
@@ -761,14 +788,14 @@ void w8_launch(const GemmW8A16Params &p, int steps_per_slice, hipStream_t s) {
   hipLaunchKernelGGL((gemm_w8a16_kernel<NW, DEPTH, FAST, 8>), grid, dim3(NW * 64), 0, s, p, steps_per_slice);
 }
 
-template <int NW, int DEPTH>
+template <int NW, int DEPTH, int MT = 1>
 hipError_t w8_launch_wide(const GemmW8A16Params &p, int first_steps, int other_steps, hipStream_t s) {
   constexpr size_t lds = (size_t)NW * 16 * 64 * sizeof(float4);
-  static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_w8a16_wide_kernel<NW, DEPTH>),
+  static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_w8a16_wide_kernel<NW, DEPTH, MT>),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return attr;
   dim3 grid((unsigned)(p.N / W8_COLS_WIDE), p.split);
-  hipLaunchKernelGGL((gemm_w8a16_wide_kernel<NW, DEPTH>), grid, dim3(NW * 64), lds, s, p, first_steps, other_steps);
+  hipLaunchKernelGGL((gemm_w8a16_wide_kernel<NW, DEPTH, MT>), grid, dim3(NW * 64), lds, s, p, first_steps, other_steps);
   return hipGetLastError();
 }
 }  // namespace
@@ -777,22 +804,27 @@ int gemm_w8a16_split(const GemmW8A16Params &p) { return w8_config(p).split; }
 
 size_t gemm_w8a16_workspace_bytes(const GemmW8A16Params &p) {
   if (p.split <= 1) return 0;
-  return (size_t)p.split * 16 * (size_t)((p.N + 255) / 256 * 256) * sizeof(float);  // per-slice partial tiles, 16 rows of fp32
+  // per-slice partial tiles: 16 rows of fp32, 32 when a launch takes two groups of rows
+  return (size_t)p.split * (p.M > 16 ? 32 : 16) * (size_t)((p.N + 255) / 256 * 256) * sizeof(float);
 }
 
 size_t gemm_w8a16_counters(const GemmW8A16Params &p) { return p.split <= 1 ? 0 : (size_t)((p.N + 255) / 256); }
 
 static hipError_t launch_gemm_w8a16_rows(const GemmW8A16Params &p, hipStream_t s, const char **name);
 
-// More than 16 rows of A: the decode kernels once per group of 16 rows, one launch after the other on the stream (they
-// share the split-K workspace, which every launch leaves ready for the next).  W is read once per group, so this is
-// for the handful of rows beside the decode shape (M = 64 at [8192, 28672]: four passes over W, against 13 ms on the
-// generic family's kernel); a prefill-sized M wants the tiled matmul kernels on dequantised weights instead.
+static bool w8_wide(const GemmW8A16Params &p);
+
+// More rows of A than a launch takes (32 on the 16-byte-load kernel, 16 on the other): the decode kernels once per
+// group of rows, one launch after the other on the stream (they share the split-K workspace, which every launch leaves
+// ready for the next).  W is read once per launch, so this is for the rows beside the decode shape (M = 64 at
+// [8192, 28672]: two passes over W, against 13 ms on the generic family's kernel); a prefill-sized M wants the tiled
+// matmul kernels on dequantised weights instead.
 hipError_t launch_gemm_w8a16(const GemmW8A16Params &p, hipStream_t s, const char **name) {
-  if (p.M <= 16) return launch_gemm_w8a16_rows(p, s, name);
-  for (int64_t m0 = 0; m0 < p.M; m0 += 16) {
+  const int64_t rows = w8_wide(p) ? 32 : 16;
+  if (p.M <= rows) return launch_gemm_w8a16_rows(p, s, name);
+  for (int64_t m0 = 0; m0 < p.M; m0 += rows) {
     GemmW8A16Params q = p;
-    q.M = std::min<int64_t>(16, p.M - m0);
+    q.M = std::min<int64_t>(rows, p.M - m0);
     q.a = (const uint16_t *)p.a + m0 * p.lda;
     q.c = (uint16_t *)p.c + m0 * p.ldc;
     hipError_t e = launch_gemm_w8a16_rows(q, s, name);
@@ -801,13 +833,17 @@ hipError_t launch_gemm_w8a16(const GemmW8A16Params &p, hipStream_t s, const char
   return hipSuccess;
 }
 
+static bool w8_fast(const GemmW8A16Params &p) {
+  return p.K % 32 == 0 && p.N % W8_COLS == 0 && p.lda % 8 == 0 && p.ldw % 8 == 0 && ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.w & 7) == 0;
+}
+static bool w8_wide(const GemmW8A16Params &p) { return w8_fast(p) && w8_config(p).cw == 16 && ((uintptr_t)p.w & 15) == 0; }
+
 static hipError_t launch_gemm_w8a16_rows(const GemmW8A16Params &p, hipStream_t s, const char **name) {
   W8Config c = w8_config(p);
   const int steps = (int)((p.K + 31) / 32);
   const int sps = (steps + p.split - 1) / p.split;
-  const bool fast = p.K % 32 == 0 && p.N % W8_COLS == 0 && p.lda % 8 == 0 && p.ldw % 8 == 0 &&
-                    ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.w & 7) == 0;
-  const bool wide = fast && c.cw == 16 && ((uintptr_t)p.w & 15) == 0;
+  const bool fast = w8_fast(p);
+  const bool wide = w8_wide(p);
   if (wide) {
     *name = "gemm_w8a16_wide_kernel";
     // slice 0 gets `bias` steps more than an even share (see the kernel's tail), taken evenly from the others
@@ -819,6 +855,7 @@ static hipError_t launch_gemm_w8a16_rows(const GemmW8A16Params &p, hipStream_t s
       if (sps - take >= 8 && sps * p.split == steps) { first = sps + take * (p.split - 1); other = sps - take; }
     }
     // one step in flight per wavefront; two measured 1.2 us slower at the decode shape
+    if (p.M > 16) return w8_launch_wide<8, 1, 2>(p, first, other, s);
     if (c.depth == 2) return w8_launch_wide<8, 2>(p, first, other, s);
     return w8_launch_wide<8, 1>(p, first, other, s);
   }
