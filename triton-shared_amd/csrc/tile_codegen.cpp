@@ -1012,9 +1012,9 @@ struct Gen {
     // operands of a 16-bit type are staged in that type (their values are exactly representable), others as fp32
     auto narrow = [](const std::string &t) { return t == "f16" || t == "bf16"; };
     const size_t a_size = narrow(A.dtype) ? 2 : 4, b_size = narrow(B.dtype) ? 2 : 4;
-    if (((size_t)(M * K) * a_size + 15) / 16 * 16 + (size_t)(K * N) * b_size > 48 * 1024)
+    if (((size_t)(M * K) * a_size + 15) / 16 * 16 + (size_t)(K * N) * b_size > 96 * 1024)
       no("a matrix product whose operands need " + std::to_string(((size_t)(M * K) * a_size + 15) / 16 * 16 + (size_t)(K * N) * b_size) +
-         " bytes of LDS (limit 49152)");
+         " bytes of LDS (limit 98304)");
     // The 16-bit matrix-core path reads 16-byte fragments of 32 consecutive rows at once: rows K elements apart would
     // fall into the same few banks (measured: more cycles of bank conflict than of anything else), so its rows are K + 8
     // elements apart when that still fits.
@@ -1023,7 +1023,7 @@ struct Gen {
     const size_t band_bytes = (size_t)32 * N * 4;
     const bool shaped = !(!is_float(A.dtype) && !is_float(B.dtype)) && M % 32 == 0 && N % 32 == 0 && ((both16 && K % 16 == 0) || (both32 && K % 2 == 0)) &&
                         band_bytes <= 32 * 1024;
-    const int64_t KP = (shaped && both16 && (size_t)(M + N) * (K + 8) * 2 + band_bytes <= 60 * 1024) ? K + 8 : K;  // row pitch of the staged operands
+    const int64_t KP = (shaped && both16 && (size_t)(M + N) * (K + 8) * 2 + band_bytes <= 112 * 1024) ? K + 8 : K;  // row pitch of the staged operands
     const size_t a_bytes = ((size_t)(M * KP) * a_size + 15) / 16 * 16, bytes = a_bytes + (size_t)(KP * N) * b_size;
     // integers (i8 x i8 -> i32 and the like): staged as 32-bit integers, multiplied and added with wrap-around
     const bool integer = !is_float(A.dtype) && !is_float(B.dtype) && !is_float(R.dtype);
@@ -1044,7 +1044,7 @@ struct Gen {
     close_loop();
     // for the 16-bit matrix-core path B is staged transposed ([N][K], K contiguous), so that a lane's eight consecutive k
     // of a column are one 16-byte LDS read, as they are for A
-    const bool mfma = !integer && shaped && bytes + band_bytes <= 60 * 1024;
+    const bool mfma = !integer && shaped && bytes + band_bytes <= 112 * 1024;
     open_element_loop(B.shape);
     if (mfma && both16)
       os << pad() << "db" << id << "[" << idx1(B.shape) << " * " << KP << " + " << idx0(B.shape) << "] = " << put(B.dtype, at(s.operands[1], idx0(B.shape), idx1(B.shape))) << ";\n";
