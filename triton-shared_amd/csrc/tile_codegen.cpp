@@ -745,14 +745,37 @@ struct Gen {
         decl << "  __shared__ " << ctype(val(o.result).dtype) << " " << name << "[" << elems << "];\n";
         out_bytes += (bytes + 15) / 16 * 16;
         staged[o.result] = {name, pitch};
-        open_element_loop(o.acc.sizes);
+        // Two loops, as for the run's own loads: every load is issued before the first loaded value is looked at.  (In
+        // one loop, `lds[i] = valid ? *p : other` waits for each load before the next goes out: the K block of a
+        // flash-attention step, 16 loads per thread, cost most of the step.)  16-bit floats travel as raw bits.
         {
-          std::string pred, addr = address(o.acc, idx0(o.acc.sizes), idx1(o.acc.sizes), pred);
-          os << pad() << staged_at(o.result, idx0(o.acc.sizes), idx1(o.acc.sizes)) << " = "
-             << (pred.empty() ? mem_read(o.acc, addr) : "(" + pred + ") ? " + mem_read(o.acc, addr) + " : " + other_of(o.acc, idx0(o.acc.sizes), idx1(o.acc.sizes)))
-             << ";\n";
+          const std::string &el = o.acc.elem;
+          const bool r16 = el == "f16" || el == "bf16";
+          const std::string ct = ctype(val(o.result).dtype);
+          const bool opaque = r16 || ct == "float" || ct == "int" || ct == "long long" || ct == "double";
+          const std::string tmp = "stg" + std::to_string(o.result);
+          const std::string i0s = idx0(o.acc.sizes), i1s = idx1(o.acc.sizes);
+          os << pad() << "{\n";
+          indent++;
+          os << pad() << (r16 ? std::string("unsigned") : ct) << " " << tmp << "[" << (count(o.acc.sizes) + 255) / 256 << "];\n";
+          open_element_loop(o.acc.sizes);
+          {
+            std::string pred, addr = address(o.acc, i0s, i1s, pred);
+            const std::string raw = r16 ? "((const unsigned short *)p.ptr[" + std::to_string(o.acc.base_arg) + "])[" + addr + "]" : mem_read(o.acc, addr);
+            os << pad() << (pred.empty() ? "" : "if (" + pred + ") ") << tmp << "[n] = " << raw << ";\n";
+          }
+          close_loop();
+          open_element_loop(o.acc.sizes);
+          {
+            std::string pred, addr = address(o.acc, i0s, i1s, pred);
+            if (opaque) os << pad() << "asm volatile(\"\" : \"+v\"(" << tmp << "[n]));\n";
+            const std::string got = r16 ? std::string(el == "f16" ? "up_f16(" : "up_bf16(") + "(unsigned short)" + tmp + "[n])" : tmp + "[n]";
+            os << pad() << staged_at(o.result, i0s, i1s) << " = " << (pred.empty() ? got : "(" + pred + ") ? " + got + " : " + other_of(o.acc, i0s, i1s)) << ";\n";
+          }
+          close_loop();
+          indent--;
+          os << pad() << "}\n";
         }
-        close_loop();
         os << pad() << "__syncthreads();\n";
       }
       if (two_phase) {
@@ -1059,9 +1082,45 @@ struct Gen {
     // 32x32x2 (fp32), and leave the band in LDS, from where every thread picks up the elements it owns.
     if (mfma) {
       const size_t band_off = (bytes + 15) / 16 * 16;
-      pool_bytes = std::max(pool_bytes, band_off + band_bytes);
       uses_mfma = true;
       os << pad() << "float *const dc" << id << " = (float *)(pool + " << band_off << ");\n";
+      // When the whole result fits next to the operands, the wavefronts take its 32 x 32 blocks in turn and meet once:
+      // two barriers instead of two per band, and no wavefront idles because a band has fewer than four column blocks
+      // (a [128, 64] x [64, 64] product of a flash-attention step: 4 bands of 2 blocks).
+      if (band_off + (size_t)M * N * 4 <= 112 * 1024) {
+        pool_bytes = std::max(pool_bytes, band_off + (size_t)M * N * 4);
+        os << pad() << "for (int blk = threadIdx.x >> 6; blk < " << (M / 32) * (N / 32) << "; blk += 4) {\n";
+        indent++;
+        os << pad() << "const int br = blk / " << N / 32 << ", bc = blk % " << N / 32 << ";\n";
+        os << pad() << "const int ln = threadIdx.x & 63, row = br * 32 + (ln & 31), col = bc * 32 + (ln & 31), kg = ln >> 5;\n";
+        os << pad() << "f32x16_t acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};\n";
+        if (both16) {
+          os << pad() << "for (int k0 = 0; k0 < " << K << "; k0 += 16) {\n";
+          indent++;
+          os << pad() << "const u16x8_t fa = *(const u16x8_t *)&da" << id << "[row * " << KP << " + k0 + 8 * kg], fb = *(const u16x8_t *)&db" << id << "[col * " << KP
+             << " + k0 + 8 * kg];\n";
+          os << pad() << "acc = " << (A.dtype == "bf16" ? "__builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fa), __builtin_bit_cast(bf16x8_t, fb)"
+                                                        : "__builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, fa), __builtin_bit_cast(f16x8_t, fb)")
+             << ", acc, 0, 0, 0);\n";
+          indent--;
+          os << pad() << "}\n";
+        } else {
+          os << pad() << "for (int k0 = 0; k0 < " << K << "; k0 += 2) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(da" << id << "[row * " << K << " + k0 + kg], db" << id
+             << "[(k0 + kg) * " << N << " + col], acc, 0, 0, 0);\n";
+        }
+        os << pad() << "#pragma unroll\n" << pad() << "for (int v = 0; v < 16; v++) dc" << id << "[(br * 32 + 8 * (v >> 2) + 4 * kg + (v & 3)) * " << N
+           << " + col] = acc[v];\n";
+        indent--;
+        os << pad() << "}\n" << pad() << "__syncthreads();\n";
+        open_element_loop(R.shape);
+        os << pad() << name << "[n] = " << rounded(R.dtype, "dc" + id + "[t] + " + at(s.operands.at(2), idx0(R.shape), idx1(R.shape))) << ";\n";
+        close_loop();
+        os << pad() << "__syncthreads();\n";
+        held[s.result] = {name, R.shape};
+        mine.push_back(s.result);
+        return;
+      }
+      pool_bytes = std::max(pool_bytes, band_off + band_bytes);
       // With few bands the band loop is unrolled, so that the slots of the result a thread fills from a band (N / 8 of
       // them, consecutive) are known at compile time and the result stays in registers.
       const bool unrolled_bands = M / 32 <= 8;
