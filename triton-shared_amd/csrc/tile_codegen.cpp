@@ -1476,7 +1476,11 @@ struct Gen {
       cur_i1.clear();
       return;
     }
-    // LDS: staging and partials in the shared pool, results in arrays of their own
+    // LDS: staging and partials in the shared pool, results in arrays of their own.  Rows that are reduced along their
+    // length are staged one element apart from a multiple of the bank count: the threads of a wavefront walk different
+    // rows at the same position, which would otherwise meet in one or two banks (rows of 64 floats: 32 threads per bank).
+    const int64_t PAD = (!scan && rank == 2 && s.axis == 1 && shape[1] % 2 == 0) ? 1 : 0;
+    const int64_t SOS = OS + PAD;  // staged pitch between lines
     std::vector<std::string> Tn(k);
     size_t off = 0;
     os << pad() << "__syncthreads();\n";
@@ -1484,7 +1488,7 @@ struct Gen {
       Tn[j] = ctype(val(s.operands[j]).dtype);
       const size_t sz = held_bytes(val(s.operands[j]).dtype);
       os << pad() << Tn[j] << " *const st" << id << "_" << j << " = (" << Tn[j] << " *)(pool + " << off << ");\n";
-      off = (off + T * sz + 15) / 16 * 16;
+      off = (off + (T + O * PAD) * sz + 15) / 16 * 16;
       os << pad() << Tn[j] << " *const pt" << id << "_" << j << " = (" << Tn[j] << " *)(pool + " << off << ");\n";
       off = (off + PS * sz + 15) / 16 * 16;
       const int64_t n_out = scan ? T : O;
@@ -1500,7 +1504,8 @@ struct Gen {
     const std::string S = "st" + id + "_", Pt = "pt" + id + "_", Out = "out" + id + "_";
     // stage
     open_element_loop(shape);
-    for (size_t j = 0; j < k; j++) os << pad() << S << j << "[t] = " << at(s.operands[j], i0, i1) << ";\n";
+    for (size_t j = 0; j < k; j++)
+      os << pad() << S << j << "[" << (PAD ? i0 + " * " + std::to_string(SOS) + " + " + i1 : std::string("t")) << "] = " << at(s.operands[j], i0, i1) << ";\n";
     close_loop();
     os << pad() << "__syncthreads();\n";
     auto final_value = [&](size_t j, const std::string &e) {  // a 16-bit sum is rounded once, here
@@ -1511,9 +1516,9 @@ struct Gen {
       os << pad() << "for (int q = threadIdx.x; q < " << PS << "; q += 256) {\n";
       indent++;
       os << pad() << "const int o = q / " << SEG << ", sg = q % " << SEG << ";\n";
-      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << " = " << S << j << "[o * " << OS << " + sg * " << LS << "];\n";
+      for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << " = " << S << j << "[o * " << SOS << " + sg * " << LS << "];\n";
       os << pad() << "for (int l = sg + " << SEG << "; l < " << L << "; l += " << SEG << ") " << fname << "(" << list("acc", "") << ", "
-         << list(S, "[o * " + std::to_string(OS) + " + l * " + std::to_string(LS) + "]") << ", " << list("acc", "") << ");\n";
+         << list(S, "[o * " + std::to_string(SOS) + " + l * " + std::to_string(LS) + "]") << ", " << list("acc", "") << ");\n";
       for (size_t j = 0; j < k; j++) {
         if (SEG == 1) os << pad() << Out << j << "[o] = " << final_value(j, "acc" + std::to_string(j)) << ";\n";
         else os << pad() << Pt << j << "[q] = acc" << j << ";\n";
