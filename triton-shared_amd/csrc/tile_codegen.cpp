@@ -55,12 +55,35 @@ struct Gen {
   // written, so that an access in a later iteration of a loop counts): a scalar store is one thread's, every read is
   // all threads', so the two are kept apart by barriers wherever they may touch the same argument.
   std::set<int> read_bases_anywhere, scalar_store_bases_anywhere;
+  std::map<int, int> uses;  // value id -> how many operands of the program name it
   void collect_bases(const std::vector<SOp> &ops) {
     for (const SOp &s : ops) {
       if (s.kind == SK::Load || s.kind == SK::ScalarLoad) read_bases_anywhere.insert(s.acc.base_arg);
       if (s.kind == SK::ScalarStore) scalar_store_bases_anywhere.insert(s.acc.base_arg);
+      for (int v : s.operands) uses[v]++;
+      for (int v : s.tile_inits) uses[v]++;
+      for (int v : s.tile_yields) uses[v]++;
+      for (int v : {s.acc.gather, s.acc.mask_value, s.acc.other_value})
+        if (v >= 0) uses[v]++;
       if (s.kind == SK::For || s.kind == SK::If) collect_bases(s.body);
     }
+  }
+  // Does computing v take a transcendental function, a division or a square root?  (Worth a register per element to a
+  // value that is used twice: every use of a value that has no register writes its whole expression out again.)
+  bool costly(int v, int depth = 0) {
+    auto d = def.find(v);
+    if (d == def.end() || depth > 24 || var.count(v) || held.count(v)) return false;
+    const SOp &o = *d->second;
+    if (o.kind == SK::Map) {
+      static const char *heavy[] = {"math.exp", "math.log", "math.sqrt", "math.rsqrt", "arith.divf", "math.erf", "math.tanh", "math.sin", "math.cos",
+                                    "math.pow", "tt.precise", "extern.", "arith.remf", "arith.divsi", "arith.divui", "arith.remsi", "arith.remui"};
+      for (const char *h : heavy)
+        if (o.name.rfind(h, 0) == 0) return true;
+    }
+    if (o.kind != SK::Map && o.kind != SK::Broadcast && o.kind != SK::ExpandDims && o.kind != SK::Splat) return false;
+    for (int x : o.operands)
+      if (costly(x, depth + 1)) return true;
+    return false;
   }
   std::ostringstream fns;                           // combiner functions of reductions and scans (before the kernel)
   std::ostringstream decl;                          // LDS arrays holding their results (top of the kernel)
@@ -663,6 +686,20 @@ struct Gen {
         if (shape.empty() || shape.size() > 4) no("a reduction over a block of rank " + std::to_string(shape.size()));
         if (s.kind == SK::Scan && shape.size() > 2) no("a scan over a block of rank " + std::to_string(shape.size()));
         if (s.kind == SK::Scan && count(shape) > TWO_PHASE_MAX) no("a scan over a block of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
+        // An operand that something else uses as well and that is costly to compute (the exponentials of a softmax: summed
+        // here, divided and stored later) gets registers now; otherwise both uses write its expression out.
+        if (count(shape) <= TWO_PHASE_MAX && shape.size() <= 2)
+          for (int o : s.operands) {
+            auto d = def.find(o);
+            if (d == def.end() || d->second->kind != SK::Map || val(o).shape != shape || held.count(o) || uses[o] < 2 || !costly(o)) continue;
+            const std::string name = "mv" + std::to_string(o);
+            os << pad() << ctype(val(o).dtype) << " " << name << "[" << (count(shape) + 255) / 256 << "];\n";
+            open_element_loop(shape);
+            os << pad() << name << "[n] = " << at(o, idx0(shape), idx1(shape)) << ";\n";
+            close_loop();
+            held[o] = {name, shape};
+            mine.push_back(o);
+          }
         reduce(s, shape);
         k++;
         continue;
