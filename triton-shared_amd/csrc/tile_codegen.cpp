@@ -203,6 +203,10 @@ struct Gen {
       const auto &sh = val(v).shape;
       if (sh.empty() || (i0 == cur_i0 && (sh.size() < 2 || i1 == cur_i1))) return it->second;
     }
+    {
+      auto lc = lds_copy.find(v);
+      if (lc != lds_copy.end()) return lc->second + "[" + linear(val(v).shape, i0, i1) + "]";
+    }
     auto d = def.find(v);
     if (d == def.end()) {
       auto mi = mirror.find(v);
@@ -557,6 +561,47 @@ struct Gen {
         for (int x : ops[q].operands) walk(x, 0);
     return found;
   }
+  // Costly vectors read through a broadcast: a value of one dimension (<= 4096 elements) that takes a transcendental
+  // function or a division and that a loop over a larger block reads at [row] for every element of the row (the
+  // exp(m_old - m_new) that rescales an attention accumulator) is computed once per element of its own, into LDS.
+  // value id -> array.  `roots` are the values the next phase evaluates.
+  std::map<int, std::string> lds_copy;
+  void hoist_costly_vectors(const std::vector<int> &roots, std::vector<int> &copies) {
+    std::vector<int> found;
+    std::function<void(int, bool, int)> walk = [&](int v, bool through_broadcast, int depth) {
+      auto d = def.find(v);
+      if (v < 0 || d == def.end() || depth > 24 || lds_copy.count(v)) return;
+      const SOp &o = *d->second;
+      const Value &V = val(v);
+      if (through_broadcast && o.kind == SK::Map && V.shape.size() == 1 && V.shape[0] > 1 && V.shape[0] <= 4096 && !held.count(v) && costly(v)) {
+        if (std::find(found.begin(), found.end(), v) == found.end()) found.push_back(v);
+        return;
+      }
+      if (o.kind == SK::Map) for (int x : o.operands) walk(x, through_broadcast, depth + 1);
+      else if (o.kind == SK::Broadcast || o.kind == SK::ExpandDims) for (int x : o.operands) walk(x, true, depth + 1);
+    };
+    for (int r : roots) walk(r, false, 0);
+    if (found.empty()) return;
+    os << pad() << "__syncthreads();\n";
+    for (int v : found) {
+      const Value &V = val(v);
+      const std::string name = "sv" + std::to_string(v);
+      if (!declared_copies.count(v)) {
+        decl << "  __shared__ " << ctype(V.dtype) << " " << name << "[" << V.shape[0] << "];\n";
+        out_bytes += ((size_t)V.shape[0] * held_bytes(V.dtype) + 15) / 16 * 16;
+        declared_copies.insert(v);
+      }
+      open_element_loop(V.shape);
+      os << pad() << name << "[t] = " << at(v, idx0(V.shape), idx1(V.shape)) << ";\n";
+      close_loop();
+    }
+    os << pad() << "__syncthreads();\n";
+    for (int v : found) {
+      lds_copy[v] = "sv" + std::to_string(v);
+      copies.push_back(v);
+    }
+  }
+  std::set<int> declared_copies;
   struct Held { std::string name; std::vector<int64_t> shape; };
   std::map<int, Held> held;
   // Loop-carried vectors that a loop also reads from blocks of another shape (the running maximum and sum of an online
@@ -599,6 +644,7 @@ struct Gen {
              s.kind == SK::Dot;
     };
     std::vector<int> mine;  // loads this body holds in registers
+    std::vector<int> copies;  // vectors this body keeps a copy of in LDS (hoist_costly_vectors)
     size_t k = 0;
     while (k < ops.size()) {
       const SOp &s = ops[k];
@@ -677,6 +723,7 @@ struct Gen {
         continue;
       }
       if (s.kind == SK::Dot) {
+        hoist_costly_vectors(s.operands, copies);
         dot(s, mine);
         k++;
         continue;
@@ -688,6 +735,7 @@ struct Gen {
         if (s.kind == SK::Scan && count(shape) > TWO_PHASE_MAX) no("a scan over a block of more than " + std::to_string(TWO_PHASE_MAX) + " elements");
         // An operand that something else uses as well and that is costly to compute (the exponentials of a softmax: summed
         // here, divided and stored later) gets registers now; otherwise both uses write its expression out.
+        hoist_costly_vectors(s.operands, copies);
         if (count(shape) <= TWO_PHASE_MAX && shape.size() <= 2)
           for (int o : s.operands) {
             auto d = def.find(o);
@@ -947,6 +995,7 @@ struct Gen {
         if (ops[q].result >= 0 && (ops[q].kind == SK::Map || (ops[q].kind == SK::Load && !held.count(ops[q].result)))) var.erase(ops[q].result);
       k = end;
     }
+    for (int v : copies) lds_copy.erase(v);
     if (defer) {
       defer->insert(defer->end(), mine.begin(), mine.end());
       return;
