@@ -53,6 +53,9 @@ __device__ inline float up_f16(unsigned short h) { _Float16 f; __builtin_memcpy(
 // The empty asm hides where f comes from: the compiler otherwise folds a multiplication into the narrowing (v_fma_mixlo_f16
 // with an addend of +0), which rounds once instead of twice and turns a product of -0 into +0.
 __device__ inline unsigned short down_f16(float f) { asm("" : "+v"(f)); _Float16 h = (_Float16)f; unsigned short r; __builtin_memcpy(&r, &h, 2); return r; }
+// for values that an fp16 holds exactly (whatever has the type f16 here): nothing to round, so nothing to hide, and the
+// compiler may cancel this against the widening before it
+__device__ inline unsigned short down_f16_exact(float f) { _Float16 h = (_Float16)f; unsigned short r; __builtin_memcpy(&r, &h, 2); return r; }
 __device__ inline float up_bf16(unsigned short h) { __bf16 b; __builtin_memcpy(&b, &h, 2); return (float)b; }
 // the hardware conversion (v_cvt_pk_bf16_f32: round to nearest even); NaNs keep their sign and high payload bits
 __device__ inline unsigned short down_bf16(float f) {
@@ -85,7 +88,7 @@ template <bool BF16>
 __device__ inline void store_h(void *base, int i, int valid, const float (&v)[W]) {
   unsigned short *p = (unsigned short *)base + i;
   hw w;
-  for (int e = 0; e < W; e++) w[e] = BF16 ? down_bf16(v[e]) : down_f16(v[e]);
+  for (int e = 0; e < W; e++) w[e] = BF16 ? down_bf16(v[e]) : down_f16_exact(v[e]);  // (stored values have been rounded to the type already)
   if (valid >= W && (((unsigned long long)p) & (2 * W - 1)) == 0) { __builtin_nontemporal_store(w, (hw *)p); return; }
   for (int e = 0; e < W && e < valid; e++) p[e] = w[e];
 }

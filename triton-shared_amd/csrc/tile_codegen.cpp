@@ -524,7 +524,7 @@ struct Gen {
   }
   void mem_write(const Access &a, const std::string &addr, const std::string &pred, const std::string &value) {
     std::string v = value;
-    if (a.elem == "f16") v = "down_f16(" + v + ")";
+    if (a.elem == "f16") v = "down_f16_exact(" + v + ")";  // (a value of type f16 is held as the float it equals)
     if (a.elem == "bf16") v = "down_bf16(" + v + ")";
     os << pad() << (pred.empty() ? "" : "if (" + pred + ") ") << "((" << memtype(a.elem) << " *)p.ptr[" << a.base_arg << "])[" << addr
        << "] = " << v << ";\n";
@@ -1154,7 +1154,7 @@ struct Gen {
     pool_bytes = std::max(pool_bytes, bytes);
     const std::string id = std::to_string(s.result);
     auto staged_type = [&](const std::string &t) { return integer ? std::string("int") : narrow(t) ? std::string("unsigned short") : std::string("float"); };
-    auto put = [&](const std::string &t, const std::string &e) { return t == "f16" ? "down_f16(" + e + ")" : t == "bf16" ? "down_bf16(" + e + ")" : e; };
+    auto put = [&](const std::string &t, const std::string &e) { return t == "f16" ? "down_f16_exact(" + e + ")" : t == "bf16" ? "down_bf16(" + e + ")" : e; };
     auto get = [&](const std::string &t, const std::string &e) { return t == "f16" ? "up_f16(" + e + ")" : t == "bf16" ? "up_bf16(" + e + ")" : e; };
     os << pad() << "__syncthreads();\n";
     os << pad() << staged_type(A.dtype) << " *const da" << id << " = (" << staged_type(A.dtype) << " *)pool;\n";
@@ -1691,6 +1691,9 @@ __device__ inline float up_f16(unsigned short h) { _Float16 f; __builtin_memcpy(
 // The empty asm hides where f comes from: the compiler otherwise folds a multiplication into the narrowing (v_fma_mixlo_f16
 // with an addend of +0), which rounds once instead of twice and turns a product of -0 into +0.
 __device__ inline unsigned short down_f16(float f) { asm("" : "+v"(f)); _Float16 h = (_Float16)f; unsigned short r; __builtin_memcpy(&r, &h, 2); return r; }
+// for values that an fp16 holds exactly (whatever has the type f16 here): nothing to round, so nothing to hide, and the
+// compiler may cancel this against the widening before it
+__device__ inline unsigned short down_f16_exact(float f) { _Float16 h = (_Float16)f; unsigned short r; __builtin_memcpy(&r, &h, 2); return r; }
 __device__ inline float up_bf16(unsigned short h) { __bf16 b; __builtin_memcpy(&b, &h, 2); return (float)b; }
 // the hardware conversion (v_cvt_pk_bf16_f32: round to nearest even); NaNs keep their sign and high payload bits
 __device__ inline unsigned short down_bf16(float f) {
