@@ -253,6 +253,8 @@ def test_gemm_whole_tile_kernel(K, M, N, Kd, dtype, pad):
                                                                    c.stride(0), 1, BM=128, BN=128, BK=64, GROUP_M=8)
     torch.cuda.synchronize()
     want_kernel = {(4096, 2048): "gemm_dma_kernel<128x256>", (4096, 2176): "gemm_dma_kernel<256x128>", (4096, 4096): "gemm_dma_kernel"}.get((M, N), "gemm_dma_kernel<128x128>")
+    if (M, N, Kd) == (256, 256, 4096):
+        want_kernel += ", K slices"     # four tiles and a long K: cut into slices (test_gemm_in_k_slices_for_skinny_products)
     assert k.function.last_kernel == want_kernel
     assert relfro(c.cpu(), a.cpu().double() @ b.cpu().double()) <= 1e-2
     assert torch.equal(Cfull[:, N:].cpu(), torch.full((M, pad), 5.0, dtype=dtype))
@@ -265,6 +267,40 @@ def test_gemm_whole_tile_kernel(K, M, N, Kd, dtype, pad):
                                                                c.stride(0), 1, BM=128, BN=128, BK=64, GROUP_M=8)
     torch.cuda.synchronize()
     assert torch.equal(c.cpu(), -a.cpu()[:, perm])
+
+
+@pytest.mark.parametrize("M,N,Kd,dtype,bt", [(128, 4096, 4096, torch.bfloat16, False), (300, 1032, 2048, torch.float16, False), (512, 2048, 8192, torch.bfloat16, True),
+                                            (1000, 2048, 4096, torch.bfloat16, False), (64, 8192, 8192, torch.float16, False), (1, 256, 4096, torch.bfloat16, False)])
+def test_gemm_in_k_slices_for_skinny_products(K, M, N, Kd, dtype, bt):
+    """Products with too few output tiles for the chip run with K cut into slices (a workgroup per tile and slice, fp32
+    partial sums, a second kernel that adds them and narrows): exact on small-integer operands whatever the order of
+    the sums, ragged rows and columns, a column-major B, the buffer around C untouched; twice on one stream (the second
+    launch reuses the workspace) and once more on another stream (a workspace of its own)."""
+    g = torch.Generator(device="cpu").manual_seed(M + N + Kd)
+    pad = 8
+    A = torch.randint(-3, 4, (M, Kd), generator=g).to(dtype).to(DEV)
+    Bm = torch.randint(-2, 3, (N + pad, Kd) if bt else (Kd, N + pad), generator=g).to(dtype).to(DEV)
+    b = Bm[:N].t() if bt else Bm[:, :N]
+    Cfull = torch.full((M + 3, N + pad), 5.0, dtype=dtype, device=DEV)
+    c = Cfull[:M, :N]
+    grid = (triton.cdiv(M, 128) * triton.cdiv(N, 128),)
+    want = A.float() @ b.float()          # |sums| stay far below 2^11 * max: exact in fp32, and in 16 bits when small enough
+    exact = want.abs().max().item() <= (256 if dtype == torch.bfloat16 else 2048)
+    def launch():
+        return K.matmul_tiles[grid](A, b, c, M, N, Kd, A.stride(0), 1, b.stride(0), b.stride(1), c.stride(0), 1, BM=128, BN=128, BK=64, GROUP_M=8)
+    for _ in range(2):
+        k = launch()
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and k.function.last_kernel.endswith("K slices"), k.function.last_kernel
+    assert torch.equal(c.float(), want.to(dtype).float()) if exact else relfro(c.float(), want) <= 1e-2
+    assert torch.equal(Cfull[:, N:].cpu(), torch.full((M + 3, pad), 5.0, dtype=dtype)) and torch.equal(Cfull[M:].cpu(), torch.full((3, N + pad), 5.0, dtype=dtype))
+    c.fill_(7.0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch()
+    side.synchronize()
+    assert torch.equal(c.float(), want.to(dtype).float()) if exact else relfro(c.float(), want) <= 1e-2
 
 
 @pytest.mark.parametrize("M,N,Kd,dtype,kernel", [(4000, 2048, 96, torch.bfloat16, "gemm_dma_kernel<128x256>"), (1000, 1032, 64, torch.float16, "gemm_dma_kernel<128x128>"),

@@ -33,6 +33,10 @@ struct TtsGemmParams {
   int b_block_rows;
   int gather_mul32;       // bit 0: a_rows[m] * lda, bit 1: id * b_block_stride is a 32-bit product that wraps, as the source computes it
   int is_f32;             // fp32 operands and result (kernels_gemm.hip: gemm_f32_kernel); is_bf16 is then 0
+  // K in `split` slices, one workgroup per (tile, slice), for products with too few tiles to occupy the chip: slice s
+  // leaves its fp32 sums at partial[s * M * N + m * N + n], and a second kernel adds the slices and narrows (1 = none)
+  int split;
+  float *partial;
 };
 
 namespace tts_gemm_device {
@@ -330,7 +334,9 @@ template <bool E> struct EdgeTile { static constexpr bool value = E; };
 // PF: the workgroup has a fifth wavefront that fetches nothing into the stages; it touches lines of B some K tiles ahead
 // of the four that work (below).
 constexpr int F_PF_AHEAD = 8;
-template <bool BF16, int TM, int TN, class Ep, bool BT = false, bool AT = false, bool PF = false>
+// SK: the grid holds p.split workgroups per tile; workgroup (tile, s) walks the s-th share of the K tiles and leaves its sums
+// in p.partial.
+template <bool BF16, int TM, int TN, class Ep, bool BT = false, bool AT = false, bool PF = false, bool SK = false>
 __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, int tiles_n, const Ep &ep) {
   using T = DmaTile<TM, TN>;
   constexpr int BM = T::BM, BN = T::BN, STAGES = T::STAGES, A_BYTES = T::A_BYTES, STAGE_BYTES = T::STAGE_BYTES, ROWB = T::B_ROW_BYTES;
@@ -351,6 +357,8 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
 
   int bid = blockIdx.x;
   const int nwg = tiles_m * tiles_n;
+  const int slice = SK ? bid / nwg : 0;
+  if (SK) bid -= slice * nwg;
   if (nwg % 8 == 0) bid = (bid % 8) * (nwg / 8) + bid / 8;  // consecutive ids on one XCD
   const int group = 4 * tiles_n;                             // 4-tile-tall column groups
   const int g0 = (bid / group) * 4;
@@ -395,7 +403,9 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
     b_base += 2 * ((p.gather_mul32 & 2) ? (int64_t)(int)((uint32_t)which * (uint32_t)p.b_block_stride) : (int64_t)which * p.b_block_stride);
   }
 
-  const int nk = (int)(p.K / F_BK);
+  const int nk_all = (int)(p.K / F_BK);
+  const int k_begin = SK ? (int)((int64_t)slice * nk_all / p.split) : 0;
+  const int nk = SK ? (int)((int64_t)(slice + 1) * nk_all / p.split) - k_begin : nk_all;
   // Row tiles with matrices of their own walk K from different starting tiles (matrix id tiles in, wrapping round): the
   // workgroups of a launch start together, and matrices that lie a power of two apart in memory would otherwise be read
   // at the same offsets at the same time.  (The sum over K is taken in that order; 1.5 us of 45 on the measured case.)
@@ -496,6 +506,7 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   auto dma_one = [&](int t, int n) {  // n < A_DMA: A part, else B part of tile t, into stage t % STAGES
     int tc = min(t, nk - 1) + k_first;
     if (tc >= nk) tc -= nk;
+    tc += k_begin;
     const uint32_t st = lds0 + (t % STAGES) * STAGE_BYTES;
     if (n < A_DMA) {
       const uint32_t at = st + (A_DMA * wave_u + n) * 1024;
@@ -596,6 +607,22 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   // are narrowed at once (v_cvt_pk_bf16_f32 for bf16: round to nearest even, NaNs quieted), the pair is exchanged with
   // the neighbouring lane, and the even lane stores row r at columns (n, n+1), the odd lane row r+1 at (n-1, n):
   // half as many store instructions as one 2-byte store per element, and a handful of VALU ops per pair.
+  if constexpr (SK) {
+    // the slice's sums as they are: a lane's 32 x 32 block column by column, two rows of 32 consecutive floats per store
+    float *__restrict__ part = p.partial + (int64_t)slice * p.M * p.N;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const int64_t col = n0 + wn * TN * 32 + j * 32 + (lane & 31);
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const int64_t row = m0 + wm * TM * 32 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+          if (row < p.M && col < p.N) part[row * p.N + col] = acc[i][j][v];
+        }
+      }
+    return;
+  }
   uint16_t *__restrict__ C = (uint16_t *)p.c;
   typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
   typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));

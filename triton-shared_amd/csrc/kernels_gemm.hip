@@ -48,21 +48,56 @@ hipError_t launch_gemm_cfg(const GemmParams &p, hipStream_t s) {
 
 // PF: a fifth wavefront that touches B's lines ahead of the four that work (gemm_device.h); the accumulators then sit in
 // the 256 registers two wavefronts of a SIMD can have each, which the 128 x 256 tile fits without spilling.
-template <bool BF16, int TM, int TN, bool BT, bool AT, bool PF>
+template <bool BF16, int TM, int TN, bool BT, bool AT, bool PF, bool SK>
 __global__ __launch_bounds__(PF ? 320 : 256) void gemm_dma_kernel(GemmParams p, int tiles_m, int tiles_n) {
-  gemm_dma_body<BF16, TM, TN, IdentityEp, BT, AT, PF>(p, tiles_m, tiles_n, IdentityEp());
+  gemm_dma_body<BF16, TM, TN, IdentityEp, BT, AT, PF, SK>(p, tiles_m, tiles_n, IdentityEp());
+}
+
+// Adds the K slices' partial sums in slice order and narrows: four columns per thread (N is a multiple of 8).
+template <bool BF16>
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmParams p) {
+  const int64_t quads = p.N / 4, idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= p.M * quads) return;
+  const int64_t m = idx / quads, n = (idx % quads) * 4;
+  const float4 *src = reinterpret_cast<const float4 *>(p.partial + m * p.N + n);
+  float4 t = src[0];
+  for (int sl = 1; sl < p.split; sl++) {
+    const float4 u = src[(int64_t)sl * p.M * quads];
+    t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+  }
+  typedef float f32x4_t __attribute__((ext_vector_type(4)));
+  typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+  typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+  const f32x4_t v = {t.x, t.y, t.z, t.w};
+  uint16_t *dst = (uint16_t *)p.c + m * p.ldc + n;
+  const uint2 w = BF16 ? __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t)) : __builtin_bit_cast(uint2, __builtin_convertvector(v, f16x4_t));
+  reinterpret_cast<uint32_t *>(dst)[0] = w.x;  // (rows of C are 4-byte aligned: gemm_dma_ok)
+  reinterpret_cast<uint32_t *>(dst)[1] = w.y;
 }
 
 template <bool BF16, int TM, int TN, bool BT, bool AT, bool PF = false>
 hipError_t launch_gemm_dma_t(const GemmParams &p, hipStream_t s) {
   using T = DmaTile<TM, TN>;
   constexpr size_t lds = T::LDS_BYTES;
+  if constexpr (!PF) {
+    if (p.split > 1) {
+      auto kern = gemm_dma_kernel<BF16, TM, TN, BT, AT, false, true>;
+      static const hipError_t attr = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (attr != hipSuccess) return attr;
+      int tiles_m = (int)((p.M + T::BM - 1) / T::BM), tiles_n = (int)((p.N + T::BN - 1) / T::BN);
+      hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n * p.split), dim3(256), lds, s, p, tiles_m, tiles_n);
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) return e;
+      hipLaunchKernelGGL(gemm_splitk_reduce_kernel<BF16>, dim3((unsigned)((p.M * (p.N / 4) + 255) / 256)), dim3(256), 0, s, p);
+      return hipGetLastError();
+    }
+  }
   // Row tiles with weight matrices of their own (p.b_block) stream B from HBM: they get the prefetching wavefront.
   if constexpr (!PF && TM == 2 && TN == 4 && !BT && !AT) {
     static const char *pf = getenv("TTS_GEMM_PREFETCH");  // tuning aid: "0" = never, "2" = for every launch of this tile
     if (pf ? pf[0] == '2' || (pf[0] != '0' && p.b_block) : p.b_block != nullptr) return launch_gemm_dma_t<BF16, TM, TN, BT, AT, true>(p, s);
   }
-  auto kern = gemm_dma_kernel<BF16, TM, TN, BT, AT, PF>;
+  auto kern = gemm_dma_kernel<BF16, TM, TN, BT, AT, PF, false>;
   static const hipError_t attr = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return attr;
   int tiles_m = (int)((p.M + T::BM - 1) / T::BM), tiles_n = (int)((p.N + T::BN - 1) / T::BN);
@@ -675,6 +710,75 @@ constexpr int W8_WAVES = 16;
 
 }  // namespace
 
+namespace {
+// Which direct-to-LDS tile a product runs on (null: none applies), and in how many K slices.
+struct DmaCand { const char *tag; int64_t bm, bn; double eff; };
+const DmaCand DMA_CANDS[4] = {{"256x256", 256, 256, 1.0}, {"128x256", 128, 256, 0.77}, {"256x128", 256, 128, 0.73}, {"128x128", 128, 128, 0.59}};
+struct DmaChoice { const DmaCand *tile = nullptr; int split = 1; };
+
+DmaChoice choose_dma(const GemmParams &p, bool allow_split) {
+  static const char *dma_env = getenv("TTS_GEMM_DMA");      // tuning aid: "256x256", "128x256", "256x128", "128x128" or unset
+  static const char *split_env = getenv("TTS_GEMM_SPLIT");  // tuning aid: the number of K slices (1 = never split)
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    return n;
+  }();
+  auto tiles = [&](const DmaCand &c) { return ((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn); };
+  // Among the tiles that give every CU a workgroup (128 x 128: always), the one with the least padded work per unit
+  // of the tile's measured efficiency at 4096^3 (105 / 136 / 144 / 179 us): a ragged edge counts against a tile that
+  // overshoots it by more.
+  DmaChoice best;
+  double best_cost = 0;
+  for (const DmaCand &c : DMA_CANDS) {
+    if (!gemm_dma_ok(p, c.bm, c.bn)) continue;
+    if (dma_env ? std::string(dma_env) != c.tag : (tiles(c) < cus && c.bm + c.bn != 256)) continue;
+    const double cost = (double)(tiles(c) * c.bm * c.bn) / c.eff;
+    if (!best.tile || cost < best_cost) { best.tile = &c; best_cost = cost; }
+  }
+  if (!best.tile || !allow_split || p.a_rows || p.b_block) return best;
+  // Too few tiles for the chip (a skinny product: M = 128 ... 1024 against N, K in the thousands): every workgroup then walks
+  // all of K alone, at the pace one workgroup streams its operands, and the launch takes as long as with a fraction of
+  // its rows -- 4096 x 4096 weights took 50 us at M = 128, 256, 512 and 1024 alike.  K is cut into slices so that about
+  // every CU has a workgroup; each slice leaves fp32 sums that a second kernel adds.  Modelled time: the K tiles a
+  // workgroup walks at the tile's measured time per K tile (times the rounds of workgroups the chip needs), the launch's
+  // fixed cost, and the partial sums' way through memory (measured: 512 x 8192 x 8192 in four slices of 256 x 256 tiles
+  // 79 us for a model of 82; 512 x 4096 x 4096 in four of 128 x 256 34.5 for 34.5; 128 x 4096 x 4096 in eight of
+  // 128 x 128 20.9 for 22.3).
+  const int64_t nk = p.K / F_BK;
+  auto model = [&](const DmaCand &c, int split) {
+    // per K tile and workgroup with operands from HBM (the 128 x 256 tile: 0.42 us from cache)
+    const double step = c.bm + c.bn == 512 ? 0.80e-6 : c.bm + c.bn == 256 ? 0.39e-6 : c.bm == 128 ? 0.60e-6 : 0.62e-6;
+    const double wgs = (double)tiles(c) * split;
+    double t = std::max(1.0, wgs / cus) * (double)((nk + split - 1) / split) * step + 8e-6;
+    if (split > 1) t += 1.2 * split * (double)p.M * (double)p.N * 4 / 4e12 + 3e-6;
+    return t;
+  };
+  DmaChoice pick = best;
+  double pick_t = model(*best.tile, 1);
+  if (!(split_env && atoi(split_env) == 1))
+    for (const DmaCand &c : DMA_CANDS) {
+      if (!gemm_dma_ok(p, c.bm, c.bn) || (dma_env && std::string(dma_env) != c.tag)) continue;
+      const int64_t most = std::min<int64_t>(std::min<int64_t>(16, nk / 8), (2 * cus + tiles(c) - 1) / tiles(c));
+      for (int64_t sp = split_env ? atoi(split_env) : 2; sp <= most; sp++) {
+        if ((size_t)sp * p.M * p.N * 4 > ((size_t)256 << 20)) break;
+        const double t = model(c, (int)sp);
+        if (t < 0.9 * pick_t || (pick.split > 1 && t < pick_t)) { pick.tile = &c; pick.split = (int)sp; pick_t = t; }
+        if (split_env) break;
+      }
+    }
+  return pick;
+}
+}  // namespace
+
+int gemm_split(const GemmParams &p) {
+  static const char *tile_env = getenv("TTS_GEMM_TILE");
+  if (p.is_f32 || tile_env) return 1;
+  return choose_dma(p, true).split;
+}
+size_t gemm_workspace_bytes(const GemmParams &p) { return p.split > 1 ? (size_t)p.split * p.M * p.N * sizeof(float) : 0; }
+
+// p.split is what gemm_split(p) said (the caller provides p.partial for it), or 1.
 hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
   if (p.is_f32) {
     if (p.a_rows || p.b_block) return hipErrorInvalidValue;  // (the matcher takes gathered rows on 16-bit operands only)
@@ -682,37 +786,20 @@ hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
     return launch_gemm_f32(p, s);
   }
   static const char *tile_env = getenv("TTS_GEMM_TILE");  // tuning aid: set = the any-shape kernel even for whole tiles
-  static const char *dma_env = getenv("TTS_GEMM_DMA");    // tuning aid: "256x256", "128x256", "256x128", "128x128" or unset
   if (!tile_env) {
     // Whole K tiles go to the direct-to-LDS kernels.
-    static const int cus = [] {
-      int dev = 0, n = 0;
-      if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-      return n;
-    }();
-    auto tiles = [&](int64_t bm, int64_t bn) { return ((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn); };
-    // Among the tiles that give every CU a workgroup (128 x 128: always), the one with the least padded work per unit
-    // of the tile's measured efficiency at 4096^3 (105 / 136 / 144 / 179 us): a ragged edge counts against a tile that
-    // overshoots it by more.
-    struct Cand { const char *tag; int64_t bm, bn, enough; double eff; };
-    static const Cand cands[4] = {{"256x256", 256, 256, cus, 1.0}, {"128x256", 128, 256, cus, 0.77}, {"256x128", 256, 128, cus, 0.73}, {"128x128", 128, 128, 1, 0.59}};
-    const Cand *best = nullptr;
-    double best_cost = 0;
-    for (const Cand &c : cands) {
-      if (!gemm_dma_ok(p, c.bm, c.bn)) continue;
-      if (dma_env ? std::string(dma_env) != c.tag : tiles(c.bm, c.bn) < c.enough) continue;
-      const double cost = (double)(tiles(c.bm, c.bn) * c.bm * c.bn) / c.eff;
-      if (!best || cost < best_cost) { best = &c; best_cost = cost; }
-    }
+    const DmaChoice choice = choose_dma(p, p.split > 1);  // (a caller without a workspace: the tile as without slices)
+    if (p.split > 1 && choice.split != p.split) return hipErrorInvalidValue;  // gemm_split and this launch disagree
+    const DmaCand *best = choice.tile;
 #define TTS_DMA(TM, TN, TAG)                                                                                  \
   do {                                                                                                        \
     *name = TAG;                                                                                              \
     return p.is_bf16 ? launch_gemm_dma<true, TM, TN>(p, s) : launch_gemm_dma<false, TM, TN>(p, s);            \
   } while (0)
-    if (best && best->bm == 256 && best->bn == 256) TTS_DMA(4, 4, "gemm_dma_kernel");
-    if (best && best->bm == 128 && best->bn == 256) TTS_DMA(2, 4, "gemm_dma_kernel<128x256>");
-    if (best && best->bm == 256 && best->bn == 128) TTS_DMA(4, 2, "gemm_dma_kernel<256x128>");
-    if (best) TTS_DMA(2, 2, "gemm_dma_kernel<128x128>");
+    if (best && best->bm == 256 && best->bn == 256) TTS_DMA(4, 4, p.split > 1 ? "gemm_dma_kernel, K slices" : "gemm_dma_kernel");
+    if (best && best->bm == 128 && best->bn == 256) TTS_DMA(2, 4, p.split > 1 ? "gemm_dma_kernel<128x256>, K slices" : "gemm_dma_kernel<128x256>");
+    if (best && best->bm == 256 && best->bn == 128) TTS_DMA(4, 2, p.split > 1 ? "gemm_dma_kernel<256x128>, K slices" : "gemm_dma_kernel<256x128>");
+    if (best) TTS_DMA(2, 2, p.split > 1 ? "gemm_dma_kernel<128x128>, K slices" : "gemm_dma_kernel<128x128>");
 #undef TTS_DMA
   }
   // anything else: 128 x 128 x 64 tiles, two workgroups per CU (a 256 x 256 x 32 form of the same kernel measured behind it

@@ -719,7 +719,34 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
           p.a_rows = ptr_arg<const int>(args, pl, "rows_arg");
           p.b_block = ptr_arg<const int>(args, pl, "block_arg");
         }
+        p.split = 1;
+        p.partial = nullptr;
         if (pl.source.empty()) {
+          // a product with too few tiles for the chip runs in K slices, whose partial sums need memory: the stream's
+          // workspace (as for the int8-weight product), or the static array of the call that may not allocate, when
+          // they fit there (else that call runs the product without slices)
+          const int want = gemm_split(p);
+          if (want > 1) {
+            p.split = want;
+            const size_t need = gemm_workspace_bytes(p);
+            if (no_alloc) {
+              if (need <= NOALLOC_WORKSPACE_BYTES) p.partial = reinterpret_cast<float *>(noalloc_scratch());
+              else p.split = 1;
+            } else {
+              std::lock_guard<std::mutex> lock(plan->mu);
+              tts_plan::SplitK &sk = plan->split_k[stream];
+              if (sk.workspace_bytes < need) {
+                // the stream's earlier launches may still be using the old buffer: hipFree waits for the device
+                if (sk.workspace) (void)hipFree(sk.workspace);
+                sk.workspace = nullptr;
+                sk.workspace_bytes = 0;
+                hipError_t e = hipMalloc((void **)&sk.workspace, need);
+                if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(split-K workspace): ") + hipGetErrorString(e));
+                sk.workspace_bytes = need;
+              }
+              p.partial = sk.workspace;
+            }
+          }
           err = launch_gemm(p, s, &kname);
           break;
         }
