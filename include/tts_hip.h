@@ -83,10 +83,12 @@ tts_status tts_launch(tts_plan *plan, int grid_x, int grid_y, int grid_z, void *
 /* tts_launch for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as tts_launch, but
  * the call never allocates or frees device memory and never compiles: the split-K partial tiles and arrival counters
- * of the int8-weight product live in a static device array (8 MiB + 4096 counters per GPU, held until the process
- * ends; its address is looked up with hipGetSymbolAddress at the first call on each device).  A launch whose partial
- * tiles exceed that, or that would need a run-time compiled kernel or a device-side table that no earlier tts_launch
- * of the plan has created yet, returns TTS_UNSUPPORTED with the reason.  All calls on one GPU share the array:
+ * of the int8-weight product, and the partial sums of a matrix product that runs in K slices, live in a static device
+ * array (8 MiB + 4096 counters per GPU, held until the process ends; its address is looked up with
+ * hipGetSymbolAddress at the first call on each device).  An int8-weight launch whose partial tiles exceed that, or
+ * a launch that would need a run-time compiled kernel or a device-side table that no earlier tts_launch of the plan
+ * has created yet, returns TTS_UNSUPPORTED with the reason; a matrix product whose slices would not fit runs without
+ * slices.  All calls on one GPU share the array:
  * calls that overlap in time on one GPU (two streams, two threads) race on it. */
 tts_status tts_launch_noalloc(tts_plan *plan, int grid_x, int grid_y, int grid_z, void *stream, const tts_arg *args,
                               int num_args);
