@@ -87,8 +87,8 @@ tts_status tts_launch(tts_plan *plan, int grid_x, int grid_y, int grid_z, void *
  * array (8 MiB + 4096 counters per GPU, held until the process ends; its address is looked up with
  * hipGetSymbolAddress at the first call on each device).  An int8-weight launch whose partial tiles exceed that, or
  * a launch that would need a run-time compiled kernel or a device-side table that no earlier tts_launch of the plan
- * has created yet, returns TTS_UNSUPPORTED with the reason; a matrix product whose slices would not fit runs without
- * slices.  All calls on one GPU share the array:
+ * has created yet, returns TTS_UNSUPPORTED with the reason; a matrix product runs in as many slices as fit there, or
+ * without slices.  All calls on one GPU share the array:
  * calls that overlap in time on one GPU (two streams, two threads) race on it. */
 tts_status tts_launch_noalloc(tts_plan *plan, int grid_x, int grid_y, int grid_z, void *stream, const tts_arg *args,
                               int num_args);

@@ -70,3 +70,33 @@ def test_noalloc_launch_refuses_a_plan_that_still_has_to_compile(native):
     plan.launch_noalloc((4, 1, 1), stream, vals)  # now there is nothing left to allocate
     torch.cuda.synchronize()
     assert torch.equal(y, want) and want.abs().sum().item() > 0
+
+
+def test_noalloc_launch_runs_a_skinny_matmul_in_k_slices_from_the_static_array(native):
+    # a matrix product with too few output tiles for the chip runs in K slices, whose fp32 partial sums tts_launch keeps in
+    # the stream's workspace and tts_launch_noalloc in the static array, in as many slices as fit there (8 MiB: eight
+    # slices of 128 x 2048); with the same number of slices the results agree bit for bit, both adding them in slice order.
+    # A product of which not even two slices fit (1024 x 2048) runs without slices in the call that may not allocate,
+    # which changes the order of the sums: within the tolerance of the family
+    plan, _ = plan_for(native, "matmul_tiles")
+    assert plan.family == "gemm"
+    stream = torch.cuda.current_stream().cuda_stream
+    for seed, (M, N, Kd, fits) in enumerate([(128, 2048, 8192, True), (64, 1024, 4096, True), (1000, 2048, 4096, False)]):
+        torch.manual_seed(seed)
+        a = (torch.randn(M, Kd) * 0.1).bfloat16().to(DEV)
+        b = (torch.randn(Kd, N) * 0.1).bfloat16().to(DEV)
+        want = torch.full((M, N), 5.0, dtype=torch.bfloat16, device=DEV)
+        got = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+        grid = (((M + 127) // 128) * ((N + 127) // 128), 1, 1)
+        plan.launch(grid, stream, [a.data_ptr(), b.data_ptr(), want.data_ptr(), M, N, Kd, Kd, N, N])
+        torch.cuda.synchronize()
+        assert plan.last_kernel.endswith("K slices"), plan.last_kernel
+        free_before = torch.cuda.mem_get_info()[0]
+        plan.launch_noalloc(grid, stream, [a.data_ptr(), b.data_ptr(), got.data_ptr(), M, N, Kd, Kd, N, N])
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] >= free_before
+        assert plan.last_kernel.endswith("K slices") == fits, plan.last_kernel
+        ref = a.double() @ b.double()
+        assert ((got.double() - ref).norm() / ref.norm()).item() <= 1e-2
+        if fits and M * N * 4 * 16 <= (8 << 20):   # (at most 16 slices are ever taken: then both calls took the same number)
+            assert torch.equal(got, want), (M, N, Kd)

@@ -91,7 +91,7 @@ hipError_t launch_layernorm(const LayerNormParams &p, int gx, int gy, int gz, hi
 
 // C[M,N] = A[M,K] * B[K,N], 16-bit inputs, fp32 accumulate, 16-bit output (RTNE)
 using GemmParams = ::TtsGemmParams;  // gemm_device.h
-// p.split = gemm_split(p) K slices (1: none) with p.partial = gemm_workspace_bytes(p) bytes of device memory for them
+// p.split = at most gemm_split(p) K slices (1: none) with p.partial = gemm_workspace_bytes(p) bytes of device memory for them
 int gemm_split(const GemmParams &p);
 size_t gemm_workspace_bytes(const GemmParams &p);
 hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **kernel_name);

@@ -716,7 +716,7 @@ struct DmaCand { const char *tag; int64_t bm, bn; double eff; };
 const DmaCand DMA_CANDS[4] = {{"256x256", 256, 256, 1.0}, {"128x256", 128, 256, 0.77}, {"256x128", 256, 128, 0.73}, {"128x128", 128, 128, 0.59}};
 struct DmaChoice { const DmaCand *tile = nullptr; int split = 1; };
 
-DmaChoice choose_dma(const GemmParams &p, bool allow_split) {
+DmaChoice choose_dma(const GemmParams &p, int max_split) {
   static const char *dma_env = getenv("TTS_GEMM_DMA");      // tuning aid: "256x256", "128x256", "256x128", "128x128" or unset
   static const char *split_env = getenv("TTS_GEMM_SPLIT");  // tuning aid: the number of K slices (1 = never split)
   static const int cus = [] {
@@ -736,7 +736,7 @@ DmaChoice choose_dma(const GemmParams &p, bool allow_split) {
     const double cost = (double)(tiles(c) * c.bm * c.bn) / c.eff;
     if (!best.tile || cost < best_cost) { best.tile = &c; best_cost = cost; }
   }
-  if (!best.tile || !allow_split || p.a_rows || p.b_block) return best;
+  if (!best.tile || max_split < 2 || p.a_rows || p.b_block) return best;
   // Too few tiles for the chip (a skinny product: M = 128 ... 1024 against N, K in the thousands): every workgroup then walks
   // all of K alone, at the pace one workgroup streams its operands, and the launch takes as long as with a fraction of
   // its rows -- 4096 x 4096 weights took 50 us at M = 128, 256, 512 and 1024 alike.  K is cut into slices so that about
@@ -759,7 +759,7 @@ DmaChoice choose_dma(const GemmParams &p, bool allow_split) {
   if (!(split_env && atoi(split_env) == 1))
     for (const DmaCand &c : DMA_CANDS) {
       if (!gemm_dma_ok(p, c.bm, c.bn) || (dma_env && std::string(dma_env) != c.tag)) continue;
-      const int64_t most = std::min<int64_t>(std::min<int64_t>(16, nk / 8), (2 * cus + tiles(c) - 1) / tiles(c));
+      const int64_t most = std::min<int64_t>(std::min<int64_t>(std::min<int64_t>(16, max_split), nk / 8), (2 * cus + tiles(c) - 1) / tiles(c));
       for (int64_t sp = split_env ? atoi(split_env) : 2; sp <= most; sp++) {
         if ((size_t)sp * p.M * p.N * 4 > ((size_t)256 << 20)) break;
         const double t = model(c, (int)sp);
@@ -774,11 +774,11 @@ DmaChoice choose_dma(const GemmParams &p, bool allow_split) {
 int gemm_split(const GemmParams &p) {
   static const char *tile_env = getenv("TTS_GEMM_TILE");
   if (p.is_f32 || tile_env) return 1;
-  return choose_dma(p, true).split;
+  return choose_dma(p, 16).split;
 }
 size_t gemm_workspace_bytes(const GemmParams &p) { return p.split > 1 ? (size_t)p.split * p.M * p.N * sizeof(float) : 0; }
 
-// p.split is what gemm_split(p) said (the caller provides p.partial for it), or 1.
+// p.split: the most K slices p.partial has room for (what gemm_split(p) said, or fewer; 1: none).
 hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
   if (p.is_f32) {
     if (p.a_rows || p.b_block) return hipErrorInvalidValue;  // (the matcher takes gathered rows on 16-bit operands only)
@@ -788,18 +788,20 @@ hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {
   static const char *tile_env = getenv("TTS_GEMM_TILE");  // tuning aid: set = the any-shape kernel even for whole tiles
   if (!tile_env) {
     // Whole K tiles go to the direct-to-LDS kernels.
-    const DmaChoice choice = choose_dma(p, p.split > 1);  // (a caller without a workspace: the tile as without slices)
-    if (p.split > 1 && choice.split != p.split) return hipErrorInvalidValue;  // gemm_split and this launch disagree
+    // at most p.split slices: what gemm_split said, or fewer when the caller's workspace holds no more (1: none)
+    const DmaChoice choice = choose_dma(p, std::max(1, p.split));
+    GemmParams q = p;
+    q.split = choice.split;
     const DmaCand *best = choice.tile;
 #define TTS_DMA(TM, TN, TAG)                                                                                  \
   do {                                                                                                        \
     *name = TAG;                                                                                              \
-    return p.is_bf16 ? launch_gemm_dma<true, TM, TN>(p, s) : launch_gemm_dma<false, TM, TN>(p, s);            \
+    return q.is_bf16 ? launch_gemm_dma<true, TM, TN>(q, s) : launch_gemm_dma<false, TM, TN>(q, s);            \
   } while (0)
-    if (best && best->bm == 256 && best->bn == 256) TTS_DMA(4, 4, p.split > 1 ? "gemm_dma_kernel, K slices" : "gemm_dma_kernel");
-    if (best && best->bm == 128 && best->bn == 256) TTS_DMA(2, 4, p.split > 1 ? "gemm_dma_kernel<128x256>, K slices" : "gemm_dma_kernel<128x256>");
-    if (best && best->bm == 256 && best->bn == 128) TTS_DMA(4, 2, p.split > 1 ? "gemm_dma_kernel<256x128>, K slices" : "gemm_dma_kernel<256x128>");
-    if (best) TTS_DMA(2, 2, p.split > 1 ? "gemm_dma_kernel<128x128>, K slices" : "gemm_dma_kernel<128x128>");
+    if (best && best->bm == 256 && best->bn == 256) TTS_DMA(4, 4, q.split > 1 ? "gemm_dma_kernel, K slices" : "gemm_dma_kernel");
+    if (best && best->bm == 128 && best->bn == 256) TTS_DMA(2, 4, q.split > 1 ? "gemm_dma_kernel<128x256>, K slices" : "gemm_dma_kernel<128x256>");
+    if (best && best->bm == 256 && best->bn == 128) TTS_DMA(4, 2, q.split > 1 ? "gemm_dma_kernel<256x128>, K slices" : "gemm_dma_kernel<256x128>");
+    if (best) TTS_DMA(2, 2, q.split > 1 ? "gemm_dma_kernel<128x128>, K slices" : "gemm_dma_kernel<128x128>");
 #undef TTS_DMA
   }
   // anything else: 128 x 128 x 64 tiles, two workgroups per CU (a 256 x 256 x 32 form of the same kernel measured behind it

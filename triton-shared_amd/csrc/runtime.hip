@@ -729,8 +729,10 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
           if (want > 1) {
             p.split = want;
             const size_t need = gemm_workspace_bytes(p);
-            if (no_alloc) {
-              if (need <= NOALLOC_WORKSPACE_BYTES) p.partial = reinterpret_cast<float *>(noalloc_scratch());
+            if (no_alloc) {  // as many slices as the static array holds
+              const size_t one = (size_t)p.M * p.N * sizeof(float);
+              p.split = (int)std::min<size_t>((size_t)want, NOALLOC_WORKSPACE_BYTES / one);
+              if (p.split > 1) p.partial = reinterpret_cast<float *>(noalloc_scratch());
               else p.split = 1;
             } else {
               std::lock_guard<std::mutex> lock(plan->mu);
