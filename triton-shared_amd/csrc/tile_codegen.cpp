@@ -614,8 +614,22 @@ struct Gen {
       else var.erase(h.first);
     }
   }
-  static std::string idx0(const std::vector<int64_t> &shape) { return shape.size() >= 2 ? "(t / " + std::to_string(shape.back()) + ")" : "t"; }
-  static std::string idx1(const std::vector<int64_t> &shape) { return shape.size() >= 2 ? "(t % " + std::to_string(shape.back()) + ")" : "0"; }
+  // Row and column of element t of a block.  Every loop that names t names n as well, with t = threadIdx.x + 256 n; with
+  // rows of a multiple of 256 elements the row depends on n alone, which is a constant once the loop is unrolled (or the
+  // same in every thread where it is not): written that way, the row's address arithmetic (row * pitch in 64 bits, per
+  // element and access: quarter-rate multiplies) is the scalar unit's or the compiler's, not every lane's.
+  static std::string idx0(const std::vector<int64_t> &shape) {
+    if (shape.size() < 2) return "t";
+    const int64_t C = shape.back();
+    if (C % 256 == 0) return C == 256 ? "n" : "(n / " + std::to_string(C / 256) + ")";
+    return "(t / " + std::to_string(C) + ")";
+  }
+  static std::string idx1(const std::vector<int64_t> &shape) {
+    if (shape.size() < 2) return "0";
+    const int64_t C = shape.back();
+    if (C % 256 == 0) return C == 256 ? "(int)threadIdx.x" : "((int)threadIdx.x + 256 * (n % " + std::to_string(C / 256) + "))";
+    return "(t % " + std::to_string(C) + ")";
+  }
   std::string cur_i0, cur_i1;  // the index expressions of the element loop being written
   void open_element_loop(const std::vector<int64_t> &shape) {
     const int64_t T = count(shape);
@@ -957,7 +971,7 @@ struct Gen {
           if (reads_held) {
             open_element_loop(shape);
           } else {
-            os << pad() << "for (int t = threadIdx.x; t < " << T << "; t += 256) {\n";
+            os << pad() << "for (int n = 0, t = threadIdx.x; t < " << T << "; t += 256, n++) {\n";
             indent++;
             map_vars({-1});
             cur_i0 = i0;
