@@ -1111,3 +1111,15 @@ def narrow_scaled_with_row_max(x_ptr, y_ptr, m_ptr, n_cols, scale, BLOCK: tl.con
     x = tl.load(x_ptr + r * n_cols + c, mask=c < n_cols, other=0.0)
     tl.store(m_ptr + r, tl.max(tl.abs(x), axis=0))
     tl.store(y_ptr + r * n_cols + c, (x * scale).to(y_ptr.dtype.element_ty), mask=c < n_cols)
+
+
+@triton.jit
+def stamp_tiles(out_ptr, R, C, BR: tl.constexpr, BC: tl.constexpr):
+    # every element gets its program's ids and the grid's extents: rows on program_id(0), columns on program_id(1)
+    p0 = tl.program_id(0)
+    p1 = tl.program_id(1)
+    r = p0 * BR + tl.arange(0, BR)
+    c = p1 * BC + tl.arange(0, BC)
+    v = p0 * 100 + p1 + 10000 * tl.num_programs(0) + 1000000 * tl.num_programs(1)
+    tile = tl.zeros((BR, BC), dtype=tl.int32) + v
+    tl.store(out_ptr + r[:, None] * C + c[None, :], tile, mask=(r[:, None] < R) & (c[None, :] < C))

@@ -604,6 +604,23 @@ def test_w8a16_beyond_the_decode_shape(K, oracle_cpu, M, N, Kd, BM, kernel):
     assert torch.equal(cd[M:].cpu(), torch.full((3, N), 5.0, dtype=torch.float16))
 
 
+@pytest.mark.parametrize("R,C,BR,BC", [(150, 700, 32, 256), (64, 64, 32, 32), (33, 1000, 8, 128), (40, 300, 16, 64)])
+def test_programs_keep_their_ids_when_the_launcher_swaps_the_grid(R, C, BR, BC):
+    # a program whose stores are contiguous along the dimension program_id(1) walks is launched with the grid's x and y
+    # exchanged (neighbouring workgroups then write neighbouring columns); program_id and num_programs must not notice
+    import extra_kernels as X
+    import numpy as np
+    out = torch.full((R + 1, C), -1, dtype=torch.int32, device=DEV)
+    g0, g1 = triton.cdiv(R, BR), triton.cdiv(C, BC)
+    k = X.stamp_tiles[(g0, g1)](out, R, C, BR=BR, BC=BC)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    rows, cols = np.arange(R)[:, None] // BR, np.arange(C)[None, :] // BC
+    want = rows * 100 + cols + 10000 * g0 + 1000000 * g1
+    assert np.array_equal(out[:R].cpu().numpy(), want)
+    assert bool((out[R] == -1).all())
+
+
 @pytest.mark.parametrize("R,C,BR,BC", [(200, 300, 64, 64), (513, 130, 32, 128), (64, 64, 64, 64), (1000, 77, 128, 32)])
 def test_tiled_transpose_goes_through_lds(R, C, BR, BC):
     # tl.trans of a loaded tile: the load is copied to LDS (pitch = columns + 1) and read back transposed, so that both

@@ -505,6 +505,19 @@ def test_memory_effects_keep_their_order_inside_a_program(native, tmp_path):
     assert "__syncthreads();" in body[first_read:write] and "__syncthreads();" in body[write:second_read]
 
 
+def test_generic_source_asks_for_a_swapped_grid_when_program_id_1_walks_the_contiguous_dimension(native, tmp_path):
+    # tiles of a row-major matrix with rows on program_id(0) and columns on program_id(1): the hardware starts workgroups
+    # along x first, so the launcher is asked to exchange x and y (the mark at the top of the source).  A transpose, whose
+    # stores are contiguous along what program_id(0) walks, is left as it is.
+    import extra_kernels as X
+    sig = {"out_ptr": "*i32", "R": "i32", "C": "i32", "BR": "constexpr", "BC": "constexpr"}
+    body = _generic_source(tmp_path, compile_ttir(X.stamp_tiles, sig, {"BR": 32, "BC": 256}))
+    assert body.startswith("// tts: swap_xy\n") and "swap_xy ? blockIdx.y : blockIdx.x" in body
+    sig = {"src": "*fp32", "dst": "*fp32", "R": "i32", "C": "i32", "BR": "constexpr", "BC": "constexpr"}
+    body = _generic_source(tmp_path, compile_ttir(X.transpose_tiles, sig, {"BR": 64, "BC": 64}))
+    assert not body.startswith("// tts: swap_xy")
+
+
 def test_declined_details_of_a_handwritten_family_fall_through(native):
     import extra_kernels as X
     from triton_shared_amd.examples import kernels as K

@@ -43,6 +43,7 @@ struct Plan {
 // every kernel argument by index: { void *ptr[N]; long long ival[N]; double fval[N]; }, N = TILE_MAX_ARGS.
 constexpr int TILE_MAX_ARGS = 32;
 std::string tile_program_source(const Program &p);
+bool tile_program_swaps_grid(const std::string &source);  // the launcher exchanges the grid's x and y for this source (when y fits)
 // Matmul family with ops between the K loop and the store: the source of the functor that applies them to one
 // accumulator value (tile_codegen.cpp), compiled at run time together with the kernels of gemm_device.h.
 std::string gemm_epilogue_source(const Program &p, const std::vector<const SOp *> &ops, int acc, int out, int64_t BM, int64_t BN);

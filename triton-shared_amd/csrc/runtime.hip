@@ -628,7 +628,7 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
     const char *kname = "";
     // one workgroup of 256 threads per Triton program, on the kernel generated for the program (compiled at its first use)
     auto run_tile_program = [&](RtcModule **slot, const std::string &source) -> tts_status {
-      struct { void *ptr[TILE_MAX_ARGS]; long long ival[TILE_MAX_ARGS]; double fval[TILE_MAX_ARGS]; } a{};
+      struct { void *ptr[TILE_MAX_ARGS]; long long ival[TILE_MAX_ARGS]; double fval[TILE_MAX_ARGS]; int swap_xy; } a{};
       for (int i = 0; i < n; i++) {
         if (args[i].kind == TTS_ARG_PTR) a.ptr[i] = args[i].v.ptr;
         else if (args[i].kind == TTS_ARG_INT) a.ival[i] = args[i].v.i;
@@ -644,7 +644,9 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
         }
       }
       kname = "tile_program (hipRTC)";
-      err = rtc_launch(*slot, gx, gy, gz, 256, &a, sizeof a, s);
+      // the program asks for neighbouring workgroups along program_id(1) (tile_codegen.cpp); grid.y holds 65535 at most
+      a.swap_xy = tile_program_swaps_grid(source) && gy > 1 && gx <= 65535 ? 1 : 0;
+      err = a.swap_xy ? rtc_launch(*slot, gy, gx, gz, 256, &a, sizeof a, s) : rtc_launch(*slot, gx, gy, gz, 256, &a, sizeof a, s);
       return TTS_OK;
     };
     if (b->fallback) {
