@@ -194,6 +194,16 @@ def make_workloads(torch, triton, K):
         return dict(desc=f"C = leaky_relu(A @ B) bf16 {n}^3, BM=BN=128 BK=64 (matmul family, the activation compiled into the kernel's epilogue)",
                     work=2 * n ** 3, bound="mfma", dtype="bf16", make=make, set_bytes=3 * n * n * 2)
 
+    def skinny_matmul(m, n, kd):
+        def make():
+            a = (torch.randn(m, kd, device=dev) * 0.02).bfloat16()
+            b = (torch.randn(kd, n, device=dev) * 0.02).bfloat16()
+            c = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+            return lambda: K.matmul_tiles[(triton.cdiv(m, 128) * triton.cdiv(n, 128),)](a, b, c, m, n, kd, kd, 1, n, 1, n, 1, BM=128, BN=128, BK=64, GROUP_M=8)
+        return dict(desc=f"matmul bf16 {m}x{n}x{kd}: too few output tiles for the chip, so K runs in slices (a workgroup per tile and slice, fp32 partial sums, "
+                         "a second kernel adds and narrows; the time is the two kernels')",
+                    work=2 * m * n * kd, bound="mfma", dtype="bf16", make=make, set_bytes=(m * kd + kd * n + m * n) * 2)
+
     def expert_rows(tokens, kd, nd, experts):
         def make():
             a = (torch.randn(tokens, kd, device=dev) * 0.02).bfloat16()
@@ -236,6 +246,7 @@ def make_workloads(torch, triton, K):
     W["next_fused_silu_2p26"] = fused_silu(1 << 26)
     W["next_matmul_act_4096"] = matmul_act(4096)
     W["next_expert_rows_4096"] = expert_rows(4096, 2048, 2048, 8)
+    W["next_matmul_skinny_512"] = skinny_matmul(512, 8192, 8192)
     W["next_take_rows_2p26"] = take_rows(1 << 16, 1024)
     W["next_row_sums_2p26"] = row_sums(1 << 16, 1024)
     W["next_block_cumsum_2p26"] = block_cumsum(1 << 26)
