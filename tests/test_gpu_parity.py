@@ -584,10 +584,13 @@ def test_gemm_with_column_major_a_and_with_strides_no_kernel_takes(K):
 
 @pytest.mark.parametrize("M,N,Kd,BM,kernel", [(17, 384, 512, 16, "gemm_w8a16_kernel"), (64, 384, 512, 16, "gemm_w8a16_kernel"),
                                              (40, 512, 1024, 16, "gemm_w8a16_wide_kernel"), (100, 1024, 2048, 64, "gemm_w8a16_wide_kernel"),
-                                             (33, 200, 100, 32, "gemm_w8a16_kernel")])
+                                             (33, 200, 100, 32, "gemm_w8a16_kernel"),
+                                             # from 193 rows: the weights widened to fp16 once, then the tiled matmul kernels
+                                             (193, 512, 1024, 16, "gemm_w8a16_widen_kernel + matmul"), (300, 1032, 2048, 64, "gemm_w8a16_widen_kernel + matmul"),
+                                             (200, 260, 96, 64, "gemm_w8a16_kernel")])   # (N not a multiple of 8: the decode kernels, 13 launches)
 def test_w8a16_beyond_the_decode_shape(K, oracle_cpu, M, N, Kd, BM, kernel):
     # the reference's matmul lowering has no shape limit (ConversionPatterns.hpp:1128-1201); the decode kernels take 16
-    # rows, more rows run as one launch of them per group of 16 (the last group ragged), whatever the program's BM
+    # or 32 rows, more rows run as one launch of them per group of rows (the last group ragged), whatever the program's BM
     torch.manual_seed(M)
     a = torch.randn(M, Kd).half()
     w = torch.randint(-127, 128, (Kd, N), dtype=torch.int8)

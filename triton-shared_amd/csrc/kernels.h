@@ -124,10 +124,12 @@ struct GemmW8A16Params {
   float *workspace;        // split-K partial sums, gemm_w8a16_workspace_bytes() large, or null when split == 1
   int *counters;           // gemm_w8a16_counters() arrival counters, zero between launches (clear them once)
   int split;
+  void *widened;           // gemm_w8a16_widened_bytes() of device memory for the weights as fp16 (many rows of A), or null
 };
 int gemm_w8a16_split(const GemmW8A16Params &p);  // how many K slices the kernel wants (from shapes and pitches)
 size_t gemm_w8a16_workspace_bytes(const GemmW8A16Params &p);
 size_t gemm_w8a16_counters(const GemmW8A16Params &p);
+size_t gemm_w8a16_widened_bytes(const GemmW8A16Params &p);  // 0: this shape runs on the decode kernels
 hipError_t launch_gemm_w8a16(const GemmW8A16Params &p, hipStream_t s, const char **kernel_name);
 
 }  // namespace tts

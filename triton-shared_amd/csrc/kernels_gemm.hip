@@ -903,12 +903,57 @@ static hipError_t launch_gemm_w8a16_rows(const GemmW8A16Params &p, hipStream_t s
 
 static bool w8_wide(const GemmW8A16Params &p);
 
+// Many rows of A (a prefill-sized M): the decode kernels would read W once per 32 rows.  The weights are widened once,
+// as the source does it -- w.to(f16) * scale[None, :], one fp16 rounding -- into a [K, N] fp16 matrix, and the tiled
+// matmul kernels multiply (fp16 operands, fp32 accumulation: the same arithmetic as the decode kernels').  From 193
+// rows up, where the passes of the decode kernel cost what widening (W read, twice its bytes written) and one tiled
+// product do.  Eight columns per thread: 8-byte weight loads, 16-byte scale loads and stores.
+// Measured at [8192, 28672]: 304 us at M = 129, 351 at 256, 452 at 512, 952 at 2048, against 50 us per 32 rows on the
+// decode kernels: from seven launches of those on, the widened product is ahead.
+constexpr int64_t W8_WIDEN_FROM_ROWS = 193;
+__global__ __launch_bounds__(256) void gemm_w8a16_widen_kernel(GemmW8A16Params p) {
+  const int64_t octs = p.N / 8, idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= p.K * octs) return;
+  const int64_t k = idx / octs, n = (idx % octs) * 8;
+  const uint2 q = *reinterpret_cast<const uint2 *>(p.w + k * p.ldw + n);
+  const uint4 sv = *reinterpret_cast<const uint4 *>((const uint16_t *)p.scale + n);
+  const uint32_t qs[2] = {q.x, q.y}, ss[4] = {sv.x, sv.y, sv.z, sv.w};
+  uint32_t out[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    // bytes 2c and 2c + 1 of the eight: [b0, 0, b1, 0], then 0x6400 | (b ^ 0x80) = 1152 + b as fp16 (exact), as in the decode kernels
+    const uint32_t word = qs[c / 2] >> (16 * (c & 1));
+    const uint32_t pair = ((word & 0xffu) | ((word & 0xff00u) << 8)) ^ 0x64806480u;
+    out[c] = pk_sub_1152_mul(pair, ss[c]);
+  }
+  *reinterpret_cast<uint4 *>((uint16_t *)p.widened + k * p.N + n) = make_uint4(out[0], out[1], out[2], out[3]);
+}
+static bool w8_widens(const GemmW8A16Params &p) {
+  return p.M >= W8_WIDEN_FROM_ROWS && p.N % 8 == 0 && p.ldw % 8 == 0 && ((uintptr_t)p.w & 7) == 0 && ((uintptr_t)p.scale & 15) == 0;
+}
+
 // More rows of A than a launch takes (32 on the 16-byte-load kernel, 16 on the other): the decode kernels once per
 // group of rows, one launch after the other on the stream (they share the split-K workspace, which every launch leaves
 // ready for the next).  W is read once per launch, so this is for the rows beside the decode shape (M = 64 at
 // [8192, 28672]: two passes over W, against 13 ms on the generic family's kernel); a prefill-sized M wants the tiled
 // matmul kernels on dequantised weights instead.
+size_t gemm_w8a16_widened_bytes(const GemmW8A16Params &p) { return w8_widens(p) ? (size_t)p.K * p.N * 2 : 0; }
+
 hipError_t launch_gemm_w8a16(const GemmW8A16Params &p, hipStream_t s, const char **name) {
+  if (p.widened && w8_widens(p)) {
+    hipLaunchKernelGGL(gemm_w8a16_widen_kernel, dim3((unsigned)((p.K * (p.N / 8) + 255) / 256)), dim3(256), 0, s, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    GemmParams g{};
+    g.a = p.a; g.b = p.widened; g.c = p.c;
+    g.M = p.M; g.N = p.N; g.K = p.K;
+    g.lda = p.lda; g.ldb = p.N; g.ldc = p.ldc;
+    g.split = 1;
+    const char *inner = nullptr;
+    e = launch_gemm(g, s, &inner);
+    *name = "gemm_w8a16_widen_kernel + matmul";
+    return e;
+  }
   const int64_t rows = w8_wide(p) ? 32 : 16;
   if (p.M <= rows) return launch_gemm_w8a16_rows(p, s, name);
   for (int64_t m0 = 0; m0 < p.M; m0 += rows) {

@@ -90,6 +90,8 @@ struct tts_plan {
   // launched on: launches on one stream run one after the other, launches on different streams may overlap and must
   // not share them.  Counters are zero between launches.
   struct SplitK {
+    void *widened = nullptr;  // the int8-weight product's weights as fp16, for launches with many rows
+    size_t widened_bytes = 0;
     float *workspace = nullptr;
     size_t workspace_bytes = 0;
     int *counters = nullptr;
@@ -102,6 +104,7 @@ struct tts_plan {
   ~tts_plan() {
     for (auto &kv : split_k) {
       if (kv.second.workspace) (void)hipFree(kv.second.workspace);
+      if (kv.second.widened) (void)hipFree(kv.second.widened);
       if (kv.second.counters) (void)hipFree(kv.second.counters);
     }
     rtc_release(fused);
@@ -827,6 +830,23 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
           }
           p.workspace = sk.workspace;
           p.counters = sk.counters;
+        }
+        p.widened = nullptr;
+        if (!no_alloc) {  // (the call that may not allocate stays on the decode kernels, a launch per 32 rows)
+          const size_t need = gemm_w8a16_widened_bytes(p);
+          if (need) {
+            std::lock_guard<std::mutex> lock(plan->mu);
+            tts_plan::SplitK &sk = plan->split_k[stream];
+            if (sk.widened_bytes < need) {
+              if (sk.widened) (void)hipFree(sk.widened);  // (waits for the device: earlier launches may still read it)
+              sk.widened = nullptr;
+              sk.widened_bytes = 0;
+              hipError_t e = hipMalloc(&sk.widened, need);
+              if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(widened weights): ") + hipGetErrorString(e));
+              sk.widened_bytes = need;
+            }
+            p.widened = sk.widened;
+          }
         }
         err = launch_gemm_w8a16(p, s, &kname);
         break;
