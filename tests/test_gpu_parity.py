@@ -303,6 +303,51 @@ def test_gemm_in_k_slices_for_skinny_products(K, M, N, Kd, dtype, bt):
     assert torch.equal(c.float(), want.to(dtype).float()) if exact else relfro(c.float(), want) <= 1e-2
 
 
+@pytest.mark.parametrize("case", [
+    # (batches, M, N, K, dtype, shared B, expected in the kernel's name)
+    (8, 256, 384, 256, torch.bfloat16, False, "gemm_dma_kernel"),       # whole tiles
+    (5, 130, 264, 96, torch.float16, False, "gemm_dma_kernel"),          # ragged rows and columns
+    (3, 200, 136, 2048, torch.bfloat16, True, "K slices"),               # too few tiles: K slices, one workspace part per product; B shared
+    (4, 70, 75, 50, torch.bfloat16, False, "gemm_mfma_kernel"),          # nothing aligned: the any-shape kernel
+    (3, 100, 72, 40, torch.float32, False, "gemm_f32_kernel"),           # fp32 operands
+])
+def test_batched_matmul_runs_on_the_matmul_kernels(case):
+    """A batch of products of one shape (tiles on program_id(0), the product on program_id(1), every operand at a batch
+    stride) is proved product by product (each an exact cover of its own C, evenly spaced, results apart) and runs as
+    one launch with the batch on grid.y: exact on small-integer operands, the padding around each C untouched."""
+    import extra_kernels as X
+    Bn, M, N, Kd, dtype, shared_b, kernel = case
+    g = torch.Generator(device="cpu").manual_seed(Bn * 1000 + M + N + Kd)
+    pad = 8
+    A = torch.randint(-3, 4, (Bn, M, Kd), generator=g).to(dtype).to(DEV)
+    Bm = torch.randint(-2, 3, (1 if shared_b else Bn, Kd, N + pad), generator=g).to(dtype).to(DEV)
+    b = Bm[:, :, :N]
+    Cfull = torch.full((Bn, M + 2, N + pad), 5.0, dtype=dtype, device=DEV)
+    c = Cfull[:, :M, :N]
+    grid = (triton.cdiv(M, 128) * triton.cdiv(N, 128), Bn)
+    k = X.batched_matmul[grid](A, b, c, M, N, Kd, A.stride(0), A.stride(1), 0 if shared_b else b.stride(0), b.stride(1), c.stride(0), c.stride(1), BM=128, BN=128, BK=32)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and kernel in k.function.last_kernel, k.function.last_kernel
+    want = torch.matmul(A.float(), b.float())           # small integers: the sums are exact in fp32 in any order, and narrowed once
+    assert torch.equal(c.float(), want.to(dtype).float())
+    assert torch.equal(Cfull[:, :, N:].cpu(), torch.full((Bn, M + 2, pad), 5.0, dtype=dtype)) and torch.equal(Cfull[:, M:].cpu(), torch.full((Bn, 2, N + pad), 5.0, dtype=dtype))
+
+
+def test_batched_matmul_with_overlapping_results_stays_on_the_generic_family():
+    import extra_kernels as X
+    # two products whose results land on the same C are not one batch of independent products: the launch falls back to
+    # the program-per-tile kernel (here both products are the same, so that the result does not depend on who writes last)
+    M = N = Kd = 128
+    g = torch.Generator(device="cpu").manual_seed(7)
+    A = torch.randint(-3, 4, (1, M, Kd), generator=g).bfloat16().to(DEV)
+    Bm = torch.randint(-2, 3, (1, Kd, N), generator=g).bfloat16().to(DEV)
+    c = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+    k = X.batched_matmul[(1, 2)](A, Bm, c, M, N, Kd, 0, A.stride(1), 0, Bm.stride(1), 0, c.stride(0), BM=128, BN=128, BK=32)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and k.function.last_kernel == "tile_program (hipRTC)", k.function.last_kernel
+    assert torch.equal(c.float(), A[0].float() @ Bm[0].float())
+
+
 @pytest.mark.parametrize("M,N,Kd,dtype,kernel", [(4000, 2048, 96, torch.bfloat16, "gemm_dma_kernel<128x256>"), (1000, 1032, 64, torch.float16, "gemm_dma_kernel<128x128>"),
                                                 (130, 264, 96, torch.bfloat16, "gemm_dma_kernel<128x128>"), (4100, 4104, 64, torch.bfloat16, "gemm_dma_kernel"),
                                                 (4090, 2056, 32, torch.float16, "gemm_dma_kernel<256x128>"), (1, 8, 32, torch.bfloat16, "gemm_dma_kernel<128x128>")])

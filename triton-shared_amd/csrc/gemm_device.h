@@ -37,10 +37,25 @@ struct TtsGemmParams {
   // leaves its fp32 sums at partial[s * M * N + m * N + n], and a second kernel adds the slices and narrows (1 = none)
   int split;
   float *partial;
+  // A batch of products of one shape (grid.y of the launch = batches): batch b reads a + b * batch_a and b + b * batch_b
+  // and writes c + b * batch_c (in elements); 1 / 0 for a single product
+  int batches;
+  int64_t batch_a, batch_b, batch_c;
 };
 
 namespace tts_gemm_device {
 typedef TtsGemmParams GemmParams;
+
+// the product of batch blockIdx.y of a launch (esize: bytes per element of the operands and of C)
+__device__ __forceinline__ GemmParams of_batch(const GemmParams &p, int esize) {
+  GemmParams q = p;
+  const int64_t by = blockIdx.y;
+  q.a = (const char *)p.a + by * p.batch_a * esize;
+  q.b = (const char *)p.b + by * p.batch_b * esize;
+  q.c = (char *)p.c + by * p.batch_c * esize;
+  if (p.partial) q.partial = p.partial + by * (int64_t)p.split * p.M * p.N;
+  return q;
+}
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;

@@ -26,7 +26,7 @@ struct IdentityEp {
 // the kernels' device code is in gemm_device.h (it is also compiled at run time, with a fused epilogue)
 template <bool BF16, int TM, int TN, int BK>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(GemmParams p, int tiles_m, int tiles_n) {
-  gemm_mfma_body<BF16, TM, TN, BK>(p, tiles_m, tiles_n, IdentityEp());
+  gemm_mfma_body<BF16, TM, TN, BK>(of_batch(p, 2), tiles_m, tiles_n, IdentityEp());
 }
 
 template <bool BF16, int TM, int TN, int BK>
@@ -41,7 +41,7 @@ hipError_t launch_gemm_cfg(const GemmParams &p, hipStream_t s) {
     configured = true;
   }
   int tiles_m = (int)((p.M + BM - 1) / BM), tiles_n = (int)((p.N + BN - 1) / BN);
-  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), lds, s, p, tiles_m, tiles_n);
+  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, std::max(1, p.batches)), dim3(256), lds, s, p, tiles_m, tiles_n);
   return hipGetLastError();
 }
 
@@ -50,12 +50,13 @@ hipError_t launch_gemm_cfg(const GemmParams &p, hipStream_t s) {
 // the 256 registers two wavefronts of a SIMD can have each, which the 128 x 256 tile fits without spilling.
 template <bool BF16, int TM, int TN, bool BT, bool AT, bool PF, bool SK>
 __global__ __launch_bounds__(PF ? 320 : 256) void gemm_dma_kernel(GemmParams p, int tiles_m, int tiles_n) {
-  gemm_dma_body<BF16, TM, TN, IdentityEp, BT, AT, PF, SK>(p, tiles_m, tiles_n, IdentityEp());
+  gemm_dma_body<BF16, TM, TN, IdentityEp, BT, AT, PF, SK>(of_batch(p, 2), tiles_m, tiles_n, IdentityEp());
 }
 
 // Adds the K slices' partial sums in slice order and narrows: four columns per thread (N is a multiple of 8).
 template <bool BF16>
-__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmParams p) {
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(GemmParams batch) {
+  const GemmParams p = of_batch(batch, 2);
   const int64_t quads = p.N / 4, idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= p.M * quads) return;
   const int64_t m = idx / quads, n = (idx % quads) * 4;
@@ -85,10 +86,10 @@ hipError_t launch_gemm_dma_t(const GemmParams &p, hipStream_t s) {
       static const hipError_t attr = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       if (attr != hipSuccess) return attr;
       int tiles_m = (int)((p.M + T::BM - 1) / T::BM), tiles_n = (int)((p.N + T::BN - 1) / T::BN);
-      hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n * p.split), dim3(256), lds, s, p, tiles_m, tiles_n);
+      hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n * p.split, std::max(1, p.batches)), dim3(256), lds, s, p, tiles_m, tiles_n);
       hipError_t e = hipGetLastError();
       if (e != hipSuccess) return e;
-      hipLaunchKernelGGL(gemm_splitk_reduce_kernel<BF16>, dim3((unsigned)((p.M * (p.N / 4) + 255) / 256)), dim3(256), 0, s, p);
+      hipLaunchKernelGGL(gemm_splitk_reduce_kernel<BF16>, dim3((unsigned)((p.M * (p.N / 4) + 255) / 256), std::max(1, p.batches)), dim3(256), 0, s, p);
       return hipGetLastError();
     }
   }
@@ -101,7 +102,7 @@ hipError_t launch_gemm_dma_t(const GemmParams &p, hipStream_t s) {
   static const hipError_t attr = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (attr != hipSuccess) return attr;
   int tiles_m = (int)((p.M + T::BM - 1) / T::BM), tiles_n = (int)((p.N + T::BN - 1) / T::BN);
-  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(PF ? 320 : 256), lds, s, p, tiles_m, tiles_n);
+  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n, std::max(1, p.batches)), dim3(PF ? 320 : 256), lds, s, p, tiles_m, tiles_n);
   return hipGetLastError();
 }
 
@@ -119,6 +120,7 @@ bool gemm_dma_ok(const GemmParams &p, int64_t bm, int64_t bn) {
   if (p.a_trans && (p.M % 8 != 0 || p.a_rows || p.b_block)) return false;
   if ((p.a_rows || p.b_block) && bm != 128) return false;  // gathered rows: 128-row tiles (64-bit A addresses per lane)
   if (p.b_block && p.b_block_rows % bm != 0) return false;
+  if (p.batches > 1 && (p.batch_a % 8 != 0 || p.batch_b % 8 != 0 || p.batch_c % 2 != 0)) return false;  // every product aligned like the first
   return p.M >= 1 && p.N >= 8 && p.N % 8 == 0 && p.K % F_BK == 0 && p.K >= F_BK && p.lda % 8 == 0 && p.ldb % 8 == 0 &&
          ((uintptr_t)p.a & 15) == 0 && ((uintptr_t)p.b & 15) == 0 && p.lda < (p.a_trans ? (1 << 25) : (1 << 22)) && p.ldb < (p.b_trans ? (1 << 22) : (1 << 25)) &&
          (!p.b_block || p.b_block_stride % 8 == 0) && p.ldc % 2 == 0 && ((uintptr_t)p.c & 3) == 0;  // C is written in 4-byte pairs
@@ -139,7 +141,8 @@ bool gemm_fast_path_ok(const GemmParams &p) { return !p.a_trans && !p.b_trans &&
 constexpr int F32_BK = 16;
 
 template <int T>
-__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams p, int tiles_m, int tiles_n) {
+__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmParams batch, int tiles_m, int tiles_n) {
+  const GemmParams p = of_batch(batch, 4);
   constexpr int BT = 64 * T;          // rows of A / columns of B per workgroup
   constexpr int PITCH = BT + 4;       // floats between k rows in LDS
   constexpr int CH = BT / 64;         // chunks of 4 floats per thread and operand tile (BT x 16 floats = 4 BT chunks)
@@ -262,13 +265,14 @@ hipError_t launch_gemm_f32(const GemmParams &p, hipStream_t s) {
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
     return n;
   }();
-  const int64_t big = ((p.M + 127) / 128) * ((p.N + 127) / 128);
+  const int batches = std::max(1, p.batches);
+  const int64_t big = ((p.M + 127) / 128) * ((p.N + 127) / 128) * batches;
   if (big >= 2 * cus) {
     const int tiles_m = (int)((p.M + 127) / 128), tiles_n = (int)((p.N + 127) / 128);
-    hipLaunchKernelGGL(gemm_f32_kernel<2>, dim3(tiles_m * tiles_n), dim3(256), 0, s, p, tiles_m, tiles_n);
+    hipLaunchKernelGGL(gemm_f32_kernel<2>, dim3(tiles_m * tiles_n, batches), dim3(256), 0, s, p, tiles_m, tiles_n);
   } else {
     const int tiles_m = (int)((p.M + 63) / 64), tiles_n = (int)((p.N + 63) / 64);
-    hipLaunchKernelGGL(gemm_f32_kernel<1>, dim3(tiles_m * tiles_n), dim3(256), 0, s, p, tiles_m, tiles_n);
+    hipLaunchKernelGGL(gemm_f32_kernel<1>, dim3(tiles_m * tiles_n, batches), dim3(256), 0, s, p, tiles_m, tiles_n);
   }
   return hipGetLastError();
 }
@@ -724,7 +728,8 @@ DmaChoice choose_dma(const GemmParams &p, int max_split) {
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
     return n;
   }();
-  auto tiles = [&](const DmaCand &c) { return ((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn); };
+  // (tiles of all the batch's products: they share the launch)
+  auto tiles = [&](const DmaCand &c) { return ((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn) * std::max(1, p.batches); };
   // Among the tiles that give every CU a workgroup (128 x 128: always), the one with the least padded work per unit
   // of the tile's measured efficiency at 4096^3 (105 / 136 / 144 / 179 us): a ragged edge counts against a tile that
   // overshoots it by more.
@@ -751,7 +756,7 @@ DmaChoice choose_dma(const GemmParams &p, int max_split) {
     const double step = c.bm + c.bn == 512 ? 0.80e-6 : c.bm + c.bn == 256 ? 0.39e-6 : c.bm == 128 ? 0.60e-6 : 0.62e-6;
     const double wgs = (double)tiles(c) * split;
     double t = std::max(1.0, wgs / cus) * (double)((nk + split - 1) / split) * step + 8e-6;
-    if (split > 1) t += 1.2 * split * (double)p.M * (double)p.N * 4 / 4e12 + 3e-6;
+    if (split > 1) t += 1.2 * split * (double)p.M * (double)p.N * std::max(1, p.batches) * 4 / 4e12 + 3e-6;
     return t;
   };
   DmaChoice pick = best;
@@ -761,7 +766,7 @@ DmaChoice choose_dma(const GemmParams &p, int max_split) {
       if (!gemm_dma_ok(p, c.bm, c.bn) || (dma_env && std::string(dma_env) != c.tag)) continue;
       const int64_t most = std::min<int64_t>(std::min<int64_t>(std::min<int64_t>(16, max_split), nk / 8), (2 * cus + tiles(c) - 1) / tiles(c));
       for (int64_t sp = split_env ? atoi(split_env) : 2; sp <= most; sp++) {
-        if ((size_t)sp * p.M * p.N * 4 > ((size_t)256 << 20)) break;
+        if ((size_t)sp * p.M * p.N * std::max(1, p.batches) * 4 > ((size_t)256 << 20)) break;
         const double t = model(c, (int)sp);
         if (t < 0.9 * pick_t || (pick.split > 1 && t < pick_t)) { pick.tile = &c; pick.split = (int)sp; pick_t = t; }
         if (split_env) break;
@@ -776,7 +781,7 @@ int gemm_split(const GemmParams &p) {
   if (p.is_f32 || tile_env) return 1;
   return choose_dma(p, 16).split;
 }
-size_t gemm_workspace_bytes(const GemmParams &p) { return p.split > 1 ? (size_t)p.split * p.M * p.N * sizeof(float) : 0; }
+size_t gemm_workspace_bytes(const GemmParams &p) { return p.split > 1 ? (size_t)p.split * p.M * p.N * std::max(1, p.batches) * sizeof(float) : 0; }
 
 // p.split: the most K slices p.partial has room for (what gemm_split(p) said, or fewer; 1: none).
 hipError_t launch_gemm(const GemmParams &p, hipStream_t s, const char **name) {

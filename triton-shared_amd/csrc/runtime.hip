@@ -9,8 +9,11 @@
 // cached; the device kernels receive closed forms of it.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+#include <array>
 #include <cstring>
 #include <list>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <set>
@@ -286,6 +289,8 @@ struct DenseGemm {
   bool a_trans = false, b_trans = false;  // column-major operands (the tutorial's `b.T`): the pitch is the other stride
   std::vector<int> tile_pid;  // per BM x BN tile (row-major over the tile grid): linear id of the program that computes it
   int tiles_n = 0;
+  // a batch of products of this shape: product b reads A and B and writes C batch_a * b, batch_b * b, batch_c * b elements further on
+  int64_t batches = 1, batch_a = 0, batch_b = 0, batch_c = 0;
 };
 
 DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
@@ -330,9 +335,17 @@ DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
   if (a_wraps) need(r.ev0("a_mod") == d.M * sam, "A rows wrap around with a period other than M");
   if (b_wraps) need(r.ev0("b_mod") == d.N * sbn, "B columns wrap around with a period other than N");
   // tiles: every program's origin, offsets consistent with a dense layout, exact cover
+  // A grid with a whole multiple of that many programs may be a batch of products (a batch index on another grid axis,
+  // tutorial-style bmm): the programs then fall into groups that differ by constant offsets into A, B and C, each group
+  // an exact cover of its own C, the offsets in arithmetic progression, the C's apart.
   const int64_t tm = (d.M + BM - 1) / BM, tn = (d.N + BN - 1) / BN;
-  need((int64_t)r.g[0] * r.g[1] * r.g[2] == tm * tn, "the grid does not have one program per output tile");
-  std::vector<char> seen(tm * tn, 0);
+  const int64_t programs = (int64_t)r.g[0] * r.g[1] * r.g[2];
+  need(programs % (tm * tn) == 0 && programs >= tm * tn, "the grid does not have one program per output tile");
+  d.batches = programs / (tm * tn);
+  need(d.batches == 1 || (!a_wraps && !b_wraps), "a batch of products with wrapped operands");
+  need(d.batches <= 65535, "more than 65535 products in a batch");
+  std::map<std::array<int64_t, 3>, int> batch_of;  // offsets (A, B, C) of a product beyond those of a single one -> its place in `seen`
+  std::vector<std::vector<char>> seen;
   d.tile_pid.assign(tm * tn, 0);
   d.tiles_n = (int)tn;
   for (int z = 0; z < r.g[2]; z++)
@@ -341,16 +354,39 @@ DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
         EvalEnv e = r.env(x, y, z);
         int64_t r0 = r.ev("r0", e), c0 = r.ev("c0", e);
         need(r0 >= 0 && c0 >= 0 && r0 % BM == 0 && c0 % BN == 0 && r0 / BM < tm && c0 / BN < tn, "a program's tile origin is off the tile grid");
-        char &s = seen[(r0 / BM) * tn + c0 / BN];
+        const std::array<int64_t, 3> off = {r.ev("a_base", e) - r0 * sam, r.ev("b_base", e) - c0 * sbn, r.ev("c_base", e) - (r0 * d.ldc + c0)};
+        if (d.batches == 1) {
+          need(off[0] == 0, "A tile offset is not row0 * its row stride");
+          need(off[1] == 0, "B tile offset is not col0 * its column stride");
+          need(off[2] == 0, "C tile offset is not row0 * ldc + col0");
+        }
+        auto at = batch_of.find(off);
+        if (at == batch_of.end()) {
+          need((int64_t)batch_of.size() < d.batches, "the programs do not fall into products of one shape");
+          at = batch_of.emplace(off, (int)seen.size()).first;
+          seen.emplace_back(tm * tn, 0);
+        }
+        char &s = seen[at->second][(r0 / BM) * tn + c0 / BN];
         need(!s, "two programs compute the same output tile");
         s = 1;
-        d.tile_pid[(r0 / BM) * tn + c0 / BN] = x + r.g[0] * (y + r.g[1] * z);
-        need(r.ev("a_base", e) == r0 * sam, "A tile offset is not row0 * its row stride");
-        need(r.ev("b_base", e) == c0 * sbn, "B tile offset is not col0 * its column stride");
+        if (d.batches == 1) d.tile_pid[(r0 / BM) * tn + c0 / BN] = x + r.g[0] * (y + r.g[1] * z);
         if (a_wraps) need(r.ev("a_wrapped", e) == r0 * sam, "the wrapped part of A's offset is not row0 * its row stride");
         if (b_wraps) need(r.ev("b_wrapped", e) == c0 * sbn, "the wrapped part of B's offset is not col0 * its column stride");
-        need(r.ev("c_base", e) == r0 * d.ldc + c0, "C tile offset is not row0 * ldc + col0");
       }
+  if (d.batches > 1) {
+    // (every product has tm * tn distinct tiles, and there are batches * tm * tn programs: all covers are exact)
+    need((int64_t)batch_of.size() == d.batches, "the programs do not fall into products of one shape");
+    std::vector<std::array<int64_t, 3>> offs;
+    for (auto &kv : batch_of) offs.push_back(kv.first);
+    std::sort(offs.begin(), offs.end(), [](const std::array<int64_t, 3> &a, const std::array<int64_t, 3> &b) { return a[2] < b[2]; });
+    need(offs[0][0] == 0 && offs[0][1] == 0 && offs[0][2] == 0, "the first product of a batch does not start at the arguments' addresses");
+    d.batch_a = offs[1][0];
+    d.batch_b = offs[1][1];
+    d.batch_c = offs[1][2];
+    for (int64_t b = 0; b < d.batches; b++)
+      need(offs[b][0] == b * d.batch_a && offs[b][1] == b * d.batch_b && offs[b][2] == b * d.batch_c, "the products of a batch are not evenly spaced");
+    need(d.batch_c >= (d.M - 1) * d.ldc + d.N, "the results of a batch's products overlap");
+  }
   return d;
 }
 
@@ -403,7 +439,9 @@ void bind_gemm(const Resolver &r, Bound &b) {
   p.a_trans = d.a_trans; p.b_trans = d.b_trans;
   p.is_bf16 = (int)r.pl.k.at("is_bf16");
   p.is_f32 = r.pl.k.count("is_f32") ? (int)r.pl.k.at("is_f32") : 0;
+  p.batches = (int)d.batches; p.batch_a = d.batch_a; p.batch_b = d.batch_b; p.batch_c = d.batch_c;
   if (p.is_f32 && !r.pl.source.empty()) throw Unsupported("gemm: a fused epilogue on fp32 operands");
+  if (p.batches > 1 && !r.pl.source.empty()) throw Unsupported("gemm: a fused epilogue on a batch of products");
   if (!r.pl.source.empty()) {  // a fused epilogue looks up the program that owns an element
     may_allocate("a table of tile owners on the device");
     hipError_t e = hipMalloc((void **)&b.tile_pid, d.tile_pid.size() * sizeof(int));
@@ -414,12 +452,14 @@ void bind_gemm(const Resolver &r, Bound &b) {
   std::ostringstream os;
   os << "kernel=gemm_mfma\nM=" << p.M << "\nN=" << p.N << "\nK=" << p.K << "\nlda=" << p.lda << "\nldb=" << p.ldb
      << "\nldc=" << p.ldc << "\nbf16=" << p.is_bf16 << "\nf32=" << p.is_f32 << "\na_trans=" << p.a_trans << "\nb_trans=" << p.b_trans << "\n";
+  if (p.batches > 1) os << "batches=" << p.batches << "\nbatch_a=" << p.batch_a << "\nbatch_b=" << p.batch_b << "\nbatch_c=" << p.batch_c << "\n";
   b.describe = os.str();
 }
 
 void bind_w8a16(const Resolver &r, Bound &b) {
   DenseGemm d = prove_dense_gemm(r, "gemm_w8a16");
   if (d.a_trans || d.b_trans) throw Unsupported("gemm_w8a16: only row-major operands are implemented");
+  if (d.batches > 1) throw Unsupported("gemm_w8a16: a batch of products");
   GemmW8A16Params &p = b.w8;
   p.M = d.M; p.N = d.N; p.K = d.K; p.lda = d.lda; p.ldw = d.ldb; p.ldc = d.ldc;
   p.split = gemm_w8a16_split(p);
@@ -735,7 +775,7 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
             p.split = want;
             const size_t need = gemm_workspace_bytes(p);
             if (no_alloc) {  // as many slices as the static array holds
-              const size_t one = (size_t)p.M * p.N * sizeof(float);
+              const size_t one = (size_t)p.M * p.N * std::max(1, p.batches) * sizeof(float);
               p.split = (int)std::min<size_t>((size_t)want, NOALLOC_WORKSPACE_BYTES / one);
               if (p.split > 1) p.partial = reinterpret_cast<float *>(noalloc_scratch());
               else p.split = 1;
