@@ -204,6 +204,15 @@ def make_workloads(torch, triton, K):
                          "a second kernel adds and narrows; the time is the two kernels')",
                     work=2 * m * n * kd, bound="mfma", dtype="bf16", make=make, set_bytes=(m * kd + kd * n + m * n) * 2)
 
+    def batched_matmul(batches, m, n, kd):
+        def make():
+            a = (torch.randn(batches, m, kd, device=dev) * 0.02).bfloat16()
+            b = (torch.randn(batches, kd, n, device=dev) * 0.02).bfloat16()
+            c = torch.empty(batches, m, n, dtype=torch.bfloat16, device=dev)
+            return lambda: K.batched_matmul[(triton.cdiv(m, 128) * triton.cdiv(n, 128), batches)](a, b, c, m, n, kd, m * kd, kd, kd * n, n, m * n, n, BM=128, BN=128, BK=64)
+        return dict(desc=f"{batches} matmuls bf16 {m}x{n}x{kd} in one launch: tiles on program_id(0), the product on program_id(1) (matmul family: the batch on grid.y)",
+                    work=2 * batches * m * n * kd, bound="mfma", dtype="bf16", make=make, set_bytes=batches * (m * kd + kd * n + m * n) * 2)
+
     def expert_rows(tokens, kd, nd, experts):
         def make():
             a = (torch.randn(tokens, kd, device=dev) * 0.02).bfloat16()
@@ -247,6 +256,7 @@ def make_workloads(torch, triton, K):
     W["next_matmul_act_4096"] = matmul_act(4096)
     W["next_expert_rows_4096"] = expert_rows(4096, 2048, 2048, 8)
     W["next_matmul_skinny_512"] = skinny_matmul(512, 8192, 8192)
+    W["next_matmul_batched_16x2048"] = batched_matmul(16, 2048, 2048, 2048)
     W["next_take_rows_2p26"] = take_rows(1 << 16, 1024)
     W["next_row_sums_2p26"] = row_sums(1 << 16, 1024)
     W["next_block_cumsum_2p26"] = block_cumsum(1 << 26)

@@ -1123,26 +1123,3 @@ def stamp_tiles(out_ptr, R, C, BR: tl.constexpr, BC: tl.constexpr):
     v = p0 * 100 + p1 + 10000 * tl.num_programs(0) + 1000000 * tl.num_programs(1)
     tile = tl.zeros((BR, BC), dtype=tl.int32) + v
     tl.store(out_ptr + r[:, None] * C + c[None, :], tile, mask=(r[:, None] < R) & (c[None, :] < C))
-
-
-@triton.jit
-def batched_matmul(a_ptr, b_ptr, c_ptr, M, N, K, s_ab, s_am, s_bb, s_bk, s_cb, s_cm, BM: tl.constexpr, BN: tl.constexpr, BK: tl.constexpr):
-    # C[b] = A[b] @ B[b]: tiles of one product on program_id(0), the product on program_id(1); a batch stride of 0 shares an operand
-    pid = tl.program_id(0)
-    bid = tl.program_id(1)
-    nn = tl.cdiv(N, BN)
-    pm = pid // nn
-    pn = pid % nn
-    rm = pm * BM + tl.arange(0, BM)
-    rn = pn * BN + tl.arange(0, BN)
-    rk = tl.arange(0, BK)
-    pa = a_ptr + bid * s_ab + rm[:, None] * s_am + rk[None, :]
-    pb = b_ptr + bid * s_bb + rk[:, None] * s_bk + rn[None, :]
-    acc = tl.zeros((BM, BN), dtype=tl.float32)
-    for k in range(0, tl.cdiv(K, BK)):
-        a = tl.load(pa, mask=(rm[:, None] < M) & (rk[None, :] < K - k * BK), other=0.0)
-        b = tl.load(pb, mask=(rk[:, None] < K - k * BK) & (rn[None, :] < N), other=0.0)
-        acc += tl.dot(a, b)
-        pa += BK
-        pb += BK * s_bk
-    tl.store(c_ptr + bid * s_cb + rm[:, None] * s_cm + rn[None, :], acc.to(c_ptr.dtype.element_ty), mask=(rm[:, None] < M) & (rn[None, :] < N))

@@ -311,11 +311,10 @@ def test_gemm_in_k_slices_for_skinny_products(K, M, N, Kd, dtype, bt):
     (4, 70, 75, 50, torch.bfloat16, False, "gemm_mfma_kernel"),          # nothing aligned: the any-shape kernel
     (3, 100, 72, 40, torch.float32, False, "gemm_f32_kernel"),           # fp32 operands
 ])
-def test_batched_matmul_runs_on_the_matmul_kernels(case):
+def test_batched_matmul_runs_on_the_matmul_kernels(K, case):
     """A batch of products of one shape (tiles on program_id(0), the product on program_id(1), every operand at a batch
     stride) is proved product by product (each an exact cover of its own C, evenly spaced, results apart) and runs as
     one launch with the batch on grid.y: exact on small-integer operands, the padding around each C untouched."""
-    import extra_kernels as X
     Bn, M, N, Kd, dtype, shared_b, kernel = case
     g = torch.Generator(device="cpu").manual_seed(Bn * 1000 + M + N + Kd)
     pad = 8
@@ -325,7 +324,7 @@ def test_batched_matmul_runs_on_the_matmul_kernels(case):
     Cfull = torch.full((Bn, M + 2, N + pad), 5.0, dtype=dtype, device=DEV)
     c = Cfull[:, :M, :N]
     grid = (triton.cdiv(M, 128) * triton.cdiv(N, 128), Bn)
-    k = X.batched_matmul[grid](A, b, c, M, N, Kd, A.stride(0), A.stride(1), 0 if shared_b else b.stride(0), b.stride(1), c.stride(0), c.stride(1), BM=128, BN=128, BK=32)
+    k = K.batched_matmul[grid](A, b, c, M, N, Kd, A.stride(0), A.stride(1), 0 if shared_b else b.stride(0), b.stride(1), c.stride(0), c.stride(1), BM=128, BN=128, BK=32)
     torch.cuda.synchronize()
     assert k.function.family == "gemm" and kernel in k.function.last_kernel, k.function.last_kernel
     want = torch.matmul(A.float(), b.float())           # small integers: the sums are exact in fp32 in any order, and narrowed once
@@ -333,8 +332,7 @@ def test_batched_matmul_runs_on_the_matmul_kernels(case):
     assert torch.equal(Cfull[:, :, N:].cpu(), torch.full((Bn, M + 2, pad), 5.0, dtype=dtype)) and torch.equal(Cfull[:, M:].cpu(), torch.full((Bn, 2, N + pad), 5.0, dtype=dtype))
 
 
-def test_batched_matmul_with_overlapping_results_stays_on_the_generic_family():
-    import extra_kernels as X
+def test_batched_matmul_with_overlapping_results_stays_on_the_generic_family(K):
     # two products whose results land on the same C are not one batch of independent products: the launch falls back to
     # the program-per-tile kernel (here both products are the same, so that the result does not depend on who writes last)
     M = N = Kd = 128
@@ -342,7 +340,7 @@ def test_batched_matmul_with_overlapping_results_stays_on_the_generic_family():
     A = torch.randint(-3, 4, (1, M, Kd), generator=g).bfloat16().to(DEV)
     Bm = torch.randint(-2, 3, (1, Kd, N), generator=g).bfloat16().to(DEV)
     c = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
-    k = X.batched_matmul[(1, 2)](A, Bm, c, M, N, Kd, 0, A.stride(1), 0, Bm.stride(1), 0, c.stride(0), BM=128, BN=128, BK=32)
+    k = K.batched_matmul[(1, 2)](A, Bm, c, M, N, Kd, 0, A.stride(1), 0, Bm.stride(1), 0, c.stride(0), BM=128, BN=128, BK=32)
     torch.cuda.synchronize()
     assert k.function.family == "gemm" and k.function.last_kernel == "tile_program (hipRTC)", k.function.last_kernel
     assert torch.equal(c.float(), A[0].float() @ Bm[0].float())
