@@ -1123,3 +1123,25 @@ def stamp_tiles(out_ptr, R, C, BR: tl.constexpr, BC: tl.constexpr):
     v = p0 * 100 + p1 + 10000 * tl.num_programs(0) + 1000000 * tl.num_programs(1)
     tile = tl.zeros((BR, BC), dtype=tl.int32) + v
     tl.store(out_ptr + r[:, None] * C + c[None, :], tile, mask=(r[:, None] < R) & (c[None, :] < C))
+
+
+@triton.jit
+def softmax_row_in_pieces(x_ptr, y_ptr, cnt_ptr, stride, N, BLOCK: tl.constexpr):
+    # a row longer than a block: running maximum and sum carried through the loop as scalars (an online softmax), and a
+    # carried integer that counts the positive elements
+    row = tl.program_id(0)
+    m_i = -float("inf")
+    l_i = 0.0
+    pos = 0
+    for s in range(0, N, BLOCK):
+        cols = s + tl.arange(0, BLOCK)
+        x = tl.load(x_ptr + row * stride + cols, mask=cols < N, other=-float("inf"))
+        m_new = tl.maximum(m_i, tl.max(x, 0))
+        l_i = l_i * tl.exp(m_i - m_new) + tl.sum(tl.exp(x - m_new), 0)
+        m_i = m_new
+        pos += tl.sum((x > 0).to(tl.int32), 0)
+    for s in range(0, N, BLOCK):
+        cols = s + tl.arange(0, BLOCK)
+        x = tl.load(x_ptr + row * stride + cols, mask=cols < N, other=0.0)
+        tl.store(y_ptr + row * stride + cols, tl.exp(x - m_i) / l_i, mask=cols < N)
+    tl.store(cnt_ptr + row, pos)

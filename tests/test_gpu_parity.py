@@ -788,6 +788,24 @@ def test_narrowing_rounds_to_nearest_even_in_both_generated_families(dtype):
     assert torch.equal(got.view(torch.int16)[sel], want[:rows * cols].view(torch.int16)[sel]) and torch.isnan(got[~sel]).all()
 
 
+@pytest.mark.parametrize("rows,N,BLOCK", [(7, 5000, 1024), (3, 1024, 1024), (5, 777, 256), (2, 1, 64)])
+def test_tile_program_carries_scalars_through_a_loop(rows, N, BLOCK):
+    """Scalars that are not index expressions (a running maximum and sum, a count) carried by a loop: the reference
+    carries them as scf.for iter_args like any other value.  An online softmax over rows read in pieces against
+    torch.softmax (1e-6: the pieces rescale the sum), the count of positive elements exact."""
+    import extra_kernels as X
+    torch.manual_seed(N)
+    x = torch.randn(rows, N + 3, device=DEV)
+    y = torch.full_like(x, -1.0)
+    cnt = torch.zeros(rows, dtype=torch.int32, device=DEV)
+    k = X.softmax_row_in_pieces[(rows,)](x, y, cnt, x.stride(0), N, BLOCK=BLOCK)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    assert (y[:, :N] - torch.softmax(x[:, :N], 1)).abs().max().item() <= 1e-6
+    assert torch.equal(y[:, N:].cpu(), torch.full((rows, 3), -1.0))
+    assert torch.equal(cnt.cpu(), (x[:, :N] > 0).sum(1).int().cpu())
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.int32])
 def test_tile_program_load_after_store_sees_the_store(dtype):
     # the serial reference finishes the store before the next load of the same buffer starts

@@ -1027,10 +1027,16 @@ struct Gen {
     // loop-carried block values live in per-thread arrays (element-wise programs never move a value between
     // elements, so each thread carries the elements it owns), each of <= 16384 elements; values of one shape are
     // initialised and stepped together
+    // A carried scalar that is not an index expression (a running maximum or sum, as in a softmax over a row read in
+    // pieces) is one variable per thread: every thread holds the same value, as it does for a reduction's result.
     std::vector<std::vector<int64_t>> cshapes;
+    auto scalar = [&](size_t q) { return val(s.tile_args[q]).shape.empty(); };
+    for (size_t q = 0; q < s.tile_args.size(); q++)
+      if (scalar(q)) os << pad() << ctype(val(s.tile_args[q]).dtype) << " car" << L << "_" << q << " = " << at(s.tile_inits[q], "0", "0") << ";\n";
     for (size_t q = 0; q < s.tile_args.size(); q++) {
       const Value &V = val(s.tile_args[q]);
-      if (V.shape.empty() || V.shape.size() > 4) no("a loop-carried value of rank " + std::to_string(V.shape.size()));
+      if (scalar(q)) continue;
+      if (V.shape.size() > 4) no("a loop-carried value of rank " + std::to_string(V.shape.size()));
       if (count(V.shape) > 2 * TWO_PHASE_MAX) no("a loop-carried block value of more than " + std::to_string(2 * TWO_PHASE_MAX) + " elements");
       if (std::find(cshapes.begin(), cshapes.end(), V.shape) == cshapes.end()) cshapes.push_back(V.shape);
       os << pad() << ctype(V.dtype) << " car" << L << "_" << q << "[" << (count(V.shape) + 255) / 256 << "];\n";
@@ -1067,6 +1073,10 @@ struct Gen {
     }
     if (any_mirror) os << pad() << "__syncthreads();\n";
     for (size_t q = 0; q < s.tile_args.size(); q++) {
+      if (scalar(q)) {
+        var[s.tile_args[q]] = "car" + L + "_" + std::to_string(q);
+        continue;
+      }
       held[s.tile_args[q]] = {"car" + L + "_" + std::to_string(q), val(s.tile_args[q]).shape};
       if (!mirrored[q].empty()) mirror[s.tile_args[q]] = mirrored[q];
     }
@@ -1080,10 +1090,13 @@ struct Gen {
     loop_depth++;
     body(s.body, &body_held);
     loop_depth--;
+    // the scalars' new values first, their assignment last: the blocks' new values may be written in terms of the old scalars
+    for (size_t q = 0; q < s.tile_args.size(); q++)
+      if (scalar(q)) os << pad() << "const " << ctype(val(s.tile_args[q]).dtype) << " nys" << L << "_" << q << " = " << at(s.tile_yields[q], "0", "0") << ";\n";
     // With LDS copies: every new value is computed (and every reader of the old copies is done) before a copy changes, and
     // the new copies are complete before the next iteration reads them.
     if (any_mirror) {
-      for (size_t q = 0; q < s.tile_args.size(); q++) os << pad() << ctype(val(s.tile_args[q]).dtype) << " nyv" << L << "_" << q << "[" << (count(val(s.tile_args[q]).shape) + 255) / 256 << "];\n";
+      for (size_t q = 0; q < s.tile_args.size(); q++) if (!scalar(q)) os << pad() << ctype(val(s.tile_args[q]).dtype) << " nyv" << L << "_" << q << "[" << (count(val(s.tile_args[q]).shape) + 255) / 256 << "];\n";
       for (const auto &cshape : cshapes) {
         open_element_loop(cshape);
         for (size_t q = 0; q < s.tile_args.size(); q++)
@@ -1111,6 +1124,8 @@ struct Gen {
         if (val(s.tile_args[q]).shape == cshape) os << pad() << "car" << L << "_" << q << "[n] = ny" << q << ";\n";
       close_loop();
     }
+    for (size_t q = 0; q < s.tile_args.size(); q++)
+      if (scalar(q)) os << pad() << "car" << L << "_" << q << " = nys" << L << "_" << q << ";\n";
     for (int v : body_held) {
       held.erase(v);
       var.erase(v);
@@ -1127,6 +1142,10 @@ struct Gen {
       held.erase(s.tile_args[q]);
       var.erase(s.tile_args[q]);
       mirror.erase(s.tile_args[q]);
+      if (scalar(q)) {
+        if (s.results[q] >= 0) var[s.results[q]] = "car" + L + "_" + std::to_string(q);
+        continue;
+      }
       if (s.results[q] >= 0) {
         held[s.results[q]] = {"car" + L + "_" + std::to_string(q), val(s.tile_args[q]).shape};
         if (!mirrored[q].empty()) mirror[s.results[q]] = mirrored[q];  // (a result read from another shape after the loop)
