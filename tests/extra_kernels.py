@@ -1145,3 +1145,20 @@ def softmax_row_in_pieces(x_ptr, y_ptr, cnt_ptr, stride, N, BLOCK: tl.constexpr)
         x = tl.load(x_ptr + row * stride + cols, mask=cols < N, other=0.0)
         tl.store(y_ptr + row * stride + cols, tl.exp(x - m_i) / l_i, mask=cols < N)
     tl.store(cnt_ptr + row, pos)
+
+
+@triton.jit
+def scale_add_2d(x_ptr, y_ptr, out_ptr, n_cols, stride, alpha, ROWS_ON_X: tl.constexpr, BLOCK: tl.constexpr):
+    # out[r, c] = alpha * x[r, c] + y[r, c] + r + c / 1024 on a two-dimensional grid, rows on either axis: the result
+    # tells which program wrote an element
+    if ROWS_ON_X:
+        row = tl.program_id(0)
+        cb = tl.program_id(1)
+    else:
+        row = tl.program_id(1)
+        cb = tl.program_id(0)
+    cols = cb * BLOCK + tl.arange(0, BLOCK)
+    m = cols < n_cols
+    x = tl.load(x_ptr + row * stride + cols, mask=m, other=0.0)
+    y = tl.load(y_ptr + row * stride + cols, mask=m, other=0.0)
+    tl.store(out_ptr + row * stride + cols, alpha * x + y, mask=m)

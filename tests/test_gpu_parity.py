@@ -926,6 +926,29 @@ def test_fused_map_interpreter_and_compiled_kernel_agree(K, kernel, monkeypatch)
     assert torch.equal(outs[0], outs[1])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("rows,n_cols,BLOCK,rows_on_x", [(37, 100, 16, True), (37, 100, 16, False), (5, 1000, 64, True), (300, 70, 32, False),
+                                                         (3, 5000, 1024, True), (9, 3000, 512, False), (1, 8, 8, True), (70000, 24, 8, False)])
+def test_fused_map_small_blocks_share_a_workgroup(rows, n_cols, BLOCK, rows_on_x, dtype):
+    """Programs whose blocks need fewer than 256 threads share a workgroup, and the launch walks the grid along the
+    axis on which the output advances least: every element still comes from its own program (bit-exact against the
+    same two roundings in torch), ragged last column blocks stay masked, the padding between rows is untouched."""
+    import extra_kernels as X
+    torch.manual_seed(rows + n_cols)
+    stride = n_cols + 5
+    x = torch.randn(rows, stride, device=DEV).to(dtype)
+    y = torch.randn(rows, stride, device=DEV).to(dtype)
+    out = torch.full((rows, stride), 7.0, dtype=dtype, device=DEV)
+    nb = triton.cdiv(n_cols, BLOCK)
+    grid = (rows, nb) if rows_on_x else (nb, rows)
+    k = X.scale_add_2d[grid](x, y, out, n_cols, stride, 0.5, ROWS_ON_X=rows_on_x, BLOCK=BLOCK)
+    torch.cuda.synchronize()
+    assert k.function.family == "fused_map" and k.function.last_kernel == "fused_map (hipRTC)", k.function.last_kernel
+    want = ((0.5 * x[:, :n_cols].float()).to(dtype) + y[:, :n_cols]) if dtype != torch.float32 else 0.5 * x[:, :n_cols] + y[:, :n_cols]
+    assert torch.equal(out[:, :n_cols], want)
+    assert torch.equal(out[:, n_cols:].cpu(), torch.full((rows, 5), 7.0, dtype=dtype))
+
+
 def test_fused_map_two_ops(K):
     import extra_kernels as X
     n = 3000

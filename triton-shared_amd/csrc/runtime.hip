@@ -663,9 +663,14 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
   return guarded([&]() {
     if (gx < 0 || gy < 0 || gz < 0) throw Invalid("negative grid");
     if ((int64_t)gx * gy * gz == 0) return TTS_OK;  // backend/driver.py:117
-    if (gy > 65535 || gz > 65535) throw Unsupported("grid y/z extents above 65535");
     auto b = resolve(plan, gx, gy, gz, args, n);
     const Plan &pl = plan->plan;
+    {
+      // the compiled fused map numbers its programs itself (a one-dimensional launch); the others use the device's grid
+      const char *mode = getenv("TTS_FUSED_MAP");
+      const bool own_numbering = pl.family == Family::FusedMap && !b->fallback && !(mode && std::string(mode) == "interpreter");
+      if ((gy > 65535 || gz > 65535) && !own_numbering) throw Unsupported("grid y/z extents above 65535");
+    }
     hipStream_t s = (hipStream_t)stream;
     hipError_t err = hipSuccess;
     const char *kname = "";
