@@ -581,3 +581,19 @@ def test_gathered_rows_matmul_binds_to_the_matrix_product_family(native):
     sig32 = {k: (v.replace("bf16", "fp32")) for k, v in sig.items()}
     text = native.ttir_to_structured(compile_ttir(K.expert_rows_matmul, sig32, {"BM": 32, "BN": 32, "BK": 32}))
     assert native.PlanHandle(native.structured_to_plan(text)[0]).family == "tile_program"
+
+
+def test_batched_matmul_and_carried_scalars_plan(native):
+    """A batch index on another grid axis leaves the matmul in its family (the launcher proves the batch's structure
+    from the arguments); a loop that carries a running maximum and sum as scalars is a generic program whose source
+    keeps them in one variable per thread."""
+    from triton_shared_amd.examples import kernels as K
+    import extra_kernels as X
+    sig = {"a_ptr": "*bf16", "b_ptr": "*bf16", "c_ptr": "*bf16", "M": "i32", "N": "i32", "K": "i32", "s_ab": "i32", "s_am": "i32", "s_bb": "i32",
+           "s_bk": "i32", "s_cb": "i32", "s_cm": "i32", "BM": "constexpr", "BN": "constexpr", "BK": "constexpr"}
+    s = native.ttir_to_structured(compile_ttir(K.batched_matmul, sig, {"BM": 128, "BN": 128, "BK": 64}))
+    assert native.PlanHandle(native.structured_to_plan(s)[0]).family == "gemm"
+    sig = {"x_ptr": "*fp32", "y_ptr": "*fp32", "cnt_ptr": "*i32", "stride": "i32", "N": "i32", "BLOCK": "constexpr"}
+    s = native.ttir_to_structured(compile_ttir(X.softmax_row_in_pieces, sig, {"BLOCK": 1024}))
+    plan = native.PlanHandle(native.structured_to_plan(s)[0])
+    assert plan.family == "tile_program"
