@@ -487,7 +487,15 @@ struct Gen {
       std::string term = "(" + ex(a.offsets[d]) + " + " + i + " * " + ex(a.strides[d]) + ")";
       if (!a.mods.empty() && a.mods[d] >= 0) term = "wrap(" + term + ", " + ex(a.mods[d]) + ")";
       sum += (d ? " + " : "") + term;
-      if (!a.dims.empty()) pred += std::string(pred.empty() ? "" : " && ") + i + " < " + ex(a.dims[d]);
+      // (An index lies in [0, size): comparing it with the extent clamped to that range is the same, and the clamped
+      // extent is a 32-bit value that is the same in every lane, where the extent itself is a 64-bit one.  For extents
+      // that do not change inside a loop, where it measured faster: LayerNorm's dx on fp16 [4096, 8192] 51 -> 45 us;
+      // a softmax over rows read in pieces, whose extents follow the loop, 284 -> 306 us with it.)
+      if (!a.dims.empty()) {
+        const bool fixed = !P.pool.depends_on(a.dims[d], EK::IV) && !P.pool.depends_on(a.dims[d], EK::Iter);
+        pred += std::string(pred.empty() ? "" : " && ") + i + " < " +
+                (fixed ? "(int)smin(smax(" + ex(a.dims[d]) + ", 0LL), " + std::to_string(a.sizes[d]) + "LL)" : ex(a.dims[d]));
+      }
     }
     if (a.sizes.empty()) sum = ex(a.offsets.at(0));
     return sum;
