@@ -1162,3 +1162,31 @@ def scale_add_2d(x_ptr, y_ptr, out_ptr, n_cols, stride, alpha, ROWS_ON_X: tl.con
     x = tl.load(x_ptr + row * stride + cols, mask=m, other=0.0)
     y = tl.load(y_ptr + row * stride + cols, mask=m, other=0.0)
     tl.store(out_ptr + row * stride + cols, alpha * x + y, mask=m)
+
+
+@triton.jit
+def while_halve(x_ptr, y_ptr, n, BLOCK: tl.constexpr):
+    # y = x / 2^floor(log2 n): a `while` that carries an integer and a block
+    offs = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    acc = tl.load(x_ptr + offs, mask=offs < n, other=0.0)
+    k = n
+    while k > 1:
+        acc = acc * 0.5
+        k = k // 2
+    tl.store(y_ptr + offs, acc, mask=offs < n)
+
+
+@triton.jit
+def while_sum_until(x_ptr, out_ptr, cnt_ptr, stride, n, limit, BLOCK: tl.constexpr):
+    # a row is summed piece by piece until the sum reaches `limit` or the row ends: how often the loop runs depends on
+    # the data, and differs from program to program
+    row = tl.program_id(0)
+    k = 0
+    acc = 0.0
+    while (k < n) & (acc < limit):
+        cols = k + tl.arange(0, BLOCK)
+        x = tl.load(x_ptr + row * stride + cols, mask=cols < n, other=0.0)
+        acc += tl.sum(x, 0)
+        k += BLOCK
+    tl.store(out_ptr + row, acc)
+    tl.store(cnt_ptr + row, k)

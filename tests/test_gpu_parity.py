@@ -788,6 +788,41 @@ def test_narrowing_rounds_to_nearest_even_in_both_generated_families(dtype):
     assert torch.equal(got.view(torch.int16)[sel], want[:rows * cols].view(torch.int16)[sel]) and torch.isnan(got[~sel]).all()
 
 
+def test_tile_program_while_loops():
+    """`while` (scf.while whose condition passes the loop's arguments on, the form the frontend writes) runs as a loop
+    that every thread of a program leaves together: a trip count that depends on an argument, and one that depends on
+    the data and differs from program to program (small integers: the sums are exact)."""
+    import extra_kernels as X
+    for n in (1, 2, 1000, 1025):
+        x = torch.randn(n, device=DEV)
+        y = torch.full((n + 3,), 9.0, device=DEV)
+        k = X.while_halve[(triton.cdiv(n, 256),)](x, y, n, BLOCK=256)
+        torch.cuda.synchronize()
+        assert k.function.family == "tile_program"
+        assert torch.equal(y[:n], x * 0.5 ** (n.bit_length() - 1)) and torch.equal(y[n:].cpu(), torch.full((3,), 9.0))
+    rows, n, B = 9, 3000, 256
+    g = torch.Generator(device="cpu").manual_seed(5)
+    x = torch.randint(0, 4, (rows, n + 5), generator=g).float()
+    x[3] = 0.0                                    # never reaches the limit: runs to the end of the row
+    x[4, 0] = 1000.0                              # reaches it in the first piece
+    limit = 700.0
+    out = torch.zeros(rows, device=DEV)
+    cnt = torch.zeros(rows, dtype=torch.int32, device=DEV)
+    k = X.while_sum_until[(rows,)](x.to(DEV), out, cnt, x.stride(0), n, limit, BLOCK=B)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    want_sum, want_cnt = [], []
+    for r in range(rows):
+        kk, acc = 0, 0.0
+        while kk < n and acc < limit:
+            acc += float(x[r, kk:min(kk + B, n)].sum())
+            kk += B
+        want_sum.append(acc)
+        want_cnt.append(kk)
+    assert out.cpu().tolist() == want_sum and cnt.cpu().tolist() == want_cnt
+    assert len(set(want_cnt)) > 2                 # the programs did leave after different numbers of rounds
+
+
 @pytest.mark.parametrize("rows,N,BLOCK", [(7, 5000, 1024), (3, 1024, 1024), (5, 777, 256), (2, 1, 64)])
 def test_tile_program_carries_scalars_through_a_loop(rows, N, BLOCK):
     """Scalars that are not index expressions (a running maximum and sum, a count) carried by a loop: the reference

@@ -597,3 +597,8 @@ def test_batched_matmul_and_carried_scalars_plan(native):
     s = native.ttir_to_structured(compile_ttir(X.softmax_row_in_pieces, sig, {"BLOCK": 1024}))
     plan = native.PlanHandle(native.structured_to_plan(s)[0])
     assert plan.family == "tile_program"
+    # `while`: a counted loop with an exit (an If without a body, ival = 2) that dead-code elimination keeps
+    sig = {"x_ptr": "*fp32", "out_ptr": "*fp32", "cnt_ptr": "*i32", "stride": "i32", "n": "i32", "limit": "fp32", "BLOCK": "constexpr"}
+    s = native.ttir_to_structured(compile_ttir(X.while_sum_until, sig, {"BLOCK": 256}))
+    assert "ub=" in s and "2147483647" in s and "ival=2" in s
+    assert native.PlanHandle(native.structured_to_plan(s)[0]).family == "tile_program"

@@ -1224,6 +1224,14 @@ class Lowerer {
     if (n == "tt.return" || n == "tt.assert") return;  // assertions are dropped, as the reference does (triton_assert.mlir)
     if (n == "scf.for") return lower_for(op);
     if (n == "cf.if" || n == "scf.if") return lower_if(op);
+    if (n == "tts.break_unless") {  // where a `while` leaves its loop (ttir.cpp: parse_while): an If without a body, ival = 2
+      SOp s;
+      s.kind = SK::If;
+      s.operands.push_back(data_of(op.operands.at(0)));
+      s.ival = 2;
+      cur_->push_back(s);
+      return;
+    }
     if (n == "tt.load") return lower_load(op);
     if (n == "tt.store") return lower_store(op);
     if (n == "tt.reduce" || n == "tt.scan") return lower_reduce(op);
@@ -1447,7 +1455,7 @@ class Lowerer {
         } else if (s.kind == SK::If) {
           bool res_live = false;
           for (int r : s.results) res_live |= live[r];
-          const bool eff = mark(s.body);
+          const bool eff = mark(s.body) || s.ival == 2;  // (a loop's exit is an effect: what the loop does depends on it)
           if (eff || res_live) {
             any_effect |= eff;
             for (int v : s.operands) use(v);
@@ -1502,7 +1510,7 @@ class Lowerer {
             keep = scan(s.body) || need_loop.count(s.loop);
             for (int r : s.results) keep = keep || (r >= 0 && live[r]);
           } else if (s.kind == SK::If) {
-            keep = scan(s.body);
+            keep = scan(s.body) || s.ival == 2;
             for (int r : s.results) keep = keep || live[r];
           } else if (!s.results.empty()) keep = live[s.results[0]];
           else keep = s.result >= 0 && live[s.result];
@@ -1553,7 +1561,7 @@ class Lowerer {
             s.results.clear();
             s.tile_yields.clear();
           }
-          keep = sweep(s.body) || res_live;
+          keep = sweep(s.body) || res_live || s.ival == 2;
         }
         else if (!s.results.empty()) keep = live[s.results[0]];
         else keep = s.result >= 0 && live[s.result];

@@ -46,7 +46,8 @@ enum class SK {
   ExpandDims,  // tensor.expand_shape
   Broadcast,   // linalg.generic broadcast
   For,         // scf.for
-  If,          // body runs iff the scalar i1 operand is true (false when ival = 1); no results (cf.cond_br trees, scf.if)
+  If,          // body runs iff the scalar i1 operand is true (false when ival = 1); no results (cf.cond_br trees, scf.if).
+               // ival = 2, no body: the enclosing loop ends here unless the operand is true (scf.while's scf.condition)
 };
 
 struct Access {          // the tts.make_tptr + mask part of a load/store

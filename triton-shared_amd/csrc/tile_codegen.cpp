@@ -672,6 +672,13 @@ struct Gen {
     while (k < ops.size()) {
       const SOp &s = ops[k];
       if (s.kind == SK::For) { loop(s); k++; continue; }
+      if (s.kind == SK::If && s.ival == 2) {  // a `while` leaves its loop: every thread does, the condition is a scalar
+        if (!loop_depth) no("a loop exit outside a loop");
+        map_vars({-1});
+        os << pad() << "if (!(" << at(s.operands.at(0), "0", "0") << ")) break;\n";
+        k++;
+        continue;
+      }
       if (s.kind == SK::If) {  // the condition is a scalar, the same for every thread: barriers inside are safe
         map_vars({-1});
         // results: a variable per scalar, a per-thread array per block, declared once (the `then` side comes first)

@@ -207,6 +207,109 @@ static void parse_results(const std::string &lhs, Op &op) {
   }
 }
 
+using Renames = std::map<std::string, std::string>;
+static void copy_block(const Block &src, Block &dst, const Renames &m);
+static void collect_defs(const Block &b, std::vector<std::string> &out);
+
+// scf.while (%a = %x, ...) : (types) -> (types) { <before> scf.condition(%c) %a, ... } do { ^bb0(%a: type, ...): <after>
+// scf.yield ... }, in the form the frontend writes for `while cond:` -- the condition passes the loop's arguments on
+// unchanged -- becomes a counted loop that is left through a break: scf.for over [0, 2^31 - 1) whose body is the `before`
+// ops, "tts.break_unless %c", and the `after` ops with their yield.  Where it breaks, the carried values are the
+// arguments of that round, which is what scf.while returns.
+static void parse_while(const std::string &rest, Op &op, Lines &L, Block &blk) {
+  const std::string tag = "_w" + std::to_string(op.line);
+  std::vector<std::string> names, inits;
+  const size_t open = rest.find('(');
+  const size_t colon = top_colon(rest);
+  if (open != std::string::npos && (colon == std::string::npos || open < colon)) {
+    int depth = 0;
+    size_t close = open;
+    for (; close < rest.size(); close++) {
+      if (rest[close] == '(') depth++;
+      if (rest[close] == ')' && --depth == 0) break;
+    }
+    for (auto &pair : split_top(rest.substr(open + 1, close - open - 1), {","})) {
+      const size_t q = pair.find('=');
+      if (q == std::string::npos) continue;
+      names.push_back(trim(pair.substr(0, q)));
+      inits.push_back(trim(pair.substr(q + 1)));
+    }
+  }
+  const size_t arrow = rest.rfind("->"), brace = rest.rfind('{');
+  if (arrow == std::string::npos || brace == std::string::npos || brace < arrow) throw Unsupported("malformed scf.while: " + rest);
+  op.result_types = parse_type_list(trim(rest.substr(arrow + 2, brace - arrow - 2)));
+  if (op.result_types.size() != names.size() || op.results.size() != names.size())
+    throw Unsupported("scf.while whose results are not its arguments (line " + std::to_string(op.line) + ")");
+  Block before, after;
+  parse_block(L, before);
+  if (L.i >= L.v.size() || L.v[L.i] != "} do {") throw Unsupported("scf.while without a do region");
+  L.i++;
+  if (L.i < L.v.size() && L.v[L.i][0] == '^') {
+    const std::string hdr = L.v[L.i++];
+    const size_t o = hdr.find('('), c2 = hdr.rfind(')');
+    if (o != std::string::npos)
+      for (auto &a : split_top(hdr.substr(o + 1, c2 - o - 1), {","})) {
+        const size_t col = a.find(':');
+        after.arg_names.push_back(trim(a.substr(0, col)));
+        after.arg_types.push_back(parse_type(a.substr(col + 1)));
+      }
+  }
+  parse_block(L, after);
+  if (L.i >= L.v.size() || L.v[L.i] != "}") throw Unsupported("scf.while region not closed");
+  L.i++;
+  if (before.ops.empty() || before.ops.back()->name != "scf.condition") throw Unsupported("scf.while whose first region does not end in scf.condition");
+  const Op &cond = *before.ops.back();
+  if (cond.operands.size() != names.size() + 1 || after.arg_names.size() != names.size())
+    throw Unsupported("scf.while whose condition passes on other values than the loop's arguments (line " + std::to_string(op.line) + ")");
+  for (size_t j = 0; j < names.size(); j++)
+    if (cond.operands[j + 1] != names[j])
+      throw Unsupported("scf.while whose condition passes on other values than the loop's arguments (line " + std::to_string(op.line) + ")");
+  // the two regions are siblings and may use the same names for different values: the first one's get a suffix
+  Renames first, second;
+  {
+    std::vector<std::string> defs;
+    collect_defs(before, defs);
+    for (auto &d : defs) first[d] = d + tag;
+    for (auto &n : names) first[n] = n + tag;
+    for (size_t j = 0; j < names.size(); j++) second[after.arg_names[j]] = names[j] + tag;
+  }
+  auto constant = [&](const std::string &name, const std::string &value) {
+    auto c = std::make_unique<Op>();
+    c->name = "arith.constant";
+    c->line = op.line;
+    c->results.push_back(name);
+    c->literal = value;
+    Type t;
+    t.elem = "i32";
+    c->result_types.push_back(t);
+    blk.ops.push_back(std::move(c));
+  };
+  constant("%lb" + tag, "0");
+  constant("%ub" + tag, "2147483647");
+  constant("%st" + tag, "1");
+  op.name = "scf.for";
+  op.iv = "%iv" + tag;
+  op.operands = {"%lb" + tag, "%ub" + tag, "%st" + tag};
+  for (auto &n : names) op.iter_names.push_back(n + tag);
+  op.iter_inits = inits;
+  op.regions.emplace_back();
+  Block &body = op.regions.back();
+  {
+    Block renamed_before;
+    copy_block(before, renamed_before, first);
+    auto brk = std::make_unique<Op>();
+    brk->name = "tts.break_unless";
+    brk->line = op.line;
+    brk->operands.push_back(renamed_before.ops.back()->operands.at(0));
+    renamed_before.ops.pop_back();
+    for (auto &o : renamed_before.ops) body.ops.push_back(std::move(o));
+    body.ops.push_back(std::move(brk));
+    Block renamed_after;
+    copy_block(after, renamed_after, second);
+    for (auto &o : renamed_after.ops) body.ops.push_back(std::move(o));
+  }
+}
+
 static void parse_for(const std::string &rest, Op &op, Lines &L) {
   // %iv = %lb to %ub step %st [iter_args(%a = %x, ...) -> (types)] : i32 {
   size_t eq = rest.find(" = ");
@@ -277,6 +380,11 @@ static void parse_op(Lines &L, Block &blk) {
 
   if (op->name == "scf.for") {
     parse_for(rest, *op, L);
+    blk.ops.push_back(std::move(op));
+    return;
+  }
+  if (op->name == "scf.while") {
+    parse_while(rest, *op, L, blk);
     blk.ops.push_back(std::move(op));
     return;
   }
@@ -419,7 +527,7 @@ static void parse_op(Lines &L, Block &blk) {
 static void parse_block(Lines &L, Block &blk) {
   while (L.i < L.v.size()) {
     const std::string &line = L.v[L.i];
-    if (line == "}" || starts_with(line, "})") || starts_with(line, "} else")) return;
+    if (line == "}" || starts_with(line, "})") || starts_with(line, "} else") || line == "} do {") return;
     parse_op(L, blk);
   }
 }
@@ -427,8 +535,6 @@ static void parse_block(Lines &L, Block &blk) {
 // ---------------------------------------------------------------- copies of ops under new names
 // Tail duplication (a block reached from two branches) and the inlining of calls both copy ops; every copy gets
 // its own SSA names, so that nothing keyed by name downstream sees two definitions of one value.
-using Renames = std::map<std::string, std::string>;
-
 static std::string renamed(const std::string &name, const Renames &m) {
   auto whole = m.find(name);  // one result of a pack ("%r#1") replaced by itself
   if (whole != m.end()) return whole->second;
