@@ -247,7 +247,7 @@ static void parse_while(const std::string &rest, Op &op, Lines &L, Block &blk) {
   if (L.i < L.v.size() && L.v[L.i][0] == '^') {
     const std::string hdr = L.v[L.i++];
     const size_t o = hdr.find('('), c2 = hdr.rfind(')');
-    if (o != std::string::npos)
+    if (o != std::string::npos && c2 != std::string::npos && c2 > o)
       for (auto &a : split_top(hdr.substr(o + 1, c2 - o - 1), {","})) {
         const size_t col = a.find(':');
         after.arg_names.push_back(trim(a.substr(0, col)));
@@ -442,15 +442,17 @@ static void parse_op(Lines &L, Block &blk) {
     op->regions.emplace_back();
     Block &rb = op->regions.back();
     // ^bb0(%a: f32, %b: f32):
+    if (L.i >= L.v.size()) throw Unsupported("region of " + op->name + " cut short");
     std::string hdr = L.v[L.i++];
     size_t o = hdr.find('('), c2 = hdr.rfind(')');
-    if (!starts_with(hdr, "^") || o == std::string::npos) throw Unsupported("expected block header: " + hdr);
+    if (!starts_with(hdr, "^") || o == std::string::npos || c2 == std::string::npos || c2 < o) throw Unsupported("expected block header: " + hdr);
     for (auto &a : split_top(hdr.substr(o + 1, c2 - o - 1), {","})) {
       size_t col = a.find(':');
       rb.arg_names.push_back(trim(a.substr(0, col)));
       rb.arg_types.push_back(parse_type(a.substr(col + 1)));
     }
     parse_block(L, rb);
+    if (L.i >= L.v.size()) throw Unsupported("region of " + op->name + " not closed");
     std::string tail = L.v[L.i++];  // }) : (types) -> types
     if (!starts_with(tail, "})")) throw Unsupported("region of " + op->name + " not closed: " + tail);
     {  // the generic form carries the attributes here: }) {axis = 0 : i32} : (types) -> types
@@ -462,6 +464,7 @@ static void parse_op(Lines &L, Block &blk) {
     }
     size_t col = tail.find(':');
     size_t arrow = tail.find("->");
+    if (col == std::string::npos || arrow == std::string::npos || arrow < col) throw Unsupported("region of " + op->name + " without its types: " + tail);
     op->types = parse_type_list(tail.substr(col + 1, arrow - col - 1));
     op->result_types = parse_type_list(tail.substr(arrow + 2));
     blk.ops.push_back(std::move(op));
