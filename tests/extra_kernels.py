@@ -1190,3 +1190,31 @@ def while_sum_until(x_ptr, out_ptr, cnt_ptr, stride, n, limit, BLOCK: tl.constex
         k += BLOCK
     tl.store(out_ptr + row, acc)
     tl.store(cnt_ptr + row, k)
+
+
+@triton.jit
+def while_carried_pointer(x_ptr, out_ptr, stride, n, BLOCK: tl.constexpr):
+    # a block of pointers carried by a `while`, stepped along the row
+    row = tl.program_id(0)
+    offs = tl.arange(0, BLOCK)
+    p = x_ptr + row * stride + offs
+    k = 0
+    acc = tl.zeros((BLOCK,), dtype=tl.float32)
+    while k < n:
+        acc += tl.load(p, mask=k + offs < n, other=0.0)
+        p += BLOCK
+        k += BLOCK
+    tl.store(out_ptr + row, tl.sum(acc, 0))
+
+
+@triton.jit
+def while_inside_for(x_ptr, out_ptr, n, BLOCK: tl.constexpr):
+    # a `while` inside a `for`: out = x * sum over i < n of (i + i // 2 + i // 4 + ...)
+    offs = tl.arange(0, BLOCK)
+    acc = tl.zeros((BLOCK,), dtype=tl.float32)
+    for i in range(0, n):
+        k = i
+        while k > 0:
+            acc += tl.load(x_ptr + offs) * k
+            k = k // 2
+    tl.store(out_ptr + offs, acc)

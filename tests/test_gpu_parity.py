@@ -821,6 +821,23 @@ def test_tile_program_while_loops():
         want_cnt.append(kk)
     assert out.cpu().tolist() == want_sum and cnt.cpu().tolist() == want_cnt
     assert len(set(want_cnt)) > 2                 # the programs did leave after different numbers of rounds
+    # a carried block of pointers; a `while` inside a `for`
+    xs = torch.randint(-3, 4, (5, 1000 + 7), generator=g).float()
+    out = torch.zeros(5, device=DEV)
+    X.while_carried_pointer[(5,)](xs.to(DEV), out, xs.stride(0), 1000, BLOCK=256)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), xs[:, :1000].sum(1))
+    xv = torch.randint(-2, 3, (256,), generator=g).float()
+    out = torch.zeros(256, device=DEV)
+    X.while_inside_for[(1,)](xv.to(DEV), out, 37, BLOCK=256)
+    torch.cuda.synchronize()
+    total = 0
+    for i in range(37):
+        kk = i
+        while kk > 0:
+            total += kk
+            kk //= 2
+    assert torch.equal(out.cpu(), xv * total)
 
 
 @pytest.mark.parametrize("rows,N,BLOCK", [(7, 5000, 1024), (3, 1024, 1024), (5, 777, 256), (2, 1, 64)])
