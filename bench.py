@@ -157,6 +157,16 @@ def make_workloads(torch, triton, K):
         return dict(desc=f"fused map out = silu(g) * u fp16 N={n}, BLOCK=1024 (10 elementwise ops, compiled with hipRTC)",
                     work=3 * n * 2, bound="hbm", dtype="f16", make=make, set_bytes=3 * n * 2)
 
+    def rotary(seq, heads, half):
+        def make():
+            x = torch.randn(seq, heads * 2 * half, device=dev).half()
+            c, sn = torch.randn(seq, half, device=dev), torch.randn(seq, half, device=dev)
+            o = torch.empty_like(x)
+            return lambda: K.rotary_embedding[(seq, heads)](x, c, sn, o, heads * 2 * half, HALF=half)
+        nbytes = seq * heads * 2 * half * 4 + seq * half * 8
+        return dict(desc=f"rotary embedding fp16 [{seq}, {heads} x {2 * half}], a program per (position, head) with blocks of {half} elements "
+                         "(fused map: programs this small share a workgroup)", work=nbytes, bound="hbm", dtype="f16", make=make, set_bytes=nbytes)
+
     def take_rows(rows, cols):
         def make():
             src = torch.randn(rows, cols, device=dev)
@@ -253,6 +263,7 @@ def make_workloads(torch, triton, K):
     W["stream_read_2p28"] = stream_read(1 << 28)
     W["next_fused_gelu_2p26"] = fused_gelu(1 << 26)
     W["next_fused_silu_2p26"] = fused_silu(1 << 26)
+    W["next_rotary_8192x32x128"] = rotary(8192, 32, 64)
     W["next_matmul_act_4096"] = matmul_act(4096)
     W["next_expert_rows_4096"] = expert_rows(4096, 2048, 2048, 8)
     W["next_matmul_skinny_512"] = skinny_matmul(512, 8192, 8192)

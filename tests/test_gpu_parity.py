@@ -1001,6 +1001,24 @@ def test_fused_map_small_blocks_share_a_workgroup(rows, n_cols, BLOCK, rows_on_x
     assert torch.equal(out[:, n_cols:].cpu(), torch.full((rows, 5), 7.0, dtype=dtype))
 
 
+@pytest.mark.parametrize("seq,heads,half", [(33, 5, 64), (7, 3, 16), (2, 1, 128)])
+def test_fused_map_rotary_embedding(K, seq, heads, half):
+    # a program per (position, head) on blocks of `half` elements, two outputs: fp32 products and differences rounded
+    # one by one, as torch rounds them, then narrowed: bit-exact
+    torch.manual_seed(seq)
+    x = torch.randn(seq, heads * 2 * half, device=DEV).half()
+    c, sn = torch.randn(seq, half, device=DEV), torch.randn(seq, half, device=DEV)
+    out = torch.zeros_like(x)
+    k = K.rotary_embedding[(seq, heads)](x, c, sn, out, x.stride(0), HALF=half)
+    torch.cuda.synchronize()
+    assert k.function.family == "fused_map" and k.function.last_kernel == "fused_map (hipRTC)"
+    xv = x.float().view(seq, heads, 2, half)
+    x1, x2 = xv[:, :, 0], xv[:, :, 1]
+    cc, ss = c[:, None, :], sn[:, None, :]
+    want = torch.stack([x1 * cc - x2 * ss, x2 * cc + x1 * ss], 2).half().view(seq, -1)
+    assert torch.equal(out, want)
+
+
 def test_fused_map_two_ops(K):
     import extra_kernels as X
     n = 3000

@@ -315,3 +315,18 @@ def batched_matmul(a_ptr, b_ptr, c_ptr, M, N, K, s_ab, s_am, s_bb, s_bk, s_cb, s
         pa += BK
         pb += BK * s_bk
     tl.store(c_ptr + bid * s_cb + rm[:, None] * s_cm + rn[None, :], acc.to(c_ptr.dtype.element_ty), mask=(rm[:, None] < M) & (rn[None, :] < N))
+
+
+@triton.jit
+def rotary_embedding(x_ptr, cos_ptr, sin_ptr, out_ptr, stride_s, HALF: tl.constexpr):
+    """Rotary position embedding on [seq, heads * 2 * HALF] fp16: one program per (position, head), blocks of HALF elements."""
+    s = tl.program_id(0)
+    h = tl.program_id(1)
+    d = tl.arange(0, HALF)
+    base = s * stride_s + h * 2 * HALF
+    x1 = tl.load(x_ptr + base + d).to(tl.float32)
+    x2 = tl.load(x_ptr + base + HALF + d).to(tl.float32)
+    c = tl.load(cos_ptr + s * HALF + d)
+    sn = tl.load(sin_ptr + s * HALF + d)
+    tl.store(out_ptr + base + d, (x1 * c - x2 * sn).to(tl.float16))
+    tl.store(out_ptr + base + HALF + d, (x2 * c + x1 * sn).to(tl.float16))
