@@ -11,9 +11,11 @@ does not find its input in the 256 MB Infinity Cache left by the previous one.
 Prints ONE JSON line.  The headline workload is the LayerNorm forward, fp16
 [4096, 8192] (the third of the five configurations: HBM-bound at a size that
 neither fits the caches nor is dominated by the launch); the other four
-configurations, two steady-state sizes, the two stream ceilings of the machine
-(a copy and a read-only reduction, through this backend) and the workloads of
-the generic families are reported in "kernels".
+configurations, two steady-state sizes, the stream ceilings of the machine
+(a copy and a read-only reduction through this backend, and the HIP runtime's
+own device-to-device copy as an independent figure) and the workloads of the
+generic families are reported in "kernels"; "summary", the last key of the
+line, repeats [us, fraction of peak] for every workload.
 
 Per kernel: `us` = mean kernel duration from HIP events around the K timed
 launches (the line's ms_per_step); `launch_us` = median / min / std of the
@@ -243,6 +245,16 @@ def make_workloads(torch, triton, K):
         return dict(desc=f"stream ceiling, 1:1 read/write: z = x fp32 N={n}, BLOCK=4096 (fused map with no ops)", work=8 * n, bound="hbm",
                     dtype="f32", make=make, set_bytes=8 * n)
 
+    def runtime_copy(n):
+        # the HIP runtime's own device-to-device copy (what torch.Tensor.copy_ enqueues for two contiguous tensors of one
+        # type): a mover this backend did not write, as an independent figure for what a 1:1 stream reaches on the machine
+        def make():
+            x = torch.rand(n, device=dev)
+            z = torch.empty_like(x)
+            return dict(direct=lambda: z.copy_(x), kernel="hipMemcpyAsync device-to-device (the runtime's copy kernel, not this backend)")
+        return dict(desc=f"independent stream ceiling, 1:1 read/write: the HIP runtime's device-to-device copy of fp32 N={n} (not a kernel of this backend)",
+                    work=8 * n, bound="hbm", dtype="f32", make=make, set_bytes=8 * n)
+
     def stream_read(n):
         def make():
             x = torch.rand(n, device=dev)
@@ -261,6 +273,7 @@ def make_workloads(torch, triton, K):
     W["diag_cfg4_zero_operands"] = gemm(zeros=True)
     W["stream_copy_2p28"] = stream_copy(1 << 28)
     W["stream_read_2p28"] = stream_read(1 << 28)
+    W["stream_runtime_copy_2p28"] = runtime_copy(1 << 28)
     W["next_fused_gelu_2p26"] = fused_gelu(1 << 26)
     W["next_fused_silu_2p26"] = fused_silu(1 << 26)
     W["next_rotary_8192x32x128"] = rotary(8192, 32, 64)
@@ -279,33 +292,39 @@ def time_workload(torch, spy, wl, steps, warmup, rotating_only=False):
     sets = max(1, min(32, math.ceil(ROTATE_BYTES / wl["set_bytes"])))
     if wl["set_bytes"] > 1e9:
         sets = 1
-    launches = []
-    plan = None
+    stream = torch.cuda.current_stream().cuda_stream
+    launches = []   # one closure per buffer set: enqueues the workload's kernel on torch's current stream
+    frontends = []  # the same launch through the Triton JIT dispatch (None for a workload that is not a Triton kernel)
+    plan, ttir, direct_kernel = None, None, None
     for _ in range(sets):
         fn = wl["make"]()
+        if isinstance(fn, dict):  # not a kernel of this backend (the runtime's own copy): called as it is
+            direct_kernel = fn["kernel"]
+            launches.append(fn["direct"])
+            frontends.append(None)
+            continue
         k = fn()  # compiles on first use, launches once through the full frontend
         plan = k.function
         ttir = k.asm.get("ttir") if hasattr(k, "asm") else None
         grid, vals = spy.last
-        launches.append((grid, plan.pack(vals), len(vals), fn))
+        arr, n = plan.pack(vals), len(vals)
+        launches.append(lambda plan=plan, grid=grid, arr=arr, n=n: plan.launch_packed(grid, stream, arr, n))
+        frontends.append(fn)
     torch.cuda.synchronize()
-    stream = torch.cuda.current_stream().cuda_stream
     # Warm-up: `warmup` steps at least, and on until the GPU has been busy for RAMP_SECONDS: after an idle
     # period the device takes tens of milliseconds of load to reach its sustained clocks (a 4096^3 GEMM
     # measured 125 us per launch in the first 10 ms of load and 113 us from 30 ms on).
     t_ramp, done = time.perf_counter(), 0
     while done < warmup or time.perf_counter() - t_ramp < RAMP_SECONDS:
         for i in range(max(warmup, 20)):
-            g, arr, n, _ = launches[(done + i) % sets]
-            plan.launch_packed(g, stream, arr, n)
+            launches[(done + i) % sets]()
         done += max(warmup, 20)
         torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     start.record()
     for i in range(steps):
-        g, arr, n, _ = launches[i % sets]
-        plan.launch_packed(g, stream, arr, n)
+        launches[i % sets]()
     stop.record()
     torch.cuda.synchronize()
     wall_us = (time.perf_counter() - t0) * 1e6 / steps
@@ -315,41 +334,42 @@ def time_workload(torch, spy, wl, steps, warmup, rotating_only=False):
     singles = max(steps, 100) if wl["set_bytes"] < 1e9 else steps
     pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(singles)]
     for i, (e0, e1) in enumerate(pairs):
-        g, arr, n, _ = launches[i % sets]
         e0.record()
-        plan.launch_packed(g, stream, arr, n)
+        launches[i % sets]()
         e1.record()
     torch.cuda.synchronize()
     per = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in pairs)
     mean = sum(per) / len(per)
     launch_us = dict(median=round(per[len(per) // 2], 3), min=round(per[0], 3),
                      std=round((sum((v - mean) ** 2 for v in per) / len(per)) ** 0.5, 3), n=len(per))
+    kernel_name = lambda: direct_kernel if plan is None else plan.last_kernel
     if rotating_only:
-        kernel = plan.last_kernel
-        del launches
+        kernel = kernel_name()
+        del launches, frontends
         torch.cuda.empty_cache()
         return dict(us=us, hot_us=us, wall_us=wall_us, kernel=kernel, sets=sets, frontend_us=0.0, warmup_steps_run=done, ttir=ttir,
                     launch_us=launch_us)
     # same measurement on one buffer set ("hot": inputs may sit in the Infinity Cache), for information
-    g, arr, n, _ = launches[0]
     for _ in range(warmup):
-        plan.launch_packed(g, stream, arr, n)
+        launches[0]()
     start.record()
     for _ in range(steps):
-        plan.launch_packed(g, stream, arr, n)
+        launches[0]()
     stop.record()
     torch.cuda.synchronize()
     hot_us = start.elapsed_time(stop) * 1e3 / steps
     # the same launch through the Triton JIT dispatch (Python overhead included), for information
-    fn = launches[0][3]
-    t0 = time.perf_counter()
-    for _ in range(20):
-        fn()
-    torch.cuda.synchronize()
-    frontend_us = (time.perf_counter() - t0) * 1e6 / 20
-    del launches
+    frontend_us = 0.0
+    if frontends[0] is not None:
+        t0 = time.perf_counter()
+        for _ in range(20):
+            frontends[0]()
+        torch.cuda.synchronize()
+        frontend_us = (time.perf_counter() - t0) * 1e6 / 20
+    kernel = kernel_name()
+    del launches, frontends
     torch.cuda.empty_cache()
-    return dict(us=us, hot_us=hot_us, wall_us=wall_us, kernel=plan.last_kernel, sets=sets, frontend_us=frontend_us, ttir=ttir,
+    return dict(us=us, hot_us=hot_us, wall_us=wall_us, kernel=kernel, sets=sets, frontend_us=frontend_us, ttir=ttir,
                 warmup_steps_run=done, launch_us=launch_us)
 
 
@@ -499,6 +519,13 @@ def main():
     head = kernels[args.workload]
     wl = W[args.workload]
     unit = "GB/s" if wl["bound"] == "hbm" else "TFLOP/s"
+    # The five configurations and their two steady-state sizes go last in "kernels", and a compact "summary"
+    # ([us per launch, fraction of the peak that bounds the kernel] per workload) ends the line, so that a reader who keeps
+    # only the end of this (long) line still has every configuration's figure.
+    last = ("cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "cfg1_2p28", "cfg2_1m")
+    order = [n for n in kernels if n not in last] + [n for n in last if n in kernels]
+    kernels = {n: kernels[n] for n in order}
+    summary = {n: [round(kernels[n]["us"], 2), kernels[n]["roofline"]["frac"]] for n in order}
     line = {
         "metric": "achieved HBM GB/s & bf16 TFLOP/s as % of MI355X roofline per kernel",
         "value": head["roofline"]["achieved"],
@@ -516,6 +543,7 @@ def main():
         "roofline": head["roofline"],
         "cpu_baseline": head.get("cpu_baseline"),
         "kernels": kernels,
+        "summary": summary,
     }
     print(json.dumps(line))
 

@@ -276,6 +276,18 @@ def test_gemm_launches_the_product_kernels_decline_go_to_the_generic_family(nati
     assert d["kernel"] == "gemm_mfma" and d["a_trans"] == "0" and d["b_trans"] == "0"
 
 
+def test_gemm_declines_negative_pitches(native):
+    # a negative pitch of A or B would become an unsigned byte offset in the product kernels, and a pitch of C that is
+    # not positive makes the rows of C overlap or run backwards: such launches go to the generic family's kernel
+    plan, _ = plan_for(native, "matmul_tiles.small")
+    for vals in ([0, 0, 0, 70, 90, 40, -40, 90, 90], [0, 0, 0, 70, 90, 40, 40, -90, 90], [0, 0, 0, 70, 90, 40, 40, 90, -90],
+                 [0, 0, 0, 70, 90, 40, 40, 90, 0]):
+        d = plan.describe_launch((9, 1, 1), vals)
+        assert d["kernel"] == "tile_program" and "pitch" in d["fallback_reason"], (vals, d)
+    d = plan.describe_launch((9, 1, 1), [0, 0, 0, 70, 90, 40, 0, 90, 90])    # a pitch of 0: one row of A for every row of C
+    assert d["kernel"] == "gemm_mfma" and d["lda"] == "0"
+
+
 def test_w8a16_binding(native):
     plan, _ = plan_for(native, "w8a16_matmul.small")
     M, N, K = 13, 70, 100

@@ -100,3 +100,64 @@ def test_noalloc_launch_runs_a_skinny_matmul_in_k_slices_from_the_static_array(n
         assert ((got.double() - ref).norm() / ref.norm()).item() <= 1e-2
         if fits and M * N * 4 * 16 <= (8 << 20):   # (at most 16 slices are ever taken: then both calls took the same number)
             assert torch.equal(got, want), (M, N, Kd)
+
+
+def test_noalloc_refusal_leaves_a_matmul_with_epilogue_on_its_kernel(native):
+    """A matrix product with a fused epilogue needs a compiled kernel and, per launch shape, a device table of tile
+    owners: the launch that may not allocate refuses both, and the refusal must not be remembered as "this launch belongs
+    to the generic family" -- the same launch through tts_launch afterwards runs the product kernel with its epilogue."""
+    import triton
+    import triton_shared_amd as tsa
+    import extra_kernels as X
+    tsa.activate()
+    g = torch.Generator(device="cpu").manual_seed(3)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def operands(M, N, K):
+        a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).to(DEV)
+        b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).to(DEV)
+        return a, b, torch.full((M, N), 7, device=DEV, dtype=torch.bfloat16)
+
+    M, N, K = 512, 768, 96
+    a, b, c = operands(M, N, K)
+    grid = (triton.cdiv(M, 128), triton.cdiv(N, 128), 1)
+    k = X.matmul_leaky[grid[:2]](a, b, c, M, N, K, a.stride(0), b.stride(0), c.stride(0), 0.5, BM=128, BN=128, BK=64)
+    torch.cuda.synchronize()
+    assert k.function.family == "gemm" and k.function.last_kernel.startswith("gemm_dma_kernel + epilogue")
+    want = torch.nn.functional.leaky_relu(a.float() @ b.float(), 0.5)
+    assert torch.equal(c.float(), want)
+    n_args = len(k.function.arg_kinds)
+
+    def values(a, b, c, M, N, K):
+        vals = [a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, a.stride(0), b.stride(0), c.stride(0), 0.5]
+        assert len(vals) == n_args, (n_args, k.function.arg_kinds)
+        return vals
+
+    # (1) a plan that has compiled nothing yet: refused, then launched the ordinary way on the product kernel
+    fresh = native.PlanHandle(k.kernel)
+    c.fill_(7)
+    with pytest.raises(NotImplementedError, match="allocates"):
+        fresh.launch_noalloc(grid, stream, values(a, b, c, M, N, K))
+    torch.cuda.synchronize()
+    assert torch.all(c == 7)                     # nothing ran
+    fresh.launch(grid, stream, values(a, b, c, M, N, K))
+    torch.cuda.synchronize()
+    assert fresh.last_kernel.startswith("gemm_dma_kernel + epilogue"), fresh.last_kernel
+    assert torch.equal(c.float(), want)
+    c.fill_(7)
+    fresh.launch_noalloc(grid, stream, values(a, b, c, M, N, K))   # kernel compiled, table of this shape built: runs
+    torch.cuda.synchronize()
+    assert fresh.last_kernel.startswith("gemm_dma_kernel + epilogue") and torch.equal(c.float(), want)
+    # (2) the kernel is compiled, but a new shape needs a new table of tile owners: refused, not rebound to the generic
+    # family; a smaller problem than the first, as the second call of two in a row
+    M2, N2, K2 = 256, 512, 64
+    a2, b2, c2 = operands(M2, N2, K2)
+    grid2 = (triton.cdiv(M2, 128), triton.cdiv(N2, 128), 1)
+    with pytest.raises(NotImplementedError, match="allocates"):
+        fresh.launch_noalloc(grid2, stream, values(a2, b2, c2, M2, N2, K2))
+    d = fresh.describe_launch(grid2, values(a2, b2, c2, M2, N2, K2))
+    assert d["kernel"] == "gemm_mfma", d
+    fresh.launch(grid2, stream, values(a2, b2, c2, M2, N2, K2))
+    torch.cuda.synchronize()
+    assert fresh.last_kernel.startswith("gemm_dma_kernel + epilogue"), fresh.last_kernel
+    assert torch.equal(c2.float(), torch.nn.functional.leaky_relu(a2.float() @ b2.float(), 0.5))

@@ -45,10 +45,17 @@ struct Invalid : std::runtime_error {
   using std::runtime_error::runtime_error;
 };
 
+// What tts_launch_noalloc refuses.  Not an Unsupported: a launch that the matrix-product families decline for a reason of
+// their own goes on to the generic family's kernel and its binding is cached as such, whereas this refusal says nothing
+// about the launch -- the same launch through tts_launch must still find the family's kernel, so nothing is cached.
+struct WouldAllocate : std::runtime_error {
+  using std::runtime_error::runtime_error;
+};
+
 thread_local bool g_no_alloc = false;  // set while tts_launch_noalloc runs on this thread
 void may_allocate(const char *what) {
   if (g_no_alloc)
-    throw Unsupported(std::string("tts_launch_noalloc: this launch needs ") + what + ", which allocates; run it once through tts_launch first");
+    throw WouldAllocate(std::string("tts_launch_noalloc: this launch needs ") + what + ", which allocates; run it once through tts_launch first");
 }
 
 // Everything a launch needs besides the pointers, resolved for one (scalars, grid).
@@ -101,6 +108,27 @@ struct tts_plan {
     size_t counters_count = 0;
   };
   std::unordered_map<void *, SplitK> split_k;
+  // Buffers a stream has outgrown.  Launches already enqueued (by this or another thread) may still use them, so they are
+  // neither freed nor reused before the plan goes: growing never waits for the device.  A buffer grows to at least twice
+  // its size, so the retired ones of a stream together are smaller than the one in use.
+  std::vector<void *> retired;
+  // A buffer of at least `need` bytes in *buf (of *have bytes); called with `mu` held.
+  hipError_t grow(void **buf, size_t *have, size_t need) {
+    if (*have >= need) return hipSuccess;
+    size_t got = std::max(need, 2 * *have);
+    void *fresh = nullptr;
+    hipError_t e = hipMalloc(&fresh, got);
+    if (e != hipSuccess && got > need) {
+      (void)hipGetLastError();
+      got = need;
+      e = hipMalloc(&fresh, got);
+    }
+    if (e != hipSuccess) return e;
+    if (*buf) retired.push_back(*buf);
+    *buf = fresh;
+    *have = got;
+    return hipSuccess;
+  }
   RtcModule *fused = nullptr;  // the kernel compiled for this plan at its first launch (fused maps, tile programs)
   RtcModule *gemm_rtc[2] = {nullptr, nullptr};  // matrix products with a fused epilogue: one kernel per tiling
   RtcModule *fallback = nullptr;  // the generic family's kernel for a matrix-product plan (launches the product kernels decline)
@@ -110,6 +138,7 @@ struct tts_plan {
       if (kv.second.widened) (void)hipFree(kv.second.widened);
       if (kv.second.counters) (void)hipFree(kv.second.counters);
     }
+    for (void *p : retired) (void)hipFree(p);
     rtc_release(fused);
     rtc_release(fallback);
     for (RtcModule *m : gemm_rtc) rtc_release(m);
@@ -316,6 +345,10 @@ DenseGemm prove_dense_gemm(const Resolver &r, const char *F) {
   d.lda = d.a_trans ? sak : sam;
   d.ldb = d.b_trans ? sbn : sbk;
   need(d.M > 0 && d.N > 0, "empty problem");
+  // a pitch of 0 is a broadcast operand, which the kernels read correctly; a negative one would become an unsigned byte
+  // offset in the kernels, and rows of C that overlap or run backwards are not a dense product
+  need(d.lda >= 0 && d.ldb >= 0, "a negative pitch of A or B");
+  need(d.ldc > 0, "a pitch of C that is not positive");
   // K: the loop must sweep K in full blocks followed by at most one partial block
   int64_t trip = r.ev0("trip");
   need(trip >= 0 && trip < (1 << 24), "unreasonable K trip count");
@@ -529,6 +562,8 @@ tts_status guarded(F &&f) {
   try {
     return f();
   } catch (const Unsupported &e) {
+    return fail(TTS_UNSUPPORTED, e.what());
+  } catch (const WouldAllocate &e) {
     return fail(TTS_UNSUPPORTED, e.what());
   } catch (const Invalid &e) {
     return fail(TTS_INVALID, e.what());
@@ -787,15 +822,8 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
             } else {
               std::lock_guard<std::mutex> lock(plan->mu);
               tts_plan::SplitK &sk = plan->split_k[stream];
-              if (sk.workspace_bytes < need) {
-                // the stream's earlier launches may still be using the old buffer: hipFree waits for the device
-                if (sk.workspace) (void)hipFree(sk.workspace);
-                sk.workspace = nullptr;
-                sk.workspace_bytes = 0;
-                hipError_t e = hipMalloc((void **)&sk.workspace, need);
-                if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(split-K workspace): ") + hipGetErrorString(e));
-                sk.workspace_bytes = need;
-              }
+              hipError_t e = plan->grow((void **)&sk.workspace, &sk.workspace_bytes, need);
+              if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(split-K workspace): ") + hipGetErrorString(e));
               p.partial = sk.workspace;
             }
           }
@@ -854,24 +882,19 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
           const size_t need = gemm_w8a16_workspace_bytes(p), ncount = gemm_w8a16_counters(p);
           std::lock_guard<std::mutex> lock(plan->mu);
           tts_plan::SplitK &sk = plan->split_k[stream];
-          if (sk.workspace_bytes < need) {
-            // the stream's earlier launches may still be using the old buffer: hipFree waits for the device
-            if (sk.workspace) (void)hipFree(sk.workspace);
-            sk.workspace = nullptr;
-            sk.workspace_bytes = 0;
-            hipError_t e = hipMalloc((void **)&sk.workspace, need);
-            if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(split-K workspace): ") + hipGetErrorString(e));
-            sk.workspace_bytes = need;
-          }
+          hipError_t e = plan->grow((void **)&sk.workspace, &sk.workspace_bytes, need);
+          if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(split-K workspace): ") + hipGetErrorString(e));
           if (sk.counters_count < ncount) {
-            if (sk.counters) (void)hipFree(sk.counters);
-            sk.counters = nullptr;
-            sk.counters_count = 0;
-            hipError_t e = hipMalloc((void **)&sk.counters, ncount * sizeof(int));
-            if (e == hipSuccess) e = hipMemset(sk.counters, 0, ncount * sizeof(int));
+            // (new counters start at zero; the old ones, which launches in flight may still be bumping, are retired)
+            int *fresh = nullptr;
+            const size_t count = std::max(ncount, 2 * sk.counters_count);
+            e = hipMalloc((void **)&fresh, count * sizeof(int));
+            if (e == hipSuccess) e = hipMemset(fresh, 0, count * sizeof(int));
             if (e == hipSuccess) e = hipDeviceSynchronize();  // the fill has landed before a launch on any stream reads the counters
             if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(split-K counters): ") + hipGetErrorString(e));
-            sk.counters_count = ncount;
+            if (sk.counters) plan->retired.push_back(sk.counters);
+            sk.counters = fresh;
+            sk.counters_count = count;
           }
           p.workspace = sk.workspace;
           p.counters = sk.counters;
@@ -882,14 +905,8 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
           if (need) {
             std::lock_guard<std::mutex> lock(plan->mu);
             tts_plan::SplitK &sk = plan->split_k[stream];
-            if (sk.widened_bytes < need) {
-              if (sk.widened) (void)hipFree(sk.widened);  // (waits for the device: earlier launches may still read it)
-              sk.widened = nullptr;
-              sk.widened_bytes = 0;
-              hipError_t e = hipMalloc(&sk.widened, need);
-              if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(widened weights): ") + hipGetErrorString(e));
-              sk.widened_bytes = need;
-            }
+            hipError_t e = plan->grow(&sk.widened, &sk.widened_bytes, need);
+            if (e != hipSuccess) return fail(TTS_HIP_ERROR, std::string("hipMalloc(widened weights): ") + hipGetErrorString(e));
             p.widened = sk.widened;
           }
         }
