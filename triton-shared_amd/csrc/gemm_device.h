@@ -671,12 +671,258 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
   else store_tile(EdgeTile<false>());
 }
 
+
+// ------------------------- the 256 x 256 tile on v_mfma_f32_16x16x32 (row-major operands, whole K tiles)
+// The same tile, the same ring of four direct-to-LDS stages and the same A swizzle as gemm_dma_body<4, 4>, with the matrix
+// instruction of shape 16 x 16 x 32 instead of 32 x 32 x 16.  Under the board's power limit the time of a large product is the
+// energy it dissipates, and on operands of the prescribed distribution the 16 x 16 x 32 instruction sustains 0.79 of the
+// peak rate from registers where 32 x 32 x 16 sustains 0.70 to 0.73 (measured with no data movement at all; on all-zero
+// operands both reach 0.90); LDS and global traffic per flop are the same for both.  4096^3: 101-104 us against 104-110 for
+// the 32 x 32 x 16 body in the same runs, bit for bit the same result.
+//
+// A wavefront's 128 x 128 part of C is 8 x 8 blocks of 16 x 16, four accumulator registers each, held transposed (the B
+// operand goes in as the instruction's first source): a lane holds four consecutive columns of one row, which the epilogue
+// can narrow and pack without cross-lane moves.  One K tile of 32 is one instruction's depth.
+//   A operand of row block i: row 16 i + lane % 16, k 8 (lane / 16) .. +7: one 16-byte LDS read; the four chunks of 16 rows
+//     are 1 KB of consecutive LDS whatever the swizzle.
+//   B operand of column block j: `ds_read_b64_tr_b16` twice (k 0-3 and 4-7 of the lane's octet), lane r of a 16-lane group
+//     addressing k row 8 (lane / 16) + r / 4, columns 4 (r % 4) .. +3 of the block.  Two k octets share a half wavefront, so
+//     the stage's swizzle also flips chunk bit 1 with k bit 3: position q of k row k holds chunk q ^ ((k & 3) << 2) ^ (((k >> 3) & 1) << 1).
+// Phases of a tile t: (0) the 32 products of column blocks 0-3, with the eight reads of B blocks 4-7 of tile t and half of
+// the loads of tile t + 3 behind them; wait for the own loads of tile t + 1, barrier; (1) the 32 products of column blocks
+// 4-7, with the reads of all of A (8) and of B blocks 0-3 (8) of tile t + 1 and the other half of the loads.  A's operands
+// alternate between two register sets (the K loop is unrolled by two), B's blocks 0-3 and 4-7 each have one.
+// The matrix instruction is issued from inline assembly, in place on the accumulation registers: left to the register
+// allocator (the instruction's result may overlap its addend arbitrarily, so nothing ties them) the 64 accumulators rotate
+// through both register files and are copied back at the loop's end, 520 moves per two tiles.
+// Epilogue: every wavefront narrows 16 rows at a time into a patch of LDS of its own (the stages are free by then) and
+// stores whole 256-byte row segments with 16-byte nontemporal stores: 33.5 MB written for 33.5 MB of C where 4-byte
+// stores of 64-byte segments wrote 51 MB.
+// Loops over compile-time indices, and every lambda of the body below is marked always_inline: the accumulators and
+// operand registers must become registers whatever the size of the epilogue functor.  (With a functor of a few hundred
+// operations the inliner left the epilogue's lambda out of line, the accumulators, passed to it by reference, lived in
+// scratch memory, and the compiler read them right behind matrix instructions it had not seen being issued.)
+template <int V>
+struct IntConstant {
+  static constexpr int value = V;
+};
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(IntConstant<I>());
+    static_for<I + 1, N>(f);
+  }
+}
+
+template <bool BF16, class Ep>
+__device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m, int tiles_n, const Ep &ep) {
+  using T = DmaTile<4, 4>;
+  constexpr int BM = T::BM, BN = T::BN, STAGES = T::STAGES, A_BYTES = T::A_BYTES, STAGE_BYTES = T::STAGE_BYTES, ROWB = T::B_ROW_BYTES;
+  constexpr int A_DMA = T::A_DMA, B_DMA = T::B_DMA, DMA = T::DMA;
+  static_assert(A_DMA == 4 && B_DMA == 4 && ROWB == 512, "256 x 256 x 32 stages");
+#ifdef TTS_GEMM_RTC
+  __shared__ __align__(16) char dma_smem[T::LDS_BYTES];
+#else
+  extern __shared__ __align__(16) char dma_smem[];
+#endif
+  char *smem = dma_smem;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  int bid = blockIdx.x;
+  const int nwg = tiles_m * tiles_n;
+  if (nwg % 8 == 0) bid = (bid % 8) * (nwg / 8) + bid / 8;  // consecutive ids on one XCD
+  const int group = 4 * tiles_n;                             // 4-tile-tall column groups
+  const int g0 = (bid / group) * 4;
+  const int gh = min(tiles_m - g0, 4);
+  const int tile_m = g0 + (bid % group) % gh, tile_n = (bid % group) / gh;
+  const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+  const char *a_base = (const char *)((const uint16_t *)p.a + m0 * p.lda);
+  const char *b_base = (const char *)((const uint16_t *)p.b + n0);
+  const int nk = (int)(p.K / F_BK);
+
+  uint32_t a_voff[A_DMA], b_voff[B_DMA];
+#pragma unroll
+  for (int i = 0; i < A_DMA; i++) {
+    // rows past M (the last row tile of a ragged problem) fetch row M - 1 again: they only reach outputs nobody stores
+    const int row = min(16 * (A_DMA * wave + i) + lane / 4, (int)(p.M - 1 - m0));
+    const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
+    a_voff[i] = (uint32_t)((row * p.lda + 8 * chunk) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < B_DMA; i++) {
+    const int krow = 2 * (B_DMA * wave + i) + lane / 32;
+    // likewise, chunks of columns past N fetch the last whole chunk of the row (N is a multiple of 8)
+    const int chunk = min((lane & 31) ^ ((krow & 3) << 2) ^ (((krow >> 3) & 1) << 1), (int)((p.N - n0) / 8 - 1));
+    b_voff[i] = (uint32_t)((krow * p.ldb + 8 * chunk) * 2);
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)TTS_LDS(smem);
+  const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
+  auto dma = [&](const char *sbase, uint32_t voff, uint32_t lds) __attribute__((always_inline)) {
+#ifdef TTS_GEMM_RTC
+    // (an older run-time compiler does not see that the tile's base address is the same in every lane: say so)
+    const uint64_t b = (uint64_t)(uintptr_t)sbase;
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    sbase = (const char *)(uintptr_t)(((uint64_t)hi << 32) | (uint64_t)lo);
+#endif
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(voff), "s"(sbase) : "memory", "m0");
+  };
+  auto dma_one = [&](int t, int n) __attribute__((always_inline)) {  // n < A_DMA: A part, else B part of tile t (past the last tile: the last again), into stage t % STAGES
+    const int tc = min(t, nk - 1);
+    const uint32_t st = lds0 + (t % STAGES) * STAGE_BYTES;
+    if (n < A_DMA) dma(a_base + (int64_t)tc * F_BK * 2, a_voff[n], st + (A_DMA * wave_u + n) * 1024);
+    else dma(b_base + (int64_t)tc * F_BK * p.ldb * 2, b_voff[n - A_DMA], st + A_BYTES + (B_DMA * wave_u + n - A_DMA) * 1024);
+  };
+
+  const int l16 = lane & 15, q = lane >> 4;
+  const int a_off = (wm * 128 + l16) * 64 + ((q ^ ((l16 >> 2) & 3)) << 4);
+  const int b_sw = ((l16 >> 2) << 2) ^ ((q & 1) << 1);
+  const int b_chunk = wn * 16 + ((l16 & 3) >> 1);
+  const int b_off = A_BYTES + (8 * q + (l16 >> 2)) * ROWB + 8 * (l16 & 1);
+
+  f32x4 acc[8][8];
+  static_for<0, 64>([&](auto n) __attribute__((always_inline)) { acc[n.value / 8][n.value % 8] = (f32x4){0.f, 0.f, 0.f, 0.f}; });
+  uint4 A[2][8], B0[4], B1[4];
+  auto read_a = [&](int t, int i, uint4 (&a)[8]) {
+    a[i] = *reinterpret_cast<const uint4 *>(smem + (t % STAGES) * STAGE_BYTES + a_off + i * 1024);
+  };
+  auto read_b = [&](int t, int j, int h, uint4 &b) __attribute__((always_inline)) {  // column block j of the wavefront's eight, k half h of the lane's octet
+    const char *bp = smem + (t % STAGES) * STAGE_BYTES + b_off + h * 4 * ROWB + (((b_chunk + 2 * j) ^ b_sw) << 4);
+    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)TTS_LDS(bp));
+    uint2 v2 = __builtin_bit_cast(uint2, v);
+    if (h == 0) { b.x = v2.x; b.y = v2.y; } else { b.z = v2.x; b.w = v2.y; }
+  };
+  typedef uint32_t u32x4_r __attribute__((ext_vector_type(4)));
+  auto mfma16 = [&](int i, int j, const uint4 &a, const uint4 &b) __attribute__((always_inline)) {
+    if constexpr (BF16)
+      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(__builtin_bit_cast(u32x4_r, b)), "v"(__builtin_bit_cast(u32x4_r, a)));
+    else
+      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(__builtin_bit_cast(u32x4_r, b)), "v"(__builtin_bit_cast(u32x4_r, a)));
+  };
+  auto tile = [&](int t, uint4 (&Ac)[8], uint4 (&An)[8]) {
+    static_for<0, 32>([&](auto slot) __attribute__((always_inline)) {
+      constexpr int n = decltype(slot)::value;
+      __builtin_amdgcn_sched_barrier(0);
+      mfma16(n >> 2, n & 3, Ac[n >> 2], B0[n & 3]);
+      if constexpr (n < 8) read_b(t, 4 + (n >> 1), n & 1, B1[n >> 1]);
+      if constexpr (n % 8 == 7) dma_one(t + STAGES - 1, n / 8);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    // own loads of tile t + 1 have landed (later ones may be in flight); own reads of tile t are complete
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(DMA * (STAGES - 3) + DMA / 2, 0));
+    __syncthreads();
+    static_for<0, 32>([&](auto slot) __attribute__((always_inline)) {
+      constexpr int n = decltype(slot)::value;
+      __builtin_amdgcn_sched_barrier(0);
+      mfma16(n >> 2, 4 + (n & 3), Ac[n >> 2], B1[n & 3]);
+      if constexpr (n < 8) read_a(t + 1, n, An);
+      else if constexpr (n < 16) read_b(t + 1, (n - 8) >> 1, n & 1, B0[(n - 8) >> 1]);
+      if constexpr (n % 8 == 7) dma_one(t + STAGES - 1, 4 + n / 8);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+  };
+
+  // prologue: STAGES - 1 tiles in flight; tile 0 landed; its first operands read
+  for (int t = 0; t < STAGES - 1; t++) static_for<0, DMA>([&](auto n) __attribute__((always_inline)) { dma_one(t, n.value); });
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(DMA * (STAGES - 2), 15));
+  __syncthreads();
+  static_for<0, 8>([&](auto i) __attribute__((always_inline)) { read_a(0, i.value, A[0]); });
+  static_for<0, 4>([&](auto j) __attribute__((always_inline)) {
+    read_b(0, j.value, 0, B0[j.value]);
+    read_b(0, j.value, 1, B0[j.value]);
+  });
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+  int t = 0;
+  for (; t + 1 < nk; t += 2) {
+    tile(t, A[0], A[1]);
+    tile(t + 1, A[1], A[0]);
+  }
+  if (t < nk) tile(t, A[0], A[1]);
+  // the last matrix instructions have written their accumulators (the compiler does not know what the assembly issued)
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));  // the surplus loads land before the stages are reused
+  __syncthreads();                                  // every wavefront has read its last operands
+
+  // acc[i][j][v] is C(row 16 i + lane % 16, column 16 j + 4 (lane / 16) + v) of the wavefront's part
+  uint16_t *__restrict__ C = (uint16_t *)p.c;
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  constexpr int PITCH = 272;  // bytes per staged row of 128 columns
+  char *mine = smem + wave * (2 * 16 * PITCH);
+  // A fused epilogue evaluates the stored value with the ids of the Triton program that owns the element (Ep::BM x Ep::BN
+  // blocks; 0: no functor).  Blocks of 16 x 16 never straddle two owners, and a wavefront's 128 x 128 part has GI x GJ of
+  // them: they are looked up once each, and what the functor computes from the program's ids alone is then the same
+  // expression on the same values for every element of an owner, which the compiler evaluates once.  (Looked up per
+  // element, every one of the 256 evaluations per lane is separate code: a functor with the tutorial's grouped tile
+  // order and a bias per row and column took eight minutes to compile.)
+  constexpr int EBM = Ep::BM, EBN = Ep::BN;
+  constexpr bool OWNED = EBM >= 16 && EBN >= 16 && (128 % EBM == 0 || EBM % 128 == 0) && (128 % EBN == 0 || EBN % 128 == 0);
+  constexpr int GI = OWNED && EBM < 128 ? 128 / EBM : 1, GJ = OWNED && EBN < 128 ? 128 / EBN : 1;
+  int owner[GI][GJ];
+  if constexpr (OWNED)
+    static_for<0, GI * GJ>([&](auto gc) __attribute__((always_inline)) {
+      constexpr int gi = decltype(gc)::value / GJ, gj = decltype(gc)::value % GJ;
+      const int64_t r0 = m0 + wm * 128 + gi * (128 / GI), c0 = n0 + wn * 128 + gj * (128 / GJ);
+      owner[gi][gj] = (r0 < p.M && c0 < p.N) ? ep.tile_pid[(r0 / EBM) * ep.tiles_n + c0 / EBN] : 0;  // (outside C: nobody's)
+    });
+  auto value = [&](auto ic, auto jc, float a, int64_t row, int64_t col) __attribute__((always_inline)) -> float {
+    if constexpr (OWNED) return ep.at(owner[decltype(ic)::value * 16 / (128 / GI)][decltype(jc)::value * 16 / (128 / GJ)], a, (int)(row % EBM), (int)(col % EBN));
+    else return ep(a, row, col);
+  };
+  auto store_tile = [&](auto edge) __attribute__((always_inline)) {
+    // EDGE: the tile sticks out of C (ragged M, or N that is not a multiple of the tile): elements outside are neither
+    // evaluated (the functor may read a bias or a residual at the element's position) nor stored.
+    constexpr bool EDGE = decltype(edge)::value;
+    static_for<0, 8>([&](auto ic) __attribute__((always_inline)) {
+      constexpr int i = decltype(ic)::value;
+      char *reg = mine + (i & 1) * (16 * PITCH);
+      const int64_t er = m0 + wm * 128 + i * 16 + l16;
+      static_for<0, 8>([&](auto jc) __attribute__((always_inline)) {
+        constexpr int j = decltype(jc)::value;
+        const int64_t ec = n0 + wn * 128 + j * 16 + 4 * q;
+        float o[4];
+        static_for<0, 4>([&](auto vc) __attribute__((always_inline)) {
+          constexpr int v = decltype(vc)::value;
+          o[v] = (!EDGE || (er < p.M && ec + v < p.N)) ? value(ic, jc, acc[i][j][v], er, ec + v) : 0.f;
+        });
+        const f32x2_t p01 = {o[0], o[1]}, p23 = {o[2], o[3]};
+        uint2 w;
+        if (BF16) {
+          w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector(p01, bf16x2_t));
+          w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector(p23, bf16x2_t));
+        } else {
+          w.x = __builtin_bit_cast(uint32_t, __builtin_convertvector(p01, f16x2_t));
+          w.y = __builtin_bit_cast(uint32_t, __builtin_convertvector(p23, f16x2_t));
+        }
+        *reinterpret_cast<uint2 *>(reg + l16 * PITCH + (j * 16 + 4 * q) * 2) = w;
+      });
+      // (a wavefront's LDS accesses complete in order: its reads below see its writes above)
+      static_for<0, 4>([&](auto kc) __attribute__((always_inline)) {
+        constexpr int k = decltype(kc)::value;
+        const int id = k * 64 + lane, row = id >> 4, ch = id & 15;
+        const uint4 v = *reinterpret_cast<const uint4 *>(reg + row * PITCH + ch * 16);
+        const int64_t gr = m0 + wm * 128 + i * 16 + row, gc = n0 + wn * 128 + ch * 8;
+        // (rows of C need only be 4-byte aligned: a store of four dwords wants dword alignment, no more)
+        typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+        const u32x4_a4 w = {v.x, v.y, v.z, v.w};
+        if (!EDGE || (gr < p.M && gc < p.N)) __builtin_nontemporal_store(w, reinterpret_cast<u32x4_a4 *>(C + gr * p.ldc + gc));
+      });
+    });
+  };
+  // (with a functor only the guarded form is compiled: it is evaluated 256 times per lane, which is most of the code)
+  if (EBM > 0 || m0 + BM > p.M || n0 + BN > p.N) store_tile(EdgeTile<true>());
+  else if constexpr (EBM == 0) store_tile(EdgeTile<false>());
+}
+
 }  // namespace tts_gemm_device
 
 #ifdef TTS_GEMM_RTC
 extern "C" __global__ __launch_bounds__(256) void gemm_rtc(TtsGemmParams p, int tiles_m, int tiles_n, TtsEp ep) {
 #if TTS_GEMM_RTC == 0
-  tts_gemm_device::gemm_dma_body<TTS_GEMM_BF16 != 0, 4, 4>(p, tiles_m, tiles_n, ep);
+  tts_gemm_device::gemm_dma16_body<TTS_GEMM_BF16 != 0>(p, tiles_m, tiles_n, ep);
 #else
   tts_gemm_device::gemm_mfma_body<TTS_GEMM_BF16 != 0, 2, 2, 64>(p, tiles_m, tiles_n, ep);
 #endif

@@ -20,6 +20,7 @@ namespace {
 using namespace tts_gemm_device;
 
 struct IdentityEp {
+  static constexpr int BM = 0, BN = 0;  // (no owner to look up: see the generated functor, tile_codegen.cpp)
   __device__ __forceinline__ float operator()(float x, int64_t, int64_t) const { return x; }
 };
 
@@ -50,7 +51,9 @@ hipError_t launch_gemm_cfg(const GemmParams &p, hipStream_t s) {
 // the 256 registers two wavefronts of a SIMD can have each, which the 128 x 256 tile fits without spilling.
 template <bool BF16, int TM, int TN, bool BT, bool AT, bool PF, bool SK>
 __global__ __launch_bounds__(PF ? 320 : 256) void gemm_dma_kernel(GemmParams p, int tiles_m, int tiles_n) {
-  gemm_dma_body<BF16, TM, TN, IdentityEp, BT, AT, PF, SK>(of_batch(p, 2), tiles_m, tiles_n, IdentityEp());
+  // whole 256 x 256 tiles of row-major operands: the body on the 16 x 16 x 32 matrix instruction (gemm_device.h)
+  if constexpr (TM == 4 && TN == 4 && !BT && !AT && !PF && !SK) gemm_dma16_body<BF16>(of_batch(p, 2), tiles_m, tiles_n, IdentityEp());
+  else gemm_dma_body<BF16, TM, TN, IdentityEp, BT, AT, PF, SK>(of_batch(p, 2), tiles_m, tiles_n, IdentityEp());
 }
 
 // Adds the K slices' partial sums in slice order and narrows: four columns per thread (N is a multiple of 8).

@@ -114,7 +114,26 @@ struct Gen {
   static bool is_float(const std::string &t) { return t[0] == 'f' || t[0] == 'b'; }
 
   // ---- index expressions -------------------------------------------------
+  // name_index_exprs: every operation node of the pool becomes a local (`const long long x<id> = ...;` in index_locals,
+  // operands before their users), and ex() returns the local's name: a caller that evaluates its expression many times on
+  // the same leaves (the matrix-product epilogue, once per accumulator element) then has the shared part in one place.
+  bool name_index_exprs = false;
+  std::ostringstream index_locals;
+  std::map<int, std::string> named_exprs;
   std::string ex(int id) {
+    if (!name_index_exprs) return ex_text(id);
+    const EK k = P.pool.at(id).k;
+    if (k == EK::Const || k == EK::Arg || k == EK::Pid || k == EK::NProg || k == EK::IV || k == EK::Iter || k == EK::Result || k == EK::Data)
+      return ex_text(id);
+    auto it = named_exprs.find(id);
+    if (it != named_exprs.end()) return it->second;
+    const std::string text = ex_text(id);  // (names the operands first)
+    const std::string name = "x" + std::to_string(id);
+    index_locals << "    const long long " << name << " = " << text << ";\n";
+    named_exprs[id] = name;
+    return name;
+  }
+  std::string ex_text(int id) {
     const Expr &e = P.pool.at(id);
     auto w = [&](const std::string &s) { return e.bits == 32 ? "(long long)(int)(" + s + ")" : "(" + s + ")"; };
     auto u = [&](const char *op) {  // wrapping arithmetic through unsigned
@@ -133,8 +152,8 @@ struct Gen {
       case EK::Add: return u("+");
       case EK::Sub: return u("-");
       case EK::Mul: return u("*");
-      case EK::DivS: return w("sdiv(" + ex(e.a) + ", " + ex(e.b) + ")");
-      case EK::RemS: return w("srem(" + ex(e.a) + ", " + ex(e.b) + ")");
+      case EK::DivS: return e.bits == 32 ? "sdiv32(" + ex(e.a) + ", " + ex(e.b) + ")" : "(sdiv(" + ex(e.a) + ", " + ex(e.b) + "))";
+      case EK::RemS: return e.bits == 32 ? "srem32(" + ex(e.a) + ", " + ex(e.b) + ")" : "(srem(" + ex(e.a) + ", " + ex(e.b) + "))";
       case EK::MinS: return "smin(" + ex(e.a) + ", " + ex(e.b) + ")";
       case EK::MaxS: return "smax(" + ex(e.a) + ", " + ex(e.b) + ")";
       case EK::Sext: return ex(e.a);
@@ -1759,6 +1778,21 @@ __device__ inline long long smin(long long a, long long b) { return a < b ? a : 
 __device__ inline long long smax(long long a, long long b) { return a > b ? a : b; }
 __device__ inline long long sdiv(long long a, long long b) { return b == 0 ? 0 : a / b; }
 __device__ inline long long srem(long long a, long long b) { return b == 0 ? 0 : a % b; }
+// The same on 32-bit values (what the index arithmetic of a Triton program almost always is): one unsigned 32-bit division,
+// a tenth of the 64-bit one's instructions, and no branch, so that equal divisions of neighbouring code merge.  Truncates
+// toward zero, 0 for a zero divisor, and the most negative value over -1 wraps, as the 64-bit form does after narrowing.
+__device__ inline long long sdiv32(long long a, long long b) {
+  const int x = (int)a, y = (int)b;
+  const unsigned ux = x < 0 ? 0u - (unsigned)x : (unsigned)x, uy = y < 0 ? 0u - (unsigned)y : (unsigned)y;
+  const unsigned uq = ux / (uy == 0u ? 1u : uy);
+  return y == 0 ? 0LL : (long long)(int)((x ^ y) < 0 ? 0u - uq : uq);
+}
+__device__ inline long long srem32(long long a, long long b) {
+  const int x = (int)a, y = (int)b;
+  const unsigned ux = x < 0 ? 0u - (unsigned)x : (unsigned)x, uy = y < 0 ? 0u - (unsigned)y : (unsigned)y;
+  const unsigned ur = ux % (uy == 0u ? 1u : uy);
+  return y == 0 ? 0LL : (long long)(int)(x < 0 ? 0u - ur : ur);
+}
 __device__ inline long long wrap(long long x, long long m) { return m > 0 ? ((x % m) + m) % m : x; }
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef unsigned short u16x8_t __attribute__((ext_vector_type(8)));
@@ -1863,19 +1897,25 @@ std::string gemm_epilogue_source(const Program &p, const std::vector<const SOp *
         p.values.at(d->second->operands[0]).dtype == "f32")
       shown = d->second->operands[0];
   }
+  g.name_index_exprs = true;
   const std::string expr = g.at(shown, "i0", "i1");
   if (!g.fns.str().empty() || g.pool_bytes || g.out_bytes) throw Unsupported("an epilogue that needs more than one element at a time");
   std::string pre = TILE_PRELUDE;
   const std::string n = std::to_string(TILE_MAX_ARGS);
   for (size_t pos = 0; (pos = pre.find("%N%", pos)) != std::string::npos;) pre.replace(pos, 3, n);
   std::ostringstream all;
+  // `at`: the stored value of element (i0, i1) of the block of program q (its linear id); the call operator looks the owner
+  // of (row, col) up.  A kernel that knows which of its elements share an owner (BM, BN say how far one owner reaches)
+  // looks it up once for all of them and calls `at`, so that what depends on the program alone is computed once.
   all << pre << "struct TtsEp {\n  Args p;\n  const int *tile_pid;\n  int tiles_n, gx, gy, gz;\n"
-      << "  __device__ __forceinline__ float operator()(float acc, long long row, long long col) const {\n"
-      << "    const int i0 = (int)(row % " << BM << "), i1 = (int)(col % " << BN << ");\n"
-      << "    const int q = tile_pid[(row / " << BM << ") * tiles_n + col / " << BN << "];\n"
+      << "  static constexpr int BM = " << BM << ", BN = " << BN << ";\n"
+      << "  __device__ __forceinline__ float at(int q, float acc, int i0, int i1) const {\n"
       << "    const long long pidx = q % gx, pidy = (q / gx) % gy, pidz = q / (gx * gy), npx = gx, npy = gy, npz = gz;\n"
       << "    (void)i0; (void)i1; (void)pidx; (void)pidy; (void)pidz; (void)npx; (void)npy; (void)npz;\n"
-      << "    return " << expr << ";\n  }\n};\n";
+      << g.index_locals.str()
+      << "    return " << expr << ";\n  }\n"
+      << "  __device__ __forceinline__ float operator()(float acc, long long row, long long col) const {\n"
+      << "    return at(tile_pid[(row / BM) * tiles_n + col / BN], acc, (int)(row % BM), (int)(col % BN));\n  }\n};\n";
   return all.str();
 }
 
