@@ -356,6 +356,16 @@ static hipError_t rtc_compile_with(const std::string &source, const char *entry,
     return e;
   }
   if (!cached && !dir.empty()) write_file(dir, name, code);
+  if (getenv("TTS_RTC_REPORT")) {  // tuning aid: what the run-time compiler made of the kernel
+    int regs = -1, scratch = -1, lds = -1;
+    (void)hipFuncGetAttribute(&regs, HIP_FUNC_ATTRIBUTE_NUM_REGS, m->fn);
+    (void)hipFuncGetAttribute(&scratch, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, m->fn);
+    (void)hipFuncGetAttribute(&lds, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, m->fn);
+    int major = 0, minor = 0;
+    hiprtcVersion(&major, &minor);
+    fprintf(stderr, "tts rtc: %s: %d registers, %d bytes of scratch per lane, %d bytes of LDS, %zu bytes of code (%s, hipRTC %d.%d)\n", entry, regs,
+            scratch, lds, code.size(), cached ? "from the cache" : "compiled", major, minor);
+  }
   *out = m;
   return hipSuccess;
 }

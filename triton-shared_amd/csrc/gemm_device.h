@@ -768,7 +768,10 @@ __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m
 #endif
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds), "v"(voff), "s"(sbase) : "memory", "m0");
   };
-  auto dma_one = [&](int t, int n) __attribute__((always_inline)) {  // n < A_DMA: A part, else B part of tile t (past the last tile: the last again), into stage t % STAGES
+  // n < A_DMA: A part, else B part of tile t, into stage t % STAGES.  Loads past the last tile fetch the last tile again, so
+  // that the wait count is the same in every iteration (a scalar branch around every load and between two waits instead
+  // cost 5 us of 110: sixteen branches per tile in between the matrix instructions).
+  auto dma_one = [&](int t, int n) __attribute__((always_inline)) {
     const int tc = min(t, nk - 1);
     const uint32_t st = lds0 + (t % STAGES) * STAGE_BYTES;
     if (n < A_DMA) dma(a_base + (int64_t)tc * F_BK * 2, a_voff[n], st + (A_DMA * wave_u + n) * 1024);
@@ -800,7 +803,7 @@ __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m
     else
       asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(__builtin_bit_cast(u32x4_r, b)), "v"(__builtin_bit_cast(u32x4_r, a)));
   };
-  auto tile = [&](int t, uint4 (&Ac)[8], uint4 (&An)[8]) {
+  auto tile = [&](int t, uint4 (&Ac)[8], uint4 (&An)[8]) __attribute__((always_inline)) {
     static_for<0, 32>([&](auto slot) __attribute__((always_inline)) {
       constexpr int n = decltype(slot)::value;
       __builtin_amdgcn_sched_barrier(0);
@@ -835,15 +838,23 @@ __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m
   });
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
   int t = 0;
-  for (; t + 1 < nk; t += 2) {
+  for (; t + 1 < nk; t += 2) {  // two tiles per turn: A's register sets take turns
     tile(t, A[0], A[1]);
     tile(t + 1, A[1], A[0]);
   }
   if (t < nk) tile(t, A[0], A[1]);
-  // the last matrix instructions have written their accumulators (the compiler does not know what the assembly issued)
-  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));  // the surplus loads land before the stages are reused
-  __syncthreads();                                  // every wavefront has read its last operands
+  // The compiler does not know that the assembly above issued matrix instructions, so it leaves no wait states between
+  // one of them and a read of its result (the epilogue's, or a spill the register allocator places right behind the
+  // loop).  The sixteen accumulators the last tile wrote last pass through this statement, so whatever reads them comes
+  // after its wait states; the others were written at least sixteen instructions (256 cycles) earlier.
+  asm volatile("s_nop 15\n\ts_nop 15"
+               : "+a"(acc[4][4]), "+a"(acc[4][5]), "+a"(acc[4][6]), "+a"(acc[4][7]), "+a"(acc[5][4]), "+a"(acc[5][5]), "+a"(acc[5][6]), "+a"(acc[5][7]),
+                 "+a"(acc[6][4]), "+a"(acc[6][5]), "+a"(acc[6][6]), "+a"(acc[6][7]), "+a"(acc[7][4]), "+a"(acc[7][5]), "+a"(acc[7][6]), "+a"(acc[7][7])
+               :
+               : "memory");
+  // Every wavefront has read its last operands: the last tile's stage is free.  The other three still receive the surplus
+  // loads of the last iterations, which nobody waits for before the kernel's end.
+  __syncthreads();
 
   // acc[i][j][v] is C(row 16 i + lane % 16, column 16 j + 4 (lane / 16) + v) of the wavefront's part
   uint16_t *__restrict__ C = (uint16_t *)p.c;
@@ -851,7 +862,10 @@ __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m
   typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
   typedef float f32x2_t __attribute__((ext_vector_type(2)));
   constexpr int PITCH = 272;  // bytes per staged row of 128 columns
-  char *mine = smem + wave * (2 * 16 * PITCH);
+  // (one patch of 16 rows per wavefront, in the last tile's stage; a wavefront's LDS accesses complete in order, so the
+  // next 16 rows' writes come after this 16 rows' reads)
+  static_assert(4 * 16 * PITCH <= STAGE_BYTES, "the four wavefronts' patches fit one stage");
+  char *mine = smem + ((nk + STAGES - 1) % STAGES) * STAGE_BYTES + wave * (16 * PITCH);
   // A fused epilogue evaluates the stored value with the ids of the Triton program that owns the element (Ep::BM x Ep::BN
   // blocks; 0: no functor).  Blocks of 16 x 16 never straddle two owners, and a wavefront's 128 x 128 part has GI x GJ of
   // them: they are looked up once each, and what the functor computes from the program's ids alone is then the same
@@ -872,21 +886,28 @@ __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m
     if constexpr (OWNED) return ep.at(owner[decltype(ic)::value * 16 / (128 / GI)][decltype(jc)::value * 16 / (128 / GJ)], a, (int)(row % EBM), (int)(col % EBN));
     else return ep(a, row, col);
   };
+  // this lane's chunk of row lane / 16 of the wavefront's part
+  uint16_t *c_lane = C + (m0 + wm * 128 + (lane >> 4)) * p.ldc + n0 + wn * 128 + (lane & 15) * 8;
   auto store_tile = [&](auto edge) __attribute__((always_inline)) {
     // EDGE: the tile sticks out of C (ragged M, or N that is not a multiple of the tile): elements outside are neither
     // evaluated (the functor may read a bias or a residual at the element's position) nor stored.
     constexpr bool EDGE = decltype(edge)::value;
+    // rows and columns of the wavefront's part that lie inside C (N is a multiple of 8: a lane's four columns, and a
+    // stored chunk's eight, are inside or outside together)
+    const int rows_left = (int)min((int64_t)128, p.M - (m0 + wm * 128)), cols_left = (int)min((int64_t)128, p.N - (n0 + wn * 128));
     static_for<0, 8>([&](auto ic) __attribute__((always_inline)) {
       constexpr int i = decltype(ic)::value;
-      char *reg = mine + (i & 1) * (16 * PITCH);
+      char *reg = mine;
       const int64_t er = m0 + wm * 128 + i * 16 + l16;
+      const bool row_in = !EDGE || i * 16 + l16 < rows_left;
       static_for<0, 8>([&](auto jc) __attribute__((always_inline)) {
         constexpr int j = decltype(jc)::value;
         const int64_t ec = n0 + wn * 128 + j * 16 + 4 * q;
+        const bool in = !EDGE || (row_in && j * 16 + 4 * q < cols_left);
         float o[4];
         static_for<0, 4>([&](auto vc) __attribute__((always_inline)) {
           constexpr int v = decltype(vc)::value;
-          o[v] = (!EDGE || (er < p.M && ec + v < p.N)) ? value(ic, jc, acc[i][j][v], er, ec + v) : 0.f;
+          o[v] = in ? value(ic, jc, acc[i][j][v], er, ec + v) : 0.f;
         });
         const f32x2_t p01 = {o[0], o[1]}, p23 = {o[2], o[3]};
         uint2 w;
@@ -900,21 +921,25 @@ __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m
         *reinterpret_cast<uint2 *>(reg + l16 * PITCH + (j * 16 + 4 * q) * 2) = w;
       });
       // (a wavefront's LDS accesses complete in order: its reads below see its writes above)
+      uint4 chunk[4];
       static_for<0, 4>([&](auto kc) __attribute__((always_inline)) {
         constexpr int k = decltype(kc)::value;
-        const int id = k * 64 + lane, row = id >> 4, ch = id & 15;
-        const uint4 v = *reinterpret_cast<const uint4 *>(reg + row * PITCH + ch * 16);
-        const int64_t gr = m0 + wm * 128 + i * 16 + row, gc = n0 + wn * 128 + ch * 8;
+        chunk[k] = *reinterpret_cast<const uint4 *>(reg + (4 * k + (lane >> 4)) * PITCH + (lane & 15) * 16);
+      });
+      static_for<0, 4>([&](auto kc) __attribute__((always_inline)) {
+        constexpr int k = decltype(kc)::value;
+        const int row = 4 * k + (lane >> 4), ch = lane & 15;  // row of the sixteen, 16-byte chunk of the row
         // (rows of C need only be 4-byte aligned: a store of four dwords wants dword alignment, no more)
         typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
-        const u32x4_a4 w = {v.x, v.y, v.z, v.w};
-        if (!EDGE || (gr < p.M && gc < p.N)) __builtin_nontemporal_store(w, reinterpret_cast<u32x4_a4 *>(C + gr * p.ldc + gc));
+        const u32x4_a4 w = {chunk[k].x, chunk[k].y, chunk[k].z, chunk[k].w};
+        if (!EDGE || (i * 16 + row < rows_left && ch * 8 < cols_left))
+          __builtin_nontemporal_store(w, reinterpret_cast<u32x4_a4 *>(c_lane + (int64_t)(i * 16 + 4 * k) * p.ldc));
       });
     });
   };
-  // (with a functor only the guarded form is compiled: it is evaluated 256 times per lane, which is most of the code)
-  if (EBM > 0 || m0 + BM > p.M || n0 + BN > p.N) store_tile(EdgeTile<true>());
-  else if constexpr (EBM == 0) store_tile(EdgeTile<false>());
+  if (m0 + BM > p.M || n0 + BN > p.N) store_tile(EdgeTile<true>());
+  else store_tile(EdgeTile<false>());
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));  // the surplus loads land before the LDS goes away
 }
 
 }  // namespace tts_gemm_device
