@@ -245,14 +245,15 @@ def make_workloads(torch, triton, K):
         return dict(desc=f"stream ceiling, 1:1 read/write: z = x fp32 N={n}, BLOCK=4096 (fused map with no ops)", work=8 * n, bound="hbm",
                     dtype="f32", make=make, set_bytes=8 * n)
 
-    def runtime_copy(n):
+    def runtime_copy(n, like=None):
         # the HIP runtime's own device-to-device copy (what torch.Tensor.copy_ enqueues for two contiguous tensors of one
         # type): a mover this backend did not write, as an independent figure for what a 1:1 stream reaches on the machine
         def make():
             x = torch.rand(n, device=dev)
             z = torch.empty_like(x)
             return dict(direct=lambda: z.copy_(x), kernel="hipMemcpyAsync device-to-device (the runtime's copy kernel, not this backend)")
-        return dict(desc=f"independent stream ceiling, 1:1 read/write: the HIP runtime's device-to-device copy of fp32 N={n} (not a kernel of this backend)",
+        what = f" -- the bytes {like} moves, as a plain copy" if like else ""
+        return dict(desc=f"independent stream ceiling, 1:1 read/write: the HIP runtime's device-to-device copy of fp32 N={n} (not a kernel of this backend){what}",
                     work=8 * n, bound="hbm", dtype="f32", make=make, set_bytes=8 * n)
 
     def stream_read(n):
@@ -274,6 +275,10 @@ def make_workloads(torch, triton, K):
     W["stream_copy_2p28"] = stream_copy(1 << 28)
     W["stream_read_2p28"] = stream_read(1 << 28)
     W["stream_runtime_copy_2p28"] = runtime_copy(1 << 28)
+    # what a 1:1 stream reaches falls with its footprint (0.75 of the 8 TB/s figure up to 1 GiB moved, 0.69 from 6 GiB on):
+    # the same footprints as the two row-wise configurations, moved by the runtime's copy
+    W["stream_runtime_copy_as_cfg2_1m"] = runtime_copy(781 << 20, like="cfg2_1m")
+    W["stream_runtime_copy_as_cfg3"] = runtime_copy(4096 * 8192 // 2, like="cfg3")
     W["next_fused_gelu_2p26"] = fused_gelu(1 << 26)
     W["next_fused_silu_2p26"] = fused_silu(1 << 26)
     W["next_rotary_8192x32x128"] = rotary(8192, 32, 64)

@@ -1218,3 +1218,29 @@ def while_inside_for(x_ptr, out_ptr, n, BLOCK: tl.constexpr):
             acc += tl.load(x_ptr + offs) * k
             k = k // 2
     tl.store(out_ptr + offs, acc)
+
+
+@triton.jit
+def grid_stamp(out_ptr, BLOCK: tl.constexpr):
+    # every program writes a block of integers made from its ids and the grid's extents: what a launch hands to
+    # program_id / num_programs on each axis, whatever the extents are
+    x = tl.program_id(0)
+    y = tl.program_id(1)
+    z = tl.program_id(2)
+    nx = tl.num_programs(0)
+    ny = tl.num_programs(1)
+    offs = tl.arange(0, BLOCK)
+    lin = (z * ny + y) * nx + x
+    vals = x * 1000003 + y * 7 + z * 131 + offs * 3 + tl.num_programs(2)
+    tl.store(out_ptr + lin * BLOCK + offs, vals)
+
+
+@triton.jit
+def add_rows_2d(x_ptr, y_ptr, z_ptr, n_cols, BLOCK: tl.constexpr):
+    # z = x + y on [rows, n_cols]: column blocks on program_id(0), rows on program_id(1)
+    row = tl.program_id(1)
+    cols = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    mask = cols < n_cols
+    a = tl.load(x_ptr + row * n_cols + cols, mask=mask)
+    b = tl.load(y_ptr + row * n_cols + cols, mask=mask)
+    tl.store(z_ptr + row * n_cols + cols, a + b, mask=mask)

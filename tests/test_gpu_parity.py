@@ -1946,3 +1946,42 @@ def test_gemm_with_fused_epilogue(M, N, K, kernel, dtype):
     z = a.double() @ b.double()
     want = z * torch.sigmoid(z * 0.25)
     assert ((c.double() - want).norm() / want.norm()) <= 1e-2
+
+
+# ------------------------------------------------------------------ grids beyond the device's extents
+def test_grid_extents_beyond_the_device_limit():
+    """The reference's launcher loops over any grid (backend/driver.py:116-133); the device's grid holds 65535 along y and
+    z.  A (3, 70000) grid and a (2, 3, 66000) one run as one-dimensional launches whose kernels number the programs
+    themselves: every program must see its own ids and the grid's extents (closed form; the small grid of the same kernel
+    is checked against the lane interpreter as well)."""
+    import extra_kernels as X
+    from oracle import ttir_lanes
+    BLOCK = 16
+
+    def expect(gx, gy, gz):
+        z, y, x, o = np.meshgrid(np.arange(gz), np.arange(gy), np.arange(gx), np.arange(BLOCK), indexing="ij")
+        return (x * 1000003 + y * 7 + z * 131 + o * 3 + gz).astype(np.int32).reshape(-1)
+
+    for grid in [(3, 5, 2), (3, 70000, 1), (2, 3, 66000)]:
+        gx, gy, gz = grid
+        out = torch.full((gx * gy * gz * BLOCK + 8,), -1, dtype=torch.int32, device=DEV)
+        k = X.grid_stamp[grid](out, BLOCK=BLOCK)
+        torch.cuda.synchronize()
+        assert k.function.family == "tile_program"
+        got = out.cpu().numpy()
+        assert np.array_equal(got[:-8], expect(gx, gy, gz)), grid
+        assert (got[-8:] == -1).all()
+        if grid == (3, 5, 2):
+            mem = {0: np.full(gx * gy * gz * BLOCK, -1, np.int32)}
+            ttir_lanes.Interpreter(k.asm["ttir"]).run(grid, [None], mem)
+            assert np.array_equal(mem[0], expect(gx, gy, gz))
+    # the hand-written elementwise family (or the compiled fused map, whichever takes it) on rows along program_id(1)
+    rows, n_cols = 66000, 1500
+    g = torch.Generator(device="cpu").manual_seed(1)
+    x = torch.rand(rows, n_cols, generator=g).to(DEV)
+    y = torch.rand(rows, n_cols, generator=g).to(DEV)
+    z = torch.full((rows, n_cols), -1.0, device=DEV)
+    k = X.add_rows_2d[(triton.cdiv(n_cols, 1024), rows)](x, y, z, n_cols, BLOCK=1024)
+    torch.cuda.synchronize()
+    assert k.function.family in ("map1d", "fused_map"), k.function.family
+    assert torch.equal(z, x + y)     # one IEEE addition per element: bit for bit

@@ -714,7 +714,9 @@ __device__ __forceinline__ void static_for(F &&f) {
   }
 }
 
-template <bool BF16, class Ep>
+// SK: the grid holds p.split workgroups per tile; workgroup (tile, s) walks the s-th share of the K tiles and leaves its fp32
+// sums in p.partial (a lane's four consecutive columns of a row are one 16-byte store, straight from the registers).
+template <bool BF16, class Ep, bool SK = false>
 __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m, int tiles_n, const Ep &ep) {
   using T = DmaTile<4, 4>;
   constexpr int BM = T::BM, BN = T::BN, STAGES = T::STAGES, A_BYTES = T::A_BYTES, STAGE_BYTES = T::STAGE_BYTES, ROWB = T::B_ROW_BYTES;
@@ -731,6 +733,8 @@ __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m
 
   int bid = blockIdx.x;
   const int nwg = tiles_m * tiles_n;
+  const int slice = SK ? bid / nwg : 0;
+  if (SK) bid -= slice * nwg;
   if (nwg % 8 == 0) bid = (bid % 8) * (nwg / 8) + bid / 8;  // consecutive ids on one XCD
   const int group = 4 * tiles_n;                             // 4-tile-tall column groups
   const int g0 = (bid / group) * 4;
@@ -739,7 +743,9 @@ __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m
   const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
   const char *a_base = (const char *)((const uint16_t *)p.a + m0 * p.lda);
   const char *b_base = (const char *)((const uint16_t *)p.b + n0);
-  const int nk = (int)(p.K / F_BK);
+  const int nk_all = (int)(p.K / F_BK);
+  const int k_begin = SK ? (int)((int64_t)slice * nk_all / p.split) : 0;
+  const int nk = SK ? (int)((int64_t)(slice + 1) * nk_all / p.split) - k_begin : nk_all;
 
   uint32_t a_voff[A_DMA], b_voff[B_DMA];
 #pragma unroll
@@ -772,7 +778,7 @@ __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m
   // that the wait count is the same in every iteration (a scalar branch around every load and between two waits instead
   // cost 5 us of 110: sixteen branches per tile in between the matrix instructions).
   auto dma_one = [&](int t, int n) __attribute__((always_inline)) {
-    const int tc = min(t, nk - 1);
+    const int tc = min(t, nk - 1) + k_begin;
     const uint32_t st = lds0 + (t % STAGES) * STAGE_BYTES;
     if (n < A_DMA) dma(a_base + (int64_t)tc * F_BK * 2, a_voff[n], st + (A_DMA * wave_u + n) * 1024);
     else dma(b_base + (int64_t)tc * F_BK * p.ldb * 2, b_voff[n - A_DMA], st + A_BYTES + (B_DMA * wave_u + n - A_DMA) * 1024);
@@ -857,6 +863,16 @@ __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m
   __syncthreads();
 
   // acc[i][j][v] is C(row 16 i + lane % 16, column 16 j + 4 (lane / 16) + v) of the wavefront's part
+  if constexpr (SK) {
+    float *__restrict__ part = p.partial + (int64_t)slice * p.M * p.N;
+    static_for<0, 64>([&](auto bc) __attribute__((always_inline)) {
+      constexpr int i = decltype(bc)::value / 8, j = decltype(bc)::value % 8;
+      const int64_t row = m0 + wm * 128 + i * 16 + l16, col = n0 + wn * 128 + j * 16 + 4 * q;
+      if (row < p.M && col < p.N) *reinterpret_cast<f32x4 *>(part + row * p.N + col) = acc[i][j];  // (N is a multiple of 8)
+    });
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));  // the surplus loads land before the LDS goes away
+    return;
+  }
   uint16_t *__restrict__ C = (uint16_t *)p.c;
   typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
   typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));

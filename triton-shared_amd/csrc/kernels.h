@@ -29,6 +29,7 @@ struct Map1DParams {
   int masked;
   int op;    // 0 add 1 sub 2 mul 3 div 4 maximum 5 minimum
   int swap;  // operands of `op` are (y, x)
+  int lin_gx = 0, lin_gy = 0;  // set by the launch: a one-dimensional launch numbers the programs of a grid this wide and tall itself
 };
 hipError_t launch_map1d(const Map1DParams &p, int gx, int gy, int gz, hipStream_t s, const char **kernel_name);
 
@@ -86,6 +87,7 @@ struct LayerNormParams {
   int64_t N;
   float eps;
   int elem_kind;  // the element type of x, y, w and b: 0 fp16, 1 bf16, 2 fp32
+  int lin_gx = 0, lin_gy = 0;  // set by the launch: a one-dimensional launch numbers the programs of a grid this wide and tall itself
 };
 hipError_t launch_layernorm(const LayerNormParams &p, int gx, int gy, int gz, hipStream_t s, const char **kernel_name);
 

@@ -52,7 +52,7 @@ hipError_t launch_gemm_cfg(const GemmParams &p, hipStream_t s) {
 template <bool BF16, int TM, int TN, bool BT, bool AT, bool PF, bool SK>
 __global__ __launch_bounds__(PF ? 320 : 256) void gemm_dma_kernel(GemmParams p, int tiles_m, int tiles_n) {
   // whole 256 x 256 tiles of row-major operands: the body on the 16 x 16 x 32 matrix instruction (gemm_device.h)
-  if constexpr (TM == 4 && TN == 4 && !BT && !AT && !PF && !SK) gemm_dma16_body<BF16>(of_batch(p, 2), tiles_m, tiles_n, IdentityEp());
+  if constexpr (TM == 4 && TN == 4 && !BT && !AT && !PF) gemm_dma16_body<BF16, IdentityEp, SK>(of_batch(p, 2), tiles_m, tiles_n, IdentityEp());
   else gemm_dma_body<BF16, TM, TN, IdentityEp, BT, AT, PF, SK>(of_batch(p, 2), tiles_m, tiles_n, IdentityEp());
 }
 

@@ -26,6 +26,26 @@ __device__ __forceinline__ int64_t affine(const Affine &a, int px, int py, int p
   return a.c0 + a.c[0] * px + a.c[1] * py + a.c[2] * pz;
 }
 
+// The program a workgroup runs.  The device's grid holds 65535 along y and z, the reference's launcher loops over any
+// extents (backend/driver.py:116-133): for such grids the launch is one-dimensional and the kernel numbers the programs
+// itself, x fastest (lin_gx != 0).
+struct ProgramId {
+  int x, y, z;
+};
+__device__ __forceinline__ ProgramId program_id(int lin_gx, int lin_gy) {
+  if (!lin_gx) return {(int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z};
+  const int64_t lin = blockIdx.x;
+  return {(int)(lin % lin_gx), (int)((lin / lin_gx) % lin_gy), (int)(lin / ((int64_t)lin_gx * lin_gy))};
+}
+// the launch grid for gx x gy x gz programs (and what the kernel needs to number them)
+template <class P>
+dim3 program_grid(P &p, int gx, int gy, int gz) {
+  if (gy <= 65535 && gz <= 65535) return dim3(gx, gy, gz);
+  p.lin_gx = gx;
+  p.lin_gy = gy;
+  return dim3((unsigned)((int64_t)gx * gy * gz));
+}
+
 // Wavefront reductions with DPP cross-lane operands (no LDS round trips): quad swaps, half-row and
 // row mirrors leave every lane of a 16-lane row with the row's result; row_bcast15 / row_bcast31 fold
 // the four rows into lane 63, which is then broadcast.  Lanes a step does not write take the
@@ -89,7 +109,8 @@ __device__ __forceinline__ void ntstore(float4 *p, float4 v) {
 
 template <int OP, bool SWAP>
 __global__ __launch_bounds__(256) void map1d_f32_kernel(Map1DParams p) {
-  const int px = blockIdx.x, py = blockIdx.y, pz = blockIdx.z;
+  const ProgramId id = program_id(p.lin_gx, p.lin_gy);
+  const int px = id.x, py = id.y, pz = id.z;
   const float *__restrict__ x = p.x + affine(p.xo, px, py, pz);
   const float *__restrict__ y = p.y + affine(p.yo, px, py, pz);
   float *__restrict__ z = p.z + affine(p.zo, px, py, pz);
@@ -163,9 +184,8 @@ __device__ __forceinline__ float block_sum_256(float v, float *red) {
 // ---------------------------------------------------------------- softmax
 // T threads share one row; thread t holds elements t, t+T, ... (NPL of them).
 // VEC (block == NPL * T, NPL % 4 == 0, d_in >= 4): thread t holds the four-element chunks t, t+T, ...
-// instead and moves each with one 16-byte access.  Rows need no 16-byte alignment for that (global
-// accesses of several dwords only need dword alignment).  Every load is unconditional: a chunk that
-// sticks out of the row is read from the row's last four elements and shifted into place.
+// of a grid laid on the 16-byte boundaries of memory instead, and moves each with one aligned 16-byte
+// access (the grid starts up to three elements before the row; see the loads below).
 typedef float f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
 // IO: the element type of the rows in memory (0 fp16, 1 bf16, 2 fp32); a 16-bit row is widened after the load and narrowed
@@ -197,6 +217,8 @@ __global__ __launch_bounds__(WG) void softmax_f32_kernel(SoftmaxParams p, int gx
   const E *__restrict__ in = (const E *)p.in + affine(p.in_off, px, py, pz);
   E *__restrict__ out = (E *)p.out + affine(p.out_off, px, py, pz);
   const int d_in = active ? (int)p.d_in : 0, d_out = active ? (int)p.d_out : 0;
+  // fp32 rows moved in 16-byte chunks: elements between the 16-byte boundary at or below the row's start and the row
+  const int lead = (VEC && IO == 2 && active) ? (int)(((uintptr_t)in >> 2) & 3) : 0;
   // lanes beyond d_in hold `other` and take part in the reductions, as a filled
   // tile does; lanes beyond the block do not exist
   float v[NPL];
@@ -215,24 +237,24 @@ __global__ __launch_bounds__(WG) void softmax_f32_kernel(SoftmaxParams p, int gx
       }
     }
   } else if constexpr (VEC) {
-    const int last = max(d_in - 4, 0);  // inactive rows (d_in == 0) read the first row's start and store nothing
-    f32x4_a4 win[NPL / 4];
-#pragma unroll
-    for (int j = 0; j < NPL / 4; j++) win[j] = *reinterpret_cast<const f32x4_a4 *>(in + min(4 * (t + j * T), last));
+    // The chunk grid lies on 16-byte boundaries of memory: it starts `lead` elements before the row (rows of 781 floats are
+    // 3124 bytes apart, so a row starts 0, 4, 8 or 12 bytes past a boundary), every chunk is one aligned 16-byte load, and
+    // chunks past the row's end are not loaded at all.  Slots outside the row -- before its first element, after its last
+    // -- hold `other`: together they are the block's padding, block - d_in slots, as in a filled tile.  (The bytes read
+    // before the row and after it lie in the same aligned 16 bytes as an element of the row, so they are mapped.)
+    const f32x4_t *grid = reinterpret_cast<const f32x4_t *>(in - lead);
+    const int slots = lead + d_in;
+    f32x4_t win[NPL / 4];
 #pragma unroll
     for (int j = 0; j < NPL / 4; j++) {
-      const int i0 = 4 * (t + j * T);
-      const int shift = i0 - min(i0, last);  // chunk element c is window[c + shift]
-      const f32x4_a4 w = win[j];
+      win[j] = (f32x4_t){p.other, p.other, p.other, p.other};
+      if (4 * (t + j * T) < slots) win[j] = grid[t + j * T];
+    }
 #pragma unroll
-      for (int c = 0; c < 4; c++) {
-        float x = p.other;
-        if (shift == 0) x = w[c];
+    for (int j = 0; j < NPL / 4; j++) {
+      const int s0 = 4 * (t + j * T);
 #pragma unroll
-        for (int sft = 1; sft < 4; sft++)
-          if (c + sft < 4 && shift == sft) x = w[c + sft];
-        v[4 * j + c] = i0 + c < d_in ? x : p.other;
-      }
+      for (int c = 0; c < 4; c++) v[4 * j + c] = (s0 + c >= lead && s0 + c < slots) ? win[j][c] : p.other;
     }
   } else {
 #pragma unroll
@@ -283,17 +305,21 @@ __global__ __launch_bounds__(WG) void softmax_f32_kernel(SoftmaxParams p, int gx
       if (i0 < d_out) ntstore(reinterpret_cast<uint4 *>(out + i0), make_uint4(o[0], o[1], o[2], o[3]));
     }
   } else if constexpr (VEC) {
+    // slot s of the grid is element s - lead of the row; the output row's chunks are aligned stores when it sits at the
+    // same offset from a 16-byte boundary as the input row (dword-aligned ones otherwise)
+    E *ogrid = out - lead;
+    const int oslots = lead + d_out;
 #pragma unroll
     for (int j = 0; j < NPL / 4; j++) {
-      const int i0 = 4 * (t + j * T);
+      const int s0 = 4 * (t + j * T);
       f32x4_a4 w;
 #pragma unroll
       for (int c = 0; c < 4; c++) w[c] = v[4 * j + c] * rsum;
-      if (i0 + 4 <= d_out) __builtin_nontemporal_store(w, reinterpret_cast<f32x4_a4 *>(out + i0));
+      if (s0 >= lead && s0 + 4 <= oslots) __builtin_nontemporal_store(w, reinterpret_cast<f32x4_a4 *>(ogrid + s0));
       else
 #pragma unroll
         for (int c = 0; c < 4; c++)
-          if (i0 + c < d_out) out[i0 + c] = w[c];
+          if (s0 + c >= lead && s0 + c < oslots) ogrid[s0 + c] = w[c];
     }
   } else {
 #pragma unroll
@@ -311,7 +337,13 @@ hipError_t launch_softmax_io(const SoftmaxParams &p, int gx, int gy, int gz, hip
   dim3 grid((unsigned)((programs + rows_per_wg - 1) / rows_per_wg));
   constexpr int EPC = IO == 2 ? 4 : 8;  // elements per 16-byte chunk
   constexpr bool CAN_VEC = NPL % EPC == 0;
-  bool vec = CAN_VEC && p.block == NPL * WAVES * WAVE && p.d_in >= 4;
+  // (fp32: a row's chunk grid starts up to 3 elements before the row and its NPL * T slots must hold the row as well: rows
+  // that fill the block to its last three elements must start on 16-byte boundaries, all of them)
+  auto rows_on_boundaries = [&](const Affine &a, const void *base) {
+    return (a.c0 | a.c[0] | a.c[1] | a.c[2]) % 4 == 0 && ((uintptr_t)base & 15) == 0;
+  };
+  bool vec = CAN_VEC && p.block == NPL * WAVES * WAVE && p.d_in >= 4 &&
+             (IO != 2 || p.d_in + 3 <= p.block || rows_on_boundaries(p.in_off, p.in));
   if (IO != 2) {  // whole chunks of aligned rows only
     auto aligned = [](const Affine &a) { return (a.c0 | a.c[0] | a.c[1] | a.c[2]) % 8 == 0; };
     vec = vec && p.d_in % 8 == 0 && p.d_out % 8 == 0 && aligned(p.in_off) && aligned(p.out_off) && (((uintptr_t)p.in | (uintptr_t)p.out) & 15) == 0;
@@ -382,7 +414,8 @@ __global__ __launch_bounds__(256, CPT <= 4 ? 8 : 4) void layernorm_fwd_kernel(La
   using E = typename T::elem;
   constexpr int EPC = T::EPC;
   __shared__ float red[4];
-  const int px = blockIdx.x, py = blockIdx.y, pz = blockIdx.z;
+  const ProgramId id = program_id(p.lin_gx, p.lin_gy);
+  const int px = id.x, py = id.y, pz = id.z;
   const E *__restrict__ x = (const E *)p.x + affine(p.x_off, px, py, pz);
   const E *__restrict__ w = (const E *)p.w + affine(p.w_off, px, py, pz);
   const E *__restrict__ b = (const E *)p.b + affine(p.b_off, px, py, pz);
@@ -588,7 +621,8 @@ __global__ __launch_bounds__(256) void layernorm_fwd_long_kernel(LayerNormParams
   using T = LnType<KIND>;
   using E = typename T::elem;
   __shared__ float red[4];
-  const int px = blockIdx.x, py = blockIdx.y, pz = blockIdx.z;
+  const ProgramId id = program_id(p.lin_gx, p.lin_gy);
+  const int px = id.x, py = id.y, pz = id.z;
   const E *__restrict__ x = (const E *)p.x + affine(p.x_off, px, py, pz);
   const E *__restrict__ w = (const E *)p.w + affine(p.w_off, px, py, pz);
   const E *__restrict__ b = (const E *)p.b + affine(p.b_off, px, py, pz);
@@ -639,7 +673,7 @@ hipError_t launch_layernorm_t(const LayerNormParams &p, dim3 grid, hipStream_t s
     min_rows = 2 * (int64_t)persistent_grid;
   }
   auto row_invariant = [](const Affine &a) { return (a.c[0] | a.c[1] | a.c[2]) == 0; };
-  if (fast && cpt && persistent_grid > 0 && grid.y == 1 && grid.z == 1 && (int64_t)grid.x >= min_rows && row_invariant(p.w_off) &&
+  if (fast && cpt && persistent_grid > 0 && !p.lin_gx && grid.y == 1 && grid.z == 1 && (int64_t)grid.x >= min_rows && row_invariant(p.w_off) &&
       row_invariant(p.b_off)) {
     const int rows = (int)grid.x;
     const dim3 pg((unsigned)persistent_grid);
@@ -885,8 +919,9 @@ hipError_t launch_mapn_n(const MapNParams &p, dim3 grid, hipStream_t s) {
 
 }  // namespace
 
-hipError_t launch_map1d(const Map1DParams &p, int gx, int gy, int gz, hipStream_t s, const char **name) {
-  dim3 grid(gx, gy, gz);
+hipError_t launch_map1d(const Map1DParams &params, int gx, int gy, int gz, hipStream_t s, const char **name) {
+  Map1DParams p = params;
+  const dim3 grid = program_grid(p, gx, gy, gz);
   *name = "map1d_f32_kernel";
   switch (p.op) {
     case 0: return launch_map1d_op<0>(p, grid, s);
@@ -931,8 +966,9 @@ hipError_t launch_softmax(const SoftmaxParams &p, int gx, int gy, int gz, hipStr
   return hipErrorInvalidValue;
 }
 
-hipError_t launch_layernorm(const LayerNormParams &p, int gx, int gy, int gz, hipStream_t s, const char **name) {
-  dim3 grid(gx, gy, gz);
+hipError_t launch_layernorm(const LayerNormParams &params, int gx, int gy, int gz, hipStream_t s, const char **name) {
+  LayerNormParams p = params;
+  const dim3 grid = program_grid(p, gx, gy, gz);
   return p.elem_kind == 2 ? launch_layernorm_t<2>(p, grid, s, name) : p.elem_kind == 1 ? launch_layernorm_t<1>(p, grid, s, name) : launch_layernorm_t<0>(p, grid, s, name);
 }
 

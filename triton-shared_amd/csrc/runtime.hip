@@ -701,17 +701,21 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
     auto b = resolve(plan, gx, gy, gz, args, n);
     const Plan &pl = plan->plan;
     {
-      // the compiled fused map numbers its programs itself (a one-dimensional launch); the others use the device's grid
+      // The device's grid holds 65535 along y and z; the reference's launcher loops over any extents
+      // (backend/driver.py:116-133).  For larger ones every family launches one-dimensionally and numbers its programs
+      // itself, as the compiled fused map and the row softmax always do (the matrix products use tilings of their own);
+      // only the fused map's interpreter (a tuning aid) is left out.
       const char *mode = getenv("TTS_FUSED_MAP");
-      const bool own_numbering = pl.family == Family::FusedMap && !b->fallback && !(mode && std::string(mode) == "interpreter");
-      if ((gy > 65535 || gz > 65535) && !own_numbering) throw Unsupported("grid y/z extents above 65535");
+      const bool interpreter = pl.family == Family::FusedMap && !b->fallback && mode && std::string(mode) == "interpreter";
+      if ((gy > 65535 || gz > 65535) && interpreter) throw Unsupported("grid y/z extents above 65535 on the fused map's interpreter");
+      if ((int64_t)gx * gy * gz > INT32_MAX) throw Unsupported("more than 2^31 - 1 programs in a launch");
     }
     hipStream_t s = (hipStream_t)stream;
     hipError_t err = hipSuccess;
     const char *kname = "";
     // one workgroup of 256 threads per Triton program, on the kernel generated for the program (compiled at its first use)
     auto run_tile_program = [&](RtcModule **slot, const std::string &source) -> tts_status {
-      struct { void *ptr[TILE_MAX_ARGS]; long long ival[TILE_MAX_ARGS]; double fval[TILE_MAX_ARGS]; int swap_xy; } a{};
+      struct { void *ptr[TILE_MAX_ARGS]; long long ival[TILE_MAX_ARGS]; double fval[TILE_MAX_ARGS]; int swap_xy, lgx, lgy, lgz; } a{};
       for (int i = 0; i < n; i++) {
         if (args[i].kind == TTS_ARG_PTR) a.ptr[i] = args[i].v.ptr;
         else if (args[i].kind == TTS_ARG_INT) a.ival[i] = args[i].v.i;
@@ -729,7 +733,13 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
       kname = "tile_program (hipRTC)";
       // the program asks for neighbouring workgroups along program_id(1) (tile_codegen.cpp); grid.y holds 65535 at most
       a.swap_xy = tile_program_swaps_grid(source) && gy > 1 && gx <= 65535 ? 1 : 0;
-      err = a.swap_xy ? rtc_launch(*slot, gy, gx, gz, 256, &a, sizeof a, s) : rtc_launch(*slot, gx, gy, gz, 256, &a, sizeof a, s);
+      if ((a.swap_xy ? gx : gy) > 65535 || gz > 65535) {  // the kernel numbers the programs itself (x fastest)
+        a.swap_xy = 0;
+        a.lgx = gx; a.lgy = gy; a.lgz = gz;
+        err = rtc_launch(*slot, (int)((int64_t)gx * gy * gz), 1, 1, 256, &a, sizeof a, s);
+      } else {
+        err = a.swap_xy ? rtc_launch(*slot, gy, gx, gz, 256, &a, sizeof a, s) : rtc_launch(*slot, gx, gy, gz, 256, &a, sizeof a, s);
+      }
       return TTS_OK;
     };
     if (b->fallback) {

@@ -1851,9 +1851,13 @@ std::string tile_program_source(const Program &p) {
   if (stores_walk_columns_with_pid1(p)) all << SWAP_MARK;
   all << pre << g.fns.str();
   // swap_xy: the launcher has exchanged the grid's x and y (see SWAP_MARK)
-  all << "extern \"C\" __global__ __launch_bounds__(256) void tile_program(const Args p, const int swap_xy) {\n"
-      << "  const long long pidx = swap_xy ? blockIdx.y : blockIdx.x, pidy = swap_xy ? blockIdx.x : blockIdx.y, pidz = blockIdx.z;\n"
-      << "  const long long npx = swap_xy ? gridDim.y : gridDim.x, npy = swap_xy ? gridDim.x : gridDim.y, npz = gridDim.z;\n"
+  // lgx != 0: the launch is one-dimensional and numbers the programs of an lgx x lgy x lgz grid itself, x fastest (the
+  // device's grid holds 65535 along y and z; the reference's launcher loops over any extents, backend/driver.py:116-133)
+  all << "extern \"C\" __global__ __launch_bounds__(256) void tile_program(const Args p, const int swap_xy, const int lgx, const int lgy, const int lgz) {\n"
+      << "  const long long lin = blockIdx.x;\n"
+      << "  const long long pidx = lgx ? lin % lgx : swap_xy ? blockIdx.y : blockIdx.x, pidy = lgx ? (lin / lgx) % lgy : swap_xy ? blockIdx.x : blockIdx.y,\n"
+      << "                  pidz = lgx ? lin / ((long long)lgx * lgy) : blockIdx.z;\n"
+      << "  const long long npx = lgx ? lgx : swap_xy ? gridDim.y : gridDim.x, npy = lgx ? lgy : swap_xy ? gridDim.x : gridDim.y, npz = lgx ? lgz : gridDim.z;\n"
       << "  (void)pidx; (void)pidy; (void)pidz; (void)npx; (void)npy; (void)npz;\n";
   if (g.pool_bytes) all << "  __shared__ __attribute__((aligned(16))) unsigned char pool[" << g.pool_bytes << "];\n";
   all << g.decl.str() << g.os.str() << "}\n";
