@@ -683,8 +683,8 @@ __device__ __forceinline__ void gemm_dma_body(const GemmParams &p, int tiles_m, 
 // A wavefront's 128 x 128 part of C is 8 x 8 blocks of 16 x 16, four accumulator registers each, held transposed (the B
 // operand goes in as the instruction's first source): a lane holds four consecutive columns of one row, which the epilogue
 // can narrow and pack without cross-lane moves.  One K tile of 32 is one instruction's depth.
-//   A operand of row block i: row 16 i + lane % 16, k 8 (lane / 16) .. +7: one 16-byte LDS read; the four chunks of 16 rows
-//     are 1 KB of consecutive LDS whatever the swizzle.
+//   A operand of row block i: row 16 i + lane % 16, k 8 (lane / 16) .. +7: one 16-byte LDS read (A's swizzle is chosen
+//     for the order in which such a read serves its lanes: see a_swizzle).
 //   B operand of column block j: `ds_read_b64_tr_b16` twice (k 0-3 and 4-7 of the lane's octet), lane r of a 16-lane group
 //     addressing k row 8 (lane / 16) + r / 4, columns 4 (r % 4) .. +3 of the block.  Two k octets share a half wavefront, so
 //     the stage's swizzle also flips chunk bit 1 with k bit 3: position q of k row k holds chunk q ^ ((k & 3) << 2) ^ (((k >> 3) & 1) << 1).
@@ -747,12 +747,19 @@ __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m
   const int k_begin = SK ? (int)((int64_t)slice * nk_all / p.split) : 0;
   const int nk = SK ? (int)((int64_t)(slice + 1) * nk_all / p.split) - k_begin : nk_all;
 
+  // A's swizzle: position q of row r holds chunk q ^ a_swizzle((r / 4) & 3).  A 16-byte LDS read serves sixteen lanes per
+  // cycle, and not sixteen neighbours: lanes 0-3 go with 12-15, 20-23 and 24-27 (of the eight quads of a half wavefront,
+  // those whose number has an even count of set bits, then the others; found by letting two lanes alone read one bank).
+  // With this instruction's operand layout (lane l: row l % 16, chunk l / 16) such a cycle holds row quads 0 and 3 of one
+  // chunk and 1 and 2 of the next, and the swizzle (0, 2, 3, 1) puts the four into different banks; the plain
+  // (r / 4) & 3 of the 32 x 32 x 16 body, conflict-free for that body's layout, made every A read here take twice its cycles.
+  auto a_swizzle = [](int row_quad) __attribute__((always_inline)) { return ((row_quad >> 1) & 1) | (((row_quad & 1) ^ ((row_quad >> 1) & 1)) << 1); };
   uint32_t a_voff[A_DMA], b_voff[B_DMA];
 #pragma unroll
   for (int i = 0; i < A_DMA; i++) {
     // rows past M (the last row tile of a ragged problem) fetch row M - 1 again: they only reach outputs nobody stores
     const int row = min(16 * (A_DMA * wave + i) + lane / 4, (int)(p.M - 1 - m0));
-    const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
+    const int chunk = (lane & 3) ^ a_swizzle((lane >> 4) & 3);
     a_voff[i] = (uint32_t)((row * p.lda + 8 * chunk) * 2);
   }
 #pragma unroll
@@ -785,7 +792,7 @@ __device__ __forceinline__ void gemm_dma16_body(const GemmParams &p, int tiles_m
   };
 
   const int l16 = lane & 15, q = lane >> 4;
-  const int a_off = (wm * 128 + l16) * 64 + ((q ^ ((l16 >> 2) & 3)) << 4);
+  const int a_off = (wm * 128 + l16) * 64 + ((q ^ a_swizzle((l16 >> 2) & 3)) << 4);
   const int b_sw = ((l16 >> 2) << 2) ^ ((q & 1) << 1);
   const int b_chunk = wn * 16 + ((l16 & 3) >> 1);
   const int b_off = A_BYTES + (8 * q + (l16 >> 2)) * ROWB + 8 * (l16 & 1);
