@@ -237,6 +237,27 @@ def make_workloads(torch, triton, K):
                          "loaded expert id per 128 rows (matmul family: the direct-to-LDS kernel takes the index vector and the id table; a fifth wavefront touches B's lines ahead)",
                     work=2 * tokens * kd * nd, bound="mfma", dtype="bf16", make=make, set_bytes=(tokens * kd + experts * kd * nd + tokens * nd) * 2)
 
+    def rms_norm(rows, cols):
+        def make():
+            x = torch.randn(rows, cols, device=dev).half()
+            w = (1 + 0.1 * torch.randn(cols, device=dev)).half()
+            y = torch.empty_like(x)
+            return lambda: K.rms_norm_rows[(rows,)](x, w, y, x.stride(0), cols, 1e-6, BLOCK=cols)
+        work = 2 * rows * cols * 2 + cols * 2
+        return dict(desc=f"RMSNorm fp16 [{rows}, {cols}], a row per program (generic family: eight neighbouring 16-bit elements per thread, 16-byte accesses)",
+                    work=work, bound="hbm", dtype="f16", make=make, set_bytes=work)
+
+    def layer_norm_dx(rows, cols):
+        def make():
+            x, dy = torch.randn(rows, cols, device=dev).half(), torch.randn(rows, cols, device=dev).half()
+            w = (1 + 0.1 * torch.randn(cols, device=dev)).half()
+            mean, rstd = torch.randn(rows, device=dev) * 0.1, 0.5 + torch.rand(rows, device=dev)
+            dx = torch.empty_like(x)
+            return lambda: K.layer_norm_dx_rows[(rows,)](dx, dy, x, w, mean, rstd, x.stride(0), cols, BLOCK=cols)
+        work = 3 * rows * cols * 2 + cols * 2 + 2 * rows * 4
+        return dict(desc=f"LayerNorm input gradient fp16 [{rows}, {cols}], a row per program, two row reductions (generic family, 16-byte accesses)",
+                    work=work, bound="hbm", dtype="f16", make=make, set_bytes=work)
+
     def stream_copy(n):
         def make():
             x = torch.rand(n, device=dev)
@@ -282,6 +303,8 @@ def make_workloads(torch, triton, K):
     W["next_fused_gelu_2p26"] = fused_gelu(1 << 26)
     W["next_fused_silu_2p26"] = fused_silu(1 << 26)
     W["next_rotary_8192x32x128"] = rotary(8192, 32, 64)
+    W["next_rms_norm_4096x8192"] = rms_norm(4096, 8192)
+    W["next_layer_norm_dx_4096x8192"] = layer_norm_dx(4096, 8192)
     W["next_matmul_act_4096"] = matmul_act(4096)
     W["next_expert_rows_4096"] = expert_rows(4096, 2048, 2048, 8)
     W["next_matmul_skinny_512"] = skinny_matmul(512, 8192, 8192)

@@ -1244,3 +1244,37 @@ def add_rows_2d(x_ptr, y_ptr, z_ptr, n_cols, BLOCK: tl.constexpr):
     a = tl.load(x_ptr + row * n_cols + cols, mask=mask)
     b = tl.load(y_ptr + row * n_cols + cols, mask=mask)
     tl.store(z_ptr + row * n_cols + cols, a + b, mask=mask)
+
+
+@triton.jit
+def scale_tile_and_row_sums(x_ptr, s_ptr, y_ptr, sums_ptr, n_rows, n_cols, pitch, BR: tl.constexpr, BC: tl.constexpr):
+    # y = x * s[None, :] on [BR, BC] tiles (x and y in a 16-bit type, s in fp32), and each tile's row sums of x
+    r = tl.program_id(0) * BR + tl.arange(0, BR)
+    c = tl.program_id(1) * BC + tl.arange(0, BC)
+    m = (r[:, None] < n_rows) & (c[None, :] < n_cols)
+    x = tl.load(x_ptr + r[:, None] * pitch + c[None, :], mask=m, other=0.0).to(tl.float32)
+    s = tl.load(s_ptr + c, mask=c < n_cols, other=0.0)
+    tl.store(y_ptr + r[:, None] * pitch + c[None, :], (x * s[None, :]).to(y_ptr.dtype.element_ty), mask=m)
+    tl.store(sums_ptr + tl.program_id(1) * n_rows + r, tl.sum(x, axis=1), mask=r < n_rows)
+
+
+@triton.jit
+def running_mean_of_rows(x_ptr, y_ptr, n_rows, n_cols, pitch, BLOCK: tl.constexpr):
+    # y[r, :] = mean(x[0..r, :]) for a block of columns: a carried fp32 accumulator next to 16-bit loads and stores
+    c = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = c < n_cols
+    acc = tl.zeros((BLOCK,), dtype=tl.float32)
+    for r in range(0, n_rows):
+        acc += tl.load(x_ptr + r * pitch + c, mask=m, other=0.0).to(tl.float32)
+        tl.store(y_ptr + r * pitch + c, (acc / (r + 1)).to(y_ptr.dtype.element_ty), mask=m)
+
+
+@triton.jit
+def widen_and_count(x_ptr, y_ptr, k_ptr, n, BLOCK: tl.constexpr):
+    # fp32 copy of a 16-bit block, and an i32 block counting the elements up to each position that are positive
+    # (4-byte stores next to 16-bit loads)
+    o = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    m = o < n
+    x = tl.load(x_ptr + o, mask=m, other=-1.0).to(tl.float32)
+    tl.store(y_ptr + o, x * 2.0, mask=m)
+    tl.store(k_ptr + o, tl.where(x > 0, o, -o), mask=m)

@@ -1701,6 +1701,96 @@ def test_tile_program_norms_and_reductions_of_the_tutorials():
     torch.testing.assert_close(lse, torch.logsumexp(b.double(), 1).float(), rtol=1e-6, atol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("n_cols,block,pitch,lead", [
+    (8192, 8192, 8192, 0),     # whole rows, every group moves in one access
+    (5000, 8192, 5000, 0),     # rows end on a group boundary; the groups behind are invalid as a whole
+    (4001, 4096, 4008, 0),     # rows end inside a group
+    (4001, 4096, 4001, 0),     # odd row pitch: every other row starts off a 16-byte boundary
+    (4096, 4096, 4096, 3),     # the tensors themselves start off a 16-byte boundary
+    (2048, 2048, 2056, 8),
+])
+def test_tile_program_wide_16_bit_rows(dtype, n_cols, block, pitch, lead):
+    """Blocks of 16-bit elements with whole groups of 2048 along the contiguous dimension give every thread eight
+    neighbouring elements and move them in 16-byte accesses where a group is aligned, element by element where it is not:
+    RMSNorm and the input gradient of LayerNorm on aligned, ragged and misaligned rows against float64 closed forms."""
+    torch.manual_seed(n_cols + lead)
+    dt = getattr(torch, dtype)
+    rows = 9
+    def rows_view(fill):
+        buf = torch.full((lead + rows * pitch + 16,), fill, device=DEV, dtype=dt)
+        return buf, buf[lead:lead + rows * pitch].view(rows, pitch)[:, :n_cols]
+    xb, x = rows_view(7.0)
+    x.copy_(torch.randn(rows, n_cols, device=DEV))
+    wb = torch.zeros(lead + n_cols, device=DEV, dtype=dt)
+    w = wb[lead:]
+    w.copy_(1 + 0.1 * torch.randn(n_cols, device=DEV))
+    yb, y = rows_view(5.0)
+    k = K_mod().rms_norm_rows[(rows,)](x, w, y, pitch, n_cols, 1e-6, BLOCK=block)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    xd = x.double()
+    want = xd / torch.sqrt((xd * xd).mean(1, keepdim=True) + 1e-6) * w.double()
+    tol = 2e-2 if dtype == "bfloat16" else 4e-3
+    assert (y.double() - want).abs().max() <= tol * max(1.0, want.abs().max().item())
+    keep = torch.ones_like(yb, dtype=torch.bool)
+    keep[lead:lead + rows * pitch].view(rows, pitch)[:, :n_cols] = False
+    assert (yb[keep] == 5.0).all()                              # nothing written outside the rows
+    # the gradient: three 16-bit row tensors, two scalars per row, two reductions
+    dyb, dy = rows_view(3.0)
+    dy.copy_(torch.randn(rows, n_cols, device=DEV))
+    mean, rstd = torch.randn(rows, device=DEV) * 0.1, 0.5 + torch.rand(rows, device=DEV)
+    dxb, dx = rows_view(5.0)
+    K_mod().layer_norm_dx_rows[(rows,)](dx, dy, x, w, mean, rstd, pitch, n_cols, BLOCK=block)
+    torch.cuda.synchronize()
+    xhat = (xd - mean.double()[:, None]) * rstd.double()[:, None]
+    wdy = w.double() * dy.double()
+    want = (wdy - (xhat * (xhat * wdy).mean(1, keepdim=True) + wdy.mean(1, keepdim=True))) * rstd.double()[:, None]
+    assert (dx.double() - want).abs().max() <= tol * max(1.0, want.abs().max().item())
+    assert (dxb[keep] == 5.0).all()
+
+
+def test_tile_program_wide_blocks_of_rows_loops_and_mixed_widths():
+    """The wide element order next to what shares a program with it: tiles of rows with a row reduction and a vector of
+    another shape, a carried accumulator in a loop, 4-byte stores next to 16-bit loads."""
+    import extra_kernels as X
+    torch.manual_seed(5)
+    for dt in (torch.float16, torch.bfloat16):
+        n_rows, n_cols, pitch = 11, 4100, 4104
+        xb = torch.randn(n_rows, pitch, device=DEV).to(dt)
+        x = xb[:, :n_cols]
+        s = torch.randn(n_cols, device=DEV)
+        yb = torch.full_like(xb, 5.0)
+        sums = torch.zeros(3, n_rows, device=DEV)
+        k = X.scale_tile_and_row_sums[(triton.cdiv(n_rows, 4), triton.cdiv(n_cols, 2048))](x, s, yb, sums, n_rows, n_cols, pitch, BR=4, BC=2048)
+        torch.cuda.synchronize()
+        assert k.function.family == "tile_program"
+        want = (x.double() * s.double()).to(dt)
+        assert (yb[:, :n_cols].double() - want.double()).abs().max() <= (0.07 if dt == torch.bfloat16 else 0.01)
+        assert (yb[:, n_cols:] == 5.0).all()
+        for j in range(3):
+            torch.testing.assert_close(sums[j].double(), x[:, j * 2048:(j + 1) * 2048].double().sum(1), rtol=1e-5, atol=1e-4)
+        # a carried accumulator
+        n_rows, n_cols = 6, 4096 + 24
+        x = torch.randn(n_rows, n_cols, device=DEV).to(dt)
+        y = torch.zeros_like(x)
+        X.running_mean_of_rows[(triton.cdiv(n_cols, 2048),)](x, y, n_rows, n_cols, n_cols, BLOCK=2048)
+        torch.cuda.synchronize()
+        want = x.double().cumsum(0) / torch.arange(1, n_rows + 1, device=DEV).double()[:, None]
+        assert (y.double() - want).abs().max() <= (0.03 if dt == torch.bfloat16 else 4e-3)
+        # 4-byte results of 16-bit loads, off a 16-byte boundary as well
+        for lead in (0, 2):
+            n = 3 * 2048 + 77
+            xs = torch.randn(lead + n, device=DEV).to(dt)[lead:]
+            yf = torch.full((lead + n + 8,), 5.0, device=DEV)
+            ki = torch.full((lead + n + 8,), 5, device=DEV, dtype=torch.int32)
+            X.widen_and_count[(triton.cdiv(n, 2048),)](xs, yf[lead:], ki[lead:], n, BLOCK=2048)
+            torch.cuda.synchronize()
+            assert torch.equal(yf[lead:lead + n], xs.float() * 2) and (yf[lead + n:] == 5).all() and (yf[:lead] == 5).all()
+            o = torch.arange(n, device=DEV, dtype=torch.int32)
+            assert torch.equal(ki[lead:lead + n], torch.where(xs.float() > 0, o, -o)) and (ki[lead + n:] == 5).all()
+
+
 def test_compiled_kernels_are_cached_on_disk(tmp_path, monkeypatch):
     """The code object of a run-time compiled kernel is written to the cache directory at the first launch and loaded
     from there by the next plan of the same source (the reference caches its compiled launchers the same way,

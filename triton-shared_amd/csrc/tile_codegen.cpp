@@ -30,6 +30,7 @@
 // whose address waits for another load's result, or a select between a loaded value and `other` right
 // after the load, serialises the whole run (see the notes at the two places).
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <map>
@@ -90,6 +91,7 @@ struct Gen {
   std::ostringstream decl;                          // LDS arrays holding their results (top of the kernel)
   size_t pool_bytes = 0, out_bytes = 0;             // staging pool shared by all reductions; result arrays
   bool uses_mfma = false;
+  bool uses_dummy = false;  // wide loads of invalid groups read this instead
 
   explicit Gen(const Program &p) : P(p) {}
 
@@ -112,6 +114,7 @@ struct Gen {
     return ctype(t);
   }
   static bool is_float(const std::string &t) { return t[0] == 'f' || t[0] == 'b'; }
+  static bool is16(const std::string &t) { return t == "f16" || t == "bf16"; }
 
   // ---- index expressions -------------------------------------------------
   // name_index_exprs: every operation node of the pool becomes a local (`const long long x<id> = ...;` in index_locals,
@@ -642,19 +645,68 @@ struct Gen {
       else var.erase(h.first);
     }
   }
-  // Row and column of element t of a block.  Every loop that names t names n as well, with t = threadIdx.x + 256 n; with
-  // rows of a multiple of 256 elements the row depends on n alone, which is a constant once the loop is unrolled (or the
-  // same in every thread where it is not): written that way, the row's address arithmetic (row * pitch in 64 bits, per
-  // element and access: quarter-rate multiplies) is the scalar unit's or the compiler's, not every lane's.
-  static std::string idx0(const std::vector<int64_t> &shape) {
+  // Which element a thread holds in slot n of a block.  Ordinarily t = threadIdx.x + 256 n: a wavefront's accesses are
+  // contiguous, one element per lane.  For 16-bit data that is 2 bytes per lane and access; a program whose blocks of
+  // 16-bit elements have whole groups of 2048 along the contiguous dimension is written "wide" instead: a thread owns
+  // eight neighbouring elements, t = 8 threadIdx.x + (n & 7) + 2048 (n >> 3), and a group of eight that is valid as a
+  // whole and 16-byte aligned moves in one access (two for 4-byte elements).  Only blocks of the one shape `wide_shape`
+  // are laid out that way; every other shape of the program keeps the ordinary order.  Programs with scans, matrix
+  // products or index shuffles (whose code relies on the ordinary order) are never wide.
+  bool wide_mode = false;
+  std::vector<int64_t> wide_shape;
+  bool wide(const std::vector<int64_t> &shape) const { return wide_mode && shape == wide_shape; }
+  bool vector_access(const Access &a) const {  // eight neighbouring elements are eight neighbouring addresses
+    if (a.gather >= 0 || a.sizes.empty() || a.strides.size() != a.sizes.size() || a.offsets.size() != a.sizes.size()) return false;
+    if (a.elem != "f16" && a.elem != "bf16" && a.elem != "f32" && a.elem != "i32") return false;
+    for (int m : a.mods)
+      if (m >= 0) return false;
+    int64_t st = 0;
+    return P.pool.is_const(a.strides.back(), &st) && st == 1;
+  }
+  void choose_wide_shape() {
+    if (const char *e = getenv("TTS_TILE_WIDE"))
+      if (e[0] == '0') return;
+    bool refuse = false;
+    std::vector<int64_t> best;
+    std::function<void(const std::vector<SOp> &)> scan = [&](const std::vector<SOp> &ops) {
+      for (const SOp &s : ops) {
+        if (s.kind == SK::Scan || s.kind == SK::Dot) refuse = true;
+        if (s.kind == SK::Map && (s.name.rfind("tt.trans", 0) == 0 || s.name == "tt.cat" || s.name == "tt.join" || s.name.rfind("tt.split", 0) == 0 ||
+                                  s.name == "tt.reshape" || s.name == "tt.unsplat"))
+          refuse = true;
+        if ((s.kind == SK::Load || s.kind == SK::Store) && (s.acc.elem == "f16" || s.acc.elem == "bf16") && vector_access(s.acc)) {
+          const auto &sz = s.acc.sizes;
+          if (sz.size() <= 2 && sz.back() % 2048 == 0 && count(sz) <= TWO_PHASE_MAX && (best.empty() || count(sz) > count(best))) best = sz;
+        }
+        if (s.kind == SK::For || s.kind == SK::If) scan(s.body);
+      }
+    };
+    scan(P.body);
+    if (refuse || best.empty()) return;
+    wide_mode = true;
+    wide_shape = best;
+  }
+  // (i0, i1) moved by `delta` along the contiguous dimension: called once with i0 (use .first) and once with i1 (.second)
+  static std::pair<std::string, std::string> along(const std::vector<int64_t> &shape, const std::string &i, const std::string &delta) {
+    return {shape.size() < 2 ? "(" + i + delta + ")" : i, shape.size() < 2 ? i : "(" + i + delta + ")"};
+  }
+  std::string element_of_slot(const std::vector<int64_t> &shape) const {
+    return wide(shape) ? "8 * (int)threadIdx.x + (n & 7) + 2048 * (n >> 3)" : "threadIdx.x + 256 * n";
+  }
+  // Row and column of element t of a block.  Every loop that names t names n as well (element_of_slot); with rows of a
+  // multiple of 256 elements the row depends on n alone, which is a constant once the loop is unrolled (or the same in
+  // every thread where it is not): written that way, the row's address arithmetic (row * pitch in 64 bits, per element
+  // and access: quarter-rate multiplies) is the scalar unit's or the compiler's, not every lane's.
+  std::string idx0(const std::vector<int64_t> &shape) const {
     if (shape.size() < 2) return "t";
     const int64_t C = shape.back();
     if (C % 256 == 0) return C == 256 ? "n" : "(n / " + std::to_string(C / 256) + ")";
     return "(t / " + std::to_string(C) + ")";
   }
-  static std::string idx1(const std::vector<int64_t> &shape) {
+  std::string idx1(const std::vector<int64_t> &shape) const {
     if (shape.size() < 2) return "0";
     const int64_t C = shape.back();
+    if (wide(shape)) return "(8 * (int)threadIdx.x + (n & 7) + 2048 * ((n >> 3) % " + std::to_string(C / 2048) + "))";
     if (C % 256 == 0) return C == 256 ? "(int)threadIdx.x" : "((int)threadIdx.x + 256 * (n % " + std::to_string(C / 256) + "))";
     return "(t % " + std::to_string(C) + ")";
   }
@@ -665,7 +717,8 @@ struct Gen {
     cur_i1 = idx1(shape);
     os << pad() << "#pragma unroll\n" << pad() << "for (int n = 0; n < " << (T + 255) / 256 << "; n++) {\n";
     indent++;
-    os << pad() << "const int t = threadIdx.x + 256 * n;\n" << pad() << "if (t >= " << T << ") break;\n";
+    os << pad() << "const int t = " << element_of_slot(shape) << ";\n";
+    if (T % 256) os << pad() << "if (t >= " << T << ") break;\n";  // (whole slots otherwise: 256 threads, launch bounds say so)
     map_vars(shape);
   }
   void close_loop() {
@@ -962,9 +1015,124 @@ struct Gen {
             close_loop();
             fill.clear();
           };
+          // Wide blocks: when every group of eight of these loads starts on a 16-byte boundary (the same answer in every
+          // thread of the program: the block's first element is aligned and, for blocks of rows, so is the row pitch), a
+          // group moves in one 16-byte access (two for 4-byte elements), unconditionally: a group whose first element is
+          // valid is read whole (what lies past the valid extent inside an aligned 16 bytes is on the same page), any
+          // other from a dummy; a second loop unpacks, widens and fills in `other`.  No branch sits between the loads, so
+          // none waits for another.  Otherwise the loads go element by element, as they would in the ordinary order.
+          auto wide_load = [&](const SOp &o) { return wide(ls) && mine_here(o) && vector_access(o.acc); };
+          {
+            bool any_wide = false;
+            for (size_t q = k; q < end; q++) any_wide = any_wide || wide_load(ops[q]);
+            if (any_wide) {
+              const int64_t G = count(ls) / 2048;
+              uses_dummy = true;
+              std::string aligned;
+              for (size_t q = k; q < end; q++)
+                if (wide_load(ops[q])) {
+                  const SOp &o = ops[q];
+                  std::string unused;
+                  const int esz = is16(o.acc.elem) ? 2 : 4;
+                  aligned += std::string(aligned.empty() ? "" : " && ") + "((unsigned long long)((const " + memtype(o.acc.elem) + " *)p.ptr[" + std::to_string(o.acc.base_arg) +
+                             "] + (" + address(o.acc, "0", "0", unused) + ")) & 15) == 0";
+                  if (ls.size() == 2) aligned += " && (((unsigned long long)(" + ex(o.acc.strides[0]) + ") * " + std::to_string(esz) + ") & 15) == 0";
+                }
+              os << pad() << "if (" << aligned << ") {\n";
+              indent++;
+              for (size_t q = k; q < end; q++)
+                if (wide_load(ops[q])) os << pad() << "u32x4_t rw" << ops[q].result << "[" << G * (is16(ops[q].acc.elem) ? 1 : 2) << "];\n";
+              os << pad() << "#pragma unroll\n" << pad() << "for (int g = 0; g < " << G << "; g++) {\n";
+              indent++;
+              os << pad() << "const int n = 8 * g;\n" << pad() << "const int t = " << element_of_slot(ls) << ";\n";
+              for (size_t q = k; q < end; q++)
+                if (wide_load(ops[q])) {
+                  const SOp &o = ops[q];
+                  const std::string id = std::to_string(o.result), mt = memtype(o.acc.elem);
+                  std::string pred, addr = address(o.acc, l0, l1, pred);
+                  os << pad() << "{\n";
+                  indent++;
+                  os << pad() << "const u32x4_t *const src = " << (pred.empty() ? "" : "!(" + pred + ") ? (const u32x4_t *)tts_dummy : ") << "(const u32x4_t *)((const " << mt
+                     << " *)p.ptr[" << o.acc.base_arg << "] + (" << addr << "));\n";
+                  if (is16(o.acc.elem)) os << pad() << "rw" << id << "[g] = src[0];\n";
+                  else {  // the second 16 bytes may lie on another page than the first: read only if their first element is valid
+                    std::string pred4;
+                    address(o.acc, along(ls, l0, " + 4").first, along(ls, l1, " + 4").second, pred4);
+                    os << pad() << "rw" << id << "[2 * g] = src[0];\n" << pad() << "rw" << id << "[2 * g + 1] = "
+                       << (pred4.empty() ? "src[1]" : "*(!(" + pred4 + ") ? (const u32x4_t *)tts_dummy : src + 1)") << ";\n";
+                  }
+                  indent--;
+                  os << pad() << "}\n";
+                }
+              indent--;
+              os << pad() << "}\n";
+              open_element_loop(ls);
+              for (size_t q = k; q < end; q++)
+                if (wide_load(ops[q])) {
+                  const SOp &o = ops[q];
+                  const std::string id = std::to_string(o.result);
+                  std::string pred, addr = address(o.acc, l0, l1, pred);
+                  std::string got;
+                  if (is16(o.acc.elem)) {
+                    const std::string word = "rw" + id + "[n >> 3][(n & 7) >> 1]";
+                    got = std::string(o.acc.elem == "f16" ? "up_f16(" : "up_bf16(") + "(unsigned short)((n & 1) ? " + word + " >> 16 : " + word + "))";
+                  } else {
+                    const std::string word = "rw" + id + "[n >> 2][n & 3]";
+                    got = o.acc.elem == "f32" ? "__uint_as_float(" + word + ")" : "(int)" + word;
+                  }
+                  os << pad() << "ld" << id << "[n] = " << (pred.empty() ? got : "(" + pred + ") ? " + got + " : " + other_of(o.acc, l0, l1)) << ";\n";
+                }
+              close_loop();
+              indent--;
+              os << pad() << "} else {\n";
+              indent++;
+              open_element_loop(ls);
+              for (size_t q = k; q < end; q++)
+                if (wide_load(ops[q])) {
+                  const SOp &o = ops[q];
+                  const std::string name = "ld" + std::to_string(o.result);
+                  std::string pred, addr = address(o.acc, l0, l1, pred);
+                  if (pred.empty()) os << pad() << name << "[n] = " << mem_read(o.acc, addr) << ";\n";
+                  else if (is16(o.acc.elem))
+                    os << pad() << "if (" << pred << ") " << name << "[n] = __uint_as_float(((const unsigned short *)p.ptr[" << o.acc.base_arg << "])[" << addr << "]);\n";
+                  else os << pad() << "if (" << pred << ") " << name << "[n] = " << mem_read(o.acc, addr) << ";\n";
+                }
+              close_loop();
+              bool any_masked = false;
+              for (size_t q = k; q < end; q++) any_masked = any_masked || (wide_load(ops[q]) && !ops[q].acc.dims.empty());
+              if (any_masked) {
+                open_element_loop(ls);
+                for (size_t q = k; q < end; q++)
+                  if (wide_load(ops[q]) && !ops[q].acc.dims.empty()) {
+                    const SOp &o = ops[q];
+                    const std::string name = "ld" + std::to_string(o.result);
+                    std::string pred, addr = address(o.acc, l0, l1, pred);
+                    if (is16(o.acc.elem)) {
+                      os << pad() << "asm volatile(\"\" : \"+v\"(" << name << "[n]));\n";
+                      os << pad() << name << "[n] = (" << pred << ") ? " << (o.acc.elem == "f16" ? "up_f16(" : "up_bf16(") << "(unsigned short)__float_as_uint(" << name
+                         << "[n])) : " << other_of(o.acc, l0, l1) << ";\n";
+                    } else
+                      os << pad() << "if (!(" << pred << ")) " << name << "[n] = " << other_of(o.acc, l0, l1) << ";\n";
+                  }
+                close_loop();
+              }
+              indent--;
+              os << pad() << "}\n";
+              for (size_t q = k; q < end; q++)
+                if (wide_load(ops[q])) {
+                  const std::string name = "ld" + std::to_string(ops[q].result);
+                  held[ops[q].result] = {name, ls};
+                  var[ops[q].result] = name + "[n]";
+                  mine.push_back(ops[q].result);
+                }
+            }
+          }
+          bool any_classic = false;
+          for (size_t q = k; q < end; q++) any_classic = any_classic || (mine_here(ops[q]) && !wide_load(ops[q]));
+          if (!any_classic) continue;
           open_element_loop(ls);
           for (size_t q = k; q < end; q++)
-            if (mine_here(ops[q])) {
+            if (mine_here(ops[q]) && !wide_load(ops[q])) {
               const std::string name = "ld" + std::to_string(ops[q].result);
               std::string pred, addr = address(ops[q].acc, l0, l1, pred);
               bool needs_filled = false;  // indexed or masked by a load that still lacks its `other`
@@ -992,6 +1160,9 @@ struct Gen {
           fill_others();
         }
         if (any_load) os << pad() << "__syncthreads();\n";
+        if (stores && wide(shape))  // wide stores collect a group's eight values (see the Store case below)
+          for (size_t q = k; q < end; q++)
+            if (ops[q].kind == SK::Store && vector_access(ops[q].acc)) os << pad() << "unsigned sv" << q << "[8];\n";
         if (stores) open_element_loop(shape);
       } else {
         std::set<int> load_bases;
@@ -1032,6 +1203,35 @@ struct Gen {
             all_store_bases.insert(o.acc.base_arg);
             const Value &sv = val(o.operands.at(0));
             if (sv.shape != shape) no("a stored value whose shape is not the block's");
+            if (two_phase && wide(shape) && vector_access(o.acc)) {
+              // the eighth element of a group writes the group: one 16-byte access (two for 4-byte elements) when all
+              // eight are valid and the first is 16-byte aligned, element by element otherwise
+              const bool half = is16(o.acc.elem);
+              const std::string sv = "sv" + std::to_string(q), mt = memtype(o.acc.elem), value = at(o.operands[0], i0, i1);
+              const std::string bits = o.acc.elem == "f16" ? "(unsigned)down_f16_exact(" + value + ")" : o.acc.elem == "bf16" ? "(unsigned)down_bf16(" + value + ")"
+                                       : o.acc.elem == "f32" ? "__float_as_uint(" + value + ")" : "(unsigned)(" + value + ")";
+              os << pad() << sv << "[n & 7] = " << bits << ";\n";
+              std::string pred_last, pred_e, addr0 = address(o.acc, along(shape, i0, " - 7").first, along(shape, i1, " - 7").second, pred_e);
+              address(o.acc, i0, i1, pred_last);
+              address(o.acc, along(shape, i0, " - 7 + e").first, along(shape, i1, " - 7 + e").second, pred_e);
+              os << pad() << "if ((n & 7) == 7) {\n";
+              indent++;
+              os << pad() << mt << " *const dst = (" << mt << " *)p.ptr[" << o.acc.base_arg << "] + (" << addr0 << ");\n";
+              os << pad() << "if (" << (pred_last.empty() ? "" : "(" + pred_last + ") && ") << "((unsigned long long)dst & 15) == 0) {\n";
+              if (half)
+                os << pad() << "  *(u32x4_t *)dst = u32x4_t{" << sv << "[0] | " << sv << "[1] << 16, " << sv << "[2] | " << sv << "[3] << 16, " << sv << "[4] | " << sv
+                   << "[5] << 16, " << sv << "[6] | " << sv << "[7] << 16};\n";
+              else
+                os << pad() << "  ((u32x4_t *)dst)[0] = u32x4_t{" << sv << "[0], " << sv << "[1], " << sv << "[2], " << sv << "[3]};\n"
+                   << pad() << "  ((u32x4_t *)dst)[1] = u32x4_t{" << sv << "[4], " << sv << "[5], " << sv << "[6], " << sv << "[7]};\n";
+              os << pad() << "} else {\n";
+              os << pad() << "  #pragma unroll\n" << pad() << "  for (int e = 0; e < 8; e++)\n";
+              os << pad() << "    if (" << (pred_e.empty() ? "true" : pred_e) << ") " << (half ? "dst[e] = (unsigned short)" + sv + "[e]" : "((unsigned *)dst)[e] = " + sv + "[e]") << ";\n";
+              os << pad() << "}\n";
+              indent--;
+              os << pad() << "}\n";
+              continue;
+            }
             std::string pred, addr = address(o.acc, i0, i1, pred);
             mem_write(o.acc, addr, pred, at(o.operands[0], i0, i1));
           }
@@ -1514,7 +1714,7 @@ struct Gen {
       for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << ";\n";
       os << pad() << unroll << "for (int q = 0; q < " << LQ << "; q++) {\n";
       indent++;
-      os << pad() << "const int n = o * " << LQ << " + q;\n" << pad() << "const int t = threadIdx.x + 256 * n;\n";
+      os << pad() << "const int n = o * " << LQ << " + q;\n" << pad() << "const int t = " << element_of_slot(shape) << ";\n";
       for (size_t j = 0; j < k; j++) os << pad() << "const " << Tn[j] << " el" << j << " = " << at(s.operands[j], i0, i1) << ";\n";
       os << pad() << "if (q == 0) { ";
       for (size_t j = 0; j < k; j++) os << "acc" << j << " = el" << j << "; ";
@@ -1795,6 +1995,7 @@ __device__ inline long long srem32(long long a, long long b) {
 }
 __device__ inline long long wrap(long long x, long long m) { return m > 0 ? ((x % m) + m) % m : x; }
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
 typedef unsigned short u16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
@@ -1843,6 +2044,7 @@ std::string tile_program_source(const Program &p) {
   const std::string n = std::to_string(TILE_MAX_ARGS);
   for (size_t pos = 0; (pos = pre.find("%N%", pos)) != std::string::npos;) pre.replace(pos, 3, n);
   g.collect_bases(p.body);
+  g.choose_wide_shape();
   g.body(p.body);
   // (a CU has 160 KB of LDS and the compiler lets one workgroup declare all of it; 128 KB leaves room for a second, small one)
   if (g.pool_bytes + g.out_bytes > 128 * 1024)
@@ -1850,6 +2052,7 @@ std::string tile_program_source(const Program &p) {
   std::ostringstream all;
   if (stores_walk_columns_with_pid1(p)) all << SWAP_MARK;
   all << pre << g.fns.str();
+  if (g.uses_dummy) all << "__device__ __attribute__((aligned(16))) unsigned tts_dummy[8];\n";
   // swap_xy: the launcher has exchanged the grid's x and y (see SWAP_MARK)
   // lgx != 0: the launch is one-dimensional and numbers the programs of an lgx x lgy x lgz grid itself, x fastest (the
   // device's grid holds 65535 along y and z; the reference's launcher loops over any extents, backend/driver.py:116-133)

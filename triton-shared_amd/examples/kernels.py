@@ -330,3 +330,35 @@ def rotary_embedding(x_ptr, cos_ptr, sin_ptr, out_ptr, stride_s, HALF: tl.conste
     sn = tl.load(sin_ptr + s * HALF + d)
     tl.store(out_ptr + base + d, (x1 * c - x2 * sn).to(tl.float16))
     tl.store(out_ptr + base + HALF + d, (x2 * c + x1 * sn).to(tl.float16))
+
+
+@triton.jit
+def rms_norm_rows(x_ptr, w_ptr, y_ptr, pitch, n_cols, eps, BLOCK: tl.constexpr):
+    """RMSNorm of rows, one row per program: y = x / sqrt(mean(x^2) + eps) * w; 16-bit or fp32 tensors, fp32 arithmetic."""
+    row = tl.program_id(0)
+    c = tl.arange(0, BLOCK)
+    m = c < n_cols
+    x = tl.load(x_ptr + row * pitch + c, mask=m, other=0.0).to(tl.float32)
+    ms = tl.sum(x * x, axis=0) / n_cols
+    w = tl.load(w_ptr + c, mask=m, other=0.0).to(tl.float32)
+    tl.store(y_ptr + row * pitch + c, (x * tl.rsqrt(ms + eps) * w).to(y_ptr.dtype.element_ty), mask=m)
+
+
+@triton.jit
+def layer_norm_dx_rows(dx_ptr, dy_ptr, x_ptr, w_ptr, mean_ptr, rstd_ptr, pitch, n_cols, BLOCK: tl.constexpr):
+    """The input gradient of LayerNorm, one row per program, from the forward's saved mean and rstd:
+    dx = (w dy - (xhat mean(xhat w dy) + mean(w dy))) rstd with xhat = (x - mean) rstd."""
+    row = tl.program_id(0)
+    c = tl.arange(0, BLOCK)
+    m = c < n_cols
+    x = tl.load(x_ptr + row * pitch + c, mask=m, other=0.0).to(tl.float32)
+    dy = tl.load(dy_ptr + row * pitch + c, mask=m, other=0.0).to(tl.float32)
+    w = tl.load(w_ptr + c, mask=m, other=0.0).to(tl.float32)
+    mean = tl.load(mean_ptr + row)
+    rstd = tl.load(rstd_ptr + row)
+    xhat = tl.where(m, (x - mean) * rstd, 0.0)
+    wdy = tl.where(m, w * dy, 0.0)
+    c1 = tl.sum(xhat * wdy, axis=0) / n_cols
+    c2 = tl.sum(wdy, axis=0) / n_cols
+    dx = (wdy - (xhat * c1 + c2)) * rstd
+    tl.store(dx_ptr + row * pitch + c, dx.to(dx_ptr.dtype.element_ty), mask=m)
