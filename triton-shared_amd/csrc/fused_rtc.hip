@@ -251,6 +251,7 @@ std::string source_of(const MapNParams &p) {
 struct RtcModule {
   hipModule_t module = nullptr;
   hipFunction_t fn = nullptr;
+  int resident = 0;  // workgroups of 256 threads a CU holds at once (0: not asked yet)
 };
 
 std::string fused_map_source(const MapNParams &p) { return source_of(p); }
@@ -383,6 +384,14 @@ void rtc_release(RtcModule *m) {
 hipError_t rtc_launch(RtcModule *m, int gx, int gy, int gz, int block, void *args, size_t size, hipStream_t s) {
   void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
   return hipModuleLaunchKernel(m->fn, gx, gy, gz, block, 1, 1, 0, s, nullptr, config);
+}
+
+int rtc_resident_workgroups(RtcModule *m) {
+  if (m->resident == 0) {
+    int n = 0;
+    m->resident = hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&n, m->fn, 256, 0) == hipSuccess && n > 0 ? n : 1;
+  }
+  return m->resident;
 }
 
 const char *gemm_device_source() {

@@ -58,6 +58,7 @@ hipError_t launch_mapn(const MapNParams &p, int gx, int gy, int gz, hipStream_t 
 struct RtcModule;
 hipError_t rtc_compile(const std::string &source, const char *entry, RtcModule **out, std::string *err);
 hipError_t rtc_launch(RtcModule *m, int gx, int gy, int gz, int block, void *args, size_t size, hipStream_t s);
+int rtc_resident_workgroups(RtcModule *m);  // how many workgroups of 256 threads of this kernel a CU holds at once (asked once, then kept)
 const char *gemm_device_source();  // the text of gemm_device.h
 void rtc_release(RtcModule *m);
 // The fused map's register program printed as HIP source and compiled once.

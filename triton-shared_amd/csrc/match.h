@@ -42,7 +42,8 @@ struct Plan {
 // (tile_codegen.cpp).  Throws Unsupported for anything else.  The kernel's argument block holds
 // every kernel argument by index: { void *ptr[N]; long long ival[N]; double fval[N]; }, N = TILE_MAX_ARGS.
 constexpr int TILE_MAX_ARGS = 32;
-std::string tile_program_source(const Program &p);
+std::string tile_program_source(const Program &p, bool allow_persistent = true);  // (persistent: see tile_program_is_persistent)
+bool tile_program_is_persistent(const std::string &source);  // the kernel walks the programs itself: any one-dimensional launch, lgx/lgy/lgz = the grid
 bool tile_program_swaps_grid(const std::string &source);  // the launcher exchanges the grid's x and y for this source (when y fits)
 // Matmul family with ops between the K loop and the store: the source of the functor that applies them to one
 // accumulator value (tile_codegen.cpp), compiled at run time together with the kernels of gemm_device.h.

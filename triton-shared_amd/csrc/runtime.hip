@@ -130,6 +130,7 @@ struct tts_plan {
     return hipSuccess;
   }
   RtcModule *fused = nullptr;  // the kernel compiled for this plan at its first launch (fused maps, tile programs)
+  bool fused_is_plain = false; // a tile program whose source is persistent but whose kernel with a workgroup per program was kept
   RtcModule *gemm_rtc[2] = {nullptr, nullptr};  // matrix products with a fused epilogue: one kernel per tiling
   RtcModule *fallback = nullptr;  // the generic family's kernel for a matrix-product plan (launches the product kernels decline)
   ~tts_plan() {
@@ -687,6 +688,15 @@ tts_status tts_plan_describe_launch(tts_plan *plan, int gx, int gy, int gz, cons
 
 namespace {
 
+int compute_units() {  // of the current device (256 when the query fails)
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    return n;
+  }();
+  return cus;
+}
+
 // tts_launch and tts_launch_noalloc (no_alloc: nothing below may allocate device memory or compile)
 tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, const tts_arg *args, int n, bool no_alloc) {
   if (!plan || (n > 0 && !args)) return fail(TTS_INVALID, "null argument");
@@ -721,6 +731,7 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
         else if (args[i].kind == TTS_ARG_INT) a.ival[i] = args[i].v.i;
         else a.fval[i] = args[i].v.f;
       }
+      bool persistent = false;
       {
         std::lock_guard<std::mutex> lock(plan->mu);
         if (!*slot) {
@@ -728,12 +739,35 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
           std::string why;
           hipError_t ce = rtc_compile(source, "tile_program", slot, &why);
           if (ce != hipSuccess) return fail(TTS_HIP_ERROR, "tile_program: " + why + "\n--- source ---\n" + source);
+          // A persistent kernel keeps what its programs share in registers.  When that costs it workgroups per CU (fewer
+          // than four fit), the kernel with a workgroup per program is compiled as well, and the one of which more fit
+          // is kept (LayerNorm's input gradient on rows of 8192: 2 against 3 per CU, 50 us against 41).
+          if (slot == &plan->fused && tile_program_is_persistent(source) && rtc_resident_workgroups(*slot) < 4) {
+            const std::string plain = tile_program_source(pl.prog, false);
+            RtcModule *other = nullptr;
+            if (rtc_compile(plain, "tile_program", &other, &why) == hipSuccess && rtc_resident_workgroups(other) > rtc_resident_workgroups(*slot)) {
+              rtc_release(*slot);
+              *slot = other;
+              plan->fused_is_plain = true;
+            } else if (other) {
+              rtc_release(other);
+            }
+          }
         }
+        persistent = tile_program_is_persistent(source) && !(slot == &plan->fused && plan->fused_is_plain);
       }
       kname = "tile_program (hipRTC)";
       // the program asks for neighbouring workgroups along program_id(1) (tile_codegen.cpp); grid.y holds 65535 at most
       a.swap_xy = tile_program_swaps_grid(source) && gy > 1 && gx <= 65535 ? 1 : 0;
-      if ((a.swap_xy ? gx : gy) > 65535 || gz > 65535) {  // the kernel numbers the programs itself (x fastest)
+      if (persistent) {
+        // as many workgroups as the device holds at once, four per CU at most, walk the programs (RMSNorm of 4096 rows:
+        // 768 / 1024 / 2048 workgroups took 26.5 / 25.6 / 26.2 us; a kernel whose registers admit three per CU runs a
+        // quarter of 1024 workgroups after the others)
+        a.swap_xy = 0;
+        a.lgx = gx; a.lgy = gy; a.lgz = gz;
+        const int64_t per_cu = std::min(4, rtc_resident_workgroups(*slot));
+        err = rtc_launch(*slot, (int)std::min<int64_t>((int64_t)gx * gy * gz, per_cu * compute_units()), 1, 1, 256, &a, sizeof a, s);
+      } else if ((a.swap_xy ? gx : gy) > 65535 || gz > 65535) {  // the kernel numbers the programs itself (x fastest)
         a.swap_xy = 0;
         a.lgx = gx; a.lgy = gy; a.lgz = gz;
         err = rtc_launch(*slot, (int)((int64_t)gx * gy * gz), 1, 1, 256, &a, sizeof a, s);

@@ -633,7 +633,7 @@ struct Gen {
     }
   }
   std::set<int> declared_copies;
-  struct Held { std::string name; std::vector<int64_t> shape; };
+  struct Held { std::string name; std::vector<int64_t> shape; std::string expr; };  // expr: what to write instead of name[n], if anything
   std::map<int, Held> held;
   // Loop-carried vectors that a loop also reads from blocks of another shape (the running maximum and sum of an online
   // softmax next to its [BM, BN] scores): besides the owning threads' registers they are kept in an LDS array, written
@@ -641,7 +641,7 @@ struct Gen {
   std::map<int, std::string> mirror;
   void map_vars(const std::vector<int64_t> &shape) {
     for (auto &h : held) {
-      if (h.second.shape == shape) var[h.first] = h.second.name + "[n]";
+      if (h.second.shape == shape) var[h.first] = h.second.expr.empty() ? h.second.name + "[n]" : h.second.expr;
       else var.erase(h.first);
     }
   }
@@ -689,6 +689,40 @@ struct Gen {
   // (i0, i1) moved by `delta` along the contiguous dimension: called once with i0 (use .first) and once with i1 (.second)
   static std::pair<std::string, std::string> along(const std::vector<int64_t> &shape, const std::string &i, const std::string &delta) {
     return {shape.size() < 2 ? "(" + i + delta + ")" : i, shape.size() < 2 ? i : "(" + i + delta + ")"};
+  }
+  // A wide program whose body loads a block that is the same for every program (a row of weights next to the row it
+  // scales: its address and extent name no program id, loop variable or loaded value, and nothing stores to its argument)
+  // is written "persistent": the launch has a few workgroups per CU, each walks the programs lin = blockIdx.x,
+  // blockIdx.x + gridDim.x, ... and the shared blocks are loaded once per workgroup, before that loop (hoisted: their
+  // code goes to hoist_os).  Read again by every program they stay in L2, but the L2 -> CU traffic is that of a second
+  // row (RMSNorm fp16 [4096, 8192]: 27.5 -> 25.5 us).
+  bool persistent = false;
+  std::set<int> hoisted;  // value ids of the loads emitted before the program loop
+  std::ostringstream hoist_os;
+  std::ostringstream loop_top;  // first statements of the program loop
+  void choose_persistent() {
+    if (!wide_mode) return;
+    if (const char *e = getenv("TTS_TILE_PERSISTENT"))
+      if (e[0] == '0') return;
+    std::set<int> stored;
+    std::function<void(const std::vector<SOp> &)> scan = [&](const std::vector<SOp> &ops) {
+      for (const SOp &s : ops) {
+        if (s.kind == SK::Store || s.kind == SK::ScalarStore) stored.insert(s.acc.base_arg);
+        if (s.kind == SK::For || s.kind == SK::If) scan(s.body);
+      }
+    };
+    scan(P.body);
+    for (const SOp &s : P.body) {
+      if (s.kind != SK::Load || !wide(s.acc.sizes) || !vector_access(s.acc) || stored.count(s.acc.base_arg) || s.acc.other_value >= 0) continue;
+      std::vector<int> es = s.acc.offsets;
+      es.insert(es.end(), s.acc.strides.begin(), s.acc.strides.end());
+      es.insert(es.end(), s.acc.dims.begin(), s.acc.dims.end());
+      bool fixed = true;
+      for (int e : es)
+        for (EK k : {EK::Pid, EK::IV, EK::Iter, EK::Result, EK::Data}) fixed = fixed && (e < 0 || !P.pool.depends_on(e, k));
+      if (fixed) hoisted.insert(s.result);
+    }
+    persistent = !hoisted.empty();
   }
   std::string element_of_slot(const std::vector<int64_t> &shape) const {
     return wide(shape) ? "8 * (int)threadIdx.x + (n & 7) + 2048 * (n >> 3)" : "threadIdx.x + 256 * n";
@@ -986,7 +1020,18 @@ struct Gen {
           bool any = false;
           for (size_t q = k; q < end; q++)
             if (mine_here(ops[q])) {
-              os << pad() << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << (count(ls) + 255) / 256 << "];\n";
+              if (hoisted.count(ops[q].result)) {
+                // (16-bit blocks that stay in registers for the whole launch stay packed, two elements per register, and
+                // are widened where they are used)
+                if (is16(ops[q].acc.elem)) {
+                  hoist_os << "  u32x4_t rw" << ops[q].result << "[" << count(ls) / 2048 << "];\n";
+                  // (the empty asm says the words may have changed: the compiler would otherwise widen them once, before
+                  // the loop, and keep twice the registers for the whole launch)
+                  for (int64_t g = 0; g < count(ls) / 2048; g++) loop_top << "    asm volatile(\"\" : \"+v\"(rw" << ops[q].result << "[" << g << "]));\n";
+                }
+                else hoist_os << "  " << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << (count(ls) + 255) / 256 << "];\n";
+              }
+              else os << pad() << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << (count(ls) + 255) / 256 << "];\n";
               any = true;
             }
           if (!any) continue;
@@ -1021,8 +1066,15 @@ struct Gen {
           // valid is read whole (what lies past the valid extent inside an aligned 16 bytes is on the same page), any
           // other from a dummy; a second loop unpacks, widens and fills in `other`.  No branch sits between the loads, so
           // none waits for another.  Otherwise the loads go element by element, as they would in the ordinary order.
-          auto wide_load = [&](const SOp &o) { return wide(ls) && mine_here(o) && vector_access(o.acc); };
-          {
+          auto wide_load_any = [&](const SOp &o) { return wide(ls) && mine_here(o) && vector_access(o.acc); };
+          for (int pass = 0; pass < 2; pass++) {  // pass 0: the loads hoisted out of the program loop, into hoist_os
+            auto wide_load = [&](const SOp &o) { return wide_load_any(o) && (hoisted.count(o.result) != 0) == (pass == 0); };
+            const int saved_indent = indent;
+            if (pass == 0) {
+              os.swap(hoist_os);
+              indent = 1;
+            }
+            auto packed = [&](const SOp &o) { return pass == 0 && is16(o.acc.elem); };
             bool any_wide = false;
             for (size_t q = k; q < end; q++) any_wide = any_wide || wide_load(ops[q]);
             if (any_wide) {
@@ -1041,7 +1093,7 @@ struct Gen {
               os << pad() << "if (" << aligned << ") {\n";
               indent++;
               for (size_t q = k; q < end; q++)
-                if (wide_load(ops[q])) os << pad() << "u32x4_t rw" << ops[q].result << "[" << G * (is16(ops[q].acc.elem) ? 1 : 2) << "];\n";
+                if (wide_load(ops[q]) && !packed(ops[q])) os << pad() << "u32x4_t rw" << ops[q].result << "[" << G * (is16(ops[q].acc.elem) ? 1 : 2) << "];\n";
               os << pad() << "#pragma unroll\n" << pad() << "for (int g = 0; g < " << G << "; g++) {\n";
               indent++;
               os << pad() << "const int n = 8 * g;\n" << pad() << "const int t = " << element_of_slot(ls) << ";\n";
@@ -1068,7 +1120,7 @@ struct Gen {
               os << pad() << "}\n";
               open_element_loop(ls);
               for (size_t q = k; q < end; q++)
-                if (wide_load(ops[q])) {
+                if (wide_load(ops[q]) && !packed(ops[q])) {
                   const SOp &o = ops[q];
                   const std::string id = std::to_string(o.result);
                   std::string pred, addr = address(o.acc, l0, l1, pred);
@@ -1086,9 +1138,26 @@ struct Gen {
               indent--;
               os << pad() << "} else {\n";
               indent++;
+              for (size_t q = k; q < end; q++)
+                if (wide_load(ops[q]) && packed(ops[q])) os << pad() << "unsigned tm" << ops[q].result << "[" << count(ls) / 256 << "] = {};\n";
               open_element_loop(ls);
               for (size_t q = k; q < end; q++)
-                if (wide_load(ops[q])) {
+                if (wide_load(ops[q]) && packed(ops[q])) {
+                  std::string pred, addr = address(ops[q].acc, l0, l1, pred);
+                  os << pad() << (pred.empty() ? "" : "if (" + pred + ") ") << "tm" << ops[q].result << "[n] = ((const unsigned short *)p.ptr[" << ops[q].acc.base_arg << "])[" << addr << "];\n";
+                }
+              close_loop();
+              for (size_t q = k; q < end; q++)
+                if (wide_load(ops[q]) && packed(ops[q])) {
+                  os << pad() << "#pragma unroll\n" << pad() << "for (int g = 0; g < " << G << "; g++)\n";
+                  os << pad() << "  rw" << ops[q].result << "[g] = u32x4_t{";
+                  for (int c = 0; c < 4; c++)
+                    os << (c ? ", " : "") << "tm" << ops[q].result << "[8 * g + " << 2 * c << "] | tm" << ops[q].result << "[8 * g + " << 2 * c + 1 << "] << 16";
+                  os << "};\n";
+                }
+              open_element_loop(ls);
+              for (size_t q = k; q < end; q++)
+                if (wide_load(ops[q]) && !packed(ops[q])) {
                   const SOp &o = ops[q];
                   const std::string name = "ld" + std::to_string(o.result);
                   std::string pred, addr = address(o.acc, l0, l1, pred);
@@ -1099,11 +1168,11 @@ struct Gen {
                 }
               close_loop();
               bool any_masked = false;
-              for (size_t q = k; q < end; q++) any_masked = any_masked || (wide_load(ops[q]) && !ops[q].acc.dims.empty());
+              for (size_t q = k; q < end; q++) any_masked = any_masked || (wide_load(ops[q]) && !packed(ops[q]) && !ops[q].acc.dims.empty());
               if (any_masked) {
                 open_element_loop(ls);
                 for (size_t q = k; q < end; q++)
-                  if (wide_load(ops[q]) && !ops[q].acc.dims.empty()) {
+                  if (wide_load(ops[q]) && !packed(ops[q]) && !ops[q].acc.dims.empty()) {
                     const SOp &o = ops[q];
                     const std::string name = "ld" + std::to_string(o.result);
                     std::string pred, addr = address(o.acc, l0, l1, pred);
@@ -1120,13 +1189,27 @@ struct Gen {
               os << pad() << "}\n";
               for (size_t q = k; q < end; q++)
                 if (wide_load(ops[q])) {
-                  const std::string name = "ld" + std::to_string(ops[q].result);
-                  held[ops[q].result] = {name, ls};
-                  var[ops[q].result] = name + "[n]";
-                  mine.push_back(ops[q].result);
+                  const SOp &o = ops[q];
+                  if (packed(o)) {
+                    const std::string word = "rw" + std::to_string(o.result) + "[n >> 3][(n & 7) >> 1]";
+                    std::string pred, addr = address(o.acc, l0, l1, pred);
+                    const std::string got = std::string(o.acc.elem == "f16" ? "up_f16(" : "up_bf16(") + "(unsigned short)((n & 1) ? " + word + " >> 16 : " + word + "))";
+                    held[o.result] = {"rw" + std::to_string(o.result), ls, "(" + (pred.empty() ? got : "(" + pred + ") ? " + got + " : " + other_of(o.acc, l0, l1)) + ")"};
+                    var[o.result] = held[o.result].expr;
+                  } else {
+                    const std::string name = "ld" + std::to_string(o.result);
+                    held[o.result] = {name, ls};
+                    var[o.result] = name + "[n]";
+                  }
+                  mine.push_back(o.result);
                 }
             }
+            if (pass == 0) {
+              os.swap(hoist_os);
+              indent = saved_indent;
+            }
           }
+          auto wide_load = wide_load_any;
           bool any_classic = false;
           for (size_t q = k; q < end; q++) any_classic = any_classic || (mine_here(ops[q]) && !wide_load(ops[q]));
           if (!any_classic) continue;
@@ -1219,11 +1302,11 @@ struct Gen {
               os << pad() << mt << " *const dst = (" << mt << " *)p.ptr[" << o.acc.base_arg << "] + (" << addr0 << ");\n";
               os << pad() << "if (" << (pred_last.empty() ? "" : "(" + pred_last + ") && ") << "((unsigned long long)dst & 15) == 0) {\n";
               if (half)
-                os << pad() << "  *(u32x4_t *)dst = u32x4_t{" << sv << "[0] | " << sv << "[1] << 16, " << sv << "[2] | " << sv << "[3] << 16, " << sv << "[4] | " << sv
-                   << "[5] << 16, " << sv << "[6] | " << sv << "[7] << 16};\n";
+                os << pad() << "  __builtin_nontemporal_store(u32x4_t{" << sv << "[0] | " << sv << "[1] << 16, " << sv << "[2] | " << sv << "[3] << 16, " << sv << "[4] | " << sv
+                   << "[5] << 16, " << sv << "[6] | " << sv << "[7] << 16}, (u32x4_t *)dst);\n";
               else
-                os << pad() << "  ((u32x4_t *)dst)[0] = u32x4_t{" << sv << "[0], " << sv << "[1], " << sv << "[2], " << sv << "[3]};\n"
-                   << pad() << "  ((u32x4_t *)dst)[1] = u32x4_t{" << sv << "[4], " << sv << "[5], " << sv << "[6], " << sv << "[7]};\n";
+                os << pad() << "  __builtin_nontemporal_store(u32x4_t{" << sv << "[0], " << sv << "[1], " << sv << "[2], " << sv << "[3]}, (u32x4_t *)dst);\n"
+                   << pad() << "  __builtin_nontemporal_store(u32x4_t{" << sv << "[4], " << sv << "[5], " << sv << "[6], " << sv << "[7]}, (u32x4_t *)dst + 1);\n";
               os << pad() << "} else {\n";
               os << pad() << "  #pragma unroll\n" << pad() << "  for (int e = 0; e < 8; e++)\n";
               os << pad() << "    if (" << (pred_e.empty() ? "true" : pred_e) << ") " << (half ? "dst[e] = (unsigned short)" + sv + "[e]" : "((unsigned *)dst)[e] = " + sv + "[e]") << ";\n";
@@ -2010,6 +2093,7 @@ namespace {
 // the line below, and the launcher swaps the grid's x and y (x + bias[None, :] on [32, 256] tiles of an 8192 x 8192 matrix,
 // row blocks on program_id(0): 119 us; with column blocks there: 100).
 const char *const SWAP_MARK = "// tts: swap_xy\n";
+const char *const PERSISTENT_MARK = "// tts: persistent\n";  // the launcher starts a few workgroups per CU, which walk the programs
 bool stores_walk_columns_with_pid1(const Program &p) {
   int votes_for = 0, votes_against = 0;
   std::function<void(const std::vector<SOp> &)> scan = [&](const std::vector<SOp> &ops) {
@@ -2035,9 +2119,21 @@ bool stores_walk_columns_with_pid1(const Program &p) {
 }
 }  // namespace
 
-bool tile_program_swaps_grid(const std::string &source) { return source.compare(0, strlen(SWAP_MARK), SWAP_MARK) == 0; }
+namespace {
+// The body of a persistent kernel's program loop with the thread's index read from a variable that an empty asm renews in
+// every iteration: what depends on it alone -- 32 element masks, 32 64-bit element offsets -- is otherwise computed once,
+// before the loop, and held in registers for the whole launch (LayerNorm's input gradient: 211 registers instead of 149).
+std::string per_program_thread_index(std::string body) {
+  const std::string from = "threadIdx.x", to = "tidx";
+  for (size_t pos = 0; (pos = body.find(from, pos)) != std::string::npos; pos += to.size()) body.replace(pos, from.size(), to);
+  return "    unsigned tidx = threadIdx.x;\n    asm volatile(\"\" : \"+v\"(tidx));\n" + body;
+}
+}  // namespace
 
-std::string tile_program_source(const Program &p) {
+bool tile_program_swaps_grid(const std::string &source) { return source.compare(0, strlen(SWAP_MARK), SWAP_MARK) == 0; }
+bool tile_program_is_persistent(const std::string &source) { return source.compare(0, strlen(PERSISTENT_MARK), PERSISTENT_MARK) == 0; }
+
+std::string tile_program_source(const Program &p, bool allow_persistent) {
   if ((int)p.arg_names.size() > TILE_MAX_ARGS) throw Unsupported("tile_program: more than " + std::to_string(TILE_MAX_ARGS) + " kernel arguments");
   Gen g(p);
   std::string pre = TILE_PRELUDE;
@@ -2045,25 +2141,40 @@ std::string tile_program_source(const Program &p) {
   for (size_t pos = 0; (pos = pre.find("%N%", pos)) != std::string::npos;) pre.replace(pos, 3, n);
   g.collect_bases(p.body);
   g.choose_wide_shape();
+  if (allow_persistent) g.choose_persistent();
+  if (g.persistent) g.indent = 2;
   g.body(p.body);
   // (a CU has 160 KB of LDS and the compiler lets one workgroup declare all of it; 128 KB leaves room for a second, small one)
   if (g.pool_bytes + g.out_bytes > 128 * 1024)
     throw Unsupported("tile_program: the reductions of this program need " + std::to_string(g.pool_bytes + g.out_bytes) + " bytes of LDS (limit 131072)");
   std::ostringstream all;
-  if (stores_walk_columns_with_pid1(p)) all << SWAP_MARK;
+  if (g.persistent) all << PERSISTENT_MARK;
+  else if (stores_walk_columns_with_pid1(p)) all << SWAP_MARK;
   all << pre << g.fns.str();
   if (g.uses_dummy) all << "__device__ __attribute__((aligned(16))) unsigned tts_dummy[8];\n";
   // swap_xy: the launcher has exchanged the grid's x and y (see SWAP_MARK)
   // lgx != 0: the launch is one-dimensional and numbers the programs of an lgx x lgy x lgz grid itself, x fastest (the
   // device's grid holds 65535 along y and z; the reference's launcher loops over any extents, backend/driver.py:116-133)
-  all << "extern \"C\" __global__ __launch_bounds__(256) void tile_program(const Args p, const int swap_xy, const int lgx, const int lgy, const int lgz) {\n"
-      << "  const long long lin = blockIdx.x;\n"
-      << "  const long long pidx = lgx ? lin % lgx : swap_xy ? blockIdx.y : blockIdx.x, pidy = lgx ? (lin / lgx) % lgy : swap_xy ? blockIdx.x : blockIdx.y,\n"
-      << "                  pidz = lgx ? lin / ((long long)lgx * lgy) : blockIdx.z;\n"
-      << "  const long long npx = lgx ? lgx : swap_xy ? gridDim.y : gridDim.x, npy = lgx ? lgy : swap_xy ? gridDim.x : gridDim.y, npz = lgx ? lgz : gridDim.z;\n"
-      << "  (void)pidx; (void)pidy; (void)pidz; (void)npx; (void)npy; (void)npz;\n";
+  all << "extern \"C\" __global__ __launch_bounds__(256) void tile_program(const Args p, const int swap_xy, const int lgx, const int lgy, const int lgz) {\n";
   if (g.pool_bytes) all << "  __shared__ __attribute__((aligned(16))) unsigned char pool[" << g.pool_bytes << "];\n";
-  all << g.decl.str() << g.os.str() << "}\n";
+  all << g.decl.str();
+  if (g.persistent) {
+    // a one-dimensional launch of any number of workgroups (lgx, lgy, lgz always hold the grid); what the programs share
+    // is loaded first; the barrier at the end keeps a program's LDS arrays from the next program's writes
+    all << g.hoist_os.str()
+        << "  for (unsigned lin = blockIdx.x; lin < (unsigned)lgx * (unsigned)lgy * (unsigned)lgz; lin += gridDim.x) {  // (fewer than 2^31 programs: the launcher sees to it)\n"
+        << "    const long long pidx = lin % (unsigned)lgx, pidy = (lin / (unsigned)lgx) % (unsigned)lgy, pidz = lin / ((unsigned)lgx * (unsigned)lgy);\n"
+        << "    const long long npx = lgx, npy = lgy, npz = lgz;\n"
+        << "    (void)pidx; (void)pidy; (void)pidz; (void)npx; (void)npy; (void)npz; (void)swap_xy;\n"
+        << g.loop_top.str() << per_program_thread_index(g.os.str()) << "    __syncthreads();\n  }\n}\n";
+  } else {
+    all << "  const long long lin = blockIdx.x;\n"
+        << "  const long long pidx = lgx ? lin % lgx : swap_xy ? blockIdx.y : blockIdx.x, pidy = lgx ? (lin / lgx) % lgy : swap_xy ? blockIdx.x : blockIdx.y,\n"
+        << "                  pidz = lgx ? lin / ((long long)lgx * lgy) : blockIdx.z;\n"
+        << "  const long long npx = lgx ? lgx : swap_xy ? gridDim.y : gridDim.x, npy = lgx ? lgy : swap_xy ? gridDim.x : gridDim.y, npz = lgx ? lgz : gridDim.z;\n"
+        << "  (void)pidx; (void)pidy; (void)pidz; (void)npx; (void)npy; (void)npz;\n"
+        << g.os.str() << "}\n";
+  }
   for (int b : g.all_inline_bases)
     if (g.all_store_bases.count(b))
       throw Unsupported("tile_program: an argument is both stored to and read by a load that is not of its body's block shape");
