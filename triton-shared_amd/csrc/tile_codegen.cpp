@@ -1031,7 +1031,8 @@ struct Gen {
                 }
                 else hoist_os << "  " << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << (count(ls) + 255) / 256 << "];\n";
               }
-              else os << pad() << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << (count(ls) + 255) / 256 << "];\n";
+              else  // (inside a program loop a slot that a masked load leaves unwritten would otherwise hold, and carry, the last program's)
+                os << pad() << ctype(val(ops[q].result).dtype) << " ld" << ops[q].result << "[" << (count(ls) + 255) / 256 << "]" << (persistent ? " = {}" : "") << ";\n";
               any = true;
             }
           if (!any) continue;
