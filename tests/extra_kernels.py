@@ -1278,3 +1278,26 @@ def widen_and_count(x_ptr, y_ptr, k_ptr, n, BLOCK: tl.constexpr):
     x = tl.load(x_ptr + o, mask=m, other=-1.0).to(tl.float32)
     tl.store(y_ptr + o, x * 2.0, mask=m)
     tl.store(k_ptr + o, tl.where(x > 0, o, -o), mask=m)
+
+
+@triton.jit
+def quantize_rows_int8(x_ptr, q_ptr, s_ptr, n_cols, pitch, BLOCK: tl.constexpr):
+    # row-wise symmetric int8 quantisation: q = round-half-away(x / (max|x| / 127)), one row per program
+    row = tl.program_id(0)
+    c = tl.arange(0, BLOCK)
+    m = c < n_cols
+    x = tl.load(x_ptr + row * pitch + c, mask=m, other=0.0).to(tl.float32)
+    scale = tl.max(tl.abs(x), axis=0) / 127.0
+    q = x / scale
+    q = tl.where(q >= 0, q + 0.5, q - 0.5).to(tl.int8)
+    tl.store(q_ptr + row * pitch + c, q, mask=m)
+    tl.store(s_ptr + row, scale)
+
+
+@triton.jit
+def dequantize_rows_int8(q_ptr, s_ptr, y_ptr, n_cols, pitch, BLOCK: tl.constexpr):
+    row = tl.program_id(0)
+    c = tl.arange(0, BLOCK)
+    m = c < n_cols
+    q = tl.load(q_ptr + row * pitch + c, mask=m, other=0)
+    tl.store(y_ptr + row * pitch + c, (q.to(tl.float32) * tl.load(s_ptr + row)).to(y_ptr.dtype.element_ty), mask=m)

@@ -1791,6 +1791,38 @@ def test_tile_program_wide_blocks_of_rows_loops_and_mixed_widths():
             assert torch.equal(ki[lead:lead + n], torch.where(xs.float() > 0, o, -o)) and (ki[lead + n:] == 5).all()
 
 
+@pytest.mark.parametrize("n_cols,pitch,lead", [(4096, 4096, 0), (4000, 4000, 0), (4093, 4099, 0), (2048, 2048, 5)])
+def test_tile_program_wide_rows_with_int8_neighbours(n_cols, pitch, lead):
+    """Row-wise int8 quantisation and its inverse: 1-byte blocks next to 16-bit ones take the wide element order too
+    (eight bytes per thread, one 8-byte access where a group is whole and aligned); exact against torch."""
+    import extra_kernels as X
+    torch.manual_seed(n_cols)
+    rows = 7
+    xb = torch.zeros(lead + rows * pitch, device=DEV, dtype=torch.float16)
+    x = xb[lead:].view(rows, pitch)[:, :n_cols]
+    x.copy_(torch.randn(rows, n_cols, device=DEV))
+    qb = torch.full((lead + rows * pitch + 8,), 5, device=DEV, dtype=torch.int8)
+    q = qb[lead:lead + rows * pitch].view(rows, pitch)[:, :n_cols]
+    s = torch.zeros(rows, device=DEV)
+    k = X.quantize_rows_int8[(rows,)](x, q, s, n_cols, pitch, BLOCK=4096)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    xf = x.float().cpu()                                              # (on the host: IEEE division, as the kernel's is)
+    scale = xf.abs().amax(1) / torch.full((rows,), 127.0)
+    assert torch.equal(s.cpu(), scale)
+    t = xf / scale[:, None]
+    want = torch.where(t >= 0, t + 0.5, t - 0.5).to(torch.int8)      # (the conversion truncates toward zero, as the kernel's does)
+    assert torch.equal(q.cpu(), want)
+    keep = torch.ones_like(qb, dtype=torch.bool)
+    keep[lead:lead + rows * pitch].view(rows, pitch)[:, :n_cols] = False
+    assert (qb[keep] == 5).all()
+    yb = torch.full((lead + rows * pitch,), 3.0, device=DEV, dtype=torch.float16)
+    y = yb[lead:].view(rows, pitch)[:, :n_cols]
+    X.dequantize_rows_int8[(rows,)](q, s, y, n_cols, pitch, BLOCK=4096)
+    torch.cuda.synchronize()
+    assert torch.equal(y.cpu(), (want.float() * scale[:, None]).half())
+
+
 def test_compiled_kernels_are_cached_on_disk(tmp_path, monkeypatch):
     """The code object of a run-time compiled kernel is written to the cache directory at the first launch and loaded
     from there by the next plan of the same source (the reference caches its compiled launchers the same way,

@@ -115,6 +115,7 @@ struct Gen {
   }
   static bool is_float(const std::string &t) { return t[0] == 'f' || t[0] == 'b'; }
   static bool is16(const std::string &t) { return t == "f16" || t == "bf16"; }
+  static int mem_bytes(const std::string &t) { return t == "i8" ? 1 : is16(t) ? 2 : 4; }  // of the element types vector_access takes
 
   // ---- index expressions -------------------------------------------------
   // name_index_exprs: every operation node of the pool becomes a local (`const long long x<id> = ...;` in index_locals,
@@ -657,7 +658,7 @@ struct Gen {
   bool wide(const std::vector<int64_t> &shape) const { return wide_mode && shape == wide_shape; }
   bool vector_access(const Access &a) const {  // eight neighbouring elements are eight neighbouring addresses
     if (a.gather >= 0 || a.sizes.empty() || a.strides.size() != a.sizes.size() || a.offsets.size() != a.sizes.size()) return false;
-    if (a.elem != "f16" && a.elem != "bf16" && a.elem != "f32" && a.elem != "i32") return false;
+    if (a.elem != "f16" && a.elem != "bf16" && a.elem != "f32" && a.elem != "i32" && a.elem != "i8") return false;
     for (int m : a.mods)
       if (m >= 0) return false;
     int64_t st = 0;
@@ -1086,15 +1087,17 @@ struct Gen {
                 if (wide_load(ops[q])) {
                   const SOp &o = ops[q];
                   std::string unused;
-                  const int esz = is16(o.acc.elem) ? 2 : 4;
+                  const int esz = mem_bytes(o.acc.elem);
+                  const std::string mask = esz == 1 ? "7" : "15";  // a group of eight 1-byte elements is one 8-byte access
                   aligned += std::string(aligned.empty() ? "" : " && ") + "((unsigned long long)((const " + memtype(o.acc.elem) + " *)p.ptr[" + std::to_string(o.acc.base_arg) +
-                             "] + (" + address(o.acc, "0", "0", unused) + ")) & 15) == 0";
-                  if (ls.size() == 2) aligned += " && (((unsigned long long)(" + ex(o.acc.strides[0]) + ") * " + std::to_string(esz) + ") & 15) == 0";
+                             "] + (" + address(o.acc, "0", "0", unused) + ")) & " + mask + ") == 0";
+                  if (ls.size() == 2) aligned += " && (((unsigned long long)(" + ex(o.acc.strides[0]) + ") * " + std::to_string(esz) + ") & " + mask + ") == 0";
                 }
               os << pad() << "if (" << aligned << ") {\n";
               indent++;
               for (size_t q = k; q < end; q++)
-                if (wide_load(ops[q]) && !packed(ops[q])) os << pad() << "u32x4_t rw" << ops[q].result << "[" << G * (is16(ops[q].acc.elem) ? 1 : 2) << "];\n";
+                if (wide_load(ops[q]) && !packed(ops[q]))
+                  os << pad() << (mem_bytes(ops[q].acc.elem) == 1 ? "u32x2_t rw" : "u32x4_t rw") << ops[q].result << "[" << G * (mem_bytes(ops[q].acc.elem) == 4 ? 2 : 1) << "];\n";
               os << pad() << "#pragma unroll\n" << pad() << "for (int g = 0; g < " << G << "; g++) {\n";
               indent++;
               os << pad() << "const int n = 8 * g;\n" << pad() << "const int t = " << element_of_slot(ls) << ";\n";
@@ -1105,9 +1108,10 @@ struct Gen {
                   std::string pred, addr = address(o.acc, l0, l1, pred);
                   os << pad() << "{\n";
                   indent++;
-                  os << pad() << "const u32x4_t *const src = " << (pred.empty() ? "" : "!(" + pred + ") ? (const u32x4_t *)tts_dummy : ") << "(const u32x4_t *)((const " << mt
+                  const std::string vt = mem_bytes(o.acc.elem) == 1 ? "u32x2_t" : "u32x4_t";
+                  os << pad() << "const " << vt << " *const src = " << (pred.empty() ? "" : "!(" + pred + ") ? (const " + vt + " *)tts_dummy : ") << "(const " << vt << " *)((const " << mt
                      << " *)p.ptr[" << o.acc.base_arg << "] + (" << addr << "));\n";
-                  if (is16(o.acc.elem)) os << pad() << "rw" << id << "[g] = src[0];\n";
+                  if (mem_bytes(o.acc.elem) <= 2) os << pad() << "rw" << id << "[g] = src[0];\n";
                   else {  // the second 16 bytes may lie on another page than the first: read only if their first element is valid
                     std::string pred4;
                     address(o.acc, along(ls, l0, " + 4").first, along(ls, l1, " + 4").second, pred4);
@@ -1129,6 +1133,8 @@ struct Gen {
                   if (is16(o.acc.elem)) {
                     const std::string word = "rw" + id + "[n >> 3][(n & 7) >> 1]";
                     got = std::string(o.acc.elem == "f16" ? "up_f16(" : "up_bf16(") + "(unsigned short)((n & 1) ? " + word + " >> 16 : " + word + "))";
+                  } else if (mem_bytes(o.acc.elem) == 1) {
+                    got = "(signed char)(rw" + id + "[n >> 3][(n & 7) >> 2] >> (8 * (n & 3)))";
                   } else {
                     const std::string word = "rw" + id + "[n >> 2][n & 3]";
                     got = o.acc.elem == "f32" ? "__uint_as_float(" + word + ")" : "(int)" + word;
@@ -1290,10 +1296,10 @@ struct Gen {
             if (two_phase && wide(shape) && vector_access(o.acc)) {
               // the eighth element of a group writes the group: one 16-byte access (two for 4-byte elements) when all
               // eight are valid and the first is 16-byte aligned, element by element otherwise
-              const bool half = is16(o.acc.elem);
+              const bool half = is16(o.acc.elem), byte = mem_bytes(o.acc.elem) == 1;
               const std::string sv = "sv" + std::to_string(q), mt = memtype(o.acc.elem), value = at(o.operands[0], i0, i1);
               const std::string bits = o.acc.elem == "f16" ? "(unsigned)down_f16_exact(" + value + ")" : o.acc.elem == "bf16" ? "(unsigned)down_bf16(" + value + ")"
-                                       : o.acc.elem == "f32" ? "__float_as_uint(" + value + ")" : "(unsigned)(" + value + ")";
+                                       : o.acc.elem == "f32" ? "__float_as_uint(" + value + ")" : byte ? "(unsigned)(unsigned char)(" + value + ")" : "(unsigned)(" + value + ")";
               os << pad() << sv << "[n & 7] = " << bits << ";\n";
               std::string pred_last, pred_e, addr0 = address(o.acc, along(shape, i0, " - 7").first, along(shape, i1, " - 7").second, pred_e);
               address(o.acc, i0, i1, pred_last);
@@ -1301,8 +1307,11 @@ struct Gen {
               os << pad() << "if ((n & 7) == 7) {\n";
               indent++;
               os << pad() << mt << " *const dst = (" << mt << " *)p.ptr[" << o.acc.base_arg << "] + (" << addr0 << ");\n";
-              os << pad() << "if (" << (pred_last.empty() ? "" : "(" + pred_last + ") && ") << "((unsigned long long)dst & 15) == 0) {\n";
-              if (half)
+              os << pad() << "if (" << (pred_last.empty() ? "" : "(" + pred_last + ") && ") << "((unsigned long long)dst & " << (byte ? 7 : 15) << ") == 0) {\n";
+              if (byte)
+                os << pad() << "  __builtin_nontemporal_store(u32x2_t{" << sv << "[0] | " << sv << "[1] << 8 | " << sv << "[2] << 16 | " << sv << "[3] << 24, " << sv << "[4] | " << sv
+                   << "[5] << 8 | " << sv << "[6] << 16 | " << sv << "[7] << 24}, (u32x2_t *)dst);\n";
+              else if (half)
                 os << pad() << "  __builtin_nontemporal_store(u32x4_t{" << sv << "[0] | " << sv << "[1] << 16, " << sv << "[2] | " << sv << "[3] << 16, " << sv << "[4] | " << sv
                    << "[5] << 16, " << sv << "[6] | " << sv << "[7] << 16}, (u32x4_t *)dst);\n";
               else
@@ -1310,7 +1319,7 @@ struct Gen {
                    << pad() << "  __builtin_nontemporal_store(u32x4_t{" << sv << "[4], " << sv << "[5], " << sv << "[6], " << sv << "[7]}, (u32x4_t *)dst + 1);\n";
               os << pad() << "} else {\n";
               os << pad() << "  #pragma unroll\n" << pad() << "  for (int e = 0; e < 8; e++)\n";
-              os << pad() << "    if (" << (pred_e.empty() ? "true" : pred_e) << ") " << (half ? "dst[e] = (unsigned short)" + sv + "[e]" : "((unsigned *)dst)[e] = " + sv + "[e]") << ";\n";
+              os << pad() << "    if (" << (pred_e.empty() ? "true" : pred_e) << ") " << (byte ? "dst[e] = (signed char)" + sv + "[e]" : half ? "dst[e] = (unsigned short)" + sv + "[e]" : "((unsigned *)dst)[e] = " + sv + "[e]") << ";\n";
               os << pad() << "}\n";
               indent--;
               os << pad() << "}\n";
@@ -2080,6 +2089,7 @@ __device__ inline long long srem32(long long a, long long b) {
 __device__ inline long long wrap(long long x, long long m) { return m > 0 ? ((x % m) + m) % m : x; }
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2_t __attribute__((ext_vector_type(2)));
 typedef unsigned short u16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
