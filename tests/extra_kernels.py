@@ -1301,3 +1301,16 @@ def dequantize_rows_int8(q_ptr, s_ptr, y_ptr, n_cols, pitch, BLOCK: tl.constexpr
     m = c < n_cols
     q = tl.load(q_ptr + row * pitch + c, mask=m, other=0)
     tl.store(y_ptr + row * pitch + c, (q.to(tl.float32) * tl.load(s_ptr + row)).to(y_ptr.dtype.element_ty), mask=m)
+
+
+@triton.jit
+def scale_rows_on_a_2d_grid(x_ptr, w_ptr, y_ptr, n_rows, n_cols, BLOCK: tl.constexpr):
+    # y[b, r, :] = x[b, r, :] * w + (b - r): one row per program, rows on program_id(0), batches on program_id(1); w is the
+    # same block for every program
+    r = tl.program_id(0)
+    b = tl.program_id(1)
+    c = tl.arange(0, BLOCK)
+    m = c < n_cols
+    w = tl.load(w_ptr + c, mask=m, other=0.0).to(tl.float32)
+    x = tl.load(x_ptr + (b * n_rows + r) * n_cols + c, mask=m, other=0.0).to(tl.float32)
+    tl.store(y_ptr + (b * n_rows + r) * n_cols + c, (x * w + (b - r)).to(y_ptr.dtype.element_ty), mask=m)

@@ -1791,6 +1791,32 @@ def test_tile_program_wide_blocks_of_rows_loops_and_mixed_widths():
             assert torch.equal(ki[lead:lead + n], torch.where(xs.float() > 0, o, -o)) and (ki[lead + n:] == 5).all()
 
 
+def test_tile_program_persistent_programs_walk_the_whole_grid():
+    """A program whose block of weights is the same for every program runs as a loop over programs in a launch of a few
+    workgroups per CU: more programs than such a launch has workgroups, on one- and two-dimensional grids."""
+    import extra_kernels as X
+    torch.manual_seed(3)
+    rows, n = 5000, 2048
+    x = torch.randn(rows, n, device=DEV).half()
+    w = (1 + 0.1 * torch.randn(n, device=DEV)).half()
+    y = torch.zeros_like(x)
+    k = K_mod().rms_norm_rows[(rows,)](x, w, y, n, n, 1e-6, BLOCK=2048)
+    torch.cuda.synchronize()
+    assert k.function.family == "tile_program"
+    xd = x.double()
+    want = xd / torch.sqrt((xd * xd).mean(1, keepdim=True) + 1e-6) * w.double()
+    assert (y.double() - want).abs().max() <= 4e-3 * want.abs().max().item()
+    batches, rows, n = 3, 700, 2040
+    x = torch.randn(batches, rows, n, device=DEV).bfloat16()
+    w = torch.randn(n, device=DEV).bfloat16()
+    y = torch.zeros_like(x)
+    X.scale_rows_on_a_2d_grid[(rows, batches)](x, w, y, rows, n, BLOCK=2048)
+    torch.cuda.synchronize()
+    shift = torch.arange(batches, device=DEV)[:, None, None] - torch.arange(rows, device=DEV)[None, :, None]
+    want = (x.float() * w.float() + shift.float()).bfloat16()
+    assert torch.equal(y, want)
+
+
 @pytest.mark.parametrize("n_cols,pitch,lead", [(4096, 4096, 0), (4000, 4000, 0), (4093, 4099, 0), (2048, 2048, 5)])
 def test_tile_program_wide_rows_with_int8_neighbours(n_cols, pitch, lead):
     """Row-wise int8 quantisation and its inverse: 1-byte blocks next to 16-bit ones take the wide element order too
