@@ -1785,8 +1785,13 @@ struct Gen {
         const size_t sz = held_bytes(val(s.operands[j]).dtype);
         os << pad() << Tn[j] << " *const wp" << id << "_" << j << " = (" << Tn[j] << " *)(pool + " << off << ");\n";
         off = (off + O * 4 * sz + 15) / 16 * 16;
-        decl << "  __shared__ " << Tn[j] << " out" << id << "_" << j << "[" << O << "];\n";
-        out_bytes += (O * sz + 15) / 16 * 16;
+        // (a single result: every thread folds the four wavefronts' partials itself and keeps the result in a register,
+        // which saves the round through LDS and a barrier)
+        if (O == 1) decl << "  " << Tn[j] << " out" << id << "_" << j << "[1];\n";
+        else {
+          decl << "  __shared__ " << Tn[j] << " out" << id << "_" << j << "[" << O << "];\n";
+          out_bytes += (O * sz + 15) / 16 * 16;
+        }
       }
       pool_bytes = std::max(pool_bytes, off);
       auto list = [&](const std::string &pre, const std::string &post) {
@@ -1830,13 +1835,15 @@ struct Gen {
       os << "}\n";
       indent--;
       os << pad() << "}\n" << pad() << "__syncthreads();\n";
-      os << pad() << "for (int o = threadIdx.x; o < " << O << "; o += 256) {\n";
+      if (O == 1) os << pad() << "{\n" << pad() << "  const int o = 0;\n";
+      else os << pad() << "for (int o = threadIdx.x; o < " << O << "; o += 256) {\n";
       indent++;
       for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " acc" << j << " = wp" << id << "_" << j << "[o * 4];\n";
-      os << pad() << "for (int w = 1; w < 4; w++) " << fname << "(" << list("acc", "") << ", " << list("wp" + id + "_", "[o * 4 + w]") << ", " << list("acc", "") << ");\n";
+      os << pad() << "#pragma unroll\n" << pad() << "for (int w = 1; w < 4; w++) " << fname << "(" << list("acc", "") << ", " << list("wp" + id + "_", "[o * 4 + w]") << ", " << list("acc", "") << ");\n";
       for (size_t j = 0; j < k; j++) os << pad() << "out" << id << "_" << j << "[o] = " << final_value(j, "acc" + std::to_string(j)) << ";\n";
       indent--;
-      os << pad() << "}\n" << pad() << "__syncthreads();\n";
+      os << pad() << "}\n";
+      if (O != 1) os << pad() << "__syncthreads();\n";
       cur_i0.clear();
       cur_i1.clear();
       return;
@@ -2131,6 +2138,19 @@ bool stores_walk_columns_with_pid1(const Program &p) {
 }  // namespace
 
 namespace {
+// Two barriers with nothing between them are one.
+std::string without_double_barriers(std::string src) {
+  const std::string bar = "__syncthreads();\n";
+  for (size_t pos = src.find(bar); pos != std::string::npos; pos = src.find(bar, pos + bar.size())) {
+    for (;;) {
+      size_t next = pos + bar.size(), q = next;
+      while (q < src.size() && src[q] == ' ') q++;
+      if (src.compare(q, bar.size(), bar) != 0) break;
+      src.erase(next, q + bar.size() - next);
+    }
+  }
+  return src;
+}
 // The body of a persistent kernel's program loop with the thread's index read from a variable that an empty asm renews in
 // every iteration: what depends on it alone -- 32 element masks, 32 64-bit element offsets -- is otherwise computed once,
 // before the loop, and held in registers for the whole launch (LayerNorm's input gradient: 211 registers instead of 149).
@@ -2189,7 +2209,7 @@ std::string tile_program_source(const Program &p, bool allow_persistent) {
   for (int b : g.all_inline_bases)
     if (g.all_store_bases.count(b))
       throw Unsupported("tile_program: an argument is both stored to and read by a load that is not of its body's block shape");
-  return all.str();
+  return without_double_barriers(all.str());
 }
 
 // What a matmul kernel does to its accumulator between the K loop and the store (an activation, a bias, a residual, the
