@@ -720,7 +720,7 @@ struct Gen {
       es.insert(es.end(), s.acc.dims.begin(), s.acc.dims.end());
       bool fixed = true;
       for (int e : es)
-        for (EK k : {EK::Pid, EK::IV, EK::Iter, EK::Result, EK::Data}) fixed = fixed && (e < 0 || !P.pool.depends_on(e, k));
+        for (EK k : {EK::Pid, EK::NProg, EK::IV, EK::Iter, EK::Result, EK::Data}) fixed = fixed && (e < 0 || !P.pool.depends_on(e, k));  // (what the code before the program loop can name: arguments and constants)
       if (fixed) hoisted.insert(s.result);
     }
     persistent = !hoisted.empty();
