@@ -270,10 +270,12 @@ def test_gemm_whole_tile_kernel(K, M, N, Kd, dtype, pad):
 
 
 @pytest.mark.parametrize("M,N,Kd,dtype,bt", [(128, 4096, 4096, torch.bfloat16, False), (300, 1032, 2048, torch.float16, False), (512, 2048, 8192, torch.bfloat16, True),
-                                            (1000, 2048, 4096, torch.bfloat16, False), (64, 8192, 8192, torch.float16, False), (1, 256, 4096, torch.bfloat16, False)])
+                                            (1000, 2048, 4096, torch.bfloat16, False), (64, 8192, 8192, torch.float16, False), (1, 256, 4096, torch.bfloat16, False),
+                                            (512, 8192, 8192, torch.bfloat16, False), (500, 4104, 8192, torch.float16, False), (768, 2048, 16384, torch.bfloat16, False)])
 def test_gemm_in_k_slices_for_skinny_products(K, M, N, Kd, dtype, bt):
     """Products with too few output tiles for the chip run with K cut into slices (a workgroup per tile and slice, fp32
-    partial sums, a second kernel that adds them and narrows): exact on small-integer operands whatever the order of
+    partial sums; a second kernel adds them and narrows, or, on 256 x 256 tiles, the slice of a tile that arrives last
+    does): exact on small-integer operands whatever the order of
     the sums, ragged rows and columns, a column-major B, the buffer around C untouched; twice on one stream (the second
     launch reuses the workspace) and once more on another stream (a workspace of its own)."""
     g = torch.Generator(device="cpu").manual_seed(M + N + Kd)
