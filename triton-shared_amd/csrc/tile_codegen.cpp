@@ -1123,7 +1123,12 @@ struct Gen {
                 }
               indent--;
               os << pad() << "}\n";
-              open_element_loop(ls);
+              bool any_packed = false, any_unpacked = false;
+              for (size_t q = k; q < end; q++) {
+                any_packed = any_packed || (wide_load(ops[q]) && packed(ops[q]));
+                any_unpacked = any_unpacked || (wide_load(ops[q]) && !packed(ops[q]));
+              }
+              if (any_unpacked) open_element_loop(ls);
               for (size_t q = k; q < end; q++)
                 if (wide_load(ops[q]) && !packed(ops[q])) {
                   const SOp &o = ops[q];
@@ -1141,19 +1146,19 @@ struct Gen {
                   }
                   os << pad() << "ld" << id << "[n] = " << (pred.empty() ? got : "(" + pred + ") ? " + got + " : " + other_of(o.acc, l0, l1)) << ";\n";
                 }
-              close_loop();
+              if (any_unpacked) close_loop();
               indent--;
               os << pad() << "} else {\n";
               indent++;
               for (size_t q = k; q < end; q++)
                 if (wide_load(ops[q]) && packed(ops[q])) os << pad() << "unsigned tm" << ops[q].result << "[" << count(ls) / 256 << "] = {};\n";
-              open_element_loop(ls);
+              if (any_packed) open_element_loop(ls);
               for (size_t q = k; q < end; q++)
                 if (wide_load(ops[q]) && packed(ops[q])) {
                   std::string pred, addr = address(ops[q].acc, l0, l1, pred);
                   os << pad() << (pred.empty() ? "" : "if (" + pred + ") ") << "tm" << ops[q].result << "[n] = ((const unsigned short *)p.ptr[" << ops[q].acc.base_arg << "])[" << addr << "];\n";
                 }
-              close_loop();
+              if (any_packed) close_loop();
               for (size_t q = k; q < end; q++)
                 if (wide_load(ops[q]) && packed(ops[q])) {
                   os << pad() << "#pragma unroll\n" << pad() << "for (int g = 0; g < " << G << "; g++)\n";
@@ -1162,7 +1167,7 @@ struct Gen {
                     os << (c ? ", " : "") << "tm" << ops[q].result << "[8 * g + " << 2 * c << "] | tm" << ops[q].result << "[8 * g + " << 2 * c + 1 << "] << 16";
                   os << "};\n";
                 }
-              open_element_loop(ls);
+              if (any_unpacked) open_element_loop(ls);
               for (size_t q = k; q < end; q++)
                 if (wide_load(ops[q]) && !packed(ops[q])) {
                   const SOp &o = ops[q];
@@ -1173,7 +1178,7 @@ struct Gen {
                     os << pad() << "if (" << pred << ") " << name << "[n] = __uint_as_float(((const unsigned short *)p.ptr[" << o.acc.base_arg << "])[" << addr << "]);\n";
                   else os << pad() << "if (" << pred << ") " << name << "[n] = " << mem_read(o.acc, addr) << ";\n";
                 }
-              close_loop();
+              if (any_unpacked) close_loop();
               bool any_masked = false;
               for (size_t q = k; q < end; q++) any_masked = any_masked || (wide_load(ops[q]) && !packed(ops[q]) && !ops[q].acc.dims.empty());
               if (any_masked) {
