@@ -1819,6 +1819,30 @@ def test_tile_program_persistent_programs_walk_the_whole_grid():
     assert torch.equal(y, want)
 
 
+def test_tile_program_wide_rows_of_random_extent_and_alignment():
+    """Seeded random row counts, row lengths, pitches and starting offsets through a wide, persistent elementwise program
+    (16-bit rows scaled by a shared vector): bit-exact against torch, nothing written outside the rows."""
+    import extra_kernels as X
+    rng = torch.Generator(device="cpu").manual_seed(77)
+    for trial in range(24):
+        dt = (torch.float16, torch.bfloat16)[trial % 2]
+        batches = int(torch.randint(1, 4, (1,), generator=rng))
+        rows = int(torch.randint(1, 40, (1,), generator=rng))
+        n = int(torch.randint(1, 2049, (1,), generator=rng))
+        lead = int(torch.randint(0, 9, (1,), generator=rng))
+        total = batches * rows * n
+        xb = torch.randn(lead + total + 8, device=DEV).to(dt)
+        wb = torch.randn(lead + n + 8, device=DEV).to(dt)
+        yb = torch.full((lead + total + 8,), 5.0, device=DEV, dtype=dt)
+        x, w, y = xb[lead:lead + total].view(batches, rows, n), wb[lead:lead + n], yb[lead:lead + total].view(batches, rows, n)
+        X.scale_rows_on_a_2d_grid[(rows, batches)](x, w, y, rows, n, BLOCK=2048)
+        torch.cuda.synchronize()
+        shift = torch.arange(batches, device=DEV)[:, None, None] - torch.arange(rows, device=DEV)[None, :, None]
+        want = (x.float() * w.float() + shift.float()).to(dt)
+        assert torch.equal(y, want), (trial, batches, rows, n, lead)
+        assert (yb[:lead] == 5.0).all() and (yb[lead + total:] == 5.0).all(), (trial, batches, rows, n, lead)
+
+
 @pytest.mark.parametrize("n_cols,pitch,lead", [(4096, 4096, 0), (4000, 4000, 0), (4093, 4099, 0), (2048, 2048, 5)])
 def test_tile_program_wide_rows_with_int8_neighbours(n_cols, pitch, lead):
     """Row-wise int8 quantisation and its inverse: 1-byte blocks next to 16-bit ones take the wide element order too
