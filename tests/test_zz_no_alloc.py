@@ -91,6 +91,11 @@ def test_noalloc_launch_runs_a_skinny_matmul_in_k_slices_from_the_static_array(n
         plan.launch(grid, stream, [a.data_ptr(), b.data_ptr(), want.data_ptr(), M, N, Kd, Kd, N, N])
         torch.cuda.synchronize()
         assert plan.last_kernel.endswith("K slices"), plan.last_kernel
+        # (the entry point's first call on a device looks the static array's address up, which is when the runtime gives
+        # the array its memory: free memory is compared around a later call)
+        plan.launch_noalloc(grid, stream, [a.data_ptr(), b.data_ptr(), got.data_ptr(), M, N, Kd, Kd, N, N])
+        torch.cuda.synchronize()
+        got.fill_(7.0)
         free_before = torch.cuda.mem_get_info()[0]
         plan.launch_noalloc(grid, stream, [a.data_ptr(), b.data_ptr(), got.data_ptr(), M, N, Kd, Kd, N, N])
         torch.cuda.synchronize()
