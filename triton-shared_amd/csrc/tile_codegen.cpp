@@ -698,6 +698,11 @@ struct Gen {
   // code goes to hoist_os).  Read again by every program they stay in L2, but the L2 -> CU traffic is that of a second
   // row (RMSNorm fp16 [4096, 8192]: 27.5 -> 25.5 us).
   bool persistent = false;
+  // In a persistent kernel every wide 16-bit load stays packed (two elements per register, widened where used): RMSNorm
+  // on rows of 8192 then takes 75 registers instead of 111.  (With a workgroup per program the compiler keeps packed and
+  // widened values side by side and takes more registers than without: 121 against 108; the launcher compiles that form,
+  // unpacked, when the persistent one holds too few workgroups per CU.)
+  bool pack_wide = false;
   std::set<int> hoisted;  // value ids of the loads emitted before the program loop
   std::ostringstream hoist_os;
   std::ostringstream loop_top;  // first statements of the program loop
@@ -724,6 +729,7 @@ struct Gen {
       if (fixed) hoisted.insert(s.result);
     }
     persistent = !hoisted.empty();
+    pack_wide = persistent;
   }
   std::string element_of_slot(const std::vector<int64_t> &shape) const {
     return wide(shape) ? "8 * (int)threadIdx.x + (n & 7) + 2048 * (n >> 3)" : "threadIdx.x + 256 * n";
@@ -1021,7 +1027,9 @@ struct Gen {
           bool any = false;
           for (size_t q = k; q < end; q++)
             if (mine_here(ops[q])) {
-              if (hoisted.count(ops[q].result)) {
+              if (pack_wide && !hoisted.count(ops[q].result) && wide(ls) && vector_access(ops[q].acc) && is16(ops[q].acc.elem))
+                os << pad() << "u32x4_t rw" << ops[q].result << "[" << count(ls) / 2048 << "];\n";
+              else if (hoisted.count(ops[q].result)) {
                 // (16-bit blocks that stay in registers for the whole launch stay packed, two elements per register, and
                 // are widened where they are used)
                 if (is16(ops[q].acc.elem)) {
@@ -1076,7 +1084,7 @@ struct Gen {
               os.swap(hoist_os);
               indent = 1;
             }
-            auto packed = [&](const SOp &o) { return pass == 0 && is16(o.acc.elem); };
+            auto packed = [&](const SOp &o) { return (pass == 0 || pack_wide) && is16(o.acc.elem); };
             bool any_wide = false;
             for (size_t q = k; q < end; q++) any_wide = any_wide || wide_load(ops[q]);
             if (any_wide) {
