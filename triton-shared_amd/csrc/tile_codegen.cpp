@@ -58,15 +58,16 @@ struct Gen {
   // all threads', so the two are kept apart by barriers wherever they may touch the same argument.
   std::set<int> read_bases_anywhere, scalar_store_bases_anywhere;
   std::map<int, int> uses;  // value id -> how many operands of the program name it
+  std::map<int, std::vector<const SOp *>> users;  // value id -> the ops that name it
   void collect_bases(const std::vector<SOp> &ops) {
     for (const SOp &s : ops) {
       if (s.kind == SK::Load || s.kind == SK::ScalarLoad) read_bases_anywhere.insert(s.acc.base_arg);
       if (s.kind == SK::ScalarStore) scalar_store_bases_anywhere.insert(s.acc.base_arg);
-      for (int v : s.operands) uses[v]++;
-      for (int v : s.tile_inits) uses[v]++;
-      for (int v : s.tile_yields) uses[v]++;
+      for (int v : s.operands) uses[v]++, users[v].push_back(&s);
+      for (int v : s.tile_inits) uses[v]++, users[v].push_back(&s);
+      for (int v : s.tile_yields) uses[v]++, users[v].push_back(&s);
       for (int v : {s.acc.gather, s.acc.mask_value, s.acc.other_value})
-        if (v >= 0) uses[v]++;
+        if (v >= 0) uses[v]++, users[v].push_back(&s);
       if (s.kind == SK::For || s.kind == SK::If) collect_bases(s.body);
     }
   }
@@ -87,6 +88,26 @@ struct Gen {
       if (costly(x, depth + 1)) return true;
     return false;
   }
+  // Is v only ever read element by element, by ops over blocks of its own shape (through any chain of elementwise ops,
+  // down to block stores)?  Then the thread that owns an element is the only one that needs it.
+  bool read_in_place_only(int v, const std::vector<int64_t> &shape, int depth = 0) {
+    if (depth > 32) return false;
+    auto u = users.find(v);
+    if (u == users.end()) return true;
+    for (const SOp *o : u->second) {
+      if (o->kind == SK::Store) {
+        if (o->acc.sizes != shape || o->acc.gather == v) return false;  // (offsets of a scatter are read by index expressions)
+        continue;
+      }
+      if (o->kind != SK::Map || o->result < 0 || val(o->result).shape != shape) return false;
+      if (o->name.rfind("tt.", 0) == 0 && o->name != "tt.clampf.none" && o->name != "tt.clampf.all" && o->name != "tt.precise_sqrt" && o->name != "tt.precise_divf" &&
+          o->name != "tt.mulhiui" && o->name != "tt.bitcast")
+        return false;  // transposes, reshapes, joins and the like read other elements
+      if (!read_in_place_only(o->result, shape, depth + 1)) return false;
+    }
+    return true;
+  }
+  std::vector<int> kept_by_scan;  // results of the last scan that stay in the owning threads' registers (see reduce())
   std::ostringstream fns;                           // combiner functions of reductions and scans (before the kernel)
   std::ostringstream decl;                          // LDS arrays holding their results (top of the kernel)
   size_t pool_bytes = 0, out_bytes = 0;             // staging pool shared by all reductions; result arrays
@@ -892,6 +913,8 @@ struct Gen {
             mine.push_back(o);
           }
         reduce(s, shape);
+        mine.insert(mine.end(), kept_by_scan.begin(), kept_by_scan.end());
+        kept_by_scan.clear();
         k++;
         continue;
       }
@@ -1868,6 +1891,10 @@ struct Gen {
       std::vector<std::string> Tn(k);
       const int64_t LQ = L / 256, slots = O * LQ;
       size_t off = 0;
+      // Results that are only read element by element, in blocks of this shape, stay in the registers of the threads that
+      // own them: no copy in LDS, and no barrier after the last step.
+      bool in_registers = true;
+      for (size_t j = 0; j < k; j++) in_registers = in_registers && read_in_place_only(s.results.empty() ? s.result : s.results[j], shape);
       os << pad() << "__syncthreads();\n";
       for (size_t j = 0; j < k; j++) {
         Tn[j] = ctype(val(s.operands[j]).dtype);
@@ -1876,8 +1903,10 @@ struct Gen {
         off = (off + slots * 4 * sz + 15) / 16 * 16;
         os << pad() << Tn[j] << " *const wq" << id << "_" << j << " = (" << Tn[j] << " *)(pool + " << off << ");\n";  // what precedes each piece in its line
         off = (off + slots * 4 * sz + 15) / 16 * 16;
-        decl << "  __shared__ " << Tn[j] << " out" << id << "_" << j << "[" << T << "];\n";
-        out_bytes += (T * sz + 15) / 16 * 16;
+        if (!in_registers) {
+          decl << "  __shared__ " << Tn[j] << " out" << id << "_" << j << "[" << T << "];\n";
+          out_bytes += (T * sz + 15) / 16 * 16;
+        }
       }
       pool_bytes = std::max(pool_bytes, off);
       auto list = [&](const std::string &pre, const std::string &post) {
@@ -1948,9 +1977,21 @@ struct Gen {
       os << pad() << "const int first = (n / " << LQ << ") * " << LQ * 4 << ", pieces = (n % " << LQ << ") * 4 + (threadIdx.x >> 6);\n";
       for (size_t j = 0; j < k; j++) os << pad() << Tn[j] << " res" << j << " = sc" << id << "_" << j << "[n];\n";
       os << pad() << "if (pieces > 0) " << fname << "(" << list("wq" + id + "_", "[first + pieces]") << ", " << list("sc" + id + "_", "[n]") << ", " << list("res", "") << ");\n";
-      for (size_t j = 0; j < k; j++) os << pad() << "out" << id << "_" << j << "[t] = res" << j << ";\n";
+      for (size_t j = 0; j < k; j++) {
+        if (in_registers) os << pad() << "sc" << id << "_" << j << "[n] = res" << j << ";\n";
+        else os << pad() << "out" << id << "_" << j << "[t] = res" << j << ";\n";
+      }
       indent--;
-      os << pad() << "}\n" << pad() << "__syncthreads();\n";
+      os << pad() << "}\n";
+      if (in_registers) {
+        for (size_t j = 0; j < k; j++) {
+          const int r = s.results.empty() ? s.result : s.results[j];
+          held[r] = {"sc" + id + "_" + std::to_string(j), shape};
+          kept_by_scan.push_back(r);
+        }
+      } else {
+        os << pad() << "__syncthreads();\n";
+      }
       cur_i0.clear();
       cur_i1.clear();
       return;
