@@ -740,12 +740,12 @@ tts_status launch_impl(tts_plan *plan, int gx, int gy, int gz, void *stream, con
           hipError_t ce = rtc_compile(source, "tile_program", slot, &why);
           if (ce != hipSuccess) return fail(TTS_HIP_ERROR, "tile_program: " + why + "\n--- source ---\n" + source);
           // A persistent kernel keeps what its programs share in registers.  When that costs it workgroups per CU (fewer
-          // than four fit), the kernel with a workgroup per program is compiled as well, and the one of which more fit
-          // is kept (LayerNorm's input gradient on rows of 8192: 2 against 3 per CU, 50 us against 41).
+          // than four fit), the kernel with a workgroup per program is compiled as well, and kept unless fewer of it fit
+          // (LayerNorm's input gradient on rows of 8192: 2 against 3 per CU, 50 us against 41).
           if (slot == &plan->fused && tile_program_is_persistent(source) && rtc_resident_workgroups(*slot) < 4) {
             const std::string plain = tile_program_source(pl.prog, false);
             RtcModule *other = nullptr;
-            if (rtc_compile(plain, "tile_program", &other, &why) == hipSuccess && rtc_resident_workgroups(other) > rtc_resident_workgroups(*slot)) {
+            if (rtc_compile(plain, "tile_program", &other, &why) == hipSuccess && rtc_resident_workgroups(other) >= rtc_resident_workgroups(*slot)) {
               rtc_release(*slot);
               *slot = other;
               plan->fused_is_plain = true;
