@@ -277,6 +277,17 @@ def make_workloads(torch, triton, K):
         return dict(desc=f"independent stream ceiling, 1:1 read/write: the HIP runtime's device-to-device copy of fp32 N={n} (not a kernel of this backend){what}",
                     work=8 * n, bound="hbm", dtype="f32", make=make, set_bytes=8 * n)
 
+    def vendor_matmul(n):
+        # the vendor library's product of the same operands (what torch.matmul enqueues for two bf16 matrices: hipBLASLt): a
+        # kernel this backend did not write, timed the same way, as an independent figure for what the machine reaches on cfg4
+        def make():
+            a = (torch.randn(n, n, device=dev) * 0.02).bfloat16()
+            b = (torch.randn(n, n, device=dev) * 0.02).bfloat16()
+            c = torch.empty(n, n, dtype=torch.bfloat16, device=dev)
+            return dict(direct=lambda: torch.matmul(a, b, out=c), kernel="torch.matmul (hipBLASLt, not this backend)")
+        return dict(desc=f"independent reference for cfg4: torch.matmul of the same bf16 {n}x{n}x{n} operands (the vendor library, not a kernel of this backend)",
+                    work=2 * n ** 3, bound="mfma", dtype="bf16", make=make, set_bytes=3 * n * n * 2)
+
     def stream_read(n):
         def make():
             x = torch.rand(n, device=dev)
@@ -293,6 +304,7 @@ def make_workloads(torch, triton, K):
     W["cfg1_2p28"] = vec_add(1 << 28)
     W["cfg2_1m"] = softmax(1 << 20)
     W["diag_cfg4_zero_operands"] = gemm(zeros=True)
+    W["ref_vendor_matmul_as_cfg4"] = vendor_matmul(4096)
     W["stream_copy_2p28"] = stream_copy(1 << 28)
     W["stream_read_2p28"] = stream_read(1 << 28)
     W["stream_runtime_copy_2p28"] = runtime_copy(1 << 28)
