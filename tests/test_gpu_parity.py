@@ -1819,6 +1819,39 @@ def test_tile_program_persistent_programs_walk_the_whole_grid():
     assert torch.equal(y, want)
 
 
+def test_tile_program_wide_and_ordinary_element_order_agree(monkeypatch):
+    """The same program planned with and without the wide element order (and with and without the program loop) writes
+    the same bits: an elementwise program exactly, a program with a row reduction to within the reduction's rounding."""
+    import extra_kernels as X
+    from triton_shared_amd import _native as native
+    from test_planner import compile_ttir
+    torch.manual_seed(21)
+    stream = torch.cuda.current_stream().cuda_stream
+    batches, rows, n = 2, 37, 2040
+    x = torch.randn(batches, rows, n, device=DEV).bfloat16()
+    w = torch.randn(n, device=DEV).bfloat16()
+    sig = {"x_ptr": "*bf16", "w_ptr": "*bf16", "y_ptr": "*bf16", "n_rows": "i32", "n_cols": "i32", "BLOCK": "constexpr"}
+    ttir = compile_ttir(X.scale_rows_on_a_2d_grid, sig, {"BLOCK": 2048})
+    sig2 = {"x_ptr": "*bf16", "w_ptr": "*bf16", "y_ptr": "*bf16", "pitch": "i32", "n_cols": "i32", "eps": "fp32", "BLOCK": "constexpr"}
+    ttir2 = compile_ttir(K_mod().rms_norm_rows, sig2, {"BLOCK": 2048})
+    outs, norms = [], []
+    for wide, persistent in (("1", "1"), ("1", "0"), ("0", "0")):
+        monkeypatch.setenv("TTS_TILE_WIDE", wide)
+        monkeypatch.setenv("TTS_TILE_PERSISTENT", persistent)
+        plan = native.PlanHandle(native.structured_to_plan(native.ttir_to_structured(ttir))[0])
+        y = torch.zeros_like(x)
+        plan.launch((rows, batches, 1), stream, [x.data_ptr(), w.data_ptr(), y.data_ptr(), rows, n])
+        plan2 = native.PlanHandle(native.structured_to_plan(native.ttir_to_structured(ttir2))[0])
+        z = torch.zeros(batches * rows, n, device=DEV, dtype=torch.bfloat16)
+        plan2.launch((batches * rows, 1, 1), stream, [x.data_ptr(), w.data_ptr(), z.data_ptr(), n, n, 1e-6])
+        torch.cuda.synchronize()
+        outs.append(y)
+        norms.append(z)
+    assert torch.equal(outs[0], outs[2]) and torch.equal(outs[1], outs[2])
+    for z in norms[:2]:
+        assert (z.float() - norms[2].float()).abs().max() <= 2e-2 * norms[2].float().abs().max()
+
+
 def test_tile_program_wide_rows_of_random_extent_and_alignment():
     """Seeded random row counts, row lengths, pitches and starting offsets through a wide, persistent elementwise program
     (16-bit rows scaled by a shared vector): bit-exact against torch, nothing written outside the rows."""
